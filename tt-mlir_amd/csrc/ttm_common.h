@@ -1,0 +1,61 @@
+// Shared helpers of the gfx950 kernel library: error reporting, launch checks, tile addressing.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "ttmlir_amd_hip.h"
+
+// native clang vectors (usable with the nontemporal load/store builtins)
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define TTM_EXPORT extern "C" __attribute__((visibility("default")))
+
+int ttm_set_error(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+
+#define TTM_HIP(expr)                                                                          \
+  do {                                                                                         \
+    hipError_t _e = (expr);                                                                    \
+    if (_e != hipSuccess)                                                                      \
+      return ttm_set_error(TTM_ERR_HIP, "%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), \
+                           __FILE__, __LINE__);                                                \
+  } while (0)
+
+#define TTM_REQUIRE(cond, ...)                                        \
+  do {                                                                \
+    if (!(cond)) return ttm_set_error(TTM_ERR_INVALID, __VA_ARGS__);  \
+  } while (0)
+
+#define TTM_LAUNCH_CHECK() TTM_HIP(hipGetLastError())
+
+int ttm_option(const char *name);  // 0 when unset
+
+static inline int64_t ttm_round_up32(int64_t v) { return (v + 31) / 32 * 32; }
+static inline int64_t ttm_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+static inline int ttm_dtype_bytes(int dtype) {
+  switch (dtype) {
+  case TTM_F32: case TTM_U32: case TTM_I32: return 4;
+  case TTM_F16: case TTM_BF16: case TTM_U16: return 2;
+  case TTM_U8: return 1;
+  default: return 0;
+  }
+}
+
+// Element offset of (r, c) inside a tiled [Rt*32, Ct*32] matrix: tiles row-major, faces
+// (0,0) (0,1) (1,0) (1,1), 16 contiguous elements per face row.
+__host__ __device__ static inline int64_t ttm_tiled_offset(int64_t r, int64_t c, int64_t ct) {
+  int64_t tile = (r >> 5) * ct + (c >> 5);
+  int face = (int)(((r >> 4) & 1) * 2 + ((c >> 4) & 1));
+  return tile * 1024 + face * 256 + (r & 15) * 16 + (c & 15);
+}
+
+__device__ static inline float ttm_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
+__device__ static inline uint16_t ttm_f32_to_bf16(float f) {  // round to nearest even, quiet NaN
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);
+  u += 0x7FFFu + ((u >> 16) & 1);
+  return (uint16_t)(u >> 16);
+}
