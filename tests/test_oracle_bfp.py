@@ -120,7 +120,8 @@ def test_invariants(orc, fmt, W):
     _, ex = np.frexp(np.max(np.abs(t), axis=1))
     unit = np.ldexp(1.0, ex - 1 - (W - 1))[:, None]
     sat = np.abs(ty) == unit * (2 ** W - 1)
-    assert np.all((np.abs(t - ty) <= unit / 2) | sat)
+    # alignment bits are truncated before rounding, so a hair over half a unit is possible
+    assert np.all((np.abs(t - ty) <= unit / 2 * (1 + 2.0 ** -16)) | sat)
     assert np.all(np.abs(t - ty)[sat] <= unit.repeat(16, 1)[sat])
     # sign symmetry
     yn = orc.bfp_unpack(orc.bfp_pack(-x, fmt), x.shape, fmt)
