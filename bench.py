@@ -1,0 +1,243 @@
+"""Benchmark of the hot path on one MI355X.
+
+Primary line (BASELINE.json metric "bfp8_b matmul TFLOP/s ..."): the config-3 linear layer at
+M=2048 -- bf16 activations [2048,4096] x bfp8_b weights [4096,14336], fused bias + GELU, fp32
+accumulate -- one kernel launch per step, inputs resident in HBM.  The same JSON line carries
+the pack / unpack / tilize bandwidth figures of config 2 and the decode-shape (M=32) linear under
+"secondary", each with its own roofline object, and the CPU baseline timed on this host.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload linear2048|pack_bfp8|...]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import __graft_entry__ as entry  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0        # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA peak
+
+
+def _events_time(hip, stream, fn, steps):
+    a, b = hip.Event(), hip.Event()
+    a.record(stream)
+    for _ in range(steps):
+        fn()
+    b.record(stream)
+    b.sync()
+    return a.elapsed_ms(b) / steps
+
+
+def _wall_time(torch, fn, steps):
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+class Workload:
+    """name, bound ('hbm'|'mfma'), algorithmic work per launch, fn() launching exactly one kernel."""
+
+    def __init__(self, name, bound, work, unit_work, fn, desc, extra=None):
+        self.name, self.bound, self.work, self.unit_work, self.fn, self.desc = name, bound, work, unit_work, fn, desc
+        self.extra = extra or {}
+
+
+def make_workloads(torch, hip, datagen, dev, names):
+    s = hip.current_stream()
+    out = {}
+    R = C = 8192
+    ntiles = (R // 32) * (C // 32)
+    need_c2 = any(n in names for n in ("pack_bfp8", "unpack_bfp8", "pack_bfp4", "unpack_bfp4", "tilize_f32",
+                                       "untilize_f32", "copy"))
+    if need_c2:
+        x = datagen.c2_outliers(R, C, seed=0).to(dev)
+        y = torch.empty_like(x)
+        for fmt, nm in ((hip.BFP8B, "bfp8"), (hip.BFP4B, "bfp4")):
+            tb = hip.bfp_tile_bytes(fmt)
+            p = torch.empty(ntiles * tb, dtype=torch.uint8, device=dev)
+            hip.call("ttm_bfp_pack", hip.ptr(x), hip.F32, hip.ROW_MAJOR, hip.ptr(p), fmt, 1, R, C, s)
+            work = R * C * 4 + ntiles * tb
+            out["pack_" + nm] = Workload(
+                "pack_" + nm, "hbm", work, "bytes",
+                (lambda p=p, fmt=fmt: hip.call("ttm_bfp_pack", hip.ptr(x), hip.F32, hip.ROW_MAJOR, hip.ptr(p), fmt, 1, R, C, s)),
+                "config 2: fp32 [8192,8192] row-major -> %s_b tiles (tilize fused)" % nm)
+            out["unpack_" + nm] = Workload(
+                "unpack_" + nm, "hbm", work, "bytes",
+                (lambda p=p, fmt=fmt: hip.call("ttm_bfp_unpack", hip.ptr(p), fmt, hip.ptr(y), hip.F32, hip.ROW_MAJOR, 1, R, C, s)),
+                "config 2: %s_b tiles -> fp32 [8192,8192] row-major (untilize fused)" % nm)
+        out["tilize_f32"] = Workload("tilize_f32", "hbm", 2 * R * C * 4, "bytes",
+                                     lambda: hip.call("ttm_tilize", hip.ptr(x), hip.ptr(y), 1, R, C, 4, s),
+                                     "config 2: tilize fp32 [8192,8192]")
+        out["untilize_f32"] = Workload("untilize_f32", "hbm", 2 * R * C * 4, "bytes",
+                                       lambda: hip.call("ttm_untilize", hip.ptr(x), hip.ptr(y), 1, R, C, 4, s),
+                                       "config 2: untilize fp32 [8192,8192]")
+        out["copy"] = Workload("copy", "hbm", 2 * R * C * 4, "bytes",
+                               lambda: hip.call("ttm_copy_kernel", hip.ptr(x), hip.ptr(y), R * C * 4, s),
+                               "plain 16 B/lane copy of 256 MiB (measured HBM ceiling)")
+    for M in (2048, 32):
+        nm = "linear%d" % M
+        if nm not in names:
+            continue
+        K, N = 4096, 14336
+        a, w, bias = datagen.c3_linear(M)
+        ad, wd, bd = a.to(dev), w.to(dev), bias.reshape(1, -1).to(dev)
+        at = torch.empty(M * K, dtype=torch.bfloat16, device=dev)
+        hip.call("ttm_tilize", hip.ptr(ad), hip.ptr(at), 1, M, K, 2, s)
+        wt = torch.empty((K // 32) * (N // 32) * 1088, dtype=torch.uint8, device=dev)
+        hip.call("ttm_bfp_pack", hip.ptr(wd), hip.F32, hip.ROW_MAJOR, hip.ptr(wt), hip.BFP8B, 1, K, N, s)
+        bt = torch.zeros(32 * N, dtype=torch.bfloat16, device=dev)
+        hip.call("ttm_tilize", hip.ptr(bd), hip.ptr(bt), 1, 1, N, 2, s)
+        ot = torch.empty(M * N, dtype=torch.bfloat16, device=dev)
+        torch.cuda.synchronize()
+        del wd
+        fn = (lambda at=at, wt=wt, bt=bt, ot=ot, M=M: hip.call(
+            "ttm_linear", hip.ptr(at), hip.BF16, hip.ptr(wt), hip.BFP8B, 0, hip.ptr(bt), hip.BF16, hip.TILE,
+            hip.ptr(ot), hip.BF16, 1, 1, M, N, K, hip.ACT["gelu"], s))
+        if M == 2048:
+            out[nm] = Workload(nm, "mfma", 2.0 * M * N * K, "flop", fn,
+                               "config 3: bf16 [2048,4096] x bfp8_b [4096,14336] + bias + GELU",
+                               dict(host=(a, w, bias), dev=(at, wt, bt, ot)))
+        else:
+            nbytes = (K // 32) * (N // 32) * 1088 + 2 * M * K + 2 * M * N + 2 * N
+            out[nm] = Workload(nm, "hbm", nbytes, "bytes", fn,
+                               "config 3 decode: bf16 [32,4096] x bfp8_b [4096,14336] + bias + GELU (weight streaming)",
+                               dict(flop=2.0 * M * N * K))
+    return out
+
+
+def roofline(w, kernel_ms):
+    if w.bound == "hbm":
+        achieved = w.work / (kernel_ms * 1e-3) / 1e9
+        peak, unit = HBM_PEAK_GBS, "GB/s"
+    else:
+        achieved = w.work / (kernel_ms * 1e-3) / 1e12
+        peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+    return {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": None, "kernel_us": round(kernel_ms * 1e3, 2),
+            "algorithmic_work": w.work, "work_unit": w.unit_work}
+
+
+def cpu_baseline_linear(orc, datagen, budget_rows=256):
+    """The CPU path (scalar f32 loops, one thread) on a row sample of config 3, M=2048."""
+    import numpy as np
+    import torch
+    a, w, bias = datagen.c3_linear(2048)
+    weff = orc.bfp_unpack(orc.bfp_pack(w.numpy(), 8), w.shape, 8)      # the weights the device multiplies
+    rows = a[:budget_rows].float().numpy()
+    K, N = w.shape
+    orc.set_threads(1)
+    t0 = time.perf_counter()
+    y = orc.linear(rows, weff, bias.float().numpy(), "gelu", rowstream=True)
+    dt = time.perf_counter() - t0
+    one = 2.0 * budget_rows * N * K / dt / 1e12
+    cores = min(16, orc.max_threads())
+    orc.set_threads(cores)
+    big = a[:budget_rows * 4].float().numpy()
+    t0 = time.perf_counter()
+    orc.linear(big, weff, bias.float().numpy(), "gelu", rowstream=True)
+    dtn = time.perf_counter() - t0
+    orc.set_threads(1)
+    alln = 2.0 * budget_rows * 4 * N * K / dtn / 1e12
+    return {"value": round(one, 6), "unit": "TFLOP/s", "cores": 1, "kind": "port",
+            "sample": "oracle scalar f32 linear+bias+GELU on rows 0..%d of config 3 (M=2048, K=4096, N=14336), "
+                      "dequantised bfp8_b weights, %.1f s" % (budget_rows - 1, dt),
+            "all_cores": {"value": round(alln, 6), "cores": cores, "rows": budget_rows * 4, "seconds": round(dtn, 2)}}, y
+
+
+def cpu_baseline_pack(orc, datagen, rows=8192):
+    x = datagen.c2_outliers(rows, 8192, seed=0).numpy()
+    orc.set_threads(1)
+    t0 = time.perf_counter()
+    orc.bfp_pack(x, 8)
+    dt = time.perf_counter() - t0
+    nbytes = rows * 8192 * 4 + (rows // 32) * 256 * 1088
+    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "oracle bfp8_b pack of %d x 8192 fp32 rows of config 2, %.2f s" % (rows, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="linear2048")
+    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (one MI355X per box); run with --gpus 1",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    entry.load_package()
+    from ttmlir_amd import hip, datagen
+    hip.lib()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    stream = hip.current_stream()
+    sec_names = [n for n in args.secondary.split(",") if n and n != args.workload]
+    wl = make_workloads(torch, hip, datagen, dev, [args.workload] + sec_names)
+    if args.workload not in wl:
+        raise SystemExit("unknown workload " + args.workload)
+
+    def measure(w, steps, warmup):
+        for _ in range(warmup):
+            w.fn()
+        ms = _wall_time(torch, w.fn, steps)                    # timed region: exactly `steps` launches
+        kms = _events_time(hip, stream, w.fn, steps)           # HIP events on the launch stream
+        return ms, kms
+
+    prim = wl[args.workload]
+    ms, kms = measure(prim, args.steps, args.warmup)
+    rl = roofline(prim, kms)
+    if prim.bound == "mfma":
+        value, unit, metric = prim.work / (ms * 1e-3) / 1e12, "TFLOP/s", "bfp8_b matmul TFLOP/s"
+    else:
+        value, unit, metric = prim.work / (ms * 1e-3) / 1e9, "GB/s", prim.name + " GB/s"
+    secondary = []
+    for n in sec_names:
+        w = wl[n]
+        sms, skms = measure(w, max(10, args.steps // 2), max(3, args.warmup // 2))
+        r = roofline(w, skms)
+        secondary.append({"workload": n, "desc": w.desc, "ms_per_step": round(sms, 5), "roofline": r})
+
+    result = {
+        "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16 x bfp8_b -> f32 accumulate" if "linear" in prim.name else "u8/f32 bits",
+        "data": "synthetic",
+        "config": {"workload": prim.desc, "name": prim.name, "device": hip.device_name()},
+        "roofline": rl, "secondary": secondary,
+    }
+    if not args.no_cpu_baseline:
+        orc = entry.load_oracle()
+        if "linear" in prim.name:
+            cb, y_cpu = cpu_baseline_linear(orc, datagen)
+            result["cpu_baseline"] = cb
+            # the same rows from the GPU output, as a last sanity check of what was timed
+            if prim.name == "linear2048":
+                import numpy as np
+                at, wt, bt, ot = prim.extra["dev"]
+                o = torch.empty((2048, 14336), dtype=torch.bfloat16, device=dev)
+                hip.call("ttm_untilize", hip.ptr(ot), hip.ptr(o), 1, 2048, 14336, 2, stream)
+                torch.cuda.synchronize()
+                g = o[: y_cpu.shape[0]].float().cpu().numpy()
+                result["check"] = {"rows": int(y_cpu.shape[0]),
+                                   "max_abs_err_vs_cpu": float(np.max(np.abs(g - orc.round_bf16(y_cpu))))}
+        else:
+            result["cpu_baseline"] = cpu_baseline_pack(orc, datagen)
+        result["cpu_baseline_pack_bfp8"] = cpu_baseline_pack(orc, datagen)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

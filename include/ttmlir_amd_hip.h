@@ -90,6 +90,19 @@ int ttm_bfp_pack(const void *src, int src_dtype, int src_layout, void *dst, int 
 int ttm_bfp_unpack(const void *src, int fmt, void *dst, int dst_dtype, int dst_layout, int64_t batch,
                    int64_t rows, int64_t cols, void *stream);
 
+/* ---- matmul / linear: ::ttnn::matmul, ::ttnn::linear
+ * (runtime/lib/ttnn/operations/matmul/matmul.cpp:47-83, 86-125; semantics
+ * include/ttmlir/Dialect/TTIR/IR/TTIROps.td:5169-5290).
+ * out[b] = act(a[b] . w[b or 0] + bias), fp32 accumulation.  Every operand is in TILE layout:
+ * a [batch, M, K] BFloat16; w [w_batch, K, N] BFloat16, BFP_BFloat8 or BFP_BFloat4 packed tiles
+ * (transpose_w: w holds [w_batch, N, K], BFloat16 only); bias BFloat16 [N] either TILE (a [1,N]
+ * tensor padded to 32 rows) or ROW_MAJOR, may be NULL; out [batch, M, N] BFloat16.
+ * w_batch is 1 (weights shared by every batch entry) or equal to batch.  act is TTM_ACT_*,
+ * applied after the bias (tools/golden/mapping.py:7792-7796). */
+int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias,
+               int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch,
+               int64_t M, int64_t N, int64_t K, int act, void *stream);
+
 /* Kernel-variant selection for measurement (name -> small integer); unknown names fail. */
 int ttm_set_option(const char *name, int value);
 int ttm_get_option(const char *name, int *value);

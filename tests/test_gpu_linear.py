@@ -1,0 +1,173 @@
+"""GPU parity: ttm_linear (bf16 x bf16 / bfp8_b / bfp4_b, fused bias + activation) against the CPU
+oracle on identical seeded inputs.  Tolerances (north star): PCC >= 0.99; the max-abs error is
+asserted per weight dtype below.  The oracle multiplies the *dequantised* weights, so the
+comparison isolates the kernel (accumulation order, bf16 output rounding, fast GELU), not the
+block-float quantisation error; that is covered separately against the unquantised weights with
+the reference's own bars (PCC 0.99 bfp8 / 0.98 bfp4, test_weight_dtype_conversion.py:39,78)."""
+import numpy as np
+import pytest
+import torch
+
+from ttmlir_amd import datagen
+
+pytestmark = pytest.mark.gpu
+
+
+def tilize_dev(hip, t, dev):
+    """[.., R, C] torch tensor (2 or 4 byte dtype) -> device tensor in tile order."""
+    t = t.contiguous().to(dev)
+    b = int(np.prod(t.shape[:-2], dtype=np.int64))
+    r, c = t.shape[-2], t.shape[-1]
+    pr, pc = (r + 31) // 32 * 32, (c + 31) // 32 * 32
+    out = torch.zeros(b * pr * pc, dtype=t.dtype, device=dev)
+    hip.call("ttm_tilize", hip.ptr(t), hip.ptr(out), b, r, c, t.element_size(), hip.current_stream())
+    return out
+
+
+def untilize_dev(hip, t, shape, dev):
+    b = int(np.prod(shape[:-2], dtype=np.int64))
+    out = torch.empty(shape, dtype=t.dtype, device=dev)
+    hip.call("ttm_untilize", hip.ptr(t), hip.ptr(out), b, shape[-2], shape[-1], t.element_size(), hip.current_stream())
+    return out
+
+
+def pack_weight(hip, w_f32, fmt, dev):
+    K, N = w_f32.shape[-2:]
+    b = int(np.prod(w_f32.shape[:-2], dtype=np.int64))
+    nt = b * ((K + 31) // 32) * ((N + 31) // 32)
+    out = torch.empty(nt * hip.bfp_tile_bytes(fmt), dtype=torch.uint8, device=dev)
+    wd = w_f32.contiguous().to(dev)
+    hip.call("ttm_bfp_pack", hip.ptr(wd), hip.F32, hip.ROW_MAJOR, hip.ptr(out), fmt, b, K, N, hip.current_stream())
+    return out
+
+
+def run_linear(hip, dev, a, w, bias, act, wfmt, transpose_w=False, bias_tiled=True):
+    """a [..,M,K] bf16, w [..,K,N] f32 (or [..,N,K] when transpose_w); returns [..,M,N] bf16 on the host
+    together with the weights the kernel actually multiplied (dequantised, [..,K,N])."""
+    M, K = a.shape[-2:]
+    N = w.shape[-2] if transpose_w else w.shape[-1]
+    batch = int(np.prod(a.shape[:-2], dtype=np.int64))
+    wbatch = int(np.prod(w.shape[:-2], dtype=np.int64))
+    at = tilize_dev(hip, a, dev)
+    if wfmt == hip.BF16:
+        wq = w.to(torch.bfloat16)
+        wt = tilize_dev(hip, wq, dev)
+        w_eff = wq.float()
+    else:
+        wt = pack_weight(hip, w, wfmt, dev)
+        back = torch.empty(w.shape, dtype=torch.float32, device=dev)
+        hip.call("ttm_bfp_unpack", hip.ptr(wt), wfmt, hip.ptr(back), hip.F32, hip.ROW_MAJOR, wbatch, K, N,
+                 hip.current_stream())
+        w_eff = back.cpu()
+    bt = None
+    if bias is not None:
+        bt = tilize_dev(hip, bias.reshape(1, -1), dev) if bias_tiled else bias.to(dev)
+    Mp, Np = (M + 31) // 32 * 32, (N + 31) // 32 * 32
+    out = torch.full((batch * Mp * Np,), float("nan"), dtype=torch.bfloat16, device=dev)
+    hip.call("ttm_linear", hip.ptr(at), hip.BF16, hip.ptr(wt), wfmt, int(transpose_w),
+             hip.ptr(bt) if bt is not None else None, hip.BF16, hip.TILE if bias_tiled else hip.ROW_MAJOR,
+             hip.ptr(out), hip.BF16, batch, wbatch, M, N, K, hip.ACT[act], hip.current_stream())
+    res = untilize_dev(hip, out, tuple(a.shape[:-2]) + (M, N), dev)
+    torch.cuda.synchronize()
+    return res.cpu(), (w_eff.transpose(-1, -2) if transpose_w else w_eff)
+
+
+def check(orc, metrics, got_bf16, a, w_eff, bias, act, max_abs, pcc=0.99):
+    a32 = a.float().numpy()
+    if a32.ndim == 2:
+        want = orc.linear(a32, w_eff.numpy(), None if bias is None else bias.float().numpy(), act)
+    else:
+        want = orc.matmul(a32, w_eff.numpy())
+        assert bias is None and act is None
+    want = orc.round_bf16(want)                      # the CPU path casts f32 back to bf16 at the end
+    got = got_bf16.float().numpy()
+    assert np.all(np.isfinite(got))
+    err = float(np.max(np.abs(got - want)))
+    p = metrics.get_pcc(want, got)
+    assert p >= pcc, "pcc %.5f" % p
+    assert err <= max_abs, "max abs err %.4g > %.4g" % (err, max_abs)
+    return err, p
+
+
+@pytest.fixture(scope="module")
+def metrics():
+    import oracle.metrics as m
+    return m
+
+
+def test_c1_bf16_matmul(hip, dev, orc, metrics):
+    a, b = datagen.c1_matmul()
+    got, w_eff = run_linear(hip, dev, a, b.float(), None, None, hip.BF16)
+    # |C| ~ sqrt(512) ~ 23 -> bf16 half-ulp 0.0625 at 16..32; allow one bf16 ulp (0.25 at 32..64)
+    check(orc, metrics, got, a, w_eff, None, None, max_abs=0.25)
+
+
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4", "bf16"])
+@pytest.mark.parametrize("M,K,N,act,bias", [
+    (256, 512, 256, None, False), (256, 256, 512, "gelu", True), (512, 128, 256, "silu", True),
+    (64, 96, 160, "sigmoid", True), (32, 512, 64, "gelu", True), (17, 200, 100, "relu", True),
+    (288, 64, 320, "gelu", True), (1, 64, 32, None, True)])
+def test_linear_shapes(hip, dev, orc, metrics, wfmt_name, M, K, N, act, bias):
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B, "bf16": hip.BF16}[wfmt_name]
+    a = datagen.randn((M, K), seed=M + K, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=N, std=0.05)
+    b = datagen.randn((N,), seed=7, std=0.5, dtype=torch.bfloat16) if bias else None
+    got, w_eff = run_linear(hip, dev, a, w, b, act, wfmt)
+    # outputs are O(1); one bf16 ulp at |y| < 4 is 2^-6... allow 2^-5 for accumulation-order effects
+    check(orc, metrics, got, a, w_eff, b, act, max_abs=2.0 ** -5)
+
+
+def test_linear_row_major_bias_and_transposed_weights(hip, dev, orc, metrics):
+    a = datagen.randn((96, 128), seed=1, dtype=torch.bfloat16)
+    w = datagen.randn((128, 192), seed=2, std=0.05)
+    b = datagen.randn((192,), seed=3, std=0.5, dtype=torch.bfloat16)
+    got, w_eff = run_linear(hip, dev, a, w, b, "gelu", hip.BFP8B, bias_tiled=False)
+    check(orc, metrics, got, a, w_eff, b, "gelu", max_abs=2.0 ** -5)
+    for M in (96, 32):
+        a = datagen.randn((M, 128), seed=1, dtype=torch.bfloat16)
+        got, w_eff = run_linear(hip, dev, a, w.t().contiguous(), b, None, hip.BF16, transpose_w=True)
+        check(orc, metrics, got, a, w_eff, b, None, max_abs=2.0 ** -5)
+
+
+def test_batched_matmul(hip, dev, orc, metrics):
+    a = datagen.randn((2, 3, 64, 96), seed=4, dtype=torch.bfloat16)
+    w = datagen.randn((2, 3, 96, 64), seed=5, std=0.1)
+    got, w_eff = run_linear(hip, dev, a, w, None, None, hip.BF16)
+    check(orc, metrics, got, a, w_eff, None, None, max_abs=2.0 ** -5)
+    w1 = datagen.randn((1, 96, 64), seed=6, std=0.1)          # RHS with a single batch broadcasts
+    got, w_eff = run_linear(hip, dev, a, w1, None, None, hip.BF16)
+    want = orc.round_bf16(orc.matmul(a.float().numpy(), w_eff.numpy()))
+    assert np.max(np.abs(got.float().numpy() - want)) <= 2.0 ** -5
+
+
+@pytest.mark.parametrize("M", [32, 2048])
+def test_c3_linear_band(hip, dev, orc, metrics, M):
+    """Config 3 at full size; the oracle checks a band of rows and columns it finishes in seconds."""
+    a, w, bias = datagen.c3_linear(M)
+    got, w_eff = run_linear(hip, dev, a, w, bias, "gelu", hip.BFP8B)
+    rows = slice(0, 32) if M == 32 else slice(1000, 1032)
+    cols = slice(7000, 7512)
+    want = orc.round_bf16(orc.linear(a[rows].float().numpy(), w_eff[:, cols].contiguous().numpy(),
+                                     bias[cols].float().numpy(), "gelu"))
+    g = got[rows, cols].float().numpy()
+    # |y| up to ~6 -> bf16 ulp 2^-5; accumulation over K=4096 in a different order adds less than that
+    assert np.max(np.abs(g - want)) <= 2.0 ** -5
+    assert metrics.get_pcc(want, g) >= 0.99
+    # quantisation itself against the unquantised weights: the reference's own bar for bfp8 weights
+    ref = torch.nn.functional.gelu(a[rows].float() @ w[:, cols] + bias[cols].float())
+    assert metrics.get_pcc(ref.numpy(), g) >= 0.99
+    # linearity in the activations at full size: f(2a) - 2 f(a) == 0 without bias/activation (exact in bf16/f32)
+    g1, _ = run_linear(hip, dev, a, w, None, None, hip.BFP8B)
+    g2, _ = run_linear(hip, dev, (a.float() * 2).to(torch.bfloat16), w, None, None, hip.BFP8B)
+    assert torch.equal(g2.float(), g1.float() * 2)
+
+
+@pytest.mark.parametrize("wfmt_name,bar", [("bfp8", 0.99), ("bfp4", 0.98)])
+def test_weight_dtype_bars(hip, dev, metrics, wfmt_name, bar):
+    """test/python/golden/ttir_ops/matmul/test_weight_dtype_conversion.py:15-88 shapes, PCC vs torch."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    a = datagen.randn((64, 128), seed=0, dtype=torch.bfloat16)
+    w = datagen.randn((128, 64), seed=1)
+    got, _ = run_linear(hip, dev, a, w, None, None, wfmt)
+    ref = a.float() @ w.to(torch.bfloat16).float()
+    assert metrics.get_pcc(ref.numpy(), got.float().numpy()) >= bar
