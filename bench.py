@@ -125,7 +125,7 @@ def roofline(w, kernel_ms):
             "algorithmic_work": w.work, "work_unit": w.unit_work}
 
 
-def cpu_baseline_linear(orc, datagen, budget_rows=256):
+def cpu_baseline_linear(orc, datagen, budget_rows=512):
     """The CPU path (scalar f32 loops, one thread) on a row sample of config 3, M=2048."""
     import numpy as np
     import torch
