@@ -103,6 +103,59 @@ int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int trans
                int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch,
                int64_t M, int64_t N, int64_t K, int act, void *stream);
 
+/* ---- elementwise: ::ttnn::<unary>, ::ttnn::<binary>
+ * (runtime/lib/ttnn/operations/eltwise/unary/unary.cpp:159-205, eltwise/binary/binary.cpp:38-126;
+ * CPU lowering lib/Conversion/TTIRToLinalg/EltwiseUnary.cpp:251-326).  `op` is the value of
+ * EltwiseUnaryOpType / EltwiseBinaryOpType (include/ttmlir/Target/TTNN/operations/eltwise.fbs).
+ * fp32 math, result stored in `dtype` (TTM_BF16 or TTM_F32).  Unary takes a [batch, rows, cols]
+ * tensor in `layout`.  Binary broadcasts numpy-style: the three shapes have `rank` entries (<= 8);
+ * `layout` is the layout of all three tensors.  The zero padding of TILE tensors is preserved. */
+int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows,
+                      int64_t cols, float param, void *stream);
+int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape,
+                       void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream);
+
+/* ---- typecast between plain dtypes: ::ttnn::typecast
+ * (runtime/lib/ttnn/operations/layout/typecast.cpp:14-31).  Layout is preserved, so n counts the
+ * (padded) elements.  Float -> integer truncates toward zero and saturates; integer narrowing
+ * saturates (runtime/include/tt/runtime/utils.h:26-150). */
+int ttm_typecast(const void *in, int src_dtype, void *out, int dst_dtype, int64_t n, void *stream);
+
+/* ---- row-wise ops on TILE tensors [batch, rows, cols], reduced over the last dim, fp32 math.
+ * rms_norm: ::ttnn::rms_norm (runtime/lib/ttnn/operations/normalization/rms_norm.cpp:10-49;
+ *   op order lib/Dialect/TTIR/Transforms/DecomposeComposites.cpp:47-111); weight / bias are [cols]
+ *   vectors of the same dtype, TILE (a [1,cols] tensor) or ROW_MAJOR, may be NULL.
+ * softmax: ::ttnn::softmax over the last dim, always max-subtracted
+ *   (normalization/softmax.cpp:12-36; lib/Conversion/TTIRToLinalg/TTIRToLinalg.cpp:944-1017).
+ * reduce: ::ttnn::sum/mean/max/min over the last dim (reduction/reduction.cpp:13-63); op is
+ *   ReductionOpType; the result is the TILE tensor [batch, rows, 1]. */
+int ttm_rms_norm(const void *x, const void *weight, int weight_layout, const void *bias, int bias_layout,
+                 void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, float eps, void *stream);
+int ttm_softmax_lastdim(const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols,
+                        void *stream);
+int ttm_reduce_lastdim(int op, const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols,
+                       void *stream);
+
+/* ---- generic data movement: reshape / permute / transpose / slice / concat / repeat_interleave
+ * (runtime/lib/ttnn/operations/data_movement/ *.cpp).  A view of `rank` extents maps view index v to
+ * the logical linear index src_base + sum v[d]*src_stride[d] of the source and likewise of the
+ * destination; logical indices are row-major over [batch, rows, cols] and converted to the
+ * layout of each tensor.  Padding of a TILE destination is not written. */
+int ttm_copy_view(const void *src, int64_t src_rows, int64_t src_cols, int src_layout, void *dst,
+                  int64_t dst_rows, int64_t dst_cols, int dst_layout, int elem_bytes, int rank,
+                  const int64_t *extent, const int64_t *src_stride, int64_t src_base,
+                  const int64_t *dst_stride, int64_t dst_base, void *stream);
+
+/* ---- attention: ::ttnn::transformer::scaled_dot_product_attention
+ * (runtime/lib/ttnn/operations/transformer/scaled_dot_product_attention.cpp:14-55; golden
+ * tools/golden/mapping.py:8398-8500).  q [B,Hq,Sq,D], k/v [B,Hkv,Sk,D], out [B,Hq,Sq,D], all
+ * BFloat16 TILE; query head h reads kv head h / (Hq/Hkv); mask is additive BFloat16 TILE
+ * [B,mask_heads,Sq,Sk] (mask_heads 1 or Hq) or NULL; is_causal masks key > query; scale <= 0
+ * means 1/sqrt(D); softmax in fp32. */
+int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype,
+             int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale,
+             void *stream);
+
 /* Kernel-variant selection for measurement (name -> small integer); unknown names fail. */
 int ttm_set_option(const char *name, int value);
 int ttm_get_option(const char *name, int *value);

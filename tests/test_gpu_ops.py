@@ -1,0 +1,265 @@
+"""GPU parity of the bandwidth kernels, data movement and attention against the CPU oracle on
+identical seeded inputs.  Tolerances: fp32 tensors -- values agree to 1e-5 relative (different
+transcendental implementations); bf16 tensors -- at most one bf16 ulp of the result (2^-8
+relative); PCC >= 0.99 everywhere (north star), asserted much tighter."""
+import numpy as np
+import pytest
+import torch
+
+from ttmlir_amd import datagen
+from test_gpu_linear import tilize_dev, untilize_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def bf16_ulps(got, want):
+    """|got - want| in units of the bf16 spacing at |want| (both f32 arrays holding bf16 values)."""
+    _, e = np.frexp(np.clip(np.abs(want), 2.0 ** -126, 3e38))
+    with np.errstate(invalid="ignore"):
+        d = np.where(got == want, 0.0, np.abs(got - want))          # equal infinities count as exact
+    return d / np.ldexp(1.0, e - 8)
+
+
+UNARY = ["abs", "ceil", "cos", "floor", "gelu", "isfinite", "logical_not", "neg", "relu", "sqrt", "rsqrt", "sigmoid",
+         "sin", "reciprocal", "sign", "tanh", "atan", "exp", "erf", "erfc", "log", "expm1", "relu6", "silu", "leaky_relu"]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_unary(hip, dev, orc, dtype):
+    x = datagen.randn((70, 33), seed=1, std=2.0)
+    x[0, :4] = torch.tensor([0.0, -0.0, 1.0, -1.0])
+    for name in UNARY:
+        xi = x.abs() + 0.01 if name in ("sqrt", "rsqrt", "log") else x
+        if dtype == "bf16":
+            xi = xi.to(torch.bfloat16)
+        xd = xi.to(dev)
+        out = torch.empty_like(xd)
+        hip.call("ttm_eltwise_unary", orc.UNARY[name], hip.ptr(xd), hip.ptr(out), hip.BF16 if dtype == "bf16" else hip.F32,
+                 hip.ROW_MAJOR, 1, 70, 33, 0.1, hip.current_stream())
+        torch.cuda.synchronize()
+        want = orc.unary(name, xi.float().numpy(), 0.1)
+        got = out.float().cpu().numpy()
+        if dtype == "f32":
+            assert np.allclose(got, want, rtol=1e-5, atol=1e-6), name
+        else:
+            assert np.max(bf16_ulps(got, orc.round_bf16(want))) <= 1.0, name
+
+
+@pytest.mark.parametrize("layout", ["tile", "row_major"])
+@pytest.mark.parametrize("ashape,bshape", [((64, 96), (64, 96)), ((2, 3, 40, 50), (2, 3, 40, 50)), ((64, 96), (1, 96)),
+                                           ((2, 64, 96), (64, 1)), ((2, 1, 33, 70), (1, 3, 1, 70)), ((4, 32, 32), (1,)),
+                                           ((1, 128), (5, 128, 1))])
+def test_binary_broadcast(hip, dev, orc, layout, ashape, bshape):
+    a = datagen.randn(ashape, seed=2, dtype=torch.bfloat16)
+    b = datagen.randn(bshape, seed=3, dtype=torch.bfloat16) + 3.0
+    oshape = tuple(np.broadcast_shapes(ashape, bshape))
+    rank = len(oshape)
+    pad = lambda s: np.array((1,) * (rank - len(s)) + tuple(s), dtype=np.int64)
+    tiled = layout == "tile"
+    r2 = lambda t: t.reshape((1,) * (2 - t.dim()) + tuple(t.shape)) if t.dim() < 2 else t
+    for name in ("add", "multiply", "subtract", "divide", "gt"):
+        if tiled:
+            ad, bd = tilize_dev(hip, r2(a), dev), tilize_dev(hip, r2(b), dev)
+            Rp, Cp = (oshape[-2] + 31) // 32 * 32, (oshape[-1] + 31) // 32 * 32
+            od = torch.empty(int(np.prod(oshape[:-2], dtype=np.int64)) * Rp * Cp, dtype=torch.bfloat16, device=dev)
+        else:
+            ad, bd = a.to(dev), b.to(dev)
+            od = torch.empty(oshape, dtype=torch.bfloat16, device=dev)
+        sa, sb, so = pad(ashape), pad(bshape), pad(oshape)          # keep the shape arrays alive over the call
+        hip.call("ttm_eltwise_binary", orc.BINARY[name], hip.ptr(ad), sa.ctypes.data, hip.ptr(bd),
+                 sb.ctypes.data, hip.ptr(od), so.ctypes.data, rank, hip.BF16,
+                 hip.TILE if tiled else hip.ROW_MAJOR, hip.current_stream())
+        res = untilize_dev(hip, od, oshape, dev) if tiled else od
+        torch.cuda.synchronize()
+        want = orc.round_bf16(orc.binary(name, a.float().numpy(), b.float().numpy()))
+        assert np.array_equal(res.float().cpu().numpy(), want), name   # one rounding of an exact f32 op: bit exact
+        if tiled:  # padding of the tiled result is zero
+            full = od.float().cpu().numpy()
+            assert np.count_nonzero(full) == np.count_nonzero(want)
+
+
+def test_unary_keeps_tile_padding_zero(hip, dev, orc):
+    x = datagen.randn((2, 40, 50), seed=21, dtype=torch.bfloat16)
+    xt = tilize_dev(hip, x, dev)
+    for name in ("exp", "reciprocal", "gelu"):
+        out = torch.full_like(xt, float("nan"))
+        hip.call("ttm_eltwise_unary", orc.UNARY[name], hip.ptr(xt), hip.ptr(out), hip.BF16, hip.TILE, 2, 40, 50, 0.0,
+                 hip.current_stream())
+        torch.cuda.synchronize()
+        want = orc.round_bf16(orc.unary(name, x.float().numpy()))
+        full = out.float().cpu().numpy()
+        wt = orc.tilize(want)
+        assert np.array_equal(full == 0, wt == 0)                               # padding (and only padding) is zero
+        assert np.max(bf16_ulps(untilize_dev(hip, out, x.shape, dev).float().cpu().numpy(), want)) <= 1.0
+
+
+def test_typecast(hip, dev, orc):
+    x = datagen.randn((1000,), seed=4, std=300.0)
+    x[:6] = torch.tensor([0.0, -0.0, 1e10, -1e10, 65535.4, -7.9])
+    xd = x.to(dev)
+    s = hip.current_stream()
+    out = torch.empty(1000, dtype=torch.bfloat16, device=dev)
+    hip.call("ttm_typecast", hip.ptr(xd), hip.F32, hip.ptr(out), hip.BF16, 1000, s)
+    assert np.array_equal(out.view(torch.int16).cpu().numpy().view(np.uint16), orc.f32_to_bf16(x.numpy()))
+    back = torch.empty(1000, dtype=torch.float32, device=dev)
+    hip.call("ttm_typecast", hip.ptr(out), hip.BF16, hip.ptr(back), hip.F32, 1000, s)
+    assert torch.equal(back.cpu(), out.float().cpu())
+    i32 = torch.empty(1000, dtype=torch.int32, device=dev)
+    hip.call("ttm_typecast", hip.ptr(xd), hip.F32, hip.ptr(i32), hip.I32, 1000, s)
+    want = np.clip(np.trunc(x.double().numpy()), -2 ** 31, 2 ** 31 - 1).astype(np.int64)
+    assert np.array_equal(i32.cpu().numpy().astype(np.int64), want)
+    u8 = torch.empty(1000, dtype=torch.uint8, device=dev)
+    hip.call("ttm_typecast", hip.ptr(i32), hip.I32, hip.ptr(u8), hip.U8, 1000, s)
+    assert np.array_equal(u8.cpu().numpy().astype(np.int64), np.clip(want, 0, 255))   # saturating narrowing
+    f16 = torch.empty(1000, dtype=torch.float16, device=dev)
+    hip.call("ttm_typecast", hip.ptr(out), hip.BF16, hip.ptr(f16), hip.F16, 1000, s)
+    torch.cuda.synchronize()
+    sel = np.abs(out.float().cpu().numpy()) < 65504
+    assert np.array_equal(f16.view(torch.int16).cpu().numpy().view(np.uint16)[sel],
+                          orc.bf16_to_f16(out.view(torch.int16).cpu().numpy().view(np.uint16))[sel])
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("shape,wl,bias", [((512, 4096), "tile", False), ((64, 96), "tile", True), ((3, 40, 70), "rm", True),
+                                           ((1, 33), "tile", False), ((2, 2, 32, 256), "rm", False)])
+def test_rms_norm(hip, dev, orc, dtype, shape, wl, bias):
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    x = datagen.randn(shape, seed=5, dtype=tdt)
+    C = shape[-1]
+    w = (1.0 + 0.02 * datagen.randn((C,), seed=6)).to(tdt)
+    b = datagen.randn((C,), seed=7, std=0.1).to(tdt) if bias else None
+    xt = tilize_dev(hip, x, dev)
+    vec = lambda v: tilize_dev(hip, v.reshape(1, -1), dev) if wl == "tile" else v.to(dev)
+    wd, bd = vec(w), (vec(b) if bias else None)
+    out = torch.full_like(xt, float("nan"))
+    batch, R = int(np.prod(shape[:-2], dtype=np.int64)), shape[-2]
+    lay = hip.TILE if wl == "tile" else hip.ROW_MAJOR
+    hip.call("ttm_rms_norm", hip.ptr(xt), hip.ptr(wd), lay, hip.ptr(bd) if bias else None, lay, hip.ptr(out),
+             hip.BF16 if dtype == "bf16" else hip.F32, batch, R, C, 1e-5, hip.current_stream())
+    res = untilize_dev(hip, out, shape, dev)
+    torch.cuda.synchronize()
+    want = orc.rms_norm(x.float().numpy(), w.float().numpy(), None if b is None else b.float().numpy(), 1e-5)
+    got = res.float().cpu().numpy()
+    if dtype == "f32":
+        assert np.allclose(got, want, rtol=2e-5, atol=1e-6)
+    else:
+        assert np.max(bf16_ulps(got, orc.round_bf16(want))) <= 1.0
+    assert np.all(np.isfinite(out.float().cpu().numpy()))          # padding written as zeros, not left NaN
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("shape", [(64, 96), (2, 3, 40, 70), (1, 2048), (32, 2048)])
+def test_softmax_and_reduce_lastdim(hip, dev, orc, dtype, shape):
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    hdt = hip.BF16 if dtype == "bf16" else hip.F32
+    x = datagen.randn(shape, seed=8, std=3.0, dtype=tdt)
+    xt = tilize_dev(hip, x, dev)
+    batch, R, C = int(np.prod(shape[:-2], dtype=np.int64)), shape[-2], shape[-1]
+    out = torch.full_like(xt, float("nan"))
+    hip.call("ttm_softmax_lastdim", hip.ptr(xt), hip.ptr(out), hdt, batch, R, C, hip.current_stream())
+    res = untilize_dev(hip, out, shape, dev).float().cpu().numpy()
+    want = orc.softmax(x.float().numpy(), -1)
+    if dtype == "f32":
+        assert np.allclose(res, want, rtol=2e-5, atol=1e-7)
+    else:
+        assert np.max(bf16_ulps(res, orc.round_bf16(want))) <= 1.0
+    Rp = (R + 31) // 32 * 32
+    for op in ("sum", "mean", "max", "min"):
+        o = torch.full((batch * Rp * 32,), float("nan"), dtype=tdt, device=dev)
+        hip.call("ttm_reduce_lastdim", orc.REDUCE[op], hip.ptr(xt), hip.ptr(o), hdt, batch, R, C, hip.current_stream())
+        got = untilize_dev(hip, o, tuple(shape[:-1]) + (1,), dev).float().cpu().numpy()
+        w = orc.reduce(op, x.float().numpy(), -1, keepdim=True)
+        if dtype == "f32":
+            assert np.allclose(got, w, rtol=1e-5, atol=1e-4), op
+        else:
+            assert np.max(bf16_ulps(got, orc.round_bf16(w))) <= 1.0, op
+        assert np.all(np.isfinite(o.float().cpu().numpy()))
+
+
+def view_copy(hip, dev, src, src_shape, src_tiled, dst_shape, dst_tiled, extent, sstride, dstride, sbase=0, dbase=0,
+              dst=None):
+    r2 = lambda s: (1,) * (2 - len(s)) + tuple(s) if len(s) < 2 else tuple(s)
+    ss, ds = r2(src_shape), r2(dst_shape)
+    if dst is None:
+        n = int(np.prod(ds[:-2], dtype=np.int64)) * ((ds[-2] + 31) // 32 * 32) * ((ds[-1] + 31) // 32 * 32) if dst_tiled \
+            else int(np.prod(ds, dtype=np.int64))
+        dst = torch.zeros(n, dtype=src.dtype, device=dev)
+    e, s1, s2 = (np.array(v, dtype=np.int64) for v in (extent, sstride, dstride))
+    hip.call("ttm_copy_view", hip.ptr(src), ss[-2], ss[-1], hip.TILE if src_tiled else hip.ROW_MAJOR, hip.ptr(dst),
+             ds[-2], ds[-1], hip.TILE if dst_tiled else hip.ROW_MAJOR, src.element_size(), len(extent),
+             e.ctypes.data, s1.ctypes.data, sbase, s2.ctypes.data, dbase, hip.current_stream())
+    return dst
+
+
+def strides(shape):
+    s, acc = [], 1
+    for d in reversed(shape):
+        s.insert(0, acc)
+        acc *= d
+    return s
+
+
+def test_copy_view_reshape_permute_slice_concat(hip, dev, orc):
+    x = datagen.randn((2, 48, 64), seed=9, dtype=torch.bfloat16)
+    xt = tilize_dev(hip, x, dev)
+    # reshape [2,48,64] -> [2,48,4,16] -> permute (0,2,1,3) -> [2,4,48,16], tiled in and out
+    oshape = (2, 4, 48, 16)
+    in4 = strides((2, 48, 4, 16))
+    out = view_copy(hip, dev, xt, (2, 48, 64), True, oshape, True, oshape, [in4[0], in4[2], in4[1], in4[3]], strides(oshape))
+    got = untilize_dev(hip, out, oshape, dev).cpu()
+    assert torch.equal(got, x.reshape(2, 48, 4, 16).permute(0, 2, 1, 3))
+    # slice [:, 8:40:2, 16:48] to row-major
+    sl = x[:, 8:40:2, 16:48]
+    i3 = strides((2, 48, 64))
+    out = view_copy(hip, dev, xt, (2, 48, 64), True, sl.shape, False, sl.shape, [i3[0], 2 * i3[1], i3[2]],
+                    strides(sl.shape), sbase=8 * 64 + 16)
+    assert torch.equal(out.reshape(sl.shape).cpu(), sl)
+    # concat along dim 1 of two tiled tensors into a tiled [2, 96, 64]
+    y = datagen.randn((2, 48, 64), seed=10, dtype=torch.bfloat16)
+    yt = tilize_dev(hip, y, dev)
+    cshape = (2, 96, 64)
+    dst = view_copy(hip, dev, xt, x.shape, True, cshape, True, x.shape, strides(x.shape), strides(cshape))
+    dst = view_copy(hip, dev, yt, y.shape, True, cshape, True, y.shape, strides(y.shape), strides(cshape), dbase=48 * 64, dst=dst)
+    assert torch.equal(untilize_dev(hip, dst, cshape, dev).cpu(), torch.cat([x, y], dim=1))
+    # repeat_interleave(3, dim=0): view [2,3,48,64] with source stride 0 on the repeat dim
+    rshape = (6, 48, 64)
+    dst = view_copy(hip, dev, xt, x.shape, True, rshape, True, (2, 3, 48, 64), [i3[0], 0, i3[1], i3[2]],
+                    strides((2, 3, 48, 64)))
+    assert torch.equal(untilize_dev(hip, dst, rshape, dev).cpu(), x.repeat_interleave(3, dim=0))
+    # transpose of the last two dims on fp32, ragged
+    z = datagen.randn((3, 40, 50), seed=11)
+    zt = tilize_dev(hip, z, dev)
+    tshape = (3, 50, 40)
+    zs = strides(z.shape)
+    dst = view_copy(hip, dev, zt, z.shape, True, tshape, True, tshape, [zs[0], zs[2], zs[1]], strides(tshape))
+    torch.cuda.synchronize()
+    assert torch.equal(untilize_dev(hip, dst, tshape, dev).cpu(), z.transpose(1, 2))
+    assert np.array_equal(dst.cpu().numpy(), orc.tilize(z.transpose(1, 2).contiguous().numpy()))   # padding stays zero
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,mask", [
+    (1, 4, 2, 128, 128, 64, True, None), (2, 2, 2, 96, 160, 128, False, None), (1, 8, 2, 256, 256, 128, True, None),
+    (1, 2, 1, 70, 70, 32, True, None), (1, 2, 2, 64, 100, 64, False, "b1"), (2, 2, 1, 64, 64, 64, False, "bh"),
+    (1, 1, 1, 40, 300, 256, False, None)])
+def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask):
+    import oracle.metrics as metrics
+    q = datagen.randn((B, Hq, Sq, D), seed=12, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, Sk, D), seed=13, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, Sk, D), seed=14, dtype=torch.bfloat16)
+    m = None
+    if mask:
+        m = datagen.randn((B, 1 if mask == "b1" else Hq, Sq, Sk), seed=15, dtype=torch.bfloat16)
+    qt, kt, vt = (tilize_dev(hip, t, dev) for t in (q, k, v))
+    mt = tilize_dev(hip, m, dev) if m is not None else None
+    out = torch.full_like(qt, float("nan"))
+    hip.call("ttm_sdpa", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(mt) if mt is not None else None,
+             m.shape[1] if m is not None else 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, Sq, Sk, D, int(causal), 0.0,
+             hip.current_stream())
+    res = untilize_dev(hip, out, q.shape, dev).float().cpu().numpy()
+    torch.cuda.synchronize()
+    want = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), None if m is None else m.float().numpy(),
+                    is_causal=causal)
+    assert np.all(np.isfinite(out.float().cpu().numpy()))
+    # probabilities are rounded to bf16 before P.V (relative 2^-9 each) and the output once more
+    assert np.max(np.abs(res - want)) <= 2.0 ** -6
+    assert metrics.get_pcc(want, res) >= 0.9999

@@ -1,0 +1,137 @@
+"""Pins the oracle's f32 compute functions against library routines (torch on the CPU) and
+closed forms.  Tolerances are those of f32 evaluation order, written per check."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+
+def rnd(shape, seed, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * scale).astype(np.float32)
+
+
+def test_linear_matches_torch(orc):
+    a, b, bias = rnd((37, 53), 0), rnd((53, 29), 1), rnd((29,), 2)
+    want = torch.from_numpy(a).double() @ torch.from_numpy(b).double() + torch.from_numpy(bias).double()
+    got = orc.linear(a, b, bias)
+    assert np.allclose(got, want.numpy(), rtol=1e-5, atol=1e-5)
+    # transposes address the stored operand with its last two dims swapped
+    assert np.array_equal(orc.linear(a.T.copy(), b, bias, transpose_a=True), got)
+    assert np.array_equal(orc.linear(a, b.T.copy(), bias, transpose_b=True), got)
+    # the row-streaming variant keeps the same per-element accumulation order: bit identical
+    assert np.array_equal(orc.linear(a, b, bias, rowstream=True), got)
+    # a dropped bias or a swapped activation order would show here
+    g = orc.linear(a, b, bias, act="gelu")
+    assert np.allclose(g, F.gelu(want).float().numpy(), rtol=1e-5, atol=1e-5)
+    s = orc.linear(a, b, bias, act="silu")
+    assert np.allclose(s, F.silu(want).float().numpy(), rtol=1e-5, atol=1e-5)
+
+
+def test_identity_and_known_matmul(orc):
+    a = rnd((8, 8), 3)
+    assert np.array_equal(orc.linear(a, np.eye(8, dtype=np.float32)), a)
+    x = np.array([[1, 2], [3, 4]], dtype=np.float32)
+    y = np.array([[5, 6], [7, 8]], dtype=np.float32)
+    assert orc.linear(x, y).tolist() == [[19, 22], [43, 50]]
+
+
+def test_batched_matmul_broadcast(orc):
+    a, b = rnd((2, 3, 5, 7), 4), rnd((1, 7, 4), 5)
+    want = torch.from_numpy(a) @ torch.from_numpy(b)
+    assert np.allclose(orc.matmul(a, b), want.numpy(), rtol=1e-5, atol=1e-5)
+    b2 = rnd((2, 3, 7, 4), 6)
+    assert np.allclose(orc.matmul(a, b2), (torch.from_numpy(a) @ torch.from_numpy(b2)).numpy(), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("name,fn", [
+    ("gelu", F.gelu), ("silu", F.silu), ("sigmoid", torch.sigmoid), ("exp", torch.exp), ("neg", torch.neg),
+    ("rsqrt", torch.rsqrt), ("sqrt", torch.sqrt), ("tanh", torch.tanh), ("erf", torch.erf), ("relu", torch.relu),
+    ("abs", torch.abs), ("reciprocal", torch.reciprocal), ("log", torch.log), ("sin", torch.sin), ("cos", torch.cos),
+    ("floor", torch.floor), ("ceil", torch.ceil), ("sign", torch.sign)])
+def test_unary_matches_torch(orc, name, fn):
+    x = rnd((1000,), 7, 3.0)
+    if name in ("rsqrt", "sqrt", "log"):
+        x = np.abs(x) + 0.01
+    want = fn(torch.from_numpy(x).double()).float().numpy()
+    assert np.allclose(orc.unary(name, x), want, rtol=2e-6, atol=2e-7)
+
+
+def test_gelu_doc_example(orc):
+    # include/ttmlir/Dialect/TTIR/IR/TTIROps.td:529-537: gelu([1, -1, 0...]) -> [0.8413, -0.1587, 0]
+    y = orc.unary("gelu", np.array([1.0, -1.0, 0.0], dtype=np.float32))
+    assert np.allclose(y, [0.8413447, -0.1586553, 0.0], atol=1e-6)
+
+
+def test_binary_broadcast(orc):
+    a, b = rnd((2, 1, 5, 7), 8), rnd((3, 1, 7), 9)
+    for name, fn in (("add", np.add), ("multiply", np.multiply), ("subtract", np.subtract), ("divide", np.divide)):
+        assert np.array_equal(orc.binary(name, a, b), fn(a, b))
+    assert np.array_equal(orc.binary("gt", a, b), (a > b).astype(np.float32))
+
+
+def test_rms_norm_matches_torch(orc):
+    x, w, b = rnd((6, 40), 10), rnd((40,), 11), rnd((40,), 12)
+    want = F.rms_norm(torch.from_numpy(x), (40,), torch.from_numpy(w), 1e-5) + torch.from_numpy(b)
+    assert np.allclose(orc.rms_norm(x, w, b, 1e-5), want.numpy(), rtol=1e-5, atol=1e-6)
+    # closed form: a constant row c normalises to c / sqrt(c^2 + eps)
+    c = np.full((1, 16), 3.0, dtype=np.float32)
+    assert np.allclose(orc.rms_norm(c, None, None, 0.0), 1.0)
+    # eps matters: a dropped eps would turn an all-zero row into NaN
+    assert np.array_equal(orc.rms_norm(np.zeros((1, 8), np.float32), None, None, 1e-5), np.zeros((1, 8), np.float32))
+
+
+def test_softmax_and_reduce(orc):
+    x = rnd((3, 5, 17), 13, 4.0)
+    for dim in (-1, 1, 0):
+        want = F.softmax(torch.from_numpy(x).double(), dim=dim).float().numpy()
+        got = orc.softmax(x, dim)
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-7)
+        assert np.allclose(got.sum(axis=dim), 1.0, atol=1e-5)
+    big = np.array([[1000.0, 1000.0, -1000.0]], dtype=np.float32)        # max subtraction keeps this finite
+    assert np.allclose(orc.softmax(big), [[0.5, 0.5, 0.0]])
+    for op, fn in (("sum", np.sum), ("mean", np.mean), ("max", np.max), ("min", np.min)):
+        for dim in (-1, 0, 1):
+            assert np.allclose(orc.reduce(op, x, dim), fn(x.astype(np.float64), axis=dim), rtol=1e-5, atol=1e-5)
+    assert orc.reduce("sum", x, -1, keepdim=True).shape == (3, 5, 1)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_sdpa_matches_torch(orc, causal):
+    B, Hq, Hkv, S, D = 2, 4, 2, 24, 16
+    q, k, v = rnd((B, Hq, S, D), 14), rnd((B, Hkv, S, D), 15), rnd((B, Hkv, S, D), 16)
+    kr = torch.from_numpy(k).repeat_interleave(Hq // Hkv, dim=1)
+    vr = torch.from_numpy(v).repeat_interleave(Hq // Hkv, dim=1)
+    want = F.scaled_dot_product_attention(torch.from_numpy(q), kr, vr, is_causal=causal)
+    assert np.allclose(orc.sdpa(q, k, v, is_causal=causal), want.numpy(), rtol=1e-4, atol=1e-5)
+    if not causal:
+        mask = rnd((B, 1, S, S), 17)
+        want = F.scaled_dot_product_attention(torch.from_numpy(q), kr, vr, attn_mask=torch.from_numpy(mask), scale=0.3)
+        assert np.allclose(orc.sdpa(q, k, v, mask=mask, scale=0.3), want.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_sdpa_uniform_keys_average_values(orc):
+    # q = 0 -> uniform attention: causal row i is the mean of v[0..i]
+    q = np.zeros((1, 1, 4, 8), np.float32)
+    k = rnd((1, 1, 4, 8), 18)
+    v = rnd((1, 1, 4, 8), 19)
+    out = orc.sdpa(q, k, v, is_causal=True)[0, 0]
+    for i in range(4):
+        assert np.allclose(out[i], v[0, 0, : i + 1].mean(axis=0), atol=1e-6)
+
+
+def test_pcc_special_cases():
+    import oracle.metrics as m
+    a = np.array([1.0, 2.0, 3.0, 4.0])
+    assert m.get_pcc(a, a) == 1.0
+    assert abs(m.get_pcc(a, 2 * a + 1) - 1.0) < 1e-12
+    assert abs(m.get_pcc(a, -a) + 1.0) < 1e-12
+    assert m.get_pcc(np.zeros(4), np.ones(4)) == 0.0                 # any-nonzero mismatch
+    assert m.get_pcc(np.full(4, np.nan), np.full(4, np.nan)) == 1.0
+    assert m.get_pcc(np.full(4, 2.0), np.full(4, 2.0 + 1e-9)) == 1.0  # two constants -> isclose
+    assert m.get_pcc(np.zeros((0,)), np.zeros((0,))) == 1.0
+    assert m.get_pcc(np.array([3.0]), np.array([3.1])) == 1.0         # single non-zero golden: cosine sign
+    x = np.random.default_rng(0).standard_normal(1000)
+    y = x + 0.1 * np.random.default_rng(1).standard_normal(1000)
+    assert abs(m.get_pcc(x, y) - np.corrcoef(x, y)[0, 1]) < 1e-12
+    at, rt = m.get_atol_rtol(np.array([1.0, 2.0]), np.array([1.5, 2.0]))
+    assert at == 0.5 and abs(rt - 0.5 / 1.5) < 1e-12

@@ -1,0 +1,226 @@
+// Row-wise bandwidth kernels on tile-ordered tensors: RMSNorm, softmax and reductions over the
+// last dimension.  A workgroup owns one tile row (32 logical rows x all columns), which is one
+// contiguous run of tiles in memory.  Thread (r = tid % 32, j = tid / 32) walks the chunks of row
+// r with stride 8; for every step the 256 lanes together read whole tiles, so global accesses are
+// contiguous.  Partial results of the 8 lanes of a row meet in LDS.  Math is fp32; columns beyond
+// the logical width are masked with the operation's identity, rows beyond the logical height are
+// written as zeros.
+#include "ttm_common.h"
+#include "ttm_math.h"
+
+enum { RW_RMSNORM = 0, RW_SOFTMAX = 1, RW_SUM = 2, RW_MEAN = 3, RW_MAX = 4, RW_MIN = 5 };
+
+struct RowArgs {
+  const void *x;
+  void *out;
+  const void *w, *b;   // rmsnorm weight / bias (same dtype as x) or null
+  int w_tiled, b_tiled;
+  int64_t rows, cols;  // logical extent of the last two dims
+  int rt, ct;          // tiles per batch entry
+  float eps;
+  int out_ct;          // reductions: column tiles of the output (1), keepdim layout [.., rows, 1]
+};
+
+template <int ELEM>
+struct ChunkPos {  // chunk q of row r inside a tile row
+  int64_t off;     // element offset from the start of the tile row
+  int c0;          // logical column of the chunk's first element
+};
+template <int ELEM>
+__device__ __forceinline__ ChunkPos<ELEM> chunk_pos(int r, int q) {
+  constexpr int EPC = 16 / ELEM;
+  int tile = q / (2 * ELEM), fx = (q % (2 * ELEM)) / ELEM, part = q % ELEM;
+  ChunkPos<ELEM> p;
+  p.off = (int64_t)tile * 1024 + ((r >> 4) * 2 + fx) * 256 + (r & 15) * 16 + part * EPC;
+  p.c0 = tile * 32 + fx * 16 + part * EPC;
+  return p;
+}
+
+template <int ELEM>
+__device__ __forceinline__ void load_vals(const void *base, int64_t off, float (&f)[16 / ELEM]) {
+  u32x4 v = *(const u32x4 *)((const uint8_t *)base + off * ELEM);
+  if (ELEM == 2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(v[i] << 16);
+      f[2 * i + 1] = __uint_as_float(v[i] & 0xFFFF0000u);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(v[i]);
+  }
+}
+template <int ELEM>
+__device__ __forceinline__ void store_vals(void *base, int64_t off, const float (&f)[16 / ELEM]) {
+  u32x4 v;
+  if (ELEM == 2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = (uint32_t)ttm_f32_to_bf16(f[2 * i]) | ((uint32_t)ttm_f32_to_bf16(f[2 * i + 1]) << 16);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __float_as_uint(f[i]);
+  }
+  *(u32x4 *)((uint8_t *)base + off * ELEM) = v;
+}
+
+// weight / bias vector element c: tiled [1, C] tensor (row 0 of a 32-row tile) or plain [C]
+template <int ELEM>
+__device__ __forceinline__ void load_vec(const void *v, int tiled, int c0, float (&f)[16 / ELEM]) {
+  int64_t off = tiled ? (int64_t)(c0 >> 5) * 1024 + ((c0 >> 4) & 1) * 256 + (c0 & 15) : c0;
+  load_vals<ELEM>(v, off, f);
+}
+
+template <int MODE, int ELEM>
+__global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
+  constexpr int EPC = 16 / ELEM;
+  __shared__ float part[8][32];
+  __shared__ float part2[8][32];
+  const int tid = threadIdx.x, r = tid & 31, j = tid >> 5;
+  const int64_t trow = blockIdx.x;                       // tile row over all batch entries
+  const int64_t row = (trow % p.rt) * 32 + r;            // logical row inside the batch entry
+  const bool row_ok = row < p.rows;
+  const int nq = p.ct * 2 * ELEM;                        // chunks per row
+  const uint8_t *x = (const uint8_t *)p.x + trow * p.ct * 1024 * ELEM;
+  const int cols = (int)p.cols;
+
+  constexpr bool IS_MAX = MODE == RW_SOFTMAX || MODE == RW_MAX;
+  float acc = IS_MAX ? -INFINITY : (MODE == RW_MIN ? INFINITY : 0.0f);
+  for (int q = j; q < nq; q += 8) {
+    ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
+    float f[EPC];
+    load_vals<ELEM>(x, cp.off, f);
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) {
+      bool ok = cp.c0 + i < cols;
+      if (MODE == RW_RMSNORM) acc += ok ? f[i] * f[i] : 0.0f;
+      else if (IS_MAX) acc = ok ? fmaxf(acc, f[i]) : acc;
+      else if (MODE == RW_MIN) acc = ok ? fminf(acc, f[i]) : acc;
+      else acc += ok ? f[i] : 0.0f;
+    }
+  }
+  part[j][r] = acc;
+  __syncthreads();
+  float stat = part[0][r];
+#pragma unroll
+  for (int k = 1; k < 8; ++k) {
+    float o = part[k][r];
+    stat = IS_MAX ? fmaxf(stat, o) : (MODE == RW_MIN ? fminf(stat, o) : stat + o);
+  }
+
+  if (MODE == RW_SUM || MODE == RW_MEAN || MODE == RW_MAX || MODE == RW_MIN) {
+    // output [.., rows, 1] in tile order: one column tile per tile row; zero padded
+    if (MODE == RW_MEAN) stat = stat / (float)cols;
+    uint8_t *o = (uint8_t *)p.out + trow * 1024 * ELEM;
+    // 256 lanes clear the tile (1024 elements), then column 0 is written
+    for (int e = tid; e < 1024 * ELEM / 16; e += 256) ((u32x4 *)o)[e] = u32x4{0, 0, 0, 0};
+    __syncthreads();
+    if (j == 0 && row_ok) {
+      int64_t off = ((r >> 4) * 2) * 256 + (r & 15) * 16;
+      if (ELEM == 2) ((uint16_t *)o)[off] = ttm_f32_to_bf16(stat);
+      else ((float *)o)[off] = stat;
+    }
+    return;
+  }
+
+  uint8_t *o = (uint8_t *)p.out + trow * p.ct * 1024 * ELEM;
+  if (MODE == RW_RMSNORM) {
+    const float rs = 1.0f / sqrtf(stat / (float)cols + p.eps);
+    for (int q = j; q < nq; q += 8) {
+      ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
+      float f[EPC], w[EPC], b[EPC];
+      load_vals<ELEM>(x, cp.off, f);
+      if (p.w) load_vec<ELEM>(p.w, p.w_tiled, cp.c0, w);
+      if (p.b) load_vec<ELEM>(p.b, p.b_tiled, cp.c0, b);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) {
+        float v = f[i] * rs;
+        if (p.w) v *= w[i];
+        if (p.b) v += b[i];
+        f[i] = (row_ok && cp.c0 + i < cols) ? v : 0.0f;
+      }
+      store_vals<ELEM>(o, cp.off, f);
+    }
+  } else {  // softmax: second pass for the sum of exponentials, third pass writes
+    const float mx = stat;
+    float sum = 0.0f;
+    for (int q = j; q < nq; q += 8) {
+      ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
+      float f[EPC];
+      load_vals<ELEM>(x, cp.off, f);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) sum += cp.c0 + i < cols ? expf(f[i] - mx) : 0.0f;
+    }
+    part2[j][r] = sum;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) tot += part2[k][r];
+    const float inv = 1.0f / tot;
+    for (int q = j; q < nq; q += 8) {
+      ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
+      float f[EPC];
+      load_vals<ELEM>(x, cp.off, f);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) f[i] = (row_ok && cp.c0 + i < cols) ? expf(f[i] - mx) * inv : 0.0f;
+      store_vals<ELEM>(o, cp.off, f);
+    }
+  }
+}
+
+template <int MODE>
+static int launch_rowwise(const RowArgs &p, int dtype, int64_t trows, hipStream_t s) {
+  TTM_REQUIRE(trows < (1ll << 31), "row-wise kernel: tensor too large");
+  if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_k<MODE, 2>), dim3((unsigned)trows), dim3(256), 0, s, p);
+  else hipLaunchKernelGGL((ttm_rowwise_k<MODE, 4>), dim3((unsigned)trows), dim3(256), 0, s, p);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+static int fill_args(RowArgs &p, const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols,
+                     const char *who) {
+  TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "%s: dtype must be BFloat16 or Float32 (got %d)", who, dtype);
+  TTM_REQUIRE(batch >= 0 && rows >= 0 && cols >= 0, "%s: negative dimension", who);
+  TTM_REQUIRE(x && out, "%s: null pointer", who);
+  TTM_REQUIRE(((uintptr_t)x & 15) == 0 && ((uintptr_t)out & 15) == 0, "%s: pointers must be 16-byte aligned", who);
+  p.x = x; p.out = out; p.w = p.b = nullptr; p.w_tiled = p.b_tiled = 0;
+  p.rows = rows; p.cols = cols;
+  p.rt = (int)ttm_cdiv(rows, 32); p.ct = (int)ttm_cdiv(cols, 32);
+  p.eps = 0.0f; p.out_ct = 1;
+  return TTM_OK;
+}
+
+TTM_EXPORT int ttm_rms_norm(const void *x, const void *weight, int weight_layout, const void *bias, int bias_layout,
+                            void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, float eps, void *stream) {
+  if (batch == 0 || rows == 0 || cols == 0) return TTM_OK;
+  RowArgs p;
+  int rc = fill_args(p, x, out, dtype, batch, rows, cols, "ttm_rms_norm");
+  if (rc) return rc;
+  TTM_REQUIRE((((uintptr_t)weight | (uintptr_t)bias) & 15) == 0, "ttm_rms_norm: weight/bias must be 16-byte aligned");
+  p.w = weight; p.b = bias; p.w_tiled = weight_layout == TTM_TILE; p.b_tiled = bias_layout == TTM_TILE; p.eps = eps;
+  return launch_rowwise<RW_RMSNORM>(p, dtype, batch * p.rt, (hipStream_t)stream);
+}
+
+TTM_EXPORT int ttm_softmax_lastdim(const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols,
+                                   void *stream) {
+  if (batch == 0 || rows == 0 || cols == 0) return TTM_OK;
+  RowArgs p;
+  int rc = fill_args(p, x, out, dtype, batch, rows, cols, "ttm_softmax_lastdim");
+  if (rc) return rc;
+  return launch_rowwise<RW_SOFTMAX>(p, dtype, batch * p.rt, (hipStream_t)stream);
+}
+
+TTM_EXPORT int ttm_reduce_lastdim(int op, const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols,
+                                  void *stream) {
+  TTM_REQUIRE(op >= 0 && op <= 3, "ttm_reduce_lastdim: op must be Sum(0), Mean(1), Max(2) or Min(3), got %d", op);
+  if (batch == 0 || rows == 0 || cols == 0) return TTM_OK;
+  RowArgs p;
+  int rc = fill_args(p, x, out, dtype, batch, rows, cols, "ttm_reduce_lastdim");
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  switch (op) {
+  case 0: return launch_rowwise<RW_SUM>(p, dtype, batch * p.rt, s);
+  case 1: return launch_rowwise<RW_MEAN>(p, dtype, batch * p.rt, s);
+  case 2: return launch_rowwise<RW_MAX>(p, dtype, batch * p.rt, s);
+  default: return launch_rowwise<RW_MIN>(p, dtype, batch * p.rt, s);
+  }
+}

@@ -1,0 +1,209 @@
+// Fused scaled-dot-product attention (prefill): softmax(Q K^T * scale + mask) V with grouped-query
+// heads, causal masking, fp32 online softmax, bf16 MFMA.  Q [B,Hq,Sq,D], K/V [B,Hkv,Sk,D], mask
+// (optional, additive) [B,1|Hq,Sq,Sk], out [B,Hq,Sq,D]; all bf16 in tile order.
+//
+// Everything is computed transposed so that no accumulator ever has to be shuffled between lanes:
+//   S^T[key][q] = K . Q^T     (MFMA A = K rows, 8 consecutive d per lane straight from the tiled K;
+//                              MFMA B = Q, kept in registers for the whole key loop)
+//   O^T[d][q]   = V^T . P^T   (MFMA B = P^T taken directly from the S^T accumulator registers: a lane
+//                              holds q = lane % 32 and keys 8g + 4h + {0..3}; the k-slot order this
+//                              implies is matched on the V^T side)
+// A lane therefore owns one query column of every accumulator: the running max / sum and the
+// rescale factor are per-lane scalars, shared only with lane ^ 32.
+// Workgroup = 4 wavefronts x 32 queries; K and V^T blocks of 32 keys are staged in LDS.
+#include "ttm_common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct SdpaArgs {
+  const uint8_t *q, *k, *v, *mask;
+  uint8_t *out;
+  int B, Hq, Hkv, Sq, Sk;
+  int sqt, skt;      // tiles along the sequence dims
+  int mask_heads;    // 1 or Hq
+  int causal;
+  float scale;
+};
+
+__device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
+  return (uint32_t)ttm_f32_to_bf16(a) | ((uint32_t)ttm_f32_to_bf16(b) << 16);
+}
+
+template <int DT>  // head_dim / 32
+__global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
+  constexpr int D = DT * 32;
+  constexpr int VPITCH = 40;                           // V^T row pitch in bf16 (32 keys + pad)
+  __shared__ __attribute__((aligned(16))) uint8_t ldsK[32 * D * 2];
+  __shared__ __attribute__((aligned(16))) uint16_t ldsV[D * VPITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int qb = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int hk = h / (p.Hq / p.Hkv);
+  const int qt = qb * 4 + wave;                         // this wave's query tile
+  const bool wave_ok = qt < p.sqt;
+  const int l31 = lane & 31, hh = lane >> 5;
+  const int64_t q_mat = ((int64_t)b * p.Hq + h) * p.sqt * DT * 2048;
+  const int64_t kv_mat = ((int64_t)b * p.Hkv + hk) * p.skt * DT * 2048;
+
+  // Q fragments: B operand, lane (q = l31, hh): d = 16 s + 8 hh .. +7
+  bf16x8 qf[2 * DT];
+#pragma unroll
+  for (int s = 0; s < 2 * DT; ++s) {
+    u32x4 v = {0, 0, 0, 0};
+    if (wave_ok)
+      v = *(const u32x4 *)(p.q + q_mat + ((int64_t)qt * DT + (s >> 1)) * 2048 + ((l31 >> 4) * 2 + (s & 1)) * 512 +
+                           (l31 & 15) * 32 + hh * 16);
+    qf[s] = *(bf16x8 *)&v;
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[d][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+  const int q_glob = qt * 32 + l31;
+
+  // number of key tiles any wave of this workgroup needs
+  int kt_end = p.skt;
+  if (p.causal) kt_end = min(kt_end, (min(qb * 4 + 4, p.sqt) * 32 + 31) / 32);
+  for (int kt = 0; kt < kt_end; ++kt) {
+    __syncthreads();  // previous block fully consumed
+    {
+      // K block: DT tiles, contiguous (32 * D * 2 bytes); copied as is
+      const u32x4 *src = (const u32x4 *)(p.k + kv_mat + (int64_t)kt * DT * 2048);
+      for (int c = tid; c < DT * 128; c += 256) ((u32x4 *)ldsK)[c] = src[c];
+      // V block -> V^T[d][key]
+      const u32x4 *vs = (const u32x4 *)(p.v + kv_mat + (int64_t)kt * DT * 2048);
+      for (int c = tid; c < DT * 128; c += 256) {
+        u32x4 v = vs[c];
+        int tile = c >> 7, cc = c & 127;
+        int face = cc >> 5, row = (cc & 31) >> 1, half = cc & 1;
+        int key = (face >> 1) * 16 + row;
+        int d0 = tile * 32 + (face & 1) * 16 + half * 8;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          ldsV[(d0 + 2 * i) * VPITCH + key] = (uint16_t)(v[i] & 0xFFFF);
+          ldsV[(d0 + 2 * i + 1) * VPITCH + key] = (uint16_t)(v[i] >> 16);
+        }
+      }
+    }
+    __syncthreads();
+    const bool skip = !wave_ok || (p.causal && kt * 32 > qt * 32 + 31);
+    if (skip) continue;
+
+    // S^T = K . Q^T for 32 keys x 32 queries
+    f32x16 s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+#pragma unroll
+    for (int st = 0; st < 2 * DT; ++st) {
+      u32x4 kv = *(const u32x4 *)(ldsK + (st >> 1) * 2048 + ((l31 >> 4) * 2 + (st & 1)) * 512 + (l31 & 15) * 32 + hh * 16);
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&kv, qf[st], s, 0, 0, 0);
+    }
+    // scale, mask; lane holds q = q_glob, keys kt*32 + 8g + 4hh + r
+    float mx = -INFINITY;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int key0 = kt * 32 + g * 8 + hh * 4;
+      float mk[4] = {0.f, 0.f, 0.f, 0.f};
+      if (p.mask) {
+        const int64_t mm = ((int64_t)b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
+        const int kin = g * 8 + hh * 4;
+        const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
+                            (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
+        u32x2 raw = *(const u32x2 *)mp;
+        mk[0] = __uint_as_float(raw.x << 16); mk[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+        mk[2] = __uint_as_float(raw.y << 16); mk[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float v = s[g * 4 + r] * p.scale + mk[r];
+        const int key = key0 + r;
+        if (key >= p.Sk || (p.causal && key > q_glob)) v = -INFINITY;
+        s[g * 4 + r] = v;
+        mx = fmaxf(mx, v);
+      }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    // fully masked so far: keep everything at zero without producing NaN
+    const float m_use = m_new == -INFINITY ? 0.0f : m_new;
+    const float alpha = __expf(m_run - m_use);
+    float rs = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      float e = __expf(s[r] - m_use);
+      s[r] = e;
+      rs += e;
+    }
+    rs += __shfl_xor(rs, 32);
+    l_run = l_run * alpha + rs;
+    m_run = m_new;
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
+    // O^T += V^T . P^T, two k16 steps
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      u32x4 pb;
+      pb.x = pack_bf16_rne(s[8 * t + 0], s[8 * t + 1]);
+      pb.y = pack_bf16_rne(s[8 * t + 2], s[8 * t + 3]);
+      pb.z = pack_bf16_rne(s[8 * t + 4], s[8 * t + 5]);
+      pb.w = pack_bf16_rne(s[8 * t + 6], s[8 * t + 7]);
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        const uint16_t *vr = ldsV + (d * 32 + l31) * VPITCH + 16 * t + 4 * hh;
+        u32x2 lo = *(const u32x2 *)vr, hi = *(const u32x2 *)(vr + 8);
+        u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va, *(bf16x8 *)&pb, o[d], 0, 0, 0);
+      }
+    }
+  }
+  if (!wave_ok) return;
+  const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+  const bool q_ok = q_glob < p.Sq;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int din = g * 8 + hh * 4;
+      u32x2 ov;
+      ov.x = q_ok ? pack_bf16_rne(o[d][g * 4 + 0] * inv, o[d][g * 4 + 1] * inv) : 0u;
+      ov.y = q_ok ? pack_bf16_rne(o[d][g * 4 + 2] * inv, o[d][g * 4 + 3] * inv) : 0u;
+      uint8_t *op = p.out + q_mat + ((int64_t)qt * DT + d) * 2048 +
+                    (((l31 >> 4) * 2 + (din >> 4)) * 256 + (l31 & 15) * 16 + (din & 15)) * 2;
+      *(u32x2 *)op = ov;
+    }
+}
+
+TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
+                        int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
+                        int is_causal, float scale, void *stream) {
+  TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa: tensors must be BFloat16 (got %d)", dtype);
+  TTM_REQUIRE(B >= 0 && Hq >= 0 && Hkv > 0 && Sq >= 0 && Sk >= 0 && D > 0, "ttm_sdpa: bad dimension");
+  TTM_REQUIRE(Hq % Hkv == 0, "ttm_sdpa: query heads (%ld) must be a multiple of kv heads (%ld)", (long)Hq, (long)Hkv);
+  TTM_REQUIRE(D % 32 == 0 && (D == 32 || D == 64 || D == 128 || D == 256), "ttm_sdpa: head_dim must be 32, 64, 128 or 256 (got %ld)", (long)D);
+  TTM_REQUIRE(mask == nullptr || mask_heads == 1 || mask_heads == Hq, "ttm_sdpa: mask heads must be 1 or Hq");
+  if (B == 0 || Hq == 0 || Sq == 0) return TTM_OK;
+  TTM_REQUIRE(Sk > 0, "ttm_sdpa: empty key sequence");
+  TTM_REQUIRE(q && k && v && out, "ttm_sdpa: null pointer");
+  TTM_REQUIRE(Hq <= 65535 && B <= 65535, "ttm_sdpa: too many heads or batches");
+  SdpaArgs p;
+  p.q = (const uint8_t *)q; p.k = (const uint8_t *)k; p.v = (const uint8_t *)v; p.mask = (const uint8_t *)mask;
+  p.out = (uint8_t *)out;
+  p.B = (int)B; p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.Sq = (int)Sq; p.Sk = (int)Sk;
+  p.sqt = (int)ttm_cdiv(Sq, 32); p.skt = (int)ttm_cdiv(Sk, 32);
+  p.mask_heads = mask_heads; p.causal = is_causal;
+  p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)D);
+  dim3 grid((unsigned)ttm_cdiv(p.sqt, 4), (unsigned)Hq, (unsigned)B), block(256);
+  hipStream_t s = (hipStream_t)stream;
+  switch (D) {
+  case 32: hipLaunchKernelGGL(ttm_sdpa_k<1>, grid, block, 0, s, p); break;
+  case 64: hipLaunchKernelGGL(ttm_sdpa_k<2>, grid, block, 0, s, p); break;
+  case 128: hipLaunchKernelGGL(ttm_sdpa_k<4>, grid, block, 0, s, p); break;
+  default: hipLaunchKernelGGL(ttm_sdpa_k<8>, grid, block, 0, s, p); break;
+  }
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
