@@ -1,0 +1,142 @@
+/*
+ * ttmlir_amd_runtime.h -- C ABI over the C++ host runtime (libttmlir_amd_rt.so).
+ *
+ * The C++ API in tt-mlir_amd/runtime/runtime.h mirrors tt::runtime (tt-mlir
+ * runtime/include/tt/runtime/runtime.h:31-308).  This header exposes the same calls with opaque
+ * handles so that any language with a C FFI can load a `.ttnn` flatbuffer, convert inputs to the
+ * program's layouts, submit and read results -- the role the nanobind module plays in the reference
+ * (runtime/python/runtime/runtime.cpp:29-847).  Each function names the tt::runtime call it wraps.
+ *
+ * Every function returns 0 on success and 1 on failure; ttrt_last_error() holds the message of the
+ * C++ exception (the reference throws std::runtime_error from LOG_FATAL).  Handles are owned by
+ * the caller and released with the matching *_free / *_destroy.
+ */
+#ifndef TTMLIR_AMD_RUNTIME_H
+#define TTMLIR_AMD_RUNTIME_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ttrt_binary ttrt_binary;
+typedef struct ttrt_device ttrt_device;
+typedef struct ttrt_tensor ttrt_tensor;
+typedef struct ttrt_builder ttrt_builder;
+
+/* (storage, layout, dtype) with the enum values of the flatbuffer schema
+ * (StorageType: Host 0, Device 1; TensorLayout: RowMajor 0, Tile 1; DataType as in Common/types.fbs) */
+typedef struct ttrt_layout {
+  int storage, layout, dtype;
+} ttrt_layout;
+
+const char *ttrt_last_error(void);
+
+/* ---- Binary: Flatbuffer::loadFromPath / loadFromMemory, getProgramInputs/Outputs (runtime/lib/binary.cpp:164-188, 422-440) */
+int ttrt_binary_load_file(const char *path, ttrt_binary **out);
+int ttrt_binary_load_memory(const void *data, size_t size, ttrt_binary **out);
+int ttrt_binary_store(const ttrt_binary *bin, const char *path);
+void ttrt_binary_free(ttrt_binary *bin);
+int ttrt_binary_num_programs(const ttrt_binary *bin, uint32_t *n);
+int ttrt_binary_program_name(const ttrt_binary *bin, uint32_t program, char *buf, size_t len);
+int ttrt_binary_program_is_private(const ttrt_binary *bin, uint32_t program, int *is_private);
+int ttrt_binary_num_inputs(const ttrt_binary *bin, uint32_t program, uint32_t *n);
+int ttrt_binary_num_outputs(const ttrt_binary *bin, uint32_t program, uint32_t *n);
+/* is_output 0: input `index`, 1: output `index`.  shape receives up to 8 extents. */
+int ttrt_binary_tensor_desc(const ttrt_binary *bin, uint32_t program, int is_output, uint32_t index, uint32_t *shape,
+                            int *rank, ttrt_layout *layout);
+int ttrt_binary_ops_text(const ttrt_binary *bin, uint32_t program, char *buf, size_t len);
+int ttrt_binary_info(const ttrt_binary *bin, char *identifier5, char *version, size_t version_len);
+
+/* ---- Device: getNumAvailableDevices / openMeshDevice / closeMeshDevice (runtime.h:151-157) */
+int ttrt_num_devices(uint32_t *n);
+int ttrt_device_open(ttrt_device **out);
+int ttrt_device_close(ttrt_device *dev);
+int ttrt_device_name(ttrt_device *dev, char *buf, size_t len);
+
+/* ---- Tensors: createOwnedHostTensor / createBorrowedHostTensor (runtime.h:56-69); stride may be NULL
+ * (contiguous) and counts elements */
+int ttrt_tensor_create_host(const void *data, const uint32_t *shape, int rank, const int64_t *stride, uint32_t itemsize,
+                            int dtype, int borrowed, ttrt_tensor **out);
+void ttrt_tensor_free(ttrt_tensor *t);
+int ttrt_tensor_desc(const ttrt_tensor *t, uint32_t *shape, int *rank, ttrt_layout *layout, uint64_t *bytes);
+int ttrt_tensor_is_allocated(const ttrt_tensor *t, int *allocated);
+int ttrt_tensor_set_retain(ttrt_tensor *t, int retain);
+int ttrt_tensor_get_retain(const ttrt_tensor *t, int *retain);
+int ttrt_tensor_deallocate(ttrt_tensor *t, int force);                         /* deallocateTensor (runtime.h:244) */
+
+/* getLayout (runtime.h:234-235), toLayout (227-228; retain: -1 unset, 0, 1), toHost (221-222), wait (212-217),
+ * memcpy(void*, Tensor, optional<DataType>) (237-238; target_dtype -1 = none), memcpy(Tensor, Tensor) (240) */
+int ttrt_get_layout(const ttrt_binary *bin, uint32_t program, uint32_t input, ttrt_layout *layout);
+int ttrt_to_layout(ttrt_tensor *t, ttrt_device *dev, const ttrt_layout *layout, int retain, ttrt_tensor **out);
+int ttrt_to_host(ttrt_tensor *t, int untilize, ttrt_tensor **out);
+int ttrt_wait(ttrt_tensor *t);
+int ttrt_memcpy_out(void *dst, const ttrt_tensor *src, int target_dtype);
+int ttrt_memcpy_tensor(ttrt_tensor *dst, const ttrt_tensor *src);
+
+/* submit (runtime.h:299-301): outputs receives up to max_outputs new handles */
+int ttrt_submit(ttrt_device *dev, const ttrt_binary *bin, uint32_t program, ttrt_tensor *const *inputs, uint32_t num_inputs,
+                ttrt_tensor **outputs, uint32_t max_outputs, uint32_t *num_outputs);
+
+/* ---- debug hooks (runtime/include/tt/runtime/debug.h:77-157): post-operator callback.  The callback
+ * may call ttrt_hook_output to fetch the op's output as an untilized host tensor (NULL if none). */
+typedef void (*ttrt_op_callback)(uint32_t op_index, const char *op_name, const char *debug_info, void *hook_ctx, void *user);
+int ttrt_set_post_op_callback(ttrt_op_callback cb, void *user);
+int ttrt_clear_callbacks(void);
+int ttrt_hook_output(void *hook_ctx, ttrt_tensor **out);
+int ttrt_stat(const char *name, int64_t *value);
+int ttrt_stats_clear(void);
+
+/* ---- host dtype casts used for unsupported host dtypes (runtime/lib/common/utils.cpp:267-360) */
+int ttrt_buffer_cast(const void *src, void *dst, int from_dtype, int to_dtype, int64_t n);
+
+/* ---- program writer (no counterpart in the reference runtime: its binaries come from the compiler).
+ * Tensor ids are the flatbuffer global_ids; 0 means "no tensor". */
+int ttrt_pb_create(ttrt_builder **out);
+void ttrt_pb_destroy(ttrt_builder *pb);
+int ttrt_pb_begin_program(ttrt_builder *pb, const char *name, int is_private);
+int ttrt_pb_end_program(ttrt_builder *pb, uint32_t *program_index);
+int ttrt_pb_input(ttrt_builder *pb, const uint32_t *shape, int rank, const ttrt_layout *layout, uint32_t *id);
+int ttrt_pb_output(ttrt_builder *pb, uint32_t id);
+int ttrt_pb_finish(ttrt_builder *pb, uint8_t **data, size_t *size);              /* free with ttrt_free_bytes */
+void ttrt_free_bytes(uint8_t *data);
+int ttrt_pb_tensor_desc(ttrt_builder *pb, uint32_t id, uint32_t *shape, int *rank, ttrt_layout *layout);
+int ttrt_pb_to_layout(ttrt_builder *pb, uint32_t in, int layout, int dtype, int storage, uint32_t *out);
+int ttrt_pb_typecast(ttrt_builder *pb, uint32_t in, int dtype, uint32_t *out);
+int ttrt_pb_to_device(ttrt_builder *pb, uint32_t in, uint32_t *out);
+int ttrt_pb_from_device(ttrt_builder *pb, uint32_t in, uint32_t *out);
+int ttrt_pb_matmul(ttrt_builder *pb, uint32_t a, uint32_t b, int transpose_a, int transpose_b, const char *activation,
+                   int out_dtype, uint32_t *out);
+int ttrt_pb_linear(ttrt_builder *pb, uint32_t a, uint32_t b, uint32_t bias, int transpose_a, int transpose_b,
+                   const char *activation, int out_dtype, uint32_t *out);
+int ttrt_pb_unary(ttrt_builder *pb, uint32_t type, uint32_t in, int has_param, float param, uint32_t *out);
+int ttrt_pb_binary(ttrt_builder *pb, uint32_t type, uint32_t lhs, uint32_t rhs, uint32_t *out);
+int ttrt_pb_rms_norm(ttrt_builder *pb, uint32_t in, uint32_t weight, uint32_t bias, float eps, uint32_t *out);
+int ttrt_pb_softmax(ttrt_builder *pb, uint32_t in, int dim, uint32_t *out);
+int ttrt_pb_reduction(ttrt_builder *pb, uint32_t type, uint32_t in, const int32_t *dims, int ndims, int keep_dim, uint32_t *out);
+int ttrt_pb_sdpa(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t mask, int is_causal, int has_scale, float scale,
+                 uint32_t *out);
+int ttrt_pb_reshape(ttrt_builder *pb, uint32_t in, const uint32_t *shape, int rank, uint32_t *out);
+int ttrt_pb_permute(ttrt_builder *pb, uint32_t in, const int64_t *perm, int rank, uint32_t *out);
+int ttrt_pb_transpose(ttrt_builder *pb, uint32_t in, int dim0, int dim1, uint32_t *out);
+int ttrt_pb_concat(ttrt_builder *pb, const uint32_t *ins, int n, int dim, uint32_t *out);
+int ttrt_pb_slice(ttrt_builder *pb, uint32_t in, const int64_t *begins, const int64_t *ends, const int64_t *steps, int rank,
+                  uint32_t *out);
+int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_t repeats, int dim, uint32_t *out);
+int ttrt_pb_constant(ttrt_builder *pb, const void *data, size_t bytes, int in_dtype, const uint32_t *shape, int rank,
+                     const ttrt_layout *layout, uint32_t *out);
+int ttrt_pb_full(ttrt_builder *pb, const uint32_t *shape, int rank, float value, int dtype, int layout, uint32_t *out);
+int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force);
+/* out_shapes: n_out entries of 8 extents each, out_ranks / out_layouts per entry */
+int ttrt_pb_load_cached(ttrt_builder *pb, uint32_t program_index, const char *callee, const uint32_t *ins, int n_in,
+                        const uint32_t *out_shapes, const int *out_ranks, const ttrt_layout *out_layouts, int n_out,
+                        uint32_t *outs);
+int ttrt_pb_func_call(ttrt_builder *pb, uint32_t program_index, const uint32_t *ins, int n_in, const uint32_t *out_shapes,
+                      const int *out_ranks, const ttrt_layout *out_layouts, int n_out, uint32_t *outs);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

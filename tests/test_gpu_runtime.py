@@ -1,0 +1,259 @@
+"""End-to-end through the drop-in boundary on the GPU: `.ttnn` flatbuffer -> Binary -> to_layout ->
+submit -> wait -> to_host, compared with the CPU oracle evaluating the same op graph in f32 with a
+bf16 cast after every op (the CPU path's per-op cast back, HoistCPUOps.cpp:219-245).
+Bars: layouts bit exact; values PCC >= 0.99 (asserted tighter) with the max-abs error stated."""
+import numpy as np
+import pytest
+import torch
+
+from ttmlir_amd import datagen, programs, runtime as rt, harness
+
+pytestmark = pytest.mark.gpu
+DT, TL, ST = rt.DataType, rt.TensorLayout, rt.StorageType
+
+
+@pytest.fixture(scope="module")
+def device(dev):
+    d = rt.open_mesh_device()
+    yield d
+    rt.close_mesh_device(d)
+
+
+@pytest.fixture(scope="module")
+def metrics():
+    import oracle.metrics as m
+    return m
+
+
+def bf(x):
+    return x.to(torch.bfloat16)
+
+
+def test_c1_matmul_program(device, orc, metrics):
+    a, b = datagen.c1_matmul()
+    binary = rt.Binary.load_from_memory(programs.c1_matmul())
+    ins = [rt.to_layout(rt.from_torch(t), device, rt.get_layout(binary, 0, i)) for i, t in enumerate((a, b))]
+    outs = rt.submit(device, binary, 0, ins)
+    rt.wait(outs)
+    c = rt.to_torch(outs[0])                                   # already a host row-major tensor
+    want = orc.round_bf16(orc.linear(a.float().numpy(), b.float().numpy()))
+    assert metrics.get_pcc(want, c.float().numpy()) >= 0.9999
+    assert np.max(np.abs(c.float().numpy() - want)) <= 0.25   # one bf16 ulp at |c| in [32, 64)
+    # layout of the tilized operand, bit exact, read back without untilizing
+    tiled = rt.to_numpy(rt.to_host(outs[1], untilize=False)[0])
+    assert np.array_equal(tiled.view(np.uint16), orc.tilize(a.view(torch.int16).numpy().view(np.uint16)))
+    assert np.array_equal(rt.to_numpy(rt.to_host(outs[1], untilize=True)[0]), a.view(torch.int16).numpy().view(np.uint16))
+
+
+@pytest.mark.parametrize("shape", [(64, 128), (2, 40, 50), (33,), (1, 1, 32, 32)])
+@pytest.mark.parametrize("dtype", [DT.BFloat16, DT.Float32, DT.BFP_BFloat8, DT.BFP_BFloat4])
+def test_to_layout_round_trip(device, orc, shape, dtype):
+    """runtime/test/ttnn/python/n150/test_runtime_api.py:71 analogue: host -> device tile (-> block float) -> host."""
+    x = datagen.randn(shape, seed=1)
+    h = rt.from_torch(x)
+    d = rt.to_layout(h, device, rt.Layout(ST.Device, TL.Tile, dtype), retain=None)
+    assert not h.is_allocated()                                 # toLayout consumes its input unless it is retained
+    assert d.layout == rt.Layout(ST.Device, TL.Tile, dtype)
+    back = rt.to_host(d, untilize=True)[0]
+    got = rt.to_numpy(back)
+    if dtype == DT.Float32:
+        assert np.array_equal(got, x.numpy())
+    elif dtype == DT.BFloat16:
+        assert np.array_equal(got, orc.f32_to_bf16(x.numpy()))
+    else:
+        fmt = 8 if dtype == DT.BFP_BFloat8 else 4
+        assert back.layout.dtype == DT.Float32               # block float reads back as float32
+        x2 = x.numpy().reshape((1,) * (2 - x.dim()) + tuple(x.shape)) if x.dim() < 2 else x.numpy()
+        want = orc.bfp_unpack(orc.bfp_pack(x2, fmt), x2.shape, fmt).reshape(shape)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        raw = rt.to_numpy(rt.to_host(d, untilize=False)[0])   # packed tile bytes, bit exact
+        assert np.array_equal(raw, orc.bfp_pack(x2, fmt))
+    keep = rt.from_torch(x)
+    keep.set_retain(True)
+    rt.to_layout(keep, device, rt.Layout(ST.Device, TL.Tile, DT.BFloat16))
+    assert keep.is_allocated()
+
+
+def test_c3_linear_program_and_const_eval_cache(device, orc, metrics):
+    M, K, N = 96, 256, 320
+    a, w, bias = datagen.c3_linear(M, K, N, seed=2)
+    binary = rt.Binary.load_from_memory(programs.c3_linear(M, K, N))
+    assert binary.get_program_name(1) == "c3_linear"
+    rt.clear_stats()
+    tins = [a, bf(w), bias]
+    ins = [rt.to_layout(rt.from_torch(t), device, rt.get_layout(binary, 1, i), retain=True) for i, t in enumerate(tins)]
+    y1 = rt.to_torch(rt.to_host(rt.submit(device, binary, 1, ins)[0], untilize=True)[0])
+    y2 = rt.to_torch(rt.to_host(rt.submit(device, binary, 1, ins)[0], untilize=True)[0])
+    assert rt.get_stat("ConstEvalCacheMiss") == 1 and rt.get_stat("ConstEvalCacheHit") == 1   # weights packed once
+    assert torch.equal(y1, y2)
+    wq = orc.bfp_unpack(orc.bfp_pack(bf(w).float().numpy(), 8), (K, N), 8)
+    want = orc.round_bf16(orc.linear(a.float().numpy(), wq, bias.float().numpy(), "gelu"))
+    assert np.max(np.abs(y1.float().numpy() - want)) <= 2.0 ** -6
+    assert metrics.get_pcc(want, y1.float().numpy()) >= 0.9999
+    # a new weight tensor (new version) invalidates the cache entry
+    ins[1] = rt.to_layout(rt.from_torch(bf(w * 2)), device, rt.get_layout(binary, 1, 1), retain=True)
+    y3 = rt.to_torch(rt.to_host(rt.submit(device, binary, 1, ins)[0], untilize=True)[0])
+    assert rt.get_stat("ConstEvalCacheMiss") == 2
+    assert not torch.equal(y1, y3)
+
+
+def oracle_mlp(orc, x, nw, wg, wu, wd, eps):
+    r = orc.round_bf16
+    q8 = lambda w: orc.bfp_unpack(orc.bfp_pack(w, 8), w.shape, 8)
+    q4 = lambda w: orc.bfp_unpack(orc.bfp_pack(w, 4), w.shape, 4)
+    h = r(orc.rms_norm(x, nw, None, eps))
+    g = r(orc.linear(h, q8(wg), None, "silu"))
+    u = r(orc.linear(h, q8(wu)))
+    m = r(orc.binary("multiply", g, u))
+    return r(orc.linear(m, q4(wd)))
+
+
+def test_c4_mlp_program_small(device, orc, metrics):
+    d = datagen.c4_mlp(tokens=96, hidden=256, ffn=512, seed=3)
+    binary = rt.Binary.load_from_memory(programs.c4_mlp(96, 256, 512))
+    tins = [d["x"], d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    (y,) = harness.execute(binary, 1, tins, device)
+    f = lambda t: t.float().numpy()
+    want = oracle_mlp(orc, f(d["x"]), f(d["norm_w"]), f(bf(d["wg"])), f(bf(d["wu"])), f(bf(d["wd"])), 1e-5)
+    err = np.max(np.abs(f(y) - want))
+    # three chained bf16 roundings; outputs are O(0.05): allow 2 bf16 ulps there (2^-11)
+    assert err <= 2.0 ** -10, err
+    assert metrics.get_pcc(want, f(y)) >= 0.999
+
+
+def test_c4_mlp_full_size_band(device, orc, metrics):
+    d = datagen.c4_mlp()
+    binary = rt.Binary.load_from_memory(programs.c4_mlp())
+    tins = [d["x"], d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    (y,) = harness.execute(binary, 1, tins, device)
+    assert tuple(y.shape) == (512, 4096) and bool(torch.isfinite(y.float()).all())
+    # torch (library) evaluation of the unquantised block on a row band: the reference's bars for bfp8 / bfp4 weights
+    rows = slice(100, 132)
+    x = d["x"][rows].float()
+    h = torch.nn.functional.rms_norm(x, (4096,), d["norm_w"].float(), 1e-5)
+    ref = (torch.nn.functional.silu(h @ bf(d["wg"]).float()) * (h @ bf(d["wu"]).float())) @ bf(d["wd"]).float()
+    assert metrics.get_pcc(ref.numpy(), y[rows].float().numpy()) >= 0.98
+
+
+def oracle_decoder(orc, d):
+    r = orc.round_bf16
+    f = lambda t: t.float().numpy()
+    q8 = lambda w: orc.bfp_unpack(orc.bfp_pack(f(bf(w)), 8), tuple(w.shape), 8)
+    S, H, nq, nkv, hd = d["seq"], d["hidden"], d["n_q"], d["n_kv"], d["head_dim"]
+    x = f(d["x"])[0]
+    h = r(orc.rms_norm(x, f(d["attn_norm_w"]), None, d["eps"]))
+    q = r(orc.linear(h, q8(d["wq"]))).reshape(S, nq, hd).transpose(1, 0, 2)[None]
+    k = r(orc.linear(h, q8(d["wk"]))).reshape(S, nkv, hd).transpose(1, 0, 2)[None]
+    v = r(orc.linear(h, q8(d["wv"]))).reshape(S, nkv, hd).transpose(1, 0, 2)[None]
+    a = r(orc.sdpa(np.ascontiguousarray(q), np.ascontiguousarray(k), np.ascontiguousarray(v), is_causal=True))
+    merged = a[0].transpose(1, 0, 2).reshape(S, nq * hd)
+    x1 = r(x + r(orc.linear(np.ascontiguousarray(merged), q8(d["wo"]))))
+    mlp = oracle_mlp(orc, x1, f(d["mlp_norm_w"]), f(bf(d["wg"])), f(bf(d["wu"])), f(bf(d["wd"])), d["eps"])
+    return r(x1 + mlp)[None]
+
+
+def test_c5_decoder_layer_small(device, orc, metrics):
+    d = datagen.c5_decoder(seq=96, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, seed=4)
+    binary = rt.Binary.load_from_memory(programs.c5_decoder(96, 256, 4, 2, 64, 512))
+    tins = [d["x"], d["attn_norm_w"], bf(d["wq"]), bf(d["wk"]), bf(d["wv"]), bf(d["wo"]), d["mlp_norm_w"], bf(d["wg"]), bf(d["wu"]),
+            bf(d["wd"])]
+    (y,) = harness.execute(binary, 1, tins, device)
+    want = oracle_decoder(orc, d)
+    got = y.float().numpy()
+    # the residual stream is O(1..4): one bf16 ulp there is 2^-6; intermediate roundings may flip a neighbour
+    assert np.max(np.abs(got - want)) <= 2.0 ** -5
+    assert metrics.get_pcc(want, got) >= 0.9999
+
+
+def test_generic_ops_program(device, orc):
+    """One program that exercises the glue ops; checked against numpy on the same values."""
+    pb = rt.ProgramBuilder()
+    pb.begin_program("glue")
+    x = pb.input((2, 48, 64), DT.BFloat16)
+    y = pb.input((2, 48, 64), DT.BFloat16)
+    s = pb.binary(programs.BINARY["add"], x, y)
+    e = pb.unary(programs.UNARY["exp"], pb.unary(programs.UNARY["neg"], pb.unary(programs.UNARY["abs"], s)))
+    sm = pb.softmax(e, -1)
+    red = pb.reduction(programs.REDUCE["sum"], sm, [-1], keep_dim=False)
+    rmax = pb.reduction(programs.REDUCE["max"], x, [1], keep_dim=True)
+    perm = pb.permute(pb.reshape(x, (2, 48, 4, 16)), (0, 2, 1, 3))
+    cat = pb.concat([x, y], 1)
+    sl = pb.slice(cat, [0, 8, 16], [2, 88, 48], [1, 2, 1])
+    rep = pb.repeat_interleave(x, 3, 0)
+    tr = pb.transpose(x, -2, -1)
+    cst = pb.constant(np.arange(64, dtype=np.float32), DT.Float32, DT.BFloat16)
+    addc = pb.binary(programs.BINARY["add"], x, cst)
+    fl = pb.binary(programs.BINARY["multiply"], x, pb.full((1,), 0.5, DT.BFloat16))
+    f32 = pb.typecast(x, DT.Float32)
+    sm0 = pb.softmax(f32, 1)
+    host = pb.from_device(pb.to_layout(s, TL.RowMajor))
+    for t in (s, sm, red, rmax, perm, cat, sl, rep, tr, addc, fl, f32, sm0, host):
+        pb.output(t)
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    a = datagen.randn((2, 48, 64), seed=5, dtype=torch.bfloat16)
+    b = datagen.randn((2, 48, 64), seed=6, dtype=torch.bfloat16)
+    outs = harness.execute(binary, 0, [a, b], device)
+    r = lambda t: torch.from_numpy(orc.round_bf16(t.float().numpy()))
+    A, B = a.float(), b.float()
+    S = r(A + B)
+    assert torch.equal(outs[0].float(), S)
+    E = r(torch.exp(r(-r(S.abs()))))
+    SM = torch.softmax(E, -1)
+    assert torch.allclose(outs[1].float(), SM, atol=2.0 ** -9, rtol=2.0 ** -7)
+    assert tuple(outs[2].shape) == (2, 48) and torch.allclose(outs[2].float(), r(SM).sum(-1), atol=2.0 ** -6)
+    assert tuple(outs[3].shape) == (2, 1, 64) and torch.equal(outs[3].float(), A.max(1, keepdim=True).values)
+    assert torch.equal(outs[4], a.reshape(2, 48, 4, 16).permute(0, 2, 1, 3))
+    assert torch.equal(outs[5], torch.cat([a, b], 1))
+    assert torch.equal(outs[6], torch.cat([a, b], 1)[:, 8:88:2, 16:48])
+    assert torch.equal(outs[7], a.repeat_interleave(3, 0))
+    assert torch.equal(outs[8], a.transpose(-2, -1))
+    assert torch.equal(outs[9].float(), r(A + torch.arange(64, dtype=torch.float32)))
+    assert torch.equal(outs[10].float(), r(A * 0.5))
+    assert outs[11].dtype == torch.float32 and torch.equal(outs[11], A)
+    assert torch.allclose(outs[12], torch.softmax(A, 1), rtol=2e-5, atol=1e-7)
+    assert torch.equal(outs[13].float(), S)
+
+
+def test_post_op_hook_sees_intermediates(device, orc):
+    binary = rt.Binary.load_from_memory(programs.c4_mlp(64, 128, 256))
+    d = datagen.c4_mlp(64, 128, 256, seed=7)
+    seen = []
+
+    def hook(idx, name, dbg, get_output):
+        t = get_output()
+        seen.append((idx, name, None if t is None else rt.to_torch(t)))
+
+    rt.set_post_op_callback(hook)
+    try:
+        harness.execute(binary, 1, [d["x"], d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])], device)
+    finally:
+        rt.clear_callbacks()
+    names = [n for _, n, _ in seen]
+    # the const-eval program's typecasts run inside the first op of the main program
+    assert names[:3] == ["TypecastOp"] * 3 and names[3] == "LoadCachedOp" and names[4] == "RMSNormOp"
+    rms = [t for _, n, t in seen if n == "RMSNormOp"][0]
+    want = orc.round_bf16(orc.rms_norm(d["x"].float().numpy(), d["norm_w"].float().numpy(), None, 1e-5))
+    assert np.max(np.abs(rms.float().numpy() - want)) <= 2.0 ** -6
+    assert [t is None for _, n, t in seen if n == "DeallocateOp"] == [True, True, True]
+
+
+def test_submit_errors(device):
+    binary = rt.Binary.load_from_memory(programs.c3_linear(32, 64, 64))
+    a = rt.from_torch(torch.zeros(32, 64, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="expects 3 inputs"):
+        rt.submit(device, binary, 1, [a])
+    w = rt.from_torch(torch.zeros(64, 64, dtype=torch.bfloat16))
+    b = rt.from_torch(torch.zeros(64, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="layout the program expects"):
+        rt.submit(device, binary, 1, [a, w, b])                   # host row-major, program wants device tiles
+    with pytest.raises(RuntimeError, match="out of range"):
+        rt.submit(device, binary, 7, [])
+    bad = rt.to_layout(rt.from_torch(torch.zeros(32, 32, dtype=torch.bfloat16)), device, rt.get_layout(binary, 1, 0))
+    with pytest.raises(RuntimeError, match="wrong shape"):
+        rt.submit(device, binary, 1, [bad, bad, bad])
+    # an op outside the supported subset is reported by name
+    freed = rt.to_layout(a, device, rt.get_layout(binary, 1, 0))
+    rt.deallocate_tensor(freed, force=True)
+    with pytest.raises(RuntimeError, match="deallocated"):
+        rt.to_host(freed)

@@ -1,0 +1,163 @@
+"""Host-side runtime logic that needs no GPU: the flatbuffer codec, binary inspection, host tensor
+creation (strides, unsupported dtype aliases) and the buffer casts with the reference's
+known-answer vectors."""
+import ctypes
+import struct
+
+import numpy as np
+import pytest
+
+from ttmlir_amd import runtime as rt, programs
+
+DT, TL, ST = rt.DataType, rt.TensorLayout, rt.StorageType
+
+
+def test_runtime_abi_symbols():
+    l = ctypes.CDLL(rt.LIB_PATH)
+    names = rt.declared_functions()
+    assert len(names) > 60
+    for n in names:
+        assert hasattr(l, n), "declared but not exported: " + n
+
+
+def test_binary_wire_format_and_inspection(tmp_path):
+    data = programs.c1_matmul()
+    # size-prefixed flatbuffer with file identifier "TTNN" (include/ttmlir/Target/TTNN/binary.fbs:17-19)
+    assert struct.unpack("<I", data[:4])[0] == len(data) - 4
+    assert data[8:12] == b"TTNN"
+    root = struct.unpack("<I", data[4:8])[0]
+    assert 0 < root < len(data) - 4 and root % 4 == 0
+    b = rt.Binary.load_from_memory(data)
+    assert b.info() == ("TTNN", "0.1.0")
+    assert b.get_num_programs() == 1 and b.get_program_name(0) == "c1_matmul"
+    ins, outs = b.get_program_inputs(0), b.get_program_outputs(0)
+    assert [s for s, _ in ins] == [(256, 512), (512, 256)]
+    assert all(l == rt.Layout(ST.Host, TL.RowMajor, DT.BFloat16) for _, l in ins)
+    assert outs[0] == ((256, 256), rt.Layout(ST.Host, TL.RowMajor, DT.BFloat16))
+    assert outs[1] == ((256, 512), rt.Layout(ST.Device, TL.Tile, DT.BFloat16))
+    text = b.get_program_ops_as_text(0)
+    assert [l.split()[1] for l in text.strip().splitlines()] == ["ToDeviceOp", "ToLayoutOp", "ToDeviceOp", "ToLayoutOp", "MatmulOp",
+                                                                "ToLayoutOp", "FromDeviceOp"]
+    p = tmp_path / "c1.ttnn"
+    b.store(p)
+    assert rt.Binary.load_from_path(p).get_program_name(0) == "c1_matmul"
+    assert rt.get_layout(b, 0, 1) == rt.Layout(ST.Host, TL.RowMajor, DT.BFloat16)
+
+
+def test_const_eval_program_structure():
+    b = rt.Binary.load_from_memory(programs.c4_mlp(tokens=64, hidden=128, ffn=256))
+    assert b.get_num_programs() == 2
+    assert b.is_program_private(0) and not b.is_program_private(1)
+    assert [l.dtype for _, l in b.get_program_outputs(0)] == [DT.BFP_BFloat8, DT.BFP_BFloat8, DT.BFP_BFloat4]
+    ops = [l.split()[1] for l in b.get_program_ops_as_text(1).strip().splitlines()]
+    assert ops == ["LoadCachedOp", "RMSNormOp", "LinearOp", "MatmulOp", "EltwiseBinaryOp", "DeallocateOp", "DeallocateOp", "MatmulOp",
+                   "DeallocateOp"]
+
+
+def test_decoder_program_shapes():
+    b = rt.Binary.load_from_memory(programs.c5_decoder(seq=64, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512))
+    assert b.get_program_outputs(1)[0][0] == (1, 64, 256)
+    assert len(b.get_program_inputs(1)) == 10
+    assert "ScaledDotProductAttentionOp" in b.get_program_ops_as_text(1)
+
+
+@pytest.mark.parametrize("bad", [b"", b"\x00" * 8, b"\x10\x00\x00\x00" + b"\x00" * 16, b"garbage-that-is-not-a-flatbuffer!"])
+def test_malformed_binaries_are_rejected(bad):
+    with pytest.raises(RuntimeError):
+        rt.Binary.load_from_memory(bad)
+
+
+def test_truncated_binary_is_rejected():
+    data = programs.c1_matmul()
+    with pytest.raises(RuntimeError):
+        rt.Binary.load_from_memory(data[: len(data) // 2])
+    wrong = bytearray(data)
+    wrong[8:12] = b"TTM0"
+    with pytest.raises(RuntimeError):
+        rt.Binary.load_from_memory(bytes(wrong))
+
+
+def test_buffer_cast_known_answers():
+    # runtime/test/common/gtest/test_handle_float_bfloat_buffer_cast.cpp:8-46
+    f16 = np.array([0xBC00, 0, 0xBC00], dtype=np.uint16).view(np.float16)
+    assert rt.buffer_cast(f16, DT.Float16, DT.BFloat16).tolist() == [0xBF80, 0, 0xBF80]
+    bf = np.array([0xBF80, 0, 0xBF80], dtype=np.uint16)
+    assert rt.buffer_cast(bf, DT.BFloat16, DT.Float16).view(np.uint16).tolist() == [0xBC00, 0, 0xBC00]
+    mm = np.array([0xFBFF, 0x7BFF], dtype=np.uint16).view(np.float16)
+    assert rt.buffer_cast(mm, DT.Float16, DT.BFloat16).tolist() == [0xC780, 0x4780]
+
+
+def test_integer_buffer_casts_saturate():
+    # runtime/test/common/gtest/test_handle_integer_buffer_cast.cpp:8-66: clamp to the destination range
+    i64 = np.array([0, -1, 2 ** 31 - 1, 2 ** 31, -2 ** 31 - 1, 2 ** 62, -2 ** 62], dtype=np.int64)
+    assert rt.buffer_cast(i64, DT.Int64, DT.Int32).tolist() == [0, -1, 2 ** 31 - 1, 2 ** 31 - 1, -2 ** 31, 2 ** 31 - 1, -2 ** 31]
+    u64 = np.array([0, 2 ** 32 - 1, 2 ** 32, 2 ** 63], dtype=np.uint64)
+    assert rt.buffer_cast(u64, DT.UInt64, DT.UInt32).tolist() == [0, 2 ** 32 - 1, 2 ** 32 - 1, 2 ** 32 - 1]
+    i16 = np.array([-5, 0, 7, -32768, 32767], dtype=np.int16)
+    assert rt.buffer_cast(i16, DT.Int16, DT.UInt16).tolist() == [0, 0, 7, 0, 32767]
+    u16 = np.array([0, 32767, 32768, 65535], dtype=np.uint16)
+    assert rt.buffer_cast(u16, DT.UInt16, DT.Int16).tolist() == [0, 32767, 32767, 32767]
+    i8 = np.array([-128, -1, 0, 127], dtype=np.int8)
+    assert rt.buffer_cast(i8, DT.Int8, DT.UInt8).tolist() == [0, 0, 0, 127]
+    assert rt.buffer_cast(np.array([1, 2 ** 31 - 1], dtype=np.int32), DT.Int32, DT.Int64).tolist() == [1, 2 ** 31 - 1]
+    assert rt.buffer_cast(np.array([2 ** 32 - 1], dtype=np.uint32), DT.UInt32, DT.Int64).tolist() == [2 ** 32 - 1]
+    f64 = np.array([1.5, -2.25, 1e300], dtype=np.float64)
+    assert rt.buffer_cast(f64, DT.Float64, DT.Float32).tolist() == [1.5, -2.25, float("inf")]
+    with pytest.raises(RuntimeError):
+        rt.buffer_cast(f64, DT.Float64, DT.Int32)
+
+
+def test_owned_host_tensor_gathers_strides():
+    # runtime/test/ttnn/gtest/test_owned_host_tensor_strided.cpp:44-92: element strides, non-contiguous source
+    base = np.arange(24, dtype=np.float32).reshape(4, 6)
+    t = rt.create_owned_host_tensor(base, DT.Float32, stride=None)
+    assert np.array_equal(rt.to_numpy(t), base)
+    # view of every other column: shape [4,3], strides (6, 2) elements
+    src = np.ascontiguousarray(base)
+    h = ctypes.c_void_p()
+    shape = (ctypes.c_uint32 * 8)(4, 3)
+    stride = (ctypes.c_int64 * 8)(6, 2)
+    assert rt.lib().ttrt_tensor_create_host(ctypes.c_void_p(src.ctypes.data), shape, 2, stride, 4, DT.Float32, 0, ctypes.byref(h)) == 0
+    assert np.array_equal(rt.to_numpy(rt.Tensor(h)), base[:, ::2])
+    # a transposed view
+    stride = (ctypes.c_int64 * 8)(1, 6)
+    shape = (ctypes.c_uint32 * 8)(6, 4)
+    assert rt.lib().ttrt_tensor_create_host(ctypes.c_void_p(src.ctypes.data), shape, 2, stride, 4, DT.Float32, 0, ctypes.byref(h)) == 0
+    assert np.array_equal(rt.to_numpy(rt.Tensor(h)), base.T)
+    # borrowed tensors must be contiguous
+    assert rt.lib().ttrt_tensor_create_host(ctypes.c_void_p(src.ctypes.data), shape, 2, stride, 4, DT.Float32, 1, ctypes.byref(h)) == 1
+    assert b"non-contiguous" in rt.lib().ttrt_last_error()
+
+
+def test_unsupported_host_dtypes_are_aliased():
+    # i64 -> i32 with saturation on the way in, cast back on the way out (runtime/lib/ttnn/runtime.cpp:120-141, 999-1041)
+    x = np.array([[1, -2, 2 ** 40], [3, 4, -2 ** 40]], dtype=np.int64)
+    t = rt.create_owned_host_tensor(x, DT.Int64)
+    assert t.layout.dtype == DT.Int32
+    back = rt.to_numpy(t, target_dtype=DT.Int64)
+    assert back.dtype == np.int64 and back.tolist() == [[1, -2, 2 ** 31 - 1], [3, 4, -2 ** 31]]
+    f = rt.create_owned_host_tensor(np.array([1.5, 2.5], dtype=np.float64), DT.Float64)
+    assert f.layout.dtype == DT.Float32 and rt.to_numpy(f).tolist() == [1.5, 2.5]
+    b = rt.create_owned_host_tensor(np.array([True, False, True]), DT.Bool)
+    assert b.layout.dtype == DT.BFloat16 and rt.to_numpy(b).tolist() == [0x3F80, 0, 0x3F80]
+    h = rt.create_owned_host_tensor(np.array([1.0, -2.0], dtype=np.float16), DT.Float16)
+    assert h.layout.dtype == DT.BFloat16 and rt.to_numpy(h).tolist() == [0x3F80, 0xC000]
+
+
+def test_borrowed_tensor_aliases_and_retain_flag():
+    a = np.arange(6, dtype=np.float32).reshape(2, 3)
+    t = rt.create_borrowed_host_tensor(a, DT.Float32)
+    a[0, 0] = 42.0
+    assert rt.to_numpy(t)[0, 0] == 42.0
+    assert not t.get_retain()
+    t.set_retain(True)
+    assert t.get_retain()
+    with pytest.raises(RuntimeError):
+        rt.create_owned_host_tensor(np.zeros(4, np.uint8), DT.BFP_BFloat8)
+
+
+def test_submit_without_device_fails_cleanly():
+    if rt.get_num_available_devices() > 0:
+        pytest.skip("a GPU is visible")
+    with pytest.raises(RuntimeError):
+        rt.open_mesh_device()

@@ -91,7 +91,8 @@ def build_runtime(force=False, jobs=8, verbose=True):
             if verbose and out.strip():
                 print(out)
     if force or not _newer(RT_LIB, objs):
-        _run([CXX, "-shared", "-fPIC", "-pthread", "-o", RT_LIB] + objs + ["-ldl"])
+        _run([CXX, "-shared", "-fPIC", "-pthread", "-o", RT_LIB] + objs +
+             ["-L", LIBDIR, "-lttmlir_amd_hip", "-Wl,-rpath,$ORIGIN", "-ldl"])
     return RT_LIB
 
 

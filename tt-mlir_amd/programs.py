@@ -1,0 +1,122 @@
+"""`.ttnn` programs of the benchmark configurations, written with the ProgramBuilder.
+
+The reference produces these binaries with its compiler (ttmlir-opt + ttmlir-translate); none is
+checked in, so each configuration is rebuilt here op by op in the form the compiler emits:
+weights enter as bf16 device tensors and are converted to block-float by a private const-eval
+program reached through ttcore.load_cached (TTNNWeightDtypeConversion.cpp:102-131,
+test/ttmlir/Silicon/TTNN/n150/mixed_precision/linear.mlir:9); inputs are expected in
+Device / Tile / bf16 layout, which callers obtain with to_layout(get_layout(...)).
+"""
+from . import runtime as rt
+
+DT, TL, ST = rt.DataType, rt.TensorLayout, rt.StorageType
+# EltwiseUnaryOpType / EltwiseBinaryOpType / ReductionOpType values
+UNARY = dict(abs=0, ceil=1, cos=2, floor=3, gelu=4, isfinite=5, logical_not=6, neg=7, relu=8, sqrt=9, rsqrt=10,
+             sigmoid=11, sin=12, reciprocal=13, sign=14, tan=15, tanh=16, atan=17, exp=18, erf=19, erfc=20, log=21,
+             expm1=22, leaky_relu=23, relu6=25, silu=26)
+BINARY = dict(add=0, multiply=1, subtract=3, eq=4, ne=5, ge=6, gt=7, le=8, lt=9, divide=10)
+REDUCE = dict(sum=0, mean=1, max=2, min=3)
+
+
+def _consteval_pack(pb, name, shapes_dtypes):
+    """Private program: typecast each bf16 weight to its block-float dtype.  Returns (index, out descs)."""
+    pb.begin_program(name, private=True)
+    outs = []
+    for shape, dtype in shapes_dtypes:
+        w = pb.input(shape, DT.BFloat16)
+        o = pb.typecast(w, dtype)
+        pb.output(o)
+        outs.append((tuple(shape), rt.Layout(ST.Device, TL.Tile, dtype)))
+    return pb.end_program(), outs
+
+
+def c1_matmul():
+    """Config 1: to_layout(TILE) -> matmul [256,512] x [512,256] -> to_layout(ROW_MAJOR); inputs on the host."""
+    pb = rt.ProgramBuilder()
+    pb.begin_program("c1_matmul")
+    a = pb.input((256, 512), DT.BFloat16, TL.RowMajor, ST.Host)
+    b = pb.input((512, 256), DT.BFloat16, TL.RowMajor, ST.Host)
+    at = pb.to_layout(pb.to_device(a), TL.Tile)
+    bt = pb.to_layout(pb.to_device(b), TL.Tile)
+    c = pb.matmul(at, bt)
+    out = pb.from_device(pb.to_layout(c, TL.RowMajor))
+    pb.output(out)
+    pb.output(at)      # the tilized operand, so the layout can be checked bit-exactly
+    pb.end_program()
+    return pb.finish()
+
+
+def c3_linear(M, K=4096, N=14336, weight_dtype=DT.BFP_BFloat8, activation="gelu"):
+    """Config 3: linear with block-float weights (packed once by a const-eval program), bias + GELU."""
+    pb = rt.ProgramBuilder()
+    ce, ce_outs = _consteval_pack(pb, "c3_linear_const_eval_0", [((K, N), weight_dtype)])
+    pb.begin_program("c3_linear")
+    a = pb.input((M, K), DT.BFloat16)
+    w = pb.input((K, N), DT.BFloat16)
+    bias = pb.input((N,), DT.BFloat16)
+    (wq,) = pb.load_cached(ce, "c3_linear_const_eval_0", [w], ce_outs)
+    y = pb.linear(a, wq, bias, activation=activation)
+    pb.output(y)
+    pb.end_program()
+    return pb.finish()
+
+
+def _mlp(pb, x, norm_w, wg, wu, wd, eps):
+    h = pb.rms_norm(x, norm_w, 0, eps)
+    g = pb.linear(h, wg, 0, activation="silu")
+    u = pb.matmul(h, wu)
+    m = pb.binary(BINARY["multiply"], g, u)
+    pb.deallocate(g)
+    pb.deallocate(u)
+    d = pb.matmul(m, wd)
+    pb.deallocate(m)
+    return d
+
+
+def c4_mlp(tokens=512, hidden=4096, ffn=14336, eps=1e-5):
+    """Config 4: RMSNorm -> gate/up (bfp8_b) -> SiLU(gate)*up -> down (bfp4_b)."""
+    pb = rt.ProgramBuilder()
+    ce, ce_outs = _consteval_pack(pb, "c4_mlp_const_eval_0", [((hidden, ffn), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8),
+                                                             ((ffn, hidden), DT.BFP_BFloat4)])
+    pb.begin_program("c4_mlp")
+    x = pb.input((tokens, hidden), DT.BFloat16)
+    nw = pb.input((hidden,), DT.BFloat16)
+    wg, wu, wd = pb.input((hidden, ffn), DT.BFloat16), pb.input((hidden, ffn), DT.BFloat16), pb.input((ffn, hidden), DT.BFloat16)
+    qg, qu, qd = pb.load_cached(ce, "c4_mlp_const_eval_0", [wg, wu, wd], ce_outs)
+    pb.output(_mlp(pb, x, nw, qg, qu, qd, eps))
+    pb.end_program()
+    return pb.finish()
+
+
+def c5_decoder(seq=2048, hidden=4096, n_q=32, n_kv=8, head_dim=128, ffn=14336, eps=1e-5):
+    """Config 5: Llama-3-8B-shaped decoder layer, batch 1 prefill (op mix of
+    test/ttmlir/models/single_blocks_and_layers/llama_3_8b_prefill_layer.mlir:54-304 without rotary embedding)."""
+    pb = rt.ProgramBuilder()
+    dq, dkv = n_q * head_dim, n_kv * head_dim
+    ce, ce_outs = _consteval_pack(pb, "c5_decoder_const_eval_0", [
+        ((hidden, dq), DT.BFP_BFloat8), ((hidden, dkv), DT.BFP_BFloat8), ((hidden, dkv), DT.BFP_BFloat8),
+        ((dq, hidden), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8),
+        ((ffn, hidden), DT.BFP_BFloat4)])
+    pb.begin_program("c5_decoder_layer")
+    x = pb.input((1, seq, hidden), DT.BFloat16)
+    anw = pb.input((hidden,), DT.BFloat16)
+    wq, wk, wv, wo = (pb.input(s, DT.BFloat16) for s in ((hidden, dq), (hidden, dkv), (hidden, dkv), (dq, hidden)))
+    mnw = pb.input((hidden,), DT.BFloat16)
+    wg, wu, wd = pb.input((hidden, ffn), DT.BFloat16), pb.input((hidden, ffn), DT.BFloat16), pb.input((ffn, hidden), DT.BFloat16)
+    qq, qk, qv, qo, qg, qu, qd = pb.load_cached(ce, "c5_decoder_const_eval_0", [wq, wk, wv, wo, wg, wu, wd], ce_outs)
+    h = pb.rms_norm(x, anw, 0, eps)
+    q = pb.permute(pb.reshape(pb.matmul(h, qq), (1, seq, n_q, head_dim)), (0, 2, 1, 3))
+    k = pb.permute(pb.reshape(pb.matmul(h, qk), (1, seq, n_kv, head_dim)), (0, 2, 1, 3))
+    v = pb.permute(pb.reshape(pb.matmul(h, qv), (1, seq, n_kv, head_dim)), (0, 2, 1, 3))
+    pb.deallocate(h)
+    attn = pb.sdpa(q, k, v, 0, is_causal=True)
+    for t in (q, k, v):
+        pb.deallocate(t)
+    merged = pb.reshape(pb.permute(attn, (0, 2, 1, 3)), (1, seq, dq))
+    pb.deallocate(attn)
+    x1 = pb.binary(BINARY["add"], x, pb.matmul(merged, qo))
+    d = _mlp(pb, x1, mnw, qg, qu, qd, eps)
+    out = pb.binary(BINARY["add"], x1, d)
+    pb.output(out)
+    pb.end_program()
+    return pb.finish()

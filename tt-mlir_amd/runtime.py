@@ -1,0 +1,502 @@
+"""Python surface of the host runtime (ctypes over lib/libttmlir_amd_rt.so).
+
+Mirrors the calls a tt-mlir harness makes on `ttrt.runtime` / `_ttmlir_runtime`
+(tools/builder/base/builder_runtime.py:112-169, 694-803; tools/ttrt/common/run.py:534-873):
+load a binary, open a device, create host tensors, get_layout / to_layout, submit, wait, to_host,
+memcpy.  Tensors cross the boundary as numpy arrays (bf16 as uint16 bit patterns or torch tensors).
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libttmlir_amd_rt.so")
+HEADER = os.path.join(os.path.dirname(_HERE), "include", "ttmlir_amd_runtime.h")
+
+
+class RuntimeError_(RuntimeError):
+    pass
+
+
+class DataType:
+    Float32, Float16, BFloat16, BFP_Float8, BFP_BFloat8, BFP_Float4, BFP_BFloat4, BFP_Float2, BFP_BFloat2 = range(9)
+    UInt32, UInt16, UInt8, Int32, Float64, Int64, UInt64, Int16, Int8, Bool = range(9, 19)
+
+
+class TensorLayout:
+    RowMajor, Tile = 0, 1
+
+
+class StorageType:
+    Host, Device = 0, 1
+
+
+class Layout(ctypes.Structure):
+    _fields_ = [("storage", ctypes.c_int), ("layout", ctypes.c_int), ("dtype", ctypes.c_int)]
+
+    def __repr__(self):
+        return "Layout(storage=%d, layout=%d, dtype=%d)" % (self.storage, self.layout, self.dtype)
+
+    def __eq__(self, o):
+        return (self.storage, self.layout, self.dtype) == (o.storage, o.layout, o.dtype)
+
+
+_NP_DTYPE = {DataType.Float32: np.float32, DataType.Float16: np.float16, DataType.BFloat16: np.uint16, DataType.UInt32: np.uint32,
+             DataType.UInt16: np.uint16, DataType.UInt8: np.uint8, DataType.Int32: np.int32, DataType.Float64: np.float64,
+             DataType.Int64: np.int64, DataType.UInt64: np.uint64, DataType.Int16: np.int16, DataType.Int8: np.int8,
+             DataType.Bool: np.bool_}
+_ITEMSIZE = {k: np.dtype(v).itemsize for k, v in _NP_DTYPE.items()}
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError_("native runtime library missing: %s (run `python tt-mlir_amd/build.py`)" % LIB_PATH)
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.ttrt_last_error.restype = ctypes.c_char_p
+    return _lib
+
+
+def declared_functions():
+    import re
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ttrt_\w+)\s*\(", text)) - {"ttrt_op_callback"})
+
+
+def _ck(status, what):
+    if status != 0:
+        raise RuntimeError_("%s: %s" % (what, lib().ttrt_last_error().decode()))
+
+
+def _call(name, *args):
+    _ck(getattr(lib(), name)(*args), name)
+
+
+def _shape_arg(shape):
+    arr = (ctypes.c_uint32 * 8)(*[int(s) for s in shape])
+    return arr, len(shape)
+
+
+class Binary:
+    def __init__(self, handle):
+        self.h = handle
+
+    @staticmethod
+    def load_from_path(path):
+        h = ctypes.c_void_p()
+        _call("ttrt_binary_load_file", str(path).encode(), ctypes.byref(h))
+        return Binary(h)
+
+    @staticmethod
+    def load_from_memory(data):
+        h = ctypes.c_void_p()
+        buf = (ctypes.c_uint8 * len(data)).from_buffer_copy(data)
+        _call("ttrt_binary_load_memory", buf, ctypes.c_size_t(len(data)), ctypes.byref(h))
+        return Binary(h)
+
+    def store(self, path):
+        _call("ttrt_binary_store", self.h, str(path).encode())
+
+    def get_num_programs(self):
+        n = ctypes.c_uint32()
+        _call("ttrt_binary_num_programs", self.h, ctypes.byref(n))
+        return n.value
+
+    def get_program_name(self, i):
+        buf = ctypes.create_string_buffer(256)
+        _call("ttrt_binary_program_name", self.h, i, buf, 256)
+        return buf.value.decode()
+
+    def is_program_private(self, i):
+        v = ctypes.c_int()
+        _call("ttrt_binary_program_is_private", self.h, i, ctypes.byref(v))
+        return bool(v.value)
+
+    def _descs(self, program, is_output):
+        n = ctypes.c_uint32()
+        _call("ttrt_binary_num_outputs" if is_output else "ttrt_binary_num_inputs", self.h, program, ctypes.byref(n))
+        out = []
+        for i in range(n.value):
+            shape, rank, lay = (ctypes.c_uint32 * 8)(), ctypes.c_int(), Layout()
+            _call("ttrt_binary_tensor_desc", self.h, program, int(is_output), i, shape, ctypes.byref(rank), ctypes.byref(lay))
+            out.append((tuple(shape[: rank.value]), lay))
+        return out
+
+    def get_program_inputs(self, program):
+        return self._descs(program, False)
+
+    def get_program_outputs(self, program):
+        return self._descs(program, True)
+
+    def get_program_ops_as_text(self, program):
+        buf = ctypes.create_string_buffer(1 << 16)
+        _call("ttrt_binary_ops_text", self.h, program, buf, 1 << 16)
+        return buf.value.decode()
+
+    def info(self):
+        ident, ver = ctypes.create_string_buffer(5), ctypes.create_string_buffer(64)
+        _call("ttrt_binary_info", self.h, ident, ver, 64)
+        return ident.value.decode(), ver.value.decode()
+
+    def __del__(self):
+        try:
+            lib().ttrt_binary_free(self.h)
+        except Exception:
+            pass
+
+
+class Device:
+    def __init__(self, handle):
+        self.h = handle
+
+    def name(self):
+        buf = ctypes.create_string_buffer(256)
+        _call("ttrt_device_name", self.h, buf, 256)
+        return buf.value.decode()
+
+
+class Tensor:
+    def __init__(self, handle, keepalive=None):
+        self.h = handle
+        self._keepalive = keepalive  # borrowed host memory must outlive the tensor
+
+    def desc(self):
+        shape, rank, lay, nbytes = (ctypes.c_uint32 * 8)(), ctypes.c_int(), Layout(), ctypes.c_uint64()
+        _call("ttrt_tensor_desc", self.h, shape, ctypes.byref(rank), ctypes.byref(lay), ctypes.byref(nbytes))
+        return tuple(shape[: rank.value]), lay, nbytes.value
+
+    @property
+    def shape(self):
+        return self.desc()[0]
+
+    @property
+    def layout(self):
+        return self.desc()[1]
+
+    def is_allocated(self):
+        v = ctypes.c_int()
+        _call("ttrt_tensor_is_allocated", self.h, ctypes.byref(v))
+        return bool(v.value)
+
+    def set_retain(self, retain):
+        _call("ttrt_tensor_set_retain", self.h, int(retain))
+
+    def get_retain(self):
+        v = ctypes.c_int()
+        _call("ttrt_tensor_get_retain", self.h, ctypes.byref(v))
+        return bool(v.value)
+
+    def __del__(self):
+        try:
+            lib().ttrt_tensor_free(self.h)
+        except Exception:
+            pass
+
+
+def get_num_available_devices():
+    n = ctypes.c_uint32()
+    _call("ttrt_num_devices", ctypes.byref(n))
+    return n.value
+
+
+def open_mesh_device():
+    h = ctypes.c_void_p()
+    _call("ttrt_device_open", ctypes.byref(h))
+    return Device(h)
+
+
+def close_mesh_device(dev):
+    _call("ttrt_device_close", dev.h)
+    dev.h = None
+
+
+def _host(array, dtype, borrowed, stride=None):
+    a = np.asarray(array)
+    if stride is None:
+        a = np.ascontiguousarray(a)
+    shape, rank = _shape_arg(a.shape)
+    st = None
+    if stride is not None:
+        st = (ctypes.c_int64 * 8)(*[int(s) for s in stride])
+    h = ctypes.c_void_p()
+    _call("ttrt_tensor_create_host", ctypes.c_void_p(a.ctypes.data), shape, rank, st, a.dtype.itemsize, dtype, int(borrowed),
+          ctypes.byref(h))
+    return Tensor(h, keepalive=a if borrowed else None)
+
+
+def create_owned_host_tensor(array, dtype, stride=None):
+    """createOwnedHostTensor: copies (and gathers strides); `array` is numpy, bf16 as uint16 bits."""
+    return _host(array, dtype, False, stride)
+
+
+def create_borrowed_host_tensor(array, dtype):
+    """createBorrowedHostTensor: aliases the numpy buffer, which the returned object keeps alive."""
+    return _host(array, dtype, True)
+
+
+def from_torch(t, borrowed=False):
+    """Host tensor from a CPU torch tensor (bf16 / f32 / f16 / ints)."""
+    import torch
+    m = {torch.float32: (DataType.Float32, None), torch.bfloat16: (DataType.BFloat16, torch.int16),
+         torch.float16: (DataType.Float16, None), torch.int32: (DataType.Int32, None), torch.int64: (DataType.Int64, None),
+         torch.uint8: (DataType.UInt8, None), torch.float64: (DataType.Float64, None), torch.int16: (DataType.Int16, None),
+         torch.int8: (DataType.Int8, None), torch.bool: (DataType.Bool, None)}
+    dt, view = m[t.dtype]
+    a = t.contiguous()
+    arr = a.view(view).numpy().view(np.uint16) if view is not None else a.numpy()
+    return _host(arr, dt, borrowed)
+
+
+def get_layout(binary, program, input_index):
+    lay = Layout()
+    _call("ttrt_get_layout", binary.h, program, input_index, ctypes.byref(lay))
+    return lay
+
+
+def to_layout(tensor, device, layout, retain=None):
+    h = ctypes.c_void_p()
+    _call("ttrt_to_layout", tensor.h, device.h, ctypes.byref(layout), -1 if retain is None else int(retain), ctypes.byref(h))
+    return Tensor(h, keepalive=tensor._keepalive)
+
+
+def to_host(tensor, untilize=False):
+    h = ctypes.c_void_p()
+    _call("ttrt_to_host", tensor.h, int(untilize), ctypes.byref(h))
+    return [Tensor(h)]
+
+
+def wait(tensor_or_list):
+    for t in (tensor_or_list if isinstance(tensor_or_list, (list, tuple)) else [tensor_or_list]):
+        _call("ttrt_wait", t.h)
+
+
+def submit(device, binary, program, inputs):
+    ins = (ctypes.c_void_p * max(1, len(inputs)))(*[t.h for t in inputs])
+    outs = (ctypes.c_void_p * 64)()
+    n = ctypes.c_uint32()
+    _call("ttrt_submit", device.h, binary.h, program, ins, len(inputs), outs, 64, ctypes.byref(n))
+    return [Tensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
+
+
+def deallocate_tensor(tensor, force=False):
+    _call("ttrt_tensor_deallocate", tensor.h, int(force))
+
+
+def memcpy(dst_array, src_tensor, target_dtype=None):
+    """memcpy(void*, Tensor, optional<DataType>) into a numpy array."""
+    _call("ttrt_memcpy_out", ctypes.c_void_p(dst_array.ctypes.data), src_tensor.h, -1 if target_dtype is None else target_dtype)
+
+
+def to_numpy(tensor, target_dtype=None):
+    """Host tensor -> numpy array (bf16 as uint16 bits; block-float host tensors as raw bytes)."""
+    shape, lay, nbytes = tensor.desc()
+    if lay.storage != StorageType.Host:
+        tensor = to_host(tensor, untilize=True)[0]
+        shape, lay, nbytes = tensor.desc()
+    dt = lay.dtype if target_dtype is None else target_dtype
+    if dt not in _NP_DTYPE or lay.layout == TensorLayout.Tile:
+        out = np.empty(nbytes, dtype=np.uint8)
+        memcpy(out, tensor)
+        return out
+    out = np.empty(shape, dtype=_NP_DTYPE[dt])
+    memcpy(out, tensor, target_dtype)
+    return out
+
+
+def to_torch(tensor):
+    import torch
+    a = to_numpy(tensor)
+    lay = tensor.desc()[1]
+    if lay.dtype == DataType.BFloat16:
+        return torch.from_numpy(a.view(np.int16)).view(torch.bfloat16)
+    return torch.from_numpy(a)
+
+
+def buffer_cast(src, from_dtype, to_dtype):
+    src = np.ascontiguousarray(src)
+    dst = np.empty(src.shape, dtype=_NP_DTYPE[to_dtype])
+    _call("ttrt_buffer_cast", ctypes.c_void_p(src.ctypes.data), ctypes.c_void_p(dst.ctypes.data), from_dtype, to_dtype, ctypes.c_int64(src.size))
+    return dst
+
+
+def get_stat(name):
+    v = ctypes.c_int64()
+    _call("ttrt_stat", name.encode(), ctypes.byref(v))
+    return v.value
+
+
+def clear_stats():
+    _call("ttrt_stats_clear")
+
+
+_CB_TYPE = ctypes.CFUNCTYPE(None, ctypes.c_uint32, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_void_p)
+_cb_keep = None
+
+
+def set_post_op_callback(fn):
+    """fn(op_index, op_name, debug_info, get_output) with get_output() -> host Tensor or None."""
+    global _cb_keep
+
+    def tramp(idx, name, dbg, hook, user):
+        def get_output():
+            h = ctypes.c_void_p()
+            _call("ttrt_hook_output", ctypes.c_void_p(hook), ctypes.byref(h))
+            return Tensor(h) if h.value else None
+        fn(idx, name.decode(), dbg.decode(), get_output)
+
+    _cb_keep = _CB_TYPE(tramp)
+    _call("ttrt_set_post_op_callback", _cb_keep, None)
+
+
+def clear_callbacks():
+    global _cb_keep
+    _call("ttrt_clear_callbacks")
+    _cb_keep = None
+
+
+class ProgramBuilder:
+    """Writes `.ttnn` programs; ids are flatbuffer global_ids (0 = no tensor)."""
+
+    def __init__(self):
+        self.h = ctypes.c_void_p()
+        _call("ttrt_pb_create", ctypes.byref(self.h))
+
+    def __del__(self):
+        try:
+            lib().ttrt_pb_destroy(self.h)
+        except Exception:
+            pass
+
+    def begin_program(self, name, private=False):
+        _call("ttrt_pb_begin_program", self.h, name.encode(), int(private))
+
+    def end_program(self):
+        i = ctypes.c_uint32()
+        _call("ttrt_pb_end_program", self.h, ctypes.byref(i))
+        return i.value
+
+    def input(self, shape, dtype, layout=TensorLayout.Tile, storage=StorageType.Device):
+        s, r = _shape_arg(shape)
+        out = ctypes.c_uint32()
+        _call("ttrt_pb_input", self.h, s, r, ctypes.byref(Layout(storage, layout, dtype)), ctypes.byref(out))
+        return out.value
+
+    def output(self, t):
+        _call("ttrt_pb_output", self.h, t)
+
+    def finish(self):
+        data, size = ctypes.POINTER(ctypes.c_uint8)(), ctypes.c_size_t()
+        _call("ttrt_pb_finish", self.h, ctypes.byref(data), ctypes.byref(size))
+        out = ctypes.string_at(data, size.value)
+        lib().ttrt_free_bytes(data)
+        return out
+
+    def desc(self, t):
+        shape, rank, lay = (ctypes.c_uint32 * 8)(), ctypes.c_int(), Layout()
+        _call("ttrt_pb_tensor_desc", self.h, t, shape, ctypes.byref(rank), ctypes.byref(lay))
+        return tuple(shape[: rank.value]), lay
+
+    def _op(self, name, *args):
+        out = ctypes.c_uint32()
+        _call(name, self.h, *args, ctypes.byref(out))
+        return out.value
+
+    def to_layout(self, t, layout, dtype=None, storage=StorageType.Device):
+        return self._op("ttrt_pb_to_layout", t, layout, -1 if dtype is None else dtype, storage)
+
+    def typecast(self, t, dtype):
+        return self._op("ttrt_pb_typecast", t, dtype)
+
+    def to_device(self, t):
+        return self._op("ttrt_pb_to_device", t)
+
+    def from_device(self, t):
+        return self._op("ttrt_pb_from_device", t)
+
+    def matmul(self, a, b, transpose_a=False, transpose_b=False, activation="", out_dtype=DataType.BFloat16):
+        return self._op("ttrt_pb_matmul", a, b, int(transpose_a), int(transpose_b), activation.encode(), out_dtype)
+
+    def linear(self, a, b, bias=0, transpose_a=False, transpose_b=False, activation="", out_dtype=DataType.BFloat16):
+        return self._op("ttrt_pb_linear", a, b, bias, int(transpose_a), int(transpose_b), activation.encode(), out_dtype)
+
+    def unary(self, type_, t, param=None):
+        return self._op("ttrt_pb_unary", type_, t, int(param is not None), ctypes.c_float(param or 0.0))
+
+    def binary(self, type_, a, b):
+        return self._op("ttrt_pb_binary", type_, a, b)
+
+    def rms_norm(self, t, weight=0, bias=0, eps=1e-5):
+        return self._op("ttrt_pb_rms_norm", t, weight, bias, ctypes.c_float(eps))
+
+    def softmax(self, t, dim=-1):
+        return self._op("ttrt_pb_softmax", t, dim)
+
+    def reduction(self, type_, t, dims, keep_dim=False):
+        d = (ctypes.c_int32 * max(1, len(dims)))(*dims)
+        return self._op("ttrt_pb_reduction", type_, t, d, len(dims), int(keep_dim))
+
+    def sdpa(self, q, k, v, mask=0, is_causal=False, scale=None):
+        return self._op("ttrt_pb_sdpa", q, k, v, mask, int(is_causal), int(scale is not None), ctypes.c_float(scale or 0.0))
+
+    def reshape(self, t, shape):
+        s, r = _shape_arg(shape)
+        return self._op("ttrt_pb_reshape", t, s, r)
+
+    def permute(self, t, perm):
+        p = (ctypes.c_int64 * len(perm))(*perm)
+        return self._op("ttrt_pb_permute", t, p, len(perm))
+
+    def transpose(self, t, dim0, dim1):
+        return self._op("ttrt_pb_transpose", t, dim0, dim1)
+
+    def concat(self, ts, dim):
+        a = (ctypes.c_uint32 * len(ts))(*ts)
+        return self._op("ttrt_pb_concat", a, len(ts), dim)
+
+    def slice(self, t, begins, ends, steps=None):
+        n = len(begins)
+        steps = steps or [1] * n
+        mk = lambda v: (ctypes.c_int64 * n)(*v)
+        return self._op("ttrt_pb_slice", t, mk(begins), mk(ends), mk(steps), n)
+
+    def repeat_interleave(self, t, repeats, dim):
+        return self._op("ttrt_pb_repeat_interleave", t, repeats, dim)
+
+    def constant(self, array, in_dtype, dtype=None, layout=TensorLayout.Tile, storage=StorageType.Device):
+        a = np.ascontiguousarray(array)
+        s, r = _shape_arg(a.shape)
+        lay = Layout(storage, layout, in_dtype if dtype is None else dtype)
+        return self._op("ttrt_pb_constant", ctypes.c_void_p(a.ctypes.data), ctypes.c_size_t(a.nbytes), in_dtype, s, r, ctypes.byref(lay))
+
+    def full(self, shape, value, dtype, layout=TensorLayout.Tile):
+        s, r = _shape_arg(shape)
+        return self._op("ttrt_pb_full", s, r, ctypes.c_float(value), dtype, layout)
+
+    def deallocate(self, t, force=False):
+        _call("ttrt_pb_deallocate", self.h, t, int(force))
+
+    def _multi(self, name, head, ins, out_descs):
+        n_out = len(out_descs)
+        shapes = (ctypes.c_uint32 * (8 * n_out))()
+        ranks = (ctypes.c_int * n_out)()
+        lays = (Layout * n_out)()
+        for i, (shape, lay) in enumerate(out_descs):
+            for j, s in enumerate(shape):
+                shapes[8 * i + j] = s
+            ranks[i] = len(shape)
+            lays[i] = lay
+        ia = (ctypes.c_uint32 * max(1, len(ins)))(*ins)
+        outs = (ctypes.c_uint32 * n_out)()
+        _call(name, self.h, *head, ia, len(ins), shapes, ranks, lays, n_out, outs)
+        return list(outs)
+
+    def load_cached(self, program_index, callee, ins, out_descs):
+        return self._multi("ttrt_pb_load_cached", (program_index, callee.encode()), ins, out_descs)
+
+    def func_call(self, program_index, ins, out_descs):
+        return self._multi("ttrt_pb_func_call", (program_index,), ins, out_descs)

@@ -1,0 +1,363 @@
+// C ABI over the C++ runtime (include/ttmlir_amd_runtime.h): exception -> status translation and
+// opaque handles.
+#include <cstring>
+#include <string>
+
+#include "program_builder.h"
+#include "runtime_impl.h"
+#include "ttmlir_amd_runtime.h"
+
+using namespace tt::runtime;
+using ttmlir_amd::ProgramBuilder;
+
+struct ttrt_binary { Binary b; };
+struct ttrt_device { Device d; };
+struct ttrt_tensor { Tensor t; };
+struct ttrt_builder { ProgramBuilder pb; };
+
+#define TTRT_EXPORT extern "C" __attribute__((visibility("default")))
+
+static thread_local std::string g_err;
+
+template <typename F>
+static int guard(F &&f) {
+  try {
+    f();
+    return 0;
+  } catch (const std::exception &e) {
+    g_err = e.what();
+    return 1;
+  } catch (...) {
+    g_err = "unknown C++ exception";
+    return 1;
+  }
+}
+static void need(const void *p, const char *what) {
+  if (!p) throw std::runtime_error(std::string("null argument: ") + what);
+}
+static Layout toLayoutStruct(const ttrt_layout &l) {
+  return Layout{static_cast<StorageType>(l.storage), static_cast<TensorLayout>(l.layout), static_cast<DataType>(l.dtype)};
+}
+static ttrt_layout fromLayoutStruct(const Layout &l) {
+  return ttrt_layout{static_cast<int>(l.storageType), static_cast<int>(l.layout), static_cast<int>(l.dataType)};
+}
+static void copyStr(const std::string &s, char *buf, size_t len) {
+  if (!buf || !len) return;
+  size_t n = std::min(len - 1, s.size());
+  std::memcpy(buf, s.data(), n);
+  buf[n] = 0;
+}
+static std::vector<std::uint32_t> shapeVec(const uint32_t *shape, int rank) {
+  if (rank < 0 || rank > 8) throw std::runtime_error("rank must be 0..8");
+  if (rank > 0) need(shape, "shape");
+  return std::vector<std::uint32_t>(shape, shape + rank);
+}
+static void writeShape(const std::vector<std::uint32_t> &s, uint32_t *shape, int *rank) {
+  if (s.size() > 8) throw std::runtime_error("tensor rank above 8");
+  if (rank) *rank = static_cast<int>(s.size());
+  if (shape) for (size_t i = 0; i < s.size(); ++i) shape[i] = s[i];
+}
+
+TTRT_EXPORT const char *ttrt_last_error(void) { return g_err.c_str(); }
+
+// ---- binary
+TTRT_EXPORT int ttrt_binary_load_file(const char *path, ttrt_binary **out) {
+  return guard([&] { need(path, "path"); need(out, "out"); *out = new ttrt_binary{Binary::loadFromPath(path)}; });
+}
+TTRT_EXPORT int ttrt_binary_load_memory(const void *data, size_t size, ttrt_binary **out) {
+  return guard([&] { need(out, "out"); *out = new ttrt_binary{Binary::loadFromMemory(data, size)}; });
+}
+TTRT_EXPORT int ttrt_binary_store(const ttrt_binary *bin, const char *path) {
+  return guard([&] { need(bin, "binary"); need(path, "path"); bin->b.store(path); });
+}
+TTRT_EXPORT void ttrt_binary_free(ttrt_binary *bin) { delete bin; }
+TTRT_EXPORT int ttrt_binary_num_programs(const ttrt_binary *bin, uint32_t *n) {
+  return guard([&] { need(bin, "binary"); need(n, "n"); *n = bin->b.getNumPrograms(); });
+}
+TTRT_EXPORT int ttrt_binary_program_name(const ttrt_binary *bin, uint32_t program, char *buf, size_t len) {
+  return guard([&] { need(bin, "binary"); copyStr(bin->b.getProgramName(program), buf, len); });
+}
+TTRT_EXPORT int ttrt_binary_program_is_private(const ttrt_binary *bin, uint32_t program, int *is_private) {
+  return guard([&] { need(bin, "binary"); need(is_private, "is_private"); *is_private = bin->b.isProgramPrivate(program); });
+}
+TTRT_EXPORT int ttrt_binary_num_inputs(const ttrt_binary *bin, uint32_t program, uint32_t *n) {
+  return guard([&] { need(bin, "binary"); need(n, "n"); *n = static_cast<uint32_t>(bin->b.getProgramInputs(program).size()); });
+}
+TTRT_EXPORT int ttrt_binary_num_outputs(const ttrt_binary *bin, uint32_t program, uint32_t *n) {
+  return guard([&] { need(bin, "binary"); need(n, "n"); *n = static_cast<uint32_t>(bin->b.getProgramOutputs(program).size()); });
+}
+TTRT_EXPORT int ttrt_binary_tensor_desc(const ttrt_binary *bin, uint32_t program, int is_output, uint32_t index, uint32_t *shape,
+                                        int *rank, ttrt_layout *layout) {
+  return guard([&] {
+    need(bin, "binary");
+    auto v = is_output ? bin->b.getProgramOutputs(program) : bin->b.getProgramInputs(program);
+    if (index >= v.size()) throw std::runtime_error("tensor index out of range");
+    writeShape(v[index].shape, shape, rank);
+    if (layout) *layout = fromLayoutStruct(v[index].layout);
+  });
+}
+TTRT_EXPORT int ttrt_binary_ops_text(const ttrt_binary *bin, uint32_t program, char *buf, size_t len) {
+  return guard([&] { need(bin, "binary"); copyStr(bin->b.getProgramOpsAsText(program), buf, len); });
+}
+TTRT_EXPORT int ttrt_binary_info(const ttrt_binary *bin, char *identifier5, char *version, size_t version_len) {
+  return guard([&] {
+    need(bin, "binary");
+    copyStr(bin->b.getFileIdentifier(), identifier5, 5);
+    copyStr(bin->b.getVersion(), version, version_len);
+  });
+}
+
+// ---- device
+TTRT_EXPORT int ttrt_num_devices(uint32_t *n) {
+  return guard([&] { need(n, "n"); *n = static_cast<uint32_t>(getNumAvailableDevices()); });
+}
+TTRT_EXPORT int ttrt_device_open(ttrt_device **out) {
+  return guard([&] { need(out, "out"); *out = new ttrt_device{openMeshDevice()}; });
+}
+TTRT_EXPORT int ttrt_device_close(ttrt_device *dev) {
+  return guard([&] { need(dev, "device"); closeMeshDevice(dev->d); delete dev; });
+}
+TTRT_EXPORT int ttrt_device_name(ttrt_device *dev, char *buf, size_t len) {
+  return guard([&] { need(dev, "device"); copyStr(getDeviceName(dev->d), buf, len); });
+}
+
+// ---- tensors
+TTRT_EXPORT int ttrt_tensor_create_host(const void *data, const uint32_t *shape, int rank, const int64_t *stride, uint32_t itemsize,
+                                        int dtype, int borrowed, ttrt_tensor **out) {
+  return guard([&] {
+    need(out, "out");
+    auto s = shapeVec(shape, rank);
+    std::vector<std::int64_t> st = stride ? std::vector<std::int64_t>(stride, stride + rank) : utils::calculateStride(s);
+    DataType dt = static_cast<DataType>(dtype);
+    Tensor t = borrowed ? createBorrowedHostTensor(const_cast<void *>(data), s, st, itemsize, dt) : createOwnedHostTensor(data, s, st, itemsize, dt);
+    *out = new ttrt_tensor{t};
+  });
+}
+TTRT_EXPORT void ttrt_tensor_free(ttrt_tensor *t) { delete t; }
+TTRT_EXPORT int ttrt_tensor_desc(const ttrt_tensor *t, uint32_t *shape, int *rank, ttrt_layout *layout, uint64_t *bytes) {
+  return guard([&] {
+    need(t, "tensor");
+    writeShape(t->t.handle->shape, shape, rank);
+    if (layout) *layout = fromLayoutStruct(getTensorLayout(t->t));
+    if (bytes) *bytes = t->t.handle->bytes;
+  });
+}
+TTRT_EXPORT int ttrt_tensor_is_allocated(const ttrt_tensor *t, int *allocated) {
+  return guard([&] { need(t, "tensor"); need(allocated, "allocated"); *allocated = isTensorAllocated(t->t); });
+}
+TTRT_EXPORT int ttrt_tensor_set_retain(ttrt_tensor *t, int retain) {
+  return guard([&] { need(t, "tensor"); setTensorRetain(t->t, retain != 0); });
+}
+TTRT_EXPORT int ttrt_tensor_get_retain(const ttrt_tensor *t, int *retain) {
+  return guard([&] { need(t, "tensor"); need(retain, "retain"); *retain = getTensorRetain(t->t); });
+}
+TTRT_EXPORT int ttrt_tensor_deallocate(ttrt_tensor *t, int force) {
+  return guard([&] { need(t, "tensor"); deallocateTensor(t->t, force != 0); });
+}
+
+TTRT_EXPORT int ttrt_get_layout(const ttrt_binary *bin, uint32_t program, uint32_t input, ttrt_layout *layout) {
+  return guard([&] { need(bin, "binary"); need(layout, "layout"); *layout = fromLayoutStruct(getLayout(bin->b, program, input)); });
+}
+TTRT_EXPORT int ttrt_to_layout(ttrt_tensor *t, ttrt_device *dev, const ttrt_layout *layout, int retain, ttrt_tensor **out) {
+  return guard([&] {
+    need(t, "tensor"); need(dev, "device"); need(layout, "layout"); need(out, "out");
+    std::optional<bool> r = retain < 0 ? std::nullopt : std::optional<bool>(retain != 0);
+    *out = new ttrt_tensor{toLayout(t->t, dev->d, toLayoutStruct(*layout), r)};
+  });
+}
+TTRT_EXPORT int ttrt_to_host(ttrt_tensor *t, int untilize, ttrt_tensor **out) {
+  return guard([&] { need(t, "tensor"); need(out, "out"); *out = new ttrt_tensor{toHost(t->t, untilize != 0, true).at(0)}; });
+}
+TTRT_EXPORT int ttrt_wait(ttrt_tensor *t) {
+  return guard([&] { need(t, "tensor"); wait(t->t); });
+}
+TTRT_EXPORT int ttrt_memcpy_out(void *dst, const ttrt_tensor *src, int target_dtype) {
+  return guard([&] {
+    need(src, "tensor");
+    std::optional<DataType> dt = target_dtype < 0 ? std::nullopt : std::optional<DataType>(static_cast<DataType>(target_dtype));
+    tt::runtime::memcpy(dst, src->t, dt);
+  });
+}
+TTRT_EXPORT int ttrt_memcpy_tensor(ttrt_tensor *dst, const ttrt_tensor *src) {
+  return guard([&] { need(dst, "dst"); need(src, "src"); tt::runtime::memcpy(dst->t, src->t); });
+}
+
+TTRT_EXPORT int ttrt_submit(ttrt_device *dev, const ttrt_binary *bin, uint32_t program, ttrt_tensor *const *inputs, uint32_t num_inputs,
+                            ttrt_tensor **outputs, uint32_t max_outputs, uint32_t *num_outputs) {
+  return guard([&] {
+    need(dev, "device"); need(bin, "binary"); need(num_outputs, "num_outputs");
+    std::vector<Tensor> ins;
+    for (uint32_t i = 0; i < num_inputs; ++i) {
+      need(inputs[i], "input tensor");
+      ins.push_back(inputs[i]->t);
+    }
+    std::vector<Tensor> outs = submit(dev->d, bin->b, program, ins);
+    if (outs.size() > max_outputs) throw std::runtime_error("program returns more outputs than the caller's buffer holds");
+    *num_outputs = static_cast<uint32_t>(outs.size());
+    for (size_t i = 0; i < outs.size(); ++i) outputs[i] = new ttrt_tensor{outs[i]};
+  });
+}
+
+// ---- hooks
+struct HookCtx {
+  CallbackContext cc;
+  OpContext oc;
+};
+TTRT_EXPORT int ttrt_set_post_op_callback(ttrt_op_callback cb, void *user) {
+  return guard([&] {
+    need(reinterpret_cast<const void *>(cb), "callback");
+    debug::Hooks::get(std::nullopt, debug::CallbackFn([cb, user](Binary, CallbackContext cc, OpContext oc) {
+                        HookCtx h{cc, oc};
+                        auto type = static_cast<ttmlir_amd::schema::OpType>(oc.op.scalar<std::uint8_t>(ttmlir_amd::schema::Operation::f_type_type, 0));
+                        std::string dbg = getOpDebugString(oc);
+                        cb(oc.index, ttmlir_amd::schema::opTypeName(type), dbg.c_str(), &h, user);
+                      }));
+  });
+}
+TTRT_EXPORT int ttrt_clear_callbacks(void) {
+  return guard([&] { debug::Hooks::get().unregisterHooks(); });
+}
+TTRT_EXPORT int ttrt_hook_output(void *hook_ctx, ttrt_tensor **out) {
+  return guard([&] {
+    need(hook_ctx, "hook context"); need(out, "out");
+    auto *h = static_cast<HookCtx *>(hook_ctx);
+    auto m = getOpOutputTensor(h->oc, h->cc);
+    *out = m.empty() ? nullptr : new ttrt_tensor{m.begin()->second};
+  });
+}
+TTRT_EXPORT int ttrt_stat(const char *name, int64_t *value) {
+  return guard([&] { need(name, "name"); need(value, "value"); *value = debug::Stats::get().getStat(name); });
+}
+TTRT_EXPORT int ttrt_stats_clear(void) {
+  return guard([&] { debug::Stats::get().clear(); });
+}
+TTRT_EXPORT int ttrt_buffer_cast(const void *src, void *dst, int from_dtype, int to_dtype, int64_t n) {
+  return guard([&] { utils::handleBufferCast(src, dst, static_cast<DataType>(from_dtype), static_cast<DataType>(to_dtype), n); });
+}
+
+// ---- program writer
+TTRT_EXPORT int ttrt_pb_create(ttrt_builder **out) {
+  return guard([&] { need(out, "out"); *out = new ttrt_builder{}; });
+}
+TTRT_EXPORT void ttrt_pb_destroy(ttrt_builder *pb) { delete pb; }
+TTRT_EXPORT int ttrt_pb_begin_program(ttrt_builder *pb, const char *name, int is_private) {
+  return guard([&] { need(pb, "builder"); need(name, "name"); pb->pb.beginProgram(name, is_private != 0); });
+}
+TTRT_EXPORT int ttrt_pb_end_program(ttrt_builder *pb, uint32_t *program_index) {
+  return guard([&] { need(pb, "builder"); uint32_t i = pb->pb.endProgram(); if (program_index) *program_index = i; });
+}
+static ProgramBuilder::Desc descOf(const uint32_t *shape, int rank, const ttrt_layout *l) {
+  need(l, "layout");
+  return ProgramBuilder::Desc{shapeVec(shape, rank), static_cast<DataType>(l->dtype), static_cast<TensorLayout>(l->layout),
+                              static_cast<StorageType>(l->storage)};
+}
+TTRT_EXPORT int ttrt_pb_input(ttrt_builder *pb, const uint32_t *shape, int rank, const ttrt_layout *layout, uint32_t *id) {
+  return guard([&] {
+    need(pb, "builder"); need(id, "id");
+    auto d = descOf(shape, rank, layout);
+    *id = pb->pb.input(d.shape, d.dtype, d.layout, d.storage);
+  });
+}
+TTRT_EXPORT int ttrt_pb_output(ttrt_builder *pb, uint32_t id) {
+  return guard([&] { need(pb, "builder"); pb->pb.output(id); });
+}
+TTRT_EXPORT int ttrt_pb_finish(ttrt_builder *pb, uint8_t **data, size_t *size) {
+  return guard([&] {
+    need(pb, "builder"); need(data, "data"); need(size, "size");
+    auto v = pb->pb.finish();
+    *data = static_cast<uint8_t *>(std::malloc(v.size()));
+    if (!*data) throw std::runtime_error("out of memory");
+    std::memcpy(*data, v.data(), v.size());
+    *size = v.size();
+  });
+}
+TTRT_EXPORT void ttrt_free_bytes(uint8_t *data) { std::free(data); }
+TTRT_EXPORT int ttrt_pb_tensor_desc(ttrt_builder *pb, uint32_t id, uint32_t *shape, int *rank, ttrt_layout *layout) {
+  return guard([&] {
+    need(pb, "builder");
+    const auto &d = pb->pb.desc(id);
+    writeShape(d.shape, shape, rank);
+    if (layout) *layout = ttrt_layout{static_cast<int>(d.storage), static_cast<int>(d.layout), static_cast<int>(d.dtype)};
+  });
+}
+#define PB_OP(call) return guard([&] { need(pb, "builder"); need(out, "out"); *out = pb->pb.call; })
+TTRT_EXPORT int ttrt_pb_to_layout(ttrt_builder *pb, uint32_t in, int layout, int dtype, int storage, uint32_t *out) {
+  PB_OP(toLayout(in, static_cast<TensorLayout>(layout), dtype, static_cast<StorageType>(storage)));
+}
+TTRT_EXPORT int ttrt_pb_typecast(ttrt_builder *pb, uint32_t in, int dtype, uint32_t *out) { PB_OP(typecast(in, static_cast<DataType>(dtype))); }
+TTRT_EXPORT int ttrt_pb_to_device(ttrt_builder *pb, uint32_t in, uint32_t *out) { PB_OP(toDevice(in)); }
+TTRT_EXPORT int ttrt_pb_from_device(ttrt_builder *pb, uint32_t in, uint32_t *out) { PB_OP(fromDevice(in)); }
+TTRT_EXPORT int ttrt_pb_matmul(ttrt_builder *pb, uint32_t a, uint32_t b, int ta, int tb, const char *activation, int out_dtype, uint32_t *out) {
+  PB_OP(matmul(a, b, ta != 0, tb != 0, activation ? activation : "", static_cast<DataType>(out_dtype)));
+}
+TTRT_EXPORT int ttrt_pb_linear(ttrt_builder *pb, uint32_t a, uint32_t b, uint32_t bias, int ta, int tb, const char *activation, int out_dtype,
+                               uint32_t *out) {
+  PB_OP(linear(a, b, bias, ta != 0, tb != 0, activation ? activation : "", static_cast<DataType>(out_dtype)));
+}
+TTRT_EXPORT int ttrt_pb_unary(ttrt_builder *pb, uint32_t type, uint32_t in, int has_param, float param, uint32_t *out) {
+  PB_OP(unary(type, in, has_param != 0, param));
+}
+TTRT_EXPORT int ttrt_pb_binary(ttrt_builder *pb, uint32_t type, uint32_t lhs, uint32_t rhs, uint32_t *out) { PB_OP(binary(type, lhs, rhs)); }
+TTRT_EXPORT int ttrt_pb_rms_norm(ttrt_builder *pb, uint32_t in, uint32_t weight, uint32_t bias, float eps, uint32_t *out) {
+  PB_OP(rmsNorm(in, weight, bias, eps));
+}
+TTRT_EXPORT int ttrt_pb_softmax(ttrt_builder *pb, uint32_t in, int dim, uint32_t *out) { PB_OP(softmax(in, dim)); }
+TTRT_EXPORT int ttrt_pb_reduction(ttrt_builder *pb, uint32_t type, uint32_t in, const int32_t *dims, int ndims, int keep_dim, uint32_t *out) {
+  PB_OP(reduction(type, in, std::vector<int>(dims, dims + ndims), keep_dim != 0));
+}
+TTRT_EXPORT int ttrt_pb_sdpa(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t mask, int is_causal, int has_scale, float scale,
+                             uint32_t *out) {
+  PB_OP(sdpa(q, k, v, mask, is_causal != 0, has_scale != 0, scale));
+}
+TTRT_EXPORT int ttrt_pb_reshape(ttrt_builder *pb, uint32_t in, const uint32_t *shape, int rank, uint32_t *out) { PB_OP(reshape(in, shapeVec(shape, rank))); }
+TTRT_EXPORT int ttrt_pb_permute(ttrt_builder *pb, uint32_t in, const int64_t *perm, int rank, uint32_t *out) {
+  PB_OP(permute(in, std::vector<std::int64_t>(perm, perm + rank)));
+}
+TTRT_EXPORT int ttrt_pb_transpose(ttrt_builder *pb, uint32_t in, int dim0, int dim1, uint32_t *out) { PB_OP(transpose(in, dim0, dim1)); }
+TTRT_EXPORT int ttrt_pb_concat(ttrt_builder *pb, const uint32_t *ins, int n, int dim, uint32_t *out) {
+  PB_OP(concat(std::vector<ProgramBuilder::Id>(ins, ins + n), dim));
+}
+TTRT_EXPORT int ttrt_pb_slice(ttrt_builder *pb, uint32_t in, const int64_t *begins, const int64_t *ends, const int64_t *steps, int rank,
+                              uint32_t *out) {
+  PB_OP(slice(in, std::vector<std::int64_t>(begins, begins + rank), std::vector<std::int64_t>(ends, ends + rank),
+              std::vector<std::int64_t>(steps, steps + rank)));
+}
+TTRT_EXPORT int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_t repeats, int dim, uint32_t *out) {
+  PB_OP(repeatInterleave(in, repeats, dim));
+}
+TTRT_EXPORT int ttrt_pb_constant(ttrt_builder *pb, const void *data, size_t bytes, int in_dtype, const uint32_t *shape, int rank,
+                                 const ttrt_layout *layout, uint32_t *out) {
+  return guard([&] {
+    need(pb, "builder"); need(out, "out"); need(data, "data");
+    auto d = descOf(shape, rank, layout);
+    *out = pb->pb.constant(data, bytes, static_cast<DataType>(in_dtype), d.shape, d.dtype, d.layout, d.storage);
+  });
+}
+TTRT_EXPORT int ttrt_pb_full(ttrt_builder *pb, const uint32_t *shape, int rank, float value, int dtype, int layout, uint32_t *out) {
+  PB_OP(full(shapeVec(shape, rank), value, static_cast<DataType>(dtype), static_cast<TensorLayout>(layout)));
+}
+TTRT_EXPORT int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force) {
+  return guard([&] { need(pb, "builder"); pb->pb.deallocate(in, force != 0); });
+}
+static std::vector<ProgramBuilder::Desc> outDescs(const uint32_t *out_shapes, const int *out_ranks, const ttrt_layout *out_layouts, int n_out) {
+  std::vector<ProgramBuilder::Desc> v;
+  for (int i = 0; i < n_out; ++i) v.push_back(descOf(out_shapes + 8 * i, out_ranks[i], out_layouts + i));
+  return v;
+}
+TTRT_EXPORT int ttrt_pb_load_cached(ttrt_builder *pb, uint32_t program_index, const char *callee, const uint32_t *ins, int n_in,
+                                    const uint32_t *out_shapes, const int *out_ranks, const ttrt_layout *out_layouts, int n_out, uint32_t *outs) {
+  return guard([&] {
+    need(pb, "builder"); need(outs, "outs");
+    auto ids = pb->pb.loadCached(program_index, callee ? callee : "", std::vector<ProgramBuilder::Id>(ins, ins + n_in),
+                                 outDescs(out_shapes, out_ranks, out_layouts, n_out));
+    for (size_t i = 0; i < ids.size(); ++i) outs[i] = ids[i];
+  });
+}
+TTRT_EXPORT int ttrt_pb_func_call(ttrt_builder *pb, uint32_t program_index, const uint32_t *ins, int n_in, const uint32_t *out_shapes,
+                                  const int *out_ranks, const ttrt_layout *out_layouts, int n_out, uint32_t *outs) {
+  return guard([&] {
+    need(pb, "builder"); need(outs, "outs");
+    auto ids = pb->pb.funcCall(program_index, std::vector<ProgramBuilder::Id>(ins, ins + n_in), outDescs(out_shapes, out_ranks, out_layouts, n_out));
+    for (size_t i = 0; i < ids.size(); ++i) outs[i] = ids[i];
+  });
+}

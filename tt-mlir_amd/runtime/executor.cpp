@@ -1,0 +1,761 @@
+// Program executor: walks the operations of one TTNN program and runs each through the gfx950
+// kernel library.  Structure follows runtime/lib/ttnn/program_executor.cpp:146-266 (tensor pool keyed
+// by global_id, pre/post hooks around every op, outputs gathered at the end) with one runner per
+// flatbuffer op table (runtime/lib/ttnn/operations/**).  Ops outside the supported subset fail with
+// the op name, like the reference's LOG_FATAL("Unsupported operation type").
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <sstream>
+
+#include "runtime_impl.h"
+
+namespace tt::runtime {
+
+using namespace ::ttmlir_amd;
+using schema::OpType;
+
+namespace {
+
+int ttmDtype(DataType dt) { return static_cast<int>(dt); }
+int ttmLayout(TensorLayout l) { return static_cast<int>(l); }
+
+struct ProgramContext {
+  std::shared_ptr<DeviceState> dev;
+  Binary binary;
+  std::uint32_t programIndex = 0;
+  std::unordered_map<std::uint32_t, Tensor> pool;  // global_id -> live tensor
+
+  Tensor &get(const fb::Table &ref, const char *what) {
+    TTRT_ASSERT(static_cast<bool>(ref), std::string("missing tensor reference: ") + what);
+    std::uint32_t id = ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
+    auto it = pool.find(id);
+    TTRT_ASSERT(it != pool.end(), std::string("tensor ") + std::to_string(id) + " (" + what + ") is not in the tensor pool");
+    TTRT_ASSERT(isTensorAllocated(it->second), std::string("tensor ") + std::to_string(id) + " (" + what + ") was deallocated");
+    return it->second;
+  }
+  void put(const fb::Table &ref, Tensor t) {
+    std::uint32_t id = ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
+    pool[id] = std::move(t);
+  }
+  void *stream() const { return dev->stream; }
+};
+
+// ---- helpers
+Tensor onDevice(ProgramContext &ctx, const Tensor &t) { return t.handle->storage == StorageType::Device ? t : toDevice(t, ctx.dev); }
+
+// a device tensor in (layout, dtype); never frees its argument
+Tensor as(ProgramContext &ctx, const Tensor &t, TensorLayout layout, DataType dtype) { return convertOnDevice(onDevice(ctx, t), layout, dtype); }
+
+Tensor convertTo(ProgramContext &ctx, const Tensor &t, const Layout &target) {
+  Tensor cur = t;
+  const bool change = cur.handle->layout != target.layout || cur.handle->dtype != target.dataType;
+  if (change || target.storageType == StorageType::Device) cur = as(ctx, cur, target.layout, target.dataType);
+  if (target.storageType == StorageType::Host && cur.handle->storage == StorageType::Device) cur = fromDevice(cur);
+  return cur;
+}
+
+std::vector<std::int64_t> rowMajorStrides(const std::vector<std::uint32_t> &shape) {
+  std::vector<std::int64_t> s(shape.size(), 1);
+  for (int i = static_cast<int>(shape.size()) - 2; i >= 0; --i) s[i] = s[i + 1] * shape[i + 1];
+  return s;
+}
+
+bool hasPadding(const std::vector<std::uint32_t> &shape) {
+  Dims3 d = dims3(shape);
+  return d.rows % 32 != 0 || d.cols % 32 != 0;
+}
+
+// zero a freshly made tile tensor whose padding the producing kernel does not write
+void zeroIfPadded(ProgramContext &ctx, const Tensor &t) {
+  if (t.handle->layout == TensorLayout::Tile && hasPadding(t.handle->shape))
+    TTM_CALL(ttm_fill_u32(t.handle->data.get(), 0, (t.handle->bytes + 3) / 4, ctx.stream()));
+}
+
+// generic strided copy between two device tensors (any layouts) through ttm_copy_view
+void copyView(ProgramContext &ctx, const Tensor &src, const Tensor &dst, const std::vector<std::int64_t> &extent,
+              const std::vector<std::int64_t> &sstride, std::int64_t sbase, const std::vector<std::int64_t> &dstride,
+              std::int64_t dbase) {
+  TTRT_ASSERT(src.handle->dtype == dst.handle->dtype, "copyView: dtype mismatch");
+  TTRT_ASSERT(!utils::isBlockFormatDataType(src.handle->dtype), "data movement on block-float tensors is not supported");
+  // collapse to at most 8 view dims by merging leading ones when needed
+  std::vector<std::int64_t> e = extent, ss = sstride, ds = dstride;
+  TTRT_ASSERT(e.size() <= 8, "copyView: rank above 8");
+  Dims3 sd = dims3(src.handle->shape), dd = dims3(dst.handle->shape);
+  TTM_CALL(ttm_copy_view(src.handle->data.get(), sd.rows, sd.cols, ttmLayout(src.handle->layout), dst.handle->data.get(), dd.rows,
+                         dd.cols, ttmLayout(dst.handle->layout), static_cast<int>(utils::dataTypeElementSize(src.handle->dtype)),
+                         static_cast<int>(e.size()), e.data(), ss.data(), sbase, ds.data(), dbase, ctx.stream()));
+}
+
+std::vector<std::int64_t> toI64(const std::vector<std::uint32_t> &v) { return std::vector<std::int64_t>(v.begin(), v.end()); }
+
+Tensor makeOut(ProgramContext &ctx, const fb::Table &outRef, DataType dtype, TensorLayout layout) {
+  return makeDeviceTensor(ctx.dev, shapeFromTensorRef(outRef), dtype, layout);
+}
+
+// final cast of an op result to what the program's TensorRef declares (dtype and layout)
+Tensor finish(ProgramContext &ctx, const Tensor &t, const fb::Table &outRef) {
+  Layout want = layoutFromTensorRef(outRef);
+  if (want.storageType == StorageType::Host) return convertTo(ctx, t, want);
+  return as(ctx, t, want.layout, want.dataType);
+}
+
+int activationCode(std::string_view s) {
+  if (s.empty()) return TTM_ACT_NONE;
+  if (s == "gelu") return TTM_ACT_GELU;
+  if (s == "silu") return TTM_ACT_SILU;
+  if (s == "sigmoid") return TTM_ACT_SIGMOID;
+  if (s == "relu") return TTM_ACT_RELU;
+  fatal("unsupported fused activation '" + std::string(s) + "'");
+}
+
+// ---- layout ops (runtime/lib/ttnn/operations/layout/*.cpp)
+void runToLayout(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = ctx.get(op.table(schema::ToLayoutOp::f_in), "to_layout in");
+  auto outRef = op.table(schema::ToLayoutOp::f_out);
+  Layout want = layoutFromTensorRef(outRef);
+  want.layout = static_cast<TensorLayout>(op.scalar<std::uint16_t>(schema::ToLayoutOp::f_layout, 0));
+  if (op.has(schema::ToLayoutOp::f_dtype)) want.dataType = static_cast<DataType>(op.scalar<std::uint16_t>(schema::ToLayoutOp::f_dtype, 0));
+  ctx.put(outRef, convertTo(ctx, in, want));
+}
+void runTypecast(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = ctx.get(op.table(schema::TypecastOp::f_in), "typecast in");
+  DataType dt = static_cast<DataType>(op.scalar<std::uint16_t>(schema::TypecastOp::f_dtype, 0));
+  TensorLayout l = utils::isBlockFormatDataType(dt) ? TensorLayout::Tile : in.handle->layout;
+  Tensor out = as(ctx, in, l, dt);
+  auto outRef = op.table(schema::TypecastOp::f_out);
+  if (layoutFromTensorRef(outRef).storageType == StorageType::Host) out = fromDevice(out);
+  ctx.put(outRef, out);
+}
+void runToDevice(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = ctx.get(op.table(schema::ToDeviceOp::f_in), "to_device in");
+  ctx.put(op.table(schema::ToDeviceOp::f_out), onDevice(ctx, in));
+}
+void runFromDevice(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = ctx.get(op.table(schema::FromDeviceOp::f_in), "from_device in");
+  ctx.put(op.table(schema::FromDeviceOp::f_out), in.handle->storage == StorageType::Device ? fromDevice(in) : in);
+}
+void runToMemoryConfig(const fb::Table &op, ProgramContext &ctx) {
+  // one memory space on this device: the tensor is passed through
+  ctx.put(op.table(schema::ToMemoryConfigOp::f_out), ctx.get(op.table(schema::ToMemoryConfigOp::f_in0), "to_memory_config in"));
+}
+
+// ---- matmul / linear (runtime/lib/ttnn/operations/matmul/matmul.cpp:47-125)
+Tensor transposeLast2(ProgramContext &ctx, const Tensor &t) {
+  std::vector<std::uint32_t> shape = t.handle->shape;
+  TTRT_ASSERT(shape.size() >= 2, "transpose needs rank >= 2");
+  std::vector<std::uint32_t> oshape = shape;
+  std::swap(oshape[oshape.size() - 1], oshape[oshape.size() - 2]);
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, t.handle->dtype, t.handle->layout);
+  zeroIfPadded(ctx, out);
+  auto ss = rowMajorStrides(shape);
+  std::swap(ss[ss.size() - 1], ss[ss.size() - 2]);
+  copyView(ctx, t, out, toI64(oshape), ss, 0, rowMajorStrides(oshape), 0);
+  return out;
+}
+
+void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &bRef, const fb::Table &biasRef, const fb::Table &outRef,
+                   bool transposeA, bool transposeB, std::string_view activation) {
+  Tensor a = as(ctx, ctx.get(aRef, "matmul a"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor b = onDevice(ctx, ctx.get(bRef, "matmul b"));
+  if (!utils::isBlockFormatDataType(b.handle->dtype)) b = as(ctx, b, TensorLayout::Tile, DataType::BFloat16);
+  TTRT_ASSERT(b.handle->layout == TensorLayout::Tile, "matmul: weights must be in tile layout");
+  if (transposeA) a = transposeLast2(ctx, a);
+  if (transposeB && utils::isBlockFormatDataType(b.handle->dtype)) {
+    // block-float rows share exponents along n: transpose through bf16
+    b = transposeLast2(ctx, as(ctx, b, TensorLayout::Tile, DataType::BFloat16));
+    transposeB = false;
+  }
+  const auto &as_ = a.handle->shape, &bs = b.handle->shape;
+  TTRT_ASSERT(!as_.empty() && !bs.empty(), "matmul: scalar operands are not supported");
+  Dims3 ad = dims3(as_), bd = dims3(bs);
+  std::int64_t M = ad.rows, K = ad.cols;
+  std::int64_t Kb = transposeB ? bd.cols : bd.rows, N = transposeB ? bd.rows : bd.cols;
+  if (as_.size() == 1) { M = 1; K = as_[0]; }
+  TTRT_ASSERT(K == Kb, "matmul: inner dimensions differ (" + std::to_string(K) + " vs " + std::to_string(Kb) + ")");
+  std::int64_t batch = ad.batch, wbatch = bd.batch;
+  TTRT_ASSERT(wbatch == 1 || wbatch == batch, "matmul: RHS batch must be 1 or match the LHS batch");
+  // shared weights: fold the LHS batch into M when that does not cross tile padding
+  if (wbatch == 1 && batch > 1 && M % 32 == 0) { M *= batch; batch = 1; }
+  const void *biasPtr = nullptr;
+  int biasLayout = TTM_TILE;
+  Tensor bias;
+  if (biasRef) {
+    bias = as(ctx, ctx.get(biasRef, "linear bias"), TensorLayout::Tile, DataType::BFloat16);
+    TTRT_ASSERT(volume(bias.handle->shape) == N, "linear: bias must have N elements");
+    biasPtr = bias.handle->data.get();
+  }
+  Tensor out = makeOut(ctx, outRef, DataType::BFloat16, TensorLayout::Tile);
+  TTM_CALL(ttm_linear(a.handle->data.get(), TTM_BF16, b.handle->data.get(), ttmDtype(b.handle->dtype), transposeB ? 1 : 0, biasPtr,
+                      TTM_BF16, biasLayout, out.handle->data.get(), TTM_BF16, batch, wbatch == 1 ? 1 : batch, M, N, K,
+                      activationCode(activation), ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+void runMatmul(const fb::Table &op, ProgramContext &ctx) {
+  runMatmulLike(ctx, op.table(schema::MatmulOp::f_a), op.table(schema::MatmulOp::f_b), fb::Table(), op.table(schema::MatmulOp::f_out),
+                op.scalar<std::uint8_t>(schema::MatmulOp::f_transpose_a, 0) != 0,
+                op.scalar<std::uint8_t>(schema::MatmulOp::f_transpose_b, 0) != 0, op.string(schema::MatmulOp::f_activation));
+}
+void runLinear(const fb::Table &op, ProgramContext &ctx) {
+  runMatmulLike(ctx, op.table(schema::LinearOp::f_a), op.table(schema::LinearOp::f_b), op.table(schema::LinearOp::f_bias),
+                op.table(schema::LinearOp::f_out), op.scalar<std::uint8_t>(schema::LinearOp::f_transpose_a, 0) != 0,
+                op.scalar<std::uint8_t>(schema::LinearOp::f_transpose_b, 0) != 0, op.string(schema::LinearOp::f_activation));
+}
+
+// ---- eltwise (runtime/lib/ttnn/operations/eltwise/{unary,binary}/*.cpp)
+DataType computeDtype(DataType dt) { return dt == DataType::Float32 ? DataType::Float32 : DataType::BFloat16; }
+
+void runEltwiseUnary(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in0 = ctx.get(op.table(schema::EltwiseUnaryOp::f_in), "unary in");
+  auto outRef = op.table(schema::EltwiseUnaryOp::f_out);
+  Layout want = layoutFromTensorRef(outRef);
+  DataType dt = computeDtype(want.dataType);
+  Tensor in = as(ctx, in0, in0.handle->layout, dt);
+  std::uint32_t type = op.scalar<std::uint32_t>(schema::EltwiseUnaryOp::f_type, 0);
+  float param = 0.0f;
+  if (auto prm = op.table(schema::EltwiseUnaryOp::f_params)) param = prm.scalar<float>(schema::EltwiseOpWithFloatParams::f_parameter, 0.0f);
+  Tensor out = makeDeviceTensor(ctx.dev, in.handle->shape, dt, in.handle->layout);
+  Dims3 d = dims3(in.handle->shape);
+  TTM_CALL(ttm_eltwise_unary(static_cast<int>(type), in.handle->data.get(), out.handle->data.get(), ttmDtype(dt),
+                             ttmLayout(in.handle->layout), d.batch, d.rows, d.cols, param, ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+void runEltwiseBinary(const fb::Table &op, ProgramContext &ctx) {
+  Tensor l0 = ctx.get(op.table(schema::EltwiseBinaryOp::f_lhs), "binary lhs"), r0 = ctx.get(op.table(schema::EltwiseBinaryOp::f_rhs), "binary rhs");
+  auto outRef = op.table(schema::EltwiseBinaryOp::f_out);
+  Layout want = layoutFromTensorRef(outRef);
+  DataType dt = computeDtype(want.dataType);
+  TensorLayout lay = want.storageType == StorageType::Device ? want.layout : onDevice(ctx, l0).handle->layout;
+  Tensor l = as(ctx, l0, lay, dt), r = as(ctx, r0, lay, dt);
+  std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
+  size_t rank = std::max<size_t>(1, oshape.size());
+  auto pad = [&](const std::vector<std::uint32_t> &s) {
+    std::vector<std::int64_t> o(rank, 1);
+    for (size_t i = 0; i < s.size(); ++i) o[rank - s.size() + i] = s[i];
+    return o;
+  };
+  TTRT_ASSERT(l.handle->shape.size() <= rank && r.handle->shape.size() <= rank, "binary: operand rank exceeds the output rank");
+  auto ls = pad(l.handle->shape), rs = pad(r.handle->shape), os = pad(oshape);
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, dt, lay);
+  std::uint32_t type = op.scalar<std::uint32_t>(schema::EltwiseBinaryOp::f_type, 0);
+  TTM_CALL(ttm_eltwise_binary(static_cast<int>(type), l.handle->data.get(), ls.data(), r.handle->data.get(), rs.data(),
+                              out.handle->data.get(), os.data(), static_cast<int>(rank), ttmDtype(dt), ttmLayout(lay), ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// ---- normalization / reduction (runtime/lib/ttnn/operations/normalization/*.cpp, reduction/reduction.cpp)
+void runRmsNorm(const fb::Table &op, ProgramContext &ctx) {
+  auto outRef = op.table(schema::RMSNormOp::f_out);
+  DataType dt = computeDtype(layoutFromTensorRef(outRef).dataType);
+  Tensor x = as(ctx, ctx.get(op.table(schema::RMSNormOp::f_input), "rms_norm input"), TensorLayout::Tile, dt);
+  Tensor w, b;
+  Dims3 d = dims3(x.handle->shape);
+  if (auto wr = op.table(schema::RMSNormOp::f_weight)) {
+    w = as(ctx, ctx.get(wr, "rms_norm weight"), TensorLayout::Tile, dt);
+    TTRT_ASSERT(volume(w.handle->shape) == d.cols, "rms_norm: weight must have as many elements as the last dim");
+  }
+  if (auto br = op.table(schema::RMSNormOp::f_bias)) {
+    b = as(ctx, ctx.get(br, "rms_norm bias"), TensorLayout::Tile, dt);
+    TTRT_ASSERT(volume(b.handle->shape) == d.cols, "rms_norm: bias must have as many elements as the last dim");
+  }
+  float eps = op.scalar<float>(schema::RMSNormOp::f_epsilon, 0.0f);
+  Tensor out = makeDeviceTensor(ctx.dev, x.handle->shape, dt, TensorLayout::Tile);
+  TTM_CALL(ttm_rms_norm(x.handle->data.get(), w ? w.handle->data.get() : nullptr, TTM_TILE, b ? b.handle->data.get() : nullptr, TTM_TILE,
+                        out.handle->data.get(), ttmDtype(dt), d.batch, d.rows, d.cols, eps, ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// move dimension `dim` to the end (or back) with one strided copy
+Tensor moveDimLast(ProgramContext &ctx, const Tensor &t, int dim, bool inverse, const std::vector<std::uint32_t> &origShape) {
+  const int rank = static_cast<int>(origShape.size());
+  std::vector<int> perm;  // perm[i] = source dim of output dim i for the forward move
+  for (int i = 0; i < rank; ++i) if (i != dim) perm.push_back(i);
+  perm.push_back(dim);
+  std::vector<std::uint32_t> moved(rank);
+  for (int i = 0; i < rank; ++i) moved[i] = origShape[perm[i]];
+  const std::vector<std::uint32_t> &srcShape = inverse ? moved : origShape, &dstShape = inverse ? origShape : moved;
+  Tensor out = makeDeviceTensor(ctx.dev, dstShape, t.handle->dtype, t.handle->layout);
+  zeroIfPadded(ctx, out);
+  auto ss = rowMajorStrides(srcShape), ds = rowMajorStrides(dstShape);
+  std::vector<std::int64_t> extent(rank), sst(rank), dst(rank);
+  for (int i = 0; i < rank; ++i) {  // iterate in the order of `moved`
+    extent[i] = moved[i];
+    sst[i] = inverse ? ss[i] : ss[perm[i]];
+    dst[i] = inverse ? ds[perm[i]] : ds[i];
+  }
+  copyView(ctx, t, out, extent, sst, 0, dst, 0);
+  return out;
+}
+
+void runSoftmax(const fb::Table &op, ProgramContext &ctx) {
+  auto outRef = op.table(schema::SoftmaxOp::f_out);
+  DataType dt = computeDtype(layoutFromTensorRef(outRef).dataType);
+  Tensor x = as(ctx, ctx.get(op.table(schema::SoftmaxOp::f_in), "softmax in"), TensorLayout::Tile, dt);
+  const int rank = static_cast<int>(x.handle->shape.size());
+  int dim = op.scalar<std::int32_t>(schema::SoftmaxOp::f_dimension, 0);
+  if (dim < 0) dim += rank;
+  TTRT_ASSERT(dim >= 0 && dim < rank, "softmax: dimension out of range");
+  const std::vector<std::uint32_t> orig = x.handle->shape;
+  if (dim != rank - 1) x = moveDimLast(ctx, x, dim, false, orig);
+  Dims3 d = dims3(x.handle->shape);
+  Tensor out = makeDeviceTensor(ctx.dev, x.handle->shape, dt, TensorLayout::Tile);
+  TTM_CALL(ttm_softmax_lastdim(x.handle->data.get(), out.handle->data.get(), ttmDtype(dt), d.batch, d.rows, d.cols, ctx.stream()));
+  if (dim != rank - 1) out = moveDimLast(ctx, out, dim, true, orig);
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+void runReduction(const fb::Table &op, ProgramContext &ctx) {
+  auto outRef = op.table(schema::ReductionOp::f_out);
+  DataType dt = computeDtype(layoutFromTensorRef(outRef).dataType);
+  Tensor x = as(ctx, ctx.get(op.table(schema::ReductionOp::f_in), "reduction in"), TensorLayout::Tile, dt);
+  const int rank = static_cast<int>(x.handle->shape.size());
+  auto dims = op.scalars<std::int32_t>(schema::ReductionOp::f_dim_arg);
+  std::uint32_t type = op.scalar<std::uint32_t>(schema::ReductionOp::f_type, 0);
+  std::vector<int> rd;
+  for (std::uint32_t i = 0; i < dims.size(); ++i) rd.push_back(dims[i] < 0 ? dims[i] + rank : dims[i]);
+  if (rd.empty()) for (int i = 0; i < rank; ++i) rd.push_back(i);
+  std::sort(rd.begin(), rd.end(), std::greater<int>());
+  // reduce one dim at a time, innermost first; the reduced dim is kept as size 1.  A mean over several
+  // dims is a mean of means (equal group sizes), so every op applies dim by dim.
+  for (int dim : rd) {
+    TTRT_ASSERT(dim >= 0 && dim < rank, "reduction: dimension out of range");
+    const std::vector<std::uint32_t> orig = x.handle->shape;
+    Tensor cur = dim != rank - 1 ? moveDimLast(ctx, x, dim, false, orig) : x;
+    Dims3 d = dims3(cur.handle->shape);
+    std::vector<std::uint32_t> rshape = cur.handle->shape;
+    rshape.back() = 1;
+    Tensor red = makeDeviceTensor(ctx.dev, rshape, dt, TensorLayout::Tile);
+    TTM_CALL(ttm_reduce_lastdim(static_cast<int>(type), cur.handle->data.get(), red.handle->data.get(), ttmDtype(dt), d.batch, d.rows,
+                                d.cols, ctx.stream()));
+    if (dim != rank - 1) {
+      std::vector<std::uint32_t> back = orig;
+      back[dim] = 1;
+      red = moveDimLast(ctx, red, dim, true, back);
+    }
+    x = red;
+  }
+  // keep_dim = false only changes the logical shape; relayout through a strided copy
+  std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
+  if (oshape != x.handle->shape) {
+    TTRT_ASSERT(volume(oshape) == volume(x.handle->shape), "reduction: output shape does not match");
+    Tensor out = makeDeviceTensor(ctx.dev, oshape, dt, TensorLayout::Tile);
+    zeroIfPadded(ctx, out);
+    std::vector<std::int64_t> e{volume(oshape)}, one{1};
+    copyView(ctx, x, out, e, one, 0, one, 0);
+    x = out;
+  }
+  ctx.put(outRef, finish(ctx, x, outRef));
+}
+
+// ---- attention (runtime/lib/ttnn/operations/transformer/scaled_dot_product_attention.cpp:14-55)
+void runSdpa(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::ScaledDotProductAttentionOp;
+  Tensor q = as(ctx, ctx.get(op.table(S::f_query), "sdpa query"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor k = as(ctx, ctx.get(op.table(S::f_key), "sdpa key"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor v = as(ctx, ctx.get(op.table(S::f_value), "sdpa value"), TensorLayout::Tile, DataType::BFloat16);
+  TTRT_ASSERT(q.handle->shape.size() == 4 && k.handle->shape.size() == 4 && v.handle->shape.size() == 4, "sdpa: q, k, v must be rank 4");
+  TTRT_ASSERT(!op.has(S::f_sliding_window_size) && !op.table(S::f_attention_sink), "sdpa: sliding window / attention sink are not supported");
+  const auto &qs = q.handle->shape, &ks = k.handle->shape;
+  TTRT_ASSERT(k.handle->shape == v.handle->shape && qs[0] == ks[0] && qs[3] == ks[3], "sdpa: q/k/v shapes do not agree");
+  Tensor mask;
+  int maskHeads = 1;
+  if (auto mr = op.table(S::f_attention_mask)) {
+    mask = as(ctx, ctx.get(mr, "sdpa mask"), TensorLayout::Tile, DataType::BFloat16);
+    const auto &ms = mask.handle->shape;
+    TTRT_ASSERT(ms.size() == 4 && ms[0] == qs[0] && ms[2] == qs[2] && ms[3] == ks[2] && (ms[1] == 1 || ms[1] == qs[1]),
+                "sdpa: mask must be [B, 1|Hq, Sq, Sk]");
+    maskHeads = static_cast<int>(ms[1]);
+  }
+  bool causal = op.scalar<std::uint8_t>(S::f_is_causal, 0) != 0;
+  TTRT_ASSERT(!(causal && mask), "sdpa: is_causal and an explicit mask are mutually exclusive");
+  float scale = op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f;
+  auto outRef = op.table(S::f_out);
+  Tensor out = makeDeviceTensor(ctx.dev, qs, DataType::BFloat16, TensorLayout::Tile);
+  TTM_CALL(ttm_sdpa(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(), mask ? mask.handle->data.get() : nullptr, maskHeads,
+                    out.handle->data.get(), TTM_BF16, qs[0], qs[1], ks[1], qs[2], ks[2], qs[3], causal ? 1 : 0, scale, ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// ---- data movement (runtime/lib/ttnn/operations/data_movement/*.cpp)
+bool sameTiling(const std::vector<std::uint32_t> &a, const std::vector<std::uint32_t> &b) {
+  // physical tile order is unchanged when the last dim is kept and no padding is involved
+  if (a.empty() || b.empty() || a.back() != b.back()) return false;
+  Dims3 da = dims3(a), db = dims3(b);
+  return da.rows % 32 == 0 && db.rows % 32 == 0 && da.cols % 32 == 0 && a.size() >= 2 && b.size() >= 2;
+}
+
+Tensor reshapeTo(ProgramContext &ctx, const Tensor &in, const std::vector<std::uint32_t> &oshape) {
+  TTRT_ASSERT(volume(in.handle->shape) == volume(oshape), "reshape: element count differs");
+  if (in.handle->layout == TensorLayout::RowMajor || sameTiling(in.handle->shape, oshape)) {
+    auto t = std::make_shared<TensorImpl>();  // alias: same buffer, new logical shape
+    t->shape = oshape; t->dtype = in.handle->dtype; t->layout = in.handle->layout; t->storage = in.handle->storage;
+    t->data = in.handle->data; t->bytes = in.handle->bytes; t->device = in.handle->device; t->version = in.handle->version;
+    return Tensor{t};
+  }
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, in.handle->dtype, in.handle->layout);
+  zeroIfPadded(ctx, out);
+  std::vector<std::int64_t> e{volume(oshape)}, one{1};
+  copyView(ctx, in, out, e, one, 0, one, 0);
+  return out;
+}
+
+void runReshape(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = onDevice(ctx, ctx.get(op.table(schema::ReshapeOp::f_in), "reshape in"));
+  auto outRef = op.table(schema::ReshapeOp::f_out);
+  ctx.put(outRef, finish(ctx, reshapeTo(ctx, in, shapeFromTensorRef(outRef)), outRef));
+}
+
+Tensor permuteTo(ProgramContext &ctx, const Tensor &in, const std::vector<int> &perm) {
+  const auto &shape = in.handle->shape;
+  const size_t rank = shape.size();
+  TTRT_ASSERT(perm.size() == rank, "permute: permutation rank differs from the tensor rank");
+  std::vector<std::uint32_t> oshape(rank);
+  auto ss = rowMajorStrides(shape);
+  std::vector<std::int64_t> sst(rank);
+  for (size_t i = 0; i < rank; ++i) {
+    TTRT_ASSERT(perm[i] >= 0 && static_cast<size_t>(perm[i]) < rank, "permute: index out of range");
+    oshape[i] = shape[perm[i]];
+    sst[i] = ss[perm[i]];
+  }
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, in.handle->dtype, in.handle->layout);
+  zeroIfPadded(ctx, out);
+  copyView(ctx, in, out, toI64(oshape), sst, 0, rowMajorStrides(oshape), 0);
+  return out;
+}
+void runPermute(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = onDevice(ctx, ctx.get(op.table(schema::PermuteOp::f_in), "permute in"));
+  auto pv = op.scalars<std::int64_t>(schema::PermuteOp::f_permutation);
+  std::vector<int> perm;
+  for (std::uint32_t i = 0; i < pv.size(); ++i) perm.push_back(static_cast<int>(pv[i] < 0 ? pv[i] + pv.size() : pv[i]));
+  auto outRef = op.table(schema::PermuteOp::f_out);
+  ctx.put(outRef, finish(ctx, permuteTo(ctx, in, perm), outRef));
+}
+void runTranspose(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = onDevice(ctx, ctx.get(op.table(schema::TransposeOp::f_in), "transpose in"));
+  int rank = static_cast<int>(in.handle->shape.size());
+  int d0 = op.scalar<std::int32_t>(schema::TransposeOp::f_dim0, 0), d1 = op.scalar<std::int32_t>(schema::TransposeOp::f_dim1, 0);
+  if (d0 < 0) d0 += rank;
+  if (d1 < 0) d1 += rank;
+  std::vector<int> perm(rank);
+  for (int i = 0; i < rank; ++i) perm[i] = i;
+  TTRT_ASSERT(d0 >= 0 && d0 < rank && d1 >= 0 && d1 < rank, "transpose: dim out of range");
+  std::swap(perm[d0], perm[d1]);
+  auto outRef = op.table(schema::TransposeOp::f_out);
+  ctx.put(outRef, finish(ctx, permuteTo(ctx, in, perm), outRef));
+}
+void runConcat(const fb::Table &op, ProgramContext &ctx) {
+  auto ins = op.tables(schema::ConcatOp::f_inputs);
+  TTRT_ASSERT(ins.size() >= 1, "concat: no inputs");
+  auto outRef = op.table(schema::ConcatOp::f_out);
+  std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
+  Tensor first = onDevice(ctx, ctx.get(ins[0], "concat in"));
+  int rank = static_cast<int>(oshape.size());
+  int dim = op.scalar<std::int32_t>(schema::ConcatOp::f_dim, 0);
+  if (dim < 0) dim += rank;
+  TTRT_ASSERT(dim >= 0 && dim < rank, "concat: dim out of range");
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, first.handle->dtype, first.handle->layout);
+  zeroIfPadded(ctx, out);
+  auto os = rowMajorStrides(oshape);
+  std::int64_t at = 0;
+  for (std::uint32_t i = 0; i < ins.size(); ++i) {
+    Tensor t = as(ctx, ctx.get(ins[i], "concat in"), first.handle->layout, first.handle->dtype);
+    TTRT_ASSERT(static_cast<int>(t.handle->shape.size()) == rank, "concat: rank mismatch");
+    copyView(ctx, t, out, toI64(t.handle->shape), rowMajorStrides(t.handle->shape), 0, os, at * os[dim]);
+    at += t.handle->shape[dim];
+  }
+  TTRT_ASSERT(at == oshape[dim], "concat: inputs do not add up to the output extent");
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+void runSlice(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = onDevice(ctx, ctx.get(op.table(schema::SliceOp::f_in), "slice in"));
+  TTRT_ASSERT(op.scalar<std::uint8_t>(schema::SliceOp::f_params_type, 0) == static_cast<std::uint8_t>(schema::SliceOpParams::SliceStaticOpParams),
+              "slice: only static begins/ends are supported");
+  auto prm = op.table(schema::SliceOp::f_params);
+  auto begins = prm.scalars<std::int64_t>(schema::SliceStaticOpParams::f_begins), ends = prm.scalars<std::int64_t>(schema::SliceStaticOpParams::f_ends);
+  auto steps = op.scalars<std::int64_t>(schema::SliceOp::f_step);
+  const auto &shape = in.handle->shape;
+  const size_t rank = shape.size();
+  TTRT_ASSERT(begins.size() == rank && ends.size() == rank, "slice: begins/ends rank mismatch");
+  auto ss = rowMajorStrides(shape);
+  std::vector<std::uint32_t> oshape(rank);
+  std::vector<std::int64_t> sst(rank);
+  std::int64_t base = 0;
+  for (size_t i = 0; i < rank; ++i) {
+    std::int64_t b = begins[i], e = ends[i], st = i < steps.size() ? steps[i] : 1;
+    if (b < 0) b += shape[i];
+    if (e < 0) e += shape[i];
+    TTRT_ASSERT(st > 0 && b >= 0 && e <= static_cast<std::int64_t>(shape[i]) && b <= e, "slice: bad range");
+    oshape[i] = static_cast<std::uint32_t>((e - b + st - 1) / st);
+    sst[i] = ss[i] * st;
+    base += b * ss[i];
+  }
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, in.handle->dtype, in.handle->layout);
+  zeroIfPadded(ctx, out);
+  copyView(ctx, in, out, toI64(oshape), sst, base, rowMajorStrides(oshape), 0);
+  auto outRef = op.table(schema::SliceOp::f_out);
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+void runRepeatInterleave(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = onDevice(ctx, ctx.get(op.table(schema::RepeatInterleaveOp::f_input), "repeat_interleave in"));
+  const auto &shape = in.handle->shape;
+  int rank = static_cast<int>(shape.size());
+  int dim = op.scalar<std::int32_t>(schema::RepeatInterleaveOp::f_dim, 0);
+  if (dim < 0) dim += rank;
+  std::uint32_t rep = op.scalar<std::uint32_t>(schema::RepeatInterleaveOp::f_repeats, 1);
+  TTRT_ASSERT(dim >= 0 && dim < rank && rep >= 1, "repeat_interleave: bad arguments");
+  std::vector<std::uint32_t> oshape = shape;
+  oshape[dim] *= rep;
+  // view [.., shape[dim], rep, ..]: the rep axis has source stride 0
+  std::vector<std::int64_t> extent, sst, dstv;
+  auto ss = rowMajorStrides(shape), os = rowMajorStrides(oshape);
+  for (int i = 0; i < rank; ++i) {
+    extent.push_back(shape[i]);
+    sst.push_back(ss[i]);
+    dstv.push_back(i == dim ? os[i] * rep : os[i]);
+    if (i == dim) { extent.push_back(rep); sst.push_back(0); dstv.push_back(os[i]); }
+  }
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, in.handle->dtype, in.handle->layout);
+  zeroIfPadded(ctx, out);
+  copyView(ctx, in, out, extent, sst, 0, dstv, 0);
+  auto outRef = op.table(schema::RepeatInterleaveOp::f_out);
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// ---- creation (runtime/lib/ttnn/operations/creation/*.cpp)
+void runConstant(const fb::Table &op, ProgramContext &ctx) {
+  auto outRef = op.table(schema::ConstantOp::f_out);
+  auto bytes = op.scalars<std::uint8_t>(schema::ConstantOp::f_input);
+  DataType in = static_cast<DataType>(op.scalar<std::uint16_t>(schema::ConstantOp::f_input_dtype, 0));
+  std::vector<std::uint32_t> shape = shapeFromTensorRef(outRef);
+  TTRT_ASSERT(static_cast<std::int64_t>(bytes.size()) == volume(shape) * utils::dataTypeElementSize(in), "constant: payload size does not match the shape");
+  Tensor h = createOwnedHostTensor(bytes.data(), shape, {}, utils::dataTypeElementSize(in), in);
+  ctx.put(outRef, convertTo(ctx, h, layoutFromTensorRef(outRef)));
+}
+void fillTensor(ProgramContext &ctx, const fb::Table &outRef, double value) {
+  Layout want = layoutFromTensorRef(outRef);
+  std::vector<std::uint32_t> shape = shapeFromTensorRef(outRef);
+  std::int64_t n = volume(shape);
+  std::vector<float> host(static_cast<size_t>(n), static_cast<float>(value));
+  Tensor h = createOwnedHostTensor(host.data(), shape, {}, 4, DataType::Float32);
+  ctx.put(outRef, convertTo(ctx, h, want));
+}
+void runFull(const fb::Table &op, ProgramContext &ctx) {
+  double v = 0.0;
+  auto fv = op.table(schema::FullOp::f_fill_value);
+  auto kind = op.scalar<std::uint8_t>(schema::FullOp::f_fill_value_type, 0);
+  if (kind == static_cast<std::uint8_t>(schema::NumberType::FP)) v = fv.scalar<float>(schema::FloatingPointType::f_value, 0.0f);
+  else if (kind == static_cast<std::uint8_t>(schema::NumberType::I32)) v = fv.scalar<std::int32_t>(schema::IntegralType::f_value, 0);
+  fillTensor(ctx, op.table(schema::FullOp::f_out), v);
+}
+void runNamedFull(const fb::Table &op, ProgramContext &ctx) {
+  auto t = op.scalar<std::uint32_t>(schema::NamedFullOp::f_type, 0);
+  fillTensor(ctx, op.table(schema::NamedFullOp::f_out), t == static_cast<std::uint32_t>(schema::NamedFullOpType::Ones) ? 1.0 : 0.0);
+}
+void runEmpty(const fb::Table &op, ProgramContext &ctx) {
+  auto outRef = op.table(schema::EmptyOp::f_out);
+  Layout want = layoutFromTensorRef(outRef);
+  Tensor t = makeDeviceTensor(ctx.dev, shapeFromTensorRef(outRef), want.dataType, want.layout);
+  TTM_CALL(ttm_fill_u32(t.handle->data.get(), 0, (t.handle->bytes + 3) / 4, ctx.stream()));
+  ctx.put(outRef, t);
+}
+
+void runDeallocate(const fb::Table &op, ProgramContext &ctx) {
+  auto ref = op.table(schema::DeallocateOp::f_in);
+  std::uint32_t id = ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
+  auto it = ctx.pool.find(id);
+  if (it == ctx.pool.end()) return;
+  if (getTensorRetain(it->second)) return;  // runtime/lib/ttnn/operations/deletion/deallocate.cpp:16-18
+  ctx.pool.erase(it);                        // other aliases (reshape views) keep the buffer alive
+}
+
+// ---- const-eval (runtime/lib/ttnn/operations/cache/load_cached.cpp:20-90)
+struct CacheEntry {
+  std::vector<std::uint64_t> inputVersions;
+  std::vector<Tensor> outputs;
+};
+std::mutex g_cacheMu;
+std::map<std::pair<std::uint64_t, std::uint32_t>, CacheEntry> g_constEvalCache;
+
+void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
+  auto ins = op.tables(schema::LoadCachedOp::f_inputs), outs = op.tables(schema::LoadCachedOp::f_outputs);
+  std::uint32_t prog = op.scalar<std::uint32_t>(schema::LoadCachedOp::f_program_idx, 0);
+  std::vector<Tensor> inputs;
+  std::vector<std::uint64_t> versions;
+  for (std::uint32_t i = 0; i < ins.size(); ++i) {
+    inputs.push_back(ctx.get(ins[i], "load_cached in"));
+    versions.push_back(inputs.back().handle->version);
+  }
+  auto key = std::make_pair(ctx.binary.id(), prog);
+  {
+    std::lock_guard<std::mutex> g(g_cacheMu);
+    auto it = g_constEvalCache.find(key);
+    if (it != g_constEvalCache.end() && it->second.inputVersions == versions) {
+      debug::Stats::get().incrementStat("ConstEvalCacheHit");
+      for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], it->second.outputs.at(i));
+      return;
+    }
+  }
+  debug::Stats::get().incrementStat("ConstEvalCacheMiss");
+  std::vector<Tensor> results = executeProgram(ctx.dev, ctx.binary, prog, inputs);
+  TTRT_ASSERT(results.size() == outs.size(), "load_cached: callee returned a different number of outputs");
+  for (auto &t : results) setTensorRetain(t, true);
+  {
+    std::lock_guard<std::mutex> g(g_cacheMu);
+    g_constEvalCache[key] = CacheEntry{versions, results};
+  }
+  for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], results[i]);
+}
+void runFuncCall(const fb::Table &op, ProgramContext &ctx) {
+  auto ins = op.tables(schema::FuncCallOp::f_inputs), outs = op.tables(schema::FuncCallOp::f_outputs);
+  std::vector<Tensor> inputs;
+  for (std::uint32_t i = 0; i < ins.size(); ++i) inputs.push_back(ctx.get(ins[i], "func_call in"));
+  std::vector<Tensor> results = executeProgram(ctx.dev, ctx.binary, op.scalar<std::uint32_t>(schema::FuncCallOp::f_program_id, 0), inputs);
+  TTRT_ASSERT(results.size() == outs.size(), "func_call: callee returned a different number of outputs");
+  for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], results[i]);
+}
+
+void runOperation(const fb::Table &operation, ProgramContext &ctx) {
+  auto type = static_cast<OpType>(operation.scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
+  fb::Table op = operation.table(schema::Operation::f_type);
+  switch (type) {
+  case OpType::GetDeviceOp: return;
+  case OpType::ToLayoutOp: return runToLayout(op, ctx);
+  case OpType::TypecastOp: return runTypecast(op, ctx);
+  case OpType::ToDeviceOp: return runToDevice(op, ctx);
+  case OpType::FromDeviceOp: return runFromDevice(op, ctx);
+  case OpType::ToMemoryConfigOp: return runToMemoryConfig(op, ctx);
+  case OpType::MatmulOp: return runMatmul(op, ctx);
+  case OpType::LinearOp: return runLinear(op, ctx);
+  case OpType::EltwiseUnaryOp: return runEltwiseUnary(op, ctx);
+  case OpType::EltwiseBinaryOp: return runEltwiseBinary(op, ctx);
+  case OpType::RMSNormOp: return runRmsNorm(op, ctx);
+  case OpType::SoftmaxOp: return runSoftmax(op, ctx);
+  case OpType::ReductionOp: return runReduction(op, ctx);
+  case OpType::ScaledDotProductAttentionOp: return runSdpa(op, ctx);
+  case OpType::ReshapeOp: return runReshape(op, ctx);
+  case OpType::PermuteOp: return runPermute(op, ctx);
+  case OpType::TransposeOp: return runTranspose(op, ctx);
+  case OpType::ConcatOp: return runConcat(op, ctx);
+  case OpType::SliceOp: return runSlice(op, ctx);
+  case OpType::RepeatInterleaveOp: return runRepeatInterleave(op, ctx);
+  case OpType::ConstantOp: return runConstant(op, ctx);
+  case OpType::FullOp: return runFull(op, ctx);
+  case OpType::NamedFullOp: return runNamedFull(op, ctx);
+  case OpType::EmptyOp: return runEmpty(op, ctx);
+  case OpType::DeallocateOp: return runDeallocate(op, ctx);
+  case OpType::LoadCachedOp: return runLoadCached(op, ctx);
+  case OpType::FuncCallOp: return runFuncCall(op, ctx);
+  default: fatal(std::string("Unsupported operation type: ") + schema::opTypeName(type));
+  }
+}
+
+}  // namespace
+
+std::vector<Tensor> executeProgram(const std::shared_ptr<DeviceState> &dev, const Binary &binary, std::uint32_t programIndex,
+                                   std::vector<Tensor> &inputs) {
+  auto programs = binary.handle->root.tables(schema::TTNNBinary::f_programs);
+  TTRT_ASSERT(programIndex < programs.size(), "submit: program index out of range");
+  fb::Table program = programs[programIndex];
+  ProgramContext ctx;
+  ctx.dev = dev; ctx.binary = binary; ctx.programIndex = programIndex;
+  auto ins = program.tables(schema::Program::f_inputs);
+  TTRT_ASSERT(ins.size() == inputs.size(), "submit: program '" + std::string(program.string(schema::Program::f_name)) + "' expects " +
+                                               std::to_string(ins.size()) + " inputs, got " + std::to_string(inputs.size()));
+  for (std::uint32_t i = 0; i < ins.size(); ++i) {
+    TTRT_ASSERT(isTensorAllocated(inputs[i]), "submit: input " + std::to_string(i) + " is deallocated");
+    std::vector<std::uint32_t> want = shapeFromTensorRef(ins[i]);
+    TTRT_ASSERT(want == inputs[i].handle->shape, "submit: input " + std::to_string(i) + " has the wrong shape");
+    // callers must bring every input to the layout in the flatbuffer (docs/src/specs/runtime-stitching.md:50-66)
+    TTRT_ASSERT(getTensorLayout(inputs[i]) == layoutFromTensorRef(ins[i]),
+                "submit: input " + std::to_string(i) + " is not in the layout the program expects (use toLayout(getLayout(...)))");
+    ctx.put(ins[i], inputs[i]);
+  }
+  auto ops = program.tables(schema::Program::f_operations);
+  auto &hooks = debug::Hooks::get();
+  for (std::uint32_t i = 0; i < ops.size(); ++i) {
+    OpContext oc{ops[i], i};
+    CallbackContext cc{&ctx};
+    if (hooks.preOperatorCallback) (*hooks.preOperatorCallback)(binary, cc, oc);
+    runOperation(ops[i], ctx);
+    if (hooks.postOperatorCallback) (*hooks.postOperatorCallback)(binary, cc, oc);
+  }
+  std::vector<Tensor> outputs;
+  auto outs = program.tables(schema::Program::f_outputs);
+  for (std::uint32_t i = 0; i < outs.size(); ++i) outputs.push_back(ctx.get(outs[i], "program output"));
+  return outputs;
+}
+
+// ---- hook-side access to the running program (runtime/include/tt/runtime/runtime.h:246-297)
+static fb::Table firstOutputRef(const fb::Table &operation, std::vector<fb::Table> *all = nullptr) {
+  auto type = static_cast<OpType>(operation.scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
+  fb::Table op = operation.table(schema::Operation::f_type);
+  int slot = -1;
+  switch (type) {
+  case OpType::ToLayoutOp: slot = schema::ToLayoutOp::f_out; break;
+  case OpType::TypecastOp: slot = schema::TypecastOp::f_out; break;
+  case OpType::ToDeviceOp: slot = schema::ToDeviceOp::f_out; break;
+  case OpType::FromDeviceOp: slot = schema::FromDeviceOp::f_out; break;
+  case OpType::ToMemoryConfigOp: slot = schema::ToMemoryConfigOp::f_out; break;
+  case OpType::MatmulOp: slot = schema::MatmulOp::f_out; break;
+  case OpType::LinearOp: slot = schema::LinearOp::f_out; break;
+  case OpType::EltwiseUnaryOp: slot = schema::EltwiseUnaryOp::f_out; break;
+  case OpType::EltwiseBinaryOp: slot = schema::EltwiseBinaryOp::f_out; break;
+  case OpType::RMSNormOp: slot = schema::RMSNormOp::f_out; break;
+  case OpType::SoftmaxOp: slot = schema::SoftmaxOp::f_out; break;
+  case OpType::ReductionOp: slot = schema::ReductionOp::f_out; break;
+  case OpType::ScaledDotProductAttentionOp: slot = schema::ScaledDotProductAttentionOp::f_out; break;
+  case OpType::ReshapeOp: slot = schema::ReshapeOp::f_out; break;
+  case OpType::PermuteOp: slot = schema::PermuteOp::f_out; break;
+  case OpType::TransposeOp: slot = schema::TransposeOp::f_out; break;
+  case OpType::ConcatOp: slot = schema::ConcatOp::f_out; break;
+  case OpType::SliceOp: slot = schema::SliceOp::f_out; break;
+  case OpType::RepeatInterleaveOp: slot = schema::RepeatInterleaveOp::f_out; break;
+  case OpType::ConstantOp: slot = schema::ConstantOp::f_out; break;
+  case OpType::FullOp: slot = schema::FullOp::f_out; break;
+  case OpType::NamedFullOp: slot = schema::NamedFullOp::f_out; break;
+  case OpType::EmptyOp: slot = schema::EmptyOp::f_out; break;
+  default: break;
+  }
+  (void)all;
+  return slot >= 0 ? op.table(slot) : fb::Table();
+}
+
+std::unordered_map<std::uint32_t, Tensor> getOpOutputTensor(OpContext oc, CallbackContext cc) {
+  std::unordered_map<std::uint32_t, Tensor> out;
+  auto *ctx = static_cast<ProgramContext *>(cc.programContext);
+  fb::Table ref = firstOutputRef(oc.op);
+  if (!ref || !ctx) return out;
+  std::uint32_t id = ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
+  auto it = ctx->pool.find(id);
+  if (it == ctx->pool.end() || !isTensorAllocated(it->second)) return out;
+  out[0] = toHost(it->second, /*untilize=*/true)[0];
+  return out;
+}
+
+std::optional<Tensor> retrieveTensorFromPool(CallbackContext cc, std::uint32_t globalId, bool untilize) {
+  auto *ctx = static_cast<ProgramContext *>(cc.programContext);
+  if (!ctx) return std::nullopt;
+  auto it = ctx->pool.find(globalId);
+  if (it == ctx->pool.end() || !isTensorAllocated(it->second)) return std::nullopt;
+  return toHost(it->second, untilize)[0];
+}
+
+void updateTensorInPool(CallbackContext cc, std::uint32_t globalId, Tensor src) {
+  auto *ctx = static_cast<ProgramContext *>(cc.programContext);
+  TTRT_ASSERT(ctx != nullptr, "updateTensorInPool: no program context");
+  auto it = ctx->pool.find(globalId);
+  TTRT_ASSERT(it != ctx->pool.end(), "updateTensorInPool: tensor is not in the pool");
+  Tensor &dst = it->second;
+  TTRT_ASSERT(dst.handle->shape == src.handle->shape, "updateTensorInPool: shape mismatch");
+  // normalise the source to the destination's layout, then overwrite the payload in place
+  Layout want = getTensorLayout(dst);
+  Tensor conv = src;
+  if (want.storageType == StorageType::Device || conv.handle->layout != want.layout || conv.handle->dtype != want.dataType)
+    conv = convertOnDevice(conv.handle->storage == StorageType::Device ? conv : toDevice(conv, ctx->dev), want.layout, want.dataType);
+  if (want.storageType == StorageType::Host && conv.handle->storage == StorageType::Device) conv = fromDevice(conv);
+  memcpy(dst, conv);
+}
+
+}  // namespace tt::runtime

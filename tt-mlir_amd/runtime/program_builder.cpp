@@ -1,0 +1,526 @@
+#include "program_builder.h"
+
+#include <algorithm>
+
+namespace ttmlir_amd {
+
+using namespace schema;
+using Off = fb::Builder::Off;
+using ::tt::runtime::fatal;
+
+ProgramBuilder::Id ProgramBuilder::newTensor(const Desc &d) {
+  tensors_.push_back(d);
+  return static_cast<Id>(tensors_.size() - 1);
+}
+
+const ProgramBuilder::Desc &ProgramBuilder::desc(Id t) const {
+  if (t == 0 || t >= tensors_.size()) fatal("ProgramBuilder: unknown tensor id " + std::to_string(t));
+  return tensors_[t];
+}
+
+Off ProgramBuilder::memoryConfig(StorageType storage) {
+  b_.startTable(MemoryConfig::kNumFields);
+  b_.addScalarDefault<std::uint16_t>(MemoryConfig::f_tensor_memory_layout, static_cast<std::uint16_t>(TensorMemoryLayout::Interleaved), 0);
+  b_.addScalarDefault<std::uint16_t>(MemoryConfig::f_buffer_type,
+                                     static_cast<std::uint16_t>(storage == StorageType::Device ? BufferType::DRAM : BufferType::SystemMemory), 0);
+  return b_.endTable();
+}
+
+Off ProgramBuilder::tensorRef(Id t) {
+  const Desc &d = desc(t);
+  std::vector<std::int32_t> shape(d.shape.begin(), d.shape.end());
+  Off shapeOff = b_.createScalarVector(shape);
+  Off memcfg = memoryConfig(d.storage);
+  b_.startTable(MemoryDesc::kNumFields);
+  b_.addScalarDefault<std::uint16_t>(MemoryDesc::f_storage_type, static_cast<std::uint16_t>(d.storage), 0);
+  std::int32_t tile[2] = {d.layout == TensorLayout::Tile ? 32 : 1, d.layout == TensorLayout::Tile ? 32 : 1};
+  b_.addStruct(MemoryDesc::f_tile_shape, tile, sizeof(tile), 4);
+  b_.addScalarDefault<std::uint16_t>(MemoryDesc::f_data_type, static_cast<std::uint16_t>(d.dtype), 0);
+  b_.addOffset(MemoryDesc::f_memory_config, memcfg);
+  Off md = b_.endTable();
+  b_.startTable(LayoutDesc::kNumFields);
+  b_.addScalarDefault<std::uint16_t>(LayoutDesc::f_oob_val, static_cast<std::uint16_t>(OOBVal::Undef), 0);
+  b_.addOffset(LayoutDesc::f_memory_desc, md);
+  Off ld = b_.endTable();
+  b_.startTable(TensorDesc::kNumFields);
+  b_.addOffset(TensorDesc::f_shape, shapeOff);
+  b_.addOffset(TensorDesc::f_layout, ld);
+  b_.addScalarDefault<std::uint32_t>(TensorDesc::f_shard_status, static_cast<std::uint32_t>(ShardStatus::Unsharded), 0);
+  Off td = b_.endTable();
+  b_.startTable(TensorRef::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(TensorRef::f_global_id, t, 0);
+  b_.addOffset(TensorRef::f_desc, td);
+  return b_.endTable();
+}
+
+void ProgramBuilder::addOp(OpType type, Off table, const std::string &debug) {
+  if (!open_) fatal("ProgramBuilder: no program is open");
+  cur_.ops.push_back(OpRec{static_cast<std::uint8_t>(type), table, debug});
+}
+
+void ProgramBuilder::beginProgram(const std::string &name, bool isPrivate) {
+  if (open_) fatal("ProgramBuilder: a program is already open");
+  cur_ = ProgramRec{};
+  cur_.name = name;
+  cur_.isPrivate = isPrivate;
+  open_ = true;
+}
+
+ProgramBuilder::Id ProgramBuilder::input(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout, StorageType storage) {
+  Id t = newTensor(Desc{shape, dtype, layout, storage});
+  cur_.inputs.push_back(t);
+  return t;
+}
+void ProgramBuilder::output(Id t) {
+  desc(t);
+  cur_.outputs.push_back(t);
+}
+
+std::uint32_t ProgramBuilder::endProgram() {
+  if (!open_) fatal("ProgramBuilder: no program is open");
+  std::vector<Off> ops;
+  for (const OpRec &r : cur_.ops) {
+    Off dbg = b_.createString(r.debug);
+    Off loc = b_.createString("loc(\"" + cur_.name + "\")");
+    b_.startTable(Operation::kNumFields);
+    b_.addScalar<std::uint8_t>(Operation::f_type_type, r.type);
+    b_.addOffset(Operation::f_type, r.table);
+    b_.addOffset(Operation::f_debug_info, dbg);
+    b_.addOffset(Operation::f_loc_info, loc);
+    ops.push_back(b_.endTable());
+  }
+  std::vector<Off> ins, outs;
+  for (Id t : cur_.inputs) ins.push_back(tensorRef(t));
+  for (Id t : cur_.outputs) outs.push_back(tensorRef(t));
+  Off opsV = b_.createOffsetVector(ops), insV = b_.createOffsetVector(ins), outsV = b_.createOffsetVector(outs);
+  Off name = b_.createString(cur_.name);
+  b_.startTable(Program::kNumFields);
+  b_.addOffset(Program::f_name, name);
+  b_.addOffset(Program::f_inputs, insV);
+  b_.addOffset(Program::f_outputs, outsV);
+  b_.addOffset(Program::f_operations, opsV);
+  b_.addScalarDefault<std::uint8_t>(Program::f_private, cur_.isPrivate ? 1 : 0, 0);
+  std::int32_t mesh[2] = {1, 1};
+  b_.addStruct(Program::f_mesh_shape, mesh, sizeof(mesh), 4);
+  finishedPrograms_.push_back(b_.endTable());
+  open_ = false;
+  return static_cast<std::uint32_t>(finishedPrograms_.size() - 1);
+}
+
+std::vector<std::uint8_t> ProgramBuilder::finish() {
+  if (open_) fatal("ProgramBuilder: a program is still open");
+  Off programs = b_.createOffsetVector(finishedPrograms_);
+  Off hash = b_.createString("mi355x-native-writer");  // not reproducible without flatc; readers here never enforce it
+  Off git = b_.createString("0000000000000000000000000000000000000000");
+  b_.startTable(TTNNBinary::kNumFields);
+  struct { std::uint16_t major, minor; std::uint32_t patch; } ver{0, 1, 0};
+  b_.addStruct(TTNNBinary::f_version, &ver, sizeof(ver), 4);
+  b_.addOffset(TTNNBinary::f_schema_hash, hash);
+  b_.addOffset(TTNNBinary::f_ttmlir_git_hash, git);
+  b_.addOffset(TTNNBinary::f_programs, programs);
+  Off root = b_.endTable();
+  return b_.finishSizePrefixed(root, "TTNN");
+}
+
+// ------------------------------------------------------------------------------------ ops
+static std::string shapeStr(const std::vector<std::uint32_t> &s) {
+  std::string o = "[";
+  for (size_t i = 0; i < s.size(); ++i) o += (i ? "x" : "") + std::to_string(s[i]);
+  return o + "]";
+}
+
+ProgramBuilder::Id ProgramBuilder::toLayout(Id in, TensorLayout layout, int dtype, StorageType storage) {
+  Desc d = desc(in);
+  d.layout = layout;
+  d.storage = storage;
+  if (dtype >= 0) d.dtype = static_cast<DataType>(dtype);
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out), mc = memoryConfig(storage);
+  b_.startTable(ToLayoutOp::kNumFields);
+  b_.addOffset(ToLayoutOp::f_in, i);
+  b_.addScalarDefault<std::uint16_t>(ToLayoutOp::f_layout, static_cast<std::uint16_t>(layout), 0);
+  if (dtype >= 0) b_.addScalar<std::uint16_t>(ToLayoutOp::f_dtype, static_cast<std::uint16_t>(dtype));
+  b_.addOffset(ToLayoutOp::f_memcfg, mc);
+  b_.addOffset(ToLayoutOp::f_out, o);
+  addOp(OpType::ToLayoutOp, b_.endTable(), "ttnn.to_layout " + shapeStr(d.shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::typecast(Id in, DataType dtype) {
+  Desc d = desc(in);
+  d.dtype = dtype;
+  if (::tt::runtime::utils::isBlockFormatDataType(dtype)) d.layout = TensorLayout::Tile;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  b_.startTable(TypecastOp::kNumFields);
+  b_.addOffset(TypecastOp::f_in, i);
+  b_.addScalarDefault<std::uint16_t>(TypecastOp::f_dtype, static_cast<std::uint16_t>(dtype), 0);
+  b_.addOffset(TypecastOp::f_out, o);
+  addOp(OpType::TypecastOp, b_.endTable(), std::string("ttnn.typecast -> ") + ::tt::runtime::utils::dataTypeName(dtype));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::toDevice(Id in) {
+  Desc d = desc(in);
+  d.storage = StorageType::Device;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  b_.startTable(DeviceRef::kNumFields);
+  Off dev = b_.endTable();
+  b_.startTable(ToDeviceOp::kNumFields);
+  b_.addOffset(ToDeviceOp::f_in, i);
+  b_.addOffset(ToDeviceOp::f_device, dev);
+  b_.addOffset(ToDeviceOp::f_out, o);
+  addOp(OpType::ToDeviceOp, b_.endTable(), "ttnn.to_device");
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::fromDevice(Id in) {
+  Desc d = desc(in);
+  d.storage = StorageType::Host;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  b_.startTable(FromDeviceOp::kNumFields);
+  b_.addOffset(FromDeviceOp::f_in, i);
+  b_.addOffset(FromDeviceOp::f_out, o);
+  addOp(OpType::FromDeviceOp, b_.endTable(), "ttnn.from_device");
+  return out;
+}
+
+static std::vector<std::uint32_t> matmulShape(const std::vector<std::uint32_t> &a, const std::vector<std::uint32_t> &b, bool ta, bool tb) {
+  if (a.size() < 2 || b.size() < 2) fatal("ProgramBuilder: matmul operands must have rank >= 2");
+  std::uint32_t M = ta ? a[a.size() - 1] : a[a.size() - 2], K = ta ? a[a.size() - 2] : a[a.size() - 1];
+  std::uint32_t Kb = tb ? b[b.size() - 1] : b[b.size() - 2], N = tb ? b[b.size() - 2] : b[b.size() - 1];
+  if (K != Kb) fatal("ProgramBuilder: matmul inner dimensions differ");
+  std::vector<std::uint32_t> out(a.begin(), a.end() - 2);
+  if (b.size() > a.size()) out.assign(b.begin(), b.end() - 2);
+  out.push_back(M);
+  out.push_back(N);
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::matmul(Id a, Id b, bool ta, bool tb, const std::string &activation, DataType outDtype) {
+  Desc d{matmulShape(desc(a).shape, desc(b).shape, ta, tb), outDtype, TensorLayout::Tile, StorageType::Device};
+  Id out = newTensor(d);
+  Off ar = tensorRef(a), br = tensorRef(b), orf = tensorRef(out);
+  Off act = activation.empty() ? 0 : b_.createString(activation);
+  b_.startTable(MatmulOp::kNumFields);
+  b_.addOffset(MatmulOp::f_a, ar);
+  b_.addOffset(MatmulOp::f_b, br);
+  b_.addOffset(MatmulOp::f_out, orf);
+  b_.addScalarDefault<std::uint8_t>(MatmulOp::f_transpose_a, ta, 0);
+  b_.addScalarDefault<std::uint8_t>(MatmulOp::f_transpose_b, tb, 0);
+  b_.addOffset(MatmulOp::f_activation, act);
+  addOp(OpType::MatmulOp, b_.endTable(), "ttnn.matmul " + shapeStr(desc(a).shape) + " x " + shapeStr(desc(b).shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::linear(Id a, Id b, Id bias, bool ta, bool tb, const std::string &activation, DataType outDtype) {
+  Desc d{matmulShape(desc(a).shape, desc(b).shape, ta, tb), outDtype, TensorLayout::Tile, StorageType::Device};
+  Id out = newTensor(d);
+  Off ar = tensorRef(a), br = tensorRef(b), bi = bias ? tensorRef(bias) : 0, orf = tensorRef(out);
+  Off act = activation.empty() ? 0 : b_.createString(activation);
+  b_.startTable(DeviceComputeKernelConfig::kNumFields);
+  b_.addScalar<std::uint8_t>(DeviceComputeKernelConfig::f_math_fidelity, static_cast<std::uint8_t>(MathFidelity::HiFi4));
+  b_.addScalar<std::uint8_t>(DeviceComputeKernelConfig::f_fp32_dest_acc_en, 1);
+  Off cc = b_.endTable();
+  b_.startTable(LinearOp::kNumFields);
+  b_.addOffset(LinearOp::f_a, ar);
+  b_.addOffset(LinearOp::f_b, br);
+  b_.addOffset(LinearOp::f_bias, bi);
+  b_.addOffset(LinearOp::f_out, orf);
+  b_.addScalarDefault<std::uint8_t>(LinearOp::f_transpose_a, ta, 0);
+  b_.addScalarDefault<std::uint8_t>(LinearOp::f_transpose_b, tb, 0);
+  b_.addOffset(LinearOp::f_activation, act);
+  b_.addOffset(LinearOp::f_compute_config, cc);
+  addOp(OpType::LinearOp, b_.endTable(), "ttnn.linear " + shapeStr(desc(a).shape) + " x " + shapeStr(desc(b).shape) + (activation.empty() ? "" : " + " + activation));
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::unary(std::uint32_t type, Id in, bool hasParam, float param) {
+  Desc d = desc(in);
+  d.storage = StorageType::Device;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out), prm = 0;
+  if (hasParam) {
+    b_.startTable(EltwiseOpWithFloatParams::kNumFields);
+    b_.addScalar<float>(EltwiseOpWithFloatParams::f_parameter, param);
+    prm = b_.endTable();
+  }
+  b_.startTable(EltwiseUnaryOp::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(EltwiseUnaryOp::f_type, type, 0);
+  b_.addOffset(EltwiseUnaryOp::f_in, i);
+  b_.addOffset(EltwiseUnaryOp::f_out, o);
+  if (prm) {
+    b_.addScalar<std::uint8_t>(EltwiseUnaryOp::f_params_type, static_cast<std::uint8_t>(EltwiseUnaryOpParams::EltwiseOpWithFloatParams));
+    b_.addOffset(EltwiseUnaryOp::f_params, prm);
+  }
+  addOp(OpType::EltwiseUnaryOp, b_.endTable(), "ttnn.unary#" + std::to_string(type));
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::binary(std::uint32_t type, Id lhs, Id rhs) {
+  const auto &a = desc(lhs).shape, &b = desc(rhs).shape;
+  size_t rank = std::max(a.size(), b.size());
+  std::vector<std::uint32_t> shape(rank);
+  for (size_t i = 0; i < rank; ++i) {
+    std::uint32_t x = i < rank - a.size() ? 1 : a[i - (rank - a.size())], y = i < rank - b.size() ? 1 : b[i - (rank - b.size())];
+    if (x != y && x != 1 && y != 1) fatal("ProgramBuilder: binary operands do not broadcast");
+    shape[i] = std::max(x, y);
+  }
+  Desc d{shape, desc(lhs).dtype, desc(lhs).layout, StorageType::Device};
+  Id out = newTensor(d);
+  Off l = tensorRef(lhs), r = tensorRef(rhs), o = tensorRef(out);
+  b_.startTable(EltwiseBinaryOp::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(EltwiseBinaryOp::f_type, type, 0);
+  b_.addOffset(EltwiseBinaryOp::f_lhs, l);
+  b_.addOffset(EltwiseBinaryOp::f_rhs, r);
+  b_.addOffset(EltwiseBinaryOp::f_out, o);
+  addOp(OpType::EltwiseBinaryOp, b_.endTable(), "ttnn.binary#" + std::to_string(type));
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::rmsNorm(Id in, Id weight, Id bias, float eps) {
+  Desc d = desc(in);
+  d.storage = StorageType::Device;
+  d.layout = TensorLayout::Tile;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), w = weight ? tensorRef(weight) : 0, bi = bias ? tensorRef(bias) : 0, o = tensorRef(out);
+  b_.startTable(RMSNormOp::kNumFields);
+  b_.addOffset(RMSNormOp::f_input, i);
+  b_.addOffset(RMSNormOp::f_weight, w);
+  b_.addOffset(RMSNormOp::f_bias, bi);
+  b_.addScalar<float>(RMSNormOp::f_epsilon, eps);
+  b_.addOffset(RMSNormOp::f_out, o);
+  addOp(OpType::RMSNormOp, b_.endTable(), "ttnn.rms_norm " + shapeStr(d.shape));
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::softmax(Id in, int dim) {
+  Desc d = desc(in);
+  d.storage = StorageType::Device;
+  d.layout = TensorLayout::Tile;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  b_.startTable(SoftmaxOp::kNumFields);
+  b_.addOffset(SoftmaxOp::f_in, i);
+  b_.addOffset(SoftmaxOp::f_out, o);
+  b_.addScalarDefault<std::int32_t>(SoftmaxOp::f_dimension, dim, 0);
+  b_.addScalarDefault<std::uint8_t>(SoftmaxOp::f_numeric_stable, 1, 0);
+  addOp(OpType::SoftmaxOp, b_.endTable(), "ttnn.softmax dim=" + std::to_string(dim));
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::reduction(std::uint32_t type, Id in, const std::vector<int> &dims, bool keepDim) {
+  Desc d = desc(in);
+  int rank = static_cast<int>(d.shape.size());
+  std::vector<bool> red(rank, dims.empty());
+  for (int x : dims) red.at(x < 0 ? x + rank : x) = true;
+  std::vector<std::uint32_t> shape;
+  for (int i = 0; i < rank; ++i) {
+    if (!red[i]) shape.push_back(d.shape[i]);
+    else if (keepDim) shape.push_back(1);
+  }
+  Desc od{shape, d.dtype, TensorLayout::Tile, StorageType::Device};
+  Id out = newTensor(od);
+  Off i = tensorRef(in), o = tensorRef(out);
+  std::vector<std::int32_t> dv(dims.begin(), dims.end());
+  Off dimsOff = b_.createScalarVector(dv);
+  b_.startTable(ReductionOp::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(ReductionOp::f_type, type, 0);
+  b_.addOffset(ReductionOp::f_in, i);
+  b_.addOffset(ReductionOp::f_out, o);
+  b_.addOffset(ReductionOp::f_dim_arg, dimsOff);
+  b_.addScalarDefault<std::uint8_t>(ReductionOp::f_keep_dim, keepDim, 0);
+  addOp(OpType::ReductionOp, b_.endTable(), "ttnn.reduction#" + std::to_string(type));
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::sdpa(Id q, Id k, Id v, Id mask, bool causal, bool hasScale, float scale) {
+  Desc d = desc(q);
+  d.storage = StorageType::Device;
+  d.layout = TensorLayout::Tile;
+  Id out = newTensor(d);
+  using S = ScaledDotProductAttentionOp;
+  Off qr = tensorRef(q), kr = tensorRef(k), vr = tensorRef(v), mr = mask ? tensorRef(mask) : 0, o = tensorRef(out);
+  b_.startTable(S::kNumFields);
+  b_.addOffset(S::f_query, qr);
+  b_.addOffset(S::f_key, kr);
+  b_.addOffset(S::f_value, vr);
+  b_.addScalarDefault<std::uint8_t>(S::f_is_causal, causal, 0);
+  b_.addOffset(S::f_attention_mask, mr);
+  if (hasScale) b_.addScalar<float>(S::f_scale, scale);
+  b_.addOffset(S::f_out, o);
+  addOp(OpType::ScaledDotProductAttentionOp, b_.endTable(), "ttnn.scaled_dot_product_attention " + shapeStr(d.shape));
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::reshape(Id in, const std::vector<std::uint32_t> &shape) {
+  Desc d = desc(in);
+  d.shape = shape;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  std::vector<std::int32_t> sv(shape.begin(), shape.end());
+  Off s = b_.createScalarVector(sv);
+  b_.startTable(ReshapeOp::kNumFields);
+  b_.addOffset(ReshapeOp::f_in, i);
+  b_.addOffset(ReshapeOp::f_out, o);
+  b_.addOffset(ReshapeOp::f_shape, s);
+  addOp(OpType::ReshapeOp, b_.endTable(), "ttnn.reshape -> " + shapeStr(shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::permute(Id in, const std::vector<std::int64_t> &perm) {
+  Desc d = desc(in);
+  std::vector<std::uint32_t> shape(perm.size());
+  for (size_t i = 0; i < perm.size(); ++i) shape[i] = d.shape.at(static_cast<size_t>(perm[i]));
+  d.shape = shape;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out), p = b_.createScalarVector(perm);
+  b_.startTable(PermuteOp::kNumFields);
+  b_.addOffset(PermuteOp::f_in, i);
+  b_.addOffset(PermuteOp::f_permutation, p);
+  b_.addOffset(PermuteOp::f_out, o);
+  addOp(OpType::PermuteOp, b_.endTable(), "ttnn.permute -> " + shapeStr(shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::transpose(Id in, int dim0, int dim1) {
+  Desc d = desc(in);
+  int rank = static_cast<int>(d.shape.size());
+  std::swap(d.shape.at(dim0 < 0 ? dim0 + rank : dim0), d.shape.at(dim1 < 0 ? dim1 + rank : dim1));
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  b_.startTable(TransposeOp::kNumFields);
+  b_.addOffset(TransposeOp::f_in, i);
+  b_.addOffset(TransposeOp::f_out, o);
+  b_.addScalarDefault<std::int32_t>(TransposeOp::f_dim0, dim0, 0);
+  b_.addScalarDefault<std::int32_t>(TransposeOp::f_dim1, dim1, 0);
+  addOp(OpType::TransposeOp, b_.endTable(), "ttnn.transpose");
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::concat(const std::vector<Id> &ins, int dim) {
+  Desc d = desc(ins.at(0));
+  int rank = static_cast<int>(d.shape.size());
+  int ax = dim < 0 ? dim + rank : dim;
+  std::uint32_t total = 0;
+  for (Id t : ins) total += desc(t).shape.at(ax);
+  d.shape[ax] = total;
+  Id out = newTensor(d);
+  std::vector<Off> refs;
+  for (Id t : ins) refs.push_back(tensorRef(t));
+  Off iv = b_.createOffsetVector(refs), o = tensorRef(out);
+  b_.startTable(ConcatOp::kNumFields);
+  b_.addOffset(ConcatOp::f_inputs, iv);
+  b_.addOffset(ConcatOp::f_out, o);
+  b_.addScalarDefault<std::int32_t>(ConcatOp::f_dim, dim, 0);
+  addOp(OpType::ConcatOp, b_.endTable(), "ttnn.concat dim=" + std::to_string(dim));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::slice(Id in, const std::vector<std::int64_t> &begins, const std::vector<std::int64_t> &ends,
+                                         const std::vector<std::int64_t> &steps) {
+  Desc d = desc(in);
+  for (size_t i = 0; i < d.shape.size(); ++i) {
+    std::int64_t st = i < steps.size() ? steps[i] : 1;
+    d.shape[i] = static_cast<std::uint32_t>((ends.at(i) - begins.at(i) + st - 1) / st);
+  }
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  Off bv = b_.createScalarVector(begins), ev = b_.createScalarVector(ends), sv = b_.createScalarVector(steps);
+  b_.startTable(SliceStaticOpParams::kNumFields);
+  b_.addOffset(SliceStaticOpParams::f_begins, bv);
+  b_.addOffset(SliceStaticOpParams::f_ends, ev);
+  Off prm = b_.endTable();
+  b_.startTable(SliceOp::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(SliceOp::f_type, static_cast<std::uint32_t>(SliceOpType::SliceStaticOp), 0);
+  b_.addOffset(SliceOp::f_in, i);
+  b_.addOffset(SliceOp::f_out, o);
+  b_.addOffset(SliceOp::f_step, sv);
+  b_.addScalar<std::uint8_t>(SliceOp::f_params_type, static_cast<std::uint8_t>(SliceOpParams::SliceStaticOpParams));
+  b_.addOffset(SliceOp::f_params, prm);
+  addOp(OpType::SliceOp, b_.endTable(), "ttnn.slice_static -> " + shapeStr(d.shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::repeatInterleave(Id in, std::uint32_t repeats, int dim) {
+  Desc d = desc(in);
+  int rank = static_cast<int>(d.shape.size());
+  d.shape.at(dim < 0 ? dim + rank : dim) *= repeats;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  b_.startTable(RepeatInterleaveOp::kNumFields);
+  b_.addOffset(RepeatInterleaveOp::f_input, i);
+  b_.addOffset(RepeatInterleaveOp::f_out, o);
+  b_.addScalarDefault<std::uint32_t>(RepeatInterleaveOp::f_repeats, repeats, 0);
+  b_.addScalarDefault<std::int32_t>(RepeatInterleaveOp::f_dim, dim, 0);
+  addOp(OpType::RepeatInterleaveOp, b_.endTable(), "ttnn.repeat_interleave x" + std::to_string(repeats));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::constant(const void *data, size_t bytes, DataType inDtype, const std::vector<std::uint32_t> &shape,
+                                            DataType dtype, TensorLayout layout, StorageType storage) {
+  Id out = newTensor(Desc{shape, dtype, layout, storage});
+  Off payload = b_.createScalarVector(static_cast<const std::uint8_t *>(data), bytes), o = tensorRef(out);
+  b_.startTable(ConstantOp::kNumFields);
+  b_.addOffset(ConstantOp::f_input, payload);
+  b_.addScalarDefault<std::uint16_t>(ConstantOp::f_input_dtype, static_cast<std::uint16_t>(inDtype), 0);
+  b_.addScalar<std::uint16_t>(ConstantOp::f_dtype, static_cast<std::uint16_t>(dtype));
+  b_.addScalar<std::uint16_t>(ConstantOp::f_layout, static_cast<std::uint16_t>(layout));
+  b_.addOffset(ConstantOp::f_out, o);
+  addOp(OpType::ConstantOp, b_.endTable(), "ttnn.constant " + shapeStr(shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::full(const std::vector<std::uint32_t> &shape, float value, DataType dtype, TensorLayout layout) {
+  Id out = newTensor(Desc{shape, dtype, layout, StorageType::Device});
+  std::vector<std::int64_t> sv(shape.begin(), shape.end());
+  Off s = b_.createScalarVector(sv), o = tensorRef(out);
+  b_.startTable(FloatingPointType::kNumFields);
+  b_.addScalar<float>(FloatingPointType::f_value, value);
+  Off fv = b_.endTable();
+  b_.startTable(FullOp::kNumFields);
+  b_.addOffset(FullOp::f_shape, s);
+  b_.addScalar<std::uint8_t>(FullOp::f_fill_value_type, static_cast<std::uint8_t>(NumberType::FP));
+  b_.addOffset(FullOp::f_fill_value, fv);
+  b_.addScalar<std::uint16_t>(FullOp::f_dtype, static_cast<std::uint16_t>(dtype));
+  b_.addScalar<std::uint16_t>(FullOp::f_layout, static_cast<std::uint16_t>(layout));
+  b_.addOffset(FullOp::f_out, o);
+  addOp(OpType::FullOp, b_.endTable(), "ttnn.full " + shapeStr(shape));
+  return out;
+}
+void ProgramBuilder::deallocate(Id in, bool force) {
+  Off i = tensorRef(in);
+  b_.startTable(DeallocateOp::kNumFields);
+  b_.addOffset(DeallocateOp::f_in, i);
+  b_.addScalarDefault<std::uint8_t>(DeallocateOp::f_force, force, 0);
+  addOp(OpType::DeallocateOp, b_.endTable(), "ttnn.deallocate");
+}
+std::vector<ProgramBuilder::Id> ProgramBuilder::loadCached(std::uint32_t programIdx, const std::string &callee, const std::vector<Id> &ins,
+                                                           const std::vector<Desc> &outs) {
+  std::vector<Id> ids;
+  std::vector<Off> ir, orf;
+  for (Id t : ins) ir.push_back(tensorRef(t));
+  for (const Desc &d : outs) {
+    ids.push_back(newTensor(d));
+    orf.push_back(tensorRef(ids.back()));
+  }
+  Off iv = b_.createOffsetVector(ir), ov = b_.createOffsetVector(orf), name = b_.createString(callee);
+  Off hash = b_.createString(callee + "#" + std::to_string(programIdx));
+  b_.startTable(LoadCachedOp::kNumFields);
+  b_.addOffset(LoadCachedOp::f_inputs, iv);
+  b_.addOffset(LoadCachedOp::f_callee_name, name);
+  b_.addScalarDefault<std::uint32_t>(LoadCachedOp::f_program_idx, programIdx, 0);
+  b_.addOffset(LoadCachedOp::f_outputs, ov);
+  b_.addOffset(LoadCachedOp::f_program_hash, hash);
+  addOp(OpType::LoadCachedOp, b_.endTable(), "ttcore.load_cached @" + callee);
+  return ids;
+}
+std::vector<ProgramBuilder::Id> ProgramBuilder::funcCall(std::uint32_t programIdx, const std::vector<Id> &ins, const std::vector<Desc> &outs) {
+  std::vector<Id> ids;
+  std::vector<Off> ir, orf;
+  for (Id t : ins) ir.push_back(tensorRef(t));
+  for (const Desc &d : outs) {
+    ids.push_back(newTensor(d));
+    orf.push_back(tensorRef(ids.back()));
+  }
+  Off iv = b_.createOffsetVector(ir), ov = b_.createOffsetVector(orf);
+  b_.startTable(FuncCallOp::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(FuncCallOp::f_program_id, programIdx, 0);
+  b_.addOffset(FuncCallOp::f_inputs, iv);
+  b_.addOffset(FuncCallOp::f_outputs, ov);
+  addOp(OpType::FuncCallOp, b_.endTable(), "func.call #" + std::to_string(programIdx));
+  return ids;
+}
+
+}  // namespace ttmlir_amd

@@ -1,0 +1,84 @@
+// Writer of `.ttnn` flatbuffer programs for the op subset this backend executes.  The reference
+// ships no prebuilt binaries (they are produced by ttmlir-opt + ttmlir-translate, see
+// test/ttmlir/Runtime/TTNN/n150/**.mlir RUN lines), so tests and benchmarks build their programs
+// here; the wire format is the reference's (include/ttmlir/Target/TTNN/*.fbs).
+#pragma once
+#include <string>
+#include <vector>
+
+#include "runtime.h"
+
+namespace ttmlir_amd {
+
+using ::tt::target::DataType;
+using ::tt::target::StorageType;
+using ::tt::target::TensorLayout;
+
+class ProgramBuilder {
+public:
+  using Id = std::uint32_t;  // tensor global_id
+  struct Desc {
+    std::vector<std::uint32_t> shape;
+    DataType dtype;
+    TensorLayout layout;
+    StorageType storage;
+  };
+
+  void beginProgram(const std::string &name, bool isPrivate = false);
+  Id input(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout, StorageType storage);
+  void output(Id t);
+  std::uint32_t endProgram();  // returns the program index
+
+  Id toLayout(Id in, TensorLayout layout, int dtype /* -1 = keep */, StorageType storage);
+  Id typecast(Id in, DataType dtype);
+  Id toDevice(Id in);
+  Id fromDevice(Id in);
+  Id matmul(Id a, Id b, bool transposeA, bool transposeB, const std::string &activation, DataType outDtype);
+  Id linear(Id a, Id b, Id bias /* 0 = none */, bool transposeA, bool transposeB, const std::string &activation, DataType outDtype);
+  Id unary(std::uint32_t type, Id in, bool hasParam, float param);
+  Id binary(std::uint32_t type, Id lhs, Id rhs);
+  Id rmsNorm(Id in, Id weight, Id bias, float eps);
+  Id softmax(Id in, int dim);
+  Id reduction(std::uint32_t type, Id in, const std::vector<int> &dims, bool keepDim);
+  Id sdpa(Id q, Id k, Id v, Id mask, bool causal, bool hasScale, float scale);
+  Id reshape(Id in, const std::vector<std::uint32_t> &shape);
+  Id permute(Id in, const std::vector<std::int64_t> &perm);
+  Id transpose(Id in, int dim0, int dim1);
+  Id concat(const std::vector<Id> &ins, int dim);
+  Id slice(Id in, const std::vector<std::int64_t> &begins, const std::vector<std::int64_t> &ends, const std::vector<std::int64_t> &steps);
+  Id repeatInterleave(Id in, std::uint32_t repeats, int dim);
+  Id constant(const void *data, size_t bytes, DataType inDtype, const std::vector<std::uint32_t> &shape, DataType dtype,
+              TensorLayout layout, StorageType storage);
+  Id full(const std::vector<std::uint32_t> &shape, float value, DataType dtype, TensorLayout layout);
+  void deallocate(Id in, bool force);
+  std::vector<Id> loadCached(std::uint32_t programIdx, const std::string &callee, const std::vector<Id> &ins, const std::vector<Desc> &outs);
+  std::vector<Id> funcCall(std::uint32_t programIdx, const std::vector<Id> &ins, const std::vector<Desc> &outs);
+
+  const Desc &desc(Id t) const;
+  std::vector<std::uint8_t> finish();  // size-prefixed TTNN binary
+
+private:
+  struct OpRec {
+    std::uint8_t type;
+    fb::Builder::Off table;
+    std::string debug;
+  };
+  struct ProgramRec {
+    std::string name;
+    bool isPrivate = false;
+    std::vector<Id> inputs, outputs;
+    std::vector<OpRec> ops;
+  };
+  Id newTensor(const Desc &d);
+  fb::Builder::Off tensorRef(Id t);
+  fb::Builder::Off memoryConfig(StorageType storage);
+  void addOp(::ttmlir_amd::schema::OpType type, fb::Builder::Off table, const std::string &debug);
+
+  fb::Builder b_;
+  std::vector<Desc> tensors_{Desc{}};  // index = id; id 0 is "none"
+  std::vector<fb::Builder::Off> finishedPrograms_;
+  ProgramRec cur_;
+  bool open_ = false;
+};
+
+}  // namespace ttmlir_amd

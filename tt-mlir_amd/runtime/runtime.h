@@ -1,0 +1,177 @@
+// tt::runtime-style host API of the MI355X backend.  Names, argument meaning and error behaviour
+// follow runtime/include/tt/runtime/runtime.h:31-308 and types.h:112-150, 392-481 of tt-mlir, for the
+// subset a `.ttnn` program needs on one device: load a binary, create host tensors, convert them to
+// the layout the program expects, submit, wait, read back.  Errors throw std::runtime_error, like
+// the reference's LOG_FATAL (runtime/include/tt/runtime/detail/common/logger.h:301-320).
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <functional>
+#include <memory>
+#include <optional>
+#include <string>
+#include <string_view>
+#include <unordered_map>
+#include <vector>
+
+#include "flatbuffer.h"
+#include "schema_generated.h"
+
+namespace tt::target {
+using DataType = ::ttmlir_amd::schema::DataType;
+using TensorLayout = ::ttmlir_amd::schema::TensorLayout;
+using StorageType = ::ttmlir_amd::schema::StorageType;
+}  // namespace tt::target
+
+namespace tt::runtime {
+
+namespace fb = ::ttmlir_amd::fb;
+
+[[noreturn]] void fatal(const std::string &msg);
+#define TTRT_ASSERT(cond, msg)                 \
+  do {                                         \
+    if (!(cond)) ::tt::runtime::fatal(msg);    \
+  } while (0)
+
+// ---- dtype helpers (runtime/lib/common/utils.cpp:140-290)
+namespace utils {
+std::uint32_t dataTypeElementSize(::tt::target::DataType dataType);
+bool isBlockFormatDataType(::tt::target::DataType dataType);
+std::uint64_t blockFormatTileSizeBytes(::tt::target::DataType dataType);
+bool isSupportedDataType(::tt::target::DataType dataType);
+::tt::target::DataType getUnsupportedDataTypeAlias(::tt::target::DataType unsupportedDataType);
+void handleBufferCast(const void *oldBuffer, void *newBuffer, ::tt::target::DataType oldDataType,
+                      ::tt::target::DataType newDataType, std::int64_t numElements);
+std::vector<std::int64_t> calculateStride(const std::vector<std::uint32_t> &shape);
+const char *dataTypeName(::tt::target::DataType dataType);
+}  // namespace utils
+
+struct TensorDesc {
+  std::vector<std::uint32_t> shape;
+  std::vector<std::int64_t> stride;
+  ::tt::target::DataType dataType = ::tt::target::DataType::Float32;
+  std::uint32_t elementSize() const { return utils::dataTypeElementSize(dataType); }
+};
+
+// Layout of a tensor as a program sees it (runtime/include/tt/runtime/detail/ttnn/types/types.h:112-135)
+struct Layout {
+  ::tt::target::StorageType storageType = ::tt::target::StorageType::Host;
+  ::tt::target::TensorLayout layout = ::tt::target::TensorLayout::RowMajor;
+  ::tt::target::DataType dataType = ::tt::target::DataType::Float32;
+  bool operator==(const Layout &o) const { return storageType == o.storageType && layout == o.layout && dataType == o.dataType; }
+};
+
+struct DeviceState;
+struct TensorImpl;
+struct BinaryImpl;
+
+struct Device {
+  std::shared_ptr<DeviceState> handle;
+};
+struct Tensor {
+  std::shared_ptr<TensorImpl> handle;
+  explicit operator bool() const { return handle != nullptr; }
+};
+struct Event {
+  std::shared_ptr<void> handle;
+};
+
+struct MeshDeviceOptions {
+  std::vector<std::uint32_t> meshShape{1, 1};
+  std::vector<int> deviceIds;
+};
+
+// ---- binary (runtime/lib/binary.cpp)
+struct TensorRefInfo {
+  std::uint32_t globalId = 0;
+  std::vector<std::uint32_t> shape;
+  Layout layout;
+};
+struct Binary {
+  std::shared_ptr<BinaryImpl> handle;
+  static Binary loadFromPath(const std::string &path);
+  static Binary loadFromMemory(const void *data, size_t size);  // copies
+  void store(const std::string &path) const;
+  std::string getFileIdentifier() const;
+  std::string getVersion() const;
+  std::string getSchemaHash() const;
+  std::uint32_t getNumPrograms() const;
+  std::string getProgramName(std::uint32_t programIndex) const;
+  bool isProgramPrivate(std::uint32_t programIndex) const;
+  std::vector<TensorRefInfo> getProgramInputs(std::uint32_t programIndex) const;
+  std::vector<TensorRefInfo> getProgramOutputs(std::uint32_t programIndex) const;
+  std::uint32_t getNumOps(std::uint32_t programIndex) const;
+  std::string getProgramOpsAsText(std::uint32_t programIndex) const;
+  std::uint64_t id() const;
+};
+
+// ---- debug hooks (runtime/include/tt/runtime/debug.h:77-157)
+struct OpContext {
+  fb::Table op;  // the Operation table
+  std::uint32_t index = 0;
+};
+struct CallbackContext {
+  void *programContext = nullptr;
+};
+namespace debug {
+using CallbackFn = std::function<void(Binary, CallbackContext, OpContext)>;
+struct Hooks {
+  static Hooks &get(std::optional<CallbackFn> preOperator = std::nullopt, std::optional<CallbackFn> postOperator = std::nullopt);
+  std::optional<CallbackFn> preOperatorCallback, postOperatorCallback;
+  void unregisterHooks();
+};
+struct Stats {
+  static Stats &get();
+  void incrementStat(const std::string &stat, std::int64_t value = 1);
+  std::int64_t getStat(const std::string &stat) const;
+  void clear();
+  std::unordered_map<std::string, std::int64_t> counters;
+};
+}  // namespace debug
+
+// ---- API
+size_t getNumAvailableDevices();
+Device openMeshDevice(const MeshDeviceOptions &options = {});
+void closeMeshDevice(Device parentMesh);
+std::string getDeviceName(Device device);
+
+Tensor createBorrowedHostTensor(void *data, const std::vector<std::uint32_t> &shape, const std::vector<std::int64_t> &stride,
+                                std::uint32_t itemsize, ::tt::target::DataType dataType);
+Tensor createOwnedHostTensor(const void *data, const std::vector<std::uint32_t> &shape, const std::vector<std::int64_t> &stride,
+                             std::uint32_t itemsize, ::tt::target::DataType dataType);
+Tensor createEmptyTensor(Device device, Layout layout, const std::vector<std::uint32_t> &shape,
+                         const std::vector<std::int64_t> &stride, std::uint32_t itemsize);
+
+bool isTensorAllocated(Tensor tensor);
+::tt::target::DataType getTensorDataType(Tensor tensor);
+std::vector<std::byte> getTensorDataBuffer(Tensor tensor);
+std::uint32_t getTensorElementSize(Tensor tensor);
+std::uint32_t getTensorVolume(Tensor tensor);
+std::vector<std::uint32_t> getTensorShape(Tensor tensor);
+std::vector<std::int64_t> getTensorStride(Tensor tensor);
+TensorDesc getTensorDesc(Tensor tensor);
+bool getTensorRetain(Tensor tensor);
+void setTensorRetain(Tensor tensor, bool retain);
+Layout getTensorLayout(Tensor tensor);
+bool hasLayout(Tensor tensor, Layout layout);
+
+void wait(Event event);
+void wait(Tensor tensor, std::optional<std::uint8_t> cqId = std::nullopt);
+void wait(const std::vector<Tensor> &tensors, std::optional<std::uint8_t> cqId = std::nullopt);
+
+std::vector<Tensor> toHost(Tensor tensor, bool untilize = false, bool blocking = true);
+Tensor toLayout(Tensor tensor, Device device, Layout layout, std::optional<bool> retain = std::nullopt);
+Layout getLayout(Binary executableHandle, std::uint32_t programIndex, std::uint32_t inputIndex);
+void memcpy(void *dst, Tensor src, std::optional<::tt::target::DataType> targetDataType = std::nullopt);
+void memcpy(Tensor dst, Tensor src);
+void deallocateTensor(Tensor &tensor, bool force = false);
+
+std::string getOpDebugString(OpContext opContextHandle);
+std::string getOpLocInfo(OpContext opContextHandle);
+std::unordered_map<std::uint32_t, Tensor> getOpOutputTensor(OpContext opContextHandle, CallbackContext programContextHandle);
+std::optional<Tensor> retrieveTensorFromPool(CallbackContext programContextHandle, std::uint32_t globalId, bool untilize);
+void updateTensorInPool(CallbackContext programContextHandle, std::uint32_t globalId, Tensor srcTensor);
+
+std::vector<Tensor> submit(Device deviceHandle, Binary executableHandle, std::uint32_t programIndex, std::vector<Tensor> &inputs);
+
+}  // namespace tt::runtime
