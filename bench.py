@@ -110,6 +110,35 @@ def make_workloads(torch, hip, datagen, dev, names):
             out[nm] = Workload(nm, "hbm", nbytes, "bytes", fn,
                                "config 3 decode: bf16 [32,4096] x bfp8_b [4096,14336] + bias + GELU (weight streaming)",
                                dict(flop=2.0 * M * N * K))
+    # whole programs through the runtime boundary (flatbuffer -> submit -> wait)
+    for nm in ("mlp512", "decoder2048"):
+        if nm not in names:
+            continue
+        from ttmlir_amd import programs, runtime as rt
+        bfl = lambda t: t.to(torch.bfloat16)
+        if nm == "mlp512":
+            d = datagen.c4_mlp()
+            binary = rt.Binary.load_from_memory(programs.c4_mlp())
+            tins = [d["x"], d["norm_w"], bfl(d["wg"]), bfl(d["wu"]), bfl(d["wd"])]
+            flop, desc = 180388626432.0, "config 4: Llama MLP block, 512 tokens (RMSNorm, gate/up bfp8_b, SiLU*up, down bfp4_b), one submit"
+        else:
+            d = datagen.c5_decoder()
+            binary = rt.Binary.load_from_memory(programs.c5_decoder())
+            tins = [d["x"], d["attn_norm_w"], bfl(d["wq"]), bfl(d["wk"]), bfl(d["wv"]), bfl(d["wo"]), d["mlp_norm_w"], bfl(d["wg"]),
+                    bfl(d["wu"]), bfl(d["wd"])]
+            flop = 893353197568.0 + 68719476736.0
+            desc = "config 5: Llama-3-8B decoder layer, batch 1, seq 2048 prefill (dense attention FLOPs counted), one submit"
+        rdev = rt.open_mesh_device()
+        rins = [rt.to_layout(rt.from_torch(t), rdev, rt.get_layout(binary, 1, i), retain=True) for i, t in enumerate(tins)]
+        del d, tins
+
+        def run(binary=binary, rins=rins, rdev=rdev):
+            outs = rt.submit(rdev, binary, 1, rins)
+            rt.wait(outs)
+            for o in outs:
+                rt.deallocate_tensor(o, force=True)
+
+        out[nm] = Workload(nm, "mfma", flop, "flop", run, desc, dict(sync=True, keep=(rdev, rins, binary)))
     return out
 
 
@@ -169,7 +198,7 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="linear2048")
-    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32")
+    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,mlp512,decoder2048")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -193,6 +222,8 @@ def main():
         for _ in range(warmup):
             w.fn()
         ms = _wall_time(torch, w.fn, steps)                    # timed region: exactly `steps` launches
+        if w.extra.get("sync"):                                # whole programs run on the runtime's own stream and sync inside
+            return ms, ms
         kms = _events_time(hip, stream, w.fn, steps)           # HIP events on the launch stream
         return ms, kms
 
@@ -206,7 +237,8 @@ def main():
     secondary = []
     for n in sec_names:
         w = wl[n]
-        sms, skms = measure(w, max(10, args.steps // 2), max(3, args.warmup // 2))
+        heavy = bool(w.extra.get("sync"))
+        sms, skms = measure(w, 5 if heavy else max(10, args.steps // 2), 2 if heavy else max(3, args.warmup // 2))
         r = roofline(w, skms)
         secondary.append({"workload": n, "desc": w.desc, "ms_per_step": round(sms, 5), "roofline": r})
 

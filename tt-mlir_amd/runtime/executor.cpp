@@ -576,7 +576,13 @@ struct CacheEntry {
   std::vector<Tensor> outputs;
 };
 std::mutex g_cacheMu;
-std::map<std::pair<std::uint64_t, std::uint32_t>, CacheEntry> g_constEvalCache;
+using ConstEvalCache = std::map<std::pair<std::uint64_t, std::uint32_t>, CacheEntry>;
+ConstEvalCache &constEvalCache() {
+  // leaked on purpose: its tensors own device memory, which must not be released from static
+  // destructors that run after the HIP runtime has begun shutting down
+  static ConstEvalCache *c = new ConstEvalCache;
+  return *c;
+}
 
 void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
   auto ins = op.tables(schema::LoadCachedOp::f_inputs), outs = op.tables(schema::LoadCachedOp::f_outputs);
@@ -590,8 +596,8 @@ void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
   auto key = std::make_pair(ctx.binary.id(), prog);
   {
     std::lock_guard<std::mutex> g(g_cacheMu);
-    auto it = g_constEvalCache.find(key);
-    if (it != g_constEvalCache.end() && it->second.inputVersions == versions) {
+    auto it = constEvalCache().find(key);
+    if (it != constEvalCache().end() && it->second.inputVersions == versions) {
       debug::Stats::get().incrementStat("ConstEvalCacheHit");
       for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], it->second.outputs.at(i));
       return;
@@ -603,7 +609,7 @@ void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
   for (auto &t : results) setTensorRetain(t, true);
   {
     std::lock_guard<std::mutex> g(g_cacheMu);
-    g_constEvalCache[key] = CacheEntry{versions, results};
+    constEvalCache()[key] = CacheEntry{versions, results};
   }
   for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], results[i]);
 }

@@ -363,8 +363,10 @@ struct DevicePool {
   }
 };
 DevicePool &pool() {
-  static DevicePool p;
-  return p;
+  // never destroyed: tensors held by other statics (the const-eval cache) return their blocks here
+  // during process teardown, after function-local statics would already be gone
+  static DevicePool *p = new DevicePool;
+  return *p;
 }
 }  // namespace
 
