@@ -195,8 +195,8 @@ def cpu_baseline_pack(orc, datagen, rows=8192):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="linear2048")
     ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,mlp512,decoder2048")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -219,6 +219,13 @@ def main():
         raise SystemExit("unknown workload " + args.workload)
 
     def measure(w, steps, warmup):
+        # clocks settle only after some tens of milliseconds of load: keep the device busy for about 0.3 s before
+        # the `warmup` untimed steps, so that short default runs measure the steady state
+        t_end = time.perf_counter() + 0.3
+        while time.perf_counter() < t_end:
+            for _ in range(8):
+                w.fn()
+            torch.cuda.synchronize()
         for _ in range(warmup):
             w.fn()
         ms = _wall_time(torch, w.fn, steps)                    # timed region: exactly `steps` launches

@@ -36,7 +36,7 @@ struct LinearArgs {
   int act, bias_tiled;
   int64_t a_batch, w_batch, c_batch;  // byte strides between batch entries (w_batch 0 = shared weights)
   int m_blocks, n_blocks;
-  int debug;  // measurement only: 1 skips the conversion phase, 2 skips the multiply phase, 4 swaps the phase groups
+  int split, nt_split, ntw_a, ntw_b;  // two-part grid of the block-float main kernel
 };
 
 template <int ACT>
@@ -214,13 +214,15 @@ __device__ __forceinline__ void store_w(u32x4 *ldsW, int tid, const WRegs<WF> &r
 
 // bias, activation, bf16, 8-byte stores into the output face rows.  acc[a][b]: n tile a, m tile b of the
 // wavefront; a lane holds m = lane % 32 and n = 8 g + 4 (lane / 32) + r in register g * 4 + r.
-template <int ACT, int MB>
-__device__ __forceinline__ void linear_epilogue(const LinearArgs &p, uint8_t *C, f32x16 (&acc)[4][MB], int mtw, int ntw, int lane) {
+// bias, activation, bf16, and 8-byte stores into the output face rows for a wavefront's NA x MB accumulator tiles;
+// column tiles at or beyond nt_end are left alone
+template <int ACT, int NA, int MB>
+__device__ __forceinline__ void linear_epilogue(const LinearArgs &p, uint8_t *C, f32x16 (&acc)[NA][MB], int mtw, int ntw, int nt_end, int lane) {
   const int m_in = lane & 31;
 #pragma unroll
-  for (int a = 0; a < 4; ++a) {
+  for (int a = 0; a < NA; ++a) {
     const int nt = ntw + a;
-    if (nt >= p.Nt) continue;
+    if (nt >= nt_end) continue;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const int n_in = g * 8 + (lane >> 5) * 4;
@@ -244,6 +246,16 @@ __device__ __forceinline__ void linear_epilogue(const LinearArgs &p, uint8_t *C,
         *(u32x2 *)(C + off * 2) = o;
       }
     }
+  }
+}
+template <int NA, int MB>
+__device__ __forceinline__ void linear_epilogue_act(const LinearArgs &p, uint8_t *C, f32x16 (&acc)[NA][MB], int mtw, int ntw, int nt_end, int lane) {
+  switch (p.act) {   // uniform
+  case TTM_ACT_GELU: linear_epilogue<TTM_ACT_GELU>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  case TTM_ACT_SILU: linear_epilogue<TTM_ACT_SILU>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  case TTM_ACT_SIGMOID: linear_epilogue<TTM_ACT_SIGMOID>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  case TTM_ACT_RELU: linear_epilogue<TTM_ACT_RELU>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  default: linear_epilogue<TTM_ACT_NONE>(p, C, acc, mtw, ntw, nt_end, lane); break;
   }
 }
 
@@ -329,236 +341,9 @@ __global__ __launch_bounds__(256) void ttm_linear_big_k(LinearArgs p) {
     __syncthreads();
   }
 
-  switch (p.act) {
-  case TTM_ACT_GELU: linear_epilogue<TTM_ACT_GELU>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  case TTM_ACT_SILU: linear_epilogue<TTM_ACT_SILU>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  case TTM_ACT_SIGMOID: linear_epilogue<TTM_ACT_SIGMOID>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  case TTM_ACT_RELU: linear_epilogue<TTM_ACT_RELU>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  default: linear_epilogue<TTM_ACT_NONE>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  }
+  linear_epilogue_act(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, p.Nt, lane);
 }
 
-// =============================================================================================
-// Software-pipelined variant of the large-M kernel.  Raw operand data of k-step ks+1 sits in
-// registers while the MFMAs of step ks run; its dequantisation / LDS stores are cut into four
-// quarters issued between the four k16 groups of MFMAs, so VALU and LDS-write work overlaps the
-// matrix pipe instead of following it.  Two register sets alternate (loop unrolled by two): the
-// global loads of step ks+2 are issued at the top of step ks.  Loads are unconditional with
-// clamped tile indices (no branches inside the loop); only the k tail needs zeroed weights,
-// rows / columns beyond M / N are computed on clamped data and never stored.
-// =============================================================================================
-__device__ __forceinline__ void load_a_raw(const LinearArgs &p, const uint8_t *A, int mt0, int kt0, int tid, u32x4 (&a)[8]) {
-  const int ktA = min(kt0 + (tid >> 7), p.Kt - 1);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int mt = min(mt0 + i, p.Mt - 1);
-    a[i] = *((const u32x4 *)(A + ((int64_t)mt * p.Kt + ktA) * 2048) + (tid & 127));
-  }
-}
-
-template <int WF>
-__device__ __forceinline__ void load_w_raw(const LinearArgs &p, const uint8_t *W, int nt0, int kt0, int tid, WRegs<WF> &r) {
-  if constexpr (WF == WF_BF16_NK) {
-    const int ktA = min(kt0 + (tid >> 7), p.Kt - 1);
-    const bool ok = kt0 + (tid >> 7) < p.Kt;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int nt = min(nt0 + i, p.Nt - 1);
-      u32x4 v = *((const u32x4 *)(W + ((int64_t)nt * p.Kt + ktA) * 2048) + (tid & 127));
-      r.direct[i] = ok ? v : u32x4{0, 0, 0, 0};
-    }
-  } else {
-    const int tile_l = tid >> 4, w = tid & 15;
-    const int ktw = kt0 + (tile_l >> 3);
-    const bool ok = ktw < p.Kt;
-    const int kt = min(ktw, p.Kt - 1), nt = min(nt0 + (tile_l & 7), p.Nt - 1);
-    const int face = w >> 2, khalf = (w >> 1) & 1, oct = w & 1;
-    const int64_t tile = (int64_t)kt * p.Nt + nt;
-    if constexpr (WF == WF_BFP8) {
-      const uint8_t *t = W + tile * 1088;
-      r.exps = *(const u32x2 *)(t + face * 16 + khalf * 8);
-      const uint8_t *m = t + 64 + face * 256 + khalf * 128 + oct * 8;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        u32x2 v = *(const u32x2 *)(m + i * 16);
-        r.rows8[i] = ok ? v : u32x2{0, 0};   // zero magnitudes: the k tail contributes nothing
-      }
-    } else if constexpr (WF == WF_BFP4) {
-      const uint8_t *t = W + tile * 576;
-      r.exps = *(const u32x2 *)(t + face * 16 + khalf * 8);
-      const uint8_t *m = t + 64 + face * 128 + khalf * 64 + oct * 4;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        uint32_t v = *(const uint32_t *)(m + i * 8);
-        r.rows4[i] = ok ? v : 0u;
-      }
-    } else {
-      const uint8_t *m = W + tile * 2048 + face * 512 + khalf * 256 + oct * 16;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        u32x4 v = *(const u32x4 *)(m + i * 32);
-        r.rows16[i] = ok ? v : u32x4{0, 0, 0, 0};
-      }
-    }
-  }
-}
-
-// quarter q of the conversion of one raw weight register set: rows (k) 2q and 2q+1 of the lane's 8x8 weight
-// block become word q of each of the 8 output chunks.
-template <int WF>
-__device__ __forceinline__ void convert_quarter(int q, const WRegs<WF> &rw, u32x4 (&out)[8], u32x4 *ldsW, int tid) {
-  struct { const WRegs<WF> &w; } r{rw};
-  if constexpr (WF == WF_BF16_NK) {
-    ldsW[copy_lds_chunk(tid, 2 * q)] = r.w.direct[2 * q];
-    ldsW[copy_lds_chunk(tid, 2 * q + 1)] = r.w.direct[2 * q + 1];
-  } else if constexpr (WF == WF_BF16_KN) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-      out[j][q] = __builtin_amdgcn_perm(r.w.rows16[2 * q + 1][j >> 1], r.w.rows16[2 * q][j >> 1], sel);
-    }
-  } else {
-    float f[2][8];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int i = 2 * q + h;
-      uint32_t E = ((i < 4 ? r.w.exps.x : r.w.exps.y) >> (8 * (i & 3))) & 0xFFu;
-      if constexpr (WF == WF_BFP8) {
-        E = max(E, 7u);
-        const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh) {
-          const uint32_t d = hh ? r.w.rows8[i].y : r.w.rows8[i].x;
-          const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
-          const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
-#pragma unroll
-          for (int b = 0; b < 4; ++b) f[h][hh * 4 + b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
-        }
-      } else {
-        E = max(E, 3u);
-        const float scale = __uint_as_float((E - 2u) << 23), nscale = -8.0f * scale;
-        const uint32_t d = r.w.rows4[i];
-        const uint32_t sg = d & 0x88888888u, sb = sg >> 3;
-        const uint32_t t = (d ^ 0x88888888u ^ (sg - sb)) + sb;
-#pragma unroll
-        for (int b = 0; b < 8; ++b) f[h][b] = fmaf((float)((t >> (4 * b)) & 0xFu), scale, nscale);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 8; ++j) out[j][q] = pack_hi(f[0][j], f[1][j]);
-  }
-}
-
-template <int WF>
-__device__ __forceinline__ void store_converted(const u32x4 (&out)[8], u32x4 *ldsW, int tid) {
-  if constexpr (WF != WF_BF16_NK) {
-    const int tile_l = tid >> 4, w = tid & 15;
-    const int face = w >> 2, khalf = (w >> 1) & 1, oct = w & 1;
-    const int kc = (tile_l >> 3) * 4 + (face >> 1) * 2 + khalf;
-    const int n0 = (tile_l & 7) * 32 + (face & 1) * 16 + oct * 8;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) ldsW[lds_chunk(n0 + j, kc)] = out[j];
-  }
-}
-
-template <int WF>
-__global__ __launch_bounds__(256) void ttm_linear_pipe_k(LinearArgs p) {
-  extern __shared__ u32x4 smem[];  // 2 stages x (A 2048 chunks + W 2048 chunks) = 128 KiB
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wn = wave & 1, wm = wave >> 1;
-  const int nblk = p.m_blocks * p.n_blocks;
-  int bid = blockIdx.x;
-  if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
-  const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
-  const int mt0 = mb * 8, nt0 = nb * 8;
-  const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
-  const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
-  uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
-
-  f32x16 acc[4][4];
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 4; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
-
-  const int ksteps = (p.Kt + 1) / 2;
-  u32x4 areg[8];        // activations of the next step (one set: stored to LDS at the top of a step)
-  WRegs<WF> r0, r1;     // raw weights of the next step / the step after
-  u32x4 out[8];
-  // fragment row offsets are loop invariant
-  int rowW[4], rowA[4];
-#pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    rowW[t] = wn * 128 + t * 32 + (lane & 31);
-    rowA[t] = wm * 128 + t * 32 + (lane & 31);
-  }
-
-  // prologue: step 0 into stage 0, raw data of step 1 into the registers
-  load_a_raw(p, A, mt0, 0, tid, areg);
-  load_w_raw<WF>(p, W, nt0, 0, tid, r0);
-#pragma unroll
-  for (int i = 0; i < 8; ++i) smem[copy_lds_chunk(tid, i)] = areg[i];
-#pragma unroll
-  for (int q = 0; q < 4; ++q) convert_quarter<WF>(q, r0, out, smem + 2048, tid);
-  store_converted<WF>(out, smem + 2048, tid);
-  load_a_raw(p, A, mt0, 2, tid, areg);
-  load_w_raw<WF>(p, W, nt0, 2, tid, r0);
-  __syncthreads();
-
-  auto step = [&](int ks, const WRegs<WF> &cur, WRegs<WF> &nxt) {
-    u32x4 *ldsA = smem + (ks & 1) * 4096, *ldsW = ldsA + 2048;
-    u32x4 *nxtA = smem + ((ks + 1) & 1) * 4096, *nxtW = nxtA + 2048;
-    // activations of step ks+1 arrived during the previous step: park them in the idle LDS stage, then
-    // reuse the registers for step ks+2
-#pragma unroll
-    for (int i = 0; i < 8; ++i) nxtA[copy_lds_chunk(tid, i)] = areg[i];
-    load_a_raw(p, A, mt0, (ks + 2) * 2, tid, areg);
-    load_w_raw<WF>(p, W, nt0, (ks + 2) * 2, tid, nxt);
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      bf16x8 wf[4], af[4];
-      const int kc = 2 * s + (lane >> 5);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        u32x4 a = ldsW[lds_chunk(rowW[t], kc)], b = ldsA[lds_chunk(rowA[t], kc)];
-        wf[t] = *(bf16x8 *)&a;
-        af[t] = *(bf16x8 *)&b;
-      }
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 4; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[a], af[b], acc[a][b], 0, 0, 0);
-      convert_quarter<WF>(s, cur, out, nxtW, tid);
-    }
-    store_converted<WF>(out, nxtW, tid);
-    __syncthreads();
-  };
-
-  for (int ks = 0; ks < ksteps; ks += 2) {
-    step(ks, r0, r1);
-    if (ks + 1 < ksteps) step(ks + 1, r1, r0);
-  }
-
-  switch (p.act) {
-  case TTM_ACT_GELU: linear_epilogue<TTM_ACT_GELU>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  case TTM_ACT_SILU: linear_epilogue<TTM_ACT_SILU>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  case TTM_ACT_SIGMOID: linear_epilogue<TTM_ACT_SIGMOID>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  case TTM_ACT_RELU: linear_epilogue<TTM_ACT_RELU>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  default: linear_epilogue<TTM_ACT_NONE>(p, C, acc, mt0 + wm * 4, nt0 + wn * 4, lane); break;
-  }
-}
-
-// =============================================================================================
-// Eight-wavefront variant of the large-M kernel: same 256 x 256 x 64 block and LDS image, but 512
-// lanes; a wavefront owns 128 (n) x 64 (m), so two wavefronts share every SIMD.  The two are run
-// out of phase -- wavefronts 0-3 multiply first and convert the next step's operands afterwards,
-// wavefronts 4-7 convert first and multiply afterwards -- so the dequantisation VALU work of one
-// overlaps the MFMAs of the other without any software pipelining.  One register set: the global
-// loads of step ks+2 are issued as soon as the registers of step ks+1 have been converted.
-// =============================================================================================
 template <int WF>
 struct W8Regs {  // raw weights of one k-step: an 8 (k) x 4 (n) block per lane (8 x 8 for bf16 [K,N])
   uint32_t rows8[WF == WF_BFP8 ? 8 : 1];
@@ -571,454 +356,25 @@ struct W8Regs {  // raw weights of one k-step: an 8 (k) x 4 (n) block per lane (
 // activation-style copy with 512 lanes: lane covers chunk (tid & 255) of the 4 KiB k-tile pair of row tile (tid >> 8) + 2 i
 __device__ __forceinline__ int copy8_lds_chunk(int tid, int i) { return copy_lds_chunk(tid & 255, (tid >> 8) + 2 * i); }
 
+// =============================================================================================
+// Main kernel, operands staged through registers (used for bf16 weights).  512 lanes = 8 wavefronts, each
+// owning a 128 (n) x 64 (m) piece of a 256 x 256 output block (128 accumulator registers per lane); k
+// advances 64 per step.  Per step a wavefront stores the activations it fetched one step earlier into LDS,
+// converts its 8 x 4 weight block into LDS, re-issues the global loads, and runs 24 ds_read_b128 + 32 MFMA
+// on the stage converted one step earlier, all in one instruction stream.
+// The issue port of a SIMD is shared by MFMA and VALU, which makes the number of VALU instructions per
+// step the second budget next to MFMA time.  Hence: every LDS address is a per-lane constant plus an
+// immediate (the step loop is unrolled by two so the stage is an immediate too), and every global address
+// is a wavefront-uniform base, advanced on the scalar unit, plus a per-lane 32-bit constant.
+// LDS: activations 2 x 32 KiB at 0, converted weights 2 x 32 KiB at 64 KiB.
+// =============================================================================================
 template <int WF>
-__global__ __launch_bounds__(512) void ttm_linear_w8_k(LinearArgs p) {
-  extern __shared__ u32x4 smem[];  // 2 stages x (A 2048 chunks + W 2048 chunks) = 128 KiB
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wn = wave & 1, wm = (wave >> 1) & 3;
-  const bool convert_first = (p.debug & 4) ? (wave & 1) : (wave >= 4);
-  const int nblk = p.m_blocks * p.n_blocks;
-  int bid = blockIdx.x;
-  if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
-  const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
-  const int mt0 = mb * 8, nt0 = nb * 8;
-  const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
-  const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
-  uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
-
-  f32x16 acc[4][2];
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
-
-  const int ksteps = (p.Kt + 1) / 2;
-  u32x4 areg[4];
-  W8Regs<WF> wreg;
-
-  // weight unit of this lane: tile (kt_l, nt_l) of the 2 x 8 tiles, face, 8-row half, 4-column quad
-  const int tile_l = tid >> 5, wq = tid & 31;
-  const int ukt = tile_l >> 3, unt = tile_l & 7;
-  const int face = wq >> 3, khalf = (wq >> 2) & 1, quad = wq & 3;
-
-  auto load_regs = [&](int kt0) {
-    const int ktA = min(kt0 + ((tid & 255) >> 7), p.Kt - 1);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int mt = min(mt0 + (tid >> 8) + 2 * i, p.Mt - 1);
-      areg[i] = *((const u32x4 *)(A + ((int64_t)mt * p.Kt + ktA) * 2048) + (tid & 127));
-    }
-    if constexpr (WF == WF_BF16_NK) {
-      const bool ok = kt0 + ((tid & 255) >> 7) < p.Kt;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int nt = min(nt0 + (tid >> 8) + 2 * i, p.Nt - 1);
-        u32x4 v = *((const u32x4 *)(W + ((int64_t)nt * p.Kt + ktA) * 2048) + (tid & 127));
-        wreg.direct[i] = ok ? v : u32x4{0, 0, 0, 0};
-      }
-    } else {
-      const bool ok = kt0 + ukt < p.Kt;
-      const int kt = min(kt0 + ukt, p.Kt - 1), nt = min(nt0 + unt, p.Nt - 1);
-      const int64_t tile = (int64_t)kt * p.Nt + nt;
-      if constexpr (WF == WF_BFP8) {
-        const uint8_t *t = W + tile * 1088;
-        wreg.exps = *(const u32x2 *)(t + face * 16 + khalf * 8);
-        const uint8_t *m = t + 64 + face * 256 + khalf * 128 + quad * 4;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          uint32_t v = *(const uint32_t *)(m + i * 16);
-          wreg.rows8[i] = ok ? v : 0u;
-        }
-      } else if constexpr (WF == WF_BFP4) {
-        const uint8_t *t = W + tile * 576;
-        wreg.exps = *(const u32x2 *)(t + face * 16 + khalf * 8);
-        const uint8_t *m = t + 64 + face * 128 + khalf * 64 + quad * 2;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          uint16_t v = *(const uint16_t *)(m + i * 8);
-          wreg.rows4[i] = ok ? v : (uint16_t)0;
-        }
-      } else {
-        const uint8_t *m = W + tile * 2048 + face * 512 + khalf * 256 + quad * 8;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          u32x2 v = *(const u32x2 *)(m + i * 32);
-          wreg.rows16[i] = ok ? v : u32x2{0, 0};
-        }
-      }
-    }
-  };
-
-  auto convert = [&](u32x4 *ldsA, u32x4 *ldsW) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) ldsA[copy8_lds_chunk(tid, i)] = areg[i];
-    if constexpr (WF == WF_BF16_NK) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) ldsW[copy8_lds_chunk(tid, i)] = wreg.direct[i];
-    } else {
-      u32x4 out[4];
-      if constexpr (WF == WF_BF16_KN) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) out[j][q] = __builtin_amdgcn_perm(wreg.rows16[2 * q + 1][j >> 1], wreg.rows16[2 * q][j >> 1], sel);
-        }
-      } else {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float f[2][4];
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const int i = 2 * q + h;
-            uint32_t E = ((i < 4 ? wreg.exps.x : wreg.exps.y) >> (8 * (i & 3))) & 0xFFu;
-            if constexpr (WF == WF_BFP8) {
-              E = max(E, 7u);
-              const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
-              const uint32_t d = wreg.rows8[i];
-              const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
-              const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
-#pragma unroll
-              for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
-            } else {
-              E = max(E, 3u);
-              const float scale = __uint_as_float((E - 2u) << 23), nscale = -8.0f * scale;
-              const uint32_t d = wreg.rows4[i];
-              const uint32_t sg = d & 0x8888u, sb = sg >> 3;
-              const uint32_t t = (d ^ 0x8888u ^ (sg - sb)) + sb;
-#pragma unroll
-              for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (4 * b)) & 0xFu), scale, nscale);
-            }
-          }
-#pragma unroll
-          for (int j = 0; j < 4; ++j) out[j][q] = pack_hi(f[0][j], f[1][j]);
-        }
-      }
-      const int kc = ukt * 4 + (face >> 1) * 2 + khalf;
-      const int n0 = unt * 32 + (face & 1) * 16 + quad * 4;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) ldsW[lds_chunk(n0 + j, kc)] = out[j];
-    }
-  };
-
-  auto multiply = [&](const u32x4 *ldsA, const u32x4 *ldsW) {
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      bf16x8 wf[4], af[2];
-      const int kc = 2 * s + (lane >> 5);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        u32x4 a = ldsW[lds_chunk(wn * 128 + t * 32 + (lane & 31), kc)];
-        wf[t] = *(bf16x8 *)&a;
-      }
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        u32x4 b = ldsA[lds_chunk(wm * 64 + t * 32 + (lane & 31), kc)];
-        af[t] = *(bf16x8 *)&b;
-      }
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[a], af[b], acc[a][b], 0, 0, 0);
-    }
-  };
-
-  load_regs(0);
-  convert(smem, smem + 2048);
-  load_regs(2);
-  __syncthreads();
-
-  for (int ks = 0; ks < ksteps; ++ks) {
-    u32x4 *ldsA = smem + (ks & 1) * 4096, *ldsW = ldsA + 2048;
-    u32x4 *nxtA = smem + ((ks + 1) & 1) * 4096, *nxtW = nxtA + 2048;
-    if (convert_first) {   // wavefront-uniform
-      if (!(p.debug & 1)) convert(nxtA, nxtW);
-      if (!(p.debug & 8)) load_regs((ks + 2) * 2);
-      if (!(p.debug & (2 | 16))) multiply(ldsA, ldsW);
-    } else {
-      if (!(p.debug & 2)) multiply(ldsA, ldsW);
-      if (!(p.debug & (1 | 16))) convert(nxtA, nxtW);
-      if (!(p.debug & (8 | 16))) load_regs((ks + 2) * 2);
-    }
-    __syncthreads();
-  }
-
-  // epilogue
-  const int m_in = lane & 31;
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const int nt = nt0 + wn * 4 + a;
-    if (nt >= p.Nt) continue;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int n_in = g * 8 + (lane >> 5) * 4;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (p.bias) {
-        const uint16_t *bp = p.bias_tiled ? p.bias + (int64_t)nt * 1024 + (n_in >> 4) * 256 + (n_in & 15) : p.bias + nt * 32 + n_in;
-        u32x2 raw = *(const u32x2 *)bp;
-        bv[0] = __uint_as_float(raw.x << 16); bv[1] = __uint_as_float(raw.x & 0xFFFF0000u);
-        bv[2] = __uint_as_float(raw.y << 16); bv[3] = __uint_as_float(raw.y & 0xFFFF0000u);
-      }
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int mt = mt0 + wm * 2 + b;
-        if (mt >= p.Mt) continue;
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float x = acc[a][b][g * 4 + r] + bv[r];
-          switch (p.act) {
-          case TTM_ACT_GELU: x = apply_act<TTM_ACT_GELU>(x); break;
-          case TTM_ACT_SILU: x = apply_act<TTM_ACT_SILU>(x); break;
-          case TTM_ACT_SIGMOID: x = apply_act<TTM_ACT_SIGMOID>(x); break;
-          case TTM_ACT_RELU: x = apply_act<TTM_ACT_RELU>(x); break;
-          default: break;
-          }
-          v[r] = x;
-        }
-        u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-        int64_t off = ((int64_t)mt * p.Nt + nt) * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
-        *(u32x2 *)(C + off * 2) = o;
-      }
-    }
-  }
-}
-
-// =============================================================================================
-// bfp8_b weights with staged raw tiles.  Loading a lane's 8 (k) x 4 (n) weight block straight from
-// global memory means eight 4-byte accesses at a 16-byte stride: the vector memory pipe then moves
-// 1 KiB per wavefront instruction as sixteen separate segments and becomes the limiter of the whole
-// kernel.  Here the mantissa bytes of the 16 weight tiles of a k-step are copied global -> LDS as
-// whole 16-byte face rows (1 KiB contiguous per wavefront instruction), two steps ahead, and the
-// 8 x 4 blocks are picked out of that raw image with ds_read_b32.  Row r = 8 a + i of a tile sits at
-// chunk 8 a + (i ^ a), so both the copy and the eight strided reads are bank-conflict free.
-// LDS: 2 x (activations 32 KiB + dequantised weights 32 KiB) + 2 x 16 KiB raw = 160 KiB.
-// Pipeline per step ks (one barrier): multiply(ks) | store A(ks+1), raw(ks+2); dequantise raw(ks+1);
-// issue global loads of A(ks+2), exponents(ks+2), raw(ks+3).
-// =============================================================================================
-__global__ __launch_bounds__(512) void ttm_linear_w8s_k(LinearArgs p) {
-  extern __shared__ u32x4 smem[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wn = wave & 1, wm = (wave >> 1) & 3;
-  const bool convert_first = wave >= 4;
-  const int nblk = p.m_blocks * p.n_blocks;
-  int bid = blockIdx.x;
-  if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
-  const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
-  const int mt0 = mb * 8, nt0 = nb * 8;
-  const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
-  const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
-  uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
-  uint8_t *lds8 = (uint8_t *)smem;
-  constexpr int RAW0 = 8192;  // chunk index of the first raw buffer; each holds 16 tiles x 64 chunks
-
-  f32x16 acc[4][2];
-#pragma unroll
-  for (int a = 0; a < 4; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.0f;
-
-  const int ksteps = (p.Kt + 1) / 2;
-  u32x4 areg[4], wraw[2];
-  u32x2 exps;
-
-  // weight unit of this lane (dequantisation): tile (ukt, unt), face, 8-row half, 4-column quad
-  const int tile_l = tid >> 5, wq = tid & 31;
-  const int ukt = tile_l >> 3, unt = tile_l & 7;
-  const int face = wq >> 3, khalf = (wq >> 2) & 1, quad = wq & 3;
-  const int ua = face * 2 + khalf;  // 8-row group inside the tile
-  // byte offset (inside a raw buffer) of row i = 0 of the lane's block; row i is at this ^ (i << 4)
-  const uint32_t raw_rd = tile_l * 1024 + ua * 128 + ua * 16 + quad * 4;
-  // raw copy: lane moves chunk (tid & 63) of tiles (tid >> 6) and (tid >> 6) + 8
-  const int cr = tid & 63, ca = cr >> 3;
-  const int raw_wr = (cr & ~7) | ((cr & 7) ^ ca);
-
-  auto load_a = [&](int kt0) {
-    const int ktA = min(kt0 + ((tid & 255) >> 7), p.Kt - 1);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int mt = min(mt0 + (tid >> 8) + 2 * i, p.Mt - 1);
-      areg[i] = *((const u32x4 *)(A + ((int64_t)mt * p.Kt + ktA) * 2048) + (tid & 127));
-    }
-  };
-  auto load_exps = [&](int kt0) {
-    const int kt = min(kt0 + ukt, p.Kt - 1), nt = min(nt0 + unt, p.Nt - 1);
-    exps = *(const u32x2 *)(W + ((int64_t)kt * p.Nt + nt) * 1088 + face * 16 + khalf * 8);
-  };
-  auto load_raw = [&](int kt0) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int tl = (tid >> 6) + 8 * h;              // tile (kt = h, nt = tid >> 6)
-      const bool ok = kt0 + h < p.Kt;
-      const int kt = min(kt0 + h, p.Kt - 1), nt = min(nt0 + (tl & 7), p.Nt - 1);
-      u32x4 v = *((const u32x4 *)(W + ((int64_t)kt * p.Nt + nt) * 1088 + 64) + cr);
-      wraw[h] = ok ? v : u32x4{0, 0, 0, 0};            // zero magnitudes: the k tail contributes nothing
-    }
-  };
-  auto store_a = [&](u32x4 *ldsA) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) ldsA[copy8_lds_chunk(tid, i)] = areg[i];
-  };
-  auto store_raw = [&](int buf) {
-#pragma unroll
-    for (int h = 0; h < 2; ++h) smem[RAW0 + buf * 1024 + ((tid >> 6) + 8 * h) * 64 + raw_wr] = wraw[h];
-  };
-  auto dequant = [&](int buf, u32x4 *ldsW) {
-    const uint8_t *raw = lds8 + (RAW0 + buf * 1024) * 16;
-    u32x4 out[4];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      float f[2][4];
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        const int i = 2 * q + h;
-        uint32_t E = ((i < 4 ? exps.x : exps.y) >> (8 * (i & 3))) & 0xFFu;
-        E = max(E, 7u);
-        const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
-        const uint32_t d = *(const uint32_t *)(raw + (raw_rd ^ (i << 4)));
-        const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
-        const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
-#pragma unroll
-        for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) out[j][q] = pack_hi(f[0][j], f[1][j]);
-    }
-    const int kc = ukt * 4 + (face >> 1) * 2 + khalf;
-    const int n0 = unt * 32 + (face & 1) * 16 + quad * 4;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) ldsW[lds_chunk(n0 + j, kc)] = out[j];
-  };
-  auto multiply = [&](const u32x4 *ldsA, const u32x4 *ldsW) {
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      bf16x8 wf[4], af[2];
-      const int kc = 2 * s + (lane >> 5);
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        u32x4 a = ldsW[lds_chunk(wn * 128 + t * 32 + (lane & 31), kc)];
-        wf[t] = *(bf16x8 *)&a;
-      }
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        u32x4 b = ldsA[lds_chunk(wm * 64 + t * 32 + (lane & 31), kc)];
-        af[t] = *(bf16x8 *)&b;
-      }
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[a], af[b], acc[a][b], 0, 0, 0);
-    }
-  };
-
-  // prologue: step 0 converted into stage 0, raw(1) in raw buffer 1, registers hold A(1), exps(1), raw(2)
-  load_a(0);
-  load_raw(0);
-  load_exps(0);
-  store_a(smem);
-  store_raw(0);
-  load_raw(2);
-  __syncthreads();
-  dequant(0, smem + 2048);
-  store_raw(1);
-  load_a(2);
-  load_exps(2);
-  load_raw(4);
-  __syncthreads();
-
-  for (int ks = 0; ks < ksteps; ++ks) {
-    u32x4 *ldsA = smem + (ks & 1) * 4096, *ldsW = ldsA + 2048;
-    u32x4 *nxtA = smem + ((ks + 1) & 1) * 4096, *nxtW = nxtA + 2048;
-    if (convert_first) {   // wavefront-uniform
-      store_a(nxtA);
-      store_raw(ks & 1);
-      dequant((ks + 1) & 1, nxtW);
-      load_a((ks + 2) * 2);
-      load_exps((ks + 2) * 2);
-      load_raw((ks + 3) * 2);
-      multiply(ldsA, ldsW);
-    } else {
-      multiply(ldsA, ldsW);
-      store_a(nxtA);
-      store_raw(ks & 1);
-      dequant((ks + 1) & 1, nxtW);
-      load_a((ks + 2) * 2);
-      load_exps((ks + 2) * 2);
-      load_raw((ks + 3) * 2);
-    }
-    __syncthreads();
-  }
-
-  const int m_in = lane & 31;
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const int nt = nt0 + wn * 4 + a;
-    if (nt >= p.Nt) continue;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int n_in = g * 8 + (lane >> 5) * 4;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (p.bias) {
-        const uint16_t *bp = p.bias_tiled ? p.bias + (int64_t)nt * 1024 + (n_in >> 4) * 256 + (n_in & 15) : p.bias + nt * 32 + n_in;
-        u32x2 raw = *(const u32x2 *)bp;
-        bv[0] = __uint_as_float(raw.x << 16); bv[1] = __uint_as_float(raw.x & 0xFFFF0000u);
-        bv[2] = __uint_as_float(raw.y << 16); bv[3] = __uint_as_float(raw.y & 0xFFFF0000u);
-      }
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int mt = mt0 + wm * 2 + b;
-        if (mt >= p.Mt) continue;
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float x = acc[a][b][g * 4 + r] + bv[r];
-          switch (p.act) {
-          case TTM_ACT_GELU: x = apply_act<TTM_ACT_GELU>(x); break;
-          case TTM_ACT_SILU: x = apply_act<TTM_ACT_SILU>(x); break;
-          case TTM_ACT_SIGMOID: x = apply_act<TTM_ACT_SIGMOID>(x); break;
-          case TTM_ACT_RELU: x = apply_act<TTM_ACT_RELU>(x); break;
-          default: break;
-          }
-          v[r] = x;
-        }
-        u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-        int64_t off = ((int64_t)mt * p.Nt + nt) * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
-        *(u32x2 *)(C + off * 2) = o;
-      }
-    }
-  }
-}
-
-// =============================================================================================
-// Main kernel.  512 lanes = 8 wavefronts, each owning a 128 (n) x 64 (m) piece of a 256 x 256 output
-// block (128 accumulator registers per lane); k advances 64 per step.  Per step a wavefront
-//   converts : stores the activations it fetched one step earlier into LDS, dequantises its 8 x 4
-//              weight block into LDS, then issues the global loads of the step after next;
-//   multiplies: 24 ds_read_b128 + 32 MFMA from the stage converted one step earlier.
-// Wavefronts 4..7 run their conversions one step further ahead than 0..3 and wait at the block barrier
-// between multiply and convert instead of after the convert: all wavefronts execute the same
-// instruction stream, but on every SIMD one wavefront feeds the matrix core while the other runs the
-// VALU / memory instructions.
-// The issue port of a SIMD is shared by MFMA and VALU, which makes the number of VALU instructions
-// per step the second budget next to MFMA time.  Hence: every LDS address is a per-lane constant plus
-// an immediate (the step loop is unrolled by two so the stage is an immediate too), and every global
-// address is a wavefront-uniform base, advanced on the scalar unit, plus a per-lane 32-bit constant.
-// LDS: activations 2 x 32 KiB at 0, dequantised weights 2 x 32 KiB at 64 KiB.
-// =============================================================================================
-template <int WF, bool FUSED>
-__global__ __launch_bounds__(512) void ttm_linear_main_k(LinearArgs p) {
+__global__ __launch_bounds__(512) void ttm_linear_reg_k(LinearArgs p) {
   extern __shared__ u32x4 smem[];
   uint8_t *lds = (uint8_t *)smem;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
-  const bool convert_first = !FUSED && wave >= 4;
   const int nblk = p.m_blocks * p.n_blocks;
   int bid = blockIdx.x;
   if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
@@ -1044,7 +400,7 @@ __global__ __launch_bounds__(512) void ttm_linear_main_k(LinearArgs p) {
     rdW[s] = LDS_W + 16u * lds_chunk(wn * 128 + (lane & 31), 2 * s + (lane >> 5));
     rdA[s] = 16u * lds_chunk(wm * 64 + (lane & 31), 2 * s + (lane >> 5));
   }
-  uint32_t wrA = 16u * copy8_lds_chunk(tid, 0);  // activation copy: + 8192 i; bit 15 selects the stage
+  const uint32_t wrA = 16u * copy8_lds_chunk(tid, 0);  // activation copy: + 8192 i + STAGE stage
   // weight unit of this lane: tile (ukt, unt) of the 2 x 8 tiles, face, 8-row half, 4-column quad
   const int ukt = wave >> 2, unt = (tid >> 5) & 7, wq = tid & 31;
   const int face = wq >> 3, khalf = (wq >> 2) & 1, quad = wq & 3;
@@ -1126,285 +482,142 @@ __global__ __launch_bounds__(512) void ttm_linear_main_k(LinearArgs p) {
     }
   };
 
-  if constexpr (FUSED) {
-    // ---- rotated pipeline: MFMA of one stage overlaps the conversion of the next, all in one instruction stream.
-    // A step is four chunks of 16 k.  Chunk q multiplies, requests the fragments of the following chunk,
-    // stores activation register c and converts weight rows 2c, 2c+1 with c = (q + 1) % 4, and re-issues the
-    // global loads of the registers it has just consumed (5 VALU instructions are scheduled behind every MFMA:
-    // that is what the matrix core leaves free on the issue port).  The block barrier sits between chunks 2
-    // and 3: chunk 3 multiplies from fragments that were requested before the barrier and already requests
-    // chunk 0 of the next stage, so the matrix core does not drain at the barrier; its conversion quarter
-    // (c = 0) already belongs to the step after next and goes into the stage that the barrier has just freed.
-    constexpr bool BFP = WF == WF_BFP8 || WF == WF_BFP4;
-    u32x4 fw[2][4], fa[2][2], out[4];
-    u32x2 exps_next = {0, 0};
-    auto bases = [&](int kt0, const uint8_t *&Ak, const uint8_t *&Wk, uint32_t &keep) {
-      const int ktA = min(kt0 + sub_kt, p.Kt - 1);
-      Ak = A + (int64_t)ktA * 2048;
-      const int ktW = WF == WF_BF16_NK ? ktA : min(kt0 + ukt, p.Kt - 1);
-      Wk = W + (int64_t)ktW * (WF == WF_BF16_NK ? 2048 : (int64_t)p.Nt * W_TILE);
-      keep = kt0 + (WF == WF_BF16_NK ? sub_kt : ukt) >= p.Kt ? 0u : 0xFFFFFFFFu;   // k tail: zero weights
-    };
-    auto fetch = [&](int s2, uint32_t so, u32x4 (&w)[4], u32x4 (&a)[2]) {
+  // ---- rotated pipeline: MFMA of one stage overlaps the conversion of the next, all in one instruction stream.
+  // A step is four chunks of 16 k.  Chunk q multiplies, requests the fragments of the following chunk,
+  // stores activation register c and converts weight rows 2c, 2c+1 with c = (q + 1) % 4, and re-issues the
+  // global loads of the registers it has just consumed (5 VALU instructions are scheduled behind every MFMA:
+  // that is what the matrix core leaves free on the issue port).  The block barrier sits between chunks 2
+  // and 3: chunk 3 multiplies from fragments that were requested before the barrier and already requests
+  // chunk 0 of the next stage, so the matrix core does not drain at the barrier; its conversion quarter
+  // (c = 0) already belongs to the step after next and goes into the stage that the barrier has just freed.
+  constexpr bool BFP = WF == WF_BFP8 || WF == WF_BFP4;
+  u32x4 fw[2][4], fa[2][2], out[4];
+  u32x2 exps_next = {0, 0};
+  auto bases = [&](int kt0, const uint8_t *&Ak, const uint8_t *&Wk, uint32_t &keep) {
+    const int ktA = min(kt0 + sub_kt, p.Kt - 1);
+    Ak = A + (int64_t)ktA * 2048;
+    const int ktW = WF == WF_BF16_NK ? ktA : min(kt0 + ukt, p.Kt - 1);
+    Wk = W + (int64_t)ktW * (WF == WF_BF16_NK ? 2048 : (int64_t)p.Nt * W_TILE);
+    keep = kt0 + (WF == WF_BF16_NK ? sub_kt : ukt) >= p.Kt ? 0u : 0xFFFFFFFFu;   // k tail: zero weights
+  };
+  auto fetch = [&](int s2, uint32_t so, u32x4 (&w)[4], u32x4 (&a)[2]) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) w[t] = *(const u32x4 *)(lds + rdW[s2] + t * 4096 + so);
+    for (int t = 0; t < 4; ++t) w[t] = *(const u32x4 *)(lds + rdW[s2] + t * 4096 + so);
 #pragma unroll
-      for (int t = 0; t < 2; ++t) a[t] = *(const u32x4 *)(lds + rdA[s2] + t * 4096 + so);
-    };
-    // conversion quarter c into the stage at byte offset so; afterwards reloads the consumed registers from (Ak, Wk)
-    auto quarter = [&](int c, uint32_t so, const uint8_t *Ak, const uint8_t *Wk, uint32_t keep) {
-      *(u32x4 *)(lds + wrA + c * 8192 + so) = areg[c];
-      areg[c] = *(const u32x4 *)(Ak + offA[c]);
-      if constexpr (WF == WF_BF16_NK) {
-        *(u32x4 *)(lds + wrA + LDS_W + c * 8192 + so) = wreg.direct[c];
-        u32x4 v = *(const u32x4 *)(Wk + offWd[c]);
-        wreg.direct[c] = u32x4{v.x & keep, v.y & keep, v.z & keep, v.w & keep};
-      } else if constexpr (WF == WF_BF16_KN) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
-          out[j][c] = __builtin_amdgcn_perm(wreg.rows16[2 * c + 1][j >> 1], wreg.rows16[2 * c][j >> 1], sel);
-        }
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          u32x2 v = *(const u32x2 *)(Wk + offWm + (2 * c + h) * 32);
-          wreg.rows16[2 * c + h] = u32x2{v.x & keep, v.y & keep};
-        }
-      } else {
-        float f[2][4];
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          const int i = 2 * c + h;
-          uint32_t E = ((i < 4 ? wreg.exps.x : wreg.exps.y) >> (8 * (i & 3))) & 0xFFu;
-          if constexpr (WF == WF_BFP8) {
-            E = max(E, 6u);   // rows below 2^-120, and the zeroed exponents of the k tail, dequantise to zero
-            const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
-            const uint32_t d = wreg.rows8[i];
-            const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
-            const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
-            wreg.rows8[i] = *(const uint32_t *)(Wk + offWm + i * 16);
-          } else {
-            E = max(E, 2u);
-            const float scale = __uint_as_float((E - 2u) << 23), nscale = -8.0f * scale;
-            const uint32_t d = wreg.rows4[i];
-            const uint32_t sg = d & 0x8888u, sb = sg >> 3;
-            const uint32_t t = (d ^ 0x8888u ^ (sg - sb)) + sb;
-#pragma unroll
-            for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (4 * b)) & 0xFu), scale, nscale);
-            wreg.rows4[i] = *(const uint16_t *)(Wk + offWm + i * 8);
-          }
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j) out[j][c] = pack_hi(f[0][j], f[1][j]);
-      }
-      if (c == 3 && WF != WF_BF16_NK) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) *(u32x4 *)(lds + wrW[j] + so) = out[j];
-      }
-    };
-    auto mfma8 = [&](int buf) {
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&fw[buf][a], *(bf16x8 *)&fa[buf][b], acc[a][b], 0, 0, 0);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
-      }
-    };
-
-    const uint8_t *Ak, *Wk;
-    uint32_t keep;
-    // prologue: step 0 into stage 0, first quarter of step 1 into stage 1, registers refilled behind each use
-    load_regs(0);
-    bases(2, Ak, Wk, keep);
-#pragma unroll
-    for (int c = 0; c < 4; ++c) quarter(c, 0, Ak, Wk, keep);
-    if constexpr (BFP) {
-      u32x2 e = *(const u32x2 *)(Wk + offWe);
-      wreg.exps = u32x2{e.x & keep, e.y & keep};
-    }
-    __syncthreads();
-    fetch(0, 0, fw[0], fa[0]);
-    bases(4, Ak, Wk, keep);
-    quarter(0, STAGE, Ak, Wk, keep);
-
-    auto step = [&](auto stage_c, int ks) {
-      constexpr uint32_t CUR = decltype(stage_c)::value * STAGE, NXT = STAGE - CUR;
-      bases((ks + 2) * 2, Ak, Wk, keep);
-#pragma unroll
-      for (int q = 0; q < 3; ++q) {
-        fetch(q + 1, CUR, fw[(q + 1) & 1], fa[(q + 1) & 1]);
-        quarter(q + 1, NXT, Ak, Wk, keep);
-        if (q == 0 && BFP) {
-          u32x2 e = *(const u32x2 *)(Wk + offWe);
-          exps_next = u32x2{e.x & keep, e.y & keep};
-        }
-        mfma8(q & 1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if constexpr (BFP) wreg.exps = exps_next;
-      __syncthreads();
-      bases((ks + 3) * 2, Ak, Wk, keep);
-      fetch(0, NXT, fw[0], fa[0]);
-      quarter(0, CUR, Ak, Wk, keep);
-      mfma8(1);
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    // an odd number of steps is rounded up: the extra step multiplies zeroed weights
-    for (int ks = 0; ks < ksteps; ks += 2) {
-      step(std::integral_constant<int, 0>{}, ks);
-      step(std::integral_constant<int, 1>{}, ks + 1);
-    }
-  } else {
-  // stores into the stage that the write addresses currently point at, then flips them to the other stage
-  auto convert = [&]() {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *(u32x4 *)(lds + wrA + i * 8192) = areg[i];
+    for (int t = 0; t < 2; ++t) a[t] = *(const u32x4 *)(lds + rdA[s2] + t * 4096 + so);
+  };
+  // conversion quarter c into the stage at byte offset so; afterwards reloads the consumed registers from (Ak, Wk)
+  auto quarter = [&](int c, uint32_t so, const uint8_t *Ak, const uint8_t *Wk, uint32_t keep) {
+    *(u32x4 *)(lds + wrA + c * 8192 + so) = areg[c];
+    areg[c] = *(const u32x4 *)(Ak + offA[c]);
     if constexpr (WF == WF_BF16_NK) {
+      *(u32x4 *)(lds + wrA + LDS_W + c * 8192 + so) = wreg.direct[c];
+      u32x4 v = *(const u32x4 *)(Wk + offWd[c]);
+      wreg.direct[c] = u32x4{v.x & keep, v.y & keep, v.z & keep, v.w & keep};
+    } else if constexpr (WF == WF_BF16_KN) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) *(u32x4 *)(lds + wrA + LDS_W + i * 8192) = wreg.direct[i];
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+        out[j][c] = __builtin_amdgcn_perm(wreg.rows16[2 * c + 1][j >> 1], wreg.rows16[2 * c][j >> 1], sel);
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        u32x2 v = *(const u32x2 *)(Wk + offWm + (2 * c + h) * 32);
+        wreg.rows16[2 * c + h] = u32x2{v.x & keep, v.y & keep};
+      }
     } else {
-      u32x4 out[4];
-      if constexpr (WF == WF_BF16_KN) {
+      float f[2][4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const uint32_t sel = (j & 1) ? 0x07060302u : 0x05040100u;
+      for (int h = 0; h < 2; ++h) {
+        const int i = 2 * c + h;
+        uint32_t E = ((i < 4 ? wreg.exps.x : wreg.exps.y) >> (8 * (i & 3))) & 0xFFu;
+        if constexpr (WF == WF_BFP8) {
+          E = max(E, 6u);   // rows below 2^-120, and the zeroed exponents of the k tail, dequantise to zero
+          const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
+          const uint32_t d = wreg.rows8[i];
+          const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
+          const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
 #pragma unroll
-          for (int q = 0; q < 4; ++q) out[j][q] = __builtin_amdgcn_perm(wreg.rows16[2 * q + 1][j >> 1], wreg.rows16[2 * q][j >> 1], sel);
-        }
-      } else {
+          for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
+          wreg.rows8[i] = *(const uint32_t *)(Wk + offWm + i * 16);
+        } else {
+          E = max(E, 2u);
+          const float scale = __uint_as_float((E - 2u) << 23), nscale = -8.0f * scale;
+          const uint32_t d = wreg.rows4[i];
+          const uint32_t sg = d & 0x8888u, sb = sg >> 3;
+          const uint32_t t = (d ^ 0x8888u ^ (sg - sb)) + sb;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          float f[2][4];
-#pragma unroll
-          for (int h = 0; h < 2; ++h) {
-            const int i = 2 * q + h;
-            uint32_t E = ((i < 4 ? wreg.exps.x : wreg.exps.y) >> (8 * (i & 3))) & 0xFFu;
-            if constexpr (WF == WF_BFP8) {
-              E = max(E, 6u);   // rows below 2^-120 dequantise to zero
-              const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
-              const uint32_t d = wreg.rows8[i];
-              const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
-              const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
-#pragma unroll
-              for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
-            } else {
-              E = max(E, 2u);
-              const float scale = __uint_as_float((E - 2u) << 23), nscale = -8.0f * scale;
-              const uint32_t d = wreg.rows4[i];
-              const uint32_t sg = d & 0x8888u, sb = sg >> 3;
-              const uint32_t t = (d ^ 0x8888u ^ (sg - sb)) + sb;
-#pragma unroll
-              for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (4 * b)) & 0xFu), scale, nscale);
-            }
-          }
-#pragma unroll
-          for (int j = 0; j < 4; ++j) out[j][q] = pack_hi(f[0][j], f[1][j]);
+          for (int b = 0; b < 4; ++b) f[h][b] = fmaf((float)((t >> (4 * b)) & 0xFu), scale, nscale);
+          wreg.rows4[i] = *(const uint16_t *)(Wk + offWm + i * 8);
         }
       }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) *(u32x4 *)(lds + wrW[j]) = out[j];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) wrW[j] ^= STAGE;
+      for (int j = 0; j < 4; ++j) out[j][c] = pack_hi(f[0][j], f[1][j]);
     }
-    wrA ^= STAGE;
+    if (c == 3 && WF != WF_BF16_NK) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) *(u32x4 *)(lds + wrW[j] + so) = out[j];
+    }
   };
-
-  auto multiply = [&](auto stage_c) {
-    constexpr uint32_t SO = decltype(stage_c)::value * STAGE;
-    // fragments of k-chunk s + 1 are requested before the MFMAs of chunk s are issued
-    u32x4 fw[2][4], fa[2][2];
-    auto fetch = [&](int s, u32x4 (&w)[4], u32x4 (&a)[2]) {
+  auto mfma8 = [&](int buf) {
 #pragma unroll
-      for (int t = 0; t < 4; ++t) w[t] = *(const u32x4 *)(lds + rdW[s] + t * 4096 + SO);
+    for (int a = 0; a < 4; ++a)
 #pragma unroll
-      for (int t = 0; t < 2; ++t) a[t] = *(const u32x4 *)(lds + rdA[s] + t * 4096 + SO);
-    };
-    fetch(0, fw[0], fa[0]);
+      for (int b = 0; b < 2; ++b)
+        acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&fw[buf][a], *(bf16x8 *)&fa[buf][b], acc[a][b], 0, 0, 0);
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      if (s < 3) fetch(s + 1, fw[(s + 1) & 1], fa[(s + 1) & 1]);
-      if (!FUSED) __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int a = 0; a < 4; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&fw[s & 1][a], *(bf16x8 *)&fa[s & 1][b], acc[a][b], 0, 0, 0);
-      if (!FUSED) __builtin_amdgcn_sched_barrier(0);
+    for (int i = 0; i < 8; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
     }
   };
 
-  // prologue: step 0 converted by everybody; the early group also converts step 1
+  const uint8_t *Ak, *Wk;
+  uint32_t keep;
+  // prologue: step 0 into stage 0, first quarter of step 1 into stage 1, registers refilled behind each use
   load_regs(0);
-  convert();
-  load_regs(2);
-  __syncthreads();
-  const int ahead = convert_first ? 1 : 0;
-  if (convert_first) {
-    convert();
-    load_regs(4);
+  bases(2, Ak, Wk, keep);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) quarter(c, 0, Ak, Wk, keep);
+  if constexpr (BFP) {
+    u32x2 e = *(const u32x2 *)(Wk + offWe);
+    wreg.exps = u32x2{e.x & keep, e.y & keep};
   }
+  __syncthreads();
+  fetch(0, 0, fw[0], fa[0]);
+  bases(4, Ak, Wk, keep);
+  quarter(0, STAGE, Ak, Wk, keep);
 
   auto step = [&](auto stage_c, int ks) {
-    multiply(stage_c);
-    if (convert_first) __syncthreads();
-    convert();
-    load_regs((ks + 2 + ahead) * 2);
-    if (!convert_first) __syncthreads();
+    constexpr uint32_t CUR = decltype(stage_c)::value * STAGE, NXT = STAGE - CUR;
+    bases((ks + 2) * 2, Ak, Wk, keep);
+#pragma unroll
+    for (int q = 0; q < 3; ++q) {
+      fetch(q + 1, CUR, fw[(q + 1) & 1], fa[(q + 1) & 1]);
+      quarter(q + 1, NXT, Ak, Wk, keep);
+      if (q == 0 && BFP) {
+        u32x2 e = *(const u32x2 *)(Wk + offWe);
+        exps_next = u32x2{e.x & keep, e.y & keep};
+      }
+      mfma8(q & 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (BFP) wreg.exps = exps_next;
+    __syncthreads();
+    bases((ks + 3) * 2, Ak, Wk, keep);
+    fetch(0, NXT, fw[0], fa[0]);
+    quarter(0, CUR, Ak, Wk, keep);
+    mfma8(1);
+    __builtin_amdgcn_sched_barrier(0);
   };
   // an odd number of steps is rounded up: the extra step multiplies zeroed weights
   for (int ks = 0; ks < ksteps; ks += 2) {
     step(std::integral_constant<int, 0>{}, ks);
     step(std::integral_constant<int, 1>{}, ks + 1);
   }
-
-  }
-
-  // epilogue: bias, activation, bf16, 8-byte stores into the output face rows
-  const int m_in = lane & 31;
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    const int nt = nt0 + wn * 4 + a;
-    if (nt >= p.Nt) continue;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int n_in = g * 8 + (lane >> 5) * 4;
-      float bv[4] = {0.f, 0.f, 0.f, 0.f};
-      if (p.bias) {
-        const uint16_t *bp = p.bias_tiled ? p.bias + (int64_t)nt * 1024 + (n_in >> 4) * 256 + (n_in & 15) : p.bias + nt * 32 + n_in;
-        u32x2 raw = *(const u32x2 *)bp;
-        bv[0] = __uint_as_float(raw.x << 16); bv[1] = __uint_as_float(raw.x & 0xFFFF0000u);
-        bv[2] = __uint_as_float(raw.y << 16); bv[3] = __uint_as_float(raw.y & 0xFFFF0000u);
-      }
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int mt = mt0 + wm * 2 + b;
-        if (mt >= p.Mt) continue;
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float x = acc[a][b][g * 4 + r] + bv[r];
-          switch (p.act) {
-          case TTM_ACT_GELU: x = apply_act<TTM_ACT_GELU>(x); break;
-          case TTM_ACT_SILU: x = apply_act<TTM_ACT_SILU>(x); break;
-          case TTM_ACT_SIGMOID: x = apply_act<TTM_ACT_SIGMOID>(x); break;
-          case TTM_ACT_RELU: x = apply_act<TTM_ACT_RELU>(x); break;
-          default: break;
-          }
-          v[r] = x;
-        }
-        u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-        int64_t off = ((int64_t)mt * p.Nt + nt) * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
-        *(u32x2 *)(C + off * 2) = o;
-      }
-    }
-  }
+  linear_epilogue_act(p, C, acc, mt0 + wm * 2, nt0 + wn * 4, p.Nt, lane);
 }
+
 
 // =============================================================================================
 // Block-float main kernel with LDS-direct global loads.  Same tiling and the same rotated pipeline as
@@ -1427,25 +640,22 @@ __device__ __forceinline__ void lds_dma16(const void *base, uint32_t lane_off, u
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
 }
 
-template <int WF, int NWAVE>
-__global__ __launch_bounds__(NWAVE * 64) void ttm_linear_dma_k(LinearArgs p) {
+// One output block of 2 NTW x 8 tiles (NTW = 4, 3 or 2 column tiles per wavefront); bid / nblk number the blocks of
+// the column range [nt_first, nt_end) that this body covers.
+template <int WF, int NTW>
+__device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, int nblk, int nt_first, int nt_end) {
   static_assert(WF == WF_BFP8 || WF == WF_BFP4, "block-float weights only");
-  static_assert(NWAVE == 8 || NWAVE == 4, "8 wavefronts of 128 x 64 or 4 wavefronts of 128 x 128");
-  constexpr int T = NWAVE * 64;
-  constexpr int MB = 16 / NWAVE;       // row tiles (32 m) per wavefront
-  constexpr int NU = 512 / T;          // 8 x 4 weight blocks per lane and step
-  constexpr int TPW = 16 / NWAVE;      // weight tiles staged per wavefront and step
+  constexpr int MB = 2;          // row tiles (32 m) per wavefront
+  constexpr int BN = 2 * NTW;    // column tiles per block
   extern __shared__ u32x4 smem[];
   uint8_t *lds = (uint8_t *)smem;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;   // LDS byte address of the image
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wn = wave & 1, wm = wave >> 1;
-  const int nblk = p.m_blocks * p.n_blocks;
-  int bid = blockIdx.x;
-  if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
+  if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);   // consecutive blocks of one XCD share weight columns
   const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
-  const int mt0 = mb * 8, nt0 = nb * 8;
+  const int mt0 = mb * 8, nt0 = nt_first + nb * BN;
   const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
   const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
   uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
@@ -1453,9 +663,9 @@ __global__ __launch_bounds__(NWAVE * 64) void ttm_linear_dma_k(LinearArgs p) {
   constexpr uint32_t RAW_TILE = WF == WF_BFP8 ? 1024u : 512u, RAW_STAGE = 16 * RAW_TILE;
   constexpr uint32_t W_TILE = WF == WF_BFP8 ? 1088u : 576u;
 
-  f32x16 acc[4][MB];
+  f32x16 acc[NTW][MB];
 #pragma unroll
-  for (int a = 0; a < 4; ++a)
+  for (int a = 0; a < NTW; ++a)
 #pragma unroll
     for (int b = 0; b < MB; ++b)
 #pragma unroll
@@ -1465,23 +675,23 @@ __global__ __launch_bounds__(NWAVE * 64) void ttm_linear_dma_k(LinearArgs p) {
   uint32_t rdW[4], rdA[4];   // fragment reads: + 4096 t + STAGE stage
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
-    rdW[s] = LDS_W + 16u * lds_chunk(wn * 128 + (lane & 31), 2 * s + (lane >> 5));
+    rdW[s] = LDS_W + 16u * lds_chunk(wn * (32 * NTW) + (lane & 31), 2 * s + (lane >> 5));
     rdA[s] = 16u * lds_chunk(wm * (32 * MB) + (lane & 31), 2 * s + (lane >> 5));
   }
-  // weight blocks of this lane: block h lives in tile slot (tid >> 5) + (T / 32) h of the 2 x 8 tiles of a step
-  // (slot = 8 * k-tile + column tile); inside the tile: face, 8-row half, 4-column quad
-  const int unt = (tid >> 5) & 7, wq = tid & 31;
+  // weight block of this lane: tile slot tid >> 5 of the 2 x 8 tiles of a step (slot = 8 * k-tile + column tile);
+  // inside the tile: face, 8-row half, 4-column quad.  A wavefront owns two neighbouring column tiles of one
+  // k-tile; with fewer than 8 column tiles per block the wavefronts of the unused slots skip the conversion.
+  const int ukt = wave >> 2, unt = (tid >> 5) & 7, wq = tid & 31;
+  const bool converts = 2 * (wave & 3) < BN;   // wavefront-uniform
   const int face = wq >> 3, khalf = (wq >> 2) & 1, quad = wq & 3;
-  auto unit_kt = [&](int h) { return NWAVE == 8 ? wave >> 2 : h; };   // wavefront-uniform
-  uint32_t wrW[NU][4];
-#pragma unroll
-  for (int h = 0; h < NU; ++h) {
-    const int kc = unit_kt(h) * 4 + (face >> 1) * 2 + khalf;
+  uint32_t wrW[4];
+  {
+    const int kc = ukt * 4 + (face >> 1) * 2 + khalf;
     const int n0 = unt * 32 + (face & 1) * 16 + quad * 4;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) wrW[h][j] = LDS_W + 16u * lds_chunk(n0 + j, kc);
+    for (int j = 0; j < 4; ++j) wrW[j] = LDS_W + 16u * lds_chunk(n0 + j, kc);
   }
-  // raw staging reads of block 0: row i at rawRd ^ (16 i) (bfp8) or rawRd + 8 i (bfp4); block 1 is 8 tiles further
+  // raw staging reads: row i of the block at rawRd ^ (16 i) (bfp8) or rawRd + 8 i (bfp4)
   uint32_t rawRd;
   {
     const int tile_l = tid >> 5, a = face * 2 + khalf;
@@ -1489,129 +699,109 @@ __global__ __launch_bounds__(NWAVE * 64) void ttm_linear_dma_k(LinearArgs p) {
     else rawRd = LDS_RAW + tile_l * 512 + a * 64 + quad * 2;
   }
   const uint32_t offWe = (uint32_t)min(nt0 + unt, p.Nt - 1) * W_TILE + face * 16 + khalf * 8;
-  // LDS-direct loads of the activations: wavefront w fills rows (256 / NWAVE) w .. with instructions of 8 rows each;
-  // lane l writes slot l & 7 of row 8 i + (l >> 3), i.e. k-chunk slot ^ swizzle(row) (which only looks at row % 32)
+  // LDS-direct loads of the activations: wavefront w fills rows 32 w .. 32 w + 31 (row tile mt0 + w) with four
+  // instructions of 8 rows each; lane l writes slot l & 7 of row 8 i + (l >> 3), i.e. k-chunk slot ^ swizzle(row)
   uint32_t dmaA[4];
   bool dmaA_sub[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r32 = 8 * i + (lane >> 3);
-    const int kc = (lane & 7) ^ lds_swz(r32);
+    const int kc = (lane & 7) ^ lds_swz(r32);   // the swizzle only looks at the low five row bits
     dmaA[i] = (uint32_t)(((r32 >> 4) * 2 + ((kc & 3) >> 1)) * 512 + (r32 & 15) * 32 + (kc & 1) * 16);
     dmaA_sub[i] = (kc >> 2) != 0;
   }
-  int64_t a_row[MB / 2];
-#pragma unroll
-  for (int x = 0; x < MB / 2; ++x) a_row[x] = (int64_t)min(mt0 + wave * (MB / 2) + x, p.Mt - 1) * p.Kt * 2048;
-  // mantissas: the wavefront stages tile slots TPW w .. TPW w + TPW - 1
-  uint32_t dmaW;   // lane offset inside the tile (bfp8), inside the k-tile row (bfp4: two tiles per instruction)
-  int64_t w_col[TPW];
+  const int64_t a_row = (int64_t)min(mt0 + wave, p.Mt - 1) * p.Kt * 2048;
+  // mantissas: the wavefront stages its two tile slots 2 w, 2 w + 1
+  uint32_t dmaW;   // bfp8: lane offset inside the tile; bfp4: inside the k-tile row (one instruction, two tiles)
+  int64_t w_col[2] = {0, 0};
   if constexpr (WF == WF_BFP8) {
     const int a = lane >> 3;
     dmaW = 64u + (uint32_t)(8 * a + ((lane & 7) ^ a)) * 16u;   // tile parity is folded in at the call site (XOR 16)
 #pragma unroll
-    for (int x = 0; x < TPW; ++x) w_col[x] = (int64_t)min(nt0 + ((wave * TPW + x) & 7), p.Nt - 1) * W_TILE;
+    for (int x = 0; x < 2; ++x) w_col[x] = (int64_t)min(nt0 + 2 * (wave & 3) + x, p.Nt - 1) * W_TILE;
   } else {
-    dmaW = 64u + (uint32_t)(lane & 31) * 16u;
-#pragma unroll
-    for (int x = 0; x < TPW; ++x) w_col[x] = 0;
-  }
-  uint32_t dmaW4[TPW / 2];   // bfp4: lanes 0..31 fetch tile slot 2 y, lanes 32..63 slot 2 y + 1
-  if constexpr (WF == WF_BFP4) {
-#pragma unroll
-    for (int y = 0; y < TPW / 2; ++y)
-      dmaW4[y] = (uint32_t)(min(nt0 + ((wave * TPW + 2 * y + (lane >> 5)) & 7), p.Nt - 1) * (int)W_TILE) + dmaW;
+    dmaW = (uint32_t)(min(nt0 + 2 * (wave & 3) + (lane >> 5), p.Nt - 1) * (int)W_TILE) + 64u + (uint32_t)(lane & 31) * 16u;
   }
 
   const int ksteps = (p.Kt + 1) / 2;
-  u32x2 exps[NU], exps_next[NU];
-  u32x4 fw[2][4], fa[2][MB], out[NU][4];
+  u32x2 exps = {0, 0}, exps_next = {0, 0};
+  u32x4 fw[2][NTW], fa[2][MB], out[4];
 
   auto issue_a = [&](int kt0, uint32_t stage_off) {
     const int kt = min(kt0, p.Kt - 1);
     const uint32_t sub = kt0 + 1 < p.Kt ? 2048u : 0u;   // k tail: the second tile of the pair repeats the first (its weights are zero)
+    const uint8_t *base = A + a_row + (int64_t)kt * 2048;
 #pragma unroll
-    for (int i = 0; i < 2 * MB; ++i)
-      lds_dma16(A + a_row[i >> 2] + (int64_t)kt * 2048, dmaA[i & 3] + (dmaA_sub[i & 3] ? sub : 0u),
-                lds0 + stage_off + (uint32_t)(wave * (2048 / NWAVE) + i * 64) * 16u);
+    for (int i = 0; i < 4; ++i)
+      lds_dma16(base, dmaA[i] + (dmaA_sub[i] ? sub : 0u), lds0 + stage_off + (uint32_t)(wave * 256 + i * 64) * 16u);
   };
   auto issue_raw = [&](int kt0, uint32_t stage_off) {
+    if (!converts) return;
+    const int kt = min(kt0 + ukt, p.Kt - 1);
+    const uint8_t *row = W + (int64_t)kt * p.Nt * W_TILE;
     if constexpr (WF == WF_BFP8) {
 #pragma unroll
-      for (int x = 0; x < TPW; ++x) {
-        const int slot = wave * TPW + x;
-        const int kt = min(kt0 + (slot >> 3), p.Kt - 1);
-        lds_dma16(W + (int64_t)kt * p.Nt * W_TILE + w_col[x], dmaW ^ ((x & 1) << 4), lds0 + LDS_RAW + stage_off + (uint32_t)slot * 1024u);
-      }
+      for (int x = 0; x < 2; ++x)
+        lds_dma16(row + w_col[x], dmaW ^ (x << 4), lds0 + LDS_RAW + stage_off + (uint32_t)(2 * wave + x) * 1024u);
     } else {
-#pragma unroll
-      for (int y = 0; y < TPW / 2; ++y) {
-        const int slot = wave * TPW + 2 * y;
-        const int kt = min(kt0 + (slot >> 3), p.Kt - 1);
-        lds_dma16(W + (int64_t)kt * p.Nt * W_TILE, dmaW4[y], lds0 + LDS_RAW + stage_off + (uint32_t)slot * 512u);
-      }
+      lds_dma16(row, dmaW, lds0 + LDS_RAW + stage_off + (uint32_t)(2 * wave) * 512u);
     }
   };
-  auto load_exps = [&](int kt0, u32x2 (&e)[NU]) {
-#pragma unroll
-    for (int h = 0; h < NU; ++h) {
-      const int kt = min(kt0 + unit_kt(h), p.Kt - 1);
-      const uint32_t keep = kt0 + unit_kt(h) >= p.Kt ? 0u : 0xFFFFFFFFu;   // k tail: zero exponents dequantise to zero weights
-      u32x2 v = *(const u32x2 *)(W + (int64_t)kt * p.Nt * W_TILE + offWe);
-      e[h] = u32x2{v.x & keep, v.y & keep};
-    }
+  auto load_exps = [&](int kt0) {
+    const int kt = min(kt0 + ukt, p.Kt - 1);
+    const uint32_t keep = kt0 + ukt >= p.Kt ? 0u : 0xFFFFFFFFu;   // k tail: zero exponents dequantise to zero weights
+    u32x2 e = *(const u32x2 *)(W + (int64_t)kt * p.Nt * W_TILE + offWe);
+    return u32x2{e.x & keep, e.y & keep};
   };
-  auto fetch = [&](int s2, uint32_t so, u32x4 (&w)[4], u32x4 (&a)[MB]) {
+  auto fetch = [&](int s2, uint32_t so, u32x4 (&w)[NTW], u32x4 (&a)[MB]) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) w[t] = *(const u32x4 *)(lds + rdW[s2] + t * 4096 + so);
+    for (int t = 0; t < NTW; ++t) w[t] = *(const u32x4 *)(lds + rdW[s2] + t * 4096 + so);
 #pragma unroll
     for (int t = 0; t < MB; ++t) a[t] = *(const u32x4 *)(lds + rdA[s2] + t * 4096 + so);
   };
-  // conversion quarter c: rows 2c, 2c+1 of the lane's blocks from the raw stage at raw_off; c == 3 stores the blocks
+  // conversion quarter c: rows 2c, 2c+1 of the lane's block from the raw stage at raw_off; c == 3 stores the block
   auto quarter = [&](int c, uint32_t raw_off, uint32_t w_off) {
+    if (!converts) return;
+    float f[2][4];
 #pragma unroll
-    for (int h = 0; h < NU; ++h) {
-      float f[2][4];
+    for (int r = 0; r < 2; ++r) {
+      const int i = 2 * c + r;
+      uint32_t E = ((i < 4 ? exps.x : exps.y) >> (8 * (i & 3))) & 0xFFu;
+      if constexpr (WF == WF_BFP8) {
+        E = max(E, 6u);   // rows below 2^-120, and the zeroed exponents of the k tail, dequantise to zero
+        const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
+        const uint32_t d = *(const uint32_t *)(lds + (rawRd ^ (i << 4)) + raw_off);
+        const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
+        const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;   // per byte: 128 + mag or 128 - mag
 #pragma unroll
-      for (int r = 0; r < 2; ++r) {
-        const int i = 2 * c + r;
-        uint32_t E = ((i < 4 ? exps[h].x : exps[h].y) >> (8 * (i & 3))) & 0xFFu;
-        if constexpr (WF == WF_BFP8) {
-          E = max(E, 6u);   // rows below 2^-120, and the zeroed exponents of the k tail, dequantise to zero
-          const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
-          const uint32_t d = *(const uint32_t *)(lds + (rawRd ^ (i << 4)) + h * (T / 32) * RAW_TILE + raw_off);
-          const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
-          const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
+        for (int b = 0; b < 4; ++b) f[r][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
+      } else {
+        E = max(E, 2u);
+        const float scale = __uint_as_float((E - 2u) << 23), nscale = -8.0f * scale;
+        const uint32_t d = *(const uint16_t *)(lds + rawRd + i * 8 + raw_off);
+        const uint32_t sg = d & 0x8888u, sb = sg >> 3;
+        const uint32_t t = (d ^ 0x8888u ^ (sg - sb)) + sb;       // per nibble: 8 + mag or 8 - mag
 #pragma unroll
-          for (int b = 0; b < 4; ++b) f[r][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
-        } else {
-          E = max(E, 2u);
-          const float scale = __uint_as_float((E - 2u) << 23), nscale = -8.0f * scale;
-          const uint32_t d = *(const uint16_t *)(lds + rawRd + i * 8 + h * (T / 32) * RAW_TILE + raw_off);
-          const uint32_t sg = d & 0x8888u, sb = sg >> 3;
-          const uint32_t t = (d ^ 0x8888u ^ (sg - sb)) + sb;
-#pragma unroll
-          for (int b = 0; b < 4; ++b) f[r][b] = fmaf((float)((t >> (4 * b)) & 0xFu), scale, nscale);
-        }
+        for (int b = 0; b < 4; ++b) f[r][b] = fmaf((float)((t >> (4 * b)) & 0xFu), scale, nscale);
       }
+    }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) out[h][j][c] = pack_hi(f[0][j], f[1][j]);
-      if (c == 3) {
+    for (int j = 0; j < 4; ++j) out[j][c] = pack_hi(f[0][j], f[1][j]);
+    if (c == 3) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) *(u32x4 *)(lds + wrW[h][j] + w_off) = out[h][j];
-      }
+      for (int j = 0; j < 4; ++j) *(u32x4 *)(lds + wrW[j] + w_off) = out[j];
     }
   };
   auto mfma_chunk = [&](int buf) {
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < NTW; ++a)
 #pragma unroll
       for (int b = 0; b < MB; ++b)
         acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&fw[buf][a], *(bf16x8 *)&fa[buf][b], acc[a][b], 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < 4 * MB; ++i) {
+    for (int i = 0; i < NTW * MB; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 40 / (NTW * MB), 0);
     }
   };
   auto landed_barrier = [&]() {
@@ -1619,22 +809,28 @@ __global__ __launch_bounds__(NWAVE * 64) void ttm_linear_dma_k(LinearArgs p) {
     __syncthreads();
   };
 
-  // ---- prologue
+  // ---- prologue: step 0 staged and converted, step 1 staged and its first quarter converted
   issue_a(0, 0);
   issue_raw(0, 0);
   issue_raw(2, RAW_STAGE);
-  load_exps(0, exps);
+  exps = load_exps(0);
   landed_barrier();
 #pragma unroll
   for (int c = 0; c < 4; ++c) quarter(c, 0, 0);
-  load_exps(2, exps);
+  exps = load_exps(2);
   landed_barrier();            // weights of step 0 visible, raw stage 0 free
   issue_a(2, STAGE);
   issue_raw(4, 0);
-  load_exps(4, exps_next);
+  exps_next = load_exps(4);
   fetch(0, 0, fw[0], fa[0]);
   quarter(0, RAW_STAGE, STAGE);
 
+  // ---- rotated pipeline.  A step is four chunks of 16 k.  Chunk q multiplies, requests the fragments of the
+  // following chunk and converts weight rows 2c, 2c+1 with c = (q + 1) % 4; the scheduler is asked to put the
+  // conversion's VALU instructions behind the MFMAs, five apiece, which is what the matrix core leaves free
+  // on the issue port.  The block barrier sits between chunks 2 and 3: chunk 3 multiplies from fragments that
+  // were requested before the barrier and already requests chunk 0 of the next stage, so the matrix core does
+  // not drain at the barrier; its conversion quarter (c = 0) belongs to the step after next.
   auto step = [&](auto stage_c, int ks) {
     constexpr uint32_t CUR = decltype(stage_c)::value * STAGE, NXT = STAGE - CUR;
     constexpr uint32_t RCUR = decltype(stage_c)::value * RAW_STAGE, RNXT = RAW_STAGE - RCUR;
@@ -1645,11 +841,10 @@ __global__ __launch_bounds__(NWAVE * 64) void ttm_linear_dma_k(LinearArgs p) {
       mfma_chunk(q & 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-#pragma unroll
-    for (int h = 0; h < NU; ++h) exps[h] = exps_next[h];
+    exps = exps_next;
     landed_barrier();
-    // stage CUR of the activations, stage RNXT of the mantissas are free now
-    load_exps((ks + 3) * 2, exps_next);
+    // stage CUR of the activations and stage RNXT of the mantissas are free now
+    exps_next = load_exps((ks + 3) * 2);
     issue_a((ks + 2) * 2, CUR);
     issue_raw((ks + 3) * 2, RNXT);
     fetch(0, NXT, fw[0], fa[0]);
@@ -1664,14 +859,22 @@ __global__ __launch_bounds__(NWAVE * 64) void ttm_linear_dma_k(LinearArgs p) {
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be in flight towards LDS when the block ends
 
-  // epilogue: bias, activation, bf16, 8-byte stores into the output face rows
-  switch (p.act) {
-  case TTM_ACT_GELU: linear_epilogue<TTM_ACT_GELU>(p, C, acc, mt0 + wm * MB, nt0 + wn * 4, lane); break;
-  case TTM_ACT_SILU: linear_epilogue<TTM_ACT_SILU>(p, C, acc, mt0 + wm * MB, nt0 + wn * 4, lane); break;
-  case TTM_ACT_SIGMOID: linear_epilogue<TTM_ACT_SIGMOID>(p, C, acc, mt0 + wm * MB, nt0 + wn * 4, lane); break;
-  case TTM_ACT_RELU: linear_epilogue<TTM_ACT_RELU>(p, C, acc, mt0 + wm * MB, nt0 + wn * 4, lane); break;
-  default: linear_epilogue<TTM_ACT_NONE>(p, C, acc, mt0 + wm * MB, nt0 + wn * 4, lane); break;
-  }
+  linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wn * NTW, nt_end, lane);
+}
+
+// The grid is split in two parts so that the last, partly filled round of blocks can use narrower blocks:
+// blocks [0, split) cover column tiles [0, nt_split) with 2 ntw_a tiles per block, the rest covers
+// [nt_split, Nt) with 2 ntw_b tiles per block.
+template <int WF>
+__global__ __launch_bounds__(512) void ttm_linear_dma_k(LinearArgs p) {
+  const bool first = (int)blockIdx.x < p.split;
+  const int ntw = first ? p.ntw_a : p.ntw_b;
+  const int bid = first ? blockIdx.x : blockIdx.x - p.split;
+  const int nblk = first ? p.split : (int)gridDim.x - p.split;
+  const int nt_first = first ? 0 : p.nt_split, nt_end = first ? p.nt_split : p.Nt;
+  if (ntw == 4) linear_dma_block<WF, 4>(p, bid, nblk, nt_first, nt_end);
+  else if (ntw == 3) linear_dma_block<WF, 3>(p, bid, nblk, nt_first, nt_end);
+  else linear_dma_block<WF, 2>(p, bid, nblk, nt_first, nt_end);
 }
 
 // =============================================================================================
@@ -1809,10 +1012,57 @@ __global__ __launch_bounds__(256) void ttm_linear_small_k(LinearArgs p) {
   }
 }
 
+static int device_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    else cus = 256;
+  }
+  return cus;
+}
+
+// Grid of the block-float main kernel.  Whole rounds (one block per CU) use 8-tile-wide blocks.  What is left may
+// use narrower blocks (6 or 4 column tiles) when that fills more CUs: a narrower block keeps the whole activation
+// traffic of a wide one, so its measured time is 0.92 (6 tiles) and 0.78 (4 tiles) of it, and it is only chosen
+// when the estimate (block time x rounds) beats the wide block by more than 15 %.
+static void plan_dma_grid(LinearArgs &p, int cus, int force_ntw) {
+  const int mbk = p.m_blocks;
+  auto blocks_for = [&](int nt, int ntw) { return mbk * ((nt + 2 * ntw - 1) / (2 * ntw)); };
+  p.ntw_a = 4;
+  p.nt_split = 0;
+  if (force_ntw == 0 && mbk <= cus && cus % mbk == 0) {
+    const int per_round = cus / mbk;                 // column blocks per round
+    p.nt_split = (p.Nt / 8 / per_round) * per_round * 8;
+  }
+  p.split = mbk * (p.nt_split / 8);
+  const int rest = p.Nt - p.nt_split;
+  p.ntw_b = 4;
+  if (force_ntw >= 2 && force_ntw <= 4) p.ntw_b = force_ntw;
+  else {
+    static const int block_time[5] = {0, 0, 78, 92, 100};
+    const int wide = block_time[4] * ((blocks_for(rest, 4) + cus - 1) / cus);
+    int best = wide * 85 / 100;
+    for (int ntw = 3; ntw >= 2; --ntw) {
+      const int cost = block_time[ntw] * ((blocks_for(rest, ntw) + cus - 1) / cus);
+      if (cost < best) { best = cost; p.ntw_b = ntw; }
+    }
+  }
+  p.n_blocks = p.split + (rest > 0 ? blocks_for(rest, p.ntw_b) : 0);   // total blocks of the launch
+}
+
+template <typename K>
+static int set_lds_limit(K kernel, int bytes) {
+  hipError_t e = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "hipFuncSetAttribute(LDS %d): %s", bytes, hipGetErrorString(e));
+  return 0;
+}
+
 template <int WF>
 static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
+  constexpr bool BFP = WF == WF_BFP8 || WF == WF_BFP4;
   if (a.Mt == 1 || a.Mt * 32 <= ttm_option("linear_small_m_max")) {
-    // the small kernel handles one row tile per launch row: loop row tiles through grid.y
+    // the small kernel handles one row tile per launch
     LinearArgs p = a;
     for (int mt = 0; mt < a.Mt; ++mt) {
       p.A = a.A + (int64_t)mt * a.Kt * 2048;
@@ -1821,64 +1071,43 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
     }
     return 0;
   }
-  static bool attr_set = false;
-  const int lds_bytes = 2 * 4096 * 16;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void *)ttm_linear_big_k<WF>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       lds_bytes);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void *)ttm_linear_pipe_k<WF>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e == hipSuccess)
-      e = hipFuncSetAttribute((const void *)ttm_linear_w8_k<WF>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "hipFuncSetAttribute(LDS %d): %s", lds_bytes, hipGetErrorString(e));
-    attr_set = true;
-  }
+  // linear_variant: 0 = automatic, 1 = 64-bit-addressed fallback, 5 = register-staged kernel, 6 = LDS-direct kernel
   int variant = ttm_option("linear_variant");
-  if (variant == 0) variant = (WF == WF_BFP8 || WF == WF_BFP4) ? 6 : 5;
-  if constexpr (WF == WF_BFP8 || WF == WF_BFP4) {
-    if (variant == 6 || variant == 7) {
-      static bool attr6 = false;
+  // the main kernels keep per-lane 32-bit offsets into one batch entry of the activations ([N,K] weights too)
+  const bool fits32 = (int64_t)a.Mt * a.Kt * 2048 < (int64_t)1 << 32 && (int64_t)a.Nt * a.Kt * 2048 < (int64_t)1 << 32;
+  if (variant == 0) variant = !fits32 ? 1 : (BFP ? 6 : 5);
+  if ((variant == 5 || variant == 6) && !fits32) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear: operand too large for the selected kernel variant");
+  if (variant == 6 && !BFP) variant = 5;
+  const int lds_bytes = 2 * 4096 * 16;
+  if constexpr (BFP) {
+    if (variant == 6) {
+      static bool attr = false;
       const int lds6 = 131072 + (WF == WF_BFP8 ? 32768 : 16384);
-      if (!attr6) {
-        hipError_t e = hipFuncSetAttribute((const void *)ttm_linear_dma_k<WF, 8>, hipFuncAttributeMaxDynamicSharedMemorySize, lds6);
-        if (e == hipSuccess) e = hipFuncSetAttribute((const void *)ttm_linear_dma_k<WF, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, lds6);
-        if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "hipFuncSetAttribute(LDS %d): %s", lds6, hipGetErrorString(e));
-        attr6 = true;
+      if (!attr) {
+        if (int rc = set_lds_limit(ttm_linear_dma_k<WF>, lds6)) return rc;
+        attr = true;
       }
-      if (variant == 6) hipLaunchKernelGGL((ttm_linear_dma_k<WF, 8>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(512), lds6, s, a);
-      else hipLaunchKernelGGL((ttm_linear_dma_k<WF, 4>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(256), lds6, s, a);
+      LinearArgs p = a;
+      plan_dma_grid(p, device_cu_count(), ttm_option("linear_ntw"));
+      hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, 1, (unsigned)batch), dim3(512), lds6, s, p);
       return 0;
     }
   }
-  if (variant == 4 || variant == 5) {
-    static bool attr4 = false;
-    if (!attr4) {
-      hipError_t e = hipFuncSetAttribute((const void *)ttm_linear_main_k<WF, false>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-      if (e == hipSuccess) e = hipFuncSetAttribute((const void *)ttm_linear_main_k<WF, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-      if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "hipFuncSetAttribute(LDS %d): %s", lds_bytes, hipGetErrorString(e));
-      attr4 = true;
+  if (variant == 5) {
+    static bool attr = false;
+    if (!attr) {
+      if (int rc = set_lds_limit(ttm_linear_reg_k<WF>, lds_bytes)) return rc;
+      attr = true;
     }
-    if (variant == 4) hipLaunchKernelGGL((ttm_linear_main_k<WF, false>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(512), lds_bytes, s, a);
-    else hipLaunchKernelGGL((ttm_linear_main_k<WF, true>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(512), lds_bytes, s, a);
+    hipLaunchKernelGGL((ttm_linear_reg_k<WF>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(512), lds_bytes, s, a);
     return 0;
   }
-  if (variant == 8 && WF == WF_BFP8) {
-    static bool attr2 = false;
-    const int lds2 = 163840;
-    if (!attr2) {
-      hipError_t e = hipFuncSetAttribute((const void *)ttm_linear_w8s_k, hipFuncAttributeMaxDynamicSharedMemorySize, lds2);
-      if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "hipFuncSetAttribute(LDS %d): %s", lds2, hipGetErrorString(e));
-      attr2 = true;
-    }
-    hipLaunchKernelGGL(ttm_linear_w8s_k, dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(512), lds2, s, a);
-    return 0;
+  static bool attr = false;
+  if (!attr) {
+    if (int rc = set_lds_limit(ttm_linear_big_k<WF>, lds_bytes)) return rc;
+    attr = true;
   }
-  if (variant == 1)
-    hipLaunchKernelGGL((ttm_linear_big_k<WF>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(256), lds_bytes, s, a);
-  else if (variant != 3)
-    hipLaunchKernelGGL((ttm_linear_w8_k<WF>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(512), lds_bytes, s, a);
-  else
-    hipLaunchKernelGGL((ttm_linear_pipe_k<WF>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(256), lds_bytes, s, a);
+  hipLaunchKernelGGL((ttm_linear_big_k<WF>), dim3(a.m_blocks * a.n_blocks, 1, (unsigned)batch), dim3(256), lds_bytes, s, a);
   return 0;
 }
 
@@ -1909,7 +1138,7 @@ TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype
   p.w_batch = w_batch == 1 ? 0 : (int64_t)p.Kt * p.Nt * w_tile;
   p.c_batch = (int64_t)p.Mt * p.Nt * 2048;
   p.m_blocks = (p.Mt + 7) / 8; p.n_blocks = (p.Nt + 7) / 8;
-  p.debug = ttm_option("linear_debug");
+  p.split = 0; p.nt_split = 0; p.ntw_a = 4; p.ntw_b = 4;
   TTM_REQUIRE(batch <= 65535, "ttm_linear: batch too large");
   hipStream_t s = (hipStream_t)stream;
   int rc;
