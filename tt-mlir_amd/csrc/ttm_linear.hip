@@ -927,7 +927,7 @@ __global__ __launch_bounds__(256) void ttm_linear_small_k(LinearArgs p) {
       const uint8_t *m = t + 64 + face * 256 + khalf * 128 + oct * 8;
       u32x2 rows[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) rows[i] = ok ? __builtin_nontemporal_load((const u32x2 *)(m + i * 16)) : u32x2{0, 0};
+      for (int i = 0; i < 8; ++i) rows[i] = ok ? *(const u32x2 *)(m + i * 16) : u32x2{0, 0};
       dequant_bfp8_block(rows, exps, out);
     } else if constexpr (WF == WF_BFP4) {
       const uint8_t *t = W + tile * 576;
@@ -935,7 +935,7 @@ __global__ __launch_bounds__(256) void ttm_linear_small_k(LinearArgs p) {
       const uint8_t *m = t + 64 + face * 128 + khalf * 64 + oct * 4;
       uint32_t rows[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) rows[i] = ok ? __builtin_nontemporal_load((const uint32_t *)(m + i * 8)) : 0u;
+      for (int i = 0; i < 8; ++i) rows[i] = ok ? *(const uint32_t *)(m + i * 8) : 0u;
       dequant_bfp4_block(rows, exps, out);
     } else {
       const uint8_t *m = W + tile * 2048 + face * 512 + khalf * 256 + oct * 16;
@@ -1012,6 +1012,135 @@ __global__ __launch_bounds__(256) void ttm_linear_small_k(LinearArgs p) {
   }
 }
 
+// =============================================================================================
+// Decode kernel for bfp8_b weights (M <= 32 per launch): pure weight streaming, no LDS on the way in.
+// A workgroup owns 64 output columns (two weight tiles); its 8 wavefronts take every 8th k-tile and are
+// summed through LDS at the end.  Per k-tile a lane loads the 8 (k) x 4 (n) block it needs as eight
+// 4-byte words, dequantises it in registers and feeds byte j of the words to MFMA j: with
+// v_mfma_f32_16x16x32_bf16 lane l supplies row l % 16 and k = 8 (l / 16) .. + 7 of the 16 x 32 weight
+// operand, and MFMA j's row r stands for column n = 4 r + j, so one accumulator register of the four
+// MFMAs is four consecutive n again.  Loads run four k-tiles ahead (register ring).
+// =============================================================================================
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(512) void ttm_linear_decode_bfp8_k(LinearArgs p) {
+  extern __shared__ u32x4 smem[];   // partial sums: 8 wavefronts x 8 x 64 float4 = 64 KiB
+  constexpr int D = 4;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int cg = blockIdx.x;
+  const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
+  const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
+  uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
+  const int q16 = lane & 15, kg = lane >> 4;   // weight operand row and 8-k group of this lane
+  const int fc = (q16 >> 2) & 1, quad = q16 & 3, fr = kg >> 1, half = kg & 1;
+  const uint32_t nt_l = (uint32_t)min(2 * cg + (q16 >> 3), p.Nt - 1);
+  const uint32_t offW = nt_l * 1088u + 64u + (fr * 2 + fc) * 256 + half * 128 + quad * 4;   // + 16 i
+  const uint32_t offE = nt_l * 1088u + (fr * 2 + fc) * 16 + half * 8;
+  const uint32_t offA = fr * 512 + q16 * 32 + half * 16;                                     // + 1024 h
+
+  f32x4v acc[2][4];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[h][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+
+  uint32_t rows[D][8], keeps[D];
+  u32x2 ex[D];
+  u32x4 af[D][2];
+  const int nchunks = (p.Kt + 7) / 8;
+  auto load_slot = [&](int s, int c) {
+    const int kt = wave + 8 * c;
+    const int ktc = min(kt, p.Kt - 1);
+    const uint32_t keep = kt < p.Kt ? 0xFFFFFFFFu : 0u;   // past the end: zero exponents, zero weights
+    const uint8_t *Wk = W + (int64_t)ktc * p.Nt * 1088;
+    const uint8_t *Ak = A + (int64_t)ktc * 2048;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) rows[s][i] = *(const uint32_t *)(Wk + offW + i * 16);   // the eight loads share their cache lines: cached loads
+    ex[s] = *(const u32x2 *)(Wk + offE);
+    keeps[s] = keep;   // applied when the slot is consumed: masking here would wait for the load
+#pragma unroll
+    for (int h = 0; h < 2; ++h) af[s][h] = *(const u32x4 *)(Ak + offA + h * 1024);
+  };
+  auto process = [&](int s) {
+    float f[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      uint32_t E = (((i < 4 ? ex[s].x : ex[s].y) & keeps[s]) >> (8 * (i & 3))) & 0xFFu;
+      E = max(E, 6u);
+      const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
+      const uint32_t d = rows[s][i];
+      const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
+      const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) f[i][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      u32x4 w = {pack_hi(f[0][j], f[1][j]), pack_hi(f[2][j], f[3][j]), pack_hi(f[4][j], f[5][j]), pack_hi(f[6][j], f[7][j])};
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&w, *(bf16x8 *)&af[s][h], acc[h][j], 0, 0, 0);
+    }
+  };
+#pragma unroll
+  for (int s = 0; s < D; ++s) {
+    load_slot(s, s);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  // straight-line loop body (exact load counters): the chunk count is rounded up to the ring depth, and the
+  // extra chunks contribute zeros
+  for (int c0 = 0; c0 < nchunks; c0 += D) {
+#pragma unroll
+    for (int s = 0; s < D; ++s) {
+      process(s);
+      __builtin_amdgcn_sched_barrier(0);   // keep the loads in slot order, D - 1 slots ahead of their use
+      load_slot(s, c0 + s + D);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  // partial sums -> LDS as float4 (four consecutive n of one m): slot ((wave * 8 + h * 4 + i) * 64 + lane)
+  f32x4v *part = (f32x4v *)smem;
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      part[(wave * 8 + h * 4 + i) * 64 + lane] = f32x4v{acc[h][0][i], acc[h][1][i], acc[h][2][i], acc[h][3][i]};
+  __syncthreads();
+  // thread t finishes slot t of the 512: (h, i, lane) = (t >> 8, (t >> 6) & 3, t & 63)
+  f32x4v sum = part[tid];
+#pragma unroll
+  for (int w = 1; w < 8; ++w) sum += part[w * 512 + tid];
+  const int h = tid >> 8, i = (tid >> 6) & 3;
+  const int nt = 2 * cg + (kg >> 1);
+  if (nt >= p.Nt) return;
+  const int n_in = 16 * (kg & 1) + 4 * i;
+  float bv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (p.bias) {
+    const uint16_t *bp = p.bias_tiled ? p.bias + (int64_t)nt * 1024 + (n_in >> 4) * 256 + (n_in & 15) : p.bias + nt * 32 + n_in;
+    u32x2 raw = *(const u32x2 *)bp;
+    bv[0] = __uint_as_float(raw.x << 16); bv[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+    bv[2] = __uint_as_float(raw.y << 16); bv[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+  }
+  float v[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float x = sum[r] + bv[r];
+    switch (p.act) {
+    case TTM_ACT_GELU: x = apply_act<TTM_ACT_GELU>(x); break;
+    case TTM_ACT_SILU: x = apply_act<TTM_ACT_SILU>(x); break;
+    case TTM_ACT_SIGMOID: x = apply_act<TTM_ACT_SIGMOID>(x); break;
+    case TTM_ACT_RELU: x = apply_act<TTM_ACT_RELU>(x); break;
+    default: break;
+    }
+    v[r] = x;
+  }
+  u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+  const int64_t off = (int64_t)nt * 1024 + (h * 2 + (n_in >> 4)) * 256 + q16 * 16 + (n_in & 15);
+  *(u32x2 *)(C + off * 2) = o;
+}
+
 static int device_cu_count() {
   static int cus = 0;
   if (cus == 0) {
@@ -1064,10 +1193,12 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
   if (a.Mt == 1 || a.Mt * 32 <= ttm_option("linear_small_m_max")) {
     // the small kernel handles one row tile per launch
     LinearArgs p = a;
+    const bool decode = WF == WF_BFP8 && ttm_option("linear_variant") != 1 && (int64_t)a.Nt * 1088 < (int64_t)1 << 32;
     for (int mt = 0; mt < a.Mt; ++mt) {
       p.A = a.A + (int64_t)mt * a.Kt * 2048;
       p.C = a.C + (int64_t)mt * a.Nt * 2048;
-      hipLaunchKernelGGL((ttm_linear_small_k<WF>), dim3(a.Nt, 1, (unsigned)batch), dim3(256), 0, s, p);
+      if (decode) hipLaunchKernelGGL(ttm_linear_decode_bfp8_k, dim3((a.Nt + 1) / 2, 1, (unsigned)batch), dim3(512), 65536, s, p);
+      else hipLaunchKernelGGL((ttm_linear_small_k<WF>), dim3(a.Nt, 1, (unsigned)batch), dim3(256), 0, s, p);
     }
     return 0;
   }

@@ -1,8 +1,9 @@
 // Row-wise bandwidth kernels on tile-ordered tensors: RMSNorm, softmax and reductions over the
-// last dimension.  A workgroup owns one tile row (32 logical rows x all columns), which is one
-// contiguous run of tiles in memory.  Thread (r = tid % 32, j = tid / 32) walks the chunks of row
-// r with stride 8; for every step the 256 lanes together read whole tiles, so global accesses are
-// contiguous.  Partial results of the 8 lanes of a row meet in LDS.  Math is fp32; columns beyond
+// last dimension.  A workgroup owns RPB = 32 or 8 rows of one tile row (32 logical rows x all columns,
+// one contiguous run of tiles in memory); 8 rows per workgroup are used when whole tile rows would
+// leave most CUs without work.  Thread (r = tid % RPB, j = tid / RPB) walks the chunks of row r with
+// stride 256 / RPB; the lanes of a step read whole face rows, so global accesses are contiguous runs
+// of at least 256 bytes.  Partial results of the lanes of a row meet in LDS.  Math is fp32; columns beyond
 // the logical width are masked with the operation's identity, rows beyond the logical height are
 // written as zeros.
 #include "ttm_common.h"
@@ -70,13 +71,16 @@ __device__ __forceinline__ void load_vec(const void *v, int tiled, int c0, float
   load_vals<ELEM>(v, off, f);
 }
 
-template <int MODE, int ELEM>
+template <int MODE, int ELEM, int RPB>
 __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
   constexpr int EPC = 16 / ELEM;
-  __shared__ float part[8][32];
-  __shared__ float part2[8][32];
-  const int tid = threadIdx.x, r = tid & 31, j = tid >> 5;
-  const int64_t trow = blockIdx.x;                       // tile row over all batch entries
+  constexpr int J = 256 / RPB;                           // lanes per row
+  __shared__ float part[J][RPB];
+  __shared__ float part2[J][RPB];
+  const int tid = threadIdx.x, j = tid / RPB;
+  const int r = (int)(blockIdx.x % (32 / RPB)) * RPB + tid % RPB;   // row inside the tile row
+  const int rl = tid % RPB;
+  const int64_t trow = blockIdx.x / (32 / RPB);          // tile row over all batch entries
   const int64_t row = (trow % p.rt) * 32 + r;            // logical row inside the batch entry
   const bool row_ok = row < p.rows;
   const int nq = p.ct * 2 * ELEM;                        // chunks per row
@@ -85,7 +89,8 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
 
   constexpr bool IS_MAX = MODE == RW_SOFTMAX || MODE == RW_MAX;
   float acc = IS_MAX ? -INFINITY : (MODE == RW_MIN ? INFINITY : 0.0f);
-  for (int q = j; q < nq; q += 8) {
+  #pragma unroll 4
+  for (int q = j; q < nq; q += J) {
     ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
     float f[EPC];
     load_vals<ELEM>(x, cp.off, f);
@@ -98,12 +103,12 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
       else acc += ok ? f[i] : 0.0f;
     }
   }
-  part[j][r] = acc;
+  part[j][rl] = acc;
   __syncthreads();
-  float stat = part[0][r];
+  float stat = part[0][rl];
 #pragma unroll
-  for (int k = 1; k < 8; ++k) {
-    float o = part[k][r];
+  for (int k = 1; k < J; ++k) {
+    float o = part[k][rl];
     stat = IS_MAX ? fmaxf(stat, o) : (MODE == RW_MIN ? fminf(stat, o) : stat + o);
   }
 
@@ -111,8 +116,11 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
     // output [.., rows, 1] in tile order: one column tile per tile row; zero padded
     if (MODE == RW_MEAN) stat = stat / (float)cols;
     uint8_t *o = (uint8_t *)p.out + trow * 1024 * ELEM;
-    // 256 lanes clear the tile (1024 elements), then column 0 is written
-    for (int e = tid; e < 1024 * ELEM / 16; e += 256) ((u32x4 *)o)[e] = u32x4{0, 0, 0, 0};
+    // the lanes clear the block's rows of the tile (both faces), then column 0 is written
+    for (int e = tid; e < RPB * 2 * (16 * ELEM / 16); e += 256) {
+      const int rr = (int)(blockIdx.x % (32 / RPB)) * RPB + e / (2 * ELEM), fx = (e / ELEM) & 1, part_i = e % ELEM;
+      ((u32x4 *)o)[(((rr >> 4) * 2 + fx) * 256 + (rr & 15) * 16) * ELEM / 16 + part_i] = u32x4{0, 0, 0, 0};
+    }
     __syncthreads();
     if (j == 0 && row_ok) {
       int64_t off = ((r >> 4) * 2) * 256 + (r & 15) * 16;
@@ -125,7 +133,8 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
   uint8_t *o = (uint8_t *)p.out + trow * p.ct * 1024 * ELEM;
   if (MODE == RW_RMSNORM) {
     const float rs = 1.0f / sqrtf(stat / (float)cols + p.eps);
-    for (int q = j; q < nq; q += 8) {
+    #pragma unroll 4
+  for (int q = j; q < nq; q += J) {
       ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
       float f[EPC], w[EPC], b[EPC];
       load_vals<ELEM>(x, cp.off, f);
@@ -143,20 +152,22 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
   } else {  // softmax: second pass for the sum of exponentials, third pass writes
     const float mx = stat;
     float sum = 0.0f;
-    for (int q = j; q < nq; q += 8) {
+    #pragma unroll 4
+  for (int q = j; q < nq; q += J) {
       ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
       float f[EPC];
       load_vals<ELEM>(x, cp.off, f);
 #pragma unroll
       for (int i = 0; i < EPC; ++i) sum += cp.c0 + i < cols ? expf(f[i] - mx) : 0.0f;
     }
-    part2[j][r] = sum;
+    part2[j][rl] = sum;
     __syncthreads();
     float tot = 0.0f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) tot += part2[k][r];
+    for (int k = 0; k < J; ++k) tot += part2[k][rl];
     const float inv = 1.0f / tot;
-    for (int q = j; q < nq; q += 8) {
+    #pragma unroll 4
+  for (int q = j; q < nq; q += J) {
       ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
       float f[EPC];
       load_vals<ELEM>(x, cp.off, f);
@@ -169,9 +180,14 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
 
 template <int MODE>
 static int launch_rowwise(const RowArgs &p, int dtype, int64_t trows, hipStream_t s) {
-  TTM_REQUIRE(trows < (1ll << 31), "row-wise kernel: tensor too large");
-  if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_k<MODE, 2>), dim3((unsigned)trows), dim3(256), 0, s, p);
-  else hipLaunchKernelGGL((ttm_rowwise_k<MODE, 4>), dim3((unsigned)trows), dim3(256), 0, s, p);
+  TTM_REQUIRE(trows < (1ll << 29), "row-wise kernel: tensor too large");
+  if (trows >= 1024) {   // enough tile rows to fill the device with one workgroup each
+    if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_k<MODE, 2, 32>), dim3((unsigned)trows), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((ttm_rowwise_k<MODE, 4, 32>), dim3((unsigned)trows), dim3(256), 0, s, p);
+  } else {
+    if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_k<MODE, 2, 8>), dim3((unsigned)trows * 4), dim3(256), 0, s, p);
+    else hipLaunchKernelGGL((ttm_rowwise_k<MODE, 4, 8>), dim3((unsigned)trows * 4), dim3(256), 0, s, p);
+  }
   TTM_LAUNCH_CHECK();
   return TTM_OK;
 }
