@@ -171,3 +171,32 @@ def test_weight_dtype_bars(hip, dev, metrics, wfmt_name, bar):
     got, _ = run_linear(hip, dev, a, w, None, None, wfmt)
     ref = a.float() @ w.to(torch.bfloat16).float()
     assert metrics.get_pcc(ref.numpy(), got.float().numpy()) >= bar
+
+
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4"])
+@pytest.mark.parametrize("option,value", [("linear_ntw", 4), ("linear_ntw", 3), ("linear_ntw", 2), ("linear_split_k", 2),
+                                          ("linear_split_k", 3), ("linear_variant", 1), ("linear_variant", 5)])
+def test_block_float_kernel_configurations(hip, dev, orc, metrics, wfmt_name, option, value):
+    """Every block width of the LDS-direct kernel, the split-K path with its reduction kernel, the register-staged
+    kernel and the 64-bit-addressed fallback, on a ragged shape with an odd number of k-tiles."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    M, K, N = 330, 7 * 32 + 8, 21 * 32 + 5
+    a = datagen.randn((M, K), seed=11, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=12, std=0.05)
+    b = datagen.randn((N,), seed=13, std=0.5, dtype=torch.bfloat16)
+    hip.set_option(option, value)
+    try:
+        got, w_eff = run_linear(hip, dev, a, w, b, "gelu", wfmt)
+    finally:
+        hip.set_option(option, 0)
+    check(orc, metrics, got, a, w_eff, b, "gelu", max_abs=2.0 ** -5)
+
+
+def test_split_k_is_chosen_for_long_skinny_reductions(hip, dev, orc, metrics):
+    """M = 128, N = 256, K = 8192: one round of blocks would use 2 CUs; the launcher splits K."""
+    M, K, N = 128, 8192, 256
+    a = datagen.randn((M, K), seed=21, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=22, std=0.02)
+    got, w_eff = run_linear(hip, dev, a, w, None, None, hip.BFP8B)
+    # |y| ~ 0.02 * sqrt(8192) ~ 1.8: one bf16 ulp below 4 is 2^-6; allow 2^-5
+    check(orc, metrics, got, a, w_eff, None, None, max_abs=2.0 ** -5)

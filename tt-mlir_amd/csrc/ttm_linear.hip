@@ -37,6 +37,8 @@ struct LinearArgs {
   int64_t a_batch, w_batch, c_batch;  // byte strides between batch entries (w_batch 0 = shared weights)
   int m_blocks, n_blocks;
   int split, nt_split, ntw_a, ntw_b;  // two-part grid of the block-float main kernel
+  int k_slice;                        // k-tiles per grid.y slice (split-K); Kt when the reduction is not split
+  float *partial;                     // split-K: fp32 partial sums [slices][Mt * Nt * 1024] in output tile order
 };
 
 template <int ACT>
@@ -248,6 +250,63 @@ __device__ __forceinline__ void linear_epilogue(const LinearArgs &p, uint8_t *C,
     }
   }
 }
+// split-K: fp32 partial sums of a wavefront's accumulator tiles, same element order as the bf16 output
+template <int NA, int MB>
+__device__ __forceinline__ void linear_store_partial(const LinearArgs &p, float *P, f32x16 (&acc)[NA][MB], int mtw, int ntw, int nt_end, int lane) {
+  const int m_in = lane & 31;
+#pragma unroll
+  for (int a = 0; a < NA; ++a) {
+    const int nt = ntw + a;
+    if (nt >= nt_end) continue;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int n_in = g * 8 + (lane >> 5) * 4;
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const int mt = mtw + b;
+        if (mt >= p.Mt) continue;
+        const int64_t off = ((int64_t)mt * p.Nt + nt) * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
+        *(f32x4 *)(P + off) = f32x4{acc[a][b][g * 4], acc[a][b][g * 4 + 1], acc[a][b][g * 4 + 2], acc[a][b][g * 4 + 3]};
+      }
+    }
+  }
+}
+
+// split-K: sums the slices, then bias, activation and bf16 as in the fused epilogue; one lane per four elements
+__global__ __launch_bounds__(256) void ttm_linear_reduce_k(LinearArgs p, int slices) {
+  const int64_t per = (int64_t)p.Mt * p.Nt * 1024;
+  const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;   // group of four consecutive elements
+  if (q * 4 >= per) return;
+  const float *P = p.partial + (int64_t)blockIdx.z * slices * per + q * 4;
+  f32x4 sum = *(const f32x4 *)P;
+  for (int s = 1; s < slices; ++s) sum += *(const f32x4 *)(P + s * per);
+  const int64_t off = q * 4;
+  const int nt = (int)((off >> 10) % p.Nt), in = (int)(off & 1023);
+  const int n_in = ((in >> 8) & 1) * 16 + (in & 15);
+  float bv[4] = {0.f, 0.f, 0.f, 0.f};
+  if (p.bias) {
+    const uint16_t *bp = p.bias_tiled ? p.bias + (int64_t)nt * 1024 + (n_in >> 4) * 256 + (n_in & 15) : p.bias + nt * 32 + n_in;
+    u32x2 raw = *(const u32x2 *)bp;
+    bv[0] = __uint_as_float(raw.x << 16); bv[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+    bv[2] = __uint_as_float(raw.y << 16); bv[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+  }
+  float v[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float x = sum[r] + bv[r];
+    switch (p.act) {
+    case TTM_ACT_GELU: x = apply_act<TTM_ACT_GELU>(x); break;
+    case TTM_ACT_SILU: x = apply_act<TTM_ACT_SILU>(x); break;
+    case TTM_ACT_SIGMOID: x = apply_act<TTM_ACT_SIGMOID>(x); break;
+    case TTM_ACT_RELU: x = apply_act<TTM_ACT_RELU>(x); break;
+    default: break;
+    }
+    v[r] = x;
+  }
+  uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
+  *(u32x2 *)(C + off * 2) = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+}
+
 template <int NA, int MB>
 __device__ __forceinline__ void linear_epilogue_act(const LinearArgs &p, uint8_t *C, f32x16 (&acc)[NA][MB], int mtw, int ntw, int nt_end, int lane) {
   switch (p.act) {   // uniform
@@ -723,11 +782,14 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     dmaW = (uint32_t)(min(nt0 + 2 * (wave & 3) + (lane >> 5), p.Nt - 1) * (int)W_TILE) + 64u + (uint32_t)(lane & 31) * 16u;
   }
 
-  const int ksteps = (p.Kt + 1) / 2;
+  // split-K: this block reduces k-tiles [kbase, kt_end); k-tiles past kt_end get zero weights
+  const int kbase = blockIdx.y * p.k_slice, kt_end = min(p.Kt, kbase + p.k_slice);
+  const int ksteps = (kt_end - kbase + 1) / 2;
   u32x2 exps = {0, 0}, exps_next = {0, 0};
   u32x4 fw[2][NTW], fa[2][MB], out[4];
 
   auto issue_a = [&](int kt0, uint32_t stage_off) {
+    kt0 += kbase;
     const int kt = min(kt0, p.Kt - 1);
     const uint32_t sub = kt0 + 1 < p.Kt ? 2048u : 0u;   // k tail: the second tile of the pair repeats the first (its weights are zero)
     const uint8_t *base = A + a_row + (int64_t)kt * 2048;
@@ -737,7 +799,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   };
   auto issue_raw = [&](int kt0, uint32_t stage_off) {
     if (!converts) return;
-    const int kt = min(kt0 + ukt, p.Kt - 1);
+    const int kt = min(kbase + kt0 + ukt, p.Kt - 1);
     const uint8_t *row = W + (int64_t)kt * p.Nt * W_TILE;
     if constexpr (WF == WF_BFP8) {
 #pragma unroll
@@ -748,8 +810,9 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     }
   };
   auto load_exps = [&](int kt0) {
+    kt0 += kbase;
     const int kt = min(kt0 + ukt, p.Kt - 1);
-    const uint32_t keep = kt0 + ukt >= p.Kt ? 0u : 0xFFFFFFFFu;   // k tail: zero exponents dequantise to zero weights
+    const uint32_t keep = kt0 + ukt >= kt_end ? 0u : 0xFFFFFFFFu;   // k tail: zero exponents dequantise to zero weights
     u32x2 e = *(const u32x2 *)(W + (int64_t)kt * p.Nt * W_TILE + offWe);
     return u32x2{e.x & keep, e.y & keep};
   };
@@ -859,7 +922,9 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be in flight towards LDS when the block ends
 
-  linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wn * NTW, nt_end, lane);
+  if (p.partial) linear_store_partial(p, p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * ((int64_t)p.Mt * p.Nt * 1024), acc,
+                                      mt0 + wm * MB, nt0 + wn * NTW, nt_end, lane);
+  else linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wn * NTW, nt_end, lane);
 }
 
 // The grid is split in two parts so that the last, partly filled round of blocks can use narrower blocks:
@@ -1219,8 +1284,33 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         attr = true;
       }
       LinearArgs p = a;
-      plan_dma_grid(p, device_cu_count(), ttm_option("linear_ntw"));
-      hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, 1, (unsigned)batch), dim3(512), lds6, s, p);
+      const int cus = device_cu_count();
+      plan_dma_grid(p, cus, ttm_option("linear_ntw"));
+      // split-K when the output alone gives less than half a round of blocks and the reduction is long
+      int slices = ttm_option("linear_split_k");
+      if (slices == 0) {
+        slices = 1;
+        const int ksteps = (a.Kt + 1) / 2;
+        while (slices < 8 && p.n_blocks * slices * 2 <= cus && ksteps / (slices * 2) >= 16) slices *= 2;
+      }
+      slices = slices < 1 ? 1 : (slices > a.Kt ? a.Kt : slices);
+      if (slices > 1) {
+        p.k_slice = (a.Kt + slices - 1) / slices;
+        slices = (a.Kt + p.k_slice - 1) / p.k_slice;
+      }
+      if (slices <= 1) {
+        hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, 1, (unsigned)batch), dim3(512), lds6, s, p);
+        return 0;
+      }
+      const int64_t per = (int64_t)a.Mt * a.Nt * 1024;
+      void *ws = nullptr;
+      hipError_t e = hipMallocAsync(&ws, (size_t)(per * slices * batch) * sizeof(float), s);
+      if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "ttm_linear: split-K workspace: %s", hipGetErrorString(e));
+      p.partial = (float *)ws;
+      hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), lds6, s, p);
+      hipLaunchKernelGGL(ttm_linear_reduce_k, dim3((unsigned)((per / 4 + 255) / 256), 1, (unsigned)batch), dim3(256), 0, s, p, slices);
+      e = hipFreeAsync(ws, s);
+      if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "ttm_linear: split-K workspace release: %s", hipGetErrorString(e));
       return 0;
     }
   }
@@ -1270,6 +1360,7 @@ TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype
   p.c_batch = (int64_t)p.Mt * p.Nt * 2048;
   p.m_blocks = (p.Mt + 7) / 8; p.n_blocks = (p.Nt + 7) / 8;
   p.split = 0; p.nt_split = 0; p.ntw_a = 4; p.ntw_b = 4;
+  p.k_slice = p.Kt; p.partial = nullptr;
   TTM_REQUIRE(batch <= 65535, "ttm_linear: batch too large");
   hipStream_t s = (hipStream_t)stream;
   int rc;
