@@ -40,6 +40,32 @@ __global__ __launch_bounds__(256) void ttm_copy_view_k(const T *__restrict__ src
   }
 }
 
+// 16 bytes per lane: the innermost view dimension is contiguous on both sides and everything that positions a
+// group of V = 16 / elem_bytes elements is a multiple of V, so a group never leaves its row or its 16-wide face row
+template <int ELEM>
+__global__ __launch_bounds__(256) void ttm_copy_view_vec_k(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, ViewArgs p,
+                                                           int64_t total) {
+  constexpr int V = 16 / ELEM;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    int64_t rem = i, ls = p.sbase, ld = p.dbase;
+    {
+      const int64_t e = p.extent[p.rank - 1] / V;
+      const int64_t v = rem % e;
+      rem /= e;
+      ls += v * V;
+      ld += v * V;
+    }
+#pragma unroll 1
+    for (int d = p.rank - 2; d >= 0; --d) {
+      int64_t v = rem % p.extent[d];
+      rem /= p.extent[d];
+      ls += v * p.sstride[d];
+      ld += v * p.dstride[d];
+    }
+    dst[phys_offset(ld, p.drows, p.dcols, p.dtiled) / V] = src[phys_offset(ls, p.srows, p.scols, p.stiled) / V];
+  }
+}
+
 TTM_EXPORT int ttm_copy_view(const void *src, int64_t src_rows, int64_t src_cols, int src_layout, void *dst,
                              int64_t dst_rows, int64_t dst_cols, int dst_layout, int elem_bytes, int rank,
                              const int64_t *extent, const int64_t *src_stride, int64_t src_base,
@@ -61,9 +87,26 @@ TTM_EXPORT int ttm_copy_view(const void *src, int64_t src_rows, int64_t src_cols
   p.sbase = src_base; p.dbase = dst_base;
   p.srows = src_rows; p.scols = src_cols; p.drows = dst_rows; p.dcols = dst_cols;
   p.stiled = src_layout == TTM_TILE; p.dtiled = dst_layout == TTM_TILE;
+  hipStream_t s = (hipStream_t)stream;
+  {
+    const int64_t V = 16 / elem_bytes;
+    bool vec = rank >= 1 && src_stride[rank - 1] == 1 && dst_stride[rank - 1] == 1 && extent[rank - 1] % V == 0 &&
+               src_base % V == 0 && dst_base % V == 0 && src_cols % V == 0 && dst_cols % V == 0 &&
+               ((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0;
+    for (int d = 0; vec && d < rank - 1; ++d) vec = src_stride[d] % V == 0 && dst_stride[d] % V == 0;
+    if (vec) {
+      const int64_t groups = total / V;
+      int64_t vblocks = ttm_cdiv(groups, 256);
+      unsigned vgrid = (unsigned)(vblocks > 262144 ? 262144 : vblocks);
+      if (elem_bytes == 4) hipLaunchKernelGGL(ttm_copy_view_vec_k<4>, dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
+      else if (elem_bytes == 2) hipLaunchKernelGGL(ttm_copy_view_vec_k<2>, dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
+      else hipLaunchKernelGGL(ttm_copy_view_vec_k<1>, dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
+      TTM_LAUNCH_CHECK();
+      return TTM_OK;
+    }
+  }
   int64_t blocks = ttm_cdiv(total, 256);
   unsigned grid = (unsigned)(blocks > 262144 ? 262144 : blocks);
-  hipStream_t s = (hipStream_t)stream;
   if (elem_bytes == 4) hipLaunchKernelGGL(ttm_copy_view_k<uint32_t>, dim3(grid), dim3(256), 0, s, (const uint32_t *)src, (uint32_t *)dst, p, total);
   else if (elem_bytes == 2) hipLaunchKernelGGL(ttm_copy_view_k<uint16_t>, dim3(grid), dim3(256), 0, s, (const uint16_t *)src, (uint16_t *)dst, p, total);
   else hipLaunchKernelGGL(ttm_copy_view_k<uint8_t>, dim3(grid), dim3(256), 0, s, (const uint8_t *)src, (uint8_t *)dst, p, total);
