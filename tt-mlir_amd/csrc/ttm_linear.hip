@@ -786,16 +786,18 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   const int kbase = blockIdx.y * p.k_slice, kt_end = min(p.Kt, kbase + p.k_slice);
   const int ksteps = (kt_end - kbase + 1) / 2;
   u32x2 exps = {0, 0}, exps_next = {0, 0};
+  uint32_t keep = 0, keep_next = 0;
   u32x4 fw[2][NTW], fa[2][MB], out[4];
 
-  auto issue_a = [&](int kt0, uint32_t stage_off) {
+  // instructions [i0, i1) of the four that stage this wavefront's 32 activation rows of step kt0
+  auto issue_a = [&](int kt0, uint32_t stage_off, int i0 = 0, int i1 = 4) {
     kt0 += kbase;
     const int kt = min(kt0, p.Kt - 1);
     const uint32_t sub = kt0 + 1 < p.Kt ? 2048u : 0u;   // k tail: the second tile of the pair repeats the first (its weights are zero)
     const uint8_t *base = A + a_row + (int64_t)kt * 2048;
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      lds_dma16(base, dmaA[i] + (dmaA_sub[i] ? sub : 0u), lds0 + stage_off + (uint32_t)(wave * 256 + i * 64) * 16u);
+      if (i >= i0 && i < i1) lds_dma16(base, dmaA[i] + (dmaA_sub[i] ? sub : 0u), lds0 + stage_off + (uint32_t)(wave * 256 + i * 64) * 16u);
   };
   auto issue_raw = [&](int kt0, uint32_t stage_off) {
     if (!converts) return;
@@ -809,12 +811,14 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
       lds_dma16(row, dmaW, lds0 + LDS_RAW + stage_off + (uint32_t)(2 * wave) * 512u);
     }
   };
-  auto load_exps = [&](int kt0) {
+  // exponents of step kt0: the raw load and, separately, the k-tail mask (zero exponents dequantise to zero weights).
+  // The mask is applied when the value is taken into use; masking right behind the load would wait for it, and with
+  // it for every LDS-direct load issued before.
+  auto load_exps = [&](int kt0, uint32_t &keep) {
     kt0 += kbase;
     const int kt = min(kt0 + ukt, p.Kt - 1);
-    const uint32_t keep = kt0 + ukt >= kt_end ? 0u : 0xFFFFFFFFu;   // k tail: zero exponents dequantise to zero weights
-    u32x2 e = *(const u32x2 *)(W + (int64_t)kt * p.Nt * W_TILE + offWe);
-    return u32x2{e.x & keep, e.y & keep};
+    keep = kt0 + ukt >= kt_end ? 0u : 0xFFFFFFFFu;
+    return *(const u32x2 *)(W + (int64_t)kt * p.Nt * W_TILE + offWe);
   };
   auto fetch = [&](int s2, uint32_t so, u32x4 (&w)[NTW], u32x4 (&a)[MB]) {
 #pragma unroll
@@ -864,7 +868,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
 #pragma unroll
     for (int i = 0; i < NTW * MB; ++i) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 40 / (NTW * MB), 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 32 / (NTW * MB), 0);
     }
   };
   auto landed_barrier = [&]() {
@@ -876,15 +880,17 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   issue_a(0, 0);
   issue_raw(0, 0);
   issue_raw(2, RAW_STAGE);
-  exps = load_exps(0);
+  exps = load_exps(0, keep);
   landed_barrier();
+  exps = u32x2{exps.x & keep, exps.y & keep};
 #pragma unroll
   for (int c = 0; c < 4; ++c) quarter(c, 0, 0);
-  exps = load_exps(2);
+  exps = load_exps(2, keep);
   landed_barrier();            // weights of step 0 visible, raw stage 0 free
+  exps = u32x2{exps.x & keep, exps.y & keep};
   issue_a(2, STAGE);
   issue_raw(4, 0);
-  exps_next = load_exps(4);
+  exps_next = load_exps(4, keep_next);
   fetch(0, 0, fw[0], fa[0]);
   quarter(0, RAW_STAGE, STAGE);
 
@@ -899,17 +905,21 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     constexpr uint32_t RCUR = decltype(stage_c)::value * RAW_STAGE, RNXT = RAW_STAGE - RCUR;
 #pragma unroll
     for (int q = 0; q < 3; ++q) {
+      // the global-memory pipe takes about 16 cycles per LDS-direct instruction: the activation loads of a step are
+      // spread over three chunks (1 + 2 + 1) so that no wavefront queues behind the whole block's burst
+      if (q == 0 && ks > 0) issue_a((ks + 1) * 2, NXT, 1, 3);
+      if (q == 1 && ks > 0) issue_a((ks + 1) * 2, NXT, 3, 4);
       fetch(q + 1, CUR, fw[(q + 1) & 1], fa[(q + 1) & 1]);
       quarter(q + 1, RNXT, NXT);
       mfma_chunk(q & 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    exps = exps_next;
     landed_barrier();
+    exps = u32x2{exps_next.x & keep_next, exps_next.y & keep_next};
     // stage CUR of the activations and stage RNXT of the mantissas are free now
-    exps_next = load_exps((ks + 3) * 2);
-    issue_a((ks + 2) * 2, CUR);
+    exps_next = load_exps((ks + 3) * 2, keep_next);
     issue_raw((ks + 3) * 2, RNXT);
+    issue_a((ks + 2) * 2, CUR, 0, 1);
     fetch(0, NXT, fw[0], fa[0]);
     quarter(0, RCUR, CUR);
     mfma_chunk(1);
