@@ -8,15 +8,19 @@
 // input (columns = m), so a lane's four accumulator registers of one group are four consecutive
 // n of one m: an 8-byte store into the output face row, and bias is a per-register constant.
 //
-// LDS image (both operands): [row][8 chunks of 8 k] with chunk index XOR (row & 7); a fragment
-// read is one ds_read_b128 per lane and is bank-conflict free.
+// LDS image (both operands): [row][8 chunks of 8 k] with the chunk slot XOR-swizzled by the row (lds_swz);
+// a fragment read is one ds_read_b128 per lane and is bank-conflict free.
 //
-// Weight dequantisation (bfp8_b).  A lane owns an 8(k) x 8(n) block: eight 8-byte row loads plus the
-// eight row exponents.  Sign-magnitude bytes are turned into offset-binary bytes with packed
-// integer ops (t = 128 +- mag), so an element is cvt_f32_ubyte + one fma:
+// Weight dequantisation (bfp8_b).  A lane owns an 8 (k) x 4 (n) block (8 x 8 in the fallback and small-M
+// kernels): eight row words plus the eight row exponents.  Sign-magnitude bytes are turned into
+// offset-binary bytes with packed integer ops (t = 128 +- mag), so an element is cvt_f32_ubyte + one fma:
 //     w = t * 2^(E-133) - 128 * 2^(E-133)          (exact)
 // and pairs along k are packed to bf16 by taking the high halves (exact: 7 significant bits).
-// Rows whose shared exponent is below 7 (|w| < 2^-120) are flushed towards zero.
+// Rows whose shared exponent is below 7 (|w| < 2^-120) are flushed to zero.
+//
+// Kernels, by use: ttm_linear_dma_k (block-float weights, M > 64), ttm_linear_reg_k (bf16 weights, M > 64),
+// ttm_linear_big_k (64-bit-addressed fallback), ttm_linear_decode_bfp8_k / ttm_linear_small_k (M <= 64),
+// ttm_linear_reduce_k (second half of a split-K launch).
 #include <type_traits>
 
 #include "ttm_common.h"
@@ -914,8 +918,8 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
 
   // ---- rotated pipeline.  A step is four chunks of 16 k.  Chunk q multiplies, requests the fragments of the
   // following chunk and converts weight rows 2c, 2c+1 with c = (q + 1) % 4; the scheduler is asked to put the
-  // conversion's VALU instructions behind the MFMAs, five apiece, which is what the matrix core leaves free
-  // on the issue port.  The block barrier sits between chunks 2 and 3: chunk 3 multiplies from fragments that
+  // conversion's VALU instructions behind the MFMAs, four apiece (the matrix core leaves five to six slots free
+  // on the issue port).  The block barrier sits between chunks 2 and 3: chunk 3 multiplies from fragments that
   // were requested before the barrier and already requests chunk 0 of the next stage, so the matrix core does
   // not drain at the barrier; its conversion quarter (c = 0) belongs to the step after next.
 #ifdef TTM_LINEAR_TRACE
