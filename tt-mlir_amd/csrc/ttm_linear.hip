@@ -40,7 +40,7 @@ struct LinearArgs {
   int act, bias_tiled;
   int64_t a_batch, w_batch, c_batch;  // byte strides between batch entries (w_batch 0 = shared weights)
   int m_blocks, n_blocks;
-  int split, nt_split, ntw_a, ntw_b;  // two-part grid of the block-float main kernel
+  int ntw;                            // block-float main kernel: column tiles per wavefront (block width / 2)
   int k_slice;                        // k-tiles per grid.y slice (split-K); Kt when the reduction is not split
   float *partial;                     // split-K: fp32 partial sums [slices][Mt * Nt * 1024] in output tile order
 };
@@ -972,19 +972,11 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   else linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wn * NTW, nt_end, lane);
 }
 
-// The grid is split in two parts so that the last, partly filled round of blocks can use narrower blocks:
-// blocks [0, split) cover column tiles [0, nt_split) with 2 ntw_a tiles per block, the rest covers
-// [nt_split, Nt) with 2 ntw_b tiles per block.
 template <int WF>
 __global__ __launch_bounds__(512) void ttm_linear_dma_k(LinearArgs p) {
-  const bool first = (int)blockIdx.x < p.split;
-  const int ntw = first ? p.ntw_a : p.ntw_b;
-  const int bid = first ? blockIdx.x : blockIdx.x - p.split;
-  const int nblk = first ? p.split : (int)gridDim.x - p.split;
-  const int nt_first = first ? 0 : p.nt_split, nt_end = first ? p.nt_split : p.Nt;
-  if (ntw == 4) linear_dma_block<WF, 4>(p, bid, nblk, nt_first, nt_end);
-  else if (ntw == 3) linear_dma_block<WF, 3>(p, bid, nblk, nt_first, nt_end);
-  else linear_dma_block<WF, 2>(p, bid, nblk, nt_first, nt_end);
+  if (p.ntw == 4) linear_dma_block<WF, 4>(p, blockIdx.x, gridDim.x, 0, p.Nt);
+  else if (p.ntw == 3) linear_dma_block<WF, 3>(p, blockIdx.x, gridDim.x, 0, p.Nt);
+  else linear_dma_block<WF, 2>(p, blockIdx.x, gridDim.x, 0, p.Nt);
 }
 
 // =============================================================================================
@@ -1261,33 +1253,31 @@ static int device_cu_count() {
   return cus;
 }
 
-// Grid of the block-float main kernel.  Whole rounds (one block per CU) use 8-tile-wide blocks.  What is left may
-// use narrower blocks (6 or 4 column tiles) when that fills more CUs: a narrower block keeps the whole activation
-// traffic of a wide one, so its measured time is 0.92 (6 tiles) and 0.78 (4 tiles) of it, and it is only chosen
-// when the estimate (block time x rounds) beats the wide block by more than 15 %.
-static void plan_dma_grid(LinearArgs &p, int cus, int force_ntw) {
-  const int mbk = p.m_blocks;
-  auto blocks_for = [&](int nt, int ntw) { return mbk * ((nt + 2 * ntw - 1) / (2 * ntw)); };
-  p.ntw_a = 4;
-  p.nt_split = 0;
-  if (force_ntw == 0 && mbk <= cus && cus % mbk == 0) {
-    const int per_round = cus / mbk;                 // column blocks per round
-    p.nt_split = (p.Nt / 8 / per_round) * per_round * 8;
-  }
-  p.split = mbk * (p.nt_split / 8);
-  const int rest = p.Nt - p.nt_split;
-  p.ntw_b = 4;
-  if (force_ntw >= 2 && force_ntw <= 4) p.ntw_b = force_ntw;
-  else {
-    static const int block_time[5] = {0, 0, 78, 92, 100};
-    const int wide = block_time[4] * ((blocks_for(rest, 4) + cus - 1) / cus);
-    int best = wide * 85 / 100;
-    for (int ntw = 3; ntw >= 2; --ntw) {
-      const int cost = block_time[ntw] * ((blocks_for(rest, ntw) + cus - 1) / cus);
-      if (cost < best) { best = cost; p.ntw_b = ntw; }
+// Grid of the block-float main kernel: block width (8, 6 or 4 column tiles) and number of k-slices, chosen by a
+// small cost model fitted to measurements on the config shapes.  A block costs (k-steps + 12) x 1.65 us at full width
+// (the 12 stand for prologue and epilogue), 0.92 / 0.78 of that at 6 / 4 tiles (a narrower block keeps the whole
+// activation traffic of a wide one); blocks run in rounds of one per CU; a split reduction adds its fp32 partial
+// traffic, (slices + 0.5) x M x N x 4 bytes, at 4 TB/s.  force_* != 0 pin a choice (tests, measurements).
+static int plan_dma_grid(LinearArgs &p, int cus, int force_ntw, int force_slices) {
+  const int mbk = p.m_blocks, ksteps = (p.Kt + 1) / 2;
+  static const double width_cost[5] = {0, 0, 0.78, 0.92, 1.0};
+  double best = 1e30;
+  int best_ntw = 4, best_slices = 1;
+  for (int ntw = 4; ntw >= 2; --ntw) {
+    if (force_ntw && ntw != force_ntw) continue;
+    const int blocks = mbk * ((p.Nt + 2 * ntw - 1) / (2 * ntw));
+    for (int slices = 1; slices <= 8; slices *= 2) {
+      if (force_slices ? slices != 1 : (slices > 1 && ksteps / slices < 8)) continue;
+      const int rounds = (blocks * slices + cus - 1) / cus;
+      double t = rounds * width_cost[ntw] * ((ksteps + slices - 1) / slices + 12) * 1.65;
+      if (slices > 1) t += (slices + 0.5) * (double)p.Mt * p.Nt * 4096.0 / 4.0e6;
+      if (t < best * 0.97) { best = t; best_ntw = ntw; best_slices = slices; }   // ties go to the wider, unsplit choice
     }
   }
-  p.n_blocks = p.split + (rest > 0 ? blocks_for(rest, p.ntw_b) : 0);   // total blocks of the launch
+  if (force_slices) best_slices = force_slices;
+  p.ntw = best_ntw;
+  p.n_blocks = mbk * ((p.Nt + 2 * best_ntw - 1) / (2 * best_ntw));   // blocks per k-slice
+  return best_slices;
 }
 
 template <typename K>
@@ -1330,17 +1320,11 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       }
       LinearArgs p = a;
       const int cus = device_cu_count();
-      plan_dma_grid(p, cus, ttm_option("linear_ntw"));
-      // split-K when the output alone gives less than half a round of blocks and the reduction is long
-      int slices = ttm_option("linear_split_k");
-      if (slices == 0) {
-        slices = 1;
-        const int ksteps = (a.Kt + 1) / 2;
-        while (slices < 8 && p.n_blocks * slices * 2 <= cus && ksteps / (slices * 2) >= 16) slices *= 2;
-      }
+      int slices = plan_dma_grid(p, cus, ttm_option("linear_ntw"), ttm_option("linear_split_k"));
       slices = slices < 1 ? 1 : (slices > a.Kt ? a.Kt : slices);
       if (slices > 1) {
         p.k_slice = (a.Kt + slices - 1) / slices;
+        p.k_slice += p.k_slice & 1;                         // whole k-steps per slice
         slices = (a.Kt + p.k_slice - 1) / p.k_slice;
       }
       if (slices <= 1) {
@@ -1349,6 +1333,16 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       }
       const int64_t per = (int64_t)a.Mt * a.Nt * 1024;
       void *ws = nullptr;
+      static bool pool_kept = false;
+      if (!pool_kept) {   // keep freed workspace memory in the stream-ordered pool instead of returning it at every sync
+        int dev = 0;
+        hipMemPool_t pool;
+        uint64_t keep = UINT64_MAX;
+        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess)
+          (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
+        (void)hipGetLastError();
+        pool_kept = true;
+      }
       hipError_t e = hipMallocAsync(&ws, (size_t)(per * slices * batch) * sizeof(float), s);
       if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "ttm_linear: split-K workspace: %s", hipGetErrorString(e));
       p.partial = (float *)ws;
@@ -1404,7 +1398,7 @@ TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype
   p.w_batch = w_batch == 1 ? 0 : (int64_t)p.Kt * p.Nt * w_tile;
   p.c_batch = (int64_t)p.Mt * p.Nt * 2048;
   p.m_blocks = (p.Mt + 7) / 8; p.n_blocks = (p.Nt + 7) / 8;
-  p.split = 0; p.nt_split = 0; p.ntw_a = 4; p.ntw_b = 4;
+  p.ntw = 4;
   p.k_slice = p.Kt; p.partial = nullptr;
   TTM_REQUIRE(batch <= 65535, "ttm_linear: batch too large");
   hipStream_t s = (hipStream_t)stream;
