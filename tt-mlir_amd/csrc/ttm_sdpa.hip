@@ -66,28 +66,44 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
   // number of key tiles any wave of this workgroup needs
   int kt_end = p.skt;
   if (p.causal) kt_end = min(kt_end, (min(qb * 4 + 4, p.sqt) * 32 + 31) / 32);
+  // K and V blocks travel global -> registers -> LDS; the loads of block kt + 1 are issued before block kt is
+  // computed, so their latency hides behind the MFMA and softmax work
+  constexpr int NC = (DT * 128 + 255) / 256;   // 16-byte chunks of a K (or V) block per lane
+  u32x4 kreg[NC], vreg[NC];
+  auto load_block = [&](int kt) {
+    const u32x4 *ks = (const u32x4 *)(p.k + kv_mat + (int64_t)kt * DT * 2048);
+    const u32x4 *vs = (const u32x4 *)(p.v + kv_mat + (int64_t)kt * DT * 2048);
+#pragma unroll
+    for (int i = 0; i < NC; ++i) {
+      if (tid + 256 * i < DT * 128) {
+        kreg[i] = ks[tid + 256 * i];
+        vreg[i] = vs[tid + 256 * i];
+      }
+    }
+  };
+  if (kt_end > 0) load_block(0);
   for (int kt = 0; kt < kt_end; ++kt) {
     __syncthreads();  // previous block fully consumed
-    {
-      // K block: DT tiles, contiguous (32 * D * 2 bytes); copied as is
-      const u32x4 *src = (const u32x4 *)(p.k + kv_mat + (int64_t)kt * DT * 2048);
-      for (int c = tid; c < DT * 128; c += 256) ((u32x4 *)ldsK)[c] = src[c];
-      // V block -> V^T[d][key]
-      const u32x4 *vs = (const u32x4 *)(p.v + kv_mat + (int64_t)kt * DT * 2048);
-      for (int c = tid; c < DT * 128; c += 256) {
-        u32x4 v = vs[c];
-        int tile = c >> 7, cc = c & 127;
-        int face = cc >> 5, row = (cc & 31) >> 1, half = cc & 1;
-        int key = (face >> 1) * 16 + row;
-        int d0 = tile * 32 + (face & 1) * 16 + half * 8;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          ldsV[(d0 + 2 * i) * VPITCH + key] = (uint16_t)(v[i] & 0xFFFF);
-          ldsV[(d0 + 2 * i + 1) * VPITCH + key] = (uint16_t)(v[i] >> 16);
-        }
+    for (int i = 0; i < NC; ++i) {
+      const int c = tid + 256 * i;
+      if (c >= DT * 128) break;
+      // K block: DT tiles, contiguous (32 * D * 2 bytes); copied as is
+      ((u32x4 *)ldsK)[c] = kreg[i];
+      // V block -> V^T[d][key]
+      const u32x4 v = vreg[i];
+      const int tile = c >> 7, cc = c & 127;
+      const int face = cc >> 5, row = (cc & 31) >> 1, half = cc & 1;
+      const int key = (face >> 1) * 16 + row;
+      const int d0 = tile * 32 + (face & 1) * 16 + half * 8;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        ldsV[(d0 + 2 * e) * VPITCH + key] = (uint16_t)(v[e] & 0xFFFF);
+        ldsV[(d0 + 2 * e + 1) * VPITCH + key] = (uint16_t)(v[e] >> 16);
       }
     }
     __syncthreads();
+    if (kt + 1 < kt_end) load_block(kt + 1);
     const bool skip = !wave_ok || (p.causal && kt * 32 > qt * 32 + 31);
     if (skip) continue;
 
@@ -100,49 +116,65 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
       u32x4 kv = *(const u32x4 *)(ldsK + (st >> 1) * 2048 + ((l31 >> 4) * 2 + (st & 1)) * 512 + (l31 & 15) * 32 + hh * 16);
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&kv, qf[st], s, 0, 0, 0);
     }
-    // scale, mask; lane holds q = q_glob, keys kt*32 + 8g + 4hh + r
+    // scale, mask; lane holds q = q_glob, keys kt*32 + 8g + 4hh + r.  Scores are kept in the log2 domain
+    // (scale and mask multiplied by log2 e) so that the exponential is a bare v_exp_f32.
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float scale2 = p.scale * LOG2E;
+    // masking by position is only needed on the diagonal block of a causal pass and on a ragged last block
+    const bool edge = (p.causal && kt * 32 + 31 > qt * 32) || kt * 32 + 32 > p.Sk;   // wavefront-uniform
     float mx = -INFINITY;
+    if (p.mask || edge) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int key0 = kt * 32 + g * 8 + hh * 4;
-      float mk[4] = {0.f, 0.f, 0.f, 0.f};
-      if (p.mask) {
-        const int64_t mm = ((int64_t)b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
-        const int kin = g * 8 + hh * 4;
-        const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
-                            (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
-        u32x2 raw = *(const u32x2 *)mp;
-        mk[0] = __uint_as_float(raw.x << 16); mk[1] = __uint_as_float(raw.x & 0xFFFF0000u);
-        mk[2] = __uint_as_float(raw.y << 16); mk[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+      for (int g = 0; g < 4; ++g) {
+        const int key0 = kt * 32 + g * 8 + hh * 4;
+        float mk[4] = {0.f, 0.f, 0.f, 0.f};
+        if (p.mask) {
+          const int64_t mm = ((int64_t)b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
+          const int kin = g * 8 + hh * 4;
+          const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
+                              (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
+          u32x2 raw = *(const u32x2 *)mp;
+          mk[0] = __uint_as_float(raw.x << 16); mk[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+          mk[2] = __uint_as_float(raw.y << 16); mk[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = fmaf(s[g * 4 + r], scale2, mk[r] * LOG2E);
+          const int key = key0 + r;
+          if (key >= p.Sk || (p.causal && key > q_glob)) v = -INFINITY;
+          s[g * 4 + r] = v;
+          mx = fmaxf(mx, v);
+        }
       }
+    } else {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float v = s[g * 4 + r] * p.scale + mk[r];
-        const int key = key0 + r;
-        if (key >= p.Sk || (p.causal && key > q_glob)) v = -INFINITY;
-        s[g * 4 + r] = v;
-        mx = fmaxf(mx, v);
+      for (int r = 0; r < 16; ++r) {
+        s[r] *= scale2;
+        mx = fmaxf(mx, s[r]);
       }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
     // fully masked so far: keep everything at zero without producing NaN
     const float m_use = m_new == -INFINITY ? 0.0f : m_new;
-    const float alpha = __expf(m_run - m_use);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
     float rs = 0.0f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      float e = __expf(s[r] - m_use);
+      float e = __builtin_amdgcn_exp2f(s[r] - m_use);
       s[r] = e;
       rs += e;
     }
     rs += __shfl_xor(rs, 32);
     l_run = l_run * alpha + rs;
     m_run = m_new;
+    // the running maximum seldom moves after the first blocks: rescale only when some lane needs it
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
 #pragma unroll
-    for (int d = 0; d < DT; ++d)
+      for (int d = 0; d < DT; ++d)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
+        for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
+    }
     // O^T += V^T . P^T, two k16 steps
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
