@@ -38,6 +38,19 @@ __device__ __forceinline__ ChunkPos<ELEM> chunk_pos(int r, int q) {
 }
 
 template <int ELEM>
+__device__ __forceinline__ void unpack_vals(u32x4 v, float (&f)[16 / ELEM]) {
+  if (ELEM == 2) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(v[i] << 16);
+      f[2 * i + 1] = __uint_as_float(v[i] & 0xFFFF0000u);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = __uint_as_float(v[i]);
+  }
+}
+template <int ELEM>
 __device__ __forceinline__ void load_vals(const void *base, int64_t off, float (&f)[16 / ELEM]) {
   u32x4 v = *(const u32x4 *)((const uint8_t *)base + off * ELEM);
   if (ELEM == 2) {
@@ -178,9 +191,102 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
   }
 }
 
+// RMSNorm / softmax for rows of up to 16 chunks per lane (4096 bf16 or 2048 fp32 columns): 8 rows per workgroup,
+// 32 lanes per row.  The row slice of a lane is read from global memory once and parked in LDS (64 KiB per
+// workgroup, each lane reads back only what it wrote, so no barrier is involved) for the output pass.  The loops
+// are kept rolled (8 loads in flight per lane): fully unrolled, the once-executed code ran at instruction-fetch speed.
+template <int MODE, int ELEM>
+__global__ __launch_bounds__(256) void ttm_rowwise_resident_k(RowArgs p) {
+  constexpr int EPC = 16 / ELEM, RPB = 8, J = 32, NQ = 16;
+  __shared__ u32x4 park[NQ * 256];
+  __shared__ float part[J][RPB];
+  __shared__ float part2[J][RPB];
+  const int tid = threadIdx.x, j = tid / RPB, rl = tid % RPB;
+  const int r = (int)(blockIdx.x % 4) * RPB + rl;
+  const int trow = (int)(blockIdx.x / 4);
+  const int row = (trow % p.rt) * 32 + r;
+  const bool row_ok = row < p.rows;
+  const int nq = p.ct * 2 * ELEM;
+  const uint8_t *x = (const uint8_t *)p.x + (int64_t)trow * p.ct * 1024 * ELEM;
+  uint8_t *o = (uint8_t *)p.out + (int64_t)trow * p.ct * 1024 * ELEM;
+  const int cols = (int)p.cols;
+  const int nk = (nq - j + J - 1) / J;   // chunks of this lane
+  float acc = MODE == RW_SOFTMAX ? -INFINITY : 0.0f;
+#pragma unroll 8
+  for (int k = 0; k < nk; ++k) {
+    const ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, j + k * J);
+    const u32x4 v = *(const u32x4 *)(x + cp.off * ELEM);
+    park[k * 256 + tid] = v;
+    float f[EPC];
+    unpack_vals<ELEM>(v, f);
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) {
+      const bool ok = cp.c0 + i < cols;
+      if (MODE == RW_RMSNORM) acc += ok ? f[i] * f[i] : 0.0f;
+      else acc = ok ? fmaxf(acc, f[i]) : acc;
+    }
+  }
+  part[j][rl] = acc;
+  __syncthreads();
+  float stat = part[0][rl];
+#pragma unroll
+  for (int k = 1; k < J; ++k) stat = MODE == RW_SOFTMAX ? fmaxf(stat, part[k][rl]) : stat + part[k][rl];
+  float mul = 0.0f;
+  if (MODE == RW_RMSNORM) mul = 1.0f / sqrtf(stat / (float)cols + p.eps);
+  else {
+    float sum = 0.0f;
+#pragma unroll 4
+    for (int k = 0; k < nk; ++k) {
+      const int c0 = chunk_pos<ELEM>(r, j + k * J).c0;
+      float f[EPC];
+      unpack_vals<ELEM>(park[k * 256 + tid], f);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) sum += c0 + i < cols ? expf(f[i] - stat) : 0.0f;
+    }
+    part2[j][rl] = sum;
+    __syncthreads();
+    float tot = 0.0f;
+#pragma unroll
+    for (int k = 0; k < J; ++k) tot += part2[k][rl];
+    mul = 1.0f / tot;
+  }
+#pragma unroll 4
+  for (int k = 0; k < nk; ++k) {
+    const ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, j + k * J);
+    float f[EPC], w[EPC], b[EPC];
+    unpack_vals<ELEM>(park[k * 256 + tid], f);
+    if (MODE == RW_RMSNORM) {
+      if (p.w) load_vec<ELEM>(p.w, p.w_tiled, cp.c0, w);
+      if (p.b) load_vec<ELEM>(p.b, p.b_tiled, cp.c0, b);
+    }
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) {
+      float v;
+      if (MODE == RW_RMSNORM) {
+        v = f[i] * mul;
+        if (p.w) v *= w[i];
+        if (p.b) v += b[i];
+      } else {
+        v = expf(f[i] - stat) * mul;
+      }
+      f[i] = (row_ok && cp.c0 + i < cols) ? v : 0.0f;
+    }
+    store_vals<ELEM>(o, cp.off, f);
+  }
+}
+
 template <int MODE>
 static int launch_rowwise(const RowArgs &p, int dtype, int64_t trows, hipStream_t s) {
   TTM_REQUIRE(trows < (1ll << 29), "row-wise kernel: tensor too large");
+  if constexpr (MODE == RW_RMSNORM || MODE == RW_SOFTMAX) {
+    const int elem = dtype == TTM_BF16 ? 2 : 4;
+    if (p.ct * 2 * elem <= 16 * 32) {   // a lane's share of the row fits in registers
+      if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_resident_k<MODE, 2>), dim3((unsigned)trows * 4), dim3(256), 0, s, p);
+      else hipLaunchKernelGGL((ttm_rowwise_resident_k<MODE, 4>), dim3((unsigned)trows * 4), dim3(256), 0, s, p);
+      TTM_LAUNCH_CHECK();
+      return TTM_OK;
+    }
+  }
   if (trows >= 1024) {   // enough tile rows to fill the device with one workgroup each
     if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_k<MODE, 2, 32>), dim3((unsigned)trows), dim3(256), 0, s, p);
     else hipLaunchKernelGGL((ttm_rowwise_k<MODE, 4, 32>), dim3((unsigned)trows), dim3(256), 0, s, p);
