@@ -200,3 +200,21 @@ def test_split_k_is_chosen_for_long_skinny_reductions(hip, dev, orc, metrics):
     got, w_eff = run_linear(hip, dev, a, w, None, None, hip.BFP8B)
     # |y| ~ 0.02 * sqrt(8192) ~ 1.8: one bf16 ulp below 4 is 2^-6; allow 2^-5
     check(orc, metrics, got, a, w_eff, None, None, max_abs=2.0 ** -5)
+
+
+@pytest.mark.parametrize("split", [0, 2])
+def test_batched_block_float_matmul(hip, dev, orc, metrics, split):
+    """Batched contraction with per-batch bfp8_b weights and with one shared weight matrix, with and without
+    a split reduction (the fp32 partials are laid out per batch entry and k-slice)."""
+    a = datagen.randn((3, 96, 160), seed=31, dtype=torch.bfloat16)
+    w = datagen.randn((3, 160, 96), seed=32, std=0.1)
+    hip.set_option("linear_split_k", split)
+    try:
+        got, w_eff = run_linear(hip, dev, a, w, None, None, hip.BFP8B)
+        check(orc, metrics, got, a, w_eff, None, None, max_abs=2.0 ** -5)
+        w1 = datagen.randn((1, 160, 96), seed=33, std=0.1)
+        got, w_eff = run_linear(hip, dev, a, w1, None, None, hip.BFP8B)
+    finally:
+        hip.set_option("linear_split_k", 0)
+    want = orc.round_bf16(orc.matmul(a.float().numpy(), w_eff.numpy()))
+    assert np.max(np.abs(got.float().numpy() - want)) <= 2.0 ** -5
