@@ -49,6 +49,13 @@ int ttrt_binary_tensor_desc(const ttrt_binary *bin, uint32_t program, int is_out
                             int *rank, ttrt_layout *layout);
 int ttrt_binary_ops_text(const ttrt_binary *bin, uint32_t program, char *buf, size_t len);
 int ttrt_binary_info(const ttrt_binary *bin, char *identifier5, char *version, size_t version_len);
+/* JSON views of one program: which = 0 inputs, 1 outputs, 2 operations (Binary::getProgram{Inputs,Outputs,Ops}AsJson,
+ * runtime/lib/binary.cpp:197-224).  Returns the length needed (without the terminator) in *needed; buf may be NULL. */
+int ttrt_binary_program_json(const ttrt_binary *bin, uint32_t program, int which, char *buf, size_t len, size_t *needed);
+/* Embedded golden tensor of the operation at location `loc` on device 0 (Binary::getDebugInfoGolden, binary.cpp:233-253):
+ * *found = 0 when there is none.  shape receives up to 8 extents; *data points into the binary. */
+int ttrt_binary_golden(const ttrt_binary *bin, const char *loc, int *found, int64_t *shape, int *rank, int *dtype,
+                       const uint8_t **data, size_t *size, char *name, size_t name_len);
 
 /* ---- Device: getNumAvailableDevices / openMeshDevice / closeMeshDevice (runtime.h:151-157) */
 int ttrt_num_devices(uint32_t *n);
@@ -86,6 +93,8 @@ typedef void (*ttrt_op_callback)(uint32_t op_index, const char *op_name, const c
 int ttrt_set_post_op_callback(ttrt_op_callback cb, void *user);
 int ttrt_clear_callbacks(void);
 int ttrt_hook_output(void *hook_ctx, ttrt_tensor **out);
+/* location string of the operation a hook is running for (getOpLocInfo, runtime.h) */
+int ttrt_hook_loc(void *hook_ctx, char *buf, size_t len);
 int ttrt_stat(const char *name, int64_t *value);
 int ttrt_stats_clear(void);
 
@@ -129,6 +138,10 @@ int ttrt_pb_constant(ttrt_builder *pb, const void *data, size_t bytes, int in_dt
                      const ttrt_layout *layout, uint32_t *out);
 int ttrt_pb_full(ttrt_builder *pb, const uint32_t *shape, int rank, float value, int dtype, int layout, uint32_t *out);
 int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force);
+/* location of the operation added last, and an expected (golden) tensor to embed for a location; data is row-major */
+int ttrt_pb_last_op_loc(ttrt_builder *pb, char *buf, size_t len);
+int ttrt_pb_golden(ttrt_builder *pb, const char *loc, const char *name, const void *data, size_t bytes, const int64_t *shape,
+                   int rank, int dtype);
 /* out_shapes: n_out entries of 8 extents each, out_ranks / out_layouts per entry */
 int ttrt_pb_load_cached(ttrt_builder *pb, uint32_t program_index, const char *callee, const uint32_t *ins, int n_in,
                         const uint32_t *out_shapes, const int *out_ranks, const ttrt_layout *out_layouts, int n_out,

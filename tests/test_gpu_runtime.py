@@ -97,15 +97,21 @@ def test_c3_linear_program_and_const_eval_cache(device, orc, metrics):
     assert not torch.equal(y1, y3)
 
 
-def oracle_mlp(orc, x, nw, wg, wu, wd, eps):
+def oracle_mlp_stages(orc, x, nw, wg, wu, wd, eps):
     r = orc.round_bf16
     q8 = lambda w: orc.bfp_unpack(orc.bfp_pack(w, 8), w.shape, 8)
     q4 = lambda w: orc.bfp_unpack(orc.bfp_pack(w, 4), w.shape, 4)
-    h = r(orc.rms_norm(x, nw, None, eps))
-    g = r(orc.linear(h, q8(wg), None, "silu"))
-    u = r(orc.linear(h, q8(wu)))
-    m = r(orc.binary("multiply", g, u))
-    return r(orc.linear(m, q4(wd)))
+    st = {}
+    st["norm"] = h = r(orc.rms_norm(x, nw, None, eps))
+    st["gate"] = g = r(orc.linear(h, q8(wg), None, "silu"))
+    st["up"] = u = r(orc.linear(h, q8(wu)))
+    st["product"] = m = r(orc.binary("multiply", g, u))
+    st["down"] = r(orc.linear(m, q4(wd)))
+    return st
+
+
+def oracle_mlp(orc, x, nw, wg, wu, wd, eps):
+    return oracle_mlp_stages(orc, x, nw, wg, wu, wd, eps)["down"]
 
 
 def test_c4_mlp_program_small(device, orc, metrics):
@@ -236,6 +242,29 @@ def test_post_op_hook_sees_intermediates(device, orc):
     want = orc.round_bf16(orc.rms_norm(d["x"].float().numpy(), d["norm_w"].float().numpy(), None, 1e-5))
     assert np.max(np.abs(rms.float().numpy() - want)) <= 2.0 ** -6
     assert [t is None for _, n, t in seen if n == "DeallocateOp"] == [True, True, True]
+
+
+def test_embedded_goldens_are_checked_per_operation(device, orc):
+    """`ttrt run --enable-golden` flow: every op with a golden embedded in the binary is compared in the post-op hook."""
+    d = datagen.c4_mlp(64, 128, 256, seed=11)
+    f = lambda t: t.float().numpy()
+    st = oracle_mlp_stages(orc, f(d["x"]), f(d["norm_w"]), f(bf(d["wg"])), f(bf(d["wu"])), f(bf(d["wd"])), 1e-5)
+    binary = rt.Binary.load_from_memory(programs.c4_mlp(64, 128, 256, goldens=st))
+    tins = [d["x"], d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    (y,), report = harness.execute(binary, 1, tins, device, enable_golden=True)
+    assert sorted(v["name"] for v in report.values()) == sorted(st)
+    assert [v["op"] for v in report.values()] == ["RMSNormOp", "LinearOp", "MatmulOp", "EltwiseBinaryOp", "MatmulOp"]
+    for loc, v in report.items():
+        assert v["pass"] and v["pcc"] >= 0.999, (loc, v)
+    assert np.max(np.abs(f(y) - st["down"])) == report[[k for k, v in report.items() if v["name"] == "down"][0]]["max_abs"]
+    # a wrong golden is reported as a failure for that op only
+    bad = dict(st)
+    bad["up"] = -st["up"]
+    binary = rt.Binary.load_from_memory(programs.c4_mlp(64, 128, 256, goldens=bad))
+    _, report = harness.execute(binary, 1, tins, device, enable_golden=True)
+    assert {v["name"]: v["pass"] for v in report.values()} == dict(norm=True, gate=True, up=False, product=True, down=True)
+    # the hook is gone afterwards
+    harness.execute(binary, 1, tins, device)
 
 
 def test_submit_errors(device):

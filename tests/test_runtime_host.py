@@ -54,6 +54,76 @@ def test_const_eval_program_structure():
                    "DeallocateOp"]
 
 
+def test_json_views_of_a_program():
+    b = rt.Binary.load_from_memory(programs.c4_mlp(tokens=64, hidden=128, ffn=256))
+    ins = b.get_program_inputs_as_json(1)
+    assert [t["desc"]["shape"] for t in ins] == [[64, 128], [128], [128, 256], [128, 256], [256, 128]]
+    md = ins[0]["desc"]["layout"]["memory_desc"]
+    assert md["data_type"] == "BFloat16" and md["tile_shape"] == {"y": 32, "x": 32} and md["storage_type"] == "DRAM"
+    assert len({t["global_id"] for t in ins}) == 5
+    outs = b.get_program_outputs_as_json(1)
+    assert [t["desc"]["shape"] for t in outs] == [[64, 128]]
+    assert [t["desc"]["layout"]["memory_desc"]["data_type"] for t in b.get_program_outputs_as_json(0)] == [
+        "BFP_BFloat8", "BFP_BFloat8", "BFP_BFloat4"]
+    ops = b.get_program_ops_as_json(1)
+    text = b.get_program_ops_as_text(1).strip().splitlines()
+    assert [o["type_type"] for o in ops] == [l.split()[1] for l in text]
+    assert all(set(o) == {"type_type", "debug_info", "loc_info"} for o in ops)
+    assert [o["loc_info"] for o in ops] == ['loc("c4_mlp"("op%d"))' % i for i in range(len(ops))]
+    with pytest.raises(RuntimeError, match="out of range"):
+        b.get_program_ops_as_json(5)
+
+
+def test_embedded_goldens_round_trip():
+    """DebugInfo.golden_info (include/ttmlir/Target/Common/debug_info.fbs:6-26) written by the builder and read back."""
+    pb = rt.ProgramBuilder()
+    pb.begin_program("g")
+    a, w = pb.input((32, 64), DT.BFloat16), pb.input((64, 32), DT.BFloat16)
+    c = pb.matmul(a, w)
+    loc_mm = pb.last_op_loc()
+    r = pb.unary(programs.UNARY["relu"], c)
+    loc_relu = pb.last_op_loc()
+    assert (loc_mm, loc_relu) == ('loc("g"("op0"))', 'loc("g"("op1"))')
+    want = np.linspace(-4, 4, 32 * 32, dtype=np.float32).reshape(32, 32)
+    bits = (want.view(np.uint32) >> 16).astype(np.uint16)
+    pb.golden(loc_mm, bits, DT.BFloat16, "product")
+    pb.golden(loc_relu, np.array([[1.5, -2.25, 3.0]], dtype=np.float32), DT.Float32, "relu")
+    pb.golden("input_0", np.arange(6, dtype=np.int32).reshape(1, 2, 3), DT.Int32)
+    pb.output(r)
+    pb.end_program()
+    b = rt.Binary.load_from_memory(pb.finish())
+    name, got = b.get_debug_info_golden(loc_mm)
+    assert name == "product" and got.dtype == np.float32 and got.shape == (32, 32)
+    assert np.array_equal(got.view(np.uint32), bits.astype(np.uint32) << 16)
+    name, got = b.get_debug_info_golden(loc_relu)
+    assert name == "relu" and np.array_equal(got, np.array([[1.5, -2.25, 3.0]], dtype=np.float32))
+    name, got = b.get_debug_info_golden("input_0")
+    assert name == "" and got.dtype == np.int32 and np.array_equal(got, np.arange(6).reshape(1, 2, 3))
+    assert b.get_debug_info_golden('loc("g"("op7"))') is None
+    # binaries without debug info answer "no golden" rather than failing
+    assert rt.Binary.load_from_memory(programs.c1_matmul()).get_debug_info_golden(loc_mm) is None
+    # golden with a byte count that does not match shape x dtype is refused when it is recorded
+    with pytest.raises(RuntimeError, match="golden"):
+        pb2 = rt.ProgramBuilder()
+        pb2.begin_program("h")
+        pb2.golden("x", np.zeros(5, dtype=np.uint8), DT.Float32)
+
+
+def test_program_goldens_option_marks_each_stage():
+    st = {k: np.full(s, i + 1, dtype=np.float32) for i, (k, s) in enumerate(
+        dict(norm=(64, 128), gate=(64, 256), up=(64, 256), product=(64, 256), down=(64, 128)).items())}
+    b = rt.Binary.load_from_memory(programs.c4_mlp(64, 128, 256, goldens=st))
+    ops = b.get_program_ops_as_json(1)
+    found = {}
+    for o in ops:
+        g = b.get_debug_info_golden(o["loc_info"])
+        if g is not None:
+            found[g[0]] = (o["type_type"], g[1])
+    assert {k: v[0] for k, v in found.items()} == dict(norm="RMSNormOp", gate="LinearOp", up="MatmulOp", product="EltwiseBinaryOp",
+                                                        down="MatmulOp")
+    assert all(np.array_equal(found[k][1], st[k]) for k in st)
+
+
 def test_decoder_program_shapes():
     b = rt.Binary.load_from_memory(programs.c5_decoder(seq=64, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512))
     assert b.get_program_outputs(1)[0][0] == (1, 64, 256)

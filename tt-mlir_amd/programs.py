@@ -7,6 +7,8 @@ program reached through ttcore.load_cached (TTNNWeightDtypeConversion.cpp:102-13
 test/ttmlir/Silicon/TTNN/n150/mixed_precision/linear.mlir:9); inputs are expected in
 Device / Tile / bf16 layout, which callers obtain with to_layout(get_layout(...)).
 """
+import numpy as np
+
 from . import runtime as rt
 
 DT, TL, ST = rt.DataType, rt.TensorLayout, rt.StorageType
@@ -61,20 +63,36 @@ def c3_linear(M, K=4096, N=14336, weight_dtype=DT.BFP_BFloat8, activation="gelu"
     return pb.finish()
 
 
-def _mlp(pb, x, norm_w, wg, wu, wd, eps):
+def _bf16_bits(a):
+    """float32 array -> bf16 bit patterns, round to nearest even."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def _mlp(pb, x, norm_w, wg, wu, wd, eps, goldens=None):
+    """goldens: optional {"norm" | "gate" | "up" | "product" | "down": float32 array}; each is embedded as the
+    expected bf16 output of the operation that computes it (DebugInfo.golden_info, keyed by the op's location)."""
+    def mark(key):
+        if goldens and key in goldens:
+            pb.golden(pb.last_op_loc(), _bf16_bits(goldens[key]), DT.BFloat16, key)
     h = pb.rms_norm(x, norm_w, 0, eps)
+    mark("norm")
     g = pb.linear(h, wg, 0, activation="silu")
+    mark("gate")
     u = pb.matmul(h, wu)
+    mark("up")
     m = pb.binary(BINARY["multiply"], g, u)
+    mark("product")
     pb.deallocate(g)
     pb.deallocate(u)
     d = pb.matmul(m, wd)
+    mark("down")
     pb.deallocate(m)
     return d
 
 
-def c4_mlp(tokens=512, hidden=4096, ffn=14336, eps=1e-5):
-    """Config 4: RMSNorm -> gate/up (bfp8_b) -> SiLU(gate)*up -> down (bfp4_b)."""
+def c4_mlp(tokens=512, hidden=4096, ffn=14336, eps=1e-5, goldens=None):
+    """Config 4: RMSNorm -> gate/up (bfp8_b) -> SiLU(gate)*up -> down (bfp4_b).  goldens: see _mlp."""
     pb = rt.ProgramBuilder()
     ce, ce_outs = _consteval_pack(pb, "c4_mlp_const_eval_0", [((hidden, ffn), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8),
                                                              ((ffn, hidden), DT.BFP_BFloat4)])
@@ -83,7 +101,7 @@ def c4_mlp(tokens=512, hidden=4096, ffn=14336, eps=1e-5):
     nw = pb.input((hidden,), DT.BFloat16)
     wg, wu, wd = pb.input((hidden, ffn), DT.BFloat16), pb.input((hidden, ffn), DT.BFloat16), pb.input((ffn, hidden), DT.BFloat16)
     qg, qu, qd = pb.load_cached(ce, "c4_mlp_const_eval_0", [wg, wu, wd], ce_outs)
-    pb.output(_mlp(pb, x, nw, qg, qu, qd, eps))
+    pb.output(_mlp(pb, x, nw, qg, qu, qd, eps, goldens))
     pb.end_program()
     return pb.finish()
 

@@ -138,6 +138,45 @@ class Binary:
         _call("ttrt_binary_ops_text", self.h, program, buf, 1 << 16)
         return buf.value.decode()
 
+    def _json(self, program, which):
+        import json
+        need = ctypes.c_size_t()
+        _call("ttrt_binary_program_json", self.h, program, which, None, 0, ctypes.byref(need))
+        buf = ctypes.create_string_buffer(need.value + 1)
+        _call("ttrt_binary_program_json", self.h, program, which, buf, need.value + 1, None)
+        return json.loads(buf.value.decode())
+
+    def get_program_inputs_as_json(self, program):
+        """Parsed JSON view of the program's input TensorRefs (Binary.getProgramInputsAsJson)."""
+        return self._json(program, 0)
+
+    def get_program_outputs_as_json(self, program):
+        return self._json(program, 1)
+
+    def get_program_ops_as_json(self, program):
+        """[{type_type, debug_info, loc_info}, ...] (Binary.getProgramOpsAsJson)."""
+        return self._json(program, 2)
+
+    def get_debug_info_golden(self, loc):
+        """Embedded golden tensor for an op location as (name, numpy array) or None (Binary.getDebugInfoGolden).
+        bf16 goldens come back as float32 values."""
+        import numpy as np
+        found, rank, dtype = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        shape = (ctypes.c_int64 * 8)()
+        data, size = ctypes.POINTER(ctypes.c_uint8)(), ctypes.c_size_t()
+        name = ctypes.create_string_buffer(256)
+        _call("ttrt_binary_golden", self.h, loc.encode(), ctypes.byref(found), shape, ctypes.byref(rank), ctypes.byref(dtype),
+              ctypes.byref(data), ctypes.byref(size), name, 256)
+        if not found.value:
+            return None
+        raw = np.ctypeslib.as_array(data, shape=(size.value,)).copy()
+        shp = tuple(shape[: rank.value])
+        if dtype.value == DataType.BFloat16:
+            arr = (raw.view(np.uint16).astype(np.uint32) << 16).view(np.float32).reshape(shp)
+        else:
+            arr = raw.view(_NP_DTYPE[dtype.value]).reshape(shp)
+        return name.value.decode(), arr
+
     def info(self):
         ident, ver = ctypes.create_string_buffer(5), ctypes.create_string_buffer(64)
         _call("ttrt_binary_info", self.h, ident, ver, 64)
@@ -347,6 +386,12 @@ def set_post_op_callback(fn):
             h = ctypes.c_void_p()
             _call("ttrt_hook_output", ctypes.c_void_p(hook), ctypes.byref(h))
             return Tensor(h) if h.value else None
+
+        def get_loc():
+            buf = ctypes.create_string_buffer(512)
+            _call("ttrt_hook_loc", ctypes.c_void_p(hook), buf, 512)
+            return buf.value.decode()
+        get_output.loc = get_loc
         fn(idx, name.decode(), dbg.decode(), get_output)
 
     _cb_keep = _CB_TYPE(tramp)
@@ -400,6 +445,18 @@ class ProgramBuilder:
         shape, rank, lay = (ctypes.c_uint32 * 8)(), ctypes.c_int(), Layout()
         _call("ttrt_pb_tensor_desc", self.h, t, shape, ctypes.byref(rank), ctypes.byref(lay))
         return tuple(shape[: rank.value]), lay
+
+    def last_op_loc(self):
+        buf = ctypes.create_string_buffer(512)
+        _call("ttrt_pb_last_op_loc", self.h, buf, 512)
+        return buf.value.decode()
+
+    def golden(self, loc, array, dtype, name=""):
+        """Embed an expected tensor for the op at `loc`: numpy array (bf16 as uint16 bits) of runtime dtype `dtype`."""
+        import numpy as np
+        a = np.ascontiguousarray(array)
+        shape = (ctypes.c_int64 * max(1, a.ndim))(*a.shape)
+        _call("ttrt_pb_golden", self.h, loc.encode(), name.encode(), a.ctypes.data_as(ctypes.c_void_p), a.nbytes, shape, a.ndim, dtype)
 
     def _op(self, name, *args):
         out = ctypes.c_uint32()

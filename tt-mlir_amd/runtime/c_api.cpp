@@ -99,6 +99,34 @@ TTRT_EXPORT int ttrt_binary_tensor_desc(const ttrt_binary *bin, uint32_t program
 TTRT_EXPORT int ttrt_binary_ops_text(const ttrt_binary *bin, uint32_t program, char *buf, size_t len) {
   return guard([&] { need(bin, "binary"); copyStr(bin->b.getProgramOpsAsText(program), buf, len); });
 }
+TTRT_EXPORT int ttrt_binary_program_json(const ttrt_binary *bin, uint32_t program, int which, char *buf, size_t len, size_t *needed) {
+  return guard([&] {
+    need(bin, "binary");
+    std::string j = which == 0 ? bin->b.getProgramInputsAsJson(program)
+                  : which == 1 ? bin->b.getProgramOutputsAsJson(program)
+                               : bin->b.getProgramOpsAsJson(program);
+    if (needed) *needed = j.size();
+    if (buf && len) copyStr(j, buf, len);
+  });
+}
+TTRT_EXPORT int ttrt_binary_golden(const ttrt_binary *bin, const char *loc, int *found, int64_t *shape, int *rank, int *dtype,
+                                   const uint8_t **data, size_t *size, char *name, size_t name_len) {
+  return guard([&] {
+    need(bin, "binary"); need(loc, "loc"); need(found, "found");
+    auto m = bin->b.getDebugInfoGolden(loc);
+    auto it = m.find(0);
+    *found = it != m.end();
+    if (!*found) return;
+    const GoldenTensorInfo &g = it->second;
+    if (g.shape.size() > 8) throw std::runtime_error("golden tensor rank above 8");
+    if (rank) *rank = static_cast<int>(g.shape.size());
+    if (shape) for (size_t i = 0; i < g.shape.size(); ++i) shape[i] = g.shape[i];
+    if (dtype) *dtype = static_cast<int>(g.dataType);
+    if (data) *data = g.data;
+    if (size) *size = g.size;
+    if (name && name_len) copyStr(g.name, name, name_len);
+  });
+}
 TTRT_EXPORT int ttrt_binary_info(const ttrt_binary *bin, char *identifier5, char *version, size_t version_len) {
   return guard([&] {
     need(bin, "binary");
@@ -225,6 +253,12 @@ TTRT_EXPORT int ttrt_hook_output(void *hook_ctx, ttrt_tensor **out) {
     *out = m.empty() ? nullptr : new ttrt_tensor{m.begin()->second};
   });
 }
+TTRT_EXPORT int ttrt_hook_loc(void *hook_ctx, char *buf, size_t len) {
+  return guard([&] {
+    need(hook_ctx, "hook context");
+    copyStr(getOpLocInfo(static_cast<HookCtx *>(hook_ctx)->oc), buf, len);
+  });
+}
 TTRT_EXPORT int ttrt_stat(const char *name, int64_t *value) {
   return guard([&] { need(name, "name"); need(value, "value"); *value = debug::Stats::get().getStat(name); });
 }
@@ -338,6 +372,16 @@ TTRT_EXPORT int ttrt_pb_full(ttrt_builder *pb, const uint32_t *shape, int rank, 
 }
 TTRT_EXPORT int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force) {
   return guard([&] { need(pb, "builder"); pb->pb.deallocate(in, force != 0); });
+}
+TTRT_EXPORT int ttrt_pb_last_op_loc(ttrt_builder *pb, char *buf, size_t len) {
+  return guard([&] { need(pb, "builder"); copyStr(pb->pb.lastOpLoc(), buf, len); });
+}
+TTRT_EXPORT int ttrt_pb_golden(ttrt_builder *pb, const char *loc, const char *name, const void *data, size_t bytes, const int64_t *shape,
+                               int rank, int dtype) {
+  return guard([&] {
+    need(pb, "builder"); need(loc, "loc"); need(data, "data");
+    pb->pb.golden(loc, name ? name : "", data, bytes, std::vector<std::int64_t>(shape, shape + rank), static_cast<DataType>(dtype));
+  });
 }
 static std::vector<ProgramBuilder::Desc> outDescs(const uint32_t *out_shapes, const int *out_ranks, const ttrt_layout *out_layouts, int n_out) {
   std::vector<ProgramBuilder::Desc> v;

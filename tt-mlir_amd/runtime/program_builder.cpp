@@ -58,6 +58,47 @@ void ProgramBuilder::addOp(OpType type, Off table, const std::string &debug) {
   cur_.ops.push_back(OpRec{static_cast<std::uint8_t>(type), table, debug});
 }
 
+static std::string opLoc(const std::string &program, std::uint32_t index) {
+  return "loc(\"" + program + "\"(\"op" + std::to_string(index) + "\"))";
+}
+
+std::string ProgramBuilder::lastOpLoc() const {
+  if (!open_ || cur_.ops.empty()) fatal("ProgramBuilder: no operation to name");
+  return opLoc(cur_.name, static_cast<std::uint32_t>(cur_.ops.size() - 1));
+}
+
+void ProgramBuilder::golden(const std::string &loc, const std::string &name, const void *data, size_t bytes,
+                            const std::vector<std::int64_t> &shape, DataType dtype) {
+  if (!open_) fatal("ProgramBuilder: no program is open");
+  std::uint64_t volume = 1;
+  for (std::int64_t d : shape) {
+    if (d < 0) fatal("ProgramBuilder: golden tensor has a negative dimension");
+    volume *= static_cast<std::uint64_t>(d);
+  }
+  if (::tt::runtime::utils::isBlockFormatDataType(dtype))
+    fatal("ProgramBuilder: golden tensors hold plain element types, not block-float tiles");
+  const std::uint32_t elem = ::tt::runtime::utils::dataTypeElementSize(dtype);
+  if (volume * elem != bytes)
+    fatal("ProgramBuilder: golden tensor of " + std::to_string(bytes) + " bytes does not match its shape and dtype (" +
+          std::to_string(volume * elem) + " bytes)");
+  std::vector<std::int64_t> stride(shape.size(), 1);
+  for (int d = static_cast<int>(shape.size()) - 2; d >= 0; --d) stride[d] = stride[d + 1] * shape[d + 1];
+  Off nameOff = b_.createString(name);
+  Off shapeOff = b_.createScalarVector(shape), strideOff = b_.createScalarVector(stride);
+  Off dataOff = b_.createScalarVector(static_cast<const std::uint8_t *>(data), bytes);
+  b_.startTable(GoldenTensor::kNumFields);
+  b_.addOffset(GoldenTensor::f_name, nameOff);
+  b_.addOffset(GoldenTensor::f_shape, shapeOff);
+  b_.addOffset(GoldenTensor::f_stride, strideOff);
+  b_.addScalar<std::uint16_t>(GoldenTensor::f_dtype, static_cast<std::uint16_t>(dtype));
+  b_.addOffset(GoldenTensor::f_data, dataOff);
+  Off gt = b_.endTable();
+  b_.startTable(GoldenDeviceTensor::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(GoldenDeviceTensor::f_device, 0, 0);
+  b_.addOffset(GoldenDeviceTensor::f_value, gt);
+  cur_.goldens.emplace_back(loc, b_.endTable());
+}
+
 void ProgramBuilder::beginProgram(const std::string &name, bool isPrivate) {
   if (open_) fatal("ProgramBuilder: a program is already open");
   cur_ = ProgramRec{};
@@ -79,9 +120,10 @@ void ProgramBuilder::output(Id t) {
 std::uint32_t ProgramBuilder::endProgram() {
   if (!open_) fatal("ProgramBuilder: no program is open");
   std::vector<Off> ops;
+  std::uint32_t opIndex = 0;
   for (const OpRec &r : cur_.ops) {
     Off dbg = b_.createString(r.debug);
-    Off loc = b_.createString("loc(\"" + cur_.name + "\")");
+    Off loc = b_.createString(opLoc(cur_.name, opIndex++));
     b_.startTable(Operation::kNumFields);
     b_.addScalar<std::uint8_t>(Operation::f_type_type, r.type);
     b_.addOffset(Operation::f_type, r.table);
@@ -94,7 +136,28 @@ std::uint32_t ProgramBuilder::endProgram() {
   for (Id t : cur_.outputs) outs.push_back(tensorRef(t));
   Off opsV = b_.createOffsetVector(ops), insV = b_.createOffsetVector(ins), outsV = b_.createOffsetVector(outs);
   Off name = b_.createString(cur_.name);
+  Off debugInfo = 0;
+  if (!cur_.goldens.empty()) {
+    // one GoldenKV per location, each with the single device-0 tensor
+    std::vector<Off> kvs;
+    for (const auto &g : cur_.goldens) {
+      Off key = b_.createString(g.first);
+      Off vals = b_.createOffsetVector(std::vector<Off>{g.second});
+      b_.startTable(GoldenKV::kNumFields);
+      b_.addOffset(GoldenKV::f_key, key);
+      b_.addOffset(GoldenKV::f_value, vals);
+      kvs.push_back(b_.endTable());
+    }
+    Off map = b_.createOffsetVector(kvs);
+    b_.startTable(GoldenInfo::kNumFields);
+    b_.addOffset(GoldenInfo::f_golden_map, map);
+    Off info = b_.endTable();
+    b_.startTable(DebugInfo::kNumFields);
+    b_.addOffset(DebugInfo::f_golden_info, info);
+    debugInfo = b_.endTable();
+  }
   b_.startTable(Program::kNumFields);
+  if (debugInfo) b_.addOffset(Program::f_debug_info, debugInfo);
   b_.addOffset(Program::f_name, name);
   b_.addOffset(Program::f_inputs, insV);
   b_.addOffset(Program::f_outputs, outsV);

@@ -54,6 +54,13 @@ public:
   std::vector<Id> loadCached(std::uint32_t programIdx, const std::string &callee, const std::vector<Id> &ins, const std::vector<Desc> &outs);
   std::vector<Id> funcCall(std::uint32_t programIdx, const std::vector<Id> &ins, const std::vector<Desc> &outs);
 
+  // Location string of the operation added last ("loc(\"<program>\"(\"op<k>\"))"); goldens are keyed by it.
+  std::string lastOpLoc() const;
+  // Embeds an expected tensor for the operation at `loc` into the open program's debug info
+  // (Common/debug_info.fbs: GoldenInfo.golden_map); data is row-major, contiguous.
+  void golden(const std::string &loc, const std::string &name, const void *data, size_t bytes,
+              const std::vector<std::int64_t> &shape, DataType dtype);
+
   const Desc &desc(Id t) const;
   std::vector<std::uint8_t> finish();  // size-prefixed TTNN binary
 
@@ -68,6 +75,7 @@ private:
     bool isPrivate = false;
     std::vector<Id> inputs, outputs;
     std::vector<OpRec> ops;
+    std::vector<std::pair<std::string, fb::Builder::Off>> goldens;   // loc -> GoldenDeviceTensor table
   };
   Id newTensor(const Desc &d);
   fb::Builder::Off tensorRef(Id t);

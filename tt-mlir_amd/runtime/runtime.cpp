@@ -314,6 +314,84 @@ std::string Binary::getProgramOpsAsText(std::uint32_t i) const {
   return os.str();
 }
 
+// ---- JSON views and embedded goldens
+static std::string jsonEscape(std::string_view in) {
+  std::string o;
+  for (char c : in) {
+    switch (c) {
+    case '"': o += "\\\""; break;
+    case '\\': o += "\\\\"; break;
+    case '\n': o += "\\n"; break;
+    case '\t': o += "\\t"; break;
+    default:
+      if (static_cast<unsigned char>(c) < 0x20) { char b[8]; snprintf(b, sizeof(b), "\\u%04x", c); o += b; }
+      else o += c;
+    }
+  }
+  return o;
+}
+static std::string tensorRefJson(const fb::Table &ref) {
+  std::ostringstream os;
+  Layout l = layoutFromTensorRef(ref);
+  os << "{\"global_id\": " << ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0) << ", \"desc\": {\"shape\": [";
+  auto shp = shapeFromTensorRef(ref);
+  for (size_t i = 0; i < shp.size(); ++i) os << (i ? ", " : "") << shp[i];
+  os << "], \"layout\": {\"memory_desc\": {\"storage_type\": \"" << (l.storageType == StorageType::Device ? "DRAM" : "System")
+     << "\", \"tile_shape\": " << (l.layout == TensorLayout::Tile ? "{\"y\": 32, \"x\": 32}" : "{\"y\": 1, \"x\": 1}")
+     << ", \"data_type\": \"" << utils::dataTypeName(l.dataType) << "\"}}}}";
+  return os.str();
+}
+static std::string refsJson(const fb::TableVector &v) {
+  std::string o = "[";
+  for (std::uint32_t k = 0; k < v.size(); ++k) o += (k ? ", " : "") + tensorRefJson(v[k]);
+  return o + "]";
+}
+std::string Binary::getProgramInputsAsJson(std::uint32_t i) const { return refsJson(programAt(*this, i).tables(schema::Program::f_inputs)); }
+std::string Binary::getProgramOutputsAsJson(std::uint32_t i) const { return refsJson(programAt(*this, i).tables(schema::Program::f_outputs)); }
+std::string Binary::getProgramOpsAsJson(std::uint32_t i) const {
+  auto ops = programAt(*this, i).tables(schema::Program::f_operations);
+  std::ostringstream os;
+  os << "[";
+  for (std::uint32_t k = 0; k < ops.size(); ++k) {
+    auto t = static_cast<schema::OpType>(ops[k].scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
+    os << (k ? ", " : "") << "{\"type_type\": \"" << schema::opTypeName(t) << "\", \"debug_info\": \""
+       << jsonEscape(ops[k].string(schema::Operation::f_debug_info)) << "\", \"loc_info\": \""
+       << jsonEscape(ops[k].string(schema::Operation::f_loc_info)) << "\"}";
+  }
+  os << "]";
+  return os.str();
+}
+std::unordered_map<std::uint32_t, GoldenTensorInfo> Binary::getDebugInfoGolden(const std::string &loc) const {
+  std::unordered_map<std::uint32_t, GoldenTensorInfo> out;
+  for (std::uint32_t pi = 0; pi < getNumPrograms(); ++pi) {
+    auto dbg = programAt(*this, pi).table(schema::Program::f_debug_info);
+    if (!dbg) continue;
+    auto info = dbg.table(schema::DebugInfo::f_golden_info);
+    if (!info) continue;
+    auto kvs = info.tables(schema::GoldenInfo::f_golden_map);
+    for (std::uint32_t k = 0; k < kvs.size(); ++k) {
+      if (kvs[k].string(schema::GoldenKV::f_key) != loc) continue;
+      auto vals = kvs[k].tables(schema::GoldenKV::f_value);
+      for (std::uint32_t v = 0; v < vals.size(); ++v) {
+        auto gt = vals[v].table(schema::GoldenDeviceTensor::f_value);
+        if (!gt) continue;
+        GoldenTensorInfo g;
+        g.name = std::string(gt.string(schema::GoldenTensor::f_name));
+        auto shp = gt.scalars<std::int64_t>(schema::GoldenTensor::f_shape);
+        auto str = gt.scalars<std::int64_t>(schema::GoldenTensor::f_stride);
+        for (std::uint32_t q = 0; q < shp.size(); ++q) g.shape.push_back(shp[q]);
+        for (std::uint32_t q = 0; q < str.size(); ++q) g.stride.push_back(str[q]);
+        g.dataType = static_cast<::tt::target::DataType>(gt.scalar<std::uint16_t>(schema::GoldenTensor::f_dtype, 0));
+        auto data = gt.scalars<std::uint8_t>(schema::GoldenTensor::f_data);
+        g.data = data.data();
+        g.size = data.size();
+        out[vals[v].scalar<std::uint32_t>(schema::GoldenDeviceTensor::f_device, 0)] = g;
+      }
+    }
+  }
+  return out;
+}
+
 Layout getLayout(Binary binary, std::uint32_t programIndex, std::uint32_t inputIndex) {
   auto inputs = programAt(binary, programIndex).tables(schema::Program::f_inputs);
   TTRT_ASSERT(inputIndex < inputs.size(), "getLayout: input index out of range");

@@ -87,6 +87,14 @@ struct TensorRefInfo {
   std::vector<std::uint32_t> shape;
   Layout layout;
 };
+// golden tensor embedded in a program's debug info (include/ttmlir/Target/Common/debug_info.fbs:5-27)
+struct GoldenTensorInfo {
+  std::string name;
+  std::vector<std::int64_t> shape, stride;
+  ::tt::target::DataType dataType = ::tt::target::DataType::Float32;
+  const std::uint8_t *data = nullptr;   // points into the binary; valid while the Binary is alive
+  std::size_t size = 0;
+};
 struct Binary {
   std::shared_ptr<BinaryImpl> handle;
   static Binary loadFromPath(const std::string &path);
@@ -102,6 +110,11 @@ struct Binary {
   std::vector<TensorRefInfo> getProgramOutputs(std::uint32_t programIndex) const;
   std::uint32_t getNumOps(std::uint32_t programIndex) const;
   std::string getProgramOpsAsText(std::uint32_t programIndex) const;
+  // JSON views of one program (runtime/lib/binary.cpp:197-224) and the goldens keyed by op location (:233-253)
+  std::string getProgramOpsAsJson(std::uint32_t programIndex) const;
+  std::string getProgramInputsAsJson(std::uint32_t programIndex) const;
+  std::string getProgramOutputsAsJson(std::uint32_t programIndex) const;
+  std::unordered_map<std::uint32_t, GoldenTensorInfo> getDebugInfoGolden(const std::string &loc) const;
   std::uint64_t id() const;
 };
 
