@@ -87,13 +87,28 @@ int ttrt_memcpy_tensor(ttrt_tensor *dst, const ttrt_tensor *src);
 int ttrt_submit(ttrt_device *dev, const ttrt_binary *bin, uint32_t program, ttrt_tensor *const *inputs, uint32_t num_inputs,
                 ttrt_tensor **outputs, uint32_t max_outputs, uint32_t *num_outputs);
 
-/* ---- debug hooks (runtime/include/tt/runtime/debug.h:77-157): post-operator callback.  The callback
- * may call ttrt_hook_output to fetch the op's output as an untilized host tensor (NULL if none). */
+/* ---- debug hooks (runtime/include/tt/runtime/debug.h:77-157): callbacks before / after every operation and before /
+ * after every program (nested const-eval and func-call programs included).  hook_ctx is valid only inside the callback.
+ * ttrt_hook_output: the op's first output as an untilized host tensor (NULL if none) - getOpOutputTensor, runtime.h:250.
+ * ttrt_hook_input_refs / output_refs: global ids of the op's operands / results - getOpInputRefs / getOpOutputRefs,
+ *   runtime.h:252-262; in a program callback both report nothing.
+ * ttrt_hook_retrieve: host copy of any live tensor of the running program (NULL if not in the pool) -
+ *   retrieveTensorFromPool, runtime.h:267-273.
+ * ttrt_hook_update: overwrite the payload of a pool tensor from src, converting src to the pool tensor's layout -
+ *   updateTensorInPool, runtime.h:275-283. */
 typedef void (*ttrt_op_callback)(uint32_t op_index, const char *op_name, const char *debug_info, void *hook_ctx, void *user);
+typedef void (*ttrt_program_callback)(uint32_t program_index, void *hook_ctx, void *user);
+int ttrt_set_pre_op_callback(ttrt_op_callback cb, void *user);
 int ttrt_set_post_op_callback(ttrt_op_callback cb, void *user);
+int ttrt_set_program_callbacks(ttrt_program_callback pre, ttrt_program_callback post, void *user);
 int ttrt_clear_callbacks(void);
 int ttrt_hook_output(void *hook_ctx, ttrt_tensor **out);
-/* location string of the operation a hook is running for (getOpLocInfo, runtime.h) */
+int ttrt_hook_input_refs(void *hook_ctx, uint32_t *ids, uint32_t cap, uint32_t *count);
+int ttrt_hook_output_refs(void *hook_ctx, uint32_t *ids, uint32_t cap, uint32_t *count);
+int ttrt_hook_retrieve(void *hook_ctx, uint32_t global_id, int untilize, ttrt_tensor **out);
+int ttrt_hook_update(void *hook_ctx, uint32_t global_id, const ttrt_tensor *src);
+int ttrt_hook_program_index(void *hook_ctx, uint32_t *index);
+/* location string of the operation a hook is running for (getOpLocInfo, runtime.h:248) */
 int ttrt_hook_loc(void *hook_ctx, char *buf, size_t len);
 int ttrt_stat(const char *name, int64_t *value);
 int ttrt_stats_clear(void);

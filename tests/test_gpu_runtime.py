@@ -244,6 +244,65 @@ def test_post_op_hook_sees_intermediates(device, orc):
     assert [t is None for _, n, t in seen if n == "DeallocateOp"] == [True, True, True]
 
 
+def test_hooks_can_read_and_replace_pool_tensors(device, orc):
+    """Pre / post operator and program callbacks, operand references, retrieveTensorFromPool / updateTensorInPool
+    (runtime/include/tt/runtime/runtime.h:246-297; use in tools/builder/base/builder_runtime.py:353-451)."""
+    binary = rt.Binary.load_from_memory(programs.c4_mlp(64, 128, 256))
+    d = datagen.c4_mlp(64, 128, 256, seed=9)
+    f = lambda t: t.float().numpy()
+    tins = [d["x"], d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    events, refs, seen_in = [], {}, {}
+
+    def pre(idx, name, dbg, hook):
+        events.append(("pre", hook.program_index(), idx, name))
+        if hook.program_index() == 1 and name == "LinearOp":
+            ids = hook.input_refs()
+            seen_in["linear"] = [None if hook.retrieve(i) is None else tuple(hook.retrieve(i).shape) for i in ids]
+
+    def post(idx, name, dbg, hook):
+        events.append(("post", hook.program_index(), idx, name))
+        if hook.program_index() != 1:
+            return
+        refs[idx] = (name, hook.input_refs(), hook.output_refs())
+        if name == "RMSNormOp":
+            # replace the normalised activations by zeros: everything downstream must become exactly zero
+            (out_id,) = hook.output_refs()
+            hook.update(out_id, rt.from_torch(torch.zeros(64, 128, dtype=torch.bfloat16)))
+            back = rt.to_torch(hook.retrieve(out_id))
+            assert back.shape == (64, 128) and not back.any()
+            tiled = hook.retrieve(out_id, untilize=False)
+            assert tiled.layout.layout == rt.TensorLayout.Tile
+
+    programs_seen = []
+    rt.set_pre_op_callback(pre)
+    rt.set_post_op_callback(post)
+    rt.set_program_callbacks(lambda i, h: programs_seen.append(("begin", i)), lambda i, h: programs_seen.append(("end", i)))
+    try:
+        (y,) = harness.execute(binary, 1, tins, device)
+    finally:
+        rt.clear_callbacks()
+    assert not f(y).any()
+    # the private const-eval program runs nested inside the main program's LoadCachedOp
+    assert programs_seen == [("begin", 1), ("begin", 0), ("end", 0), ("end", 1)]
+    assert events[0] == ("pre", 1, 0, "LoadCachedOp") and events[1][:2] == ("pre", 0)
+    assert [e[0] for e in events].count("pre") == [e[0] for e in events].count("post")
+    ins = binary.get_program_inputs_as_json(1)
+    in_ids = [t["global_id"] for t in ins]
+    name, i_refs, o_refs = refs[0]
+    assert name == "LoadCachedOp" and i_refs == in_ids[2:] and len(o_refs) == 3
+    name, i_refs, o_refs = refs[1]
+    assert name == "RMSNormOp" and i_refs == in_ids[:2] and len(o_refs) == 1
+    norm_id = o_refs[0]
+    name, i_refs, _ = refs[2]
+    assert name == "LinearOp" and i_refs == [norm_id, refs[0][2][0]]
+    assert seen_in["linear"] == [(64, 128), (128, 256)]
+    assert refs[5] == ("DeallocateOp", [refs[2][2][0]], [])
+    # hooks are gone: the same run gives the ordinary result again
+    (y2,) = harness.execute(binary, 1, tins, device)
+    want = oracle_mlp(orc, f(d["x"]), f(d["norm_w"]), f(bf(d["wg"])), f(bf(d["wu"])), f(bf(d["wd"])), 1e-5)
+    assert np.max(np.abs(f(y2) - want)) <= 2.0 ** -10
+
+
 def test_embedded_goldens_are_checked_per_operation(device, orc):
     """`ttrt run --enable-golden` flow: every op with a golden embedded in the binary is compared in the post-op hook."""
     d = datagen.c4_mlp(64, 128, 256, seed=11)
@@ -265,6 +324,48 @@ def test_embedded_goldens_are_checked_per_operation(device, orc):
     assert {v["name"]: v["pass"] for v in report.values()} == dict(norm=True, gate=True, up=False, product=True, down=True)
     # the hook is gone afterwards
     harness.execute(binary, 1, tins, device)
+
+
+def test_ttrt_run_checks_embedded_goldens_and_saves_artifacts(orc, tmp_path):
+    """`ttrt run --enable-golden --save-artifacts` (tools/ttrt/common/run.py:534-873, 1160-1172)."""
+    import json
+    from ttmlir_amd import ttrt
+    d = datagen.c4_mlp(64, 128, 256, seed=5)
+    f = lambda t: t.float().numpy()
+    tins = [d["x"], d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    st = oracle_mlp_stages(orc, *[f(t) for t in tins], 1e-5)
+    gold = dict(st, output_0=st["down"], **{"input_%d" % k: f(t) for k, t in enumerate(tins)})
+    good = tmp_path / "mlp.ttnn"
+    good.write_bytes(programs.c4_mlp(64, 128, 256, goldens=gold))
+    res, art = tmp_path / "res.json", tmp_path / "art"
+    rc = ttrt.main(["run", str(good), "--enable-golden", "--loops", "2", "--save-artifacts", "--artifact-dir", str(art),
+                    "--result-file", str(res), "--non-zero", "--benchmark"])
+    (rec,) = json.loads(res.read_text())
+    assert rc == 0 and rec["result"] == "pass", rec
+    (prog,) = rec["program_results"]                     # the private const-eval program is not run on its own
+    assert prog["program_index"] == 1 and [l["loop"] for l in prog["loops"]] == [0, 1]
+    assert all(l["total_duration_ns"] >= l["submit_ns"] > 0 for l in prog["loops"])
+    rep = prog["golden_report"]
+    assert len(rep) == 6 and all(v["result"] == "pass" and v["actual_pcc"] >= 0.999 for v in rep.values())
+    folder = art / "mlp" / "run" / "program_1"
+    assert (art / "mlp" / "mlp.ttnn").read_bytes() == good.read_bytes()
+    assert torch.equal(torch.load(folder / "input_0.pt", weights_only=True), d["x"])
+    y = torch.load(folder / "device_output_0.pt", weights_only=True)
+    assert np.max(np.abs(f(y) - st["down"])) <= 2.0 ** -10
+    assert set(json.loads((folder / "golden_results.json").read_text())) == set(rep)
+    # without the embedded inputs the run uses seeded random inputs: the stage goldens no longer match
+    bad = tmp_path / "bad.ttnn"
+    bad.write_bytes(programs.c4_mlp(64, 128, 256, goldens=dict(st, output_0=st["down"])))
+    rc = ttrt.main(["run", str(good), str(bad), "--enable-golden", "--result-file", str(res)])
+    recs = json.loads(res.read_text())
+    assert rc == 1 and [r["result"] for r in recs] == ["pass", "error"]
+    assert "golden comparison failed" in recs[1]["exception"]
+    # plain run, seeded: two runs give identical outputs
+    for name in ("a", "b"):
+        assert ttrt.main(["run", str(bad), "--seed", "3", "--save-artifacts", "--artifact-dir", str(tmp_path / name),
+                          "--result-file", str(res)]) == 0
+    ya, yb = (torch.load(tmp_path / n / "bad" / "run" / "program_1" / "device_output_0.pt", weights_only=True) for n in ("a", "b"))
+    assert torch.equal(ya, yb) and bool(ya.float().abs().sum() > 0)
 
 
 def test_submit_errors(device):

@@ -124,6 +124,41 @@ def test_program_goldens_option_marks_each_stage():
     assert all(np.array_equal(found[k][1], st[k]) for k in st)
 
 
+def test_ttrt_read_and_error_records(tmp_path, capsys):
+    import json
+    from ttmlir_amd import ttrt
+    path = tmp_path / "c4.ttnn"
+    path.write_bytes(programs.c4_mlp(64, 128, 256, goldens={"norm": np.ones((64, 128), np.float32),
+                                                              "output_0": np.zeros((64, 128), np.float32)}))
+    assert ttrt.main(["read", str(path)]) == 0
+    info = json.loads(capsys.readouterr().out)
+    assert info["file_identifier"] == "TTNN" and [p["private"] for p in info["programs"]] == [True, False]
+    assert [o["type_type"] for o in info["ops"][1]][:2] == ["LoadCachedOp", "RMSNormOp"]
+    assert info["goldens"][0] == []
+    assert [(g["loc"], g["name"], g["shape"]) for g in info["goldens"][1]] == [
+        ('loc("c4_mlp"("op1"))', "norm", [64, 128]), ("output_0", "output_0", [64, 128])]
+    assert ttrt.main(["read", str(path), "--section", "version"]) == 0
+    assert set(json.loads(capsys.readouterr().out)) == {"file_path", "file_identifier", "version"}
+    # a binary that cannot be read becomes an error record and a non-zero exit code, not a traceback
+    res = tmp_path / "r.json"
+    assert ttrt.main(["run", str(tmp_path / "missing.ttnn"), "--result-file", str(res)]) == 1
+    (rec,) = json.loads(res.read_text())
+    assert rec["result"] == "error" and "cannot open" in rec["exception"] and rec["program_results"] == []
+
+
+def test_ttrt_input_initialisers():
+    import torch
+    from ttmlir_amd import ttrt
+    g = torch.Generator().manual_seed(0)
+    a = ttrt.make_input((4, 8), DT.BFloat16, "randn", g)
+    want = torch.randn((4, 8), generator=torch.Generator().manual_seed(0)).to(torch.bfloat16)
+    assert a.dtype == torch.bfloat16 and torch.equal(a, want)
+    assert torch.equal(ttrt.make_input((2, 3), DT.Float32, "arange", g), torch.arange(6.0).reshape(2, 3))
+    idx = ttrt.make_input((16,), DT.Int32, "randn", g)
+    assert idx.dtype == torch.int32 and int(idx.min()) >= 0 and int(idx.max()) < 8
+    assert ttrt.make_input((2, 2), DT.BFP_BFloat8, "ones", g).dtype == torch.bfloat16
+
+
 def test_decoder_program_shapes():
     b = rt.Binary.load_from_memory(programs.c5_decoder(seq=64, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512))
     assert b.get_program_outputs(1)[0][0] == (1, 64, 256)

@@ -374,34 +374,89 @@ def clear_stats():
 
 
 _CB_TYPE = ctypes.CFUNCTYPE(None, ctypes.c_uint32, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_void_p, ctypes.c_void_p)
-_cb_keep = None
+_PROGRAM_CB_TYPE = ctypes.CFUNCTYPE(None, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p)
+_cb_keep = {}
+
+
+class HookContext:
+    """What a callback may ask about the operation / program it runs for; valid only inside the callback.
+    Calling the object returns the op's first output (kept for callbacks written as get_output())."""
+
+    def __init__(self, hook):
+        self._h = ctypes.c_void_p(hook)
+
+    def output(self):
+        """First output of the op as an untilized host Tensor, or None (getOpOutputTensor)."""
+        h = ctypes.c_void_p()
+        _call("ttrt_hook_output", self._h, ctypes.byref(h))
+        return Tensor(h) if h.value else None
+
+    __call__ = output
+
+    def loc(self):
+        buf = ctypes.create_string_buffer(512)
+        _call("ttrt_hook_loc", self._h, buf, 512)
+        return buf.value.decode()
+
+    def _refs(self, fn):
+        ids, n = (ctypes.c_uint32 * 64)(), ctypes.c_uint32()
+        _call(fn, self._h, ids, 64, ctypes.byref(n))
+        return list(ids[: n.value])
+
+    def input_refs(self):
+        """global ids of the op's tensor operands (getOpInputRefs)."""
+        return self._refs("ttrt_hook_input_refs")
+
+    def output_refs(self):
+        return self._refs("ttrt_hook_output_refs")
+
+    def retrieve(self, global_id, untilize=True):
+        """Host copy of a live tensor of the running program, or None (retrieveTensorFromPool)."""
+        h = ctypes.c_void_p()
+        _call("ttrt_hook_retrieve", self._h, global_id, int(untilize), ctypes.byref(h))
+        return Tensor(h) if h.value else None
+
+    def update(self, global_id, tensor):
+        """Overwrite the payload of a pool tensor; `tensor` is converted to the pool tensor's layout (updateTensorInPool)."""
+        _call("ttrt_hook_update", self._h, global_id, tensor.h)
+
+    def program_index(self):
+        i = ctypes.c_uint32()
+        _call("ttrt_hook_program_index", self._h, ctypes.byref(i))
+        return i.value
+
+
+def _op_trampoline(fn):
+    def tramp(idx, name, dbg, hook, user):
+        fn(idx, name.decode(), dbg.decode(), HookContext(hook))
+    return _CB_TYPE(tramp)
 
 
 def set_post_op_callback(fn):
-    """fn(op_index, op_name, debug_info, get_output) with get_output() -> host Tensor or None."""
-    global _cb_keep
+    """fn(op_index, op_name, debug_info, hook: HookContext), after every operation."""
+    _cb_keep["post_op"] = _op_trampoline(fn)
+    _call("ttrt_set_post_op_callback", _cb_keep["post_op"], None)
 
-    def tramp(idx, name, dbg, hook, user):
-        def get_output():
-            h = ctypes.c_void_p()
-            _call("ttrt_hook_output", ctypes.c_void_p(hook), ctypes.byref(h))
-            return Tensor(h) if h.value else None
 
-        def get_loc():
-            buf = ctypes.create_string_buffer(512)
-            _call("ttrt_hook_loc", ctypes.c_void_p(hook), buf, 512)
-            return buf.value.decode()
-        get_output.loc = get_loc
-        fn(idx, name.decode(), dbg.decode(), get_output)
+def set_pre_op_callback(fn):
+    """fn(op_index, op_name, debug_info, hook: HookContext), before every operation."""
+    _cb_keep["pre_op"] = _op_trampoline(fn)
+    _call("ttrt_set_pre_op_callback", _cb_keep["pre_op"], None)
 
-    _cb_keep = _CB_TYPE(tramp)
-    _call("ttrt_set_post_op_callback", _cb_keep, None)
+
+def set_program_callbacks(pre=None, post=None):
+    """pre / post: fn(program_index, hook: HookContext) around every program, nested ones included."""
+    def wrap(fn):
+        if fn is None:
+            return _PROGRAM_CB_TYPE()
+        return _PROGRAM_CB_TYPE(lambda idx, hook, user: fn(idx, HookContext(hook)))
+    _cb_keep["pre_program"], _cb_keep["post_program"] = wrap(pre), wrap(post)
+    _call("ttrt_set_program_callbacks", _cb_keep["pre_program"], _cb_keep["post_program"], None)
 
 
 def clear_callbacks():
-    global _cb_keep
     _call("ttrt_clear_callbacks")
-    _cb_keep = None
+    _cb_keep.clear()
 
 
 class ProgramBuilder:

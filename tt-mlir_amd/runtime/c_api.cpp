@@ -231,15 +231,74 @@ struct HookCtx {
   CallbackContext cc;
   OpContext oc;
 };
+static debug::CallbackFn wrapOpCallback(ttrt_op_callback cb, void *user) {
+  return debug::CallbackFn([cb, user](Binary, CallbackContext cc, OpContext oc) {
+    HookCtx h{cc, oc};
+    auto type = static_cast<ttmlir_amd::schema::OpType>(oc.op.scalar<std::uint8_t>(ttmlir_amd::schema::Operation::f_type_type, 0));
+    std::string dbg = getOpDebugString(oc);
+    cb(oc.index, ttmlir_amd::schema::opTypeName(type), dbg.c_str(), &h, user);
+  });
+}
+static debug::ProgramCallbackFn wrapProgramCallback(ttrt_program_callback cb, void *user) {
+  return debug::ProgramCallbackFn([cb, user](Binary, CallbackContext cc) {
+    HookCtx h{cc, OpContext{}};
+    cb(static_cast<uint32_t>(getProgramIndex(cc)), &h, user);
+  });
+}
 TTRT_EXPORT int ttrt_set_post_op_callback(ttrt_op_callback cb, void *user) {
   return guard([&] {
     need(reinterpret_cast<const void *>(cb), "callback");
-    debug::Hooks::get(std::nullopt, debug::CallbackFn([cb, user](Binary, CallbackContext cc, OpContext oc) {
-                        HookCtx h{cc, oc};
-                        auto type = static_cast<ttmlir_amd::schema::OpType>(oc.op.scalar<std::uint8_t>(ttmlir_amd::schema::Operation::f_type_type, 0));
-                        std::string dbg = getOpDebugString(oc);
-                        cb(oc.index, ttmlir_amd::schema::opTypeName(type), dbg.c_str(), &h, user);
-                      }));
+    debug::Hooks::get(std::nullopt, wrapOpCallback(cb, user));
+  });
+}
+TTRT_EXPORT int ttrt_set_pre_op_callback(ttrt_op_callback cb, void *user) {
+  return guard([&] {
+    need(reinterpret_cast<const void *>(cb), "callback");
+    debug::Hooks::get(wrapOpCallback(cb, user));
+  });
+}
+TTRT_EXPORT int ttrt_set_program_callbacks(ttrt_program_callback pre, ttrt_program_callback post, void *user) {
+  return guard([&] {
+    debug::Hooks::get(std::nullopt, std::nullopt,
+                      pre ? std::optional<debug::ProgramCallbackFn>(wrapProgramCallback(pre, user)) : std::nullopt,
+                      post ? std::optional<debug::ProgramCallbackFn>(wrapProgramCallback(post, user)) : std::nullopt);
+  });
+}
+static void copyRefIds(const std::vector<TensorRef> &refs, uint32_t *ids, uint32_t cap, uint32_t *count) {
+  need(count, "count");
+  *count = static_cast<uint32_t>(refs.size());
+  if (refs.size() > cap) fatal("hook: the id array is too small for this operation's tensor references");
+  for (size_t i = 0; i < refs.size(); ++i) ids[i] = getTensorRefGlobalId(refs[i]);
+}
+TTRT_EXPORT int ttrt_hook_input_refs(void *hook_ctx, uint32_t *ids, uint32_t cap, uint32_t *count) {
+  return guard([&] {
+    need(hook_ctx, "hook context");
+    copyRefIds(getOpInputRefs(static_cast<HookCtx *>(hook_ctx)->oc), ids, cap, count);
+  });
+}
+TTRT_EXPORT int ttrt_hook_output_refs(void *hook_ctx, uint32_t *ids, uint32_t cap, uint32_t *count) {
+  return guard([&] {
+    need(hook_ctx, "hook context");
+    copyRefIds(getOpOutputRefs(static_cast<HookCtx *>(hook_ctx)->oc), ids, cap, count);
+  });
+}
+TTRT_EXPORT int ttrt_hook_retrieve(void *hook_ctx, uint32_t global_id, int untilize, ttrt_tensor **out) {
+  return guard([&] {
+    need(hook_ctx, "hook context"); need(out, "out");
+    auto t = retrieveTensorFromPool(static_cast<HookCtx *>(hook_ctx)->cc, global_id, untilize != 0);
+    *out = t.has_value() ? new ttrt_tensor{*t} : nullptr;
+  });
+}
+TTRT_EXPORT int ttrt_hook_update(void *hook_ctx, uint32_t global_id, const ttrt_tensor *src) {
+  return guard([&] {
+    need(hook_ctx, "hook context"); need(src, "source tensor");
+    updateTensorInPool(static_cast<HookCtx *>(hook_ctx)->cc, global_id, src->t);
+  });
+}
+TTRT_EXPORT int ttrt_hook_program_index(void *hook_ctx, uint32_t *index) {
+  return guard([&] {
+    need(hook_ctx, "hook context"); need(index, "index");
+    *index = static_cast<uint32_t>(getProgramIndex(static_cast<HookCtx *>(hook_ctx)->cc));
   });
 }
 TTRT_EXPORT int ttrt_clear_callbacks(void) {

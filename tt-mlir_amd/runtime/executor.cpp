@@ -680,13 +680,15 @@ std::vector<Tensor> executeProgram(const std::shared_ptr<DeviceState> &dev, cons
   }
   auto ops = program.tables(schema::Program::f_operations);
   auto &hooks = debug::Hooks::get();
+  CallbackContext cc{&ctx};
+  if (hooks.preProgramCallback) (*hooks.preProgramCallback)(binary, cc);
   for (std::uint32_t i = 0; i < ops.size(); ++i) {
     OpContext oc{ops[i], i};
-    CallbackContext cc{&ctx};
     if (hooks.preOperatorCallback) (*hooks.preOperatorCallback)(binary, cc, oc);
     runOperation(ops[i], ctx);
     if (hooks.postOperatorCallback) (*hooks.postOperatorCallback)(binary, cc, oc);
   }
+  if (hooks.postProgramCallback) (*hooks.postProgramCallback)(binary, cc);
   std::vector<Tensor> outputs;
   auto outs = program.tables(schema::Program::f_outputs);
   for (std::uint32_t i = 0; i < outs.size(); ++i) outputs.push_back(ctx.get(outs[i], "program output"));
@@ -694,51 +696,103 @@ std::vector<Tensor> executeProgram(const std::shared_ptr<DeviceState> &dev, cons
 }
 
 // ---- hook-side access to the running program (runtime/include/tt/runtime/runtime.h:246-297)
-static fb::Table firstOutputRef(const fb::Table &operation, std::vector<fb::Table> *all = nullptr) {
+namespace {
+// Tensor operands of an operation as the flatbuffer names them: `ins` in operand order (absent optional operands are
+// skipped), `outs` in result order.  Ops outside the supported subset report nothing.
+struct OpRefs {
+  std::vector<fb::Table> ins, outs;
+};
+
+OpRefs opRefs(const fb::Table &operation) {
   auto type = static_cast<OpType>(operation.scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
   fb::Table op = operation.table(schema::Operation::f_type);
-  int slot = -1;
+  OpRefs r;
+  auto in = [&](int slot) { if (fb::Table t = op.table(slot)) r.ins.push_back(t); };
+  auto out = [&](int slot) { if (fb::Table t = op.table(slot)) r.outs.push_back(t); };
+  auto inVec = [&](int slot) {
+    auto v = op.tables(slot);
+    for (std::uint32_t i = 0; i < v.size(); ++i) r.ins.push_back(v[i]);
+  };
+  auto outVec = [&](int slot) {
+    auto v = op.tables(slot);
+    for (std::uint32_t i = 0; i < v.size(); ++i) r.outs.push_back(v[i]);
+  };
   switch (type) {
-  case OpType::ToLayoutOp: slot = schema::ToLayoutOp::f_out; break;
-  case OpType::TypecastOp: slot = schema::TypecastOp::f_out; break;
-  case OpType::ToDeviceOp: slot = schema::ToDeviceOp::f_out; break;
-  case OpType::FromDeviceOp: slot = schema::FromDeviceOp::f_out; break;
-  case OpType::ToMemoryConfigOp: slot = schema::ToMemoryConfigOp::f_out; break;
-  case OpType::MatmulOp: slot = schema::MatmulOp::f_out; break;
-  case OpType::LinearOp: slot = schema::LinearOp::f_out; break;
-  case OpType::EltwiseUnaryOp: slot = schema::EltwiseUnaryOp::f_out; break;
-  case OpType::EltwiseBinaryOp: slot = schema::EltwiseBinaryOp::f_out; break;
-  case OpType::RMSNormOp: slot = schema::RMSNormOp::f_out; break;
-  case OpType::SoftmaxOp: slot = schema::SoftmaxOp::f_out; break;
-  case OpType::ReductionOp: slot = schema::ReductionOp::f_out; break;
-  case OpType::ScaledDotProductAttentionOp: slot = schema::ScaledDotProductAttentionOp::f_out; break;
-  case OpType::ReshapeOp: slot = schema::ReshapeOp::f_out; break;
-  case OpType::PermuteOp: slot = schema::PermuteOp::f_out; break;
-  case OpType::TransposeOp: slot = schema::TransposeOp::f_out; break;
-  case OpType::ConcatOp: slot = schema::ConcatOp::f_out; break;
-  case OpType::SliceOp: slot = schema::SliceOp::f_out; break;
-  case OpType::RepeatInterleaveOp: slot = schema::RepeatInterleaveOp::f_out; break;
-  case OpType::ConstantOp: slot = schema::ConstantOp::f_out; break;
-  case OpType::FullOp: slot = schema::FullOp::f_out; break;
-  case OpType::NamedFullOp: slot = schema::NamedFullOp::f_out; break;
-  case OpType::EmptyOp: slot = schema::EmptyOp::f_out; break;
+  case OpType::ToLayoutOp: in(schema::ToLayoutOp::f_in); out(schema::ToLayoutOp::f_out); break;
+  case OpType::TypecastOp: in(schema::TypecastOp::f_in); out(schema::TypecastOp::f_out); break;
+  case OpType::ToDeviceOp: in(schema::ToDeviceOp::f_in); out(schema::ToDeviceOp::f_out); break;
+  case OpType::FromDeviceOp: in(schema::FromDeviceOp::f_in); out(schema::FromDeviceOp::f_out); break;
+  case OpType::ToMemoryConfigOp: in(schema::ToMemoryConfigOp::f_in0); out(schema::ToMemoryConfigOp::f_out); break;
+  case OpType::MatmulOp: in(schema::MatmulOp::f_a); in(schema::MatmulOp::f_b); out(schema::MatmulOp::f_out); break;
+  case OpType::LinearOp:
+    in(schema::LinearOp::f_a); in(schema::LinearOp::f_b); in(schema::LinearOp::f_bias); out(schema::LinearOp::f_out);
+    break;
+  case OpType::EltwiseUnaryOp: in(schema::EltwiseUnaryOp::f_in); out(schema::EltwiseUnaryOp::f_out); break;
+  case OpType::EltwiseBinaryOp:
+    in(schema::EltwiseBinaryOp::f_lhs); in(schema::EltwiseBinaryOp::f_rhs); out(schema::EltwiseBinaryOp::f_out);
+    break;
+  case OpType::RMSNormOp:
+    in(schema::RMSNormOp::f_input); in(schema::RMSNormOp::f_weight); in(schema::RMSNormOp::f_bias); out(schema::RMSNormOp::f_out);
+    break;
+  case OpType::SoftmaxOp: in(schema::SoftmaxOp::f_in); out(schema::SoftmaxOp::f_out); break;
+  case OpType::ReductionOp: in(schema::ReductionOp::f_in); out(schema::ReductionOp::f_out); break;
+  case OpType::ScaledDotProductAttentionOp:
+    in(schema::ScaledDotProductAttentionOp::f_query); in(schema::ScaledDotProductAttentionOp::f_key);
+    in(schema::ScaledDotProductAttentionOp::f_value); in(schema::ScaledDotProductAttentionOp::f_attention_mask);
+    out(schema::ScaledDotProductAttentionOp::f_out);
+    break;
+  case OpType::ReshapeOp: in(schema::ReshapeOp::f_in); out(schema::ReshapeOp::f_out); break;
+  case OpType::PermuteOp: in(schema::PermuteOp::f_in); out(schema::PermuteOp::f_out); break;
+  case OpType::TransposeOp: in(schema::TransposeOp::f_in); out(schema::TransposeOp::f_out); break;
+  case OpType::ConcatOp: inVec(schema::ConcatOp::f_inputs); out(schema::ConcatOp::f_out); break;
+  case OpType::SliceOp: in(schema::SliceOp::f_in); out(schema::SliceOp::f_out); break;
+  case OpType::RepeatInterleaveOp: in(schema::RepeatInterleaveOp::f_input); out(schema::RepeatInterleaveOp::f_out); break;
+  case OpType::ConstantOp: out(schema::ConstantOp::f_out); break;
+  case OpType::FullOp: out(schema::FullOp::f_out); break;
+  case OpType::NamedFullOp: out(schema::NamedFullOp::f_out); break;
+  case OpType::EmptyOp: out(schema::EmptyOp::f_out); break;
+  case OpType::DeallocateOp: in(schema::DeallocateOp::f_in); break;
+  case OpType::LoadCachedOp: inVec(schema::LoadCachedOp::f_inputs); outVec(schema::LoadCachedOp::f_outputs); break;
+  case OpType::FuncCallOp: inVec(schema::FuncCallOp::f_inputs); outVec(schema::FuncCallOp::f_outputs); break;
   default: break;
   }
-  (void)all;
-  return slot >= 0 ? op.table(slot) : fb::Table();
+  return r;
+}
+
+std::vector<TensorRef> wrapRefs(const std::vector<fb::Table> &tables) {
+  std::vector<TensorRef> out;
+  for (const auto &t : tables) out.push_back(TensorRef{t});
+  return out;
+}
+}  // namespace
+
+std::vector<TensorRef> getOpOutputRefs(OpContext oc) { return wrapRefs(opRefs(oc.op).outs); }
+std::vector<TensorRef> getOpInputRefs(OpContext oc) { return wrapRefs(opRefs(oc.op).ins); }
+std::vector<std::uint32_t> getTensorRefShape(TensorRef ref) { return shapeFromTensorRef(ref.table); }
+::tt::target::DataType getTensorRefDataType(TensorRef ref) { return layoutFromTensorRef(ref.table).dataType; }
+std::uint32_t getTensorRefGlobalId(TensorRef ref) { return ref.table.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0); }
+size_t getProgramIndex(CallbackContext cc) {
+  auto *ctx = static_cast<ProgramContext *>(cc.programContext);
+  TTRT_ASSERT(ctx != nullptr, "getProgramIndex: no program context");
+  return ctx->programIndex;
 }
 
 std::unordered_map<std::uint32_t, Tensor> getOpOutputTensor(OpContext oc, CallbackContext cc) {
   std::unordered_map<std::uint32_t, Tensor> out;
   auto *ctx = static_cast<ProgramContext *>(cc.programContext);
-  fb::Table ref = firstOutputRef(oc.op);
-  if (!ref || !ctx) return out;
-  std::uint32_t id = ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
+  OpRefs refs = opRefs(oc.op);
+  if (refs.outs.empty() || !ctx) return out;
+  std::uint32_t id = refs.outs.front().scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
   auto it = ctx->pool.find(id);
   if (it == ctx->pool.end() || !isTensorAllocated(it->second)) return out;
   out[0] = toHost(it->second, /*untilize=*/true)[0];
   return out;
 }
+
+std::optional<Tensor> retrieveTensorFromPool(CallbackContext cc, TensorRef ref, bool untilize) {
+  return retrieveTensorFromPool(cc, getTensorRefGlobalId(ref), untilize);
+}
+void updateTensorInPool(CallbackContext cc, TensorRef ref, Tensor src) { updateTensorInPool(cc, getTensorRefGlobalId(ref), src); }
 
 std::optional<Tensor> retrieveTensorFromPool(CallbackContext cc, std::uint32_t globalId, bool untilize) {
   auto *ctx = static_cast<ProgramContext *>(cc.programContext);

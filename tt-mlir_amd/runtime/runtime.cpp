@@ -756,15 +756,20 @@ std::vector<Tensor> submit(Device device, Binary binary, std::uint32_t programIn
 
 // ---------------------------------------------------------------------------- debug
 namespace debug {
-Hooks &Hooks::get(std::optional<CallbackFn> pre, std::optional<CallbackFn> post) {
+Hooks &Hooks::get(std::optional<CallbackFn> pre, std::optional<CallbackFn> post, std::optional<ProgramCallbackFn> preProgram,
+                  std::optional<ProgramCallbackFn> postProgram) {
   static Hooks h;
   if (pre.has_value()) h.preOperatorCallback = pre;
   if (post.has_value()) h.postOperatorCallback = post;
+  if (preProgram.has_value()) h.preProgramCallback = preProgram;
+  if (postProgram.has_value()) h.postProgramCallback = postProgram;
   return h;
 }
 void Hooks::unregisterHooks() {
   preOperatorCallback.reset();
   postOperatorCallback.reset();
+  preProgramCallback.reset();
+  postProgramCallback.reset();
 }
 static std::mutex g_statsMu;
 Stats &Stats::get() {

@@ -126,11 +126,19 @@ struct OpContext {
 struct CallbackContext {
   void *programContext = nullptr;
 };
+// a TensorRef table of the binary, as hooks see an operation's operands (runtime/include/tt/runtime/types.h TensorRef)
+struct TensorRef {
+  fb::Table table;
+};
 namespace debug {
 using CallbackFn = std::function<void(Binary, CallbackContext, OpContext)>;
+using ProgramCallbackFn = std::function<void(Binary, CallbackContext)>;
 struct Hooks {
-  static Hooks &get(std::optional<CallbackFn> preOperator = std::nullopt, std::optional<CallbackFn> postOperator = std::nullopt);
+  static Hooks &get(std::optional<CallbackFn> preOperator = std::nullopt, std::optional<CallbackFn> postOperator = std::nullopt,
+                    std::optional<ProgramCallbackFn> preProgram = std::nullopt,
+                    std::optional<ProgramCallbackFn> postProgram = std::nullopt);
   std::optional<CallbackFn> preOperatorCallback, postOperatorCallback;
+  std::optional<ProgramCallbackFn> preProgramCallback, postProgramCallback;
   void unregisterHooks();
 };
 struct Stats {
@@ -182,8 +190,16 @@ void deallocateTensor(Tensor &tensor, bool force = false);
 std::string getOpDebugString(OpContext opContextHandle);
 std::string getOpLocInfo(OpContext opContextHandle);
 std::unordered_map<std::uint32_t, Tensor> getOpOutputTensor(OpContext opContextHandle, CallbackContext programContextHandle);
+std::vector<TensorRef> getOpOutputRefs(OpContext opContextHandle);
+std::vector<TensorRef> getOpInputRefs(OpContext opContextHandle);
+std::vector<std::uint32_t> getTensorRefShape(TensorRef tensorRef);
+::tt::target::DataType getTensorRefDataType(TensorRef tensorRef);
+std::uint32_t getTensorRefGlobalId(TensorRef tensorRef);
+std::optional<Tensor> retrieveTensorFromPool(CallbackContext programContextHandle, TensorRef tensorRef, bool untilize);
 std::optional<Tensor> retrieveTensorFromPool(CallbackContext programContextHandle, std::uint32_t globalId, bool untilize);
+void updateTensorInPool(CallbackContext programContextHandle, TensorRef tensorRef, Tensor srcTensor);
 void updateTensorInPool(CallbackContext programContextHandle, std::uint32_t globalId, Tensor srcTensor);
+size_t getProgramIndex(CallbackContext programContextHandle);
 
 std::vector<Tensor> submit(Device deviceHandle, Binary executableHandle, std::uint32_t programIndex, std::vector<Tensor> &inputs);
 
