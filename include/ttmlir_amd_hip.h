@@ -67,6 +67,18 @@ int ttm_event_record(void *event, void *stream);
 int ttm_event_sync(void *event);
 int ttm_event_elapsed_ms(float *ms, void *start, void *stop);
 
+/* ---- HIP graphs, the device side of trace capture / replay (ttnn begin_trace_capture / end_trace_capture /
+ * execute_trace as called from runtime/lib/ttnn/operations/trace/{begin_trace_capture,end_trace_capture,
+ * execute_trace}.cpp).  Between begin and end every launch made through this library on `stream` is recorded, not run;
+ * end returns an executable graph (and the number of recorded nodes) that ttm_graph_launch replays with one launch.
+ * Recorded launches name their operand addresses: the caller keeps those allocations alive and in place until
+ * ttm_graph_destroy.  Host transfers and synchronisation are not legal on a capturing stream. */
+int ttm_graph_begin_capture(void *stream);
+int ttm_graph_end_capture(void *stream, void **graph_exec, size_t *num_nodes);
+int ttm_graph_launch(void *graph_exec, void *stream);
+int ttm_graph_destroy(void *graph_exec);
+int ttm_stream_is_capturing(void *stream, int *capturing);
+
 /* Plain 16-byte-per-lane device copy kernel: the measured HBM ceiling the layout kernels are
  * compared with, and the calibration kernel for FETCH_SIZE / WRITE_SIZE counters. */
 int ttm_copy_kernel(const void *src, void *dst, size_t bytes, void *stream);

@@ -152,6 +152,16 @@ int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_t repeats, i
 int ttrt_pb_constant(ttrt_builder *pb, const void *data, size_t bytes, int in_dtype, const uint32_t *shape, int rank,
                      const ttrt_layout *layout, uint32_t *out);
 int ttrt_pb_full(ttrt_builder *pb, const uint32_t *shape, int rank, float value, int dtype, int layout, uint32_t *out);
+int ttrt_pb_empty(ttrt_builder *pb, const uint32_t *shape, int rank, int dtype, int layout, uint32_t *out);
+int ttrt_pb_copy(ttrt_builder *pb, uint32_t src, uint32_t dst);
+int ttrt_pb_write_tensor(ttrt_builder *pb, uint32_t host, uint32_t device);
+/* trace ops (include/ttmlir/Target/TTNN/operations/trace.fbs); the trace id is a rank-0 UInt32 host tensor */
+int ttrt_pb_begin_trace_capture(ttrt_builder *pb, uint32_t *trace_id);
+int ttrt_pb_end_trace_capture(ttrt_builder *pb, uint32_t trace_id);
+int ttrt_pb_execute_trace(ttrt_builder *pb, uint32_t trace_id, int blocking);
+int ttrt_pb_capture_or_execute_trace(ttrt_builder *pb, uint32_t capture_program, uint32_t execute_program,
+                                     uint32_t allocate_slots_program, const uint32_t *ins, int n_in, const uint32_t *out_shapes,
+                                     const int *out_ranks, const ttrt_layout *out_layouts, int n_out, uint32_t *outs);
 int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force);
 /* location of the operation added last, and an expected (golden) tensor to embed for a location; data is row-major */
 int ttrt_pb_last_op_loc(ttrt_builder *pb, char *buf, size_t len);

@@ -368,6 +368,78 @@ def test_ttrt_run_checks_embedded_goldens_and_saves_artifacts(orc, tmp_path):
     assert torch.equal(ya, yb) and bool(ya.float().abs().sum() > 0)
 
 
+def _run_traced(binary, device, x, resident):
+    ins = [rt.from_torch(x)] + resident
+    outs = rt.submit(device, binary, binary.get_num_programs() - 1, ins)
+    y = rt.to_torch(rt.to_host(outs[0], untilize=True)[0])
+    return y
+
+
+def test_traced_program_replays_as_a_graph(device, orc):
+    """capture_or_execute_trace (runtime/lib/ttnn/operations/trace/capture_or_execute_trace.cpp:262-357): first submit
+    allocates slots and captures, later submits replay; every replay is compared with the same program run op by op."""
+    T, H, F = 32, 256, 512
+    traced = rt.Binary.load_from_memory(programs.traced_mlp(T, H, F))
+    eager = rt.Binary.load_from_memory(programs.traced_mlp(T, H, F, trace=False))
+    other = rt.Binary.load_from_memory(programs.c4_mlp(96, 256, 512))
+    d = datagen.c4_mlp(T, H, F, seed=21)
+    main = traced.get_num_programs() - 1
+    assert [traced.get_program_name(i) for i in range(1, 5)] == [
+        "trace_0_traced_mlp", "allocate_slots_trace_0_traced_mlp", "run_and_capture_trace_0_traced_mlp", "execute_trace_0_traced_mlp"]
+
+    def resident(binary, prog, wscale=1.0):
+        ts = [d["norm_w"], bf(d["wg"] * wscale), bf(d["wu"]), bf(d["wd"])]
+        return [rt.to_layout(rt.from_torch(t), device, rt.get_layout(binary, prog, k + 1), retain=True) for k, t in enumerate(ts)]
+
+    res_t, res_e = resident(traced, main), resident(eager, 1)
+    rt.clear_stats()
+    f = lambda t: t.float().numpy()
+    g = torch.Generator().manual_seed(5)
+    od = datagen.c4_mlp(96, 256, 512, seed=3)
+    for it in range(5):
+        x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+        y = _run_traced(traced, device, x, res_t)
+        want = _run_traced(eager, device, x, res_e)
+        assert torch.equal(y, want), "replay %d differs from the op-by-op run" % it
+        if it == 0:
+            ref = oracle_mlp(orc, f(x), f(d["norm_w"]), f(bf(d["wg"])), f(bf(d["wu"])), f(bf(d["wd"])), 1e-5)
+            assert np.max(np.abs(f(y) - ref)) <= 2.0 ** -10
+        # unrelated work between replays allocates and frees device memory; the trace's buffers must stay its own
+        harness.execute(other, 1, [od["x"], od["norm_w"], bf(od["wg"]), bf(od["wu"]), bf(od["wd"])], device)
+    assert (rt.get_stat("TraceCacheMiss"), rt.get_stat("CapturedTrace"), rt.get_stat("ExecutedTrace")) == (1, 1, 4)
+    # a parameter replaced by the caller (new tensor, new version) is copied into its slot before the replay
+    res_t2, res_e2 = resident(traced, main, 2.0), resident(eager, 1, 2.0)
+    x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+    y2 = _run_traced(traced, device, x, res_t2)
+    assert torch.equal(y2, _run_traced(eager, device, x, res_e2))
+    assert not torch.equal(y2, _run_traced(traced, device, x, res_t))
+    assert rt.get_stat("CapturedTrace") == 1 and rt.get_stat("ExecutedTrace") == 6
+
+
+def test_host_transfer_inside_a_capture_is_refused_cleanly(device):
+    pb = rt.ProgramBuilder()
+
+    def body(pb, a):
+        y = pb.unary(programs.UNARY["relu"], a[0])
+        pb.from_device(y)                                  # not recordable
+        return [y]
+    emit = programs.add_traced(pb, "bad", [((32, 64), DT.BFloat16, False)], body,
+                               [((32, 64), rt.Layout(ST.Device, TL.Tile, DT.BFloat16))])
+    pb.begin_program("bad")
+    x = pb.input((32, 64), DT.BFloat16, TL.RowMajor, ST.Host)
+    pb.output(emit(pb, [x])[0])
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    xin = torch.randn(32, 64).to(torch.bfloat16)
+    with pytest.raises(RuntimeError, match="while a trace is being captured"):
+        rt.submit(device, binary, 4, [rt.from_torch(xin)])
+    # the stream is usable again and a well-formed trace still captures
+    good = rt.Binary.load_from_memory(programs.c3_linear(32, 64, 64))
+    a, w, bias = datagen.c3_linear(32, 64, 64, seed=1)
+    (y,) = harness.execute(good, 1, [a, bf(w), bias], device)
+    assert bool(torch.isfinite(y.float()).all())
+
+
 def test_submit_errors(device):
     binary = rt.Binary.load_from_memory(programs.c3_linear(32, 64, 64))
     a = rt.from_torch(torch.zeros(32, 64, dtype=torch.bfloat16))

@@ -5,6 +5,8 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "ttm_common.h"
 
@@ -146,8 +148,104 @@ TTM_EXPORT int ttm_stream_create(void **stream) {
   *stream = (void *)s;
   return TTM_OK;
 }
+namespace {
+struct StreamWorkspace {
+  void *ptr = nullptr;
+  size_t bytes = 0;
+  bool recorded = false;          // handed out while the stream was capturing
+  std::vector<void *> retired;    // outgrown allocations that a graph may still name
+};
+std::mutex g_ws_mu;
+std::map<std::pair<int, hipStream_t>, StreamWorkspace> g_ws;
+}  // namespace
+
+int ttm_stream_workspace(hipStream_t stream, size_t bytes, void **ptr) {
+  int dev = 0;
+  TTM_HIP(hipGetDevice(&dev));
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  TTM_HIP(hipStreamIsCapturing(stream, &st));
+  const bool capturing = st != hipStreamCaptureStatusNone;
+  std::lock_guard<std::mutex> g(g_ws_mu);
+  StreamWorkspace &w = g_ws[{dev, stream}];
+  if (w.bytes < bytes) {
+    if (capturing)
+      return ttm_set_error(TTM_ERR_INVALID,
+                           "a kernel needs %zu bytes of stream workspace while the stream is capturing: run the same work "
+                           "once outside the capture first", bytes);
+    if (w.ptr) {
+      if (w.recorded) {
+        w.retired.push_back(w.ptr);
+      } else {
+        TTM_HIP(hipStreamSynchronize(stream));
+        TTM_HIP(hipFree(w.ptr));
+      }
+      w.ptr = nullptr; w.bytes = 0; w.recorded = false;
+    }
+    const size_t unit = (size_t)2 << 20;
+    size_t want = (bytes + unit - 1) / unit * unit;
+    TTM_HIP(hipMalloc(&w.ptr, want));
+    w.bytes = want;
+  }
+  w.recorded |= capturing;
+  *ptr = w.ptr;
+  return TTM_OK;
+}
+
 TTM_EXPORT int ttm_stream_destroy(void *stream) {
-  if (stream) TTM_HIP(hipStreamDestroy((hipStream_t)stream));
+  if (!stream) return TTM_OK;
+  TTM_HIP(hipStreamSynchronize((hipStream_t)stream));
+  {
+    int dev = 0;
+    TTM_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> g(g_ws_mu);
+    auto it = g_ws.find({dev, (hipStream_t)stream});
+    if (it != g_ws.end()) {
+      if (it->second.ptr) (void)hipFree(it->second.ptr);
+      for (void *q : it->second.retired) (void)hipFree(q);
+      g_ws.erase(it);
+    }
+  }
+  TTM_HIP(hipStreamDestroy((hipStream_t)stream));
+  return TTM_OK;
+}
+
+// ---- HIP graphs: record the launches issued on a stream once, replay them with one launch
+TTM_EXPORT int ttm_graph_begin_capture(void *stream) {
+  TTM_REQUIRE(stream != nullptr, "ttm_graph_begin_capture: capture needs a stream of its own, not the null stream");
+  // relaxed mode: allocation calls made by the capturing thread stay legal (they are not recorded)
+  TTM_HIP(hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeRelaxed));
+  return TTM_OK;
+}
+TTM_EXPORT int ttm_graph_end_capture(void *stream, void **graph_exec, size_t *num_nodes) {
+  TTM_REQUIRE(stream && graph_exec, "ttm_graph_end_capture: null argument");
+  *graph_exec = nullptr;
+  hipGraph_t graph = nullptr;
+  TTM_HIP(hipStreamEndCapture((hipStream_t)stream, &graph));
+  TTM_REQUIRE(graph != nullptr, "ttm_graph_end_capture: the capture was invalidated");
+  size_t n = 0;
+  hipError_t e = hipGraphGetNodes(graph, nullptr, &n);
+  if (e == hipSuccess && num_nodes) *num_nodes = n;
+  hipGraphExec_t exec = nullptr;
+  e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(e));
+  *graph_exec = (void *)exec;
+  return TTM_OK;
+}
+TTM_EXPORT int ttm_graph_launch(void *graph_exec, void *stream) {
+  TTM_REQUIRE(graph_exec != nullptr, "ttm_graph_launch: null graph");
+  TTM_HIP(hipGraphLaunch((hipGraphExec_t)graph_exec, (hipStream_t)stream));
+  return TTM_OK;
+}
+TTM_EXPORT int ttm_graph_destroy(void *graph_exec) {
+  if (graph_exec) TTM_HIP(hipGraphExecDestroy((hipGraphExec_t)graph_exec));
+  return TTM_OK;
+}
+TTM_EXPORT int ttm_stream_is_capturing(void *stream, int *capturing) {
+  TTM_REQUIRE(capturing != nullptr, "ttm_stream_is_capturing: null out pointer");
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  TTM_HIP(hipStreamIsCapturing((hipStream_t)stream, &st));
+  *capturing = st != hipStreamCaptureStatusNone;
   return TTM_OK;
 }
 TTM_EXPORT int ttm_stream_sync(void *stream) {

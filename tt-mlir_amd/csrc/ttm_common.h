@@ -32,6 +32,12 @@ int ttm_set_error(int code, const char *fmt, ...) __attribute__((format(printf, 
 
 int ttm_option(const char *name);  // 0 when unset
 
+// Scratch memory of a stream for kernels that need device memory beyond their operands (split-K partial sums).
+// One grow-only allocation per (device, stream): launches on a stream are ordered, so consecutive users do not overlap.
+// Growing allocates with hipMalloc and is refused while the stream is capturing; an allocation that a captured graph may
+// have recorded is never freed before the stream is destroyed.
+int ttm_stream_workspace(hipStream_t stream, size_t bytes, void **ptr);
+
 static inline int64_t ttm_round_up32(int64_t v) { return (v + 31) / 32 * 32; }
 static inline int64_t ttm_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

@@ -1333,23 +1333,10 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       }
       const int64_t per = (int64_t)a.Mt * a.Nt * 1024;
       void *ws = nullptr;
-      static bool pool_kept = false;
-      if (!pool_kept) {   // keep freed workspace memory in the stream-ordered pool instead of returning it at every sync
-        int dev = 0;
-        hipMemPool_t pool;
-        uint64_t keep = UINT64_MAX;
-        if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetDefaultMemPool(&pool, dev) == hipSuccess)
-          (void)hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &keep);
-        (void)hipGetLastError();
-        pool_kept = true;
-      }
-      hipError_t e = hipMallocAsync(&ws, (size_t)(per * slices * batch) * sizeof(float), s);
-      if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "ttm_linear: split-K workspace: %s", hipGetErrorString(e));
+      if (int rc = ttm_stream_workspace(s, (size_t)(per * slices * batch) * sizeof(float), &ws)) return rc;
       p.partial = (float *)ws;
       hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), lds6, s, p);
       hipLaunchKernelGGL(ttm_linear_reduce_k, dim3((unsigned)((per / 4 + 255) / 256), 1, (unsigned)batch), dim3(256), 0, s, p, slices);
-      e = hipFreeAsync(ws, s);
-      if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "ttm_linear: split-K workspace release: %s", hipGetErrorString(e));
       return 0;
     }
   }

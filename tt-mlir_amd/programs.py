@@ -142,3 +142,90 @@ def c5_decoder(seq=2048, hidden=4096, n_q=32, n_kv=8, head_dim=128, ffn=14336, e
     pb.output(out)
     pb.end_program()
     return pb.finish()
+
+
+def add_traced(pb, name, args, body, out_descs):
+    """Adds the four private programs the compiler's trace hoisting emits for a traced region
+    (test/ttmlir/Dialect/TTNN/trace/scenarios/single_add_no_consteval.mlir:5-45) and returns a function that emits the
+    `capture_or_execute_trace` op into the program that is open when it is called.
+
+    args: [(shape, dtype, resident)] - resident arguments live on the device (parameters, const-eval results, caches) and
+    are their own slots; the others arrive on the host, row-major, and are staged into device slots.
+    body(pb, ids) -> [result ids] builds the traced computation on Device / Tile tensors.
+    out_descs: [(shape, Layout)] of the results.
+
+      trace_0_<name>(args..., out slots...)            body, then ttnn.copy of every result into its slot; returns nothing
+      allocate_slots_trace_0_<name>(resident args...)  -> input slots (resident args pass through), output slots
+      run_and_capture_trace_0_<name>(host args..., input slots..., output slots...) -> trace id
+                                                       write_tensor, one eager run, capture of a second run, one replay
+      execute_trace_0_<name>(trace id)                 ttnn.execute_trace
+    """
+    dev_lay = lambda dt: rt.Layout(ST.Device, TL.Tile, dt)
+    # the traced function
+    pb.begin_program("trace_0_" + name, private=True)
+    ids = [pb.input(shape, dt) for shape, dt, _ in args]
+    slots = [pb.input(shape, lay.dtype, lay.layout, lay.storage) for shape, lay in out_descs]
+    for res, slot in zip(body(pb, ids), slots):
+        pb.copy(res, slot)
+    trace_fn = pb.end_program()
+    # slot allocation
+    pb.begin_program("allocate_slots_trace_0_" + name, private=True)
+    resident = iter([pb.input(shape, dt) for shape, dt, res in args if res])
+    for shape, dt, res in args:
+        pb.output(next(resident) if res else pb.empty(shape, dt))
+    for shape, lay in out_descs:
+        pb.output(pb.empty(shape, lay.dtype, lay.layout))
+    allocate = pb.end_program()
+    # capture
+    pb.begin_program("run_and_capture_trace_0_" + name, private=True)
+    staged = [pb.input(shape, dt, TL.RowMajor, ST.Host) for shape, dt, res in args if not res]
+    in_slots = [pb.input(shape, dt) for shape, dt, _ in args]
+    out_slots = [pb.input(shape, lay.dtype, lay.layout, lay.storage) for shape, lay in out_descs]
+    host = iter(staged)
+    for (shape, dt, res), slot in zip(args, in_slots):
+        if not res:
+            pb.write_tensor(next(host), slot)
+    pb.func_call(trace_fn, in_slots + out_slots, [])
+    tid = pb.begin_trace_capture()
+    pb.func_call(trace_fn, in_slots + out_slots, [])
+    pb.end_trace_capture(tid)
+    pb.execute_trace(tid)
+    pb.output(tid)
+    capture = pb.end_program()
+    # replay
+    pb.begin_program("execute_trace_0_" + name, private=True)
+    tid = pb.input((), DT.UInt32, TL.RowMajor, ST.Host)
+    pb.execute_trace(tid)
+    execute = pb.end_program()
+
+    def emit(pb, operands):
+        return pb.capture_or_execute_trace(capture, execute, allocate, operands, out_descs)
+    return emit
+
+
+def traced_mlp(tokens=32, hidden=4096, ffn=14336, eps=1e-5, trace=True):
+    """Decode-sized MLP block (config 4 at `tokens` rows) whose whole body is one traced region: activations arrive on the
+    host, weights are device-resident parameters packed by const-eval outside the trace
+    (test/ttmlir/Dialect/TTNN/trace/scenarios/matmul_multiply_consteval.mlir).  trace=False builds the same program with
+    the body inline, for comparison."""
+    pb = rt.ProgramBuilder()
+    ce, ce_outs = _consteval_pack(pb, "traced_mlp_const_eval_0", [((hidden, ffn), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8),
+                                                                  ((ffn, hidden), DT.BFP_BFloat4)])
+    out_desc = ((tokens, hidden), rt.Layout(ST.Device, TL.Tile, DT.BFloat16))
+    emit = None
+    if trace:
+        args = [((tokens, hidden), DT.BFloat16, False), ((hidden,), DT.BFloat16, True), ((hidden, ffn), DT.BFP_BFloat8, True),
+                ((hidden, ffn), DT.BFP_BFloat8, True), ((ffn, hidden), DT.BFP_BFloat4, True)]
+        emit = add_traced(pb, "traced_mlp", args, lambda pb, a: [_mlp(pb, a[0], a[1], a[2], a[3], a[4], eps)], [out_desc])
+    pb.begin_program("traced_mlp")
+    x = pb.input((tokens, hidden), DT.BFloat16, TL.RowMajor, ST.Host)
+    nw = pb.input((hidden,), DT.BFloat16)
+    wg, wu, wd = pb.input((hidden, ffn), DT.BFloat16), pb.input((hidden, ffn), DT.BFloat16), pb.input((ffn, hidden), DT.BFloat16)
+    qg, qu, qd = pb.load_cached(ce, "traced_mlp_const_eval_0", [wg, wu, wd], ce_outs)
+    if trace:
+        (y,) = emit(pb, [x, nw, qg, qu, qd])
+    else:
+        y = _mlp(pb, pb.to_layout(pb.to_device(x), TL.Tile), nw, qg, qu, qd, eps)
+    pb.output(y)
+    pb.end_program()
+    return pb.finish()

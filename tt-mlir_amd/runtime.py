@@ -589,6 +589,28 @@ class ProgramBuilder:
         s, r = _shape_arg(shape)
         return self._op("ttrt_pb_full", s, r, ctypes.c_float(value), dtype, layout)
 
+    def empty(self, shape, dtype, layout=TensorLayout.Tile):
+        s, r = _shape_arg(shape)
+        return self._op("ttrt_pb_empty", s, r, dtype, layout)
+
+    def copy(self, src, dst):
+        _call("ttrt_pb_copy", self.h, src, dst)
+
+    def write_tensor(self, host, device):
+        _call("ttrt_pb_write_tensor", self.h, host, device)
+
+    def begin_trace_capture(self):
+        return self._op("ttrt_pb_begin_trace_capture")
+
+    def end_trace_capture(self, trace_id):
+        _call("ttrt_pb_end_trace_capture", self.h, trace_id)
+
+    def execute_trace(self, trace_id, blocking=False):
+        _call("ttrt_pb_execute_trace", self.h, trace_id, int(blocking))
+
+    def capture_or_execute_trace(self, capture_program, execute_program, allocate_slots_program, ins, out_descs):
+        return self._multi("ttrt_pb_capture_or_execute_trace", (capture_program, execute_program, allocate_slots_program), ins, out_descs)
+
     def deallocate(self, t, force=False):
         _call("ttrt_pb_deallocate", self.h, t, int(force))
 

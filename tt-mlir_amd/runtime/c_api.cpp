@@ -429,6 +429,22 @@ TTRT_EXPORT int ttrt_pb_constant(ttrt_builder *pb, const void *data, size_t byte
 TTRT_EXPORT int ttrt_pb_full(ttrt_builder *pb, const uint32_t *shape, int rank, float value, int dtype, int layout, uint32_t *out) {
   PB_OP(full(shapeVec(shape, rank), value, static_cast<DataType>(dtype), static_cast<TensorLayout>(layout)));
 }
+TTRT_EXPORT int ttrt_pb_empty(ttrt_builder *pb, const uint32_t *shape, int rank, int dtype, int layout, uint32_t *out) {
+  PB_OP(empty(shapeVec(shape, rank), static_cast<DataType>(dtype), static_cast<TensorLayout>(layout)));
+}
+TTRT_EXPORT int ttrt_pb_copy(ttrt_builder *pb, uint32_t src, uint32_t dst) {
+  return guard([&] { need(pb, "builder"); pb->pb.copy(src, dst); });
+}
+TTRT_EXPORT int ttrt_pb_write_tensor(ttrt_builder *pb, uint32_t host, uint32_t device) {
+  return guard([&] { need(pb, "builder"); pb->pb.writeTensor(host, device); });
+}
+TTRT_EXPORT int ttrt_pb_begin_trace_capture(ttrt_builder *pb, uint32_t *out) { PB_OP(beginTraceCapture()); }
+TTRT_EXPORT int ttrt_pb_end_trace_capture(ttrt_builder *pb, uint32_t trace_id) {
+  return guard([&] { need(pb, "builder"); pb->pb.endTraceCapture(trace_id); });
+}
+TTRT_EXPORT int ttrt_pb_execute_trace(ttrt_builder *pb, uint32_t trace_id, int blocking) {
+  return guard([&] { need(pb, "builder"); pb->pb.executeTrace(trace_id, blocking != 0); });
+}
 TTRT_EXPORT int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force) {
   return guard([&] { need(pb, "builder"); pb->pb.deallocate(in, force != 0); });
 }
@@ -453,6 +469,18 @@ TTRT_EXPORT int ttrt_pb_load_cached(ttrt_builder *pb, uint32_t program_index, co
     need(pb, "builder"); need(outs, "outs");
     auto ids = pb->pb.loadCached(program_index, callee ? callee : "", std::vector<ProgramBuilder::Id>(ins, ins + n_in),
                                  outDescs(out_shapes, out_ranks, out_layouts, n_out));
+    for (size_t i = 0; i < ids.size(); ++i) outs[i] = ids[i];
+  });
+}
+TTRT_EXPORT int ttrt_pb_capture_or_execute_trace(ttrt_builder *pb, uint32_t capture_program, uint32_t execute_program,
+                                                 uint32_t allocate_slots_program, const uint32_t *ins, int n_in,
+                                                 const uint32_t *out_shapes, const int *out_ranks, const ttrt_layout *out_layouts,
+                                                 int n_out, uint32_t *outs) {
+  return guard([&] {
+    need(pb, "builder"); need(outs, "outs");
+    auto ids = pb->pb.captureOrExecuteTrace(capture_program, execute_program, allocate_slots_program,
+                                            std::vector<ProgramBuilder::Id>(ins, ins + n_in),
+                                            outDescs(out_shapes, out_ranks, out_layouts, n_out));
     for (size_t i = 0; i < ids.size(); ++i) outs[i] = ids[i];
   });
 }

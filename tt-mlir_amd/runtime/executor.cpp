@@ -622,6 +622,129 @@ void runFuncCall(const fb::Table &op, ProgramContext &ctx) {
   for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], results[i]);
 }
 
+// ---- traces (runtime/lib/ttnn/operations/trace/*.cpp): a trace is a HIP graph recorded on the device's stream
+Tensor makeTraceIdTensor(std::uint32_t id) {
+  Tensor t = makeHostTensor({}, DataType::UInt32, TensorLayout::RowMajor);
+  std::memcpy(t.handle->data.get(), &id, sizeof(id));
+  return t;
+}
+std::uint32_t traceIdOf(const Tensor &t) {
+  TTRT_ASSERT(t.handle->storage == StorageType::Host && t.handle->dtype == DataType::UInt32 && t.handle->bytes >= 4,
+              "Trace ID must be a UINT32 host scalar");
+  std::uint32_t id = 0;
+  std::memcpy(&id, t.handle->data.get(), sizeof(id));
+  return id;
+}
+void runBeginTraceCapture(const fb::Table &op, ProgramContext &ctx) {
+  std::uint32_t id = ctx.dev->nextTraceId++;
+  beginTraceCapture(ctx.dev, id);
+  ctx.put(op.table(schema::BeginTraceCaptureOp::f_trace_id), makeTraceIdTensor(id));
+}
+void runEndTraceCapture(const fb::Table &op, ProgramContext &ctx) {
+  endTraceCapture(ctx.dev, traceIdOf(ctx.get(op.table(schema::EndTraceCaptureOp::f_trace_id), "end_trace_capture trace id")));
+}
+void runExecuteTrace(const fb::Table &op, ProgramContext &ctx) {
+  executeTrace(ctx.dev, traceIdOf(ctx.get(op.table(schema::ExecuteTraceOp::f_trace_id), "execute_trace trace id")),
+               op.scalar<std::uint8_t>(schema::ExecuteTraceOp::f_blocking, 0) != 0);
+}
+
+// dst <- src for tensors of one shape; src is brought to dst's layout and dtype first (on the device)
+void overwriteTensor(ProgramContext &ctx, Tensor &dst, const Tensor &src, const char *what) {
+  TTRT_ASSERT(dst.handle->shape == src.handle->shape, std::string(what) + ": shape mismatch");
+  Tensor conv = src;
+  if (conv.handle->layout != dst.handle->layout || conv.handle->dtype != dst.handle->dtype)
+    conv = as(ctx, conv, dst.handle->layout, dst.handle->dtype);
+  TTRT_ASSERT(conv.handle->bytes == dst.handle->bytes, std::string(what) + ": size mismatch");
+  if (conv.handle->storage == StorageType::Device && dst.handle->storage == StorageType::Device)
+    TTM_CALL(ttm_copy_kernel(conv.handle->data.get(), dst.handle->data.get(), dst.handle->bytes, ctx.stream()));
+  else
+    memcpy(dst, conv);
+}
+void runWriteTensor(const fb::Table &op, ProgramContext &ctx) {
+  Tensor &host = ctx.get(op.table(schema::WriteTensorOp::f_host_tensor), "write_tensor host");
+  Tensor &dev = ctx.get(op.table(schema::WriteTensorOp::f_device_tensor), "write_tensor device");
+  TTRT_ASSERT(host.handle->storage == StorageType::Host && dev.handle->storage == StorageType::Device,
+              "write_tensor: source must be on host and destination on device");
+  overwriteTensor(ctx, dev, host, "write_tensor");
+  dev.handle->version = host.handle->version;
+}
+void runCopy(const fb::Table &op, ProgramContext &ctx) {
+  Tensor &src = ctx.get(op.table(schema::CopyOp::f_src), "copy src");
+  Tensor &dst = ctx.get(op.table(schema::CopyOp::f_dst), "copy dst");
+  overwriteTensor(ctx, dst, src, "copy");
+}
+
+bool inDeviceMemory(const fb::Table &ref) { return layoutFromTensorRef(ref).storageType == StorageType::Device; }
+
+// Copies the current values of the op's inputs into the persistent input slots; a slot whose version equals its
+// input's already holds the data (device-resident inputs are their own slots).
+void updateTraceInputSlots(const fb::Table &op, ProgramContext &ctx, std::vector<Tensor> &slots, bool deviceResidentOnly) {
+  auto ins = op.tables(schema::CaptureOrExecuteTraceOp::f_inputs);
+  TTRT_ASSERT(ins.size() == slots.size(), "capture_or_execute_trace: mismatched number of input slots");
+  for (std::uint32_t i = 0; i < ins.size(); ++i) {
+    const bool resident = inDeviceMemory(ins[i]);
+    if (deviceResidentOnly && !resident) continue;
+    Tensor &in = ctx.get(ins[i], "trace input");
+    if (in.handle->version == slots[i].handle->version) continue;
+    overwriteTensor(ctx, slots[i], in, "trace input slot");
+    slots[i].handle->version = in.handle->version;
+  }
+}
+void publishTraceOutputs(const fb::Table &op, ProgramContext &ctx, const std::vector<Tensor> &slots) {
+  auto outs = op.tables(schema::CaptureOrExecuteTraceOp::f_outputs);
+  TTRT_ASSERT(outs.size() == slots.size(), "capture_or_execute_trace: mismatched number of output slots");
+  for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], slots[i]);
+}
+void runCaptureOrExecuteTrace(const fb::Table &op, ProgramContext &ctx) {
+  const std::uint32_t captureId = op.scalar<std::uint32_t>(schema::CaptureOrExecuteTraceOp::f_capture_program_id, 0);
+  const std::uint32_t executeId = op.scalar<std::uint32_t>(schema::CaptureOrExecuteTraceOp::f_execute_program_id, 0);
+  const std::uint32_t allocateId = op.scalar<std::uint32_t>(schema::CaptureOrExecuteTraceOp::f_allocate_slots_program_id, 0);
+  auto ins = op.tables(schema::CaptureOrExecuteTraceOp::f_inputs);
+  auto outs = op.tables(schema::CaptureOrExecuteTraceOp::f_outputs);
+  TraceKey key{ctx.binary.id(), ctx.programIndex, captureId, executeId};
+  auto hit = ctx.dev->traceCache.find(key);
+  if (hit == ctx.dev->traceCache.end()) {
+    // allocate the persistent slots once: the allocation program takes the device-resident inputs (their own slots)
+    // and returns the input slots followed by the output slots
+    std::vector<Tensor> resident;
+    for (std::uint32_t i = 0; i < ins.size(); ++i)
+      if (inDeviceMemory(ins[i])) resident.push_back(ctx.get(ins[i], "trace input"));
+    std::vector<Tensor> slots = executeProgram(ctx.dev, ctx.binary, allocateId, resident);
+    TTRT_ASSERT(slots.size() == ins.size() + outs.size(), "capture_or_execute_trace: mismatched number of trace slots, expected " +
+                                                              std::to_string(ins.size() + outs.size()) + " got " + std::to_string(slots.size()));
+    for (Tensor &t : slots) setTensorRetain(t, true);
+    std::vector<Tensor> inputSlots(slots.begin(), slots.begin() + ins.size()), outputSlots(slots.begin() + ins.size(), slots.end());
+    updateTraceInputSlots(op, ctx, inputSlots, /*deviceResidentOnly=*/true);
+    // capture program arguments: host-staged inputs, input slots, output slots; it returns the new trace id
+    std::vector<Tensor> args;
+    for (std::uint32_t i = 0; i < ins.size(); ++i)
+      if (!inDeviceMemory(ins[i])) args.push_back(ctx.get(ins[i], "trace input"));
+    args.insert(args.end(), inputSlots.begin(), inputSlots.end());
+    args.insert(args.end(), outputSlots.begin(), outputSlots.end());
+    std::vector<Tensor> ret = executeProgram(ctx.dev, ctx.binary, captureId, args);
+    TTRT_ASSERT(ret.size() == 1, "Capture program must return exactly the new trace id");
+    const std::uint32_t traceId = traceIdOf(ret[0]);
+    auto it = ctx.dev->traces.find(traceId);
+    TTRT_ASSERT(it != ctx.dev->traces.end(), "capture program returned a trace id that was not captured");
+    // the capture program wrote the host inputs into their slots itself
+    for (std::uint32_t i = 0; i < ins.size(); ++i)
+      if (!inDeviceMemory(ins[i])) inputSlots[i].handle->version = ctx.get(ins[i], "trace input").handle->version;
+    it->second.inputSlots = std::move(inputSlots);
+    it->second.outputSlots = std::move(outputSlots);
+    ctx.dev->traceCache[key] = traceId;
+    publishTraceOutputs(op, ctx, it->second.outputSlots);  // the capture program replayed the trace once
+    debug::Stats::get().incrementStat("TraceCacheMiss");
+    debug::Stats::get().incrementStat("CapturedTrace");
+    return;
+  }
+  TraceData &td = ctx.dev->traces.at(hit->second);
+  updateTraceInputSlots(op, ctx, td.inputSlots, /*deviceResidentOnly=*/false);
+  std::vector<Tensor> idArg{makeTraceIdTensor(td.traceId)};
+  executeProgram(ctx.dev, ctx.binary, executeId, idArg);
+  publishTraceOutputs(op, ctx, td.outputSlots);
+  debug::Stats::get().incrementStat("ExecutedTrace");
+}
+
 void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   auto type = static_cast<OpType>(operation.scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
   fb::Table op = operation.table(schema::Operation::f_type);
@@ -653,6 +776,12 @@ void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   case OpType::DeallocateOp: return runDeallocate(op, ctx);
   case OpType::LoadCachedOp: return runLoadCached(op, ctx);
   case OpType::FuncCallOp: return runFuncCall(op, ctx);
+  case OpType::BeginTraceCaptureOp: return runBeginTraceCapture(op, ctx);
+  case OpType::EndTraceCaptureOp: return runEndTraceCapture(op, ctx);
+  case OpType::ExecuteTraceOp: return runExecuteTrace(op, ctx);
+  case OpType::CaptureOrExecuteTraceOp: return runCaptureOrExecuteTrace(op, ctx);
+  case OpType::WriteTensorOp: return runWriteTensor(op, ctx);
+  case OpType::CopyOp: return runCopy(op, ctx);
   default: fatal(std::string("Unsupported operation type: ") + schema::opTypeName(type));
   }
 }
@@ -754,6 +883,14 @@ OpRefs opRefs(const fb::Table &operation) {
   case OpType::DeallocateOp: in(schema::DeallocateOp::f_in); break;
   case OpType::LoadCachedOp: inVec(schema::LoadCachedOp::f_inputs); outVec(schema::LoadCachedOp::f_outputs); break;
   case OpType::FuncCallOp: inVec(schema::FuncCallOp::f_inputs); outVec(schema::FuncCallOp::f_outputs); break;
+  case OpType::CaptureOrExecuteTraceOp:
+    inVec(schema::CaptureOrExecuteTraceOp::f_inputs); outVec(schema::CaptureOrExecuteTraceOp::f_outputs);
+    break;
+  case OpType::WriteTensorOp: in(schema::WriteTensorOp::f_host_tensor); in(schema::WriteTensorOp::f_device_tensor); break;
+  case OpType::CopyOp: in(schema::CopyOp::f_src); in(schema::CopyOp::f_dst); break;
+  case OpType::BeginTraceCaptureOp: out(schema::BeginTraceCaptureOp::f_trace_id); break;
+  case OpType::EndTraceCaptureOp: in(schema::EndTraceCaptureOp::f_trace_id); break;
+  case OpType::ExecuteTraceOp: in(schema::ExecuteTraceOp::f_trace_id); break;
   default: break;
   }
   return r;

@@ -542,6 +542,75 @@ ProgramBuilder::Id ProgramBuilder::full(const std::vector<std::uint32_t> &shape,
   addOp(OpType::FullOp, b_.endTable(), "ttnn.full " + shapeStr(shape));
   return out;
 }
+ProgramBuilder::Id ProgramBuilder::empty(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout) {
+  Id out = newTensor(Desc{shape, dtype, layout, StorageType::Device});
+  std::vector<std::int64_t> sv(shape.begin(), shape.end());
+  Off s = b_.createScalarVector(sv), o = tensorRef(out);
+  b_.startTable(EmptyOp::kNumFields);
+  b_.addOffset(EmptyOp::f_shape, s);
+  b_.addScalar<std::uint16_t>(EmptyOp::f_dtype, static_cast<std::uint16_t>(dtype));
+  b_.addScalar<std::uint16_t>(EmptyOp::f_layout, static_cast<std::uint16_t>(layout));
+  b_.addOffset(EmptyOp::f_out, o);
+  addOp(OpType::EmptyOp, b_.endTable(), "ttnn.empty " + shapeStr(shape));
+  return out;
+}
+void ProgramBuilder::copy(Id src, Id dst) {
+  Off s = tensorRef(src), d = tensorRef(dst);
+  b_.startTable(CopyOp::kNumFields);
+  b_.addOffset(CopyOp::f_src, s);
+  b_.addOffset(CopyOp::f_dst, d);
+  addOp(OpType::CopyOp, b_.endTable(), "ttnn.copy");
+}
+void ProgramBuilder::writeTensor(Id host, Id device) {
+  Off h = tensorRef(host), d = tensorRef(device);
+  b_.startTable(WriteTensorOp::kNumFields);
+  b_.addOffset(WriteTensorOp::f_host_tensor, h);
+  b_.addOffset(WriteTensorOp::f_device_tensor, d);
+  b_.addScalarDefault<std::uint8_t>(WriteTensorOp::f_blocking, 1, 0);
+  addOp(OpType::WriteTensorOp, b_.endTable(), "ttnn.write_tensor");
+}
+ProgramBuilder::Id ProgramBuilder::beginTraceCapture() {
+  Id out = newTensor(Desc{{}, DataType::UInt32, TensorLayout::RowMajor, StorageType::Host});
+  Off o = tensorRef(out);
+  b_.startTable(BeginTraceCaptureOp::kNumFields);
+  b_.addOffset(BeginTraceCaptureOp::f_trace_id, o);
+  addOp(OpType::BeginTraceCaptureOp, b_.endTable(), "ttnn.begin_trace_capture");
+  return out;
+}
+void ProgramBuilder::endTraceCapture(Id traceId) {
+  Off t = tensorRef(traceId);
+  b_.startTable(EndTraceCaptureOp::kNumFields);
+  b_.addOffset(EndTraceCaptureOp::f_trace_id, t);
+  addOp(OpType::EndTraceCaptureOp, b_.endTable(), "ttnn.end_trace_capture");
+}
+void ProgramBuilder::executeTrace(Id traceId, bool blocking) {
+  Off t = tensorRef(traceId);
+  b_.startTable(ExecuteTraceOp::kNumFields);
+  b_.addOffset(ExecuteTraceOp::f_trace_id, t);
+  b_.addScalarDefault<std::uint8_t>(ExecuteTraceOp::f_blocking, blocking, 0);
+  addOp(OpType::ExecuteTraceOp, b_.endTable(), "ttnn.execute_trace");
+}
+std::vector<ProgramBuilder::Id> ProgramBuilder::captureOrExecuteTrace(std::uint32_t captureProgram, std::uint32_t executeProgram,
+                                                                      std::uint32_t allocateSlotsProgram, const std::vector<Id> &ins,
+                                                                      const std::vector<Desc> &outs) {
+  std::vector<Id> ids;
+  std::vector<Off> ir, orf;
+  for (Id t : ins) ir.push_back(tensorRef(t));
+  for (const Desc &d : outs) {
+    ids.push_back(newTensor(d));
+    orf.push_back(tensorRef(ids.back()));
+  }
+  Off iv = b_.createOffsetVector(ir), ov = b_.createOffsetVector(orf);
+  b_.startTable(CaptureOrExecuteTraceOp::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(CaptureOrExecuteTraceOp::f_capture_program_id, captureProgram, 0);
+  b_.addScalarDefault<std::uint32_t>(CaptureOrExecuteTraceOp::f_execute_program_id, executeProgram, 0);
+  b_.addScalarDefault<std::uint32_t>(CaptureOrExecuteTraceOp::f_allocate_slots_program_id, allocateSlotsProgram, 0);
+  b_.addOffset(CaptureOrExecuteTraceOp::f_inputs, iv);
+  b_.addOffset(CaptureOrExecuteTraceOp::f_outputs, ov);
+  addOp(OpType::CaptureOrExecuteTraceOp, b_.endTable(),
+        "ttnn.capture_or_execute_trace capture #" + std::to_string(captureProgram) + " execute #" + std::to_string(executeProgram));
+  return ids;
+}
 void ProgramBuilder::deallocate(Id in, bool force) {
   Off i = tensorRef(in);
   b_.startTable(DeallocateOp::kNumFields);

@@ -50,6 +50,14 @@ public:
   Id constant(const void *data, size_t bytes, DataType inDtype, const std::vector<std::uint32_t> &shape, DataType dtype,
               TensorLayout layout, StorageType storage);
   Id full(const std::vector<std::uint32_t> &shape, float value, DataType dtype, TensorLayout layout);
+  Id empty(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout);
+  void copy(Id src, Id dst);                 // ttnn.copy: dst <- src, both on device
+  void writeTensor(Id host, Id device);      // ttnn.write_tensor: device <- host
+  Id beginTraceCapture();                    // returns the trace id tensor (rank-0 UInt32 on host)
+  void endTraceCapture(Id traceId);
+  void executeTrace(Id traceId, bool blocking);
+  std::vector<Id> captureOrExecuteTrace(std::uint32_t captureProgram, std::uint32_t executeProgram, std::uint32_t allocateSlotsProgram,
+                                        const std::vector<Id> &ins, const std::vector<Desc> &outs);
   void deallocate(Id in, bool force);
   std::vector<Id> loadCached(std::uint32_t programIdx, const std::string &callee, const std::vector<Id> &ins, const std::vector<Desc> &outs);
   std::vector<Id> funcCall(std::uint32_t programIdx, const std::vector<Id> &ins, const std::vector<Desc> &outs);

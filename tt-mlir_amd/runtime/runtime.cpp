@@ -7,7 +7,10 @@
 #include <fstream>
 #include <limits>
 #include <map>
+#include <mutex>
+#include <set>
 #include <sstream>
+#include <thread>
 
 #include "runtime_impl.h"
 
@@ -406,15 +409,37 @@ struct DevicePool {
   std::mutex mu;
   std::multimap<size_t, void *> freeBlocks;
   size_t cachedBytes = 0;
+  // While a trace is being recorded on this thread, blocks that are released stay with the recording (they may be
+  // reused by later launches of the same recording, whose order the graph keeps) and every block the recording
+  // touched is pinned: it never returns to freeBlocks until the trace is released.
+  bool recording = false;
+  std::thread::id recorder;
+  std::multimap<size_t, void *> recordFree;
+  std::map<void *, size_t> recordTouched;
+  std::set<void *> pinned;
+
+  static size_t rounded(size_t bytes) { return std::max<size_t>(512, (bytes + 511) / 512 * 512); }
+  bool recordingHere() const { return recording && recorder == std::this_thread::get_id(); }
+
   void *alloc(size_t bytes) {
-    size_t sz = std::max<size_t>(512, (bytes + 511) / 512 * 512);
+    size_t sz = rounded(bytes);
     {
       std::lock_guard<std::mutex> g(mu);
+      const bool rec = recordingHere();
+      if (rec) {
+        auto it = recordFree.find(sz);
+        if (it != recordFree.end()) {
+          void *p = it->second;
+          recordFree.erase(it);
+          return p;
+        }
+      }
       auto it = freeBlocks.find(sz);
       if (it != freeBlocks.end()) {
         void *p = it->second;
         freeBlocks.erase(it);
         cachedBytes -= sz;
+        if (rec) { recordTouched[p] = sz; pinned.insert(p); }
         return p;
       }
     }
@@ -424,13 +449,49 @@ struct DevicePool {
       release();
       TTM_CALL(ttm_malloc(&p, sz));
     }
+    std::lock_guard<std::mutex> g(mu);
+    if (recordingHere()) { recordTouched[p] = sz; pinned.insert(p); }
     return p;
   }
   void free(void *p, size_t bytes) {
-    size_t sz = std::max<size_t>(512, (bytes + 511) / 512 * 512);
+    size_t sz = rounded(bytes);
     std::lock_guard<std::mutex> g(mu);
+    if (recordingHere()) {
+      // a block that existed before the recording and is released inside it may still be read by recorded launches
+      recordTouched[p] = sz;
+      pinned.insert(p);
+      recordFree.emplace(sz, p);
+      return;
+    }
+    if (pinned.count(p)) return;  // owned by a trace; comes back through unpin()
     freeBlocks.emplace(sz, p);
     cachedBytes += sz;
+  }
+  void beginRecording() {
+    std::lock_guard<std::mutex> g(mu);
+    TTRT_ASSERT(!recording, "a trace is already being recorded");
+    recording = true;
+    recorder = std::this_thread::get_id();
+    recordFree.clear();
+    recordTouched.clear();
+  }
+  std::vector<std::pair<void *, size_t>> endRecording() {
+    std::lock_guard<std::mutex> g(mu);
+    std::vector<std::pair<void *, size_t>> out(recordTouched.begin(), recordTouched.end());
+    recording = false;
+    recordFree.clear();
+    recordTouched.clear();
+    return out;
+  }
+  // blocks of a released trace go back into circulation, except those a live tensor still holds (their deleter returns them)
+  void unpin(const std::vector<std::pair<void *, size_t>> &blocks, const std::set<void *> &stillHeld) {
+    std::lock_guard<std::mutex> g(mu);
+    for (const auto &b : blocks) {
+      pinned.erase(b.first);
+      if (stillHeld.count(b.first)) continue;
+      freeBlocks.emplace(b.second, b.first);
+      cachedBytes += b.second;
+    }
   }
   void release() {
     std::lock_guard<std::mutex> g(mu);
@@ -470,9 +531,74 @@ Device openMeshDevice(const MeshDeviceOptions &options) {
   return Device{st};
 }
 
+void requireNotCapturing(const std::shared_ptr<DeviceState> &dev, const char *what) {
+  TTRT_ASSERT(!(dev && dev->capturing), std::string(what) + " is not possible while a trace is being captured: "
+                                           "host transfers and waits cannot be recorded");
+}
+
+void beginTraceCapture(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId) {
+  TTRT_ASSERT(dev && dev->open, "begin_trace_capture: device is not open");
+  TTRT_ASSERT(!dev->capturing, "begin_trace_capture: a capture is already in progress on this device");
+  pool().beginRecording();
+  int rc = ttm_graph_begin_capture(dev->stream);
+  if (rc != 0) {
+    pool().unpin(pool().endRecording(), {});
+    hipCheck(rc, "ttm_graph_begin_capture");
+  }
+  dev->capturing = true;
+  dev->capturingTraceId = traceId;
+}
+
+void endTraceCapture(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId) {
+  TTRT_ASSERT(dev && dev->capturing, "end_trace_capture: no capture is in progress");
+  TTRT_ASSERT(dev->capturingTraceId == traceId, "end_trace_capture: trace id does not match the capture in progress");
+  dev->capturing = false;
+  TraceData td;
+  td.traceId = traceId;
+  td.blocks = pool().endRecording();
+  int rc = ttm_graph_end_capture(dev->stream, &td.graphExec, &td.numNodes);
+  if (rc != 0) {
+    pool().unpin(td.blocks, {});
+    hipCheck(rc, "ttm_graph_end_capture");
+  }
+  dev->traces[traceId] = std::move(td);
+}
+
+void abortTraceCapture(const std::shared_ptr<DeviceState> &dev) {
+  if (!dev || !dev->capturing) return;
+  dev->capturing = false;
+  auto blocks = pool().endRecording();
+  void *exec = nullptr;
+  size_t nodes = 0;
+  if (ttm_graph_end_capture(dev->stream, &exec, &nodes) == 0 && exec) ttm_graph_destroy(exec);
+  pool().unpin(blocks, {});
+}
+
+void executeTrace(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId, bool blocking) {
+  TTRT_ASSERT(dev && dev->open, "execute_trace: device is not open");
+  TTRT_ASSERT(!dev->capturing, "execute_trace: a capture is in progress");
+  auto it = dev->traces.find(traceId);
+  TTRT_ASSERT(it != dev->traces.end(), "execute_trace: unknown trace id " + std::to_string(traceId));
+  TTM_CALL(ttm_graph_launch(it->second.graphExec, dev->stream));
+  if (blocking) TTM_CALL(ttm_stream_sync(dev->stream));
+}
+
+void releaseTrace(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId) {
+  auto it = dev->traces.find(traceId);
+  if (it == dev->traces.end()) return;
+  TTM_CALL(ttm_stream_sync(dev->stream));
+  TTM_CALL(ttm_graph_destroy(it->second.graphExec));
+  pool().unpin(it->second.blocks, {});
+  for (auto kv = dev->traceCache.begin(); kv != dev->traceCache.end();)
+    kv = kv->second == traceId ? dev->traceCache.erase(kv) : std::next(kv);
+  dev->traces.erase(it);
+}
+
 void closeMeshDevice(Device d) {
   TTRT_ASSERT(d.handle && d.handle->open, "closeMeshDevice: device is not open");
+  TTRT_ASSERT(!d.handle->capturing, "closeMeshDevice: a trace capture is in progress");
   TTM_CALL(ttm_stream_sync(d.handle->stream));
+  while (!d.handle->traces.empty()) releaseTrace(d.handle, d.handle->traces.begin()->first);
   pool().release();
   TTM_CALL(ttm_stream_destroy(d.handle->stream));
   d.handle->stream = nullptr;
@@ -601,8 +727,10 @@ std::vector<std::byte> getTensorDataBuffer(Tensor t) {
 void wait(Event) {}
 void wait(Tensor t, std::optional<std::uint8_t>) {
   TTRT_ASSERT(t.handle != nullptr, "wait: null tensor");
-  if (t.handle->storage == StorageType::Device && t.handle->device && t.handle->device->open)
+  if (t.handle->storage == StorageType::Device && t.handle->device && t.handle->device->open) {
+    requireNotCapturing(t.handle->device, "wait");
     TTM_CALL(ttm_stream_sync(t.handle->device->stream));
+  }
 }
 void wait(const std::vector<Tensor> &ts, std::optional<std::uint8_t> cq) {
   for (const auto &t : ts) wait(t, cq);
@@ -622,6 +750,7 @@ static int ttmDtype(DataType dt) { return static_cast<int>(dt); }  // same numbe
 
 Tensor toDevice(const Tensor &h, const std::shared_ptr<DeviceState> &dev) {
   TTRT_ASSERT(h.handle->storage == StorageType::Host, "toDevice: tensor is not on the host");
+  requireNotCapturing(dev, "a host to device transfer");
   Tensor d = makeDeviceTensor(dev, h.handle->shape, h.handle->dtype, h.handle->layout);
   TTM_CALL(ttm_memcpy_h2d(d.handle->data.get(), h.handle->data.get(), h.handle->bytes, dev->stream));
   TTM_CALL(ttm_stream_sync(dev->stream));  // the host buffer may be borrowed: do not outlive the call
@@ -630,6 +759,7 @@ Tensor toDevice(const Tensor &h, const std::shared_ptr<DeviceState> &dev) {
 
 Tensor fromDevice(const Tensor &d) {
   TTRT_ASSERT(d.handle->storage == StorageType::Device, "fromDevice: tensor is not on the device");
+  requireNotCapturing(d.handle->device, "a device to host transfer");
   Tensor h = makeHostTensor(d.handle->shape, d.handle->dtype, d.handle->layout);
   TTM_CALL(ttm_memcpy_d2h(h.handle->data.get(), d.handle->data.get(), d.handle->bytes, d.handle->device->stream));
   TTM_CALL(ttm_stream_sync(d.handle->device->stream));
@@ -738,9 +868,11 @@ void memcpy(Tensor dst, Tensor src) {
   if (!dDev && !sDev) {
     std::memcpy(dst.handle->data.get(), src.handle->data.get(), src.handle->bytes);
   } else if (dDev && !sDev) {
+    requireNotCapturing(dst.handle->device, "a host to device copy");
     TTM_CALL(ttm_memcpy_h2d(dst.handle->data.get(), src.handle->data.get(), src.handle->bytes, dst.handle->device->stream));
     TTM_CALL(ttm_stream_sync(dst.handle->device->stream));
   } else if (!dDev && sDev) {
+    requireNotCapturing(src.handle->device, "a device to host copy");
     TTM_CALL(ttm_memcpy_d2h(dst.handle->data.get(), src.handle->data.get(), src.handle->bytes, src.handle->device->stream));
     TTM_CALL(ttm_stream_sync(src.handle->device->stream));
   } else {
@@ -751,7 +883,12 @@ void memcpy(Tensor dst, Tensor src) {
 std::vector<Tensor> submit(Device device, Binary binary, std::uint32_t programIndex, std::vector<Tensor> &inputs) {
   TTRT_ASSERT(device.handle && device.handle->open, "submit: device is not open");
   TTRT_ASSERT(binary.handle != nullptr, "submit: null binary");
-  return executeProgram(device.handle, binary, programIndex, inputs);
+  try {
+    return executeProgram(device.handle, binary, programIndex, inputs);
+  } catch (...) {
+    abortTraceCapture(device.handle);  // an op that failed while a trace was being recorded must not leave the stream capturing
+    throw;
+  }
 }
 
 // ---------------------------------------------------------------------------- debug

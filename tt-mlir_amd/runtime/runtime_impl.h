@@ -1,7 +1,10 @@
 // Internal state behind the opaque handles of runtime.h.
 #pragma once
 #include <atomic>
+#include <map>
 #include <mutex>
+#include <tuple>
+#include <utility>
 
 #include "runtime.h"
 #include "ttmlir_amd_hip.h"
@@ -15,13 +18,45 @@ using ::tt::target::TensorLayout;
 void hipCheck(int status, const char *what);
 #define TTM_CALL(expr) ::tt::runtime::hipCheck((expr), #expr)
 
+// One captured trace: an executable HIP graph plus everything its recorded launches name.  The slots are the
+// persistent tensors the trace reads and writes (TraceData, runtime/include/tt/runtime/detail/ttnn/types/trace_cache.h);
+// `blocks` are the device allocations that held intermediates while the trace was recorded - they stay out of
+// circulation until the trace is released, so a replay can never write into memory that was handed to someone else.
+struct TraceData {
+  std::uint32_t traceId = 0;
+  void *graphExec = nullptr;
+  size_t numNodes = 0;
+  std::vector<Tensor> inputSlots, outputSlots;
+  std::vector<std::pair<void *, size_t>> blocks;
+};
+
+// (binary id, main program, capture program, execute program): MainProgramKey + CaptureExecuteProgramKey of the reference
+using TraceKey = std::tuple<std::uint64_t, std::uint32_t, std::uint32_t, std::uint32_t>;
+
 struct DeviceState {
   int deviceId = 0;
   void *stream = nullptr;  // hipStream_t: all work of this device is ordered on it
   bool open = false;
   std::mutex mu;           // submit is re-entrant per device, one program at a time per stream
+  // trace state
+  bool capturing = false;                         // between begin_trace_capture and end_trace_capture
+  std::uint32_t capturingTraceId = 0;
+  std::uint32_t nextTraceId = 1;
+  std::map<std::uint32_t, TraceData> traces;      // by trace id: graphs recorded on this device
+  std::map<TraceKey, std::uint32_t> traceCache;   // capture_or_execute_trace -> trace id
   ~DeviceState();
 };
+
+// trace capture on a device's stream (runtime.cpp): device allocations made or released between begin and end belong to
+// the trace afterwards
+void beginTraceCapture(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId);
+void endTraceCapture(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId);
+void executeTrace(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId, bool blocking);
+void releaseTrace(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId);
+void abortTraceCapture(const std::shared_ptr<DeviceState> &dev);  // no-op when no capture is in progress
+// fails with `what` in the message when the device's stream is recording a trace (host transfers and waits are not
+// recordable)
+void requireNotCapturing(const std::shared_ptr<DeviceState> &dev, const char *what);
 
 struct TensorImpl {
   std::vector<std::uint32_t> shape;  // logical shape
