@@ -168,6 +168,39 @@ int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int 
              int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale,
              void *stream);
 
+/* ---- decode path: rotary embedding, KV-cache writes, attention of one new token over the cache.  TILE layout
+ * throughout; positions (update index, current position, page table) are Int32 / UInt32 values in DEVICE memory, read
+ * by the kernels, so the launches can be recorded into a graph and replayed with new positions.
+ *
+ * ttm_rotary_embedding: ::ttnn::experimental::rotary_embedding (runtime/lib/ttnn/operations/transformer/
+ *   rotary_embedding.cpp:14-31; formula include/ttmlir/Dialect/TTNN/IR/TTNNOps.td:4002-4016 and
+ *   test/python/golden/ttir_ops/fusing/test_rope_fusing.py:24-33): out = x * cos + rotate_half(x) * sin with
+ *   rotate_half(x) = concat(-x[D/2:], x[:D/2]).  x / out [batch, rows, cols], cos / sin [cache_rows, cols], BFloat16 or
+ *   Float32; row s uses cache row s, or cache row token_index for every row when token_index >= 0 (decode mode).
+ * ttm_update_cache: ::ttnn::update_cache (operations/kv_cache/update_cache.cpp:14-60; golden tools/golden/mapping.py:
+ *   3614-3671): cache[batch_offset + b, h, *update_index, :] = input[0, h, b, :] for b < input_users; cache
+ *   [users, heads, max_seq, head_dim], input [1, heads, input_users, head_dim]; an index outside [0, max_seq) writes nothing.
+ * ttm_fill_cache: ::ttnn::fill_cache (operations/kv_cache/fill_cache.cpp:12-18; golden mapping.py:3582-3611):
+ *   cache[batch_offset, :, 0:seq, :] = input[0, :, :, :], input [1, heads, seq, head_dim]; the rows up to the next
+ *   multiple of 32 receive the input's tile padding (zeros), as in the golden.
+ * ttm_sdpa_decode: ::ttnn::transformer::scaled_dot_product_attention_decode and its paged form
+ *   (operations/transformer/scaled_dot_product_attention_decode.cpp, paged_scaled_dot_product_attention_decode.cpp;
+ *   golden mapping.py:2417-2481): q / out [1, batch, heads, head_dim]; k / v [batch, kv_heads, seq, head_dim], or with a
+ *   page table [batch, pages_per_user] pages [blocks, kv_heads, page_block, head_dim] where seq = pages_per_user *
+ *   page_block; BFloat16.  scores = (q k^T + mask) * scale, mask additive BFloat16 [batch, 1, mask_heads, seq] or NULL;
+ *   with is_causal and cur_pos [batch] keys after cur_pos[b] are excluded; scale <= 0 means 1/sqrt(head_dim); softmax in
+ *   fp32.  Uses the stream's workspace for per-slice partial results. */
+int ttm_rotary_embedding(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype, int64_t batch,
+                         int64_t rows, int64_t cols, int64_t cache_rows, int64_t token_index, void *stream);
+int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users, int64_t heads,
+                     int64_t max_seq, int64_t head_dim, int64_t input_users, int64_t batch_offset, void *stream);
+int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t users, int64_t heads, int64_t max_seq,
+                   int64_t head_dim, int64_t seq, int64_t batch_offset, void *stream);
+int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
+                    const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out, int dtype,
+                    int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal,
+                    float scale, void *stream);
+
 /* Kernel-variant selection for measurement (name -> small integer); unknown names fail. */
 int ttm_set_option(const char *name, int value);
 int ttm_get_option(const char *name, int *value);

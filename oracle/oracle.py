@@ -38,6 +38,10 @@ def lib():
             "orc_tilize": ([vp, vp, i64, i64, i64, i32], None),
             "orc_untilize": ([vp, vp, i64, i64, i64, i32], None),
             "orc_bfp_tile_bytes": ([i32], i64),
+            "orc_rotary_embedding_f32": ([vp, vp, vp, vp, i64, i64, i64, i64], None),
+            "orc_update_cache_f32": ([vp, vp, i64, i64, i64, i64, i64, i64], None),
+            "orc_fill_cache_f32": ([vp, vp, i64, i64, i64, i64, i64], None),
+            "orc_sdpa_decode_f32": ([vp, vp, vp, vp, vp, i32, vp, i64, i64, i64, i64, i64, i32, f32], None),
             "orc_bfp_pack_tiles": ([vp, vp, i64, i32], None),
             "orc_bfp_unpack_tiles": ([vp, vp, i64, i32], None),
             "orc_bfp_pack_rm": ([vp, vp, i64, i64, i64, i32], None),
@@ -292,4 +296,45 @@ def sdpa(q, k, v, mask=None, is_causal=False, scale=None):
     out = np.empty_like(q)
     lib().orc_sdpa_f32(_p(q), _p(k), _p(v), _p(mask), mh, _p(out), B, Hq, Hkv, Sq, Sk, D, int(is_causal),
                        float(scale) if scale else 0.0)
+    return out
+
+
+def rotary_embedding(x, cos, sin, token_index=None):
+    """x [..., rows, D], cos / sin [..., cache_rows, D] (leading 1s dropped)."""
+    x = _c(x, np.float32)
+    D = x.shape[-1]
+    cos, sin = _c(cos, np.float32).reshape(-1, D), _c(sin, np.float32).reshape(-1, D)
+    rows = x.shape[-2]
+    out = np.empty_like(x)
+    lib().orc_rotary_embedding_f32(_p(x), _p(cos), _p(sin), _p(out), x.size // (rows * D), rows, D,
+                                   -1 if token_index is None else int(token_index))
+    return out
+
+
+def update_cache(cache, inp, update_index, batch_offset=0):
+    cache, inp = _c(cache, np.float32).copy(), _c(inp, np.float32)
+    U, H, S, D = cache.shape
+    lib().orc_update_cache_f32(_p(cache), _p(inp), H, S, D, inp.shape[2], int(update_index), int(batch_offset))
+    return cache
+
+
+def fill_cache(cache, inp, batch_offset=0):
+    cache, inp = _c(cache, np.float32).copy(), _c(inp, np.float32)
+    U, H, S, D = cache.shape
+    lib().orc_fill_cache_f32(_p(cache), _p(inp), H, S, D, inp.shape[2], int(batch_offset))
+    return cache
+
+
+def sdpa_decode(q, k, v, cur_pos=None, mask=None, is_causal=True, scale=None):
+    q, k, v = _c(q, np.float32), _c(k, np.float32), _c(v, np.float32)
+    _, B, H, D = q.shape
+    _, Hkv, S, _ = k.shape
+    cp = None if cur_pos is None else np.ascontiguousarray(cur_pos, dtype=np.int32)
+    mh = 1
+    if mask is not None:
+        mask = _c(mask, np.float32)
+        mh = mask.shape[2]
+    out = np.empty_like(q)
+    lib().orc_sdpa_decode_f32(_p(q), _p(k), _p(v), _p(cp), _p(mask), mh, _p(out), B, H, Hkv, S, D, int(is_causal),
+                              float(scale) if scale else 0.0)
     return out

@@ -524,3 +524,81 @@ void orc_sdpa_f32(const float *q, const float *k, const float *v, const float *m
     free(s);
   }
 }
+
+/* ------------------------------------------------------------------ decode path
+ * Rotary embedding: out = x * cos + rotate_half(x) * sin, rotate_half(x) = concat(-x[D/2:], x[:D/2])
+ * (include/ttmlir/Dialect/TTNN/IR/TTNNOps.td:4002-4016; test/python/golden/ttir_ops/fusing/test_rope_fusing.py:24-33).
+ * x [batch, rows, D]; cos / sin [cache_rows, D]; row s reads cache row s, or row token_index when token_index >= 0. */
+void orc_rotary_embedding_f32(const float *x, const float *cosc, const float *sinc, float *out, int64_t batch,
+                              int64_t rows, int64_t D, int64_t token_index) {
+  const int64_t half = D / 2;
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t s = 0; s < rows; ++s) {
+      const float *xr = x + (b * rows + s) * D;
+      const int64_t cr = token_index >= 0 ? token_index : s;
+      const float *c = cosc + cr * D, *sn = sinc + cr * D;
+      float *o = out + (b * rows + s) * D;
+      for (int64_t d = 0; d < D; ++d) {
+        const float rot = d < half ? -xr[d + half] : xr[d - half];
+        o[d] = xr[d] * c[d] + rot * sn[d];
+      }
+    }
+}
+
+/* update_cache (tools/golden/mapping.py:3614-3671): cache [U,H,S,D] in place;
+ * cache[batch_offset + b, h, idx, :] = input[0, h, b, :], input [1,H,Bin,D]. */
+void orc_update_cache_f32(float *cache, const float *input, int64_t H, int64_t S, int64_t D, int64_t Bin,
+                          int64_t idx, int64_t batch_offset) {
+  for (int64_t b = 0; b < Bin; ++b)
+    for (int64_t h = 0; h < H; ++h)
+      memcpy(cache + (((batch_offset + b) * H + h) * S + idx) * D, input + (h * Bin + b) * D, sizeof(float) * D);
+}
+
+/* fill_cache (tools/golden/mapping.py:3582-3611 with the runner's batch_offset, operations/kv_cache/fill_cache.cpp:
+ * 12-18): cache[batch_offset, :, :seq, :] = input[0]; rows seq .. round_up(seq, 32) become 0 when they exist. */
+void orc_fill_cache_f32(float *cache, const float *input, int64_t H, int64_t S, int64_t D, int64_t seq,
+                        int64_t batch_offset) {
+  int64_t padded = (seq + 31) / 32 * 32;
+  for (int64_t h = 0; h < H; ++h) {
+    float *dst = cache + ((batch_offset * H + h) * S) * D;
+    memcpy(dst, input + h * seq * D, sizeof(float) * seq * D);
+    if (seq < padded && padded <= S) memset(dst + seq * D, 0, sizeof(float) * (padded - seq) * D);
+  }
+}
+
+/* Attention of one new token (tools/golden/mapping.py:2417-2481): q [1,B,H,D], k / v [B,Hkv,S,D], mask (optional)
+ * [B,1,mask_heads,S] additive BEFORE the scale, cur_pos (optional, with is_causal) excludes keys j > cur_pos[b];
+ * scale <= 0 means 1/sqrt(D).  out [1,B,H,D]. */
+void orc_sdpa_decode_f32(const float *q, const float *k, const float *v, const int32_t *cur_pos, const float *mask,
+                         int mask_heads, float *out, int64_t B, int64_t H, int64_t Hkv, int64_t S, int64_t D,
+                         int is_causal, float scale) {
+  if (!(scale > 0.0f)) scale = 1.0f / sqrtf((float)D);
+  int64_t rep = H / Hkv;
+  float *s = (float *)malloc(sizeof(float) * S);
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t h = 0; h < H; ++h) {
+      const float *qi = q + (b * H + h) * D;
+      int64_t hk = h / rep;
+      float mx = -INFINITY;
+      for (int64_t j = 0; j < S; ++j) {
+        const float *kj = k + ((b * Hkv + hk) * S + j) * D;
+        float acc = 0.0f;
+        for (int64_t d = 0; d < D; ++d) acc += qi[d] * kj[d];
+        if (mask) acc += mask[(b * mask_heads + (mask_heads == 1 ? 0 : h)) * S + j];
+        else if (is_causal && cur_pos && j > cur_pos[b]) acc = -INFINITY;
+        acc *= scale;
+        s[j] = acc;
+        mx = acc > mx ? acc : mx;
+      }
+      float sum = 0.0f;
+      for (int64_t j = 0; j < S; ++j) { s[j] = expf(s[j] - mx); sum += s[j]; }
+      float *o = out + (b * H + h) * D;
+      for (int64_t d = 0; d < D; ++d) o[d] = 0.0f;
+      for (int64_t j = 0; j < S; ++j) {
+        float p = s[j] / sum;
+        const float *vj = v + ((b * Hkv + hk) * S + j) * D;
+        for (int64_t d = 0; d < D; ++d) o[d] += p * vj[d];
+      }
+    }
+  free(s);
+}

@@ -1,0 +1,177 @@
+"""Decode-path kernels through the C ABI against the CPU oracle: rotary embedding, KV-cache update / fill (bit exact:
+they move or scale bf16 values the oracle reproduces exactly or within one rounding), attention of one token over a cache
+(PCC >= 0.9999, max-abs stated)."""
+import numpy as np
+import pytest
+import torch
+
+from ttmlir_amd import datagen
+from test_gpu_linear import tilize_dev, untilize_dev
+
+pytestmark = pytest.mark.gpu
+
+
+def f32(t):
+    return t.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("B,H,S,D,cache_rows,token", [(1, 8, 64, 128, 64, None), (2, 4, 40, 64, 96, None), (1, 3, 7, 32, 32, None),
+                                                       (1, 32, 32, 128, 2048, 1234), (4, 1, 8, 64, 64, 5)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rotary_embedding(hip, dev, orc, B, H, S, D, cache_rows, token, dtype):
+    x = datagen.randn((B, H, S, D), seed=40, dtype=dtype)
+    ang = datagen.randn((1, 1, cache_rows, D // 2), seed=41, dtype=torch.float32) * 2.0
+    cos = torch.cat([ang.cos(), ang.cos()], -1).to(dtype)
+    sin = torch.cat([ang.sin(), ang.sin()], -1).to(dtype)
+    xt, ct, st = (tilize_dev(hip, t, dev) for t in (x, cos, sin))
+    out = torch.full_like(xt, float("nan"))
+    hip.call("ttm_rotary_embedding", hip.ptr(xt), hip.ptr(ct), hip.ptr(st), hip.ptr(out), hip.BF16 if dtype == torch.bfloat16 else hip.F32,
+             B * H, S, D, cache_rows, -1 if token is None else token, hip.current_stream())
+    got = f32(untilize_dev(hip, out, x.shape, dev))
+    want = orc.rotary_embedding(f32(x), f32(cos), f32(sin), token_index=token)
+    if dtype == torch.float32:
+        # two products and a sum in fp32; the compiler may contract them into fused multiply-adds
+        assert np.max(np.abs(got - want)) <= 1e-6 * max(1.0, np.max(np.abs(want)))
+    else:
+        assert np.max(np.abs(got - orc.round_bf16(want))) <= 2.0 ** -8 * np.maximum(1.0, np.max(np.abs(want)))
+        assert np.mean(got == orc.round_bf16(want)) > 0.99      # differences are single roundings at ties of fused vs separate ops
+    assert bool(torch.isfinite(out.float()).all())              # padding rows are written too (as zeros)
+
+
+def test_rotary_embedding_rejects_bad_shapes(hip, dev):
+    z = torch.zeros(32 * 48, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(hip.TTMError, match="multiple of 32"):
+        hip.call("ttm_rotary_embedding", hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.BF16, 1, 32, 48, 32, -1, hip.current_stream())
+    with pytest.raises(hip.TTMError, match="cached positions"):
+        hip.call("ttm_rotary_embedding", hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.BF16, 1, 32, 32, 32, 32, hip.current_stream())
+    with pytest.raises(hip.TTMError, match="caches hold"):
+        hip.call("ttm_rotary_embedding", hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.BF16, 1, 33, 32, 32, -1, hip.current_stream())
+
+
+@pytest.mark.parametrize("U,H,S,D,Bin,off,idx", [(1, 8, 128, 128, 1, 0, 5), (4, 2, 96, 64, 2, 1, 95), (32, 8, 64, 128, 32, 0, 33),
+                                                  (2, 3, 40, 32, 1, 1, 39)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_update_cache_bit_exact(hip, dev, orc, U, H, S, D, Bin, off, idx, dtype):
+    cache = datagen.randn((U, H, S, D), seed=42, dtype=dtype)
+    upd = datagen.randn((1, H, Bin, D), seed=43, dtype=dtype)
+    ct, ut = tilize_dev(hip, cache, dev), tilize_dev(hip, upd, dev)
+    index = torch.tensor([idx], dtype=torch.int32, device=dev)
+    code = hip.BF16 if dtype == torch.bfloat16 else hip.F32
+    hip.call("ttm_update_cache", hip.ptr(ct), hip.ptr(ut), hip.ptr(index), code, U, H, S, D, Bin, off, hip.current_stream())
+    got = f32(untilize_dev(hip, ct, cache.shape, dev))
+    assert np.array_equal(got, orc.update_cache(f32(cache), f32(upd), idx, off))
+    # an index outside the cache writes nothing
+    before = ct.clone()
+    index.fill_(S)
+    hip.call("ttm_update_cache", hip.ptr(ct), hip.ptr(ut), hip.ptr(index), code, U, H, S, D, Bin, off, hip.current_stream())
+    assert torch.equal(ct, before)
+    with pytest.raises(hip.TTMError, match="outside the cache"):
+        hip.call("ttm_update_cache", hip.ptr(ct), hip.ptr(ut), hip.ptr(index), code, U, H, S, D, Bin, U, hip.current_stream())
+
+
+@pytest.mark.parametrize("U,H,S,D,seq,off", [(1, 8, 128, 128, 128, 0), (4, 2, 96, 64, 40, 3), (2, 3, 64, 32, 1, 1), (2, 1, 64, 64, 33, 0)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fill_cache_bit_exact(hip, dev, orc, U, H, S, D, seq, off, dtype):
+    cache = datagen.randn((U, H, S, D), seed=44, dtype=dtype)
+    fill = datagen.randn((1, H, seq, D), seed=45, dtype=dtype)
+    ct, ft = tilize_dev(hip, cache, dev), tilize_dev(hip, fill, dev)
+    hip.call("ttm_fill_cache", hip.ptr(ct), hip.ptr(ft), hip.BF16 if dtype == torch.bfloat16 else hip.F32, U, H, S, D, seq, off,
+             hip.current_stream())
+    got = f32(untilize_dev(hip, ct, cache.shape, dev))
+    assert np.array_equal(got, orc.fill_cache(f32(cache), f32(fill), off))
+
+
+def _decode_case(hip, dev, orc, B, H, Hkv, S, D, cur, mask_heads=None, causal=True, scale=0.0, paged=None, seed=50):
+    import oracle.metrics as metrics
+    q = datagen.randn((1, B, H, D), seed=seed, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, S, D), seed=seed + 1, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, S, D), seed=seed + 2, dtype=torch.bfloat16)
+    m = datagen.randn((B, 1, mask_heads, S), seed=seed + 3, dtype=torch.bfloat16) if mask_heads else None
+    cp = None if cur is None else torch.tensor(cur, dtype=torch.int32, device=dev)
+    qt = tilize_dev(hip, q, dev)
+    mt = tilize_dev(hip, m, dev) if m is not None else None
+    table, pages, block = None, 0, 0
+    if paged:
+        # scatter the cache into shuffled pages [blocks, Hkv, block, D] behind a page table [B, S / block]
+        block = paged
+        pages = S // block
+        perm = torch.randperm(B * pages, generator=torch.Generator().manual_seed(seed)).reshape(B, pages)
+        kp = torch.zeros((B * pages, Hkv, block, D), dtype=torch.bfloat16)
+        vp = torch.zeros_like(kp)
+        for b in range(B):
+            for j in range(pages):
+                kp[perm[b, j]] = k[b, :, j * block:(j + 1) * block]
+                vp[perm[b, j]] = v[b, :, j * block:(j + 1) * block]
+        kt, vt = tilize_dev(hip, kp, dev), tilize_dev(hip, vp, dev)
+        table = perm.to(torch.int32).to(dev)
+    else:
+        kt, vt = tilize_dev(hip, k, dev), tilize_dev(hip, v, dev)
+    out = torch.full_like(qt, float("nan"))
+    hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp) if cp is not None else None,
+             hip.ptr(mt) if mt is not None else None, mask_heads or 1, hip.ptr(table) if table is not None else None, pages, block,
+             hip.ptr(out), hip.BF16, B, H, Hkv, S, D, int(causal), scale, hip.current_stream())
+    got = f32(untilize_dev(hip, out, q.shape, dev))
+    want = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur, mask=None if m is None else f32(m), is_causal=causal,
+                           scale=scale or None)
+    assert bool(torch.isfinite(out.float()).all())
+    # fp32 scores and probabilities, output rounded to bf16 once: half a bf16 ulp of values up to ~4 plus summation order
+    assert np.max(np.abs(got - want)) <= 2.0 ** -6, np.max(np.abs(got - want))
+    assert metrics.get_pcc(want, got) >= 0.9999
+
+
+@pytest.mark.parametrize("B,H,Hkv,S,D,cur", [
+    (1, 32, 8, 2048, 128, [1500]),            # Llama-3-8B decode, one user
+    (8, 32, 8, 1024, 128, [0, 1, 31, 32, 33, 500, 1022, 1023]),
+    (32, 8, 8, 256, 64, list(range(0, 256, 8))),
+    (2, 8, 1, 512, 32, [100, 511]),           # one kv head serving 8 query heads, single column tile
+    (3, 12, 4, 96, 96, [95, 40, 7]),          # three column tiles
+    (1, 16, 2, 8192, 256, [8000]),            # long cache: several slices per kv head
+])
+def test_sdpa_decode_causal(hip, dev, orc, B, H, Hkv, S, D, cur):
+    _decode_case(hip, dev, orc, B, H, Hkv, S, D, cur)
+
+
+def test_sdpa_decode_mask_scale_and_full_attention(hip, dev, orc):
+    _decode_case(hip, dev, orc, 2, 8, 2, 256, 64, None, causal=False)
+    _decode_case(hip, dev, orc, 2, 8, 2, 256, 64, None, mask_heads=8, scale=0.2)
+    _decode_case(hip, dev, orc, 2, 8, 2, 256, 64, None, mask_heads=1, scale=0.05)
+    _decode_case(hip, dev, orc, 2, 8, 2, 256, 64, [7, 200], causal=False)       # positions are ignored without is_causal
+
+
+@pytest.mark.parametrize("block", [32, 64, 256])
+def test_sdpa_decode_paged(hip, dev, orc, block):
+    _decode_case(hip, dev, orc, 4, 32, 8, 1024, 128, [3, 200, 640, 1023], paged=block)
+
+
+def test_sdpa_decode_ignores_garbage_after_the_current_position(hip, dev, orc):
+    # cache rows that were never written may hold NaN / Inf bit patterns: they must not leak into the output
+    B, H, Hkv, S, D = 2, 8, 2, 512, 128
+    q = datagen.randn((1, B, H, D), seed=60, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, S, D), seed=61, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, S, D), seed=62, dtype=torch.bfloat16)
+    cur = [70, 300]
+    kb, vb = k.clone(), v.clone()
+    for b, c in enumerate(cur):
+        kb[b, :, c + 1:] = float("nan")
+        vb[b, :, c + 1:] = float("inf")
+    cp = torch.tensor(cur, dtype=torch.int32, device=dev)
+    qt, kt, vt = (tilize_dev(hip, t, dev) for t in (q, kb, vb))
+    out = torch.full_like(qt, float("nan"))
+    hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, None, 0, 0, hip.ptr(out), hip.BF16,
+             B, H, Hkv, S, D, 1, 0.0, hip.current_stream())
+    got = f32(untilize_dev(hip, out, q.shape, dev))
+    want = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur)
+    assert np.all(np.isfinite(got)) and np.max(np.abs(got - want)) <= 2.0 ** -6
+
+
+def test_sdpa_decode_rejects_unsupported(hip, dev):
+    z = torch.zeros(1 << 16, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(hip.TTMError, match="query heads per kv head"):
+        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, hip.ptr(z), hip.BF16, 1, 16, 1, 32, 32,
+                 1, 0.0, hip.current_stream())
+    with pytest.raises(hip.TTMError, match="multiple of 32"):
+        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, hip.ptr(z), hip.BF16, 1, 8, 8, 40, 32,
+                 1, 0.0, hip.current_stream())
+    with pytest.raises(hip.TTMError, match="page table"):
+        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, hip.ptr(z), 3, 32, hip.ptr(z), hip.BF16, 1, 8, 8,
+                 64, 32, 1, 0.0, hip.current_stream())

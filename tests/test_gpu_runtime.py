@@ -440,6 +440,79 @@ def test_host_transfer_inside_a_capture_is_refused_cleanly(device):
     assert bool(torch.isfinite(y.float()).all())
 
 
+def _decode_setup(users, hidden, n_q, n_kv, hd, ffn, max_seq, seed):
+    g = torch.Generator().manual_seed(seed)
+    rn = lambda *shape, scale=1.0: torch.randn(shape, generator=g) * scale
+    w = dict(anw=bf(1.0 + 0.02 * rn(hidden)), wq=bf(rn(hidden, n_q * hd, scale=0.05)), wk=bf(rn(hidden, n_kv * hd, scale=0.05)),
+             wv=bf(rn(hidden, n_kv * hd, scale=0.05)), wo=bf(rn(n_q * hd, hidden, scale=0.05)), mnw=bf(1.0 + 0.02 * rn(hidden)),
+             wg=bf(rn(hidden, ffn, scale=0.05)), wu=bf(rn(hidden, ffn, scale=0.05)), wd=bf(rn(ffn, hidden, scale=0.05)))
+    kc, vc = bf(rn(users, n_kv, max_seq, hd)), bf(rn(users, n_kv, max_seq, hd))
+    inv = 1.0 / (10000.0 ** (torch.arange(0, hd // 2).float() / (hd // 2)))
+    ang = torch.arange(max_seq).float()[:, None] * inv[None, :]
+    cos, sin = bf(torch.cat([ang.cos(), ang.cos()], -1)), bf(torch.cat([ang.sin(), ang.sin()], -1))
+    xs = [bf(rn(users, hidden)) for _ in range(4)]
+    return w, kc, vc, cos, sin, xs
+
+
+def oracle_decode_step(orc, x, cos_row, sin_row, pos, kc, vc, w, users, n_q, n_kv, hd):
+    r, f = orc.round_bf16, lambda t: t.float().numpy()
+    q8 = lambda t: orc.bfp_unpack(orc.bfp_pack(f(t), 8), tuple(t.shape), 8)
+    h = r(orc.rms_norm(x, f(w["anw"]), None, 1e-5))
+    q = r(orc.linear(h, q8(w["wq"]))).reshape(1, users, n_q, hd)
+    k = r(orc.linear(h, q8(w["wk"]))).reshape(1, users, n_kv, hd)
+    v = r(orc.linear(h, q8(w["wv"]))).reshape(1, users, n_kv, hd)
+    q = r(orc.rotary_embedding(q, cos_row, sin_row, token_index=0))
+    k = r(orc.rotary_embedding(k, cos_row, sin_row, token_index=0))
+    kc = orc.update_cache(kc, np.ascontiguousarray(k.transpose(0, 2, 1, 3)), pos)
+    vc = orc.update_cache(vc, np.ascontiguousarray(v.transpose(0, 2, 1, 3)), pos)
+    attn = r(orc.sdpa_decode(q, kc, vc, cur_pos=[pos] * users))
+    x1 = r(x + r(orc.linear(attn.reshape(users, n_q * hd), q8(w["wo"]))))
+    mlp = oracle_mlp(orc, x1, f(w["mnw"]), f(w["wg"]), f(w["wu"]), f(w["wd"]), 1e-5)
+    return r(x1 + mlp), kc, vc
+
+
+def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
+    """Three decode steps of a Llama-style layer with KV caches updated in place (rotary embedding, update_cache,
+    scaled_dot_product_attention_decode), op by op and as one traced region replayed from a HIP graph."""
+    users, hidden, n_q, n_kv, hd, ffn, max_seq = 8, 256, 4, 2, 64, 512, 128
+    w, kc0, vc0, cos, sin, xs = _decode_setup(users, hidden, n_q, n_kv, hd, ffn, max_seq, seed=31)
+    f = lambda t: t.float().numpy()
+    order = ["anw", "wq", "wk", "wv", "wo", "mnw", "wg", "wu", "wd"]
+    results = {}
+    for mode in ("eager", "traced"):
+        binary = rt.Binary.load_from_memory(programs.decode_layer(users, hidden, n_q, n_kv, hd, ffn, max_seq, trace=mode == "traced"))
+        main = binary.get_num_programs() - 1
+        lay = lambda k: rt.get_layout(binary, main, k)
+        caches = [rt.to_layout(rt.from_torch(t.clone()), device, lay(5 + i), retain=True) for i, t in enumerate((kc0, vc0))]
+        weights = [rt.to_layout(rt.from_torch(w[n]), device, lay(7 + i), retain=True) for i, n in enumerate(order)]
+        outs = []
+        for step, pos in enumerate((40, 41, 42)):
+            step_in = [xs[step], cos[pos].reshape(1, 1, 1, hd), sin[pos].reshape(1, 1, 1, hd), torch.tensor([pos], dtype=torch.int32),
+                       torch.full((users,), pos, dtype=torch.int32)]
+            ins = [rt.to_layout(rt.from_torch(t.contiguous()), device, lay(i)) for i, t in enumerate(step_in)] + caches + weights
+            (y,) = rt.submit(device, binary, main, ins)
+            outs.append(rt.to_torch(rt.to_host(y, untilize=True)[0]))
+        results[mode] = (outs, [rt.to_torch(rt.to_host(c, untilize=True)[0]) for c in caches])
+        if mode == "traced":
+            assert rt.get_stat("CapturedTrace") >= 1
+    # the replayed graph runs the same kernels on the same data: identical to the op-by-op run, caches included
+    for a, b in zip(results["eager"][0] + results["eager"][1], results["traced"][0] + results["traced"][1]):
+        assert torch.equal(a, b)
+    # against the CPU oracle, step by step
+    kc, vc = f(kc0), f(vc0)
+    for step, pos in enumerate((40, 41, 42)):
+        want, kc, vc = oracle_decode_step(orc, f(xs[step]), f(cos[pos])[None], f(sin[pos])[None], pos, kc, vc, w, users, n_q, n_kv, hd)
+        got = f(results["eager"][0][step])
+        # a chain of eight bf16-rounded ops on values of order 1
+        assert np.max(np.abs(got - want)) <= 2.0 ** -5, (step, np.max(np.abs(got - want)))
+        assert metrics.get_pcc(want, got) >= 0.999
+    gk, gv = (f(t) for t in results["eager"][1])
+    assert np.max(np.abs(gk - kc)) <= 2.0 ** -6 and np.max(np.abs(gv - vc)) <= 2.0 ** -6
+    untouched = np.ones(max_seq, bool)
+    untouched[40:43] = False
+    assert np.array_equal(gk[:, :, untouched], f(kc0)[:, :, untouched]) and np.array_equal(gv[:, :, untouched], f(vc0)[:, :, untouched])
+
+
 def test_submit_errors(device):
     binary = rt.Binary.load_from_memory(programs.c3_linear(32, 64, 64))
     a = rt.from_torch(torch.zeros(32, 64, dtype=torch.bfloat16))

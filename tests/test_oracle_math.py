@@ -135,3 +135,65 @@ def test_pcc_special_cases():
     assert abs(m.get_pcc(x, y) - np.corrcoef(x, y)[0, 1]) < 1e-12
     at, rt = m.get_atol_rtol(np.array([1.0, 2.0]), np.array([1.5, 2.0]))
     assert at == 0.5 and abs(rt - 0.5 / 1.5) < 1e-12
+
+
+# ---- decode path
+def test_rotary_embedding_is_a_plane_rotation(orc):
+    # pair (x[d], x[d + D/2]) with cos = cos(t), sin = sin(t) is the complex product (x1 + i x2) e^{it}
+    B, S, D = 3, 5, 16
+    x = rnd((B, S, D), 30)
+    theta = np.random.default_rng(31).uniform(-3, 3, (S, D // 2)).astype(np.float32)
+    cos = np.concatenate([np.cos(theta), np.cos(theta)], axis=-1)
+    sin = np.concatenate([np.sin(theta), np.sin(theta)], axis=-1)
+    out = orc.rotary_embedding(x, cos, sin)
+    z = (x[..., : D // 2].astype(np.complex128) + 1j * x[..., D // 2:]) * np.exp(1j * theta.astype(np.float64))
+    assert np.allclose(out[..., : D // 2], z.real, atol=1e-5) and np.allclose(out[..., D // 2:], z.imag, atol=1e-5)
+    # special cases: cos = 1, sin = 0 is the identity; cos = 0, sin = 1 is rotate_half itself
+    one, zero = np.ones((S, D), np.float32), np.zeros((S, D), np.float32)
+    assert np.array_equal(orc.rotary_embedding(x, one, zero), x)
+    rh = orc.rotary_embedding(x, zero, one)
+    assert np.array_equal(rh[..., : D // 2], -x[..., D // 2:]) and np.array_equal(rh[..., D // 2:], x[..., : D // 2])
+    # decode mode: every row uses the cache row named by token_index
+    t3 = orc.rotary_embedding(x, cos, sin, token_index=3)
+    assert np.allclose(t3[:, 0], orc.rotary_embedding(x[:, :1], cos[3:4], sin[3:4])[:, 0], atol=0)
+    assert np.allclose(t3[:, 4], orc.rotary_embedding(x[:, 4:5], cos[3:4], sin[3:4])[:, 0], atol=0)
+
+
+def test_cache_update_and_fill_match_slice_assignment(orc):
+    U, H, S, D, Bin = 4, 3, 64, 8, 2
+    cache = rnd((U, H, S, D), 32)
+    upd = rnd((1, H, Bin, D), 33)
+    got = orc.update_cache(cache, upd, 37, batch_offset=1)
+    want = torch.from_numpy(cache.copy())
+    want[1:3, :, 37, :] = torch.from_numpy(upd)[0].permute(1, 0, 2)      # tools/golden/mapping.py:3664-3671
+    assert np.array_equal(got, want.numpy())
+    assert np.array_equal(orc.update_cache(cache, upd[:, :, :1], 0)[0, :, 0], upd[0, :, 0])
+    fill = rnd((1, H, 40, D), 34)
+    got = orc.fill_cache(cache, fill, batch_offset=2)
+    want = cache.copy()
+    want[2, :, :40] = fill[0]
+    want[2, :, 40:64] = 0                                                  # rows up to the tile boundary are cleared
+    assert np.array_equal(got, want)
+    assert np.array_equal(orc.fill_cache(cache, fill[:, :, :32])[0, :, 32:], cache[0, :, 32:])   # aligned: nothing cleared
+
+
+@pytest.mark.parametrize("H,Hkv", [(4, 4), (8, 2)])
+def test_sdpa_decode_against_library_attention(orc, H, Hkv):
+    B, S, D = 3, 48, 16
+    q, k, v = rnd((1, B, H, D), 35), rnd((B, Hkv, S, D), 36), rnd((B, Hkv, S, D), 37)
+    cur = np.array([0, 17, 47], np.int32)
+    got = orc.sdpa_decode(q, k, v, cur_pos=cur)
+    qt = torch.from_numpy(q)[0].unsqueeze(2)                               # [B, H, 1, D]
+    kr = torch.from_numpy(k).repeat_interleave(H // Hkv, dim=1)
+    vr = torch.from_numpy(v).repeat_interleave(H // Hkv, dim=1)
+    keep = (torch.arange(S)[None, :] <= torch.from_numpy(cur).long()[:, None])[:, None, None, :]
+    want = F.scaled_dot_product_attention(qt, kr, vr, attn_mask=keep).squeeze(2).unsqueeze(0)
+    assert np.allclose(got, want.numpy(), rtol=1e-4, atol=1e-5)
+    # the prefill oracle with one query row per head agrees when nothing is masked
+    full = orc.sdpa(np.ascontiguousarray(qt.numpy()), k, v)
+    assert np.allclose(orc.sdpa_decode(q, k, v, is_causal=False)[0], full[:, :, 0], rtol=1e-5, atol=1e-6)
+    # additive mask enters before the scale: (q k + m) * s
+    m = rnd((B, 1, H, S), 38)
+    got = orc.sdpa_decode(q, k, v, mask=m, scale=0.25)
+    want = F.scaled_dot_product_attention(qt, kr, vr, attn_mask=torch.from_numpy(m).permute(0, 2, 1, 3) * 0.25, scale=0.25)
+    assert np.allclose(got[0], want.squeeze(2).numpy(), rtol=1e-4, atol=1e-5)

@@ -38,7 +38,7 @@ int ttm_option(const char *name);  // 0 when unset
 // have recorded is never freed before the stream is destroyed.
 int ttm_stream_workspace(hipStream_t stream, size_t bytes, void **ptr);
 
-static inline int64_t ttm_round_up32(int64_t v) { return (v + 31) / 32 * 32; }
+__host__ __device__ static inline int64_t ttm_round_up32(int64_t v) { return (v + 31) / 32 * 32; }
 static inline int64_t ttm_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 static inline int ttm_dtype_bytes(int dtype) {

@@ -1,0 +1,452 @@
+// Decode-path transformer kernels: rotary embedding, KV-cache update / fill, single-token attention over a KV cache.
+// All tensors are TILE layout (32 x 32 tiles of four 16 x 16 faces); every kernel here is bound by HBM bandwidth.
+#include "ttm_common.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4v __attribute__((ext_vector_type(4)));
+
+// 8 consecutive elements <-> 8 floats
+__device__ __forceinline__ void load8(const uint16_t *p, float *v) {
+  const u32x4 r = *(const u32x4 *)p;
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    v[2 * j] = __uint_as_float(w[j] << 16);
+    v[2 * j + 1] = __uint_as_float(w[j] & 0xFFFF0000u);
+  }
+}
+__device__ __forceinline__ void load8(const float *p, float *v) {
+  const f32x4 a = *(const f32x4 *)p, b = *(const f32x4 *)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void store8(uint16_t *p, const float *v) {
+  u32x4 r;
+  r.x = ttm_f32_to_bf16(v[0]) | ((uint32_t)ttm_f32_to_bf16(v[1]) << 16);
+  r.y = ttm_f32_to_bf16(v[2]) | ((uint32_t)ttm_f32_to_bf16(v[3]) << 16);
+  r.z = ttm_f32_to_bf16(v[4]) | ((uint32_t)ttm_f32_to_bf16(v[5]) << 16);
+  r.w = ttm_f32_to_bf16(v[6]) | ((uint32_t)ttm_f32_to_bf16(v[7]) << 16);
+  *(u32x4 *)p = r;
+}
+__device__ __forceinline__ void store8(float *p, const float *v) {
+  *(f32x4 *)p = f32x4{v[0], v[1], v[2], v[3]};
+  *(f32x4 *)(p + 4) = f32x4{v[4], v[5], v[6], v[7]};
+}
+
+// ------------------------------------------------------------------------------------------------ rotary embedding
+// out[b, s, d] = x[b, s, d] * cos[r, d] + rot(x)[b, s, d] * sin[r, d],  rot(x)[d] = d < D/2 ? -x[d + D/2] : x[d - D/2],
+// r = token_index when given, else s.  One thread per 8 consecutive columns of a face row: the partner columns
+// d +- D/2 are 8 consecutive elements of another face row because D/2 is a multiple of 16.
+template <typename T>
+__global__ __launch_bounds__(256) void ttm_rotary_k(const T *__restrict__ x, const T *__restrict__ cosc,
+                                                    const T *__restrict__ sinc, T *__restrict__ out, int64_t rows_pad,
+                                                    int64_t cols, int64_t per_batch, int64_t total8, int64_t token_index) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const int64_t ct = cols >> 5, half = cols >> 1;
+  const int64_t e = i * 8, b = e / per_batch, o = e % per_batch;
+  // o -> (row, col) of the tiled [rows_pad, cols] matrix
+  const int64_t tile = o >> 10;
+  const int in = (int)(o & 1023), face = in >> 8, fr = (in >> 4) & 15, fc = in & 15;
+  const int64_t r = (tile / ct) * 32 + (face >> 1) * 16 + fr, c = (tile % ct) * 32 + (face & 1) * 16 + fc;
+  const int64_t cr = token_index >= 0 ? token_index : r;
+  const int64_t pc = c < half ? c + half : c - half;
+  const float sign = c < half ? -1.0f : 1.0f;
+  const T *xp = x + b * per_batch;
+  const int64_t co = ttm_tiled_offset(cr, c, ct);
+  float xv[8], pv[8], cv[8], sv[8], ov[8];
+  load8(xp + o, xv);
+  load8(xp + ttm_tiled_offset(r, pc, ct), pv);
+  load8(cosc + co, cv);
+  load8(sinc + co, sv);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) ov[j] = xv[j] * cv[j] + sign * pv[j] * sv[j];
+  store8(out + b * per_batch + o, ov);
+}
+
+// ------------------------------------------------------------------------------------------------ cache update / fill
+// cache[batch_offset + b, h, *index, :] = input[0, h, b, :]; one thread per 8 elements (never straddles a face row)
+template <typename T>
+__global__ __launch_bounds__(256) void ttm_update_cache_k(T *__restrict__ cache, const T *__restrict__ input,
+                                                          const int32_t *__restrict__ index, int64_t heads, int64_t seq_pad,
+                                                          int64_t max_seq, int64_t dim, int64_t in_users, int64_t in_users_pad,
+                                                          int64_t batch_offset, int64_t total8) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const int64_t pos = index[0];
+  if (pos < 0 || pos >= max_seq) return;          // out of range positions write nothing
+  const int64_t d8 = dim >> 3;
+  const int64_t c = (i % d8) * 8, b = (i / d8) % in_users, h = i / (d8 * in_users);
+  const int64_t ct = dim >> 5;
+  const T *src = input + h * in_users_pad * dim + ttm_tiled_offset(b, c, ct);
+  T *dst = cache + ((batch_offset + b) * heads + h) * seq_pad * dim + ttm_tiled_offset(pos, c, ct);
+  *(u32x4 *)dst = *(const u32x4 *)src;
+  if (sizeof(T) == 4) *(u32x4 *)(dst + 4) = *(const u32x4 *)(src + 4);
+}
+
+// cache[batch_offset, h, 0:seq_tiles*32, :] = input[0, h, :, :] tile by tile (the padding rows of the last tile come along)
+__global__ __launch_bounds__(256) void ttm_fill_cache_k(u32x4 *__restrict__ cache, const u32x4 *__restrict__ input,
+                                                        int64_t head_stride_cache16, int64_t head_stride_in16, int64_t base16,
+                                                        int64_t total16) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total16) return;
+  const int64_t h = i / head_stride_in16, o = i % head_stride_in16;
+  cache[base16 + h * head_stride_cache16 + o] = input[i];
+}
+
+// ------------------------------------------------------------------------------------------------ attention, one query token
+// q [1, B, H, D], k / v [B, Hkv, S, D] (or pages [blocks, Hkv, block, D] behind a page table), out [1, B, H, D], bf16 tiles.
+// grid (splits, B * Hkv), 256 threads.  A block owns the G = H / Hkv query heads of one kv head and one slice of the keys:
+//   1. scores = Q K^T with v_mfma_f32_16x16x32_bf16 (queries are the 16 rows, padded with zeros), written to LDS
+//      as (score + mask) * scale, -inf outside the valid keys;
+//   2. softmax numerators and their sum per query head, in place in LDS;
+//   3. P V on the vector ALU: a wave reads half tiles of V (16 keys x 32 columns, 1 KiB contiguous), every lane keeps
+//      8 columns x G heads of partial sums, lanes are combined once per column tile;
+//   4. (max, sum, unnormalised output) go to the split's slot of the workspace; ttm_sdpa_decode_combine_k merges the slots.
+struct DecodeArgs {
+  const uint16_t *q, *k, *v, *mask;
+  const int32_t *cur_pos, *page_table;
+  float *part;        // [B * Hkv][splits][G][D + 2]
+  uint16_t *out;
+  int B, H, Hkv, G, S, D, splits, keys_per_split, block, pages_per_user, mask_heads, is_causal;
+  float scale;
+};
+
+constexpr int kMaxG = 8;
+
+__device__ __forceinline__ const uint16_t *kv_tile_row(const uint16_t *base, const DecodeArgs &p, int b, int hk, int key_tile) {
+  // start of the row of tiles holding keys [32 key_tile, 32 key_tile + 32) of (b, hk)
+  const int64_t row_elems = (int64_t)32 * p.D;
+  if (p.page_table) {
+    const int tiles_per_block = p.block >> 5;
+    const int page = p.page_table[(int64_t)b * p.pages_per_user + key_tile / tiles_per_block];
+    return base + (((int64_t)page * p.Hkv + hk) * tiles_per_block + key_tile % tiles_per_block) * row_elems;
+  }
+  return base + (((int64_t)b * p.Hkv + hk) * (p.S >> 5) + key_tile) * row_elems;
+}
+
+__global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
+  extern __shared__ float lds[];
+  const int split = blockIdx.x, bh = blockIdx.y, b = bh / p.Hkv, hk = bh % p.Hkv;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int G = p.G, D = p.D, DT = D >> 5;
+  const int k0 = split * p.keys_per_split;
+  int valid = p.S;
+  if (p.is_causal && p.cur_pos) {
+    int cp = p.cur_pos[b] + 1;
+    valid = cp < valid ? (cp < 0 ? 0 : cp) : valid;
+  }
+  int k1 = k0 + p.keys_per_split;
+  k1 = k1 < valid ? k1 : valid;
+  const int nkeys = k1 > k0 ? k1 - k0 : 0;
+  const int ngroups = (nkeys + 15) >> 4;
+  float *sc = lds;                                        // [G][keys_per_split]
+  float *osum = lds + (size_t)G * p.keys_per_split;       // [G][D]
+  float *stat = osum + (size_t)G * D;                     // [G][2]: max, sum
+  float *slot = p.part + ((size_t)bh * p.splits + split) * G * (D + 2);
+
+  for (int i = tid; i < G * D; i += 256) osum[i] = 0.0f;
+  if (nkeys == 0) {
+    for (int i = tid; i < G * (D + 2); i += 256) {
+      const int c = i % (D + 2);
+      slot[i] = c == D ? -INFINITY : 0.0f;
+    }
+    return;
+  }
+
+  // ---- 1. scores
+  {
+    // query fragments: lane supplies query row lane % 16, columns 32 c + 8 (lane / 16) .. + 7
+    const int g = lane & 15, dq = (lane >> 4) * 8;
+    bf16x8 qf[8];
+    const int h = hk * G + g;
+    const uint16_t *qb = p.q + (int64_t)b * ttm_round_up32(p.H) * D;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+      u32x4 z = {0, 0, 0, 0};
+      if (c < DT && g < G) z = *(const u32x4 *)(qb + ttm_tiled_offset(h, 32 * c + dq, DT));
+      qf[c] = *(bf16x8 *)&z;
+    }
+    const int hrow = hk * G;  // mask rows of this block's heads
+    for (int g0 = wave; g0 < ngroups; g0 += 8) {
+      // two groups of 16 keys per pass, all their loads issued before the first product
+      u32x4 kf[2][8];
+      int grp[2];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        grp[u] = g0 + 4 * u < ngroups ? g0 + 4 * u : g0;   // the tail repeats a valid group and skips its result
+        const int key = k0 + grp[u] * 16 + (lane & 15);     // this lane's key column of the B operand
+        const uint16_t *kt = kv_tile_row(p.k, p, b, hk, key >> 5);
+        // inside a tile: face (key half, column half), row key % 16, columns dq % 16 .. + 7
+        const int in_tile = (((key >> 4) & 1) * 2 + (dq >> 4)) * 256 + (key & 15) * 16 + (dq & 15);
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+          if (c < DT) kf[u][c] = *(const u32x4 *)(kt + (int64_t)c * 1024 + in_tile);
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        if (u == 1 && g0 + 4 >= ngroups) break;
+        f32x4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < 8; ++c)
+          if (c < DT) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[c], *(bf16x8 *)&kf[u][c], acc, 0, 0, 0);
+        // acc[i] = score of query 4 (lane / 16) + i against key lane % 16 of the group
+        const int kk = grp[u] * 16 + (lane & 15);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int gq = (lane >> 4) * 4 + i;
+          if (gq < G) {
+            float sv = acc[i];
+            if (p.mask) {
+              const int mh = p.mask_heads == 1 ? 0 : hrow + gq;
+              const int64_t mrows = ttm_round_up32(p.mask_heads);
+              sv += ttm_bf16_to_f32(p.mask[(int64_t)b * mrows * p.S + ttm_tiled_offset(mh, k0 + kk, p.S >> 5)]);
+            }
+            sc[gq * p.keys_per_split + kk] = (k0 + kk < k1) ? sv * p.scale : -INFINITY;
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- 2. softmax numerators: wave w serves heads w, w + 4, ...
+  const int padded = ngroups * 16;
+  for (int g = wave; g < G; g += 4) {
+    float *row = sc + g * p.keys_per_split;
+    float m = -INFINITY;
+    for (int i = lane; i < padded; i += 64) m = fmaxf(m, row[i]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+    float l = 0.0f;
+    for (int i = lane; i < padded; i += 64) {
+      const float e = (m == -INFINITY) ? 0.0f : __expf(row[i] - m);
+      row[i] = e;
+      l += e;
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
+    if (lane == 0) { stat[2 * g] = m; stat[2 * g + 1] = l; }
+  }
+  __syncthreads();
+
+  // ---- 3. P V: work items are (column tile, key-group stride class); lane covers key (lane % 32) / 2 of a 16-key group
+  // and columns 16 (lane / 32) + 8 (lane % 2) .. + 7 of the 32-column tile
+  {
+    const int share = DT == 1 ? 4 : (DT == 2 ? 2 : 1);   // with one or two column tiles several waves split the keys of one
+    const int items = DT * share;
+    const int krow = (lane & 31) >> 1;
+    for (int item = wave; item < items; item += 4) {
+      const int dt = item % DT, kfirst = item / DT;
+      float o[kMaxG][8];
+#pragma unroll
+      for (int g = 0; g < kMaxG; ++g)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[g][j] = 0.0f;
+      for (int g0 = kfirst; g0 < ngroups; g0 += 4 * share) {
+        // four half tiles of V in flight
+        u32x4 raw[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int grp = g0 + u * share < ngroups ? g0 + u * share : g0;
+          const int key = k0 + grp * 16;               // first key of the group; a group never straddles a tile half
+          const uint16_t *vt = kv_tile_row(p.v, p, b, hk, key >> 5) + (int64_t)dt * 1024 + ((key >> 4) & 1) * 512;
+          raw[u] = *(const u32x4 *)(vt + lane * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int grp = g0 + u * share;
+          const int kk = grp * 16 + krow;
+          const bool live = grp < ngroups && kk < nkeys;   // rows past the valid keys may hold anything, NaN included
+          const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
+          float vv[8];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            vv[2 * j] = live ? __uint_as_float(w[j] << 16) : 0.0f;
+            vv[2 * j + 1] = live ? __uint_as_float(w[j] & 0xFFFF0000u) : 0.0f;
+          }
+#pragma unroll
+          for (int g = 0; g < kMaxG; ++g) {
+            if (g < G) {
+              const float pg = live ? sc[g * p.keys_per_split + kk] : 0.0f;
+#pragma unroll
+              for (int j = 0; j < 8; ++j) o[g][j] += pg * vv[j];
+            }
+          }
+        }
+      }
+      // combine the 16 lanes that hold the same columns (they differ in bits 1..4 of the lane id)
+#pragma unroll
+      for (int g = 0; g < kMaxG; ++g) {
+        if (g < G) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            float v = o[g][j];
+            v += __shfl_xor(v, 2);
+            v += __shfl_xor(v, 4);
+            v += __shfl_xor(v, 8);
+            v += __shfl_xor(v, 16);
+            o[g][j] = v;
+          }
+        }
+      }
+      if (((lane >> 1) & 15) == 0) {
+        const int col = dt * 32 + (lane >> 5) * 16 + (lane & 1) * 8;
+#pragma unroll
+        for (int g = 0; g < kMaxG; ++g)
+          if (g < G)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+              if (share == 1) osum[g * D + col + j] = o[g][j];
+              else atomicAdd(&osum[g * D + col + j], o[g][j]);
+            }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- 4. the split's slot
+  for (int i = tid; i < G * (D + 2); i += 256) {
+    const int g = i / (D + 2), c = i % (D + 2);
+    slot[i] = c < D ? osum[g * D + c] : stat[2 * g + (c - D)];
+  }
+}
+
+// merges the slots of one (b, kv head): out = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M)
+__global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
+  const int bh = blockIdx.x, b = bh / p.Hkv, hk = bh % p.Hkv;
+  const int G = p.G, D = p.D;
+  const float *base = p.part + (size_t)bh * p.splits * G * (D + 2);
+  for (int i = threadIdx.x; i < G * D; i += 256) {
+    const int g = i / D, c = i % D;
+    float M = -INFINITY;
+    for (int s = 0; s < p.splits; ++s) M = fmaxf(M, base[((size_t)s * G + g) * (D + 2) + D]);
+    float num = 0.0f, den = 0.0f;
+    for (int s = 0; s < p.splits; ++s) {
+      const float *sl = base + ((size_t)s * G + g) * (D + 2);
+      const float w = (sl[D] == -INFINITY) ? 0.0f : __expf(sl[D] - M);
+      num += sl[c] * w;
+      den += sl[D + 1] * w;
+    }
+    const int h = hk * G + g;
+    p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(h, c, D >> 5)] = ttm_f32_to_bf16(den > 0.0f ? num / den : 0.0f);
+  }
+  if (hk == p.Hkv - 1) {   // padding rows of the last head tile
+    const int pad = (int)ttm_round_up32(p.H) - p.H;
+    for (int i = threadIdx.x; i < pad * D; i += 256)
+      p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(p.H + i / D, i % D, D >> 5)] = 0;
+  }
+}
+
+}  // namespace
+
+TTM_EXPORT int ttm_rotary_embedding(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype,
+                                    int64_t batch, int64_t rows, int64_t cols, int64_t cache_rows, int64_t token_index,
+                                    void *stream) {
+  TTM_REQUIRE(x && cos_cache && sin_cache && out, "ttm_rotary_embedding: null pointer");
+  TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_rotary_embedding: dtype must be BFloat16 or Float32");
+  TTM_REQUIRE(batch >= 0 && rows > 0 && cols > 0 && cols % 32 == 0, "ttm_rotary_embedding: head dim must be a positive multiple of 32");
+  if (token_index >= 0)
+    TTM_REQUIRE(token_index < cache_rows, "ttm_rotary_embedding: token_index %lld outside the %lld cached positions",
+                (long long)token_index, (long long)cache_rows);
+  else
+    TTM_REQUIRE(cache_rows >= rows, "ttm_rotary_embedding: cos / sin caches hold %lld positions, input has %lld",
+                (long long)cache_rows, (long long)rows);
+  if (batch == 0) return TTM_OK;
+  const int64_t rows_pad = ttm_round_up32(rows), per_batch = rows_pad * cols, total8 = batch * per_batch / 8;
+  const dim3 grid((unsigned)ttm_cdiv(total8, 256));
+  if (dtype == TTM_BF16)
+    hipLaunchKernelGGL(ttm_rotary_k<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x,
+                       (const uint16_t *)cos_cache, (const uint16_t *)sin_cache, (uint16_t *)out, rows_pad, cols, per_batch,
+                       total8, token_index);
+  else
+    hipLaunchKernelGGL(ttm_rotary_k<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float *)x, (const float *)cos_cache,
+                       (const float *)sin_cache, (float *)out, rows_pad, cols, per_batch, total8, token_index);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+TTM_EXPORT int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users,
+                                int64_t heads, int64_t max_seq, int64_t head_dim, int64_t input_users, int64_t batch_offset,
+                                void *stream) {
+  TTM_REQUIRE(cache && input && update_index, "ttm_update_cache: null pointer");
+  TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_update_cache: dtype must be BFloat16 or Float32");
+  TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_update_cache: head dim must be a positive multiple of 32");
+  TTM_REQUIRE(batch_offset >= 0 && input_users >= 0 && batch_offset + input_users <= users,
+              "ttm_update_cache: users [%lld, %lld) outside the cache's %lld", (long long)batch_offset,
+              (long long)(batch_offset + input_users), (long long)users);
+  const int64_t total8 = heads * input_users * (head_dim / 8);
+  if (total8 == 0) return TTM_OK;
+  const dim3 grid((unsigned)ttm_cdiv(total8, 256));
+  const int64_t seq_pad = ttm_round_up32(max_seq), in_pad = ttm_round_up32(input_users);
+  if (dtype == TTM_BF16)
+    hipLaunchKernelGGL(ttm_update_cache_k<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, (uint16_t *)cache,
+                       (const uint16_t *)input, update_index, heads, seq_pad, max_seq, head_dim, input_users, in_pad, batch_offset,
+                       total8);
+  else
+    hipLaunchKernelGGL(ttm_update_cache_k<float>, grid, dim3(256), 0, (hipStream_t)stream, (float *)cache, (const float *)input,
+                       update_index, heads, seq_pad, max_seq, head_dim, input_users, in_pad, batch_offset, total8);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+TTM_EXPORT int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t users, int64_t heads, int64_t max_seq,
+                              int64_t head_dim, int64_t seq, int64_t batch_offset, void *stream) {
+  TTM_REQUIRE(cache && input, "ttm_fill_cache: null pointer");
+  const int eb = ttm_dtype_bytes(dtype);
+  TTM_REQUIRE(eb == 2 || eb == 4, "ttm_fill_cache: element size must be 2 or 4 bytes");
+  TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_fill_cache: head dim must be a positive multiple of 32");
+  TTM_REQUIRE(batch_offset >= 0 && batch_offset < users, "ttm_fill_cache: batch offset %lld outside the cache's %lld users",
+              (long long)batch_offset, (long long)users);
+  TTM_REQUIRE(seq >= 0 && seq <= max_seq, "ttm_fill_cache: %lld positions do not fit a cache of %lld", (long long)seq, (long long)max_seq);
+  const int64_t in16 = ttm_round_up32(seq) * head_dim * eb / 16, cache16 = ttm_round_up32(max_seq) * head_dim * eb / 16;
+  const int64_t total16 = heads * in16;
+  if (total16 == 0) return TTM_OK;
+  hipLaunchKernelGGL(ttm_fill_cache_k, dim3((unsigned)ttm_cdiv(total16, 256)), dim3(256), 0, (hipStream_t)stream, (u32x4 *)cache,
+                     (const u32x4 *)input, cache16, in16, batch_offset * heads * cache16, total16);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
+                               int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out,
+                               int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
+                               int is_causal, float scale, void *stream) {
+  TTM_REQUIRE(q && k && v && out, "ttm_sdpa_decode: null pointer");
+  TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa_decode: tensors must be BFloat16");
+  TTM_REQUIRE(batch > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "ttm_sdpa_decode: heads must be a multiple of kv heads");
+  const int64_t G = heads / kv_heads;
+  TTM_REQUIRE(G <= kMaxG, "ttm_sdpa_decode: at most %d query heads per kv head (got %lld)", kMaxG, (long long)G);
+  TTM_REQUIRE(head_dim % 32 == 0 && head_dim >= 32 && head_dim <= 256, "ttm_sdpa_decode: head dim must be a multiple of 32 up to 256");
+  TTM_REQUIRE(seq > 0 && seq % 32 == 0, "ttm_sdpa_decode: cache length must be a positive multiple of 32");
+  TTM_REQUIRE(!mask || mask_heads == 1 || mask_heads == heads, "ttm_sdpa_decode: mask must have 1 or %lld head rows", (long long)heads);
+  if (page_table)
+    TTM_REQUIRE(page_block > 0 && page_block % 32 == 0 && pages_per_user * page_block == seq,
+                "ttm_sdpa_decode: page table of %lld blocks x %lld positions does not cover %lld positions",
+                (long long)pages_per_user, (long long)page_block, (long long)seq);
+  hipStream_t s = (hipStream_t)stream;
+  // enough blocks to fill the device, slices small enough for the score rows to fit in LDS
+  int64_t splits = ttm_cdiv(512, batch * kv_heads);
+  const int64_t max_keys = (48 * 1024 / 4) / G / 32 * 32;
+  if (splits > seq / 256) splits = seq / 256 > 0 ? seq / 256 : 1;
+  if (ttm_cdiv(seq, splits) > max_keys) splits = ttm_cdiv(seq, max_keys);
+  const int64_t keys = ttm_round_up32(ttm_cdiv(seq, splits));
+  splits = ttm_cdiv(seq, keys);
+  DecodeArgs p;
+  p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.v = (const uint16_t *)v; p.mask = (const uint16_t *)mask;
+  p.cur_pos = cur_pos; p.page_table = page_table; p.out = (uint16_t *)out;
+  p.B = (int)batch; p.H = (int)heads; p.Hkv = (int)kv_heads; p.G = (int)G; p.S = (int)seq; p.D = (int)head_dim;
+  p.splits = (int)splits; p.keys_per_split = (int)keys; p.block = (int)page_block; p.pages_per_user = (int)pages_per_user;
+  p.mask_heads = mask_heads; p.is_causal = is_causal;
+  p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)head_dim);
+  void *ws = nullptr;
+  if (int rc = ttm_stream_workspace(s, (size_t)(batch * kv_heads * splits * G * (head_dim + 2)) * sizeof(float), &ws)) return rc;
+  p.part = (float *)ws;
+  const size_t lds = (size_t)(G * keys + G * head_dim + 2 * G) * sizeof(float);
+  hipLaunchKernelGGL(ttm_sdpa_decode_k, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
+  TTM_LAUNCH_CHECK();
+  hipLaunchKernelGGL(ttm_sdpa_decode_combine_k, dim3((unsigned)(batch * kv_heads)), dim3(256), 0, s, p);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}

@@ -149,8 +149,9 @@ def add_traced(pb, name, args, body, out_descs):
     (test/ttmlir/Dialect/TTNN/trace/scenarios/single_add_no_consteval.mlir:5-45) and returns a function that emits the
     `capture_or_execute_trace` op into the program that is open when it is called.
 
-    args: [(shape, dtype, resident)] - resident arguments live on the device (parameters, const-eval results, caches) and
-    are their own slots; the others arrive on the host, row-major, and are staged into device slots.
+    args: [(shape, dtype, resident[, layout])] - resident arguments live on the device (parameters, const-eval results,
+    caches) and are their own slots; the others arrive on the host, row-major, and are staged into device slots.  The
+    device layout is TILE unless given (positions and page tables stay row-major).
     body(pb, ids) -> [result ids] builds the traced computation on Device / Tile tensors.
     out_descs: [(shape, Layout)] of the results.
 
@@ -160,29 +161,29 @@ def add_traced(pb, name, args, body, out_descs):
                                                        write_tensor, one eager run, capture of a second run, one replay
       execute_trace_0_<name>(trace id)                 ttnn.execute_trace
     """
-    dev_lay = lambda dt: rt.Layout(ST.Device, TL.Tile, dt)
+    args = [(a[0], a[1], a[2], a[3] if len(a) > 3 else TL.Tile) for a in args]
     # the traced function
     pb.begin_program("trace_0_" + name, private=True)
-    ids = [pb.input(shape, dt) for shape, dt, _ in args]
+    ids = [pb.input(shape, dt, lay) for shape, dt, _, lay in args]
     slots = [pb.input(shape, lay.dtype, lay.layout, lay.storage) for shape, lay in out_descs]
     for res, slot in zip(body(pb, ids), slots):
         pb.copy(res, slot)
     trace_fn = pb.end_program()
     # slot allocation
     pb.begin_program("allocate_slots_trace_0_" + name, private=True)
-    resident = iter([pb.input(shape, dt) for shape, dt, res in args if res])
-    for shape, dt, res in args:
-        pb.output(next(resident) if res else pb.empty(shape, dt))
+    resident = iter([pb.input(shape, dt, lay) for shape, dt, res, lay in args if res])
+    for shape, dt, res, lay in args:
+        pb.output(next(resident) if res else pb.empty(shape, dt, lay))
     for shape, lay in out_descs:
         pb.output(pb.empty(shape, lay.dtype, lay.layout))
     allocate = pb.end_program()
     # capture
     pb.begin_program("run_and_capture_trace_0_" + name, private=True)
-    staged = [pb.input(shape, dt, TL.RowMajor, ST.Host) for shape, dt, res in args if not res]
-    in_slots = [pb.input(shape, dt) for shape, dt, _ in args]
+    staged = [pb.input(shape, dt, TL.RowMajor, ST.Host) for shape, dt, res, _ in args if not res]
+    in_slots = [pb.input(shape, dt, lay) for shape, dt, _, lay in args]
     out_slots = [pb.input(shape, lay.dtype, lay.layout, lay.storage) for shape, lay in out_descs]
     host = iter(staged)
-    for (shape, dt, res), slot in zip(args, in_slots):
+    for (shape, dt, res, _), slot in zip(args, in_slots):
         if not res:
             pb.write_tensor(next(host), slot)
     pb.func_call(trace_fn, in_slots + out_slots, [])
@@ -227,5 +228,70 @@ def traced_mlp(tokens=32, hidden=4096, ffn=14336, eps=1e-5, trace=True):
     else:
         y = _mlp(pb, pb.to_layout(pb.to_device(x), TL.Tile), nw, qg, qu, qd, eps)
     pb.output(y)
+    pb.end_program()
+    return pb.finish()
+
+
+def _decode_body(pb, a, users, hidden, n_q, n_kv, head_dim, eps):
+    """One decode step of a Llama-style layer for `users` sequences that share a position (op mix of
+    test/ttmlir/models/single_blocks_and_layers/llama_3_8b_decode_layer.mlir after RoPE / cache / attention fusing):
+    a = [x, cos, sin, update_index, cur_pos, k_cache, v_cache, attn_norm_w, wq, wk, wv, wo, mlp_norm_w, wg, wu, wd]."""
+    x, cos, sin, upd, cur, kc, vc, anw, wq, wk, wv, wo, mnw, wg, wu, wd = a
+    h = pb.rms_norm(x, anw, 0, eps)
+    q = pb.reshape(pb.matmul(h, wq), (1, users, n_q, head_dim))
+    k = pb.reshape(pb.matmul(h, wk), (1, users, n_kv, head_dim))
+    v = pb.reshape(pb.matmul(h, wv), (1, users, n_kv, head_dim))
+    # decode-mode RoPE: cos / sin hold the row of the current position, token_index = 0
+    # (lib/Dialect/TTNN/Transforms/Fusing/RoPEFusingPattern.cpp:1143-1149)
+    q = pb.rotary_embedding(q, cos, sin, token_index=0)
+    k = pb.rotary_embedding(k, cos, sin, token_index=0)
+    pb.update_cache(kc, pb.permute(k, (0, 2, 1, 3)), upd)
+    pb.update_cache(vc, pb.permute(v, (0, 2, 1, 3)), upd)
+    attn = pb.sdpa_decode(q, kc, vc, cur_pos=cur, is_causal=True)
+    merged = pb.reshape(attn, (users, n_q * head_dim))
+    x1 = pb.binary(BINARY["add"], x, pb.matmul(merged, wo))
+    d = _mlp(pb, x1, mnw, wg, wu, wd, eps)
+    return pb.binary(BINARY["add"], x1, d)
+
+
+def decode_layer(users=32, hidden=4096, n_q=32, n_kv=8, head_dim=128, ffn=14336, max_seq=2048, eps=1e-5, trace=False):
+    """Decoder layer, one new token per user, KV caches updated in place.  Inputs: x [users, hidden], cos / sin
+    [1, 1, 1, head_dim] of the current position, update_index [1] and cur_pos [users] (Int32), k / v caches
+    [users, n_kv, max_seq, head_dim], then the weights in bf16 (packed to block-float by const-eval).  With trace=True
+    the step is one traced region: activations, rotary rows and positions are staged from the host, caches and weights
+    are device resident."""
+    pb = rt.ProgramBuilder()
+    dq, dkv = n_q * head_dim, n_kv * head_dim
+    name = "decode_layer"
+    ce, ce_outs = _consteval_pack(pb, name + "_const_eval_0", [
+        ((hidden, dq), DT.BFP_BFloat8), ((hidden, dkv), DT.BFP_BFloat8), ((hidden, dkv), DT.BFP_BFloat8),
+        ((dq, hidden), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8),
+        ((ffn, hidden), DT.BFP_BFloat4)])
+    cache_shape = (users, n_kv, max_seq, head_dim)
+    step = [((users, hidden), DT.BFloat16, False), ((1, 1, 1, head_dim), DT.BFloat16, False), ((1, 1, 1, head_dim), DT.BFloat16, False),
+            ((1,), DT.Int32, False, TL.RowMajor), ((users,), DT.Int32, False, TL.RowMajor),
+            (cache_shape, DT.BFloat16, True), (cache_shape, DT.BFloat16, True)]
+    wshapes = [(hidden,), (hidden, dq), (hidden, dkv), (hidden, dkv), (dq, hidden), (hidden,), (hidden, ffn), (hidden, ffn), (ffn, hidden)]
+    wdtypes = [DT.BFloat16, DT.BFP_BFloat8, DT.BFP_BFloat8, DT.BFP_BFloat8, DT.BFP_BFloat8, DT.BFloat16, DT.BFP_BFloat8, DT.BFP_BFloat8,
+               DT.BFP_BFloat4]
+    out_desc = ((users, hidden), rt.Layout(ST.Device, TL.Tile, DT.BFloat16))
+    body = lambda pb, a: [_decode_body(pb, a, users, hidden, n_q, n_kv, head_dim, eps)]
+    emit = None
+    if trace:
+        emit = add_traced(pb, name, step + [(s, d, True) for s, d in zip(wshapes, wdtypes)], body, [out_desc])
+    pb.begin_program(name)
+    ins = []
+    for a in step:
+        shape, dt, resident = a[0], a[1], a[2]
+        lay = a[3] if len(a) > 3 else TL.Tile
+        if trace and not resident:
+            ins.append(pb.input(shape, dt, TL.RowMajor, ST.Host))
+        else:
+            ins.append(pb.input(shape, dt, lay))
+    raw = [pb.input(s, DT.BFloat16) for s in wshapes]
+    packed = pb.load_cached(ce, name + "_const_eval_0", [raw[1], raw[2], raw[3], raw[4], raw[6], raw[7], raw[8]], ce_outs)
+    weights = [raw[0], packed[0], packed[1], packed[2], packed[3], raw[5], packed[4], packed[5], packed[6]]
+    out = emit(pb, ins + weights)[0] if trace else body(pb, ins + weights)[0]
+    pb.output(out)
     pb.end_program()
     return pb.finish()

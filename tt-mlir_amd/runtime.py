@@ -555,6 +555,19 @@ class ProgramBuilder:
     def sdpa(self, q, k, v, mask=0, is_causal=False, scale=None):
         return self._op("ttrt_pb_sdpa", q, k, v, mask, int(is_causal), int(scale is not None), ctypes.c_float(scale or 0.0))
 
+    def rotary_embedding(self, t, cos_cache, sin_cache, token_index=None):
+        return self._op("ttrt_pb_rotary_embedding", t, cos_cache, sin_cache, int(token_index is not None), token_index or 0)
+
+    def update_cache(self, cache, t, update_index, batch_offset=0):
+        _call("ttrt_pb_update_cache", self.h, cache, t, update_index, batch_offset)
+
+    def fill_cache(self, cache, t, batch_offset=0):
+        _call("ttrt_pb_fill_cache", self.h, cache, t, batch_offset)
+
+    def sdpa_decode(self, q, k, v, cur_pos=0, mask=0, page_table=0, is_causal=True, scale=None):
+        return self._op("ttrt_pb_sdpa_decode", q, k, v, page_table, mask, cur_pos, int(is_causal), int(scale is not None),
+                        ctypes.c_float(scale or 0.0))
+
     def reshape(self, t, shape):
         s, r = _shape_arg(shape)
         return self._op("ttrt_pb_reshape", t, s, r)

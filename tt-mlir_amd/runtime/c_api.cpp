@@ -402,6 +402,20 @@ TTRT_EXPORT int ttrt_pb_sdpa(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t 
                              uint32_t *out) {
   PB_OP(sdpa(q, k, v, mask, is_causal != 0, has_scale != 0, scale));
 }
+TTRT_EXPORT int ttrt_pb_rotary_embedding(ttrt_builder *pb, uint32_t in, uint32_t cos_cache, uint32_t sin_cache, int has_token_index,
+                                         uint32_t token_index, uint32_t *out) {
+  PB_OP(rotaryEmbedding(in, cos_cache, sin_cache, has_token_index != 0, token_index));
+}
+TTRT_EXPORT int ttrt_pb_update_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t update_index, uint32_t batch_offset) {
+  return guard([&] { need(pb, "builder"); pb->pb.updateCache(cache, in, update_index, batch_offset); });
+}
+TTRT_EXPORT int ttrt_pb_fill_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t batch_offset) {
+  return guard([&] { need(pb, "builder"); pb->pb.fillCache(cache, in, batch_offset); });
+}
+TTRT_EXPORT int ttrt_pb_sdpa_decode(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t page_table, uint32_t mask, uint32_t cur_pos,
+                                    int is_causal, int has_scale, float scale, uint32_t *out) {
+  PB_OP(sdpaDecode(q, k, v, page_table, mask, cur_pos, is_causal != 0, has_scale != 0, scale));
+}
 TTRT_EXPORT int ttrt_pb_reshape(ttrt_builder *pb, uint32_t in, const uint32_t *shape, int rank, uint32_t *out) { PB_OP(reshape(in, shapeVec(shape, rank))); }
 TTRT_EXPORT int ttrt_pb_permute(ttrt_builder *pb, uint32_t in, const int64_t *perm, int rank, uint32_t *out) {
   PB_OP(permute(in, std::vector<std::int64_t>(perm, perm + rank)));

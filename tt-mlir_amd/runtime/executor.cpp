@@ -378,6 +378,131 @@ void runSdpa(const fb::Table &op, ProgramContext &ctx) {
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 
+// ---- decode path (runtime/lib/ttnn/operations/transformer/rotary_embedding.cpp, scaled_dot_product_attention_decode.cpp,
+// paged_scaled_dot_product_attention_decode.cpp; operations/kv_cache/{update_cache,fill_cache}.cpp)
+int floatCode(DataType dt, const char *what) {
+  if (dt == DataType::BFloat16) return TTM_BF16;
+  if (dt == DataType::Float32) return TTM_F32;
+  fatal(std::string(what) + ": tensors must be BFloat16 or Float32");
+}
+// positions (update index, current positions, page table) as 32-bit integers in device memory, row-major
+Tensor devicePositions(ProgramContext &ctx, const Tensor &t, const char *what) {
+  TTRT_ASSERT(t.handle->dtype == DataType::Int32 || t.handle->dtype == DataType::UInt32,
+              std::string(what) + " must be a 32-bit integer tensor");
+  return as(ctx, t, TensorLayout::RowMajor, t.handle->dtype);
+}
+
+void runRotaryEmbedding(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::RotaryEmbeddingOp;
+  Tensor &in = ctx.get(op.table(S::f_input), "rotary_embedding input");
+  const DataType dt = in.handle->dtype == DataType::Float32 ? DataType::Float32 : DataType::BFloat16;
+  Tensor x = as(ctx, in, TensorLayout::Tile, dt);
+  Tensor cosc = as(ctx, ctx.get(op.table(S::f_cos_cache), "rotary_embedding cos"), TensorLayout::Tile, dt);
+  Tensor sinc = as(ctx, ctx.get(op.table(S::f_sin_cache), "rotary_embedding sin"), TensorLayout::Tile, dt);
+  const auto &xs = x.handle->shape, &cs = cosc.handle->shape;
+  TTRT_ASSERT(xs.size() == 4 && cs.size() == 4 && sinc.handle->shape == cs, "rotary_embedding: all tensors must be 4D, cos and sin of one shape");
+  TTRT_ASSERT(cs[0] == 1 && cs[1] == 1 && cs[3] == xs[3], "rotary_embedding: cos / sin caches must be [1, 1, positions, head_dim]");
+  const std::int64_t token = op.has(S::f_token_index) ? op.scalar<std::uint32_t>(S::f_token_index, 0) : -1;
+  auto outRef = op.table(S::f_out);
+  Tensor out = makeDeviceTensor(ctx.dev, xs, dt, TensorLayout::Tile);
+  TTM_CALL(ttm_rotary_embedding(x.handle->data.get(), cosc.handle->data.get(), sinc.handle->data.get(), out.handle->data.get(),
+                                floatCode(dt, "rotary_embedding"), static_cast<std::int64_t>(xs[0]) * xs[1], xs[2], xs[3], cs[2], token,
+                                ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// the cache operand of the in-place cache ops: it must already be what the kernels write into
+Tensor &cacheOperand(ProgramContext &ctx, const fb::Table &ref, const char *what) {
+  Tensor &cache = ctx.get(ref, what);
+  TTRT_ASSERT(cache.handle->storage == StorageType::Device && cache.handle->layout == TensorLayout::Tile && cache.handle->shape.size() == 4,
+              std::string(what) + " must be a 4D device tensor in tile layout");
+  return cache;
+}
+void runUpdateCache(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::UpdateCacheOp;
+  Tensor &cache = cacheOperand(ctx, op.table(S::f_cache), "update_cache cache");
+  const auto &cs = cache.handle->shape;
+  Tensor in = as(ctx, ctx.get(op.table(S::f_input), "update_cache input"), TensorLayout::Tile, cache.handle->dtype);
+  const auto &is = in.handle->shape;
+  TTRT_ASSERT(is.size() == 4 && is[0] == 1 && is[1] == cs[1] && is[3] == cs[3],
+              "update_cache: input must be [1, heads, users, head_dim] matching the cache");
+  Tensor index = devicePositions(ctx, ctx.get(op.table(S::f_update_index), "update_cache index"), "update_cache: update_index");
+  TTM_CALL(ttm_update_cache(cache.handle->data.get(), in.handle->data.get(), static_cast<const std::int32_t *>(index.handle->data.get()),
+                            floatCode(cache.handle->dtype, "update_cache"), cs[0], cs[1], cs[2], cs[3], is[2],
+                            op.scalar<std::uint32_t>(S::f_batch_offset, 0), ctx.stream()));
+  cache.handle->version = nextTensorVersion();
+}
+void runFillCache(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::FillCacheOp;
+  Tensor &cache = cacheOperand(ctx, op.table(S::f_cache), "fill_cache cache");
+  const auto &cs = cache.handle->shape;
+  Tensor in = as(ctx, ctx.get(op.table(S::f_input), "fill_cache input"), TensorLayout::Tile, cache.handle->dtype);
+  const auto &is = in.handle->shape;
+  // lib/Dialect/TTNN/IR/TTNNOps.cpp:4896-4946
+  TTRT_ASSERT(is.size() == 4 && is[1] == cs[1] && is[3] == cs[3], "fill_cache: cache and input must agree on dims 1 and 3");
+  TTRT_ASSERT(is[2] <= cs[2], "fill_cache: input has more positions than the cache");
+  TTRT_ASSERT(is[0] == 1, "fill_cache: input must hold one user");
+  TTM_CALL(ttm_fill_cache(cache.handle->data.get(), in.handle->data.get(), floatCode(cache.handle->dtype, "fill_cache"), cs[0], cs[1], cs[2],
+                          cs[3], is[2], op.scalar<std::uint32_t>(S::f_batch_offset, 0), ctx.stream()));
+  cache.handle->version = nextTensorVersion();
+}
+
+void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRef, const fb::Table &vRef, const fb::Table &pageRef,
+                const fb::Table &maskRef, const fb::Table &posRef, bool causal, float scale, const fb::Table &outRef) {
+  Tensor q = as(ctx, ctx.get(qRef, "sdpa_decode query"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor k = as(ctx, ctx.get(kRef, "sdpa_decode key"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor v = as(ctx, ctx.get(vRef, "sdpa_decode value"), TensorLayout::Tile, DataType::BFloat16);
+  const auto &qs = q.handle->shape, &ks = k.handle->shape;
+  TTRT_ASSERT(qs.size() == 4 && ks.size() == 4 && v.handle->shape == ks && qs[0] == 1 && qs[3] == ks[3],
+              "sdpa_decode: query must be [1, batch, heads, head_dim], key / value 4D with the same head_dim");
+  const std::int64_t B = qs[1], H = qs[2], Hkv = ks[1], D = qs[3];
+  Tensor table;
+  std::int64_t pages = 0, block = 0, S = ks[2];
+  if (pageRef) {
+    table = devicePositions(ctx, ctx.get(pageRef, "sdpa_decode page table"), "sdpa_decode: page_table");
+    const auto &ts = table.handle->shape;
+    TTRT_ASSERT(ts.size() == 2 && ts[0] == B, "sdpa_decode: page table must be [batch, blocks per user]");
+    pages = ts[1]; block = ks[2]; S = pages * block;
+  } else {
+    TTRT_ASSERT(ks[0] == B, "sdpa_decode: key / value batch differs from the query's");
+  }
+  Tensor mask, pos;
+  int maskHeads = 1;
+  if (maskRef) {
+    mask = as(ctx, ctx.get(maskRef, "sdpa_decode mask"), TensorLayout::Tile, DataType::BFloat16);
+    const auto &ms = mask.handle->shape;
+    TTRT_ASSERT(ms.size() == 4 && ms[0] == B && ms[1] == 1 && (ms[2] == 1 || ms[2] == H) && ms[3] == S,
+                "sdpa_decode: mask must be [batch, 1, 1|heads, positions]");
+    maskHeads = static_cast<int>(ms[2]);
+  }
+  if (posRef) {
+    pos = devicePositions(ctx, ctx.get(posRef, "sdpa_decode cur_pos"), "sdpa_decode: cur_pos_tensor");
+    TTRT_ASSERT(volume(pos.handle->shape) == B, "sdpa_decode: cur_pos_tensor must hold one position per user");
+  }
+  Tensor out = makeDeviceTensor(ctx.dev, qs, DataType::BFloat16, TensorLayout::Tile);
+  TTM_CALL(ttm_sdpa_decode(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
+                           pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
+                           mask ? mask.handle->data.get() : nullptr, maskHeads,
+                           table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
+                           out.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+void runSdpaDecode(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::ScaledDotProductAttentionDecodeOp;
+  TTRT_ASSERT(!op.has(S::f_sliding_window_size) && !op.table(S::f_attention_sink), "sdpa_decode: sliding window / attention sink are not supported");
+  sdpaDecode(ctx, op.table(S::f_query), op.table(S::f_key), op.table(S::f_value), fb::Table(), op.table(S::f_attention_mask),
+             op.table(S::f_cur_pos_tensor), op.scalar<std::uint8_t>(S::f_is_causal, 0) != 0,
+             op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f, op.table(S::f_out));
+}
+void runPagedSdpaDecode(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::PagedScaledDotProductAttentionDecodeOp;
+  TTRT_ASSERT(!op.has(S::f_sliding_window_size) && !op.table(S::f_attention_sink), "paged sdpa_decode: sliding window / attention sink are not supported");
+  TTRT_ASSERT(static_cast<bool>(op.table(S::f_page_table)), "paged sdpa_decode: page table missing");
+  sdpaDecode(ctx, op.table(S::f_query), op.table(S::f_key), op.table(S::f_value), op.table(S::f_page_table), op.table(S::f_attention_mask),
+             op.table(S::f_cur_pos_tensor), op.scalar<std::uint8_t>(S::f_is_causal, 0) != 0,
+             op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f, op.table(S::f_out));
+}
+
 // ---- data movement (runtime/lib/ttnn/operations/data_movement/*.cpp)
 bool sameTiling(const std::vector<std::uint32_t> &a, const std::vector<std::uint32_t> &b) {
   // physical tile order is unchanged when the last dim is kept and no padding is involved
@@ -776,6 +901,11 @@ void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   case OpType::DeallocateOp: return runDeallocate(op, ctx);
   case OpType::LoadCachedOp: return runLoadCached(op, ctx);
   case OpType::FuncCallOp: return runFuncCall(op, ctx);
+  case OpType::RotaryEmbeddingOp: return runRotaryEmbedding(op, ctx);
+  case OpType::UpdateCacheOp: return runUpdateCache(op, ctx);
+  case OpType::FillCacheOp: return runFillCache(op, ctx);
+  case OpType::ScaledDotProductAttentionDecodeOp: return runSdpaDecode(op, ctx);
+  case OpType::PagedScaledDotProductAttentionDecodeOp: return runPagedSdpaDecode(op, ctx);
   case OpType::BeginTraceCaptureOp: return runBeginTraceCapture(op, ctx);
   case OpType::EndTraceCaptureOp: return runEndTraceCapture(op, ctx);
   case OpType::ExecuteTraceOp: return runExecuteTrace(op, ctx);
@@ -883,6 +1013,24 @@ OpRefs opRefs(const fb::Table &operation) {
   case OpType::DeallocateOp: in(schema::DeallocateOp::f_in); break;
   case OpType::LoadCachedOp: inVec(schema::LoadCachedOp::f_inputs); outVec(schema::LoadCachedOp::f_outputs); break;
   case OpType::FuncCallOp: inVec(schema::FuncCallOp::f_inputs); outVec(schema::FuncCallOp::f_outputs); break;
+  case OpType::RotaryEmbeddingOp:
+    in(schema::RotaryEmbeddingOp::f_input); in(schema::RotaryEmbeddingOp::f_cos_cache); in(schema::RotaryEmbeddingOp::f_sin_cache);
+    out(schema::RotaryEmbeddingOp::f_out);
+    break;
+  case OpType::UpdateCacheOp:
+    in(schema::UpdateCacheOp::f_cache); in(schema::UpdateCacheOp::f_input); in(schema::UpdateCacheOp::f_update_index);
+    break;
+  case OpType::FillCacheOp: in(schema::FillCacheOp::f_cache); in(schema::FillCacheOp::f_input); break;
+  case OpType::ScaledDotProductAttentionDecodeOp: {
+    using S = schema::ScaledDotProductAttentionDecodeOp;
+    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
+    break;
+  }
+  case OpType::PagedScaledDotProductAttentionDecodeOp: {
+    using S = schema::PagedScaledDotProductAttentionDecodeOp;
+    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_page_table); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
+    break;
+  }
   case OpType::CaptureOrExecuteTraceOp:
     inVec(schema::CaptureOrExecuteTraceOp::f_inputs); outVec(schema::CaptureOrExecuteTraceOp::f_outputs);
     break;

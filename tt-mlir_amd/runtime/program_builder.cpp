@@ -414,6 +414,68 @@ ProgramBuilder::Id ProgramBuilder::sdpa(Id q, Id k, Id v, Id mask, bool causal, 
   return out;
 }
 
+ProgramBuilder::Id ProgramBuilder::rotaryEmbedding(Id in, Id cosCache, Id sinCache, bool hasTokenIndex, std::uint32_t tokenIndex) {
+  Desc d = desc(in);
+  d.storage = StorageType::Device;
+  d.layout = TensorLayout::Tile;
+  Id out = newTensor(d);
+  using S = RotaryEmbeddingOp;
+  Off i = tensorRef(in), c = tensorRef(cosCache), sn = tensorRef(sinCache), o = tensorRef(out);
+  b_.startTable(S::kNumFields);
+  b_.addOffset(S::f_input, i);
+  b_.addOffset(S::f_cos_cache, c);
+  b_.addOffset(S::f_sin_cache, sn);
+  if (hasTokenIndex) b_.addScalar<std::uint32_t>(S::f_token_index, tokenIndex);
+  b_.addOffset(S::f_out, o);
+  addOp(OpType::RotaryEmbeddingOp, b_.endTable(), "ttnn.rotary_embedding " + shapeStr(d.shape));
+  return out;
+}
+void ProgramBuilder::updateCache(Id cache, Id in, Id updateIndex, std::uint32_t batchOffset) {
+  Off c = tensorRef(cache), i = tensorRef(in), u = tensorRef(updateIndex);
+  b_.startTable(UpdateCacheOp::kNumFields);
+  b_.addOffset(UpdateCacheOp::f_cache, c);
+  b_.addOffset(UpdateCacheOp::f_input, i);
+  b_.addOffset(UpdateCacheOp::f_update_index, u);
+  b_.addScalarDefault<std::uint32_t>(UpdateCacheOp::f_batch_offset, batchOffset, 0);
+  addOp(OpType::UpdateCacheOp, b_.endTable(), "ttnn.update_cache");
+}
+void ProgramBuilder::fillCache(Id cache, Id in, std::uint32_t batchOffset) {
+  Off c = tensorRef(cache), i = tensorRef(in);
+  b_.startTable(FillCacheOp::kNumFields);
+  b_.addOffset(FillCacheOp::f_cache, c);
+  b_.addOffset(FillCacheOp::f_input, i);
+  b_.addScalarDefault<std::uint32_t>(FillCacheOp::f_batch_offset, batchOffset, 0);
+  addOp(OpType::FillCacheOp, b_.endTable(), "ttnn.fill_cache");
+}
+ProgramBuilder::Id ProgramBuilder::sdpaDecode(Id q, Id k, Id v, Id pageTable, Id mask, Id curPos, bool causal, bool hasScale, float scale) {
+  Desc d = desc(q);
+  d.storage = StorageType::Device;
+  d.layout = TensorLayout::Tile;
+  Id out = newTensor(d);
+  Off qr = tensorRef(q), kr = tensorRef(k), vr = tensorRef(v), pt = pageTable ? tensorRef(pageTable) : 0, mr = mask ? tensorRef(mask) : 0,
+      cp = curPos ? tensorRef(curPos) : 0, o = tensorRef(out);
+  if (pageTable) {
+    using S = PagedScaledDotProductAttentionDecodeOp;
+    b_.startTable(S::kNumFields);
+    b_.addOffset(S::f_query, qr); b_.addOffset(S::f_key, kr); b_.addOffset(S::f_value, vr); b_.addOffset(S::f_page_table, pt);
+    b_.addScalarDefault<std::uint8_t>(S::f_is_causal, causal, 0);
+    b_.addOffset(S::f_attention_mask, mr); b_.addOffset(S::f_cur_pos_tensor, cp);
+    if (hasScale) b_.addScalar<float>(S::f_scale, scale);
+    b_.addOffset(S::f_out, o);
+    addOp(OpType::PagedScaledDotProductAttentionDecodeOp, b_.endTable(), "ttnn.paged_scaled_dot_product_attention_decode " + shapeStr(d.shape));
+  } else {
+    using S = ScaledDotProductAttentionDecodeOp;
+    b_.startTable(S::kNumFields);
+    b_.addOffset(S::f_query, qr); b_.addOffset(S::f_key, kr); b_.addOffset(S::f_value, vr);
+    b_.addScalarDefault<std::uint8_t>(S::f_is_causal, causal, 0);
+    b_.addOffset(S::f_attention_mask, mr); b_.addOffset(S::f_cur_pos_tensor, cp);
+    if (hasScale) b_.addScalar<float>(S::f_scale, scale);
+    b_.addOffset(S::f_out, o);
+    addOp(OpType::ScaledDotProductAttentionDecodeOp, b_.endTable(), "ttnn.scaled_dot_product_attention_decode " + shapeStr(d.shape));
+  }
+  return out;
+}
+
 ProgramBuilder::Id ProgramBuilder::reshape(Id in, const std::vector<std::uint32_t> &shape) {
   Desc d = desc(in);
   d.shape = shape;

@@ -50,6 +50,11 @@ public:
   Id constant(const void *data, size_t bytes, DataType inDtype, const std::vector<std::uint32_t> &shape, DataType dtype,
               TensorLayout layout, StorageType storage);
   Id full(const std::vector<std::uint32_t> &shape, float value, DataType dtype, TensorLayout layout);
+  Id rotaryEmbedding(Id in, Id cosCache, Id sinCache, bool hasTokenIndex, std::uint32_t tokenIndex);
+  void updateCache(Id cache, Id in, Id updateIndex, std::uint32_t batchOffset);
+  void fillCache(Id cache, Id in, std::uint32_t batchOffset);
+  // pageTable = 0 writes ScaledDotProductAttentionDecodeOp, otherwise the paged op
+  Id sdpaDecode(Id q, Id k, Id v, Id pageTable, Id mask, Id curPos, bool causal, bool hasScale, float scale);
   Id empty(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout);
   void copy(Id src, Id dst);                 // ttnn.copy: dst <- src, both on device
   void writeTensor(Id host, Id device);      // ttnn.write_tensor: device <- host

@@ -613,6 +613,7 @@ std::string getDeviceName(Device) {
 
 // ============================================================================ tensors
 static std::atomic<std::uint64_t> g_tensorVersion{1};
+std::uint64_t nextTensorVersion() { return g_tensorVersion++; }
 
 Tensor makeHostTensor(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout) {
   auto t = std::make_shared<TensorImpl>();

@@ -86,6 +86,7 @@ std::int64_t volume(const std::vector<std::uint32_t> &shape);
 std::int64_t paddedVolume(const std::vector<std::uint32_t> &shape);
 size_t tensorBytes(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout);
 
+std::uint64_t nextTensorVersion();  // a tensor written in place takes a new version
 Tensor makeDeviceTensor(const std::shared_ptr<DeviceState> &dev, const std::vector<std::uint32_t> &shape, DataType dtype,
                         TensorLayout layout);
 Tensor makeHostTensor(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout);
