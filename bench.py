@@ -110,7 +110,55 @@ def make_workloads(torch, hip, datagen, dev, names):
             out[nm] = Workload(nm, "hbm", nbytes, "bytes", fn,
                                "config 3 decode: bf16 [32,4096] x bfp8_b [4096,14336] + bias + GELU (weight streaming)",
                                dict(flop=2.0 * M * N * K))
+    if "sdpa_decode32" in names:
+        B, H, Hkv, S, D = 32, 32, 8, 2048, 128
+        q = datagen.randn((1, B, H, D), seed=1, dtype=torch.bfloat16).to(dev)
+        kv = [datagen.randn((B, Hkv, S, D), seed=2 + i, dtype=torch.bfloat16).to(dev) for i in range(2)]
+        qt, o = torch.empty(B * 32 * D, dtype=torch.bfloat16, device=dev), torch.empty(B * 32 * D, dtype=torch.bfloat16, device=dev)
+        hip.call("ttm_tilize", hip.ptr(q), hip.ptr(qt), B, H, D, 2, s)
+        kvt = [torch.empty_like(t) for t in kv]
+        for t, tt in zip(kv, kvt):
+            hip.call("ttm_tilize", hip.ptr(t), hip.ptr(tt), B * Hkv, S, D, 2, s)
+        cur = torch.full((B,), S - 1, dtype=torch.int32, device=dev)
+        torch.cuda.synchronize()
+        del kv
+        out["sdpa_decode32"] = Workload(
+            "sdpa_decode32", "hbm", 2 * B * Hkv * S * D * 2 + 2 * B * H * D * 2, "bytes",
+            lambda: hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kvt[0]), hip.ptr(kvt[1]), hip.ptr(cur), None, 1, None, 0, 0,
+                             hip.ptr(o), hip.BF16, B, H, Hkv, S, D, 1, 0.0, s),
+            "decode attention: 32 users x 32 heads (8 kv heads) x 1 token over a full 2048-position bf16 KV cache",
+            dict(keep=(qt, kvt, cur, o)))
     # whole programs through the runtime boundary (flatbuffer -> submit -> wait)
+    for nm in ("decode32", "decode32_traced"):
+        if nm not in names:
+            continue
+        from ttmlir_amd import programs, runtime as rt
+        users, hidden, n_q, n_kv, hd, ffn, max_seq, pos = 32, 4096, 32, 8, 128, 14336, 2048, 2047
+        binary = rt.Binary.load_from_memory(programs.decode_layer(users, hidden, n_q, n_kv, hd, ffn, max_seq, trace=nm.endswith("traced"),
+                                                                  host_inputs=False))
+        main = binary.get_num_programs() - 1
+        r16 = lambda shape, seed, scale=1.0: (datagen.randn(shape, seed=seed, dtype=torch.float32) * scale).to(torch.bfloat16)
+        wshapes = [(hidden,), (hidden, n_q * hd), (hidden, n_kv * hd), (hidden, n_kv * hd), (n_q * hd, hidden), (hidden,), (hidden, ffn),
+                   (hidden, ffn), (ffn, hidden)]
+        tins = [r16((users, hidden), 1), r16((1, 1, 1, hd), 2), r16((1, 1, 1, hd), 3), torch.tensor([pos], dtype=torch.int32),
+                torch.full((users,), pos, dtype=torch.int32), r16((users, n_kv, max_seq, hd), 4), r16((users, n_kv, max_seq, hd), 5)]
+        tins += [r16(sh, 10 + i, 0.02) for i, sh in enumerate(wshapes)]
+        rdev = rt.open_mesh_device()
+        rins = [rt.to_layout(rt.from_torch(t), rdev, rt.get_layout(binary, main, i), retain=True) for i, t in enumerate(tins)]
+        del tins
+        # bytes one step must move: block-float weights once, both caches up to the current position, activations
+        wbytes = sum((a // 32) * (b // 32) * 1088 for a, b in (wshapes[1], wshapes[2], wshapes[3], wshapes[4], wshapes[6], wshapes[7]))
+        wbytes += (ffn // 32) * (hidden // 32) * 576
+        nbytes = wbytes + 2 * users * n_kv * (pos + 1) * hd * 2
+
+        def run(binary=binary, rins=rins, rdev=rdev, main=main):
+            outs = rt.submit(rdev, binary, main, rins)
+            rt.wait(outs)
+
+        out[nm] = Workload(nm, "hbm", nbytes, "bytes", run,
+                           "Llama-3-8B decoder layer, one token for 32 users at position 2047 (weights bfp8_b / bfp4_b, bf16 KV cache "
+                           "updated in place), one submit" + (" replaying a captured HIP graph" if nm.endswith("traced") else ""),
+                           dict(sync=True, steps=50, keep=(rdev, rins, binary)))
     for nm in ("mlp512", "decoder2048"):
         if nm not in names:
             continue
@@ -207,7 +255,8 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="linear2048")
-    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,mlp512,decoder2048")
+    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,sdpa_decode32,mlp512,decoder2048,"
+                                           "decode32,decode32_traced")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -254,7 +303,7 @@ def main():
     for n in sec_names:
         w = wl[n]
         heavy = bool(w.extra.get("sync"))
-        sms, skms = measure(w, 5 if heavy else max(10, args.steps // 2), 2 if heavy else max(3, args.warmup // 2))
+        sms, skms = measure(w, w.extra.get("steps", 5) if heavy else max(10, args.steps // 2), 2 if heavy else max(3, args.warmup // 2))
         r = roofline(w, skms)
         secondary.append({"workload": n, "desc": w.desc, "ms_per_step": round(sms, 5), "roofline": r})
 

@@ -19,7 +19,7 @@
 // Rows whose shared exponent is below 7 (|w| < 2^-120) are flushed to zero.
 //
 // Kernels, by use: ttm_linear_dma_k (block-float weights, M > 64), ttm_linear_reg_k (bf16 weights, M > 64),
-// ttm_linear_big_k (64-bit-addressed fallback), ttm_linear_decode_bfp8_k / ttm_linear_small_k (M <= 64),
+// ttm_linear_big_k (64-bit-addressed fallback), ttm_linear_decode_k / ttm_linear_small_k (M <= 64),
 // ttm_linear_reduce_k (second half of a split-K launch).
 #include <type_traits>
 
@@ -1125,9 +1125,13 @@ __global__ __launch_bounds__(256) void ttm_linear_small_k(LinearArgs p) {
 // =============================================================================================
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
-__global__ __launch_bounds__(512) void ttm_linear_decode_bfp8_k(LinearArgs p) {
+// BFP4 = true reads bfp4_b tiles (576 bytes, two elements per byte, low nibble first): a lane's 4 (n) of a k row are one
+// 16-bit word, whose nibbles are spread into the bytes of a word before the same sign-magnitude -> offset-binary step.
+template <bool BFP4>
+__global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   extern __shared__ u32x4 smem[];   // partial sums: 8 wavefronts x 8 x 64 float4 = 64 KiB
   constexpr int D = 4;
+  constexpr uint32_t TB = BFP4 ? 576u : 1088u, FACE = BFP4 ? 128u : 256u, ROW = BFP4 ? 8u : 16u;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int cg = blockIdx.x;
@@ -1137,8 +1141,8 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_bfp8_k(LinearArgs p) {
   const int q16 = lane & 15, kg = lane >> 4;   // weight operand row and 8-k group of this lane
   const int fc = (q16 >> 2) & 1, quad = q16 & 3, fr = kg >> 1, half = kg & 1;
   const uint32_t nt_l = (uint32_t)min(2 * cg + (q16 >> 3), p.Nt - 1);
-  const uint32_t offW = nt_l * 1088u + 64u + (fr * 2 + fc) * 256 + half * 128 + quad * 4;   // + 16 i
-  const uint32_t offE = nt_l * 1088u + (fr * 2 + fc) * 16 + half * 8;
+  const uint32_t offW = nt_l * TB + 64u + (fr * 2 + fc) * FACE + half * (FACE / 2) + quad * (ROW / 4);   // + ROW i
+  const uint32_t offE = nt_l * TB + (fr * 2 + fc) * 16 + half * 8;
   const uint32_t offA = fr * 512 + q16 * 32 + half * 16;                                     // + 1024 h
 
   f32x4v acc[2][4];
@@ -1155,10 +1159,11 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_bfp8_k(LinearArgs p) {
     const int kt = wave + 8 * c;
     const int ktc = min(kt, p.Kt - 1);
     const uint32_t keep = kt < p.Kt ? 0xFFFFFFFFu : 0u;   // past the end: zero exponents, zero weights
-    const uint8_t *Wk = W + (int64_t)ktc * p.Nt * 1088;
+    const uint8_t *Wk = W + (int64_t)ktc * p.Nt * TB;
     const uint8_t *Ak = A + (int64_t)ktc * 2048;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) rows[s][i] = *(const uint32_t *)(Wk + offW + i * 16);   // the eight loads share their cache lines: cached loads
+    for (int i = 0; i < 8; ++i)   // the eight loads share their cache lines: cached loads
+      rows[s][i] = BFP4 ? (uint32_t) * (const uint16_t *)(Wk + offW + i * ROW) : *(const uint32_t *)(Wk + offW + i * ROW);
     ex[s] = *(const u32x2 *)(Wk + offE);
     keeps[s] = keep;   // applied when the slot is consumed: masking here would wait for the load
 #pragma unroll
@@ -1169,11 +1174,17 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_bfp8_k(LinearArgs p) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       uint32_t E = (((i < 4 ? ex[s].x : ex[s].y) & keeps[s]) >> (8 * (i & 3))) & 0xFFu;
-      E = max(E, 6u);
-      const float scale = __uint_as_float((E - 6u) << 23), nscale = -128.0f * scale;
-      const uint32_t d = rows[s][i];
-      const uint32_t sg = d & 0x80808080u, sb = sg >> 7;
-      const uint32_t t = (d ^ 0x80808080u ^ (sg - sb)) + sb;
+      // value = magnitude x 2^(E - 127 - 6) (bfp8_b) or 2^(E - 127 - 2) (bfp4_b); smaller exponents flush to zero
+      constexpr uint32_t EB = BFP4 ? 2u : 6u, SIGN = BFP4 ? 0x08080808u : 0x80808080u, SH = BFP4 ? 3u : 7u;
+      E = max(E, EB);
+      const float scale = __uint_as_float((E - EB) << 23), nscale = (BFP4 ? -8.0f : -128.0f) * scale;
+      uint32_t d = rows[s][i];
+      if (BFP4) {   // nibbles n3 n2 n1 n0 of the low half -> one per byte
+        d = (d | (d << 8)) & 0x00FF00FFu;
+        d = (d | (d << 4)) & 0x0F0F0F0Fu;
+      }
+      const uint32_t sg = d & SIGN, sb = sg >> SH;
+      const uint32_t t = (d ^ SIGN ^ (sg - sb)) + sb;
 #pragma unroll
       for (int b = 0; b < 4; ++b) f[i][b] = fmaf((float)((t >> (8 * b)) & 0xFFu), scale, nscale);
     }
@@ -1293,11 +1304,12 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
   if (a.Mt == 1 || a.Mt * 32 <= ttm_option("linear_small_m_max")) {
     // the small kernel handles one row tile per launch
     LinearArgs p = a;
-    const bool decode = WF == WF_BFP8 && ttm_option("linear_variant") != 1 && (int64_t)a.Nt * 1088 < (int64_t)1 << 32;
+    const bool decode = BFP && ttm_option("linear_variant") != 1 && (int64_t)a.Nt * 1088 < (int64_t)1 << 32;
     for (int mt = 0; mt < a.Mt; ++mt) {
       p.A = a.A + (int64_t)mt * a.Kt * 2048;
       p.C = a.C + (int64_t)mt * a.Nt * 2048;
-      if (decode) hipLaunchKernelGGL(ttm_linear_decode_bfp8_k, dim3((a.Nt + 1) / 2, 1, (unsigned)batch), dim3(512), 65536, s, p);
+      if (decode && WF == WF_BFP4) hipLaunchKernelGGL(ttm_linear_decode_k<true>, dim3((a.Nt + 1) / 2, 1, (unsigned)batch), dim3(512), 65536, s, p);
+      else if (decode) hipLaunchKernelGGL(ttm_linear_decode_k<false>, dim3((a.Nt + 1) / 2, 1, (unsigned)batch), dim3(512), 65536, s, p);
       else hipLaunchKernelGGL((ttm_linear_small_k<WF>), dim3(a.Nt, 1, (unsigned)batch), dim3(256), 0, s, p);
     }
     return 0;

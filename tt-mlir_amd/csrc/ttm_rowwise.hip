@@ -275,11 +275,138 @@ __global__ __launch_bounds__(256) void ttm_rowwise_resident_k(RowArgs p) {
   }
 }
 
+// RMSNorm / softmax with one row per workgroup, for rows of up to NK = 2, 4 or 8 chunks per lane (at most 16384 bf16 or
+// 8192 fp32 columns).
+// The row stays in registers between the reduction and the output pass, weights are fetched while the reduction is in
+// flight, and a workgroup issues all its loads at once: a [32, 4096] input is 32 short workgroups instead of 4 long ones.
+// Consecutive rows of a face share 128-byte lines, so the row -> workgroup map gives every XCD (workgroup id mod 8)
+// a contiguous range of rows and its L2 sees each line of that range whole.
+template <int MODE, int ELEM, int NK>
+__global__ __launch_bounds__(256) void ttm_rowwise_row_k(RowArgs p, int total_rows) {
+  constexpr int EPC = 16 / ELEM;
+  __shared__ float red[4], red2[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int per_xcd = total_rows / 8;                    // total_rows is a multiple of 32
+  const int lrow = (int)(blockIdx.x % 8) * per_xcd + (int)(blockIdx.x / 8);
+  const int r = lrow & 31, trow = lrow >> 5;
+  const int row = (trow % p.rt) * 32 + r;
+  const bool row_ok = row < p.rows;
+  const int nq = p.ct * 2 * ELEM, cols = (int)p.cols;
+  const uint8_t *x = (const uint8_t *)p.x + (int64_t)trow * p.ct * 1024 * ELEM;
+  uint8_t *o = (uint8_t *)p.out + (int64_t)trow * p.ct * 1024 * ELEM;
+  u32x4 v[NK];
+#pragma unroll
+  for (int k = 0; k < NK; ++k) {
+    const int q = tid + k * 256;
+    v[k] = u32x4{0, 0, 0, 0};
+    if (q < nq && row_ok) v[k] = *(const u32x4 *)(x + chunk_pos<ELEM>(r, q).off * ELEM);
+  }
+  u32x4 wraw[NK], braw[NK];   // weight / bias chunks, still packed
+  if (MODE == RW_RMSNORM) {
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+      const int q = tid + k * 256;
+      if (q < nq) {
+        const int c0 = chunk_pos<ELEM>(r, q).c0;
+        const int64_t tiled = (int64_t)(c0 >> 5) * 1024 + ((c0 >> 4) & 1) * 256 + (c0 & 15);
+        if (p.w) wraw[k] = *(const u32x4 *)((const uint8_t *)p.w + (p.w_tiled ? tiled : c0) * ELEM);
+        if (p.b) braw[k] = *(const u32x4 *)((const uint8_t *)p.b + (p.b_tiled ? tiled : c0) * ELEM);
+      }
+    }
+  }
+  float acc = MODE == RW_SOFTMAX ? -INFINITY : 0.0f;
+#pragma unroll
+  for (int k = 0; k < NK; ++k) {
+    const int q = tid + k * 256;
+    if (q < nq) {
+      const int c0 = chunk_pos<ELEM>(r, q).c0;
+      float f[EPC];
+      unpack_vals<ELEM>(v[k], f);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) {
+        const bool ok = c0 + i < cols;
+        if (MODE == RW_RMSNORM) acc += ok ? f[i] * f[i] : 0.0f;
+        else acc = ok ? fmaxf(acc, f[i]) : acc;
+      }
+    }
+  }
+#pragma unroll
+  for (int s = 32; s > 0; s >>= 1) acc = MODE == RW_SOFTMAX ? fmaxf(acc, __shfl_xor(acc, s)) : acc + __shfl_xor(acc, s);
+  if (lane == 0) red[wave] = acc;
+  __syncthreads();
+  const float stat = MODE == RW_SOFTMAX ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : red[0] + red[1] + red[2] + red[3];
+  float mul;
+  if (MODE == RW_RMSNORM) {
+    mul = 1.0f / sqrtf(stat / (float)cols + p.eps);
+  } else {
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+      const int q = tid + k * 256;
+      if (q < nq) {
+        const int c0 = chunk_pos<ELEM>(r, q).c0;
+        float f[EPC];
+        unpack_vals<ELEM>(v[k], f);
+#pragma unroll
+        for (int i = 0; i < EPC; ++i) sum += c0 + i < cols ? expf(f[i] - stat) : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) sum += __shfl_xor(sum, s);
+    if (lane == 0) red2[wave] = sum;
+    __syncthreads();
+    mul = 1.0f / (red2[0] + red2[1] + red2[2] + red2[3]);
+  }
+#pragma unroll
+  for (int k = 0; k < NK; ++k) {
+    const int q = tid + k * 256;
+    if (q < nq) {
+      const ChunkPos<ELEM> cp = chunk_pos<ELEM>(r, q);
+      float f[EPC], w[EPC], b[EPC];
+      unpack_vals<ELEM>(v[k], f);
+      if (MODE == RW_RMSNORM) {
+        if (p.w) unpack_vals<ELEM>(wraw[k], w);
+        if (p.b) unpack_vals<ELEM>(braw[k], b);
+      }
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) {
+        float y;
+        if (MODE == RW_RMSNORM) {
+          y = f[i] * mul;
+          if (p.w) y *= w[i];
+          if (p.b) y += b[i];
+        } else {
+          y = expf(f[i] - stat) * mul;
+        }
+        f[i] = (row_ok && cp.c0 + i < cols) ? y : 0.0f;
+      }
+      store_vals<ELEM>(o, cp.off, f);
+    }
+  }
+}
+
 template <int MODE>
 static int launch_rowwise(const RowArgs &p, int dtype, int64_t trows, hipStream_t s) {
   TTM_REQUIRE(trows < (1ll << 29), "row-wise kernel: tensor too large");
   if constexpr (MODE == RW_RMSNORM || MODE == RW_SOFTMAX) {
     const int elem = dtype == TTM_BF16 ? 2 : 4;
+    if (p.ct * 2 * elem <= 8 * 256 && trows * 32 < (1 << 24) && ttm_option("rowwise_variant") != 1) {   // one row per workgroup
+      const int total = (int)(trows * 32), nq = p.ct * 2 * elem;
+      const dim3 grid((unsigned)total), block(256);
+#define TTM_ROW_LAUNCH(E, N) hipLaunchKernelGGL((ttm_rowwise_row_k<MODE, E, N>), grid, block, 0, s, p, total)
+      if (dtype == TTM_BF16) {
+        if (nq <= 512) TTM_ROW_LAUNCH(2, 2);
+        else if (nq <= 1024) TTM_ROW_LAUNCH(2, 4);
+        else TTM_ROW_LAUNCH(2, 8);
+      } else {
+        if (nq <= 512) TTM_ROW_LAUNCH(4, 2);
+        else if (nq <= 1024) TTM_ROW_LAUNCH(4, 4);
+        else TTM_ROW_LAUNCH(4, 8);
+      }
+#undef TTM_ROW_LAUNCH
+      TTM_LAUNCH_CHECK();
+      return TTM_OK;
+    }
     if (p.ct * 2 * elem <= 16 * 32) {   // a lane's share of the row fits in registers
       if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_resident_k<MODE, 2>), dim3((unsigned)trows * 4), dim3(256), 0, s, p);
       else hipLaunchKernelGGL((ttm_rowwise_resident_k<MODE, 4>), dim3((unsigned)trows * 4), dim3(256), 0, s, p);

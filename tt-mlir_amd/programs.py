@@ -254,12 +254,13 @@ def _decode_body(pb, a, users, hidden, n_q, n_kv, head_dim, eps):
     return pb.binary(BINARY["add"], x1, d)
 
 
-def decode_layer(users=32, hidden=4096, n_q=32, n_kv=8, head_dim=128, ffn=14336, max_seq=2048, eps=1e-5, trace=False):
+def decode_layer(users=32, hidden=4096, n_q=32, n_kv=8, head_dim=128, ffn=14336, max_seq=2048, eps=1e-5, trace=False,
+                 host_inputs=True):
     """Decoder layer, one new token per user, KV caches updated in place.  Inputs: x [users, hidden], cos / sin
     [1, 1, 1, head_dim] of the current position, update_index [1] and cur_pos [users] (Int32), k / v caches
     [users, n_kv, max_seq, head_dim], then the weights in bf16 (packed to block-float by const-eval).  With trace=True
-    the step is one traced region: activations, rotary rows and positions are staged from the host, caches and weights
-    are device resident."""
+    the step is one traced region: activations, rotary rows and positions are staged from the host (or, with
+    host_inputs=False, are device tensors the caller updates in place), caches and weights are device resident."""
     pb = rt.ProgramBuilder()
     dq, dkv = n_q * head_dim, n_kv * head_dim
     name = "decode_layer"
@@ -268,8 +269,9 @@ def decode_layer(users=32, hidden=4096, n_q=32, n_kv=8, head_dim=128, ffn=14336,
         ((dq, hidden), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8), ((hidden, ffn), DT.BFP_BFloat8),
         ((ffn, hidden), DT.BFP_BFloat4)])
     cache_shape = (users, n_kv, max_seq, head_dim)
-    step = [((users, hidden), DT.BFloat16, False), ((1, 1, 1, head_dim), DT.BFloat16, False), ((1, 1, 1, head_dim), DT.BFloat16, False),
-            ((1,), DT.Int32, False, TL.RowMajor), ((users,), DT.Int32, False, TL.RowMajor),
+    on_dev = not host_inputs
+    step = [((users, hidden), DT.BFloat16, on_dev), ((1, 1, 1, head_dim), DT.BFloat16, on_dev), ((1, 1, 1, head_dim), DT.BFloat16, on_dev),
+            ((1,), DT.Int32, on_dev, TL.RowMajor), ((users,), DT.Int32, on_dev, TL.RowMajor),
             (cache_shape, DT.BFloat16, True), (cache_shape, DT.BFloat16, True)]
     wshapes = [(hidden,), (hidden, dq), (hidden, dkv), (hidden, dkv), (dq, hidden), (hidden,), (hidden, ffn), (hidden, ffn), (ffn, hidden)]
     wdtypes = [DT.BFloat16, DT.BFP_BFloat8, DT.BFP_BFloat8, DT.BFP_BFloat8, DT.BFP_BFloat8, DT.BFloat16, DT.BFP_BFloat8, DT.BFP_BFloat8,
