@@ -192,6 +192,33 @@ def test_block_float_kernel_configurations(hip, dev, orc, metrics, wfmt_name, op
     check(orc, metrics, got, a, w_eff, b, "gelu", max_abs=2.0 ** -5)
 
 
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4"])
+@pytest.mark.parametrize("split", [0, 1, 3, 5])
+def test_decode_kernel_k_slices(hip, dev, orc, metrics, wfmt_name, split):
+    """M <= 32 path: split-K of the weight-streaming kernel (fp32 partials + reduction with bias and activation), forced
+    to several slice counts and left automatic, on a ragged K with a tail tile and a batch of two."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    M, K, N = 19, 37 * 32 + 11, 5 * 32 + 7
+    a = datagen.randn((2, M, K), seed=41, dtype=torch.bfloat16)
+    w = datagen.randn((2, K, N), seed=42, std=0.05)
+    b = datagen.randn((N,), seed=43, std=0.5, dtype=torch.bfloat16)
+    hip.set_option("linear_decode_split", split)
+    try:
+        got, w_eff = run_linear(hip, dev, a, w, b, "silu", wfmt)
+    finally:
+        hip.set_option("linear_decode_split", 0)
+    for i in range(2):   # the oracle's linear takes one matrix at a time
+        check(orc, metrics, got[i], a[i], w_eff[i], b, "silu", max_abs=2.0 ** -5)
+
+
+def test_decode_kernel_splits_narrow_outputs_by_itself(hip, dev, orc, metrics):
+    """[32, 4096] x bfp4_b [4096, 1024]: 16 column groups on a 256-CU device -> the launcher slices K."""
+    a = datagen.randn((32, 4096), seed=44, dtype=torch.bfloat16)
+    w = datagen.randn((4096, 1024), seed=45, std=0.02)
+    got, w_eff = run_linear(hip, dev, a, w, None, None, hip.BFP4B)
+    check(orc, metrics, got, a, w_eff, None, None, max_abs=2.0 ** -5)
+
+
 def test_split_k_is_chosen_for_long_skinny_reductions(hip, dev, orc, metrics):
     """M = 128, N = 256, K = 8192: one round of blocks would use 2 CUs; the launcher splits K."""
     M, K, N = 128, 8192, 256

@@ -1154,11 +1154,14 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   uint32_t rows[D][8], keeps[D];
   u32x2 ex[D];
   u32x4 af[D][2];
-  const int nchunks = (p.Kt + 7) / 8;
+  // split-K: workgroup y of the grid takes k-tiles [y k_slice, (y + 1) k_slice) and leaves fp32 partial sums
+  const int kbase = p.partial ? (int)blockIdx.y * p.k_slice : 0;
+  const int kend = p.partial ? min(kbase + p.k_slice, p.Kt) : p.Kt;
+  const int nchunks = (kend - kbase + 7) / 8;
   auto load_slot = [&](int s, int c) {
-    const int kt = wave + 8 * c;
-    const int ktc = min(kt, p.Kt - 1);
-    const uint32_t keep = kt < p.Kt ? 0xFFFFFFFFu : 0u;   // past the end: zero exponents, zero weights
+    const int kt = kbase + wave + 8 * c;
+    const int ktc = min(kt, kend - 1);
+    const uint32_t keep = kt < kend ? 0xFFFFFFFFu : 0u;   // past the end: zero exponents, zero weights
     const uint8_t *Wk = W + (int64_t)ktc * p.Nt * TB;
     const uint8_t *Ak = A + (int64_t)ktc * 2048;
 #pragma unroll
@@ -1229,6 +1232,12 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   const int nt = 2 * cg + (kg >> 1);
   if (nt >= p.Nt) return;
   const int n_in = 16 * (kg & 1) + 4 * i;
+  const int64_t off = (int64_t)nt * 1024 + (h * 2 + (n_in >> 4)) * 256 + q16 * 16 + (n_in & 15);
+  if (p.partial) {   // bias, activation and rounding happen in ttm_linear_reduce_k
+    const int64_t per = (int64_t)p.Nt * 1024;
+    *(f32x4v *)(p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * per + off) = sum;
+    return;
+  }
   float bv[4] = {0.f, 0.f, 0.f, 0.f};
   if (p.bias) {
     const uint16_t *bp = p.bias_tiled ? p.bias + (int64_t)nt * 1024 + (n_in >> 4) * 256 + (n_in & 15) : p.bias + nt * 32 + n_in;
@@ -1250,7 +1259,6 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
     v[r] = x;
   }
   u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-  const int64_t off = (int64_t)nt * 1024 + (h * 2 + (n_in >> 4)) * 256 + q16 * 16 + (n_in & 15);
   *(u32x2 *)(C + off * 2) = o;
 }
 
@@ -1305,12 +1313,41 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
     // the small kernel handles one row tile per launch
     LinearArgs p = a;
     const bool decode = BFP && ttm_option("linear_variant") != 1 && (int64_t)a.Nt * 1088 < (int64_t)1 << 32;
+    // the decode kernel has one workgroup per 64 columns: narrow outputs split K until there is one workgroup per CU,
+    // as long as a slice keeps 32 k-tiles (four per wavefront, the depth of its load ring); the slices leave fp32
+    // partial sums that ttm_linear_reduce_k finishes.  Measured at M = 32: [4096, 4096] 14.3 -> 10.6 us,
+    // [14336, 4096] 38 -> 19 us with 4 slices; 8 slices or splitting a [4096, 14336] weight are slower than not splitting.
+    int slices = 1;
+    if (decode) {
+      const int64_t groups = (int64_t)((a.Nt + 1) / 2) * batch;
+      slices = ttm_option("linear_decode_split");
+      if (slices <= 0) {
+        slices = (int)(device_cu_count() / groups);
+        if (slices > a.Kt / 32) slices = a.Kt / 32;
+      }
+      if (slices > a.Kt) slices = a.Kt;
+      if (slices < 1) slices = 1;
+      if (slices > 1) {
+        p.k_slice = (a.Kt + slices - 1) / slices;
+        slices = (a.Kt + p.k_slice - 1) / p.k_slice;
+      }
+    }
+    const int64_t per = (int64_t)a.Nt * 1024;
+    if (slices > 1) {
+      void *ws = nullptr;
+      if (int rc = ttm_stream_workspace(s, (size_t)(per * slices * batch) * sizeof(float), &ws)) return rc;
+      p.partial = (float *)ws;
+      p.Mt = 1;   // the reduction sees one row tile per launch
+    }
     for (int mt = 0; mt < a.Mt; ++mt) {
       p.A = a.A + (int64_t)mt * a.Kt * 2048;
       p.C = a.C + (int64_t)mt * a.Nt * 2048;
-      if (decode && WF == WF_BFP4) hipLaunchKernelGGL(ttm_linear_decode_k<true>, dim3((a.Nt + 1) / 2, 1, (unsigned)batch), dim3(512), 65536, s, p);
-      else if (decode) hipLaunchKernelGGL(ttm_linear_decode_k<false>, dim3((a.Nt + 1) / 2, 1, (unsigned)batch), dim3(512), 65536, s, p);
+      const dim3 grid((a.Nt + 1) / 2, slices, (unsigned)batch);
+      if (decode && WF == WF_BFP4) hipLaunchKernelGGL(ttm_linear_decode_k<true>, grid, dim3(512), 65536, s, p);
+      else if (decode) hipLaunchKernelGGL(ttm_linear_decode_k<false>, grid, dim3(512), 65536, s, p);
       else hipLaunchKernelGGL((ttm_linear_small_k<WF>), dim3(a.Nt, 1, (unsigned)batch), dim3(256), 0, s, p);
+      if (slices > 1)
+        hipLaunchKernelGGL(ttm_linear_reduce_k, dim3((unsigned)((per / 4 + 255) / 256), 1, (unsigned)batch), dim3(256), 0, s, p, slices);
     }
     return 0;
   }
