@@ -6,6 +6,7 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4v __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 
 // 8 consecutive elements <-> 8 floats
 __device__ __forceinline__ void load8(const uint16_t *p, float *v) {
@@ -100,10 +101,11 @@ __global__ __launch_bounds__(256) void ttm_fill_cache_k(u32x4 *__restrict__ cach
 // grid (splits, B * Hkv), 256 threads.  A block owns the G = H / Hkv query heads of one kv head and one slice of the keys:
 //   1. scores = Q K^T with v_mfma_f32_16x16x32_bf16 (queries are the 16 rows, padded with zeros), written to LDS
 //      as (score + mask) * scale, -inf outside the valid keys;
-//   2. softmax numerators and their sum per query head, in place in LDS;
-//   3. P V on the vector ALU: a wave reads half tiles of V (16 keys x 32 columns, 1 KiB contiguous), every lane keeps
-//      8 columns x G heads of partial sums, lanes are combined once per column tile;
-//   4. (max, sum, unnormalised output) go to the split's slot of the workspace; ttm_sdpa_decode_combine_k merges the slots.
+//   2. softmax numerators per query head, rounded to bf16 and stored as pairs of keys 16 apart, and their sum;
+//   3. P V on the vector ALU with v_dot2_f32_bf16: a wave reads the two halves of a V tile (2 x 1 KiB contiguous), every
+//      lane keeps 8 columns x G heads of partial sums, lanes are combined once per column tile;
+//   4. (max, sum, unnormalised output) go to the split's slot of the workspace; ttm_sdpa_decode_combine_k merges the slots
+//      (merging in the last workgroup to arrive was measured: the device-scope fences it needs double the kernel time).
 struct DecodeArgs {
   const uint16_t *q, *k, *v, *mask;
   const int32_t *cur_pos, *page_table;
@@ -114,6 +116,9 @@ struct DecodeArgs {
 };
 
 constexpr int kMaxG = 8;
+#ifndef SPLIT_TARGET
+#define SPLIT_TARGET 512
+#endif
 
 __device__ __forceinline__ const uint16_t *kv_tile_row(const uint16_t *base, const DecodeArgs &p, int b, int hk, int key_tile) {
   // start of the row of tiles holding keys [32 key_tile, 32 key_tile + 32) of (b, hk)
@@ -141,9 +146,10 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
   k1 = k1 < valid ? k1 : valid;
   const int nkeys = k1 > k0 ? k1 - k0 : 0;
   const int ngroups = (nkeys + 15) >> 4;
-  float *sc = lds;                                        // [G][keys_per_split]
+  float *sc = lds;                                        // [G][keys_per_split] scores
   float *osum = lds + (size_t)G * p.keys_per_split;       // [G][D]
   float *stat = osum + (size_t)G * D;                     // [G][2]: max, sum
+  uint32_t *pp = (uint32_t *)(stat + 2 * G);              // [G][keys_per_split / 2] bf16 pairs of softmax numerators
   float *slot = p.part + ((size_t)bh * p.splits + split) * G * (D + 2);
 
   for (int i = tid; i < G * D; i += 256) osum[i] = 0.0f;
@@ -152,8 +158,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
       const int c = i % (D + 2);
       slot[i] = c == D ? -INFINITY : 0.0f;
     }
-    return;
-  }
+  } else {
 
   // ---- 1. scores
   {
@@ -211,19 +216,25 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
   }
   __syncthreads();
 
-  // ---- 2. softmax numerators: wave w serves heads w, w + 4, ...
-  const int padded = ngroups * 16;
+  // ---- 2. softmax numerators: wave w serves heads w, w + 4, ...  The numerators are rounded to bf16 and stored in pairs
+  // (key r, key r + 16 of a 32-key tile) so that the next phase multiplies two keys per instruction; their sum is taken
+  // over the rounded values, which keeps numerator and denominator consistent.
+  const int padded = ngroups * 16, ntiles = (ngroups + 1) >> 1;
   for (int g = wave; g < G; g += 4) {
-    float *row = sc + g * p.keys_per_split;
+    const float *row = sc + g * p.keys_per_split;
+    uint32_t *prow = pp + g * (p.keys_per_split >> 1);
     float m = -INFINITY;
     for (int i = lane; i < padded; i += 64) m = fmaxf(m, row[i]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
     float l = 0.0f;
-    for (int i = lane; i < padded; i += 64) {
-      const float e = (m == -INFINITY) ? 0.0f : __expf(row[i] - m);
-      row[i] = e;
-      l += e;
+    for (int i = lane; i < ntiles * 16; i += 64) {
+      const int klo = (i >> 4) * 32 + (i & 15), khi = klo + 16;
+      const float elo = (m == -INFINITY || klo >= padded) ? 0.0f : __expf(row[klo] - m);
+      const float ehi = (m == -INFINITY || khi >= padded) ? 0.0f : __expf(row[khi] - m);
+      const uint32_t blo = ttm_f32_to_bf16(elo), bhi = ttm_f32_to_bf16(ehi);
+      prow[i] = blo | (bhi << 16);
+      l += __uint_as_float(blo << 16) + __uint_as_float(bhi << 16);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);
@@ -231,47 +242,54 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
   }
   __syncthreads();
 
-  // ---- 3. P V: work items are (column tile, key-group stride class); lane covers key (lane % 32) / 2 of a 16-key group
-  // and columns 16 (lane / 32) + 8 (lane % 2) .. + 7 of the 32-column tile
+  // ---- 3. P V with v_dot2_f32_bf16: work items are (column tile, stride class of key tiles).  Per key tile a lane reads
+  // 8 columns of key r (faces 0 / 1) and of key r + 16 (faces 2 / 3), r = (lane % 32) / 2, columns
+  // 16 (lane / 32) + 8 (lane % 2) .. + 7; the two rows are interleaved to (v[r][d], v[r + 16][d]) pairs and multiplied with
+  // the stored (p[r], p[r + 16]) pair.
   {
     const int share = DT == 1 ? 4 : (DT == 2 ? 2 : 1);   // with one or two column tiles several waves split the keys of one
     const int items = DT * share;
     const int krow = (lane & 31) >> 1;
+    constexpr int UT = 4;                                  // key tiles in flight per pass (8 KiB per wave)
     for (int item = wave; item < items; item += 4) {
-      const int dt = item % DT, kfirst = item / DT;
+      const int dt = item % DT, tfirst = item / DT;
       float o[kMaxG][8];
 #pragma unroll
       for (int g = 0; g < kMaxG; ++g)
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[g][j] = 0.0f;
-      for (int g0 = kfirst; g0 < ngroups; g0 += 4 * share) {
-        // four half tiles of V in flight
-        u32x4 raw[4];
+      for (int t0 = tfirst; t0 < ntiles; t0 += UT * share) {
+        u32x4 ra[UT], rb[UT];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int grp = g0 + u * share < ngroups ? g0 + u * share : g0;
-          const int key = k0 + grp * 16;               // first key of the group; a group never straddles a tile half
-          const uint16_t *vt = kv_tile_row(p.v, p, b, hk, key >> 5) + (int64_t)dt * 1024 + ((key >> 4) & 1) * 512;
-          raw[u] = *(const u32x4 *)(vt + lane * 8);
+        for (int u = 0; u < UT; ++u) {
+          const int t = t0 + u * share < ntiles ? t0 + u * share : t0;
+          const uint16_t *vt = kv_tile_row(p.v, p, b, hk, (k0 >> 5) + t) + (int64_t)dt * 1024;
+          ra[u] = *(const u32x4 *)(vt + lane * 8);
+          rb[u] = *(const u32x4 *)(vt + 512 + lane * 8);
         }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int grp = g0 + u * share;
-          const int kk = grp * 16 + krow;
-          const bool live = grp < ngroups && kk < nkeys;   // rows past the valid keys may hold anything, NaN included
-          const uint32_t w[4] = {raw[u].x, raw[u].y, raw[u].z, raw[u].w};
-          float vv[8];
+        for (int u = 0; u < UT; ++u) {
+          const int t = t0 + u * share;
+          if (t >= ntiles) break;
+          uint32_t a[4] = {ra[u].x, ra[u].y, ra[u].z, ra[u].w}, c[4] = {rb[u].x, rb[u].y, rb[u].z, rb[u].w};
+          if (t * 32 + 32 > nkeys) {   // boundary tile: rows past the valid keys may hold anything, NaN included
+            const bool la = t * 32 + krow < nkeys, lb = t * 32 + 16 + krow < nkeys;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { a[j] = la ? a[j] : 0u; c[j] = lb ? c[j] : 0u; }
+          }
+          uint32_t vp[8];   // vp[2 j] = (a.col 2j, c.col 2j), vp[2 j + 1] = (a.col 2j+1, c.col 2j+1)
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            vv[2 * j] = live ? __uint_as_float(w[j] << 16) : 0.0f;
-            vv[2 * j + 1] = live ? __uint_as_float(w[j] & 0xFFFF0000u) : 0.0f;
+            vp[2 * j] = __builtin_amdgcn_perm(c[j], a[j], 0x05040100u);
+            vp[2 * j + 1] = __builtin_amdgcn_perm(c[j], a[j], 0x07060302u);
           }
 #pragma unroll
           for (int g = 0; g < kMaxG; ++g) {
             if (g < G) {
-              const float pg = live ? sc[g * p.keys_per_split + kk] : 0.0f;
+              const uint32_t pg = pp[g * (p.keys_per_split >> 1) + t * 16 + krow];
 #pragma unroll
-              for (int j = 0; j < 8; ++j) o[g][j] += pg * vv[j];
+              for (int j = 0; j < 8; ++j)
+                o[g][j] = __builtin_amdgcn_fdot2_f32_bf16(*(bf16x2 *)&vp[j], *(const bf16x2 *)&pg, o[g][j], false);
             }
           }
         }
@@ -311,14 +329,16 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
     const int g = i / (D + 2), c = i % (D + 2);
     slot[i] = c < D ? osum[g * D + c] : stat[2 * g + (c - D)];
   }
+  }  // nkeys != 0
 }
 
 // merges the slots of one (b, kv head): out = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M)
 __global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
-  const int bh = blockIdx.x, b = bh / p.Hkv, hk = bh % p.Hkv;
+  const int bh = blockIdx.x, tid0 = threadIdx.x;
+  const int b = bh / p.Hkv, hk = bh % p.Hkv;
   const int G = p.G, D = p.D;
   const float *base = p.part + (size_t)bh * p.splits * G * (D + 2);
-  for (int i = threadIdx.x; i < G * D; i += 256) {
+  for (int i = tid0; i < G * D; i += 256) {
     const int g = i / D, c = i % D;
     float M = -INFINITY;
     for (int s = 0; s < p.splits; ++s) M = fmaxf(M, base[((size_t)s * G + g) * (D + 2) + D]);
@@ -334,7 +354,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
   }
   if (hk == p.Hkv - 1) {   // padding rows of the last head tile
     const int pad = (int)ttm_round_up32(p.H) - p.H;
-    for (int i = threadIdx.x; i < pad * D; i += 256)
+    for (int i = tid0; i < pad * D; i += 256)
       p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(p.H + i / D, i % D, D >> 5)] = 0;
   }
 }
@@ -427,8 +447,8 @@ TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, cons
                 (long long)pages_per_user, (long long)page_block, (long long)seq);
   hipStream_t s = (hipStream_t)stream;
   // enough blocks to fill the device, slices small enough for the score rows to fit in LDS
-  int64_t splits = ttm_cdiv(512, batch * kv_heads);
-  const int64_t max_keys = (48 * 1024 / 4) / G / 32 * 32;
+  int64_t splits = ttm_cdiv(SPLIT_TARGET, batch * kv_heads);
+  const int64_t max_keys = (48 * 1024 / 6) / G / 32 * 32;   // 4 bytes of score + 2 of numerator per key and head
   if (splits > seq / 256) splits = seq / 256 > 0 ? seq / 256 : 1;
   if (ttm_cdiv(seq, splits) > max_keys) splits = ttm_cdiv(seq, max_keys);
   const int64_t keys = ttm_round_up32(ttm_cdiv(seq, splits));
@@ -443,7 +463,7 @@ TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, cons
   void *ws = nullptr;
   if (int rc = ttm_stream_workspace(s, (size_t)(batch * kv_heads * splits * G * (head_dim + 2)) * sizeof(float), &ws)) return rc;
   p.part = (float *)ws;
-  const size_t lds = (size_t)(G * keys + G * head_dim + 2 * G) * sizeof(float);
+  const size_t lds = (size_t)(G * keys + G * head_dim + 2 * G + G * keys / 2) * sizeof(float);
   hipLaunchKernelGGL(ttm_sdpa_decode_k, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
   TTM_LAUNCH_CHECK();
   hipLaunchKernelGGL(ttm_sdpa_decode_combine_k, dim3((unsigned)(batch * kv_heads)), dim3(256), 0, s, p);
