@@ -146,13 +146,14 @@ def test_c3_linear_band(hip, dev, orc, metrics, M):
     a, w, bias = datagen.c3_linear(M)
     got, w_eff = run_linear(hip, dev, a, w, bias, "gelu", hip.BFP8B)
     rows = slice(0, 32) if M == 32 else slice(1000, 1032)
-    cols = slice(7000, 7512)
-    want = orc.round_bf16(orc.linear(a[rows].float().numpy(), w_eff[:, cols].contiguous().numpy(),
-                                     bias[cols].float().numpy(), "gelu"))
-    g = got[rows, cols].float().numpy()
-    # |y| up to ~6 -> bf16 ulp 2^-5; accumulation over K=4096 in a different order adds less than that
-    assert np.max(np.abs(g - want)) <= 2.0 ** -5
-    assert metrics.get_pcc(want, g) >= 0.99
+    # two column bands, one in each round of blocks at M = 2048
+    for cols in (slice(7000, 7512), slice(13900, 14336)):
+        want = orc.round_bf16(orc.linear(a[rows].float().numpy(), w_eff[:, cols].contiguous().numpy(),
+                                         bias[cols].float().numpy(), "gelu"))
+        g = got[rows, cols].float().numpy()
+        # |y| up to ~6 -> bf16 ulp 2^-5; accumulation over K=4096 in a different order adds less than that
+        assert np.max(np.abs(g - want)) <= 2.0 ** -5
+        assert metrics.get_pcc(want, g) >= 0.99
     # quantisation itself against the unquantised weights: the reference's own bar for bfp8 weights
     ref = torch.nn.functional.gelu(a[rows].float() @ w[:, cols] + bias[cols].float())
     assert metrics.get_pcc(ref.numpy(), g) >= 0.99
@@ -217,6 +218,27 @@ def test_decode_kernel_splits_narrow_outputs_by_itself(hip, dev, orc, metrics):
     w = datagen.randn((4096, 1024), seed=45, std=0.02)
     got, w_eff = run_linear(hip, dev, a, w, None, None, hip.BFP4B)
     check(orc, metrics, got, a, w_eff, None, None, max_abs=2.0 ** -5)
+
+
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4"])
+def test_two_part_grid_with_ragged_remainder(hip, dev, orc, metrics, wfmt_name):
+    """The optional two-part grid: 300 column blocks and a bit on a 256-CU device run as one full round of 8-tile-wide
+    blocks plus the remaining 353 column tiles (the last one ragged) in 6-tile-wide blocks of the same launch.  Compared with the single-part grid bit for bit
+    (same per-element accumulation order) and with the oracle on three column bands."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    M, K, N = 200, 96, 300 * 256 + 40
+    a = datagen.randn((M, K), seed=51, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=52, std=0.1)
+    b = datagen.randn((N,), seed=53, std=0.5, dtype=torch.bfloat16)
+    one, w_eff = run_linear(hip, dev, a, w, b, "relu", wfmt)
+    hip.set_option("linear_two_part", 1)
+    try:
+        got, _ = run_linear(hip, dev, a, w, b, "relu", wfmt)
+    finally:
+        hip.set_option("linear_two_part", 0)
+    assert torch.equal(got, one)
+    for cols in (slice(0, 512), slice(65536 - 256, 65536 + 256), slice(N - 300, N)):
+        check(orc, metrics, got[:, cols], a, w_eff[:, cols].contiguous(), b[cols], "relu", max_abs=2.0 ** -5)
 
 
 def test_split_k_is_chosen_for_long_skinny_reductions(hip, dev, orc, metrics):

@@ -41,6 +41,8 @@ struct LinearArgs {
   int64_t a_batch, w_batch, c_batch;  // byte strides between batch entries (w_batch 0 = shared weights)
   int m_blocks, n_blocks;
   int ntw;                            // block-float main kernel: column tiles per wavefront (block width / 2)
+  int nt_split, n_blocks1, ntw2;      // two-part grid: blocks [0, n_blocks1) cover column tiles [0, nt_split) at width ntw,
+                                      // the rest cover [nt_split, Nt) at width ntw2; nt_split = 0: one part
   int k_slice;                        // k-tiles per grid.y slice (split-K); Kt when the reduction is not split
   float *partial;                     // split-K: fp32 partial sums [slices][Mt * Nt * 1024] in output tile order
 };
@@ -974,9 +976,14 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
 
 template <int WF>
 __global__ __launch_bounds__(512) void ttm_linear_dma_k(LinearArgs p) {
-  if (p.ntw == 4) linear_dma_block<WF, 4>(p, blockIdx.x, gridDim.x, 0, p.Nt);
-  else if (p.ntw == 3) linear_dma_block<WF, 3>(p, blockIdx.x, gridDim.x, 0, p.Nt);
-  else linear_dma_block<WF, 2>(p, blockIdx.x, gridDim.x, 0, p.Nt);
+  int bid = blockIdx.x, nblk = gridDim.x, first = 0, end = p.Nt, ntw = p.ntw;
+  if (p.nt_split > 0) {   // workgroup-uniform
+    if (bid < p.n_blocks1) { nblk = p.n_blocks1; end = p.nt_split; }
+    else { bid -= p.n_blocks1; nblk -= p.n_blocks1; first = p.nt_split; ntw = p.ntw2; }
+  }
+  if (ntw == 4) linear_dma_block<WF, 4>(p, bid, nblk, first, end);
+  else if (ntw == 3) linear_dma_block<WF, 3>(p, bid, nblk, first, end);
+  else linear_dma_block<WF, 2>(p, bid, nblk, first, end);
 }
 
 // =============================================================================================
@@ -1277,7 +1284,7 @@ static int device_cu_count() {
 // (the 12 stand for prologue and epilogue), 0.92 / 0.78 of that at 6 / 4 tiles (a narrower block keeps the whole
 // activation traffic of a wide one); blocks run in rounds of one per CU; a split reduction adds its fp32 partial
 // traffic, (slices + 0.5) x M x N x 4 bytes, at 4 TB/s.  force_* != 0 pin a choice (tests, measurements).
-static int plan_dma_grid(LinearArgs &p, int cus, int force_ntw, int force_slices) {
+static int plan_dma_grid(LinearArgs &p, int cus, int force_ntw, int force_slices, int two_part = 0) {
   const int mbk = p.m_blocks, ksteps = (p.Kt + 1) / 2;
   static const double width_cost[5] = {0, 0, 0.78, 0.92, 1.0};
   double best = 1e30;
@@ -1296,6 +1303,32 @@ static int plan_dma_grid(LinearArgs &p, int cus, int force_ntw, int force_slices
   if (force_slices) best_slices = force_slices;
   p.ntw = best_ntw;
   p.n_blocks = mbk * ((p.Nt + 2 * best_ntw - 1) / (2 * best_ntw));   // blocks per k-slice
+  p.nt_split = 0;
+  // Optional (linear_two_part = 1): unsplit, full-width grids whose last round is partly filled keep the full rounds at
+  // 8 tiles and cover the remaining columns with narrower blocks when the model says those cost fewer CU-rounds.
+  // [2048, 4096] x [4096, 14336]: 256 blocks of 8 tiles + 256 blocks of 6 tiles instead of 448 of 8 - modelled 1.92
+  // rounds instead of 2, measured 262 us instead of 250, so it is off unless asked for.
+  if (best_slices == 1 && best_ntw == 4 && !force_ntw && two_part != 0) {
+    const int full_rounds = p.n_blocks / cus;
+    const int cols1 = full_rounds * cus / mbk;            // column blocks (8 tiles) the full rounds cover
+    const int rem = p.Nt - 8 * cols1;                      // column tiles left
+    if (full_rounds >= 1 && rem > 0 && p.n_blocks % cus != 0) {
+      const double step = (ksteps + 12) * 1.65;
+      double t_one = ((p.n_blocks + cus - 1) / cus) * step, t_best = t_one;
+      int pick = 0;
+      for (int ntw2 = 3; ntw2 >= 2; --ntw2) {
+        const int blocks2 = mbk * ((rem + 2 * ntw2 - 1) / (2 * ntw2));
+        const double t = full_rounds * step + ((blocks2 + cus - 1) / cus) * width_cost[ntw2] * step;
+        if (t < t_best * 0.99) { t_best = t; pick = ntw2; }
+      }
+      if (pick) {
+        p.nt_split = 8 * cols1;
+        p.n_blocks1 = mbk * cols1;
+        p.ntw2 = pick;
+        p.n_blocks = p.n_blocks1 + mbk * ((rem + 2 * pick - 1) / (2 * pick));
+      }
+    }
+  }
   return best_slices;
 }
 
@@ -1369,7 +1402,7 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       }
       LinearArgs p = a;
       const int cus = device_cu_count();
-      int slices = plan_dma_grid(p, cus, ttm_option("linear_ntw"), ttm_option("linear_split_k"));
+      int slices = plan_dma_grid(p, cus, ttm_option("linear_ntw"), ttm_option("linear_split_k"), ttm_option("linear_two_part") == 1);
       slices = slices < 1 ? 1 : (slices > a.Kt ? a.Kt : slices);
       if (slices > 1) {
         p.k_slice = (a.Kt + slices - 1) / slices;
@@ -1436,6 +1469,7 @@ TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype
   p.m_blocks = (p.Mt + 7) / 8; p.n_blocks = (p.Nt + 7) / 8;
   p.ntw = 4;
   p.k_slice = p.Kt; p.partial = nullptr;
+  p.nt_split = p.n_blocks1 = p.ntw2 = 0;
   TTM_REQUIRE(batch <= 65535, "ttm_linear: batch too large");
   hipStream_t s = (hipStream_t)stream;
   int rc;
