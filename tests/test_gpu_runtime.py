@@ -513,6 +513,44 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
     assert np.array_equal(gk[:, :, untouched], f(kc0)[:, :, untouched]) and np.array_equal(gv[:, :, untouched], f(vc0)[:, :, untouched])
 
 
+@pytest.mark.parametrize("shape,mid,perm,final", [
+    ((2, 40, 96), (2, 40, 3, 32), (0, 2, 1, 3), (6, 40, 32)),          # reshape -> permute -> reshape, ragged rows
+    ((1, 64, 256), (1, 64, 4, 64), (0, 2, 1, 3), (1, 4, 64, 64)),      # head split as in the decoder layer
+    ((4, 33, 64), (4, 33, 2, 32), (2, 0, 1, 3), (8, 33, 32)),
+])
+def test_reshape_permute_pairs_are_fused_without_changing_results(device, shape, mid, perm, final):
+    """Adjacent reshape / permute pairs run as one strided copy when no callback is registered; with a callback every
+    operation materialises its own output.  Both must equal torch's reshape / permute bit for bit."""
+    pb = rt.ProgramBuilder()
+    pb.begin_program("views")
+    x = pb.input(shape, DT.BFloat16)
+    y = pb.reshape(pb.permute(pb.reshape(x, mid), perm), final)
+    z = pb.permute(pb.reshape(x, mid), perm)            # same head, second consumer of x: fused as well
+    pb.output(y)
+    pb.output(z)
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    xin = torch.randn(shape).to(torch.bfloat16)
+    want_z = xin.reshape(mid).permute(perm).contiguous()
+    want_y = want_z.reshape(final)
+    rt.clear_stats()
+    y0, z0 = harness.execute(binary, 0, [xin], device)
+    fused_copies = rt.get_stat("CopyViewLaunch")
+    seen = []
+    rt.set_post_op_callback(lambda idx, name, dbg, hook: seen.append(name))
+    try:
+        y1, z1 = harness.execute(binary, 0, [xin], device)
+    finally:
+        rt.clear_callbacks()
+    assert seen == ["ReshapeOp", "PermuteOp", "ReshapeOp", "ReshapeOp", "PermuteOp"]
+    for got in (y0, y1):
+        assert torch.equal(got, want_y)
+    for got in (z0, z1):
+        assert torch.equal(got, want_z)
+    unfused_copies = rt.get_stat("CopyViewLaunch") - fused_copies
+    assert fused_copies < unfused_copies, (fused_copies, unfused_copies)
+
+
 def test_submit_errors(device):
     binary = rt.Binary.load_from_memory(programs.c3_linear(32, 64, 64))
     a = rt.from_torch(torch.zeros(32, 64, dtype=torch.bfloat16))

@@ -4,6 +4,7 @@
 // flatbuffer op table (runtime/lib/ttnn/operations/**).  Ops outside the supported subset fail with
 // the op name, like the reference's LOG_FATAL("Unsupported operation type").
 #include <algorithm>
+#include <set>
 #include <cmath>
 #include <cstring>
 #include <map>
@@ -26,6 +27,19 @@ struct ProgramContext {
   Binary binary;
   std::uint32_t programIndex = 0;
   std::unordered_map<std::uint32_t, Tensor> pool;  // global_id -> live tensor
+  // reshape / permute fusion (only when no hooks are registered): a reshape whose single consumer is the next permute is
+  // not materialised (`deferred` keeps its source and logical shape), and a permute whose single consumer is the next
+  // reshape writes the reshaped tensor directly (the reshape's index goes into `skip`)
+  struct DeferredView {
+    Tensor source;
+    std::vector<std::uint32_t> shape;
+  };
+  std::vector<fb::Table> ops;
+  std::uint32_t opIndex = 0;
+  bool fuseViews = false;
+  std::unordered_map<std::uint32_t, int> uses;      // consumers of a tensor (deallocations not counted; program outputs are)
+  std::unordered_map<std::uint32_t, DeferredView> deferred;
+  std::set<std::uint32_t> skip;
 
   Tensor &get(const fb::Table &ref, const char *what) {
     TTRT_ASSERT(static_cast<bool>(ref), std::string("missing tensor reference: ") + what);
@@ -41,6 +55,95 @@ struct ProgramContext {
   }
   void *stream() const { return dev->stream; }
 };
+
+// Tensor operands of an operation as the flatbuffer names them: `ins` in operand order (absent optional operands are
+// skipped), `outs` in result order.  Ops outside the supported subset report nothing.
+struct OpRefs {
+  std::vector<fb::Table> ins, outs;
+};
+
+OpRefs opRefs(const fb::Table &operation) {
+  auto type = static_cast<OpType>(operation.scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
+  fb::Table op = operation.table(schema::Operation::f_type);
+  OpRefs r;
+  auto in = [&](int slot) { if (fb::Table t = op.table(slot)) r.ins.push_back(t); };
+  auto out = [&](int slot) { if (fb::Table t = op.table(slot)) r.outs.push_back(t); };
+  auto inVec = [&](int slot) {
+    auto v = op.tables(slot);
+    for (std::uint32_t i = 0; i < v.size(); ++i) r.ins.push_back(v[i]);
+  };
+  auto outVec = [&](int slot) {
+    auto v = op.tables(slot);
+    for (std::uint32_t i = 0; i < v.size(); ++i) r.outs.push_back(v[i]);
+  };
+  switch (type) {
+  case OpType::ToLayoutOp: in(schema::ToLayoutOp::f_in); out(schema::ToLayoutOp::f_out); break;
+  case OpType::TypecastOp: in(schema::TypecastOp::f_in); out(schema::TypecastOp::f_out); break;
+  case OpType::ToDeviceOp: in(schema::ToDeviceOp::f_in); out(schema::ToDeviceOp::f_out); break;
+  case OpType::FromDeviceOp: in(schema::FromDeviceOp::f_in); out(schema::FromDeviceOp::f_out); break;
+  case OpType::ToMemoryConfigOp: in(schema::ToMemoryConfigOp::f_in0); out(schema::ToMemoryConfigOp::f_out); break;
+  case OpType::MatmulOp: in(schema::MatmulOp::f_a); in(schema::MatmulOp::f_b); out(schema::MatmulOp::f_out); break;
+  case OpType::LinearOp:
+    in(schema::LinearOp::f_a); in(schema::LinearOp::f_b); in(schema::LinearOp::f_bias); out(schema::LinearOp::f_out);
+    break;
+  case OpType::EltwiseUnaryOp: in(schema::EltwiseUnaryOp::f_in); out(schema::EltwiseUnaryOp::f_out); break;
+  case OpType::EltwiseBinaryOp:
+    in(schema::EltwiseBinaryOp::f_lhs); in(schema::EltwiseBinaryOp::f_rhs); out(schema::EltwiseBinaryOp::f_out);
+    break;
+  case OpType::RMSNormOp:
+    in(schema::RMSNormOp::f_input); in(schema::RMSNormOp::f_weight); in(schema::RMSNormOp::f_bias); out(schema::RMSNormOp::f_out);
+    break;
+  case OpType::SoftmaxOp: in(schema::SoftmaxOp::f_in); out(schema::SoftmaxOp::f_out); break;
+  case OpType::ReductionOp: in(schema::ReductionOp::f_in); out(schema::ReductionOp::f_out); break;
+  case OpType::ScaledDotProductAttentionOp:
+    in(schema::ScaledDotProductAttentionOp::f_query); in(schema::ScaledDotProductAttentionOp::f_key);
+    in(schema::ScaledDotProductAttentionOp::f_value); in(schema::ScaledDotProductAttentionOp::f_attention_mask);
+    out(schema::ScaledDotProductAttentionOp::f_out);
+    break;
+  case OpType::ReshapeOp: in(schema::ReshapeOp::f_in); out(schema::ReshapeOp::f_out); break;
+  case OpType::PermuteOp: in(schema::PermuteOp::f_in); out(schema::PermuteOp::f_out); break;
+  case OpType::TransposeOp: in(schema::TransposeOp::f_in); out(schema::TransposeOp::f_out); break;
+  case OpType::ConcatOp: inVec(schema::ConcatOp::f_inputs); out(schema::ConcatOp::f_out); break;
+  case OpType::SliceOp: in(schema::SliceOp::f_in); out(schema::SliceOp::f_out); break;
+  case OpType::RepeatInterleaveOp: in(schema::RepeatInterleaveOp::f_input); out(schema::RepeatInterleaveOp::f_out); break;
+  case OpType::ConstantOp: out(schema::ConstantOp::f_out); break;
+  case OpType::FullOp: out(schema::FullOp::f_out); break;
+  case OpType::NamedFullOp: out(schema::NamedFullOp::f_out); break;
+  case OpType::EmptyOp: out(schema::EmptyOp::f_out); break;
+  case OpType::DeallocateOp: in(schema::DeallocateOp::f_in); break;
+  case OpType::LoadCachedOp: inVec(schema::LoadCachedOp::f_inputs); outVec(schema::LoadCachedOp::f_outputs); break;
+  case OpType::FuncCallOp: inVec(schema::FuncCallOp::f_inputs); outVec(schema::FuncCallOp::f_outputs); break;
+  case OpType::RotaryEmbeddingOp:
+    in(schema::RotaryEmbeddingOp::f_input); in(schema::RotaryEmbeddingOp::f_cos_cache); in(schema::RotaryEmbeddingOp::f_sin_cache);
+    out(schema::RotaryEmbeddingOp::f_out);
+    break;
+  case OpType::UpdateCacheOp:
+    in(schema::UpdateCacheOp::f_cache); in(schema::UpdateCacheOp::f_input); in(schema::UpdateCacheOp::f_update_index);
+    break;
+  case OpType::FillCacheOp: in(schema::FillCacheOp::f_cache); in(schema::FillCacheOp::f_input); break;
+  case OpType::ScaledDotProductAttentionDecodeOp: {
+    using S = schema::ScaledDotProductAttentionDecodeOp;
+    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
+    break;
+  }
+  case OpType::PagedScaledDotProductAttentionDecodeOp: {
+    using S = schema::PagedScaledDotProductAttentionDecodeOp;
+    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_page_table); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
+    break;
+  }
+  case OpType::CaptureOrExecuteTraceOp:
+    inVec(schema::CaptureOrExecuteTraceOp::f_inputs); outVec(schema::CaptureOrExecuteTraceOp::f_outputs);
+    break;
+  case OpType::WriteTensorOp: in(schema::WriteTensorOp::f_host_tensor); in(schema::WriteTensorOp::f_device_tensor); break;
+  case OpType::CopyOp: in(schema::CopyOp::f_src); in(schema::CopyOp::f_dst); break;
+  case OpType::BeginTraceCaptureOp: out(schema::BeginTraceCaptureOp::f_trace_id); break;
+  case OpType::EndTraceCaptureOp: in(schema::EndTraceCaptureOp::f_trace_id); break;
+  case OpType::ExecuteTraceOp: in(schema::ExecuteTraceOp::f_trace_id); break;
+  default: break;
+  }
+  return r;
+}
+
 
 // ---- helpers
 Tensor onDevice(ProgramContext &ctx, const Tensor &t) { return t.handle->storage == StorageType::Device ? t : toDevice(t, ctx.dev); }
@@ -83,6 +186,7 @@ void copyView(ProgramContext &ctx, const Tensor &src, const Tensor &dst, const s
   std::vector<std::int64_t> e = extent, ss = sstride, ds = dstride;
   TTRT_ASSERT(e.size() <= 8, "copyView: rank above 8");
   Dims3 sd = dims3(src.handle->shape), dd = dims3(dst.handle->shape);
+  debug::Stats::get().incrementStat("CopyViewLaunch");
   TTM_CALL(ttm_copy_view(src.handle->data.get(), sd.rows, sd.cols, ttmLayout(src.handle->layout), dst.handle->data.get(), dd.rows,
                          dd.cols, ttmLayout(dst.handle->layout), static_cast<int>(utils::dataTypeElementSize(src.handle->dtype)),
                          static_cast<int>(e.size()), e.data(), ss.data(), sbase, ds.data(), dbase, ctx.stream()));
@@ -526,14 +630,44 @@ Tensor reshapeTo(ProgramContext &ctx, const Tensor &in, const std::vector<std::u
   return out;
 }
 
+std::uint32_t refId(const fb::Table &ref) { return ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0); }
+
+// the operation after the current one, if it is of `type`, consumes `produced` as its first operand, and is the only
+// consumer of it; its output must keep the producer's layout so that no conversion hides between the two
+fb::Table fusableNext(ProgramContext &ctx, OpType type, int inSlot, int outSlot, const fb::Table &produced, const Tensor &like) {
+  if (!ctx.fuseViews || ctx.opIndex + 1 >= ctx.ops.size()) return fb::Table();
+  const fb::Table &next = ctx.ops[ctx.opIndex + 1];
+  if (static_cast<OpType>(next.scalar<std::uint8_t>(schema::Operation::f_type_type, 0)) != type) return fb::Table();
+  fb::Table nop = next.table(schema::Operation::f_type);
+  fb::Table in = nop.table(inSlot), out = nop.table(outSlot);
+  if (!in || !out || refId(in) != refId(produced)) return fb::Table();
+  auto u = ctx.uses.find(refId(produced));
+  if (u == ctx.uses.end() || u->second != 1) return fb::Table();
+  Layout a = layoutFromTensorRef(produced), b = layoutFromTensorRef(out);
+  if (!(a == b) || a.storageType != StorageType::Device || a.layout != like.handle->layout || a.dataType != like.handle->dtype)
+    return fb::Table();
+  return nop;
+}
+
 void runReshape(const fb::Table &op, ProgramContext &ctx) {
   Tensor in = onDevice(ctx, ctx.get(op.table(schema::ReshapeOp::f_in), "reshape in"));
   auto outRef = op.table(schema::ReshapeOp::f_out);
-  ctx.put(outRef, finish(ctx, reshapeTo(ctx, in, shapeFromTensorRef(outRef)), outRef));
+  std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
+  const bool copies = in.handle->layout == TensorLayout::Tile && !sameTiling(in.handle->shape, oshape);
+  if (copies && !utils::isBlockFormatDataType(in.handle->dtype) &&
+      fusableNext(ctx, OpType::PermuteOp, schema::PermuteOp::f_in, schema::PermuteOp::f_out, outRef, in)) {
+    TTRT_ASSERT(volume(in.handle->shape) == volume(oshape), "reshape: element count differs");
+    ctx.deferred[refId(outRef)] = ProgramContext::DeferredView{in, oshape};   // the permute reads the source directly
+    return;
+  }
+  ctx.put(outRef, finish(ctx, reshapeTo(ctx, in, oshape), outRef));
 }
 
-Tensor permuteTo(ProgramContext &ctx, const Tensor &in, const std::vector<int> &perm) {
-  const auto &shape = in.handle->shape;
+// out[i0, i1, ...] = in[i_perm...]; `viewShape` reinterprets the input's elements under another logical shape first (a
+// reshape is the identity on flat indices), `finalShape` gives the output another logical shape of the same volume
+Tensor permuteTo(ProgramContext &ctx, const Tensor &in, const std::vector<int> &perm, const std::vector<std::uint32_t> *viewShape = nullptr,
+                 const std::vector<std::uint32_t> *finalShape = nullptr) {
+  const auto &shape = viewShape ? *viewShape : in.handle->shape;
   const size_t rank = shape.size();
   TTRT_ASSERT(perm.size() == rank, "permute: permutation rank differs from the tensor rank");
   std::vector<std::uint32_t> oshape(rank);
@@ -544,18 +678,39 @@ Tensor permuteTo(ProgramContext &ctx, const Tensor &in, const std::vector<int> &
     oshape[i] = shape[perm[i]];
     sst[i] = ss[perm[i]];
   }
-  Tensor out = makeDeviceTensor(ctx.dev, oshape, in.handle->dtype, in.handle->layout);
+  if (finalShape) TTRT_ASSERT(volume(*finalShape) == volume(oshape), "reshape: element count differs");
+  Tensor out = makeDeviceTensor(ctx.dev, finalShape ? *finalShape : oshape, in.handle->dtype, in.handle->layout);
   zeroIfPadded(ctx, out);
   copyView(ctx, in, out, toI64(oshape), sst, 0, rowMajorStrides(oshape), 0);
   return out;
 }
 void runPermute(const fb::Table &op, ProgramContext &ctx) {
-  Tensor in = onDevice(ctx, ctx.get(op.table(schema::PermuteOp::f_in), "permute in"));
+  auto inRef = op.table(schema::PermuteOp::f_in);
   auto pv = op.scalars<std::int64_t>(schema::PermuteOp::f_permutation);
   std::vector<int> perm;
   for (std::uint32_t i = 0; i < pv.size(); ++i) perm.push_back(static_cast<int>(pv[i] < 0 ? pv[i] + pv.size() : pv[i]));
   auto outRef = op.table(schema::PermuteOp::f_out);
-  ctx.put(outRef, finish(ctx, permuteTo(ctx, in, perm), outRef));
+  Tensor in;
+  std::vector<std::uint32_t> viewShape;
+  auto d = ctx.deferred.find(refId(inRef));
+  if (d != ctx.deferred.end()) {
+    in = d->second.source;
+    viewShape = d->second.shape;
+    ctx.deferred.erase(d);
+  } else {
+    in = onDevice(ctx, ctx.get(inRef, "permute in"));
+  }
+  const std::vector<std::uint32_t> *view = viewShape.empty() ? nullptr : &viewShape;
+  if (in.handle->layout == TensorLayout::Tile && !utils::isBlockFormatDataType(in.handle->dtype)) {
+    if (fb::Table rs = fusableNext(ctx, OpType::ReshapeOp, schema::ReshapeOp::f_in, schema::ReshapeOp::f_out, outRef, in)) {
+      auto finalRef = rs.table(schema::ReshapeOp::f_out);
+      std::vector<std::uint32_t> finalShape = shapeFromTensorRef(finalRef);
+      ctx.put(finalRef, permuteTo(ctx, in, perm, view, &finalShape));
+      ctx.skip.insert(ctx.opIndex + 1);
+      return;
+    }
+  }
+  ctx.put(outRef, finish(ctx, permuteTo(ctx, in, perm, view), outRef));
 }
 void runTranspose(const fb::Table &op, ProgramContext &ctx) {
   Tensor in = onDevice(ctx, ctx.get(op.table(schema::TransposeOp::f_in), "transpose in"));
@@ -939,9 +1094,22 @@ std::vector<Tensor> executeProgram(const std::shared_ptr<DeviceState> &dev, cons
   }
   auto ops = program.tables(schema::Program::f_operations);
   auto &hooks = debug::Hooks::get();
+  // with callbacks registered every operation must leave its own output in the pool: no fusion then
+  ctx.fuseViews = !hooks.preOperatorCallback && !hooks.postOperatorCallback;
+  if (ctx.fuseViews) {
+    for (std::uint32_t i = 0; i < ops.size(); ++i) {
+      ctx.ops.push_back(ops[i]);
+      if (static_cast<OpType>(ops[i].scalar<std::uint8_t>(schema::Operation::f_type_type, 0)) == OpType::DeallocateOp) continue;
+      for (const auto &ref : opRefs(ops[i]).ins) ++ctx.uses[refId(ref)];
+    }
+    auto pouts = program.tables(schema::Program::f_outputs);
+    for (std::uint32_t i = 0; i < pouts.size(); ++i) ++ctx.uses[refId(pouts[i])];
+  }
   CallbackContext cc{&ctx};
   if (hooks.preProgramCallback) (*hooks.preProgramCallback)(binary, cc);
   for (std::uint32_t i = 0; i < ops.size(); ++i) {
+    if (ctx.skip.count(i)) continue;   // folded into the operation before it
+    ctx.opIndex = i;
     OpContext oc{ops[i], i};
     if (hooks.preOperatorCallback) (*hooks.preOperatorCallback)(binary, cc, oc);
     runOperation(ops[i], ctx);
@@ -956,94 +1124,6 @@ std::vector<Tensor> executeProgram(const std::shared_ptr<DeviceState> &dev, cons
 
 // ---- hook-side access to the running program (runtime/include/tt/runtime/runtime.h:246-297)
 namespace {
-// Tensor operands of an operation as the flatbuffer names them: `ins` in operand order (absent optional operands are
-// skipped), `outs` in result order.  Ops outside the supported subset report nothing.
-struct OpRefs {
-  std::vector<fb::Table> ins, outs;
-};
-
-OpRefs opRefs(const fb::Table &operation) {
-  auto type = static_cast<OpType>(operation.scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
-  fb::Table op = operation.table(schema::Operation::f_type);
-  OpRefs r;
-  auto in = [&](int slot) { if (fb::Table t = op.table(slot)) r.ins.push_back(t); };
-  auto out = [&](int slot) { if (fb::Table t = op.table(slot)) r.outs.push_back(t); };
-  auto inVec = [&](int slot) {
-    auto v = op.tables(slot);
-    for (std::uint32_t i = 0; i < v.size(); ++i) r.ins.push_back(v[i]);
-  };
-  auto outVec = [&](int slot) {
-    auto v = op.tables(slot);
-    for (std::uint32_t i = 0; i < v.size(); ++i) r.outs.push_back(v[i]);
-  };
-  switch (type) {
-  case OpType::ToLayoutOp: in(schema::ToLayoutOp::f_in); out(schema::ToLayoutOp::f_out); break;
-  case OpType::TypecastOp: in(schema::TypecastOp::f_in); out(schema::TypecastOp::f_out); break;
-  case OpType::ToDeviceOp: in(schema::ToDeviceOp::f_in); out(schema::ToDeviceOp::f_out); break;
-  case OpType::FromDeviceOp: in(schema::FromDeviceOp::f_in); out(schema::FromDeviceOp::f_out); break;
-  case OpType::ToMemoryConfigOp: in(schema::ToMemoryConfigOp::f_in0); out(schema::ToMemoryConfigOp::f_out); break;
-  case OpType::MatmulOp: in(schema::MatmulOp::f_a); in(schema::MatmulOp::f_b); out(schema::MatmulOp::f_out); break;
-  case OpType::LinearOp:
-    in(schema::LinearOp::f_a); in(schema::LinearOp::f_b); in(schema::LinearOp::f_bias); out(schema::LinearOp::f_out);
-    break;
-  case OpType::EltwiseUnaryOp: in(schema::EltwiseUnaryOp::f_in); out(schema::EltwiseUnaryOp::f_out); break;
-  case OpType::EltwiseBinaryOp:
-    in(schema::EltwiseBinaryOp::f_lhs); in(schema::EltwiseBinaryOp::f_rhs); out(schema::EltwiseBinaryOp::f_out);
-    break;
-  case OpType::RMSNormOp:
-    in(schema::RMSNormOp::f_input); in(schema::RMSNormOp::f_weight); in(schema::RMSNormOp::f_bias); out(schema::RMSNormOp::f_out);
-    break;
-  case OpType::SoftmaxOp: in(schema::SoftmaxOp::f_in); out(schema::SoftmaxOp::f_out); break;
-  case OpType::ReductionOp: in(schema::ReductionOp::f_in); out(schema::ReductionOp::f_out); break;
-  case OpType::ScaledDotProductAttentionOp:
-    in(schema::ScaledDotProductAttentionOp::f_query); in(schema::ScaledDotProductAttentionOp::f_key);
-    in(schema::ScaledDotProductAttentionOp::f_value); in(schema::ScaledDotProductAttentionOp::f_attention_mask);
-    out(schema::ScaledDotProductAttentionOp::f_out);
-    break;
-  case OpType::ReshapeOp: in(schema::ReshapeOp::f_in); out(schema::ReshapeOp::f_out); break;
-  case OpType::PermuteOp: in(schema::PermuteOp::f_in); out(schema::PermuteOp::f_out); break;
-  case OpType::TransposeOp: in(schema::TransposeOp::f_in); out(schema::TransposeOp::f_out); break;
-  case OpType::ConcatOp: inVec(schema::ConcatOp::f_inputs); out(schema::ConcatOp::f_out); break;
-  case OpType::SliceOp: in(schema::SliceOp::f_in); out(schema::SliceOp::f_out); break;
-  case OpType::RepeatInterleaveOp: in(schema::RepeatInterleaveOp::f_input); out(schema::RepeatInterleaveOp::f_out); break;
-  case OpType::ConstantOp: out(schema::ConstantOp::f_out); break;
-  case OpType::FullOp: out(schema::FullOp::f_out); break;
-  case OpType::NamedFullOp: out(schema::NamedFullOp::f_out); break;
-  case OpType::EmptyOp: out(schema::EmptyOp::f_out); break;
-  case OpType::DeallocateOp: in(schema::DeallocateOp::f_in); break;
-  case OpType::LoadCachedOp: inVec(schema::LoadCachedOp::f_inputs); outVec(schema::LoadCachedOp::f_outputs); break;
-  case OpType::FuncCallOp: inVec(schema::FuncCallOp::f_inputs); outVec(schema::FuncCallOp::f_outputs); break;
-  case OpType::RotaryEmbeddingOp:
-    in(schema::RotaryEmbeddingOp::f_input); in(schema::RotaryEmbeddingOp::f_cos_cache); in(schema::RotaryEmbeddingOp::f_sin_cache);
-    out(schema::RotaryEmbeddingOp::f_out);
-    break;
-  case OpType::UpdateCacheOp:
-    in(schema::UpdateCacheOp::f_cache); in(schema::UpdateCacheOp::f_input); in(schema::UpdateCacheOp::f_update_index);
-    break;
-  case OpType::FillCacheOp: in(schema::FillCacheOp::f_cache); in(schema::FillCacheOp::f_input); break;
-  case OpType::ScaledDotProductAttentionDecodeOp: {
-    using S = schema::ScaledDotProductAttentionDecodeOp;
-    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
-    break;
-  }
-  case OpType::PagedScaledDotProductAttentionDecodeOp: {
-    using S = schema::PagedScaledDotProductAttentionDecodeOp;
-    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_page_table); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
-    break;
-  }
-  case OpType::CaptureOrExecuteTraceOp:
-    inVec(schema::CaptureOrExecuteTraceOp::f_inputs); outVec(schema::CaptureOrExecuteTraceOp::f_outputs);
-    break;
-  case OpType::WriteTensorOp: in(schema::WriteTensorOp::f_host_tensor); in(schema::WriteTensorOp::f_device_tensor); break;
-  case OpType::CopyOp: in(schema::CopyOp::f_src); in(schema::CopyOp::f_dst); break;
-  case OpType::BeginTraceCaptureOp: out(schema::BeginTraceCaptureOp::f_trace_id); break;
-  case OpType::EndTraceCaptureOp: in(schema::EndTraceCaptureOp::f_trace_id); break;
-  case OpType::ExecuteTraceOp: in(schema::ExecuteTraceOp::f_trace_id); break;
-  default: break;
-  }
-  return r;
-}
-
 std::vector<TensorRef> wrapRefs(const std::vector<fb::Table> &tables) {
   std::vector<TensorRef> out;
   for (const auto &t : tables) out.push_back(TensorRef{t});
