@@ -240,8 +240,16 @@ def test_copy_view_reshape_permute_slice_concat(hip, dev, orc):
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,mask", [
     (1, 4, 2, 128, 128, 64, True, None), (2, 2, 2, 96, 160, 128, False, None), (1, 8, 2, 256, 256, 128, True, None),
     (1, 2, 1, 70, 70, 32, True, None), (1, 2, 2, 64, 100, 64, False, "b1"), (2, 2, 1, 64, 64, 64, False, "bh"),
-    (1, 1, 1, 40, 300, 256, False, None)])
-def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask):
+    (1, 1, 1, 40, 300, 256, False, None),
+    # odd and ragged key-tile counts for the 64-keys-per-pass kernel, masks on its second half, causal with Sq != Sk
+    (1, 2, 2, 160, 96, 128, False, None), (1, 4, 1, 33, 33, 128, True, None), (1, 2, 2, 96, 224, 64, False, "bh"),
+    (2, 4, 4, 130, 190, 128, False, "b1"), (1, 4, 2, 192, 320, 128, True, None), (1, 2, 1, 320, 192, 32, True, None),
+    (1, 8, 2, 1024, 1024, 128, True, None)])
+@pytest.mark.parametrize("variant", [0, 1])
+def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask, variant):
+    if variant == 1 and Sq * Sk >= 512 * 512:
+        pytest.skip("the 32-key kernel is covered by the small shapes")
+    hip.set_option("sdpa_variant", variant)
     import oracle.metrics as metrics
     q = datagen.randn((B, Hq, Sq, D), seed=12, dtype=torch.bfloat16)
     k = datagen.randn((B, Hkv, Sk, D), seed=13, dtype=torch.bfloat16)
@@ -252,9 +260,12 @@ def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask):
     qt, kt, vt = (tilize_dev(hip, t, dev) for t in (q, k, v))
     mt = tilize_dev(hip, m, dev) if m is not None else None
     out = torch.full_like(qt, float("nan"))
-    hip.call("ttm_sdpa", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(mt) if mt is not None else None,
-             m.shape[1] if m is not None else 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, Sq, Sk, D, int(causal), 0.0,
-             hip.current_stream())
+    try:
+        hip.call("ttm_sdpa", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(mt) if mt is not None else None,
+                 m.shape[1] if m is not None else 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, Sq, Sk, D, int(causal), 0.0,
+                 hip.current_stream())
+    finally:
+        hip.set_option("sdpa_variant", 0)
     res = untilize_dev(hip, out, q.shape, dev).float().cpu().numpy()
     torch.cuda.synchronize()
     want = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), None if m is None else m.float().numpy(),

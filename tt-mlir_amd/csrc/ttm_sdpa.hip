@@ -209,6 +209,211 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
     }
 }
 
+// Same computation with 64 keys per pass (head_dim <= 128): half as many barriers and loop turns, two independent
+// accumulator chains for S, and V^T written to LDS as 32-bit pairs of neighbouring keys (the two lanes that hold keys
+// k and k + 1 of the same 8 columns trade halves with a quad permute) instead of 16-bit scatters.
+__device__ __forceinline__ uint32_t quad_xor2(uint32_t v) {   // value of lane ^ 2
+  return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E /* quad_perm [2,3,0,1] */, 0xF, 0xF, true);
+}
+
+template <int DT>  // head_dim / 32
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void ttm_sdpa64_k(SdpaArgs p) {
+  constexpr int D = DT * 32;
+  constexpr int VPITCH = 68;                           // V^T row pitch in bf16 (64 keys + pad): rows 34 words apart
+  __shared__ __attribute__((aligned(16))) uint8_t ldsK[64 * D * 2];
+  __shared__ __attribute__((aligned(16))) uint16_t ldsV[D * VPITCH];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int qb = gridDim.x - 1 - blockIdx.x, h = blockIdx.y, b = blockIdx.z;   // longest (causal) workgroups first
+  const int hk = h / (p.Hq / p.Hkv);
+  const int qt = qb * 4 + wave;                         // this wave's query tile
+  const bool wave_ok = qt < p.sqt;
+  const int l31 = lane & 31, hh = lane >> 5;
+  const int64_t q_mat = ((int64_t)b * p.Hq + h) * p.sqt * DT * 2048;
+  const int64_t kv_mat = ((int64_t)b * p.Hkv + hk) * p.skt * DT * 2048;
+
+  bf16x8 qf[2 * DT];
+#pragma unroll
+  for (int s = 0; s < 2 * DT; ++s) {
+    u32x4 v = {0, 0, 0, 0};
+    if (wave_ok)
+      v = *(const u32x4 *)(p.q + q_mat + ((int64_t)qt * DT + (s >> 1)) * 2048 + ((l31 >> 4) * 2 + (s & 1)) * 512 +
+                           (l31 & 15) * 32 + hh * 16);
+    qf[s] = *(bf16x8 *)&v;
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[d][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+  const int q_glob = qt * 32 + l31, q_last = qt * 32 + 31;
+
+  int kt_end = p.skt;                                   // 32-key tiles any wave of this workgroup needs
+  if (p.causal) kt_end = min(kt_end, (min(qb * 4 + 4, p.sqt) * 32 + 31) / 32);
+  const int kb_end = (kt_end + 1) >> 1;                 // 64-key passes
+  // a lane moves DT 16-byte chunks of K and of V per pass: chunk c = tid + 256 i lies in tile row c / (DT * 128)
+  u32x4 kreg[DT], vreg[DT];
+  auto load_block = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < DT; ++i) {
+      const int c = tid + 256 * i, tr = c / (DT * 128), cc = c % (DT * 128);
+      const int kt = min(2 * kb + tr, p.skt - 1);       // an odd tile count repeats the last tile; its keys are masked
+      kreg[i] = ((const u32x4 *)(p.k + kv_mat + (int64_t)kt * DT * 2048))[cc];
+      vreg[i] = ((const u32x4 *)(p.v + kv_mat + (int64_t)kt * DT * 2048))[cc];
+    }
+  };
+  if (kb_end > 0) load_block(0);
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = p.scale * LOG2E;
+  for (int kb = 0; kb < kb_end; ++kb) {
+    __syncthreads();  // previous block fully consumed
+#pragma unroll
+    for (int i = 0; i < DT; ++i) {
+      const int c = tid + 256 * i, tr = c / (DT * 128), cc = c % (DT * 128);
+      ((u32x4 *)ldsK)[c] = kreg[i];
+      // V: this lane holds 8 columns of one key; lane ^ 2 holds the same columns of the neighbouring key
+      const u32x4 v = vreg[i];
+      const int tile = cc >> 7, c7 = cc & 127;
+      const int face = c7 >> 5, row = (c7 & 31) >> 1, half = c7 & 1;
+      const bool odd = row & 1;
+      const int key = 32 * tr + (face >> 1) * 16 + (row & ~1);          // even key of the pair
+      const int d0 = tile * 32 + (face & 1) * 16 + half * 8 + (odd ? 4 : 0);
+      // the even lane keeps columns 0..3 and receives the odd lane's columns 0..3; the odd lane the other way round
+      const uint32_t send0 = odd ? v.x : v.z, send1 = odd ? v.y : v.w;
+      const uint32_t got0 = quad_xor2(send0), got1 = quad_xor2(send1);
+      const uint32_t mine0 = odd ? v.z : v.x, mine1 = odd ? v.w : v.y;
+      const uint32_t e0 = odd ? got0 : mine0, o0 = odd ? mine0 : got0;  // even key's word, odd key's word
+      const uint32_t e1 = odd ? got1 : mine1, o1 = odd ? mine1 : got1;
+      uint32_t *vt = (uint32_t *)(ldsV + d0 * VPITCH + key);
+      vt[0] = __builtin_amdgcn_perm(o0, e0, 0x05040100u);
+      vt[VPITCH / 2] = __builtin_amdgcn_perm(o0, e0, 0x07060302u);
+      vt[VPITCH] = __builtin_amdgcn_perm(o1, e1, 0x05040100u);
+      vt[3 * VPITCH / 2] = __builtin_amdgcn_perm(o1, e1, 0x07060302u);
+    }
+    __syncthreads();
+    if (kb + 1 < kb_end) load_block(kb + 1);
+    const int key_base = kb * 64;
+    if (!wave_ok || (p.causal && key_base > q_last)) continue;
+    // the second half of the pass is skipped when the causal limit or the key count makes it empty for this wave
+    const bool second = !(p.causal && key_base + 32 > q_last) && key_base + 32 < p.Sk;   // wavefront-uniform
+
+    f32x16 s0, s1;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s0[r] = 0.0f; s1[r] = 0.0f; }
+#pragma unroll
+    for (int st = 0; st < 2 * DT; ++st) {
+      const uint8_t *kp = ldsK + (st >> 1) * 2048 + ((l31 >> 4) * 2 + (st & 1)) * 512 + (l31 & 15) * 32 + hh * 16;
+      u32x4 ka = *(const u32x4 *)kp;
+      s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&ka, qf[st], s0, 0, 0, 0);
+      if (second) {
+        u32x4 kb2 = *(const u32x4 *)(kp + DT * 2048);
+        s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&kb2, qf[st], s1, 0, 0, 0);
+      }
+    }
+    // scale, mask; a lane holds q = q_glob and keys key_base + 32 half + 8 g + 4 hh + r.  Scores stay in the log2
+    // domain so that the exponential is a bare v_exp_f32.
+    const bool edge = (p.causal && key_base + 63 > qt * 32) || key_base + 64 > p.Sk;   // wavefront-uniform
+    float mx = -INFINITY;
+    auto finish_scores = [&](f32x16 &s, int half) {
+      if (p.mask || edge) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int kin = g * 8 + hh * 4;
+          const int key0 = key_base + 32 * half + kin;
+          float mk[4] = {0.f, 0.f, 0.f, 0.f};
+          if (p.mask) {
+            const int kt = min(2 * kb + half, p.skt - 1);
+            const int64_t mm = ((int64_t)b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
+            const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
+                                (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
+            u32x2 raw = *(const u32x2 *)mp;
+            mk[0] = __uint_as_float(raw.x << 16); mk[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+            mk[2] = __uint_as_float(raw.y << 16); mk[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float v = fmaf(s[g * 4 + r], scale2, mk[r] * LOG2E);
+            const int key = key0 + r;
+            if (key >= p.Sk || (p.causal && key > q_glob)) v = -INFINITY;
+            s[g * 4 + r] = v;
+            mx = fmaxf(mx, v);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          s[r] *= scale2;
+          mx = fmaxf(mx, s[r]);
+        }
+      }
+    };
+    finish_scores(s0, 0);
+    if (second) finish_scores(s1, 1);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new == -INFINITY ? 0.0f : m_new;   // fully masked so far: stay at zero without producing NaN
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    float rs = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float e = __builtin_amdgcn_exp2f(s0[r] - m_use);
+      s0[r] = e;
+      rs += e;
+    }
+    if (second) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float e = __builtin_amdgcn_exp2f(s1[r] - m_use);
+        s1[r] = e;
+        rs += e;
+      }
+    }
+    rs += __shfl_xor(rs, 32);
+    l_run = l_run * alpha + rs;
+    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {   // the running maximum seldom moves after the first passes
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
+    }
+    // O^T += V^T . P^T, k16 steps over the 32 or 64 keys
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (t >= 2 && !second) break;
+      const f32x16 &s = t < 2 ? s0 : s1;
+      const int t8 = 8 * (t & 1);
+      u32x4 pb;
+      pb.x = pack_bf16_rne(s[t8 + 0], s[t8 + 1]);
+      pb.y = pack_bf16_rne(s[t8 + 2], s[t8 + 3]);
+      pb.z = pack_bf16_rne(s[t8 + 4], s[t8 + 5]);
+      pb.w = pack_bf16_rne(s[t8 + 6], s[t8 + 7]);
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        const uint16_t *vr = ldsV + (d * 32 + l31) * VPITCH + 16 * t + 4 * hh;
+        u32x2 lo = *(const u32x2 *)vr, hi = *(const u32x2 *)(vr + 8);
+        u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va, *(bf16x8 *)&pb, o[d], 0, 0, 0);
+      }
+    }
+  }
+  if (!wave_ok) return;
+  const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+  const bool q_ok = q_glob < p.Sq;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int din = g * 8 + hh * 4;
+      u32x2 ov;
+      ov.x = q_ok ? pack_bf16_rne(o[d][g * 4 + 0] * inv, o[d][g * 4 + 1] * inv) : 0u;
+      ov.y = q_ok ? pack_bf16_rne(o[d][g * 4 + 2] * inv, o[d][g * 4 + 3] * inv) : 0u;
+      uint8_t *op = p.out + q_mat + ((int64_t)qt * DT + d) * 2048 +
+                    (((l31 >> 4) * 2 + (din >> 4)) * 256 + (l31 & 15) * 16 + (din & 15)) * 2;
+      *(u32x2 *)op = ov;
+    }
+}
+
 TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
                         int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                         int is_causal, float scale, void *stream) {
@@ -230,11 +435,12 @@ TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void 
   p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)D);
   dim3 grid((unsigned)ttm_cdiv(p.sqt, 4), (unsigned)Hq, (unsigned)B), block(256);
   hipStream_t s = (hipStream_t)stream;
+  const bool wide = ttm_option("sdpa_variant") != 1;   // 64 keys per pass unless the 32-key kernel is asked for
   switch (D) {
-  case 32: hipLaunchKernelGGL(ttm_sdpa_k<1>, grid, block, 0, s, p); break;
-  case 64: hipLaunchKernelGGL(ttm_sdpa_k<2>, grid, block, 0, s, p); break;
-  case 128: hipLaunchKernelGGL(ttm_sdpa_k<4>, grid, block, 0, s, p); break;
-  default: hipLaunchKernelGGL(ttm_sdpa_k<8>, grid, block, 0, s, p); break;
+  case 32: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<1>, grid, block, 0, s, p); else hipLaunchKernelGGL(ttm_sdpa_k<1>, grid, block, 0, s, p); break;
+  case 64: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<2>, grid, block, 0, s, p); else hipLaunchKernelGGL(ttm_sdpa_k<2>, grid, block, 0, s, p); break;
+  case 128: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<4>, grid, block, 0, s, p); else hipLaunchKernelGGL(ttm_sdpa_k<4>, grid, block, 0, s, p); break;
+  default: hipLaunchKernelGGL(ttm_sdpa_k<8>, grid, block, 0, s, p); break;   // 256 columns: the 64-key staging would not fit in LDS
   }
   TTM_LAUNCH_CHECK();
   return TTM_OK;
