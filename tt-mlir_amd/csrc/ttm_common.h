@@ -59,9 +59,12 @@ __host__ __device__ static inline int64_t ttm_tiled_offset(int64_t r, int64_t c,
 }
 
 __device__ static inline float ttm_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
-__device__ static inline uint16_t ttm_f32_to_bf16(float f) {  // round to nearest even, quiet NaN
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);
-  u += 0x7FFFu + ((u >> 16) & 1);
-  return (uint16_t)(u >> 16);
+// f32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950; NaN stays a quiet NaN)
+typedef __bf16 ttm_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float ttm_f32x2 __attribute__((ext_vector_type(2)));
+__device__ static inline uint32_t ttm_pack_bf16x2(float lo, float hi) {
+  ttm_f32x2 v = {lo, hi};
+  ttm_bf16x2 h = __builtin_convertvector(v, ttm_bf16x2);
+  return *(uint32_t *)&h;
 }
+__device__ static inline uint16_t ttm_f32_to_bf16(float f) { return (uint16_t)(ttm_pack_bf16x2(f, 0.0f) & 0xFFFFu); }

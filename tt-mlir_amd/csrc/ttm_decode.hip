@@ -24,10 +24,10 @@ __device__ __forceinline__ void load8(const float *p, float *v) {
 }
 __device__ __forceinline__ void store8(uint16_t *p, const float *v) {
   u32x4 r;
-  r.x = ttm_f32_to_bf16(v[0]) | ((uint32_t)ttm_f32_to_bf16(v[1]) << 16);
-  r.y = ttm_f32_to_bf16(v[2]) | ((uint32_t)ttm_f32_to_bf16(v[3]) << 16);
-  r.z = ttm_f32_to_bf16(v[4]) | ((uint32_t)ttm_f32_to_bf16(v[5]) << 16);
-  r.w = ttm_f32_to_bf16(v[6]) | ((uint32_t)ttm_f32_to_bf16(v[7]) << 16);
+  r.x = ttm_pack_bf16x2(v[0], v[1]);
+  r.y = ttm_pack_bf16x2(v[2], v[3]);
+  r.z = ttm_pack_bf16x2(v[4], v[5]);
+  r.w = ttm_pack_bf16x2(v[6], v[7]);
   *(u32x4 *)p = r;
 }
 __device__ __forceinline__ void store8(float *p, const float *v) {
@@ -232,9 +232,9 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
       const int klo = (i >> 4) * 32 + (i & 15), khi = klo + 16;
       const float elo = (m == -INFINITY || klo >= padded) ? 0.0f : __expf(row[klo] - m);
       const float ehi = (m == -INFINITY || khi >= padded) ? 0.0f : __expf(row[khi] - m);
-      const uint32_t blo = ttm_f32_to_bf16(elo), bhi = ttm_f32_to_bf16(ehi);
-      prow[i] = blo | (bhi << 16);
-      l += __uint_as_float(blo << 16) + __uint_as_float(bhi << 16);
+      const uint32_t pair = ttm_pack_bf16x2(elo, ehi);
+      prow[i] = pair;
+      l += __uint_as_float(pair << 16) + __uint_as_float(pair & 0xFFFF0000u);
     }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o);

@@ -69,7 +69,7 @@ __device__ __forceinline__ void store_vals(void *base, int64_t off, const float 
   u32x4 v;
   if (ELEM == 2) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = (uint32_t)ttm_f32_to_bf16(f[2 * i]) | ((uint32_t)ttm_f32_to_bf16(f[2 * i + 1]) << 16);
+    for (int i = 0; i < 4; ++i) v[i] = ttm_pack_bf16x2(f[2 * i], f[2 * i + 1]);
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = __float_as_uint(f[i]);

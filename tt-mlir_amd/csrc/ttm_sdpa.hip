@@ -27,7 +27,7 @@ struct SdpaArgs {
 };
 
 __device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
-  return (uint32_t)ttm_f32_to_bf16(a) | ((uint32_t)ttm_f32_to_bf16(b) << 16);
+  return ttm_pack_bf16x2(a, b);
 }
 
 template <int DT>  // head_dim / 32
@@ -216,14 +216,13 @@ __device__ __forceinline__ uint32_t quad_xor2(uint32_t v) {   // value of lane ^
   return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E /* quad_perm [2,3,0,1] */, 0xF, 0xF, true);
 }
 
+constexpr int kSdpaVPitch = 68;   // V^T row pitch in bf16 (64 keys + pad): rows 34 words apart
+
+// one block of 128 queries (4 wavefronts x 32) of head h against all the keys it needs
 template <int DT>  // head_dim / 32
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void ttm_sdpa64_k(SdpaArgs p) {
-  constexpr int D = DT * 32;
-  constexpr int VPITCH = 68;                           // V^T row pitch in bf16 (64 keys + pad): rows 34 words apart
-  __shared__ __attribute__((aligned(16))) uint8_t ldsK[64 * D * 2];
-  __shared__ __attribute__((aligned(16))) uint16_t ldsV[D * VPITCH];
+__device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *ldsK, uint16_t *ldsV) {
+  constexpr int VPITCH = kSdpaVPitch;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int qb = gridDim.x - 1 - blockIdx.x, h = blockIdx.y, b = blockIdx.z;   // longest (causal) workgroups first
   const int hk = h / (p.Hq / p.Hkv);
   const int qt = qb * 4 + wave;                         // this wave's query tile
   const bool wave_ok = qt < p.sqt;
@@ -414,6 +413,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+
+// Causal attention gives query block qb work proportional to qb + 1.  With one workgroup per query block all workgroups of a
+// launch are resident at once and the launch lasts as long as the heaviest of them; a workgroup therefore takes the pair
+// (last - i, i), heavy block first, so that every workgroup has the same amount of work.
+template <int DT>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void ttm_sdpa64_k(SdpaArgs p, int paired) {
+  constexpr int D = DT * 32;
+  __shared__ __attribute__((aligned(16))) uint8_t ldsK[64 * D * 2];
+  __shared__ __attribute__((aligned(16))) uint16_t ldsV[D * kSdpaVPitch];
+  const int nqb = (p.sqt + 3) / 4, h = blockIdx.y, b = blockIdx.z;
+  if (!paired) {
+    sdpa64_query_block<DT>(p, nqb - 1 - (int)blockIdx.x, h, b, ldsK, ldsV);
+    return;
+  }
+  const int heavy = nqb - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
+  sdpa64_query_block<DT>(p, heavy, h, b, ldsK, ldsV);
+  if (light < heavy) sdpa64_query_block<DT>(p, light, h, b, ldsK, ldsV);
+}
+
 TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
                         int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                         int is_causal, float scale, void *stream) {
@@ -435,11 +453,15 @@ TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void 
   p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)D);
   dim3 grid((unsigned)ttm_cdiv(p.sqt, 4), (unsigned)Hq, (unsigned)B), block(256);
   hipStream_t s = (hipStream_t)stream;
-  const bool wide = ttm_option("sdpa_variant") != 1;   // 64 keys per pass unless the 32-key kernel is asked for
+  const int variant = ttm_option("sdpa_variant");   // 1 = 32 keys per pass, 2 = 64 keys without pairing query blocks
+  const bool wide = variant != 1;
+  const int nqb = (int)ttm_cdiv(p.sqt, 4);
+  const int paired = is_causal && nqb >= 2 && variant != 2;
+  const dim3 grid64(paired ? (unsigned)((nqb + 1) / 2) : (unsigned)nqb, (unsigned)Hq, (unsigned)B);
   switch (D) {
-  case 32: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<1>, grid, block, 0, s, p); else hipLaunchKernelGGL(ttm_sdpa_k<1>, grid, block, 0, s, p); break;
-  case 64: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<2>, grid, block, 0, s, p); else hipLaunchKernelGGL(ttm_sdpa_k<2>, grid, block, 0, s, p); break;
-  case 128: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<4>, grid, block, 0, s, p); else hipLaunchKernelGGL(ttm_sdpa_k<4>, grid, block, 0, s, p); break;
+  case 32: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<1>, grid64, block, 0, s, p, paired); else hipLaunchKernelGGL(ttm_sdpa_k<1>, grid, block, 0, s, p); break;
+  case 64: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<2>, grid64, block, 0, s, p, paired); else hipLaunchKernelGGL(ttm_sdpa_k<2>, grid, block, 0, s, p); break;
+  case 128: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<4>, grid64, block, 0, s, p, paired); else hipLaunchKernelGGL(ttm_sdpa_k<4>, grid, block, 0, s, p); break;
   default: hipLaunchKernelGGL(ttm_sdpa_k<8>, grid, block, 0, s, p); break;   // 256 columns: the 64-key staging would not fit in LDS
   }
   TTM_LAUNCH_CHECK();
