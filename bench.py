@@ -195,7 +195,7 @@ def make_workloads(torch, hip, datagen, dev, names):
 # constants of the committed kernels, not computed here.
 MEASURED_TRAFFIC_BYTES = {
     "linear2048": 390.5e6, "linear32": 65.7e6, "pack_bfp8": 341.4e6, "unpack_bfp8": 340.1e6, "pack_bfp4": 308.1e6,
-    "unpack_bfp4": 306.5e6, "tilize_f32": 537.0e6, "untilize_f32": 537.0e6, "copy": 536.9e6,
+    "unpack_bfp4": 306.5e6, "tilize_f32": 537.0e6, "untilize_f32": 537.0e6, "copy": 536.9e6, "sdpa_decode32": 270.4e6,
 }
 
 
