@@ -114,6 +114,16 @@ int ttm_bfp_unpack(const void *src, int fmt, void *dst, int dst_dtype, int dst_l
 int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias,
                int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch,
                int64_t M, int64_t N, int64_t K, int act, void *stream);
+/* ttm_linear followed by one element-wise op with a second BFloat16 TILE tensor of the output's shape, in the same pass:
+ * out = round(round(act(a w + bias)) (+ | *) tail).  This is what the executor calls for a MatmulOp / LinearOp whose only
+ * consumer is the next `add` (residual connection) or `multiply` (SiLU(gate) * up, runtime/lib/ttnn/operations/eltwise/
+ * binary/binary.cpp:38-126); both roundings are kept so that the result equals the two ops run one after the other. */
+#define TTM_TAIL_NONE 0
+#define TTM_TAIL_ADD 1
+#define TTM_TAIL_MUL 2
+int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias, int bias_dtype,
+                    int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N,
+                    int64_t K, int act, int tail_op, const void *tail, void *stream);
 
 /* ---- elementwise: ::ttnn::<unary>, ::ttnn::<binary>
  * (runtime/lib/ttnn/operations/eltwise/unary/unary.cpp:159-205, eltwise/binary/binary.cpp:38-126;

@@ -241,6 +241,46 @@ def test_two_part_grid_with_ragged_remainder(hip, dev, orc, metrics, wfmt_name):
         check(orc, metrics, got[:, cols], a, w_eff[:, cols].contiguous(), b[cols], "relu", max_abs=2.0 ** -5)
 
 
+@pytest.mark.parametrize("tail", ["add", "multiply"])
+@pytest.mark.parametrize("wfmt_name,M,K,N,option,value", [
+    ("bfp8", 32, 1200, 200, None, 0),                 # decode kernel
+    ("bfp4", 20, 1200, 200, "linear_decode_split", 3),  # decode kernel with k-slices: tail applied by the reduction
+    ("bf16", 32, 256, 96, None, 0),                   # small-M kernel for bf16 weights
+    ("bfp8", 330, 232, 677, None, 0),                 # LDS-direct main kernel, ragged
+    ("bfp4", 330, 232, 677, "linear_split_k", 2),     # split-K main kernel
+    ("bf16", 288, 160, 320, None, 0),                 # register-staged kernel
+    ("bfp8", 96, 96, 160, "linear_variant", 1),       # 64-bit-addressed fallback
+])
+def test_linear_with_fused_tail_equals_two_ops(hip, dev, orc, metrics, tail, wfmt_name, M, K, N, option, value):
+    """ttm_linear_tail (add / multiply with a second tensor in the epilogue) against ttm_linear followed by the oracle's
+    binary op on the rounded result: bit exact on every kernel path, because both roundings are kept."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B, "bf16": hip.BF16}[wfmt_name]
+    a = datagen.randn((M, K), seed=61, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=62, std=0.05)
+    b = datagen.randn((N,), seed=63, std=0.5, dtype=torch.bfloat16)
+    t = datagen.randn((M, N), seed=64, dtype=torch.bfloat16)
+    if option:
+        hip.set_option(option, value)
+    try:
+        plain, _ = run_linear(hip, dev, a, w, b, "silu", wfmt)
+        at = tilize_dev(hip, a, dev)
+        wt = tilize_dev(hip, w.to(torch.bfloat16), dev) if wfmt == hip.BF16 else pack_weight(hip, w, wfmt, dev)
+        bt, tt = tilize_dev(hip, b.reshape(1, -1), dev), tilize_dev(hip, t, dev)
+        out = torch.full_like(tt, float("nan"))
+        hip.call("ttm_linear_tail", hip.ptr(at), hip.BF16, hip.ptr(wt), wfmt, 0, hip.ptr(bt), hip.BF16, hip.TILE, hip.ptr(out), hip.BF16,
+                 1, 1, M, N, K, hip.ACT["silu"], 1 if tail == "add" else 2, hip.ptr(tt), hip.current_stream())
+        got = untilize_dev(hip, out, (M, N), dev).cpu()
+        torch.cuda.synchronize()
+    finally:
+        if option:
+            hip.set_option(option, 0)
+    want = orc.round_bf16(orc.binary(tail, plain.float().numpy(), t.float().numpy()))
+    assert np.array_equal(got.float().numpy(), want)
+    with pytest.raises(hip.TTMError, match="tail op needs its operand"):
+        hip.call("ttm_linear_tail", hip.ptr(at), hip.BF16, hip.ptr(wt), wfmt, 0, None, hip.BF16, hip.TILE, hip.ptr(out), hip.BF16,
+                 1, 1, M, N, K, 0, 1, None, hip.current_stream())
+
+
 def test_split_k_is_chosen_for_long_skinny_reductions(hip, dev, orc, metrics):
     """M = 128, N = 256, K = 8192: one round of blocks would use 2 CUs; the launcher splits K."""
     M, K, N = 128, 8192, 256

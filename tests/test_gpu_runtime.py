@@ -551,6 +551,25 @@ def test_reshape_permute_pairs_are_fused_without_changing_results(device, shape,
     assert fused_copies < unfused_copies, (fused_copies, unfused_copies)
 
 
+def test_fused_epilogue_tails_do_not_change_program_results(device):
+    """Without callbacks the executor folds `x + matmul(...)` and `silu(gate) * matmul(...)` into the matmul's epilogue; with a
+    callback registered every op runs on its own.  Both runs of the decoder layer must agree bit for bit."""
+    d = datagen.c5_decoder(seq=96, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, seed=8)
+    binary = rt.Binary.load_from_memory(programs.c5_decoder(seq=96, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512))
+    tins = [d["x"], d["attn_norm_w"], bf(d["wq"]), bf(d["wk"]), bf(d["wv"]), bf(d["wo"]), d["mlp_norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    rt.clear_stats()
+    (fused,) = harness.execute(binary, 1, tins, device)
+    assert rt.get_stat("FusedLinearTail") == 3          # attention residual, gate * up, MLP residual
+    seen = []
+    rt.set_post_op_callback(lambda idx, name, dbg, hook: seen.append(name))
+    try:
+        (plain,) = harness.execute(binary, 1, tins, device)
+    finally:
+        rt.clear_callbacks()
+    assert seen.count("EltwiseBinaryOp") == 3 and rt.get_stat("FusedLinearTail") == 3
+    assert torch.equal(fused, plain)
+
+
 def test_submit_errors(device):
     binary = rt.Binary.load_from_memory(programs.c3_linear(32, 64, 64))
     a = rt.from_torch(torch.zeros(32, 64, dtype=torch.bfloat16))

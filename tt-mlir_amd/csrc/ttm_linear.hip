@@ -45,6 +45,8 @@ struct LinearArgs {
                                       // the rest cover [nt_split, Nt) at width ntw2; nt_split = 0: one part
   int k_slice;                        // k-tiles per grid.y slice (split-K); Kt when the reduction is not split
   float *partial;                     // split-K: fp32 partial sums [slices][Mt * Nt * 1024] in output tile order
+  int tail;                           // 0 none, 1 add, 2 multiply: element-wise tail with a tensor laid out like the output
+  int64_t tail_delta;                 // byte distance from an output element to its tail operand
 };
 
 template <int ACT>
@@ -63,6 +65,24 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   f32x2_t v = {a, b};
   bf16x2_t h = __builtin_convertvector(v, bf16x2_t);
   return *(uint32_t *)&h;
+}
+
+// Four consecutive outputs -> bf16, optionally followed by the element-wise tail.  The result is rounded to bf16 before the
+// tail and again after it, exactly as a separate binary op on the stored result would do.
+__device__ __forceinline__ u32x2 finish_quad(const LinearArgs &p, const uint8_t *cptr, const float (&v)[4]) {
+  u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+  if (p.tail != 0) {   // uniform
+    const u32x2 r = *(const u32x2 *)(cptr + p.tail_delta);
+    const float y[4] = {__uint_as_float(o.x << 16), __uint_as_float(o.x & 0xFFFF0000u), __uint_as_float(o.y << 16),
+                        __uint_as_float(o.y & 0xFFFF0000u)};
+    const float t[4] = {__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xFFFF0000u), __uint_as_float(r.y << 16),
+                        __uint_as_float(r.y & 0xFFFF0000u)};
+    float z[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) z[i] = p.tail == 1 ? y[i] + t[i] : y[i] * t[i];
+    o = u32x2{pack_bf16(z[0], z[1]), pack_bf16(z[2], z[3])};
+  }
+  return o;
 }
 
 // LDS image of an operand block: [row][8 chunks of 8 k], chunk slot XOR-swizzled by the row so that every
@@ -249,9 +269,8 @@ __device__ __forceinline__ void linear_epilogue(const LinearArgs &p, uint8_t *C,
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) v[r] = apply_act<ACT>(acc[a][b][g * 4 + r] + bv[r]);
-        u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
         int64_t off = ((int64_t)mt * p.Nt + nt) * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
-        *(u32x2 *)(C + off * 2) = o;
+        *(u32x2 *)(C + off * 2) = finish_quad(p, C + off * 2, v);
       }
     }
   }
@@ -310,7 +329,7 @@ __global__ __launch_bounds__(256) void ttm_linear_reduce_k(LinearArgs p, int sli
     v[r] = x;
   }
   uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
-  *(u32x2 *)(C + off * 2) = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+  *(u32x2 *)(C + off * 2) = finish_quad(p, C + off * 2, v);
 }
 
 template <int NA, int MB>
@@ -1115,9 +1134,8 @@ __global__ __launch_bounds__(256) void ttm_linear_small_k(LinearArgs p) {
       }
       v[r] = x;
     }
-    u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
     int64_t off = (int64_t)nt * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
-    *(u32x2 *)(C + off * 2) = o;
+    *(u32x2 *)(C + off * 2) = finish_quad(p, C + off * 2, v);
   }
 }
 
@@ -1265,8 +1283,7 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
     }
     v[r] = x;
   }
-  u32x2 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-  *(u32x2 *)(C + off * 2) = o;
+  *(u32x2 *)(C + off * 2) = finish_quad(p, C + off * 2, v);
 }
 
 static int device_cu_count() {
@@ -1443,6 +1460,17 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
 TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias,
                           int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch,
                           int64_t w_batch, int64_t M, int64_t N, int64_t K, int act, void *stream) {
+  return ttm_linear_tail(a, a_dtype, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, act,
+                         TTM_TAIL_NONE, nullptr, stream);
+}
+
+TTM_EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias,
+                               int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch,
+                               int64_t M, int64_t N, int64_t K, int act, int tail_op, const void *tail, void *stream) {
+  TTM_REQUIRE(tail_op >= TTM_TAIL_NONE && tail_op <= TTM_TAIL_MUL, "ttm_linear: unknown tail op %d", tail_op);
+  TTM_REQUIRE((tail_op == TTM_TAIL_NONE) == (tail == nullptr), "ttm_linear: a tail op needs its operand, and only then");
+  TTM_REQUIRE(((uintptr_t)tail & 15) == 0, "ttm_linear: the tail operand must be 16-byte aligned");
+  TTM_REQUIRE(tail != out, "ttm_linear: the tail operand must not be the output");
   TTM_REQUIRE(a_dtype == TTM_BF16 && out_dtype == TTM_BF16, "ttm_linear: activations and output must be BFloat16");
   TTM_REQUIRE(w_dtype == TTM_BF16 || w_dtype == TTM_BFP8B || w_dtype == TTM_BFP4B,
               "ttm_linear: weights must be BFloat16, BFP_BFloat8 or BFP_BFloat4 (got %d)", w_dtype);
@@ -1470,6 +1498,8 @@ TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype
   p.ntw = 4;
   p.k_slice = p.Kt; p.partial = nullptr;
   p.nt_split = p.n_blocks1 = p.ntw2 = 0;
+  p.tail = tail_op;
+  p.tail_delta = tail ? (const uint8_t *)tail - (const uint8_t *)out : 0;
   TTM_REQUIRE(batch <= 65535, "ttm_linear: batch too large");
   hipStream_t s = (hipStream_t)stream;
   int rc;

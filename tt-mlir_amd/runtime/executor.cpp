@@ -245,6 +245,8 @@ void runToMemoryConfig(const fb::Table &op, ProgramContext &ctx) {
   ctx.put(op.table(schema::ToMemoryConfigOp::f_out), ctx.get(op.table(schema::ToMemoryConfigOp::f_in0), "to_memory_config in"));
 }
 
+std::uint32_t refId(const fb::Table &ref);
+
 // ---- matmul / linear (runtime/lib/ttnn/operations/matmul/matmul.cpp:47-125)
 Tensor transposeLast2(ProgramContext &ctx, const Tensor &t) {
   std::vector<std::uint32_t> shape = t.handle->shape;
@@ -291,10 +293,51 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
     biasPtr = bias.handle->data.get();
   }
   Tensor out = makeOut(ctx, outRef, DataType::BFloat16, TensorLayout::Tile);
-  TTM_CALL(ttm_linear(a.handle->data.get(), TTM_BF16, b.handle->data.get(), ttmDtype(b.handle->dtype), transposeB ? 1 : 0, biasPtr,
-                      TTM_BF16, biasLayout, out.handle->data.get(), TTM_BF16, batch, wbatch == 1 ? 1 : batch, M, N, K,
-                      activationCode(activation), ctx.stream()));
-  ctx.put(outRef, finish(ctx, out, outRef));
+  // an `add` or `multiply` that is the only consumer of this result and comes next runs in the kernel's epilogue
+  // (residual connections, SiLU(gate) * up); its output takes this op's place
+  Tensor tail;
+  int tailOp = TTM_TAIL_NONE;
+  fb::Table finalRef = outRef;
+  // deallocations of other tensors may sit between the two ops (the compiler frees the matmul's operand right after it)
+  std::uint32_t nextIdx = ctx.opIndex + 1;
+  auto opType = [&](std::uint32_t i) { return static_cast<OpType>(ctx.ops[i].scalar<std::uint8_t>(schema::Operation::f_type_type, 0)); };
+  std::vector<std::uint32_t> freedBetween;
+  while (ctx.fuseViews && nextIdx < ctx.ops.size() && opType(nextIdx) == OpType::DeallocateOp) {
+    freedBetween.push_back(refId(ctx.ops[nextIdx].table(schema::Operation::f_type).table(schema::DeallocateOp::f_in)));
+    ++nextIdx;
+  }
+  if (ctx.fuseViews && nextIdx < ctx.ops.size()) {
+    const fb::Table &next = ctx.ops[nextIdx];
+    if (opType(nextIdx) == OpType::EltwiseBinaryOp) {
+      using B = schema::EltwiseBinaryOp;
+      fb::Table bop = next.table(schema::Operation::f_type);
+      const std::uint32_t kind = bop.scalar<std::uint32_t>(B::f_type, 0);
+      fb::Table lhs = bop.table(B::f_lhs), rhs = bop.table(B::f_rhs), bout = bop.table(B::f_out);
+      const std::uint32_t mine = refId(outRef);
+      auto uses = ctx.uses.find(mine);
+      const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
+      if ((kind == 0 || kind == 1) && lhs && rhs && bout && (refId(lhs) == mine) != (refId(rhs) == mine) && uses != ctx.uses.end() &&
+          uses->second == 1 && layoutFromTensorRef(outRef) == plain && layoutFromTensorRef(bout) == plain &&
+          shapeFromTensorRef(bout) == shapeFromTensorRef(outRef)) {
+        const std::uint32_t otherId = refId(refId(lhs) == mine ? rhs : lhs);
+        const bool freed = std::find(freedBetween.begin(), freedBetween.end(), otherId) != freedBetween.end() ||
+                           std::find(freedBetween.begin(), freedBetween.end(), mine) != freedBetween.end();
+        auto it = ctx.pool.find(otherId);
+        if (!freed && it != ctx.pool.end() && isTensorAllocated(it->second) && getTensorLayout(it->second) == plain &&
+            it->second.handle->shape == out.handle->shape) {
+          tail = it->second;
+          tailOp = kind == 0 ? TTM_TAIL_ADD : TTM_TAIL_MUL;
+          finalRef = bout;
+          ctx.skip.insert(nextIdx);
+          debug::Stats::get().incrementStat("FusedLinearTail");
+        }
+      }
+    }
+  }
+  TTM_CALL(ttm_linear_tail(a.handle->data.get(), TTM_BF16, b.handle->data.get(), ttmDtype(b.handle->dtype), transposeB ? 1 : 0, biasPtr,
+                           TTM_BF16, biasLayout, out.handle->data.get(), TTM_BF16, batch, wbatch == 1 ? 1 : batch, M, N, K,
+                           activationCode(activation), tailOp, tail ? tail.handle->data.get() : nullptr, ctx.stream()));
+  ctx.put(finalRef, finish(ctx, out, finalRef));
 }
 void runMatmul(const fb::Table &op, ProgramContext &ctx) {
   runMatmulLike(ctx, op.table(schema::MatmulOp::f_a), op.table(schema::MatmulOp::f_b), fb::Table(), op.table(schema::MatmulOp::f_out),
