@@ -570,6 +570,42 @@ def test_fused_epilogue_tails_do_not_change_program_results(device):
     assert torch.equal(fused, plain)
 
 
+def test_concurrent_submits_from_two_threads(device, orc):
+    """submit is re-entrant: two threads drive the same device at once (the reference runs one thread per submesh,
+    test/python/golden/test_data_parallel.py:58-75); programs are serialised per device and both get their own results."""
+    import threading
+    plain = rt.Binary.load_from_memory(programs.c4_mlp(64, 128, 256))
+    traced = rt.Binary.load_from_memory(programs.traced_mlp(32, 128, 256))
+    d = datagen.c4_mlp(64, 128, 256, seed=17)
+    weights = [d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    g = torch.Generator().manual_seed(9)
+    xs_a = [torch.randn((64, 128), generator=g).to(torch.bfloat16) for _ in range(8)]
+    xs_b = [torch.randn((32, 128), generator=g).to(torch.bfloat16) for _ in range(8)]
+    want_a = [harness.execute(plain, 1, [x] + weights, device)[0] for x in xs_a]
+    res_b = [rt.to_layout(rt.from_torch(t), device, rt.get_layout(traced, 5, k + 1), retain=True) for k, t in enumerate(weights)]
+    want_b = [_run_traced(traced, device, x, res_b) for x in xs_b]
+    # a second traced binary captures its graph inside thread b, while thread a converts layouts and reads results back
+    traced = rt.Binary.load_from_memory(programs.traced_mlp(32, 128, 256))
+    got_a, got_b, errors = [None] * 8, [None] * 8, []
+
+    def worker(kind):
+        try:
+            for i in range(8):
+                if kind == "a":
+                    got_a[i] = harness.execute(plain, 1, [xs_a[i]] + weights, device)[0]
+                else:
+                    got_b[i] = _run_traced(traced, device, xs_b[i], res_b)
+        except Exception as e:   # surfaced in the main thread below
+            errors.append(e)
+    threads = [threading.Thread(target=worker, args=(k,)) for k in ("a", "b")]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    assert all(torch.equal(a, b) for a, b in zip(got_a, want_a)) and all(torch.equal(a, b) for a, b in zip(got_b, want_b))
+
+
 def test_submit_errors(device):
     binary = rt.Binary.load_from_memory(programs.c3_linear(32, 64, 64))
     a = rt.from_torch(torch.zeros(32, 64, dtype=torch.bfloat16))

@@ -729,6 +729,7 @@ void wait(Event) {}
 void wait(Tensor t, std::optional<std::uint8_t>) {
   TTRT_ASSERT(t.handle != nullptr, "wait: null tensor");
   if (t.handle->storage == StorageType::Device && t.handle->device && t.handle->device->open) {
+    std::lock_guard<std::recursive_mutex> g(t.handle->device->mu);
     requireNotCapturing(t.handle->device, "wait");
     TTM_CALL(ttm_stream_sync(t.handle->device->stream));
   }
@@ -818,6 +819,7 @@ Tensor convertOnDevice(const Tensor &src, TensorLayout layout, DataType dtype) {
 Tensor toLayout(Tensor tensor, Device device, Layout layout, std::optional<bool> retain) {
   TTRT_ASSERT(isTensorAllocated(tensor), "toLayout: tensor is deallocated");
   TTRT_ASSERT(device.handle && device.handle->open, "toLayout: device is not open");
+  std::lock_guard<std::recursive_mutex> g(device.handle->mu);
   Tensor cur = tensor;
   const bool needsDevice = layout.storageType == StorageType::Device || cur.handle->layout != layout.layout ||
                            cur.handle->dtype != layout.dataType;
@@ -841,6 +843,8 @@ Tensor toLayout(Tensor tensor, Device device, Layout layout, std::optional<bool>
 std::vector<Tensor> toHost(Tensor tensor, bool untilize, bool /*blocking*/) {
   TTRT_ASSERT(isTensorAllocated(tensor), "toHost: tensor is deallocated");
   if (tensor.handle->storage == StorageType::Host) return {tensor};
+  std::unique_lock<std::recursive_mutex> g;
+  if (tensor.handle->device) g = std::unique_lock<std::recursive_mutex>(tensor.handle->device->mu);
   Tensor cur = tensor;
   if (untilize) {
     // block-float tensors read back as float32 (runtime/lib/ttnn/runtime.cpp:450-466)
@@ -866,6 +870,9 @@ void memcpy(Tensor dst, Tensor src) {
   TTRT_ASSERT(isTensorAllocated(dst) && isTensorAllocated(src), "memcpy: tensor is deallocated");
   TTRT_ASSERT(dst.handle->bytes == src.handle->bytes, "memcpy: tensors differ in size");
   const bool dDev = dst.handle->storage == StorageType::Device, sDev = src.handle->storage == StorageType::Device;
+  std::unique_lock<std::recursive_mutex> g;
+  if (dDev && dst.handle->device) g = std::unique_lock<std::recursive_mutex>(dst.handle->device->mu);
+  else if (sDev && src.handle->device) g = std::unique_lock<std::recursive_mutex>(src.handle->device->mu);
   if (!dDev && !sDev) {
     std::memcpy(dst.handle->data.get(), src.handle->data.get(), src.handle->bytes);
   } else if (dDev && !sDev) {
@@ -884,6 +891,9 @@ void memcpy(Tensor dst, Tensor src) {
 std::vector<Tensor> submit(Device device, Binary binary, std::uint32_t programIndex, std::vector<Tensor> &inputs) {
   TTRT_ASSERT(device.handle && device.handle->open, "submit: device is not open");
   TTRT_ASSERT(binary.handle != nullptr, "submit: null binary");
+  // one program at a time per device: its launches share one stream, one workspace and, while a trace is being captured,
+  // one recording.  Threads that drive different devices do not meet here (test/python/.../test_data_parallel.py:58-75).
+  std::lock_guard<std::recursive_mutex> programLock(device.handle->mu);
   try {
     return executeProgram(device.handle, binary, programIndex, inputs);
   } catch (...) {

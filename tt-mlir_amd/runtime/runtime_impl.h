@@ -37,7 +37,10 @@ struct DeviceState {
   int deviceId = 0;
   void *stream = nullptr;  // hipStream_t: all work of this device is ordered on it
   bool open = false;
-  std::mutex mu;           // submit is re-entrant per device, one program at a time per stream
+  // Work on the stream of a device is issued by one thread at a time: submit, toLayout, toHost, wait and device copies
+  // take this lock (recursive: a hook running inside submit may call toHost).  A capture in progress is thereby never
+  // interleaved with the launches or the synchronisation of another thread.
+  std::recursive_mutex mu;
   // trace state
   bool capturing = false;                         // between begin_trace_capture and end_trace_capture
   std::uint32_t capturingTraceId = 0;
