@@ -124,6 +124,11 @@ int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int trans
 int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias, int bias_dtype,
                     int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N,
                     int64_t K, int act, int tail_op, const void *tail, void *stream);
+/* out0 = a w0 and out1 = a w1 in one launch, for two weight tensors of one shape and format applied to the same activations
+ * (the K and V projections of an attention layer); the two weight tensors and the two outputs may live anywhere.  No bias,
+ * activation or tail.  One launch fills the device where two small ones would each leave part of it idle. */
+int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M, int64_t N,
+                    int64_t K, void *stream);
 
 /* ---- elementwise: ::ttnn::<unary>, ::ttnn::<binary>
  * (runtime/lib/ttnn/operations/eltwise/unary/unary.cpp:159-205, eltwise/binary/binary.cpp:38-126;

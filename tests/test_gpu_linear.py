@@ -307,3 +307,28 @@ def test_batched_block_float_matmul(hip, dev, orc, metrics, split):
         hip.set_option("linear_split_k", 0)
     want = orc.round_bf16(orc.matmul(a.float().numpy(), w_eff.numpy()))
     assert np.max(np.abs(got.float().numpy() - want)) <= 2.0 ** -5
+
+
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4"])
+@pytest.mark.parametrize("M,K,N,second_first", [(32, 4096, 1024, False), (20, 1200, 200, True), (330, 232, 677, False),
+                                                (2048, 512, 1024, True)])
+def test_linear_pair_equals_two_launches(hip, dev, wfmt_name, M, K, N, second_first):
+    """ttm_linear_pair (two weight matrices of one shape against the same activations in one launch) against two ttm_linear
+    calls: bit exact, whichever of the two allocations lies first in memory (the stride between them is signed)."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    a = datagen.randn((M, K), seed=71, dtype=torch.bfloat16)
+    ws = [datagen.randn((K, N), seed=72 + i, std=0.05) for i in range(2)]
+    want = [run_linear(hip, dev, a, w, None, None, wfmt)[0] for w in ws]
+    at = tilize_dev(hip, a, dev)
+    wt = [pack_weight(hip, w, wfmt, dev) for w in ws]
+    Mp, Np = (M + 31) // 32 * 32, (N + 31) // 32 * 32
+    both = torch.full((2, Mp * Np), float("nan"), dtype=torch.bfloat16, device=dev)
+    o = [both[1], both[0]] if second_first else [both[0], both[1]]
+    hip.call("ttm_linear_pair", hip.ptr(at), hip.ptr(wt[0]), hip.ptr(wt[1]), wfmt, hip.ptr(o[0]), hip.ptr(o[1]), M, N, K,
+             hip.current_stream())
+    for i in range(2):
+        got = untilize_dev(hip, o[i], (M, N), dev).cpu()
+        assert torch.equal(got, want[i])
+    with pytest.raises(hip.TTMError, match="two distinct"):
+        hip.call("ttm_linear_pair", hip.ptr(at), hip.ptr(wt[0]), hip.ptr(wt[0]), wfmt, hip.ptr(o[0]), hip.ptr(o[1]), M, N, K,
+                 hip.current_stream())

@@ -560,6 +560,7 @@ def test_fused_epilogue_tails_do_not_change_program_results(device):
     rt.clear_stats()
     (fused,) = harness.execute(binary, 1, tins, device)
     assert rt.get_stat("FusedLinearTail") == 3          # attention residual, gate * up, MLP residual
+    assert rt.get_stat("PairedMatmul") == 1             # K and V projections in one launch
     seen = []
     rt.set_post_op_callback(lambda idx, name, dbg, hook: seen.append(name))
     try:

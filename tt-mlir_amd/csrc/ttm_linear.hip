@@ -1464,9 +1464,11 @@ TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype
                          TTM_TAIL_NONE, nullptr, stream);
 }
 
-TTM_EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias,
-                               int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch,
-                               int64_t M, int64_t N, int64_t K, int act, int tail_op, const void *tail, void *stream) {
+// strides: optional byte strides between batch entries of the activations, weights and output, for operands that are not
+// stored back to back (a pair of weight matrices applied to the same activations)
+static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias, int bias_dtype,
+                        int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K,
+                        int act, int tail_op, const void *tail, const int64_t *strides, void *stream) {
   TTM_REQUIRE(tail_op >= TTM_TAIL_NONE && tail_op <= TTM_TAIL_MUL, "ttm_linear: unknown tail op %d", tail_op);
   TTM_REQUIRE((tail_op == TTM_TAIL_NONE) == (tail == nullptr), "ttm_linear: a tail op needs its operand, and only then");
   TTM_REQUIRE(((uintptr_t)tail & 15) == 0, "ttm_linear: the tail operand must be 16-byte aligned");
@@ -1500,6 +1502,7 @@ TTM_EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_
   p.nt_split = p.n_blocks1 = p.ntw2 = 0;
   p.tail = tail_op;
   p.tail_delta = tail ? (const uint8_t *)tail - (const uint8_t *)out : 0;
+  if (strides) { p.a_batch = strides[0]; p.w_batch = strides[1]; p.c_batch = strides[2]; }
   TTM_REQUIRE(batch <= 65535, "ttm_linear: batch too large");
   hipStream_t s = (hipStream_t)stream;
   int rc;
@@ -1510,4 +1513,20 @@ TTM_EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_
   if (rc) return rc;
   TTM_LAUNCH_CHECK();
   return TTM_OK;
+}
+
+TTM_EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias,
+                               int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch,
+                               int64_t M, int64_t N, int64_t K, int act, int tail_op, const void *tail, void *stream) {
+  return linear_entry(a, a_dtype, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, act,
+                      tail_op, tail, nullptr, stream);
+}
+
+TTM_EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M,
+                               int64_t N, int64_t K, void *stream) {
+  TTM_REQUIRE(w0 && w1 && out0 && out1 && w0 != w1 && out0 != out1, "ttm_linear_pair: two distinct weight and output tensors are needed");
+  TTM_REQUIRE((((uintptr_t)w1 | (uintptr_t)out1) & 15) == 0, "ttm_linear_pair: operands must be 16-byte aligned");
+  const int64_t strides[3] = {0, (const uint8_t *)w1 - (const uint8_t *)w0, (uint8_t *)out1 - (uint8_t *)out0};
+  return linear_entry(a, TTM_BF16, w0, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, out0, TTM_BF16, 2, 2, M, N, K, TTM_ACT_NONE,
+                      TTM_TAIL_NONE, nullptr, strides, stream);
 }

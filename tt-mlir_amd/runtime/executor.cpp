@@ -334,6 +334,42 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
       }
     }
   }
+  // A second matmul of the same activations with a weight tensor of the same shape and format (the K and V projections)
+  // a few ops further on runs in this launch; only reshapes, permutes and deallocations of other tensors may lie between.
+  if (ctx.fuseViews && tailOp == TTM_TAIL_NONE && !biasRef && activation.empty() && !transposeA && !transposeB && batch == 1 &&
+      utils::isBlockFormatDataType(b.handle->dtype) && layoutFromTensorRef(outRef) == Layout{StorageType::Device, TensorLayout::Tile, DataType::BFloat16}) {
+    for (std::uint32_t j = ctx.opIndex + 1; j < ctx.ops.size() && j <= ctx.opIndex + 4; ++j) {
+      const OpType t = opType(j);
+      fb::Table nop = ctx.ops[j].table(schema::Operation::f_type);
+      if (t == OpType::ReshapeOp || t == OpType::PermuteOp) continue;
+      if (t == OpType::DeallocateOp) {
+        const std::uint32_t freed = refId(nop.table(schema::DeallocateOp::f_in));
+        if (freed == refId(aRef) || freed == refId(outRef)) break;
+        continue;
+      }
+      if (t != OpType::MatmulOp || ctx.skip.count(j)) break;
+      using M2 = schema::MatmulOp;
+      fb::Table a2 = nop.table(M2::f_a), b2 = nop.table(M2::f_b), out2 = nop.table(M2::f_out);
+      if (!a2 || !b2 || !out2 || refId(a2) != refId(aRef) || nop.scalar<std::uint8_t>(M2::f_transpose_a, 0) ||
+          nop.scalar<std::uint8_t>(M2::f_transpose_b, 0) || !nop.string(M2::f_activation).empty())
+        break;
+      auto wit = ctx.pool.find(refId(b2));
+      if (wit == ctx.pool.end() || !isTensorAllocated(wit->second) || wit->second.handle->storage != StorageType::Device ||
+          wit->second.handle->dtype != b.handle->dtype || wit->second.handle->shape != b.handle->shape ||
+          wit->second.handle->data.get() == b.handle->data.get() || !(layoutFromTensorRef(out2) == layoutFromTensorRef(outRef)) ||
+          shapeFromTensorRef(out2) != shapeFromTensorRef(outRef))
+        break;
+      // the second matmul must not be followed by a fusable tail of its own: it keeps its plain form here
+      Tensor outB = makeOut(ctx, out2, DataType::BFloat16, TensorLayout::Tile);
+      TTM_CALL(ttm_linear_pair(a.handle->data.get(), b.handle->data.get(), wit->second.handle->data.get(), ttmDtype(b.handle->dtype),
+                               out.handle->data.get(), outB.handle->data.get(), M, N, K, ctx.stream()));
+      ctx.put(outRef, out);
+      ctx.put(out2, outB);
+      ctx.skip.insert(j);
+      debug::Stats::get().incrementStat("PairedMatmul");
+      return;
+    }
+  }
   TTM_CALL(ttm_linear_tail(a.handle->data.get(), TTM_BF16, b.handle->data.get(), ttmDtype(b.handle->dtype), transposeB ? 1 : 0, biasPtr,
                            TTM_BF16, biasLayout, out.handle->data.get(), TTM_BF16, batch, wbatch == 1 ? 1 : batch, M, N, K,
                            activationCode(activation), tailOp, tail ? tail.handle->data.get() : nullptr, ctx.stream()));
