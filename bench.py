@@ -98,9 +98,15 @@ def make_workloads(torch, hip, datagen, dev, names):
         ot = torch.empty(M * N, dtype=torch.bfloat16, device=dev)
         torch.cuda.synchronize()
         del wd
-        fn = (lambda at=at, wt=wt, bt=bt, ot=ot, M=M: hip.call(
-            "ttm_linear", hip.ptr(at), hip.BF16, hip.ptr(wt), hip.BFP8B, 0, hip.ptr(bt), hip.BF16, hip.TILE,
-            hip.ptr(ot), hip.BF16, 1, 1, M, N, K, hip.ACT["gelu"], s))
+        # decode streams the weights once per launch: ten copies are cycled (624 MB) so that every launch reads them from
+        # HBM and not from the 256 MB last-level cache, as a layer stack of distinct weights would
+        wts = [wt] + ([wt.clone() for _ in range(9)] if M == 32 else [])
+        turn = [0]
+
+        def fn(at=at, wts=wts, bt=bt, ot=ot, M=M, turn=turn):
+            turn[0] = (turn[0] + 1) % len(wts)
+            hip.call("ttm_linear", hip.ptr(at), hip.BF16, hip.ptr(wts[turn[0]]), hip.BFP8B, 0, hip.ptr(bt), hip.BF16, hip.TILE,
+                     hip.ptr(ot), hip.BF16, 1, 1, M, N, K, hip.ACT["gelu"], s)
         if M == 2048:
             out[nm] = Workload(nm, "mfma", 2.0 * M * N * K, "flop", fn,
                                "config 3: bf16 [2048,4096] x bfp8_b [4096,14336] + bias + GELU",
@@ -108,7 +114,8 @@ def make_workloads(torch, hip, datagen, dev, names):
         else:
             nbytes = (K // 32) * (N // 32) * 1088 + 2 * M * K + 2 * M * N + 2 * N
             out[nm] = Workload(nm, "hbm", nbytes, "bytes", fn,
-                               "config 3 decode: bf16 [32,4096] x bfp8_b [4096,14336] + bias + GELU (weight streaming)",
+                               "config 3 decode: bf16 [32,4096] x bfp8_b [4096,14336] + bias + GELU (weight streaming; ten weight "
+                               "copies cycled, so each launch reads HBM)",
                                dict(flop=2.0 * M * N * K))
     if "sdpa_decode32" in names:
         B, H, Hkv, S, D = 32, 32, 8, 2048, 128
@@ -315,6 +322,16 @@ def main():
         "config": {"workload": prim.desc, "name": prim.name, "device": hip.device_name()},
         "roofline": rl, "secondary": secondary,
     }
+    if prim.name == "linear2048":
+        # the vendor library's plain bf16 x bf16 GEMM at the same M, N, K (weights already bf16: no block-float decode, no
+        # bias, no GELU), as a reference point for what the matrix cores sustain on this device at this shape
+        xa = torch.randn(2048, 4096, device=dev).to(torch.bfloat16)
+        xw = (0.02 * torch.randn(4096, 14336, device=dev)).to(torch.bfloat16)
+        lib_w = Workload("library_gemm", "mfma", prim.work, "flop", lambda: torch.matmul(xa, xw), "torch.matmul bf16 x bf16")
+        lms, _ = measure(lib_w, max(10, args.steps // 2), max(3, args.warmup // 2))
+        result["library_gemm"] = {"what": "torch.matmul bf16 [2048,4096] x bf16 [4096,14336] (vendor BLAS, no decode / bias / GELU)",
+                                  "ms_per_step": round(lms, 5), "value": round(prim.work / (lms * 1e-3) / 1e12, 1), "unit": "TFLOP/s"}
+        del xa, xw
     if not args.no_cpu_baseline:
         orc = entry.load_oracle()
         if "linear" in prim.name:

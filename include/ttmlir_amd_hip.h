@@ -172,6 +172,16 @@ int ttm_copy_view(const void *src, int64_t src_rows, int64_t src_cols, int src_l
                   int64_t dst_rows, int64_t dst_cols, int dst_layout, int elem_bytes, int rank,
                   const int64_t *extent, const int64_t *src_stride, int64_t src_base,
                   const int64_t *dst_stride, int64_t dst_base, void *stream);
+/* ttm_copy_view whose destination base is advanced by a position held in DEVICE memory (read by the kernel, so the
+ * launch can be recorded into a graph): dst_base + *index * index_stride; an *index outside [0, index_limit) writes
+ * nothing.  With dst = a KV cache [users, heads, max_seq, head_dim], index_stride = head_dim and index_limit = max_seq
+ * this is ::ttnn::update_cache (runtime/lib/ttnn/operations/kv_cache/update_cache.cpp:14-60) reading its input through a
+ * view, i.e. with the permute / reshape that produces the [1, heads, users, head_dim] operand folded in. */
+int ttm_copy_view_at(const void *src, int64_t src_rows, int64_t src_cols, int src_layout, void *dst,
+                     int64_t dst_rows, int64_t dst_cols, int dst_layout, int elem_bytes, int rank,
+                     const int64_t *extent, const int64_t *src_stride, int64_t src_base,
+                     const int64_t *dst_stride, int64_t dst_base, const int32_t *index, int64_t index_stride,
+                     int64_t index_limit, void *stream);
 
 /* ---- attention: ::ttnn::transformer::scaled_dot_product_attention
  * (runtime/lib/ttnn/operations/transformer/scaled_dot_product_attention.cpp:14-55; golden

@@ -479,8 +479,11 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
     f = lambda t: t.float().numpy()
     order = ["anw", "wq", "wk", "wv", "wo", "mnw", "wg", "wu", "wd"]
     results = {}
-    for mode in ("eager", "traced"):
+    for mode in ("eager", "traced", "callbacks"):
         binary = rt.Binary.load_from_memory(programs.decode_layer(users, hidden, n_q, n_kv, hd, ffn, max_seq, trace=mode == "traced"))
+        rt.clear_stats()
+        if mode == "callbacks":   # with a callback registered nothing is fused: every op leaves its own output
+            rt.set_post_op_callback(lambda idx, name, dbg, hook: None)
         main = binary.get_num_programs() - 1
         lay = lambda k: rt.get_layout(binary, main, k)
         caches = [rt.to_layout(rt.from_torch(t.clone()), device, lay(5 + i), retain=True) for i, t in enumerate((kc0, vc0))]
@@ -493,11 +496,20 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
             (y,) = rt.submit(device, binary, main, ins)
             outs.append(rt.to_torch(rt.to_host(y, untilize=True)[0]))
         results[mode] = (outs, [rt.to_torch(rt.to_host(c, untilize=True)[0]) for c in caches])
+        rt.clear_callbacks()
         if mode == "traced":
             assert rt.get_stat("CapturedTrace") >= 1
-    # the replayed graph runs the same kernels on the same data: identical to the op-by-op run, caches included
-    for a, b in zip(results["eager"][0] + results["eager"][1], results["traced"][0] + results["traced"][1]):
-        assert torch.equal(a, b)
+        # both cache writes read their permuted operand as a view (K after the rotary embedding, V straight from the
+        # reshaped projection), the K and V projections share a launch; nothing of this with a callback registered
+        # (a traced program runs its body op by op only until the graph is recorded)
+        fused, paired = rt.get_stat("FusedCacheUpdate"), rt.get_stat("PairedMatmul")
+        assert (fused, paired) == {"eager": (6, 3), "callbacks": (0, 0)}.get(mode, (fused, paired))
+        assert mode != "traced" or (fused in (2, 4) and paired * 2 == fused)
+    # the replayed graph runs the same kernels on the same data: identical to the op-by-op run, caches included; so is
+    # the unfused run
+    for other in ("traced", "callbacks"):
+        for a, b in zip(results["eager"][0] + results["eager"][1], results[other][0] + results[other][1]):
+            assert torch.equal(a, b)
     # against the CPU oracle, step by step
     kc, vc = f(kc0), f(vc0)
     for step, pos in enumerate((40, 41, 42)):
@@ -549,6 +561,46 @@ def test_reshape_permute_pairs_are_fused_without_changing_results(device, shape,
         assert torch.equal(got, want_z)
     unfused_copies = rt.get_stat("CopyViewLaunch") - fused_copies
     assert fused_copies < unfused_copies, (fused_copies, unfused_copies)
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("index,offset", [(5, 0), (63, 2), (64, 0), (-1, 1)])
+def test_update_cache_reads_a_permuted_view(device, dtype, index, offset):
+    """update_cache(cache, permute(reshape(x)), index, batch_offset): without callbacks the reshape and the permute are
+    never materialised, the cache write is one strided copy from x.  Equal, bit for bit, to the op-by-op run and to
+    the definition cache[offset + b, h, index, :] = x[b, h, :]; an index outside the cache writes nothing."""
+    users, heads, max_seq, hd, in_users = 6, 3, 64, 32, 4
+    tdt, ddt = (torch.bfloat16, DT.BFloat16) if dtype == "bf16" else (torch.float32, DT.Float32)
+    pb = rt.ProgramBuilder()
+    pb.begin_program("cache_write")
+    cache = pb.input((users, heads, max_seq, hd), ddt)
+    x = pb.input((in_users, heads * hd), ddt)
+    idx = pb.input((1,), DT.Int32, TL.RowMajor)
+    pb.update_cache(cache, pb.permute(pb.reshape(x, (1, in_users, heads, hd)), (0, 2, 1, 3)), idx, batch_offset=offset)
+    pb.output(pb.unary(programs.UNARY["relu"], x))    # a program needs a result; the cache is updated in place
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    g = torch.Generator().manual_seed(17)
+    c0 = torch.randn((users, heads, max_seq, hd), generator=g).to(tdt)
+    xin = torch.randn((in_users, heads * hd), generator=g).to(tdt)
+    want = c0.clone()
+    if 0 <= index < max_seq:
+        want[offset:offset + in_users, :, index, :] = xin.reshape(in_users, heads, hd)
+    got = {}
+    for mode in ("fused", "callbacks"):
+        rt.clear_stats()
+        if mode == "callbacks":
+            rt.set_post_op_callback(lambda i, name, dbg, hook: None)
+        try:
+            cdev = rt.to_layout(rt.from_torch(c0.clone()), device, rt.get_layout(binary, 0, 0), retain=True)
+            ins = [cdev, rt.to_layout(rt.from_torch(xin), device, rt.get_layout(binary, 0, 1)),
+                   rt.to_layout(rt.from_torch(torch.tensor([index], dtype=torch.int32)), device, rt.get_layout(binary, 0, 2))]
+            rt.submit(device, binary, 0, ins)
+            got[mode] = rt.to_torch(rt.to_host(cdev, untilize=True)[0])
+        finally:
+            rt.clear_callbacks()
+        assert rt.get_stat("FusedCacheUpdate") == (1 if mode == "fused" else 0)
+        assert torch.equal(got[mode], want), mode
 
 
 def test_fused_epilogue_tails_do_not_change_program_results(device):

@@ -28,11 +28,14 @@ struct ProgramContext {
   std::uint32_t programIndex = 0;
   std::unordered_map<std::uint32_t, Tensor> pool;  // global_id -> live tensor
   // reshape / permute fusion (only when no hooks are registered): a reshape whose single consumer is the next permute is
-  // not materialised (`deferred` keeps its source and logical shape), and a permute whose single consumer is the next
-  // reshape writes the reshaped tensor directly (the reshape's index goes into `skip`)
+  // not materialised, nor is a permute whose single consumer is the next update_cache (`deferred` keeps the source, the
+  // logical shape of the result and, per result dimension, the stride in the source's row-major element order); a
+  // permute whose single consumer is the next reshape writes the reshaped tensor directly (the reshape's index goes
+  // into `skip`)
   struct DeferredView {
     Tensor source;
     std::vector<std::uint32_t> shape;
+    std::vector<std::int64_t> strides;
   };
   std::vector<fb::Table> ops;
   std::uint32_t opIndex = 0;
@@ -605,6 +608,32 @@ void runUpdateCache(const fb::Table &op, ProgramContext &ctx) {
   using S = schema::UpdateCacheOp;
   Tensor &cache = cacheOperand(ctx, op.table(S::f_cache), "update_cache cache");
   const auto &cs = cache.handle->shape;
+  if (auto d = ctx.deferred.find(refId(op.table(S::f_input))); d != ctx.deferred.end()) {
+    // the input is a permuted / reshaped view that was not materialised: one strided copy from its source into the cache
+    // row of the position.  cache[batch_offset + b, h, *index, :] = view[0, h, b, :]
+    const ProgramContext::DeferredView v = d->second;
+    ctx.deferred.erase(d);
+    const auto &is = v.shape;
+    TTRT_ASSERT(is.size() == 4 && is[0] == 1 && is[1] == cs[1] && is[3] == cs[3],
+                "update_cache: input must be [1, heads, users, head_dim] matching the cache");
+    const std::int64_t users = cs[0], heads = cs[1], maxSeq = cs[2], hd = cs[3];
+    const std::int64_t offset = op.scalar<std::uint32_t>(S::f_batch_offset, 0);
+    TTRT_ASSERT(offset + is[2] <= users, "update_cache: batch_offset + input users exceeds the cache");
+    TTRT_ASSERT(v.source.handle->dtype == cache.handle->dtype, "update_cache: fused input has another element type than the cache");
+    Tensor index = devicePositions(ctx, ctx.get(op.table(S::f_update_index), "update_cache index"), "update_cache: update_index");
+    const std::int64_t extent[3] = {heads, static_cast<std::int64_t>(is[2]), hd};
+    const std::int64_t sst[3] = {v.strides[1], v.strides[2], v.strides[3]};
+    const std::int64_t dst[3] = {maxSeq * hd, heads * maxSeq * hd, 1};
+    Dims3 sd = dims3(v.source.handle->shape), dd = dims3(cs);
+    debug::Stats::get().incrementStat("CopyViewLaunch");
+    debug::Stats::get().incrementStat("FusedCacheUpdate");
+    TTM_CALL(ttm_copy_view_at(v.source.handle->data.get(), sd.rows, sd.cols, ttmLayout(v.source.handle->layout), cache.handle->data.get(),
+                              dd.rows, dd.cols, TTM_TILE, static_cast<int>(utils::dataTypeElementSize(cache.handle->dtype)), 3, extent,
+                              sst, 0, dst, offset * heads * maxSeq * hd, static_cast<const std::int32_t *>(index.handle->data.get()), hd,
+                              maxSeq, ctx.stream()));
+    cache.handle->version = nextTensorVersion();
+    return;
+  }
   Tensor in = as(ctx, ctx.get(op.table(S::f_input), "update_cache input"), TensorLayout::Tile, cache.handle->dtype);
   const auto &is = in.handle->shape;
   TTRT_ASSERT(is.size() == 4 && is[0] == 1 && is[1] == cs[1] && is[3] == cs[3],
@@ -736,32 +765,55 @@ void runReshape(const fb::Table &op, ProgramContext &ctx) {
   if (copies && !utils::isBlockFormatDataType(in.handle->dtype) &&
       fusableNext(ctx, OpType::PermuteOp, schema::PermuteOp::f_in, schema::PermuteOp::f_out, outRef, in)) {
     TTRT_ASSERT(volume(in.handle->shape) == volume(oshape), "reshape: element count differs");
-    ctx.deferred[refId(outRef)] = ProgramContext::DeferredView{in, oshape};   // the permute reads the source directly
+    ctx.deferred[refId(outRef)] = ProgramContext::DeferredView{in, oshape, rowMajorStrides(oshape)};   // the permute reads the source directly
     return;
   }
   ctx.put(outRef, finish(ctx, reshapeTo(ctx, in, oshape), outRef));
 }
 
-// out[i0, i1, ...] = in[i_perm...]; `viewShape` reinterprets the input's elements under another logical shape first (a
-// reshape is the identity on flat indices), `finalShape` gives the output another logical shape of the same volume
-Tensor permuteTo(ProgramContext &ctx, const Tensor &in, const std::vector<int> &perm, const std::vector<std::uint32_t> *viewShape = nullptr,
-                 const std::vector<std::uint32_t> *finalShape = nullptr) {
-  const auto &shape = viewShape ? *viewShape : in.handle->shape;
-  const size_t rank = shape.size();
+// A strided view of `source` written out as a tensor of its own: element v of the view (row-major over `shape`) is
+// the source element with row-major index sum v[d] * strides[d].  `finalShape` gives the output another logical shape
+// of the same volume (a reshape is the identity on flat indices).
+Tensor materialiseView(ProgramContext &ctx, const ProgramContext::DeferredView &v, const std::vector<std::uint32_t> *finalShape = nullptr) {
+  if (finalShape) TTRT_ASSERT(volume(*finalShape) == volume(v.shape), "reshape: element count differs");
+  Tensor out = makeDeviceTensor(ctx.dev, finalShape ? *finalShape : v.shape, v.source.handle->dtype, v.source.handle->layout);
+  zeroIfPadded(ctx, out);
+  copyView(ctx, v.source, out, toI64(v.shape), v.strides, 0, rowMajorStrides(v.shape), 0);
+  return out;
+}
+// out[i0, i1, ...] = in[i_perm...] as a view of the input (or of the view `in` already is)
+ProgramContext::DeferredView permutedView(const ProgramContext::DeferredView &in, const std::vector<int> &perm) {
+  const size_t rank = in.shape.size();
   TTRT_ASSERT(perm.size() == rank, "permute: permutation rank differs from the tensor rank");
-  std::vector<std::uint32_t> oshape(rank);
-  auto ss = rowMajorStrides(shape);
-  std::vector<std::int64_t> sst(rank);
+  ProgramContext::DeferredView out{in.source, std::vector<std::uint32_t>(rank), std::vector<std::int64_t>(rank)};
   for (size_t i = 0; i < rank; ++i) {
     TTRT_ASSERT(perm[i] >= 0 && static_cast<size_t>(perm[i]) < rank, "permute: index out of range");
-    oshape[i] = shape[perm[i]];
-    sst[i] = ss[perm[i]];
+    out.shape[i] = in.shape[perm[i]];
+    out.strides[i] = in.strides[perm[i]];
   }
-  if (finalShape) TTRT_ASSERT(volume(*finalShape) == volume(oshape), "reshape: element count differs");
-  Tensor out = makeDeviceTensor(ctx.dev, finalShape ? *finalShape : oshape, in.handle->dtype, in.handle->layout);
-  zeroIfPadded(ctx, out);
-  copyView(ctx, in, out, toI64(oshape), sst, 0, rowMajorStrides(oshape), 0);
   return out;
+}
+Tensor permuteTo(ProgramContext &ctx, const Tensor &in, const std::vector<int> &perm) {
+  return materialiseView(ctx, permutedView(ProgramContext::DeferredView{in, in.handle->shape, rowMajorStrides(in.handle->shape)}, perm));
+}
+// the next operation is an update_cache that is the only consumer of `produced` (as its input) and whose cache holds
+// the element type of `like`: it can read the view directly
+bool feedsUpdateCache(ProgramContext &ctx, const fb::Table &produced, const Tensor &like) {
+  if (!ctx.fuseViews || ctx.opIndex + 1 >= ctx.ops.size()) return false;
+  const fb::Table &next = ctx.ops[ctx.opIndex + 1];
+  if (static_cast<OpType>(next.scalar<std::uint8_t>(schema::Operation::f_type_type, 0)) != OpType::UpdateCacheOp) return false;
+  fb::Table nop = next.table(schema::Operation::f_type);
+  fb::Table in = nop.table(schema::UpdateCacheOp::f_input), cache = nop.table(schema::UpdateCacheOp::f_cache);
+  if (!in || !cache || refId(in) != refId(produced)) return false;
+  auto u = ctx.uses.find(refId(produced));
+  if (u == ctx.uses.end() || u->second != 1) return false;
+  Layout a = layoutFromTensorRef(produced);
+  if (a.storageType != StorageType::Device || a.layout != TensorLayout::Tile || a.dataType != like.handle->dtype ||
+      like.handle->layout != TensorLayout::Tile)
+    return false;
+  auto c = ctx.pool.find(refId(cache));
+  return c != ctx.pool.end() && isTensorAllocated(c->second) && c->second.handle->storage == StorageType::Device &&
+         c->second.handle->layout == TensorLayout::Tile && c->second.handle->dtype == like.handle->dtype;
 }
 void runPermute(const fb::Table &op, ProgramContext &ctx) {
   auto inRef = op.table(schema::PermuteOp::f_in);
@@ -769,27 +821,31 @@ void runPermute(const fb::Table &op, ProgramContext &ctx) {
   std::vector<int> perm;
   for (std::uint32_t i = 0; i < pv.size(); ++i) perm.push_back(static_cast<int>(pv[i] < 0 ? pv[i] + pv.size() : pv[i]));
   auto outRef = op.table(schema::PermuteOp::f_out);
-  Tensor in;
-  std::vector<std::uint32_t> viewShape;
+  ProgramContext::DeferredView in;
   auto d = ctx.deferred.find(refId(inRef));
   if (d != ctx.deferred.end()) {
-    in = d->second.source;
-    viewShape = d->second.shape;
+    in = d->second;
     ctx.deferred.erase(d);
   } else {
-    in = onDevice(ctx, ctx.get(inRef, "permute in"));
+    Tensor t = onDevice(ctx, ctx.get(inRef, "permute in"));
+    in = ProgramContext::DeferredView{t, t.handle->shape, rowMajorStrides(t.handle->shape)};
   }
-  const std::vector<std::uint32_t> *view = viewShape.empty() ? nullptr : &viewShape;
-  if (in.handle->layout == TensorLayout::Tile && !utils::isBlockFormatDataType(in.handle->dtype)) {
-    if (fb::Table rs = fusableNext(ctx, OpType::ReshapeOp, schema::ReshapeOp::f_in, schema::ReshapeOp::f_out, outRef, in)) {
+  ProgramContext::DeferredView view = permutedView(in, perm);
+  const Tensor &src = in.source;
+  if (src.handle->layout == TensorLayout::Tile && !utils::isBlockFormatDataType(src.handle->dtype)) {
+    if (feedsUpdateCache(ctx, outRef, src)) {
+      ctx.deferred[refId(outRef)] = view;   // the cache write reads the source directly
+      return;
+    }
+    if (fb::Table rs = fusableNext(ctx, OpType::ReshapeOp, schema::ReshapeOp::f_in, schema::ReshapeOp::f_out, outRef, src)) {
       auto finalRef = rs.table(schema::ReshapeOp::f_out);
       std::vector<std::uint32_t> finalShape = shapeFromTensorRef(finalRef);
-      ctx.put(finalRef, permuteTo(ctx, in, perm, view, &finalShape));
+      ctx.put(finalRef, materialiseView(ctx, view, &finalShape));
       ctx.skip.insert(ctx.opIndex + 1);
       return;
     }
   }
-  ctx.put(outRef, finish(ctx, permuteTo(ctx, in, perm, view), outRef));
+  ctx.put(outRef, finish(ctx, materialiseView(ctx, view), outRef));
 }
 void runTranspose(const fb::Table &op, ProgramContext &ctx) {
   Tensor in = onDevice(ctx, ctx.get(op.table(schema::TransposeOp::f_in), "transpose in"));
