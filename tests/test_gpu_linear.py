@@ -332,3 +332,62 @@ def test_linear_pair_equals_two_launches(hip, dev, wfmt_name, M, K, N, second_fi
     with pytest.raises(hip.TTMError, match="two distinct"):
         hip.call("ttm_linear_pair", hip.ptr(at), hip.ptr(wt[0]), hip.ptr(wt[0]), wfmt, hip.ptr(o[0]), hip.ptr(o[1]), M, N, K,
                  hip.current_stream())
+
+
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4"])
+@pytest.mark.parametrize("M,K,N,option,value,act,bias", [
+    (330, 200, 677, None, 0, "gelu", True),          # odd number of k-tiles, ragged everywhere
+    (330, 232, 677, "linear_split_k", 2, None, False),  # k-slices read the zero image past their end
+    (300, 520, 200, "linear_split_k", 4, "silu", True),
+    (512, 256, 1024, "linear_ntw", 3, None, True),   # 6-tile-wide blocks: the last block has columns to spare
+    (512, 256, 320, "linear_ntw", 2, "relu", False),
+    (2048, 512, 2048, None, 0, None, True),
+])
+def test_two_pass_launch_equals_the_fused_kernel(hip, dev, wfmt_name, M, K, N, option, value, act, bias):
+    """linear_two_pass = 2 dequantises the weights once into bf16 fragment images and runs the main loop without the
+    conversion; = 1 keeps the fused kernel.  Same arithmetic in the same order: bit-identical results."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    a = datagen.randn((M, K), seed=81, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=82, std=0.05)
+    b = datagen.randn((N,), seed=83, std=0.5, dtype=torch.bfloat16) if bias else None
+    got = {}
+    if option:
+        hip.set_option(option, value)
+    try:
+        for mode in (1, 2):
+            hip.set_option("linear_two_pass", mode)
+            got[mode], _ = run_linear(hip, dev, a, w, b, act, wfmt)
+    finally:
+        hip.set_option("linear_two_pass", 0)
+        if option:
+            hip.set_option(option, 0)
+    assert torch.equal(got[1], got[2])
+
+
+def test_two_pass_launch_with_batches_pairs_and_tails(hip, dev, orc, metrics):
+    """The image pass covers every weight set of a launch: per-batch weights, one shared set, a pair of separately
+    allocated matrices, and the element-wise tail still runs in the second pass's epilogue."""
+    try:
+        res = {}
+        for mode in (1, 2):
+            hip.set_option("linear_two_pass", mode)
+            a = datagen.randn((3, 288, 160), seed=91, dtype=torch.bfloat16)
+            own, _ = run_linear(hip, dev, a, datagen.randn((3, 160, 96), seed=92, std=0.1), None, None, hip.BFP8B)
+            shared, _ = run_linear(hip, dev, a, datagen.randn((1, 160, 96), seed=93, std=0.1), None, None, hip.BFP4B)
+            M, K, N = 330, 232, 677
+            x = datagen.randn((M, K), seed=94, dtype=torch.bfloat16)
+            ws = [pack_weight(hip, datagen.randn((K, N), seed=95 + i, std=0.05), hip.BFP8B, dev) for i in range(2)]
+            xt, tt = tilize_dev(hip, x, dev), tilize_dev(hip, datagen.randn((M, N), seed=97, dtype=torch.bfloat16), dev)
+            Mp, Np = (M + 31) // 32 * 32, (N + 31) // 32 * 32
+            both = torch.full((2, Mp * Np), float("nan"), dtype=torch.bfloat16, device=dev)
+            hip.call("ttm_linear_pair", hip.ptr(xt), hip.ptr(ws[1]), hip.ptr(ws[0]), hip.BFP8B, hip.ptr(both[0]), hip.ptr(both[1]), M, N, K,
+                     hip.current_stream())
+            tail = torch.full((Mp * Np,), float("nan"), dtype=torch.bfloat16, device=dev)
+            hip.call("ttm_linear_tail", hip.ptr(xt), hip.BF16, hip.ptr(ws[0]), hip.BFP8B, 0, None, hip.BF16, hip.TILE, hip.ptr(tail), hip.BF16,
+                     1, 1, M, N, K, hip.ACT["silu"], 2, hip.ptr(tt), hip.current_stream())
+            torch.cuda.synchronize()
+            res[mode] = [own, shared, both.cpu(), tail.cpu()]
+    finally:
+        hip.set_option("linear_two_pass", 0)
+    for x, y in zip(res[1], res[2]):
+        assert torch.equal(x.view(torch.int16), y.view(torch.int16))   # bit patterns: the padding may hold NaN

@@ -45,6 +45,7 @@ struct LinearArgs {
                                       // the rest cover [nt_split, Nt) at width ntw2; nt_split = 0: one part
   int k_slice;                        // k-tiles per grid.y slice (split-K); Kt when the reduction is not split
   float *partial;                     // split-K: fp32 partial sums [slices][Mt * Nt * 1024] in output tile order
+  int img_zero_step;                  // two-pass launch: W points at the dequantised images, this step index holds zeros
   int tail;                           // 0 none, 1 add, 2 multiply: element-wise tail with a tensor laid out like the output
   int64_t tail_delta;                 // byte distance from an output element to its tail operand
 };
@@ -739,7 +740,10 @@ TTM_EXPORT int ttm_debug_trace(void *dst, size_t bytes) {
 #define TTM_TRACE(slot) do { } while (0)
 #endif
 
-template <int WF, int NTW>
+// IMG = true is the second pass of a two-pass launch: p.W holds the weights already dequantised to bf16, one 4 KiB
+// LDS fragment image per (k-step, column tile) (ttm_linear_image_k), so a step's weights are a straight LDS-direct copy
+// and the conversion, the raw staging area and the exponent loads drop out of the loop.
+template <int WF, int NTW, bool IMG = false>
 __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, int nblk, int nt_first, int nt_end) {
   static_assert(WF == WF_BFP8 || WF == WF_BFP4, "block-float weights only");
   constexpr int MB = 2;          // row tiles (32 m) per wavefront
@@ -837,7 +841,19 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     for (int i = 0; i < 4; ++i)
       if (i >= i0 && i < i1) lds_dma16(base, dmaA[i] + (dmaA_sub[i] ? sub : 0u), lds0 + stage_off + (uint32_t)(wave * 256 + i * 64) * 16u);
   };
+  // second pass: instructions [i0, i1) of the four that copy this wavefront's column tile image of step `step` (counted
+  // from the slice's first k-step) into the weight stage; steps past the slice's end read the all-zero image
+  auto issue_img = [&](int step, uint32_t stage_off, int i0 = 0, int i1 = 4) {
+    if (wave >= BN) return;   // wavefront-uniform: one image per column tile of the block
+    const int ksg = (kbase >> 1) + step;
+    const int ksc = kbase + 2 * step < kt_end ? ksg : p.img_zero_step;
+    const uint8_t *base = W + ((int64_t)ksc * p.Nt + min(nt0 + wave, p.Nt - 1)) * 4096;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i >= i0 && i < i1) lds_dma16(base, (uint32_t)(lane * 16 + i * 1024), lds0 + LDS_W + stage_off + (uint32_t)(wave * 4096 + i * 1024));
+  };
   auto issue_raw = [&](int kt0, uint32_t stage_off) {
+    if constexpr (IMG) return;
     if (!converts) return;
     const int kt = min(kbase + kt0 + ukt, p.Kt - 1);
     const uint8_t *row = W + (int64_t)kt * p.Nt * W_TILE;
@@ -853,6 +869,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   // The mask is applied when the value is taken into use; masking right behind the load would wait for it, and with
   // it for every LDS-direct load issued before.
   auto load_exps = [&](int kt0, uint32_t &keep) {
+    if constexpr (IMG) { keep = 0; return u32x2{0, 0}; }
     kt0 += kbase;
     const int kt = min(kt0 + ukt, p.Kt - 1);
     keep = kt0 + ukt >= kt_end ? 0u : 0xFFFFFFFFu;
@@ -866,6 +883,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   };
   // conversion quarter c: rows 2c, 2c+1 of the lane's block from the raw stage at raw_off; c == 3 stores the block
   auto quarter = [&](int c, uint32_t raw_off, uint32_t w_off) {
+    if constexpr (IMG) return;
     if (!converts) return;
     float f[2][4];
 #pragma unroll
@@ -921,6 +939,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
 
   // ---- prologue: step 0 staged and converted, step 1 staged and its first quarter converted
   issue_a(0, 0);
+  if constexpr (IMG) issue_img(0, 0);
   issue_raw(0, 0);
   issue_raw(2, RAW_STAGE);
   exps = load_exps(0, keep);
@@ -932,6 +951,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   landed_barrier();            // weights of step 0 visible, raw stage 0 free
   exps = u32x2{exps.x & keep, exps.y & keep};
   issue_a(2, STAGE);
+  if constexpr (IMG) issue_img(1, STAGE);
   issue_raw(4, 0);
   exps_next = load_exps(4, keep_next);
   fetch(0, 0, fw[0], fa[0]);
@@ -956,6 +976,10 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
       // spread over three chunks (1 + 2 + 1) so that no wavefront queues behind the whole block's burst
       if (q == 0 && ks > 0) issue_a((ks + 1) * 2, NXT, 1, 3);
       if (q == 1 && ks > 0) issue_a((ks + 1) * 2, NXT, 3, 4);
+      if constexpr (IMG) {
+        if (q == 0 && ks > 0) issue_img(ks + 1, NXT, 1, 3);
+        if (q == 1 && ks > 0) issue_img(ks + 1, NXT, 3, 4);
+      }
       fetch(q + 1, CUR, fw[(q + 1) & 1], fa[(q + 1) & 1]);
       quarter(q + 1, RNXT, NXT);
       mfma_chunk(q & 1);
@@ -975,6 +999,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     exps_next = load_exps((ks + 3) * 2, keep_next);
     issue_raw((ks + 3) * 2, RNXT);
     issue_a((ks + 2) * 2, CUR, 0, 1);
+    if constexpr (IMG) issue_img(ks + 2, CUR, 0, 1);
     fetch(0, NXT, fw[0], fa[0]);
     quarter(0, RCUR, CUR);
     mfma_chunk(1);
@@ -1003,6 +1028,69 @@ __global__ __launch_bounds__(512) void ttm_linear_dma_k(LinearArgs p) {
   if (ntw == 4) linear_dma_block<WF, 4>(p, bid, nblk, first, end);
   else if (ntw == 3) linear_dma_block<WF, 3>(p, bid, nblk, first, end);
   else linear_dma_block<WF, 2>(p, bid, nblk, first, end);
+}
+
+template <int WF>
+__global__ __launch_bounds__(512) void ttm_linear_img_k(LinearArgs p) {
+  int bid = blockIdx.x, nblk = gridDim.x, first = 0, end = p.Nt, ntw = p.ntw;
+  if (p.nt_split > 0) {   // workgroup-uniform
+    if (bid < p.n_blocks1) { nblk = p.n_blocks1; end = p.nt_split; }
+    else { bid -= p.n_blocks1; nblk -= p.n_blocks1; first = p.nt_split; ntw = p.ntw2; }
+  }
+  if (ntw == 4) linear_dma_block<WF, 4, true>(p, bid, nblk, first, end);
+  else if (ntw == 3) linear_dma_block<WF, 3, true>(p, bid, nblk, first, end);
+  else linear_dma_block<WF, 2, true>(p, bid, nblk, first, end);
+}
+
+// First pass of a two-pass launch: block-float tiles -> bf16 LDS fragment images.  img[(ks * Nt + nt) * 4096 ..] is the
+// 32 (n) x 64 (k) block of k-step ks and column tile nt exactly as the main loop wants it in LDS (row n, eight 16-byte
+// chunks of 8 k, chunk slot swizzled by the row).  k-tiles at or past Kt - the second half of the last step when Kt is
+// odd, and the extra step ks = ceil(Kt / 2) that slices read past their end - are zeros.  Same arithmetic as the fused
+// kernel's conversion, so both routes give identical results.
+// grid (ceil(Nt / 4), ceil(Kt / 2) + 1, weight sets), 256 lanes: half-wavefront h converts k-tile 2 ks + (h >> 2) of
+// column tile 4 x + (h & 3); a lane owns an 8 (k) x 4 (n) block as in the decode kernel.
+template <bool BFP4>
+__global__ __launch_bounds__(256) void ttm_linear_image_k(const uint8_t *W, int64_t w_batch, uint8_t *img, int64_t img_batch, int Nt, int Kt) {
+  constexpr uint32_t TB = BFP4 ? 576u : 1088u, FACE = BFP4 ? 128u : 256u, ROW = BFP4 ? 8u : 16u;
+  const int tid = threadIdx.x, h = tid >> 5, wq = tid & 31;
+  const int ks = blockIdx.y, nt = 4 * blockIdx.x + (h & 3), kt = 2 * ks + (h >> 2);
+  if (nt >= Nt) return;
+  const int face = wq >> 3, khalf = (wq >> 2) & 1, quad = wq & 3;
+  u32x4 out[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) out[j] = u32x4{0, 0, 0, 0};
+  if (kt < Kt) {
+    const uint8_t *t = W + (int64_t)blockIdx.z * w_batch + ((int64_t)kt * Nt + nt) * TB;
+    const u32x2 ex = *(const u32x2 *)(t + face * 16 + khalf * 8);
+    const uint8_t *m = t + 64 + face * FACE + khalf * (FACE / 2) + quad * (ROW / 4);
+    uint32_t rows[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) rows[i] = BFP4 ? (uint32_t) * (const uint16_t *)(m + i * ROW) : *(const uint32_t *)(m + i * ROW);
+    float f[8][4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      uint32_t E = ((i < 4 ? ex.x : ex.y) >> (8 * (i & 3))) & 0xFFu;
+      constexpr uint32_t EB = BFP4 ? 2u : 6u, SIGN = BFP4 ? 0x08080808u : 0x80808080u, SH = BFP4 ? 3u : 7u;
+      E = max(E, EB);
+      const float scale = __uint_as_float((E - EB) << 23), nscale = (BFP4 ? -8.0f : -128.0f) * scale;
+      uint32_t d = rows[i];
+      if (BFP4) {
+        d = (d | (d << 8)) & 0x00FF00FFu;
+        d = (d | (d << 4)) & 0x0F0F0F0Fu;
+      }
+      const uint32_t sg = d & SIGN, sb = sg >> SH;
+      const uint32_t tt = (d ^ SIGN ^ (sg - sb)) + sb;
+#pragma unroll
+      for (int b = 0; b < 4; ++b) f[i][b] = fmaf((float)((tt >> (8 * b)) & 0xFFu), scale, nscale);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      out[j] = u32x4{pack_hi(f[0][j], f[1][j]), pack_hi(f[2][j], f[3][j]), pack_hi(f[4][j], f[5][j]), pack_hi(f[6][j], f[7][j])};
+  }
+  u32x4 *dst = (u32x4 *)(img + (int64_t)blockIdx.z * img_batch + ((int64_t)ks * Nt + nt) * 4096);
+  const int kc = (h >> 2) * 4 + (face >> 1) * 2 + khalf, n0 = (face & 1) * 16 + quad * 4;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) dst[lds_chunk(n0 + j, kc)] = out[j];
 }
 
 // =============================================================================================
@@ -1426,16 +1514,49 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         p.k_slice += p.k_slice & 1;                         // whole k-steps per slice
         slices = (a.Kt + p.k_slice - 1) / p.k_slice;
       }
-      if (slices <= 1) {
-        hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, 1, (unsigned)batch), dim3(512), lds6, s, p);
-        return 0;
+      // Two passes when the conversion is repeated often enough: every block of 256 rows dequantises the weights it
+      // multiplies, so with M / 256 row blocks the same conversion runs M / 256 times.  The first pass writes the weights
+      // once as bf16 fragment images into the stream's workspace, the second runs the main loop without conversion
+      // (measured at [2048, 4096] x [4096, 14336]: 243 us fused; 30 us for the image pass + 193 us for the second pass).
+      // Modelled: the fused loop costs what plan_dma_grid says, the second pass 0.78 of it, the first pass 3 us +
+      // (tile bytes + 2048) per tile at 5.5 TB/s.  Launches that split K are left fused: measured, their second pass gains
+      // under 10 % ([2048, 14336] x [14336, 4096]: 232 us fused, 242 us in two passes).
+      // linear_two_pass: 0 = by the model, 1 = never, 2 = always.
+      const int ksteps = (a.Kt + 1) / 2;
+      const int64_t sets = a.w_batch == 0 ? 1 : batch;
+      const int64_t img_set = (int64_t)(ksteps + 1) * a.Nt * 4096;
+      bool two_pass = ttm_option("linear_two_pass") == 2;
+      if (ttm_option("linear_two_pass") == 0) {
+        static const double width_cost[5] = {0, 0, 0.78, 0.92, 1.0};
+        const int64_t rounds = ((int64_t)p.n_blocks * slices * batch + cus - 1) / cus;
+        const double fused = rounds * width_cost[p.ntw] * ((ksteps + slices - 1) / slices + 12) * 1.65;
+        const double first = 3.0 + (double)sets * a.Kt * a.Nt * ((WF == WF_BFP8 ? 1088.0 : 576.0) + 2048.0) / 5.5e6;
+        two_pass = slices == 1 && 0.22 * fused > first && img_set < ((int64_t)1 << 31);
       }
       const int64_t per = (int64_t)a.Mt * a.Nt * 1024;
-      void *ws = nullptr;
-      if (int rc = ttm_stream_workspace(s, (size_t)(per * slices * batch) * sizeof(float), &ws)) return rc;
-      p.partial = (float *)ws;
-      hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), lds6, s, p);
-      hipLaunchKernelGGL(ttm_linear_reduce_k, dim3((unsigned)((per / 4 + 255) / 256), 1, (unsigned)batch), dim3(256), 0, s, p, slices);
+      const size_t img_bytes = two_pass ? (size_t)((img_set * sets + 255) / 256 * 256) : 0;
+      const size_t part_bytes = slices > 1 ? (size_t)(per * slices * batch) * sizeof(float) : 0;
+      uint8_t *ws = nullptr;
+      if (img_bytes + part_bytes > 0)
+        if (int rc = ttm_stream_workspace(s, img_bytes + part_bytes, (void **)&ws)) return rc;
+      if (slices > 1) p.partial = (float *)(ws + img_bytes);
+      if (two_pass) {
+        static bool attr2 = false;
+        if (!attr2) {
+          if (int rc = set_lds_limit(ttm_linear_img_k<WF>, 131072)) return rc;
+          attr2 = true;
+        }
+        hipLaunchKernelGGL((ttm_linear_image_k<WF == WF_BFP4>), dim3((a.Nt + 3) / 4, ksteps + 1, (unsigned)sets), dim3(256), 0, s, a.W, a.w_batch,
+                           ws, img_set, a.Nt, a.Kt);
+        p.W = ws;
+        p.w_batch = a.w_batch == 0 ? 0 : img_set;
+        p.img_zero_step = ksteps;
+        hipLaunchKernelGGL((ttm_linear_img_k<WF>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), 131072, s, p);
+      } else {
+        hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), lds6, s, p);
+      }
+      if (slices > 1)
+        hipLaunchKernelGGL(ttm_linear_reduce_k, dim3((unsigned)((per / 4 + 255) / 256), 1, (unsigned)batch), dim3(256), 0, s, p, slices);
       return 0;
     }
   }
@@ -1500,6 +1621,7 @@ static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, 
   p.ntw = 4;
   p.k_slice = p.Kt; p.partial = nullptr;
   p.nt_split = p.n_blocks1 = p.ntw2 = 0;
+  p.img_zero_step = 0;
   p.tail = tail_op;
   p.tail_delta = tail ? (const uint8_t *)tail - (const uint8_t *)out : 0;
   if (strides) { p.a_batch = strides[0]; p.w_batch = strides[1]; p.c_batch = strides[2]; }
