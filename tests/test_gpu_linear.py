@@ -342,6 +342,9 @@ def test_linear_pair_equals_two_launches(hip, dev, wfmt_name, M, K, N, second_fi
     (512, 256, 1024, "linear_ntw", 3, None, True),   # 6-tile-wide blocks: the last block has columns to spare
     (512, 256, 320, "linear_ntw", 2, "relu", False),
     (2048, 512, 2048, None, 0, None, True),
+    (512, 256, 1024, "linear_ntw", 7, "gelu", True),  # 7-tile-wide blocks (wide and narrow wavefronts), 32 tiles = 4 x 7 + 4
+    (330, 200, 677, "linear_ntw", 7, None, False),   # ragged rows and columns, 22 tiles = 3 x 7 + 1
+    (256, 64, 224, "linear_ntw", 7, "silu", True),   # exactly one block
 ])
 def test_two_pass_launch_equals_the_fused_kernel(hip, dev, wfmt_name, M, K, N, option, value, act, bias):
     """linear_two_pass = 2 dequantises the weights once into bf16 fragment images and runs the main loop without the

@@ -743,17 +743,27 @@ TTM_EXPORT int ttm_debug_trace(void *dst, size_t bytes) {
 // IMG = true is the second pass of a two-pass launch: p.W holds the weights already dequantised to bf16, one 4 KiB
 // LDS fragment image per (k-step, column tile) (ttm_linear_image_k), so a step's weights are a straight LDS-direct copy
 // and the conversion, the raw staging area and the exponent loads drop out of the loop.
-template <int WF, int NTW, bool IMG = false>
+// BN_ = 7 (second pass only) is a block of seven column tiles: the wavefronts of one half take four of them (this body
+// with NTW = 4), those of the other half three (NTW = 3), and the two halves are dealt out so that every SIMD runs one
+// wavefront of each kind.  Both bodies execute the same sequence of barriers.
+template <int WF, int NTW, bool IMG = false, int BN_ = 2 * NTW>
 __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, int nblk, int nt_first, int nt_end) {
   static_assert(WF == WF_BFP8 || WF == WF_BFP4, "block-float weights only");
+  static_assert(BN_ == 2 * NTW || (IMG && BN_ == 7 && (NTW == 4 || NTW == 3)), "uneven blocks exist for the second pass only");
   constexpr int MB = 2;          // row tiles (32 m) per wavefront
-  constexpr int BN = 2 * NTW;    // column tiles per block
+  constexpr int BN = BN_;        // column tiles per block
   extern __shared__ u32x4 smem[];
   uint8_t *lds = (uint8_t *)smem;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;   // LDS byte address of the image
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wn = wave & 1, wm = wave >> 1;
+  int wn, wm, wcol;   // column half, row quarter, first column tile of this wavefront inside the block
+  if constexpr (BN_ == 2 * NTW) {
+    wn = wave & 1; wm = wave >> 1; wcol = wn * NTW;
+  } else {   // wavefronts w and w + 4 share a SIMD: one of them is the wide one
+    const int sd = wave & 3, hf = wave >> 2;
+    wn = (sd & 1) ^ hf; wm = (sd >> 1) + 2 * hf; wcol = wn ? BN_ - NTW : 0;
+  }
   if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);   // consecutive blocks of one XCD share weight columns
   const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
   const int mt0 = mb * 8, nt0 = nt_first + nb * BN;
@@ -776,7 +786,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   uint32_t rdW[4], rdA[4];   // fragment reads: + 4096 t + STAGE stage
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
-    rdW[s] = LDS_W + 16u * lds_chunk(wn * (32 * NTW) + (lane & 31), 2 * s + (lane >> 5));
+    rdW[s] = LDS_W + 16u * lds_chunk(wcol * 32 + (lane & 31), 2 * s + (lane >> 5));
     rdA[s] = 16u * lds_chunk(wm * (32 * MB) + (lane & 31), 2 * s + (lane >> 5));
   }
   // weight block of this lane: tile slot tid >> 5 of the 2 x 8 tiles of a step (slot = 8 * k-tile + column tile);
@@ -1014,8 +1024,8 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be in flight towards LDS when the block ends
 
   if (p.partial) linear_store_partial(p, p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * ((int64_t)p.Mt * p.Nt * 1024), acc,
-                                      mt0 + wm * MB, nt0 + wn * NTW, nt_end, lane);
-  else linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wn * NTW, nt_end, lane);
+                                      mt0 + wm * MB, nt0 + wcol, nt_end, lane);
+  else linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wcol, nt_end, lane);
 }
 
 template <int WF>
@@ -1037,7 +1047,11 @@ __global__ __launch_bounds__(512) void ttm_linear_img_k(LinearArgs p) {
     if (bid < p.n_blocks1) { nblk = p.n_blocks1; end = p.nt_split; }
     else { bid -= p.n_blocks1; nblk -= p.n_blocks1; first = p.nt_split; ntw = p.ntw2; }
   }
-  if (ntw == 4) linear_dma_block<WF, 4, true>(p, bid, nblk, first, end);
+  if (ntw == 7) {   // seven tiles wide: wide and narrow wavefronts (wavefront-uniform branch)
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if ((((wave & 3) & 1) ^ (wave >> 2)) == 0) linear_dma_block<WF, 4, true, 7>(p, bid, nblk, first, end);
+    else linear_dma_block<WF, 3, true, 7>(p, bid, nblk, first, end);
+  } else if (ntw == 4) linear_dma_block<WF, 4, true>(p, bid, nblk, first, end);
   else if (ntw == 3) linear_dma_block<WF, 3, true>(p, bid, nblk, first, end);
   else linear_dma_block<WF, 2, true>(p, bid, nblk, first, end);
 }
@@ -1507,7 +1521,8 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       }
       LinearArgs p = a;
       const int cus = device_cu_count();
-      int slices = plan_dma_grid(p, cus, ttm_option("linear_ntw"), ttm_option("linear_split_k"), ttm_option("linear_two_part") == 1);
+      const int force_ntw = ttm_option("linear_ntw") == 7 ? 0 : ttm_option("linear_ntw");   // 7 exists in the second pass only
+      int slices = plan_dma_grid(p, cus, force_ntw, ttm_option("linear_split_k"), ttm_option("linear_two_part") == 1);
       slices = slices < 1 ? 1 : (slices > a.Kt ? a.Kt : slices);
       if (slices > 1) {
         p.k_slice = (a.Kt + slices - 1) / slices;
@@ -1540,6 +1555,16 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       if (img_bytes + part_bytes > 0)
         if (int rc = ttm_stream_workspace(s, img_bytes + part_bytes, (void **)&ws)) return rc;
       if (slices > 1) p.partial = (float *)(ws + img_bytes);
+      if (two_pass && slices == 1 && p.nt_split == 0) {
+        // without the conversion a block may be seven tiles wide (the wavefronts of a SIMD take 4 + 3): worth it when
+        // that fills the last round, e.g. 8 x 448 tiles = 448 blocks of 8 (1.75 rounds on 256 CUs, paid as 2) against 512
+        // blocks of 7 (2 rounds at 7/8 of the work each).  linear_ntw = 7 forces it.
+        const int64_t blocks7 = (int64_t)p.m_blocks * ((a.Nt + 6) / 7);
+        const int64_t rounds8 = ((int64_t)p.n_blocks * batch + cus - 1) / cus, rounds7 = (blocks7 * batch + cus - 1) / cus;
+        static const double width_cost8[5] = {0, 0, 0.78, 0.92, 1.0};
+        const bool pick7 = ttm_option("linear_ntw") == 7 || (ttm_option("linear_ntw") == 0 && rounds7 * 0.92 < rounds8 * width_cost8[p.ntw] * 0.98);
+        if (pick7) { p.ntw = 7; p.n_blocks = (int)blocks7; }
+      }
       if (two_pass) {
         static bool attr2 = false;
         if (!attr2) {
