@@ -237,6 +237,53 @@ def test_copy_view_reshape_permute_slice_concat(hip, dev, orc):
     assert np.array_equal(dst.cpu().numpy(), orc.tilize(z.transpose(1, 2).contiguous().numpy()))   # padding stays zero
 
 
+@pytest.mark.parametrize("batch", [4, 5])
+def test_copy_view_index_width_boundary(hip, dev, batch):
+    """The copy kernels index with 32 bits when every logical and padded offset stays below 2^29 elements and with 64
+    bits otherwise: [4, 8192, 16384] bf16 (2^29 elements, 1 GiB) is the largest narrow case, [5, ...] the first wide one.
+    A head-split permute of both, tile layout in and out, compared with torch on the device."""
+    R, C, H = 8192, 16384, 8
+    g = torch.Generator(device="cpu").manual_seed(3)
+    base = torch.randint(-30000, 30000, (R, C // 64), generator=g, dtype=torch.int16)
+    x = base.repeat(1, 64).view(torch.bfloat16).to(dev).unsqueeze(0).repeat(batch, 1, 1)      # [batch, R, C], cheap to make
+    x += torch.arange(batch, device=dev, dtype=torch.bfloat16).view(batch, 1, 1)              # batches differ
+    xt = torch.empty(batch * R * C, dtype=torch.bfloat16, device=dev)
+    hip.call("ttm_tilize", hip.ptr(x), hip.ptr(xt), batch, R, C, 2, hip.current_stream())
+    oshape = (batch, H, R, C // H)
+    in4 = strides((batch, R, H, C // H))
+    out = view_copy(hip, dev, xt, (batch, R, C), True, oshape, True, oshape, [in4[0], in4[2], in4[1], in4[3]], strides(oshape))
+    got = torch.empty(oshape, dtype=torch.bfloat16, device=dev)
+    hip.call("ttm_untilize", hip.ptr(out), hip.ptr(got), batch * H, R, C // H, 2, hip.current_stream())
+    torch.cuda.synchronize()
+    want = x.view(batch, R, H, C // H).permute(0, 2, 1, 3)
+    assert torch.equal(got.view(torch.int16), want.contiguous().view(torch.int16))
+
+
+@pytest.mark.parametrize("index,limit", [(0, 16), (15, 16), (16, 16), (-3, 16)])
+@pytest.mark.parametrize("elem", ["bf16", "f32"])
+def test_copy_view_at_positions_the_destination_from_device_memory(hip, dev, elem, index, limit):
+    """ttm_copy_view_at: destination base + *index * index_stride with *index read by the kernel; outside [0, limit)
+    nothing is written.  A [3, 40] block goes to row block `index` of a [limit * 3, 40] row-major tensor, from a tiled
+    source read through a transposing view."""
+    dt = torch.bfloat16 if elem == "bf16" else torch.float32
+    src = datagen.randn((40, 3), seed=12, dtype=dt)
+    st = tilize_dev(hip, src, dev)
+    dst0 = datagen.randn((limit * 3, 40), seed=13, dtype=dt)
+    dst = dst0.clone().to(dev)
+    idx = torch.tensor([index], dtype=torch.int32, device=dev)
+    e, s1, s2 = (np.array(v, dtype=np.int64) for v in ([3, 40], [1, 3], [40, 1]))
+    hip.call("ttm_copy_view_at", hip.ptr(st), 40, 3, hip.TILE, hip.ptr(dst), limit * 3, 40, hip.ROW_MAJOR, src.element_size(), 2,
+             e.ctypes.data, s1.ctypes.data, 0, s2.ctypes.data, 0, hip.ptr(idx), 3 * 40, limit, hip.current_stream())
+    torch.cuda.synchronize()
+    want = dst0.clone()
+    if 0 <= index < limit:
+        want[3 * index:3 * index + 3] = src.t()
+    assert torch.equal(dst.cpu(), want)
+    with pytest.raises(hip.TTMError, match="null index"):
+        hip.call("ttm_copy_view_at", hip.ptr(st), 40, 3, hip.TILE, hip.ptr(dst), limit * 3, 40, hip.ROW_MAJOR, src.element_size(), 2,
+                 e.ctypes.data, s1.ctypes.data, 0, s2.ctypes.data, 0, None, 3 * 40, limit, hip.current_stream())
+
+
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,mask", [
     (1, 4, 2, 128, 128, 64, True, None), (2, 2, 2, 96, 160, 128, False, None), (1, 8, 2, 256, 256, 128, True, None),
     (1, 2, 1, 70, 70, 32, True, None), (1, 2, 2, 64, 100, 64, False, "b1"), (2, 2, 1, 64, 64, 64, False, "bh"),
