@@ -345,6 +345,9 @@ def test_linear_pair_equals_two_launches(hip, dev, wfmt_name, M, K, N, second_fi
     (512, 256, 1024, "linear_ntw", 7, "gelu", True),  # 7-tile-wide blocks (wide and narrow wavefronts), 32 tiles = 4 x 7 + 4
     (330, 200, 677, "linear_ntw", 7, None, False),   # ragged rows and columns, 22 tiles = 3 x 7 + 1
     (256, 64, 224, "linear_ntw", 7, "silu", True),   # exactly one block
+    (2048, 256, 10240, None, 0, "gelu", True),       # more blocks than CUs: several rounds, XCD-aware block order
+    (2048, 192, 10240, "linear_ntw", 7, None, True),
+    (2080, 256, 9000, "linear_ntw", 4, "relu", False),
 ])
 def test_two_pass_launch_equals_the_fused_kernel(hip, dev, wfmt_name, M, K, N, option, value, act, bias):
     """linear_two_pass = 2 dequantises the weights once into bf16 fragment images and runs the main loop without the
