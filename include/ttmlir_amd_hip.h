@@ -214,11 +214,26 @@ int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int 
  *   page table [batch, pages_per_user] pages [blocks, kv_heads, page_block, head_dim] where seq = pages_per_user *
  *   page_block; BFloat16.  scores = (q k^T + mask) * scale, mask additive BFloat16 [batch, 1, mask_heads, seq] or NULL;
  *   with is_causal and cur_pos [batch] keys after cur_pos[b] are excluded; scale <= 0 means 1/sqrt(head_dim); softmax in
- *   fp32.  Uses the stream's workspace for per-slice partial results. */
+ *   fp32.  Uses the stream's workspace for per-slice partial results.
+ * ttm_paged_update_cache: ::ttnn::experimental::paged_update_cache (operations/kv_cache/paged_update_cache.cpp:14-57;
+ *   shapes lib/Dialect/TTNN/IR/TTNNOps.cpp:4719-4820; golden tools/golden/mapping.py:8926-8963): cache
+ *   [blocks, heads, block_size, head_dim], input [1, users, heads, head_dim], update_index [users], page_table
+ *   [users, pages_per_user] or NULL.  cache[page_table[u, p / block_size], h, p % block_size, :] = input[0, u, h, :] with
+ *   p = update_index[u]; without a page table the cache is [users, heads, max_seq, head_dim] and user u writes entry u
+ *   (entry 0 when share_cache).  Positions, pages and blocks out of range write nothing (the golden clamps them).
+ * ttm_paged_fill_cache: ::ttnn::experimental::paged_fill_cache (operations/kv_cache/paged_fill_cache.cpp; golden
+ *   mapping.py:8966-9008): input [in_batch, heads, seq, head_dim], page_table [table_rows, pages_per_user], batch_idx
+ *   [in_batch] or NULL (then row b).  cache[page_table[row(b), s / block_size], h, s % block_size, :] = input[b, h, s, :]. */
 int ttm_rotary_embedding(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype, int64_t batch,
                          int64_t rows, int64_t cols, int64_t cache_rows, int64_t token_index, void *stream);
 int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users, int64_t heads,
                      int64_t max_seq, int64_t head_dim, int64_t input_users, int64_t batch_offset, void *stream);
+int ttm_paged_update_cache(void *cache, const void *input, const int32_t *update_index, const int32_t *page_table, int dtype,
+                           int64_t blocks, int64_t heads, int64_t block_size, int64_t head_dim, int64_t users,
+                           int64_t pages_per_user, int share_cache, void *stream);
+int ttm_paged_fill_cache(void *cache, const void *input, const int32_t *page_table, const int32_t *batch_idx, int dtype,
+                         int64_t blocks, int64_t heads, int64_t block_size, int64_t head_dim, int64_t in_batch, int64_t seq,
+                         int64_t table_rows, int64_t pages_per_user, void *stream);
 int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t users, int64_t heads, int64_t max_seq,
                    int64_t head_dim, int64_t seq, int64_t batch_offset, void *stream);
 int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,

@@ -148,6 +148,11 @@ int ttrt_pb_rotary_embedding(ttrt_builder *pb, uint32_t in, uint32_t cos_cache, 
                              uint32_t token_index, uint32_t *out);
 int ttrt_pb_update_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t update_index, uint32_t batch_offset);
 int ttrt_pb_fill_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t batch_offset);
+/* PagedUpdateCacheOp / PagedFillCacheOp (include/ttmlir/Target/TTNN/operations/kv_cache.fbs:19-32); page_table 0 = static
+ * cache, batch_idx 0 = absent */
+int ttrt_pb_paged_update_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t update_index, uint32_t page_table,
+                               int share_cache);
+int ttrt_pb_paged_fill_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t page_table, uint32_t batch_idx);
 int ttrt_pb_sdpa_decode(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t page_table, uint32_t mask, uint32_t cur_pos,
                         int is_causal, int has_scale, float scale, uint32_t *out);
 int ttrt_pb_reshape(ttrt_builder *pb, uint32_t in, const uint32_t *shape, int rank, uint32_t *out);

@@ -325,6 +325,51 @@ def fill_cache(cache, inp, batch_offset=0):
     return cache
 
 
+def paged_update_cache(cache, inp, update_index, page_table=None, share_cache=False):
+    """tools/golden/mapping.py:8926-8963 with the operand shapes of the TTNN op (lib/Dialect/TTNN/IR/TTNNOps.cpp:4719-4820):
+    cache [blocks, heads, block_size, dim], inp [1, users, heads, dim], update_index [users], page_table [users, pages].
+    cache[page_table[u, p // block_size], :, p % block_size, :] = inp[0, u] with p = update_index[u]; without a page table
+    user u owns cache entry u (entry 0 when the cache is shared).  Out-of-range positions, pages and blocks write nothing
+    (the golden clamps them instead; valid inputs never get there)."""
+    cache, inp = _c(cache, np.float32).copy(), _c(inp, np.float32)
+    blocks, _, bs, _ = cache.shape
+    for u in range(inp.shape[1]):
+        p = int(update_index[u])
+        if p < 0:
+            continue
+        if page_table is not None:
+            page = p // bs
+            if page >= page_table.shape[1]:
+                continue
+            blk, off = int(page_table[u, page]), p % bs
+        else:
+            if p >= bs:
+                continue
+            blk, off = (0 if share_cache else u), p
+        if 0 <= blk < blocks:
+            cache[blk, :, off, :] = inp[0, u]
+    return cache
+
+
+def paged_fill_cache(cache, inp, page_table, batch_idx=None):
+    """tools/golden/mapping.py:8966-9008: cache [blocks, heads, block_size, dim], inp [batch, heads, seq, dim];
+    cache[page_table[row(b), s // block_size], :, s % block_size, :] = inp[b, :, s, :], row(b) = batch_idx[b] or b."""
+    cache, inp = _c(cache, np.float32).copy(), _c(inp, np.float32)
+    blocks, _, bs, _ = cache.shape
+    for b in range(inp.shape[0]):
+        row = int(batch_idx[b]) if batch_idx is not None else b
+        if not 0 <= row < page_table.shape[0]:
+            continue
+        for sq in range(inp.shape[2]):
+            page = sq // bs
+            if page >= page_table.shape[1]:
+                continue
+            blk = int(page_table[row, page])
+            if 0 <= blk < blocks:
+                cache[blk, :, sq % bs, :] = inp[b, :, sq, :]
+    return cache
+
+
 def sdpa_decode(q, k, v, cur_pos=None, mask=None, is_causal=True, scale=None):
     q, k, v = _c(q, np.float32), _c(k, np.float32), _c(v, np.float32)
     _, B, H, D = q.shape

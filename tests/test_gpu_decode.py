@@ -175,3 +175,67 @@ def test_sdpa_decode_rejects_unsupported(hip, dev):
     with pytest.raises(hip.TTMError, match="page table"):
         hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, hip.ptr(z), 3, 32, hip.ptr(z), hip.BF16, 1, 8, 8,
                  64, 32, 1, 0.0, hip.current_stream())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("blocks,H,bs,D,users,pages,paged", [(12, 8, 64, 128, 4, 3, True), (40, 2, 32, 64, 32, 1, True), (6, 3, 96, 32, 5, 2, True),
+                                                             (4, 8, 128, 128, 4, 0, False), (1, 2, 40, 64, 3, 0, False)])
+def test_paged_update_cache_bit_exact(hip, dev, orc, dtype, blocks, H, bs, D, users, pages, paged):
+    """ttm_paged_update_cache against the oracle: shuffled page tables, positions in every page, positions and block
+    numbers out of range (nothing written), the static form with per-user entries and with one shared entry."""
+    g = torch.Generator().manual_seed(60)
+    cache = datagen.randn((blocks, H, bs, D), seed=61, dtype=dtype)
+    inp = datagen.randn((1, users, H, D), seed=62, dtype=dtype)
+    code = hip.BF16 if dtype == torch.bfloat16 else hip.F32
+    cap = pages * bs if paged else bs
+    pos = torch.randint(0, cap, (users,), generator=g, dtype=torch.int32)
+    pos[0] = cap - 1
+    if users > 2:
+        pos[1], pos[2] = -1, cap                          # skipped users
+    table = None
+    if paged:
+        table = torch.randperm(blocks, generator=g)[:users * pages].reshape(users, pages).to(torch.int32) if users * pages <= blocks \
+            else torch.randint(0, blocks, (users, pages), generator=g, dtype=torch.int32)
+        if users > 3:
+            table[3, int(pos[3]) // bs] = blocks          # a block number past the cache
+        # two users writing the same cell would race: keep (block, offset) unique among the writers
+        seen = set()
+        for u in range(users):
+            if 0 <= int(pos[u]) < cap:
+                key = (int(table[u, int(pos[u]) // bs]), int(pos[u]) % bs)
+                if key in seen:
+                    pos[u] = -1
+                seen.add(key)
+    shared = (not paged) and blocks == 1
+    if shared:
+        pos[:] = -1
+        pos[users - 1] = 7                                # one writer into the shared entry
+    ct, it = tilize_dev(hip, cache, dev), tilize_dev(hip, inp, dev)
+    pos_d, table_d = pos.to(dev), table.to(dev) if paged else None       # kept alive across the launch
+    hip.call("ttm_paged_update_cache", hip.ptr(ct), hip.ptr(it), hip.ptr(pos_d), hip.ptr(table_d) if paged else None, code,
+             blocks, H, bs, D, users, pages, int(shared), hip.current_stream())
+    got = f32(untilize_dev(hip, ct, cache.shape, dev))
+    want = orc.paged_update_cache(f32(cache), f32(inp), pos.numpy(), table.numpy() if paged else None, share_cache=shared)
+    assert np.array_equal(got, want)
+    assert not np.array_equal(want, f32(cache))          # something was written
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("blocks,H,bs,D,batch,seq,rows,pages,with_idx", [(14, 8, 64, 128, 1, 200, 3, 4, True), (8, 2, 32, 64, 2, 64, 2, 2, False),
+                                                                        (6, 3, 32, 32, 1, 33, 2, 1, True)])
+def test_paged_fill_cache_bit_exact(hip, dev, orc, dtype, blocks, H, bs, D, batch, seq, rows, pages, with_idx):
+    """ttm_paged_fill_cache against the oracle: a prefill longer than one block, ragged sequence lengths (the last block
+    keeps its old rows past the sequence), sequences longer than the page table (the excess is dropped)."""
+    g = torch.Generator().manual_seed(70)
+    cache = datagen.randn((blocks, H, bs, D), seed=71, dtype=dtype)
+    inp = datagen.randn((batch, H, seq, D), seed=72, dtype=dtype)
+    code = hip.BF16 if dtype == torch.bfloat16 else hip.F32
+    table = torch.randperm(blocks, generator=g)[:rows * pages].reshape(rows, pages).to(torch.int32)
+    idx = torch.tensor([rows - 1] * batch, dtype=torch.int32) if with_idx else None
+    ct, it = tilize_dev(hip, cache, dev), tilize_dev(hip, inp, dev)
+    table_d, idx_d = table.to(dev), idx.to(dev) if with_idx else None    # kept alive across the launch
+    hip.call("ttm_paged_fill_cache", hip.ptr(ct), hip.ptr(it), hip.ptr(table_d), hip.ptr(idx_d) if with_idx else None, code,
+             blocks, H, bs, D, batch, seq, rows, pages, hip.current_stream())
+    got = f32(untilize_dev(hip, ct, cache.shape, dev))
+    want = orc.paged_fill_cache(f32(cache), f32(inp), table.numpy(), idx.numpy() if with_idx else None)
+    assert np.array_equal(got, want)

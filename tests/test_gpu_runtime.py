@@ -678,3 +678,51 @@ def test_submit_errors(device):
     rt.deallocate_tensor(freed, force=True)
     with pytest.raises(RuntimeError, match="deallocated"):
         rt.to_host(freed)
+
+
+def test_paged_cache_program_fill_update_attend(device, orc, metrics):
+    """A paged decode step as one program: paged_fill_cache writes a prefill of 70 positions for user 1 through the page
+    table, paged_update_cache appends one position per user at its own index, paged_scaled_dot_product_attention_decode
+    attends over the pages.  The caches (updated in place) are bit-exact against the oracle, the attention output within
+    the decode kernel's tolerance."""
+    users, H, Hkv, hd, bs, pages = 2, 4, 2, 64, 32, 4
+    blocks = users * pages + 1
+    pb = rt.ProgramBuilder()
+    pb.begin_program("paged_step")
+    kc = pb.input((blocks, Hkv, bs, hd), DT.BFloat16)
+    vc = pb.input((blocks, Hkv, bs, hd), DT.BFloat16)
+    table = pb.input((users, pages), DT.Int32, TL.RowMajor)
+    kfill = pb.input((1, Hkv, 70, hd), DT.BFloat16)
+    vfill = pb.input((1, Hkv, 70, hd), DT.BFloat16)
+    row = pb.input((1,), DT.Int32, TL.RowMajor)
+    knew = pb.input((1, users, Hkv, hd), DT.BFloat16)
+    vnew = pb.input((1, users, Hkv, hd), DT.BFloat16)
+    pos = pb.input((users,), DT.Int32, TL.RowMajor)
+    q = pb.input((1, users, H, hd), DT.BFloat16)
+    pb.paged_fill_cache(kc, kfill, table, row)
+    pb.paged_fill_cache(vc, vfill, table, row)
+    pb.paged_update_cache(kc, knew, pos, table)
+    pb.paged_update_cache(vc, vnew, pos, table)
+    pb.output(pb.sdpa_decode(q, kc, vc, cur_pos=pos, page_table=table, is_causal=True))
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    g = torch.Generator().manual_seed(23)
+    rn = lambda *shape: bf(torch.randn(shape, generator=g))
+    kc0, vc0 = rn(blocks, Hkv, bs, hd), rn(blocks, Hkv, bs, hd)
+    tbl = torch.randperm(blocks, generator=g)[:users * pages].reshape(users, pages).to(torch.int32)
+    kf, vf, kn, vn, qq = rn(1, Hkv, 70, hd), rn(1, Hkv, 70, hd), rn(1, users, Hkv, hd), rn(1, users, Hkv, hd), rn(1, users, H, hd)
+    positions = torch.tensor([40, 70], dtype=torch.int32)        # user 0 continues an older sequence, user 1 its prefill
+    tins = [kc0.clone(), vc0.clone(), tbl, kf, vf, torch.tensor([1], dtype=torch.int32), kn, vn, positions, qq]
+    devs = [rt.to_layout(rt.from_torch(t.contiguous()), device, rt.get_layout(binary, 0, i), retain=i < 2) for i, t in enumerate(tins)]
+    (y,) = rt.submit(device, binary, 0, devs)
+    got = rt.to_torch(rt.to_host(y, untilize=True)[0]).float().numpy()
+    gk, gv = (rt.to_torch(rt.to_host(devs[i], untilize=True)[0]).float().numpy() for i in (0, 1))
+    f = lambda t: t.float().numpy()
+    wk = orc.paged_update_cache(orc.paged_fill_cache(f(kc0), f(kf), tbl.numpy(), np.array([1])), f(kn), positions.numpy(), tbl.numpy())
+    wv = orc.paged_update_cache(orc.paged_fill_cache(f(vc0), f(vf), tbl.numpy(), np.array([1])), f(vn), positions.numpy(), tbl.numpy())
+    assert np.array_equal(gk, wk) and np.array_equal(gv, wv)
+    # gather each user's pages into a contiguous cache for the oracle's attention
+    gather = lambda c: np.stack([np.concatenate([c[int(tbl[u, p])] for p in range(pages)], axis=1) for u in range(users)])
+    want = orc.sdpa_decode(f(qq), gather(wk), gather(wv), cur_pos=positions.tolist())
+    assert np.max(np.abs(got - want)) <= 2.0 ** -6
+    assert metrics.get_pcc(want, got) >= 0.9999

@@ -177,6 +177,49 @@ def test_cache_update_and_fill_match_slice_assignment(orc):
     assert np.array_equal(orc.fill_cache(cache, fill[:, :, :32])[0, :, 32:], cache[0, :, 32:])   # aligned: nothing cleared
 
 
+def test_paged_cache_writes_by_hand_and_against_the_unpaged_ops(orc):
+    """Known answers written out cell by cell for a 2-user page table, then the relation that ties the paged ops to the
+    unpaged ones: with the identity page table (page p of user u is block u * pages + p) a paged cache is the unpaged
+    cache [users, heads, pages * block, dim] viewed block-wise, so both routes must leave the same bytes."""
+    blocks, H, bs, D = 5, 2, 32, 8
+    cache = rnd((blocks, H, bs, D), 40)
+    inp = rnd((1, 2, H, D), 41)
+    table = np.array([[2, 0], [1, 3]], dtype=np.int32)
+    got = orc.paged_update_cache(cache, inp, np.array([33, 5]), table)
+    want = cache.copy()
+    want[0, :, 1, :] = inp[0, 0]        # user 0, position 33 = second page (block 0), offset 1
+    want[1, :, 5, :] = inp[0, 1]        # user 1, position 5 = first page (block 1), offset 5
+    assert np.array_equal(got, want)
+    # positions past the table, negative positions and block numbers outside the cache write nothing
+    assert np.array_equal(orc.paged_update_cache(cache, inp, np.array([64, -1]), table), cache)
+    assert np.array_equal(orc.paged_update_cache(cache, inp, np.array([0, 0]), np.array([[7, 0], [-2, 3]], dtype=np.int32)), cache)
+    # static cache: user u owns entry u, or entry 0 for everyone when shared (the last user wins)
+    got = orc.paged_update_cache(cache, inp, np.array([3, 9]))
+    want = cache.copy()
+    want[0, :, 3, :], want[1, :, 9, :] = inp[0, 0], inp[0, 1]
+    assert np.array_equal(got, want)
+    got = orc.paged_update_cache(cache, inp, np.array([3, 3]), share_cache=True)
+    assert np.array_equal(got[0, :, 3, :], inp[0, 1]) and np.array_equal(got[1:], cache[1:])
+    # fill: 40 positions of one sequence through row 1 of the table: 32 rows into block 1, 8 into block 3
+    fill = rnd((1, H, 40, D), 42)
+    got = orc.paged_fill_cache(cache, fill, table, batch_idx=np.array([1]))
+    want = cache.copy()
+    want[1] = fill[0, :, :32]
+    want[3, :, :8] = fill[0, :, 32:]
+    assert np.array_equal(got, want)
+    # identity page table against the unpaged ops
+    users, pages = 3, 2
+    flat = rnd((users, H, pages * bs, D), 43)
+    paged = flat.reshape(users, H, pages, bs, D).transpose(0, 2, 1, 3, 4).reshape(users * pages, H, bs, D).copy()
+    ident = np.arange(users * pages, dtype=np.int32).reshape(users, pages)
+    back = lambda c: c.reshape(users, pages, H, bs, D).transpose(0, 2, 1, 3, 4).reshape(users, H, pages * bs, D)
+    seq = rnd((1, H, 2 * bs, D), 44)
+    assert np.array_equal(back(orc.paged_fill_cache(paged, seq, ident, batch_idx=np.array([2]))), orc.fill_cache(flat, seq, batch_offset=2))
+    step = rnd((1, users, H, D), 45)
+    same_pos = orc.update_cache(flat, np.ascontiguousarray(step.transpose(0, 2, 1, 3)), 45)
+    assert np.array_equal(back(orc.paged_update_cache(paged, step, np.array([45, 45, 45]), ident)), same_pos)
+
+
 @pytest.mark.parametrize("H,Hkv", [(4, 4), (8, 2)])
 def test_sdpa_decode_against_library_attention(orc, H, Hkv):
     B, S, D = 3, 48, 16

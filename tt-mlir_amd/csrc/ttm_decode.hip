@@ -96,6 +96,65 @@ __global__ __launch_bounds__(256) void ttm_fill_cache_k(u32x4 *__restrict__ cach
   cache[base16 + h * head_stride_cache16 + o] = input[i];
 }
 
+// Paged cache writes.  The cache is [blocks, heads, block_size, dim]; a user's positions live in the blocks its row of
+// the page table names.  Without a page table the cache is [users, heads, max_seq, dim] (block_size = max_seq) and user
+// u owns entry u (entry 0 for all users when the cache is shared).  Positions, page numbers and block numbers outside
+// their ranges write nothing.
+//
+// update: cache[block(u, pos_u), h, pos_u % block_size, :] = input[0, u, h, :] with pos_u = index[u]; one thread per 8 elements
+template <typename T>
+__global__ __launch_bounds__(256) void ttm_paged_update_cache_k(T *__restrict__ cache, const T *__restrict__ input,
+                                                                const int32_t *__restrict__ index, const int32_t *__restrict__ table,
+                                                                int64_t blocks, int64_t heads, int64_t block_size, int64_t dim,
+                                                                int64_t users, int64_t pages, int shared, int64_t total8) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const int64_t d8 = dim >> 3, ct = dim >> 5;
+  const int64_t c = (i % d8) * 8, h = (i / d8) % heads, u = i / (d8 * heads);
+  const int64_t pos = index[u];
+  if (pos < 0) return;
+  int64_t blk, off;
+  if (table) {
+    const int64_t page = pos / block_size;
+    if (page >= pages) return;
+    blk = table[u * pages + page];
+    off = pos % block_size;
+  } else {
+    if (pos >= block_size) return;
+    blk = shared ? 0 : u;
+    off = pos;
+  }
+  if (blk < 0 || blk >= blocks) return;
+  const int64_t heads_pad = ttm_round_up32(heads), bs_pad = ttm_round_up32(block_size);
+  const T *src = input + u * heads_pad * dim + ttm_tiled_offset(h, c, ct);
+  T *dst = cache + (blk * heads + h) * bs_pad * dim + ttm_tiled_offset(off, c, ct);
+  *(u32x4 *)dst = *(const u32x4 *)src;
+  if (sizeof(T) == 4) *(u32x4 *)(dst + 4) = *(const u32x4 *)(src + 4);
+}
+
+// fill: cache[table[row(b), s / block_size], h, s % block_size, :] = input[b, h, s, :] for s < seq, where row(b) is
+// batch_idx[b] when given and b otherwise; one thread per 8 elements
+template <typename T>
+__global__ __launch_bounds__(256) void ttm_paged_fill_cache_k(T *__restrict__ cache, const T *__restrict__ input,
+                                                              const int32_t *__restrict__ table, const int32_t *__restrict__ batch_idx,
+                                                              int64_t blocks, int64_t heads, int64_t block_size, int64_t dim,
+                                                              int64_t seq, int64_t table_rows, int64_t pages, int64_t total8) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const int64_t d8 = dim >> 3, ct = dim >> 5;
+  const int64_t c = (i % d8) * 8, s = (i / d8) % seq, h = (i / (d8 * seq)) % heads, b = i / (d8 * seq * heads);
+  const int64_t row = batch_idx ? batch_idx[b] : b;
+  const int64_t page = s / block_size;
+  if (row < 0 || row >= table_rows || page >= pages) return;
+  const int64_t blk = table[row * pages + page];
+  if (blk < 0 || blk >= blocks) return;
+  const int64_t seq_pad = ttm_round_up32(seq), bs_pad = ttm_round_up32(block_size);
+  const T *src = input + (b * heads + h) * seq_pad * dim + ttm_tiled_offset(s, c, ct);
+  T *dst = cache + (blk * heads + h) * bs_pad * dim + ttm_tiled_offset(s % block_size, c, ct);
+  *(u32x4 *)dst = *(const u32x4 *)src;
+  if (sizeof(T) == 4) *(u32x4 *)(dst + 4) = *(const u32x4 *)(src + 4);
+}
+
 // ------------------------------------------------------------------------------------------------ attention, one query token
 // q [1, B, H, D], k / v [B, Hkv, S, D] (or pages [blocks, Hkv, block, D] behind a page table), out [1, B, H, D], bf16 tiles.
 // grid (splits, B * Hkv), 256 threads.  A block owns the G = H / Hkv query heads of one kv head and one slice of the keys:
@@ -425,6 +484,52 @@ TTM_EXPORT int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t
   if (total16 == 0) return TTM_OK;
   hipLaunchKernelGGL(ttm_fill_cache_k, dim3((unsigned)ttm_cdiv(total16, 256)), dim3(256), 0, (hipStream_t)stream, (u32x4 *)cache,
                      (const u32x4 *)input, cache16, in16, batch_offset * heads * cache16, total16);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+TTM_EXPORT int ttm_paged_update_cache(void *cache, const void *input, const int32_t *update_index, const int32_t *page_table,
+                                      int dtype, int64_t blocks, int64_t heads, int64_t block_size, int64_t head_dim, int64_t users,
+                                      int64_t pages_per_user, int share_cache, void *stream) {
+  TTM_REQUIRE(cache && input && update_index, "ttm_paged_update_cache: null pointer");
+  TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_paged_update_cache: dtype must be BFloat16 or Float32");
+  TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_paged_update_cache: head dim must be a positive multiple of 32");
+  TTM_REQUIRE(blocks > 0 && heads > 0 && block_size > 0 && users >= 0, "ttm_paged_update_cache: bad extents");
+  TTM_REQUIRE(!page_table || pages_per_user > 0, "ttm_paged_update_cache: a page table needs pages_per_user > 0");
+  TTM_REQUIRE(page_table || share_cache || users <= blocks, "ttm_paged_update_cache: %lld users do not fit a cache of %lld entries",
+              (long long)users, (long long)blocks);
+  const int64_t total8 = users * heads * (head_dim / 8);
+  if (total8 == 0) return TTM_OK;
+  const dim3 grid((unsigned)ttm_cdiv(total8, 256));
+  if (dtype == TTM_BF16)
+    hipLaunchKernelGGL(ttm_paged_update_cache_k<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, (uint16_t *)cache,
+                       (const uint16_t *)input, update_index, page_table, blocks, heads, block_size, head_dim, users, pages_per_user,
+                       share_cache, total8);
+  else
+    hipLaunchKernelGGL(ttm_paged_update_cache_k<float>, grid, dim3(256), 0, (hipStream_t)stream, (float *)cache, (const float *)input,
+                       update_index, page_table, blocks, heads, block_size, head_dim, users, pages_per_user, share_cache, total8);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+TTM_EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_t *page_table, const int32_t *batch_idx, int dtype,
+                                    int64_t blocks, int64_t heads, int64_t block_size, int64_t head_dim, int64_t in_batch, int64_t seq,
+                                    int64_t table_rows, int64_t pages_per_user, void *stream) {
+  TTM_REQUIRE(cache && input && page_table, "ttm_paged_fill_cache: null pointer");
+  TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_paged_fill_cache: dtype must be BFloat16 or Float32");
+  TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_paged_fill_cache: head dim must be a positive multiple of 32");
+  TTM_REQUIRE(blocks > 0 && heads > 0 && block_size > 0 && in_batch >= 0 && seq >= 0 && table_rows > 0 && pages_per_user > 0,
+              "ttm_paged_fill_cache: bad extents");
+  const int64_t total8 = in_batch * heads * seq * (head_dim / 8);
+  if (total8 == 0) return TTM_OK;
+  const dim3 grid((unsigned)ttm_cdiv(total8, 256));
+  if (dtype == TTM_BF16)
+    hipLaunchKernelGGL(ttm_paged_fill_cache_k<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, (uint16_t *)cache,
+                       (const uint16_t *)input, page_table, batch_idx, blocks, heads, block_size, head_dim, seq, table_rows,
+                       pages_per_user, total8);
+  else
+    hipLaunchKernelGGL(ttm_paged_fill_cache_k<float>, grid, dim3(256), 0, (hipStream_t)stream, (float *)cache, (const float *)input,
+                       page_table, batch_idx, blocks, heads, block_size, head_dim, seq, table_rows, pages_per_user, total8);
   TTM_LAUNCH_CHECK();
   return TTM_OK;
 }

@@ -564,6 +564,12 @@ class ProgramBuilder:
     def fill_cache(self, cache, t, batch_offset=0):
         _call("ttrt_pb_fill_cache", self.h, cache, t, batch_offset)
 
+    def paged_update_cache(self, cache, t, update_index, page_table=0, share_cache=False):
+        _call("ttrt_pb_paged_update_cache", self.h, cache, t, update_index, page_table, int(share_cache))
+
+    def paged_fill_cache(self, cache, t, page_table, batch_idx=0):
+        _call("ttrt_pb_paged_fill_cache", self.h, cache, t, page_table, batch_idx)
+
     def sdpa_decode(self, q, k, v, cur_pos=0, mask=0, page_table=0, is_causal=True, scale=None):
         return self._op("ttrt_pb_sdpa_decode", q, k, v, page_table, mask, cur_pos, int(is_causal), int(scale is not None),
                         ctypes.c_float(scale or 0.0))

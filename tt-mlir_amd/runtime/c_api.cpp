@@ -412,6 +412,13 @@ TTRT_EXPORT int ttrt_pb_update_cache(ttrt_builder *pb, uint32_t cache, uint32_t 
 TTRT_EXPORT int ttrt_pb_fill_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t batch_offset) {
   return guard([&] { need(pb, "builder"); pb->pb.fillCache(cache, in, batch_offset); });
 }
+TTRT_EXPORT int ttrt_pb_paged_update_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t update_index, uint32_t page_table,
+                                           int share_cache) {
+  return guard([&] { need(pb, "builder"); pb->pb.pagedUpdateCache(cache, in, update_index, page_table, share_cache != 0); });
+}
+TTRT_EXPORT int ttrt_pb_paged_fill_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t page_table, uint32_t batch_idx) {
+  return guard([&] { need(pb, "builder"); pb->pb.pagedFillCache(cache, in, page_table, batch_idx); });
+}
 TTRT_EXPORT int ttrt_pb_sdpa_decode(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t page_table, uint32_t mask, uint32_t cur_pos,
                                     int is_causal, int has_scale, float scale, uint32_t *out) {
   PB_OP(sdpaDecode(q, k, v, page_table, mask, cur_pos, is_causal != 0, has_scale != 0, scale));

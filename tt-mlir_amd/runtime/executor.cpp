@@ -124,6 +124,16 @@ OpRefs opRefs(const fb::Table &operation) {
     in(schema::UpdateCacheOp::f_cache); in(schema::UpdateCacheOp::f_input); in(schema::UpdateCacheOp::f_update_index);
     break;
   case OpType::FillCacheOp: in(schema::FillCacheOp::f_cache); in(schema::FillCacheOp::f_input); break;
+  case OpType::PagedUpdateCacheOp: {
+    using S = schema::PagedUpdateCacheOp;
+    in(S::f_cache); in(S::f_input); in(S::f_update_index); in(S::f_page_table);
+    break;
+  }
+  case OpType::PagedFillCacheOp: {
+    using S = schema::PagedFillCacheOp;
+    in(S::f_cache); in(S::f_input); in(S::f_page_table); in(S::f_batch_idx_tensor);
+    break;
+  }
   case OpType::ScaledDotProductAttentionDecodeOp: {
     using S = schema::ScaledDotProductAttentionDecodeOp;
     in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
@@ -656,6 +666,59 @@ void runFillCache(const fb::Table &op, ProgramContext &ctx) {
   TTRT_ASSERT(is[0] == 1, "fill_cache: input must hold one user");
   TTM_CALL(ttm_fill_cache(cache.handle->data.get(), in.handle->data.get(), floatCode(cache.handle->dtype, "fill_cache"), cs[0], cs[1], cs[2],
                           cs[3], is[2], op.scalar<std::uint32_t>(S::f_batch_offset, 0), ctx.stream()));
+  cache.handle->version = nextTensorVersion();
+}
+
+// runtime/lib/ttnn/operations/kv_cache/paged_update_cache.cpp:14-57; shapes lib/Dialect/TTNN/IR/TTNNOps.cpp:4719-4820
+void runPagedUpdateCache(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::PagedUpdateCacheOp;
+  Tensor &cache = cacheOperand(ctx, op.table(S::f_cache), "paged_update_cache cache");
+  const auto &cs = cache.handle->shape;
+  Tensor in = as(ctx, ctx.get(op.table(S::f_input), "paged_update_cache input"), TensorLayout::Tile, cache.handle->dtype);
+  const auto &is = in.handle->shape;
+  Tensor index = devicePositions(ctx, ctx.get(op.table(S::f_update_index), "paged_update_cache index"), "paged_update_cache: update_index");
+  TTRT_ASSERT(index.handle->shape.size() == 1, "paged_update_cache: update_index must be 1D");
+  const std::int64_t users = index.handle->shape[0];
+  TTRT_ASSERT(is.size() == 4 && is[0] == 1 && is[1] == users && is[2] == cs[1] && is[3] == cs[3],
+              "paged_update_cache: input must be [1, users, heads, head_dim] matching the cache and the update index");
+  const bool shared = op.scalar<std::uint8_t>(S::f_share_cache, 0) != 0;
+  Tensor table;
+  std::int64_t pages = 0;
+  if (fb::Table tref = op.table(S::f_page_table)) {
+    table = devicePositions(ctx, ctx.get(tref, "paged_update_cache page table"), "paged_update_cache: page_table");
+    const auto &ts = table.handle->shape;
+    TTRT_ASSERT(ts.size() == 2 && ts[0] == users, "paged_update_cache: page table must be [users, pages]");
+    TTRT_ASSERT(cs[2] % 32 == 0, "paged_update_cache: block size must be divisible by 32");
+    pages = ts[1];
+  } else {
+    TTRT_ASSERT(shared ? cs[0] == 1 : users <= static_cast<std::int64_t>(cs[0]), "paged_update_cache: more users than cache entries");
+  }
+  TTM_CALL(ttm_paged_update_cache(cache.handle->data.get(), in.handle->data.get(), static_cast<const std::int32_t *>(index.handle->data.get()),
+                                  table.handle ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr,
+                                  floatCode(cache.handle->dtype, "paged_update_cache"), cs[0], cs[1], cs[2], cs[3], users, pages,
+                                  shared ? 1 : 0, ctx.stream()));
+  cache.handle->version = nextTensorVersion();
+}
+// runtime/lib/ttnn/operations/kv_cache/paged_fill_cache.cpp; golden tools/golden/mapping.py:8966-9008
+void runPagedFillCache(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::PagedFillCacheOp;
+  Tensor &cache = cacheOperand(ctx, op.table(S::f_cache), "paged_fill_cache cache");
+  const auto &cs = cache.handle->shape;
+  Tensor in = as(ctx, ctx.get(op.table(S::f_input), "paged_fill_cache input"), TensorLayout::Tile, cache.handle->dtype);
+  const auto &is = in.handle->shape;
+  TTRT_ASSERT(is.size() == 4 && is[1] == cs[1] && is[3] == cs[3], "paged_fill_cache: input must be [batch, heads, seq, head_dim] matching the cache");
+  Tensor table = devicePositions(ctx, ctx.get(op.table(S::f_page_table), "paged_fill_cache page table"), "paged_fill_cache: page_table");
+  const auto &ts = table.handle->shape;
+  TTRT_ASSERT(ts.size() == 2, "paged_fill_cache: page table must be [users, pages]");
+  Tensor rows;
+  if (fb::Table bref = op.table(S::f_batch_idx_tensor)) {
+    rows = devicePositions(ctx, ctx.get(bref, "paged_fill_cache batch index"), "paged_fill_cache: batch_idx_tensor");
+    TTRT_ASSERT(volume(rows.handle->shape) >= is[0], "paged_fill_cache: one batch index per input batch entry is needed");
+  }
+  TTM_CALL(ttm_paged_fill_cache(cache.handle->data.get(), in.handle->data.get(), static_cast<const std::int32_t *>(table.handle->data.get()),
+                                rows.handle ? static_cast<const std::int32_t *>(rows.handle->data.get()) : nullptr,
+                                floatCode(cache.handle->dtype, "paged_fill_cache"), cs[0], cs[1], cs[2], cs[3], is[0], is[2], ts[0], ts[1],
+                                ctx.stream()));
   cache.handle->version = nextTensorVersion();
 }
 
@@ -1193,6 +1256,8 @@ void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   case OpType::FuncCallOp: return runFuncCall(op, ctx);
   case OpType::RotaryEmbeddingOp: return runRotaryEmbedding(op, ctx);
   case OpType::UpdateCacheOp: return runUpdateCache(op, ctx);
+  case OpType::PagedUpdateCacheOp: return runPagedUpdateCache(op, ctx);
+  case OpType::PagedFillCacheOp: return runPagedFillCache(op, ctx);
   case OpType::FillCacheOp: return runFillCache(op, ctx);
   case OpType::ScaledDotProductAttentionDecodeOp: return runSdpaDecode(op, ctx);
   case OpType::PagedScaledDotProductAttentionDecodeOp: return runPagedSdpaDecode(op, ctx);

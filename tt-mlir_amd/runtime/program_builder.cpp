@@ -447,6 +447,27 @@ void ProgramBuilder::fillCache(Id cache, Id in, std::uint32_t batchOffset) {
   b_.addScalarDefault<std::uint32_t>(FillCacheOp::f_batch_offset, batchOffset, 0);
   addOp(OpType::FillCacheOp, b_.endTable(), "ttnn.fill_cache");
 }
+void ProgramBuilder::pagedUpdateCache(Id cache, Id in, Id updateIndex, Id pageTable, bool shareCache) {
+  using S = PagedUpdateCacheOp;
+  Off c = tensorRef(cache), i = tensorRef(in), u = tensorRef(updateIndex), t = pageTable ? tensorRef(pageTable) : 0;
+  b_.startTable(S::kNumFields);
+  b_.addOffset(S::f_cache, c);
+  b_.addOffset(S::f_input, i);
+  b_.addOffset(S::f_update_index, u);
+  b_.addScalarDefault<std::uint8_t>(S::f_share_cache, shareCache ? 1 : 0, 0);
+  if (pageTable) b_.addOffset(S::f_page_table, t);
+  addOp(OpType::PagedUpdateCacheOp, b_.endTable(), "ttnn.paged_update_cache");
+}
+void ProgramBuilder::pagedFillCache(Id cache, Id in, Id pageTable, Id batchIdx) {
+  using S = PagedFillCacheOp;
+  Off c = tensorRef(cache), i = tensorRef(in), t = tensorRef(pageTable), bi = batchIdx ? tensorRef(batchIdx) : 0;
+  b_.startTable(S::kNumFields);
+  b_.addOffset(S::f_cache, c);
+  b_.addOffset(S::f_input, i);
+  b_.addOffset(S::f_page_table, t);
+  if (batchIdx) b_.addOffset(S::f_batch_idx_tensor, bi);
+  addOp(OpType::PagedFillCacheOp, b_.endTable(), "ttnn.paged_fill_cache");
+}
 ProgramBuilder::Id ProgramBuilder::sdpaDecode(Id q, Id k, Id v, Id pageTable, Id mask, Id curPos, bool causal, bool hasScale, float scale) {
   Desc d = desc(q);
   d.storage = StorageType::Device;

@@ -53,6 +53,8 @@ public:
   Id rotaryEmbedding(Id in, Id cosCache, Id sinCache, bool hasTokenIndex, std::uint32_t tokenIndex);
   void updateCache(Id cache, Id in, Id updateIndex, std::uint32_t batchOffset);
   void fillCache(Id cache, Id in, std::uint32_t batchOffset);
+  void pagedUpdateCache(Id cache, Id in, Id updateIndex, Id pageTable, bool shareCache);   // pageTable 0: static cache
+  void pagedFillCache(Id cache, Id in, Id pageTable, Id batchIdx);                         // batchIdx 0: row b of the table
   // pageTable = 0 writes ScaledDotProductAttentionDecodeOp, otherwise the paged op
   Id sdpaDecode(Id q, Id k, Id v, Id pageTable, Id mask, Id curPos, bool causal, bool hasScale, float scale);
   Id empty(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout);
