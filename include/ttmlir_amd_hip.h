@@ -226,6 +226,12 @@ int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int 
  *   [in_batch] or NULL (then row b).  cache[page_table[row(b), s / block_size], h, s % block_size, :] = input[b, h, s, :]. */
 int ttm_rotary_embedding(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype, int64_t batch,
                          int64_t rows, int64_t cols, int64_t cache_rows, int64_t token_index, void *stream);
+/* The head split in front of the rotary embedding folded in: x is the [batch, heads * head_dim] TILE matrix a projection
+ * leaves, out is [batch, heads, head_dim] (= [1, batch, heads, head_dim]) TILE with zero padding rows; decode mode only
+ * (token_index >= 0), since rows are heads here. */
+int ttm_rotary_embedding_split_heads(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype,
+                                     int64_t batch, int64_t heads, int64_t head_dim, int64_t cache_rows, int64_t token_index,
+                                     void *stream);
 int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users, int64_t heads,
                      int64_t max_seq, int64_t head_dim, int64_t input_users, int64_t batch_offset, void *stream);
 int ttm_paged_update_cache(void *cache, const void *input, const int32_t *update_index, const int32_t *page_table, int dtype,
@@ -240,6 +246,13 @@ int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *
                     const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out, int dtype,
                     int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal,
                     float scale, void *stream);
+/* ttm_sdpa_decode whose output already has its heads concatenated: out is the [batch, heads * head_dim] TILE matrix that
+ * ::ttnn::experimental::nlp_concat_heads_decode (runtime/lib/ttnn/operations/transformer/nlp_concat_heads_decode.cpp) or
+ * a reshape would make of [1, batch, heads, head_dim]; padding rows below the last user are written as zeros. */
+int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
+                                 int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block,
+                                 void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
+                                 int64_t head_dim, int is_causal, float scale, void *stream);
 
 /* Kernel-variant selection for measurement (name -> small integer); unknown names fail. */
 int ttm_set_option(const char *name, int value);

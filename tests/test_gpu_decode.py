@@ -239,3 +239,47 @@ def test_paged_fill_cache_bit_exact(hip, dev, orc, dtype, blocks, H, bs, D, batc
     got = f32(untilize_dev(hip, ct, cache.shape, dev))
     want = orc.paged_fill_cache(f32(cache), f32(inp), table.numpy(), idx.numpy() if with_idx else None)
     assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,H,D", [(32, 32, 128), (8, 8, 64), (5, 3, 32), (40, 2, 96)])
+def test_rotary_embedding_split_heads_equals_reshape_then_rotary(hip, dev, dtype, B, H, D):
+    """ttm_rotary_embedding_split_heads on the [users, heads * head_dim] matrix a projection leaves against the plain
+    kernel on the reshaped tensor: bit-identical, padding rows zero."""
+    x = datagen.randn((B, H * D), seed=80, dtype=dtype)
+    cos = datagen.randn((1, 1, 4, D), seed=81, dtype=dtype)
+    sin = datagen.randn((1, 1, 4, D), seed=82, dtype=dtype)
+    code = hip.BF16 if dtype == torch.bfloat16 else hip.F32
+    xt, ct, st = tilize_dev(hip, x, dev), tilize_dev(hip, cos, dev), tilize_dev(hip, sin, dev)
+    x4 = tilize_dev(hip, x.reshape(1, B, H, D), dev)
+    want = torch.full_like(x4, float("nan"))
+    hip.call("ttm_rotary_embedding", hip.ptr(x4), hip.ptr(ct), hip.ptr(st), hip.ptr(want), code, B, H, D, 4, 2, hip.current_stream())
+    got = torch.full_like(x4, float("nan"))
+    hip.call("ttm_rotary_embedding_split_heads", hip.ptr(xt), hip.ptr(ct), hip.ptr(st), hip.ptr(got), code, B, H, D, 4, 2, hip.current_stream())
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    with pytest.raises(hip.TTMError, match="token_index"):
+        hip.call("ttm_rotary_embedding_split_heads", hip.ptr(xt), hip.ptr(ct), hip.ptr(st), hip.ptr(got), code, B, H, D, 4, -1, hip.current_stream())
+
+
+@pytest.mark.parametrize("B,H,Hkv,S,D", [(32, 32, 8, 512, 128), (5, 8, 2, 256, 64), (33, 4, 4, 128, 32)])
+def test_sdpa_decode_concat_heads_equals_reshape_of_the_plain_output(hip, dev, B, H, Hkv, S, D):
+    """ttm_sdpa_decode_concat_heads writes [users, heads * head_dim]: the same values as ttm_sdpa_decode followed by a
+    reshape, zero padding rows below the last user."""
+    q = datagen.randn((1, B, H, D), seed=90, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, S, D), seed=91, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, S, D), seed=92, dtype=torch.bfloat16)
+    cp = torch.randint(0, S, (B,), generator=torch.Generator().manual_seed(93), dtype=torch.int32).to(dev)
+    qt, kt, vt = tilize_dev(hip, q, dev), tilize_dev(hip, k, dev), tilize_dev(hip, v, dev)
+    plain = torch.full_like(qt, float("nan"))
+    args = lambda out: (hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, None, 0, 0, hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 1, 0.0,
+                        hip.current_stream())
+    hip.call("ttm_sdpa_decode", *args(plain))
+    Bp = (B + 31) // 32 * 32
+    merged = torch.full((Bp * H * D,), float("nan"), dtype=torch.bfloat16, device=dev)
+    hip.call("ttm_sdpa_decode_concat_heads", *args(merged))
+    want = untilize_dev(hip, plain, q.shape, dev).reshape(B, H * D)
+    got = untilize_dev(hip, merged, (B, H * D), dev)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert torch.equal(merged, tilize_dev(hip, want.cpu(), dev))          # padding rows are zero

@@ -505,6 +505,9 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
         fused, paired = rt.get_stat("FusedCacheUpdate"), rt.get_stat("PairedMatmul")
         assert (fused, paired) == {"eager": (6, 3), "callbacks": (0, 0)}.get(mode, (fused, paired))
         assert mode != "traced" or (fused in (2, 4) and paired * 2 == fused)
+        # the head splits in front of both rotary embeddings and the head merge behind the attention are folded into
+        # those kernels
+        assert rt.get_stat("FusedHeadSplit") == fused and rt.get_stat("FusedHeadConcat") == paired
     # the replayed graph runs the same kernels on the same data: identical to the op-by-op run, caches included; so is
     # the unfused run
     for other in ("traced", "callbacks"):

@@ -39,10 +39,14 @@ __device__ __forceinline__ void store8(float *p, const float *v) {
 // out[b, s, d] = x[b, s, d] * cos[r, d] + rot(x)[b, s, d] * sin[r, d],  rot(x)[d] = d < D/2 ? -x[d + D/2] : x[d - D/2],
 // r = token_index when given, else s.  One thread per 8 consecutive columns of a face row: the partner columns
 // d +- D/2 are 8 consecutive elements of another face row because D/2 is a multiple of 16.
+// src_cols > 0: x is not laid out like `out` but is the [batch, rows * cols] matrix a projection leaves (row b holds
+// the `rows` heads of user b side by side); the head split [batch, rows * cols] -> [batch, rows, cols] happens on the
+// way in and the padding rows of `out` are written as zeros.
 template <typename T>
 __global__ __launch_bounds__(256) void ttm_rotary_k(const T *__restrict__ x, const T *__restrict__ cosc,
                                                     const T *__restrict__ sinc, T *__restrict__ out, int64_t rows_pad,
-                                                    int64_t cols, int64_t per_batch, int64_t total8, int64_t token_index) {
+                                                    int64_t cols, int64_t per_batch, int64_t total8, int64_t token_index,
+                                                    int64_t rows, int64_t src_cols) {
   int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total8) return;
   const int64_t ct = cols >> 5, half = cols >> 1;
@@ -57,8 +61,19 @@ __global__ __launch_bounds__(256) void ttm_rotary_k(const T *__restrict__ x, con
   const T *xp = x + b * per_batch;
   const int64_t co = ttm_tiled_offset(cr, c, ct);
   float xv[8], pv[8], cv[8], sv[8], ov[8];
-  load8(xp + o, xv);
-  load8(xp + ttm_tiled_offset(r, pc, ct), pv);
+  if (src_cols > 0) {
+    if (r >= rows) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ov[j] = 0.0f;
+      store8(out + b * per_batch + o, ov);
+      return;
+    }
+    load8(x + ttm_tiled_offset(b, r * cols + c, src_cols >> 5), xv);
+    load8(x + ttm_tiled_offset(b, r * cols + pc, src_cols >> 5), pv);
+  } else {
+    load8(xp + o, xv);
+    load8(xp + ttm_tiled_offset(r, pc, ct), pv);
+  }
   load8(cosc + co, cv);
   load8(sinc + co, sv);
 #pragma unroll
@@ -171,6 +186,7 @@ struct DecodeArgs {
   float *part;        // [B * Hkv][splits][G][D + 2]
   uint16_t *out;
   int B, H, Hkv, G, S, D, splits, keys_per_split, block, pages_per_user, mask_heads, is_causal;
+  int concat_heads;   // out is [B, H * D] (row b holds user b's heads side by side) instead of [B, H, D]
   float scale;
 };
 
@@ -409,7 +425,17 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
       den += sl[D + 1] * w;
     }
     const int h = hk * G + g;
-    p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(h, c, D >> 5)] = ttm_f32_to_bf16(den > 0.0f ? num / den : 0.0f);
+    const uint16_t val = ttm_f32_to_bf16(den > 0.0f ? num / den : 0.0f);
+    if (p.concat_heads) p.out[ttm_tiled_offset(b, h * D + c, (p.H * D) >> 5)] = val;
+    else p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(h, c, D >> 5)] = val;
+  }
+  if (p.concat_heads) {   // padding rows below the last user, this kv head's columns
+    if (b == p.B - 1) {
+      const int pad = (int)ttm_round_up32(p.B) - p.B;
+      for (int i = tid0; i < pad * G * D; i += 256)
+        p.out[ttm_tiled_offset(p.B + i / (G * D), hk * G * D + i % (G * D), (p.H * D) >> 5)] = 0;
+    }
+    return;
   }
   if (hk == p.Hkv - 1) {   // padding rows of the last head tile
     const int pad = (int)ttm_round_up32(p.H) - p.H;
@@ -420,10 +446,10 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
 
 }  // namespace
 
-TTM_EXPORT int ttm_rotary_embedding(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype,
-                                    int64_t batch, int64_t rows, int64_t cols, int64_t cache_rows, int64_t token_index,
-                                    void *stream) {
+static int rotary_entry(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype, int64_t batch, int64_t rows,
+                        int64_t cols, int64_t cache_rows, int64_t token_index, bool split, void *stream) {
   TTM_REQUIRE(x && cos_cache && sin_cache && out, "ttm_rotary_embedding: null pointer");
+  TTM_REQUIRE(!split || token_index >= 0, "ttm_rotary_embedding_split_heads: rows are heads here, so the position must come from token_index");
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_rotary_embedding: dtype must be BFloat16 or Float32");
   TTM_REQUIRE(batch >= 0 && rows > 0 && cols > 0 && cols % 32 == 0, "ttm_rotary_embedding: head dim must be a positive multiple of 32");
   if (token_index >= 0)
@@ -434,16 +460,29 @@ TTM_EXPORT int ttm_rotary_embedding(const void *x, const void *cos_cache, const 
                 (long long)cache_rows, (long long)rows);
   if (batch == 0) return TTM_OK;
   const int64_t rows_pad = ttm_round_up32(rows), per_batch = rows_pad * cols, total8 = batch * per_batch / 8;
+  const int64_t src_cols = split ? rows * cols : 0;
   const dim3 grid((unsigned)ttm_cdiv(total8, 256));
   if (dtype == TTM_BF16)
     hipLaunchKernelGGL(ttm_rotary_k<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x,
                        (const uint16_t *)cos_cache, (const uint16_t *)sin_cache, (uint16_t *)out, rows_pad, cols, per_batch,
-                       total8, token_index);
+                       total8, token_index, rows, src_cols);
   else
     hipLaunchKernelGGL(ttm_rotary_k<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float *)x, (const float *)cos_cache,
-                       (const float *)sin_cache, (float *)out, rows_pad, cols, per_batch, total8, token_index);
+                       (const float *)sin_cache, (float *)out, rows_pad, cols, per_batch, total8, token_index, rows, src_cols);
   TTM_LAUNCH_CHECK();
   return TTM_OK;
+}
+
+TTM_EXPORT int ttm_rotary_embedding(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype,
+                                    int64_t batch, int64_t rows, int64_t cols, int64_t cache_rows, int64_t token_index,
+                                    void *stream) {
+  return rotary_entry(x, cos_cache, sin_cache, out, dtype, batch, rows, cols, cache_rows, token_index, false, stream);
+}
+
+TTM_EXPORT int ttm_rotary_embedding_split_heads(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype,
+                                                int64_t batch, int64_t heads, int64_t head_dim, int64_t cache_rows,
+                                                int64_t token_index, void *stream) {
+  return rotary_entry(x, cos_cache, sin_cache, out, dtype, batch, heads, head_dim, cache_rows, token_index, true, stream);
 }
 
 TTM_EXPORT int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users,
@@ -534,10 +573,10 @@ TTM_EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_
   return TTM_OK;
 }
 
-TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
-                               int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out,
-                               int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
-                               int is_causal, float scale, void *stream) {
+static int sdpa_decode_entry(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
+                             const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out, int dtype, int64_t batch,
+                             int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads,
+                             void *stream) {
   TTM_REQUIRE(q && k && v && out, "ttm_sdpa_decode: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa_decode: tensors must be BFloat16");
   TTM_REQUIRE(batch > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "ttm_sdpa_decode: heads must be a multiple of kv heads");
@@ -563,7 +602,7 @@ TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, cons
   p.cur_pos = cur_pos; p.page_table = page_table; p.out = (uint16_t *)out;
   p.B = (int)batch; p.H = (int)heads; p.Hkv = (int)kv_heads; p.G = (int)G; p.S = (int)seq; p.D = (int)head_dim;
   p.splits = (int)splits; p.keys_per_split = (int)keys; p.block = (int)page_block; p.pages_per_user = (int)pages_per_user;
-  p.mask_heads = mask_heads; p.is_causal = is_causal;
+  p.mask_heads = mask_heads; p.is_causal = is_causal; p.concat_heads = concat_heads;
   p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)head_dim);
   void *ws = nullptr;
   if (int rc = ttm_stream_workspace(s, (size_t)(batch * kv_heads * splits * G * (head_dim + 2)) * sizeof(float), &ws)) return rc;
@@ -574,4 +613,20 @@ TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, cons
   hipLaunchKernelGGL(ttm_sdpa_decode_combine_k, dim3((unsigned)(batch * kv_heads)), dim3(256), 0, s, p);
   TTM_LAUNCH_CHECK();
   return TTM_OK;
+}
+
+TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
+                               int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out,
+                               int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
+                               int is_causal, float scale, void *stream) {
+  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
+                           seq, head_dim, is_causal, scale, 0, stream);
+}
+
+TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
+                                            int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block,
+                                            void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
+                                            int64_t head_dim, int is_causal, float scale, void *stream) {
+  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
+                           seq, head_dim, is_causal, scale, 1, stream);
 }

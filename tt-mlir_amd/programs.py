@@ -238,16 +238,13 @@ def _decode_body(pb, a, users, hidden, n_q, n_kv, head_dim, eps):
     a = [x, cos, sin, update_index, cur_pos, k_cache, v_cache, attn_norm_w, wq, wk, wv, wo, mlp_norm_w, wg, wu, wd]."""
     x, cos, sin, upd, cur, kc, vc, anw, wq, wk, wv, wo, mnw, wg, wu, wd = a
     h = pb.rms_norm(x, anw, 0, eps)
-    q = pb.reshape(pb.matmul(h, wq), (1, users, n_q, head_dim))
-    k = pb.reshape(pb.matmul(h, wk), (1, users, n_kv, head_dim))
-    # the value projection goes to its cache at once: reshape -> permute -> update_cache, in the order of the reference's
-    # layer (llama_3_8b_decode_layer.mlir:51-54)
+    # each projection is followed at once by its head split and what consumes it, in the order of the reference's layer
+    # (llama_3_8b_decode_layer.mlir:51-82).  Decode-mode RoPE: cos / sin hold the row of the current position,
+    # token_index = 0 (lib/Dialect/TTNN/Transforms/Fusing/RoPEFusingPattern.cpp:1143-1149)
+    q = pb.rotary_embedding(pb.reshape(pb.matmul(h, wq), (1, users, n_q, head_dim)), cos, sin, token_index=0)
+    k = pb.rotary_embedding(pb.reshape(pb.matmul(h, wk), (1, users, n_kv, head_dim)), cos, sin, token_index=0)
     v = pb.reshape(pb.matmul(h, wv), (1, users, n_kv, head_dim))
     pb.update_cache(vc, pb.permute(v, (0, 2, 1, 3)), upd)
-    # decode-mode RoPE: cos / sin hold the row of the current position, token_index = 0
-    # (lib/Dialect/TTNN/Transforms/Fusing/RoPEFusingPattern.cpp:1143-1149)
-    q = pb.rotary_embedding(q, cos, sin, token_index=0)
-    k = pb.rotary_embedding(k, cos, sin, token_index=0)
     pb.update_cache(kc, pb.permute(k, (0, 2, 1, 3)), upd)
     attn = pb.sdpa_decode(q, kc, vc, cur_pos=cur, is_causal=True)
     merged = pb.reshape(attn, (users, n_q * head_dim))

@@ -259,6 +259,8 @@ void runToMemoryConfig(const fb::Table &op, ProgramContext &ctx) {
 }
 
 std::uint32_t refId(const fb::Table &ref);
+Tensor materialiseView(ProgramContext &ctx, const ProgramContext::DeferredView &v, const std::vector<std::uint32_t> *finalShape);
+fb::Table fusableNext(ProgramContext &ctx, OpType type, int inSlot, int outSlot, const fb::Table &produced, const Tensor &like);
 
 // ---- matmul / linear (runtime/lib/ttnn/operations/matmul/matmul.cpp:47-125)
 Tensor transposeLast2(ProgramContext &ctx, const Tensor &t) {
@@ -348,13 +350,14 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
     }
   }
   // A second matmul of the same activations with a weight tensor of the same shape and format (the K and V projections)
-  // a few ops further on runs in this launch; only reshapes, permutes and deallocations of other tensors may lie between.
+  // a few ops further on runs in this launch; only reshapes, permutes, rotary embeddings and deallocations of other tensors
+  // may lie between.
   if (ctx.fuseViews && tailOp == TTM_TAIL_NONE && !biasRef && activation.empty() && !transposeA && !transposeB && batch == 1 &&
       utils::isBlockFormatDataType(b.handle->dtype) && layoutFromTensorRef(outRef) == Layout{StorageType::Device, TensorLayout::Tile, DataType::BFloat16}) {
-    for (std::uint32_t j = ctx.opIndex + 1; j < ctx.ops.size() && j <= ctx.opIndex + 4; ++j) {
+    for (std::uint32_t j = ctx.opIndex + 1; j < ctx.ops.size() && j <= ctx.opIndex + 6; ++j) {
       const OpType t = opType(j);
       fb::Table nop = ctx.ops[j].table(schema::Operation::f_type);
-      if (t == OpType::ReshapeOp || t == OpType::PermuteOp) continue;
+      if (t == OpType::ReshapeOp || t == OpType::PermuteOp || t == OpType::RotaryEmbeddingOp) continue;   // touch neither operand
       if (t == OpType::DeallocateOp) {
         const std::uint32_t freed = refId(nop.table(schema::DeallocateOp::f_in));
         if (freed == refId(aRef) || freed == refId(outRef)) break;
@@ -590,6 +593,26 @@ Tensor devicePositions(ProgramContext &ctx, const Tensor &t, const char *what) {
 
 void runRotaryEmbedding(const fb::Table &op, ProgramContext &ctx) {
   using S = schema::RotaryEmbeddingOp;
+  if (auto d = ctx.deferred.find(refId(op.table(S::f_input))); d != ctx.deferred.end()) {
+    // the input is the head split [users, heads * head_dim] -> [1, users, heads, head_dim] of a projection, not
+    // materialised (runReshape checked the shapes and that this is decode mode): the kernel splits on the way in
+    const ProgramContext::DeferredView v = d->second;
+    ctx.deferred.erase(d);
+    const DataType dt = v.source.handle->dtype;
+    Tensor cosc = as(ctx, ctx.get(op.table(S::f_cos_cache), "rotary_embedding cos"), TensorLayout::Tile, dt);
+    Tensor sinc = as(ctx, ctx.get(op.table(S::f_sin_cache), "rotary_embedding sin"), TensorLayout::Tile, dt);
+    const auto &cs = cosc.handle->shape;
+    TTRT_ASSERT(cs.size() == 4 && sinc.handle->shape == cs && cs[0] == 1 && cs[1] == 1 && cs[3] == v.shape[3],
+                "rotary_embedding: cos / sin caches must be [1, 1, positions, head_dim]");
+    auto outRef = op.table(S::f_out);
+    Tensor out = makeDeviceTensor(ctx.dev, v.shape, dt, TensorLayout::Tile);
+    debug::Stats::get().incrementStat("FusedHeadSplit");
+    TTM_CALL(ttm_rotary_embedding_split_heads(v.source.handle->data.get(), cosc.handle->data.get(), sinc.handle->data.get(),
+                                              out.handle->data.get(), floatCode(dt, "rotary_embedding"), v.shape[1], v.shape[2], v.shape[3],
+                                              cs[2], op.scalar<std::uint32_t>(S::f_token_index, 0), ctx.stream()));
+    ctx.put(outRef, finish(ctx, out, outRef));
+    return;
+  }
   Tensor &in = ctx.get(op.table(S::f_input), "rotary_embedding input");
   const DataType dt = in.handle->dtype == DataType::Float32 ? DataType::Float32 : DataType::BFloat16;
   Tensor x = as(ctx, in, TensorLayout::Tile, dt);
@@ -754,6 +777,25 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
     pos = devicePositions(ctx, ctx.get(posRef, "sdpa_decode cur_pos"), "sdpa_decode: cur_pos_tensor");
     TTRT_ASSERT(volume(pos.handle->shape) == B, "sdpa_decode: cur_pos_tensor must hold one position per user");
   }
+  // a reshape to [users, heads * head_dim] that is the only consumer of the result (the head merge in front of the output
+  // projection) is folded in: the merge kernel writes that layout directly
+  if (fb::Table rs = fusableNext(ctx, OpType::ReshapeOp, schema::ReshapeOp::f_in, schema::ReshapeOp::f_out, outRef, q)) {
+    auto finalRef = rs.table(schema::ReshapeOp::f_out);
+    const std::vector<std::uint32_t> finalShape = shapeFromTensorRef(finalRef);
+    const Dims3 fd = dims3(finalShape);
+    if (fd.batch == 1 && fd.rows == B && fd.cols == H * D) {
+      Tensor merged = makeDeviceTensor(ctx.dev, finalShape, DataType::BFloat16, TensorLayout::Tile);
+      debug::Stats::get().incrementStat("FusedHeadConcat");
+      TTM_CALL(ttm_sdpa_decode_concat_heads(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
+                                            pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
+                                            mask ? mask.handle->data.get() : nullptr, maskHeads,
+                                            table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
+                                            merged.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, ctx.stream()));
+      ctx.put(finalRef, merged);
+      ctx.skip.insert(ctx.opIndex + 1);
+      return;
+    }
+  }
   Tensor out = makeDeviceTensor(ctx.dev, qs, DataType::BFloat16, TensorLayout::Tile);
   TTM_CALL(ttm_sdpa_decode(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
                            pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
@@ -831,13 +873,34 @@ void runReshape(const fb::Table &op, ProgramContext &ctx) {
     ctx.deferred[refId(outRef)] = ProgramContext::DeferredView{in, oshape, rowMajorStrides(oshape)};   // the permute reads the source directly
     return;
   }
+  // the head split of a projection in front of a decode-mode rotary embedding: [users, heads * head_dim] ->
+  // [1, users, heads, head_dim]; the rotary kernel reads the projection's layout directly
+  if (copies && ctx.fuseViews && ctx.opIndex + 1 < ctx.ops.size() && oshape.size() == 4 && oshape[0] == 1 && oshape[3] % 32 == 0 &&
+      (in.handle->dtype == DataType::BFloat16 || in.handle->dtype == DataType::Float32)) {
+    const fb::Table &next = ctx.ops[ctx.opIndex + 1];
+    const Dims3 sd = dims3(in.handle->shape);
+    if (static_cast<OpType>(next.scalar<std::uint8_t>(schema::Operation::f_type_type, 0)) == OpType::RotaryEmbeddingOp && sd.batch == 1 &&
+        sd.rows == oshape[1] && sd.cols == static_cast<std::int64_t>(oshape[2]) * oshape[3]) {
+      using R = schema::RotaryEmbeddingOp;
+      fb::Table rop = next.table(schema::Operation::f_type);
+      fb::Table rin = rop.table(R::f_input), rout = rop.table(R::f_out);
+      auto u = ctx.uses.find(refId(outRef));
+      const Layout a = layoutFromTensorRef(outRef);
+      if (rin && rout && refId(rin) == refId(outRef) && rop.has(R::f_token_index) && u != ctx.uses.end() && u->second == 1 &&
+          a.storageType == StorageType::Device && a.layout == TensorLayout::Tile && a.dataType == in.handle->dtype &&
+          layoutFromTensorRef(rout) == a) {
+        ctx.deferred[refId(outRef)] = ProgramContext::DeferredView{in, oshape, rowMajorStrides(oshape)};
+        return;
+      }
+    }
+  }
   ctx.put(outRef, finish(ctx, reshapeTo(ctx, in, oshape), outRef));
 }
 
 // A strided view of `source` written out as a tensor of its own: element v of the view (row-major over `shape`) is
 // the source element with row-major index sum v[d] * strides[d].  `finalShape` gives the output another logical shape
 // of the same volume (a reshape is the identity on flat indices).
-Tensor materialiseView(ProgramContext &ctx, const ProgramContext::DeferredView &v, const std::vector<std::uint32_t> *finalShape = nullptr) {
+Tensor materialiseView(ProgramContext &ctx, const ProgramContext::DeferredView &v, const std::vector<std::uint32_t> *finalShape) {
   if (finalShape) TTRT_ASSERT(volume(*finalShape) == volume(v.shape), "reshape: element count differs");
   Tensor out = makeDeviceTensor(ctx.dev, finalShape ? *finalShape : v.shape, v.source.handle->dtype, v.source.handle->layout);
   zeroIfPadded(ctx, out);
@@ -857,7 +920,7 @@ ProgramContext::DeferredView permutedView(const ProgramContext::DeferredView &in
   return out;
 }
 Tensor permuteTo(ProgramContext &ctx, const Tensor &in, const std::vector<int> &perm) {
-  return materialiseView(ctx, permutedView(ProgramContext::DeferredView{in, in.handle->shape, rowMajorStrides(in.handle->shape)}, perm));
+  return materialiseView(ctx, permutedView(ProgramContext::DeferredView{in, in.handle->shape, rowMajorStrides(in.handle->shape)}, perm), nullptr);
 }
 // the next operation is an update_cache that is the only consumer of `produced` (as its input) and whose cache holds
 // the element type of `like`: it can read the view directly
@@ -908,7 +971,7 @@ void runPermute(const fb::Table &op, ProgramContext &ctx) {
       return;
     }
   }
-  ctx.put(outRef, finish(ctx, materialiseView(ctx, view), outRef));
+  ctx.put(outRef, finish(ctx, materialiseView(ctx, view, nullptr), outRef));
 }
 void runTranspose(const fb::Table &op, ProgramContext &ctx) {
   Tensor in = onDevice(ctx, ctx.get(op.table(schema::TransposeOp::f_in), "transpose in"));
