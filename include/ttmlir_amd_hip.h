@@ -192,6 +192,14 @@ int ttm_copy_view_at(const void *src, int64_t src_rows, int64_t src_cols, int sr
 int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype,
              int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale,
              void *stream);
+/* ttm_sdpa on operands that keep their heads side by side, as the projections leave them and the output projection
+ * wants them: heads_inner bit 0: q is [B, Sq, Hq * D]; bit 1: k is [B, Sk, Hkv * D]; bit 2: v likewise; bit 3: out is
+ * [B, Sq, Hq * D].  Both layouts hold the same 32 x 32 tiles in another order, so the head split (reshape + permute in
+ * front, or ::ttnn::transformer::split_query_key_value_and_split_heads) and the head merge (permute + reshape behind, or
+ * ::ttnn::transformer::concatenate_heads, runtime/lib/ttnn/operations/transformer/concatenate_heads.cpp) cost nothing. */
+int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
+                         int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal,
+                         float scale, int heads_inner, void *stream);
 
 /* ---- decode path: rotary embedding, KV-cache writes, attention of one new token over the cache.  TILE layout
  * throughout; positions (update index, current position, page table) are Int32 / UInt32 values in DEVICE memory, read

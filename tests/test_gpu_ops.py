@@ -321,3 +321,38 @@ def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask, variant):
     # probabilities are rounded to bf16 before P.V (relative 2^-9 each) and the output once more
     assert np.max(np.abs(res - want)) <= 2.0 ** -6
     assert metrics.get_pcc(want, res) >= 0.9999
+
+
+@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("flags", [15, 1, 6, 8, 9])
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", [(1, 8, 2, 256, 256, 128, True), (2, 4, 4, 96, 160, 64, False), (1, 4, 1, 70, 70, 32, True),
+                                                      (1, 2, 2, 40, 300, 256, False)])
+def test_sdpa_heads_inner_equals_the_head_major_call(hip, dev, B, Hq, Hkv, Sq, Sk, D, causal, flags, variant):
+    """ttm_sdpa_heads_inner with q / k / v / out (any subset, by flag) laid out [B, S, H * D], heads side by side, against
+    ttm_sdpa on [B, H, S, D]: both layouts hold the same tiles in another order, so the results are identical bit for
+    bit once the output is brought back to one shape."""
+    q = datagen.randn((B, Hq, Sq, D), seed=22, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, Sk, D), seed=23, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, Sk, D), seed=24, dtype=torch.bfloat16)
+    inner = lambda t: t.permute(0, 2, 1, 3).reshape(t.shape[0], t.shape[2], t.shape[1] * t.shape[3]).contiguous()
+    hip.set_option("sdpa_variant", variant)
+    try:
+        qt, kt, vt = (tilize_dev(hip, t, dev) for t in (q, k, v))
+        want_t = torch.full_like(qt, float("nan"))
+        hip.call("ttm_sdpa", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, 1, hip.ptr(want_t), hip.BF16, B, Hq, Hkv, Sq, Sk, D, int(causal), 0.0,
+                 hip.current_stream())
+        want = untilize_dev(hip, want_t, q.shape, dev).cpu()
+        qi = tilize_dev(hip, inner(q), dev) if flags & 1 else qt
+        ki = tilize_dev(hip, inner(k), dev) if flags & 2 else kt
+        vi = tilize_dev(hip, inner(v), dev) if flags & 4 else vt
+        out = torch.full_like(qt, float("nan"))
+        hip.call("ttm_sdpa_heads_inner", hip.ptr(qi), hip.ptr(ki), hip.ptr(vi), None, 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, Sq, Sk, D, int(causal),
+                 0.0, flags, hip.current_stream())
+    finally:
+        hip.set_option("sdpa_variant", 0)
+    if flags & 8:
+        got = untilize_dev(hip, out, (B, Sq, Hq * D), dev).cpu().reshape(B, Sq, Hq, D).permute(0, 2, 1, 3)
+    else:
+        got = untilize_dev(hip, out, q.shape, dev).cpu()
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)

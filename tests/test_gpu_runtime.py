@@ -616,6 +616,8 @@ def test_fused_epilogue_tails_do_not_change_program_results(device):
     (fused,) = harness.execute(binary, 1, tins, device)
     assert rt.get_stat("FusedLinearTail") == 3          # attention residual, gate * up, MLP residual
     assert rt.get_stat("PairedMatmul") == 1             # K and V projections in one launch
+    assert rt.get_stat("SdpaHeadsInner") == 1           # attention reads the projections and writes the merged heads in place
+    assert rt.get_stat("CopyViewLaunch") == 0           # no head split or merge is materialised
     seen = []
     rt.set_post_op_callback(lambda idx, name, dbg, hook: seen.append(name))
     try:

@@ -24,6 +24,11 @@ struct SdpaArgs {
   int mask_heads;    // 1 or Hq
   int causal;
   float scale;
+  // Where a row of tiles of one head lives, per operand, in bytes: matrix (b, h) starts at b * batch + h * head, its tile
+  // row t at + t * pitch (the D / 32 tiles of a tile row are contiguous).  [B, H, S, D]: pitch = D / 32 tiles, head =
+  // S / 32 * pitch, batch = H * head.  [B, S, H * D] (heads side by side, as a projection leaves them): pitch = H * D / 32
+  // tiles, head = D / 32 tiles, batch = S / 32 * pitch.  Same 32 x 32 tiles either way.
+  int64_t q_pitch, q_head, q_batch, k_pitch, k_head, k_batch, v_pitch, v_head, v_batch, o_pitch, o_head, o_batch;
 };
 
 __device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
@@ -42,8 +47,8 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
   const int qt = qb * 4 + wave;                         // this wave's query tile
   const bool wave_ok = qt < p.sqt;
   const int l31 = lane & 31, hh = lane >> 5;
-  const int64_t q_mat = ((int64_t)b * p.Hq + h) * p.sqt * DT * 2048;
-  const int64_t kv_mat = ((int64_t)b * p.Hkv + hk) * p.skt * DT * 2048;
+  const int64_t q_mat = b * p.q_batch + h * p.q_head, o_mat = b * p.o_batch + h * p.o_head;
+  const int64_t k_mat = b * p.k_batch + hk * p.k_head, v_mat = b * p.v_batch + hk * p.v_head;
 
   // Q fragments: B operand, lane (q = l31, hh): d = 16 s + 8 hh .. +7
   bf16x8 qf[2 * DT];
@@ -51,7 +56,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
   for (int s = 0; s < 2 * DT; ++s) {
     u32x4 v = {0, 0, 0, 0};
     if (wave_ok)
-      v = *(const u32x4 *)(p.q + q_mat + ((int64_t)qt * DT + (s >> 1)) * 2048 + ((l31 >> 4) * 2 + (s & 1)) * 512 +
+      v = *(const u32x4 *)(p.q + q_mat + qt * p.q_pitch + (s >> 1) * 2048 + ((l31 >> 4) * 2 + (s & 1)) * 512 +
                            (l31 & 15) * 32 + hh * 16);
     qf[s] = *(bf16x8 *)&v;
   }
@@ -71,8 +76,8 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
   constexpr int NC = (DT * 128 + 255) / 256;   // 16-byte chunks of a K (or V) block per lane
   u32x4 kreg[NC], vreg[NC];
   auto load_block = [&](int kt) {
-    const u32x4 *ks = (const u32x4 *)(p.k + kv_mat + (int64_t)kt * DT * 2048);
-    const u32x4 *vs = (const u32x4 *)(p.v + kv_mat + (int64_t)kt * DT * 2048);
+    const u32x4 *ks = (const u32x4 *)(p.k + k_mat + kt * p.k_pitch);
+    const u32x4 *vs = (const u32x4 *)(p.v + v_mat + kt * p.v_pitch);
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
       if (tid + 256 * i < DT * 128) {
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
       u32x2 ov;
       ov.x = q_ok ? pack_bf16_rne(o[d][g * 4 + 0] * inv, o[d][g * 4 + 1] * inv) : 0u;
       ov.y = q_ok ? pack_bf16_rne(o[d][g * 4 + 2] * inv, o[d][g * 4 + 3] * inv) : 0u;
-      uint8_t *op = p.out + q_mat + ((int64_t)qt * DT + d) * 2048 +
+      uint8_t *op = p.out + o_mat + qt * p.o_pitch + d * 2048 +
                     (((l31 >> 4) * 2 + (din >> 4)) * 256 + (l31 & 15) * 16 + (din & 15)) * 2;
       *(u32x2 *)op = ov;
     }
@@ -227,15 +232,15 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
   const int qt = qb * 4 + wave;                         // this wave's query tile
   const bool wave_ok = qt < p.sqt;
   const int l31 = lane & 31, hh = lane >> 5;
-  const int64_t q_mat = ((int64_t)b * p.Hq + h) * p.sqt * DT * 2048;
-  const int64_t kv_mat = ((int64_t)b * p.Hkv + hk) * p.skt * DT * 2048;
+  const int64_t q_mat = b * p.q_batch + h * p.q_head, o_mat = b * p.o_batch + h * p.o_head;
+  const int64_t k_mat = b * p.k_batch + hk * p.k_head, v_mat = b * p.v_batch + hk * p.v_head;
 
   bf16x8 qf[2 * DT];
 #pragma unroll
   for (int s = 0; s < 2 * DT; ++s) {
     u32x4 v = {0, 0, 0, 0};
     if (wave_ok)
-      v = *(const u32x4 *)(p.q + q_mat + ((int64_t)qt * DT + (s >> 1)) * 2048 + ((l31 >> 4) * 2 + (s & 1)) * 512 +
+      v = *(const u32x4 *)(p.q + q_mat + qt * p.q_pitch + (s >> 1) * 2048 + ((l31 >> 4) * 2 + (s & 1)) * 512 +
                            (l31 & 15) * 32 + hh * 16);
     qf[s] = *(bf16x8 *)&v;
   }
@@ -257,8 +262,8 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
     for (int i = 0; i < DT; ++i) {
       const int c = tid + 256 * i, tr = c / (DT * 128), cc = c % (DT * 128);
       const int kt = min(2 * kb + tr, p.skt - 1);       // an odd tile count repeats the last tile; its keys are masked
-      kreg[i] = ((const u32x4 *)(p.k + kv_mat + (int64_t)kt * DT * 2048))[cc];
-      vreg[i] = ((const u32x4 *)(p.v + kv_mat + (int64_t)kt * DT * 2048))[cc];
+      kreg[i] = ((const u32x4 *)(p.k + k_mat + kt * p.k_pitch))[cc];
+      vreg[i] = ((const u32x4 *)(p.v + v_mat + kt * p.v_pitch))[cc];
     }
   };
   if (kb_end > 0) load_block(0);
@@ -407,7 +412,7 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
       u32x2 ov;
       ov.x = q_ok ? pack_bf16_rne(o[d][g * 4 + 0] * inv, o[d][g * 4 + 1] * inv) : 0u;
       ov.y = q_ok ? pack_bf16_rne(o[d][g * 4 + 2] * inv, o[d][g * 4 + 3] * inv) : 0u;
-      uint8_t *op = p.out + q_mat + ((int64_t)qt * DT + d) * 2048 +
+      uint8_t *op = p.out + o_mat + qt * p.o_pitch + d * 2048 +
                     (((l31 >> 4) * 2 + (din >> 4)) * 256 + (l31 & 15) * 16 + (din & 15)) * 2;
       *(u32x2 *)op = ov;
     }
@@ -432,9 +437,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if (light < heavy) sdpa64_query_block<DT>(p, light, h, b, ldsK, ldsV);
 }
 
-TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
-                        int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
-                        int is_causal, float scale, void *stream) {
+static int sdpa_entry(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B,
+                      int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int heads_inner, void *stream) {
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa: tensors must be BFloat16 (got %d)", dtype);
   TTM_REQUIRE(B >= 0 && Hq >= 0 && Hkv > 0 && Sq >= 0 && Sk >= 0 && D > 0, "ttm_sdpa: bad dimension");
   TTM_REQUIRE(Hq % Hkv == 0, "ttm_sdpa: query heads (%ld) must be a multiple of kv heads (%ld)", (long)Hq, (long)Hkv);
@@ -451,6 +455,16 @@ TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void 
   p.sqt = (int)ttm_cdiv(Sq, 32); p.skt = (int)ttm_cdiv(Sk, 32);
   p.mask_heads = mask_heads; p.causal = is_causal;
   p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)D);
+  TTM_REQUIRE(heads_inner >= 0 && heads_inner < 16, "ttm_sdpa: unknown layout flags %d", heads_inner);
+  auto place = [&](bool inner, int64_t heads, int st, int64_t &pitch, int64_t &head, int64_t &batch) {
+    const int64_t dt = D / 32 * 2048;   // bytes of the tiles of one head in one tile row
+    if (inner) { pitch = heads * dt; head = dt; batch = st * pitch; }
+    else { pitch = dt; head = st * dt; batch = heads * head; }
+  };
+  place(heads_inner & 1, Hq, p.sqt, p.q_pitch, p.q_head, p.q_batch);
+  place(heads_inner & 2, Hkv, p.skt, p.k_pitch, p.k_head, p.k_batch);
+  place(heads_inner & 4, Hkv, p.skt, p.v_pitch, p.v_head, p.v_batch);
+  place(heads_inner & 8, Hq, p.sqt, p.o_pitch, p.o_head, p.o_batch);
   dim3 grid((unsigned)ttm_cdiv(p.sqt, 4), (unsigned)Hq, (unsigned)B), block(256);
   hipStream_t s = (hipStream_t)stream;
   const int variant = ttm_option("sdpa_variant");   // 1 = 32 keys per pass, 2 = 64 keys without pairing query blocks
@@ -466,4 +480,16 @@ TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void 
   }
   TTM_LAUNCH_CHECK();
   return TTM_OK;
+}
+
+TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
+                        int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
+                        int is_causal, float scale, void *stream) {
+  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, 0, stream);
+}
+
+TTM_EXPORT int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
+                                    int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
+                                    int is_causal, float scale, int heads_inner, void *stream) {
+  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner, stream);
 }

@@ -42,6 +42,9 @@ struct ProgramContext {
   bool fuseViews = false;
   std::unordered_map<std::uint32_t, int> uses;      // consumers of a tensor (deallocations not counted; program outputs are)
   std::unordered_map<std::uint32_t, DeferredView> deferred;
+  // head splits that feed scaled_dot_product_attention only: tensor id -> the [B, S, H * D] tensor it is the
+  // [B, H, S, D] view of.  The id is not in the pool; the attention kernel reads the source in place.
+  std::unordered_map<std::uint32_t, Tensor> headViews;
   std::set<std::uint32_t> skip;
 
   Tensor &get(const fb::Table &ref, const char *what) {
@@ -551,13 +554,28 @@ void runReduction(const fb::Table &op, ProgramContext &ctx) {
 // ---- attention (runtime/lib/ttnn/operations/transformer/scaled_dot_product_attention.cpp:14-55)
 void runSdpa(const fb::Table &op, ProgramContext &ctx) {
   using S = schema::ScaledDotProductAttentionOp;
-  Tensor q = as(ctx, ctx.get(op.table(S::f_query), "sdpa query"), TensorLayout::Tile, DataType::BFloat16);
-  Tensor k = as(ctx, ctx.get(op.table(S::f_key), "sdpa key"), TensorLayout::Tile, DataType::BFloat16);
-  Tensor v = as(ctx, ctx.get(op.table(S::f_value), "sdpa value"), TensorLayout::Tile, DataType::BFloat16);
-  TTRT_ASSERT(q.handle->shape.size() == 4 && k.handle->shape.size() == 4 && v.handle->shape.size() == 4, "sdpa: q, k, v must be rank 4");
+  // an operand may be a head split that was never materialised (ctx.headViews): then the tensor at hand is the
+  // [B, S, H * D] source and the kernel is told so; shapes come from the program's tensor refs
+  int inner = 0;
+  auto operand = [&](const fb::Table &ref, int bit, const char *what) {
+    auto hv = ctx.headViews.find(refId(ref));
+    if (hv != ctx.headViews.end()) {
+      Tensor t = hv->second;
+      ctx.headViews.erase(hv);
+      inner |= bit;
+      return t;
+    }
+    return as(ctx, ctx.get(ref, what), TensorLayout::Tile, DataType::BFloat16);
+  };
+  Tensor q = operand(op.table(S::f_query), 1, "sdpa query");
+  Tensor k = operand(op.table(S::f_key), 2, "sdpa key");
+  Tensor v = operand(op.table(S::f_value), 4, "sdpa value");
+  const std::vector<std::uint32_t> qs = (inner & 1) ? shapeFromTensorRef(op.table(S::f_query)) : q.handle->shape;
+  const std::vector<std::uint32_t> ks = (inner & 2) ? shapeFromTensorRef(op.table(S::f_key)) : k.handle->shape;
+  const std::vector<std::uint32_t> vs = (inner & 4) ? shapeFromTensorRef(op.table(S::f_value)) : v.handle->shape;
+  TTRT_ASSERT(qs.size() == 4 && ks.size() == 4 && vs.size() == 4, "sdpa: q, k, v must be rank 4");
   TTRT_ASSERT(!op.has(S::f_sliding_window_size) && !op.table(S::f_attention_sink), "sdpa: sliding window / attention sink are not supported");
-  const auto &qs = q.handle->shape, &ks = k.handle->shape;
-  TTRT_ASSERT(k.handle->shape == v.handle->shape && qs[0] == ks[0] && qs[3] == ks[3], "sdpa: q/k/v shapes do not agree");
+  TTRT_ASSERT(ks == vs && qs[0] == ks[0] && qs[3] == ks[3], "sdpa: q/k/v shapes do not agree");
   Tensor mask;
   int maskHeads = 1;
   if (auto mr = op.table(S::f_attention_mask)) {
@@ -571,9 +589,52 @@ void runSdpa(const fb::Table &op, ProgramContext &ctx) {
   TTRT_ASSERT(!(causal && mask), "sdpa: is_causal and an explicit mask are mutually exclusive");
   float scale = op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f;
   auto outRef = op.table(S::f_out);
-  Tensor out = makeDeviceTensor(ctx.dev, qs, DataType::BFloat16, TensorLayout::Tile);
-  TTM_CALL(ttm_sdpa(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(), mask ? mask.handle->data.get() : nullptr, maskHeads,
-                    out.handle->data.get(), TTM_BF16, qs[0], qs[1], ks[1], qs[2], ks[2], qs[3], causal ? 1 : 0, scale, ctx.stream()));
+  // The head merge behind the attention - permute (0, 2, 1, 3) and reshape to [.., Sq, Hq * D], each the only consumer of
+  // what precedes it, deallocations of other tensors between them allowed - is folded in: the kernel writes that layout.
+  fb::Table mergedRef;
+  std::vector<std::uint32_t> skipped;
+  if (ctx.fuseViews && qs[3] % 32 == 0) {
+    auto opType = [&](std::uint32_t i) { return static_cast<OpType>(ctx.ops[i].scalar<std::uint8_t>(schema::Operation::f_type_type, 0)); };
+    auto soleUse = [&](const fb::Table &r) { auto u = ctx.uses.find(refId(r)); return u != ctx.uses.end() && u->second == 1; };
+    auto nextReal = [&](std::uint32_t i, std::uint32_t avoid) {   // first op after i that is not a deallocation of another tensor
+      for (++i; i < ctx.ops.size() && opType(i) == OpType::DeallocateOp; ++i)
+        if (refId(ctx.ops[i].table(schema::Operation::f_type).table(schema::DeallocateOp::f_in)) == avoid) return static_cast<std::uint32_t>(ctx.ops.size());
+      return i;
+    };
+    const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
+    const std::uint32_t pi = nextReal(ctx.opIndex, refId(outRef));
+    if (pi < ctx.ops.size() && opType(pi) == OpType::PermuteOp && soleUse(outRef) && layoutFromTensorRef(outRef) == plain) {
+      fb::Table pop = ctx.ops[pi].table(schema::Operation::f_type);
+      fb::Table pin = pop.table(schema::PermuteOp::f_in), pout = pop.table(schema::PermuteOp::f_out);
+      auto pv = pop.scalars<std::int64_t>(schema::PermuteOp::f_permutation);
+      const bool swaps = pv.size() == 4 && pv[0] == 0 && pv[1] == 2 && pv[2] == 1 && pv[3] == 3;
+      if (pin && pout && refId(pin) == refId(outRef) && swaps && soleUse(pout) && layoutFromTensorRef(pout) == plain) {
+        const std::uint32_t ri = nextReal(pi, refId(pout));
+        if (ri < ctx.ops.size() && opType(ri) == OpType::ReshapeOp) {
+          fb::Table rop = ctx.ops[ri].table(schema::Operation::f_type);
+          fb::Table rin = rop.table(schema::ReshapeOp::f_in), rout = rop.table(schema::ReshapeOp::f_out);
+          if (rin && rout && refId(rin) == refId(pout) && layoutFromTensorRef(rout) == plain) {
+            const Dims3 fd = dims3(shapeFromTensorRef(rout));
+            if (fd.batch == qs[0] && fd.rows == qs[2] && fd.cols == static_cast<std::int64_t>(qs[1]) * qs[3]) {
+              mergedRef = rout;
+              skipped = {pi, ri};
+            }
+          }
+        }
+      }
+    }
+  }
+  if (mergedRef) inner |= 8;
+  Tensor out = makeDeviceTensor(ctx.dev, mergedRef ? shapeFromTensorRef(mergedRef) : qs, DataType::BFloat16, TensorLayout::Tile);
+  if (inner) debug::Stats::get().incrementStat("SdpaHeadsInner");
+  TTM_CALL(ttm_sdpa_heads_inner(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(), mask ? mask.handle->data.get() : nullptr,
+                                maskHeads, out.handle->data.get(), TTM_BF16, qs[0], qs[1], ks[1], qs[2], ks[2], qs[3], causal ? 1 : 0, scale,
+                                inner, ctx.stream()));
+  if (mergedRef) {
+    ctx.put(mergedRef, out);
+    for (std::uint32_t i : skipped) ctx.skip.insert(i);
+    return;
+  }
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 
@@ -941,6 +1002,36 @@ bool feedsUpdateCache(ProgramContext &ctx, const fb::Table &produced, const Tens
   return c != ctx.pool.end() && isTensorAllocated(c->second) && c->second.handle->storage == StorageType::Device &&
          c->second.handle->layout == TensorLayout::Tile && c->second.handle->dtype == like.handle->dtype;
 }
+// `view` is the head split [B, S, H * D] -> [B, H, S, D] of a tile tensor (whole tiles move, nothing inside them), and
+// the only consumer of `produced` is a scaled_dot_product_attention that takes it as query, key or value
+bool headSplitForSdpa(ProgramContext &ctx, const fb::Table &produced, const ProgramContext::DeferredView &view) {
+  if (!ctx.fuseViews || view.shape.size() != 4) return false;
+  const Tensor &src = view.source;
+  const std::int64_t B = view.shape[0], H = view.shape[1], Sq = view.shape[2], D = view.shape[3];
+  if (src.handle->dtype != DataType::BFloat16 || src.handle->layout != TensorLayout::Tile || src.handle->storage != StorageType::Device) return false;
+  if (D % 32 != 0 || !(D == 32 || D == 64 || D == 128 || D == 256)) return false;
+  const Dims3 sd = dims3(src.handle->shape);
+  if (sd.batch != B || sd.rows != Sq || sd.cols != H * D) return false;
+  if (view.strides[3] != 1 || view.strides[2] != H * D || view.strides[1] != D || (B > 1 && view.strides[0] != Sq * H * D)) return false;
+  if (!(layoutFromTensorRef(produced) == Layout{StorageType::Device, TensorLayout::Tile, DataType::BFloat16})) return false;
+  const std::uint32_t id = refId(produced);
+  auto u = ctx.uses.find(id);
+  if (u == ctx.uses.end() || u->second != 1) return false;
+  for (std::uint32_t j = ctx.opIndex + 1; j < ctx.ops.size(); ++j) {
+    const OpType t = static_cast<OpType>(ctx.ops[j].scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
+    if (t == OpType::DeallocateOp) continue;
+    bool reads = false;
+    for (const auto &ref : opRefs(ctx.ops[j]).ins) reads = reads || refId(ref) == id;
+    if (!reads) continue;
+    if (t != OpType::ScaledDotProductAttentionOp) return false;
+    using S = schema::ScaledDotProductAttentionOp;
+    fb::Table sop = ctx.ops[j].table(schema::Operation::f_type);
+    int named = 0;
+    for (int slot : {int(S::f_query), int(S::f_key), int(S::f_value)}) named += sop.table(slot) && refId(sop.table(slot)) == id;
+    return named == 1;   // not the mask, and not two operands at once
+  }
+  return false;
+}
 void runPermute(const fb::Table &op, ProgramContext &ctx) {
   auto inRef = op.table(schema::PermuteOp::f_in);
   auto pv = op.scalars<std::int64_t>(schema::PermuteOp::f_permutation);
@@ -961,6 +1052,10 @@ void runPermute(const fb::Table &op, ProgramContext &ctx) {
   if (src.handle->layout == TensorLayout::Tile && !utils::isBlockFormatDataType(src.handle->dtype)) {
     if (feedsUpdateCache(ctx, outRef, src)) {
       ctx.deferred[refId(outRef)] = view;   // the cache write reads the source directly
+      return;
+    }
+    if (headSplitForSdpa(ctx, outRef, view)) {
+      ctx.headViews[refId(outRef)] = src;   // the attention kernel reads the projection's layout in place
       return;
     }
     if (fb::Table rs = fusableNext(ctx, OpType::ReshapeOp, schema::ReshapeOp::f_in, schema::ReshapeOp::f_out, outRef, src)) {
@@ -1105,6 +1200,7 @@ void runEmpty(const fb::Table &op, ProgramContext &ctx) {
 void runDeallocate(const fb::Table &op, ProgramContext &ctx) {
   auto ref = op.table(schema::DeallocateOp::f_in);
   std::uint32_t id = ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
+  ctx.headViews.erase(id);
   auto it = ctx.pool.find(id);
   if (it == ctx.pool.end()) return;
   if (getTensorRetain(it->second)) return;  // runtime/lib/ttnn/operations/deletion/deallocate.cpp:16-18
