@@ -397,3 +397,42 @@ def test_two_pass_launch_with_batches_pairs_and_tails(hip, dev, orc, metrics):
         hip.set_option("linear_two_pass", 0)
     for x, y in zip(res[1], res[2]):
         assert torch.equal(x.view(torch.int16), y.view(torch.int16))   # bit patterns: the padding may hold NaN
+
+
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4"])
+@pytest.mark.parametrize("M,K,Ns,options", [
+    (32, 1024, (512, 128, 128), {"linear_decode_split": 2}),       # decode kernel, k-slices, reduction that knows the members
+    (20, 520, (200, 72, 72, 40), {"linear_decode_split": 1}),      # ragged everywhere, four members, direct epilogue
+    (64, 256, (96, 160), {"linear_decode_split": 3}),              # two row tiles
+    (330, 232, (677, 100, 300), {"linear_split_k": 1, "linear_two_pass": 1}),   # fused main kernel
+    (512, 256, (1024, 256, 256), {"linear_split_k": 1, "linear_two_pass": 2}),  # two passes: one image launch for all members
+    (2048, 128, (2048, 512, 512), {"linear_split_k": 1, "linear_two_pass": 2, "linear_ntw": 7}),   # 7-wide blocks, several rounds
+    (288, 160, (320, 64), {"linear_split_k": 1, "linear_two_pass": 1, "linear_ntw": 3}),
+])
+def test_linear_group_equals_separate_launches(hip, dev, wfmt_name, M, K, Ns, options):
+    """ttm_linear_group (several weight matrices of different widths against the same activations in one launch) against one
+    ttm_linear call per member under the same launch plan: bit exact."""
+    import ctypes
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    a = datagen.randn((M, K), seed=101, dtype=torch.bfloat16)
+    ws = [datagen.randn((K, N), seed=102 + i, std=0.05) for i, N in enumerate(Ns)]
+    for k, v in options.items():
+        hip.set_option(k, v)
+    try:
+        want = [run_linear(hip, dev, a, w, None, None, wfmt)[0] for w in ws]
+        at = tilize_dev(hip, a, dev)
+        wt = [pack_weight(hip, w, wfmt, dev) for w in ws]
+        Mp = (M + 31) // 32 * 32
+        outs = [torch.full((Mp * ((N + 31) // 32 * 32),), float("nan"), dtype=torch.bfloat16, device=dev) for N in Ns]
+        n = len(Ns)
+        wp = (ctypes.c_void_p * n)(*[t.data_ptr() for t in wt])
+        op = (ctypes.c_void_p * n)(*[t.data_ptr() for t in outs])
+        nn = (ctypes.c_int64 * n)(*Ns)
+        hip.call("ttm_linear_group", hip.ptr(at), n, wp, wfmt, op, nn, M, K, hip.current_stream())
+        got = [untilize_dev(hip, o, (M, N), dev).cpu() for o, N in zip(outs, Ns)]
+        torch.cuda.synchronize()
+    finally:
+        for k in options:
+            hip.set_option(k, 0)
+    for g, w in zip(got, want):
+        assert torch.equal(g, w)

@@ -500,9 +500,10 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
         if mode == "traced":
             assert rt.get_stat("CapturedTrace") >= 1
         # both cache writes read their permuted operand as a view (K after the rotary embedding, V straight from the
-        # reshaped projection), the K and V projections share a launch; nothing of this with a callback registered
+        # reshaped projection), the Q, K and V projections share a launch; nothing of this with a callback registered
         # (a traced program runs its body op by op only until the graph is recorded)
-        fused, paired = rt.get_stat("FusedCacheUpdate"), rt.get_stat("PairedMatmul")
+        fused, paired = rt.get_stat("FusedCacheUpdate"), rt.get_stat("GroupedMatmul")
+        assert rt.get_stat("GroupedMatmulMembers") == 3 * paired          # Q, K and V projections in one launch
         assert (fused, paired) == {"eager": (6, 3), "callbacks": (0, 0)}.get(mode, (fused, paired))
         assert mode != "traced" or (fused in (2, 4) and paired * 2 == fused)
         # the head splits in front of both rotary embeddings and the head merge behind the attention are folded into
@@ -615,7 +616,7 @@ def test_fused_epilogue_tails_do_not_change_program_results(device):
     rt.clear_stats()
     (fused,) = harness.execute(binary, 1, tins, device)
     assert rt.get_stat("FusedLinearTail") == 3          # attention residual, gate * up, MLP residual
-    assert rt.get_stat("PairedMatmul") == 1             # K and V projections in one launch
+    assert rt.get_stat("GroupedMatmul") == 1 and rt.get_stat("GroupedMatmulMembers") == 3   # Q, K and V projections in one launch
     assert rt.get_stat("SdpaHeadsInner") == 1           # attention reads the projections and writes the merged heads in place
     assert rt.get_stat("CopyViewLaunch") == 0           # no head split or merge is materialised
     seen = []

@@ -46,9 +46,42 @@ struct LinearArgs {
   int k_slice;                        // k-tiles per grid.y slice (split-K); Kt when the reduction is not split
   float *partial;                     // split-K: fp32 partial sums [slices][Mt * Nt * 1024] in output tile order
   int img_zero_step;                  // two-pass launch: W points at the dequantised images, this step index holds zeros
+  // group launch (group_n >= 2): several weight matrices [K, N_i] applied to the same activations, each with its own
+  // output; W / C / Nt above describe the virtual concatenation (Nt = sum of the members' column tiles) and are not
+  // dereferenced.  No bias, activation, tail or batch in a group.
+  int group_n;
+  const uint8_t *gW[4];
+  uint8_t *gC[4];
+  int gNt[4];
   int tail;                           // 0 none, 1 add, 2 multiply: element-wise tail with a tensor laid out like the output
   int64_t tail_delta;                 // byte distance from an output element to its tail operand
 };
+
+// The member of a group launch that owns column unit `u`, where a unit is `unit_tiles` column tiles and every member's
+// units are numbered one after another (a member's last unit may be partial).  Constant indices only: the arrays stay in
+// scalar registers.
+struct GroupMember {
+  const uint8_t *W;
+  uint8_t *C;
+  int Nt, local, tile_base;   // column tiles, unit index inside the member, first column tile in the concatenation
+};
+__device__ __forceinline__ GroupMember group_member(const LinearArgs &p, int u, int unit_tiles) {
+  GroupMember m = {p.gW[0], p.gC[0], p.gNt[0], u, 0};
+  int start = 0, tiles = 0;
+  bool found = false;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    if (j < p.group_n) {
+      const int n = (p.gNt[j] + unit_tiles - 1) / unit_tiles;
+      if (!found && (u < start + n || j == p.group_n - 1)) {
+        found = true;
+        m.W = p.gW[j]; m.C = p.gC[j]; m.Nt = p.gNt[j]; m.local = u - start; m.tile_base = tiles;
+      }
+      start += n; tiles += p.gNt[j];
+    }
+  }
+  return m;
+}
 
 template <int ACT>
 __device__ __forceinline__ float apply_act(float x) {
@@ -328,6 +361,12 @@ __global__ __launch_bounds__(256) void ttm_linear_reduce_k(LinearArgs p, int sli
     default: break;
     }
     v[r] = x;
+  }
+  if (p.group_n > 1) {   // one row tile (decode): tile nt of the concatenation belongs to one member
+    const GroupMember m = group_member(p, nt, 1);
+    uint8_t *Cm = m.C + ((int64_t)m.local * 1024 + in) * 2;
+    *(u32x2 *)Cm = finish_quad(p, Cm, v);
+    return;
   }
   uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
   *(u32x2 *)(C + off * 2) = finish_quad(p, C + off * 2, v);
@@ -1028,9 +1067,22 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   else linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wcol, nt_end, lane);
 }
 
+// group launch: the block's member becomes an ordinary single launch over that member's columns (p is rebound); the
+// XCD-aware renumbering is applied to the whole grid here, so the body is told not to repeat it (nblk = 1)
+__device__ __forceinline__ void linear_group_rebind(LinearArgs &p, int &bid, int &nblk, int &end) {
+  if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
+  const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
+  const GroupMember m = group_member(p, nb, p.ntw == 7 ? 7 : 2 * p.ntw);
+  p.W = m.W; p.C = m.C; p.Nt = m.Nt; p.group_n = 0;
+  bid = m.local * p.m_blocks + mb;
+  nblk = 1;
+  end = m.Nt;
+}
+
 template <int WF>
 __global__ __launch_bounds__(512) void ttm_linear_dma_k(LinearArgs p) {
   int bid = blockIdx.x, nblk = gridDim.x, first = 0, end = p.Nt, ntw = p.ntw;
+  if (p.group_n > 1) linear_group_rebind(p, bid, nblk, end);   // workgroup-uniform
   if (p.nt_split > 0) {   // workgroup-uniform
     if (bid < p.n_blocks1) { nblk = p.n_blocks1; end = p.nt_split; }
     else { bid -= p.n_blocks1; nblk -= p.n_blocks1; first = p.nt_split; ntw = p.ntw2; }
@@ -1043,6 +1095,7 @@ __global__ __launch_bounds__(512) void ttm_linear_dma_k(LinearArgs p) {
 template <int WF>
 __global__ __launch_bounds__(512) void ttm_linear_img_k(LinearArgs p) {
   int bid = blockIdx.x, nblk = gridDim.x, first = 0, end = p.Nt, ntw = p.ntw;
+  if (p.group_n > 1) linear_group_rebind(p, bid, nblk, end);   // workgroup-uniform
   if (p.nt_split > 0) {   // workgroup-uniform
     if (bid < p.n_blocks1) { nblk = p.n_blocks1; end = p.nt_split; }
     else { bid -= p.n_blocks1; nblk -= p.n_blocks1; first = p.nt_split; ntw = p.ntw2; }
@@ -1064,7 +1117,7 @@ __global__ __launch_bounds__(512) void ttm_linear_img_k(LinearArgs p) {
 // grid (ceil(Nt / 4), ceil(Kt / 2) + 1, weight sets), 256 lanes: half-wavefront h converts k-tile 2 ks + (h >> 2) of
 // column tile 4 x + (h & 3); a lane owns an 8 (k) x 4 (n) block as in the decode kernel.
 template <bool BFP4>
-__global__ __launch_bounds__(256) void ttm_linear_image_k(const uint8_t *W, int64_t w_batch, uint8_t *img, int64_t img_batch, int Nt, int Kt) {
+__device__ __forceinline__ void linear_image_body(const uint8_t *W, uint8_t *img, int Nt, int Kt) {
   constexpr uint32_t TB = BFP4 ? 576u : 1088u, FACE = BFP4 ? 128u : 256u, ROW = BFP4 ? 8u : 16u;
   const int tid = threadIdx.x, h = tid >> 5, wq = tid & 31;
   const int ks = blockIdx.y, nt = 4 * blockIdx.x + (h & 3), kt = 2 * ks + (h >> 2);
@@ -1074,7 +1127,7 @@ __global__ __launch_bounds__(256) void ttm_linear_image_k(const uint8_t *W, int6
 #pragma unroll
   for (int j = 0; j < 4; ++j) out[j] = u32x4{0, 0, 0, 0};
   if (kt < Kt) {
-    const uint8_t *t = W + (int64_t)blockIdx.z * w_batch + ((int64_t)kt * Nt + nt) * TB;
+    const uint8_t *t = W + ((int64_t)kt * Nt + nt) * TB;
     const u32x2 ex = *(const u32x2 *)(t + face * 16 + khalf * 8);
     const uint8_t *m = t + 64 + face * FACE + khalf * (FACE / 2) + quad * (ROW / 4);
     uint32_t rows[8];
@@ -1101,10 +1154,30 @@ __global__ __launch_bounds__(256) void ttm_linear_image_k(const uint8_t *W, int6
     for (int j = 0; j < 4; ++j)
       out[j] = u32x4{pack_hi(f[0][j], f[1][j]), pack_hi(f[2][j], f[3][j]), pack_hi(f[4][j], f[5][j]), pack_hi(f[6][j], f[7][j])};
   }
-  u32x4 *dst = (u32x4 *)(img + (int64_t)blockIdx.z * img_batch + ((int64_t)ks * Nt + nt) * 4096);
+  u32x4 *dst = (u32x4 *)(img + ((int64_t)ks * Nt + nt) * 4096);
   const int kc = (h >> 2) * 4 + (face >> 1) * 2 + khalf, n0 = (face & 1) * 16 + quad * 4;
 #pragma unroll
   for (int j = 0; j < 4; ++j) dst[lds_chunk(n0 + j, kc)] = out[j];
+}
+template <bool BFP4>
+__global__ __launch_bounds__(256) void ttm_linear_image_k(const uint8_t *W, int64_t w_batch, uint8_t *img, int64_t img_batch, int Nt, int Kt) {
+  linear_image_body<BFP4>(W + (int64_t)blockIdx.z * w_batch, img + (int64_t)blockIdx.z * img_batch, Nt, Kt);
+}
+// the members of a group launch: blockIdx.z picks the member, grid.x covers the widest one
+struct ImageGroup {
+  const uint8_t *W[4];
+  uint8_t *img[4];
+  int Nt[4];
+};
+template <bool BFP4>
+__global__ __launch_bounds__(256) void ttm_linear_image_group_k(ImageGroup g, int Kt) {
+  const uint8_t *W = g.W[0];
+  uint8_t *img = g.img[0];
+  int Nt = g.Nt[0];
+#pragma unroll
+  for (int j = 1; j < 4; ++j)
+    if ((int)blockIdx.z == j) { W = g.W[j]; img = g.img[j]; Nt = g.Nt[j]; }
+  linear_image_body<BFP4>(W, img, Nt, Kt);
 }
 
 // =============================================================================================
@@ -1261,13 +1334,17 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   constexpr uint32_t TB = BFP4 ? 576u : 1088u, FACE = BFP4 ? 128u : 256u, ROW = BFP4 ? 8u : 16u;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int cg = blockIdx.x;
+  int cg = blockIdx.x, Nt = p.Nt, tile_base = 0;   // column pair, column tiles of the matrix, its first tile in a group's concatenation
   const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
   const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
   uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
+  if (p.group_n > 1) {   // workgroup-uniform
+    const GroupMember m = group_member(p, cg, 2);
+    W = m.W; C = m.C; Nt = m.Nt; cg = m.local; tile_base = m.tile_base;
+  }
   const int q16 = lane & 15, kg = lane >> 4;   // weight operand row and 8-k group of this lane
   const int fc = (q16 >> 2) & 1, quad = q16 & 3, fr = kg >> 1, half = kg & 1;
-  const uint32_t nt_l = (uint32_t)min(2 * cg + (q16 >> 3), p.Nt - 1);
+  const uint32_t nt_l = (uint32_t)min(2 * cg + (q16 >> 3), Nt - 1);
   const uint32_t offW = nt_l * TB + 64u + (fr * 2 + fc) * FACE + half * (FACE / 2) + quad * (ROW / 4);   // + ROW i
   const uint32_t offE = nt_l * TB + (fr * 2 + fc) * 16 + half * 8;
   const uint32_t offA = fr * 512 + q16 * 32 + half * 16;                                     // + 1024 h
@@ -1289,7 +1366,7 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
     const int kt = kbase + wave + 8 * c;
     const int ktc = min(kt, kend - 1);
     const uint32_t keep = kt < kend ? 0xFFFFFFFFu : 0u;   // past the end: zero exponents, zero weights
-    const uint8_t *Wk = W + (int64_t)ktc * p.Nt * TB;
+    const uint8_t *Wk = W + (int64_t)ktc * Nt * TB;
     const uint8_t *Ak = A + (int64_t)ktc * 2048;
 #pragma unroll
     for (int i = 0; i < 8; ++i)   // the eight loads share their cache lines: cached loads
@@ -1357,12 +1434,12 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   for (int w = 1; w < 8; ++w) sum += part[w * 512 + tid];
   const int h = tid >> 8, i = (tid >> 6) & 3;
   const int nt = 2 * cg + (kg >> 1);
-  if (nt >= p.Nt) return;
+  if (nt >= Nt) return;
   const int n_in = 16 * (kg & 1) + 4 * i;
   const int64_t off = (int64_t)nt * 1024 + (h * 2 + (n_in >> 4)) * 256 + q16 * 16 + (n_in & 15);
   if (p.partial) {   // bias, activation and rounding happen in ttm_linear_reduce_k
-    const int64_t per = (int64_t)p.Nt * 1024;
-    *(f32x4v *)(p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * per + off) = sum;
+    const int64_t per = (int64_t)p.Nt * 1024;   // a group's partial sums are laid out as the concatenation
+    *(f32x4v *)(p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * per + (int64_t)tile_base * 1024 + off) = sum;
     return;
   }
   float bv[4] = {0.f, 0.f, 0.f, 0.f};
@@ -1403,6 +1480,14 @@ static int device_cu_count() {
 // (the 12 stand for prologue and epilogue), 0.92 / 0.78 of that at 6 / 4 tiles (a narrower block keeps the whole
 // activation traffic of a wide one); blocks run in rounds of one per CU; a split reduction adds its fp32 partial
 // traffic, (slices + 0.5) x M x N x 4 bytes, at 4 TB/s.  force_* != 0 pin a choice (tests, measurements).
+// column units of `unit_tiles` tiles in a launch: a group numbers its members' units one after another
+static int column_units(const LinearArgs &p, int unit_tiles) {
+  if (p.group_n <= 1) return (p.Nt + unit_tiles - 1) / unit_tiles;
+  int n = 0;
+  for (int j = 0; j < p.group_n; ++j) n += (p.gNt[j] + unit_tiles - 1) / unit_tiles;
+  return n;
+}
+
 static int plan_dma_grid(LinearArgs &p, int cus, int force_ntw, int force_slices, int two_part = 0) {
   const int mbk = p.m_blocks, ksteps = (p.Kt + 1) / 2;
   static const double width_cost[5] = {0, 0, 0.78, 0.92, 1.0};
@@ -1410,7 +1495,7 @@ static int plan_dma_grid(LinearArgs &p, int cus, int force_ntw, int force_slices
   int best_ntw = 4, best_slices = 1;
   for (int ntw = 4; ntw >= 2; --ntw) {
     if (force_ntw && ntw != force_ntw) continue;
-    const int blocks = mbk * ((p.Nt + 2 * ntw - 1) / (2 * ntw));
+    const int blocks = mbk * column_units(p, 2 * ntw);
     for (int slices = 1; slices <= 8; slices *= 2) {
       if (force_slices ? slices != 1 : (slices > 1 && ksteps / slices < 8)) continue;
       const int rounds = (blocks * slices + cus - 1) / cus;
@@ -1421,13 +1506,13 @@ static int plan_dma_grid(LinearArgs &p, int cus, int force_ntw, int force_slices
   }
   if (force_slices) best_slices = force_slices;
   p.ntw = best_ntw;
-  p.n_blocks = mbk * ((p.Nt + 2 * best_ntw - 1) / (2 * best_ntw));   // blocks per k-slice
+  p.n_blocks = mbk * column_units(p, 2 * best_ntw);   // blocks per k-slice
   p.nt_split = 0;
   // Optional (linear_two_part = 1): unsplit, full-width grids whose last round is partly filled keep the full rounds at
   // 8 tiles and cover the remaining columns with narrower blocks when the model says those cost fewer CU-rounds.
   // [2048, 4096] x [4096, 14336]: 256 blocks of 8 tiles + 256 blocks of 6 tiles instead of 448 of 8 - modelled 1.92
   // rounds instead of 2, measured 262 us instead of 250, so it is off unless asked for.
-  if (best_slices == 1 && best_ntw == 4 && !force_ntw && two_part != 0) {
+  if (best_slices == 1 && best_ntw == 4 && !force_ntw && two_part != 0 && p.group_n <= 1) {
     const int full_rounds = p.n_blocks / cus;
     const int cols1 = full_rounds * cus / mbk;            // column blocks (8 tiles) the full rounds cover
     const int rem = p.Nt - 8 * cols1;                      // column tiles left
@@ -1465,13 +1550,14 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
     // the small kernel handles one row tile per launch
     LinearArgs p = a;
     const bool decode = BFP && ttm_option("linear_variant") != 1 && (int64_t)a.Nt * 1088 < (int64_t)1 << 32;
+    if (a.group_n > 1 && !decode) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear_group: the selected kernel variant has no group form");
     // the decode kernel has one workgroup per 64 columns: narrow outputs split K until there is one workgroup per CU,
     // as long as a slice keeps 32 k-tiles (four per wavefront, the depth of its load ring); the slices leave fp32
     // partial sums that ttm_linear_reduce_k finishes.  Measured at M = 32: [4096, 4096] 14.3 -> 10.6 us,
     // [14336, 4096] 38 -> 19 us with 4 slices; 8 slices or splitting a [4096, 14336] weight are slower than not splitting.
     int slices = 1;
     if (decode) {
-      const int64_t groups = (int64_t)((a.Nt + 1) / 2) * batch;
+      const int64_t groups = (int64_t)column_units(a, 2) * batch;
       slices = ttm_option("linear_decode_split");
       if (slices <= 0) {
         slices = (int)(device_cu_count() / groups);
@@ -1494,7 +1580,8 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
     for (int mt = 0; mt < a.Mt; ++mt) {
       p.A = a.A + (int64_t)mt * a.Kt * 2048;
       p.C = a.C + (int64_t)mt * a.Nt * 2048;
-      const dim3 grid((a.Nt + 1) / 2, slices, (unsigned)batch);
+      for (int j = 0; j < a.group_n; ++j) p.gC[j] = a.gC[j] + (int64_t)mt * a.gNt[j] * 2048;
+      const dim3 grid(column_units(a, 2), slices, (unsigned)batch);
       if (decode && WF == WF_BFP4) hipLaunchKernelGGL(ttm_linear_decode_k<true>, grid, dim3(512), 65536, s, p);
       else if (decode) hipLaunchKernelGGL(ttm_linear_decode_k<false>, grid, dim3(512), 65536, s, p);
       else hipLaunchKernelGGL((ttm_linear_small_k<WF>), dim3(a.Nt, 1, (unsigned)batch), dim3(256), 0, s, p);
@@ -1510,6 +1597,7 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
   if (variant == 0) variant = !fits32 ? 1 : (BFP ? 6 : 5);
   if ((variant == 5 || variant == 6) && !fits32) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear: operand too large for the selected kernel variant");
   if (variant == 6 && !BFP) variant = 5;
+  if (a.group_n > 1 && variant != 6) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear_group: the selected kernel variant has no group form");
   const int lds_bytes = 2 * 4096 * 16;
   if constexpr (BFP) {
     if (variant == 6) {
@@ -1522,7 +1610,8 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       LinearArgs p = a;
       const int cus = device_cu_count();
       const int force_ntw = ttm_option("linear_ntw") == 7 ? 0 : ttm_option("linear_ntw");   // 7 exists in the second pass only
-      int slices = plan_dma_grid(p, cus, force_ntw, ttm_option("linear_split_k"), ttm_option("linear_two_part") == 1);
+      // a group is not split along K: its partial sums would need a reduction that knows the members
+      int slices = plan_dma_grid(p, cus, force_ntw, a.group_n > 1 ? 1 : ttm_option("linear_split_k"), ttm_option("linear_two_part") == 1);
       slices = slices < 1 ? 1 : (slices > a.Kt ? a.Kt : slices);
       if (slices > 1) {
         p.k_slice = (a.Kt + slices - 1) / slices;
@@ -1539,7 +1628,7 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       // linear_two_pass: 0 = by the model, 1 = never, 2 = always.
       const int ksteps = (a.Kt + 1) / 2;
       const int64_t sets = a.w_batch == 0 ? 1 : batch;
-      const int64_t img_set = (int64_t)(ksteps + 1) * a.Nt * 4096;
+      const int64_t img_set = (int64_t)(ksteps + 1) * a.Nt * 4096;   // a group: the members' image sets back to back
       bool two_pass = ttm_option("linear_two_pass") == 2;
       if (ttm_option("linear_two_pass") == 0) {
         static const double width_cost[5] = {0, 0, 0.78, 0.92, 1.0};
@@ -1559,7 +1648,7 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         // without the conversion a block may be seven tiles wide (the wavefronts of a SIMD take 4 + 3): worth it when
         // that fills the last round, e.g. 8 x 448 tiles = 448 blocks of 8 (1.75 rounds on 256 CUs, paid as 2) against 512
         // blocks of 7 (2 rounds at 7/8 of the work each).  linear_ntw = 7 forces it.
-        const int64_t blocks7 = (int64_t)p.m_blocks * ((a.Nt + 6) / 7);
+        const int64_t blocks7 = (int64_t)p.m_blocks * column_units(a, 7);
         const int64_t rounds8 = ((int64_t)p.n_blocks * batch + cus - 1) / cus, rounds7 = (blocks7 * batch + cus - 1) / cus;
         static const double width_cost8[5] = {0, 0, 0.78, 0.92, 1.0};
         const bool pick7 = ttm_option("linear_ntw") == 7 || (ttm_option("linear_ntw") == 0 && rounds7 * 0.92 < rounds8 * width_cost8[p.ntw] * 0.98);
@@ -1571,8 +1660,22 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
           if (int rc = set_lds_limit(ttm_linear_img_k<WF>, 131072)) return rc;
           attr2 = true;
         }
-        hipLaunchKernelGGL((ttm_linear_image_k<WF == WF_BFP4>), dim3((a.Nt + 3) / 4, ksteps + 1, (unsigned)sets), dim3(256), 0, s, a.W, a.w_batch,
-                           ws, img_set, a.Nt, a.Kt);
+        if (a.group_n > 1) {
+          ImageGroup g = {};
+          int widest = 0;
+          uint8_t *at = ws;
+          for (int j = 0; j < a.group_n; ++j) {
+            g.W[j] = a.gW[j]; g.img[j] = at; g.Nt[j] = a.gNt[j];
+            p.gW[j] = at;                                   // the second pass reads the images
+            at += (int64_t)(ksteps + 1) * a.gNt[j] * 4096;
+            widest = a.gNt[j] > widest ? a.gNt[j] : widest;
+          }
+          hipLaunchKernelGGL((ttm_linear_image_group_k<WF == WF_BFP4>), dim3((widest + 3) / 4, ksteps + 1, (unsigned)a.group_n), dim3(256), 0, s,
+                             g, a.Kt);
+        } else {
+          hipLaunchKernelGGL((ttm_linear_image_k<WF == WF_BFP4>), dim3((a.Nt + 3) / 4, ksteps + 1, (unsigned)sets), dim3(256), 0, s, a.W,
+                             a.w_batch, ws, img_set, a.Nt, a.Kt);
+        }
         p.W = ws;
         p.w_batch = a.w_batch == 0 ? 0 : img_set;
         p.img_zero_step = ksteps;
@@ -1647,6 +1750,8 @@ static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, 
   p.k_slice = p.Kt; p.partial = nullptr;
   p.nt_split = p.n_blocks1 = p.ntw2 = 0;
   p.img_zero_step = 0;
+  p.group_n = 0;
+  for (int j = 0; j < 4; ++j) { p.gW[j] = nullptr; p.gC[j] = nullptr; p.gNt[j] = 0; }
   p.tail = tail_op;
   p.tail_delta = tail ? (const uint8_t *)tail - (const uint8_t *)out : 0;
   if (strides) { p.a_batch = strides[0]; p.w_batch = strides[1]; p.c_batch = strides[2]; }
@@ -1676,4 +1781,43 @@ TTM_EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, in
   const int64_t strides[3] = {0, (const uint8_t *)w1 - (const uint8_t *)w0, (uint8_t *)out1 - (uint8_t *)out0};
   return linear_entry(a, TTM_BF16, w0, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, out0, TTM_BF16, 2, 2, M, N, K, TTM_ACT_NONE,
                       TTM_TAIL_NONE, nullptr, strides, stream);
+}
+
+TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N, int64_t M,
+                                int64_t K, void *stream) {
+  TTM_REQUIRE(n >= 1 && n <= 4, "ttm_linear_group: 1 to 4 members (got %d)", n);
+  TTM_REQUIRE(a && w && out && N, "ttm_linear_group: null pointer");
+  TTM_REQUIRE(w_dtype == TTM_BFP8B || w_dtype == TTM_BFP4B, "ttm_linear_group: weights must be BFP_BFloat8 or BFP_BFloat4 (got %d)", w_dtype);
+  TTM_REQUIRE(M >= 0 && K > 0, "ttm_linear_group: bad dimension");
+  for (int j = 0; j < n; ++j) {
+    TTM_REQUIRE(w[j] && out[j] && N[j] > 0, "ttm_linear_group: member %d has a null pointer or no columns", j);
+    TTM_REQUIRE((((uintptr_t)w[j] | (uintptr_t)out[j]) & 15) == 0, "ttm_linear_group: operands must be 16-byte aligned");
+    for (int i = 0; i < j; ++i) TTM_REQUIRE(out[i] != out[j], "ttm_linear_group: members %d and %d share an output", i, j);
+  }
+  if (n == 1) return ttm_linear(a, TTM_BF16, w[0], w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, out[0], TTM_BF16, 1, 1, M, N[0], K, TTM_ACT_NONE, stream);
+  if (M == 0) return TTM_OK;
+  TTM_REQUIRE(((uintptr_t)a & 15) == 0, "ttm_linear_group: operands must be 16-byte aligned");
+  LinearArgs p;
+  p.A = (const uint8_t *)a; p.W = (const uint8_t *)w[0]; p.bias = nullptr; p.C = (uint8_t *)out[0];
+  p.Mt = (int)ttm_cdiv(M, 32); p.Kt = (int)ttm_cdiv(K, 32); p.Nt = 0;
+  p.group_n = n;
+  for (int j = 0; j < 4; ++j) {
+    p.gW[j] = j < n ? (const uint8_t *)w[j] : nullptr;
+    p.gC[j] = j < n ? (uint8_t *)out[j] : nullptr;
+    p.gNt[j] = j < n ? (int)ttm_cdiv(N[j], 32) : 0;
+    p.Nt += p.gNt[j];
+  }
+  p.act = TTM_ACT_NONE; p.bias_tiled = 1;
+  p.a_batch = p.w_batch = p.c_batch = 0;
+  p.m_blocks = (p.Mt + 7) / 8; p.n_blocks = (p.Nt + 7) / 8;
+  p.ntw = 4;
+  p.k_slice = p.Kt; p.partial = nullptr;
+  p.nt_split = p.n_blocks1 = p.ntw2 = 0;
+  p.img_zero_step = 0;
+  p.tail = TTM_TAIL_NONE; p.tail_delta = 0;
+  hipStream_t s = (hipStream_t)stream;
+  const int rc = w_dtype == TTM_BFP8B ? launch_linear<WF_BFP8>(p, 1, s) : launch_linear<WF_BFP4>(p, 1, s);
+  if (rc) return rc;
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
 }

@@ -352,12 +352,15 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
       }
     }
   }
-  // A second matmul of the same activations with a weight tensor of the same shape and format (the K and V projections)
-  // a few ops further on runs in this launch; only reshapes, permutes, rotary embeddings and deallocations of other tensors
-  // may lie between.
+  // Further matmuls of the same activations with block-float weights of the same format a few ops further on (the Q, K and
+  // V projections) run in this launch; only reshapes, permutes, rotary embeddings and deallocations of other tensors may
+  // lie between, and a follower that has an add / multiply of its own to fuse is left alone.
   if (ctx.fuseViews && tailOp == TTM_TAIL_NONE && !biasRef && activation.empty() && !transposeA && !transposeB && batch == 1 &&
       utils::isBlockFormatDataType(b.handle->dtype) && layoutFromTensorRef(outRef) == Layout{StorageType::Device, TensorLayout::Tile, DataType::BFloat16}) {
-    for (std::uint32_t j = ctx.opIndex + 1; j < ctx.ops.size() && j <= ctx.opIndex + 6; ++j) {
+    struct Follower { std::uint32_t index; fb::Table out; Tensor weight; std::int64_t n; };
+    std::vector<Follower> followers;
+    const std::vector<std::uint32_t> outShape = shapeFromTensorRef(outRef);
+    for (std::uint32_t j = ctx.opIndex + 1; j < ctx.ops.size() && j <= ctx.opIndex + 10 && followers.size() < 3; ++j) {
       const OpType t = opType(j);
       fb::Table nop = ctx.ops[j].table(schema::Operation::f_type);
       if (t == OpType::ReshapeOp || t == OpType::PermuteOp || t == OpType::RotaryEmbeddingOp) continue;   // touch neither operand
@@ -374,18 +377,46 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
         break;
       auto wit = ctx.pool.find(refId(b2));
       if (wit == ctx.pool.end() || !isTensorAllocated(wit->second) || wit->second.handle->storage != StorageType::Device ||
-          wit->second.handle->dtype != b.handle->dtype || wit->second.handle->shape != b.handle->shape ||
-          wit->second.handle->data.get() == b.handle->data.get() || !(layoutFromTensorRef(out2) == layoutFromTensorRef(outRef)) ||
-          shapeFromTensorRef(out2) != shapeFromTensorRef(outRef))
+          wit->second.handle->dtype != b.handle->dtype || wit->second.handle->shape.size() != 2 || b.handle->shape.size() != 2 ||
+          wit->second.handle->shape[0] != b.handle->shape[0] || !(layoutFromTensorRef(out2) == layoutFromTensorRef(outRef)))
         break;
-      // the second matmul must not be followed by a fusable tail of its own: it keeps its plain form here
-      Tensor outB = makeOut(ctx, out2, DataType::BFloat16, TensorLayout::Tile);
-      TTM_CALL(ttm_linear_pair(a.handle->data.get(), b.handle->data.get(), wit->second.handle->data.get(), ttmDtype(b.handle->dtype),
-                               out.handle->data.get(), outB.handle->data.get(), M, N, K, ctx.stream()));
+      const std::vector<std::uint32_t> shape2 = shapeFromTensorRef(out2);
+      if (shape2.size() != outShape.size() || shape2.empty() || !std::equal(shape2.begin(), shape2.end() - 1, outShape.begin()) ||
+          shape2.back() != wit->second.handle->shape[1])
+        break;
+      // its own element-wise tail, if it has one, is worth more than the shared launch
+      std::uint32_t after = j + 1;
+      while (after < ctx.ops.size() && opType(after) == OpType::DeallocateOp) ++after;
+      if (after < ctx.ops.size() && opType(after) == OpType::EltwiseBinaryOp) {
+        fb::Table bop = ctx.ops[after].table(schema::Operation::f_type);
+        fb::Table l = bop.table(schema::EltwiseBinaryOp::f_lhs), r = bop.table(schema::EltwiseBinaryOp::f_rhs);
+        if ((l && refId(l) == refId(out2)) || (r && refId(r) == refId(out2))) break;
+      }
+      bool distinct = wit->second.handle->data.get() != b.handle->data.get();
+      for (const Follower &f : followers) distinct = distinct && f.weight.handle->data.get() != wit->second.handle->data.get();
+      if (!distinct) break;
+      followers.push_back(Follower{j, out2, wit->second, static_cast<std::int64_t>(shape2.back())});
+    }
+    if (!followers.empty()) {
+      std::vector<const void *> ws{b.handle->data.get()};
+      std::vector<void *> outs{out.handle->data.get()};
+      std::vector<std::int64_t> ns{N};
+      std::vector<Tensor> outTensors;
+      for (const Follower &f : followers) {
+        outTensors.push_back(makeOut(ctx, f.out, DataType::BFloat16, TensorLayout::Tile));
+        ws.push_back(f.weight.handle->data.get());
+        outs.push_back(outTensors.back().handle->data.get());
+        ns.push_back(f.n);
+      }
+      TTM_CALL(ttm_linear_group(a.handle->data.get(), static_cast<int>(ws.size()), ws.data(), ttmDtype(b.handle->dtype), outs.data(), ns.data(), M, K,
+                                ctx.stream()));
       ctx.put(outRef, out);
-      ctx.put(out2, outB);
-      ctx.skip.insert(j);
-      debug::Stats::get().incrementStat("PairedMatmul");
+      for (size_t i = 0; i < followers.size(); ++i) {
+        ctx.put(followers[i].out, outTensors[i]);
+        ctx.skip.insert(followers[i].index);
+      }
+      debug::Stats::get().incrementStat("GroupedMatmul");
+      debug::Stats::get().incrementStat("GroupedMatmulMembers", static_cast<std::int64_t>(ws.size()));
       return;
     }
   }
