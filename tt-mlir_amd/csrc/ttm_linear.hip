@@ -1117,10 +1117,10 @@ __global__ __launch_bounds__(512) void ttm_linear_img_k(LinearArgs p) {
 // grid (ceil(Nt / 4), ceil(Kt / 2) + 1, weight sets), 256 lanes: half-wavefront h converts k-tile 2 ks + (h >> 2) of
 // column tile 4 x + (h & 3); a lane owns an 8 (k) x 4 (n) block as in the decode kernel.
 template <bool BFP4>
-__device__ __forceinline__ void linear_image_body(const uint8_t *W, uint8_t *img, int Nt, int Kt) {
+__device__ __forceinline__ void linear_image_body(const uint8_t *W, uint8_t *img, int Nt, int Kt, int xg) {
   constexpr uint32_t TB = BFP4 ? 576u : 1088u, FACE = BFP4 ? 128u : 256u, ROW = BFP4 ? 8u : 16u;
   const int tid = threadIdx.x, h = tid >> 5, wq = tid & 31;
-  const int ks = blockIdx.y, nt = 4 * blockIdx.x + (h & 3), kt = 2 * ks + (h >> 2);
+  const int ks = blockIdx.y, nt = 4 * xg + (h & 3), kt = 2 * ks + (h >> 2);   // xg: group of four column tiles
   if (nt >= Nt) return;
   const int face = wq >> 3, khalf = (wq >> 2) & 1, quad = wq & 3;
   u32x4 out[4];
@@ -1161,23 +1161,33 @@ __device__ __forceinline__ void linear_image_body(const uint8_t *W, uint8_t *img
 }
 template <bool BFP4>
 __global__ __launch_bounds__(256) void ttm_linear_image_k(const uint8_t *W, int64_t w_batch, uint8_t *img, int64_t img_batch, int Nt, int Kt) {
-  linear_image_body<BFP4>(W + (int64_t)blockIdx.z * w_batch, img + (int64_t)blockIdx.z * img_batch, Nt, Kt);
+  linear_image_body<BFP4>(W + (int64_t)blockIdx.z * w_batch, img + (int64_t)blockIdx.z * img_batch, Nt, Kt, blockIdx.x);
 }
-// the members of a group launch: blockIdx.z picks the member, grid.x covers the widest one
+// the members of a group launch: grid.x numbers the members' groups of four column tiles one after another
 struct ImageGroup {
   const uint8_t *W[4];
   uint8_t *img[4];
   int Nt[4];
+  int n;
 };
 template <bool BFP4>
 __global__ __launch_bounds__(256) void ttm_linear_image_group_k(ImageGroup g, int Kt) {
   const uint8_t *W = g.W[0];
   uint8_t *img = g.img[0];
-  int Nt = g.Nt[0];
+  int Nt = g.Nt[0], xg = blockIdx.x, start = 0;
+  bool found = false;
 #pragma unroll
-  for (int j = 1; j < 4; ++j)
-    if ((int)blockIdx.z == j) { W = g.W[j]; img = g.img[j]; Nt = g.Nt[j]; }
-  linear_image_body<BFP4>(W, img, Nt, Kt);
+  for (int j = 0; j < 4; ++j) {
+    if (j < g.n) {
+      const int cnt = (g.Nt[j] + 3) / 4;
+      if (!found && ((int)blockIdx.x < start + cnt || j == g.n - 1)) {
+        found = true;
+        W = g.W[j]; img = g.img[j]; Nt = g.Nt[j]; xg = blockIdx.x - start;
+      }
+      start += cnt;
+    }
+  }
+  linear_image_body<BFP4>(W, img, Nt, Kt, xg);
 }
 
 // =============================================================================================
@@ -1662,16 +1672,14 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         }
         if (a.group_n > 1) {
           ImageGroup g = {};
-          int widest = 0;
+          g.n = a.group_n;
           uint8_t *at = ws;
           for (int j = 0; j < a.group_n; ++j) {
             g.W[j] = a.gW[j]; g.img[j] = at; g.Nt[j] = a.gNt[j];
             p.gW[j] = at;                                   // the second pass reads the images
             at += (int64_t)(ksteps + 1) * a.gNt[j] * 4096;
-            widest = a.gNt[j] > widest ? a.gNt[j] : widest;
           }
-          hipLaunchKernelGGL((ttm_linear_image_group_k<WF == WF_BFP4>), dim3((widest + 3) / 4, ksteps + 1, (unsigned)a.group_n), dim3(256), 0, s,
-                             g, a.Kt);
+          hipLaunchKernelGGL((ttm_linear_image_group_k<WF == WF_BFP4>), dim3(column_units(a, 4), ksteps + 1, 1), dim3(256), 0, s, g, a.Kt);
         } else {
           hipLaunchKernelGGL((ttm_linear_image_k<WF == WF_BFP4>), dim3((a.Nt + 3) / 4, ksteps + 1, (unsigned)sets), dim3(256), 0, s, a.W,
                              a.w_batch, ws, img_set, a.Nt, a.Kt);
