@@ -128,10 +128,12 @@ int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int 
  * (the K and V projections of an attention layer); the two weight tensors and the two outputs may live anywhere.  No bias,
  * activation or tail.  One launch fills the device where two small ones would each leave part of it idle. */
 /* Up to four block-float weight matrices [K, N_i] (one dtype, any widths) applied to the same activations in one launch,
- * each with its own output [M, N_i]: the Q, K and V projections of an attention layer.  No bias, activation or tail.
- * Results are those of separate ttm_linear calls up to the accumulation order the launch plan implies. */
-int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N, int64_t M,
-                     int64_t K, void *stream);
+ * each with its own output [M, N_i] and its own activation (act[i], TTM_ACT_*; NULL = none): the Q, K and V projections
+ * of an attention layer, or the gate and up projections of an MLP at token counts where one of them alone would not
+ * fill the device.  No bias or tail.  Results are those of separate ttm_linear calls up to the accumulation order the
+ * launch plan implies. */
+int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N,
+                     const int *act, int64_t M, int64_t K, void *stream);
 int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M, int64_t N,
                     int64_t K, void *stream);
 

@@ -419,7 +419,8 @@ def test_linear_group_equals_separate_launches(hip, dev, wfmt_name, M, K, Ns, op
     for k, v in options.items():
         hip.set_option(k, v)
     try:
-        want = [run_linear(hip, dev, a, w, None, None, wfmt)[0] for w in ws]
+        act_names = [(None, "silu", "gelu", "relu")[(i + M) % 4] for i in range(len(Ns))]     # a different activation per member
+        want = [run_linear(hip, dev, a, w, None, act, wfmt)[0] for w, act in zip(ws, act_names)]
         at = tilize_dev(hip, a, dev)
         wt = [pack_weight(hip, w, wfmt, dev) for w in ws]
         Mp = (M + 31) // 32 * 32
@@ -428,7 +429,8 @@ def test_linear_group_equals_separate_launches(hip, dev, wfmt_name, M, K, Ns, op
         wp = (ctypes.c_void_p * n)(*[t.data_ptr() for t in wt])
         op = (ctypes.c_void_p * n)(*[t.data_ptr() for t in outs])
         nn = (ctypes.c_int64 * n)(*Ns)
-        hip.call("ttm_linear_group", hip.ptr(at), n, wp, wfmt, op, nn, M, K, hip.current_stream())
+        acts = (ctypes.c_int * n)(*[hip.ACT[x] for x in act_names])
+        hip.call("ttm_linear_group", hip.ptr(at), n, wp, wfmt, op, nn, acts, M, K, hip.current_stream())
         got = [untilize_dev(hip, o, (M, N), dev).cpu() for o, N in zip(outs, Ns)]
         torch.cuda.synchronize()
     finally:

@@ -607,16 +607,20 @@ def test_update_cache_reads_a_permuted_view(device, dtype, index, offset):
         assert torch.equal(got[mode], want), mode
 
 
-def test_fused_epilogue_tails_do_not_change_program_results(device):
-    """Without callbacks the executor folds `x + matmul(...)` and `silu(gate) * matmul(...)` into the matmul's epilogue; with a
-    callback registered every op runs on its own.  Both runs of the decoder layer must agree bit for bit."""
-    d = datagen.c5_decoder(seq=96, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, seed=8)
-    binary = rt.Binary.load_from_memory(programs.c5_decoder(seq=96, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512))
+@pytest.mark.parametrize("seq", [64, 96])
+def test_fused_epilogue_tails_do_not_change_program_results(device, seq):
+    """Without callbacks the executor folds `x + matmul(...)` and `silu(gate) * matmul(...)` into the matmul's epilogue and
+    groups projections of the same activations; with a callback registered every op runs on its own.  Both runs of the
+    decoder layer must agree bit for bit.  At 64 tokens the gate * up product is an epilogue tail; at 96 (a count where a
+    projection alone would not fill the device) gate and up share a launch instead and the product runs by itself."""
+    d = datagen.c5_decoder(seq=seq, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, seed=8)
+    binary = rt.Binary.load_from_memory(programs.c5_decoder(seq=seq, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512))
     tins = [d["x"], d["attn_norm_w"], bf(d["wq"]), bf(d["wk"]), bf(d["wv"]), bf(d["wo"]), d["mlp_norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
     rt.clear_stats()
     (fused,) = harness.execute(binary, 1, tins, device)
-    assert rt.get_stat("FusedLinearTail") == 3          # attention residual, gate * up, MLP residual
-    assert rt.get_stat("GroupedMatmul") == 1 and rt.get_stat("GroupedMatmulMembers") == 3   # Q, K and V projections in one launch
+    tails, groups, members = {64: (3, 1, 3), 96: (2, 2, 5)}[seq]
+    assert rt.get_stat("FusedLinearTail") == tails      # attention residual, MLP residual, and gate * up at 64 tokens
+    assert rt.get_stat("GroupedMatmul") == groups and rt.get_stat("GroupedMatmulMembers") == members   # Q, K, V; gate, up
     assert rt.get_stat("SdpaHeadsInner") == 1           # attention reads the projections and writes the merged heads in place
     assert rt.get_stat("CopyViewLaunch") == 0           # no head split or merge is materialised
     seen = []
@@ -625,7 +629,7 @@ def test_fused_epilogue_tails_do_not_change_program_results(device):
         (plain,) = harness.execute(binary, 1, tins, device)
     finally:
         rt.clear_callbacks()
-    assert seen.count("EltwiseBinaryOp") == 3 and rt.get_stat("FusedLinearTail") == 3
+    assert seen.count("EltwiseBinaryOp") == 3 and rt.get_stat("FusedLinearTail") == tails
     assert torch.equal(fused, plain)
 
 

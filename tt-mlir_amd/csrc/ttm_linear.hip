@@ -48,11 +48,12 @@ struct LinearArgs {
   int img_zero_step;                  // two-pass launch: W points at the dequantised images, this step index holds zeros
   // group launch (group_n >= 2): several weight matrices [K, N_i] applied to the same activations, each with its own
   // output; W / C / Nt above describe the virtual concatenation (Nt = sum of the members' column tiles) and are not
-  // dereferenced.  No bias, activation, tail or batch in a group.
+  // dereferenced.  Each member may have its own activation; no bias, tail or batch in a group.
   int group_n;
   const uint8_t *gW[4];
   uint8_t *gC[4];
   int gNt[4];
+  int gAct[4];                        // per-member activation
   int tail;                           // 0 none, 1 add, 2 multiply: element-wise tail with a tensor laid out like the output
   int64_t tail_delta;                 // byte distance from an output element to its tail operand
 };
@@ -63,10 +64,10 @@ struct LinearArgs {
 struct GroupMember {
   const uint8_t *W;
   uint8_t *C;
-  int Nt, local, tile_base;   // column tiles, unit index inside the member, first column tile in the concatenation
+  int Nt, local, tile_base, act;   // column tiles, unit index inside the member, first column tile in the concatenation
 };
 __device__ __forceinline__ GroupMember group_member(const LinearArgs &p, int u, int unit_tiles) {
-  GroupMember m = {p.gW[0], p.gC[0], p.gNt[0], u, 0};
+  GroupMember m = {p.gW[0], p.gC[0], p.gNt[0], u, 0, p.gAct[0]};
   int start = 0, tiles = 0;
   bool found = false;
 #pragma unroll
@@ -75,7 +76,7 @@ __device__ __forceinline__ GroupMember group_member(const LinearArgs &p, int u, 
       const int n = (p.gNt[j] + unit_tiles - 1) / unit_tiles;
       if (!found && (u < start + n || j == p.group_n - 1)) {
         found = true;
-        m.W = p.gW[j]; m.C = p.gC[j]; m.Nt = p.gNt[j]; m.local = u - start; m.tile_base = tiles;
+        m.W = p.gW[j]; m.C = p.gC[j]; m.Nt = p.gNt[j]; m.local = u - start; m.tile_base = tiles; m.act = p.gAct[j];
       }
       start += n; tiles += p.gNt[j];
     }
@@ -349,11 +350,17 @@ __global__ __launch_bounds__(256) void ttm_linear_reduce_k(LinearArgs p, int sli
     bv[0] = __uint_as_float(raw.x << 16); bv[1] = __uint_as_float(raw.x & 0xFFFF0000u);
     bv[2] = __uint_as_float(raw.y << 16); bv[3] = __uint_as_float(raw.y & 0xFFFF0000u);
   }
+  GroupMember m = {};
+  int act = p.act;
+  if (p.group_n > 1) {   // one row tile (decode): tile nt of the concatenation belongs to one member
+    m = group_member(p, nt, 1);
+    act = m.act;
+  }
   float v[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     float x = sum[r] + bv[r];
-    switch (p.act) {
+    switch (act) {
     case TTM_ACT_GELU: x = apply_act<TTM_ACT_GELU>(x); break;
     case TTM_ACT_SILU: x = apply_act<TTM_ACT_SILU>(x); break;
     case TTM_ACT_SIGMOID: x = apply_act<TTM_ACT_SIGMOID>(x); break;
@@ -362,8 +369,7 @@ __global__ __launch_bounds__(256) void ttm_linear_reduce_k(LinearArgs p, int sli
     }
     v[r] = x;
   }
-  if (p.group_n > 1) {   // one row tile (decode): tile nt of the concatenation belongs to one member
-    const GroupMember m = group_member(p, nt, 1);
+  if (p.group_n > 1) {
     uint8_t *Cm = m.C + ((int64_t)m.local * 1024 + in) * 2;
     *(u32x2 *)Cm = finish_quad(p, Cm, v);
     return;
@@ -1073,7 +1079,7 @@ __device__ __forceinline__ void linear_group_rebind(LinearArgs &p, int &bid, int
   if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);
   const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
   const GroupMember m = group_member(p, nb, p.ntw == 7 ? 7 : 2 * p.ntw);
-  p.W = m.W; p.C = m.C; p.Nt = m.Nt; p.group_n = 0;
+  p.W = m.W; p.C = m.C; p.Nt = m.Nt; p.act = m.act; p.group_n = 0;
   bid = m.local * p.m_blocks + mb;
   nblk = 1;
   end = m.Nt;
@@ -1344,13 +1350,13 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   constexpr uint32_t TB = BFP4 ? 576u : 1088u, FACE = BFP4 ? 128u : 256u, ROW = BFP4 ? 8u : 16u;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  int cg = blockIdx.x, Nt = p.Nt, tile_base = 0;   // column pair, column tiles of the matrix, its first tile in a group's concatenation
+  int cg = blockIdx.x, Nt = p.Nt, tile_base = 0, act = p.act;   // column pair, column tiles of the matrix, its first tile in a group's concatenation
   const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
   const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
   uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
   if (p.group_n > 1) {   // workgroup-uniform
     const GroupMember m = group_member(p, cg, 2);
-    W = m.W; C = m.C; Nt = m.Nt; cg = m.local; tile_base = m.tile_base;
+    W = m.W; C = m.C; Nt = m.Nt; cg = m.local; tile_base = m.tile_base; act = m.act;
   }
   const int q16 = lane & 15, kg = lane >> 4;   // weight operand row and 8-k group of this lane
   const int fc = (q16 >> 2) & 1, quad = q16 & 3, fr = kg >> 1, half = kg & 1;
@@ -1463,7 +1469,7 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     float x = sum[r] + bv[r];
-    switch (p.act) {
+    switch (act) {
     case TTM_ACT_GELU: x = apply_act<TTM_ACT_GELU>(x); break;
     case TTM_ACT_SILU: x = apply_act<TTM_ACT_SILU>(x); break;
     case TTM_ACT_SIGMOID: x = apply_act<TTM_ACT_SIGMOID>(x); break;
@@ -1759,7 +1765,7 @@ static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, 
   p.nt_split = p.n_blocks1 = p.ntw2 = 0;
   p.img_zero_step = 0;
   p.group_n = 0;
-  for (int j = 0; j < 4; ++j) { p.gW[j] = nullptr; p.gC[j] = nullptr; p.gNt[j] = 0; }
+  for (int j = 0; j < 4; ++j) { p.gW[j] = nullptr; p.gC[j] = nullptr; p.gNt[j] = 0; p.gAct[j] = TTM_ACT_NONE; }
   p.tail = tail_op;
   p.tail_delta = tail ? (const uint8_t *)tail - (const uint8_t *)out : 0;
   if (strides) { p.a_batch = strides[0]; p.w_batch = strides[1]; p.c_batch = strides[2]; }
@@ -1791,8 +1797,8 @@ TTM_EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, in
                       TTM_TAIL_NONE, nullptr, strides, stream);
 }
 
-TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N, int64_t M,
-                                int64_t K, void *stream) {
+TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N,
+                                const int *act, int64_t M, int64_t K, void *stream) {
   TTM_REQUIRE(n >= 1 && n <= 4, "ttm_linear_group: 1 to 4 members (got %d)", n);
   TTM_REQUIRE(a && w && out && N, "ttm_linear_group: null pointer");
   TTM_REQUIRE(w_dtype == TTM_BFP8B || w_dtype == TTM_BFP4B, "ttm_linear_group: weights must be BFP_BFloat8 or BFP_BFloat4 (got %d)", w_dtype);
@@ -1801,8 +1807,10 @@ TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int 
     TTM_REQUIRE(w[j] && out[j] && N[j] > 0, "ttm_linear_group: member %d has a null pointer or no columns", j);
     TTM_REQUIRE((((uintptr_t)w[j] | (uintptr_t)out[j]) & 15) == 0, "ttm_linear_group: operands must be 16-byte aligned");
     for (int i = 0; i < j; ++i) TTM_REQUIRE(out[i] != out[j], "ttm_linear_group: members %d and %d share an output", i, j);
+    TTM_REQUIRE(!act || (act[j] >= TTM_ACT_NONE && act[j] <= TTM_ACT_RELU), "ttm_linear_group: unknown activation %d", act ? act[j] : 0);
   }
-  if (n == 1) return ttm_linear(a, TTM_BF16, w[0], w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, out[0], TTM_BF16, 1, 1, M, N[0], K, TTM_ACT_NONE, stream);
+  if (n == 1)
+    return ttm_linear(a, TTM_BF16, w[0], w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, out[0], TTM_BF16, 1, 1, M, N[0], K, act ? act[0] : TTM_ACT_NONE, stream);
   if (M == 0) return TTM_OK;
   TTM_REQUIRE(((uintptr_t)a & 15) == 0, "ttm_linear_group: operands must be 16-byte aligned");
   LinearArgs p;
@@ -1813,6 +1821,7 @@ TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int 
     p.gW[j] = j < n ? (const uint8_t *)w[j] : nullptr;
     p.gC[j] = j < n ? (uint8_t *)out[j] : nullptr;
     p.gNt[j] = j < n ? (int)ttm_cdiv(N[j], 32) : 0;
+    p.gAct[j] = j < n && act ? act[j] : TTM_ACT_NONE;
     p.Nt += p.gNt[j];
   }
   p.act = TTM_ACT_NONE; p.bias_tiled = 1;

@@ -352,14 +352,18 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
       }
     }
   }
-  // Further matmuls of the same activations with block-float weights of the same format a few ops further on (the Q, K and
-  // V projections) run in this launch; only reshapes, permutes, rotary embeddings and deallocations of other tensors may
-  // lie between, and a follower that has an add / multiply of its own to fuse is left alone.
-  if (ctx.fuseViews && tailOp == TTM_TAIL_NONE && !biasRef && activation.empty() && !transposeA && !transposeB && batch == 1 &&
+  // Further matmuls / bias-free linears of the same activations with block-float weights of the same format a few ops
+  // further on (the Q, K and V projections; the gate and up projections of an MLP) run in this launch, each with its own
+  // activation; only reshapes, permutes, rotary embeddings and deallocations of other tensors may lie between.  A follower
+  // that has an add / multiply of its own to fuse is left alone, unless the token count is one where a projection alone
+  // would split K to fill the device (64 < M <= 1024): there one unsplit launch for all members wins and the follower's
+  // element-wise op runs by itself.
+  if (ctx.fuseViews && tailOp == TTM_TAIL_NONE && !biasRef && !transposeA && !transposeB && batch == 1 &&
       utils::isBlockFormatDataType(b.handle->dtype) && layoutFromTensorRef(outRef) == Layout{StorageType::Device, TensorLayout::Tile, DataType::BFloat16}) {
-    struct Follower { std::uint32_t index; fb::Table out; Tensor weight; std::int64_t n; };
+    struct Follower { std::uint32_t index; fb::Table out; Tensor weight; std::int64_t n; int act; };
     std::vector<Follower> followers;
     const std::vector<std::uint32_t> outShape = shapeFromTensorRef(outRef);
+    const bool midM = M > 64 && M <= 1024;
     for (std::uint32_t j = ctx.opIndex + 1; j < ctx.ops.size() && j <= ctx.opIndex + 10 && followers.size() < 3; ++j) {
       const OpType t = opType(j);
       fb::Table nop = ctx.ops[j].table(schema::Operation::f_type);
@@ -369,12 +373,23 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
         if (freed == refId(aRef) || freed == refId(outRef)) break;
         continue;
       }
-      if (t != OpType::MatmulOp || ctx.skip.count(j)) break;
-      using M2 = schema::MatmulOp;
-      fb::Table a2 = nop.table(M2::f_a), b2 = nop.table(M2::f_b), out2 = nop.table(M2::f_out);
-      if (!a2 || !b2 || !out2 || refId(a2) != refId(aRef) || nop.scalar<std::uint8_t>(M2::f_transpose_a, 0) ||
-          nop.scalar<std::uint8_t>(M2::f_transpose_b, 0) || !nop.string(M2::f_activation).empty())
-        break;
+      if ((t != OpType::MatmulOp && t != OpType::LinearOp) || ctx.skip.count(j)) break;
+      fb::Table a2, b2, out2;
+      bool plainOperands;
+      std::string_view act2;
+      if (t == OpType::MatmulOp) {
+        using M2 = schema::MatmulOp;
+        a2 = nop.table(M2::f_a); b2 = nop.table(M2::f_b); out2 = nop.table(M2::f_out);
+        plainOperands = !nop.scalar<std::uint8_t>(M2::f_transpose_a, 0) && !nop.scalar<std::uint8_t>(M2::f_transpose_b, 0);
+        act2 = nop.string(M2::f_activation);
+      } else {
+        using L2 = schema::LinearOp;
+        a2 = nop.table(L2::f_a); b2 = nop.table(L2::f_b); out2 = nop.table(L2::f_out);
+        plainOperands = !nop.scalar<std::uint8_t>(L2::f_transpose_a, 0) && !nop.scalar<std::uint8_t>(L2::f_transpose_b, 0) &&
+                        !nop.table(L2::f_bias);
+        act2 = nop.string(L2::f_activation);
+      }
+      if (!a2 || !b2 || !out2 || refId(a2) != refId(aRef) || !plainOperands) break;
       auto wit = ctx.pool.find(refId(b2));
       if (wit == ctx.pool.end() || !isTensorAllocated(wit->second) || wit->second.handle->storage != StorageType::Device ||
           wit->second.handle->dtype != b.handle->dtype || wit->second.handle->shape.size() != 2 || b.handle->shape.size() != 2 ||
@@ -384,32 +399,35 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
       if (shape2.size() != outShape.size() || shape2.empty() || !std::equal(shape2.begin(), shape2.end() - 1, outShape.begin()) ||
           shape2.back() != wit->second.handle->shape[1])
         break;
-      // its own element-wise tail, if it has one, is worth more than the shared launch
-      std::uint32_t after = j + 1;
-      while (after < ctx.ops.size() && opType(after) == OpType::DeallocateOp) ++after;
-      if (after < ctx.ops.size() && opType(after) == OpType::EltwiseBinaryOp) {
-        fb::Table bop = ctx.ops[after].table(schema::Operation::f_type);
-        fb::Table l = bop.table(schema::EltwiseBinaryOp::f_lhs), r = bop.table(schema::EltwiseBinaryOp::f_rhs);
-        if ((l && refId(l) == refId(out2)) || (r && refId(r) == refId(out2))) break;
+      if (!midM) {   // its own element-wise tail, if it has one, is worth more than the shared launch
+        std::uint32_t after = j + 1;
+        while (after < ctx.ops.size() && opType(after) == OpType::DeallocateOp) ++after;
+        if (after < ctx.ops.size() && opType(after) == OpType::EltwiseBinaryOp) {
+          fb::Table bop = ctx.ops[after].table(schema::Operation::f_type);
+          fb::Table l = bop.table(schema::EltwiseBinaryOp::f_lhs), r = bop.table(schema::EltwiseBinaryOp::f_rhs);
+          if ((l && refId(l) == refId(out2)) || (r && refId(r) == refId(out2))) break;
+        }
       }
       bool distinct = wit->second.handle->data.get() != b.handle->data.get();
       for (const Follower &f : followers) distinct = distinct && f.weight.handle->data.get() != wit->second.handle->data.get();
       if (!distinct) break;
-      followers.push_back(Follower{j, out2, wit->second, static_cast<std::int64_t>(shape2.back())});
+      followers.push_back(Follower{j, out2, wit->second, static_cast<std::int64_t>(shape2.back()), activationCode(act2)});
     }
     if (!followers.empty()) {
       std::vector<const void *> ws{b.handle->data.get()};
       std::vector<void *> outs{out.handle->data.get()};
       std::vector<std::int64_t> ns{N};
+      std::vector<int> acts{activationCode(activation)};
       std::vector<Tensor> outTensors;
       for (const Follower &f : followers) {
         outTensors.push_back(makeOut(ctx, f.out, DataType::BFloat16, TensorLayout::Tile));
         ws.push_back(f.weight.handle->data.get());
         outs.push_back(outTensors.back().handle->data.get());
         ns.push_back(f.n);
+        acts.push_back(f.act);
       }
-      TTM_CALL(ttm_linear_group(a.handle->data.get(), static_cast<int>(ws.size()), ws.data(), ttmDtype(b.handle->dtype), outs.data(), ns.data(), M, K,
-                                ctx.stream()));
+      TTM_CALL(ttm_linear_group(a.handle->data.get(), static_cast<int>(ws.size()), ws.data(), ttmDtype(b.handle->dtype), outs.data(), ns.data(),
+                                acts.data(), M, K, ctx.stream()));
       ctx.put(outRef, out);
       for (size_t i = 0; i < followers.size(); ++i) {
         ctx.put(followers[i].out, outTensors[i]);
