@@ -229,7 +229,8 @@ int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void
  *   page table [batch, pages_per_user] pages [blocks, kv_heads, page_block, head_dim] where seq = pages_per_user *
  *   page_block; BFloat16.  scores = (q k^T + mask) * scale, mask additive BFloat16 [batch, 1, mask_heads, seq] or NULL;
  *   with is_causal and cur_pos [batch] keys after cur_pos[b] are excluded; scale <= 0 means 1/sqrt(head_dim); softmax in
- *   fp32.  Uses the stream's workspace for per-slice partial results.
+ *   fp32.  Uses the stream's workspace for per-slice partial results.  Up to 8 query heads per kv head are served by one
+ *   launch; more (multi-query attention) by several launches over the same cache.
  * ttm_paged_update_cache: ::ttnn::experimental::paged_update_cache (operations/kv_cache/paged_update_cache.cpp:14-57;
  *   shapes lib/Dialect/TTNN/IR/TTNNOps.cpp:4719-4820; golden tools/golden/mapping.py:8926-8963): cache
  *   [blocks, heads, block_size, head_dim], input [1, users, heads, head_dim], update_index [users], page_table

@@ -126,6 +126,8 @@ def _decode_case(hip, dev, orc, B, H, Hkv, S, D, cur, mask_heads=None, causal=Tr
     (2, 8, 1, 512, 32, [100, 511]),           # one kv head serving 8 query heads, single column tile
     (3, 12, 4, 96, 96, [95, 40, 7]),          # three column tiles
     (1, 16, 2, 8192, 256, [8000]),            # long cache: several slices per kv head
+    (2, 32, 1, 512, 64, [300, 511]),          # multi-query attention: 32 query heads on one kv head, four launches of 8
+    (3, 24, 2, 256, 128, [17, 200, 255]),     # 12 query heads per kv head: a launch of 8 and one of 4
 ])
 def test_sdpa_decode_causal(hip, dev, orc, B, H, Hkv, S, D, cur):
     _decode_case(hip, dev, orc, B, H, Hkv, S, D, cur)
@@ -166,8 +168,8 @@ def test_sdpa_decode_ignores_garbage_after_the_current_position(hip, dev, orc):
 
 def test_sdpa_decode_rejects_unsupported(hip, dev):
     z = torch.zeros(1 << 16, dtype=torch.bfloat16, device=dev)
-    with pytest.raises(hip.TTMError, match="query heads per kv head"):
-        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, hip.ptr(z), hip.BF16, 1, 16, 1, 32, 32,
+    with pytest.raises(hip.TTMError, match="multiple of kv heads"):
+        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, hip.ptr(z), hip.BF16, 1, 16, 3, 32, 32,
                  1, 0.0, hip.current_stream())
     with pytest.raises(hip.TTMError, match="multiple of 32"):
         hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, hip.ptr(z), hip.BF16, 1, 8, 8, 40, 32,
@@ -262,7 +264,7 @@ def test_rotary_embedding_split_heads_equals_reshape_then_rotary(hip, dev, dtype
         hip.call("ttm_rotary_embedding_split_heads", hip.ptr(xt), hip.ptr(ct), hip.ptr(st), hip.ptr(got), code, B, H, D, 4, -1, hip.current_stream())
 
 
-@pytest.mark.parametrize("B,H,Hkv,S,D", [(32, 32, 8, 512, 128), (5, 8, 2, 256, 64), (33, 4, 4, 128, 32)])
+@pytest.mark.parametrize("B,H,Hkv,S,D", [(32, 32, 8, 512, 128), (5, 8, 2, 256, 64), (33, 4, 4, 128, 32), (4, 20, 1, 128, 32)])
 def test_sdpa_decode_concat_heads_equals_reshape_of_the_plain_output(hip, dev, B, H, Hkv, S, D):
     """ttm_sdpa_decode_concat_heads writes [users, heads * head_dim]: the same values as ttm_sdpa_decode followed by a
     reshape, zero padding rows below the last user."""

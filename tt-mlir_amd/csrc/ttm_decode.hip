@@ -187,6 +187,7 @@ struct DecodeArgs {
   uint16_t *out;
   int B, H, Hkv, G, S, D, splits, keys_per_split, block, pages_per_user, mask_heads, is_causal;
   int concat_heads;   // out is [B, H * D] (row b holds user b's heads side by side) instead of [B, H, D]
+  int Gt, g0;         // query heads per kv head in the tensors, and the first of them this launch serves (it serves G of them)
   float scale;
 };
 
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
     // query fragments: lane supplies query row lane % 16, columns 32 c + 8 (lane / 16) .. + 7
     const int g = lane & 15, dq = (lane >> 4) * 8;
     bf16x8 qf[8];
-    const int h = hk * G + g;
+    const int h = hk * p.Gt + p.g0 + g;
     const uint16_t *qb = p.q + (int64_t)b * ttm_round_up32(p.H) * D;
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
@@ -248,7 +249,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
       if (c < DT && g < G) z = *(const u32x4 *)(qb + ttm_tiled_offset(h, 32 * c + dq, DT));
       qf[c] = *(bf16x8 *)&z;
     }
-    const int hrow = hk * G;  // mask rows of this block's heads
+    const int hrow = hk * p.Gt + p.g0;  // mask rows of this block's heads
     for (int g0 = wave; g0 < ngroups; g0 += 8) {
       // two groups of 16 keys per pass, all their loads issued before the first product
       u32x4 kf[2][8];
@@ -424,7 +425,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
       num += sl[c] * w;
       den += sl[D + 1] * w;
     }
-    const int h = hk * G + g;
+    const int h = hk * p.Gt + p.g0 + g;
     const uint16_t val = ttm_f32_to_bf16(den > 0.0f ? num / den : 0.0f);
     if (p.concat_heads) p.out[ttm_tiled_offset(b, h * D + c, (p.H * D) >> 5)] = val;
     else p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(h, c, D >> 5)] = val;
@@ -433,11 +434,11 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
     if (b == p.B - 1) {
       const int pad = (int)ttm_round_up32(p.B) - p.B;
       for (int i = tid0; i < pad * G * D; i += 256)
-        p.out[ttm_tiled_offset(p.B + i / (G * D), hk * G * D + i % (G * D), (p.H * D) >> 5)] = 0;
+        p.out[ttm_tiled_offset(p.B + i / (G * D), (hk * p.Gt + p.g0) * D + i % (G * D), (p.H * D) >> 5)] = 0;
     }
     return;
   }
-  if (hk == p.Hkv - 1) {   // padding rows of the last head tile
+  if (hk == p.Hkv - 1 && p.g0 + G == p.Gt) {   // padding rows of the last head tile
     const int pad = (int)ttm_round_up32(p.H) - p.H;
     for (int i = tid0; i < pad * D; i += 256)
       p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(p.H + i / D, i % D, D >> 5)] = 0;
@@ -580,8 +581,8 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
   TTM_REQUIRE(q && k && v && out, "ttm_sdpa_decode: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa_decode: tensors must be BFloat16");
   TTM_REQUIRE(batch > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "ttm_sdpa_decode: heads must be a multiple of kv heads");
-  const int64_t G = heads / kv_heads;
-  TTM_REQUIRE(G <= kMaxG, "ttm_sdpa_decode: at most %d query heads per kv head (got %lld)", kMaxG, (long long)G);
+  // a launch serves up to kMaxG query heads per kv head; more (multi-query attention) take several launches over the same cache
+  const int64_t Gt = heads / kv_heads, G = Gt < kMaxG ? Gt : kMaxG;
   TTM_REQUIRE(head_dim % 32 == 0 && head_dim >= 32 && head_dim <= 256, "ttm_sdpa_decode: head dim must be a multiple of 32 up to 256");
   TTM_REQUIRE(seq > 0 && seq % 32 == 0, "ttm_sdpa_decode: cache length must be a positive multiple of 32");
   TTM_REQUIRE(!mask || mask_heads == 1 || mask_heads == heads, "ttm_sdpa_decode: mask must have 1 or %lld head rows", (long long)heads);
@@ -604,14 +605,19 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
   p.splits = (int)splits; p.keys_per_split = (int)keys; p.block = (int)page_block; p.pages_per_user = (int)pages_per_user;
   p.mask_heads = mask_heads; p.is_causal = is_causal; p.concat_heads = concat_heads;
   p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)head_dim);
+  p.Gt = (int)Gt;
   void *ws = nullptr;
   if (int rc = ttm_stream_workspace(s, (size_t)(batch * kv_heads * splits * G * (head_dim + 2)) * sizeof(float), &ws)) return rc;
   p.part = (float *)ws;
-  const size_t lds = (size_t)(G * keys + G * head_dim + 2 * G + G * keys / 2) * sizeof(float);
-  hipLaunchKernelGGL(ttm_sdpa_decode_k, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
-  TTM_LAUNCH_CHECK();
-  hipLaunchKernelGGL(ttm_sdpa_decode_combine_k, dim3((unsigned)(batch * kv_heads)), dim3(256), 0, s, p);
-  TTM_LAUNCH_CHECK();
+  for (int64_t g0 = 0; g0 < Gt; g0 += kMaxG) {   // the launches of one call follow each other on the stream and share the workspace
+    p.g0 = (int)g0;
+    p.G = (int)(Gt - g0 < kMaxG ? Gt - g0 : kMaxG);
+    const size_t lds = (size_t)(p.G * keys + p.G * head_dim + 2 * p.G + p.G * keys / 2) * sizeof(float);
+    hipLaunchKernelGGL(ttm_sdpa_decode_k, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
+    TTM_LAUNCH_CHECK();
+    hipLaunchKernelGGL(ttm_sdpa_decode_combine_k, dim3((unsigned)(batch * kv_heads)), dim3(256), 0, s, p);
+    TTM_LAUNCH_CHECK();
+  }
   return TTM_OK;
 }
 
