@@ -416,6 +416,31 @@ def test_traced_program_replays_as_a_graph(device, orc):
     assert rt.get_stat("CapturedTrace") == 1 and rt.get_stat("ExecutedTrace") == 6
 
 
+def test_traced_program_with_grouped_two_pass_linears(device):
+    """A traced MLP at a token count where gate and up share a launch, with the two-pass route forced: the image pass, the
+    group launch and the workspace they use are recorded into the graph, and every replay equals the op-by-op run."""
+    from ttmlir_amd import hip
+    T, H, F = 256, 256, 512
+    traced = rt.Binary.load_from_memory(programs.traced_mlp(T, H, F))
+    eager = rt.Binary.load_from_memory(programs.traced_mlp(T, H, F, trace=False))
+    d = datagen.c4_mlp(T, H, F, seed=22)
+    main = traced.get_num_programs() - 1
+    resident = lambda binary, prog: [rt.to_layout(rt.from_torch(t), device, rt.get_layout(binary, prog, k + 1), retain=True)
+                                     for k, t in enumerate([d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])])]
+    res_t, res_e = resident(traced, main), resident(eager, 1)
+    g = torch.Generator().manual_seed(6)
+    hip.set_option("linear_two_pass", 2)
+    try:
+        rt.clear_stats()
+        for it in range(3):
+            x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+            assert torch.equal(_run_traced(traced, device, x, res_t), _run_traced(eager, device, x, res_e)), it
+        assert rt.get_stat("CapturedTrace") == 1 and rt.get_stat("ExecutedTrace") == 2
+        assert rt.get_stat("GroupedMatmul") >= 3
+    finally:
+        hip.set_option("linear_two_pass", 0)
+
+
 def test_host_transfer_inside_a_capture_is_refused_cleanly(device):
     pb = rt.ProgramBuilder()
 
