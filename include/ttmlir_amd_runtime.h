@@ -140,8 +140,9 @@ int ttrt_pb_binary(ttrt_builder *pb, uint32_t type, uint32_t lhs, uint32_t rhs, 
 int ttrt_pb_rms_norm(ttrt_builder *pb, uint32_t in, uint32_t weight, uint32_t bias, float eps, uint32_t *out);
 int ttrt_pb_softmax(ttrt_builder *pb, uint32_t in, int dim, uint32_t *out);
 int ttrt_pb_reduction(ttrt_builder *pb, uint32_t type, uint32_t in, const int32_t *dims, int ndims, int keep_dim, uint32_t *out);
+/* sliding_window < 0 = attribute absent; attention_sink 0 = operand absent (transformer.fbs:70-82) */
 int ttrt_pb_sdpa(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t mask, int is_causal, int has_scale, float scale,
-                 uint32_t *out);
+                 int64_t sliding_window, uint32_t attention_sink, uint32_t *out);
 /* decode path (include/ttmlir/Target/TTNN/operations/{transformer,kv_cache}.fbs); 0 = operand absent; a page table
  * selects PagedScaledDotProductAttentionDecodeOp */
 int ttrt_pb_rotary_embedding(ttrt_builder *pb, uint32_t in, uint32_t cos_cache, uint32_t sin_cache, int has_token_index,
@@ -154,7 +155,7 @@ int ttrt_pb_paged_update_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, ui
                                int share_cache);
 int ttrt_pb_paged_fill_cache(ttrt_builder *pb, uint32_t cache, uint32_t in, uint32_t page_table, uint32_t batch_idx);
 int ttrt_pb_sdpa_decode(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t page_table, uint32_t mask, uint32_t cur_pos,
-                        int is_causal, int has_scale, float scale, uint32_t *out);
+                        int is_causal, int has_scale, float scale, int64_t sliding_window, uint32_t attention_sink, uint32_t *out);
 int ttrt_pb_reshape(ttrt_builder *pb, uint32_t in, const uint32_t *shape, int rank, uint32_t *out);
 int ttrt_pb_permute(ttrt_builder *pb, uint32_t in, const int64_t *perm, int rank, uint32_t *out);
 int ttrt_pb_transpose(ttrt_builder *pb, uint32_t in, int dim0, int dim1, uint32_t *out);

@@ -41,7 +41,7 @@ def lib():
             "orc_rotary_embedding_f32": ([vp, vp, vp, vp, i64, i64, i64, i64], None),
             "orc_update_cache_f32": ([vp, vp, i64, i64, i64, i64, i64, i64], None),
             "orc_fill_cache_f32": ([vp, vp, i64, i64, i64, i64, i64], None),
-            "orc_sdpa_decode_f32": ([vp, vp, vp, vp, vp, i32, vp, i64, i64, i64, i64, i64, i32, f32], None),
+            "orc_sdpa_decode_f32": ([vp, vp, vp, vp, vp, i32, vp, i64, i64, i64, i64, i64, i32, f32, i64, vp], None),
             "orc_bfp_pack_tiles": ([vp, vp, i64, i32], None),
             "orc_bfp_unpack_tiles": ([vp, vp, i64, i32], None),
             "orc_bfp_pack_rm": ([vp, vp, i64, i64, i64, i32], None),
@@ -58,7 +58,7 @@ def lib():
             "orc_rmsnorm_f32": ([vp, vp, vp, vp, i64, i64, f32], None),
             "orc_softmax_f32": ([vp, vp, i64, i64, i64], None),
             "orc_reduce_f32": ([i32, vp, vp, i64, i64, i64], None),
-            "orc_sdpa_f32": ([vp, vp, vp, vp, i32, vp, i64, i64, i64, i64, i64, i64, i32, f32], None),
+            "orc_sdpa_f32": ([vp, vp, vp, vp, i32, vp, i64, i64, i64, i64, i64, i64, i32, f32, i64, vp], None),
         }
         for name, (args, res) in sig.items():
             fn = getattr(_lib, name)
@@ -285,7 +285,8 @@ def reduce(op, x, dim=-1, keepdim=False):
     return out if keepdim else out.reshape([s for k, s in enumerate(x.shape) if k != dim])
 
 
-def sdpa(q, k, v, mask=None, is_causal=False, scale=None):
+def sdpa(q, k, v, mask=None, is_causal=False, scale=None, sliding_window=None, attention_sink=None):
+    """attention_sink: the TTNN operand, any shape holding one value per query head ([1, Hq, 1, 1])."""
     q, k, v = _c(q, np.float32), _c(k, np.float32), _c(v, np.float32)
     B, Hq, Sq, D = q.shape
     _, Hkv, Sk, _ = k.shape
@@ -294,8 +295,9 @@ def sdpa(q, k, v, mask=None, is_causal=False, scale=None):
         mask = _c(mask, np.float32)
         mh = mask.shape[1]
     out = np.empty_like(q)
+    sink = None if attention_sink is None else _c(attention_sink, np.float32).reshape(Hq)
     lib().orc_sdpa_f32(_p(q), _p(k), _p(v), _p(mask), mh, _p(out), B, Hq, Hkv, Sq, Sk, D, int(is_causal),
-                       float(scale) if scale else 0.0)
+                       float(scale) if scale else 0.0, -1 if sliding_window is None else int(sliding_window), _p(sink))
     return out
 
 
@@ -370,7 +372,8 @@ def paged_fill_cache(cache, inp, page_table, batch_idx=None):
     return cache
 
 
-def sdpa_decode(q, k, v, cur_pos=None, mask=None, is_causal=True, scale=None):
+def sdpa_decode(q, k, v, cur_pos=None, mask=None, is_causal=True, scale=None, sliding_window=None, attention_sink=None):
+    """attention_sink: the op's [H, 32] operand (column 0 is read) or one value per head."""
     q, k, v = _c(q, np.float32), _c(k, np.float32), _c(v, np.float32)
     _, B, H, D = q.shape
     _, Hkv, S, _ = k.shape
@@ -380,6 +383,10 @@ def sdpa_decode(q, k, v, cur_pos=None, mask=None, is_causal=True, scale=None):
         mask = _c(mask, np.float32)
         mh = mask.shape[2]
     out = np.empty_like(q)
+    sink = None
+    if attention_sink is not None:
+        sink = _c(attention_sink, np.float32)
+        sink = _c(sink[:, 0] if sink.ndim == 2 else sink.reshape(H), np.float32)
     lib().orc_sdpa_decode_f32(_p(q), _p(k), _p(v), _p(cp), _p(mask), mh, _p(out), B, H, Hkv, S, D, int(is_causal),
-                              float(scale) if scale else 0.0)
+                              float(scale) if scale else 0.0, -1 if sliding_window is None else int(sliding_window), _p(sink))
     return out

@@ -488,10 +488,17 @@ void orc_reduce_f32(int op, const float *x, float *out, int64_t outer, int64_t d
 /* ------------------------------------------------------------------ scaled dot product attention
  * q [B,Hq,Sq,D], k/v [B,Hkv,Sk,D]; query head h reads kv head h / (Hq/Hkv); mask (optional)
  * is additive, [B,1,Sq,Sk] or [B,Hq,Sq,Sk] (mask_heads = 1 or Hq); causal adds -inf above the
- * diagonal; scale <= 0 means 1/sqrt(D).  Softmax in f32.                                    */
+ * diagonal; scale <= 0 means 1/sqrt(D).  Softmax in f32.
+ * window >= 0 (tools/golden/mapping.py:8450-8467): query i sees key j when 0 <= i - j < window under is_causal, when
+ * |i - j| <= window / 2 otherwise; the window replaces the causal mask and a given mask is added on top.
+ * sink (optional, one value per query head; mapping.py:8476-8494): one more logit per head in the softmax, with no
+ * value row.  The value here is the operand of the TTNN op, which the kernel multiplies by scale like the scores
+ * (lib/Conversion/TTIRToTTNN/TTIRToTTNN.cpp:3507-3533: the lowering divides the source graph's logit by scale to
+ * compensate), so the golden on logit x equals this function on x / scale.
+ * A query that sees nothing gives a row of zeros (the golden's softmax gives NaN there).                      */
 void orc_sdpa_f32(const float *q, const float *k, const float *v, const float *mask, int mask_heads,
                   float *out, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
-                  int is_causal, float scale) {
+                  int is_causal, float scale, int64_t window, const float *sink) {
   if (!(scale > 0.0f)) scale = 1.0f / sqrtf((float)D);
   int64_t rep = Hq / Hkv;
 #pragma omp parallel for num_threads(g_threads) schedule(dynamic, 4) if (g_threads > 1)
@@ -507,13 +514,18 @@ void orc_sdpa_f32(const float *q, const float *k, const float *v, const float *m
       for (int64_t d = 0; d < D; ++d) acc += qi[d] * kj[d];
       acc *= scale;
       if (mask) acc += mask[((b * mask_heads + (mask_heads == 1 ? 0 : h)) * Sq + i) * Sk + j];
-      if (is_causal && j > i) acc = -INFINITY;
+      if (window >= 0) {
+        int64_t diff = i - j, half = window / 2;
+        if (is_causal ? (diff < 0 || diff >= window) : (diff < -half || diff > half)) acc = -INFINITY;
+      } else if (is_causal && j > i) acc = -INFINITY;
       s[j] = acc;
       mx = acc > mx ? acc : mx;
     }
-    float sum = 0.0f;
-    for (int64_t j = 0; j < Sk; ++j) { s[j] = expf(s[j] - mx); sum += s[j]; }
-    float inv = 1.0f / sum;
+    float sink_logit = sink ? sink[h] * scale : -INFINITY;
+    mx = sink_logit > mx ? sink_logit : mx;
+    float sum = sink ? expf(sink_logit - mx) : 0.0f;
+    for (int64_t j = 0; j < Sk; ++j) { s[j] = mx == -INFINITY ? 0.0f : expf(s[j] - mx); sum += s[j]; }
+    float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
     float *o = out + ((b * Hq + h) * Sq + i) * D;
     for (int64_t d = 0; d < D; ++d) o[d] = 0.0f;
     for (int64_t j = 0; j < Sk; ++j) {
@@ -568,10 +580,17 @@ void orc_fill_cache_f32(float *cache, const float *input, int64_t H, int64_t S, 
 
 /* Attention of one new token (tools/golden/mapping.py:2417-2481): q [1,B,H,D], k / v [B,Hkv,S,D], mask (optional)
  * [B,1,mask_heads,S] additive BEFORE the scale, cur_pos (optional, with is_causal) excludes keys j > cur_pos[b];
- * scale <= 0 means 1/sqrt(D).  out [1,B,H,D]. */
+ * scale <= 0 means 1/sqrt(D).  out [1,B,H,D].
+ * window >= 0: of the keys up to the decode position p only the last `window` are visible, [max(0, p - window + 1), p]
+ * (mapping.py:8814-8824, the paged golden); p = cur_pos[b], or S - 1 without cur_pos, as the op's description has it
+ * (include/ttmlir/Dialect/TTNN/IR/TTNNOps.td:4131-4134; the golden leaves the window out when cur_pos is absent).
+ * sink (optional, one value per head = column 0 of the op's [H, 32] operand): one more logit per head, sink * scale, in the
+ * softmax, with no value row - the prefill op's meaning (mapping.py:8476-8494) and what the lowering's comment says of
+ * both kernels (TTIRToTTNN.cpp:3507-3508).  PARITY UNPINNED against the decode goldens for the sink: mapping.py:2417-2481
+ * ignores the operand and mapping.py:8826-8829 only unmasks the first column, neither of which is the op.          */
 void orc_sdpa_decode_f32(const float *q, const float *k, const float *v, const int32_t *cur_pos, const float *mask,
                          int mask_heads, float *out, int64_t B, int64_t H, int64_t Hkv, int64_t S, int64_t D,
-                         int is_causal, float scale) {
+                         int is_causal, float scale, int64_t window, const float *sink) {
   if (!(scale > 0.0f)) scale = 1.0f / sqrtf((float)D);
   int64_t rep = H / Hkv;
   float *s = (float *)malloc(sizeof(float) * S);
@@ -586,12 +605,19 @@ void orc_sdpa_decode_f32(const float *q, const float *k, const float *v, const i
         for (int64_t d = 0; d < D; ++d) acc += qi[d] * kj[d];
         if (mask) acc += mask[(b * mask_heads + (mask_heads == 1 ? 0 : h)) * S + j];
         else if (is_causal && cur_pos && j > cur_pos[b]) acc = -INFINITY;
+        if (window >= 0) {
+          int64_t p = cur_pos ? cur_pos[b] : S - 1;
+          if (j < p - window + 1) acc = -INFINITY;
+        }
         acc *= scale;
         s[j] = acc;
         mx = acc > mx ? acc : mx;
       }
-      float sum = 0.0f;
-      for (int64_t j = 0; j < S; ++j) { s[j] = expf(s[j] - mx); sum += s[j]; }
+      float sink_logit = sink ? sink[h] * scale : -INFINITY;
+      mx = sink_logit > mx ? sink_logit : mx;
+      float sum = sink ? expf(sink_logit - mx) : 0.0f;
+      for (int64_t j = 0; j < S; ++j) { s[j] = mx == -INFINITY ? 0.0f : expf(s[j] - mx); sum += s[j]; }
+      if (!(sum > 0.0f)) sum = 1.0f;
       float *o = out + (b * H + h) * D;
       for (int64_t d = 0; d < D; ++d) o[d] = 0.0f;
       for (int64_t j = 0; j < S; ++j) {

@@ -285,3 +285,61 @@ def test_sdpa_decode_concat_heads_equals_reshape_of_the_plain_output(hip, dev, B
     torch.cuda.synchronize()
     assert torch.equal(got, want)
     assert torch.equal(merged, tilize_dev(hip, want.cpu(), dev))          # padding rows are zero
+
+
+@pytest.mark.parametrize("B,H,Hkv,S,D,window,sink,use_pos,paged,concat", [
+    (4, 8, 2, 1024, 128, 128, False, True, False, 0), (4, 8, 2, 1024, 128, 1, False, True, False, 0),
+    (3, 4, 4, 512, 64, 100, True, True, False, 0), (2, 8, 1, 2048, 128, 700, True, True, False, 1),
+    (2, 4, 2, 256, 32, 40, True, False, False, 0), (5, 8, 2, 512, 128, 33, True, True, True, 0),
+    (2, 20, 1, 256, 64, 64, True, True, False, 0), (32, 32, 8, 2048, 128, 512, False, True, False, 1),
+    (2, 4, 2, 512, 128, None, True, True, False, 0), (2, 4, 2, 512, 128, 5000, False, True, False, 0),
+    (1, 40, 40, 320, 96, 31, True, True, False, 0)])
+def test_sdpa_decode_sliding_window_and_attention_sink(hip, dev, orc, B, H, Hkv, S, D, window, sink, use_pos, paged, concat):
+    """ttm_sdpa_decode_windowed against the oracle: windows of one key, inside one slice of the cache, across slices,
+    longer than the cache; with and without positions; the sink alone and with a window; paged caches, the merged output
+    layout, more than 8 and more than 32 query heads.  The cache in front of every user's window holds NaN / Inf."""
+    g = torch.Generator().manual_seed(130)
+    q = datagen.randn((1, B, H, D), seed=131, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, S, D), seed=132, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, S, D), seed=133, dtype=torch.bfloat16)
+    cur = torch.randint(0, S, (B,), generator=g, dtype=torch.int32)
+    cur[0] = S - 1
+    if B > 1:
+        cur[1] = 0 if window is None else min(S - 1, max(0, window - 1))
+    sk = (datagen.randn((H, 1), seed=134, dtype=torch.bfloat16) * 8).expand(H, 32).contiguous() if sink else None
+    kb, vb = k.clone(), v.clone()
+    for b in range(B):
+        p = int(cur[b]) if use_pos else S - 1
+        if use_pos:
+            kb[b, :, p + 1:], vb[b, :, p + 1:] = float("nan"), float("inf")
+        if window is not None and p - window + 1 > 0:
+            kb[b, :, :p - window + 1], vb[b, :, :p - window + 1] = float("nan"), float("inf")
+    table_d, pages, block = None, 0, 0
+    if paged:
+        block = 64
+        pages = S // block
+        table = torch.randperm(B * pages, generator=g).reshape(B, pages).to(torch.int32)
+        kp = torch.empty((B * pages, Hkv, block, D), dtype=torch.bfloat16)
+        vp = torch.empty_like(kp)
+        for b in range(B):
+            for pg in range(pages):
+                kp[table[b, pg]] = kb[b, :, pg * block:(pg + 1) * block]
+                vp[table[b, pg]] = vb[b, :, pg * block:(pg + 1) * block]
+        kt, vt, table_d = tilize_dev(hip, kp, dev), tilize_dev(hip, vp, dev), table.to(dev)
+    else:
+        kt, vt = tilize_dev(hip, kb, dev), tilize_dev(hip, vb, dev)
+    qt = tilize_dev(hip, q, dev)
+    st = tilize_dev(hip, sk, dev) if sink else None
+    cp = cur.to(dev)
+    Bp = (B + 31) // 32 * 32
+    out = torch.full((Bp * H * D,), float("nan"), dtype=torch.bfloat16, device=dev) if concat else torch.full_like(qt, float("nan"))
+    hip.call("ttm_sdpa_decode_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp) if use_pos else None, None, 1,
+             hip.ptr(table_d) if paged else None, pages, block, hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 1, 0.0, concat,
+             -1 if window is None else window, hip.ptr(st) if sink else None, hip.current_stream())
+    got = f32(untilize_dev(hip, out, (B, H * D), dev)).reshape(1, B, H, D) if concat else f32(untilize_dev(hip, out, q.shape, dev))
+    want = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur.numpy() if use_pos else None, sliding_window=window,
+                           attention_sink=None if sk is None else f32(sk))
+    assert np.all(np.isfinite(got)) and np.max(np.abs(got - want)) <= 2.0 ** -6
+    if window is not None and window < S // 2 and not sink:
+        plain = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur.numpy() if use_pos else None)
+        assert np.max(np.abs(plain - want)) > 0.02           # the window matters for this case

@@ -356,3 +356,75 @@ def test_sdpa_heads_inner_equals_the_head_major_call(hip, dev, B, Hq, Hkv, Sq, S
         got = untilize_dev(hip, out, q.shape, dev).cpu()
     torch.cuda.synchronize()
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,window,sink,mask,flags", [
+    (1, 4, 2, 256, 256, 128, True, 64, False, None, 0), (1, 4, 2, 256, 256, 128, True, 1, False, None, 0),
+    (1, 4, 2, 300, 300, 64, True, 100, True, None, 0), (2, 2, 2, 96, 160, 128, False, 40, False, None, 0),
+    (1, 2, 1, 200, 200, 32, False, 0, False, None, 0), (1, 2, 2, 160, 160, 64, False, 65, True, "b1", 0),
+    (1, 8, 2, 512, 512, 128, True, 129, True, None, 15), (1, 2, 2, 70, 70, 64, True, 1000, True, None, 0),
+    (1, 2, 2, 128, 128, 128, True, None, True, None, 0), (2, 3, 3, 64, 100, 64, False, None, True, "bh", 0),
+    (1, 1, 1, 100, 300, 256, False, 33, True, None, 0), (1, 4, 4, 640, 640, 64, True, 32, False, None, 9),
+    (1, 2, 2, 1024, 1024, 128, True, 200, True, None, 0)])
+def test_sdpa_sliding_window_and_attention_sink(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, window, sink, mask, flags, variant):
+    """ttm_sdpa_windowed against the oracle: causal windows (one key, shorter and longer than a 64-key pass, longer than
+    the sequence), symmetric windows, width 0, with and without the per-head sink, with a mask on top, ragged lengths,
+    head-inner layouts, all three kernel variants."""
+    if variant == 1 and Sq * Sk >= 512 * 512:
+        pytest.skip("the 32-key kernel is covered by the small shapes")
+    import oracle.metrics as metrics
+    q = datagen.randn((B, Hq, Sq, D), seed=112, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, Sk, D), seed=113, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, Sk, D), seed=114, dtype=torch.bfloat16)
+    m = datagen.randn((B, 1 if mask == "b1" else Hq, Sq, Sk), seed=115, dtype=torch.bfloat16) if mask else None
+    sk = (datagen.randn((1, Hq, 1, 1), seed=116, dtype=torch.bfloat16) * 8).contiguous() if sink else None
+    inner = lambda t: t.permute(0, 2, 1, 3).reshape(t.shape[0], t.shape[2], t.shape[1] * t.shape[3]).contiguous()
+    qt = tilize_dev(hip, inner(q) if flags & 1 else q, dev)
+    kt = tilize_dev(hip, inner(k) if flags & 2 else k, dev)
+    vt = tilize_dev(hip, inner(v) if flags & 4 else v, dev)
+    mt = tilize_dev(hip, m, dev) if m is not None else None
+    st = tilize_dev(hip, sk, dev) if sink else None
+    out = torch.full_like(qt, float("nan"))
+    hip.set_option("sdpa_variant", variant)
+    try:
+        hip.call("ttm_sdpa_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(mt) if mt is not None else None,
+                 m.shape[1] if m is not None else 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, Sq, Sk, D, int(causal), 0.0, flags,
+                 -1 if window is None else window, hip.ptr(st) if sink else None, hip.current_stream())
+    finally:
+        hip.set_option("sdpa_variant", 0)
+    if flags & 8:
+        res = untilize_dev(hip, out, (B, Sq, Hq * D), dev).cpu().reshape(B, Sq, Hq, D).permute(0, 2, 1, 3)
+    else:
+        res = untilize_dev(hip, out, q.shape, dev).cpu()
+    torch.cuda.synchronize()
+    res = res.float().numpy()
+    want = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), None if m is None else m.float().numpy(),
+                    is_causal=causal, sliding_window=window, attention_sink=None if sk is None else sk.float().numpy())
+    assert np.all(np.isfinite(out.float().cpu().numpy()))
+    # probabilities are rounded to bf16 before P.V (relative 2^-9 each) and the output once more
+    assert np.max(np.abs(res - want)) <= 2.0 ** -6
+    assert metrics.get_pcc(want, res) >= 0.9999
+    if window is not None and window < Sk and not sink:
+        plain = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), None if m is None else m.float().numpy(), is_causal=causal)
+        assert np.max(np.abs(plain - want)) > 0.05          # the window matters for this case
+
+
+def test_sdpa_window_does_not_read_keys_outside_it(hip, dev, orc):
+    """Causal window of 64 keys over 1024: key tiles wholly in front of a query block's window hold NaN in K and Inf in V
+    for the queries of the last block; the result for those queries is finite and equal to the oracle's on clean data."""
+    B, H, S, D, w = 1, 2, 1024, 128, 64
+    q = datagen.randn((B, H, S, D), seed=120, dtype=torch.bfloat16)
+    k = datagen.randn((B, H, S, D), seed=121, dtype=torch.bfloat16)
+    v = datagen.randn((B, H, S, D), seed=122, dtype=torch.bfloat16)
+    kb, vb = k.clone(), v.clone()
+    first_q = S - 128                                       # the last block of 128 queries
+    hidden = (first_q - w + 1) // 32 * 32                   # keys no query of that block sees
+    kb[:, :, :hidden], vb[:, :, :hidden] = float("nan"), float("inf")
+    qt, kt, vt = tilize_dev(hip, q, dev), tilize_dev(hip, kb, dev), tilize_dev(hip, vb, dev)
+    out = torch.full_like(qt, float("nan"))
+    hip.call("ttm_sdpa_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, 1, hip.ptr(out), hip.BF16, B, H, H, S, S, D, 1, 0.0, 0,
+             w, None, hip.current_stream())
+    got = untilize_dev(hip, out, q.shape, dev).float().cpu().numpy()[:, :, first_q:]
+    want = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), is_causal=True, sliding_window=w)[:, :, first_q:]
+    assert np.all(np.isfinite(got)) and np.max(np.abs(got - want)) <= 2.0 ** -6

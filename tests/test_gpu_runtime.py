@@ -761,3 +761,57 @@ def test_paged_cache_program_fill_update_attend(device, orc, metrics):
     want = orc.sdpa_decode(f(qq), gather(wk), gather(wv), cur_pos=positions.tolist())
     assert np.max(np.abs(got - want)) <= 2.0 ** -6
     assert metrics.get_pcc(want, got) >= 0.9999
+
+
+def test_attention_programs_with_sliding_window_and_sink(device, orc, metrics):
+    """ScaledDotProductAttentionOp, ScaledDotProductAttentionDecodeOp and the paged decode op with sliding_window_size and
+    attention_sink set in the flatbuffer (include/ttmlir/Target/TTNN/operations/transformer.fbs:56-82, 135-150), submitted
+    as one program: each output against the oracle with the same attributes."""
+    B, Hq, Hkv, S, D, W = 2, 4, 2, 160, 64, 48
+    users, cache, bs, pages = 3, 256, 64, 4
+    pb = rt.ProgramBuilder()
+    pb.begin_program("windowed")
+    q = pb.input((B, Hq, S, D), DT.BFloat16)
+    k = pb.input((B, Hkv, S, D), DT.BFloat16)
+    v = pb.input((B, Hkv, S, D), DT.BFloat16)
+    sink = pb.input((1, Hq, 1, 1), DT.BFloat16)
+    qd = pb.input((1, users, Hq, D), DT.BFloat16)
+    kc = pb.input((users, Hkv, cache, D), DT.BFloat16)
+    vc = pb.input((users, Hkv, cache, D), DT.BFloat16)
+    pos = pb.input((users,), DT.Int32, TL.RowMajor)
+    sinkd = pb.input((Hq, 32), DT.BFloat16)
+    kp = pb.input((users * pages, Hkv, bs, D), DT.BFloat16)
+    vp = pb.input((users * pages, Hkv, bs, D), DT.BFloat16)
+    table = pb.input((users, pages), DT.Int32, TL.RowMajor)
+    pb.output(pb.sdpa(q, k, v, is_causal=True, sliding_window=W, attention_sink=sink))
+    pb.output(pb.sdpa(q, k, v, is_causal=False, sliding_window=W))
+    pb.output(pb.sdpa_decode(qd, kc, vc, cur_pos=pos, is_causal=True, sliding_window=W, attention_sink=sinkd))
+    pb.output(pb.sdpa_decode(qd, kp, vp, cur_pos=pos, page_table=table, is_causal=True, sliding_window=W, attention_sink=sinkd))
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    g = torch.Generator().manual_seed(29)
+    rn = lambda *shape: bf(torch.randn(shape, generator=g))
+    tq, tk, tv, tsink = rn(B, Hq, S, D), rn(B, Hkv, S, D), rn(B, Hkv, S, D), bf(torch.randn((1, Hq, 1, 1), generator=g) * 6)
+    tqd, tkc, tvc = rn(1, users, Hq, D), rn(users, Hkv, cache, D), rn(users, Hkv, cache, D)
+    tpos = torch.tensor([10, 100, 255], dtype=torch.int32)
+    tsinkd = tsink.reshape(Hq, 1).expand(Hq, 32).contiguous()
+    tbl = torch.randperm(users * pages, generator=g).reshape(users, pages).to(torch.int32)
+    tkp, tvp = torch.empty((users * pages, Hkv, bs, D), dtype=torch.bfloat16), torch.empty((users * pages, Hkv, bs, D), dtype=torch.bfloat16)
+    for u in range(users):
+        for p in range(pages):
+            tkp[tbl[u, p]] = tkc[u, :, p * bs:(p + 1) * bs]
+            tvp[tbl[u, p]] = tvc[u, :, p * bs:(p + 1) * bs]
+    tins = [tq, tk, tv, tsink, tqd, tkc, tvc, tpos, tsinkd, tkp, tvp, tbl]
+    devs = [rt.to_layout(rt.from_torch(t.contiguous()), device, rt.get_layout(binary, 0, i)) for i, t in enumerate(tins)]
+    outs = rt.submit(device, binary, 0, devs)
+    got = [rt.to_torch(rt.to_host(y, untilize=True)[0]).float().numpy() for y in outs]
+    f = lambda t: t.float().numpy()
+    want = [orc.sdpa(f(tq), f(tk), f(tv), is_causal=True, sliding_window=W, attention_sink=f(tsink)),
+            orc.sdpa(f(tq), f(tk), f(tv), is_causal=False, sliding_window=W),
+            orc.sdpa_decode(f(tqd), f(tkc), f(tvc), cur_pos=tpos.numpy(), sliding_window=W, attention_sink=f(tsinkd))]
+    want.append(want[2])
+    for w_, g_ in zip(want, got):
+        assert np.max(np.abs(g_ - w_)) <= 2.0 ** -6
+        assert metrics.get_pcc(w_, g_) >= 0.9999
+    plain = orc.sdpa_decode(f(tqd), f(tkc), f(tvc), cur_pos=tpos.numpy())
+    assert np.max(np.abs(plain - want[2])) > 0.02

@@ -240,3 +240,126 @@ def test_sdpa_decode_against_library_attention(orc, H, Hkv):
     got = orc.sdpa_decode(q, k, v, mask=m, scale=0.25)
     want = F.scaled_dot_product_attention(qt, kr, vr, attn_mask=torch.from_numpy(m).permute(0, 2, 1, 3) * 0.25, scale=0.25)
     assert np.allclose(got[0], want.squeeze(2).numpy(), rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_sdpa_sliding_window_against_library_attention_with_a_band_mask(orc, causal):
+    """The window restated through torch's attention with a boolean band (tools/golden/mapping.py:8450-8467 gives the
+    band's edges), plus the cases the band's definition fixes without any formula: a causal window as long as the
+    sequence is plain causal attention, a causal window of one key returns the value rows themselves, a symmetric
+    window of width 0 (or 1: half = 0) does too."""
+    B, Hq, Hkv, S, D = 2, 4, 2, 40, 16
+    q, k, v = rnd((B, Hq, S, D), 40), rnd((B, Hkv, S, D), 41), rnd((B, Hkv, S, D), 42)
+    kr = torch.from_numpy(k).repeat_interleave(Hq // Hkv, dim=1)
+    vr = torch.from_numpy(v).repeat_interleave(Hq // Hkv, dim=1)
+    i, j = torch.arange(S)[:, None], torch.arange(S)[None, :]
+    for w in (1, 2, 7, 16, 39, 40, 100):
+        keep = ((i - j >= 0) & (i - j < w)) if causal else ((i - j).abs() <= w // 2)
+        want = F.scaled_dot_product_attention(torch.from_numpy(q), kr, vr, attn_mask=keep)
+        got = orc.sdpa(q, k, v, is_causal=causal, sliding_window=w)
+        assert np.allclose(got, want.numpy(), rtol=1e-4, atol=1e-5), w
+    if causal:
+        assert np.array_equal(orc.sdpa(q, k, v, is_causal=True, sliding_window=S), orc.sdpa(q, k, v, is_causal=True))
+        assert np.allclose(orc.sdpa(q, k, v, is_causal=True, sliding_window=1), vr.numpy(), atol=1e-6)
+    else:
+        assert np.array_equal(orc.sdpa(q, k, v, sliding_window=2 * S), orc.sdpa(q, k, v))
+        for w in (0, 1):
+            assert np.allclose(orc.sdpa(q, k, v, sliding_window=w), vr.numpy(), atol=1e-6)
+    # a mask given as well is added on top of the window
+    m = rnd((B, 1, S, S), 43)
+    keep = ((i - j >= 0) & (i - j < 5)) if causal else ((i - j).abs() <= 2)
+    want = F.scaled_dot_product_attention(torch.from_numpy(q), kr, vr,
+                                          attn_mask=torch.from_numpy(m).masked_fill(~keep, float("-inf")))
+    # (a causal op carries no mask in the reference; the oracle adds one all the same)
+    assert np.allclose(orc.sdpa(q, k, v, mask=m, is_causal=causal, sliding_window=5), want.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def test_sdpa_attention_sink_is_one_more_key_with_a_zero_value_row(orc):
+    """The sink as the golden has it (tools/golden/mapping.py:8476-8494: a column concatenated to the scores before the
+    softmax and dropped after it) is attention over one more key whose value row is zero.  With the last coordinate of
+    every query fixed at 1 and of every real key at 0, the extra key (0, ..., 0, x_h / scale) has the logit x_h for every
+    query of head h: the plain oracle on the extended tensors must equal the oracle with the sink operand x_h / scale
+    (the operand is the logit divided by the scale, lib/Conversion/TTIRToTTNN/TTIRToTTNN.cpp:3507-3533)."""
+    B, H, Sq, Sk, D = 2, 3, 9, 12, 8
+    q, k, v = rnd((B, H, Sq, D), 44), rnd((B, H, Sk, D), 45), rnd((B, H, Sk, D), 46)
+    q[..., -1] = 1.0
+    k[..., -1] = 0.0
+    x = np.array([-1.5, 0.0, 2.25], np.float32)                  # logits per head
+    for scale in (None, 0.5, 1.0):
+        s = scale if scale else 1.0 / np.sqrt(D)
+        k_ext = np.concatenate([k, np.zeros((B, H, 1, D), np.float32)], axis=2)
+        k_ext[:, :, -1, -1] = (x / s)[None, :]
+        v_ext = np.concatenate([v, np.zeros((B, H, 1, D), np.float32)], axis=2)
+        want = orc.sdpa(q, k_ext, v_ext, scale=scale)
+        got = orc.sdpa(q, k, v, scale=scale, attention_sink=(x / s).reshape(1, H, 1, 1))
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+        assert not np.allclose(got, orc.sdpa(q, k, v, scale=scale), atol=1e-3)
+    # a sink far below every score changes nothing, one far above takes all the weight
+    assert np.allclose(orc.sdpa(q, k, v, attention_sink=np.full(H, -1e4, np.float32)), orc.sdpa(q, k, v), atol=1e-6)
+    assert np.max(np.abs(orc.sdpa(q, k, v, attention_sink=np.full(H, 1e4, np.float32)))) < 1e-6
+    # grouped heads: the sink is per QUERY head
+    kg, vg = k[:, :1], v[:, :1]
+    got = orc.sdpa(q, kg, vg, attention_sink=x)
+    for h in range(H):
+        one = orc.sdpa(q[:, h:h + 1], kg, vg, attention_sink=x[h:h + 1])
+        assert np.array_equal(got[:, h:h + 1], one)
+    # causal + window + sink together, against the extended-key form with the band written as a mask
+    S = 9
+    q2, k2, v2 = q[:, :, :S], k[:, :, :S], v[:, :, :S]
+    i, j = np.arange(S)[:, None], np.arange(S)[None, :]
+    band = np.where((i - j >= 0) & (i - j < 4), 0.0, -np.inf).astype(np.float32)
+    band_ext = np.concatenate([band, np.zeros((S, 1), np.float32)], axis=1)[None, None]
+    s = 1.0 / np.sqrt(D)
+    k_ext = np.concatenate([k2, np.zeros((B, H, 1, D), np.float32)], axis=2)
+    k_ext[:, :, -1, -1] = (x / s)[None, :]
+    v_ext = np.concatenate([v2, np.zeros((B, H, 1, D), np.float32)], axis=2)
+    want = orc.sdpa(q2, k_ext, v_ext, mask=np.broadcast_to(band_ext, (B, 1, S, S + 1)))
+    got = orc.sdpa(q2, k2, v2, is_causal=True, sliding_window=4, attention_sink=x / s)
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+
+
+def test_sdpa_decode_window_and_sink(orc):
+    """Decode: the window keeps keys [max(0, p - w + 1), p] (tools/golden/mapping.py:8814-8824), checked against torch's
+    attention with that set written as a boolean mask, and against the prefill oracle's last causal row; the sink against
+    a cache that holds the extra key at position 0 (k = 0 -> logit 0, v = 0) with every position shifted by one."""
+    B, H, Hkv, S, D = 3, 4, 2, 64, 16
+    q, k, v = rnd((1, B, H, D), 47), rnd((B, Hkv, S, D), 48), rnd((B, Hkv, S, D), 49)
+    cur = np.array([3, 30, 63], np.int32)
+    qt = torch.from_numpy(q)[0].unsqueeze(2)
+    kr = torch.from_numpy(k).repeat_interleave(H // Hkv, dim=1)
+    vr = torch.from_numpy(v).repeat_interleave(H // Hkv, dim=1)
+    j, p = torch.arange(S)[None, :], torch.from_numpy(cur).long()[:, None]
+    for w in (1, 4, 17, 31, 64, 200):
+        keep = ((j <= p) & (j >= p - w + 1))[:, None, None, :]
+        want = F.scaled_dot_product_attention(qt, kr, vr, attn_mask=keep).squeeze(2).unsqueeze(0)
+        assert np.allclose(orc.sdpa_decode(q, k, v, cur_pos=cur, sliding_window=w), want.numpy(), rtol=1e-4, atol=1e-5), w
+    assert np.array_equal(orc.sdpa_decode(q, k, v, cur_pos=cur, sliding_window=S), orc.sdpa_decode(q, k, v, cur_pos=cur))
+    # window of one key: the value row at the decode position
+    one = orc.sdpa_decode(q, k, v, cur_pos=cur, sliding_window=1)
+    for b in range(B):
+        assert np.allclose(one[0, b], vr[b, :, cur[b]].numpy(), atol=1e-6)
+    # without cur_pos the window ends at the last position
+    last = orc.sdpa_decode(q, k, v, cur_pos=np.full(B, S - 1, np.int32), sliding_window=9)
+    assert np.array_equal(orc.sdpa_decode(q, k, v, is_causal=False, sliding_window=9), last)
+    # the decode of user b at position p is row p of causal windowed prefill attention over the same keys
+    qrow = np.zeros((1, H, S, D), np.float32)
+    qrow[0, :, 30] = q[0, 1]
+    pre = orc.sdpa(qrow, k[1:2], v[1:2], is_causal=True, sliding_window=17)
+    assert np.allclose(orc.sdpa_decode(q, k, v, cur_pos=cur, sliding_window=17)[0, 1], pre[0, :, 30], rtol=1e-5, atol=1e-6)
+    # sink with logit 0 = one more visible key with k = 0 and v = 0
+    k_sh = np.concatenate([np.zeros((B, Hkv, 1, D), np.float32), k[:, :, :-1]], axis=2)
+    v_sh = np.concatenate([np.zeros((B, Hkv, 1, D), np.float32), v[:, :, :-1]], axis=2)
+    cur2 = np.array([3, 30, 62], np.int32)
+    want = orc.sdpa_decode(q, k_sh, v_sh, cur_pos=cur2 + 1)
+    got = orc.sdpa_decode(q, k, v, cur_pos=cur2, attention_sink=np.zeros((H, 32), np.float32))
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
+    # the operand is multiplied by the scale like the scores: the same logits written for two scales give, with q
+    # rescaled to keep q k scale fixed, the same output
+    sink = np.tile(np.array([0.5, -2.0, 3.0, 1.0], np.float32)[:, None], (1, 32))
+    a = orc.sdpa_decode(q, k, v, cur_pos=cur, scale=0.25, attention_sink=sink)
+    b_ = orc.sdpa_decode(q * 0.5, k, v, cur_pos=cur, scale=0.5, attention_sink=sink * 0.5)
+    assert np.allclose(a, b_, rtol=1e-5, atol=1e-6)
+    assert not np.allclose(a, orc.sdpa_decode(q, k, v, cur_pos=cur, scale=0.25), atol=1e-3)
+    # the decode sink agrees with the prefill oracle's (one query row, everything visible)
+    full = orc.sdpa(np.ascontiguousarray(qt.numpy()), k, v, attention_sink=sink[:, 0])
+    assert np.allclose(orc.sdpa_decode(q, k, v, is_causal=False, attention_sink=sink)[0], full[:, :, 0], rtol=1e-5, atol=1e-6)

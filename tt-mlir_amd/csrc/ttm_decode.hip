@@ -188,6 +188,8 @@ struct DecodeArgs {
   int B, H, Hkv, G, S, D, splits, keys_per_split, block, pages_per_user, mask_heads, is_causal;
   int concat_heads;   // out is [B, H * D] (row b holds user b's heads side by side) instead of [B, H, D]
   int Gt, g0;         // query heads per kv head in the tensors, and the first of them this launch serves (it serves G of them)
+  int window;         // >= 0: only the last `window` keys up to the decode position are visible
+  const uint16_t *sink;   // [H, 32] in tiles, column 0: one more logit per head (times scale) with a zero value row; or null
   float scale;
 };
 
@@ -212,13 +214,18 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
   const int split = blockIdx.x, bh = blockIdx.y, b = bh / p.Hkv, hk = bh % p.Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int G = p.G, D = p.D, DT = D >> 5;
-  const int k0 = split * p.keys_per_split;
-  int valid = p.S;
-  if (p.is_causal && p.cur_pos) {
-    int cp = p.cur_pos[b] + 1;
-    valid = cp < valid ? (cp < 0 ? 0 : cp) : valid;
+  int valid = p.S, pos = p.S - 1;
+  if (p.cur_pos) {
+    pos = p.cur_pos[b];
+    if (p.is_causal) {
+      const int cp = pos + 1;
+      valid = cp < valid ? (cp < 0 ? 0 : cp) : valid;
+    }
   }
-  int k1 = k0 + p.keys_per_split;
+  // first visible key; the tiles in front of it are not read at all
+  const int lo = p.window >= 0 && pos + 1 > p.window ? pos + 1 - p.window : 0;
+  const int k0 = max(split * p.keys_per_split, lo & ~31);
+  int k1 = (split + 1) * p.keys_per_split;
   k1 = k1 < valid ? k1 : valid;
   const int nkeys = k1 > k0 ? k1 - k0 : 0;
   const int ngroups = (nkeys + 15) >> 4;
@@ -284,7 +291,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
               const int64_t mrows = ttm_round_up32(p.mask_heads);
               sv += ttm_bf16_to_f32(p.mask[(int64_t)b * mrows * p.S + ttm_tiled_offset(mh, k0 + kk, p.S >> 5)]);
             }
-            sc[gq * p.keys_per_split + kk] = (k0 + kk < k1) ? sv * p.scale : -INFINITY;
+            sc[gq * p.keys_per_split + kk] = (k0 + kk < k1 && k0 + kk >= lo) ? sv * p.scale : -INFINITY;
           }
         }
       }
@@ -348,8 +355,9 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
           const int t = t0 + u * share;
           if (t >= ntiles) break;
           uint32_t a[4] = {ra[u].x, ra[u].y, ra[u].z, ra[u].w}, c[4] = {rb[u].x, rb[u].y, rb[u].z, rb[u].w};
-          if (t * 32 + 32 > nkeys) {   // boundary tile: rows past the valid keys may hold anything, NaN included
-            const bool la = t * 32 + krow < nkeys, lb = t * 32 + 16 + krow < nkeys;
+          if (t * 32 + 32 > nkeys || k0 + t * 32 < lo) {   // boundary tile: rows outside the visible keys may hold anything, NaN included
+            const bool la = t * 32 + krow < nkeys && k0 + t * 32 + krow >= lo;
+            const bool lb = t * 32 + 16 + krow < nkeys && k0 + t * 32 + 16 + krow >= lo;
 #pragma unroll
             for (int j = 0; j < 4; ++j) { a[j] = la ? a[j] : 0u; c[j] = lb ? c[j] : 0u; }
           }
@@ -416,16 +424,17 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
   const float *base = p.part + (size_t)bh * p.splits * G * (D + 2);
   for (int i = tid0; i < G * D; i += 256) {
     const int g = i / D, c = i % D;
-    float M = -INFINITY;
+    const int h = hk * p.Gt + p.g0 + g;
+    const float sinkv = p.sink ? ttm_bf16_to_f32(p.sink[ttm_tiled_offset(h, 0, 1)]) * p.scale : -INFINITY;
+    float M = sinkv;
     for (int s = 0; s < p.splits; ++s) M = fmaxf(M, base[((size_t)s * G + g) * (D + 2) + D]);
-    float num = 0.0f, den = 0.0f;
+    float num = 0.0f, den = p.sink ? __expf(sinkv - M) : 0.0f;
     for (int s = 0; s < p.splits; ++s) {
       const float *sl = base + ((size_t)s * G + g) * (D + 2);
       const float w = (sl[D] == -INFINITY) ? 0.0f : __expf(sl[D] - M);
       num += sl[c] * w;
       den += sl[D + 1] * w;
     }
-    const int h = hk * p.Gt + p.g0 + g;
     const uint16_t val = ttm_f32_to_bf16(den > 0.0f ? num / den : 0.0f);
     if (p.concat_heads) p.out[ttm_tiled_offset(b, h * D + c, (p.H * D) >> 5)] = val;
     else p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(h, c, D >> 5)] = val;
@@ -577,7 +586,7 @@ TTM_EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_
 static int sdpa_decode_entry(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
                              const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out, int dtype, int64_t batch,
                              int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads,
-                             void *stream) {
+                             int64_t window, const void *sink, void *stream) {
   TTM_REQUIRE(q && k && v && out, "ttm_sdpa_decode: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa_decode: tensors must be BFloat16");
   TTM_REQUIRE(batch > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "ttm_sdpa_decode: heads must be a multiple of kv heads");
@@ -606,6 +615,8 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
   p.mask_heads = mask_heads; p.is_causal = is_causal; p.concat_heads = concat_heads;
   p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)head_dim);
   p.Gt = (int)Gt;
+  p.window = window < 0 ? -1 : (int)(window < seq ? window : seq);
+  p.sink = (const uint16_t *)sink;
   void *ws = nullptr;
   if (int rc = ttm_stream_workspace(s, (size_t)(batch * kv_heads * splits * G * (head_dim + 2)) * sizeof(float), &ws)) return rc;
   p.part = (float *)ws;
@@ -626,7 +637,7 @@ TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, cons
                                int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
                                int is_causal, float scale, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
-                           seq, head_dim, is_causal, scale, 0, stream);
+                           seq, head_dim, is_causal, scale, 0, -1, nullptr, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
@@ -634,5 +645,14 @@ TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const 
                                             void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
                                             int64_t head_dim, int is_causal, float scale, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
-                           seq, head_dim, is_causal, scale, 1, stream);
+                           seq, head_dim, is_causal, scale, 1, -1, nullptr, stream);
+}
+
+TTM_EXPORT int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
+                                        int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block,
+                                        void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
+                                        int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
+                                        const void *attention_sink, void *stream) {
+  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
+                           seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, stream);
 }

@@ -22,7 +22,10 @@ struct SdpaArgs {
   int B, Hq, Hkv, Sq, Sk;
   int sqt, skt;      // tiles along the sequence dims
   int mask_heads;    // 1 or Hq
-  int causal;
+  // query i sees key j when i - lo_off <= j <= i + hi_off.  Causal: hi_off = 0; a sliding window of w keys: lo_off = w - 1
+  // under a causal pass, lo_off = hi_off = w / 2 otherwise; kNoLimit where a side is open.
+  int hi_off, lo_off;
+  const uint8_t *sink;   // [1, Hq, 1, 1] in tiles (one tile per head, value at its first element), or null
   float scale;
   // Where a row of tiles of one head lives, per operand, in bytes: matrix (b, h) starts at b * batch + h * head, its tile
   // row t at + t * pitch (the D / 32 tiles of a tile row are contiguous).  [B, H, S, D]: pitch = D / 32 tiles, head =
@@ -30,6 +33,25 @@ struct SdpaArgs {
   // tiles, head = D / 32 tiles, batch = S / 32 * pitch.  Same 32 x 32 tiles either way.
   int64_t q_pitch, q_head, q_batch, k_pitch, k_head, k_batch, v_pitch, v_head, v_batch, o_pitch, o_head, o_batch;
 };
+
+constexpr int kNoLimit = 1 << 29;
+
+// first and one-past-last 32-key tile that the queries [q_first, q_last] can see
+__device__ __forceinline__ int first_key_tile(const SdpaArgs &p, int q_first) {
+  const int lo = q_first - p.lo_off;
+  return lo > 0 ? lo >> 5 : 0;
+}
+__device__ __forceinline__ int end_key_tile(const SdpaArgs &p, int q_last) {
+  return min(p.skt, ((q_last + p.hi_off) >> 5) + 1);
+}
+// the attention sink is one more logit per head with a zero value row: it enters the running maximum and the running
+// sum before the first key does, and the online softmax carries it from there
+__device__ __forceinline__ void sink_start(const SdpaArgs &p, int h, float scale2, float &m_run, float &l_run) {
+  if (p.sink) {
+    m_run = __uint_as_float((uint32_t)(*(const uint16_t *)(p.sink + (int64_t)h * 2048)) << 16) * scale2;
+    l_run = 1.0f;
+  }
+}
 
 __device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
   return ttm_pack_bf16x2(a, b);
@@ -67,10 +89,12 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
     for (int r = 0; r < 16; ++r) o[d][r] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
   const int q_glob = qt * 32 + l31;
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = p.scale * LOG2E;
+  sink_start(p, h, scale2, m_run, l_run);
 
-  // number of key tiles any wave of this workgroup needs
-  int kt_end = p.skt;
-  if (p.causal) kt_end = min(kt_end, (min(qb * 4 + 4, p.sqt) * 32 + 31) / 32);
+  // key tiles any wave of this workgroup needs
+  const int kt_begin = first_key_tile(p, qb * 128), kt_end = end_key_tile(p, min(qb * 4 + 4, p.sqt) * 32 - 1);
   // K and V blocks travel global -> registers -> LDS; the loads of block kt + 1 are issued before block kt is
   // computed, so their latency hides behind the MFMA and softmax work
   constexpr int NC = (DT * 128 + 255) / 256;   // 16-byte chunks of a K (or V) block per lane
@@ -86,8 +110,8 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
       }
     }
   };
-  if (kt_end > 0) load_block(0);
-  for (int kt = 0; kt < kt_end; ++kt) {
+  if (kt_end > kt_begin) load_block(kt_begin);
+  for (int kt = kt_begin; kt < kt_end; ++kt) {
     __syncthreads();  // previous block fully consumed
 #pragma unroll
     for (int i = 0; i < NC; ++i) {
@@ -109,7 +133,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
     }
     __syncthreads();
     if (kt + 1 < kt_end) load_block(kt + 1);
-    const bool skip = !wave_ok || (p.causal && kt * 32 > qt * 32 + 31);
+    const bool skip = !wave_ok || kt * 32 > qt * 32 + 31 + p.hi_off || kt * 32 + 31 < qt * 32 - p.lo_off;
     if (skip) continue;
 
     // S^T = K . Q^T for 32 keys x 32 queries
@@ -123,10 +147,8 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
     }
     // scale, mask; lane holds q = q_glob, keys kt*32 + 8g + 4hh + r.  Scores are kept in the log2 domain
     // (scale and mask multiplied by log2 e) so that the exponential is a bare v_exp_f32.
-    constexpr float LOG2E = 1.4426950408889634f;
-    const float scale2 = p.scale * LOG2E;
-    // masking by position is only needed on the diagonal block of a causal pass and on a ragged last block
-    const bool edge = (p.causal && kt * 32 + 31 > qt * 32) || kt * 32 + 32 > p.Sk;   // wavefront-uniform
+    // masking by position is only needed where a block crosses a limit of the visible range and on a ragged last block
+    const bool edge = kt * 32 + 31 > qt * 32 + p.hi_off || kt * 32 < qt * 32 + 31 - p.lo_off || kt * 32 + 32 > p.Sk;   // wavefront-uniform
     float mx = -INFINITY;
     if (p.mask || edge) {
 #pragma unroll
@@ -146,7 +168,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
         for (int r = 0; r < 4; ++r) {
           float v = fmaf(s[g * 4 + r], scale2, mk[r] * LOG2E);
           const int key = key0 + r;
-          if (key >= p.Sk || (p.causal && key > q_glob)) v = -INFINITY;
+          if (key >= p.Sk || key > q_glob + p.hi_off || key < q_glob - p.lo_off) v = -INFINITY;
           s[g * 4 + r] = v;
           mx = fmaxf(mx, v);
         }
@@ -252,9 +274,9 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
   float m_run = -INFINITY, l_run = 0.0f;
   const int q_glob = qt * 32 + l31, q_last = qt * 32 + 31;
 
-  int kt_end = p.skt;                                   // 32-key tiles any wave of this workgroup needs
-  if (p.causal) kt_end = min(kt_end, (min(qb * 4 + 4, p.sqt) * 32 + 31) / 32);
-  const int kb_end = (kt_end + 1) >> 1;                 // 64-key passes
+  // 32-key tiles any wave of this workgroup needs, and the 64-key passes that cover them
+  const int kt_begin = first_key_tile(p, qb * 128), kt_end = end_key_tile(p, min(qb * 4 + 4, p.sqt) * 32 - 1);
+  const int kb_begin = kt_begin >> 1, kb_end = (kt_end + 1) >> 1;
   // a lane moves DT 16-byte chunks of K and of V per pass: chunk c = tid + 256 i lies in tile row c / (DT * 128)
   u32x4 kreg[DT], vreg[DT];
   auto load_block = [&](int kb) {
@@ -266,10 +288,11 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
       vreg[i] = ((const u32x4 *)(p.v + v_mat + kt * p.v_pitch))[cc];
     }
   };
-  if (kb_end > 0) load_block(0);
+  if (kb_end > kb_begin) load_block(kb_begin);
   constexpr float LOG2E = 1.4426950408889634f;
   const float scale2 = p.scale * LOG2E;
-  for (int kb = 0; kb < kb_end; ++kb) {
+  sink_start(p, h, scale2, m_run, l_run);
+  for (int kb = kb_begin; kb < kb_end; ++kb) {
     __syncthreads();  // previous block fully consumed
 #pragma unroll
     for (int i = 0; i < DT; ++i) {
@@ -297,9 +320,9 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
     __syncthreads();
     if (kb + 1 < kb_end) load_block(kb + 1);
     const int key_base = kb * 64;
-    if (!wave_ok || (p.causal && key_base > q_last)) continue;
-    // the second half of the pass is skipped when the causal limit or the key count makes it empty for this wave
-    const bool second = !(p.causal && key_base + 32 > q_last) && key_base + 32 < p.Sk;   // wavefront-uniform
+    if (!wave_ok || key_base > q_last + p.hi_off || key_base + 63 < qt * 32 - p.lo_off) continue;
+    // the second half of the pass is skipped when the upper limit or the key count makes it empty for this wave
+    const bool second = key_base + 32 <= q_last + p.hi_off && key_base + 32 < p.Sk;   // wavefront-uniform
 
     f32x16 s0, s1;
 #pragma unroll
@@ -316,7 +339,7 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
     }
     // scale, mask; a lane holds q = q_glob and keys key_base + 32 half + 8 g + 4 hh + r.  Scores stay in the log2
     // domain so that the exponential is a bare v_exp_f32.
-    const bool edge = (p.causal && key_base + 63 > qt * 32) || key_base + 64 > p.Sk;   // wavefront-uniform
+    const bool edge = key_base + 63 > qt * 32 + p.hi_off || key_base < q_last - p.lo_off || key_base + 64 > p.Sk;   // wavefront-uniform
     float mx = -INFINITY;
     auto finish_scores = [&](f32x16 &s, int half) {
       if (p.mask || edge) {
@@ -338,7 +361,7 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
           for (int r = 0; r < 4; ++r) {
             float v = fmaf(s[g * 4 + r], scale2, mk[r] * LOG2E);
             const int key = key0 + r;
-            if (key >= p.Sk || (p.causal && key > q_glob)) v = -INFINITY;
+            if (key >= p.Sk || key > q_glob + p.hi_off || key < q_glob - p.lo_off) v = -INFINITY;
             s[g * 4 + r] = v;
             mx = fmaxf(mx, v);
           }
@@ -438,7 +461,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 }
 
 static int sdpa_entry(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B,
-                      int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int heads_inner, void *stream) {
+                      int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int heads_inner, int64_t window,
+                      const void *sink, void *stream) {
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa: tensors must be BFloat16 (got %d)", dtype);
   TTM_REQUIRE(B >= 0 && Hq >= 0 && Hkv > 0 && Sq >= 0 && Sk >= 0 && D > 0, "ttm_sdpa: bad dimension");
   TTM_REQUIRE(Hq % Hkv == 0, "ttm_sdpa: query heads (%ld) must be a multiple of kv heads (%ld)", (long)Hq, (long)Hkv);
@@ -453,7 +477,14 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
   p.out = (uint8_t *)out;
   p.B = (int)B; p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.Sq = (int)Sq; p.Sk = (int)Sk;
   p.sqt = (int)ttm_cdiv(Sq, 32); p.skt = (int)ttm_cdiv(Sk, 32);
-  p.mask_heads = mask_heads; p.causal = is_causal;
+  p.mask_heads = mask_heads;
+  if (window >= kNoLimit) window = kNoLimit - 1;   // longer than any sequence: no different from that length
+  p.hi_off = is_causal ? 0 : kNoLimit; p.lo_off = kNoLimit;
+  if (window >= 0) {   // a causal window holds the last `window` keys, a symmetric one window / 2 keys on either side
+    p.lo_off = is_causal ? (int)window - 1 : (int)(window / 2);
+    if (!is_causal) p.hi_off = (int)(window / 2);
+  }
+  p.sink = (const uint8_t *)sink;
   p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)D);
   TTM_REQUIRE(heads_inner >= 0 && heads_inner < 16, "ttm_sdpa: unknown layout flags %d", heads_inner);
   auto place = [&](bool inner, int64_t heads, int st, int64_t &pitch, int64_t &head, int64_t &batch) {
@@ -485,11 +516,19 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
 TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
                         int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                         int is_causal, float scale, void *stream) {
-  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, 0, stream);
+  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, 0, -1, nullptr, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
                                     int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                                     int is_causal, float scale, int heads_inner, void *stream) {
-  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner, stream);
+  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner, -1, nullptr, stream);
+}
+
+TTM_EXPORT int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
+                                 int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
+                                 int is_causal, float scale, int heads_inner, int64_t sliding_window, const void *attention_sink,
+                                 void *stream) {
+  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner,
+                    sliding_window < 0 ? -1 : sliding_window, attention_sink, stream);
 }

@@ -552,8 +552,9 @@ class ProgramBuilder:
         d = (ctypes.c_int32 * max(1, len(dims)))(*dims)
         return self._op("ttrt_pb_reduction", type_, t, d, len(dims), int(keep_dim))
 
-    def sdpa(self, q, k, v, mask=0, is_causal=False, scale=None):
-        return self._op("ttrt_pb_sdpa", q, k, v, mask, int(is_causal), int(scale is not None), ctypes.c_float(scale or 0.0))
+    def sdpa(self, q, k, v, mask=0, is_causal=False, scale=None, sliding_window=None, attention_sink=0):
+        return self._op("ttrt_pb_sdpa", q, k, v, mask, int(is_causal), int(scale is not None), ctypes.c_float(scale or 0.0),
+                        ctypes.c_int64(-1 if sliding_window is None else sliding_window), attention_sink)
 
     def rotary_embedding(self, t, cos_cache, sin_cache, token_index=None):
         return self._op("ttrt_pb_rotary_embedding", t, cos_cache, sin_cache, int(token_index is not None), token_index or 0)
@@ -570,9 +571,10 @@ class ProgramBuilder:
     def paged_fill_cache(self, cache, t, page_table, batch_idx=0):
         _call("ttrt_pb_paged_fill_cache", self.h, cache, t, page_table, batch_idx)
 
-    def sdpa_decode(self, q, k, v, cur_pos=0, mask=0, page_table=0, is_causal=True, scale=None):
+    def sdpa_decode(self, q, k, v, cur_pos=0, mask=0, page_table=0, is_causal=True, scale=None, sliding_window=None,
+                    attention_sink=0):
         return self._op("ttrt_pb_sdpa_decode", q, k, v, page_table, mask, cur_pos, int(is_causal), int(scale is not None),
-                        ctypes.c_float(scale or 0.0))
+                        ctypes.c_float(scale or 0.0), ctypes.c_int64(-1 if sliding_window is None else sliding_window), attention_sink)
 
     def reshape(self, t, shape):
         s, r = _shape_arg(shape)

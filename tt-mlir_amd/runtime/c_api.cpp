@@ -399,8 +399,8 @@ TTRT_EXPORT int ttrt_pb_reduction(ttrt_builder *pb, uint32_t type, uint32_t in, 
   PB_OP(reduction(type, in, std::vector<int>(dims, dims + ndims), keep_dim != 0));
 }
 TTRT_EXPORT int ttrt_pb_sdpa(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t mask, int is_causal, int has_scale, float scale,
-                             uint32_t *out) {
-  PB_OP(sdpa(q, k, v, mask, is_causal != 0, has_scale != 0, scale));
+                             int64_t sliding_window, uint32_t attention_sink, uint32_t *out) {
+  PB_OP(sdpa(q, k, v, mask, is_causal != 0, has_scale != 0, scale, sliding_window, attention_sink));
 }
 TTRT_EXPORT int ttrt_pb_rotary_embedding(ttrt_builder *pb, uint32_t in, uint32_t cos_cache, uint32_t sin_cache, int has_token_index,
                                          uint32_t token_index, uint32_t *out) {
@@ -420,8 +420,9 @@ TTRT_EXPORT int ttrt_pb_paged_fill_cache(ttrt_builder *pb, uint32_t cache, uint3
   return guard([&] { need(pb, "builder"); pb->pb.pagedFillCache(cache, in, page_table, batch_idx); });
 }
 TTRT_EXPORT int ttrt_pb_sdpa_decode(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t page_table, uint32_t mask, uint32_t cur_pos,
-                                    int is_causal, int has_scale, float scale, uint32_t *out) {
-  PB_OP(sdpaDecode(q, k, v, page_table, mask, cur_pos, is_causal != 0, has_scale != 0, scale));
+                                    int is_causal, int has_scale, float scale, int64_t sliding_window, uint32_t attention_sink,
+                                    uint32_t *out) {
+  PB_OP(sdpaDecode(q, k, v, page_table, mask, cur_pos, is_causal != 0, has_scale != 0, scale, sliding_window, attention_sink));
 }
 TTRT_EXPORT int ttrt_pb_reshape(ttrt_builder *pb, uint32_t in, const uint32_t *shape, int rank, uint32_t *out) { PB_OP(reshape(in, shapeVec(shape, rank))); }
 TTRT_EXPORT int ttrt_pb_permute(ttrt_builder *pb, uint32_t in, const int64_t *perm, int rank, uint32_t *out) {

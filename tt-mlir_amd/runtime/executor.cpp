@@ -623,7 +623,13 @@ void runSdpa(const fb::Table &op, ProgramContext &ctx) {
   const std::vector<std::uint32_t> ks = (inner & 2) ? shapeFromTensorRef(op.table(S::f_key)) : k.handle->shape;
   const std::vector<std::uint32_t> vs = (inner & 4) ? shapeFromTensorRef(op.table(S::f_value)) : v.handle->shape;
   TTRT_ASSERT(qs.size() == 4 && ks.size() == 4 && vs.size() == 4, "sdpa: q, k, v must be rank 4");
-  TTRT_ASSERT(!op.has(S::f_sliding_window_size) && !op.table(S::f_attention_sink), "sdpa: sliding window / attention sink are not supported");
+  const std::int64_t window = op.has(S::f_sliding_window_size) ? static_cast<std::int64_t>(op.scalar<std::uint32_t>(S::f_sliding_window_size, 0)) : std::int64_t(-1);
+  Tensor sink;
+  if (auto sr = op.table(S::f_attention_sink)) {
+    sink = as(ctx, ctx.get(sr, "sdpa attention sink"), TensorLayout::Tile, DataType::BFloat16);
+    const auto &ss = sink.handle->shape;
+    TTRT_ASSERT(ss.size() == 4 && ss[0] == 1 && ss[1] == qs[1] && ss[2] == 1 && ss[3] == 1, "sdpa: attention sink must be [1, Hq, 1, 1]");
+  }
   TTRT_ASSERT(ks == vs && qs[0] == ks[0] && qs[3] == ks[3], "sdpa: q/k/v shapes do not agree");
   Tensor mask;
   int maskHeads = 1;
@@ -676,9 +682,9 @@ void runSdpa(const fb::Table &op, ProgramContext &ctx) {
   if (mergedRef) inner |= 8;
   Tensor out = makeDeviceTensor(ctx.dev, mergedRef ? shapeFromTensorRef(mergedRef) : qs, DataType::BFloat16, TensorLayout::Tile);
   if (inner) debug::Stats::get().incrementStat("SdpaHeadsInner");
-  TTM_CALL(ttm_sdpa_heads_inner(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(), mask ? mask.handle->data.get() : nullptr,
-                                maskHeads, out.handle->data.get(), TTM_BF16, qs[0], qs[1], ks[1], qs[2], ks[2], qs[3], causal ? 1 : 0, scale,
-                                inner, ctx.stream()));
+  TTM_CALL(ttm_sdpa_windowed(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(), mask ? mask.handle->data.get() : nullptr,
+                             maskHeads, out.handle->data.get(), TTM_BF16, qs[0], qs[1], ks[1], qs[2], ks[2], qs[3], causal ? 1 : 0, scale,
+                             inner, window, sink ? sink.handle->data.get() : nullptr, ctx.stream()));
   if (mergedRef) {
     ctx.put(mergedRef, out);
     for (std::uint32_t i : skipped) ctx.skip.insert(i);
@@ -856,7 +862,8 @@ void runPagedFillCache(const fb::Table &op, ProgramContext &ctx) {
 }
 
 void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRef, const fb::Table &vRef, const fb::Table &pageRef,
-                const fb::Table &maskRef, const fb::Table &posRef, bool causal, float scale, const fb::Table &outRef) {
+                const fb::Table &maskRef, const fb::Table &posRef, bool causal, float scale, std::int64_t window,
+                const fb::Table &sinkRef, const fb::Table &outRef) {
   Tensor q = as(ctx, ctx.get(qRef, "sdpa_decode query"), TensorLayout::Tile, DataType::BFloat16);
   Tensor k = as(ctx, ctx.get(kRef, "sdpa_decode key"), TensorLayout::Tile, DataType::BFloat16);
   Tensor v = as(ctx, ctx.get(vRef, "sdpa_decode value"), TensorLayout::Tile, DataType::BFloat16);
@@ -874,8 +881,14 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
   } else {
     TTRT_ASSERT(ks[0] == B, "sdpa_decode: key / value batch differs from the query's");
   }
-  Tensor mask, pos;
+  Tensor mask, pos, sink;
   int maskHeads = 1;
+  if (sinkRef) {
+    sink = as(ctx, ctx.get(sinkRef, "sdpa_decode attention sink"), TensorLayout::Tile, DataType::BFloat16);
+    const auto &ss = sink.handle->shape;
+    TTRT_ASSERT(ss.size() == 2 && ss[0] == H && ss[1] == 32, "sdpa_decode: attention sink must be [heads, 32]");
+  }
+  const void *sinkPtr = sink ? sink.handle->data.get() : nullptr;
   if (maskRef) {
     mask = as(ctx, ctx.get(maskRef, "sdpa_decode mask"), TensorLayout::Tile, DataType::BFloat16);
     const auto &ms = mask.handle->shape;
@@ -896,38 +909,42 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
     if (fd.batch == 1 && fd.rows == B && fd.cols == H * D) {
       Tensor merged = makeDeviceTensor(ctx.dev, finalShape, DataType::BFloat16, TensorLayout::Tile);
       debug::Stats::get().incrementStat("FusedHeadConcat");
-      TTM_CALL(ttm_sdpa_decode_concat_heads(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
-                                            pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
-                                            mask ? mask.handle->data.get() : nullptr, maskHeads,
-                                            table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
-                                            merged.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, ctx.stream()));
+      TTM_CALL(ttm_sdpa_decode_windowed(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
+                                        pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
+                                        mask ? mask.handle->data.get() : nullptr, maskHeads,
+                                        table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
+                                        merged.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, 1, window, sinkPtr,
+                                        ctx.stream()));
       ctx.put(finalRef, merged);
       ctx.skip.insert(ctx.opIndex + 1);
       return;
     }
   }
   Tensor out = makeDeviceTensor(ctx.dev, qs, DataType::BFloat16, TensorLayout::Tile);
-  TTM_CALL(ttm_sdpa_decode(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
-                           pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
-                           mask ? mask.handle->data.get() : nullptr, maskHeads,
-                           table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
-                           out.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, ctx.stream()));
+  TTM_CALL(ttm_sdpa_decode_windowed(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
+                                    pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
+                                    mask ? mask.handle->data.get() : nullptr, maskHeads,
+                                    table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
+                                    out.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, 0, window, sinkPtr,
+                                    ctx.stream()));
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 void runSdpaDecode(const fb::Table &op, ProgramContext &ctx) {
   using S = schema::ScaledDotProductAttentionDecodeOp;
-  TTRT_ASSERT(!op.has(S::f_sliding_window_size) && !op.table(S::f_attention_sink), "sdpa_decode: sliding window / attention sink are not supported");
   sdpaDecode(ctx, op.table(S::f_query), op.table(S::f_key), op.table(S::f_value), fb::Table(), op.table(S::f_attention_mask),
              op.table(S::f_cur_pos_tensor), op.scalar<std::uint8_t>(S::f_is_causal, 0) != 0,
-             op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f, op.table(S::f_out));
+             op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f,
+             op.has(S::f_sliding_window_size) ? static_cast<std::int64_t>(op.scalar<std::uint32_t>(S::f_sliding_window_size, 0)) : std::int64_t(-1), op.table(S::f_attention_sink),
+             op.table(S::f_out));
 }
 void runPagedSdpaDecode(const fb::Table &op, ProgramContext &ctx) {
   using S = schema::PagedScaledDotProductAttentionDecodeOp;
-  TTRT_ASSERT(!op.has(S::f_sliding_window_size) && !op.table(S::f_attention_sink), "paged sdpa_decode: sliding window / attention sink are not supported");
   TTRT_ASSERT(static_cast<bool>(op.table(S::f_page_table)), "paged sdpa_decode: page table missing");
   sdpaDecode(ctx, op.table(S::f_query), op.table(S::f_key), op.table(S::f_value), op.table(S::f_page_table), op.table(S::f_attention_mask),
              op.table(S::f_cur_pos_tensor), op.scalar<std::uint8_t>(S::f_is_causal, 0) != 0,
-             op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f, op.table(S::f_out));
+             op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f,
+             op.has(S::f_sliding_window_size) ? static_cast<std::int64_t>(op.scalar<std::uint32_t>(S::f_sliding_window_size, 0)) : std::int64_t(-1), op.table(S::f_attention_sink),
+             op.table(S::f_out));
 }
 
 // ---- data movement (runtime/lib/ttnn/operations/data_movement/*.cpp)

@@ -395,13 +395,15 @@ ProgramBuilder::Id ProgramBuilder::reduction(std::uint32_t type, Id in, const st
   return out;
 }
 
-ProgramBuilder::Id ProgramBuilder::sdpa(Id q, Id k, Id v, Id mask, bool causal, bool hasScale, float scale) {
+ProgramBuilder::Id ProgramBuilder::sdpa(Id q, Id k, Id v, Id mask, bool causal, bool hasScale, float scale, std::int64_t slidingWindow,
+                                        Id sink) {
   Desc d = desc(q);
   d.storage = StorageType::Device;
   d.layout = TensorLayout::Tile;
   Id out = newTensor(d);
   using S = ScaledDotProductAttentionOp;
   Off qr = tensorRef(q), kr = tensorRef(k), vr = tensorRef(v), mr = mask ? tensorRef(mask) : 0, o = tensorRef(out);
+  Off sr = sink ? tensorRef(sink) : 0;
   b_.startTable(S::kNumFields);
   b_.addOffset(S::f_query, qr);
   b_.addOffset(S::f_key, kr);
@@ -409,6 +411,8 @@ ProgramBuilder::Id ProgramBuilder::sdpa(Id q, Id k, Id v, Id mask, bool causal, 
   b_.addScalarDefault<std::uint8_t>(S::f_is_causal, causal, 0);
   b_.addOffset(S::f_attention_mask, mr);
   if (hasScale) b_.addScalar<float>(S::f_scale, scale);
+  if (slidingWindow >= 0) b_.addScalar<std::uint32_t>(S::f_sliding_window_size, static_cast<std::uint32_t>(slidingWindow));
+  b_.addOffset(S::f_attention_sink, sr);
   b_.addOffset(S::f_out, o);
   addOp(OpType::ScaledDotProductAttentionOp, b_.endTable(), "ttnn.scaled_dot_product_attention " + shapeStr(d.shape));
   return out;
@@ -468,13 +472,14 @@ void ProgramBuilder::pagedFillCache(Id cache, Id in, Id pageTable, Id batchIdx) 
   if (batchIdx) b_.addOffset(S::f_batch_idx_tensor, bi);
   addOp(OpType::PagedFillCacheOp, b_.endTable(), "ttnn.paged_fill_cache");
 }
-ProgramBuilder::Id ProgramBuilder::sdpaDecode(Id q, Id k, Id v, Id pageTable, Id mask, Id curPos, bool causal, bool hasScale, float scale) {
+ProgramBuilder::Id ProgramBuilder::sdpaDecode(Id q, Id k, Id v, Id pageTable, Id mask, Id curPos, bool causal, bool hasScale, float scale,
+                                              std::int64_t slidingWindow, Id sink) {
   Desc d = desc(q);
   d.storage = StorageType::Device;
   d.layout = TensorLayout::Tile;
   Id out = newTensor(d);
   Off qr = tensorRef(q), kr = tensorRef(k), vr = tensorRef(v), pt = pageTable ? tensorRef(pageTable) : 0, mr = mask ? tensorRef(mask) : 0,
-      cp = curPos ? tensorRef(curPos) : 0, o = tensorRef(out);
+      cp = curPos ? tensorRef(curPos) : 0, o = tensorRef(out), sr = sink ? tensorRef(sink) : 0;
   if (pageTable) {
     using S = PagedScaledDotProductAttentionDecodeOp;
     b_.startTable(S::kNumFields);
@@ -482,6 +487,8 @@ ProgramBuilder::Id ProgramBuilder::sdpaDecode(Id q, Id k, Id v, Id pageTable, Id
     b_.addScalarDefault<std::uint8_t>(S::f_is_causal, causal, 0);
     b_.addOffset(S::f_attention_mask, mr); b_.addOffset(S::f_cur_pos_tensor, cp);
     if (hasScale) b_.addScalar<float>(S::f_scale, scale);
+    if (slidingWindow >= 0) b_.addScalar<std::uint32_t>(S::f_sliding_window_size, static_cast<std::uint32_t>(slidingWindow));
+    b_.addOffset(S::f_attention_sink, sr);
     b_.addOffset(S::f_out, o);
     addOp(OpType::PagedScaledDotProductAttentionDecodeOp, b_.endTable(), "ttnn.paged_scaled_dot_product_attention_decode " + shapeStr(d.shape));
   } else {
@@ -491,6 +498,8 @@ ProgramBuilder::Id ProgramBuilder::sdpaDecode(Id q, Id k, Id v, Id pageTable, Id
     b_.addScalarDefault<std::uint8_t>(S::f_is_causal, causal, 0);
     b_.addOffset(S::f_attention_mask, mr); b_.addOffset(S::f_cur_pos_tensor, cp);
     if (hasScale) b_.addScalar<float>(S::f_scale, scale);
+    if (slidingWindow >= 0) b_.addScalar<std::uint32_t>(S::f_sliding_window_size, static_cast<std::uint32_t>(slidingWindow));
+    b_.addOffset(S::f_attention_sink, sr);
     b_.addOffset(S::f_out, o);
     addOp(OpType::ScaledDotProductAttentionDecodeOp, b_.endTable(), "ttnn.scaled_dot_product_attention_decode " + shapeStr(d.shape));
   }

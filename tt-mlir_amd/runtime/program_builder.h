@@ -40,7 +40,7 @@ public:
   Id rmsNorm(Id in, Id weight, Id bias, float eps);
   Id softmax(Id in, int dim);
   Id reduction(std::uint32_t type, Id in, const std::vector<int> &dims, bool keepDim);
-  Id sdpa(Id q, Id k, Id v, Id mask, bool causal, bool hasScale, float scale);
+  Id sdpa(Id q, Id k, Id v, Id mask, bool causal, bool hasScale, float scale, std::int64_t slidingWindow = -1, Id sink = 0);
   Id reshape(Id in, const std::vector<std::uint32_t> &shape);
   Id permute(Id in, const std::vector<std::int64_t> &perm);
   Id transpose(Id in, int dim0, int dim1);
@@ -56,7 +56,8 @@ public:
   void pagedUpdateCache(Id cache, Id in, Id updateIndex, Id pageTable, bool shareCache);   // pageTable 0: static cache
   void pagedFillCache(Id cache, Id in, Id pageTable, Id batchIdx);                         // batchIdx 0: row b of the table
   // pageTable = 0 writes ScaledDotProductAttentionDecodeOp, otherwise the paged op
-  Id sdpaDecode(Id q, Id k, Id v, Id pageTable, Id mask, Id curPos, bool causal, bool hasScale, float scale);
+  Id sdpaDecode(Id q, Id k, Id v, Id pageTable, Id mask, Id curPos, bool causal, bool hasScale, float scale,
+                std::int64_t slidingWindow = -1, Id sink = 0);
   Id empty(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout);
   void copy(Id src, Id dst);                 // ttnn.copy: dst <- src, both on device
   void writeTensor(Id host, Id device);      // ttnn.write_tensor: device <- host
