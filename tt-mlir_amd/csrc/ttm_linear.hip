@@ -1343,7 +1343,15 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 
 // BFP4 = true reads bfp4_b tiles (576 bytes, two elements per byte, low nibble first): a lane's 4 (n) of a k row are one
 // 16-bit word, whose nibbles are spread into the bytes of a word before the same sign-magnitude -> offset-binary step.
-template <bool BFP4>
+//
+// TWO_TERM = true builds the bf16 operands with bit operations alone instead of int -> float conversions.  A weight is
+// +-mag x 2^(E - 133) (bfp8_b; mag x 2^(E - 129) for bfp4_b).  The bf16 number with the sign, exponent field E + 1 and
+// mantissa field mag (mag << 4 for bfp4_b) is V = +-(1 + mag / 128) x 2^(E - 126) = weight + S with S = +-2^(E - 126),
+// the same bits with a zero mantissa.  Both are made for two k rows at a time with a byte permute and three mask / shift /
+// or steps, V and S go through the matrix cores into two accumulators, and the result is their difference: twice the
+// MFMAs (which were idle) for less than half the vector instructions.  The two sums are each a few times larger than
+// their difference, so the fp32 rounding error grows by that factor - still four decimal orders below a bf16 result.
+template <bool BFP4, bool TWO_TERM>
 __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   extern __shared__ u32x4 smem[];   // partial sums: 8 wavefronts x 8 x 64 float4 = 64 KiB
   constexpr int D = 4;
@@ -1365,11 +1373,11 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   const uint32_t offE = nt_l * TB + (fr * 2 + fc) * 16 + half * 8;
   const uint32_t offA = fr * 512 + q16 * 32 + half * 16;                                     // + 1024 h
 
-  f32x4v acc[2][4];
+  f32x4v acc[2][4], accs[2][4];   // accs: the sum over the S terms (TWO_TERM)
 #pragma unroll
   for (int h = 0; h < 2; ++h)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[h][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 4; ++j) acc[h][j] = accs[h][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
 
   uint32_t rows[D][8], keeps[D];
   u32x2 ex[D];
@@ -1393,6 +1401,50 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
     for (int h = 0; h < 2; ++h) af[s][h] = *(const u32x4 *)(Ak + offA + h * 1024);
   };
   auto process = [&](int s) {
+    if constexpr (TWO_TERM) {
+      if (keeps[s] == 0u) return;   // wavefront-uniform: a k-tile past the end contributes nothing
+      // (E + 1) << 7 for the rows 2 ip and 2 ip + 1, in the two halves of a word; E is capped so that the field stays 8 bits
+      uint32_t epk[4];
+#pragma unroll
+      for (int ip = 0; ip < 4; ++ip) {
+        const uint32_t src = ip < 2 ? ex[s].x : ex[s].y;
+        uint32_t e2 = __builtin_amdgcn_perm(0u, src, (ip & 1) ? 0x0c030c02u : 0x0c010c00u);
+        typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+        const u16x2 capped = __builtin_elementwise_min(*(const u16x2 *)&e2, u16x2{0xFD, 0xFD});
+        e2 = *(const uint32_t *)&capped;
+        epk[ip] = (e2 + 0x00010001u) << 7;
+      }
+      uint32_t pr[4] = {0u, 0u, 0u, 0u};
+      if constexpr (BFP4) {
+#pragma unroll
+        for (int ip = 0; ip < 4; ++ip) pr[ip] = rows[s][2 * ip] | (rows[s][2 * ip + 1] << 16);   // four nibbles per row
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        u32x4 wv, ws;
+#pragma unroll
+        for (int ip = 0; ip < 4; ++ip) {
+          uint32_t sb, v;
+          if constexpr (BFP4) {
+            const uint32_t q = pr[ip] >> (4 * j);            // nibble j of either row in bits 0..3 and 16..19
+            sb = ((q & 0x00080008u) << 12) | epk[ip];
+            v = ((q & 0x00070007u) << 4) | sb;
+          } else {
+            const uint32_t q = __builtin_amdgcn_perm(rows[s][2 * ip + 1], rows[s][2 * ip], 0x0c040c00u + 0x00010001u * j);
+            sb = ((q & 0x00800080u) << 8) | epk[ip];
+            v = (q & 0x007F007Fu) | sb;
+          }
+          wv[ip] = v;
+          ws[ip] = sb;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&wv, *(bf16x8 *)&af[s][h], acc[h][j], 0, 0, 0);
+          accs[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&ws, *(bf16x8 *)&af[s][h], accs[h][j], 0, 0, 0);
+        }
+      }
+      return;
+    }
     float f[8][4];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -1436,6 +1488,12 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
     }
   }
 
+  if constexpr (TWO_TERM) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[h][j] -= accs[h][j];
+  }
   // partial sums -> LDS as float4 (four consecutive n of one m): slot ((wave * 8 + h * 4 + i) * 64 + lane)
   f32x4v *part = (f32x4v *)smem;
 #pragma unroll
@@ -1598,8 +1656,14 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       p.C = a.C + (int64_t)mt * a.Nt * 2048;
       for (int j = 0; j < a.group_n; ++j) p.gC[j] = a.gC[j] + (int64_t)mt * a.gNt[j] * 2048;
       const dim3 grid(column_units(a, 2), slices, (unsigned)batch);
-      if (decode && WF == WF_BFP4) hipLaunchKernelGGL(ttm_linear_decode_k<true>, grid, dim3(512), 65536, s, p);
-      else if (decode) hipLaunchKernelGGL(ttm_linear_decode_k<false>, grid, dim3(512), 65536, s, p);
+      const bool two_term = ttm_option("linear_decode_variant") != 1;   // 1 = operands by int -> float conversion
+      if (decode && WF == WF_BFP4) {
+        if (two_term) hipLaunchKernelGGL((ttm_linear_decode_k<true, true>), grid, dim3(512), 65536, s, p);
+        else hipLaunchKernelGGL((ttm_linear_decode_k<true, false>), grid, dim3(512), 65536, s, p);
+      } else if (decode) {
+        if (two_term) hipLaunchKernelGGL((ttm_linear_decode_k<false, true>), grid, dim3(512), 65536, s, p);
+        else hipLaunchKernelGGL((ttm_linear_decode_k<false, false>), grid, dim3(512), 65536, s, p);
+      }
       else hipLaunchKernelGGL((ttm_linear_small_k<WF>), dim3(a.Nt, 1, (unsigned)batch), dim3(256), 0, s, p);
       if (slices > 1)
         hipLaunchKernelGGL(ttm_linear_reduce_k, dim3((unsigned)((per / 4 + 255) / 256), 1, (unsigned)batch), dim3(256), 0, s, p, slices);
