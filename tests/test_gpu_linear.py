@@ -212,6 +212,37 @@ def test_decode_kernel_k_slices(hip, dev, orc, metrics, wfmt_name, split):
         check(orc, metrics, got[i], a[i], w_eff[i], b, "silu", max_abs=2.0 ** -5)
 
 
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4"])
+@pytest.mark.parametrize("M,K,N", [(32, 1024, 512), (7, 37 * 32 + 11, 5 * 32 + 7)])
+def test_decode_kernel_operand_constructions_agree(hip, dev, orc, metrics, wfmt_name, M, K, N):
+    """The decode kernel builds its bf16 weight operands either by int -> float conversion (linear_decode_variant 1) or
+    as two bit-built terms whose difference is the weight (default).  Weights with whole zero rows (exponent 0), rows of
+    x100 outliers (small magnitudes beside a large exponent) and both signs: each route against the oracle, and the two
+    against each other within one bf16 step of the result."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    a = datagen.randn((M, K), seed=46, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=47, std=0.05)
+    w[5:9] = 0.0
+    w[40:44, ::3] *= 100.0
+    w[:, 17] = 0.0
+    b = datagen.randn((N,), seed=48, std=0.5, dtype=torch.bfloat16)
+    res = {}
+    for variant in (1, 0):
+        hip.set_option("linear_decode_variant", variant)
+        try:
+            res[variant], w_eff = run_linear(hip, dev, a, w, b, None, wfmt)
+        finally:
+            hip.set_option("linear_decode_variant", 0)
+        check(orc, metrics, res[variant], a, w_eff, b, None, max_abs=2.0 ** -4)
+    x, y = res[0].float(), res[1].float()
+    # one bf16 step of the result, plus the fp32 accumulation error, which scales with the summands and not with the
+    # (possibly cancelling) sum: 2^-16 of sum |a| |w| is a loose bound for either route
+    summands = a.float().abs() @ w_eff.abs()
+    step = torch.maximum(x.abs(), y.abs()) * 2.0 ** -7 + summands * 2.0 ** -16 + 1e-6
+    assert torch.all((x - y).abs() <= step)
+    assert (x != y).float().mean().item() < 0.01
+
+
 def test_decode_kernel_splits_narrow_outputs_by_itself(hip, dev, orc, metrics):
     """[32, 4096] x bfp4_b [4096, 1024]: 16 column groups on a 256-CU device -> the launcher slices K."""
     a = datagen.randn((32, 4096), seed=44, dtype=torch.bfloat16)
