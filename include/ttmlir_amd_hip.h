@@ -210,13 +210,14 @@ int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void
 /* ttm_sdpa_heads_inner with the two remaining attributes of the op (include/ttmlir/Target/TTNN/operations/transformer.fbs:
  * 70-82; runtime/lib/ttnn/operations/transformer/scaled_dot_product_attention.cpp:33-45; golden tools/golden/mapping.py:
  * 8450-8494).  sliding_window >= 0: query i sees key j only when 0 <= i - j < sliding_window under is_causal, and when
- * |i - j| <= sliding_window / 2 otherwise; < 0: no window.  A mask, when given as well, is added on top.  Key tiles
+ * |i - j| <= sliding_window / 2 otherwise; < 0: no window.  A mask, when given as well, is added on top; it is
+ * [mask_batch, mask_heads, Sq, Sk] with mask_batch 1 (shared by the batch) or B (TTNNOps.td:4273-4275).  Key tiles
  * wholly outside the window are neither read nor multiplied.  attention_sink: [1, Hq, 1, 1] BFloat16 in TILE layout (one
  * tile per head) or null; per head one more logit, sink * scale, that takes part in the softmax and has no value row (the
  * kernel applies the scale to the sink as to the scores, which is what the compiler's lowering compensates for,
  * lib/Conversion/TTIRToTTNN/TTIRToTTNN.cpp:3507-3533).  A query that sees no key gives a row of zeros. */
-int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype,
-                      int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale,
+int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const void *mask, int mask_heads, int64_t mask_batch,
+                      void *out, int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale,
                       int heads_inner, int64_t sliding_window, const void *attention_sink, void *stream);
 
 /* ---- decode path: rotary embedding, KV-cache writes, attention of one new token over the cache.  TILE layout
@@ -286,12 +287,13 @@ int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, co
  * sliding_window >= 0: only the last sliding_window keys up to the decode position p are visible, keys
  * [max(0, p - sliding_window + 1), p] (golden tools/golden/mapping.py:8814-8824), p = cur_pos[b], or seq - 1 without
  * cur_pos; the cache in front of the window is not read.  attention_sink: [heads, 32] BFloat16 in TILE layout, column 0,
- * or null; one more logit per head, sink * scale, in the softmax, without a value row. */
+ * or null; one more logit per head, sink * scale, in the softmax, without a value row.  mask: [mask_batch, 1, mask_heads,
+ * seq] with mask_batch 1 (shared by the users) or batch (TTNNOps.td:4123-4125). */
 int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
-                             int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out,
-                             int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
-                             int is_causal, float scale, int concat_heads, int64_t sliding_window, const void *attention_sink,
-                             void *stream);
+                             int mask_heads, int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user,
+                             int64_t page_block, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
+                             int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
+                             const void *attention_sink, void *stream);
 
 /* Kernel-variant selection for measurement (name -> small integer); unknown names fail. */
 int ttm_set_option(const char *name, int value);

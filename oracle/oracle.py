@@ -294,6 +294,8 @@ def sdpa(q, k, v, mask=None, is_causal=False, scale=None, sliding_window=None, a
     if mask is not None:
         mask = _c(mask, np.float32)
         mh = mask.shape[1]
+        if mask.shape[0] == 1 and B > 1:               # one mask shared by the batch
+            mask = _c(np.broadcast_to(mask, (B,) + mask.shape[1:]))
     out = np.empty_like(q)
     sink = None if attention_sink is None else _c(attention_sink, np.float32).reshape(Hq)
     lib().orc_sdpa_f32(_p(q), _p(k), _p(v), _p(mask), mh, _p(out), B, Hq, Hkv, Sq, Sk, D, int(is_causal),
@@ -382,6 +384,8 @@ def sdpa_decode(q, k, v, cur_pos=None, mask=None, is_causal=True, scale=None, sl
     if mask is not None:
         mask = _c(mask, np.float32)
         mh = mask.shape[2]
+        if mask.shape[0] == 1 and B > 1:               # one mask shared by the users
+            mask = _c(np.broadcast_to(mask, (B,) + mask.shape[1:]))
     out = np.empty_like(q)
     sink = None
     if attention_sink is not None:

@@ -333,7 +333,7 @@ def test_sdpa_decode_sliding_window_and_attention_sink(hip, dev, orc, B, H, Hkv,
     cp = cur.to(dev)
     Bp = (B + 31) // 32 * 32
     out = torch.full((Bp * H * D,), float("nan"), dtype=torch.bfloat16, device=dev) if concat else torch.full_like(qt, float("nan"))
-    hip.call("ttm_sdpa_decode_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp) if use_pos else None, None, 1,
+    hip.call("ttm_sdpa_decode_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp) if use_pos else None, None, 1, 1,
              hip.ptr(table_d) if paged else None, pages, block, hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 1, 0.0, concat,
              -1 if window is None else window, hip.ptr(st) if sink else None, hip.current_stream())
     got = f32(untilize_dev(hip, out, (B, H * D), dev)).reshape(1, B, H, D) if concat else f32(untilize_dev(hip, out, q.shape, dev))
@@ -343,3 +343,24 @@ def test_sdpa_decode_sliding_window_and_attention_sink(hip, dev, orc, B, H, Hkv,
     if window is not None and window < S // 2 and not sink:
         plain = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur.numpy() if use_pos else None)
         assert np.max(np.abs(plain - want)) > 0.02           # the window matters for this case
+
+
+@pytest.mark.parametrize("mask_batch,mask_heads", [(1, 1), (1, 8), (3, 1), (3, 8)])
+def test_sdpa_decode_mask_shared_by_the_users(hip, dev, orc, mask_batch, mask_heads):
+    """The decode op's mask is [1|batch, 1, 1|heads, positions] (include/ttmlir/Dialect/TTNN/IR/TTNNOps.td:4123-4125):
+    every combination of shared and per-user, shared and per-head, with a window and a sink on top, against the oracle
+    on the broadcast mask."""
+    B, H, Hkv, S, D = 3, 8, 2, 256, 64
+    q = datagen.randn((1, B, H, D), seed=140, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, S, D), seed=141, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, S, D), seed=142, dtype=torch.bfloat16)
+    m = datagen.randn((mask_batch, 1, mask_heads, S), seed=143, dtype=torch.bfloat16) * 4
+    m[..., 200:] = float("-inf")
+    sk = (datagen.randn((H, 1), seed=144, dtype=torch.bfloat16) * 4).expand(H, 32).contiguous()
+    qt, kt, vt, mt, st = (tilize_dev(hip, t, dev) for t in (q, k, v, m, sk))
+    out = torch.full_like(qt, float("nan"))
+    hip.call("ttm_sdpa_decode_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, hip.ptr(mt), mask_heads, mask_batch, None, 0, 0,
+             hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 0, 0.0, 0, 100, hip.ptr(st), hip.current_stream())
+    got = f32(untilize_dev(hip, out, q.shape, dev))
+    want = orc.sdpa_decode(f32(q), f32(k), f32(v), mask=f32(m), is_causal=False, sliding_window=100, attention_sink=f32(sk))
+    assert np.all(np.isfinite(got)) and np.max(np.abs(got - want)) <= 2.0 ** -6

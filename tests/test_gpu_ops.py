@@ -366,7 +366,9 @@ def test_sdpa_heads_inner_equals_the_head_major_call(hip, dev, B, Hq, Hkv, Sq, S
     (1, 8, 2, 512, 512, 128, True, 129, True, None, 15), (1, 2, 2, 70, 70, 64, True, 1000, True, None, 0),
     (1, 2, 2, 128, 128, 128, True, None, True, None, 0), (2, 3, 3, 64, 100, 64, False, None, True, "bh", 0),
     (1, 1, 1, 100, 300, 256, False, 33, True, None, 0), (1, 4, 4, 640, 640, 64, True, 32, False, None, 9),
-    (1, 2, 2, 1024, 1024, 128, True, 200, True, None, 0)])
+    (1, 2, 2, 1024, 1024, 128, True, 200, True, None, 0),
+    # one mask shared by a batch of three, per head and for all heads
+    (3, 2, 2, 96, 128, 64, False, None, False, "1h", 0), (3, 4, 2, 64, 64, 128, False, 20, True, "11", 0)])
 def test_sdpa_sliding_window_and_attention_sink(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, window, sink, mask, flags, variant):
     """ttm_sdpa_windowed against the oracle: causal windows (one key, shorter and longer than a 64-key pass, longer than
     the sequence), symmetric windows, width 0, with and without the per-head sink, with a mask on top, ragged lengths,
@@ -377,7 +379,7 @@ def test_sdpa_sliding_window_and_attention_sink(hip, dev, orc, B, Hq, Hkv, Sq, S
     q = datagen.randn((B, Hq, Sq, D), seed=112, dtype=torch.bfloat16)
     k = datagen.randn((B, Hkv, Sk, D), seed=113, dtype=torch.bfloat16)
     v = datagen.randn((B, Hkv, Sk, D), seed=114, dtype=torch.bfloat16)
-    m = datagen.randn((B, 1 if mask == "b1" else Hq, Sq, Sk), seed=115, dtype=torch.bfloat16) if mask else None
+    m = datagen.randn((1 if mask[0] == "1" else B, 1 if mask[1] == "1" else Hq, Sq, Sk), seed=115, dtype=torch.bfloat16) if mask else None
     sk = (datagen.randn((1, Hq, 1, 1), seed=116, dtype=torch.bfloat16) * 8).contiguous() if sink else None
     inner = lambda t: t.permute(0, 2, 1, 3).reshape(t.shape[0], t.shape[2], t.shape[1] * t.shape[3]).contiguous()
     qt = tilize_dev(hip, inner(q) if flags & 1 else q, dev)
@@ -389,8 +391,8 @@ def test_sdpa_sliding_window_and_attention_sink(hip, dev, orc, B, Hq, Hkv, Sq, S
     hip.set_option("sdpa_variant", variant)
     try:
         hip.call("ttm_sdpa_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(mt) if mt is not None else None,
-                 m.shape[1] if m is not None else 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, Sq, Sk, D, int(causal), 0.0, flags,
-                 -1 if window is None else window, hip.ptr(st) if sink else None, hip.current_stream())
+                 m.shape[1] if m is not None else 1, m.shape[0] if m is not None else 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, Sq, Sk, D,
+                 int(causal), 0.0, flags, -1 if window is None else window, hip.ptr(st) if sink else None, hip.current_stream())
     finally:
         hip.set_option("sdpa_variant", 0)
     if flags & 8:
@@ -423,7 +425,7 @@ def test_sdpa_window_does_not_read_keys_outside_it(hip, dev, orc):
     kb[:, :, :hidden], vb[:, :, :hidden] = float("nan"), float("inf")
     qt, kt, vt = tilize_dev(hip, q, dev), tilize_dev(hip, kb, dev), tilize_dev(hip, vb, dev)
     out = torch.full_like(qt, float("nan"))
-    hip.call("ttm_sdpa_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, 1, hip.ptr(out), hip.BF16, B, H, H, S, S, D, 1, 0.0, 0,
+    hip.call("ttm_sdpa_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, 1, 1, hip.ptr(out), hip.BF16, B, H, H, S, S, D, 1, 0.0, 0,
              w, None, hip.current_stream())
     got = untilize_dev(hip, out, q.shape, dev).float().cpu().numpy()[:, :, first_q:]
     want = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), is_causal=True, sliding_window=w)[:, :, first_q:]

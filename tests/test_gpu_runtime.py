@@ -783,10 +783,12 @@ def test_attention_programs_with_sliding_window_and_sink(device, orc, metrics):
     kp = pb.input((users * pages, Hkv, bs, D), DT.BFloat16)
     vp = pb.input((users * pages, Hkv, bs, D), DT.BFloat16)
     table = pb.input((users, pages), DT.Int32, TL.RowMajor)
+    shared = pb.input((1, 1, S, S), DT.BFloat16)             # one mask for both batch entries and all heads
     pb.output(pb.sdpa(q, k, v, is_causal=True, sliding_window=W, attention_sink=sink))
     pb.output(pb.sdpa(q, k, v, is_causal=False, sliding_window=W))
     pb.output(pb.sdpa_decode(qd, kc, vc, cur_pos=pos, is_causal=True, sliding_window=W, attention_sink=sinkd))
     pb.output(pb.sdpa_decode(qd, kp, vp, cur_pos=pos, page_table=table, is_causal=True, sliding_window=W, attention_sink=sinkd))
+    pb.output(pb.sdpa(q, k, v, mask=shared, is_causal=False))
     pb.end_program()
     binary = rt.Binary.load_from_memory(pb.finish())
     g = torch.Generator().manual_seed(29)
@@ -801,7 +803,8 @@ def test_attention_programs_with_sliding_window_and_sink(device, orc, metrics):
         for p in range(pages):
             tkp[tbl[u, p]] = tkc[u, :, p * bs:(p + 1) * bs]
             tvp[tbl[u, p]] = tvc[u, :, p * bs:(p + 1) * bs]
-    tins = [tq, tk, tv, tsink, tqd, tkc, tvc, tpos, tsinkd, tkp, tvp, tbl]
+    tshared = bf(torch.randn((1, 1, S, S), generator=g) * 3)
+    tins = [tq, tk, tv, tsink, tqd, tkc, tvc, tpos, tsinkd, tkp, tvp, tbl, tshared]
     devs = [rt.to_layout(rt.from_torch(t.contiguous()), device, rt.get_layout(binary, 0, i)) for i, t in enumerate(tins)]
     outs = rt.submit(device, binary, 0, devs)
     got = [rt.to_torch(rt.to_host(y, untilize=True)[0]).float().numpy() for y in outs]
@@ -810,6 +813,7 @@ def test_attention_programs_with_sliding_window_and_sink(device, orc, metrics):
             orc.sdpa(f(tq), f(tk), f(tv), is_causal=False, sliding_window=W),
             orc.sdpa_decode(f(tqd), f(tkc), f(tvc), cur_pos=tpos.numpy(), sliding_window=W, attention_sink=f(tsinkd))]
     want.append(want[2])
+    want.append(orc.sdpa(f(tq), f(tk), f(tv), mask=f(tshared)))
     for w_, g_ in zip(want, got):
         assert np.max(np.abs(g_ - w_)) <= 2.0 ** -6
         assert metrics.get_pcc(w_, g_) >= 0.9999

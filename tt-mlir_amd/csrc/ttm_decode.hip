@@ -188,6 +188,7 @@ struct DecodeArgs {
   int B, H, Hkv, G, S, D, splits, keys_per_split, block, pages_per_user, mask_heads, is_causal;
   int concat_heads;   // out is [B, H * D] (row b holds user b's heads side by side) instead of [B, H, D]
   int Gt, g0;         // query heads per kv head in the tensors, and the first of them this launch serves (it serves G of them)
+  int mask_b;         // 1: one mask per user, 0: one mask shared by all
   int window;         // >= 0: only the last `window` keys up to the decode position are visible
   const uint16_t *sink;   // [H, 32] in tiles, column 0: one more logit per head (times scale) with a zero value row; or null
   float scale;
@@ -289,7 +290,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
             if (p.mask) {
               const int mh = p.mask_heads == 1 ? 0 : hrow + gq;
               const int64_t mrows = ttm_round_up32(p.mask_heads);
-              sv += ttm_bf16_to_f32(p.mask[(int64_t)b * mrows * p.S + ttm_tiled_offset(mh, k0 + kk, p.S >> 5)]);
+              sv += ttm_bf16_to_f32(p.mask[(int64_t)b * p.mask_b * mrows * p.S + ttm_tiled_offset(mh, k0 + kk, p.S >> 5)]);
             }
             sc[gq * p.keys_per_split + kk] = (k0 + kk < k1 && k0 + kk >= lo) ? sv * p.scale : -INFINITY;
           }
@@ -586,7 +587,7 @@ TTM_EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_
 static int sdpa_decode_entry(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
                              const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out, int dtype, int64_t batch,
                              int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads,
-                             int64_t window, const void *sink, void *stream) {
+                             int64_t window, const void *sink, int64_t mask_batch, void *stream) {
   TTM_REQUIRE(q && k && v && out, "ttm_sdpa_decode: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa_decode: tensors must be BFloat16");
   TTM_REQUIRE(batch > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "ttm_sdpa_decode: heads must be a multiple of kv heads");
@@ -617,6 +618,8 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
   p.Gt = (int)Gt;
   p.window = window < 0 ? -1 : (int)(window < seq ? window : seq);
   p.sink = (const uint16_t *)sink;
+  TTM_REQUIRE(!mask || mask_batch == 1 || mask_batch == batch, "ttm_sdpa_decode: mask batch must be 1 or %lld", (long long)batch);
+  p.mask_b = mask_batch == 1 ? 0 : 1;
   void *ws = nullptr;
   if (int rc = ttm_stream_workspace(s, (size_t)(batch * kv_heads * splits * G * (head_dim + 2)) * sizeof(float), &ws)) return rc;
   p.part = (float *)ws;
@@ -637,7 +640,7 @@ TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, cons
                                int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
                                int is_causal, float scale, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
-                           seq, head_dim, is_causal, scale, 0, -1, nullptr, stream);
+                           seq, head_dim, is_causal, scale, 0, -1, nullptr, batch, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
@@ -645,14 +648,14 @@ TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const 
                                             void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
                                             int64_t head_dim, int is_causal, float scale, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
-                           seq, head_dim, is_causal, scale, 1, -1, nullptr, stream);
+                           seq, head_dim, is_causal, scale, 1, -1, nullptr, batch, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
-                                        int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block,
-                                        void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
+                                        int mask_heads, int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user,
+                                        int64_t page_block, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
                                         int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                                         const void *attention_sink, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
-                           seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, stream);
+                           seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, stream);
 }

@@ -22,6 +22,7 @@ struct SdpaArgs {
   int B, Hq, Hkv, Sq, Sk;
   int sqt, skt;      // tiles along the sequence dims
   int mask_heads;    // 1 or Hq
+  int mask_b;        // 1: one mask per batch entry, 0: one mask shared by all
   // query i sees key j when i - lo_off <= j <= i + hi_off.  Causal: hi_off = 0; a sliding window of w keys: lo_off = w - 1
   // under a causal pass, lo_off = hi_off = w / 2 otherwise; kNoLimit where a side is open.
   int hi_off, lo_off;
@@ -156,7 +157,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
         const int key0 = kt * 32 + g * 8 + hh * 4;
         float mk[4] = {0.f, 0.f, 0.f, 0.f};
         if (p.mask) {
-          const int64_t mm = ((int64_t)b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
+          const int64_t mm = ((int64_t)b * p.mask_b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
           const int kin = g * 8 + hh * 4;
           const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
                               (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
@@ -350,7 +351,7 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
           float mk[4] = {0.f, 0.f, 0.f, 0.f};
           if (p.mask) {
             const int kt = min(2 * kb + half, p.skt - 1);
-            const int64_t mm = ((int64_t)b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
+            const int64_t mm = ((int64_t)b * p.mask_b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
             const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
                                 (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
             u32x2 raw = *(const u32x2 *)mp;
@@ -462,7 +463,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 static int sdpa_entry(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B,
                       int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int heads_inner, int64_t window,
-                      const void *sink, void *stream) {
+                      const void *sink, int64_t mask_batch, void *stream) {
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa: tensors must be BFloat16 (got %d)", dtype);
   TTM_REQUIRE(B >= 0 && Hq >= 0 && Hkv > 0 && Sq >= 0 && Sk >= 0 && D > 0, "ttm_sdpa: bad dimension");
   TTM_REQUIRE(Hq % Hkv == 0, "ttm_sdpa: query heads (%ld) must be a multiple of kv heads (%ld)", (long)Hq, (long)Hkv);
@@ -477,7 +478,8 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
   p.out = (uint8_t *)out;
   p.B = (int)B; p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.Sq = (int)Sq; p.Sk = (int)Sk;
   p.sqt = (int)ttm_cdiv(Sq, 32); p.skt = (int)ttm_cdiv(Sk, 32);
-  p.mask_heads = mask_heads;
+  TTM_REQUIRE(mask == nullptr || mask_batch == 1 || mask_batch == B, "ttm_sdpa: mask batch must be 1 or B");
+  p.mask_heads = mask_heads; p.mask_b = mask_batch == 1 ? 0 : 1;
   if (window >= kNoLimit) window = kNoLimit - 1;   // longer than any sequence: no different from that length
   p.hi_off = is_causal ? 0 : kNoLimit; p.lo_off = kNoLimit;
   if (window >= 0) {   // a causal window holds the last `window` keys, a symmetric one window / 2 keys on either side
@@ -516,19 +518,19 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
 TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
                         int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                         int is_causal, float scale, void *stream) {
-  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, 0, -1, nullptr, stream);
+  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, 0, -1, nullptr, B, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
                                     int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                                     int is_causal, float scale, int heads_inner, void *stream) {
-  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner, -1, nullptr, stream);
+  return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner, -1, nullptr, B, stream);
 }
 
-TTM_EXPORT int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
+TTM_EXPORT int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const void *mask, int mask_heads, int64_t mask_batch, void *out,
                                  int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                                  int is_causal, float scale, int heads_inner, int64_t sliding_window, const void *attention_sink,
                                  void *stream) {
   return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner,
-                    sliding_window < 0 ? -1 : sliding_window, attention_sink, stream);
+                    sliding_window < 0 ? -1 : sliding_window, attention_sink, mask_batch, stream);
 }

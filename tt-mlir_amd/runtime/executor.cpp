@@ -633,12 +633,14 @@ void runSdpa(const fb::Table &op, ProgramContext &ctx) {
   TTRT_ASSERT(ks == vs && qs[0] == ks[0] && qs[3] == ks[3], "sdpa: q/k/v shapes do not agree");
   Tensor mask;
   int maskHeads = 1;
+  std::int64_t maskBatch = 1;
   if (auto mr = op.table(S::f_attention_mask)) {
     mask = as(ctx, ctx.get(mr, "sdpa mask"), TensorLayout::Tile, DataType::BFloat16);
     const auto &ms = mask.handle->shape;
-    TTRT_ASSERT(ms.size() == 4 && ms[0] == qs[0] && ms[2] == qs[2] && ms[3] == ks[2] && (ms[1] == 1 || ms[1] == qs[1]),
-                "sdpa: mask must be [B, 1|Hq, Sq, Sk]");
+    TTRT_ASSERT(ms.size() == 4 && (ms[0] == 1 || ms[0] == qs[0]) && ms[2] == qs[2] && ms[3] == ks[2] && (ms[1] == 1 || ms[1] == qs[1]),
+                "sdpa: mask must be [1|B, 1|Hq, Sq, Sk]");
     maskHeads = static_cast<int>(ms[1]);
+    maskBatch = ms[0];
   }
   bool causal = op.scalar<std::uint8_t>(S::f_is_causal, 0) != 0;
   TTRT_ASSERT(!(causal && mask), "sdpa: is_causal and an explicit mask are mutually exclusive");
@@ -683,7 +685,7 @@ void runSdpa(const fb::Table &op, ProgramContext &ctx) {
   Tensor out = makeDeviceTensor(ctx.dev, mergedRef ? shapeFromTensorRef(mergedRef) : qs, DataType::BFloat16, TensorLayout::Tile);
   if (inner) debug::Stats::get().incrementStat("SdpaHeadsInner");
   TTM_CALL(ttm_sdpa_windowed(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(), mask ? mask.handle->data.get() : nullptr,
-                             maskHeads, out.handle->data.get(), TTM_BF16, qs[0], qs[1], ks[1], qs[2], ks[2], qs[3], causal ? 1 : 0, scale,
+                             maskHeads, maskBatch, out.handle->data.get(), TTM_BF16, qs[0], qs[1], ks[1], qs[2], ks[2], qs[3], causal ? 1 : 0, scale,
                              inner, window, sink ? sink.handle->data.get() : nullptr, ctx.stream()));
   if (mergedRef) {
     ctx.put(mergedRef, out);
@@ -883,6 +885,7 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
   }
   Tensor mask, pos, sink;
   int maskHeads = 1;
+  std::int64_t maskBatch = 1;
   if (sinkRef) {
     sink = as(ctx, ctx.get(sinkRef, "sdpa_decode attention sink"), TensorLayout::Tile, DataType::BFloat16);
     const auto &ss = sink.handle->shape;
@@ -892,9 +895,10 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
   if (maskRef) {
     mask = as(ctx, ctx.get(maskRef, "sdpa_decode mask"), TensorLayout::Tile, DataType::BFloat16);
     const auto &ms = mask.handle->shape;
-    TTRT_ASSERT(ms.size() == 4 && ms[0] == B && ms[1] == 1 && (ms[2] == 1 || ms[2] == H) && ms[3] == S,
-                "sdpa_decode: mask must be [batch, 1, 1|heads, positions]");
+    TTRT_ASSERT(ms.size() == 4 && (ms[0] == 1 || ms[0] == B) && ms[1] == 1 && (ms[2] == 1 || ms[2] == H) && ms[3] == S,
+                "sdpa_decode: mask must be [1|batch, 1, 1|heads, positions]");
     maskHeads = static_cast<int>(ms[2]);
+    maskBatch = ms[0];
   }
   if (posRef) {
     pos = devicePositions(ctx, ctx.get(posRef, "sdpa_decode cur_pos"), "sdpa_decode: cur_pos_tensor");
@@ -911,7 +915,7 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
       debug::Stats::get().incrementStat("FusedHeadConcat");
       TTM_CALL(ttm_sdpa_decode_windowed(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
                                         pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
-                                        mask ? mask.handle->data.get() : nullptr, maskHeads,
+                                        mask ? mask.handle->data.get() : nullptr, maskHeads, maskBatch,
                                         table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
                                         merged.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, 1, window, sinkPtr,
                                         ctx.stream()));
@@ -923,7 +927,7 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
   Tensor out = makeDeviceTensor(ctx.dev, qs, DataType::BFloat16, TensorLayout::Tile);
   TTM_CALL(ttm_sdpa_decode_windowed(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
                                     pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
-                                    mask ? mask.handle->data.get() : nullptr, maskHeads,
+                                    mask ? mask.handle->data.get() : nullptr, maskHeads, maskBatch,
                                     table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
                                     out.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, 0, window, sinkPtr,
                                     ctx.stream()));
