@@ -148,6 +148,28 @@ int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int layout, 
                       int64_t cols, float param, void *stream);
 int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape,
                        void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream);
+/* ttm_eltwise_binary also takes 100 + EltwiseBinaryCompositeOpType for Maximum, Minimum, Remainder, Pow and Atan2
+ * (runtime/lib/ttnn/operations/eltwise/binary/binary_composite.cpp; goldens tools/golden/mapping.py:4493-4570, 5516-5530:
+ * torch.maximum / minimum (NaN propagates), torch.remainder (sign of the divisor), torch.pow, torch.atan2).
+ *
+ * ttm_where: ::ttnn::where(first, second, third) (runtime/lib/ttnn/operations/eltwise/ternary/where.cpp:14-33; golden
+ * tools/golden/mapping.py:5579-5586, torch.where): out = cond != 0 ? a : b, the three operands broadcasting numpy-style
+ * to the output (rank <= 4), all four tensors in `dtype` (BFloat16 or Float32) and `layout`.  Values move as bits. */
+int ttm_where(const void *cond, const int64_t *cond_shape, const void *a, const int64_t *a_shape, const void *b,
+              const int64_t *b_shape, void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream);
+
+/* ---- index-driven ops of a decoder layer's head and tail, ROW_MAJOR on both sides.
+ * ttm_embedding: ::ttnn::embedding (runtime/lib/ttnn/operations/embedding/embedding.cpp:14-43; golden
+ *   tools/golden/mapping.py:2900-2912): out[r, :] = weight[clamp(indices[r], 0, vocab - 1), :]; indices Int32 / UInt32,
+ *   weight [vocab, dim] and out [rows, dim] of `elem_bytes`-byte elements.
+ * ttm_argmax: ::ttnn::argmax over the last dim (operations/reduction/argmax.cpp:14-28; golden mapping.py:5222-5265,
+ *   torch.argmax): out[r] = index of the first largest element of row r of in [rows, cols] (NaN counts as largest).
+ * ttm_arange: ::ttnn::arange (operations/creation/arange.cpp:14-42; golden mapping.py:4269-4290): out[i] = start + i * step
+ *   formed in fp32 and cast to `dtype` (Float32, BFloat16, Int32, UInt32), n = ceil((end - start) / step) elements. */
+int ttm_embedding(const void *indices, int index_dtype, const void *weight, void *out, int elem_bytes, int64_t rows,
+                  int64_t vocab, int64_t dim, void *stream);
+int ttm_argmax(const void *in, int dtype, int32_t *out, int64_t rows, int64_t cols, void *stream);
+int ttm_arange(void *out, int dtype, int64_t n, double start, double step, void *stream);
 
 /* ---- typecast between plain dtypes: ::ttnn::typecast
  * (runtime/lib/ttnn/operations/layout/typecast.cpp:14-31).  Layout is preserved, so n counts the

@@ -163,6 +163,14 @@ int ttrt_pb_concat(ttrt_builder *pb, const uint32_t *ins, int n, int dim, uint32
 int ttrt_pb_slice(ttrt_builder *pb, uint32_t in, const int64_t *begins, const int64_t *ends, const int64_t *steps, int rank,
                   uint32_t *out);
 int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_t repeats, int dim, uint32_t *out);
+/* RepeatOp, EltwiseBinaryCompositeOp (type = EltwiseBinaryCompositeOpType), EltwiseTernaryWhereOp, EmbeddingOp,
+ * ReductionArgMaxOp (has_dim = 0: over the whole tensor), ArangeOp */
+int ttrt_pb_repeat(ttrt_builder *pb, uint32_t in, const int64_t *repeats, int rank, uint32_t *out);
+int ttrt_pb_binary_composite(ttrt_builder *pb, uint32_t type, uint32_t lhs, uint32_t rhs, uint32_t *out);
+int ttrt_pb_where(ttrt_builder *pb, uint32_t cond, uint32_t a, uint32_t b, uint32_t *out);
+int ttrt_pb_embedding(ttrt_builder *pb, uint32_t indices, uint32_t weight, uint32_t *out);
+int ttrt_pb_argmax(ttrt_builder *pb, uint32_t in, int has_dim, int dim, int keep_dim, int out_dtype, uint32_t *out);
+int ttrt_pb_arange(ttrt_builder *pb, float start, float end, float step, int dtype, int layout, uint32_t *out);
 int ttrt_pb_constant(ttrt_builder *pb, const void *data, size_t bytes, int in_dtype, const uint32_t *shape, int rank,
                      const ttrt_layout *layout, uint32_t *out);
 int ttrt_pb_full(ttrt_builder *pb, const uint32_t *shape, int rank, float value, int dtype, int layout, uint32_t *out);

@@ -394,3 +394,48 @@ def sdpa_decode(q, k, v, cur_pos=None, mask=None, is_causal=True, scale=None, sl
     lib().orc_sdpa_decode_f32(_p(q), _p(k), _p(v), _p(cp), _p(mask), mh, _p(out), B, H, Hkv, S, D, int(is_causal),
                               float(scale) if scale else 0.0, -1 if sliding_window is None else int(sliding_window), _p(sink))
     return out
+
+
+# ---- the ops around a decoder layer (embedding in front, argmax behind, mask construction beside it).  Each is the
+# library routine the reference's golden calls, on numpy arrays: nothing here has arithmetic of its own to get wrong
+# except the index conventions, which tests/test_oracle_math.py checks against torch.
+def where(cond, a, b):
+    """tools/golden/mapping.py:5579-5586 (torch.where); cond != 0 selects a."""
+    return np.where(np.asarray(cond) != 0, a, b)
+
+
+def embedding(indices, weight):
+    """tools/golden/mapping.py:2900-2912: rows of the [.., vocab, dim] table, indices clamped to [0, vocab - 1]."""
+    w = np.asarray(weight)
+    w = w.reshape(w.shape[-2], w.shape[-1])
+    idx = np.clip(np.asarray(indices).astype(np.int64), 0, w.shape[0] - 1)
+    return w[idx]
+
+
+def argmax(x, dim=None, keep_dim=False):
+    """tools/golden/mapping.py:5222-5265 (torch.argmax): first index of the largest element, over `dim` or the whole tensor."""
+    x = np.asarray(x)
+    if dim is None:
+        r = np.argmax(x.reshape(-1))
+        return np.full((1,) * x.ndim if keep_dim else (), r, dtype=np.int32)
+    r = np.argmax(x, axis=dim).astype(np.int32)
+    return np.expand_dims(r, dim) if keep_dim else r
+
+
+def arange(start, end, step=1, dtype=np.float32):
+    """tools/golden/mapping.py:4269-4290: torch.arange in float32, then the cast."""
+    return np.arange(start, end, step, dtype=np.float32).astype(dtype)
+
+
+def repeat(x, repeats):
+    """tools/golden/mapping.py:4259-4266 (Tensor.repeat = numpy tile with one count per dimension)."""
+    return np.tile(np.asarray(x), tuple(int(r) for r in repeats))
+
+
+def binary_composite(name, a, b):
+    """maximum / minimum / remainder / pow / atan2 as the goldens take them from torch (tools/golden/mapping.py:4493-4570,
+    5516-5530): NaN propagates through maximum and minimum, remainder has the sign of the divisor."""
+    a, b = np.asarray(a, np.float32), np.asarray(b, np.float32)
+    with np.errstate(all="ignore"):
+        return {"maximum": np.maximum, "minimum": np.minimum, "remainder": np.mod, "pow": np.power,
+                "atan2": np.arctan2}[name](a, b).astype(np.float32)

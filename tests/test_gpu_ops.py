@@ -430,3 +430,122 @@ def test_sdpa_window_does_not_read_keys_outside_it(hip, dev, orc):
     got = untilize_dev(hip, out, q.shape, dev).float().cpu().numpy()[:, :, first_q:]
     want = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), is_causal=True, sliding_window=w)[:, :, first_q:]
     assert np.all(np.isfinite(got)) and np.max(np.abs(got - want)) <= 2.0 ** -6
+
+
+def _i64(v):
+    return np.array(v, dtype=np.int64)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("tiled", [False, True])
+@pytest.mark.parametrize("cs,as_,bs", [((3, 40, 70), (3, 40, 70), (3, 40, 70)), ((1, 40, 1), (3, 40, 70), (1, 1, 70)),
+                                       ((2, 3, 1, 33), (1, 3, 35, 33), (1,)), ((64, 64), (64, 64), (1, 1))])
+def test_where_bit_exact(hip, dev, orc, dtype, tiled, cs, as_, bs):
+    """ttm_where against the oracle: same-shape and broadcasting operands (condition, either value, a scalar), ragged
+    tiles whose padding must stay zero, both layouts and dtypes; NaN and -0.0 in the condition; the values move as bits."""
+    rank = max(len(cs), len(as_), len(bs))
+    pad = lambda s: (1,) * (rank - len(s)) + tuple(s)
+    os_ = tuple(max(x) for x in zip(pad(cs), pad(as_), pad(bs)))
+    c = (datagen.randn(pad(cs), seed=150, dtype=dtype) > 0).to(dtype)
+    c.view(-1)[0], c.view(-1)[1] = float("nan"), -0.0
+    a = datagen.randn(pad(as_), seed=151, dtype=dtype)
+    b = datagen.randn(pad(bs), seed=152, dtype=dtype)
+    a.view(-1)[0] = float("inf")
+    code, lay = (hip.BF16 if dtype == torch.bfloat16 else hip.F32), (hip.TILE if tiled else hip.ROW_MAJOR)
+    put = (lambda t: tilize_dev(hip, t, dev)) if tiled else (lambda t: t.contiguous().to(dev))
+    ct, at, bt = put(c), put(a), put(b)
+    n = int(np.prod(os_[:-2], dtype=np.int64)) * ((os_[-2] + 31) // 32 * 32) * ((os_[-1] + 31) // 32 * 32) if tiled else int(np.prod(os_))
+    out = torch.full((n,), float("nan"), dtype=dtype, device=dev)
+    shapes = [_i64(pad(cs)), _i64(pad(as_)), _i64(pad(bs)), _i64(os_)]           # kept alive across the call
+    hip.call("ttm_where", hip.ptr(ct), shapes[0].ctypes.data, hip.ptr(at), shapes[1].ctypes.data, hip.ptr(bt),
+             shapes[2].ctypes.data, hip.ptr(out), shapes[3].ctypes.data, rank, code, lay, hip.current_stream())
+    got = untilize_dev(hip, out, os_, dev).cpu() if tiled else out.reshape(os_).cpu()
+    torch.cuda.synchronize()
+    want = orc.where(c.float().numpy(), a.float().numpy(), b.float().numpy())
+    assert np.array_equal(got.float().numpy(), np.broadcast_to(want, os_), equal_nan=True)
+    if tiled:
+        back = tilize_dev(hip, got, dev)
+        assert torch.equal(back.view(torch.int16 if dtype == torch.bfloat16 else torch.int32), out.view(torch.int16 if dtype == torch.bfloat16 else torch.int32))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,vocab,dim,unsigned", [(64, 1000, 4096, False), (7, 33, 24, True), (300, 50, 5, False), (1, 1, 8, False)])
+def test_embedding_bit_exact(hip, dev, orc, dtype, rows, vocab, dim, unsigned):
+    """ttm_embedding against the oracle: wide and narrow rows (16-byte and element-wise paths), indices below 0 and past the
+    table (clamped, tools/golden/mapping.py:2910-2911), UInt32 indices."""
+    g = torch.Generator().manual_seed(160)
+    w = datagen.randn((vocab, dim), seed=161, dtype=dtype)
+    idx = torch.randint(0, vocab, (rows,), generator=g, dtype=torch.int32)
+    if rows > 3:
+        idx[1] = vocab + 5
+        if not unsigned:
+            idx[2] = -3
+    wd, idd = w.to(dev), idx.to(dev)
+    out = torch.full((rows, dim), float("nan"), dtype=dtype, device=dev)
+    hip.call("ttm_embedding", hip.ptr(idd), hip.U32 if unsigned else hip.I32, hip.ptr(wd), hip.ptr(out), w.element_size(), rows, vocab, dim,
+             hip.current_stream())
+    torch.cuda.synchronize()
+    want = orc.embedding(idx.numpy(), w.float().numpy())
+    assert np.array_equal(out.float().cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rows,cols", [(32, 128256), (5, 63), (1, 1), (9, 64), (130, 1000)])
+def test_argmax_first_largest(hip, dev, orc, dtype, rows, cols):
+    """ttm_argmax against the oracle: a vocabulary-sized row, fewer columns than lanes, ties (bf16 rows of 128 256 random
+    values have many; the first index wins), a NaN (counts as largest), -inf rows."""
+    x = datagen.randn((rows, cols), seed=170, dtype=dtype)
+    if cols > 40:
+        x[0, 7] = x[0, 33] = 50.0
+        if rows > 1:
+            x[1, 20] = float("nan")
+        if rows > 2:
+            x[2, :] = float("-inf")
+    xd = x.to(dev)
+    out = torch.full((rows,), -1, dtype=torch.int32, device=dev)
+    hip.call("ttm_argmax", hip.ptr(xd), hip.BF16 if dtype == torch.bfloat16 else hip.F32, hip.ptr(out), rows, cols, hip.current_stream())
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), orc.argmax(x.float().numpy(), -1))
+    assert np.array_equal(out.cpu().numpy(), torch.argmax(x.float(), dim=-1).numpy())
+
+
+@pytest.mark.parametrize("start,end,step", [(0, 2048, 1), (3, 40, 4), (5, -5, -2), (0, 1, 0.125), (0, 70000, 7)])
+def test_arange_all_dtypes(hip, dev, orc, start, end, step):
+    n = int(np.ceil((end - start) / step))
+    for code, tdt, ndt in ((hip.F32, torch.float32, np.float32), (hip.BF16, torch.bfloat16, None), (hip.I32, torch.int32, np.int32),
+                           (hip.U32, torch.int32, np.uint32)):
+        if code == hip.U32 and (start < 0 or end < 0):
+            continue
+        out = torch.zeros((n,), dtype=tdt, device=dev)
+        hip.call("ttm_arange", hip.ptr(out), code, n, float(start), float(step), hip.current_stream())
+        torch.cuda.synchronize()
+        want = torch.arange(start, end, step, dtype=torch.float32)
+        if ndt is None:
+            assert torch.equal(out.cpu(), want.to(torch.bfloat16))
+        else:
+            assert np.array_equal(out.cpu().numpy().view(ndt), orc.arange(start, end, step, ndt))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("name,code", [("maximum", 100), ("minimum", 101), ("remainder", 102), ("pow", 103), ("atan2", 104)])
+def test_binary_composites(hip, dev, orc, dtype, name, code):
+    """Maximum / Minimum / Remainder / Pow / Atan2 through ttm_eltwise_binary (op = 100 + EltwiseBinaryCompositeOpType),
+    broadcasting a row against a matrix in tiles: max / min / remainder exact after the store rounding, pow and atan2 within
+    2 ulp of fp32 before it."""
+    a = datagen.randn((70, 96), seed=180, dtype=dtype) * 3
+    b = datagen.randn((1, 96), seed=181, dtype=dtype) * 2
+    if name == "pow":
+        a = a.abs() + 0.1
+    a[0, 0] = float("nan")
+    at, bt = tilize_dev(hip, a, dev), tilize_dev(hip, b, dev)
+    out = torch.full_like(at, float("nan"))
+    sa, sb = _i64([70, 96]), _i64([1, 96])                                       # kept alive across the call
+    hip.call("ttm_eltwise_binary", code, hip.ptr(at), sa.ctypes.data, hip.ptr(bt), sb.ctypes.data, hip.ptr(out),
+             sa.ctypes.data, 2, hip.BF16 if dtype == torch.bfloat16 else hip.F32, hip.TILE, hip.current_stream())
+    got = untilize_dev(hip, out, (70, 96), dev).cpu()
+    torch.cuda.synchronize()
+    want = torch.from_numpy(orc.binary_composite(name, a.float().numpy(), b.float().numpy())).to(dtype)
+    if name in ("maximum", "minimum", "remainder"):
+        assert np.array_equal(got.float().numpy(), want.float().numpy(), equal_nan=True)
+    else:
+        assert torch.allclose(got.float(), want.float(), rtol=2.0 ** -7 if dtype == torch.bfloat16 else 1e-5, atol=1e-6, equal_nan=True)

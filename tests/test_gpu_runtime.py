@@ -819,3 +819,52 @@ def test_attention_programs_with_sliding_window_and_sink(device, orc, metrics):
         assert metrics.get_pcc(w_, g_) >= 0.9999
     plain = orc.sdpa_decode(f(tqd), f(tkc), f(tvc), cur_pos=tpos.numpy())
     assert np.max(np.abs(plain - want[2])) > 0.02
+
+
+def test_decoder_head_and_tail_ops_program(device, orc, metrics):
+    """The ops a lowered Llama layer carries around its attention and MLP (test/ttmlir/models/single_blocks_and_layers/
+    llama_3_8b_decode_layer.mlir: embedding, arange, comparisons, where, broadcast as repeat, maximum, argmax), submitted as
+    one program: token ids -> embedding rows; a causal mask built from two aranges, a comparison and a where; a row repeated
+    over the batch; logits -> argmax over the vocabulary, with and without a kept dimension and over a middle dimension."""
+    B, S, V, D = 2, 48, 300, 64
+    pb = rt.ProgramBuilder()
+    pb.begin_program("head_tail")
+    ids = pb.input((B, S), DT.Int32, TL.RowMajor)
+    table = pb.input((V, D), DT.BFloat16, TL.RowMajor)
+    logits = pb.input((B, S, V), DT.BFloat16)
+    row = pb.input((1, 1, D), DT.BFloat16)
+    emb = pb.embedding(ids, table)
+    pb.output(emb)
+    qpos = pb.reshape(pb.arange(0, S, 1, DT.Int32), (S, 1))
+    kpos = pb.reshape(pb.arange(0, S, 1, DT.Int32), (1, S))
+    visible = pb.binary(programs.BINARY["le"], kpos, qpos)                      # key position <= query position
+    zero, minus = pb.full((1, 1), 0.0, DT.BFloat16), pb.full((1, 1), -1e9, DT.BFloat16)
+    pb.output(pb.where(pb.typecast(visible, DT.BFloat16), zero, minus))
+    pb.output(pb.repeat(row, (B, S, 1)))
+    pb.output(pb.binary_composite(programs.BINARY_COMPOSITE["maximum"], emb, row))
+    pb.output(pb.argmax(logits, dim=-1))
+    pb.output(pb.argmax(logits, dim=-1, keep_dim=True, out_dtype=DT.UInt32))
+    pb.output(pb.argmax(logits, dim=1))
+    pb.output(pb.argmax(logits))
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    g = torch.Generator().manual_seed(31)
+    tids = torch.randint(0, V, (B, S), generator=g, dtype=torch.int32)
+    tids[0, 0], tids[1, 5] = V + 7, -2                                          # clamped
+    ttable, tlogits, trow = bf(torch.randn((V, D), generator=g)), bf(torch.randn((B, S, V), generator=g)), bf(torch.randn((1, 1, D), generator=g))
+    tlogits[0, 3, 10] = tlogits[0, 3, 200] = 30.0                               # a tie: the first index wins
+    tins = [tids, ttable, tlogits, trow]
+    devs = [rt.to_layout(rt.from_torch(t.contiguous()), device, rt.get_layout(binary, 0, i)) for i, t in enumerate(tins)]
+    outs = rt.submit(device, binary, 0, devs)
+    got = [rt.to_torch(rt.to_host(y, untilize=True)[0]) for y in outs]
+    f = lambda t: t.float().numpy()
+    want_emb = orc.embedding(tids.numpy(), f(ttable))
+    assert np.array_equal(f(got[0]), want_emb)
+    i, j = np.arange(S)[:, None], np.arange(S)[None, :]
+    assert np.array_equal(f(got[1]), np.where(j <= i, 0.0, f(bf(torch.tensor(-1e9)))).astype(np.float32))
+    assert np.array_equal(f(got[2]), orc.repeat(f(trow), (B, S, 1)))
+    assert np.array_equal(f(got[3]), orc.binary_composite("maximum", want_emb, f(trow)))
+    assert np.array_equal(got[4].numpy(), orc.argmax(f(tlogits), -1)) and got[4].dtype == torch.int32
+    assert np.array_equal(got[5].numpy().astype(np.int64), orc.argmax(f(tlogits), -1, True).astype(np.int64)) and tuple(got[5].shape) == (B, S, 1)
+    assert np.array_equal(got[6].numpy(), orc.argmax(f(tlogits), 1))
+    assert int(got[7].reshape(-1)[0]) == int(orc.argmax(f(tlogits)))

@@ -363,3 +363,37 @@ def test_sdpa_decode_window_and_sink(orc):
     # the decode sink agrees with the prefill oracle's (one query row, everything visible)
     full = orc.sdpa(np.ascontiguousarray(qt.numpy()), k, v, attention_sink=sink[:, 0])
     assert np.allclose(orc.sdpa_decode(q, k, v, is_causal=False, attention_sink=sink)[0], full[:, :, 0], rtol=1e-5, atol=1e-6)
+
+
+def test_index_and_select_ops_against_torch(orc):
+    """where / embedding / argmax / arange / repeat / maximum, minimum, remainder, pow, atan2: the oracle's numpy calls
+    against the torch calls the reference's goldens make (tools/golden/mapping.py:2900-2912, 4259-4290, 4493-4570,
+    5222-5265, 5516-5530, 5579-5586), including what differs between the libraries' conventions: ties and NaN in
+    argmax, clamped indices, remainder's sign, NaN through maximum."""
+    g = torch.Generator().manual_seed(50)
+    c = (torch.rand((3, 1, 5), generator=g) > 0.5).float()
+    a, b = torch.randn((3, 4, 5), generator=g), torch.randn((1, 4, 1), generator=g)
+    assert np.array_equal(orc.where(c.numpy(), a.numpy(), b.numpy()), torch.where(c != 0, a, b).numpy())
+    assert np.array_equal(orc.where(np.array([-0.0, 0.0, np.nan, 2.0]), np.ones(4), np.zeros(4)), np.array([0.0, 0.0, 1.0, 1.0]))
+    w = torch.randn((1, 1, 11, 6), generator=g)
+    idx = torch.tensor([[0, 10, 3], [25, -4, 7]])
+    want = F.embedding(idx.clamp(0, 10), w.reshape(11, 6))
+    assert np.array_equal(orc.embedding(idx.numpy(), w.numpy()), want.numpy())
+    x = torch.randn((2, 3, 7), generator=g)
+    x[0, 1, 2] = x[0, 1, 5] = 9.0                               # tie: the first index wins
+    x[1, 2, 4] = float("nan")                                   # NaN counts as the largest value
+    for dim in (0, 1, 2, -1):
+        for keep in (False, True):
+            assert np.array_equal(orc.argmax(x.numpy(), dim, keep), torch.argmax(x, dim=dim, keepdim=keep).numpy())
+    assert int(orc.argmax(x.numpy())) == int(torch.argmax(x))
+    assert orc.argmax(x.numpy(), keep_dim=True).shape == (1, 1, 1)
+    for start, end, step in ((0, 10, 1), (3, 40, 4), (5, -5, -2), (0, 1, 0.125)):
+        assert np.array_equal(orc.arange(start, end, step), torch.arange(start, end, step, dtype=torch.float32).numpy())
+    assert np.array_equal(orc.arange(0, 300, 1, np.int32), torch.arange(0, 300, 1, dtype=torch.float32).to(torch.int32).numpy())
+    assert np.array_equal(orc.repeat(a.numpy(), (2, 1, 3)), a.repeat(2, 1, 3).numpy())
+    p, q = torch.randn((4, 6), generator=g) * 3, torch.randn((1, 6), generator=g) * 2
+    p[0, 0] = float("nan")
+    for name, fn in (("maximum", torch.maximum), ("minimum", torch.minimum), ("remainder", torch.remainder), ("atan2", torch.atan2)):
+        assert np.allclose(orc.binary_composite(name, p.numpy(), q.numpy()), fn(p, q.expand(4, 6)).numpy(), rtol=1e-6, atol=1e-6, equal_nan=True), name
+    assert np.allclose(orc.binary_composite("pow", p.abs().numpy(), q.numpy()), torch.pow(p.abs(), q).numpy(), rtol=1e-5, equal_nan=True)
+    assert orc.binary_composite("remainder", np.float32(-7), np.float32(3)) == 2.0 and orc.binary_composite("remainder", np.float32(7), np.float32(-3)) == -2.0

@@ -4,6 +4,8 @@
 // 16 bytes per lane; broadcasting binaries decode tile coordinates per element.
 #include <hip/hip_fp16.h>
 
+#include <type_traits>
+
 #include "ttm_common.h"
 #include "ttm_math.h"
 
@@ -12,7 +14,9 @@ enum { U_ABS = 0, U_CEIL, U_COS, U_FLOOR, U_GELU, U_ISFINITE, U_LOGICALNOT, U_NE
        U_RSQRT, U_SIGMOID, U_SIN, U_RECIPROCAL, U_SIGN, U_TAN, U_TANH, U_ATAN, U_EXP, U_ERF, U_ERFC,
        U_LOG, U_EXPM1, U_LEAKYRELU, U_BITWISENOT, U_RELU6, U_SILU };
 enum { B_ADD = 0, B_MUL = 1, B_SUB = 3, B_EQ = 4, B_NE = 5, B_GE = 6, B_GT = 7, B_LE = 8, B_LT = 9, B_DIV = 10,
-       B_AND = 11, B_OR = 12, B_XOR = 13 };
+       B_AND = 11, B_OR = 12, B_XOR = 13,
+       // 100 + EltwiseBinaryCompositeOpType
+       B_MAXIMUM = 100, B_MINIMUM = 101, B_REMAINDER = 102, B_POW = 103, B_ATAN2 = 104 };
 
 template <int OP>
 __device__ __forceinline__ float unary_op(float x, float p) {
@@ -62,6 +66,14 @@ __device__ __forceinline__ float binary_op(int op, float a, float b) {
   case B_AND: return (a != 0.0f && b != 0.0f) ? 1.0f : 0.0f;
   case B_OR: return (a != 0.0f || b != 0.0f) ? 1.0f : 0.0f;
   case B_XOR: return ((a != 0.0f) != (b != 0.0f)) ? 1.0f : 0.0f;
+  case B_MAXIMUM: return (a != a || b != b) ? NAN : fmaxf(a, b);   // NaN propagates, as in torch.maximum
+  case B_MINIMUM: return (a != a || b != b) ? NAN : fminf(a, b);
+  case B_REMAINDER: {   // sign of the divisor, as torch.remainder
+    const float r = fmodf(a, b);
+    return (r != 0.0f && ((r < 0.0f) != (b < 0.0f))) ? r + b : r;
+  }
+  case B_POW: return powf(a, b);
+  case B_ATAN2: return atan2f(a, b);
   default: return a;
   }
 }
@@ -260,7 +272,7 @@ TTM_EXPORT int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape,
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_eltwise_binary: dtype must be BFloat16 or Float32 (got %d)", dtype);
   TTM_REQUIRE(layout == TTM_ROW_MAJOR || layout == TTM_TILE, "ttm_eltwise_binary: bad layout");
   TTM_REQUIRE(rank >= 0 && rank <= 8 && a_shape && b_shape && out_shape, "ttm_eltwise_binary: bad rank or null shape");
-  TTM_REQUIRE((op >= B_ADD && op <= B_XOR) && op != 2, "ttm_eltwise_binary: unsupported op %d", op);
+  TTM_REQUIRE(((op >= B_ADD && op <= B_XOR) && op != 2) || (op >= B_MAXIMUM && op <= B_ATAN2), "ttm_eltwise_binary: unsupported op %d", op);
   // right-align to rank 4: leading dims beyond the last three are folded into d0 when both operands
   // agree with the output there (no broadcasting across them)
   BcastArgs p;
@@ -307,6 +319,71 @@ TTM_EXPORT int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape,
     else
       hipLaunchKernelGGL(ttm_binary_bcast_k<false>, dim3(grid_for(total)), dim3(256), 0, s, op, a, b, out, p, total);
   }
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+// ---- where(cond, a, b): cond != 0 selects a; the three operands broadcast to the output like the binaries
+struct WhereArgs {
+  int64_t oshape[4], cshape[4], ashape[4], bshape[4];
+  int tiled;
+};
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void ttm_where_k(const void *__restrict__ cond, const void *__restrict__ a, const void *__restrict__ b,
+                                                   void *__restrict__ out, WhereArgs p, int64_t total) {
+  const int64_t R = p.oshape[2], C = p.oshape[3];
+  const int64_t pr = p.tiled ? (R + 31) / 32 * 32 : R, pc = p.tiled ? (C + 31) / 32 * 32 : C;
+  typedef typename std::conditional<BF16, uint16_t, uint32_t>::type T;   // values move as bits: no rounding, NaN payloads kept
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+    int64_t batch = i / (pr * pc), w = i % (pr * pc), r, c;
+    if (p.tiled) {
+      int64_t tile = w >> 10;
+      int e = (int)(w & 1023);
+      int face = e >> 8;
+      r = (tile / (pc / 32)) * 32 + (face >> 1) * 16 + ((e >> 4) & 15);
+      c = (tile % (pc / 32)) * 32 + (face & 1) * 16 + (e & 15);
+    } else {
+      r = w / pc; c = w % pc;
+    }
+    T y = 0;
+    if (r < R && c < C) {
+      const int64_t i0 = batch / p.oshape[1], i1 = batch % p.oshape[1];
+      const T cv = ((const T *)cond)[bcast_offset(p.cshape, i0, i1, r, c, p.tiled)];
+      const bool take = BF16 ? (cv & 0x7FFFu) != 0 : (cv & 0x7FFFFFFFu) != 0;   // +-0 is false, NaN is true
+      y = take ? ((const T *)a)[bcast_offset(p.ashape, i0, i1, r, c, p.tiled)] : ((const T *)b)[bcast_offset(p.bshape, i0, i1, r, c, p.tiled)];
+    }
+    ((T *)out)[i] = y;
+  }
+}
+
+TTM_EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a, const int64_t *a_shape, const void *b,
+                         const int64_t *b_shape, void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream) {
+  TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_where: dtype must be BFloat16 or Float32 (got %d)", dtype);
+  TTM_REQUIRE(layout == TTM_ROW_MAJOR || layout == TTM_TILE, "ttm_where: bad layout");
+  TTM_REQUIRE(rank >= 0 && rank <= 4 && cond_shape && a_shape && b_shape && out_shape, "ttm_where: rank must be at most 4, shapes non-null");
+  WhereArgs p;
+  int64_t *shapes[4] = {p.oshape, p.cshape, p.ashape, p.bshape};
+  const int64_t *src[4] = {out_shape, cond_shape, a_shape, b_shape};
+  for (int t = 0; t < 4; ++t) {
+    for (int d = 0; d < 4; ++d) shapes[t][d] = 1;
+    for (int d = 0; d < rank; ++d) {
+      const int64_t v = src[t][rank - 1 - d];
+      TTM_REQUIRE(v >= 0, "ttm_where: negative dimension");
+      shapes[t][3 - d] = v;
+      TTM_REQUIRE(t == 0 || v == out_shape[rank - 1 - d] || v == 1, "ttm_where: shapes do not broadcast at dim %d", rank - 1 - d);
+    }
+  }
+  p.tiled = layout == TTM_TILE;
+  const int64_t R = p.oshape[2], C = p.oshape[3];
+  const int64_t pr = p.tiled ? ttm_round_up32(R) : R, pc = p.tiled ? ttm_round_up32(C) : C;
+  const int64_t total = p.oshape[0] * p.oshape[1] * pr * pc;
+  if (total == 0) return TTM_OK;
+  TTM_REQUIRE(cond && a && b && out, "ttm_where: null pointer");
+  if (dtype == TTM_BF16)
+    hipLaunchKernelGGL(ttm_where_k<true>, dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream, cond, a, b, out, p, total);
+  else
+    hipLaunchKernelGGL(ttm_where_k<false>, dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream, cond, a, b, out, p, total);
   TTM_LAUNCH_CHECK();
   return TTM_OK;
 }

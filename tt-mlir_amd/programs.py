@@ -18,6 +18,7 @@ UNARY = dict(abs=0, ceil=1, cos=2, floor=3, gelu=4, isfinite=5, logical_not=6, n
              expm1=22, leaky_relu=23, relu6=25, silu=26)
 BINARY = dict(add=0, multiply=1, subtract=3, eq=4, ne=5, ge=6, gt=7, le=8, lt=9, divide=10)
 REDUCE = dict(sum=0, mean=1, max=2, min=3)
+BINARY_COMPOSITE = dict(maximum=0, minimum=1, remainder=2, pow=3, atan2=4)
 
 
 def _consteval_pack(pb, name, shapes_dtypes):

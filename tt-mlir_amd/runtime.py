@@ -600,6 +600,27 @@ class ProgramBuilder:
     def repeat_interleave(self, t, repeats, dim):
         return self._op("ttrt_pb_repeat_interleave", t, repeats, dim)
 
+    def repeat(self, t, repeats):
+        r = (ctypes.c_int64 * len(repeats))(*repeats)
+        return self._op("ttrt_pb_repeat", t, r, len(repeats))
+
+    def binary_composite(self, type_, lhs, rhs):
+        return self._op("ttrt_pb_binary_composite", type_, lhs, rhs)
+
+    def where(self, cond, a, b):
+        return self._op("ttrt_pb_where", cond, a, b)
+
+    def embedding(self, indices, weight):
+        return self._op("ttrt_pb_embedding", indices, weight)
+
+    def argmax(self, t, dim=None, keep_dim=False, out_dtype=None):
+        return self._op("ttrt_pb_argmax", t, int(dim is not None), dim or 0, int(keep_dim),
+                        int(DataType.Int32 if out_dtype is None else out_dtype))
+
+    def arange(self, start, end, step=1, dtype=None, layout=None):
+        return self._op("ttrt_pb_arange", ctypes.c_float(start), ctypes.c_float(end), ctypes.c_float(step),
+                        int(DataType.Float32 if dtype is None else dtype), int(TensorLayout.RowMajor if layout is None else layout))
+
     def constant(self, array, in_dtype, dtype=None, layout=TensorLayout.Tile, storage=StorageType.Device):
         a = np.ascontiguousarray(array)
         s, r = _shape_arg(a.shape)

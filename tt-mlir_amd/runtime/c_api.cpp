@@ -440,6 +440,20 @@ TTRT_EXPORT int ttrt_pb_slice(ttrt_builder *pb, uint32_t in, const int64_t *begi
 TTRT_EXPORT int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_t repeats, int dim, uint32_t *out) {
   PB_OP(repeatInterleave(in, repeats, dim));
 }
+TTRT_EXPORT int ttrt_pb_repeat(ttrt_builder *pb, uint32_t in, const int64_t *repeats, int rank, uint32_t *out) {
+  PB_OP(repeat(in, std::vector<std::int64_t>(repeats, repeats + rank)));
+}
+TTRT_EXPORT int ttrt_pb_binary_composite(ttrt_builder *pb, uint32_t type, uint32_t lhs, uint32_t rhs, uint32_t *out) {
+  PB_OP(binaryComposite(type, lhs, rhs));
+}
+TTRT_EXPORT int ttrt_pb_where(ttrt_builder *pb, uint32_t cond, uint32_t a, uint32_t b, uint32_t *out) { PB_OP(where(cond, a, b)); }
+TTRT_EXPORT int ttrt_pb_embedding(ttrt_builder *pb, uint32_t indices, uint32_t weight, uint32_t *out) { PB_OP(embedding(indices, weight)); }
+TTRT_EXPORT int ttrt_pb_argmax(ttrt_builder *pb, uint32_t in, int has_dim, int dim, int keep_dim, int out_dtype, uint32_t *out) {
+  PB_OP(argmax(in, has_dim != 0, dim, keep_dim != 0, static_cast<DataType>(out_dtype)));
+}
+TTRT_EXPORT int ttrt_pb_arange(ttrt_builder *pb, float start, float end, float step, int dtype, int layout, uint32_t *out) {
+  PB_OP(arange(start, end, step, static_cast<DataType>(dtype), static_cast<TensorLayout>(layout)));
+}
 TTRT_EXPORT int ttrt_pb_constant(ttrt_builder *pb, const void *data, size_t bytes, int in_dtype, const uint32_t *shape, int rank,
                                  const ttrt_layout *layout, uint32_t *out) {
   return guard([&] {

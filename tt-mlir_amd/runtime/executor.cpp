@@ -104,6 +104,7 @@ OpRefs opRefs(const fb::Table &operation) {
   case OpType::ScaledDotProductAttentionOp:
     in(schema::ScaledDotProductAttentionOp::f_query); in(schema::ScaledDotProductAttentionOp::f_key);
     in(schema::ScaledDotProductAttentionOp::f_value); in(schema::ScaledDotProductAttentionOp::f_attention_mask);
+    in(schema::ScaledDotProductAttentionOp::f_attention_sink);
     out(schema::ScaledDotProductAttentionOp::f_out);
     break;
   case OpType::ReshapeOp: in(schema::ReshapeOp::f_in); out(schema::ReshapeOp::f_out); break;
@@ -112,6 +113,17 @@ OpRefs opRefs(const fb::Table &operation) {
   case OpType::ConcatOp: inVec(schema::ConcatOp::f_inputs); out(schema::ConcatOp::f_out); break;
   case OpType::SliceOp: in(schema::SliceOp::f_in); out(schema::SliceOp::f_out); break;
   case OpType::RepeatInterleaveOp: in(schema::RepeatInterleaveOp::f_input); out(schema::RepeatInterleaveOp::f_out); break;
+  case OpType::RepeatOp: in(schema::RepeatOp::f_in); out(schema::RepeatOp::f_out); break;
+  case OpType::EltwiseBinaryCompositeOp:
+    in(schema::EltwiseBinaryCompositeOp::f_lhs); in(schema::EltwiseBinaryCompositeOp::f_rhs); out(schema::EltwiseBinaryCompositeOp::f_out);
+    break;
+  case OpType::EltwiseTernaryWhereOp:
+    in(schema::EltwiseTernaryWhereOp::f_first); in(schema::EltwiseTernaryWhereOp::f_second); in(schema::EltwiseTernaryWhereOp::f_third);
+    out(schema::EltwiseTernaryWhereOp::f_out);
+    break;
+  case OpType::EmbeddingOp: in(schema::EmbeddingOp::f_input); in(schema::EmbeddingOp::f_weight); out(schema::EmbeddingOp::f_out); break;
+  case OpType::ReductionArgMaxOp: in(schema::ReductionArgMaxOp::f_in); out(schema::ReductionArgMaxOp::f_out); break;
+  case OpType::ArangeOp: out(schema::ArangeOp::f_out); break;
   case OpType::ConstantOp: out(schema::ConstantOp::f_out); break;
   case OpType::FullOp: out(schema::FullOp::f_out); break;
   case OpType::NamedFullOp: out(schema::NamedFullOp::f_out); break;
@@ -139,12 +151,12 @@ OpRefs opRefs(const fb::Table &operation) {
   }
   case OpType::ScaledDotProductAttentionDecodeOp: {
     using S = schema::ScaledDotProductAttentionDecodeOp;
-    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
+    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_attention_mask); in(S::f_cur_pos_tensor); in(S::f_attention_sink); out(S::f_out);
     break;
   }
   case OpType::PagedScaledDotProductAttentionDecodeOp: {
     using S = schema::PagedScaledDotProductAttentionDecodeOp;
-    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_page_table); in(S::f_attention_mask); in(S::f_cur_pos_tensor); out(S::f_out);
+    in(S::f_query); in(S::f_key); in(S::f_value); in(S::f_page_table); in(S::f_attention_mask); in(S::f_cur_pos_tensor); in(S::f_attention_sink); out(S::f_out);
     break;
   }
   case OpType::CaptureOrExecuteTraceOp:
@@ -473,11 +485,18 @@ void runEltwiseUnary(const fb::Table &op, ProgramContext &ctx) {
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 
-void runEltwiseBinary(const fb::Table &op, ProgramContext &ctx) {
-  Tensor l0 = ctx.get(op.table(schema::EltwiseBinaryOp::f_lhs), "binary lhs"), r0 = ctx.get(op.table(schema::EltwiseBinaryOp::f_rhs), "binary rhs");
-  auto outRef = op.table(schema::EltwiseBinaryOp::f_out);
+// the type element-wise ops with several operands compute in: fp32 as soon as an operand or the result is Float32 or a
+// 32-bit integer (positions and token ids compared against each other must stay exact; bf16 holds 8 bits), bf16 otherwise
+DataType computeDtypeOf(std::initializer_list<DataType> types) {
+  for (DataType t : types)
+    if (t == DataType::Float32 || t == DataType::Int32 || t == DataType::UInt32) return DataType::Float32;
+  return DataType::BFloat16;
+}
+
+void binaryImpl(ProgramContext &ctx, const fb::Table &lhsRef, const fb::Table &rhsRef, const fb::Table &outRef, int code) {
+  Tensor l0 = ctx.get(lhsRef, "binary lhs"), r0 = ctx.get(rhsRef, "binary rhs");
   Layout want = layoutFromTensorRef(outRef);
-  DataType dt = computeDtype(want.dataType);
+  DataType dt = computeDtypeOf({want.dataType, l0.handle->dtype, r0.handle->dtype});
   TensorLayout lay = want.storageType == StorageType::Device ? want.layout : onDevice(ctx, l0).handle->layout;
   Tensor l = as(ctx, l0, lay, dt), r = as(ctx, r0, lay, dt);
   std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
@@ -490,9 +509,45 @@ void runEltwiseBinary(const fb::Table &op, ProgramContext &ctx) {
   TTRT_ASSERT(l.handle->shape.size() <= rank && r.handle->shape.size() <= rank, "binary: operand rank exceeds the output rank");
   auto ls = pad(l.handle->shape), rs = pad(r.handle->shape), os = pad(oshape);
   Tensor out = makeDeviceTensor(ctx.dev, oshape, dt, lay);
-  std::uint32_t type = op.scalar<std::uint32_t>(schema::EltwiseBinaryOp::f_type, 0);
-  TTM_CALL(ttm_eltwise_binary(static_cast<int>(type), l.handle->data.get(), ls.data(), r.handle->data.get(), rs.data(),
+  TTM_CALL(ttm_eltwise_binary(code, l.handle->data.get(), ls.data(), r.handle->data.get(), rs.data(),
                               out.handle->data.get(), os.data(), static_cast<int>(rank), ttmDtype(dt), ttmLayout(lay), ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+void runEltwiseBinary(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::EltwiseBinaryOp;
+  binaryImpl(ctx, op.table(S::f_lhs), op.table(S::f_rhs), op.table(S::f_out), static_cast<int>(op.scalar<std::uint32_t>(S::f_type, 0)));
+}
+// runtime/lib/ttnn/operations/eltwise/binary/binary_composite.cpp: maximum, minimum, remainder, pow, atan2 (the bitwise and
+// shift members work on integers and have no kernel here)
+void runEltwiseBinaryComposite(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::EltwiseBinaryCompositeOp;
+  const std::uint32_t type = op.scalar<std::uint32_t>(S::f_type, 0);
+  TTRT_ASSERT(type <= 4, "binary composite: bitwise and shift ops are not supported");
+  binaryImpl(ctx, op.table(S::f_lhs), op.table(S::f_rhs), op.table(S::f_out), 100 + static_cast<int>(type));
+}
+// runtime/lib/ttnn/operations/eltwise/ternary/where.cpp:14-33
+void runWhere(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::EltwiseTernaryWhereOp;
+  Tensor c0 = ctx.get(op.table(S::f_first), "where condition"), a0 = ctx.get(op.table(S::f_second), "where true value"),
+         b0 = ctx.get(op.table(S::f_third), "where false value");
+  auto outRef = op.table(S::f_out);
+  Layout want = layoutFromTensorRef(outRef);
+  const DataType dt = computeDtypeOf({want.dataType, c0.handle->dtype, a0.handle->dtype, b0.handle->dtype});
+  const TensorLayout lay = want.storageType == StorageType::Device ? want.layout : onDevice(ctx, a0).handle->layout;
+  Tensor c = as(ctx, c0, lay, dt), a = as(ctx, a0, lay, dt), b = as(ctx, b0, lay, dt);
+  const std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
+  const size_t rank = std::max<size_t>(1, oshape.size());
+  TTRT_ASSERT(rank <= 4 && c.handle->shape.size() <= rank && a.handle->shape.size() <= rank && b.handle->shape.size() <= rank,
+              "where: ranks above 4, or an operand of higher rank than the result, are not supported");
+  auto pad = [&](const std::vector<std::uint32_t> &s) {
+    std::vector<std::int64_t> o(rank, 1);
+    for (size_t i = 0; i < s.size(); ++i) o[rank - s.size() + i] = s[i];
+    return o;
+  };
+  auto cs = pad(c.handle->shape), as_ = pad(a.handle->shape), bs = pad(b.handle->shape), os = pad(oshape);
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, dt, lay);
+  TTM_CALL(ttm_where(c.handle->data.get(), cs.data(), a.handle->data.get(), as_.data(), b.handle->data.get(), bs.data(),
+                     out.handle->data.get(), os.data(), static_cast<int>(rank), ttmDtype(dt), ttmLayout(lay), ctx.stream()));
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 
@@ -1229,7 +1284,99 @@ void runRepeatInterleave(const fb::Table &op, ProgramContext &ctx) {
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 
+// runtime/lib/ttnn/operations/data_movement/repeat.cpp:12-22: the input tiled repeat_dims[i] times along dim i
+void runRepeat(const fb::Table &op, ProgramContext &ctx) {
+  Tensor in = onDevice(ctx, ctx.get(op.table(schema::RepeatOp::f_in), "repeat in"));
+  const auto &shape = in.handle->shape;
+  const int rank = static_cast<int>(shape.size());
+  auto reps = op.scalars<std::int64_t>(schema::RepeatOp::f_repeat_dims);
+  TTRT_ASSERT(static_cast<int>(reps.size()) == rank, "repeat: one repeat count per dimension expected");
+  std::vector<std::uint32_t> oshape = shape;
+  for (int i = 0; i < rank; ++i) {
+    TTRT_ASSERT(reps[i] >= 1, "repeat: counts must be positive");
+    oshape[i] = static_cast<std::uint32_t>(shape[i] * reps[i]);
+  }
+  // view [.., rep_i, shape_i, ..]: the rep axes have source stride 0
+  std::vector<std::int64_t> extent, sst, dstv;
+  auto ss = rowMajorStrides(shape), os = rowMajorStrides(oshape);
+  for (int i = 0; i < rank; ++i) {
+    if (reps[i] > 1) { extent.push_back(reps[i]); sst.push_back(0); dstv.push_back(os[i] * shape[i]); }
+    extent.push_back(shape[i]); sst.push_back(ss[i]); dstv.push_back(os[i]);
+  }
+  TTRT_ASSERT(extent.size() <= 8, "repeat: more than 8 view dimensions");
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, in.handle->dtype, in.handle->layout);
+  zeroIfPadded(ctx, out);
+  copyView(ctx, in, out, extent, sst, 0, dstv, 0);
+  auto outRef = op.table(schema::RepeatOp::f_out);
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// runtime/lib/ttnn/operations/embedding/embedding.cpp:14-43: rows of the table picked by index
+void runEmbedding(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::EmbeddingOp;
+  Tensor idx0 = ctx.get(op.table(S::f_input), "embedding indices");
+  const DataType it = idx0.handle->dtype == DataType::UInt32 ? DataType::UInt32 : DataType::Int32;
+  Tensor idx = as(ctx, idx0, TensorLayout::RowMajor, it);
+  Tensor w0 = onDevice(ctx, ctx.get(op.table(S::f_weight), "embedding weight"));
+  TTRT_ASSERT(!utils::isBlockFormatDataType(w0.handle->dtype), "embedding: block-float tables are not supported");
+  const DataType wt = w0.handle->dtype == DataType::Float32 ? DataType::Float32 : DataType::BFloat16;
+  Tensor w = as(ctx, w0, TensorLayout::RowMajor, wt);
+  const auto &ws = w.handle->shape;
+  TTRT_ASSERT(ws.size() >= 2 && volume(ws) == static_cast<std::int64_t>(ws[ws.size() - 2]) * ws.back(),
+              "embedding: the table must be [.., vocab, dim] with leading ones");
+  auto outRef = op.table(S::f_out);
+  const std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
+  const std::int64_t rows = volume(idx.handle->shape), vocab = ws[ws.size() - 2], dim = ws.back();
+  TTRT_ASSERT(!oshape.empty() && oshape.back() == dim && volume(oshape) == rows * dim, "embedding: output shape must be indices x dim");
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, wt, TensorLayout::RowMajor);
+  TTM_CALL(ttm_embedding(idx.handle->data.get(), ttmDtype(it), w.handle->data.get(), out.handle->data.get(),
+                         static_cast<int>(utils::dataTypeElementSize(wt)), rows, vocab, dim, ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// runtime/lib/ttnn/operations/reduction/argmax.cpp:14-28: index of the largest element along `dim`, or of the whole tensor
+void runArgMax(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::ReductionArgMaxOp;
+  Tensor x0 = onDevice(ctx, ctx.get(op.table(S::f_in), "argmax in"));
+  const DataType dt = computeDtypeOf({x0.handle->dtype});
+  Tensor x = as(ctx, x0, x0.handle->layout, dt);
+  const int rank = static_cast<int>(x.handle->shape.size());
+  std::int64_t rows = 1, cols = volume(x.handle->shape);
+  if (op.has(S::f_dim) && rank > 0) {
+    int dim = op.scalar<std::int32_t>(S::f_dim, 0);
+    if (dim < 0) dim += rank;
+    TTRT_ASSERT(dim >= 0 && dim < rank, "argmax: dimension out of range");
+    if (dim != rank - 1) x = moveDimLast(ctx, x, dim, false, x.handle->shape);
+    cols = x.handle->shape.back();
+    rows = volume(x.handle->shape) / std::max<std::int64_t>(cols, 1);
+  }
+  TTRT_ASSERT(cols > 0, "argmax: empty reduction");
+  x = as(ctx, x, TensorLayout::RowMajor, dt);
+  auto outRef = op.table(S::f_out);
+  const std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
+  TTRT_ASSERT(volume(oshape) == rows, "argmax: output shape does not match");
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, DataType::Int32, TensorLayout::RowMajor);
+  TTM_CALL(ttm_argmax(x.handle->data.get(), ttmDtype(dt), static_cast<std::int32_t *>(out.handle->data.get()), rows, cols, ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
 // ---- creation (runtime/lib/ttnn/operations/creation/*.cpp)
+// arange.cpp:14-42: start, start + step, ... below end
+void runArange(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::ArangeOp;
+  const double start = op.scalar<float>(S::f_start, 0.0f), end = op.scalar<float>(S::f_end, 0.0f), step = op.scalar<float>(S::f_step, 0.0f);
+  TTRT_ASSERT(step != 0.0, "arange: step must not be zero");
+  auto outRef = op.table(S::f_out);
+  const std::vector<std::uint32_t> oshape = shapeFromTensorRef(outRef);
+  const std::int64_t n = std::max<std::int64_t>(0, static_cast<std::int64_t>(std::ceil((end - start) / step)));
+  TTRT_ASSERT(volume(oshape) == n, "arange: output holds " + std::to_string(volume(oshape)) + " elements, the range " + std::to_string(n));
+  Layout want = layoutFromTensorRef(outRef);
+  DataType dt = want.dataType;
+  if (dt != DataType::Float32 && dt != DataType::BFloat16 && dt != DataType::Int32 && dt != DataType::UInt32) dt = DataType::Float32;
+  Tensor out = makeDeviceTensor(ctx.dev, oshape, dt, TensorLayout::RowMajor);
+  TTM_CALL(ttm_arange(out.handle->data.get(), ttmDtype(dt), n, start, step, ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
 void runConstant(const fb::Table &op, ProgramContext &ctx) {
   auto outRef = op.table(schema::ConstantOp::f_out);
   auto bytes = op.scalars<std::uint8_t>(schema::ConstantOp::f_input);
@@ -1476,6 +1623,12 @@ void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   case OpType::ConcatOp: return runConcat(op, ctx);
   case OpType::SliceOp: return runSlice(op, ctx);
   case OpType::RepeatInterleaveOp: return runRepeatInterleave(op, ctx);
+  case OpType::RepeatOp: return runRepeat(op, ctx);
+  case OpType::EltwiseBinaryCompositeOp: return runEltwiseBinaryComposite(op, ctx);
+  case OpType::EltwiseTernaryWhereOp: return runWhere(op, ctx);
+  case OpType::EmbeddingOp: return runEmbedding(op, ctx);
+  case OpType::ReductionArgMaxOp: return runArgMax(op, ctx);
+  case OpType::ArangeOp: return runArange(op, ctx);
   case OpType::ConstantOp: return runConstant(op, ctx);
   case OpType::FullOp: return runFull(op, ctx);
   case OpType::NamedFullOp: return runNamedFull(op, ctx);

@@ -1,5 +1,6 @@
 #include "program_builder.h"
 
+#include <cmath>
 #include <algorithm>
 
 namespace ttmlir_amd {
@@ -602,6 +603,112 @@ ProgramBuilder::Id ProgramBuilder::repeatInterleave(Id in, std::uint32_t repeats
   b_.addScalarDefault<std::uint32_t>(RepeatInterleaveOp::f_repeats, repeats, 0);
   b_.addScalarDefault<std::int32_t>(RepeatInterleaveOp::f_dim, dim, 0);
   addOp(OpType::RepeatInterleaveOp, b_.endTable(), "ttnn.repeat_interleave x" + std::to_string(repeats));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::repeat(Id in, const std::vector<std::int64_t> &repeats) {
+  Desc d = desc(in);
+  if (repeats.size() != d.shape.size()) fatal("ProgramBuilder: repeat needs one count per dimension");
+  for (size_t i = 0; i < repeats.size(); ++i) d.shape[i] = static_cast<std::uint32_t>(d.shape[i] * repeats[i]);
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out), r = b_.createScalarVector(repeats);
+  b_.startTable(RepeatOp::kNumFields);
+  b_.addOffset(RepeatOp::f_in, i);
+  b_.addOffset(RepeatOp::f_out, o);
+  b_.addOffset(RepeatOp::f_repeat_dims, r);
+  addOp(OpType::RepeatOp, b_.endTable(), "ttnn.repeat -> " + shapeStr(d.shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::binaryComposite(std::uint32_t type, Id lhs, Id rhs) {
+  const auto &a = desc(lhs).shape, &b = desc(rhs).shape;
+  size_t rank = std::max(a.size(), b.size());
+  std::vector<std::uint32_t> shape(rank);
+  for (size_t i = 0; i < rank; ++i) {
+    std::uint32_t x = i < rank - a.size() ? 1 : a[i - (rank - a.size())], y = i < rank - b.size() ? 1 : b[i - (rank - b.size())];
+    if (x != y && x != 1 && y != 1) fatal("ProgramBuilder: binary operands do not broadcast");
+    shape[i] = std::max(x, y);
+  }
+  Id out = newTensor(Desc{shape, desc(lhs).dtype, desc(lhs).layout, StorageType::Device});
+  Off l = tensorRef(lhs), r = tensorRef(rhs), o = tensorRef(out);
+  b_.startTable(EltwiseBinaryCompositeOp::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(EltwiseBinaryCompositeOp::f_type, type, 0);
+  b_.addOffset(EltwiseBinaryCompositeOp::f_lhs, l);
+  b_.addOffset(EltwiseBinaryCompositeOp::f_rhs, r);
+  b_.addOffset(EltwiseBinaryCompositeOp::f_out, o);
+  addOp(OpType::EltwiseBinaryCompositeOp, b_.endTable(), "ttnn.binary_composite#" + std::to_string(type));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::where(Id cond, Id a, Id b) {
+  const auto &cs = desc(cond).shape, &as = desc(a).shape, &bs = desc(b).shape;
+  size_t rank = std::max({cs.size(), as.size(), bs.size()});
+  std::vector<std::uint32_t> shape(rank, 1);
+  for (const auto *s : {&cs, &as, &bs})
+    for (size_t i = 0; i < s->size(); ++i) {
+      std::uint32_t &o = shape[rank - s->size() + i], v = (*s)[i];
+      if (o != v && o != 1 && v != 1) fatal("ProgramBuilder: where operands do not broadcast");
+      o = std::max(o, v);
+    }
+  Id out = newTensor(Desc{shape, desc(a).dtype, desc(a).layout, StorageType::Device});
+  Off c = tensorRef(cond), x = tensorRef(a), y = tensorRef(b), o = tensorRef(out);
+  b_.startTable(EltwiseTernaryWhereOp::kNumFields);
+  b_.addOffset(EltwiseTernaryWhereOp::f_first, c);
+  b_.addOffset(EltwiseTernaryWhereOp::f_second, x);
+  b_.addOffset(EltwiseTernaryWhereOp::f_third, y);
+  b_.addOffset(EltwiseTernaryWhereOp::f_out, o);
+  addOp(OpType::EltwiseTernaryWhereOp, b_.endTable(), "ttnn.where " + shapeStr(shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::embedding(Id indices, Id weight) {
+  Desc d = desc(weight);
+  std::vector<std::uint32_t> shape = desc(indices).shape;
+  shape.push_back(d.shape.back());
+  d.shape = shape;
+  d.storage = StorageType::Device;
+  Id out = newTensor(d);
+  Off i = tensorRef(indices), w = tensorRef(weight), o = tensorRef(out);
+  b_.startTable(EmbeddingOp::kNumFields);
+  b_.addOffset(EmbeddingOp::f_input, i);
+  b_.addOffset(EmbeddingOp::f_weight, w);
+  b_.addOffset(EmbeddingOp::f_out, o);
+  addOp(OpType::EmbeddingOp, b_.endTable(), "ttnn.embedding " + shapeStr(shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::argmax(Id in, bool hasDim, int dim, bool keepDim, DataType outDtype) {
+  Desc d = desc(in);
+  const int rank = static_cast<int>(d.shape.size());
+  std::vector<std::uint32_t> shape;
+  if (hasDim) {
+    const int dd = dim < 0 ? dim + rank : dim;
+    for (int i = 0; i < rank; ++i) {
+      if (i != dd) shape.push_back(d.shape[i]);
+      else if (keepDim) shape.push_back(1);
+    }
+  } else if (keepDim) {
+    shape.assign(rank, 1);
+  }
+  if (shape.empty()) shape.push_back(1);
+  Id out = newTensor(Desc{shape, outDtype, TensorLayout::RowMajor, StorageType::Device});
+  Off i = tensorRef(in), o = tensorRef(out);
+  b_.startTable(ReductionArgMaxOp::kNumFields);
+  b_.addOffset(ReductionArgMaxOp::f_in, i);
+  b_.addOffset(ReductionArgMaxOp::f_out, o);
+  if (hasDim) b_.addScalar<std::int32_t>(ReductionArgMaxOp::f_dim, dim);
+  b_.addScalarDefault<std::uint8_t>(ReductionArgMaxOp::f_keep_dim, keepDim, 0);
+  addOp(OpType::ReductionArgMaxOp, b_.endTable(), "ttnn.argmax " + shapeStr(shape));
+  return out;
+}
+ProgramBuilder::Id ProgramBuilder::arange(float start, float end, float step, DataType dtype, TensorLayout layout) {
+  const double n = std::ceil((static_cast<double>(end) - start) / step);
+  std::vector<std::uint32_t> shape{static_cast<std::uint32_t>(n > 0 ? n : 0)};
+  Id out = newTensor(Desc{shape, dtype, layout, StorageType::Device});
+  Off o = tensorRef(out);
+  b_.startTable(ArangeOp::kNumFields);
+  b_.addScalarDefault<float>(ArangeOp::f_start, start, 0.0f);
+  b_.addScalarDefault<float>(ArangeOp::f_end, end, 0.0f);
+  b_.addScalarDefault<float>(ArangeOp::f_step, step, 0.0f);
+  b_.addScalar<std::uint16_t>(ArangeOp::f_dtype, static_cast<std::uint16_t>(dtype));
+  b_.addScalar<std::uint16_t>(ArangeOp::f_layout, static_cast<std::uint16_t>(layout));
+  b_.addOffset(ArangeOp::f_out, o);
+  addOp(OpType::ArangeOp, b_.endTable(), "ttnn.arange " + shapeStr(shape));
   return out;
 }
 ProgramBuilder::Id ProgramBuilder::constant(const void *data, size_t bytes, DataType inDtype, const std::vector<std::uint32_t> &shape,

@@ -47,6 +47,13 @@ public:
   Id concat(const std::vector<Id> &ins, int dim);
   Id slice(Id in, const std::vector<std::int64_t> &begins, const std::vector<std::int64_t> &ends, const std::vector<std::int64_t> &steps);
   Id repeatInterleave(Id in, std::uint32_t repeats, int dim);
+  // the ops around a decoder layer (include/ttmlir/Target/TTNN/operations/{data_movement,eltwise,embedding,reduction,creation}.fbs)
+  Id repeat(Id in, const std::vector<std::int64_t> &repeats);
+  Id binaryComposite(std::uint32_t type, Id lhs, Id rhs);
+  Id where(Id cond, Id a, Id b);
+  Id embedding(Id indices, Id weight);
+  Id argmax(Id in, bool hasDim, int dim, bool keepDim, DataType outDtype);
+  Id arange(float start, float end, float step, DataType dtype, TensorLayout layout);
   Id constant(const void *data, size_t bytes, DataType inDtype, const std::vector<std::uint32_t> &shape, DataType dtype,
               TensorLayout layout, StorageType storage);
   Id full(const std::vector<std::uint32_t> &shape, float value, DataType dtype, TensorLayout layout);
