@@ -148,6 +148,11 @@ int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int layout, 
                       int64_t cols, float param, void *stream);
 int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape,
                        void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream);
+/* ttm_eltwise_unary also takes 100 + EltwiseUnaryCompositeOpType for Cbrt (100) and Log1p (103)
+ * (runtime/lib/ttnn/operations/eltwise/unary/unary_composite.cpp:104-135); ClampScalar is ttm_clamp: min(max(x, lo), hi),
+ * NaN kept (golden tools/golden/mapping.py:5267-5276, torch.clamp). */
+int ttm_clamp(const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float lo, float hi,
+              void *stream);
 /* ttm_eltwise_binary also takes 100 + EltwiseBinaryCompositeOpType for Maximum, Minimum, Remainder, Pow and Atan2
  * (runtime/lib/ttnn/operations/eltwise/binary/binary_composite.cpp; goldens tools/golden/mapping.py:4493-4570, 5516-5530:
  * torch.maximum / minimum (NaN propagates), torch.remainder (sign of the divisor), torch.pow, torch.atan2).

@@ -165,6 +165,9 @@ int ttrt_pb_slice(ttrt_builder *pb, uint32_t in, const int64_t *begins, const in
 int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_t repeats, int dim, uint32_t *out);
 /* RepeatOp, EltwiseBinaryCompositeOp (type = EltwiseBinaryCompositeOpType), EltwiseTernaryWhereOp, EmbeddingOp,
  * ReductionArgMaxOp (has_dim = 0: over the whole tensor), ArangeOp */
+/* EltwiseUnaryCompositeOp (type = EltwiseUnaryCompositeOpType: Cbrt 0, ClampScalar 1 with bounds lo / hi written as FP or,
+ * with int_bounds, as I32; Log1p 3) */
+int ttrt_pb_unary_composite(ttrt_builder *pb, uint32_t type, uint32_t in, float lo, float hi, int int_bounds, uint32_t *out);
 int ttrt_pb_repeat(ttrt_builder *pb, uint32_t in, const int64_t *repeats, int rank, uint32_t *out);
 int ttrt_pb_binary_composite(ttrt_builder *pb, uint32_t type, uint32_t lhs, uint32_t rhs, uint32_t *out);
 int ttrt_pb_where(ttrt_builder *pb, uint32_t cond, uint32_t a, uint32_t b, uint32_t *out);

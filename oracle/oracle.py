@@ -85,7 +85,8 @@ def max_threads():
 
 UNARY = dict(abs=0, ceil=1, cos=2, floor=3, gelu=4, isfinite=5, logical_not=6, neg=7, relu=8, sqrt=9,
              rsqrt=10, sigmoid=11, sin=12, reciprocal=13, sign=14, tan=15, tanh=16, atan=17, exp=18,
-             erf=19, erfc=20, log=21, expm1=22, leaky_relu=23, relu6=25, silu=26)
+             erf=19, erfc=20, log=21, expm1=22, leaky_relu=23, relu6=25, silu=26, hardsigmoid=27, mish=28, acos=29,
+             asin=30, asinh=31, cbrt=100, log1p=103)
 BINARY = dict(add=0, multiply=1, subtract=3, eq=4, ne=5, ge=6, gt=7, le=8, lt=9, divide=10)
 ACT = {None: 0, "": 0, "gelu": 1, "silu": 2, "sigmoid": 3, "relu": 4}
 REDUCE = dict(sum=0, mean=1, max=2, min=3)
@@ -439,3 +440,9 @@ def binary_composite(name, a, b):
     with np.errstate(all="ignore"):
         return {"maximum": np.maximum, "minimum": np.minimum, "remainder": np.mod, "pow": np.power,
                 "atan2": np.arctan2}[name](a, b).astype(np.float32)
+
+
+def clamp(x, lo, hi):
+    """tools/golden/mapping.py:5267-5276 (torch.clamp with scalar bounds; NaN stays NaN)."""
+    x = np.asarray(x, np.float32)
+    return np.where(np.isnan(x), x, np.minimum(np.maximum(x, np.float32(lo)), np.float32(hi))).astype(np.float32)

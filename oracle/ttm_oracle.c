@@ -297,7 +297,8 @@ void orc_bf16_to_f16(const uint16_t *in, uint16_t *out, int64_t n) {
  * include/ttmlir/Target/TTNN/operations/eltwise.fbs                                        */
 enum { U_ABS = 0, U_CEIL, U_COS, U_FLOOR, U_GELU, U_ISFINITE, U_LOGICALNOT, U_NEG, U_RELU, U_SQRT,
        U_RSQRT, U_SIGMOID, U_SIN, U_RECIPROCAL, U_SIGN, U_TAN, U_TANH, U_ATAN, U_EXP, U_ERF, U_ERFC,
-       U_LOG, U_EXPM1, U_LEAKYRELU, U_BITWISENOT, U_RELU6, U_SILU };
+       U_LOG, U_EXPM1, U_LEAKYRELU, U_BITWISENOT, U_RELU6, U_SILU, U_HARDSIGMOID, U_MISH, U_ACOS, U_ASIN, U_ASINH,
+       U_CBRT = 100, U_LOG1P = 103 };
 
 static inline float unary_f32(int op, float x, float p) {
   switch (op) {
@@ -327,6 +328,15 @@ static inline float unary_f32(int op, float x, float p) {
   case U_LEAKYRELU: return x > 0.0f ? x : p * x;
   case U_RELU6: return x < 0.0f ? 0.0f : (x > 6.0f ? 6.0f : x);
   case U_SILU: return x * (1.0f / (1.0f + expf(-x)));
+  /* torch.nn.functional.hardsigmoid = relu6(x + 3) / 6, mish = x tanh(softplus(x)) (tools/golden/mapping.py:5544-5548 and
+   * the torch definitions the other goldens call) */
+  case U_HARDSIGMOID: { float t = x + 3.0f; t = t < 0.0f ? 0.0f : (t > 6.0f ? 6.0f : t); return x != x ? x : t / 6.0f; }
+  case U_MISH: return x * tanhf(x > 20.0f ? x : log1pf(expf(x)));
+  case U_ACOS: return acosf(x);
+  case U_ASIN: return asinf(x);
+  case U_ASINH: return asinhf(x);
+  case U_CBRT: return cbrtf(x);
+  case U_LOG1P: return log1pf(x);
   default: return NAN;
   }
 }

@@ -21,7 +21,8 @@ def bf16_ulps(got, want):
 
 
 UNARY = ["abs", "ceil", "cos", "floor", "gelu", "isfinite", "logical_not", "neg", "relu", "sqrt", "rsqrt", "sigmoid",
-         "sin", "reciprocal", "sign", "tanh", "atan", "exp", "erf", "erfc", "log", "expm1", "relu6", "silu", "leaky_relu"]
+         "sin", "reciprocal", "sign", "tanh", "atan", "exp", "erf", "erfc", "log", "expm1", "relu6", "silu", "leaky_relu",
+         "hardsigmoid", "mish", "acos", "asin", "asinh", "cbrt", "log1p"]
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
@@ -29,7 +30,9 @@ def test_unary(hip, dev, orc, dtype):
     x = datagen.randn((70, 33), seed=1, std=2.0)
     x[0, :4] = torch.tensor([0.0, -0.0, 1.0, -1.0])
     for name in UNARY:
-        xi = x.abs() + 0.01 if name in ("sqrt", "rsqrt", "log") else x
+        xi = x.abs() + 0.01 if name in ("sqrt", "rsqrt", "log", "log1p") else x
+        if name in ("acos", "asin"):
+            xi = torch.tanh(x)
         if dtype == "bf16":
             xi = xi.to(torch.bfloat16)
         xd = xi.to(dev)
@@ -549,3 +552,25 @@ def test_binary_composites(hip, dev, orc, dtype, name, code):
         assert np.array_equal(got.float().numpy(), want.float().numpy(), equal_nan=True)
     else:
         assert torch.allclose(got.float(), want.float(), rtol=2.0 ** -7 if dtype == torch.bfloat16 else 1e-5, atol=1e-6, equal_nan=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("tiled", [False, True])
+def test_clamp_bit_exact(hip, dev, orc, dtype, tiled):
+    """ttm_clamp (ClampScalar) against the oracle: NaN kept, infinities clamped, tile padding left at zero even when the
+    lower bound is positive."""
+    x = datagen.randn((2, 40, 50), seed=190, dtype=dtype) * 4
+    x[0, 0, :3] = torch.tensor([float("nan"), float("inf"), float("-inf")], dtype=dtype)
+    code = hip.BF16 if dtype == torch.bfloat16 else hip.F32
+    for lo, hi in ((-1.0, 2.5), (0.5, 3.0)):
+        xd = tilize_dev(hip, x, dev) if tiled else x.to(dev)
+        out = torch.full_like(xd, float("nan"))
+        hip.call("ttm_clamp", hip.ptr(xd), hip.ptr(out), code, hip.TILE if tiled else hip.ROW_MAJOR, 2, 40, 50, lo, hi, hip.current_stream())
+        got = untilize_dev(hip, out, x.shape, dev).cpu() if tiled else out.cpu()
+        torch.cuda.synchronize()
+        want = orc.clamp(x.float().numpy(), lo, hi)
+        assert np.array_equal(got.float().numpy(), want, equal_nan=True)
+        if tiled:
+            assert torch.equal(tilize_dev(hip, got, dev).view(torch.uint8), out.view(torch.uint8))       # padding is zero
+    with pytest.raises(hip.TTMError, match="ttm_clamp"):
+        hip.call("ttm_eltwise_unary", 101, hip.ptr(xd), hip.ptr(out), code, hip.ROW_MAJOR, 2, 40, 50, 0.0, hip.current_stream())

@@ -846,6 +846,9 @@ def test_decoder_head_and_tail_ops_program(device, orc, metrics):
     pb.output(pb.argmax(logits, dim=-1, keep_dim=True, out_dtype=DT.UInt32))
     pb.output(pb.argmax(logits, dim=1))
     pb.output(pb.argmax(logits))
+    pb.output(pb.unary_composite(programs.UNARY_COMPOSITE["clamp_scalar"], emb, -0.5, 0.75))
+    pb.output(pb.unary_composite(programs.UNARY_COMPOSITE["clamp_scalar"], emb, -1, 1, int_bounds=True))
+    pb.output(pb.unary_composite(programs.UNARY_COMPOSITE["cbrt"], emb))
     pb.end_program()
     binary = rt.Binary.load_from_memory(pb.finish())
     g = torch.Generator().manual_seed(31)
@@ -868,3 +871,6 @@ def test_decoder_head_and_tail_ops_program(device, orc, metrics):
     assert np.array_equal(got[5].numpy().astype(np.int64), orc.argmax(f(tlogits), -1, True).astype(np.int64)) and tuple(got[5].shape) == (B, S, 1)
     assert np.array_equal(got[6].numpy(), orc.argmax(f(tlogits), 1))
     assert int(got[7].reshape(-1)[0]) == int(orc.argmax(f(tlogits)))
+    assert np.array_equal(f(got[8]), orc.round_bf16(orc.clamp(want_emb, -0.5, 0.75)))
+    assert np.array_equal(f(got[9]), orc.clamp(want_emb, -1.0, 1.0))
+    assert np.max(np.abs(f(got[10]) - orc.unary("cbrt", want_emb))) <= 2.0 ** -7

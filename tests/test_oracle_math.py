@@ -47,11 +47,15 @@ def test_batched_matmul_broadcast(orc):
     ("gelu", F.gelu), ("silu", F.silu), ("sigmoid", torch.sigmoid), ("exp", torch.exp), ("neg", torch.neg),
     ("rsqrt", torch.rsqrt), ("sqrt", torch.sqrt), ("tanh", torch.tanh), ("erf", torch.erf), ("relu", torch.relu),
     ("abs", torch.abs), ("reciprocal", torch.reciprocal), ("log", torch.log), ("sin", torch.sin), ("cos", torch.cos),
-    ("floor", torch.floor), ("ceil", torch.ceil), ("sign", torch.sign)])
+    ("floor", torch.floor), ("ceil", torch.ceil), ("sign", torch.sign), ("hardsigmoid", F.hardsigmoid), ("mish", F.mish),
+    ("acos", torch.acos), ("asin", torch.asin), ("asinh", torch.asinh), ("log1p", torch.log1p),
+    ("cbrt", lambda t: torch.sign(t) * torch.abs(t) ** (1.0 / 3.0))])
 def test_unary_matches_torch(orc, name, fn):
     x = rnd((1000,), 7, 3.0)
-    if name in ("rsqrt", "sqrt", "log"):
+    if name in ("rsqrt", "sqrt", "log", "log1p"):
         x = np.abs(x) + 0.01
+    if name in ("acos", "asin"):
+        x = np.tanh(x)
     want = fn(torch.from_numpy(x).double()).float().numpy()
     assert np.allclose(orc.unary(name, x), want, rtol=2e-6, atol=2e-7)
 
@@ -397,3 +401,10 @@ def test_index_and_select_ops_against_torch(orc):
         assert np.allclose(orc.binary_composite(name, p.numpy(), q.numpy()), fn(p, q.expand(4, 6)).numpy(), rtol=1e-6, atol=1e-6, equal_nan=True), name
     assert np.allclose(orc.binary_composite("pow", p.abs().numpy(), q.numpy()), torch.pow(p.abs(), q).numpy(), rtol=1e-5, equal_nan=True)
     assert orc.binary_composite("remainder", np.float32(-7), np.float32(3)) == 2.0 and orc.binary_composite("remainder", np.float32(7), np.float32(-3)) == -2.0
+
+
+def test_clamp_against_torch(orc):
+    x = rnd((500,), 51, 4.0)
+    x[:3] = [np.nan, np.inf, -np.inf]
+    for lo, hi in ((-1.0, 2.5), (0.0, 0.0), (-3.0, -1.0)):
+        assert np.array_equal(orc.clamp(x, lo, hi), torch.clamp(torch.from_numpy(x), min=lo, max=hi).numpy(), equal_nan=True)

@@ -12,14 +12,16 @@
 // op codes = EltwiseUnaryOpType / EltwiseBinaryOpType values of the TTNN flatbuffer schema
 enum { U_ABS = 0, U_CEIL, U_COS, U_FLOOR, U_GELU, U_ISFINITE, U_LOGICALNOT, U_NEG, U_RELU, U_SQRT,
        U_RSQRT, U_SIGMOID, U_SIN, U_RECIPROCAL, U_SIGN, U_TAN, U_TANH, U_ATAN, U_EXP, U_ERF, U_ERFC,
-       U_LOG, U_EXPM1, U_LEAKYRELU, U_BITWISENOT, U_RELU6, U_SILU };
+       U_LOG, U_EXPM1, U_LEAKYRELU, U_BITWISENOT, U_RELU6, U_SILU, U_HARDSIGMOID, U_MISH, U_ACOS, U_ASIN, U_ASINH,
+       // 100 + EltwiseUnaryCompositeOpType (ClampTensor, 102, is a ternary and has no kernel here)
+       U_CBRT = 100, U_CLAMP = 101, U_LOG1P = 103 };
 enum { B_ADD = 0, B_MUL = 1, B_SUB = 3, B_EQ = 4, B_NE = 5, B_GE = 6, B_GT = 7, B_LE = 8, B_LT = 9, B_DIV = 10,
        B_AND = 11, B_OR = 12, B_XOR = 13,
        // 100 + EltwiseBinaryCompositeOpType
        B_MAXIMUM = 100, B_MINIMUM = 101, B_REMAINDER = 102, B_POW = 103, B_ATAN2 = 104 };
 
 template <int OP>
-__device__ __forceinline__ float unary_op(float x, float p) {
+__device__ __forceinline__ float unary_op(float x, float p, float p2 = 0.0f) {
   switch (OP) {
   case U_ABS: return fabsf(x);
   case U_CEIL: return ceilf(x);
@@ -47,6 +49,14 @@ __device__ __forceinline__ float unary_op(float x, float p) {
   case U_LEAKYRELU: return x > 0.0f ? x : p * x;
   case U_RELU6: return fminf(fmaxf(x, 0.0f), 6.0f);
   case U_SILU: return x * (1.0f / (1.0f + expf(-x)));
+  case U_HARDSIGMOID: return fminf(fmaxf(x + 3.0f, 0.0f), 6.0f) * (1.0f / 6.0f) + (x != x ? x : 0.0f);   // relu6(x + 3) / 6
+  case U_MISH: return x * tanhf(x > 20.0f ? x : log1pf(expf(x)));                                       // x tanh(softplus(x))
+  case U_ACOS: return acosf(x);
+  case U_ASIN: return asinf(x);
+  case U_ASINH: return asinhf(x);
+  case U_CBRT: return cbrtf(x);
+  case U_CLAMP: return x != x ? x : fminf(fmaxf(x, p), p2);                                               // torch.clamp: NaN stays
+  case U_LOG1P: return log1pf(x);
   default: return x;
   }
 }
@@ -107,19 +117,19 @@ __device__ __forceinline__ void chunk_store(void *p, int64_t chunk, const float 
 
 template <int OP, bool BF16>
 __global__ __launch_bounds__(256) void ttm_unary_k(const void *__restrict__ in, void *__restrict__ out, int64_t nchunks,
-                                                   int64_t n, float param) {
+                                                   int64_t n, float param, float param2) {
   constexpr int EPC = BF16 ? 8 : 4;
   for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < nchunks; c += (int64_t)gridDim.x * 256) {
     if ((c + 1) * EPC <= n) {
       float f[EPC];
       chunk_load<BF16>(in, c, f);
 #pragma unroll
-      for (int i = 0; i < EPC; ++i) f[i] = unary_op<OP>(f[i], param);
+      for (int i = 0; i < EPC; ++i) f[i] = unary_op<OP>(f[i], param, param2);
       chunk_store<BF16>(out, c, f);
     } else {  // ragged tail
       for (int64_t i = c * EPC; i < n; ++i) {
         float x = BF16 ? ttm_bf16_to_f32(((const uint16_t *)in)[i]) : ((const float *)in)[i];
-        float y = unary_op<OP>(x, param);
+        float y = unary_op<OP>(x, param, param2);
         if (BF16) ((uint16_t *)out)[i] = ttm_f32_to_bf16(y);
         else ((float *)out)[i] = y;
       }
@@ -130,7 +140,7 @@ __global__ __launch_bounds__(256) void ttm_unary_k(const void *__restrict__ in, 
 // ragged tile-order tensors: padding must stay zero (it feeds later contractions), so decode coordinates
 template <int OP, bool BF16>
 __global__ __launch_bounds__(256) void ttm_unary_masked_k(const void *__restrict__ in, void *__restrict__ out,
-                                                          int64_t total, int64_t rows, int64_t cols, float param) {
+                                                          int64_t total, int64_t rows, int64_t cols, float param, float param2) {
   const int64_t pr = (rows + 31) / 32 * 32, pc = (cols + 31) / 32 * 32;
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
     int64_t w = i % (pr * pc), tile = w >> 10;
@@ -140,15 +150,15 @@ __global__ __launch_bounds__(256) void ttm_unary_masked_k(const void *__restrict
     float y = 0.0f;
     if (r < rows && c < cols) {
       float x = BF16 ? ttm_bf16_to_f32(((const uint16_t *)in)[i]) : ((const float *)in)[i];
-      y = unary_op<OP>(x, param);
+      y = unary_op<OP>(x, param, param2);
     }
     if (BF16) ((uint16_t *)out)[i] = ttm_f32_to_bf16(y);
     else ((float *)out)[i] = y;
   }
 }
 
-typedef void (*unary_fn)(const void *, void *, int64_t, int64_t, float);
-typedef void (*unary_masked_fn)(const void *, void *, int64_t, int64_t, int64_t, float);
+typedef void (*unary_fn)(const void *, void *, int64_t, int64_t, float, float);
+typedef void (*unary_masked_fn)(const void *, void *, int64_t, int64_t, int64_t, float, float);
 
 template <bool BF16>
 static unary_fn pick_unary(int op) {
@@ -156,7 +166,8 @@ static unary_fn pick_unary(int op) {
   switch (op) {
     U(U_ABS) U(U_CEIL) U(U_COS) U(U_FLOOR) U(U_GELU) U(U_ISFINITE) U(U_LOGICALNOT) U(U_NEG) U(U_RELU) U(U_SQRT)
     U(U_RSQRT) U(U_SIGMOID) U(U_SIN) U(U_RECIPROCAL) U(U_SIGN) U(U_TAN) U(U_TANH) U(U_ATAN) U(U_EXP) U(U_ERF)
-    U(U_ERFC) U(U_LOG) U(U_EXPM1) U(U_LEAKYRELU) U(U_RELU6) U(U_SILU)
+    U(U_ERFC) U(U_LOG) U(U_EXPM1) U(U_LEAKYRELU) U(U_RELU6) U(U_SILU) U(U_HARDSIGMOID) U(U_MISH) U(U_ACOS) U(U_ASIN)
+    U(U_ASINH) U(U_CBRT) U(U_CLAMP) U(U_LOG1P)
   default: return nullptr;
   }
 #undef U
@@ -167,7 +178,8 @@ static unary_masked_fn pick_unary_masked(int op) {
   switch (op) {
     U(U_ABS) U(U_CEIL) U(U_COS) U(U_FLOOR) U(U_GELU) U(U_ISFINITE) U(U_LOGICALNOT) U(U_NEG) U(U_RELU) U(U_SQRT)
     U(U_RSQRT) U(U_SIGMOID) U(U_SIN) U(U_RECIPROCAL) U(U_SIGN) U(U_TAN) U(U_TANH) U(U_ATAN) U(U_EXP) U(U_ERF)
-    U(U_ERFC) U(U_LOG) U(U_EXPM1) U(U_LEAKYRELU) U(U_RELU6) U(U_SILU)
+    U(U_ERFC) U(U_LOG) U(U_EXPM1) U(U_LEAKYRELU) U(U_RELU6) U(U_SILU) U(U_HARDSIGMOID) U(U_MISH) U(U_ACOS) U(U_ASIN)
+    U(U_ASINH) U(U_CBRT) U(U_CLAMP) U(U_LOG1P)
   default: return nullptr;
   }
 #undef U
@@ -178,8 +190,8 @@ static unsigned grid_for(int64_t nchunks) {
   return (unsigned)(b > 262144 ? 262144 : (b < 1 ? 1 : b));
 }
 
-TTM_EXPORT int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows,
-                                 int64_t cols, float param, void *stream) {
+static int unary_entry(int op, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float param,
+                       float param2, void *stream) {
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_eltwise_unary: dtype must be BFloat16 or Float32 (got %d)", dtype);
   TTM_REQUIRE(layout == TTM_ROW_MAJOR || layout == TTM_TILE, "ttm_eltwise_unary: bad layout");
   TTM_REQUIRE(batch >= 0 && rows >= 0 && cols >= 0, "ttm_eltwise_unary: negative dimension");
@@ -191,7 +203,7 @@ TTM_EXPORT int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, i
   if (tiled && (pr != rows || pc != cols)) {
     unary_masked_fn fn = dtype == TTM_BF16 ? pick_unary_masked<true>(op) : pick_unary_masked<false>(op);
     if (!fn) return ttm_set_error(TTM_ERR_UNSUPPORTED, "ttm_eltwise_unary: unsupported op %d", op);
-    hipLaunchKernelGGL(fn, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, in, out, n, rows, cols, param);
+    hipLaunchKernelGGL(fn, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, in, out, n, rows, cols, param, param2);
     TTM_LAUNCH_CHECK();
     return TTM_OK;
   }
@@ -200,9 +212,20 @@ TTM_EXPORT int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, i
   if (!fn) return ttm_set_error(TTM_ERR_UNSUPPORTED, "ttm_eltwise_unary: unsupported op %d", op);
   const int epc = dtype == TTM_BF16 ? 8 : 4;
   int64_t nchunks = ttm_cdiv(n, epc);
-  hipLaunchKernelGGL(fn, dim3(grid_for(nchunks)), dim3(256), 0, (hipStream_t)stream, in, out, nchunks, n, param);
+  hipLaunchKernelGGL(fn, dim3(grid_for(nchunks)), dim3(256), 0, (hipStream_t)stream, in, out, nchunks, n, param, param2);
   TTM_LAUNCH_CHECK();
   return TTM_OK;
+}
+
+TTM_EXPORT int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows,
+                                 int64_t cols, float param, void *stream) {
+  TTM_REQUIRE(op != U_CLAMP, "ttm_eltwise_unary: clamp takes two bounds, use ttm_clamp");
+  return unary_entry(op, in, out, dtype, layout, batch, rows, cols, param, 0.0f, stream);
+}
+
+TTM_EXPORT int ttm_clamp(const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float lo, float hi,
+                         void *stream) {
+  return unary_entry(U_CLAMP, in, out, dtype, layout, batch, rows, cols, lo, hi, stream);
 }
 
 // ---- binary, same shape: flat

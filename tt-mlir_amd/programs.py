@@ -15,7 +15,8 @@ DT, TL, ST = rt.DataType, rt.TensorLayout, rt.StorageType
 # EltwiseUnaryOpType / EltwiseBinaryOpType / ReductionOpType values
 UNARY = dict(abs=0, ceil=1, cos=2, floor=3, gelu=4, isfinite=5, logical_not=6, neg=7, relu=8, sqrt=9, rsqrt=10,
              sigmoid=11, sin=12, reciprocal=13, sign=14, tan=15, tanh=16, atan=17, exp=18, erf=19, erfc=20, log=21,
-             expm1=22, leaky_relu=23, relu6=25, silu=26)
+             expm1=22, leaky_relu=23, relu6=25, silu=26, hardsigmoid=27, mish=28, acos=29, asin=30, asinh=31)
+UNARY_COMPOSITE = dict(cbrt=0, clamp_scalar=1, log1p=3)
 BINARY = dict(add=0, multiply=1, subtract=3, eq=4, ne=5, ge=6, gt=7, le=8, lt=9, divide=10)
 REDUCE = dict(sum=0, mean=1, max=2, min=3)
 BINARY_COMPOSITE = dict(maximum=0, minimum=1, remainder=2, pow=3, atan2=4)

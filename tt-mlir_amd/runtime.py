@@ -600,6 +600,9 @@ class ProgramBuilder:
     def repeat_interleave(self, t, repeats, dim):
         return self._op("ttrt_pb_repeat_interleave", t, repeats, dim)
 
+    def unary_composite(self, type_, t, lo=0.0, hi=0.0, int_bounds=False):
+        return self._op("ttrt_pb_unary_composite", type_, t, ctypes.c_float(lo), ctypes.c_float(hi), int(int_bounds))
+
     def repeat(self, t, repeats):
         r = (ctypes.c_int64 * len(repeats))(*repeats)
         return self._op("ttrt_pb_repeat", t, r, len(repeats))

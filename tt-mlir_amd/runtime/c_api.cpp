@@ -440,6 +440,9 @@ TTRT_EXPORT int ttrt_pb_slice(ttrt_builder *pb, uint32_t in, const int64_t *begi
 TTRT_EXPORT int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_t repeats, int dim, uint32_t *out) {
   PB_OP(repeatInterleave(in, repeats, dim));
 }
+TTRT_EXPORT int ttrt_pb_unary_composite(ttrt_builder *pb, uint32_t type, uint32_t in, float lo, float hi, int int_bounds, uint32_t *out) {
+  PB_OP(unaryComposite(type, in, lo, hi, int_bounds != 0));
+}
 TTRT_EXPORT int ttrt_pb_repeat(ttrt_builder *pb, uint32_t in, const int64_t *repeats, int rank, uint32_t *out) {
   PB_OP(repeat(in, std::vector<std::int64_t>(repeats, repeats + rank)));
 }

@@ -114,6 +114,7 @@ OpRefs opRefs(const fb::Table &operation) {
   case OpType::SliceOp: in(schema::SliceOp::f_in); out(schema::SliceOp::f_out); break;
   case OpType::RepeatInterleaveOp: in(schema::RepeatInterleaveOp::f_input); out(schema::RepeatInterleaveOp::f_out); break;
   case OpType::RepeatOp: in(schema::RepeatOp::f_in); out(schema::RepeatOp::f_out); break;
+  case OpType::EltwiseUnaryCompositeOp: in(schema::EltwiseUnaryCompositeOp::f_in); out(schema::EltwiseUnaryCompositeOp::f_out); break;
   case OpType::EltwiseBinaryCompositeOp:
     in(schema::EltwiseBinaryCompositeOp::f_lhs); in(schema::EltwiseBinaryCompositeOp::f_rhs); out(schema::EltwiseBinaryCompositeOp::f_out);
     break;
@@ -511,6 +512,36 @@ void binaryImpl(ProgramContext &ctx, const fb::Table &lhsRef, const fb::Table &r
   Tensor out = makeDeviceTensor(ctx.dev, oshape, dt, lay);
   TTM_CALL(ttm_eltwise_binary(code, l.handle->data.get(), ls.data(), r.handle->data.get(), rs.data(),
                               out.handle->data.get(), os.data(), static_cast<int>(rank), ttmDtype(dt), ttmLayout(lay), ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+// runtime/lib/ttnn/operations/eltwise/unary/unary_composite.cpp:104-135: cbrt, log1p, clamp with scalar bounds
+void runEltwiseUnaryComposite(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::EltwiseUnaryCompositeOp;
+  const std::uint32_t type = op.scalar<std::uint32_t>(S::f_type, 0);
+  TTRT_ASSERT(type != static_cast<std::uint32_t>(schema::EltwiseUnaryCompositeOpType::ClampTensor), "clamp with tensor bounds is not supported");
+  Tensor in0 = ctx.get(op.table(S::f_in), "unary composite in");
+  auto outRef = op.table(S::f_out);
+  const DataType dt = computeDtypeOf({layoutFromTensorRef(outRef).dataType, in0.handle->dtype});
+  Tensor in = as(ctx, in0, in0.handle->layout, dt);
+  Tensor out = makeDeviceTensor(ctx.dev, in.handle->shape, dt, in.handle->layout);
+  const Dims3 d = dims3(in.handle->shape);
+  if (type == static_cast<std::uint32_t>(schema::EltwiseUnaryCompositeOpType::ClampScalar)) {
+    auto prm = op.table(S::f_params);
+    TTRT_ASSERT(static_cast<bool>(prm), "clamp: bounds missing");
+    auto number = [&](int typeSlot, int slot) {
+      const auto kind = static_cast<schema::NumberType>(prm.scalar<std::uint8_t>(typeSlot, 0));
+      auto t = prm.table(slot);
+      TTRT_ASSERT(static_cast<bool>(t), "clamp: bound missing");
+      return kind == schema::NumberType::I32 ? static_cast<float>(t.scalar<std::int32_t>(schema::IntegralType::f_value, 0))
+                                             : t.scalar<float>(schema::FloatingPointType::f_value, 0.0f);
+    };
+    using P = schema::ClampScalarOpParams;
+    TTM_CALL(ttm_clamp(in.handle->data.get(), out.handle->data.get(), ttmDtype(dt), ttmLayout(in.handle->layout), d.batch, d.rows, d.cols,
+                       number(P::f_min_type, P::f_min), number(P::f_max_type, P::f_max), ctx.stream()));
+  } else {
+    TTM_CALL(ttm_eltwise_unary(100 + static_cast<int>(type), in.handle->data.get(), out.handle->data.get(), ttmDtype(dt),
+                               ttmLayout(in.handle->layout), d.batch, d.rows, d.cols, 0.0f, ctx.stream()));
+  }
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 void runEltwiseBinary(const fb::Table &op, ProgramContext &ctx) {
@@ -1625,6 +1656,7 @@ void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   case OpType::RepeatInterleaveOp: return runRepeatInterleave(op, ctx);
   case OpType::RepeatOp: return runRepeat(op, ctx);
   case OpType::EltwiseBinaryCompositeOp: return runEltwiseBinaryComposite(op, ctx);
+  case OpType::EltwiseUnaryCompositeOp: return runEltwiseUnaryComposite(op, ctx);
   case OpType::EltwiseTernaryWhereOp: return runWhere(op, ctx);
   case OpType::EmbeddingOp: return runEmbedding(op, ctx);
   case OpType::ReductionArgMaxOp: return runArgMax(op, ctx);

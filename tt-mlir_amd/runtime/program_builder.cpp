@@ -319,6 +319,43 @@ ProgramBuilder::Id ProgramBuilder::unary(std::uint32_t type, Id in, bool hasPara
   return out;
 }
 
+ProgramBuilder::Id ProgramBuilder::unaryComposite(std::uint32_t type, Id in, float lo, float hi, bool intBounds) {
+  Desc d = desc(in);
+  d.storage = StorageType::Device;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out), prm = 0;
+  if (type == static_cast<std::uint32_t>(EltwiseUnaryCompositeOpType::ClampScalar)) {
+    auto number = [&](float v) {
+      if (intBounds) {
+        b_.startTable(IntegralType::kNumFields);
+        b_.addScalar<std::int32_t>(IntegralType::f_value, static_cast<std::int32_t>(v));
+      } else {
+        b_.startTable(FloatingPointType::kNumFields);
+        b_.addScalar<float>(FloatingPointType::f_value, v);
+      }
+      return b_.endTable();
+    };
+    Off mn = number(lo), mx = number(hi);
+    const std::uint8_t kind = static_cast<std::uint8_t>(intBounds ? NumberType::I32 : NumberType::FP);
+    b_.startTable(ClampScalarOpParams::kNumFields);
+    b_.addScalar<std::uint8_t>(ClampScalarOpParams::f_min_type, kind);
+    b_.addOffset(ClampScalarOpParams::f_min, mn);
+    b_.addScalar<std::uint8_t>(ClampScalarOpParams::f_max_type, kind);
+    b_.addOffset(ClampScalarOpParams::f_max, mx);
+    prm = b_.endTable();
+  }
+  b_.startTable(EltwiseUnaryCompositeOp::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(EltwiseUnaryCompositeOp::f_type, type, 0);
+  b_.addOffset(EltwiseUnaryCompositeOp::f_in, i);
+  b_.addOffset(EltwiseUnaryCompositeOp::f_out, o);
+  if (prm) {
+    b_.addScalar<std::uint8_t>(EltwiseUnaryCompositeOp::f_params_type, static_cast<std::uint8_t>(EltwiseUnaryCompositeOpParams::ClampScalarOpParams));
+    b_.addOffset(EltwiseUnaryCompositeOp::f_params, prm);
+  }
+  addOp(OpType::EltwiseUnaryCompositeOp, b_.endTable(), "ttnn.unary_composite#" + std::to_string(type));
+  return out;
+}
+
 ProgramBuilder::Id ProgramBuilder::binary(std::uint32_t type, Id lhs, Id rhs) {
   const auto &a = desc(lhs).shape, &b = desc(rhs).shape;
   size_t rank = std::max(a.size(), b.size());

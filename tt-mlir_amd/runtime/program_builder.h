@@ -36,6 +36,8 @@ public:
   Id matmul(Id a, Id b, bool transposeA, bool transposeB, const std::string &activation, DataType outDtype);
   Id linear(Id a, Id b, Id bias /* 0 = none */, bool transposeA, bool transposeB, const std::string &activation, DataType outDtype);
   Id unary(std::uint32_t type, Id in, bool hasParam, float param);
+  // EltwiseUnaryCompositeOp: Cbrt, ClampScalar (bounds as FP, or as I32 when intBounds), Log1p
+  Id unaryComposite(std::uint32_t type, Id in, float lo, float hi, bool intBounds);
   Id binary(std::uint32_t type, Id lhs, Id rhs);
   Id rmsNorm(Id in, Id weight, Id bias, float eps);
   Id softmax(Id in, int dim);
