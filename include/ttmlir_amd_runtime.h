@@ -168,6 +168,13 @@ int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_t repeats, i
 /* EltwiseUnaryCompositeOp (type = EltwiseUnaryCompositeOpType: Cbrt 0, ClampScalar 1 with bounds lo / hi written as FP or,
  * with int_bounds, as I32; Log1p 3) */
 int ttrt_pb_unary_composite(ttrt_builder *pb, uint32_t type, uint32_t in, float lo, float hi, int int_bounds, uint32_t *out);
+/* head merges (kind 0 ConcatenateHeadsOp, 1 NLPConcatHeadsOp, 2 NLPConcatHeadsDecodeOp with num_heads) and splits
+ * (NLPCreateQKVHeadsDecodeOp, SplitQueryKeyValueAndSplitHeadsOp with kv_input 0 = fused input); the splits write the ids of
+ * q, k, v to qkv_out[0..2] */
+int ttrt_pb_concat_heads(ttrt_builder *pb, int kind, uint32_t in, uint32_t num_heads, uint32_t *out);
+int ttrt_pb_nlp_create_qkv_heads_decode(ttrt_builder *pb, uint32_t in, uint32_t num_heads, uint32_t num_kv_heads, uint32_t *qkv_out);
+int ttrt_pb_split_qkv_and_split_heads(ttrt_builder *pb, uint32_t in, uint32_t kv_input, uint32_t num_heads, uint32_t num_kv_heads,
+                                      int transpose_key, uint32_t *qkv_out);
 int ttrt_pb_repeat(ttrt_builder *pb, uint32_t in, const int64_t *repeats, int rank, uint32_t *out);
 int ttrt_pb_binary_composite(ttrt_builder *pb, uint32_t type, uint32_t lhs, uint32_t rhs, uint32_t *out);
 int ttrt_pb_where(ttrt_builder *pb, uint32_t cond, uint32_t a, uint32_t b, uint32_t *out);

@@ -874,3 +874,46 @@ def test_decoder_head_and_tail_ops_program(device, orc, metrics):
     assert np.array_equal(f(got[8]), orc.round_bf16(orc.clamp(want_emb, -0.5, 0.75)))
     assert np.array_equal(f(got[9]), orc.clamp(want_emb, -1.0, 1.0))
     assert np.max(np.abs(f(got[10]) - orc.unary("cbrt", want_emb))) <= 2.0 ** -7
+
+
+def test_head_split_and_merge_ops(device):
+    """SplitQueryKeyValueAndSplitHeadsOp (fused input, and q + kv inputs with grouped heads and a transposed key),
+    ConcatenateHeadsOp, NLPConcatHeadsOp, NLPCreateQKVHeadsDecodeOp and NLPConcatHeadsDecodeOp as one program: pure
+    permutations, so every output equals bit for bit what the goldens' slice / reshape / permute chains give
+    (tools/golden/mapping.py:5084-5186, 5916-5924); split followed by merge returns the query part unchanged."""
+    B, S, H, Hkv, D, U = 2, 96, 4, 2, 64, 5
+    pb = rt.ProgramBuilder()
+    pb.begin_program("heads")
+    fused = pb.input((B, S, 3 * H * D), DT.BFloat16)
+    qin = pb.input((B, S, H * D), DT.BFloat16)
+    kvin = pb.input((B, S, 2 * Hkv * D), DT.BFloat16)
+    dec = pb.input((1, 1, U, (H + 2 * Hkv) * D), DT.BFloat16)
+    q1, k1, v1 = pb.split_query_key_value_and_split_heads(fused, H)
+    q2, k2, v2 = pb.split_query_key_value_and_split_heads(qin, H, Hkv, kv_input=kvin, transpose_key=True)
+    for t in (q1, k1, v1, q2, k2, v2):
+        pb.output(t)
+    pb.output(pb.concatenate_heads(q1))
+    pb.output(pb.nlp_concat_heads(q2))
+    dq, dk, dv = pb.nlp_create_qkv_heads_decode(dec, H, Hkv)
+    for t in (dq, dk, dv):
+        pb.output(t)
+    pb.output(pb.nlp_concat_heads_decode(dq, H))
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    g = torch.Generator().manual_seed(37)
+    rn = lambda *shape: bf(torch.randn(shape, generator=g))
+    tf, tq, tkv, td = rn(B, S, 3 * H * D), rn(B, S, H * D), rn(B, S, 2 * Hkv * D), rn(1, 1, U, (H + 2 * Hkv) * D)
+    devs = [rt.to_layout(rt.from_torch(t.contiguous()), device, rt.get_layout(binary, 0, i)) for i, t in enumerate((tf, tq, tkv, td))]
+    outs = rt.submit(device, binary, 0, devs)
+    got = [rt.to_torch(rt.to_host(y, untilize=True)[0]) for y in outs]
+    heads = lambda t, n: t.reshape(B, S, n, D).permute(0, 2, 1, 3)
+    hid = H * D
+    want = [heads(tf[:, :, :hid], H), heads(tf[:, :, hid:2 * hid], H), heads(tf[:, :, 2 * hid:], H),
+            heads(tq, H), heads(tkv[:, :, :Hkv * D], Hkv).transpose(-2, -1), heads(tkv[:, :, Hkv * D:], Hkv),
+            tf[:, :, :hid], tq.reshape(B, 1, S, H * D),
+            td[0, 0, :, :H * D].reshape(1, U, H, D), td[0, 0, :, H * D:(H + Hkv) * D].reshape(1, U, Hkv, D),
+            td[0, 0, :, (H + Hkv) * D:].reshape(1, U, Hkv, D), td[:, :, :, :H * D]]
+    assert len(got) == len(want)
+    for i, (g_, w_) in enumerate(zip(got, want)):
+        assert tuple(g_.shape) == tuple(w_.shape), i
+        assert torch.equal(g_, w_.contiguous()), i

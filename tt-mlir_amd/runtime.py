@@ -603,6 +603,25 @@ class ProgramBuilder:
     def unary_composite(self, type_, t, lo=0.0, hi=0.0, int_bounds=False):
         return self._op("ttrt_pb_unary_composite", type_, t, ctypes.c_float(lo), ctypes.c_float(hi), int(int_bounds))
 
+    def concatenate_heads(self, t):
+        return self._op("ttrt_pb_concat_heads", 0, t, 0)
+
+    def nlp_concat_heads(self, t):
+        return self._op("ttrt_pb_concat_heads", 1, t, 0)
+
+    def nlp_concat_heads_decode(self, t, num_heads):
+        return self._op("ttrt_pb_concat_heads", 2, t, num_heads)
+
+    def nlp_create_qkv_heads_decode(self, t, num_heads, num_kv_heads):
+        out = (ctypes.c_uint32 * 3)()
+        _call("ttrt_pb_nlp_create_qkv_heads_decode", self.h, t, num_heads, num_kv_heads, out)
+        return tuple(out)
+
+    def split_query_key_value_and_split_heads(self, t, num_heads, num_kv_heads=None, kv_input=0, transpose_key=False):
+        out = (ctypes.c_uint32 * 3)()
+        _call("ttrt_pb_split_qkv_and_split_heads", self.h, t, kv_input, num_heads, num_kv_heads or num_heads, int(transpose_key), out)
+        return tuple(out)
+
     def repeat(self, t, repeats):
         r = (ctypes.c_int64 * len(repeats))(*repeats)
         return self._op("ttrt_pb_repeat", t, r, len(repeats))

@@ -443,6 +443,24 @@ TTRT_EXPORT int ttrt_pb_repeat_interleave(ttrt_builder *pb, uint32_t in, uint32_
 TTRT_EXPORT int ttrt_pb_unary_composite(ttrt_builder *pb, uint32_t type, uint32_t in, float lo, float hi, int int_bounds, uint32_t *out) {
   PB_OP(unaryComposite(type, in, lo, hi, int_bounds != 0));
 }
+TTRT_EXPORT int ttrt_pb_concat_heads(ttrt_builder *pb, int kind, uint32_t in, uint32_t num_heads, uint32_t *out) {
+  PB_OP(concatHeads(kind, in, num_heads));
+}
+TTRT_EXPORT int ttrt_pb_nlp_create_qkv_heads_decode(ttrt_builder *pb, uint32_t in, uint32_t num_heads, uint32_t num_kv_heads, uint32_t *qkv_out) {
+  return guard([&] {
+    need(pb, "builder"); need(qkv_out, "out");
+    auto r = pb->pb.nlpCreateQkvHeadsDecode(in, num_heads, num_kv_heads);
+    for (int i = 0; i < 3; ++i) qkv_out[i] = r[i];
+  });
+}
+TTRT_EXPORT int ttrt_pb_split_qkv_and_split_heads(ttrt_builder *pb, uint32_t in, uint32_t kv_input, uint32_t num_heads, uint32_t num_kv_heads,
+                                                  int transpose_key, uint32_t *qkv_out) {
+  return guard([&] {
+    need(pb, "builder"); need(qkv_out, "out");
+    auto r = pb->pb.splitQkvAndSplitHeads(in, kv_input, num_heads, num_kv_heads, transpose_key != 0);
+    for (int i = 0; i < 3; ++i) qkv_out[i] = r[i];
+  });
+}
 TTRT_EXPORT int ttrt_pb_repeat(ttrt_builder *pb, uint32_t in, const int64_t *repeats, int rank, uint32_t *out) {
   PB_OP(repeat(in, std::vector<std::int64_t>(repeats, repeats + rank)));
 }

@@ -114,6 +114,19 @@ OpRefs opRefs(const fb::Table &operation) {
   case OpType::SliceOp: in(schema::SliceOp::f_in); out(schema::SliceOp::f_out); break;
   case OpType::RepeatInterleaveOp: in(schema::RepeatInterleaveOp::f_input); out(schema::RepeatInterleaveOp::f_out); break;
   case OpType::RepeatOp: in(schema::RepeatOp::f_in); out(schema::RepeatOp::f_out); break;
+  case OpType::ConcatenateHeadsOp: in(schema::ConcatenateHeadsOp::f_in); out(schema::ConcatenateHeadsOp::f_out); break;
+  case OpType::NLPConcatHeadsOp: in(schema::NLPConcatHeadsOp::f_in); out(schema::NLPConcatHeadsOp::f_out); break;
+  case OpType::NLPConcatHeadsDecodeOp: in(schema::NLPConcatHeadsDecodeOp::f_in); out(schema::NLPConcatHeadsDecodeOp::f_out); break;
+  case OpType::NLPCreateQKVHeadsDecodeOp: {
+    using S = schema::NLPCreateQKVHeadsDecodeOp;
+    in(S::f_input); out(S::f_q_out); out(S::f_k_out); out(S::f_v_out);
+    break;
+  }
+  case OpType::SplitQueryKeyValueAndSplitHeadsOp: {
+    using S = schema::SplitQueryKeyValueAndSplitHeadsOp;
+    in(S::f_in); in(S::f_kv_input); out(S::f_q_out); out(S::f_k_out); out(S::f_v_out);
+    break;
+  }
   case OpType::EltwiseUnaryCompositeOp: in(schema::EltwiseUnaryCompositeOp::f_in); out(schema::EltwiseUnaryCompositeOp::f_out); break;
   case OpType::EltwiseBinaryCompositeOp:
     in(schema::EltwiseBinaryCompositeOp::f_lhs); in(schema::EltwiseBinaryCompositeOp::f_rhs); out(schema::EltwiseBinaryCompositeOp::f_out);
@@ -1315,6 +1328,105 @@ void runRepeatInterleave(const fb::Table &op, ProgramContext &ctx) {
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 
+// ---- head splits and merges around the attention ops (runtime/lib/ttnn/operations/transformer/{concatenate_heads,
+// split_query_key_value_and_split_heads,nlp_concat_heads,nlp_concat_heads_decode,nlp_create_qkv_heads_decode}.cpp): each
+// result is a strided view of its operand, written out by one copy.  (Where the compiler emits reshape + permute instead,
+// the attention runners fold them away; these ops are materialised as they stand.)
+// a tensor of `shape` whose element v (row-major) is the source's row-major element base + sum v[d] * strides[d]
+Tensor stridedCopy(ProgramContext &ctx, const Tensor &src, const std::vector<std::uint32_t> &shape, const std::vector<std::int64_t> &strides,
+                   std::int64_t base, const std::vector<std::uint32_t> &finalShape) {
+  TTRT_ASSERT(volume(finalShape) == volume(shape), "head split / merge: output shape does not match");
+  Tensor out = makeDeviceTensor(ctx.dev, finalShape, src.handle->dtype, src.handle->layout);
+  zeroIfPadded(ctx, out);
+  copyView(ctx, src, out, toI64(shape), strides, base, rowMajorStrides(shape), 0);
+  return out;
+}
+Tensor plainOperand(ProgramContext &ctx, const fb::Table &ref, const char *what) {
+  Tensor t = onDevice(ctx, ctx.get(ref, what));
+  TTRT_ASSERT(!utils::isBlockFormatDataType(t.handle->dtype), std::string(what) + ": block-float tensors are not supported here");
+  return t;
+}
+// [B, H, S, D] -> [B, S, H * D] (ConcatenateHeadsOp) or [B, 1, S, H * D] (NLPConcatHeadsOp)
+void concatHeads(ProgramContext &ctx, const fb::Table &inRef, const fb::Table &outRef, const char *what) {
+  Tensor in = plainOperand(ctx, inRef, what);
+  const auto &s = in.handle->shape;
+  TTRT_ASSERT(s.size() == 4, std::string(what) + ": input must be [batch, heads, seq, head_dim]");
+  const std::int64_t H = s[1], S = s[2], D = s[3];
+  Tensor out = stridedCopy(ctx, in, {s[0], s[2], s[1], s[3]}, {H * S * D, D, S * D, 1}, 0, shapeFromTensorRef(outRef));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+void runConcatenateHeads(const fb::Table &op, ProgramContext &ctx) {
+  concatHeads(ctx, op.table(schema::ConcatenateHeadsOp::f_in), op.table(schema::ConcatenateHeadsOp::f_out), "concatenate_heads");
+}
+void runNlpConcatHeads(const fb::Table &op, ProgramContext &ctx) {
+  concatHeads(ctx, op.table(schema::NLPConcatHeadsOp::f_in), op.table(schema::NLPConcatHeadsOp::f_out), "nlp_concat_heads");
+}
+// [1, B, Hpad, D] -> [1, 1, B, num_heads * D]: the first num_heads heads of every user, side by side
+void runNlpConcatHeadsDecode(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::NLPConcatHeadsDecodeOp;
+  Tensor in = plainOperand(ctx, op.table(S::f_in), "nlp_concat_heads_decode");
+  const auto &s = in.handle->shape;
+  const std::uint32_t heads = op.scalar<std::uint32_t>(S::f_num_heads, 0);
+  TTRT_ASSERT(s.size() == 4 && s[0] == 1 && heads >= 1 && heads <= s[2], "nlp_concat_heads_decode: input must be [1, users, heads (padded), head_dim]");
+  auto outRef = op.table(S::f_out);
+  Tensor out = stridedCopy(ctx, in, {s[1], heads, s[3]}, {static_cast<std::int64_t>(s[2]) * s[3], s[3], 1}, 0, shapeFromTensorRef(outRef));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+// [1, 1, B, (H + 2 Hkv) * D] -> q [1, B, H, D], k and v [1, B, Hkv, D]
+void runNlpCreateQkvHeadsDecode(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::NLPCreateQKVHeadsDecodeOp;
+  TTRT_ASSERT(!op.table(S::f_batch_offset) && !op.has(S::f_slice_size), "nlp_create_qkv_heads_decode: batch_offset / slice_size are not supported");
+  Tensor in = plainOperand(ctx, op.table(S::f_input), "nlp_create_qkv_heads_decode");
+  const auto &s = in.handle->shape;
+  const std::int64_t H = op.scalar<std::uint32_t>(S::f_num_heads, 0);
+  const std::int64_t Hkv = op.has(S::f_num_kv_heads) ? op.scalar<std::uint32_t>(S::f_num_kv_heads, 0) : H;
+  TTRT_ASSERT(s.size() == 4 && s[0] == 1 && s[1] == 1 && H >= 1 && Hkv >= 1 && s[3] % (H + 2 * Hkv) == 0,
+              "nlp_create_qkv_heads_decode: input must be [1, 1, users, (heads + 2 kv_heads) * head_dim]");
+  const std::int64_t W = s[3], D = W / (H + 2 * Hkv);
+  const std::uint32_t B = s[2], d = static_cast<std::uint32_t>(D);
+  auto part = [&](const fb::Table &ref, std::int64_t heads, std::int64_t base) {
+    Tensor t = stridedCopy(ctx, in, {B, static_cast<std::uint32_t>(heads), d}, {W, D, 1}, base, shapeFromTensorRef(ref));
+    ctx.put(ref, finish(ctx, t, ref));
+  };
+  part(op.table(S::f_q_out), H, 0);
+  part(op.table(S::f_k_out), Hkv, H * D);
+  part(op.table(S::f_v_out), Hkv, (H + Hkv) * D);
+}
+// fused [B, S, (H + 2 Hkv) * D], or q [B, S, H * D] and kv [B, S, 2 Hkv * D] -> q [B, H, S, D], k [B, Hkv, S, D] (or
+// [B, Hkv, D, S] with transpose_key), v [B, Hkv, S, D]; golden tools/golden/mapping.py:5084-5186
+void runSplitQkvAndSplitHeads(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::SplitQueryKeyValueAndSplitHeadsOp;
+  Tensor in = plainOperand(ctx, op.table(S::f_in), "split_query_key_value_and_split_heads");
+  const auto &s = in.handle->shape;
+  const std::int64_t H = op.scalar<std::uint32_t>(S::f_num_heads, 0);
+  const std::int64_t Hkv = op.has(S::f_num_kv_heads) ? op.scalar<std::uint32_t>(S::f_num_kv_heads, 0) : H;
+  const bool transposeKey = op.scalar<std::uint8_t>(S::f_transpose_key, 0) != 0;
+  TTRT_ASSERT(s.size() == 3 && H >= 1 && Hkv >= 1, "split_query_key_value_and_split_heads: input must be [batch, seq, hidden]");
+  const std::uint32_t B = s[0], Sq = s[1];
+  Tensor kv;
+  std::int64_t D, Wq = s[2], Wkv, kBase, vBase;
+  if (auto kr = op.table(S::f_kv_input)) {
+    kv = plainOperand(ctx, kr, "split_query_key_value_and_split_heads kv");
+    const auto &ks = kv.handle->shape;
+    TTRT_ASSERT(ks.size() == 3 && ks[0] == B && ks[1] == Sq && Wq % H == 0 && ks[2] == 2 * Hkv * (Wq / H),
+                "split_query_key_value_and_split_heads: kv input must be [batch, seq, 2 * kv_heads * head_dim]");
+    D = Wq / H; Wkv = ks[2]; kBase = 0; vBase = Hkv * D;
+  } else {
+    TTRT_ASSERT(Wq % (H + 2 * Hkv) == 0, "split_query_key_value_and_split_heads: hidden size must be (heads + 2 kv_heads) * head_dim");
+    kv = in;
+    D = Wq / (H + 2 * Hkv); Wkv = Wq; kBase = H * D; vBase = (H + Hkv) * D;
+  }
+  const std::uint32_t d = static_cast<std::uint32_t>(D), h = static_cast<std::uint32_t>(H), hk = static_cast<std::uint32_t>(Hkv);
+  auto qRef = op.table(S::f_q_out), kRef = op.table(S::f_k_out), vRef = op.table(S::f_v_out);
+  Tensor q = stridedCopy(ctx, in, {B, h, Sq, d}, {Sq * Wq, D, Wq, 1}, 0, shapeFromTensorRef(qRef));
+  Tensor k = transposeKey ? stridedCopy(ctx, kv, {B, hk, d, Sq}, {Sq * Wkv, D, 1, Wkv}, kBase, shapeFromTensorRef(kRef))
+                          : stridedCopy(ctx, kv, {B, hk, Sq, d}, {Sq * Wkv, D, Wkv, 1}, kBase, shapeFromTensorRef(kRef));
+  Tensor v = stridedCopy(ctx, kv, {B, hk, Sq, d}, {Sq * Wkv, D, Wkv, 1}, vBase, shapeFromTensorRef(vRef));
+  ctx.put(qRef, finish(ctx, q, qRef));
+  ctx.put(kRef, finish(ctx, k, kRef));
+  ctx.put(vRef, finish(ctx, v, vRef));
+}
+
 // runtime/lib/ttnn/operations/data_movement/repeat.cpp:12-22: the input tiled repeat_dims[i] times along dim i
 void runRepeat(const fb::Table &op, ProgramContext &ctx) {
   Tensor in = onDevice(ctx, ctx.get(op.table(schema::RepeatOp::f_in), "repeat in"));
@@ -1655,6 +1767,11 @@ void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   case OpType::SliceOp: return runSlice(op, ctx);
   case OpType::RepeatInterleaveOp: return runRepeatInterleave(op, ctx);
   case OpType::RepeatOp: return runRepeat(op, ctx);
+  case OpType::ConcatenateHeadsOp: return runConcatenateHeads(op, ctx);
+  case OpType::NLPConcatHeadsOp: return runNlpConcatHeads(op, ctx);
+  case OpType::NLPConcatHeadsDecodeOp: return runNlpConcatHeadsDecode(op, ctx);
+  case OpType::NLPCreateQKVHeadsDecodeOp: return runNlpCreateQkvHeadsDecode(op, ctx);
+  case OpType::SplitQueryKeyValueAndSplitHeadsOp: return runSplitQkvAndSplitHeads(op, ctx);
   case OpType::EltwiseBinaryCompositeOp: return runEltwiseBinaryComposite(op, ctx);
   case OpType::EltwiseUnaryCompositeOp: return runEltwiseUnaryComposite(op, ctx);
   case OpType::EltwiseTernaryWhereOp: return runWhere(op, ctx);

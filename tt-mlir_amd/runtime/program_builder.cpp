@@ -655,6 +655,84 @@ ProgramBuilder::Id ProgramBuilder::repeat(Id in, const std::vector<std::int64_t>
   addOp(OpType::RepeatOp, b_.endTable(), "ttnn.repeat -> " + shapeStr(d.shape));
   return out;
 }
+ProgramBuilder::Id ProgramBuilder::concatHeads(int kind, Id in, std::uint32_t numHeads) {
+  Desc d = desc(in);
+  const auto s = d.shape;
+  if (s.size() != 4) fatal("ProgramBuilder: head merge needs a rank-4 input");
+  if (kind == 0) d.shape = {s[0], s[2], s[1] * s[3]};
+  else if (kind == 1) d.shape = {s[0], 1, s[2], s[1] * s[3]};
+  else d.shape = {1, 1, s[1], numHeads * s[3]};
+  d.storage = StorageType::Device;
+  Id out = newTensor(d);
+  Off i = tensorRef(in), o = tensorRef(out);
+  if (kind == 0) {
+    b_.startTable(ConcatenateHeadsOp::kNumFields);
+    b_.addOffset(ConcatenateHeadsOp::f_in, i);
+    b_.addOffset(ConcatenateHeadsOp::f_out, o);
+    addOp(OpType::ConcatenateHeadsOp, b_.endTable(), "ttnn.concatenate_heads " + shapeStr(d.shape));
+  } else if (kind == 1) {
+    b_.startTable(NLPConcatHeadsOp::kNumFields);
+    b_.addOffset(NLPConcatHeadsOp::f_in, i);
+    b_.addOffset(NLPConcatHeadsOp::f_out, o);
+    addOp(OpType::NLPConcatHeadsOp, b_.endTable(), "ttnn.nlp_concat_heads " + shapeStr(d.shape));
+  } else {
+    b_.startTable(NLPConcatHeadsDecodeOp::kNumFields);
+    b_.addOffset(NLPConcatHeadsDecodeOp::f_in, i);
+    b_.addOffset(NLPConcatHeadsDecodeOp::f_out, o);
+    b_.addScalarDefault<std::uint32_t>(NLPConcatHeadsDecodeOp::f_num_heads, numHeads, 0);
+    addOp(OpType::NLPConcatHeadsDecodeOp, b_.endTable(), "ttnn.nlp_concat_heads_decode " + shapeStr(d.shape));
+  }
+  return out;
+}
+std::array<ProgramBuilder::Id, 3> ProgramBuilder::nlpCreateQkvHeadsDecode(Id in, std::uint32_t numHeads, std::uint32_t numKvHeads) {
+  Desc d = desc(in);
+  const auto s = d.shape;
+  if (s.size() != 4 || s[3] % (numHeads + 2 * numKvHeads) != 0) fatal("ProgramBuilder: nlp_create_qkv_heads_decode input must be [1, 1, users, (heads + 2 kv) * dim]");
+  const std::uint32_t dim = s[3] / (numHeads + 2 * numKvHeads);
+  d.storage = StorageType::Device;
+  d.shape = {1, s[2], numHeads, dim};
+  Id q = newTensor(d);
+  d.shape = {1, s[2], numKvHeads, dim};
+  Id k = newTensor(d), v = newTensor(d);
+  using S = NLPCreateQKVHeadsDecodeOp;
+  Off i = tensorRef(in), qo = tensorRef(q), ko = tensorRef(k), vo = tensorRef(v);
+  b_.startTable(S::kNumFields);
+  b_.addOffset(S::f_input, i);
+  b_.addOffset(S::f_q_out, qo);
+  b_.addOffset(S::f_k_out, ko);
+  b_.addOffset(S::f_v_out, vo);
+  b_.addScalarDefault<std::uint32_t>(S::f_num_heads, numHeads, 0);
+  b_.addScalar<std::uint32_t>(S::f_num_kv_heads, numKvHeads);
+  addOp(OpType::NLPCreateQKVHeadsDecodeOp, b_.endTable(), "ttnn.nlp_create_qkv_heads_decode");
+  return {q, k, v};
+}
+std::array<ProgramBuilder::Id, 3> ProgramBuilder::splitQkvAndSplitHeads(Id in, Id kvInput, std::uint32_t numHeads, std::uint32_t numKvHeads,
+                                                                        bool transposeKey) {
+  Desc d = desc(in);
+  const auto s = d.shape;
+  if (s.size() != 3) fatal("ProgramBuilder: split_query_key_value_and_split_heads input must be [batch, seq, hidden]");
+  const std::uint32_t dim = kvInput ? s[2] / numHeads : s[2] / (numHeads + 2 * numKvHeads);
+  d.storage = StorageType::Device;
+  d.shape = {s[0], numHeads, s[1], dim};
+  Id q = newTensor(d);
+  d.shape = transposeKey ? std::vector<std::uint32_t>{s[0], numKvHeads, dim, s[1]} : std::vector<std::uint32_t>{s[0], numKvHeads, s[1], dim};
+  Id k = newTensor(d);
+  d.shape = {s[0], numKvHeads, s[1], dim};
+  Id v = newTensor(d);
+  using S = SplitQueryKeyValueAndSplitHeadsOp;
+  Off i = tensorRef(in), kv = kvInput ? tensorRef(kvInput) : 0, qo = tensorRef(q), ko = tensorRef(k), vo = tensorRef(v);
+  b_.startTable(S::kNumFields);
+  b_.addOffset(S::f_in, i);
+  b_.addOffset(S::f_kv_input, kv);
+  b_.addOffset(S::f_q_out, qo);
+  b_.addOffset(S::f_k_out, ko);
+  b_.addOffset(S::f_v_out, vo);
+  b_.addScalarDefault<std::uint32_t>(S::f_num_heads, numHeads, 0);
+  b_.addScalar<std::uint32_t>(S::f_num_kv_heads, numKvHeads);
+  b_.addScalarDefault<std::uint8_t>(S::f_transpose_key, transposeKey, 0);
+  addOp(OpType::SplitQueryKeyValueAndSplitHeadsOp, b_.endTable(), "ttnn.split_query_key_value_and_split_heads");
+  return {q, k, v};
+}
 ProgramBuilder::Id ProgramBuilder::binaryComposite(std::uint32_t type, Id lhs, Id rhs) {
   const auto &a = desc(lhs).shape, &b = desc(rhs).shape;
   size_t rank = std::max(a.size(), b.size());

@@ -3,6 +3,7 @@
 // test/ttmlir/Runtime/TTNN/n150/**.mlir RUN lines), so tests and benchmarks build their programs
 // here; the wire format is the reference's (include/ttmlir/Target/TTNN/*.fbs).
 #pragma once
+#include <array>
 #include <string>
 #include <vector>
 
@@ -51,6 +52,11 @@ public:
   Id repeatInterleave(Id in, std::uint32_t repeats, int dim);
   // the ops around a decoder layer (include/ttmlir/Target/TTNN/operations/{data_movement,eltwise,embedding,reduction,creation}.fbs)
   Id repeat(Id in, const std::vector<std::int64_t> &repeats);
+  // head splits and merges (include/ttmlir/Target/TTNN/operations/transformer.fbs:7-11, 34-45, 109-132); kind 0 =
+  // ConcatenateHeadsOp, 1 = NLPConcatHeadsOp, 2 = NLPConcatHeadsDecodeOp (numHeads used)
+  Id concatHeads(int kind, Id in, std::uint32_t numHeads);
+  std::array<Id, 3> nlpCreateQkvHeadsDecode(Id in, std::uint32_t numHeads, std::uint32_t numKvHeads);
+  std::array<Id, 3> splitQkvAndSplitHeads(Id in, Id kvInput, std::uint32_t numHeads, std::uint32_t numKvHeads, bool transposeKey);
   Id binaryComposite(std::uint32_t type, Id lhs, Id rhs);
   Id where(Id cond, Id a, Id b);
   Id embedding(Id indices, Id weight);
