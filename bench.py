@@ -135,6 +135,28 @@ def make_workloads(torch, hip, datagen, dev, names):
                              hip.ptr(o), hip.BF16, B, H, Hkv, S, D, 1, 0.0, s),
             "decode attention: 32 users x 32 heads (8 kv heads) x 1 token over a full 2048-position bf16 KV cache",
             dict(keep=(qt, kvt, cur, o)))
+    for nm, window in (("sdpa2048", -1), ("sdpa2048_window128", 128)):
+        if nm not in names:
+            continue
+        B, Hq, Hkv, S, D = 1, 32, 8, 2048, 128
+        qkv = [datagen.randn((B, h, S, D), seed=5 + i, dtype=torch.bfloat16).to(dev) for i, h in enumerate((Hq, Hkv, Hkv))]
+        tiles = [torch.empty_like(t) for t in qkv]
+        for t, tt, h in zip(qkv, tiles, (Hq, Hkv, Hkv)):
+            hip.call("ttm_tilize", hip.ptr(t), hip.ptr(tt), B * h, S, D, 2, s)
+        o = torch.empty_like(tiles[0])
+        torch.cuda.synchronize()
+        del qkv
+        # full causal pass: dense count, the convention of the decoder-layer figure (about half of it is computed);
+        # windowed pass: the visible (query, key) pairs only, sum_i min(i + 1, w), so the fraction is not flattered
+        visible = sum(min(i + 1, window) for i in range(S)) if window >= 0 else S * S
+        out[nm] = Workload(
+            nm, "mfma", 2.0 * 2 * B * Hq * visible * D, "flop",
+            lambda tiles=tiles, o=o, window=window: hip.call(
+                "ttm_sdpa_windowed", hip.ptr(tiles[0]), hip.ptr(tiles[1]), hip.ptr(tiles[2]), None, 1, 1, hip.ptr(o), hip.BF16, B, Hq, Hkv,
+                S, S, D, 1, 0.0, 0, window, None, s),
+            "config 5 attention alone: causal SDPA, 32 query / 8 kv heads, 2048 tokens, head_dim 128" +
+            (" (dense FLOPs counted)" if window < 0 else ", sliding window of %d keys (FLOPs of the visible pairs only)" % window),
+            dict(keep=(tiles, o)))
     # whole programs through the runtime boundary (flatbuffer -> submit -> wait)
     for nm in ("decode32", "decode32_traced"):
         if nm not in names:
@@ -264,7 +286,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="linear2048")
-    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,sdpa_decode32,mlp512,decoder2048,"
+    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,sdpa_decode32,sdpa2048,sdpa2048_window128,mlp512,decoder2048,"
                                            "decode32,decode32_traced")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
