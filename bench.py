@@ -286,7 +286,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="linear2048")
-    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,sdpa_decode32,sdpa2048,sdpa2048_window128,mlp512,decoder2048,"
+    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,sdpa_decode32,sdpa2048,mlp512,decoder2048,"
                                            "decode32,decode32_traced")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
