@@ -461,6 +461,232 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if (light < heavy) sdpa64_query_block<DT>(p, light, h, b, ldsK, ldsV);
 }
 
+// The same pass with eight wavefronts: wavefront w serves query tile w % 4 and the key half w / 4 of every 64-key pass,
+// with its own running maximum, sum and output; the two halves of a query tile are merged through LDS at the end.  A launch
+// that has only one workgroup per CU (a single sequence of a few thousand tokens) then still keeps two wavefronts on every
+// SIMD, so that one's softmax overlaps the other's matrix products; staging K and V is shared by twice as many lanes.
+template <int DT>  // head_dim / 32
+__device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *ldsK, uint16_t *ldsV) {
+  constexpr int VPITCH = kSdpaVPitch, NT = 512, CHUNKS = DT * 256, NCH = (CHUNKS + NT - 1) / NT;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int qw = wave & 3, kh = wave >> 2;
+  const int hk = h / (p.Hq / p.Hkv);
+  const int qt = qb * 4 + qw;                           // this wave's query tile
+  const bool wave_ok = qt < p.sqt;
+  const int l31 = lane & 31, hh = lane >> 5;
+  const int64_t q_mat = b * p.q_batch + h * p.q_head, o_mat = b * p.o_batch + h * p.o_head;
+  const int64_t k_mat = b * p.k_batch + hk * p.k_head, v_mat = b * p.v_batch + hk * p.v_head;
+
+  bf16x8 qf[2 * DT];
+#pragma unroll
+  for (int s = 0; s < 2 * DT; ++s) {
+    u32x4 v = {0, 0, 0, 0};
+    if (wave_ok)
+      v = *(const u32x4 *)(p.q + q_mat + qt * p.q_pitch + (s >> 1) * 2048 + ((l31 >> 4) * 2 + (s & 1)) * 512 +
+                           (l31 & 15) * 32 + hh * 16);
+    qf[s] = *(bf16x8 *)&v;
+  }
+  f32x16 o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[d][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+  const int q_glob = qt * 32 + l31, q_last = qt * 32 + 31;
+
+  const int kt_begin = first_key_tile(p, qb * 128), kt_end = end_key_tile(p, min(qb * 4 + 4, p.sqt) * 32 - 1);
+  const int kb_begin = kt_begin >> 1, kb_end = (kt_end + 1) >> 1;
+  u32x4 kreg[NCH], vreg[NCH];
+  auto load_block = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = tid + NT * i;
+      if (c < CHUNKS) {
+        const int tr = c / (DT * 128), cc = c % (DT * 128);
+        const int kt = min(2 * kb + tr, p.skt - 1);     // an odd tile count repeats the last tile; its keys are masked
+        kreg[i] = ((const u32x4 *)(p.k + k_mat + kt * p.k_pitch))[cc];
+        vreg[i] = ((const u32x4 *)(p.v + v_mat + kt * p.v_pitch))[cc];
+      }
+    }
+  };
+  if (kb_end > kb_begin) load_block(kb_begin);
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = p.scale * LOG2E;
+  if (kh == 0) sink_start(p, h, scale2, m_run, l_run);   // the sink belongs to one of the two halves only
+  for (int kb = kb_begin; kb < kb_end; ++kb) {
+    __syncthreads();  // previous block fully consumed
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = tid + NT * i;
+      if (c < CHUNKS) {   // uniform over a wavefront: CHUNKS is a multiple of 64
+        const int tr = c / (DT * 128), cc = c % (DT * 128);
+        ((u32x4 *)ldsK)[c] = kreg[i];
+        const u32x4 v = vreg[i];
+        const int tile = cc >> 7, c7 = cc & 127;
+        const int face = c7 >> 5, row = (c7 & 31) >> 1, half = c7 & 1;
+        const bool odd = row & 1;
+        const int key = 32 * tr + (face >> 1) * 16 + (row & ~1);          // even key of the pair
+        const int d0 = tile * 32 + (face & 1) * 16 + half * 8 + (odd ? 4 : 0);
+        const uint32_t send0 = odd ? v.x : v.z, send1 = odd ? v.y : v.w;
+        const uint32_t got0 = quad_xor2(send0), got1 = quad_xor2(send1);
+        const uint32_t mine0 = odd ? v.z : v.x, mine1 = odd ? v.w : v.y;
+        const uint32_t e0 = odd ? got0 : mine0, o0 = odd ? mine0 : got0;  // even key's word, odd key's word
+        const uint32_t e1 = odd ? got1 : mine1, o1 = odd ? mine1 : got1;
+        uint32_t *vt = (uint32_t *)(ldsV + d0 * VPITCH + key);
+        vt[0] = __builtin_amdgcn_perm(o0, e0, 0x05040100u);
+        vt[VPITCH / 2] = __builtin_amdgcn_perm(o0, e0, 0x07060302u);
+        vt[VPITCH] = __builtin_amdgcn_perm(o1, e1, 0x05040100u);
+        vt[3 * VPITCH / 2] = __builtin_amdgcn_perm(o1, e1, 0x07060302u);
+      }
+    }
+    __syncthreads();
+    if (kb + 1 < kb_end) load_block(kb + 1);
+    const int key_base = kb * 64 + 32 * kh;             // this wavefront's 32 keys of the pass
+    if (!wave_ok || key_base > q_last + p.hi_off || key_base + 31 < qt * 32 - p.lo_off || key_base >= p.Sk) continue;
+
+    f32x16 s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+#pragma unroll
+    for (int st = 0; st < 2 * DT; ++st) {
+      const uint8_t *kp = ldsK + kh * DT * 2048 + (st >> 1) * 2048 + ((l31 >> 4) * 2 + (st & 1)) * 512 + (l31 & 15) * 32 + hh * 16;
+      u32x4 ka = *(const u32x4 *)kp;
+      s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&ka, qf[st], s, 0, 0, 0);
+    }
+    const bool edge = key_base + 31 > qt * 32 + p.hi_off || key_base < q_last - p.lo_off || key_base + 32 > p.Sk;   // wavefront-uniform
+    float mx = -INFINITY;
+    if (p.mask || edge) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int kin = g * 8 + hh * 4;
+        const int key0 = key_base + kin;
+        float mk[4] = {0.f, 0.f, 0.f, 0.f};
+        if (p.mask) {
+          const int kt = min(2 * kb + kh, p.skt - 1);
+          const int64_t mm = ((int64_t)b * p.mask_b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
+          const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
+                              (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
+          u32x2 raw = *(const u32x2 *)mp;
+          mk[0] = __uint_as_float(raw.x << 16); mk[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+          mk[2] = __uint_as_float(raw.y << 16); mk[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+        }
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = fmaf(s[g * 4 + r], scale2, mk[r] * LOG2E);
+          const int key = key0 + r;
+          if (key >= p.Sk || key > q_glob + p.hi_off || key < q_glob - p.lo_off) v = -INFINITY;
+          s[g * 4 + r] = v;
+          mx = fmaxf(mx, v);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        s[r] *= scale2;
+        mx = fmaxf(mx, s[r]);
+      }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float m_use = m_new == -INFINITY ? 0.0f : m_new;   // fully masked so far: stay at zero without producing NaN
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+    float rs = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float e = __builtin_amdgcn_exp2f(s[r] - m_use);
+      s[r] = e;
+      rs += e;
+    }
+    rs += __shfl_xor(rs, 32);
+    l_run = l_run * alpha + rs;
+    m_run = m_new;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      u32x4 pb;
+      pb.x = pack_bf16_rne(s[8 * t + 0], s[8 * t + 1]);
+      pb.y = pack_bf16_rne(s[8 * t + 2], s[8 * t + 3]);
+      pb.z = pack_bf16_rne(s[8 * t + 4], s[8 * t + 5]);
+      pb.w = pack_bf16_rne(s[8 * t + 6], s[8 * t + 7]);
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        const uint16_t *vr = ldsV + (d * 32 + l31) * VPITCH + 32 * kh + 16 * t + 4 * hh;
+        u32x2 lo = *(const u32x2 *)vr, hi = *(const u32x2 *)(vr + 8);
+        u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va, *(bf16x8 *)&pb, o[d], 0, 0, 0);
+      }
+    }
+  }
+  // merge the two key halves of every query tile: the upper half hands over (max, sum) through the V region and its
+  // output, 4 DT values per lane at a time, through the K region (DT * 4 KiB = 256 lanes x DT float4)
+  __syncthreads();
+  float *ml = (float *)ldsV;
+  f32x4 *ox = (f32x4 *)ldsK;
+  const int slot = qw * 64 + lane;
+  if (kh == 1) { ml[2 * slot] = m_run; ml[2 * slot + 1] = l_run; }
+  __syncthreads();
+  float a0 = 1.0f, a1 = 0.0f;
+  if (kh == 0) {
+    const float m1 = ml[2 * slot], l1 = ml[2 * slot + 1];
+    const float m = fmaxf(m_run, m1), m_use = m == -INFINITY ? 0.0f : m;
+    a0 = __builtin_amdgcn_exp2f(m_run - m_use);
+    a1 = __builtin_amdgcn_exp2f(m1 - m_use);
+    l_run = l_run * a0 + l1 * a1;
+  }
+#pragma unroll
+  for (int r4 = 0; r4 < 4; ++r4) {
+    if (kh == 1) {
+#pragma unroll
+      for (int d = 0; d < DT; ++d) ox[slot * DT + d] = f32x4{o[d][4 * r4], o[d][4 * r4 + 1], o[d][4 * r4 + 2], o[d][4 * r4 + 3]};
+    }
+    __syncthreads();
+    if (kh == 0) {
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        const f32x4 x = ox[slot * DT + d];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[d][4 * r4 + e] = o[d][4 * r4 + e] * a0 + x[e] * a1;
+      }
+    }
+    __syncthreads();
+  }
+  if (kh != 0 || !wave_ok) return;   // no barrier follows inside this block; the next block starts with one
+  const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+  const bool q_ok = q_glob < p.Sq;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int din = g * 8 + hh * 4;
+      u32x2 ov;
+      ov.x = q_ok ? pack_bf16_rne(o[d][g * 4 + 0] * inv, o[d][g * 4 + 1] * inv) : 0u;
+      ov.y = q_ok ? pack_bf16_rne(o[d][g * 4 + 2] * inv, o[d][g * 4 + 3] * inv) : 0u;
+      uint8_t *op = p.out + o_mat + qt * p.o_pitch + d * 2048 +
+                    (((l31 >> 4) * 2 + (din >> 4)) * 256 + (l31 & 15) * 16 + (din & 15)) * 2;
+      *(u32x2 *)op = ov;
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(512) void ttm_sdpa64_split_k(SdpaArgs p, int paired) {
+  constexpr int D = DT * 32;
+  __shared__ __attribute__((aligned(16))) uint8_t ldsK[64 * D * 2];
+  __shared__ __attribute__((aligned(16))) uint16_t ldsV[D * kSdpaVPitch];
+  const int nqb = (p.sqt + 3) / 4, h = blockIdx.y, b = blockIdx.z;
+  if (!paired) {
+    sdpa64_split_block<DT>(p, nqb - 1 - (int)blockIdx.x, h, b, ldsK, ldsV);
+    return;
+  }
+  const int heavy = nqb - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
+  sdpa64_split_block<DT>(p, heavy, h, b, ldsK, ldsV);
+  if (light < heavy) sdpa64_split_block<DT>(p, light, h, b, ldsK, ldsV);   // workgroup-uniform
+}
+
 static int sdpa_entry(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B,
                       int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int heads_inner, int64_t window,
                       const void *sink, int64_t mask_batch, void *stream) {
@@ -505,6 +731,22 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
   const int nqb = (int)ttm_cdiv(p.sqt, 4);
   const int paired = is_causal && nqb >= 2 && variant != 2;
   const dim3 grid64(paired ? (unsigned)((nqb + 1) / 2) : (unsigned)nqb, (unsigned)Hq, (unsigned)B);
+  // eight wavefronts per workgroup (two key halves per query tile) when the launch would otherwise leave every SIMD with a
+  // single wavefront: fewer workgroups than twice the CUs.  sdpa_variant 3 forces it, 4 forbids it.
+  int cus = 0, devid = 0;
+  if (hipGetDevice(&devid) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, devid) != hipSuccess || cus <= 0) cus = 256;
+  const int64_t wgs = (int64_t)grid64.x * grid64.y * grid64.z;
+  const bool split = wide && D <= 128 && (variant == 3 || (variant == 0 && wgs < 2 * (int64_t)cus));
+  if (split) {
+    const dim3 block8(512);
+    switch (D) {
+    case 32: hipLaunchKernelGGL(ttm_sdpa64_split_k<1>, grid64, block8, 0, s, p, paired); break;
+    case 64: hipLaunchKernelGGL(ttm_sdpa64_split_k<2>, grid64, block8, 0, s, p, paired); break;
+    default: hipLaunchKernelGGL(ttm_sdpa64_split_k<4>, grid64, block8, 0, s, p, paired); break;
+    }
+    TTM_LAUNCH_CHECK();
+    return TTM_OK;
+  }
   switch (D) {
   case 32: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<1>, grid64, block, 0, s, p, paired); else hipLaunchKernelGGL(ttm_sdpa_k<1>, grid, block, 0, s, p); break;
   case 64: if (wide) hipLaunchKernelGGL(ttm_sdpa64_k<2>, grid64, block, 0, s, p, paired); else hipLaunchKernelGGL(ttm_sdpa_k<2>, grid, block, 0, s, p); break;
