@@ -295,7 +295,7 @@ def test_copy_view_at_positions_the_destination_from_device_memory(hip, dev, ele
     (1, 2, 2, 160, 96, 128, False, None), (1, 4, 1, 33, 33, 128, True, None), (1, 2, 2, 96, 224, 64, False, "bh"),
     (2, 4, 4, 130, 190, 128, False, "b1"), (1, 4, 2, 192, 320, 128, True, None), (1, 2, 1, 320, 192, 32, True, None),
     (1, 8, 2, 1024, 1024, 128, True, None)])
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 3, 4])   # automatic, 32-key kernel, eight-wavefront kernel forced / forbidden
 def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask, variant):
     if variant == 1 and Sq * Sk >= 512 * 512:
         pytest.skip("the 32-key kernel is covered by the small shapes")
@@ -326,7 +326,7 @@ def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask, variant):
     assert metrics.get_pcc(want, res) >= 0.9999
 
 
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, 4])
 @pytest.mark.parametrize("flags", [15, 1, 6, 8, 9])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", [(1, 8, 2, 256, 256, 128, True), (2, 4, 4, 96, 160, 64, False), (1, 4, 1, 70, 70, 32, True),
                                                       (1, 2, 2, 40, 300, 256, False)])
@@ -361,7 +361,7 @@ def test_sdpa_heads_inner_equals_the_head_major_call(hip, dev, B, Hq, Hkv, Sq, S
     assert torch.equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant", [0, 1, 2, 4])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,window,sink,mask,flags", [
     (1, 4, 2, 256, 256, 128, True, 64, False, None, 0), (1, 4, 2, 256, 256, 128, True, 1, False, None, 0),
     (1, 4, 2, 300, 300, 64, True, 100, True, None, 0), (2, 2, 2, 96, 160, 128, False, 40, False, None, 0),
