@@ -131,8 +131,9 @@ def make_workloads(torch, hip, datagen, dev, names):
         del kv
         out["sdpa_decode32"] = Workload(
             "sdpa_decode32", "hbm", 2 * B * Hkv * S * D * 2 + 2 * B * H * D * 2, "bytes",
-            lambda: hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kvt[0]), hip.ptr(kvt[1]), hip.ptr(cur), None, 1, None, 0, 0,
-                             hip.ptr(o), hip.BF16, B, H, Hkv, S, D, 1, 0.0, s),
+            lambda qt=qt, kvt=kvt, cur=cur, o=o, B=B, H=H, Hkv=Hkv, S=S, D=D: hip.call(
+                "ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kvt[0]), hip.ptr(kvt[1]), hip.ptr(cur), None, 1, None, 0, 0,
+                hip.ptr(o), hip.BF16, B, H, Hkv, S, D, 1, 0.0, s),
             "decode attention: 32 users x 32 heads (8 kv heads) x 1 token over a full 2048-position bf16 KV cache",
             dict(keep=(qt, kvt, cur, o)))
     for nm, window in (("sdpa2048", -1), ("sdpa2048_window128", 128)):
@@ -151,7 +152,7 @@ def make_workloads(torch, hip, datagen, dev, names):
         visible = sum(min(i + 1, window) for i in range(S)) if window >= 0 else S * S
         out[nm] = Workload(
             nm, "mfma", 2.0 * 2 * B * Hq * visible * D, "flop",
-            lambda tiles=tiles, o=o, window=window: hip.call(
+            lambda tiles=tiles, o=o, window=window, B=B, Hq=Hq, Hkv=Hkv, S=S, D=D: hip.call(
                 "ttm_sdpa_windowed", hip.ptr(tiles[0]), hip.ptr(tiles[1]), hip.ptr(tiles[2]), None, 1, 1, hip.ptr(o), hip.BF16, B, Hq, Hkv,
                 S, S, D, 1, 0.0, 0, window, None, s),
             "config 5 attention alone: causal SDPA, 32 query / 8 kv heads, 2048 tokens, head_dim 128" +
