@@ -732,11 +732,13 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
   const int paired = is_causal && nqb >= 2 && variant != 2;
   const dim3 grid64(paired ? (unsigned)((nqb + 1) / 2) : (unsigned)nqb, (unsigned)Hq, (unsigned)B);
   // eight wavefronts per workgroup (two key halves per query tile) when the launch would otherwise leave every SIMD with a
-  // single wavefront: fewer workgroups than twice the CUs.  sdpa_variant 3 forces it, 4 forbids it.
+  // single wavefront: no more workgroups than CUs (only one eight-wavefront workgroup fits a CU, so a larger launch would
+  // take a second round where the four-wavefront kernel runs two workgroups side by side).  sdpa_variant 3 forces it, 4
+  // forbids it.
   int cus = 0, devid = 0;
   if (hipGetDevice(&devid) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, devid) != hipSuccess || cus <= 0) cus = 256;
   const int64_t wgs = (int64_t)grid64.x * grid64.y * grid64.z;
-  const bool split = wide && D <= 128 && (variant == 3 || (variant == 0 && wgs < 2 * (int64_t)cus));
+  const bool split = wide && D <= 128 && (variant == 3 || (variant == 0 && wgs <= (int64_t)cus));
   if (split) {
     const dim3 block8(512);
     switch (D) {
