@@ -141,22 +141,26 @@ def test_batched_matmul(hip, dev, orc, metrics):
 
 
 @pytest.mark.parametrize("M", [32, 2048])
-def test_c3_linear_band(hip, dev, orc, metrics, M):
-    """Config 3 at full size; the oracle checks a band of rows and columns it finishes in seconds."""
+def test_c3_linear_full_size(hip, dev, orc, metrics, M):
+    """Config 3 at full size, every one of the M x 14336 outputs against the oracle (all host cores: 240 GFLOP at
+    M = 2048)."""
     a, w, bias = datagen.c3_linear(M)
     got, w_eff = run_linear(hip, dev, a, w, bias, "gelu", hip.BFP8B)
-    rows = slice(0, 32) if M == 32 else slice(1000, 1032)
-    # two column bands, one in each round of blocks at M = 2048
-    for cols in (slice(7000, 7512), slice(13900, 14336)):
-        want = orc.round_bf16(orc.linear(a[rows].float().numpy(), w_eff[:, cols].contiguous().numpy(),
-                                         bias[cols].float().numpy(), "gelu"))
-        g = got[rows, cols].float().numpy()
-        # |y| up to ~6 -> bf16 ulp 2^-5; accumulation over K=4096 in a different order adds less than that
-        assert np.max(np.abs(g - want)) <= 2.0 ** -5
-        assert metrics.get_pcc(want, g) >= 0.99
+    orc.set_threads(orc.max_threads())
+    try:
+        want = orc.round_bf16(orc.linear(a.float().numpy(), w_eff.contiguous().numpy(), bias.float().numpy(), "gelu"))
+    finally:
+        orc.set_threads(1)
+    g = got.float().numpy()
+    assert g.shape == want.shape == (M, 14336)
+    # |y| up to ~6 -> bf16 ulp 2^-5; accumulation over K=4096 in a different order adds less than that
+    assert np.max(np.abs(g - want)) <= 2.0 ** -5
+    assert metrics.get_pcc(want, g) >= 0.9999
+    assert np.mean(g == want) >= 0.98                  # the rest are single bf16 roundings at ties
     # quantisation itself against the unquantised weights: the reference's own bar for bfp8 weights
-    ref = torch.nn.functional.gelu(a[rows].float() @ w[:, cols] + bias[cols].float())
-    assert metrics.get_pcc(ref.numpy(), g) >= 0.99
+    rows = slice(0, 32) if M == 32 else slice(1000, 1032)
+    ref = torch.nn.functional.gelu(a[rows].float() @ w + bias.float())
+    assert metrics.get_pcc(ref.numpy(), g[rows]) >= 0.99
     # linearity in the activations at full size: f(2a) - 2 f(a) == 0 without bias/activation (exact in bf16/f32)
     g1, _ = run_linear(hip, dev, a, w, None, None, hip.BFP8B)
     g2, _ = run_linear(hip, dev, (a.float() * 2).to(torch.bfloat16), w, None, None, hip.BFP8B)

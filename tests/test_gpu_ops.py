@@ -326,6 +326,32 @@ def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask, variant):
     assert metrics.get_pcc(want, res) >= 0.9999
 
 
+def test_sdpa_config5_shape(hip, dev, orc):
+    """The attention of config 5 alone: 32 query / 8 kv heads, 2048 x 2048 causal, head dim 128 (one workgroup per CU, the
+    eight-wavefront kernel), every output against the oracle."""
+    import oracle.metrics as metrics
+    B, Hq, Hkv, S, D = 1, 32, 8, 2048, 128
+    q = datagen.randn((B, Hq, S, D), seed=112, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, S, D), seed=113, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, S, D), seed=114, dtype=torch.bfloat16)
+    qt, kt, vt = (tilize_dev(hip, t, dev) for t in (q, k, v))
+    out = torch.full_like(qt, float("nan"))
+    hip.call("ttm_sdpa", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, S, S, D, 1, 0.0,
+             hip.current_stream())
+    res = untilize_dev(hip, out, q.shape, dev).float().cpu().numpy()
+    orc.set_threads(orc.max_threads())
+    try:
+        want = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, is_causal=True)
+    finally:
+        orc.set_threads(1)
+    assert np.all(np.isfinite(res))
+    # probabilities are rounded to bf16 before P.V (relative 2^-9 each) and the output once more
+    assert np.max(np.abs(res - want)) <= 2.0 ** -6
+    assert metrics.get_pcc(want, res) >= 0.9999
+    # the first query of every head sees one key: the output is that value row, exactly
+    assert np.array_equal(res[0, :, 0, :], np.repeat(v.float().numpy()[0, :, 0, :], Hq // Hkv, axis=0))
+
+
 @pytest.mark.parametrize("variant", [0, 1, 4])
 @pytest.mark.parametrize("flags", [15, 1, 6, 8, 9])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", [(1, 8, 2, 256, 256, 128, True), (2, 4, 4, 96, 160, 64, False), (1, 4, 1, 70, 70, 32, True),
