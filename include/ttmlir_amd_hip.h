@@ -322,6 +322,21 @@ int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const 
                              int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                              const void *attention_sink, void *stream);
 
+/* ttm_sdpa_decode_windowed that allocates nothing.  It has no counterpart in the reference; it is for callers that cannot
+ * call hipMalloc: code under HIP graph capture, tight serving loops, harnesses that forbid allocation.  Same arguments, same
+ * kernels and bit-identical results; the per-slice partial results (max, sum, unnormalised output) go to a static device
+ * array of 8 MiB that the library holds on every GPU it runs on until the process ends, instead of the stream's grow-only
+ * workspace.  A call whose partial results need more (batch * kv_heads * slices * min(heads / kv_heads, 8) * (head_dim + 2)
+ * floats; the config-5 decode shape of 32 users x 8 kv heads x 2048 positions takes 1 MiB) fails with TTM_ERR_INVALID and
+ * launches nothing.  No hipMalloc, hipFree or allocating library call is made; the first call on a device looks the
+ * array's address up (hipGetSymbolAddress), so make that call outside a capture.  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU (different streams) race; calls on one stream are ordered and safe. */
+int ttm_sdpa_decode_static(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
+                           int mask_heads, int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user,
+                           int64_t page_block, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
+                           int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
+                           const void *attention_sink, void *stream);
+
 /* Kernel-variant selection for measurement (name -> small integer); unknown names fail. */
 int ttm_set_option(const char *name, int value);
 int ttm_get_option(const char *name, int *value);

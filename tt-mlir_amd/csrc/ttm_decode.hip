@@ -1,5 +1,7 @@
 // Decode-path transformer kernels: rotary embedding, KV-cache update / fill, single-token attention over a KV cache.
 // All tensors are TILE layout (32 x 32 tiles of four 16 x 16 faces); every kernel here is bound by HBM bandwidth.
+#include <mutex>
+
 #include "ttm_common.h"
 
 namespace {
@@ -584,10 +586,36 @@ TTM_EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_
   return TTM_OK;
 }
 
+// ---- scratch of ttm_sdpa_decode_static: the per-slice (max, sum, output) slots live in a device array of the library's
+// own instead of the stream's workspace, so that entry point never allocates.  Every GPU holds its own copy of the array at
+// its own address until the process ends; in host code the array's name is only a handle for hipGetSymbolAddress, the
+// kernels get the address that call returned for the current device.
+constexpr size_t kDecodeScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) float scratch[kDecodeScratchBytes / sizeof(float)];
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static float *g_scratch_ptr[kMaxDevices];   // per device, set on the first call with that device current
+
+static int decode_scratch_ptr(void **ptr) {
+  int dev = 0;
+  TTM_HIP(hipGetDevice(&dev));
+  TTM_REQUIRE(dev >= 0 && dev < kMaxDevices, "ttm_sdpa_decode_static: device ordinal %d beyond %d", dev, kMaxDevices);
+  std::lock_guard<std::mutex> g(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    float *d = nullptr;
+    TTM_HIP(hipGetSymbolAddress((void **)&d, HIP_SYMBOL(scratch)));
+    TTM_REQUIRE(d != nullptr, "ttm_sdpa_decode_static: hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = d;
+  }
+  *ptr = g_scratch_ptr[dev];
+  return TTM_OK;
+}
+
 static int sdpa_decode_entry(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
                              const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out, int dtype, int64_t batch,
                              int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads,
-                             int64_t window, const void *sink, int64_t mask_batch, void *stream) {
+                             int64_t window, const void *sink, int64_t mask_batch, bool static_scratch, void *stream) {
   TTM_REQUIRE(q && k && v && out, "ttm_sdpa_decode: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_sdpa_decode: tensors must be BFloat16");
   TTM_REQUIRE(batch > 0 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "ttm_sdpa_decode: heads must be a multiple of kv heads");
@@ -621,7 +649,16 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
   TTM_REQUIRE(!mask || mask_batch == 1 || mask_batch == batch, "ttm_sdpa_decode: mask batch must be 1 or %lld", (long long)batch);
   p.mask_b = mask_batch == 1 ? 0 : 1;
   void *ws = nullptr;
-  if (int rc = ttm_stream_workspace(s, (size_t)(batch * kv_heads * splits * G * (head_dim + 2)) * sizeof(float), &ws)) return rc;
+  const size_t part_bytes = (size_t)(batch * kv_heads * splits * G * (head_dim + 2)) * sizeof(float);
+  if (static_scratch) {
+    TTM_REQUIRE(part_bytes <= kDecodeScratchBytes,
+                "ttm_sdpa_decode_static: the per-slice partial results of this call take %zu bytes, the static scratch holds %zu "
+                "(batch * kv_heads * slices * heads-per-kv-head * (head_dim + 2) floats): use ttm_sdpa_decode_windowed",
+                part_bytes, (size_t)kDecodeScratchBytes);
+    if (int rc = decode_scratch_ptr(&ws)) return rc;
+  } else {
+    if (int rc = ttm_stream_workspace(s, part_bytes, &ws)) return rc;
+  }
   p.part = (float *)ws;
   for (int64_t g0 = 0; g0 < Gt; g0 += kMaxG) {   // the launches of one call follow each other on the stream and share the workspace
     p.g0 = (int)g0;
@@ -640,7 +677,7 @@ TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, cons
                                int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
                                int is_causal, float scale, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
-                           seq, head_dim, is_causal, scale, 0, -1, nullptr, batch, stream);
+                           seq, head_dim, is_causal, scale, 0, -1, nullptr, batch, false, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
@@ -648,7 +685,7 @@ TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const 
                                             void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
                                             int64_t head_dim, int is_causal, float scale, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
-                           seq, head_dim, is_causal, scale, 1, -1, nullptr, batch, stream);
+                           seq, head_dim, is_causal, scale, 1, -1, nullptr, batch, false, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
@@ -657,5 +694,15 @@ TTM_EXPORT int ttm_sdpa_decode_windowed(const void *q, const void *k, const void
                                         int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                                         const void *attention_sink, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
-                           seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, stream);
+                           seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, false, stream);
+}
+
+// ttm_sdpa_decode_windowed for callers that cannot allocate: the slots come from the library's static device array.
+TTM_EXPORT int ttm_sdpa_decode_static(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
+                                      int mask_heads, int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user,
+                                      int64_t page_block, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
+                                      int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
+                                      const void *attention_sink, void *stream) {
+  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
+                           seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, true, stream);
 }
