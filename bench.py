@@ -132,7 +132,7 @@ def make_workloads(torch, hip, datagen, dev, names):
         out["sdpa_decode32"] = Workload(
             "sdpa_decode32", "hbm", 2 * B * Hkv * S * D * 2 + 2 * B * H * D * 2, "bytes",
             lambda qt=qt, kvt=kvt, cur=cur, o=o, B=B, H=H, Hkv=Hkv, S=S, D=D: hip.call(
-                "ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kvt[0]), hip.ptr(kvt[1]), hip.ptr(cur), None, 1, None, 0, 0,
+                "ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kvt[0]), hip.ptr(kvt[1]), hip.ptr(cur), None, 1, None, 0, 0, 0,
                 hip.ptr(o), hip.BF16, B, H, Hkv, S, D, 1, 0.0, s),
             "decode attention: 32 users x 32 heads (8 kv heads) x 1 token over a full 2048-position bf16 KV cache",
             dict(keep=(qt, kvt, cur, o)))

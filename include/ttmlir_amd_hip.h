@@ -266,7 +266,8 @@ int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const void *m
  *   (operations/transformer/scaled_dot_product_attention_decode.cpp, paged_scaled_dot_product_attention_decode.cpp;
  *   golden mapping.py:2417-2481): q / out [1, batch, heads, head_dim]; k / v [batch, kv_heads, seq, head_dim], or with a
  *   page table [batch, pages_per_user] pages [blocks, kv_heads, page_block, head_dim] where seq = pages_per_user *
- *   page_block; BFloat16.  scores = (q k^T + mask) * scale, mask additive BFloat16 [batch, 1, mask_heads, seq] or NULL;
+ *   page_block and page_blocks = blocks (page-table entries outside [0, page_blocks), e.g. -1 in an unused slot, mask the
+ *   keys of that page instead of being followed); BFloat16.  scores = (q k^T + mask) * scale, mask additive BFloat16 [batch, 1, mask_heads, seq] or NULL;
  *   with is_causal and cur_pos [batch] keys after cur_pos[b] are excluded; scale <= 0 means 1/sqrt(head_dim); softmax in
  *   fp32.  Uses the stream's workspace for per-slice partial results.  Up to 8 query heads per kv head are served by one
  *   launch; more (multi-query attention) by several launches over the same cache.
@@ -298,7 +299,7 @@ int ttm_paged_fill_cache(void *cache, const void *input, const int32_t *page_tab
 int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t users, int64_t heads, int64_t max_seq,
                    int64_t head_dim, int64_t seq, int64_t batch_offset, void *stream);
 int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
-                    const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out, int dtype,
+                    const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
                     int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal,
                     float scale, void *stream);
 /* ttm_sdpa_decode whose output already has its heads concatenated: out is the [batch, heads * head_dim] TILE matrix that
@@ -306,7 +307,7 @@ int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *
  * a reshape would make of [1, batch, heads, head_dim]; padding rows below the last user are written as zeros. */
 int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
                                  int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block,
-                                 void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
+                                 int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
                                  int64_t head_dim, int is_causal, float scale, void *stream);
 /* ttm_sdpa_decode / ttm_sdpa_decode_concat_heads (concat_heads = 0 / 1) with the op's sliding_window_size and
  * attention_sink (runtime/lib/ttnn/operations/transformer/scaled_dot_product_attention_decode.cpp:36-50,
@@ -318,8 +319,8 @@ int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, co
  * seq] with mask_batch 1 (shared by the users) or batch (TTNNOps.td:4123-4125). */
 int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
                              int mask_heads, int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user,
-                             int64_t page_block, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
-                             int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
+                             int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads,
+                             int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                              const void *attention_sink, void *stream);
 
 /* ttm_sdpa_decode_windowed that allocates nothing.  It has no counterpart in the reference; it is for callers that cannot
@@ -333,8 +334,8 @@ int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const 
  * calls that overlap in time on one GPU (different streams) race; calls on one stream are ordered and safe. */
 int ttm_sdpa_decode_static(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
                            int mask_heads, int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user,
-                           int64_t page_block, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
-                           int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
+                           int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads,
+                           int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                            const void *attention_sink, void *stream);
 
 /* Kernel-variant selection for measurement (name -> small integer); unknown names fail. */

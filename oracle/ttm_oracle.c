@@ -590,7 +590,9 @@ void orc_fill_cache_f32(float *cache, const float *input, int64_t H, int64_t S, 
 
 /* Attention of one new token (tools/golden/mapping.py:2417-2481): q [1,B,H,D], k / v [B,Hkv,S,D], mask (optional)
  * [B,1,mask_heads,S] additive BEFORE the scale, cur_pos (optional, with is_causal) excludes keys j > cur_pos[b];
- * scale <= 0 means 1/sqrt(D).  out [1,B,H,D].
+ * scale <= 0 means 1/sqrt(D), the op's documented default (include/ttmlir/Dialect/TTNN/IR/TTNNOps.td:4130); the golden
+ * leaves the logits unscaled when `scale is None` (mapping.py:2472), a deviation from it taken on purpose, since the
+ * runtime passes the absent attribute on to the kernel, which applies the default.  out [1,B,H,D].
  * window >= 0: of the keys up to the decode position p only the last `window` are visible, [max(0, p - window + 1), p]
  * (mapping.py:8814-8824, the paged golden); p = cur_pos[b], or S - 1 without cur_pos, as the op's description has it
  * (include/ttmlir/Dialect/TTNN/IR/TTNNOps.td:4131-4134; the golden leaves the window out when cur_pos is absent).

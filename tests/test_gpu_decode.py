@@ -108,7 +108,7 @@ def _decode_case(hip, dev, orc, B, H, Hkv, S, D, cur, mask_heads=None, causal=Tr
         kt, vt = tilize_dev(hip, k, dev), tilize_dev(hip, v, dev)
     out = torch.full_like(qt, float("nan"))
     hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp) if cp is not None else None,
-             hip.ptr(mt) if mt is not None else None, mask_heads or 1, hip.ptr(table) if table is not None else None, pages, block,
+             hip.ptr(mt) if mt is not None else None, mask_heads or 1, hip.ptr(table) if table is not None else None, pages, block, (B * pages if table is not None else 0),
              hip.ptr(out), hip.BF16, B, H, Hkv, S, D, int(causal), scale, hip.current_stream())
     got = f32(untilize_dev(hip, out, q.shape, dev))
     want = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur, mask=None if m is None else f32(m), is_causal=causal,
@@ -159,7 +159,7 @@ def test_sdpa_decode_ignores_garbage_after_the_current_position(hip, dev, orc):
     cp = torch.tensor(cur, dtype=torch.int32, device=dev)
     qt, kt, vt = (tilize_dev(hip, t, dev) for t in (q, kb, vb))
     out = torch.full_like(qt, float("nan"))
-    hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, None, 0, 0, hip.ptr(out), hip.BF16,
+    hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, None, 0, 0, 0, hip.ptr(out), hip.BF16,
              B, H, Hkv, S, D, 1, 0.0, hip.current_stream())
     got = f32(untilize_dev(hip, out, q.shape, dev))
     want = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur)
@@ -169,14 +169,58 @@ def test_sdpa_decode_ignores_garbage_after_the_current_position(hip, dev, orc):
 def test_sdpa_decode_rejects_unsupported(hip, dev):
     z = torch.zeros(1 << 16, dtype=torch.bfloat16, device=dev)
     with pytest.raises(hip.TTMError, match="multiple of kv heads"):
-        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, hip.ptr(z), hip.BF16, 1, 16, 3, 32, 32,
+        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, 0, hip.ptr(z), hip.BF16, 1, 16, 3, 32, 32,
                  1, 0.0, hip.current_stream())
     with pytest.raises(hip.TTMError, match="multiple of 32"):
-        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, hip.ptr(z), hip.BF16, 1, 8, 8, 40, 32,
+        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, None, 0, 0, 0, hip.ptr(z), hip.BF16, 1, 8, 8, 40, 32,
                  1, 0.0, hip.current_stream())
     with pytest.raises(hip.TTMError, match="page table"):
-        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, hip.ptr(z), 3, 32, hip.ptr(z), hip.BF16, 1, 8, 8,
+        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, hip.ptr(z), 3, 32, 8, hip.ptr(z), hip.BF16, 1, 8, 8,
                  64, 32, 1, 0.0, hip.current_stream())
+    with pytest.raises(hip.TTMError, match="number of blocks"):
+        hip.call("ttm_sdpa_decode", hip.ptr(z), hip.ptr(z), hip.ptr(z), None, None, 1, hip.ptr(z), 2, 32, 0, hip.ptr(z), hip.BF16, 1, 8, 8,
+                 64, 32, 1, 0.0, hip.current_stream())
+
+
+def test_sdpa_decode_page_table_entries_outside_the_cache_are_masked(hip, dev, orc):
+    """Unused slots of a page table hold -1 (or stale numbers): a slot within [0, cur_pos] that names no block of the cache
+    masks its keys instead of being followed, and slots past cur_pos are not looked at; non-causal calls mask them too."""
+    B, H, Hkv, S, D, block = 3, 8, 2, 512, 64, 64
+    pages = S // block
+    q = datagen.randn((1, B, H, D), seed=150, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, S, D), seed=151, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, S, D), seed=152, dtype=torch.bfloat16)
+    cur = [300, 511, 64]
+    g = torch.Generator().manual_seed(153)
+    table = torch.randperm(B * pages, generator=g).reshape(B, pages).to(torch.int32)
+    kp = torch.zeros((B * pages, Hkv, block, D), dtype=torch.bfloat16)
+    vp = torch.zeros_like(kp)
+    for b in range(B):
+        for pg in range(pages):
+            kp[table[b, pg]] = k[b, :, pg * block:(pg + 1) * block]
+            vp[table[b, pg]] = v[b, :, pg * block:(pg + 1) * block]
+    bad = table.clone()
+    bad[0, 5:] = -1                 # past user 0's position (300 is in page 4)
+    bad[0, 2] = -1                  # inside it: keys 128..191 drop out
+    bad[1, 7] = B * pages + 5       # beyond the cache: keys 448..511 drop out
+    bad[2, 2:] = -1
+    # what the kernel must do, written for the oracle as a mask (with a mask the golden leaves the position test to the
+    # mask, tools/golden/mapping.py:2459-2470): keys past the position, and the keys of the two dropped pages
+    mask = np.zeros((B, 1, 1, S), dtype=np.float32)
+    for b in range(B):
+        mask[b, ..., cur[b] + 1:] = -np.inf
+    mask[0, ..., 128:192] = -np.inf
+    mask[1, ..., 448:512] = -np.inf
+    qt, kt, vt = tilize_dev(hip, q, dev), tilize_dev(hip, kp, dev), tilize_dev(hip, vp, dev)
+    cp, td = torch.tensor(cur, dtype=torch.int32, device=dev), bad.to(dev)
+    out = torch.full_like(qt, float("nan"))
+    hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, hip.ptr(td), pages, block, B * pages,
+             hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 1, 0.0, hip.current_stream())
+    got = f32(untilize_dev(hip, out, q.shape, dev))
+    want = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur, mask=mask, is_causal=True)
+    assert np.all(np.isfinite(got)) and np.max(np.abs(got - want)) <= 2.0 ** -6
+    plain = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur, is_causal=True)
+    assert np.max(np.abs(plain[0, :2] - want[0, :2])) > 0.02       # the dropped pages matter
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -274,7 +318,7 @@ def test_sdpa_decode_concat_heads_equals_reshape_of_the_plain_output(hip, dev, B
     cp = torch.randint(0, S, (B,), generator=torch.Generator().manual_seed(93), dtype=torch.int32).to(dev)
     qt, kt, vt = tilize_dev(hip, q, dev), tilize_dev(hip, k, dev), tilize_dev(hip, v, dev)
     plain = torch.full_like(qt, float("nan"))
-    args = lambda out: (hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, None, 0, 0, hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 1, 0.0,
+    args = lambda out: (hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, None, 0, 0, 0, hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 1, 0.0,
                         hip.current_stream())
     hip.call("ttm_sdpa_decode", *args(plain))
     Bp = (B + 31) // 32 * 32
@@ -334,7 +378,7 @@ def test_sdpa_decode_sliding_window_and_attention_sink(hip, dev, orc, B, H, Hkv,
     Bp = (B + 31) // 32 * 32
     out = torch.full((Bp * H * D,), float("nan"), dtype=torch.bfloat16, device=dev) if concat else torch.full_like(qt, float("nan"))
     hip.call("ttm_sdpa_decode_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp) if use_pos else None, None, 1, 1,
-             hip.ptr(table_d) if paged else None, pages, block, hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 1, 0.0, concat,
+             hip.ptr(table_d) if paged else None, pages, block, B * pages, hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 1, 0.0, concat,
              -1 if window is None else window, hip.ptr(st) if sink else None, hip.current_stream())
     got = f32(untilize_dev(hip, out, (B, H * D), dev)).reshape(1, B, H, D) if concat else f32(untilize_dev(hip, out, q.shape, dev))
     want = orc.sdpa_decode(f32(q), f32(k), f32(v), cur_pos=cur.numpy() if use_pos else None, sliding_window=window,
@@ -359,7 +403,7 @@ def test_sdpa_decode_mask_shared_by_the_users(hip, dev, orc, mask_batch, mask_he
     sk = (datagen.randn((H, 1), seed=144, dtype=torch.bfloat16) * 4).expand(H, 32).contiguous()
     qt, kt, vt, mt, st = (tilize_dev(hip, t, dev) for t in (q, k, v, m, sk))
     out = torch.full_like(qt, float("nan"))
-    hip.call("ttm_sdpa_decode_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, hip.ptr(mt), mask_heads, mask_batch, None, 0, 0,
+    hip.call("ttm_sdpa_decode_windowed", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, hip.ptr(mt), mask_heads, mask_batch, None, 0, 0, 0,
              hip.ptr(out), hip.BF16, B, H, Hkv, S, D, 0, 0.0, 0, 100, hip.ptr(st), hip.current_stream())
     got = f32(untilize_dev(hip, out, q.shape, dev))
     want = orc.sdpa_decode(f32(q), f32(k), f32(v), mask=f32(m), is_causal=False, sliding_window=100, attention_sink=f32(sk))

@@ -68,10 +68,19 @@ def test_to_layout_round_trip(device, orc, shape, dtype):
         assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
         raw = rt.to_numpy(rt.to_host(d, untilize=False)[0])   # packed tile bytes, bit exact
         assert np.array_equal(raw, orc.bfp_pack(x2, fmt))
+    # one decision for both sides (runtime/lib/ttnn/runtime.cpp:906-932): retain defaults to the input's own flag, the
+    # result carries it, and the input is consumed exactly when it is off
     keep = rt.from_torch(x)
     keep.set_retain(True)
-    rt.to_layout(keep, device, rt.Layout(ST.Device, TL.Tile, DT.BFloat16))
-    assert keep.is_allocated()
+    r1 = rt.to_layout(keep, device, rt.Layout(ST.Device, TL.Tile, DT.BFloat16))
+    assert keep.is_allocated() and r1.get_retain()
+    # a host input reused across loops, as tools/ttrt/common/util.py:269 does with to_layout(inputs[i], device, layout, True)
+    loop_in = rt.from_torch(x)
+    for _ in range(2):
+        r2 = rt.to_layout(loop_in, device, rt.Layout(ST.Device, TL.Tile, DT.BFloat16), retain=True)
+        assert loop_in.is_allocated() and r2.get_retain()
+    r3 = rt.to_layout(loop_in, device, rt.Layout(ST.Device, TL.Tile, DT.BFloat16), retain=False)
+    assert not loop_in.is_allocated() and not r3.get_retain()
 
 
 def test_c3_linear_program_and_const_eval_cache(device, orc, metrics):
@@ -367,6 +376,59 @@ def test_hooks_can_read_and_replace_pool_tensors(device, orc):
     (y2,) = harness.execute(binary, 1, tins, device)
     want = oracle_mlp(orc, f(d["x"]), f(d["norm_w"]), f(bf(d["wg"])), f(bf(d["wu"])), f(bf(d["wd"])), 1e-5)
     assert np.max(np.abs(f(y2) - want)) <= 2.0 ** -10
+
+
+def test_hook_update_of_a_weight_invalidates_the_const_eval_result(device, orc):
+    """updateTensorInPool gives the tensor a new version (runtime/lib/ttnn/runtime.cpp:2588), so a load_cached whose input a
+    pre-operator hook has just overwritten packs the weights again instead of returning the result for the old contents."""
+    M, K, N = 64, 128, 160
+    a, w, bias = datagen.c3_linear(M, K, N, seed=12)
+    binary = rt.Binary.load_from_memory(programs.c3_linear(M, K, N))
+    ins = [rt.to_layout(rt.from_torch(t), device, rt.get_layout(binary, 1, i), retain=True) for i, t in enumerate((a, bf(w), bias))]
+    rt.clear_stats()
+    run = lambda: rt.to_torch(rt.to_host(rt.submit(device, binary, 1, ins)[0], untilize=True)[0])
+    y1 = run()
+    assert torch.equal(run(), y1) and rt.get_stat("ConstEvalCacheMiss") == 1 and rt.get_stat("ConstEvalCacheHit") == 1
+
+    def pre(idx, name, dbg, hook):
+        if hook.program_index() == 1 and name == "LoadCachedOp":
+            (w_id,) = hook.input_refs()
+            hook.update(w_id, rt.from_torch(bf(w * 2)))
+    rt.set_pre_op_callback(pre)
+    try:
+        y2 = run()
+    finally:
+        rt.clear_callbacks()
+    assert rt.get_stat("ConstEvalCacheMiss") == 2
+    wq = orc.bfp_unpack(orc.bfp_pack(bf(w * 2).float().numpy(), 8), (K, N), 8)
+    want = orc.round_bf16(orc.linear(a.float().numpy(), wq, bias.float().numpy(), "gelu"))
+    assert np.max(np.abs(y2.float().numpy() - want)) <= 2.0 ** -6 and not torch.equal(y1, y2)
+
+
+def test_const_eval_results_die_with_their_device(orc):
+    """Const-eval results are device memory: closing the device drops them (the reference keys its cache by device as well,
+    runtime/lib/ttnn/operations/cache/load_cached.cpp:24-38), so the same binary on a reopened device packs its weights
+    again instead of meeting tensors of the closed device; destroying a binary drops its entries too."""
+    M, K, N = 64, 128, 160
+    a, w, bias = datagen.c3_linear(M, K, N, seed=13)
+    binary = rt.Binary.load_from_memory(programs.c3_linear(M, K, N))
+    results = []
+    rt.clear_stats()
+    for _ in range(2):
+        d = rt.open_mesh_device()
+        try:
+            (y,) = harness.execute(binary, 1, [a, bf(w), bias], d)
+            results.append(y)
+        finally:
+            rt.close_mesh_device(d)
+    assert rt.get_stat("ConstEvalCacheMiss") == 2 and rt.get_stat("ConstEvalCacheHit") == 0
+    assert torch.equal(results[0], results[1])
+    # a device tensor that outlives its device cannot be converted or read any more: a clear error, not a launch on a dead stream
+    d = rt.open_mesh_device()
+    t = rt.to_layout(rt.from_torch(a), d, rt.Layout(ST.Device, TL.Tile, DT.BFloat16))
+    rt.close_mesh_device(d)
+    with pytest.raises(RuntimeError, match="has been closed"):
+        rt.to_host(t, untilize=True)
 
 
 def test_embedded_goldens_are_checked_per_operation(device, orc):

@@ -20,7 +20,7 @@ def _operands(hip, dev, B, H, Hkv, S, D, seed):
 
 def _run(hip, name, qt, kt, vt, cp, B, H, Hkv, S, D, window=-1):
     out = torch.full_like(qt, float("nan"))
-    hip.call(name, hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, 1, None, 0, 0, hip.ptr(out), hip.BF16,
+    hip.call(name, hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), hip.ptr(cp), None, 1, 1, None, 0, 0, 0, hip.ptr(out), hip.BF16,
              B, H, Hkv, S, D, 1, 0.0, 0, window, None, hip.current_stream())
     torch.cuda.synchronize()
     return out
@@ -50,5 +50,5 @@ def test_static_scratch_refuses_what_does_not_fit(hip, dev):
     z = torch.zeros(1024, dtype=torch.bfloat16, device=dev)
     cp = torch.zeros(64, dtype=torch.int32, device=dev)
     with pytest.raises(hip.TTMError, match="static scratch holds"):
-        hip.call("ttm_sdpa_decode_static", hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.ptr(cp), None, 1, 1, None, 0, 0, hip.ptr(z),
+        hip.call("ttm_sdpa_decode_static", hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.ptr(cp), None, 1, 1, None, 0, 0, 0, hip.ptr(z),
                  hip.BF16, 64, 256, 32, 8192, 128, 1, 0.0, 0, -1, None, hip.current_stream())

@@ -188,6 +188,7 @@ struct DecodeArgs {
   float *part;        // [B * Hkv][splits][G][D + 2]
   uint16_t *out;
   int B, H, Hkv, G, S, D, splits, keys_per_split, block, pages_per_user, mask_heads, is_causal;
+  int blocks;         // number of blocks in a paged cache: page-table entries outside [0, blocks) are masked
   int concat_heads;   // out is [B, H * D] (row b holds user b's heads side by side) instead of [B, H, D]
   int Gt, g0;         // query heads per kv head in the tensors, and the first of them this launch serves (it serves G of them)
   int mask_b;         // 1: one mask per user, 0: one mask shared by all
@@ -201,12 +202,16 @@ constexpr int kMaxG = 8;
 #define SPLIT_TARGET 512
 #endif
 
-__device__ __forceinline__ const uint16_t *kv_tile_row(const uint16_t *base, const DecodeArgs &p, int b, int hk, int key_tile) {
-  // start of the row of tiles holding keys [32 key_tile, 32 key_tile + 32) of (b, hk)
+__device__ __forceinline__ const uint16_t *kv_tile_row(const uint16_t *base, const DecodeArgs &p, int b, int hk, int key_tile, bool &ok) {
+  // start of the row of tiles holding keys [32 key_tile, 32 key_tile + 32) of (b, hk).  A page-table entry outside the
+  // cache's blocks (an unused slot, -1) gives ok = false and the address of block 0: the caller treats those keys as masked
   const int64_t row_elems = (int64_t)32 * p.D;
+  ok = true;
   if (p.page_table) {
     const int tiles_per_block = p.block >> 5;
-    const int page = p.page_table[(int64_t)b * p.pages_per_user + key_tile / tiles_per_block];
+    int page = p.page_table[(int64_t)b * p.pages_per_user + key_tile / tiles_per_block];
+    ok = page >= 0 && page < p.blocks;
+    page = ok ? page : 0;
     return base + (((int64_t)page * p.Hkv + hk) * tiles_per_block + key_tile % tiles_per_block) * row_elems;
   }
   return base + (((int64_t)b * p.Hkv + hk) * (p.S >> 5) + key_tile) * row_elems;
@@ -264,11 +269,12 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
       // two groups of 16 keys per pass, all their loads issued before the first product
       u32x4 kf[2][8];
       int grp[2];
+      bool kok[2];
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
         grp[u] = g0 + 4 * u < ngroups ? g0 + 4 * u : g0;   // the tail repeats a valid group and skips its result
         const int key = k0 + grp[u] * 16 + (lane & 15);     // this lane's key column of the B operand
-        const uint16_t *kt = kv_tile_row(p.k, p, b, hk, key >> 5);
+        const uint16_t *kt = kv_tile_row(p.k, p, b, hk, key >> 5, kok[u]);
         // inside a tile: face (key half, column half), row key % 16, columns dq % 16 .. + 7
         const int in_tile = (((key >> 4) & 1) * 2 + (dq >> 4)) * 256 + (key & 15) * 16 + (dq & 15);
 #pragma unroll
@@ -294,7 +300,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
               const int64_t mrows = ttm_round_up32(p.mask_heads);
               sv += ttm_bf16_to_f32(p.mask[(int64_t)b * p.mask_b * mrows * p.S + ttm_tiled_offset(mh, k0 + kk, p.S >> 5)]);
             }
-            sc[gq * p.keys_per_split + kk] = (k0 + kk < k1 && k0 + kk >= lo) ? sv * p.scale : -INFINITY;
+            sc[gq * p.keys_per_split + kk] = (k0 + kk < k1 && k0 + kk >= lo && kok[u]) ? sv * p.scale : -INFINITY;
           }
         }
       }
@@ -346,10 +352,11 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
         for (int j = 0; j < 8; ++j) o[g][j] = 0.0f;
       for (int t0 = tfirst; t0 < ntiles; t0 += UT * share) {
         u32x4 ra[UT], rb[UT];
+        bool vok[UT];
 #pragma unroll
         for (int u = 0; u < UT; ++u) {
           const int t = t0 + u * share < ntiles ? t0 + u * share : t0;
-          const uint16_t *vt = kv_tile_row(p.v, p, b, hk, (k0 >> 5) + t) + (int64_t)dt * 1024;
+          const uint16_t *vt = kv_tile_row(p.v, p, b, hk, (k0 >> 5) + t, vok[u]) + (int64_t)dt * 1024;
           ra[u] = *(const u32x4 *)(vt + lane * 8);
           rb[u] = *(const u32x4 *)(vt + 512 + lane * 8);
         }
@@ -358,9 +365,9 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
           const int t = t0 + u * share;
           if (t >= ntiles) break;
           uint32_t a[4] = {ra[u].x, ra[u].y, ra[u].z, ra[u].w}, c[4] = {rb[u].x, rb[u].y, rb[u].z, rb[u].w};
-          if (t * 32 + 32 > nkeys || k0 + t * 32 < lo) {   // boundary tile: rows outside the visible keys may hold anything, NaN included
-            const bool la = t * 32 + krow < nkeys && k0 + t * 32 + krow >= lo;
-            const bool lb = t * 32 + 16 + krow < nkeys && k0 + t * 32 + 16 + krow >= lo;
+          if (t * 32 + 32 > nkeys || k0 + t * 32 < lo || !vok[u]) {   // boundary tile: rows outside the visible keys may hold anything, NaN included
+            const bool la = vok[u] && t * 32 + krow < nkeys && k0 + t * 32 + krow >= lo;
+            const bool lb = vok[u] && t * 32 + 16 + krow < nkeys && k0 + t * 32 + 16 + krow >= lo;
 #pragma unroll
             for (int j = 0; j < 4; ++j) { a[j] = la ? a[j] : 0u; c[j] = lb ? c[j] : 0u; }
           }
@@ -613,7 +620,7 @@ static int decode_scratch_ptr(void **ptr) {
 }
 
 static int sdpa_decode_entry(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
-                             const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out, int dtype, int64_t batch,
+                             const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch,
                              int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads,
                              int64_t window, const void *sink, int64_t mask_batch, bool static_scratch, void *stream) {
   TTM_REQUIRE(q && k && v && out, "ttm_sdpa_decode: null pointer");
@@ -624,10 +631,13 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
   TTM_REQUIRE(head_dim % 32 == 0 && head_dim >= 32 && head_dim <= 256, "ttm_sdpa_decode: head dim must be a multiple of 32 up to 256");
   TTM_REQUIRE(seq > 0 && seq % 32 == 0, "ttm_sdpa_decode: cache length must be a positive multiple of 32");
   TTM_REQUIRE(!mask || mask_heads == 1 || mask_heads == heads, "ttm_sdpa_decode: mask must have 1 or %lld head rows", (long long)heads);
-  if (page_table)
+  if (page_table) {
     TTM_REQUIRE(page_block > 0 && page_block % 32 == 0 && pages_per_user * page_block == seq,
                 "ttm_sdpa_decode: page table of %lld blocks x %lld positions does not cover %lld positions",
                 (long long)pages_per_user, (long long)page_block, (long long)seq);
+    TTM_REQUIRE(page_blocks > 0 && page_blocks <= INT32_MAX, "ttm_sdpa_decode: a page table needs the number of blocks in the cache (got %lld)",
+                (long long)page_blocks);
+  }
   hipStream_t s = (hipStream_t)stream;
   // enough blocks to fill the device, slices small enough for the score rows to fit in LDS
   int64_t splits = ttm_cdiv(SPLIT_TARGET, batch * kv_heads);
@@ -641,6 +651,7 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
   p.cur_pos = cur_pos; p.page_table = page_table; p.out = (uint16_t *)out;
   p.B = (int)batch; p.H = (int)heads; p.Hkv = (int)kv_heads; p.G = (int)G; p.S = (int)seq; p.D = (int)head_dim;
   p.splits = (int)splits; p.keys_per_split = (int)keys; p.block = (int)page_block; p.pages_per_user = (int)pages_per_user;
+  p.blocks = (int)page_blocks;
   p.mask_heads = mask_heads; p.is_causal = is_causal; p.concat_heads = concat_heads;
   p.scale = scale > 0.0f ? scale : 1.0f / sqrtf((float)head_dim);
   p.Gt = (int)Gt;
@@ -673,36 +684,36 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
 }
 
 TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
-                               int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, void *out,
-                               int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
+                               int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks,
+                               void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
                                int is_causal, float scale, void *stream) {
-  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
+  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, 0, -1, nullptr, batch, false, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
                                             int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block,
-                                            void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
-                                            int64_t head_dim, int is_causal, float scale, void *stream) {
-  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
+                                            int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads,
+                                            int64_t seq, int64_t head_dim, int is_causal, float scale, void *stream) {
+  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, 1, -1, nullptr, batch, false, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
                                         int mask_heads, int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user,
-                                        int64_t page_block, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
-                                        int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
+                                        int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads,
+                                        int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                                         const void *attention_sink, void *stream) {
-  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
+  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, false, stream);
 }
 
 // ttm_sdpa_decode_windowed for callers that cannot allocate: the slots come from the library's static device array.
 TTM_EXPORT int ttm_sdpa_decode_static(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask,
                                       int mask_heads, int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user,
-                                      int64_t page_block, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq,
-                                      int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
+                                      int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads,
+                                      int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                                       const void *attention_sink, void *stream) {
-  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, out, dtype, batch, heads, kv_heads,
+  return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, true, stream);
 }

@@ -973,12 +973,12 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
               "sdpa_decode: query must be [1, batch, heads, head_dim], key / value 4D with the same head_dim");
   const std::int64_t B = qs[1], H = qs[2], Hkv = ks[1], D = qs[3];
   Tensor table;
-  std::int64_t pages = 0, block = 0, S = ks[2];
+  std::int64_t pages = 0, block = 0, cacheBlocks = 0, S = ks[2];
   if (pageRef) {
     table = devicePositions(ctx, ctx.get(pageRef, "sdpa_decode page table"), "sdpa_decode: page_table");
     const auto &ts = table.handle->shape;
     TTRT_ASSERT(ts.size() == 2 && ts[0] == B, "sdpa_decode: page table must be [batch, blocks per user]");
-    pages = ts[1]; block = ks[2]; S = pages * block;
+    pages = ts[1]; block = ks[2]; cacheBlocks = ks[0]; S = pages * block;
   } else {
     TTRT_ASSERT(ks[0] == B, "sdpa_decode: key / value batch differs from the query's");
   }
@@ -1015,7 +1015,7 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
       TTM_CALL(ttm_sdpa_decode_windowed(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
                                         pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
                                         mask ? mask.handle->data.get() : nullptr, maskHeads, maskBatch,
-                                        table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
+                                        table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block, cacheBlocks,
                                         merged.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, 1, window, sinkPtr,
                                         ctx.stream()));
       ctx.put(finalRef, merged);
@@ -1027,7 +1027,7 @@ void sdpaDecode(ProgramContext &ctx, const fb::Table &qRef, const fb::Table &kRe
   TTM_CALL(ttm_sdpa_decode_windowed(q.handle->data.get(), k.handle->data.get(), v.handle->data.get(),
                                     pos ? static_cast<const std::int32_t *>(pos.handle->data.get()) : nullptr,
                                     mask ? mask.handle->data.get() : nullptr, maskHeads, maskBatch,
-                                    table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block,
+                                    table ? static_cast<const std::int32_t *>(table.handle->data.get()) : nullptr, pages, block, cacheBlocks,
                                     out.handle->data.get(), TTM_BF16, B, H, Hkv, S, D, causal ? 1 : 0, scale, 0, window, sinkPtr,
                                     ctx.stream()));
   ctx.put(outRef, finish(ctx, out, outRef));
@@ -1568,19 +1568,6 @@ void runDeallocate(const fb::Table &op, ProgramContext &ctx) {
 }
 
 // ---- const-eval (runtime/lib/ttnn/operations/cache/load_cached.cpp:20-90)
-struct CacheEntry {
-  std::vector<std::uint64_t> inputVersions;
-  std::vector<Tensor> outputs;
-};
-std::mutex g_cacheMu;
-using ConstEvalCache = std::map<std::pair<std::uint64_t, std::uint32_t>, CacheEntry>;
-ConstEvalCache &constEvalCache() {
-  // leaked on purpose: its tensors own device memory, which must not be released from static
-  // destructors that run after the HIP runtime has begun shutting down
-  static ConstEvalCache *c = new ConstEvalCache;
-  return *c;
-}
-
 void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
   auto ins = op.tables(schema::LoadCachedOp::f_inputs), outs = op.tables(schema::LoadCachedOp::f_outputs);
   std::uint32_t prog = op.scalar<std::uint32_t>(schema::LoadCachedOp::f_program_idx, 0);
@@ -1592,9 +1579,9 @@ void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
   }
   auto key = std::make_pair(ctx.binary.id(), prog);
   {
-    std::lock_guard<std::mutex> g(g_cacheMu);
-    auto it = constEvalCache().find(key);
-    if (it != constEvalCache().end() && it->second.inputVersions == versions) {
+    std::lock_guard<std::mutex> g(ctx.dev->constEvalMu);
+    auto it = ctx.dev->constEval.find(key);
+    if (it != ctx.dev->constEval.end() && it->second.inputVersions == versions) {
       debug::Stats::get().incrementStat("ConstEvalCacheHit");
       for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], it->second.outputs.at(i));
       return;
@@ -1605,8 +1592,8 @@ void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
   TTRT_ASSERT(results.size() == outs.size(), "load_cached: callee returned a different number of outputs");
   for (auto &t : results) setTensorRetain(t, true);
   {
-    std::lock_guard<std::mutex> g(g_cacheMu);
-    constEvalCache()[key] = CacheEntry{versions, results};
+    std::lock_guard<std::mutex> g(ctx.dev->constEvalMu);
+    ctx.dev->constEval[key] = ConstEvalEntry{versions, results};
   }
   for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], results[i]);
 }
@@ -1912,6 +1899,9 @@ void updateTensorInPool(CallbackContext cc, std::uint32_t globalId, Tensor src) 
     conv = convertOnDevice(conv.handle->storage == StorageType::Device ? conv : toDevice(conv, ctx->dev), want.layout, want.dataType);
   if (want.storageType == StorageType::Host && conv.handle->storage == StorageType::Device) conv = fromDevice(conv);
   memcpy(dst, conv);
+  // new contents, new version (runtime/lib/ttnn/runtime.cpp:2588): a const-eval result or a trace slot computed from the
+  // old contents no longer matches
+  dst.handle->version = nextTensorVersion();
 }
 
 }  // namespace tt::runtime

@@ -12,6 +12,7 @@
 #include <sstream>
 #include <thread>
 
+#include "device_pool.h"
 #include "runtime_impl.h"
 
 namespace tt::runtime {
@@ -220,6 +221,49 @@ size_t tensorBytes(const std::vector<std::uint32_t> &shape, DataType dtype, Tens
 // ============================================================================ binary
 static std::atomic<std::uint64_t> g_binaryId{1};
 
+// Devices that may hold cached results of a binary.  Leaked on purpose: binaries and devices may be destroyed from static
+// destructors in any order.
+namespace {
+struct DeviceRegistry {
+  std::mutex mu;
+  std::vector<std::weak_ptr<DeviceState>> devices;
+};
+DeviceRegistry &deviceRegistry() {
+  static DeviceRegistry *r = new DeviceRegistry;
+  return *r;
+}
+}  // namespace
+
+BinaryImpl::~BinaryImpl() {
+  std::vector<std::shared_ptr<DeviceState>> devs;
+  {
+    std::lock_guard<std::mutex> g(deviceRegistry().mu);
+    auto &v = deviceRegistry().devices;
+    for (auto it = v.begin(); it != v.end();) {
+      if (auto d = it->lock()) { devs.push_back(d); ++it; } else it = v.erase(it);
+    }
+  }
+  for (auto &d : devs) {
+    std::vector<ConstEvalEntry> dropped;   // their tensors return to the pool outside the lock
+    {
+      std::lock_guard<std::mutex> g(d->constEvalMu);
+      for (auto it = d->constEval.begin(); it != d->constEval.end();) {
+        if (it->first.first == id) { dropped.push_back(std::move(it->second)); it = d->constEval.erase(it); } else ++it;
+      }
+    }
+    if (!d->open) continue;
+    // traces recorded for this binary: nobody can replay them once the binary is gone
+    std::lock_guard<std::recursive_mutex> g(d->mu);
+    if (d->capturing) continue;
+    std::vector<std::uint32_t> ids;
+    for (const auto &kv : d->traceCache)
+      if (std::get<0>(kv.first) == id) ids.push_back(kv.second);
+    for (std::uint32_t t : ids) {
+      try { releaseTrace(d, t); } catch (const std::exception &) { /* a destructor must not throw */ }
+    }
+  }
+}
+
 static Binary makeBinary(std::vector<std::uint8_t> &&bytes) {
   auto impl = std::make_shared<BinaryImpl>();
   impl->bytes = std::move(bytes);
@@ -405,106 +449,12 @@ Layout getLayout(Binary binary, std::uint32_t programIndex, std::uint32_t inputI
 // Caching allocator: blocks are kept per rounded size and reused; all work of a device is ordered
 // on one stream, so reuse by a later launch is safe.  Freed to the driver at closeMeshDevice.
 namespace {
-struct DevicePool {
-  std::mutex mu;
-  std::multimap<size_t, void *> freeBlocks;
-  size_t cachedBytes = 0;
-  // While a trace is being recorded on this thread, blocks that are released stay with the recording (they may be
-  // reused by later launches of the same recording, whose order the graph keeps) and every block the recording
-  // touched is pinned: it never returns to freeBlocks until the trace is released.
-  bool recording = false;
-  std::thread::id recorder;
-  std::multimap<size_t, void *> recordFree;
-  std::map<void *, size_t> recordTouched;
-  std::set<void *> pinned;
-
-  static size_t rounded(size_t bytes) { return std::max<size_t>(512, (bytes + 511) / 512 * 512); }
-  bool recordingHere() const { return recording && recorder == std::this_thread::get_id(); }
-
-  void *alloc(size_t bytes) {
-    size_t sz = rounded(bytes);
-    {
-      std::lock_guard<std::mutex> g(mu);
-      const bool rec = recordingHere();
-      if (rec) {
-        auto it = recordFree.find(sz);
-        if (it != recordFree.end()) {
-          void *p = it->second;
-          recordFree.erase(it);
-          return p;
-        }
-      }
-      auto it = freeBlocks.find(sz);
-      if (it != freeBlocks.end()) {
-        void *p = it->second;
-        freeBlocks.erase(it);
-        cachedBytes -= sz;
-        if (rec) { recordTouched[p] = sz; pinned.insert(p); }
-        return p;
-      }
-    }
-    void *p = nullptr;
-    int rc = ttm_malloc(&p, sz);
-    if (rc != 0) {
-      release();
-      TTM_CALL(ttm_malloc(&p, sz));
-    }
-    std::lock_guard<std::mutex> g(mu);
-    if (recordingHere()) { recordTouched[p] = sz; pinned.insert(p); }
-    return p;
-  }
-  void free(void *p, size_t bytes) {
-    size_t sz = rounded(bytes);
-    std::lock_guard<std::mutex> g(mu);
-    if (recordingHere()) {
-      // a block that existed before the recording and is released inside it may still be read by recorded launches
-      recordTouched[p] = sz;
-      pinned.insert(p);
-      recordFree.emplace(sz, p);
-      return;
-    }
-    if (pinned.count(p)) return;  // owned by a trace; comes back through unpin()
-    freeBlocks.emplace(sz, p);
-    cachedBytes += sz;
-  }
-  void beginRecording() {
-    std::lock_guard<std::mutex> g(mu);
-    TTRT_ASSERT(!recording, "a trace is already being recorded");
-    recording = true;
-    recorder = std::this_thread::get_id();
-    recordFree.clear();
-    recordTouched.clear();
-  }
-  std::vector<std::pair<void *, size_t>> endRecording() {
-    std::lock_guard<std::mutex> g(mu);
-    std::vector<std::pair<void *, size_t>> out(recordTouched.begin(), recordTouched.end());
-    recording = false;
-    recordFree.clear();
-    recordTouched.clear();
-    return out;
-  }
-  // blocks of a released trace go back into circulation, except those a live tensor still holds (their deleter returns them)
-  void unpin(const std::vector<std::pair<void *, size_t>> &blocks, const std::set<void *> &stillHeld) {
-    std::lock_guard<std::mutex> g(mu);
-    for (const auto &b : blocks) {
-      pinned.erase(b.first);
-      if (stillHeld.count(b.first)) continue;
-      freeBlocks.emplace(b.second, b.first);
-      cachedBytes += b.second;
-    }
-  }
-  void release() {
-    std::lock_guard<std::mutex> g(mu);
-    if (!freeBlocks.empty()) ttm_device_sync();
-    for (auto &kv : freeBlocks) ttm_free(kv.second);
-    freeBlocks.clear();
-    cachedBytes = 0;
-  }
-};
 DevicePool &pool() {
   // never destroyed: tensors held by other statics (the const-eval cache) return their blocks here
   // during process teardown, after function-local statics would already be gone
-  static DevicePool *p = new DevicePool;
+  static DevicePool *p = new DevicePool(PoolBackend{
+      [](void **ptr, size_t bytes) { return ttm_malloc(ptr, bytes); }, [](void *ptr) { return ttm_free(ptr); },
+      []() { return ttm_device_sync(); }});
   return *p;
 }
 }  // namespace
@@ -528,6 +478,10 @@ Device openMeshDevice(const MeshDeviceOptions &options) {
   TTM_CALL(ttm_set_device(st->deviceId));
   TTM_CALL(ttm_stream_create(&st->stream));
   st->open = true;
+  {
+    std::lock_guard<std::mutex> g(deviceRegistry().mu);
+    deviceRegistry().devices.push_back(st);
+  }
   return Device{st};
 }
 
@@ -542,7 +496,7 @@ void beginTraceCapture(const std::shared_ptr<DeviceState> &dev, std::uint32_t tr
   pool().beginRecording();
   int rc = ttm_graph_begin_capture(dev->stream);
   if (rc != 0) {
-    pool().unpin(pool().endRecording(), {});
+    pool().unpin(pool().endRecording());
     hipCheck(rc, "ttm_graph_begin_capture");
   }
   dev->capturing = true;
@@ -558,7 +512,7 @@ void endTraceCapture(const std::shared_ptr<DeviceState> &dev, std::uint32_t trac
   td.blocks = pool().endRecording();
   int rc = ttm_graph_end_capture(dev->stream, &td.graphExec, &td.numNodes);
   if (rc != 0) {
-    pool().unpin(td.blocks, {});
+    pool().unpin(td.blocks);
     hipCheck(rc, "ttm_graph_end_capture");
   }
   dev->traces[traceId] = std::move(td);
@@ -571,7 +525,7 @@ void abortTraceCapture(const std::shared_ptr<DeviceState> &dev) {
   void *exec = nullptr;
   size_t nodes = 0;
   if (ttm_graph_end_capture(dev->stream, &exec, &nodes) == 0 && exec) ttm_graph_destroy(exec);
-  pool().unpin(blocks, {});
+  pool().unpin(blocks);
 }
 
 void executeTrace(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId, bool blocking) {
@@ -588,7 +542,7 @@ void releaseTrace(const std::shared_ptr<DeviceState> &dev, std::uint32_t traceId
   if (it == dev->traces.end()) return;
   TTM_CALL(ttm_stream_sync(dev->stream));
   TTM_CALL(ttm_graph_destroy(it->second.graphExec));
-  pool().unpin(it->second.blocks, {});
+  pool().unpin(it->second.blocks);
   for (auto kv = dev->traceCache.begin(); kv != dev->traceCache.end();)
     kv = kv->second == traceId ? dev->traceCache.erase(kv) : std::next(kv);
   dev->traces.erase(it);
@@ -599,6 +553,13 @@ void closeMeshDevice(Device d) {
   TTRT_ASSERT(!d.handle->capturing, "closeMeshDevice: a trace capture is in progress");
   TTM_CALL(ttm_stream_sync(d.handle->stream));
   while (!d.handle->traces.empty()) releaseTrace(d.handle, d.handle->traces.begin()->first);
+  d.handle->traceCache.clear();
+  {
+    // const-eval results are memory of this device: they go back to the pool before the pool returns it to the driver
+    std::map<std::pair<std::uint64_t, std::uint32_t>, ConstEvalEntry> dropped;
+    std::lock_guard<std::mutex> g(d.handle->constEvalMu);
+    dropped.swap(d.handle->constEval);
+  }
   pool().release();
   TTM_CALL(ttm_stream_destroy(d.handle->stream));
   d.handle->stream = nullptr;
@@ -761,6 +722,7 @@ Tensor toDevice(const Tensor &h, const std::shared_ptr<DeviceState> &dev) {
 
 Tensor fromDevice(const Tensor &d) {
   TTRT_ASSERT(d.handle->storage == StorageType::Device, "fromDevice: tensor is not on the device");
+  TTRT_ASSERT(d.handle->device && d.handle->device->open, "the tensor belongs to a device that has been closed");
   requireNotCapturing(d.handle->device, "a device to host transfer");
   Tensor h = makeHostTensor(d.handle->shape, d.handle->dtype, d.handle->layout);
   TTM_CALL(ttm_memcpy_d2h(h.handle->data.get(), d.handle->data.get(), d.handle->bytes, d.handle->device->stream));
@@ -775,6 +737,7 @@ Tensor convertOnDevice(const Tensor &src, TensorLayout layout, DataType dtype) {
   const TensorImpl &s = *src.handle;
   TTRT_ASSERT(s.storage == StorageType::Device, "convertOnDevice: tensor is not on the device");
   if (s.layout == layout && s.dtype == dtype) return src;
+  TTRT_ASSERT(s.device && s.device->open, "the tensor belongs to a device that has been closed");
   void *stream = s.device->stream;
   Dims3 d = dims3(s.shape);
   const bool srcBfp = utils::isBlockFormatDataType(s.dtype), dstBfp = utils::isBlockFormatDataType(dtype);
@@ -826,14 +789,16 @@ Tensor toLayout(Tensor tensor, Device device, Layout layout, std::optional<bool>
   if (cur.handle->storage == StorageType::Host && needsDevice) cur = toDevice(cur, device.handle);
   if (cur.handle->storage == StorageType::Device) cur = convertOnDevice(cur, layout.layout, layout.dataType);
   if (layout.storageType == StorageType::Host && cur.handle->storage == StorageType::Device) cur = fromDevice(cur);
+  // one decision for both sides, as in runtime/lib/ttnn/runtime.cpp:906-932: the result carries the flag, and the input is
+  // consumed exactly when the flag is off
+  const bool shouldRetain = retain.value_or(getTensorRetain(tensor));
   if (cur.handle == tensor.handle) {
     // already in the requested layout: hand back the same tensor, nothing to free
-    if (retain.has_value()) setTensorRetain(cur, *retain);
+    setTensorRetain(cur, shouldRetain);
     return cur;
   }
-  setTensorRetain(cur, retain.value_or(false));
-  // the input is consumed unless it asks to be kept (runtime/lib/ttnn/runtime.cpp:929-931)
-  if (!getTensorRetain(tensor) && !tensor.handle->borrowed) {
+  setTensorRetain(cur, shouldRetain);
+  if (!shouldRetain && !tensor.handle->borrowed) {   // borrowed host memory is the caller's
     Tensor t = tensor;
     deallocateTensor(t, false);
   }

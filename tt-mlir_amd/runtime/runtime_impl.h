@@ -33,6 +33,13 @@ struct TraceData {
 // (binary id, main program, capture program, execute program): MainProgramKey + CaptureExecuteProgramKey of the reference
 using TraceKey = std::tuple<std::uint64_t, std::uint32_t, std::uint32_t, std::uint32_t>;
 
+// Results of a const-eval program (runtime/lib/ttnn/operations/cache/load_cached.cpp:20-90): valid while the versions of
+// the tensors it was run on are those of the current inputs.
+struct ConstEvalEntry {
+  std::vector<std::uint64_t> inputVersions;
+  std::vector<Tensor> outputs;
+};
+
 struct DeviceState {
   int deviceId = 0;
   void *stream = nullptr;  // hipStream_t: all work of this device is ordered on it
@@ -47,6 +54,11 @@ struct DeviceState {
   std::uint32_t nextTraceId = 1;
   std::map<std::uint32_t, TraceData> traces;      // by trace id: graphs recorded on this device
   std::map<TraceKey, std::uint32_t> traceCache;   // capture_or_execute_trace -> trace id
+  // const-eval results by (binary id, program index).  They are device memory of this device, so they live and die with it
+  // (the reference keys its cache by device id as well, load_cached.cpp:24-38): dropped at closeMeshDevice, and per binary
+  // when the binary is destroyed.
+  std::mutex constEvalMu;
+  std::map<std::pair<std::uint64_t, std::uint32_t>, ConstEvalEntry> constEval;
   ~DeviceState();
 };
 
@@ -78,6 +90,7 @@ struct BinaryImpl {
   std::vector<std::uint8_t> bytes;
   fb::Table root;
   std::uint64_t id = 0;
+  ~BinaryImpl();   // drops what open devices cached for this binary (const-eval results, traces)
 };
 
 // [.., R, C] -> (batch, rows, cols); rank 0/1 tensors are a single row
