@@ -42,6 +42,46 @@ def _wall_time(torch, fn, steps):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
+def sample_sclk(torch, fn, seconds=1.2):
+    """Shader clock reported by rocm-smi while `fn` is launched back to back for `seconds`: (median MHz, samples).  The
+    matrix kernels run against the board's power limit, so the clock they are given is part of the measurement."""
+    import re
+    import statistics
+    import subprocess
+    import threading
+    vals, stop = [], [False]
+
+    def poll():
+        while not stop[0]:
+            try:
+                out = subprocess.run(["rocm-smi", "--showclocks", "--json"], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL,
+                                     text=True, timeout=5).stdout
+                card = next(iter(json.loads(out).values()))
+                for key, value in card.items():
+                    m = re.search(r"(\d+)\s*Mhz", str(value))
+                    if "sclk clock speed" in key and m:
+                        vals.append(int(m.group(1)))
+            except Exception:
+                pass
+            time.sleep(0.1)
+    for _ in range(20):
+        fn()
+    torch.cuda.synchronize()
+    th = threading.Thread(target=poll, daemon=True)
+    th.start()
+    t0, n = time.perf_counter(), 0
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(50):
+            fn()
+        n += 50
+        torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / n
+    stop[0] = True
+    th.join(timeout=6)
+    vals = vals[1:] if len(vals) > 2 else vals          # the first sample may predate the load
+    return (int(statistics.median(vals)) if vals else None), len(vals), ms
+
+
 class Workload:
     """name, bound ('hbm'|'mfma'), algorithmic work per launch, fn() launching exactly one kernel."""
 
@@ -129,13 +169,21 @@ def make_workloads(torch, hip, datagen, dev, names):
         cur = torch.full((B,), S - 1, dtype=torch.int32, device=dev)
         torch.cuda.synchronize()
         del kv
+        # the two caches of one layer (268 MB) are about the size of the 256 MB last-level cache: three pairs are cycled
+        # (805 MB), as the layers of a model would be, so that every launch reads HBM
+        caches = [kvt] + [[t.clone() for t in kvt] for _ in range(2)]
+        dturn = [0]
+
+        def dfn(qt=qt, caches=caches, cur=cur, o=o, B=B, H=H, Hkv=Hkv, S=S, D=D, dturn=dturn):
+            dturn[0] = (dturn[0] + 1) % len(caches)
+            kc, vc = caches[dturn[0]]
+            hip.call("ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kc), hip.ptr(vc), hip.ptr(cur), None, 1, None, 0, 0, 0,
+                     hip.ptr(o), hip.BF16, B, H, Hkv, S, D, 1, 0.0, s)
         out["sdpa_decode32"] = Workload(
-            "sdpa_decode32", "hbm", 2 * B * Hkv * S * D * 2 + 2 * B * H * D * 2, "bytes",
-            lambda qt=qt, kvt=kvt, cur=cur, o=o, B=B, H=H, Hkv=Hkv, S=S, D=D: hip.call(
-                "ttm_sdpa_decode", hip.ptr(qt), hip.ptr(kvt[0]), hip.ptr(kvt[1]), hip.ptr(cur), None, 1, None, 0, 0, 0,
-                hip.ptr(o), hip.BF16, B, H, Hkv, S, D, 1, 0.0, s),
-            "decode attention: 32 users x 32 heads (8 kv heads) x 1 token over a full 2048-position bf16 KV cache",
-            dict(keep=(qt, kvt, cur, o)))
+            "sdpa_decode32", "hbm", 2 * B * Hkv * S * D * 2 + 2 * B * H * D * 2, "bytes", dfn,
+            "decode attention: 32 users x 32 heads (8 kv heads) x 1 token over a full 2048-position bf16 KV cache (three cache "
+            "pairs cycled, so each launch reads HBM)",
+            dict(keep=(qt, caches, cur, o)))
     for nm, window in (("sdpa2048", -1), ("sdpa2048_window128", 128)):
         if nm not in names:
             continue
@@ -149,15 +197,67 @@ def make_workloads(torch, hip, datagen, dev, names):
         del qkv
         # full causal pass: dense count, the convention of the decoder-layer figure (about half of it is computed);
         # windowed pass: the visible (query, key) pairs only, sum_i min(i + 1, w), so the fraction is not flattered
-        visible = sum(min(i + 1, window) for i in range(S)) if window >= 0 else S * S
+        # FLOPs of the visible (query, key) pairs only: the causal triangle S (S + 1) / 2, or sum_i min(i + 1, w) under a
+        # window; the dense count 4 B Hq S^2 D (the convention of the decoder-layer figure) is reported beside it
+        visible = sum(min(i + 1, window) for i in range(S)) if window >= 0 else S * (S + 1) // 2
         out[nm] = Workload(
             nm, "mfma", 2.0 * 2 * B * Hq * visible * D, "flop",
             lambda tiles=tiles, o=o, window=window, B=B, Hq=Hq, Hkv=Hkv, S=S, D=D: hip.call(
                 "ttm_sdpa_windowed", hip.ptr(tiles[0]), hip.ptr(tiles[1]), hip.ptr(tiles[2]), None, 1, 1, hip.ptr(o), hip.BF16, B, Hq, Hkv,
                 S, S, D, 1, 0.0, 0, window, None, s),
             "config 5 attention alone: causal SDPA, 32 query / 8 kv heads, 2048 tokens, head_dim 128" +
-            (" (dense FLOPs counted)" if window < 0 else ", sliding window of %d keys (FLOPs of the visible pairs only)" % window),
-            dict(keep=(tiles, o)))
+            (" (FLOPs of the causal triangle only)" if window < 0 else ", sliding window of %d keys (FLOPs of the visible pairs only)" % window),
+            dict(keep=(tiles, o), dense_flop=2.0 * 2 * B * Hq * S * S * D))
+    # bandwidth class of the layer: RMSNorm, softmax and a last-dim reduction at config-5 sizes, SiLU(gate) * up at config 4's
+    if "rmsnorm2048" in names:
+        R_, C_ = 2048, 4096
+        xr = datagen.randn((R_, C_), seed=21, dtype=torch.bfloat16).to(dev)
+        wr = (1.0 + 0.02 * datagen.randn((1, C_), seed=22)).to(torch.bfloat16).to(dev)
+        xt_, wt_ = torch.empty_like(xr), torch.zeros(32 * C_, dtype=torch.bfloat16, device=dev)
+        hip.call("ttm_tilize", hip.ptr(xr), hip.ptr(xt_), 1, R_, C_, 2, s)
+        hip.call("ttm_tilize", hip.ptr(wr), hip.ptr(wt_), 1, 1, C_, 2, s)
+        yt_ = torch.empty_like(xt_)
+        out["rmsnorm2048"] = Workload(
+            "rmsnorm2048", "hbm", 2 * R_ * C_ * 2 + C_ * 2, "bytes",
+            lambda xt_=xt_, wt_=wt_, yt_=yt_, R_=R_, C_=C_: hip.call("ttm_rms_norm", hip.ptr(xt_), hip.ptr(wt_), hip.TILE, None, hip.TILE, hip.ptr(yt_),
+                                                       hip.BF16, 1, R_, C_, 1e-5, s),
+            "config 5 RMSNorm: bf16 [2048,4096] tiles, weight [4096], eps 1e-5", dict(keep=(xt_, wt_, yt_)))
+    if "softmax65536" in names or "reduce65536" in names:
+        R_, C_ = 32 * 2048, 2048
+        xs = (3.0 * datagen.randn((R_, C_), seed=23)).to(dev)
+        xt_ = torch.empty_like(xs)
+        hip.call("ttm_tilize", hip.ptr(xs), hip.ptr(xt_), 1, R_, C_, 4, s)
+        torch.cuda.synchronize()
+        del xs
+        if "softmax65536" in names:
+            yt_ = torch.empty_like(xt_)
+            out["softmax65536"] = Workload(
+                "softmax65536", "hbm", 2 * R_ * C_ * 4, "bytes",
+                lambda xt_=xt_, yt_=yt_, R_=R_, C_=C_: hip.call("ttm_softmax_lastdim", hip.ptr(xt_), hip.ptr(yt_), hip.F32, 1, R_, C_, s),
+                "config 5 attention scores if left unfused: softmax over the last dim of fp32 [32 x 2048, 2048] tiles",
+                dict(keep=(xt_, yt_)))
+        if "reduce65536" in names:
+            rt_ = torch.empty(R_ * 32, dtype=torch.float32, device=dev)
+            out["reduce65536"] = Workload(
+                "reduce65536", "hbm", R_ * C_ * 4 + R_ * 4, "bytes",
+                lambda xt_=xt_, rt_=rt_, R_=R_, C_=C_: hip.call("ttm_reduce_lastdim", 0, hip.ptr(xt_), hip.ptr(rt_), hip.F32, 1, R_, C_, s),
+                "sum over the last dim of fp32 [32 x 2048, 2048] tiles (one value per row)", dict(keep=(xt_, rt_)))
+    if "silu_mul512" in names:
+        import numpy as np
+        R_, C_ = 512, 14336
+        g_ = datagen.randn((R_, C_), seed=24, dtype=torch.bfloat16).to(dev)
+        u_ = datagen.randn((R_, C_), seed=25, dtype=torch.bfloat16).to(dev)
+        gt_, ut_ = torch.empty_like(g_), torch.empty_like(u_)
+        hip.call("ttm_tilize", hip.ptr(g_), hip.ptr(gt_), 1, R_, C_, 2, s)
+        hip.call("ttm_tilize", hip.ptr(u_), hip.ptr(ut_), 1, R_, C_, 2, s)
+        ot_ = torch.empty_like(gt_)
+        shp = np.array([R_, C_], dtype=np.int64)
+        out["silu_mul512"] = Workload(
+            "silu_mul512", "hbm", 3 * R_ * C_ * 2, "bytes",
+            lambda gt_=gt_, ut_=ut_, ot_=ot_, shp=shp: hip.call("ttm_eltwise_binary", 1, hip.ptr(gt_), shp.ctypes.data, hip.ptr(ut_),
+                                                                shp.ctypes.data, hip.ptr(ot_), shp.ctypes.data, 2, hip.BF16, hip.TILE, s),
+            "config 4 SiLU(gate) * up: bf16 [512,14336] tiles, two reads and one write (the SiLU itself sits in the gate "
+            "projection's epilogue)", dict(keep=(gt_, ut_, ot_, shp)))
     # whole programs through the runtime boundary (flatbuffer -> submit -> wait)
     for nm in ("decode32", "decode32_traced"):
         if nm not in names:
@@ -238,9 +338,13 @@ def roofline(w, kernel_ms):
     else:
         achieved = w.work / (kernel_ms * 1e-3) / 1e12
         peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
-    return {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(w.name), "kernel_us": round(kernel_ms * 1e3, 2),
-            "algorithmic_work": w.work, "work_unit": w.unit_work}
+    r = {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+         "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(w.name), "kernel_us": round(kernel_ms * 1e3, 2),
+         "algorithmic_work": w.work, "work_unit": w.unit_work}
+    if "dense_flop" in w.extra:   # attention: the dense count beside the FLOPs of the visible pairs that `frac` is made of
+        dense = w.extra["dense_flop"] / (kernel_ms * 1e-3) / 1e12
+        r["dense_counted"] = {"achieved": round(dense, 2), "frac": round(dense / peak, 4), "work": w.extra["dense_flop"]}
+    return r
 
 
 def cpu_baseline_linear(orc, datagen, budget_rows=512):
@@ -287,9 +391,14 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="linear2048")
-    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,sdpa_decode32,sdpa2048,mlp512,decoder2048,"
-                                           "decode32,decode32_traced")
+    ap.add_argument("--secondary", default="pack_bfp8,unpack_bfp8,pack_bfp4,unpack_bfp4,tilize_f32,untilize_f32,copy,linear32,sdpa_decode32,sdpa2048,rmsnorm2048,"
+                                           "softmax65536,reduce65536,silu_mul512,mlp512,decoder2048,decode32,decode32_traced")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-settle", action="store_true",
+                    help="skip the 0.3 s of untimed launches in front of every measurement (counter collection runs, where "
+                         "every dispatch is expensive)")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="kernel-variant option passed to ttm_set_option before anything runs (e.g. linear_two_pass=1)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (one MI355X per box); run with --gpus 1",
@@ -300,10 +409,13 @@ def main():
     entry.load_package()
     from ttmlir_amd import hip, datagen
     hip.lib()
+    for opt in args.option:
+        name, _, value = opt.partition("=")
+        hip.set_option(name, int(value))
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     stream = hip.current_stream()
-    sec_names = [n for n in args.secondary.split(",") if n and n != args.workload]
+    sec_names = [n for n in args.secondary.split(",") if n and n != args.workload and n != "none"]
     wl = make_workloads(torch, hip, datagen, dev, [args.workload] + sec_names)
     if args.workload not in wl:
         raise SystemExit("unknown workload " + args.workload)
@@ -311,7 +423,7 @@ def main():
     def measure(w, steps, warmup):
         # clocks settle only after some tens of milliseconds of load: keep the device busy for about 0.3 s before
         # the `warmup` untimed steps, so that short default runs measure the steady state
-        t_end = time.perf_counter() + 0.3
+        t_end = time.perf_counter() + (0.0 if args.no_settle else 0.3)
         while time.perf_counter() < t_end:
             for _ in range(8):
                 w.fn()
@@ -356,6 +468,31 @@ def main():
         lms, _ = measure(lib_w, max(10, args.steps // 2), max(3, args.warmup // 2))
         result["library_gemm"] = {"what": "torch.matmul bf16 [2048,4096] x bf16 [4096,14336] (vendor BLAS, no decode / bias / GELU)",
                                   "ms_per_step": round(lms, 5), "value": round(prim.work / (lms * 1e-3) / 1e12, 1), "unit": "TFLOP/s"}
+        # The matrix cores run against the board's power limit: the shader clock under this load is well below the 2400 MHz
+        # that the published peak assumes, and it depends on the operand values.  Reported: the clock while this kernel and
+        # while the vendor GEMM loop on the same operands, and the same launches on all-zero operands (no switching in the
+        # multipliers: the clock stays at its maximum), which separates what the kernel's schedule costs from what the
+        # power limit costs.
+        if not args.no_settle:
+            sclk, nsamp, loop_ms = sample_sclk(torch, prim.fn)
+            lclk, _, lloop = sample_sclk(torch, lib_w.fn)
+            at, wt, bt, ot = prim.extra["dev"]
+            keep = (at.clone(), wt.clone())
+            at.zero_(), wt.zero_()
+            zclk, _, zloop = sample_sclk(torch, prim.fn)
+            xa.zero_(), xw.zero_()
+            zlclk, _, zlloop = sample_sclk(torch, lib_w.fn)
+            at.copy_(keep[0]), wt.copy_(keep[1])
+            del keep
+            prim.fn()                                   # the output checked below comes from the real operands again
+            torch.cuda.synchronize()
+            result["clock"] = {
+                "sclk_mhz_max": 2400, "sclk_mhz_this_kernel": sclk, "loop_ms_this_kernel": round(loop_ms, 5), "samples": nsamp,
+                "sclk_mhz_library_gemm": lclk, "loop_ms_library_gemm": round(lloop, 5),
+                "zero_operands": {"sclk_mhz_this_kernel": zclk, "loop_ms_this_kernel": round(zloop, 5),
+                                  "sclk_mhz_library_gemm": zlclk, "loop_ms_library_gemm": round(zlloop, 5)},
+                "what": "rocm-smi shader clock while the launch is repeated back to back for 1.2 s, and the same with all-zero "
+                        "operands; loop_ms includes launch gaps"}
         del xa, xw
     if not args.no_cpu_baseline:
         orc = entry.load_oracle()

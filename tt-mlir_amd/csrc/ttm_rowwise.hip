@@ -385,9 +385,181 @@ __global__ __launch_bounds__(256) void ttm_rowwise_row_k(RowArgs p, int total_ro
   }
 }
 
+// All six modes with four consecutive rows per workgroup, for large row counts.  Four rows of a face are one run of whole
+// 128-byte lines (128 bytes of bf16, 256 of fp32) in every tile, so a workgroup reads and writes nothing but whole lines
+// that no other workgroup touches; consecutive lanes take consecutive 16-byte chunks of those runs.  A lane keeps its NK
+// chunks (the same row in each: 256 is a multiple of the chunks per run) in registers from the single read to the write,
+// and every load of the workgroup is in flight before the first use: 4 KiB x NK per workgroup, which is what keeps HBM
+// busy when each workgroup lives only a few microseconds.  Row statistics: shuffles over the lanes of a wavefront that
+// hold the same row, then four values per row through LDS.
+template <int MODE, int ELEM, int NK>
+__global__ __launch_bounds__(256) void ttm_rowwise_band_k(RowArgs p) {
+  constexpr int EPC = 16 / ELEM, RUN = 4 * ELEM;         // chunks per run of four face rows
+  constexpr bool IS_MAX = MODE == RW_SOFTMAX || MODE == RW_MAX;
+  constexpr bool REDUCE = MODE == RW_SUM || MODE == RW_MEAN || MODE == RW_MAX || MODE == RW_MIN;
+  __shared__ float red[4][4], red2[4][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int g4 = (int)(blockIdx.x & 7);                  // group of four rows inside the tile row
+  const int64_t trow = blockIdx.x >> 3;                  // tile row over all batch entries
+  const int rl = (tid % RUN) / ELEM, part = tid % ELEM;
+  const int r = g4 * 4 + rl;
+  const int64_t row = (trow % p.rt) * 32 + r;
+  const bool row_ok = row < p.rows;
+  const int nruns = p.ct * 2, cols = (int)p.cols;        // runs per band: one per (tile, face column)
+  const uint8_t *x = (const uint8_t *)p.x + trow * p.ct * 1024 * ELEM;
+  // chunk k of this lane: run tid / RUN + k * (256 / RUN)
+  auto run_of = [&](int k) { return tid / RUN + k * (256 / RUN); };
+  auto off_of = [&](int run) { return (int64_t)(run >> 1) * 1024 + ((r >> 4) * 2 + (run & 1)) * 256 + (r & 15) * 16 + part * EPC; };
+  auto col_of = [&](int run) { return (run >> 1) * 32 + (run & 1) * 16 + part * EPC; };
+  u32x4 v[NK];
+#pragma unroll
+  for (int k = 0; k < NK; ++k) {
+    // unconditional (a run past the end repeats the last one and is masked where it is used): a branch around a load
+    // makes the compiler wait for each load before it issues the next
+    const int run = min(run_of(k), nruns - 1);
+    v[k] = __builtin_nontemporal_load((const u32x4 *)(x + off_of(run) * ELEM));
+  }
+  u32x4 wraw[MODE == RW_RMSNORM ? NK : 1], braw[MODE == RW_RMSNORM ? NK : 1];
+  if constexpr (MODE == RW_RMSNORM) {
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+      const int c0 = col_of(min(run_of(k), nruns - 1));
+      const int64_t tiled = (int64_t)(c0 >> 5) * 1024 + ((c0 >> 4) & 1) * 256 + (c0 & 15);
+      // a null vector reads the input instead (the value is not used): no branch around the loads
+      const uint8_t *wsrc = p.w ? (const uint8_t *)p.w + (p.w_tiled ? tiled : c0) * ELEM : x;
+      const uint8_t *bsrc = p.b ? (const uint8_t *)p.b + (p.b_tiled ? tiled : c0) * ELEM : x;
+      wraw[k] = *(const u32x4 *)wsrc;
+      braw[k] = *(const u32x4 *)bsrc;
+    }
+  }
+  // the lanes of a wavefront that share a row differ in the chunk-part bits (below ELEM) and the run bits (RUN and up)
+  auto wave_combine = [&](float a, bool is_max, bool is_min) {
+#pragma unroll
+    for (int sft = 1; sft < 64; sft <<= 1) {
+      if (sft >= ELEM && sft < RUN) continue;            // the row bits
+      const float o = __shfl_xor(a, sft);
+      a = is_max ? fmaxf(a, o) : (is_min ? fminf(a, o) : a + o);
+    }
+    return a;
+  };
+  float acc = IS_MAX ? -INFINITY : (MODE == RW_MIN ? INFINITY : 0.0f);
+#pragma unroll
+  for (int k = 0; k < NK; ++k) {
+    const int run = run_of(k);
+    const int c0 = col_of(run);
+    const int lim = run < nruns ? cols : 0;
+    float f[EPC];
+    unpack_vals<ELEM>(v[k], f);
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) {
+      const bool ok = c0 + i < lim;
+      if (MODE == RW_RMSNORM) acc += ok ? f[i] * f[i] : 0.0f;
+      else if (IS_MAX) acc = ok ? fmaxf(acc, f[i]) : acc;
+      else if (MODE == RW_MIN) acc = ok ? fminf(acc, f[i]) : acc;
+      else acc += ok ? f[i] : 0.0f;
+    }
+  }
+  acc = wave_combine(acc, IS_MAX, MODE == RW_MIN);
+  if ((lane & ~(RUN - ELEM)) == 0) red[wave][rl] = acc;  // one lane per row and wavefront
+  __syncthreads();
+  float stat;
+  {
+    const float a0 = red[0][rl], a1 = red[1][rl], a2 = red[2][rl], a3 = red[3][rl];
+    stat = IS_MAX ? fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)) : (MODE == RW_MIN ? fminf(fminf(a0, a1), fminf(a2, a3)) : (a0 + a1) + (a2 + a3));
+  }
+  if constexpr (REDUCE) {
+    // output [.., rows, 1] in tile order: one column tile per tile row; this workgroup owns its four rows of it, both faces
+    if (MODE == RW_MEAN) stat = stat / (float)cols;
+    if (tid < 2 * RUN) {
+      const int fx = tid / RUN;
+      u32x4 z = u32x4{0, 0, 0, 0};
+      if (fx == 0 && part == 0 && row_ok) z.x = ELEM == 2 ? (uint32_t)ttm_f32_to_bf16(stat) : __float_as_uint(stat);
+      uint8_t *o = (uint8_t *)p.out + trow * 1024 * ELEM;
+      *(u32x4 *)(o + (int64_t)(((r >> 4) * 2 + fx) * 256 + (r & 15) * 16 + part * EPC) * ELEM) = z;
+    }
+    return;
+  } else {
+    uint8_t *o = (uint8_t *)p.out + trow * p.ct * 1024 * ELEM;
+    float mul;
+    float e[MODE == RW_SOFTMAX ? NK : 1][EPC];
+    if constexpr (MODE == RW_RMSNORM) {
+      mul = 1.0f / sqrtf(stat / (float)cols + p.eps);
+    } else {
+      float sum = 0.0f;
+#pragma unroll
+      for (int k = 0; k < NK; ++k) {
+        const int run = run_of(k);
+        const int c0 = col_of(run);
+        float f[EPC];
+        unpack_vals<ELEM>(v[k], f);
+#pragma unroll
+        for (int i = 0; i < EPC; ++i) {
+          e[k][i] = (run < nruns && c0 + i < cols) ? expf(f[i] - stat) : 0.0f;
+          sum += e[k][i];
+        }
+      }
+      sum = wave_combine(sum, false, false);
+      if ((lane & ~(RUN - ELEM)) == 0) red2[wave][rl] = sum;
+      __syncthreads();
+      mul = 1.0f / ((red2[0][rl] + red2[1][rl]) + (red2[2][rl] + red2[3][rl]));
+    }
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+      const int run = run_of(k);
+      if (run < nruns) {
+        const int c0 = col_of(run);
+        float f[EPC];
+        if constexpr (MODE == RW_RMSNORM) {
+          float w[EPC], b[EPC];
+          unpack_vals<ELEM>(v[k], f);
+          if (p.w) unpack_vals<ELEM>(wraw[k], w);
+          if (p.b) unpack_vals<ELEM>(braw[k], b);
+#pragma unroll
+          for (int i = 0; i < EPC; ++i) {
+            float y = f[i] * mul;
+            if (p.w) y *= w[i];
+            if (p.b) y += b[i];
+            f[i] = (row_ok && c0 + i < cols) ? y : 0.0f;
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < EPC; ++i) f[i] = row_ok ? e[k][i] * mul : 0.0f;
+        }
+        u32x4 ov;
+        if (ELEM == 2) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ov[i] = ttm_pack_bf16x2(f[2 * i], f[2 * i + 1]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) ov[i] = __float_as_uint(f[i]);
+        }
+        __builtin_nontemporal_store(ov, (u32x4 *)(o + off_of(run) * ELEM));
+      }
+    }
+  }
+}
+
 template <int MODE>
 static int launch_rowwise(const RowArgs &p, int dtype, int64_t trows, hipStream_t s) {
   TTM_REQUIRE(trows < (1ll << 29), "row-wise kernel: tensor too large");
+  {
+    // four rows per workgroup, whole lines, the band in registers: from one workgroup per CU upwards, rows of up to 16
+    // chunks per lane (16384 bf16 or 8192 fp32 columns).  rowwise_variant: 2 forces it, 1 and 3 exclude it.
+    const int elem = dtype == TTM_BF16 ? 2 : 4, variant = ttm_option("rowwise_variant");
+    const int nk = (int)ttm_cdiv((int64_t)p.ct * 2 * 4 * elem, 256);
+    if (nk <= 16 && trows * 8 < (1ll << 31) && (variant == 2 || (variant == 0 && trows * 8 >= 256))) {
+      const dim3 grid((unsigned)(trows * 8)), block(256);
+#define TTM_BAND_LAUNCH(E, N) hipLaunchKernelGGL((ttm_rowwise_band_k<MODE, E, N>), grid, block, 0, s, p)
+#define TTM_BAND_NK(E) \
+      do { if (nk <= 1) TTM_BAND_LAUNCH(E, 1); else if (nk <= 2) TTM_BAND_LAUNCH(E, 2); else if (nk <= 4) TTM_BAND_LAUNCH(E, 4); \
+           else if (nk <= 8) TTM_BAND_LAUNCH(E, 8); else TTM_BAND_LAUNCH(E, 16); } while (0)
+      if (dtype == TTM_BF16) TTM_BAND_NK(2); else TTM_BAND_NK(4);
+#undef TTM_BAND_NK
+#undef TTM_BAND_LAUNCH
+      TTM_LAUNCH_CHECK();
+      return TTM_OK;
+    }
+  }
   if constexpr (MODE == RW_RMSNORM || MODE == RW_SOFTMAX) {
     const int elem = dtype == TTM_BF16 ? 2 : 4;
     if (p.ct * 2 * elem <= 8 * 256 && trows * 32 < (1 << 24) && ttm_option("rowwise_variant") != 1) {   // one row per workgroup
