@@ -24,3 +24,21 @@ def test_device_pool_bookkeeping(tmp_path):
     exe = compile_cpp(tmp_path, "test_device_pool")
     r = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
     assert r.returncode == 0, r.stdout
+
+
+def test_runtime_arm_sketch_compiles_and_runs(tmp_path):
+    """The fourth dispatch arm of INTEGRATION.md: include/ttmlir_amd_runtime_arm.hpp over the C ABI, in its own namespace,
+    linked against the exported ttrt_* symbols only."""
+    import sys
+    sys.path.insert(0, ROOT)
+    import __graft_entry__ as entry
+    entry.load_package()
+    from ttmlir_amd import programs, runtime as rt
+    rt.lib()
+    path = tmp_path / "c1.ttnn"
+    path.write_bytes(programs.c1_matmul())
+    libdir = os.path.join(ROOT, "tt-mlir_amd", "lib")
+    exe = compile_cpp(tmp_path, "test_runtime_arm", ["-L", libdir, "-lttmlir_amd_rt", "-Wl,-rpath," + libdir])
+    r = subprocess.run([exe, str(path)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    assert r.returncode == 0, r.stdout
+    assert "programs=1 inputs=2 layout=(0,0,2)" in r.stdout, r.stdout      # host, row-major, bf16 inputs of config 1

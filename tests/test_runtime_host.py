@@ -2,6 +2,7 @@
 creation (strides, unsupported dtype aliases) and the buffer casts with the reference's
 known-answer vectors."""
 import ctypes
+import os
 import struct
 
 import numpy as np
@@ -266,3 +267,18 @@ def test_submit_without_device_fails_cleanly():
         pytest.skip("a GPU is visible")
     with pytest.raises(RuntimeError):
         rt.open_mesh_device()
+
+
+def test_schema_constants_are_what_the_generator_makes_of_the_schema_text():
+    """schema_generated.h / schema_names.cpp say "generated": the generator sits beside them and reproduces them from the
+    .fbs files of the tt-mlir checkout, where one is at hand (it is not on the GPU box)."""
+    import importlib.util
+    ref = "/root/reference"
+    if not os.path.isdir(os.path.join(ref, "include", "ttmlir", "Target", "TTNN")):
+        pytest.skip("no tt-mlir checkout at " + ref)
+    rtdir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "tt-mlir_amd", "runtime")
+    spec = importlib.util.spec_from_file_location("gen_schema", os.path.join(rtdir, "gen_schema.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    for fname, text in gen.generate(ref).items():
+        assert open(os.path.join(rtdir, fname)).read() == text, fname + " differs from the generator's output"

@@ -772,19 +772,6 @@ __device__ __forceinline__ void lds_dma16(const void *base, uint32_t lane_off, u
 
 // One output block of 2 NTW x 8 tiles (NTW = 4, 3 or 2 column tiles per wavefront); bid / nblk number the blocks of
 // the column range [nt_first, nt_end) that this body covers.
-// Optional instrumentation (compile with -DTTM_LINEAR_TRACE): wavefronts 0 and 4 of one block record the cycle
-// counter at eight points of every step; ttm_debug_trace copies the record out.
-#ifdef TTM_LINEAR_TRACE
-__device__ unsigned long long ttm_trace_buf[2 * 64 * 8];
-TTM_EXPORT int ttm_debug_trace(void *dst, size_t bytes) {
-  TTM_HIP(hipMemcpyFromSymbol(dst, HIP_SYMBOL(ttm_trace_buf), bytes));
-  return TTM_OK;
-}
-#define TTM_TRACE(slot) do { if (tracing && ks < 64) { unsigned long long t_ = __builtin_readcyclecounter(); if (lane == 0) ttm_trace_buf[((wave >> 2) * 64 + ks) * 8 + (slot)] = t_; } } while (0)
-#else
-#define TTM_TRACE(slot) do { } while (0)
-#endif
-
 // IMG = true is the second pass of a two-pass launch: p.W holds the weights already dequantised to bf16, one 4 KiB
 // LDS fragment image per (k-step, column tile) (ttm_linear_image_k), so a step's weights are a straight LDS-direct copy
 // and the conversion, the raw staging area and the exponent loads drop out of the loop.
@@ -1018,13 +1005,9 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   // on the issue port).  The block barrier sits between chunks 2 and 3: chunk 3 multiplies from fragments that
   // were requested before the barrier and already requests chunk 0 of the next stage, so the matrix core does
   // not drain at the barrier; its conversion quarter (c = 0) belongs to the step after next.
-#ifdef TTM_LINEAR_TRACE
-  const bool tracing = blockIdx.x == 17 && blockIdx.y == 0 && blockIdx.z == 0 && (wave == 0 || wave == 4);
-#endif
   auto step = [&](auto stage_c, int ks) {
     constexpr uint32_t CUR = decltype(stage_c)::value * STAGE, NXT = STAGE - CUR;
     constexpr uint32_t RCUR = decltype(stage_c)::value * RAW_STAGE, RNXT = RAW_STAGE - RCUR;
-    TTM_TRACE(0);
 #pragma unroll
     for (int q = 0; q < 3; ++q) {
       // the global-memory pipe takes about 16 cycles per LDS-direct instruction: the activation loads of a step are
@@ -1039,16 +1022,8 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
       quarter(q + 1, RNXT, NXT);
       mfma_chunk(q & 1);
       __builtin_amdgcn_sched_barrier(0);
-      TTM_TRACE(1 + q);
     }
-#ifdef TTM_LINEAR_TRACE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    TTM_TRACE(4);
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    TTM_TRACE(5);
-#endif
     landed_barrier();
-    TTM_TRACE(6);
     exps = u32x2{exps_next.x & keep_next, exps_next.y & keep_next};
     // stage CUR of the activations and stage RNXT of the mantissas are free now
     exps_next = load_exps((ks + 3) * 2, keep_next);
@@ -1059,7 +1034,6 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     quarter(0, RCUR, CUR);
     mfma_chunk(1);
     __builtin_amdgcn_sched_barrier(0);
-    TTM_TRACE(7);
   };
   // an odd number of steps is rounded up: the extra step multiplies zeroed weights
   for (int ks = 0; ks < ksteps; ks += 2) {

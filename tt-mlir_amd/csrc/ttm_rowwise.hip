@@ -392,6 +392,9 @@ __global__ __launch_bounds__(256) void ttm_rowwise_row_k(RowArgs p, int total_ro
 // and every load of the workgroup is in flight before the first use: 4 KiB x NK per workgroup, which is what keeps HBM
 // busy when each workgroup lives only a few microseconds.  Row statistics: shuffles over the lanes of a wavefront that
 // hold the same row, then four values per row through LDS.
+#ifndef TTM_BAND_EXP
+#define TTM_BAND_EXP expf
+#endif
 template <int MODE, int ELEM, int NK>
 __global__ __launch_bounds__(256) void ttm_rowwise_band_k(RowArgs p) {
   constexpr int EPC = 16 / ELEM, RUN = 4 * ELEM;         // chunks per run of four face rows
@@ -494,7 +497,7 @@ __global__ __launch_bounds__(256) void ttm_rowwise_band_k(RowArgs p) {
         unpack_vals<ELEM>(v[k], f);
 #pragma unroll
         for (int i = 0; i < EPC; ++i) {
-          e[k][i] = (run < nruns && c0 + i < cols) ? expf(f[i] - stat) : 0.0f;
+          e[k][i] = (run < nruns && c0 + i < cols) ? TTM_BAND_EXP(f[i] - stat) : 0.0f;
           sum += e[k][i];
         }
       }

@@ -9,7 +9,8 @@ import re
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(_HERE)
-LIB_PATH = os.path.join(_HERE, "lib", "libttmlir_amd_hip.so")
+# TTMLIR_AMD_HIP_LIB names another build of the library (a kernel variant under measurement)
+LIB_PATH = os.environ.get("TTMLIR_AMD_HIP_LIB") or os.path.join(_HERE, "lib", "libttmlir_amd_hip.so")
 HEADER = os.path.join(ROOT, "include", "ttmlir_amd_hip.h")
 
 F32, F16, BF16, BFP8B, BFP4B, U32, U16, U8, I32 = 0, 1, 2, 4, 6, 9, 10, 11, 12
