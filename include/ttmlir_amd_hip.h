@@ -323,6 +323,25 @@ int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const 
                              int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                              const void *attention_sink, void *stream);
 
+/* ---- chunked prefill over a paged cache: ::ttnn::transformer::chunked_scaled_dot_product_attention
+ * (runtime/lib/ttnn/operations/transformer/chunked_scaled_dot_product_attention.cpp; golden tools/golden/mapping.py:8847-8913)
+ * is three launches: ttm_paged_gather brings the pages of every user into a contiguous [users, heads, pages_per_user *
+ * block_size, head_dim] TILE tensor (cache [blocks, heads, block_size, head_dim], page_table [users, pages_per_user] in
+ * device memory; entries outside [0, blocks) read as zeros), ttm_chunk_causal_mask writes the additive BFloat16 TILE mask
+ * [rows, cols] of a chunk whose first query stands at position *chunk_start (device memory): 0 where col <= *chunk_start +
+ * row, -inf elsewhere, and ttm_sdpa_windowed attends with that mask.  Nothing is read on the host, so the op can be
+ * recorded into a graph and replayed with another chunk_start.
+ *
+ * ttm_rotary_embedding_llama: ::ttnn::experimental::rotary_embedding_llama (runtime/lib/ttnn/operations/transformer/
+ * rotary_embedding_llama.cpp:11-34; operand shapes lib/Dialect/TTNN/IR/TTNNOps.cpp:6293-6380): out = x * cos + (x T) * sin
+ * with the 32 x 32 BFloat16 TILE matrix T applied to every 32-column tile of a row; x / out [batch, rows, cols], cos / sin
+ * [cs_batch, cs_rows, cols] broadcast over batch (entry b % cs_batch) and, when cs_rows is 1, over rows. */
+int ttm_paged_gather(const void *cache, const int32_t *page_table, void *out, int dtype, int64_t blocks, int64_t heads,
+                     int64_t block_size, int64_t head_dim, int64_t users, int64_t pages_per_user, void *stream);
+int ttm_chunk_causal_mask(void *mask, const int32_t *chunk_start, int64_t rows, int64_t cols, void *stream);
+int ttm_rotary_embedding_llama(const void *x, const void *cos_cache, const void *sin_cache, const void *trans_mat, void *out,
+                               int dtype, int64_t batch, int64_t rows, int64_t cols, int64_t cs_batch, int64_t cs_rows, void *stream);
+
 /* ttm_sdpa_decode_windowed that allocates nothing.  It has no counterpart in the reference; it is for callers that cannot
  * call hipMalloc: code under HIP graph capture, tight serving loops, harnesses that forbid allocation.  Same arguments, same
  * kernels and bit-identical results; the per-slice partial results (max, sum, unnormalised output) go to a static device

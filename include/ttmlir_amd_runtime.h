@@ -205,6 +205,20 @@ int ttrt_pb_load_cached(ttrt_builder *pb, uint32_t program_index, const char *ca
                         uint32_t *outs);
 int ttrt_pb_func_call(ttrt_builder *pb, uint32_t program_index, const uint32_t *ins, int n_in, const uint32_t *out_shapes,
                       const int *out_ranks, const ttrt_layout *out_layouts, int n_out, uint32_t *outs);
+/* CpuOp (include/ttmlir/Target/TTNN/operations/cpu.fbs; runner runtime/lib/ttnn/operations/cpu/cpu.cpp:215-238): a call of
+ * `func_name` in the dynamic library that ttrt_pb_add_dylib embedded in the open program under dylib_id
+ * (Program.dylibs, include/ttmlir/Target/Common/types.fbs:157-160).  The function has the CPU-hoisting ABI of
+ * runtime/include/tt/runtime/detail/common/dylib.h:35-42: WrappedTensor *f(WrappedTensor *inputs) on dense row-major host
+ * tensors of 4-byte elements, outputs allocated with malloc by the callee and freed by the runtime. */
+/* RotaryEmbeddingLlamaOp, ChunkedScaledDotProductAttentionOp (include/ttmlir/Target/TTNN/operations/transformer.fbs:13-22,
+ * 150-160) */
+int ttrt_pb_rotary_embedding_llama(ttrt_builder *pb, uint32_t in, uint32_t cos_cache, uint32_t sin_cache, uint32_t trans_mat,
+                                   int decode_mode, uint32_t *out);
+int ttrt_pb_chunked_sdpa(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t page_table, uint32_t chunk_start,
+                         int has_scale, float scale, uint32_t *out);
+int ttrt_pb_add_dylib(ttrt_builder *pb, uint32_t dylib_id, const void *data, size_t size);
+int ttrt_pb_cpu_op(ttrt_builder *pb, uint32_t dylib_id, const char *func_name, const uint32_t *ins, int n_in,
+                   const uint32_t *out_shapes, const int *out_ranks, const ttrt_layout *out_layouts, int n_out, uint32_t *outs);
 
 #ifdef __cplusplus
 }

@@ -446,3 +446,33 @@ def clamp(x, lo, hi):
     """tools/golden/mapping.py:5267-5276 (torch.clamp with scalar bounds; NaN stays NaN)."""
     x = np.asarray(x, np.float32)
     return np.where(np.isnan(x), x, np.minimum(np.maximum(x, np.float32(lo)), np.float32(hi))).astype(np.float32)
+
+
+def chunked_sdpa(q, k_pages, v_pages, page_table, chunk_start, scale=None):
+    """Chunked prefill over a paged cache (tools/golden/mapping.py:8847-8913): q [B, H, Sq, D]; pages [blocks, Hkv, block, D];
+    page_table [B, pages_per_user]; query row j stands at position chunk_start + j and sees keys [0, chunk_start + j].  The
+    pages are unpaged with the table (entries clamped into range, as the golden does), the band is written as an additive
+    mask and the prefill attention of this module does the rest."""
+    q, kp, vp = _c(q, np.float32), _c(k_pages, np.float32), _c(v_pages, np.float32)
+    B, H, Sq, D = q.shape
+    blocks, Hkv, block, _ = kp.shape
+    pt = np.clip(np.asarray(page_table, dtype=np.int64), 0, blocks - 1)
+    pages = pt.shape[-1]
+    Sk = pages * block
+    unpage = lambda c: _c(c[pt.reshape(-1)].reshape(B, pages, Hkv, block, D).transpose(0, 2, 1, 3, 4).reshape(B, Hkv, Sk, D))
+    col = np.arange(Sk)[None, :]
+    row = (int(chunk_start) + np.arange(Sq))[:, None]
+    mask = np.where(col <= row, 0.0, -np.inf).astype(np.float32)[None, None]
+    return sdpa(q, unpage(kp), unpage(vp), mask=mask, is_causal=False, scale=scale)
+
+
+def rotary_embedding_llama(x, cos, sin, trans_mat):
+    """out = x * cos + (x T) * sin with the 32 x 32 matrix T applied to every 32-column tile of the last dim
+    (::ttnn::experimental::rotary_embedding_llama as called from runtime/lib/ttnn/operations/transformer/
+    rotary_embedding_llama.cpp:11-34; the op has no golden in the reference).  x [.., R, D]; cos / sin broadcast
+    against it; f32 arithmetic, as the CPU path computes."""
+    x = _c(x, np.float32)
+    T = _c(trans_mat, np.float32).reshape(32, 32)
+    xt = x.reshape(x.shape[:-1] + (x.shape[-1] // 32, 32))
+    rot = np.einsum("...tj,jc->...tc", xt, T).reshape(x.shape).astype(np.float32)
+    return (x * np.asarray(cos, dtype=np.float32) + rot * np.asarray(sin, dtype=np.float32)).astype(np.float32)

@@ -431,6 +431,149 @@ def test_const_eval_results_die_with_their_device(orc):
         rt.to_host(t, untilize=True)
 
 
+def test_cpu_op_runs_a_function_of_an_embedded_dynamic_library(device, orc, tmp_path):
+    """CpuOp (runtime/lib/ttnn/operations/cpu/cpu.cpp:215-238): the program carries a shared library as bytes
+    (Program.dylibs, runtime/lib/common/dylib.cpp:13-38); the op calls `<name>_helper(WrappedTensor *)` on host tensors and
+    takes ownership of what the callee allocated.  The library here is tests/cpp/cpu_hoisted_ops.c, compiled on the spot;
+    the device part of the program (a matmul) feeds the hoisted function through from_device, as the compiler emits it."""
+    import os
+    import subprocess
+    src = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "cpu_hoisted_ops.c")
+    so = tmp_path / "hoisted.so"
+    subprocess.run(["gcc", "-shared", "-fPIC", "-O1", "-o", str(so), src], check=True)
+    pb = rt.ProgramBuilder()
+    pb.begin_program("cpu_op")
+    pb.add_dylib(7, so.read_bytes())
+    a = pb.input((64, 96), DT.BFloat16)
+    b = pb.input((96, 32), DT.BFloat16)
+    c = pb.input((64, 32), DT.Float32, TL.RowMajor, ST.Host)
+    v = pb.input((40,), DT.Float32, TL.RowMajor, ST.Host)
+    prod = pb.from_device(pb.to_layout(pb.matmul(a, b), TL.RowMajor, DT.Float32))
+    host = lambda shape, dt: (shape, rt.Layout(ST.Host, TL.RowMajor, dt))
+    s0, s1 = pb.cpu_op(7, "cpu_hoisted_add_rowsum_0a1b2c3d_helper", [prod, c], [host((64, 32), DT.Float32), host((64,), DT.Int32)])
+    d0, d1 = pb.cpu_op(7, "cpu_hoisted_alias_helper", [v], [host((40,), DT.Float32), host((40,), DT.Float32)])
+    back = pb.matmul(pb.to_layout(pb.to_device(s0), TL.Tile, DT.BFloat16), pb.to_layout(pb.to_device(s0), TL.Tile, DT.BFloat16), transpose_b=True)
+    for t in (s0, s1, d0, d1, back):
+        pb.output(t)
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    ta, tb = datagen.randn((64, 96), seed=60, dtype=torch.bfloat16), datagen.randn((96, 32), seed=61, dtype=torch.bfloat16)
+    tc, tv = datagen.randn((64, 32), seed=62), datagen.randn((40,), seed=63)
+    for _ in range(2):      # the library is loaded once per binary; the second run finds it
+        ins = [rt.to_layout(rt.from_torch(t), device, rt.get_layout(binary, 0, i)) for i, t in enumerate((ta, tb, tc, tv))]
+        outs = rt.submit(device, binary, 0, ins)
+        rt.wait(outs)
+        got = [rt.to_torch(rt.to_host(o, untilize=True)[0]) for o in outs]
+        mm = orc.round_bf16(orc.linear(ta.float().numpy(), tb.float().numpy()))
+        want0 = mm + tc.numpy()
+        assert np.array_equal(got[0].numpy(), want0)
+        assert np.array_equal(got[1].numpy(), want0.sum(-1, dtype=np.float32).astype(np.int32))   # same order of additions
+        assert np.array_equal(got[2].numpy(), 2 * tv.numpy()) and np.array_equal(got[3].numpy(), 2 * tv.numpy())
+        s0b = orc.round_bf16(want0)
+        assert np.max(np.abs(got[4].float().numpy() - orc.round_bf16(orc.linear(s0b, s0b.T.copy())))) <= 2.0 ** -3   # |y| up to ~60
+        del outs, got
+    # a name the library does not have, a dylib id the program does not have: the reference's messages
+    for dylib, name, msg in ((7, "no_such_helper", "could not find requested op"), (8, "cpu_hoisted_alias_helper", "could not find dylib")):
+        pb = rt.ProgramBuilder()
+        pb.begin_program("bad")
+        pb.add_dylib(7, so.read_bytes())
+        x = pb.input((40,), DT.Float32, TL.RowMajor, ST.Host)
+        (o,) = pb.cpu_op(dylib, name, [x], [host((40,), DT.Float32)])
+        pb.output(o)
+        pb.end_program()
+        bad = rt.Binary.load_from_memory(pb.finish())
+        with pytest.raises(RuntimeError, match=msg):
+            rt.submit(device, bad, 0, [rt.from_torch(tv)])
+
+
+def test_chunked_prefill_attention_program(device, orc, metrics):
+    """ChunkedScaledDotProductAttentionOp: three chunks of a sequence attend over a paged cache that holds the whole prefix,
+    one program submitted with a new chunk_start_idx each time (a device-resident [1] Int32 the kernels read)."""
+    B, H, Hkv, Sq, D, block, pages = 2, 8, 2, 96, 128, 64, 6
+    Sk = block * pages
+    g = torch.Generator().manual_seed(70)
+    k = datagen.randn((B, Hkv, Sk, D), seed=71, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, Sk, D), seed=72, dtype=torch.bfloat16)
+    table = torch.randperm(B * pages + 3, generator=g)[:B * pages].reshape(B, pages).to(torch.int32)
+    kp = torch.zeros((B * pages + 3, Hkv, block, D), dtype=torch.bfloat16)
+    vp = torch.zeros_like(kp)
+    for b in range(B):
+        for p in range(pages):
+            kp[table[b, p]] = k[b, :, p * block:(p + 1) * block]
+            vp[table[b, p]] = v[b, :, p * block:(p + 1) * block]
+    pb = rt.ProgramBuilder()
+    pb.begin_program("chunked_prefill")
+    iq = pb.input((B, H, Sq, D), DT.BFloat16)
+    ik, iv = pb.input(tuple(kp.shape), DT.BFloat16), pb.input(tuple(vp.shape), DT.BFloat16)
+    it = pb.input((B, pages), DT.Int32, TL.RowMajor)
+    ist = pb.input((1,), DT.Int32, TL.RowMajor)
+    pb.output(pb.chunked_sdpa(iq, ik, iv, it, ist))
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    lay = lambda i: rt.get_layout(binary, 0, i)
+    res = [rt.to_layout(rt.from_torch(t), device, lay(1 + i), retain=True) for i, t in enumerate((kp, vp, table))]
+    f = lambda t: t.float().numpy()
+    for start in (0, 96, Sk - Sq):
+        q = datagen.randn((B, H, Sq, D), seed=73 + start, dtype=torch.bfloat16)
+        ins = [rt.to_layout(rt.from_torch(q), device, lay(0))] + res + [rt.to_layout(rt.from_torch(torch.tensor([start], dtype=torch.int32)), device, lay(4))]
+        (o,) = rt.submit(device, binary, 0, ins)
+        got = f(rt.to_torch(rt.to_host(o, untilize=True)[0]))
+        want = orc.chunked_sdpa(f(q), f(kp), f(vp), table.numpy(), start)
+        assert np.all(np.isfinite(got)) and np.max(np.abs(got - want)) <= 2.0 ** -6
+        assert metrics.get_pcc(want, got) >= 0.9999
+
+
+@pytest.mark.parametrize("decode", [False, True])
+def test_rotary_embedding_llama_program(device, orc, decode):
+    """RotaryEmbeddingLlamaOp in both modes: prefill x [1, heads, seq, head_dim] with cos / sin [1, 1, seq, head_dim];
+    decode x [1, users, heads, head_dim] with one cos / sin row per user, [1, users, 1, head_dim]."""
+    shape, cshape = ((1, 8, 70, 128), (1, 1, 70, 128)) if not decode else ((1, 5, 8, 64), (1, 5, 1, 64))
+    x = datagen.randn(shape, seed=80, dtype=torch.bfloat16)
+    ang = datagen.randn(cshape[:-1] + (cshape[-1] // 2,), seed=81) * 2.0
+    cos = torch.repeat_interleave(ang.cos(), 2, -1).to(torch.bfloat16)
+    sin = torch.repeat_interleave(ang.sin(), 2, -1).to(torch.bfloat16)
+    T = torch.zeros((1, 1, 32, 32), dtype=torch.bfloat16)
+    for i in range(16):
+        T[0, 0, 2 * i + 1, 2 * i], T[0, 0, 2 * i, 2 * i + 1] = -1.0, 1.0
+    pb = rt.ProgramBuilder()
+    pb.begin_program("rope_llama")
+    ids = [pb.input(tuple(t.shape), DT.BFloat16) for t in (x, cos, sin, T)]
+    pb.output(pb.rotary_embedding_llama(*ids, decode_mode=decode))
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    (y,) = harness.execute(binary, 0, [x, cos, sin, T], device)
+    f = lambda t: t.float().numpy()
+    want = orc.rotary_embedding_llama(f(x), f(cos), f(sin), f(T))
+    got = f(y)
+    # two products and a sum of bf16 values in fp32 (the 32-term row product has two non-zero terms), rounded once
+    assert np.max(np.abs(got - orc.round_bf16(want))) <= 2.0 ** -8 * np.maximum(1.0, np.max(np.abs(want)))
+    assert np.mean(got == orc.round_bf16(want)) > 0.99
+
+
+def test_profiler_ranges_per_operation():
+    """TTMLIR_RUNTIME_PROFILE_OPS=1 wraps every operation in a roctx range named by its type and location (the reference's
+    tracy zone + MLIR_OP_LOCATION message, runtime/lib/ttnn/program_executor.cpp:223-237); TTMLIR_RUNTIME_SYNC_AFTER_OP=1
+    adds a device wait per operation.  Both are read once per process, so the check runs in a child process."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys; sys.path.insert(0, %r)\n"
+        "import __graft_entry__ as e; e.load_package()\n"
+        "from ttmlir_amd import datagen, programs, runtime as rt, harness\n"
+        "a, b = datagen.c1_matmul()\n"
+        "binary = rt.Binary.load_from_memory(programs.c1_matmul())\n"
+        "rt.clear_stats()\n"
+        "(c, _) = harness.execute(binary, 0, [a, b])\n"
+        "print('RANGES', rt.get_stat('ProfiledOpRange'), 'OPS', len(binary.get_program_ops_as_json(0)))\n" % root)
+    env = dict(os.environ, TTMLIR_RUNTIME_PROFILE_OPS="1", TTMLIR_RUNTIME_SYNC_AFTER_OP="1")
+    r = subprocess.run([sys.executable, "-c", code], env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    assert r.returncode == 0, r.stdout
+    line = [l for l in r.stdout.splitlines() if l.startswith("RANGES")][0].split()
+    assert int(line[1]) == int(line[3]) > 0, r.stdout
+
+
 def test_embedded_goldens_are_checked_per_operation(device, orc):
     """`ttrt run --enable-golden` flow: every op with a golden embedded in the binary is compared in the post-op hook."""
     d = datagen.c4_mlp(64, 128, 256, seed=11)

@@ -408,3 +408,53 @@ def test_clamp_against_torch(orc):
     x[:3] = [np.nan, np.inf, -np.inf]
     for lo, hi in ((-1.0, 2.5), (0.0, 0.0), (-3.0, -1.0)):
         assert np.array_equal(orc.clamp(x, lo, hi), torch.clamp(torch.from_numpy(x), min=lo, max=hi).numpy(), equal_nan=True)
+
+
+def test_chunked_sdpa_is_causal_attention_of_the_chunk_over_the_unpaged_prefix(orc):
+    """tools/golden/mapping.py:8847-8913 builds the same thing from torch: unpage with the table, mask col <= start + row,
+    F.scaled_dot_product_attention.  Also fixed by the definition: a chunk that starts at 0 and spans the cache is plain
+    causal attention, and the rows of a later chunk are the last rows of the causal attention over the whole sequence."""
+    rng = np.random.default_rng(7)
+    B, H, Hkv, Sq, D, block, pages = 2, 4, 2, 40, 32, 32, 4
+    Sk = block * pages
+    k = rng.standard_normal((B, Hkv, Sk, D)).astype(np.float32)
+    v = rng.standard_normal((B, Hkv, Sk, D)).astype(np.float32)
+    table = rng.permutation(B * pages).reshape(B, pages)
+    kp = np.zeros((B * pages, Hkv, block, D), np.float32)
+    vp = np.zeros_like(kp)
+    for b in range(B):
+        for p in range(pages):
+            kp[table[b, p]] = k[b, :, p * block:(p + 1) * block]
+            vp[table[b, p]] = v[b, :, p * block:(p + 1) * block]
+    for start in (0, 17, Sk - Sq):
+        q = rng.standard_normal((B, H, Sq, D)).astype(np.float32)
+        got = orc.chunked_sdpa(q, kp, vp, table, start)
+        col, row = torch.arange(Sk).view(1, Sk), (start + torch.arange(Sq)).view(Sq, 1)
+        m = torch.zeros((1, 1, Sq, Sk)).masked_fill_(~(col <= row).view(1, 1, Sq, Sk), torch.finfo(torch.float32).min)
+        rep = lambda t: torch.repeat_interleave(torch.from_numpy(t), H // Hkv, dim=1)
+        want = F.scaled_dot_product_attention(torch.from_numpy(q), rep(k), rep(v), attn_mask=m).numpy()
+        assert np.max(np.abs(got - want)) <= 2e-6
+    # the last Sq rows of plain causal attention over all Sk positions
+    qfull = rng.standard_normal((B, H, Sk, D)).astype(np.float32)
+    full = orc.sdpa(qfull, k, v, is_causal=True)
+    assert np.max(np.abs(orc.chunked_sdpa(qfull[:, :, Sk - Sq:], kp, vp, table, Sk - Sq) - full[:, :, Sk - Sq:])) <= 2e-6
+
+
+def test_rotary_embedding_llama_with_the_pair_rotation_matrix_is_interleaved_rope(orc):
+    """No golden exists for the op; what fixes it: with the matrix that maps (x[2i], x[2i+1]) to (-x[2i+1], x[2i]) - the one
+    Llama passes - the result is the rotation of every interleaved pair by its angle; with the zero matrix it is x * cos;
+    with the identity it is x * (cos + sin)."""
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((1, 3, 40, 64)).astype(np.float32)
+    ang = rng.standard_normal((1, 1, 40, 32)).astype(np.float32)
+    cos, sin = np.repeat(np.cos(ang), 2, -1), np.repeat(np.sin(ang), 2, -1)
+    T = np.zeros((32, 32), np.float32)
+    for i in range(16):
+        T[2 * i + 1, 2 * i] = -1.0     # (x T)[2i] = -x[2i+1]
+        T[2 * i, 2 * i + 1] = 1.0      # (x T)[2i+1] = x[2i]
+    got = orc.rotary_embedding_llama(x, cos, sin, T)
+    z = (x[..., 0::2] + 1j * x[..., 1::2]) * np.exp(1j * ang)
+    want = np.stack([z.real, z.imag], -1).reshape(x.shape)
+    assert np.max(np.abs(got - want)) <= 1e-5
+    assert np.array_equal(orc.rotary_embedding_llama(x, cos, sin, np.zeros((32, 32))), x * cos)
+    assert np.allclose(orc.rotary_embedding_llama(x, cos, sin, np.eye(32)), x * cos + x * sin, atol=1e-6)

@@ -172,6 +172,73 @@ __global__ __launch_bounds__(256) void ttm_paged_fill_cache_k(T *__restrict__ ca
   if (sizeof(T) == 4) *(u32x4 *)(dst + 4) = *(const u32x4 *)(src + 4);
 }
 
+// gather: out[b, h, s, :] = cache[table[b, s / block_size], h, s % block_size, :] for s < pages * block_size, the inverse
+// of the paged fill; positions whose page is outside the cache read as zeros; one thread per 8 elements
+template <typename T>
+__global__ __launch_bounds__(256) void ttm_paged_gather_k(const T *__restrict__ cache, const int32_t *__restrict__ table, T *__restrict__ out,
+                                                          int64_t blocks, int64_t heads, int64_t block_size, int64_t dim, int64_t pages,
+                                                          int64_t total8) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const int64_t d8 = dim >> 3, ct = dim >> 5, seq = pages * block_size;
+  const int64_t c = (i % d8) * 8, s = (i / d8) % seq, h = (i / (d8 * seq)) % heads, b = i / (d8 * seq * heads);
+  const int64_t blk = table[b * pages + s / block_size];
+  T *dst = out + (b * heads + h) * seq * dim + ttm_tiled_offset(s, c, ct);
+  u32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+  if (blk >= 0 && blk < blocks) {
+    const T *src = cache + (blk * heads + h) * block_size * dim + ttm_tiled_offset(s % block_size, c, ct);
+    lo = *(const u32x4 *)src;
+    if (sizeof(T) == 4) hi = *(const u32x4 *)(src + 4);
+  }
+  *(u32x4 *)dst = lo;
+  if (sizeof(T) == 4) *(u32x4 *)(dst + 4) = hi;
+}
+
+// additive mask of a prefill chunk: query row i stands at absolute position *start + i and sees the keys up to it;
+// mask[i, j] = 0 where j <= *start + i, -inf elsewhere.  bf16 tiles [rows_pad, cols_pad]; the offset is read from device
+// memory, so the launch can be recorded into a graph and replayed for the next chunk
+__global__ __launch_bounds__(256) void ttm_chunk_mask_k(uint16_t *__restrict__ mask, const int32_t *__restrict__ start, int64_t rows_pad,
+                                                        int64_t cols_pad, int64_t total8) {
+  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total8) return;
+  const int64_t c8 = cols_pad >> 3, r = i / c8, c = (i % c8) * 8;
+  const int64_t limit = (int64_t)start[0] + r;
+  uint32_t w[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint32_t lo = c + 2 * k <= limit ? 0u : 0xFF80u, hi = c + 2 * k + 1 <= limit ? 0u : 0xFF80u;
+    w[k] = lo | (hi << 16);
+  }
+  *(u32x4 *)(mask + ttm_tiled_offset(r, c, cols_pad >> 5)) = u32x4{w[0], w[1], w[2], w[3]};
+}
+
+// rotary embedding with a transformation matrix: out = x * cos + (x T) * sin, where T is a 32 x 32 matrix applied to
+// every 32-column tile of a row (for the matrix Llama uses this rotates the interleaved pairs (x[2i], x[2i+1])).
+// x / out [batch, rows, cols] tiles; cos / sin [cs_batch, cs_rows, cols] tiles, row r of batch entry b reads cos row
+// (r if cs_rows > 1 else 0) of entry (b % cs_batch if cs_batch > 1 else 0).  One thread per element; T sits in LDS.
+__global__ __launch_bounds__(256) void ttm_rotary_llama_k(const uint16_t *__restrict__ x, const uint16_t *__restrict__ cosc,
+                                                          const uint16_t *__restrict__ sinc, const uint16_t *__restrict__ tmat,
+                                                          uint16_t *__restrict__ out, int64_t rows, int64_t rows_pad, int64_t cols,
+                                                          int64_t cs_batch, int64_t cs_rows, int64_t cs_rows_pad, int64_t total) {
+  __shared__ float T[32][33];
+  for (int e = threadIdx.x; e < 1024; e += 256) T[e >> 5][e & 31] = ttm_bf16_to_f32(tmat[ttm_tiled_offset(e >> 5, e & 31, 1)]);
+  __syncthreads();
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int64_t c = i % cols, r = (i / cols) % rows_pad, b = i / (cols * rows_pad), ct = cols >> 5;
+  const int64_t off = b * rows_pad * cols + ttm_tiled_offset(r, c, ct);
+  if (r >= rows) { out[off] = 0; return; }   // tile padding stays zero
+  const int64_t cb = cs_batch > 1 ? b % cs_batch : 0, cr = cs_rows > 1 ? r : 0;
+  const int64_t coff = cb * cs_rows_pad * cols + ttm_tiled_offset(cr, c, ct);
+  const uint16_t *xr = x + b * rows_pad * cols;
+  float rot = 0.0f;
+  const int64_t c0 = c & ~(int64_t)31;
+#pragma unroll 8
+  for (int j = 0; j < 32; ++j) rot += ttm_bf16_to_f32(xr[ttm_tiled_offset(r, c0 + j, ct)]) * T[j][c & 31];
+  // fp32 throughout, one rounding at the end (the convention of the CPU path: compute in f32, cast back)
+  out[off] = ttm_f32_to_bf16(ttm_bf16_to_f32(x[off]) * ttm_bf16_to_f32(cosc[coff]) + rot * ttm_bf16_to_f32(sinc[coff]));
+}
+
 // ------------------------------------------------------------------------------------------------ attention, one query token
 // q [1, B, H, D], k / v [B, Hkv, S, D] (or pages [blocks, Hkv, block, D] behind a page table), out [1, B, H, D], bf16 tiles.
 // grid (splits, B * Hkv), 256 threads.  A block owns the G = H / Hkv query heads of one kv head and one slice of the keys:
@@ -716,4 +783,52 @@ TTM_EXPORT int ttm_sdpa_decode_static(const void *q, const void *k, const void *
                                       const void *attention_sink, void *stream) {
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, true, stream);
+}
+
+TTM_EXPORT int ttm_paged_gather(const void *cache, const int32_t *page_table, void *out, int dtype, int64_t blocks, int64_t heads,
+                                int64_t block_size, int64_t head_dim, int64_t users, int64_t pages_per_user, void *stream) {
+  TTM_REQUIRE(cache && page_table && out, "ttm_paged_gather: null pointer");
+  TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_paged_gather: dtype must be BFloat16 or Float32");
+  TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_paged_gather: head dim must be a positive multiple of 32");
+  TTM_REQUIRE(block_size > 0 && block_size % 32 == 0, "ttm_paged_gather: block size must be a positive multiple of 32");
+  TTM_REQUIRE(blocks > 0 && heads > 0 && users >= 0 && pages_per_user > 0, "ttm_paged_gather: bad extents");
+  const int64_t total8 = users * heads * pages_per_user * block_size * (head_dim / 8);
+  if (total8 == 0) return TTM_OK;
+  const dim3 grid((unsigned)ttm_cdiv(total8, 256));
+  if (dtype == TTM_BF16)
+    hipLaunchKernelGGL(ttm_paged_gather_k<uint16_t>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t *)cache, page_table,
+                       (uint16_t *)out, blocks, heads, block_size, head_dim, pages_per_user, total8);
+  else
+    hipLaunchKernelGGL(ttm_paged_gather_k<float>, grid, dim3(256), 0, (hipStream_t)stream, (const float *)cache, page_table, (float *)out,
+                       blocks, heads, block_size, head_dim, pages_per_user, total8);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+TTM_EXPORT int ttm_chunk_causal_mask(void *mask, const int32_t *chunk_start, int64_t rows, int64_t cols, void *stream) {
+  TTM_REQUIRE(mask && chunk_start, "ttm_chunk_causal_mask: null pointer");
+  TTM_REQUIRE(rows > 0 && cols > 0, "ttm_chunk_causal_mask: bad extents");
+  const int64_t rp = ttm_round_up32(rows), cp = ttm_round_up32(cols), total8 = rp * cp / 8;
+  hipLaunchKernelGGL(ttm_chunk_mask_k, dim3((unsigned)ttm_cdiv(total8, 256)), dim3(256), 0, (hipStream_t)stream, (uint16_t *)mask,
+                     chunk_start, rp, cp, total8);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
+TTM_EXPORT int ttm_rotary_embedding_llama(const void *x, const void *cos_cache, const void *sin_cache, const void *trans_mat, void *out,
+                                          int dtype, int64_t batch, int64_t rows, int64_t cols, int64_t cs_batch, int64_t cs_rows,
+                                          void *stream) {
+  TTM_REQUIRE(x && cos_cache && sin_cache && trans_mat && out, "ttm_rotary_embedding_llama: null pointer");
+  TTM_REQUIRE(dtype == TTM_BF16, "ttm_rotary_embedding_llama: tensors must be BFloat16");
+  TTM_REQUIRE(batch >= 0 && rows > 0 && cols > 0 && cols % 32 == 0 && cols <= 256,
+              "ttm_rotary_embedding_llama: head dim must be a multiple of 32 up to 256");
+  TTM_REQUIRE(cs_batch >= 1 && (cs_rows == 1 || cs_rows == rows), "ttm_rotary_embedding_llama: cos / sin must have 1 or %lld rows",
+              (long long)rows);
+  const int64_t rp = ttm_round_up32(rows), total = batch * rp * cols;
+  if (total == 0) return TTM_OK;
+  hipLaunchKernelGGL(ttm_rotary_llama_k, dim3((unsigned)ttm_cdiv(total, 256)), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)x,
+                     (const uint16_t *)cos_cache, (const uint16_t *)sin_cache, (const uint16_t *)trans_mat, (uint16_t *)out, rows, rp, cols,
+                     cs_batch, cs_rows, ttm_round_up32(cs_rows), total);
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
 }

@@ -698,3 +698,17 @@ class ProgramBuilder:
 
     def func_call(self, program_index, ins, out_descs):
         return self._multi("ttrt_pb_func_call", (program_index,), ins, out_descs)
+
+    def rotary_embedding_llama(self, t, cos_cache, sin_cache, trans_mat, decode_mode=False):
+        return self._op("ttrt_pb_rotary_embedding_llama", t, cos_cache, sin_cache, trans_mat, int(decode_mode))
+
+    def chunked_sdpa(self, q, k, v, page_table, chunk_start, scale=None):
+        return self._op("ttrt_pb_chunked_sdpa", q, k, v, page_table, chunk_start, int(scale is not None), ctypes.c_float(scale or 0.0))
+
+    def add_dylib(self, dylib_id, data):
+        """Embed a shared library (bytes) in the open program; cpu_op calls functions of it."""
+        buf = (ctypes.c_uint8 * len(data)).from_buffer_copy(data)
+        _call("ttrt_pb_add_dylib", self.h, dylib_id, buf, len(data))
+
+    def cpu_op(self, dylib_id, func_name, ins, out_descs):
+        return self._multi("ttrt_pb_cpu_op", (dylib_id, func_name.encode()), ins, out_descs)

@@ -541,6 +541,28 @@ TTRT_EXPORT int ttrt_pb_capture_or_execute_trace(ttrt_builder *pb, uint32_t capt
     for (size_t i = 0; i < ids.size(); ++i) outs[i] = ids[i];
   });
 }
+TTRT_EXPORT int ttrt_pb_rotary_embedding_llama(ttrt_builder *pb, uint32_t in, uint32_t cos_cache, uint32_t sin_cache, uint32_t trans_mat,
+                                               int decode_mode, uint32_t *out) {
+  PB_OP(rotaryEmbeddingLlama(in, cos_cache, sin_cache, trans_mat, decode_mode != 0));
+}
+TTRT_EXPORT int ttrt_pb_chunked_sdpa(ttrt_builder *pb, uint32_t q, uint32_t k, uint32_t v, uint32_t page_table, uint32_t chunk_start,
+                                     int has_scale, float scale, uint32_t *out) {
+  PB_OP(chunkedSdpa(q, k, v, page_table, chunk_start, has_scale != 0, scale));
+}
+TTRT_EXPORT int ttrt_pb_add_dylib(ttrt_builder *pb, uint32_t dylib_id, const void *data, size_t size) {
+  return guard([&] {
+    need(pb, "builder"); need(data, "data");
+    pb->pb.addDylib(dylib_id, data, size);
+  });
+}
+TTRT_EXPORT int ttrt_pb_cpu_op(ttrt_builder *pb, uint32_t dylib_id, const char *func_name, const uint32_t *ins, int n_in,
+                               const uint32_t *out_shapes, const int *out_ranks, const ttrt_layout *out_layouts, int n_out, uint32_t *outs) {
+  return guard([&] {
+    need(pb, "builder"); need(func_name, "func_name"); need(outs, "outs");
+    auto ids = pb->pb.cpuOp(dylib_id, func_name, std::vector<ProgramBuilder::Id>(ins, ins + n_in), outDescs(out_shapes, out_ranks, out_layouts, n_out));
+    for (size_t i = 0; i < ids.size(); ++i) outs[i] = ids[i];
+  });
+}
 TTRT_EXPORT int ttrt_pb_func_call(ttrt_builder *pb, uint32_t program_index, const uint32_t *ins, int n_in, const uint32_t *out_shapes,
                                   const int *out_ranks, const ttrt_layout *out_layouts, int n_out, uint32_t *outs) {
   return guard([&] {

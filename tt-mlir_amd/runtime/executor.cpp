@@ -10,6 +10,10 @@
 #include <map>
 #include <sstream>
 
+#include <dlfcn.h>
+#include <sys/syscall.h>
+#include <unistd.h>
+
 #include "runtime_impl.h"
 
 namespace tt::runtime {
@@ -145,6 +149,17 @@ OpRefs opRefs(const fb::Table &operation) {
   case OpType::DeallocateOp: in(schema::DeallocateOp::f_in); break;
   case OpType::LoadCachedOp: inVec(schema::LoadCachedOp::f_inputs); outVec(schema::LoadCachedOp::f_outputs); break;
   case OpType::FuncCallOp: inVec(schema::FuncCallOp::f_inputs); outVec(schema::FuncCallOp::f_outputs); break;
+  case OpType::CpuOp: inVec(schema::CpuOp::f_ins); outVec(schema::CpuOp::f_outs); break;
+  case OpType::RotaryEmbeddingLlamaOp:
+    in(schema::RotaryEmbeddingLlamaOp::f_input); in(schema::RotaryEmbeddingLlamaOp::f_cos_cache);
+    in(schema::RotaryEmbeddingLlamaOp::f_sin_cache); in(schema::RotaryEmbeddingLlamaOp::f_trans_mat);
+    out(schema::RotaryEmbeddingLlamaOp::f_out);
+    break;
+  case OpType::ChunkedScaledDotProductAttentionOp:
+    in(schema::ChunkedScaledDotProductAttentionOp::f_query); in(schema::ChunkedScaledDotProductAttentionOp::f_key);
+    in(schema::ChunkedScaledDotProductAttentionOp::f_value); in(schema::ChunkedScaledDotProductAttentionOp::f_page_table);
+    in(schema::ChunkedScaledDotProductAttentionOp::f_chunk_start_idx); out(schema::ChunkedScaledDotProductAttentionOp::f_out);
+    break;
   case OpType::RotaryEmbeddingOp:
     in(schema::RotaryEmbeddingOp::f_input); in(schema::RotaryEmbeddingOp::f_cos_cache); in(schema::RotaryEmbeddingOp::f_sin_cache);
     out(schema::RotaryEmbeddingOp::f_out);
@@ -844,6 +859,70 @@ void runRotaryEmbedding(const fb::Table &op, ProgramContext &ctx) {
   TTM_CALL(ttm_rotary_embedding(x.handle->data.get(), cosc.handle->data.get(), sinc.handle->data.get(), out.handle->data.get(),
                                 floatCode(dt, "rotary_embedding"), static_cast<std::int64_t>(xs[0]) * xs[1], xs[2], xs[3], cs[2], token,
                                 ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// ::ttnn::experimental::rotary_embedding_llama (runtime/lib/ttnn/operations/transformer/rotary_embedding_llama.cpp:11-34):
+// out = x * cos + (x T) * sin with the 32 x 32 transformation matrix applied per 32-column tile.  Prefill: x
+// [1, heads, seq, head_dim], cos / sin [1, 1, seq, head_dim]; decode: x [1, users, heads, head_dim], cos / sin
+// [1, users, 1 | heads, head_dim] (lib/Dialect/TTNN/IR/TTNNOps.cpp:6293-6380 fixes dtype, layout and the matrix shape).
+void runRotaryEmbeddingLlama(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::RotaryEmbeddingLlamaOp;
+  Tensor x = as(ctx, ctx.get(op.table(S::f_input), "rotary_embedding_llama input"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor cosc = as(ctx, ctx.get(op.table(S::f_cos_cache), "rotary_embedding_llama cos"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor sinc = as(ctx, ctx.get(op.table(S::f_sin_cache), "rotary_embedding_llama sin"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor tm = as(ctx, ctx.get(op.table(S::f_trans_mat), "rotary_embedding_llama trans_mat"), TensorLayout::Tile, DataType::BFloat16);
+  const auto &xs = x.handle->shape, &cs = cosc.handle->shape, &ts = tm.handle->shape;
+  TTRT_ASSERT(xs.size() == 4 && cs.size() == 4, "rotary_embedding_llama: input and caches must be 4D");
+  TTRT_ASSERT(sinc.handle->shape == cs, "rotary_embedding_llama: cos and sin tensors must have the same shape.");
+  TTRT_ASSERT(ts.size() == 4 && ts[0] == 1 && ts[1] == 1 && ts[2] == 32 && ts[3] == 32,
+              "rotary_embedding_llama: transformation matrix must have shape (1,1,32,32)");
+  TTRT_ASSERT(xs[3] <= 256 && cs[3] == xs[3], "rotary_embedding_llama: head dimension must be <= 256 and match the caches'");
+  TTRT_ASSERT(cs[0] == 1 && (cs[1] == 1 || cs[1] == xs[1]) && (cs[2] == xs[2] || cs[2] == 1),
+              "rotary_embedding_llama: cos / sin must be [1, 1 | dim1, dim2 | 1, head_dim]");
+  auto outRef = op.table(S::f_out);
+  Tensor out = makeDeviceTensor(ctx.dev, xs, DataType::BFloat16, TensorLayout::Tile);
+  TTM_CALL(ttm_rotary_embedding_llama(x.handle->data.get(), cosc.handle->data.get(), sinc.handle->data.get(), tm.handle->data.get(),
+                                      out.handle->data.get(), TTM_BF16, static_cast<std::int64_t>(xs[0]) * xs[1], xs[2], xs[3], cs[1], cs[2],
+                                      ctx.stream()));
+  ctx.put(outRef, finish(ctx, out, outRef));
+}
+
+// ::ttnn::transformer::chunked_scaled_dot_product_attention (runtime/lib/ttnn/operations/transformer/
+// chunked_scaled_dot_product_attention.cpp:11-58; golden tools/golden/mapping.py:8847-8913): a prefill chunk
+// [users, heads, chunk_len, head_dim] attends causally over the prefix held in a paged cache; query row j stands at position
+// chunk_start_idx + j.  The pages are gathered, the mask is written and the attention kernel runs, all from device-resident
+// operands: like the reference's "flexible" overload the op keeps no host state and can be recorded into a trace.
+void runChunkedSdpa(const fb::Table &op, ProgramContext &ctx) {
+  using S = schema::ChunkedScaledDotProductAttentionOp;
+  Tensor q = as(ctx, ctx.get(op.table(S::f_query), "chunked sdpa query"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor k = as(ctx, ctx.get(op.table(S::f_key), "chunked sdpa key"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor v = as(ctx, ctx.get(op.table(S::f_value), "chunked sdpa value"), TensorLayout::Tile, DataType::BFloat16);
+  Tensor table = devicePositions(ctx, ctx.get(op.table(S::f_page_table), "chunked sdpa page table"), "chunked sdpa: page_table");
+  Tensor start = devicePositions(ctx, ctx.get(op.table(S::f_chunk_start_idx), "chunked sdpa chunk start"), "chunked sdpa: chunk_start_idx");
+  const auto &qs = q.handle->shape, &ks = k.handle->shape, &ts = table.handle->shape;
+  TTRT_ASSERT(qs.size() == 4, "Query must be a 4D tensor.");
+  TTRT_ASSERT(ks.size() == 4 && v.handle->shape == ks, "Key and value must be 4D tensors of the same shape.");
+  TTRT_ASSERT(ts.size() == 2 && ts[0] == qs[0], "Page table number of users must match query number of users.");
+  TTRT_ASSERT(volume(start.handle->shape) == 1, "Chunk start index must have shape [1]");
+  TTRT_ASSERT(qs[3] == ks[3], "Query head size must match key/value head size.");
+  TTRT_ASSERT(ks[1] != 0 && qs[1] % ks[1] == 0, "Query num heads must be divisible by key/value num heads.");
+  TTRT_ASSERT(ks[2] % 32 == 0, "Key/value block size must be divisible by 32.");
+  const std::int64_t B = qs[0], H = qs[1], Sq = qs[2], D = qs[3], Hkv = ks[1], block = ks[2], pages = ts[1], Sk = pages * block;
+  Tensor kc = makeDeviceTensor(ctx.dev, {static_cast<std::uint32_t>(B), static_cast<std::uint32_t>(Hkv), static_cast<std::uint32_t>(Sk),
+                                         static_cast<std::uint32_t>(D)}, DataType::BFloat16, TensorLayout::Tile);
+  Tensor vc = makeDeviceTensor(ctx.dev, kc.handle->shape, DataType::BFloat16, TensorLayout::Tile);
+  const auto *tp = static_cast<const std::int32_t *>(table.handle->data.get());
+  TTM_CALL(ttm_paged_gather(k.handle->data.get(), tp, kc.handle->data.get(), TTM_BF16, ks[0], Hkv, block, D, B, pages, ctx.stream()));
+  TTM_CALL(ttm_paged_gather(v.handle->data.get(), tp, vc.handle->data.get(), TTM_BF16, ks[0], Hkv, block, D, B, pages, ctx.stream()));
+  Tensor mask = makeDeviceTensor(ctx.dev, {1, 1, static_cast<std::uint32_t>(Sq), static_cast<std::uint32_t>(Sk)}, DataType::BFloat16,
+                                 TensorLayout::Tile);
+  TTM_CALL(ttm_chunk_causal_mask(mask.handle->data.get(), static_cast<const std::int32_t *>(start.handle->data.get()), Sq, Sk, ctx.stream()));
+  auto outRef = op.table(S::f_out);
+  Tensor out = makeDeviceTensor(ctx.dev, qs, DataType::BFloat16, TensorLayout::Tile);
+  TTM_CALL(ttm_sdpa_windowed(q.handle->data.get(), kc.handle->data.get(), vc.handle->data.get(), mask.handle->data.get(), 1, 1,
+                             out.handle->data.get(), TTM_BF16, B, H, Hkv, Sq, Sk, D, 0, op.has(S::f_scale) ? op.scalar<float>(S::f_scale, 0.0f) : 0.0f,
+                             0, -1, nullptr, ctx.stream()));
   ctx.put(outRef, finish(ctx, out, outRef));
 }
 
@@ -1606,6 +1685,110 @@ void runFuncCall(const fb::Table &op, ProgramContext &ctx) {
   for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], results[i]);
 }
 
+// ---- CPU-hoisted ops (runtime/lib/ttnn/operations/cpu/cpu.cpp:215-238, runtime/lib/common/dylib.cpp:13-38,
+// runtime/include/tt/runtime/detail/common/dylib.h:35-175).  A program carries its dynamic libraries as byte vectors
+// (Program.dylibs); each is loaded once per binary from an in-memory file.  The callee takes an array of WrappedTensor
+// (dense row-major host data: start, aligned start, start index, sizes then strides) and returns a malloc'ed array of
+// outputs whose data buffers, shared sizes / strides block and the array itself the runtime frees.
+struct WrappedTensor {
+  void *start;
+  void *alignedStart;
+  std::int64_t startIdx;
+  std::int64_t *sizesAndStrides;
+};
+using WrappedFunc = WrappedTensor *(*)(WrappedTensor *);
+
+void *loadLibraryFromMemory(const std::uint8_t *data, size_t size) {
+  const int fd = static_cast<int>(::syscall(SYS_memfd_create, "dylib", 1u /* MFD_CLOEXEC */));
+  TTRT_ASSERT(fd >= 0, "CpuOp: memfd_create failed");
+  size_t done = 0;
+  while (done < size) {
+    const ssize_t n = ::write(fd, data + done, size - done);
+    if (n <= 0) break;
+    done += static_cast<size_t>(n);
+  }
+  void *handle = done == size ? ::dlopen(("/proc/self/fd/" + std::to_string(fd)).c_str(), RTLD_LAZY | RTLD_LOCAL) : nullptr;
+  const std::string err = handle ? "" : (done == size ? std::string(::dlerror()) : "short write");
+  ::close(fd);   // the mapping stays
+  TTRT_ASSERT(handle != nullptr, "CpuOp: failed to open the program's dynamic library: " + err);
+  return handle;
+}
+
+// handles by (binary id, program index, dylib id); a binary's libraries stay loaded for the life of the process (the
+// reference unloads them with the program executor; code pages of a few KiB are not worth the unload hazards)
+WrappedFunc cpuFunction(ProgramContext &ctx, std::uint32_t dylibId, const std::string &name) {
+  static std::mutex mu;
+  static auto *handles = new std::map<std::tuple<std::uint64_t, std::uint32_t, std::uint32_t>, void *>;
+  std::lock_guard<std::mutex> g(mu);
+  const auto key = std::make_tuple(ctx.binary.id(), ctx.programIndex, dylibId);
+  auto it = handles->find(key);
+  if (it == handles->end()) {
+    fb::Table program = ctx.binary.handle->root.tables(schema::TTNNBinary::f_programs)[ctx.programIndex];
+    auto libs = program.tables(schema::Program::f_dylibs);
+    void *h = nullptr;
+    for (std::uint32_t i = 0; i < libs.size() && !h; ++i) {
+      if (libs[i].scalar<std::uint32_t>(schema::DynamicLib::f_dylib_id, 0) != dylibId) continue;
+      auto raw = libs[i].scalars<std::uint8_t>(schema::DynamicLib::f_raw_file);
+      h = loadLibraryFromMemory(raw.data(), raw.size());
+    }
+    TTRT_ASSERT(h != nullptr, "could not find dylib corresponding to id: " + std::to_string(dylibId));
+    it = handles->emplace(key, h).first;
+  }
+  auto fn = reinterpret_cast<WrappedFunc>(::dlsym(it->second, name.c_str()));
+  TTRT_ASSERT(fn != nullptr, "could not find requested op: \"" + name + "\" in dylib with id: " + std::to_string(dylibId));
+  return fn;
+}
+
+void runCpu(const fb::Table &op, ProgramContext &ctx) {
+  auto ins = op.tables(schema::CpuOp::f_ins), outs = op.tables(schema::CpuOp::f_outs);
+  WrappedFunc fn = cpuFunction(ctx, op.scalar<std::uint32_t>(schema::CpuOp::f_dylib_id, 0), std::string(op.string(schema::CpuOp::f_func_name)));
+  std::vector<Tensor> held;   // inputs stay alive over the call
+  std::vector<std::vector<std::int64_t>> sizesAndStrides;
+  std::vector<WrappedTensor> packed;
+  sizesAndStrides.reserve(ins.size());
+  for (std::uint32_t i = 0; i < ins.size(); ++i) {
+    Tensor t = ctx.get(ins[i], "cpu op input");
+    // the compiler brings operands of a hoisted function to the host as dense row-major f32 / i32 / u32
+    // (lib/Dialect/TTIR/Transforms/HoistCPUOps/HoistCPUOps.cpp:76-108); anything else here is a malformed program
+    TTRT_ASSERT(t.handle->storage == StorageType::Host && t.handle->layout == TensorLayout::RowMajor,
+                "CpuOp: input " + std::to_string(i) + " must be a row-major host tensor");
+    TTRT_ASSERT(utils::dataTypeElementSize(t.handle->dtype) == 4, "CpuOp: input " + std::to_string(i) + " must have 4-byte elements");
+    const std::vector<std::uint32_t> shape = shapeFromTensorRef(ins[i]);
+    TTRT_ASSERT(shape == t.handle->shape, "CpuOp: input " + std::to_string(i) + " has the wrong shape");
+    std::vector<std::int64_t> ss(2 * shape.size());
+    std::int64_t stride = 1;
+    for (size_t d = shape.size(); d-- > 0;) {
+      ss[d] = shape[d];
+      ss[shape.size() + d] = stride;
+      stride *= shape[d];
+    }
+    sizesAndStrides.push_back(std::move(ss));
+    void *data = t.handle->data.get();
+    packed.push_back(WrappedTensor{data, data, 0, sizesAndStrides.back().data()});
+    held.push_back(t);
+  }
+  WrappedTensor *result = fn(packed.data());
+  TTRT_ASSERT(result != nullptr || outs.size() == 0, "CpuOp: the function returned no outputs");
+  std::map<void *, std::shared_ptr<void>> seen;   // outputs that alias one buffer share its owner
+  for (std::uint32_t i = 0; i < outs.size(); ++i) {
+    const WrappedTensor &w = result[i];
+    const Layout lay = layoutFromTensorRef(outs[i]);
+    TTRT_ASSERT(lay.dataType == DataType::Float32 || lay.dataType == DataType::UInt32 || lay.dataType == DataType::Int32,
+                "Unsupported data type for CPU op output");
+    auto t = std::make_shared<TensorImpl>();
+    t->shape = shapeFromTensorRef(outs[i]);
+    t->dtype = lay.dataType; t->layout = TensorLayout::RowMajor; t->storage = StorageType::Host;
+    t->bytes = tensorBytes(t->shape, t->dtype, t->layout);
+    auto it = seen.find(w.start);
+    if (it == seen.end()) it = seen.emplace(w.start, std::shared_ptr<void>(w.alignedStart, [start = w.start](void *) { std::free(start); })).first;
+    t->data = it->second;
+    t->version = nextTensorVersion();
+    ctx.put(outs[i], Tensor{t});
+  }
+  if (outs.size() > 0) std::free(result[0].sizesAndStrides);   // one block for all outputs
+  std::free(result);
+}
+
 // ---- traces (runtime/lib/ttnn/operations/trace/*.cpp): a trace is a HIP graph recorded on the device's stream
 Tensor makeTraceIdTensor(std::uint32_t id) {
   Tensor t = makeHostTensor({}, DataType::UInt32, TensorLayout::RowMajor);
@@ -1772,7 +1955,10 @@ void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   case OpType::DeallocateOp: return runDeallocate(op, ctx);
   case OpType::LoadCachedOp: return runLoadCached(op, ctx);
   case OpType::FuncCallOp: return runFuncCall(op, ctx);
+  case OpType::CpuOp: return runCpu(op, ctx);
   case OpType::RotaryEmbeddingOp: return runRotaryEmbedding(op, ctx);
+  case OpType::RotaryEmbeddingLlamaOp: return runRotaryEmbeddingLlama(op, ctx);
+  case OpType::ChunkedScaledDotProductAttentionOp: return runChunkedSdpa(op, ctx);
   case OpType::UpdateCacheOp: return runUpdateCache(op, ctx);
   case OpType::PagedUpdateCacheOp: return runPagedUpdateCache(op, ctx);
   case OpType::PagedFillCacheOp: return runPagedFillCache(op, ctx);
@@ -1788,6 +1974,58 @@ void runOperation(const fb::Table &operation, ProgramContext &ctx) {
   default: fatal(std::string("Unsupported operation type: ") + schema::opTypeName(type));
   }
 }
+
+// Per-operation profiler ranges: the reference opens a tracy zone per operation and sends its MLIR location as a message
+// (runtime/lib/ttnn/program_executor.cpp:223-237); here each operation is a roctx range named "<OpType> <loc_info>", which
+// rocprofv3 --marker-trace shows around the kernels the operation launched.  TTMLIR_RUNTIME_PROFILE_OPS=1 switches the
+// ranges on (the marker library is loaded on first use); TTMLIR_RUNTIME_SYNC_AFTER_OP=1 also waits for the device at the
+// end of every operation, which makes a range's duration the operation's own (the reference's TT_RUNTIME_SYNC_AFTER_OP).
+struct Roctx {
+  int (*push)(const char *) = nullptr;
+  int (*pop)() = nullptr;
+  bool ranges = false, sync = false;
+  static Roctx &get() {
+    static Roctx r = [] {
+      Roctx x;
+      const char *on = std::getenv("TTMLIR_RUNTIME_PROFILE_OPS"), *sy = std::getenv("TTMLIR_RUNTIME_SYNC_AFTER_OP");
+      x.sync = sy && sy[0] == '1';
+      if (on && on[0] == '1') {
+        for (const char *name : {"libroctx64.so", "libroctx64.so.4", "librocprofiler-sdk-roctx.so"}) {
+          if (void *h = ::dlopen(name, RTLD_LAZY | RTLD_GLOBAL)) {
+            x.push = reinterpret_cast<int (*)(const char *)>(::dlsym(h, "roctxRangePushA"));
+            x.pop = reinterpret_cast<int (*)()>(::dlsym(h, "roctxRangePop"));
+            if (x.push && x.pop) break;
+          }
+        }
+        x.ranges = x.push && x.pop;
+        if (!x.ranges) std::fprintf(stderr, "[tt::runtime] TTMLIR_RUNTIME_PROFILE_OPS: no roctx library found, ranges are off\n");
+      }
+      return x;
+    }();
+    return r;
+  }
+};
+struct OpRange {
+  bool open = false;
+  explicit OpRange(const fb::Table &op) {
+    Roctx &r = Roctx::get();
+    if (!r.ranges) return;
+    const auto type = static_cast<OpType>(op.scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
+    const std::string name = std::string(schema::opTypeName(type)) + " " + std::string(op.string(schema::Operation::f_loc_info));
+    r.push(name.c_str());
+    open = true;
+    debug::Stats::get().incrementStat("ProfiledOpRange");
+  }
+  void close(ProgramContext &ctx) {
+    Roctx &r = Roctx::get();
+    if (r.sync && !ctx.dev->capturing) TTM_CALL(ttm_stream_sync(ctx.stream()));
+    if (open) r.pop();
+    open = false;
+  }
+  ~OpRange() {
+    if (open) Roctx::get().pop();   // an operation that threw
+  }
+};
 
 }  // namespace
 
@@ -1830,7 +2068,9 @@ std::vector<Tensor> executeProgram(const std::shared_ptr<DeviceState> &dev, cons
     ctx.opIndex = i;
     OpContext oc{ops[i], i};
     if (hooks.preOperatorCallback) (*hooks.preOperatorCallback)(binary, cc, oc);
+    OpRange range(ops[i]);
     runOperation(ops[i], ctx);
+    range.close(ctx);
     if (hooks.postOperatorCallback) (*hooks.postOperatorCallback)(binary, cc, oc);
   }
   if (hooks.postProgramCallback) (*hooks.postProgramCallback)(binary, cc);

@@ -157,8 +157,10 @@ std::uint32_t ProgramBuilder::endProgram() {
     b_.addOffset(DebugInfo::f_golden_info, info);
     debugInfo = b_.endTable();
   }
+  Off dylibsV = cur_.dylibs.empty() ? 0 : b_.createOffsetVector(cur_.dylibs);
   b_.startTable(Program::kNumFields);
   if (debugInfo) b_.addOffset(Program::f_debug_info, debugInfo);
+  if (dylibsV) b_.addOffset(Program::f_dylibs, dylibsV);
   b_.addOffset(Program::f_name, name);
   b_.addOffset(Program::f_inputs, insV);
   b_.addOffset(Program::f_outputs, outsV);
@@ -966,6 +968,67 @@ std::vector<ProgramBuilder::Id> ProgramBuilder::funcCall(std::uint32_t programId
   b_.addOffset(FuncCallOp::f_inputs, iv);
   b_.addOffset(FuncCallOp::f_outputs, ov);
   addOp(OpType::FuncCallOp, b_.endTable(), "func.call #" + std::to_string(programIdx));
+  return ids;
+}
+
+ProgramBuilder::Id ProgramBuilder::rotaryEmbeddingLlama(Id in, Id cosCache, Id sinCache, Id transMat, bool decodeMode) {
+  const Desc d = desc(in);
+  Id out = newTensor(Desc{d.shape, d.dtype, TensorLayout::Tile, StorageType::Device});
+  Off i = tensorRef(in), c = tensorRef(cosCache), s = tensorRef(sinCache), t = tensorRef(transMat), o = tensorRef(out);
+  using S = RotaryEmbeddingLlamaOp;
+  b_.startTable(S::kNumFields);
+  b_.addOffset(S::f_input, i);
+  b_.addOffset(S::f_cos_cache, c);
+  b_.addOffset(S::f_sin_cache, s);
+  b_.addOffset(S::f_trans_mat, t);
+  b_.addScalarDefault<std::uint8_t>(S::f_is_decode_mode, decodeMode ? 1 : 0, 0);
+  b_.addOffset(S::f_out, o);
+  addOp(OpType::RotaryEmbeddingLlamaOp, b_.endTable(), "ttnn.rotary_embedding_llama " + shapeStr(d.shape));
+  return out;
+}
+
+ProgramBuilder::Id ProgramBuilder::chunkedSdpa(Id q, Id k, Id v, Id pageTable, Id chunkStart, bool hasScale, float scale) {
+  const Desc d = desc(q);
+  Id out = newTensor(Desc{d.shape, DataType::BFloat16, TensorLayout::Tile, StorageType::Device});
+  Off qr = tensorRef(q), kr = tensorRef(k), vr = tensorRef(v), pr = tensorRef(pageTable), sr = tensorRef(chunkStart), o = tensorRef(out);
+  using S = ChunkedScaledDotProductAttentionOp;
+  b_.startTable(S::kNumFields);
+  b_.addOffset(S::f_query, qr);
+  b_.addOffset(S::f_key, kr);
+  b_.addOffset(S::f_value, vr);
+  b_.addOffset(S::f_page_table, pr);
+  b_.addOffset(S::f_chunk_start_idx, sr);
+  if (hasScale) b_.addScalar<float>(S::f_scale, scale);
+  b_.addOffset(S::f_out, o);
+  addOp(OpType::ChunkedScaledDotProductAttentionOp, b_.endTable(), "ttnn.chunked_scaled_dot_product_attention " + shapeStr(d.shape));
+  return out;
+}
+
+void ProgramBuilder::addDylib(std::uint32_t dylibId, const void *data, size_t bytes) {
+  if (!open_) fatal("ProgramBuilder: no program is open");
+  Off raw = b_.createScalarVector(static_cast<const std::uint8_t *>(data), bytes);
+  b_.startTable(DynamicLib::kNumFields);
+  b_.addScalarDefault<std::uint32_t>(DynamicLib::f_dylib_id, dylibId, 0);
+  b_.addOffset(DynamicLib::f_raw_file, raw);
+  cur_.dylibs.push_back(b_.endTable());
+}
+
+std::vector<ProgramBuilder::Id> ProgramBuilder::cpuOp(std::uint32_t dylibId, const std::string &funcName, const std::vector<Id> &ins,
+                                                      const std::vector<Desc> &outs) {
+  std::vector<Id> ids;
+  std::vector<Off> ir, orf;
+  for (Id t : ins) ir.push_back(tensorRef(t));
+  for (const Desc &d : outs) {
+    ids.push_back(newTensor(d));
+    orf.push_back(tensorRef(ids.back()));
+  }
+  Off iv = b_.createOffsetVector(ir), ov = b_.createOffsetVector(orf), name = b_.createString(funcName);
+  b_.startTable(CpuOp::kNumFields);
+  b_.addOffset(CpuOp::f_ins, iv);
+  b_.addOffset(CpuOp::f_outs, ov);
+  b_.addOffset(CpuOp::f_func_name, name);
+  b_.addScalarDefault<std::uint32_t>(CpuOp::f_dylib_id, dylibId, 0);
+  addOp(OpType::CpuOp, b_.endTable(), "ttnn.cpu " + funcName);
   return ids;
 }
 

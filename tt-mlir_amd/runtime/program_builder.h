@@ -66,6 +66,8 @@ public:
               TensorLayout layout, StorageType storage);
   Id full(const std::vector<std::uint32_t> &shape, float value, DataType dtype, TensorLayout layout);
   Id rotaryEmbedding(Id in, Id cosCache, Id sinCache, bool hasTokenIndex, std::uint32_t tokenIndex);
+  Id rotaryEmbeddingLlama(Id in, Id cosCache, Id sinCache, Id transMat, bool decodeMode);
+  Id chunkedSdpa(Id q, Id k, Id v, Id pageTable, Id chunkStart, bool hasScale, float scale);
   void updateCache(Id cache, Id in, Id updateIndex, std::uint32_t batchOffset);
   void fillCache(Id cache, Id in, std::uint32_t batchOffset);
   void pagedUpdateCache(Id cache, Id in, Id updateIndex, Id pageTable, bool shareCache);   // pageTable 0: static cache
@@ -84,6 +86,10 @@ public:
   void deallocate(Id in, bool force);
   std::vector<Id> loadCached(std::uint32_t programIdx, const std::string &callee, const std::vector<Id> &ins, const std::vector<Desc> &outs);
   std::vector<Id> funcCall(std::uint32_t programIdx, const std::vector<Id> &ins, const std::vector<Desc> &outs);
+  // CPU-hoisted function (include/ttmlir/Target/TTNN/operations/cpu.fbs): `funcName` of the dynamic library that
+  // addDylib put into the open program under `dylibId`
+  std::vector<Id> cpuOp(std::uint32_t dylibId, const std::string &funcName, const std::vector<Id> &ins, const std::vector<Desc> &outs);
+  void addDylib(std::uint32_t dylibId, const void *data, size_t bytes);
 
   // Location string of the operation added last ("loc(\"<program>\"(\"op<k>\"))"); goldens are keyed by it.
   std::string lastOpLoc() const;
@@ -107,6 +113,7 @@ private:
     std::vector<Id> inputs, outputs;
     std::vector<OpRec> ops;
     std::vector<std::pair<std::string, fb::Builder::Off>> goldens;   // loc -> GoldenDeviceTensor table
+    std::vector<fb::Builder::Off> dylibs;                            // DynamicLib tables
   };
   Id newTensor(const Desc &d);
   fb::Builder::Off tensorRef(Id t);
