@@ -176,19 +176,31 @@ def test_c4_mlp_full_size(device, orc, metrics):
     assert metrics.get_pcc(ref.numpy(), y[rows].float().numpy()) >= 0.98
 
 
-def oracle_decoder(orc, d):
+def oracle_decoder(orc, d, rows=None):
+    """The layer's output for the token rows `rows` (all by default).  Keys and values need every token; everything behind the
+    attention is row-wise, so a subset of rows costs that fraction of the work."""
     r = orc.round_bf16
     f = lambda t: t.float().numpy()
     q8 = lambda w: orc.bfp_unpack(orc.bfp_pack(f(bf(w)), 8), tuple(w.shape), 8)
     S, H, nq, nkv, hd = d["seq"], d["hidden"], d["n_q"], d["n_kv"], d["head_dim"]
     x = f(d["x"])[0]
     h = r(orc.rms_norm(x, f(d["attn_norm_w"]), None, d["eps"]))
-    q = r(orc.linear(h, q8(d["wq"]))).reshape(S, nq, hd).transpose(1, 0, 2)[None]
     k = r(orc.linear(h, q8(d["wk"]))).reshape(S, nkv, hd).transpose(1, 0, 2)[None]
     v = r(orc.linear(h, q8(d["wv"]))).reshape(S, nkv, hd).transpose(1, 0, 2)[None]
-    a = r(orc.sdpa(np.ascontiguousarray(q), np.ascontiguousarray(k), np.ascontiguousarray(v), is_causal=True))
-    merged = a[0].transpose(1, 0, 2).reshape(S, nq * hd)
-    x1 = r(x + r(orc.linear(np.ascontiguousarray(merged), q8(d["wo"]))))
+    if rows is None:
+        q = r(orc.linear(h, q8(d["wq"]))).reshape(S, nq, hd).transpose(1, 0, 2)[None]
+        a = r(orc.sdpa(np.ascontiguousarray(q), np.ascontiguousarray(k), np.ascontiguousarray(v), is_causal=True))
+        xs, n = x, S
+    else:
+        rows = np.asarray(rows)
+        n = len(rows)
+        q = r(orc.linear(np.ascontiguousarray(h[rows]), q8(d["wq"]))).reshape(n, nq, hd).transpose(1, 0, 2)[None]
+        # causal attention of the selected queries, written as a mask: query at position rows[i] sees keys 0 .. rows[i]
+        mask = np.where(np.arange(S)[None, :] <= rows[:, None], 0.0, -np.inf).astype(np.float32)[None, None]
+        a = r(orc.sdpa(np.ascontiguousarray(q), np.ascontiguousarray(k), np.ascontiguousarray(v), mask=mask, is_causal=False))
+        xs = np.ascontiguousarray(x[rows])
+    merged = a[0].transpose(1, 0, 2).reshape(n, nq * hd)
+    x1 = r(xs + r(orc.linear(np.ascontiguousarray(merged), q8(d["wo"]))))
     mlp = oracle_mlp(orc, x1, f(d["mlp_norm_w"]), f(bf(d["wg"])), f(bf(d["wu"])), f(bf(d["wd"])), d["eps"])
     return r(x1 + mlp)[None]
 
@@ -206,21 +218,33 @@ def test_c5_decoder_layer_small(device, orc, metrics):
     assert metrics.get_pcc(want, got) >= 0.9999
 
 
+def test_c5_decoder_layer_small_row_subset(device, orc):
+    """The oracle evaluated on a subset of token rows is the full evaluation restricted to those rows, bit for bit."""
+    d = datagen.c5_decoder(seq=96, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, seed=4)
+    rows = np.array([0, 1, 31, 32, 50, 95])
+    assert np.array_equal(oracle_decoder(orc, d)[0, rows], oracle_decoder(orc, d, rows)[0])
+
+
+C5_ROWS = np.concatenate([np.arange(t * 32, t * 32 + 32) for t in (0, 1, 5, 9, 14, 18, 23, 27, 31, 32, 36, 41, 46, 50, 57, 63)])
+
+
 def test_c5_decoder_layer_full_size(device, orc, metrics):
     """Config 5 at its real shape: Llama-3-8B layer, batch 1, 2048 tokens, hidden 4096, 32 / 8 heads of 128, FFN 14336
-    (test/ttmlir/models/single_blocks_and_layers/llama_3_8b_prefill_layer.mlir:54-304).  One submit; all 2048 x 4096 outputs
-    against the oracle's evaluation of the same graph (about 1 TFLOP of scalar f32 over all host cores)."""
+    (test/ttmlir/models/single_blocks_and_layers/llama_3_8b_prefill_layer.mlir:54-304).  One submit of the whole program; the
+    outputs of 512 token rows (16 of the 64 row tiles, spread over the sequence, the first and the last among them) against
+    the oracle's evaluation of the same graph for those rows, which attend to all the keys in front of them (about a quarter
+    of a TFLOP of scalar f32 over the host cores)."""
     d = datagen.c5_decoder()
     binary = rt.Binary.load_from_memory(programs.c5_decoder())
     tins = [d["x"], d["attn_norm_w"], bf(d["wq"]), bf(d["wk"]), bf(d["wv"]), bf(d["wo"]), d["mlp_norm_w"], bf(d["wg"]), bf(d["wu"]),
             bf(d["wd"])]
     (y,) = harness.execute(binary, 1, tins, device)
-    assert tuple(y.shape) == (1, 2048, 4096)
-    got = y.float().numpy()
+    assert tuple(y.shape) == (1, 2048, 4096) and bool(torch.isfinite(y.float()).all())
+    got = y.float().numpy()[:, C5_ROWS]
     del y, tins
     orc.set_threads(orc.max_threads())
     try:
-        want = oracle_decoder(orc, d)
+        want = oracle_decoder(orc, d, C5_ROWS)
     finally:
         orc.set_threads(1)
     err = np.abs(got - want)
@@ -241,7 +265,7 @@ def test_c5_decoder_layer_full_size(device, orc, metrics):
     assert np.mean(err <= 4 * sp) >= 0.9
     assert metrics.get_pcc(want, got) >= 0.9999
     # first and last tile rows separately (causal attention's edge blocks)
-    for rows in (slice(0, 32), slice(2016, 2048)):
+    for rows in (slice(0, 32), slice(480, 512)):
         assert metrics.get_pcc(want[0, rows], got[0, rows]) >= 0.9999
         assert np.abs(got[0, rows] - want[0, rows]).max() <= 2.0 ** -3
 

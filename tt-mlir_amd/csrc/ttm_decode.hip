@@ -265,6 +265,14 @@ struct DecodeArgs {
 };
 
 constexpr int kMaxG = 8;
+// K and V are read once per launch: streaming (nontemporal) loads keep them from displacing each other in the caches on
+// the way (measured at 32 users x 8 kv heads x 2048 positions: 59 -> 54 us).  STREAM = false when several launches share
+// one cache (more than kMaxG query heads per kv head), where the later launches profit from what the first one left.
+template <bool STREAM, typename T>
+__device__ __forceinline__ T kv_load(const T *p) {
+  if constexpr (STREAM) return __builtin_nontemporal_load(p);
+  else return *p;
+}
 #ifndef SPLIT_TARGET
 #define SPLIT_TARGET 512
 #endif
@@ -284,6 +292,7 @@ __device__ __forceinline__ const uint16_t *kv_tile_row(const uint16_t *base, con
   return base + (((int64_t)b * p.Hkv + hk) * (p.S >> 5) + key_tile) * row_elems;
 }
 
+template <bool STREAM>
 __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
   extern __shared__ float lds[];
   const int split = blockIdx.x, bh = blockIdx.y, b = bh / p.Hkv, hk = bh % p.Hkv;
@@ -346,7 +355,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
         const int in_tile = (((key >> 4) & 1) * 2 + (dq >> 4)) * 256 + (key & 15) * 16 + (dq & 15);
 #pragma unroll
         for (int c = 0; c < 8; ++c)
-          if (c < DT) kf[u][c] = *(const u32x4 *)(kt + (int64_t)c * 1024 + in_tile);
+          if (c < DT) kf[u][c] = kv_load<STREAM>((const u32x4 *)(kt + (int64_t)c * 1024 + in_tile));
       }
 #pragma unroll
       for (int u = 0; u < 2; ++u) {
@@ -424,8 +433,8 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
         for (int u = 0; u < UT; ++u) {
           const int t = t0 + u * share < ntiles ? t0 + u * share : t0;
           const uint16_t *vt = kv_tile_row(p.v, p, b, hk, (k0 >> 5) + t, vok[u]) + (int64_t)dt * 1024;
-          ra[u] = *(const u32x4 *)(vt + lane * 8);
-          rb[u] = *(const u32x4 *)(vt + 512 + lane * 8);
+          ra[u] = kv_load<STREAM>((const u32x4 *)(vt + lane * 8));
+          rb[u] = kv_load<STREAM>((const u32x4 *)(vt + 512 + lane * 8));
         }
 #pragma unroll
         for (int u = 0; u < UT; ++u) {
@@ -742,7 +751,8 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
     p.g0 = (int)g0;
     p.G = (int)(Gt - g0 < kMaxG ? Gt - g0 : kMaxG);
     const size_t lds = (size_t)(p.G * keys + p.G * head_dim + 2 * p.G + p.G * keys / 2) * sizeof(float);
-    hipLaunchKernelGGL(ttm_sdpa_decode_k, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
+    if (Gt <= kMaxG) hipLaunchKernelGGL(ttm_sdpa_decode_k<true>, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
+    else hipLaunchKernelGGL(ttm_sdpa_decode_k<false>, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
     TTM_LAUNCH_CHECK();
     hipLaunchKernelGGL(ttm_sdpa_decode_combine_k, dim3((unsigned)(batch * kv_heads)), dim3(256), 0, s, p);
     TTM_LAUNCH_CHECK();
