@@ -136,6 +136,21 @@ int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, vo
                      const int *act, int64_t M, int64_t K, void *stream);
 int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M, int64_t N,
                     int64_t K, void *stream);
+/* The front of a decode step's attention block in two launches: the Q, K and V projections of `users` <= 32 tokens (one
+ * per user, activations a [users, K] bf16 tiles, block-float weights [K, heads * head_dim] and twice
+ * [K, kv_heads * head_dim]), then in one kernel the head split, the rotary embedding of q and k with row `token_index` of
+ * the cos / sin caches ([1, 1, cache_rows, head_dim] bf16 tiles), q written as [1, users, heads, head_dim] bf16 tiles and k
+ * and v written into their caches [cache_users, kv_heads, max_seq, head_dim] at row *update_index (device memory; out of
+ * range writes nothing) of users batch_offset .. batch_offset + users - 1.  It replaces, with bit-identical results, the
+ * op sequence matmul x 3 -> reshape -> RotaryEmbeddingOp x 2 -> permute -> UpdateCacheOp x 2 of a decode layer
+ * (test/ttmlir/models/single_blocks_and_layers/llama_3_8b_decode_layer.mlir:51-82; runtime/lib/ttnn/operations/matmul/
+ * matmul.cpp:47-83, transformer/rotary_embedding.cpp:14-31, kv_cache/update_cache.cpp:14-55).
+ * ttm_linear_qkv_decode_supported returns 1 when the shapes and the selected kernel variant allow it, else 0. */
+int ttm_linear_qkv_decode_supported(int w_dtype, int64_t users, int64_t K, int64_t heads, int64_t kv_heads, int64_t head_dim);
+int ttm_linear_qkv_decode(const void *a, const void *wq, const void *wk, const void *wv, int w_dtype, int64_t users, int64_t K,
+                          int64_t heads, int64_t kv_heads, int64_t head_dim, const void *cos_cache, const void *sin_cache,
+                          int64_t cache_rows, int64_t token_index, void *q_out, void *k_cache, void *v_cache, int64_t cache_users,
+                          int64_t max_seq, const int32_t *update_index, int64_t batch_offset, void *stream);
 
 /* ---- elementwise: ::ttnn::<unary>, ::ttnn::<binary>
  * (runtime/lib/ttnn/operations/eltwise/unary/unary.cpp:159-205, eltwise/binary/binary.cpp:38-126;

@@ -408,3 +408,82 @@ def test_sdpa_decode_mask_shared_by_the_users(hip, dev, orc, mask_batch, mask_he
     got = f32(untilize_dev(hip, out, q.shape, dev))
     want = orc.sdpa_decode(f32(q), f32(k), f32(v), mask=f32(m), is_causal=False, sliding_window=100, attention_sink=f32(sk))
     assert np.all(np.isfinite(got)) and np.max(np.abs(got - want)) <= 2.0 ** -6
+
+
+@pytest.mark.parametrize("users,K,H,Hkv,D,S,pos,off,cache_users,token,rows", [
+    (32, 4096, 32, 8, 128, 2048, 2047, 0, 32, 0, 1),      # the Llama-3-8B decode step
+    (5, 256, 4, 2, 64, 96, 33, 1, 8, 2, 4),               # ragged users, padded heads, batch offset, a row of a longer cos cache
+    (1, 512, 8, 8, 32, 32, 0, 0, 1, 0, 1),
+    (32, 1024, 8, 1, 128, 64, 70, 0, 32, 0, 1),           # position outside the cache: q comes out, the caches stay
+])
+@pytest.mark.parametrize("fmt", ["bfp8", "bfp4"])
+def test_linear_qkv_decode_equals_the_op_sequence(hip, dev, orc, users, K, H, Hkv, D, S, pos, off, cache_users, token, rows, fmt):
+    """ttm_linear_qkv_decode against the ops it stands for, run one by one through the C ABI (ttm_linear_group, two
+    ttm_rotary_embedding_split_heads, the cache rows written by hand): bit-identical q and caches; and q against the oracle."""
+    from test_gpu_linear import pack_weight
+    wf = hip.BFP8B if fmt == "bfp8" else hip.BFP4B
+    a = datagen.randn((users, K), seed=90, dtype=torch.bfloat16)
+    ws = [datagen.randn((K, n * D), seed=91 + i, dtype=torch.float32) * 0.05 for i, n in enumerate((H, Hkv, Hkv))]
+    ang = datagen.randn((1, 1, rows, D // 2), seed=95, dtype=torch.float32) * 2.0
+    cos = torch.cat([ang.cos(), ang.cos()], -1).to(torch.bfloat16)
+    sin = torch.cat([ang.sin(), ang.sin()], -1).to(torch.bfloat16)
+    caches = [datagen.randn((cache_users, Hkv, S, D), seed=96 + i, dtype=torch.bfloat16) for i in range(2)]
+    at, ct, st = tilize_dev(hip, a, dev), tilize_dev(hip, cos, dev), tilize_dev(hip, sin, dev)
+    wt = [pack_weight(hip, w, wf, dev) for w in ws]
+    index = torch.tensor([pos], dtype=torch.int32, device=dev)
+    s = hip.current_stream()
+    # the op sequence; the three projections share a launch as they do in a program (a projection launched alone may split
+    # K another way and round a few sums to the neighbouring bf16 value)
+    import ctypes
+    lin = [torch.full((32 * n * D,), float("nan"), dtype=torch.bfloat16, device=dev) for n in (H, Hkv, Hkv)]
+    wp = (ctypes.c_void_p * 3)(*[t.data_ptr() for t in wt])
+    op = (ctypes.c_void_p * 3)(*[t.data_ptr() for t in lin])
+    nn = (ctypes.c_int64 * 3)(H * D, Hkv * D, Hkv * D)
+    hip.call("ttm_linear_group", hip.ptr(at), 3, wp, wf, op, nn, None, users, K, s)
+    rot = []
+    for o, n in zip(lin[:2], (H, Hkv)):
+        r = torch.full((users * ((n + 31) // 32 * 32) * D,), float("nan"), dtype=torch.bfloat16, device=dev)
+        hip.call("ttm_rotary_embedding_split_heads", hip.ptr(o), hip.ptr(ct), hip.ptr(st), hip.ptr(r), hip.BF16, users, n, D, rows, token, s)
+        rot.append(r)
+    k_rot = untilize_dev(hip, rot[1], (1, users, Hkv, D), dev)
+    v_lin = untilize_dev(hip, lin[2], (users, Hkv * D), dev).reshape(1, users, Hkv, D)
+    want_caches = [c.clone().to(dev) for c in caches]
+    if 0 <= pos < S:
+        want_caches[0][off:off + users, :, pos, :] = k_rot[0]
+        want_caches[1][off:off + users, :, pos, :] = v_lin[0]
+    # the fused entry point
+    assert hip.lib().ttm_linear_qkv_decode_supported(wf, users, K, H, Hkv, D) == 1
+    q = torch.full_like(rot[0], float("nan"))
+    ck, cv = (tilize_dev(hip, c, dev) for c in caches)
+    hip.call("ttm_linear_qkv_decode", hip.ptr(at), hip.ptr(wt[0]), hip.ptr(wt[1]), hip.ptr(wt[2]), wf, users, K, H, Hkv, D, hip.ptr(ct),
+             hip.ptr(st), rows, token, hip.ptr(q), hip.ptr(ck), hip.ptr(cv), cache_users, S, hip.ptr(index), off, s)
+    torch.cuda.synchronize()
+    assert torch.equal(q, rot[0])                                       # padding rows of q included (zeros)
+    assert torch.equal(untilize_dev(hip, ck, caches[0].shape, dev), want_caches[0])
+    assert torch.equal(untilize_dev(hip, cv, caches[1].shape, dev), want_caches[1])
+    # q against the oracle: projection on the dequantised weights, bf16, rotary embedding, bf16
+    back = torch.empty(ws[0].shape, dtype=torch.float32, device=dev)
+    hip.call("ttm_bfp_unpack", hip.ptr(wt[0]), wf, hip.ptr(back), hip.F32, hip.ROW_MAJOR, 1, K, H * D, s)
+    proj = orc.round_bf16(orc.linear(f32(a), f32(back)))
+    want_q = orc.round_bf16(orc.rotary_embedding(proj.reshape(1, users, H, D), f32(cos), f32(sin), token_index=token))
+    got_q = f32(untilize_dev(hip, q, (1, users, H, D), dev))
+    # the projection differs from the oracle's at bf16 ties of its fp32 sums (another summation order); where it agrees the
+    # rotary embedding is the oracle's arithmetic exactly
+    assert np.mean(got_q == want_q) > 0.98
+    assert np.max(np.abs(got_q - want_q)) <= 2.0 ** -7 * max(1.0, float(np.max(np.abs(want_q))))
+
+
+def test_linear_qkv_decode_rejects_what_it_cannot_fuse(hip, dev):
+    z = torch.zeros(32 * 64, dtype=torch.bfloat16, device=dev)
+    args = lambda users=4, D=64, token=0, rows=1, off=0, cu=4: (hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.ptr(z), hip.BFP8B, users, 64, 1, 1, D,
+                                                                 hip.ptr(z), hip.ptr(z), rows, token, hip.ptr(z), hip.ptr(z), hip.ptr(z), cu, 32,
+                                                                 hip.ptr(z), off, hip.current_stream())
+    assert hip.lib().ttm_linear_qkv_decode_supported(hip.BFP8B, 33, 64, 1, 1, 64) == 0
+    assert hip.lib().ttm_linear_qkv_decode_supported(hip.BF16, 4, 64, 1, 1, 64) == 0
+    assert hip.lib().ttm_linear_qkv_decode_supported(hip.BFP8B, 4, 64, 1, 1, 48) == 0
+    with pytest.raises(hip.TTMError, match="1..32 users"):
+        hip.call("ttm_linear_qkv_decode", *args(users=33))
+    with pytest.raises(hip.TTMError, match="token_index"):
+        hip.call("ttm_linear_qkv_decode", *args(token=1))
+    with pytest.raises(hip.TTMError, match="exceeds the cache"):
+        hip.call("ttm_linear_qkv_decode", *args(off=1))

@@ -819,16 +819,14 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
         rt.clear_callbacks()
         if mode == "traced":
             assert rt.get_stat("CapturedTrace") >= 1
-        # both cache writes read their permuted operand as a view (K after the rotary embedding, V straight from the
-        # reshaped projection), the Q, K and V projections share a launch; nothing of this with a callback registered
-        # (a traced program runs its body op by op only until the graph is recorded)
-        fused, paired = rt.get_stat("FusedCacheUpdate"), rt.get_stat("GroupedMatmul")
-        assert rt.get_stat("GroupedMatmulMembers") == 3 * paired          # Q, K and V projections in one launch
-        assert (fused, paired) == {"eager": (6, 3), "callbacks": (0, 0)}.get(mode, (fused, paired))
-        assert mode != "traced" or (fused in (2, 4) and paired * 2 == fused)
-        # the head splits in front of both rotary embeddings and the head merge behind the attention are folded into
-        # those kernels
-        assert rt.get_stat("FusedHeadSplit") == fused and rt.get_stat("FusedHeadConcat") == paired
+        # the Q, K and V projections, both rotary embeddings, the head splits and both cache writes are one fused step (two
+        # launches); nothing of this with a callback registered (a traced program runs its body op by op only until the graph
+        # is recorded); the head merge behind the attention is folded into the attention kernel
+        qkv = rt.get_stat("FusedQkvDecode")
+        assert qkv == {"eager": 3, "callbacks": 0}.get(mode, qkv)
+        assert mode != "traced" or qkv in (1, 2)
+        assert rt.get_stat("FusedCacheUpdate") == 0 and rt.get_stat("FusedHeadSplit") == 0 and rt.get_stat("GroupedMatmul") == 0
+        assert rt.get_stat("FusedHeadConcat") == qkv
     # the replayed graph runs the same kernels on the same data: identical to the op-by-op run, caches included; so is
     # the unfused run
     for other in ("traced", "callbacks"):

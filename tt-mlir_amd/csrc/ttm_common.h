@@ -50,6 +50,14 @@ static inline int ttm_dtype_bytes(int dtype) {
   }
 }
 
+// One element of a rotary embedding, x cos + rot(x) sin with rot(x) = sign * partner: two products and a sum, each rounded
+// to fp32 (the arithmetic of the CPU path's separate multiply and add ops; no fused multiply-add)
+__device__ __forceinline__ float ttm_rotary_value(float x, float partner, float c, float s, float sign) {
+#pragma clang fp contract(off)
+  const float a = x * c, b = (sign * partner) * s;
+  return a + b;
+}
+
 // Element offset of (r, c) inside a tiled [Rt*32, Ct*32] matrix: tiles row-major, faces
 // (0,0) (0,1) (1,0) (1,1), 16 contiguous elements per face row.
 __host__ __device__ static inline int64_t ttm_tiled_offset(int64_t r, int64_t c, int64_t ct) {

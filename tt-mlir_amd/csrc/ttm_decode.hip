@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void ttm_rotary_k(const T *__restrict__ x, con
   load8(cosc + co, cv);
   load8(sinc + co, sv);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) ov[j] = xv[j] * cv[j] + sign * pv[j] * sv[j];
+  for (int j = 0; j < 8; ++j) ov[j] = ttm_rotary_value(xv[j], pv[j], cv[j], sv[j], sign);
   store8(out + b * per_batch + o, ov);
 }
 

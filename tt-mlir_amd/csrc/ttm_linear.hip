@@ -56,6 +56,22 @@ struct LinearArgs {
   int gAct[4];                        // per-member activation
   int tail;                           // 0 none, 1 add, 2 multiply: element-wise tail with a tensor laid out like the output
   int64_t tail_delta;                 // byte distance from an output element to its tail operand
+  const struct QkvFinishArgs *qkv;    // host side only: the decode launch leaves partial sums and ttm_qkv_finish_k ends it
+};
+
+// What follows the Q, K and V projections of a decode step (one token per user): head split, rotary embedding of q and k
+// at the cos / sin row `cos_row`, q to its own tensor, k and v into the cache row of position *index.
+struct QkvFinishArgs {
+  const float *partial;               // [slices][per] fp32 in tile order over the concatenation q | k | v (one row tile)
+  int slices;
+  int64_t per;
+  int users, heads, heads_pad, kv_heads, dim;
+  const uint16_t *cosc, *sinc;        // [.., dim] bf16 tiles
+  int64_t cos_row;
+  uint16_t *q_out;                    // [1, users, heads, dim] bf16 tiles
+  uint16_t *k_cache, *v_cache;        // [cache users, kv_heads, max_seq, dim] bf16 tiles
+  int64_t max_seq, seq_pad, batch_offset;
+  const int32_t *index;               // device memory: the position all users write
 };
 
 // The member of a group launch that owns column unit `u`, where a unit is `unit_tiles` column tiles and every member's
@@ -1513,6 +1529,62 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   *(u32x2 *)(C + off * 2) = finish_quad(p, C + off * 2, v);
 }
 
+// Ends the decode step's Q / K / V launch.  One lane per four consecutive columns of one user: sums the k-slices, rounds to
+// bf16 (the projection's own output rounding), applies the rotary embedding to q and k (the partner columns d +- dim / 2 are
+// another four consecutive partial sums), and writes q in [1, users, heads, dim] order and k / v into the caches at the
+// position read from device memory (out of range: nothing is written).  Lanes past the partial sums zero the padding rows
+// of q.  The result equals ttm_linear_group + ttm_rotary_embedding_split_heads + the cache updates bit for bit.
+__global__ __launch_bounds__(256) void ttm_qkv_finish_k(QkvFinishArgs p) {
+  const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x, nq = p.per / 4;
+  const int D = p.dim, ct = D >> 5, d4 = D >> 2;
+  if (q >= nq) {
+    const int padh = p.heads_pad - p.heads;
+    const int64_t z = q - nq;
+    if (z >= (int64_t)p.users * padh * d4) return;
+    const int d = (int)(z % d4) * 4, h = p.heads + (int)((z / d4) % padh), b = (int)(z / ((int64_t)d4 * padh));
+    *(u32x2 *)(p.q_out + (int64_t)b * p.heads_pad * D + ttm_tiled_offset(h, d, ct)) = u32x2{0u, 0u};
+    return;
+  }
+  const int64_t off = q * 4;
+  const int nt = (int)(off >> 10), in = (int)(off & 1023);
+  const int m = ((in >> 9) & 1) * 16 + ((in >> 4) & 15);
+  if (m >= p.users) return;
+  const int n = nt * 32 + ((in >> 8) & 1) * 16 + (in & 15);
+  const int nQ = p.heads * D, nK = p.kv_heads * D;
+  auto sum4 = [&](int64_t o) {
+    f32x4 s = *(const f32x4 *)(p.partial + o);
+    for (int sl = 1; sl < p.slices; ++sl) s += *(const f32x4 *)(p.partial + sl * p.per + o);
+    return s;
+  };
+  auto r16 = [](float x) { return ttm_bf16_to_f32(ttm_f32_to_bf16(x)); };
+  const int64_t pos = p.index[0];
+  if (n >= nQ + nK) {   // v
+    if (pos < 0 || pos >= p.max_seq) return;
+    const int c = n - nQ - nK, hk = c / D, d = c % D;
+    const f32x4 s = sum4(off);
+    *(u32x2 *)(p.v_cache + ((p.batch_offset + m) * p.kv_heads + hk) * p.seq_pad * D + ttm_tiled_offset(pos, d, ct)) =
+        u32x2{ttm_pack_bf16x2(s.x, s.y), ttm_pack_bf16x2(s.z, s.w)};
+    return;
+  }
+  const bool isq = n < nQ;
+  if (!isq && (pos < 0 || pos >= p.max_seq)) return;
+  const int c = isq ? n : n - nQ, h = c / D, d = c % D, half = D >> 1;
+  const int pn = n - d + (d < half ? d + half : d - half);   // partner column in the concatenation
+  const float sign = d < half ? -1.0f : 1.0f;
+  const int64_t poff = (int64_t)(pn >> 5) * 1024 + ((m >> 4) * 2 + ((pn >> 4) & 1)) * 256 + (m & 15) * 16 + (pn & 15);
+  const f32x4 x = sum4(off), xp = sum4(poff);
+  const int64_t co = ttm_tiled_offset(p.cos_row, d, ct);
+  const u32x2 cr = *(const u32x2 *)(p.cosc + co), sr = *(const u32x2 *)(p.sinc + co);
+  const float cv[4] = {__uint_as_float(cr.x << 16), __uint_as_float(cr.x & 0xFFFF0000u), __uint_as_float(cr.y << 16), __uint_as_float(cr.y & 0xFFFF0000u)};
+  const float sv[4] = {__uint_as_float(sr.x << 16), __uint_as_float(sr.x & 0xFFFF0000u), __uint_as_float(sr.y << 16), __uint_as_float(sr.y & 0xFFFF0000u)};
+  float o[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) o[j] = ttm_rotary_value(r16(x[j]), r16(xp[j]), cv[j], sv[j], sign);
+  const u32x2 packed = {ttm_pack_bf16x2(o[0], o[1]), ttm_pack_bf16x2(o[2], o[3])};
+  if (isq) *(u32x2 *)(p.q_out + (int64_t)m * p.heads_pad * D + ttm_tiled_offset(h, d, ct)) = packed;
+  else *(u32x2 *)(p.k_cache + ((p.batch_offset + m) * p.kv_heads + h) * p.seq_pad * D + ttm_tiled_offset(pos, d, ct)) = packed;
+}
+
 static int device_cu_count() {
   static int cus = 0;
   if (cus == 0) {
@@ -1619,7 +1691,8 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       }
     }
     const int64_t per = (int64_t)a.Nt * 1024;
-    if (slices > 1) {
+    if (a.qkv && (!decode || a.Mt != 1 || batch != 1)) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear_qkv_decode: the selected kernel variant cannot end in the fused step");
+    if (slices > 1 || a.qkv) {
       void *ws = nullptr;
       if (int rc = ttm_stream_workspace(s, (size_t)(per * slices * batch) * sizeof(float), &ws)) return rc;
       p.partial = (float *)ws;
@@ -1639,7 +1712,12 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         else hipLaunchKernelGGL((ttm_linear_decode_k<false, false>), grid, dim3(512), 65536, s, p);
       }
       else hipLaunchKernelGGL((ttm_linear_small_k<WF>), dim3(a.Nt, 1, (unsigned)batch), dim3(256), 0, s, p);
-      if (slices > 1)
+      if (a.qkv) {
+        QkvFinishArgs f = *a.qkv;
+        f.partial = p.partial; f.slices = slices; f.per = per;
+        const int64_t lanes = per / 4 + (int64_t)f.users * (f.heads_pad - f.heads) * (f.dim / 4);
+        hipLaunchKernelGGL(ttm_qkv_finish_k, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, s, f);
+      } else if (slices > 1)
         hipLaunchKernelGGL(ttm_linear_reduce_k, dim3((unsigned)((per / 4 + 255) / 256), 1, (unsigned)batch), dim3(256), 0, s, p, slices);
     }
     return 0;
@@ -1806,6 +1884,7 @@ static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, 
   for (int j = 0; j < 4; ++j) { p.gW[j] = nullptr; p.gC[j] = nullptr; p.gNt[j] = 0; p.gAct[j] = TTM_ACT_NONE; }
   p.tail = tail_op;
   p.tail_delta = tail ? (const uint8_t *)tail - (const uint8_t *)out : 0;
+  p.qkv = nullptr;
   if (strides) { p.a_batch = strides[0]; p.w_batch = strides[1]; p.c_batch = strides[2]; }
   TTM_REQUIRE(batch <= 65535, "ttm_linear: batch too large");
   hipStream_t s = (hipStream_t)stream;
@@ -1835,8 +1914,8 @@ TTM_EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, in
                       TTM_TAIL_NONE, nullptr, strides, stream);
 }
 
-TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N,
-                                const int *act, int64_t M, int64_t K, void *stream) {
+static int linear_group_entry(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N,
+                              const int *act, int64_t M, int64_t K, const QkvFinishArgs *qkv, void *stream) {
   TTM_REQUIRE(n >= 1 && n <= 4, "ttm_linear_group: 1 to 4 members (got %d)", n);
   TTM_REQUIRE(a && w && out && N, "ttm_linear_group: null pointer");
   TTM_REQUIRE(w_dtype == TTM_BFP8B || w_dtype == TTM_BFP4B, "ttm_linear_group: weights must be BFP_BFloat8 or BFP_BFloat4 (got %d)", w_dtype);
@@ -1847,7 +1926,7 @@ TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int 
     for (int i = 0; i < j; ++i) TTM_REQUIRE(out[i] != out[j], "ttm_linear_group: members %d and %d share an output", i, j);
     TTM_REQUIRE(!act || (act[j] >= TTM_ACT_NONE && act[j] <= TTM_ACT_RELU), "ttm_linear_group: unknown activation %d", act ? act[j] : 0);
   }
-  if (n == 1)
+  if (n == 1 && !qkv)
     return ttm_linear(a, TTM_BF16, w[0], w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, out[0], TTM_BF16, 1, 1, M, N[0], K, act ? act[0] : TTM_ACT_NONE, stream);
   if (M == 0) return TTM_OK;
   TTM_REQUIRE(((uintptr_t)a & 15) == 0, "ttm_linear_group: operands must be 16-byte aligned");
@@ -1870,9 +1949,47 @@ TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int 
   p.nt_split = p.n_blocks1 = p.ntw2 = 0;
   p.img_zero_step = 0;
   p.tail = TTM_TAIL_NONE; p.tail_delta = 0;
+  p.qkv = qkv;
   hipStream_t s = (hipStream_t)stream;
   const int rc = w_dtype == TTM_BFP8B ? launch_linear<WF_BFP8>(p, 1, s) : launch_linear<WF_BFP4>(p, 1, s);
   if (rc) return rc;
   TTM_LAUNCH_CHECK();
   return TTM_OK;
+}
+
+TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N,
+                                const int *act, int64_t M, int64_t K, void *stream) {
+  return linear_group_entry(a, n, w, w_dtype, out, N, act, M, K, nullptr, stream);
+}
+
+TTM_EXPORT int ttm_linear_qkv_decode_supported(int w_dtype, int64_t users, int64_t K, int64_t heads, int64_t kv_heads, int64_t head_dim) {
+  const int64_t Nt = (heads + 2 * kv_heads) * head_dim / 32;
+  return (w_dtype == TTM_BFP8B || w_dtype == TTM_BFP4B) && users >= 1 && users <= 32 && K > 0 && heads >= 1 && kv_heads >= 1 &&
+         head_dim >= 32 && head_dim % 32 == 0 && ttm_option("linear_variant") != 1 && ttm_option("linear_small_m_max") >= 32 &&
+         Nt * 1088 < (int64_t)1 << 32;
+}
+
+TTM_EXPORT int ttm_linear_qkv_decode(const void *a, const void *wq, const void *wk, const void *wv, int w_dtype, int64_t users, int64_t K,
+                                     int64_t heads, int64_t kv_heads, int64_t head_dim, const void *cos_cache, const void *sin_cache,
+                                     int64_t cache_rows, int64_t token_index, void *q_out, void *k_cache, void *v_cache,
+                                     int64_t cache_users, int64_t max_seq, const int32_t *update_index, int64_t batch_offset,
+                                     void *stream) {
+  TTM_REQUIRE(ttm_linear_qkv_decode_supported(w_dtype, users, K, heads, kv_heads, head_dim),
+              "ttm_linear_qkv_decode: needs block-float weights, 1..32 users and a head_dim that is a multiple of 32");
+  TTM_REQUIRE(a && wq && wk && wv && cos_cache && sin_cache && q_out && k_cache && v_cache && update_index, "ttm_linear_qkv_decode: null pointer");
+  TTM_REQUIRE(cache_rows >= 1 && token_index >= 0 && token_index < cache_rows,
+              "ttm_linear_qkv_decode: token_index %lld is outside the %lld cached positions", (long long)token_index, (long long)cache_rows);
+  TTM_REQUIRE(max_seq >= 1 && batch_offset >= 0 && batch_offset + users <= cache_users,
+              "ttm_linear_qkv_decode: batch_offset + users exceeds the cache");
+  TTM_REQUIRE((((uintptr_t)cos_cache | (uintptr_t)sin_cache | (uintptr_t)q_out | (uintptr_t)k_cache | (uintptr_t)v_cache) & 15) == 0,
+              "ttm_linear_qkv_decode: operands must be 16-byte aligned");
+  QkvFinishArgs f = {};
+  f.users = (int)users; f.heads = (int)heads; f.heads_pad = (int)ttm_round_up32(heads); f.kv_heads = (int)kv_heads; f.dim = (int)head_dim;
+  f.cosc = (const uint16_t *)cos_cache; f.sinc = (const uint16_t *)sin_cache; f.cos_row = token_index;
+  f.q_out = (uint16_t *)q_out; f.k_cache = (uint16_t *)k_cache; f.v_cache = (uint16_t *)v_cache;
+  f.max_seq = max_seq; f.seq_pad = ttm_round_up32(max_seq); f.batch_offset = batch_offset; f.index = update_index;
+  const void *w[3] = {wq, wk, wv};
+  void *out[3] = {q_out, k_cache, v_cache};   // distinct, never written through these
+  const int64_t N[3] = {heads * head_dim, kv_heads * head_dim, kv_heads * head_dim};
+  return linear_group_entry(a, 3, w, w_dtype, out, N, nullptr, users, K, &f, stream);
 }

@@ -320,6 +320,132 @@ Tensor transposeLast2(ProgramContext &ctx, const Tensor &t) {
   return out;
 }
 
+// The op that consumes tensor `id` after op `from`, when the tensor has exactly one consumer (deallocations aside); else 0
+std::uint32_t soleConsumer(ProgramContext &ctx, std::uint32_t id, std::uint32_t from) {
+  auto u = ctx.uses.find(id);
+  if (u == ctx.uses.end() || u->second != 1) return 0;
+  for (std::uint32_t j = from + 1; j < ctx.ops.size(); ++j) {
+    if (static_cast<OpType>(ctx.ops[j].scalar<std::uint8_t>(schema::Operation::f_type_type, 0)) == OpType::DeallocateOp) continue;
+    for (const auto &ref : opRefs(ctx.ops[j]).ins)
+      if (refId(ref) == id) return j;
+  }
+  return 0;
+}
+
+// The front of a decode step's attention block: three projections of the same <= 32 tokens (block-float weights) whose
+// results go, each through its own chain of single-consumer ops, to
+//   q: reshape [1, users, heads, D] -> rotary_embedding(token_index)                       -> whoever reads q
+//   k: reshape [1, users, kv, D]    -> rotary_embedding(token_index) -> permute(0, 2, 1, 3) -> update_cache(k cache)
+//   v: reshape [1, users, kv, D]                                     -> permute(0, 2, 1, 3) -> update_cache(v cache)
+// (test/ttmlir/models/single_blocks_and_layers/llama_3_8b_decode_layer.mlir:51-82 after RoPE and cache fusing) run as one
+// projection launch whose partial sums a second kernel turns into q and the two cache rows.  Nothing else may sit between
+// the first projection and the last cache update except deallocations, so running the cache writes early is not observable.
+// members: (op index, out ref, weight) of the three projections.  Returns false, with nothing changed, when the pattern or a
+// shape does not fit.
+struct QkvMember { std::uint32_t index; fb::Table out; Tensor weight; };
+bool tryQkvDecode(ProgramContext &ctx, const Tensor &a, std::int64_t users, std::int64_t K, const std::vector<QkvMember> &members) {
+  if (members.size() != 3 || users > 32 || a.handle->shape.size() != 2) return false;
+  auto typeOf = [&](std::uint32_t i) { return static_cast<OpType>(ctx.ops[i].scalar<std::uint8_t>(schema::Operation::f_type_type, 0)); };
+  auto body = [&](std::uint32_t i) { return ctx.ops[i].table(schema::Operation::f_type); };
+  const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
+  struct Chain { int member = -1; std::uint32_t reshape = 0, rotary = 0, permute = 0, update = 0; std::uint32_t nh = 0; };
+  Chain q, k, v;
+  std::set<std::uint32_t> chainOps;
+  std::uint32_t D = 0, last = 0;
+  for (int mi = 0; mi < 3; ++mi) {
+    Chain c;
+    c.member = mi;
+    chainOps.insert(members[mi].index);
+    c.reshape = soleConsumer(ctx, refId(members[mi].out), members[mi].index);
+    if (!c.reshape || typeOf(c.reshape) != OpType::ReshapeOp || ctx.skip.count(c.reshape)) return false;
+    fb::Table rs = body(c.reshape).table(schema::ReshapeOp::f_out);
+    const std::vector<std::uint32_t> shape = shapeFromTensorRef(rs);
+    if (!rs || !(layoutFromTensorRef(rs) == plain) || shape.size() != 4 || shape[0] != 1 || shape[1] != users || shape[3] % 32 != 0) return false;
+    if (D && D != shape[3]) return false;
+    D = shape[3];
+    c.nh = shape[2];
+    if (static_cast<std::int64_t>(c.nh) * D != members[mi].weight.handle->shape[1]) return false;
+    std::uint32_t next = soleConsumer(ctx, refId(rs), c.reshape);
+    if (!next || ctx.skip.count(next)) return false;
+    std::uint32_t produced = refId(rs), after = c.reshape;
+    if (typeOf(next) == OpType::RotaryEmbeddingOp) {
+      using R = schema::RotaryEmbeddingOp;
+      fb::Table rop = body(next);
+      if (!rop.table(R::f_input) || refId(rop.table(R::f_input)) != produced || !rop.has(R::f_token_index) || !rop.table(R::f_out) ||
+          !(layoutFromTensorRef(rop.table(R::f_out)) == plain) || shapeFromTensorRef(rop.table(R::f_out)) != shape)
+        return false;
+      c.rotary = next;
+      produced = refId(rop.table(R::f_out));
+      after = next;
+      next = soleConsumer(ctx, produced, after);   // 0 when q has several readers: fine for q
+    }
+    if (next && !ctx.skip.count(next) && typeOf(next) == OpType::PermuteOp) {
+      fb::Table pop = body(next);
+      auto pv = pop.scalars<std::int64_t>(schema::PermuteOp::f_permutation);
+      fb::Table pout = pop.table(schema::PermuteOp::f_out);
+      if (pv.size() == 4 && pv[0] == 0 && pv[1] == 2 && pv[2] == 1 && pv[3] == 3 && pout && refId(pop.table(schema::PermuteOp::f_in)) == produced) {
+        const std::uint32_t upd = soleConsumer(ctx, refId(pout), next);
+        if (upd && !ctx.skip.count(upd) && typeOf(upd) == OpType::UpdateCacheOp &&
+            refId(body(upd).table(schema::UpdateCacheOp::f_input)) == refId(pout)) {
+          c.permute = next;
+          c.update = upd;
+        }
+      }
+    }
+    if (c.rotary && !c.update) { if (q.member >= 0) return false; q = c; }
+    else if (c.rotary && c.update) { if (k.member >= 0) return false; k = c; }
+    else if (c.update) { if (v.member >= 0) return false; v = c; }
+    else return false;
+    for (std::uint32_t o : {c.reshape, c.rotary, c.permute, c.update})
+      if (o) { chainOps.insert(o); last = std::max(last, o); }
+  }
+  if (q.member < 0 || k.member < 0 || v.member < 0 || k.nh != v.nh || q.nh % k.nh != 0) return false;
+  // only the chains and deallocations between the first projection and the last cache update
+  for (std::uint32_t j = ctx.opIndex; j <= last; ++j)
+    if (!chainOps.count(j) && typeOf(j) != OpType::DeallocateOp) return false;
+  using R = schema::RotaryEmbeddingOp;
+  using U = schema::UpdateCacheOp;
+  fb::Table rq = body(q.rotary), rk = body(k.rotary), uk = body(k.update), uv = body(v.update);
+  if (refId(rq.table(R::f_cos_cache)) != refId(rk.table(R::f_cos_cache)) || refId(rq.table(R::f_sin_cache)) != refId(rk.table(R::f_sin_cache)) ||
+      rq.scalar<std::uint32_t>(R::f_token_index, 0) != rk.scalar<std::uint32_t>(R::f_token_index, 0) ||
+      refId(uk.table(U::f_update_index)) != refId(uv.table(U::f_update_index)) ||
+      uk.scalar<std::uint32_t>(U::f_batch_offset, 0) != uv.scalar<std::uint32_t>(U::f_batch_offset, 0) ||
+      refId(uk.table(U::f_cache)) == refId(uv.table(U::f_cache)))
+    return false;
+  auto live = [&](const fb::Table &ref) {
+    auto it = ref ? ctx.pool.find(refId(ref)) : ctx.pool.end();
+    return it != ctx.pool.end() && isTensorAllocated(it->second) ? &it->second : nullptr;
+  };
+  Tensor *cosT = live(rq.table(R::f_cos_cache)), *sinT = live(rq.table(R::f_sin_cache)), *idxT = live(uk.table(U::f_update_index));
+  Tensor *kc = live(uk.table(U::f_cache)), *vc = live(uv.table(U::f_cache));
+  if (!cosT || !sinT || !idxT || !kc || !vc) return false;
+  const Layout cl = getTensorLayout(*cosT);
+  if (!(cl == plain) || !(getTensorLayout(*sinT) == plain) || !(getTensorLayout(*kc) == plain) || !(getTensorLayout(*vc) == plain)) return false;
+  const auto &cs = cosT->handle->shape, &ks = kc->handle->shape;
+  const std::uint32_t token = rq.scalar<std::uint32_t>(R::f_token_index, 0), offset = uk.scalar<std::uint32_t>(U::f_batch_offset, 0);
+  if (cs.size() != 4 || sinT->handle->shape != cs || cs[0] != 1 || cs[1] != 1 || cs[3] != D || token >= cs[2]) return false;
+  if (ks.size() != 4 || vc->handle->shape != ks || ks[1] != k.nh || ks[3] != D || offset + users > ks[0]) return false;
+  if (idxT->handle->storage != StorageType::Device || idxT->handle->layout != TensorLayout::RowMajor ||
+      (idxT->handle->dtype != DataType::Int32 && idxT->handle->dtype != DataType::UInt32) || volume(idxT->handle->shape) < 1)
+    return false;
+  const int wdt = ttmDtype(members[0].weight.handle->dtype);
+  if (!ttm_linear_qkv_decode_supported(wdt, users, K, q.nh, k.nh, D)) return false;
+
+  fb::Table qRef = rq.table(R::f_out);
+  Tensor qOut = makeOut(ctx, qRef, DataType::BFloat16, TensorLayout::Tile);
+  TTM_CALL(ttm_linear_qkv_decode(a.handle->data.get(), members[q.member].weight.handle->data.get(), members[k.member].weight.handle->data.get(),
+                                 members[v.member].weight.handle->data.get(), wdt, users, K, q.nh, k.nh, D, cosT->handle->data.get(),
+                                 sinT->handle->data.get(), cs[2], token, qOut.handle->data.get(), kc->handle->data.get(), vc->handle->data.get(),
+                                 ks[0], ks[2], static_cast<const std::int32_t *>(idxT->handle->data.get()), offset, ctx.stream()));
+  ctx.put(qRef, finish(ctx, qOut, qRef));
+  kc->handle->version = nextTensorVersion();
+  vc->handle->version = nextTensorVersion();
+  for (std::uint32_t o : chainOps)
+    if (o != ctx.opIndex) ctx.skip.insert(o);
+  debug::Stats::get().incrementStat("FusedQkvDecode");
+  return true;
+}
+
 void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &bRef, const fb::Table &biasRef, const fb::Table &outRef,
                    bool transposeA, bool transposeB, std::string_view activation) {
   Tensor a = as(ctx, ctx.get(aRef, "matmul a"), TensorLayout::Tile, DataType::BFloat16);
@@ -454,6 +580,11 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
       if (!distinct) break;
       followers.push_back(Follower{j, out2, wit->second, static_cast<std::int64_t>(shape2.back()), activationCode(act2)});
     }
+    if (followers.size() == 2 && M <= 32 && activationCode(activation) == TTM_ACT_NONE && followers[0].act == TTM_ACT_NONE &&
+        followers[1].act == TTM_ACT_NONE &&
+        tryQkvDecode(ctx, a, M, K, {QkvMember{ctx.opIndex, outRef, b}, QkvMember{followers[0].index, followers[0].out, followers[0].weight},
+                                    QkvMember{followers[1].index, followers[1].out, followers[1].weight}}))
+      return;
     if (!followers.empty()) {
       std::vector<const void *> ws{b.handle->data.get()};
       std::vector<void *> outs{out.handle->data.get()};
