@@ -136,6 +136,17 @@ int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, vo
                      const int *act, int64_t M, int64_t K, void *stream);
 int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M, int64_t N,
                     int64_t K, void *stream);
+/* x1 = residual + a w and norm_out = rms_norm(x1) * norm_weight + norm_bias for M <= 32 rows in two launches (the output
+ * projection of a decode step's attention block with its residual connection and the RMSNorm in front of the MLP):
+ * the projection leaves fp32 partial sums and the RMSNorm kernel starts from them.  a [M, K], residual, sum_out (receives x1)
+ * and norm_out [M, N] are bf16 tiles, w block-float [K, N]; norm_weight / norm_bias [N] bf16 in the given layout, or NULL.
+ * Bit-identical to ttm_linear_tail(.., TTM_TAIL_ADD, residual) followed by ttm_rms_norm (runtime/lib/ttnn/operations/
+ * matmul/matmul.cpp:47-83, eltwise/binary/binary.cpp:38-126, normalization/rms_norm.cpp:10-49).
+ * ttm_linear_add_rms_norm_supported returns 1 when the shapes and the selected kernel variants allow it, else 0. */
+int ttm_linear_add_rms_norm_supported(int w_dtype, int64_t M, int64_t N, int64_t K);
+int ttm_linear_add_rms_norm(const void *a, const void *w, int w_dtype, const void *residual, void *sum_out, const void *norm_weight,
+                            int weight_layout, const void *norm_bias, int bias_layout, float eps, void *norm_out, int64_t M, int64_t N,
+                            int64_t K, void *stream);
 /* The front of a decode step's attention block in two launches: the Q, K and V projections of `users` <= 32 tokens (one
  * per user, activations a [users, K] bf16 tiles, block-float weights [K, heads * head_dim] and twice
  * [K, kv_heads * head_dim]), then in one kernel the head split, the rotary embedding of q and k with row `token_index` of

@@ -487,3 +487,40 @@ def test_linear_qkv_decode_rejects_what_it_cannot_fuse(hip, dev):
         hip.call("ttm_linear_qkv_decode", *args(token=1))
     with pytest.raises(hip.TTMError, match="exceeds the cache"):
         hip.call("ttm_linear_qkv_decode", *args(off=1))
+
+
+@pytest.mark.parametrize("M,K,N,fmt,with_w,with_b", [
+    (32, 4096, 4096, "bfp8", True, False),      # the output projection of the Llama-3-8B decode step (K split four ways)
+    (7, 256, 512, "bfp8", True, True),          # no split, ragged rows
+    (32, 14336, 4096, "bfp4", True, False),
+    (1, 512, 96, "bfp4", False, False),
+])
+def test_linear_add_rms_norm_equals_the_op_sequence(hip, dev, orc, M, K, N, fmt, with_w, with_b):
+    """ttm_linear_add_rms_norm against ttm_linear_tail (add) followed by ttm_rms_norm: both outputs bit-identical."""
+    from test_gpu_linear import pack_weight
+    wf = hip.BFP8B if fmt == "bfp8" else hip.BFP4B
+    a = datagen.randn((M, K), seed=110, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=111, dtype=torch.float32) * 0.05
+    res = datagen.randn((M, N), seed=112, dtype=torch.bfloat16)
+    nw = (1.0 + 0.1 * datagen.randn((1, N), seed=113, dtype=torch.float32)).to(torch.bfloat16)
+    nb = (0.1 * datagen.randn((1, N), seed=114, dtype=torch.float32)).to(torch.bfloat16)
+    at, rt_, wt, nwt, nbt = tilize_dev(hip, a, dev), tilize_dev(hip, res, dev), pack_weight(hip, w, wf, dev), tilize_dev(hip, nw, dev), tilize_dev(hip, nb, dev)
+    s = hip.current_stream()
+    Np = (N + 31) // 32 * 32
+    x1 = torch.full((32 * Np,), float("nan"), dtype=torch.bfloat16, device=dev)
+    h = torch.full_like(x1, float("nan"))
+    hip.call("ttm_linear_tail", hip.ptr(at), hip.BF16, hip.ptr(wt), wf, 0, None, hip.BF16, hip.TILE, hip.ptr(x1), hip.BF16, 1, 1, M, N, K,
+             hip.ACT[None], 1, hip.ptr(rt_), s)
+    hip.call("ttm_rms_norm", hip.ptr(x1), hip.ptr(nwt) if with_w else None, hip.TILE, hip.ptr(nbt) if with_b else None, hip.TILE, hip.ptr(h),
+             hip.BF16, 1, M, N, 1e-5, s)
+    assert hip.lib().ttm_linear_add_rms_norm_supported(wf, M, N, K) == 1
+    x1f, hf = torch.full_like(x1, float("nan")), torch.full_like(x1, float("nan"))
+    hip.call("ttm_linear_add_rms_norm", hip.ptr(at), hip.ptr(wt), wf, hip.ptr(rt_), hip.ptr(x1f), hip.ptr(nwt) if with_w else None, hip.TILE,
+             hip.ptr(nbt) if with_b else None, hip.TILE, 1e-5, hip.ptr(hf), M, N, K, s)
+    torch.cuda.synchronize()
+    assert torch.equal(x1f, x1) and torch.equal(hf, h)
+    assert bool(torch.isfinite(hf.float()).all())
+    assert hip.lib().ttm_linear_add_rms_norm_supported(wf, 33, N, K) == 0 and hip.lib().ttm_linear_add_rms_norm_supported(hip.BF16, M, N, K) == 0
+    with pytest.raises(hip.TTMError, match="must not alias"):
+        hip.call("ttm_linear_add_rms_norm", hip.ptr(at), hip.ptr(wt), wf, hip.ptr(rt_), hip.ptr(rt_), None, hip.TILE, None, hip.TILE, 1e-5,
+                 hip.ptr(hf), M, N, K, s)

@@ -827,6 +827,8 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
         assert mode != "traced" or qkv in (1, 2)
         assert rt.get_stat("FusedCacheUpdate") == 0 and rt.get_stat("FusedHeadSplit") == 0 and rt.get_stat("GroupedMatmul") == 0
         assert rt.get_stat("FusedHeadConcat") == qkv
+        # the output projection, its residual add and the RMSNorm in front of the MLP are one fused step as well
+        assert rt.get_stat("FusedLinearAddNorm") == qkv
     # the replayed graph runs the same kernels on the same data: identical to the op-by-op run, caches included; so is
     # the unfused run
     for other in ("traced", "callbacks"):

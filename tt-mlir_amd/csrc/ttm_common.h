@@ -38,6 +38,12 @@ int ttm_option(const char *name);  // 0 when unset
 // have recorded is never freed before the stream is destroyed.
 int ttm_stream_workspace(hipStream_t stream, size_t bytes, void **ptr);
 
+// RMSNorm that starts from the fp32 partial sums of a split-K projection of one row tile plus a residual (ttm_rowwise.hip)
+bool ttm_rowwise_partials_supported(int64_t rows, int64_t cols);
+int ttm_rowwise_rmsnorm_from_partials(const float *partial, int slices, int64_t per, const void *residual, void *sum_out,
+                                      const void *weight, int weight_layout, const void *bias, int bias_layout, void *out,
+                                      int64_t rows, int64_t cols, float eps, hipStream_t s);
+
 __host__ __device__ static inline int64_t ttm_round_up32(int64_t v) { return (v + 31) / 32 * 32; }
 static inline int64_t ttm_cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

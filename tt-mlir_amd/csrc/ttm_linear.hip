@@ -57,6 +57,16 @@ struct LinearArgs {
   int tail;                           // 0 none, 1 add, 2 multiply: element-wise tail with a tensor laid out like the output
   int64_t tail_delta;                 // byte distance from an output element to its tail operand
   const struct QkvFinishArgs *qkv;    // host side only: the decode launch leaves partial sums and ttm_qkv_finish_k ends it
+  const struct NormFinishArgs *norm;  // host side only: ... and the RMSNorm kernel ends it (residual add, then the norm)
+};
+
+// x1 = residual + projection (stored to sum_out), then out = rms_norm(x1): the operands of the second launch
+struct NormFinishArgs {
+  const void *residual, *weight, *bias;
+  int weight_layout, bias_layout;
+  void *sum_out, *out;
+  int64_t rows, cols;
+  float eps;
 };
 
 // What follows the Q, K and V projections of a decode step (one token per user): head split, rotary embedding of q and k
@@ -1692,7 +1702,8 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
     }
     const int64_t per = (int64_t)a.Nt * 1024;
     if (a.qkv && (!decode || a.Mt != 1 || batch != 1)) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear_qkv_decode: the selected kernel variant cannot end in the fused step");
-    if (slices > 1 || a.qkv) {
+    if (a.norm && (!decode || a.Mt != 1 || batch != 1)) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear_add_rms_norm: the selected kernel variant cannot end in the fused step");
+    if (slices > 1 || a.qkv || a.norm) {
       void *ws = nullptr;
       if (int rc = ttm_stream_workspace(s, (size_t)(per * slices * batch) * sizeof(float), &ws)) return rc;
       p.partial = (float *)ws;
@@ -1717,6 +1728,11 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         f.partial = p.partial; f.slices = slices; f.per = per;
         const int64_t lanes = per / 4 + (int64_t)f.users * (f.heads_pad - f.heads) * (f.dim / 4);
         hipLaunchKernelGGL(ttm_qkv_finish_k, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, s, f);
+      } else if (a.norm) {
+        const NormFinishArgs &f = *a.norm;
+        if (int rc = ttm_rowwise_rmsnorm_from_partials(p.partial, slices, per, f.residual, f.sum_out, f.weight, f.weight_layout, f.bias,
+                                                       f.bias_layout, f.out, f.rows, f.cols, f.eps, s))
+          return rc;
       } else if (slices > 1)
         hipLaunchKernelGGL(ttm_linear_reduce_k, dim3((unsigned)((per / 4 + 255) / 256), 1, (unsigned)batch), dim3(256), 0, s, p, slices);
     }
@@ -1847,7 +1863,8 @@ TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype
 // stored back to back (a pair of weight matrices applied to the same activations)
 static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias, int bias_dtype,
                         int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K,
-                        int act, int tail_op, const void *tail, const int64_t *strides, void *stream) {
+                        int act, int tail_op, const void *tail, const int64_t *strides, void *stream,
+                        const NormFinishArgs *norm = nullptr) {
   TTM_REQUIRE(tail_op >= TTM_TAIL_NONE && tail_op <= TTM_TAIL_MUL, "ttm_linear: unknown tail op %d", tail_op);
   TTM_REQUIRE((tail_op == TTM_TAIL_NONE) == (tail == nullptr), "ttm_linear: a tail op needs its operand, and only then");
   TTM_REQUIRE(((uintptr_t)tail & 15) == 0, "ttm_linear: the tail operand must be 16-byte aligned");
@@ -1885,6 +1902,7 @@ static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, 
   p.tail = tail_op;
   p.tail_delta = tail ? (const uint8_t *)tail - (const uint8_t *)out : 0;
   p.qkv = nullptr;
+  p.norm = norm;
   if (strides) { p.a_batch = strides[0]; p.w_batch = strides[1]; p.c_batch = strides[2]; }
   TTM_REQUIRE(batch <= 65535, "ttm_linear: batch too large");
   hipStream_t s = (hipStream_t)stream;
@@ -1903,6 +1921,24 @@ TTM_EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_
                                int64_t M, int64_t N, int64_t K, int act, int tail_op, const void *tail, void *stream) {
   return linear_entry(a, a_dtype, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, act,
                       tail_op, tail, nullptr, stream);
+}
+
+TTM_EXPORT int ttm_linear_add_rms_norm_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
+  return (w_dtype == TTM_BFP8B || w_dtype == TTM_BFP4B) && M >= 1 && M <= 32 && K > 0 && N >= 1 && ttm_rowwise_partials_supported(M, N) &&
+         ttm_option("linear_variant") != 1 && ttm_option("linear_small_m_max") >= 32 && ttm_cdiv(N, 32) * 1088 < (int64_t)1 << 32;
+}
+
+TTM_EXPORT int ttm_linear_add_rms_norm(const void *a, const void *w, int w_dtype, const void *residual, void *sum_out, const void *norm_weight,
+                                       int weight_layout, const void *norm_bias, int bias_layout, float eps, void *norm_out, int64_t M,
+                                       int64_t N, int64_t K, void *stream) {
+  TTM_REQUIRE(ttm_linear_add_rms_norm_supported(w_dtype, M, N, K),
+              "ttm_linear_add_rms_norm: needs block-float weights, 1..32 rows and at most 16384 columns");
+  TTM_REQUIRE(residual && sum_out && norm_out, "ttm_linear_add_rms_norm: null pointer");
+  TTM_REQUIRE(sum_out != residual && norm_out != sum_out && norm_out != residual, "ttm_linear_add_rms_norm: the outputs must not alias the residual or each other");
+  TTM_REQUIRE((((uintptr_t)residual | (uintptr_t)norm_out) & 15) == 0, "ttm_linear_add_rms_norm: operands must be 16-byte aligned");
+  NormFinishArgs f = {residual, norm_weight, norm_bias, weight_layout, bias_layout, sum_out, norm_out, M, N, eps};
+  return linear_entry(a, TTM_BF16, w, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, sum_out, TTM_BF16, 1, 1, M, N, K, TTM_ACT_NONE, TTM_TAIL_NONE,
+                      nullptr, nullptr, stream, &f);
 }
 
 TTM_EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M,
@@ -1950,6 +1986,7 @@ static int linear_group_entry(const void *a, int n, const void *const *w, int w_
   p.img_zero_step = 0;
   p.tail = TTM_TAIL_NONE; p.tail_delta = 0;
   p.qkv = qkv;
+  p.norm = nullptr;
   hipStream_t s = (hipStream_t)stream;
   const int rc = w_dtype == TTM_BFP8B ? launch_linear<WF_BFP8>(p, 1, s) : launch_linear<WF_BFP4>(p, 1, s);
   if (rc) return rc;

@@ -20,6 +20,13 @@ struct RowArgs {
   int rt, ct;          // tiles per batch entry
   float eps;
   int out_ct;          // reductions: column tiles of the output (1), keepdim layout [.., rows, 1]
+  // ttm_rowwise_row_k<.., PRE = true>: x is not read but made on the way in from the fp32 partial sums of a split-K
+  // projection of one row tile, x = bf16(bf16(sum over slices) + residual), and also stored to sum_out
+  const float *partial;
+  int slices;
+  int64_t per;         // floats per slice
+  const void *residual;
+  void *sum_out;
 };
 
 template <int ELEM>
@@ -281,7 +288,7 @@ __global__ __launch_bounds__(256) void ttm_rowwise_resident_k(RowArgs p) {
 // flight, and a workgroup issues all its loads at once: a [32, 4096] input is 32 short workgroups instead of 4 long ones.
 // Consecutive rows of a face share 128-byte lines, so the row -> workgroup map gives every XCD (workgroup id mod 8)
 // a contiguous range of rows and its L2 sees each line of that range whole.
-template <int MODE, int ELEM, int NK>
+template <int MODE, int ELEM, int NK, bool PRE = false>
 __global__ __launch_bounds__(256) void ttm_rowwise_row_k(RowArgs p, int total_rows) {
   constexpr int EPC = 16 / ELEM;
   __shared__ float red[4], red2[4];
@@ -299,7 +306,26 @@ __global__ __launch_bounds__(256) void ttm_rowwise_row_k(RowArgs p, int total_ro
   for (int k = 0; k < NK; ++k) {
     const int q = tid + k * 256;
     v[k] = u32x4{0, 0, 0, 0};
-    if (q < nq && row_ok) v[k] = *(const u32x4 *)(x + chunk_pos<ELEM>(r, q).off * ELEM);
+    if constexpr (PRE) {   // bf16 rows made from partial sums: the projection's rounding, then the residual add's
+      static_assert(!PRE || ELEM == 2, "partial sums finish as bf16");
+      if (q < nq) {
+        const int64_t off = chunk_pos<ELEM>(r, q).off;
+        if (row_ok) {
+          f32x4 s0 = *(const f32x4 *)(p.partial + off), s1 = *(const f32x4 *)(p.partial + off + 4);
+          for (int sl = 1; sl < p.slices; ++sl) {
+            s0 += *(const f32x4 *)(p.partial + sl * p.per + off);
+            s1 += *(const f32x4 *)(p.partial + sl * p.per + off + 4);
+          }
+          const u32x4 y = {ttm_pack_bf16x2(s0.x, s0.y), ttm_pack_bf16x2(s0.z, s0.w), ttm_pack_bf16x2(s1.x, s1.y), ttm_pack_bf16x2(s1.z, s1.w)};
+          const u32x4 t = *(const u32x4 *)((const uint8_t *)p.residual + off * 2);
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            v[k][i] = ttm_pack_bf16x2(__uint_as_float(y[i] << 16) + __uint_as_float(t[i] << 16),
+                                      __uint_as_float(y[i] & 0xFFFF0000u) + __uint_as_float(t[i] & 0xFFFF0000u));
+        }
+        *(u32x4 *)((uint8_t *)p.sum_out + off * 2) = v[k];
+      }
+    } else if (q < nq && row_ok) v[k] = *(const u32x4 *)(x + chunk_pos<ELEM>(r, q).off * ELEM);
   }
   u32x4 wraw[NK], braw[NK];   // weight / bias chunks, still packed
   if (MODE == RW_RMSNORM) {
@@ -610,6 +636,33 @@ static int fill_args(RowArgs &p, const void *x, void *out, int dtype, int64_t ba
   p.rows = rows; p.cols = cols;
   p.rt = (int)ttm_cdiv(rows, 32); p.ct = (int)ttm_cdiv(cols, 32);
   p.eps = 0.0f; p.out_ct = 1;
+  p.partial = nullptr; p.slices = 0; p.per = 0; p.residual = nullptr; p.sum_out = nullptr;
+  return TTM_OK;
+}
+
+// RMSNorm of x = bf16(bf16(sum of the partial sums) + residual) for one row tile ([rows <= 32, cols] bf16 tiles), x
+// stored to sum_out on the way: what ttm_linear_reduce_k with an add tail followed by ttm_rms_norm computes, with the
+// kernel ttm_rms_norm itself uses at this size, so the two agree bit for bit.
+bool ttm_rowwise_partials_supported(int64_t rows, int64_t cols) {
+  const int v = ttm_option("rowwise_variant");
+  return rows >= 1 && rows <= 32 && cols >= 1 && ttm_cdiv(cols, 32) * 4 <= 8 * 256 && (v == 0 || v == 3);
+}
+int ttm_rowwise_rmsnorm_from_partials(const float *partial, int slices, int64_t per, const void *residual, void *sum_out,
+                                      const void *weight, int weight_layout, const void *bias, int bias_layout, void *out,
+                                      int64_t rows, int64_t cols, float eps, hipStream_t s) {
+  TTM_REQUIRE(ttm_rowwise_partials_supported(rows, cols), "rms_norm from partial sums: at most 32 rows and 16384 columns");
+  RowArgs p;
+  if (int rc = fill_args(p, residual, out, TTM_BF16, 1, rows, cols, "ttm_linear_add_rms_norm")) return rc;
+  TTM_REQUIRE(partial && sum_out && slices >= 1, "rms_norm from partial sums: null pointer");
+  TTM_REQUIRE((((uintptr_t)weight | (uintptr_t)bias | (uintptr_t)sum_out) & 15) == 0, "ttm_linear_add_rms_norm: operands must be 16-byte aligned");
+  p.w = weight; p.b = bias; p.w_tiled = weight_layout == TTM_TILE; p.b_tiled = bias_layout == TTM_TILE; p.eps = eps;
+  p.partial = partial; p.slices = slices; p.per = per; p.residual = residual; p.sum_out = sum_out;
+  const int nq = p.ct * 4;
+  const dim3 grid(32), block(256);
+  if (nq <= 512) hipLaunchKernelGGL((ttm_rowwise_row_k<RW_RMSNORM, 2, 2, true>), grid, block, 0, s, p, 32);
+  else if (nq <= 1024) hipLaunchKernelGGL((ttm_rowwise_row_k<RW_RMSNORM, 2, 4, true>), grid, block, 0, s, p, 32);
+  else hipLaunchKernelGGL((ttm_rowwise_row_k<RW_RMSNORM, 2, 8, true>), grid, block, 0, s, p, 32);
+  TTM_LAUNCH_CHECK();
   return TTM_OK;
 }
 

@@ -320,6 +320,13 @@ Tensor transposeLast2(ProgramContext &ctx, const Tensor &t) {
   return out;
 }
 
+// TTMLIR_RUNTIME_NO_DECODE_FUSION=1 keeps the decode-step fusions below off (the ops then run as the smaller fusions or
+// one by one): for measurements and for telling a fusion's fault from a kernel's
+bool decodeFusionEnabled() {
+  static const bool on = [] { const char *e = std::getenv("TTMLIR_RUNTIME_NO_DECODE_FUSION"); return !(e && e[0] == '1'); }();
+  return on;
+}
+
 // The op that consumes tensor `id` after op `from`, when the tensor has exactly one consumer (deallocations aside); else 0
 std::uint32_t soleConsumer(ProgramContext &ctx, std::uint32_t id, std::uint32_t from) {
   auto u = ctx.uses.find(id);
@@ -344,7 +351,7 @@ std::uint32_t soleConsumer(ProgramContext &ctx, std::uint32_t id, std::uint32_t 
 // shape does not fit.
 struct QkvMember { std::uint32_t index; fb::Table out; Tensor weight; };
 bool tryQkvDecode(ProgramContext &ctx, const Tensor &a, std::int64_t users, std::int64_t K, const std::vector<QkvMember> &members) {
-  if (members.size() != 3 || users > 32 || a.handle->shape.size() != 2) return false;
+  if (!decodeFusionEnabled() || members.size() != 3 || users > 32 || a.handle->shape.size() != 2) return false;
   auto typeOf = [&](std::uint32_t i) { return static_cast<OpType>(ctx.ops[i].scalar<std::uint8_t>(schema::Operation::f_type_type, 0)); };
   auto body = [&](std::uint32_t i) { return ctx.ops[i].table(schema::Operation::f_type); };
   const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
@@ -608,6 +615,44 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
       debug::Stats::get().incrementStat("GroupedMatmul");
       debug::Stats::get().incrementStat("GroupedMatmulMembers", static_cast<std::int64_t>(ws.size()));
       return;
+    }
+  }
+  // residual + projection followed at once by the RMSNorm of that sum (the end of a decode step's attention block): the
+  // projection leaves partial sums and the RMSNorm kernel starts from them, one launch fewer and no pass over the sum
+  if (decodeFusionEnabled() && tailOp == TTM_TAIL_ADD && !biasRef && !transposeB && batch == 1 && as_.size() == 2 && activationCode(activation) == TTM_ACT_NONE &&
+      utils::isBlockFormatDataType(b.handle->dtype) && ttm_linear_add_rms_norm_supported(ttmDtype(b.handle->dtype), M, N, K)) {
+    std::uint32_t j = nextIdx + 1;
+    while (j < ctx.ops.size() && opType(j) == OpType::DeallocateOp) {
+      const std::uint32_t freed = refId(ctx.ops[j].table(schema::Operation::f_type).table(schema::DeallocateOp::f_in));
+      if (freed == refId(finalRef)) break;
+      ++j;
+    }
+    if (j < ctx.ops.size() && opType(j) == OpType::RMSNormOp && !ctx.skip.count(j)) {
+      using R = schema::RMSNormOp;
+      fb::Table nop = ctx.ops[j].table(schema::Operation::f_type);
+      fb::Table nin = nop.table(R::f_input), nout = nop.table(R::f_out), wr = nop.table(R::f_weight), br = nop.table(R::f_bias);
+      const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
+      auto vec = [&](const fb::Table &ref) -> const Tensor * {   // a [N] bf16 tile tensor that is live now
+        auto it = ctx.pool.find(refId(ref));
+        if (it == ctx.pool.end() || !isTensorAllocated(it->second) || !(getTensorLayout(it->second) == plain) ||
+            static_cast<std::int64_t>(volume(it->second.handle->shape)) != N)
+          return nullptr;
+        return &it->second;
+      };
+      const Tensor *wT = wr ? vec(wr) : nullptr, *bT = br ? vec(br) : nullptr;
+      if (nin && nout && refId(nin) == refId(finalRef) && layoutFromTensorRef(nout) == plain &&
+          shapeFromTensorRef(nout) == shapeFromTensorRef(finalRef) && (!wr || wT) && (!br || bT)) {
+        Tensor normOut = makeDeviceTensor(ctx.dev, out.handle->shape, DataType::BFloat16, TensorLayout::Tile);
+        TTM_CALL(ttm_linear_add_rms_norm(a.handle->data.get(), b.handle->data.get(), ttmDtype(b.handle->dtype), tail.handle->data.get(),
+                                         out.handle->data.get(), wT ? wT->handle->data.get() : nullptr, TTM_TILE,
+                                         bT ? bT->handle->data.get() : nullptr, TTM_TILE, nop.scalar<float>(R::f_epsilon, 0.0f),
+                                         normOut.handle->data.get(), M, N, K, ctx.stream()));
+        ctx.put(finalRef, finish(ctx, out, finalRef));
+        ctx.put(nout, finish(ctx, normOut, nout));
+        ctx.skip.insert(j);
+        debug::Stats::get().incrementStat("FusedLinearAddNorm");
+        return;
+      }
     }
   }
   TTM_CALL(ttm_linear_tail(a.handle->data.get(), TTM_BF16, b.handle->data.get(), ttmDtype(b.handle->dtype), transposeB ? 1 : 0, biasPtr,
