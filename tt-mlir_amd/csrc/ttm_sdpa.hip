@@ -510,6 +510,15 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
     }
   };
   if (kb_end > kb_begin) load_block(kb_begin);
+  // per-lane part of the V^T fragment addresses: tile row kh, the face of this lane's column half, its key row and 4 columns
+  const int dhalf = (lane >> 4) & 1, s16 = lane & 15;
+  const uint8_t *vbase = (const uint8_t *)ldsV + kh * DT * 2048 + dhalf * 512;
+  const int vlo = ((4 * hh + (s16 >> 2)) * 32 + 8 * (s16 & 3) + 128 * dhalf) & 511, vhi = (vlo + 256) & 511;
+  auto tr_read = [](const uint8_t *a) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)a);
+    return *(const u32x2 *)&v;
+  };
   constexpr float LOG2E = 1.4426950408889634f;
   const float scale2 = p.scale * LOG2E;
   if (kh == 0) sink_start(p, h, scale2, m_run, l_run);   // the sink belongs to one of the two halves only
@@ -521,22 +530,10 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
       if (c < CHUNKS) {   // uniform over a wavefront: CHUNKS is a multiple of 64
         const int tr = c / (DT * 128), cc = c % (DT * 128);
         ((u32x4 *)ldsK)[c] = kreg[i];
-        const u32x4 v = vreg[i];
-        const int tile = cc >> 7, c7 = cc & 127;
-        const int face = c7 >> 5, row = (c7 & 31) >> 1, half = c7 & 1;
-        const bool odd = row & 1;
-        const int key = 32 * tr + (face >> 1) * 16 + (row & ~1);          // even key of the pair
-        const int d0 = tile * 32 + (face & 1) * 16 + half * 8 + (odd ? 4 : 0);
-        const uint32_t send0 = odd ? v.x : v.z, send1 = odd ? v.y : v.w;
-        const uint32_t got0 = quad_xor2(send0), got1 = quad_xor2(send1);
-        const uint32_t mine0 = odd ? v.z : v.x, mine1 = odd ? v.w : v.y;
-        const uint32_t e0 = odd ? got0 : mine0, o0 = odd ? mine0 : got0;  // even key's word, odd key's word
-        const uint32_t e1 = odd ? got1 : mine1, o1 = odd ? mine1 : got1;
-        uint32_t *vt = (uint32_t *)(ldsV + d0 * VPITCH + key);
-        vt[0] = __builtin_amdgcn_perm(o0, e0, 0x05040100u);
-        vt[VPITCH / 2] = __builtin_amdgcn_perm(o0, e0, 0x07060302u);
-        vt[VPITCH] = __builtin_amdgcn_perm(o1, e1, 0x05040100u);
-        vt[3 * VPITCH / 2] = __builtin_amdgcn_perm(o1, e1, 0x07060302u);
+        // V as it lies in its tiles (rows are keys), the faces of the upper 16 columns rotated by four rows so that the
+        // transposing reads below touch every bank once
+        const int c7 = cc & 127, face = c7 >> 5;
+        *(u32x4 *)((uint8_t *)ldsV + (c - c7) * 16 + face * 512 + (((c7 & 31) * 16 + 128 * (face & 1)) & 511)) = vreg[i];
       }
     }
     __syncthreads();
@@ -615,8 +612,11 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
       pb.w = pack_bf16_rne(s[8 * t + 6], s[8 * t + 7]);
 #pragma unroll
       for (int d = 0; d < DT; ++d) {
-        const uint16_t *vr = ldsV + (d * 32 + l31) * VPITCH + 32 * kh + 16 * t + 4 * hh;
-        u32x2 lo = *(const u32x2 *)vr, hi = *(const u32x2 *)(vr + 8);
+        // V^T fragment: column d * 32 + l31, keys 16 t + 4 hh .. + 3 and eight further on, by two transposing LDS reads
+        // (ds_read_b64_tr_b16: of the 16 lanes of a group, lane 4 u + c receives element c of the rows that lanes
+        // u, u + 4, u + 8, u + 12 address; lane u + 4 j addresses key j of the four, columns 4 u .. + 3)
+        const uint8_t *vb = vbase + d * 2048 + t * 1024;
+        const u32x2 lo = tr_read(vb + vlo), hi = tr_read(vb + vhi);
         u32x4 va = {lo.x, lo.y, hi.x, hi.y};
         o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va, *(bf16x8 *)&pb, o[d], 0, 0, 0);
       }
