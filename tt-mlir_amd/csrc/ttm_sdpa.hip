@@ -238,18 +238,13 @@ __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
 }
 
 // Same computation with 64 keys per pass (head_dim <= 128): half as many barriers and loop turns, two independent
-// accumulator chains for S, and V^T written to LDS as 32-bit pairs of neighbouring keys (the two lanes that hold keys
-// k and k + 1 of the same 8 columns trade halves with a quad permute) instead of 16-bit scatters.
-__device__ __forceinline__ uint32_t quad_xor2(uint32_t v) {   // value of lane ^ 2
-  return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E /* quad_perm [2,3,0,1] */, 0xF, 0xF, true);
-}
-
-constexpr int kSdpaVPitch = 68;   // V^T row pitch in bf16 (64 keys + pad): rows 34 words apart
+// accumulator chains for S; K and V go to LDS as they lie in their tiles and the V^T fragments of the second product are
+// made by transposing LDS reads.
+constexpr int kSdpaVPitch = 68;   // sizes the V staging area: head_dim rows of 68 bf16 (64 keys x head_dim bf16 are used)
 
 // one block of 128 queries (4 wavefronts x 32) of head h against all the keys it needs
 template <int DT>  // head_dim / 32
 __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *ldsK, uint16_t *ldsV) {
-  constexpr int VPITCH = kSdpaVPitch;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int hk = h / (p.Hq / p.Hkv);
   const int qt = qb * 4 + wave;                         // this wave's query tile
@@ -290,6 +285,15 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
     }
   };
   if (kb_end > kb_begin) load_block(kb_begin);
+  // per-lane part of the V^T fragment addresses: the face of this lane's column half, its key row and 4 columns
+  const int dhalf = (lane >> 4) & 1, s16 = lane & 15;
+  const uint8_t *vbase = (const uint8_t *)ldsV + dhalf * 512;
+  const int vlo = ((4 * hh + (s16 >> 2)) * 32 + 8 * (s16 & 3) + 128 * dhalf) & 511, vhi = (vlo + 256) & 511;
+  auto tr_read = [](const uint8_t *a) {
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)a);
+    return *(const u32x2 *)&v;
+  };
   constexpr float LOG2E = 1.4426950408889634f;
   const float scale2 = p.scale * LOG2E;
   sink_start(p, h, scale2, m_run, l_run);
@@ -299,24 +303,10 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
     for (int i = 0; i < DT; ++i) {
       const int c = tid + 256 * i, tr = c / (DT * 128), cc = c % (DT * 128);
       ((u32x4 *)ldsK)[c] = kreg[i];
-      // V: this lane holds 8 columns of one key; lane ^ 2 holds the same columns of the neighbouring key
-      const u32x4 v = vreg[i];
-      const int tile = cc >> 7, c7 = cc & 127;
-      const int face = c7 >> 5, row = (c7 & 31) >> 1, half = c7 & 1;
-      const bool odd = row & 1;
-      const int key = 32 * tr + (face >> 1) * 16 + (row & ~1);          // even key of the pair
-      const int d0 = tile * 32 + (face & 1) * 16 + half * 8 + (odd ? 4 : 0);
-      // the even lane keeps columns 0..3 and receives the odd lane's columns 0..3; the odd lane the other way round
-      const uint32_t send0 = odd ? v.x : v.z, send1 = odd ? v.y : v.w;
-      const uint32_t got0 = quad_xor2(send0), got1 = quad_xor2(send1);
-      const uint32_t mine0 = odd ? v.z : v.x, mine1 = odd ? v.w : v.y;
-      const uint32_t e0 = odd ? got0 : mine0, o0 = odd ? mine0 : got0;  // even key's word, odd key's word
-      const uint32_t e1 = odd ? got1 : mine1, o1 = odd ? mine1 : got1;
-      uint32_t *vt = (uint32_t *)(ldsV + d0 * VPITCH + key);
-      vt[0] = __builtin_amdgcn_perm(o0, e0, 0x05040100u);
-      vt[VPITCH / 2] = __builtin_amdgcn_perm(o0, e0, 0x07060302u);
-      vt[VPITCH] = __builtin_amdgcn_perm(o1, e1, 0x05040100u);
-      vt[3 * VPITCH / 2] = __builtin_amdgcn_perm(o1, e1, 0x07060302u);
+      // V as it lies in its tiles (rows are keys), the faces of the upper 16 columns rotated by four rows so that the
+      // transposing reads below touch every bank once
+      const int c7 = cc & 127, face = c7 >> 5;
+      *(u32x4 *)((uint8_t *)ldsV + (c - c7) * 16 + face * 512 + (((c7 & 31) * 16 + 128 * (face & 1)) & 511)) = vreg[i];
     }
     __syncthreads();
     if (kb + 1 < kb_end) load_block(kb + 1);
@@ -418,8 +408,11 @@ __device__ __forceinline__ void sdpa64_query_block(const SdpaArgs &p, int qb, in
       pb.w = pack_bf16_rne(s[t8 + 6], s[t8 + 7]);
 #pragma unroll
       for (int d = 0; d < DT; ++d) {
-        const uint16_t *vr = ldsV + (d * 32 + l31) * VPITCH + 16 * t + 4 * hh;
-        u32x2 lo = *(const u32x2 *)vr, hi = *(const u32x2 *)(vr + 8);
+        // V^T fragment: column d * 32 + l31, keys 16 t + 4 hh .. + 3 and eight further on, by two transposing LDS reads
+        // (ds_read_b64_tr_b16: of the 16 lanes of a group, lane 4 u + c receives element c of the rows that lanes
+        // u, u + 4, u + 8, u + 12 address; lane u + 4 j addresses key j of the four, columns 4 u .. + 3)
+        const uint8_t *vb = vbase + (t >> 1) * DT * 2048 + d * 2048 + (t & 1) * 1024;
+        const u32x2 lo = tr_read(vb + vlo), hi = tr_read(vb + vhi);
         u32x4 va = {lo.x, lo.y, hi.x, hi.y};
         o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va, *(bf16x8 *)&pb, o[d], 0, 0, 0);
       }
@@ -467,7 +460,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // SIMD, so that one's softmax overlaps the other's matrix products; staging K and V is shared by twice as many lanes.
 template <int DT>  // head_dim / 32
 __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *ldsK, uint16_t *ldsV) {
-  constexpr int VPITCH = kSdpaVPitch, NT = 512, CHUNKS = DT * 256, NCH = (CHUNKS + NT - 1) / NT;
+  constexpr int NT = 512, CHUNKS = DT * 256, NCH = (CHUNKS + NT - 1) / NT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int qw = wave & 3, kh = wave >> 2;
   const int hk = h / (p.Hq / p.Hkv);
