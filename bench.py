@@ -43,7 +43,7 @@ def _wall_time(torch, fn, steps):
 
 
 def sample_sclk(torch, fn, seconds=1.2):
-    """Shader clock reported by rocm-smi while `fn` is launched back to back for `seconds`: (median MHz, samples).  The
+    """Shader clock reported by the driver while `fn` is launched back to back for `seconds`: (median MHz, samples).  The
     matrix kernels run against the board's power limit, so the clock they are given is part of the measurement."""
     import re
     import statistics
@@ -51,16 +51,28 @@ def sample_sclk(torch, fn, seconds=1.2):
     import threading
     vals, stop = [], [False]
 
+    # the driver's own file first (no child process: a profiler's preloaded library initialises the GPU in every process it
+    # is loaded into, rocm-smi's interpreter included); rocm-smi only where that file is missing
+    import glob
+    dpm = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+    preloaded = "rocprof" in os.environ.get("LD_PRELOAD", "")
+
     def poll():
         while not stop[0]:
             try:
-                out = subprocess.run(["rocm-smi", "--showclocks", "--json"], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL,
-                                     text=True, timeout=5).stdout
-                card = next(iter(json.loads(out).values()))
-                for key, value in card.items():
-                    m = re.search(r"(\d+)\s*Mhz", str(value))
-                    if "sclk clock speed" in key and m:
-                        vals.append(int(m.group(1)))
+                if dpm:
+                    for line in open(dpm[0]).read().splitlines():
+                        m = re.search(r"(\d+)\s*Mhz\s*\*", line)
+                        if m:
+                            vals.append(int(m.group(1)))
+                elif not preloaded:
+                    out = subprocess.run(["rocm-smi", "--showclocks", "--json"], stdout=subprocess.PIPE, stderr=subprocess.DEVNULL,
+                                         text=True, timeout=5).stdout
+                    card = next(iter(json.loads(out).values()))
+                    for key, value in card.items():
+                        m = re.search(r"(\d+)\s*Mhz", str(value))
+                        if "sclk clock speed" in key and m:
+                            vals.append(int(m.group(1)))
             except Exception:
                 pass
             time.sleep(0.1)
@@ -322,13 +334,33 @@ def make_workloads(torch, hip, datagen, dev, names):
 
 # HBM bytes per launch of each workload's kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE) scaled by
 # what the same counters read for the plain copy kernel of known size (factors 1.9998 and 0.9996); these are measured
-# constants of the committed kernels, not computed here.  linear2048 is a two-pass launch: 184.2 MB for the pass that
-# writes the weights as bf16 fragment images plus 447.5 MB for the matrix pass (every XCD's L2 fetches the activations
-# and its share of the images again).
+# constants of the committed kernels, not computed here.  linear2048 is a two-pass launch: 183.8 MB for the pass that
+# writes the weights as bf16 fragment images plus 447.9 MB for the matrix pass (every XCD's L2 fetches the activations
+# and its share of the images again).  Each figure belongs to one version of a kernel source file: it is reported only
+# while that file still has the content it was measured on (first 12 hex digits of its SHA-1), else `traffic` is null.
 MEASURED_TRAFFIC_BYTES = {
-    "linear2048": 631.7e6, "linear32": 65.7e6, "pack_bfp8": 341.4e6, "unpack_bfp8": 340.1e6, "pack_bfp4": 308.1e6,
-    "unpack_bfp4": 306.5e6, "tilize_f32": 537.0e6, "untilize_f32": 537.0e6, "copy": 536.9e6, "sdpa_decode32": 270.4e6,
+    "linear2048": (631.7e6, "ttm_linear.hip"), "linear32": (65.7e6, "ttm_linear.hip"), "pack_bfp8": (341.4e6, "ttm_bfp.hip"),
+    "unpack_bfp8": (340.1e6, "ttm_bfp.hip"), "pack_bfp4": (308.1e6, "ttm_bfp.hip"), "unpack_bfp4": (306.5e6, "ttm_bfp.hip"),
+    "tilize_f32": (537.3e6, "ttm_layout.hip"), "untilize_f32": (537.0e6, "ttm_layout.hip"), "copy": (536.9e6, "ttm_layout.hip"),
+    "sdpa_decode32": (270.4e6, "ttm_decode.hip"), "rmsnorm2048": (34.0e6, "ttm_rowwise.hip"),
+    "softmax65536": (1073.7e6, "ttm_rowwise.hip"), "reduce65536": (545.3e6, "ttm_rowwise.hip"), "silu_mul512": (44.2e6, "ttm_eltwise.hip"),
 }
+MEASURED_ON = {"ttm_linear.hip": "8321dea48ec6", "ttm_bfp.hip": "5e8fe919a01c", "ttm_layout.hip": "61b650bd867c",
+               "ttm_decode.hip": "b17531f29ce4", "ttm_rowwise.hip": "42ca9deff5b2", "ttm_eltwise.hip": "e63e9d74edc6"}
+
+
+def measured_traffic(name):
+    import hashlib
+    entry_ = MEASURED_TRAFFIC_BYTES.get(name)
+    if entry_ is None:
+        return None
+    nbytes, source = entry_
+    try:
+        with open(os.path.join(ROOT, "tt-mlir_amd", "csrc", source), "rb") as f:
+            digest = hashlib.sha1(f.read()).hexdigest()[:12]
+    except OSError:
+        return None
+    return nbytes if digest == MEASURED_ON.get(source) else None
 
 
 def roofline(w, kernel_ms):
@@ -339,7 +371,7 @@ def roofline(w, kernel_ms):
         achieved = w.work / (kernel_ms * 1e-3) / 1e12
         peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
     r = {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-         "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC_BYTES.get(w.name), "kernel_us": round(kernel_ms * 1e3, 2),
+         "frac": round(achieved / peak, 4), "traffic": measured_traffic(w.name), "kernel_us": round(kernel_ms * 1e3, 2),
          "algorithmic_work": w.work, "work_unit": w.unit_work}
     if "dense_flop" in w.extra:   # attention: the dense count beside the FLOPs of the visible pairs that `frac` is made of
         dense = w.extra["dense_flop"] / (kernel_ms * 1e-3) / 1e12
@@ -491,7 +523,7 @@ def main():
                 "sclk_mhz_library_gemm": lclk, "loop_ms_library_gemm": round(lloop, 5),
                 "zero_operands": {"sclk_mhz_this_kernel": zclk, "loop_ms_this_kernel": round(zloop, 5),
                                   "sclk_mhz_library_gemm": zlclk, "loop_ms_library_gemm": round(zlloop, 5)},
-                "what": "rocm-smi shader clock while the launch is repeated back to back for 1.2 s, and the same with all-zero "
+                "what": "shader clock (the driver's pp_dpm_sclk) while the launch is repeated back to back for 1.2 s, and the same with all-zero "
                         "operands; loop_ms includes launch gaps"}
         del xa, xw
     if not args.no_cpu_baseline:
