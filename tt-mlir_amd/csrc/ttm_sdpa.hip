@@ -544,7 +544,7 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&ka, qf[st], s, 0, 0, 0);
     }
     const bool edge = key_base + 31 > qt * 32 + p.hi_off || key_base < q_last - p.lo_off || key_base + 32 > p.Sk;   // wavefront-uniform
-    float mx = -INFINITY;
+    float mx = -INFINITY, mul = 1.0f;
     if (p.mask || edge) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -569,12 +569,11 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
           mx = fmaxf(mx, v);
         }
       }
-    } else {
+    } else {   // plain block: the scale (positive) is folded into the exponent's multiply-add, the maximum is taken first
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        s[r] *= scale2;
-        mx = fmaxf(mx, s[r]);
-      }
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[r]);
+      mx *= scale2;
+      mul = scale2;
     }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const float m_new = fmaxf(m_run, mx);
@@ -583,7 +582,7 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
     float rs = 0.0f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float e = __builtin_amdgcn_exp2f(s[r] - m_use);
+      const float e = __builtin_amdgcn_exp2f(fmaf(s[r], mul, -m_use));
       s[r] = e;
       rs += e;
     }
