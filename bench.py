@@ -293,14 +293,19 @@ def make_workloads(torch, hip, datagen, dev, names):
         wbytes += (ffn // 32) * (hidden // 32) * 576
         nbytes = wbytes + 2 * users * n_kv * (pos + 1) * hd * 2
 
+        # a step is one submit; steps follow each other on the device's stream as the layers of a model would (each reads the
+        # caches the previous one wrote), and the timed region ends with a device-wide wait.  `latency` is one submit
+        # followed by a wait of its own
         def run(binary=binary, rins=rins, rdev=rdev, main=main):
-            outs = rt.submit(rdev, binary, main, rins)
-            rt.wait(outs)
+            rt.submit(rdev, binary, main, rins)
+
+        def run_and_wait(binary=binary, rins=rins, rdev=rdev, main=main):
+            rt.wait(rt.submit(rdev, binary, main, rins))
 
         out[nm] = Workload(nm, "hbm", nbytes, "bytes", run,
                            "Llama-3-8B decoder layer, one token for 32 users at position 2047 (weights bfp8_b / bfp4_b, bf16 KV cache "
                            "updated in place), one submit" + (" replaying a captured HIP graph" if nm.endswith("traced") else ""),
-                           dict(sync=True, steps=50, keep=(rdev, rins, binary)))
+                           dict(sync=True, steps=50, latency=run_and_wait, keep=(rdev, rins, binary)))
     for nm in ("mlp512", "decoder2048"):
         if nm not in names:
             continue
@@ -323,12 +328,16 @@ def make_workloads(torch, hip, datagen, dev, names):
         del d, tins
 
         def run(binary=binary, rins=rins, rdev=rdev):
+            for o in rt.submit(rdev, binary, 1, rins):
+                rt.deallocate_tensor(o, force=True)      # back to the stream-ordered pool; the next step may reuse it
+
+        def run_and_wait(binary=binary, rins=rins, rdev=rdev):
             outs = rt.submit(rdev, binary, 1, rins)
             rt.wait(outs)
             for o in outs:
                 rt.deallocate_tensor(o, force=True)
 
-        out[nm] = Workload(nm, "mfma", flop, "flop", run, desc, dict(sync=True, keep=(rdev, rins, binary)))
+        out[nm] = Workload(nm, "mfma", flop, "flop", run, desc, dict(sync=True, latency=run_and_wait, keep=(rdev, rins, binary)))
     return out
 
 
@@ -463,7 +472,7 @@ def main():
         for _ in range(warmup):
             w.fn()
         ms = _wall_time(torch, w.fn, steps)                    # timed region: exactly `steps` launches
-        if w.extra.get("sync"):                                # whole programs run on the runtime's own stream and sync inside
+        if w.extra.get("sync"):                                # whole programs run on the runtime's own stream: wall time of the steps
             return ms, ms
         kms = _events_time(hip, stream, w.fn, steps)           # HIP events on the launch stream
         return ms, kms
@@ -481,7 +490,10 @@ def main():
         heavy = bool(w.extra.get("sync"))
         sms, skms = measure(w, w.extra.get("steps", 5) if heavy else max(10, args.steps // 2), 2 if heavy else max(3, args.warmup // 2))
         r = roofline(w, skms)
-        secondary.append({"workload": n, "desc": w.desc, "ms_per_step": round(sms, 5), "roofline": r})
+        entry_ = {"workload": n, "desc": w.desc, "ms_per_step": round(sms, 5), "roofline": r}
+        if "latency" in w.extra:   # one step with a wait of its own (launch and wake-up latencies included)
+            entry_["latency_ms"] = round(_wall_time(torch, w.extra["latency"], 10), 5)
+        secondary.append(entry_)
 
     result = {
         "metric": metric, "value": round(value, 3), "unit": unit, "n_gpus": 1, "steps": args.steps,
