@@ -490,6 +490,18 @@ def main():
         heavy = bool(w.extra.get("sync"))
         sms, skms = measure(w, w.extra.get("steps", 5) if heavy else max(10, args.steps // 2), 2 if heavy else max(3, args.warmup // 2))
         r = roofline(w, skms)
+        if w.bound == "hbm" and not heavy and w.work < 200e6:
+            # small tensors: a launch of a few microseconds is mostly ramp; the plain copy kernel moving the same number of
+            # bytes (half read, half written) is the ceiling to hold the figure against
+            half = int(w.work // 2) // 16 * 16
+            cx = torch.empty(half, dtype=torch.uint8, device=dev)
+            cy = torch.empty_like(cx)
+            cfn = lambda cx=cx, cy=cy, half=half: hip.call("ttm_copy_kernel", hip.ptr(cx), hip.ptr(cy), half, stream)
+            for _ in range(20):
+                cfn()
+            cms = _events_time(hip, stream, cfn, 50)
+            r["copy_of_same_bytes"] = {"kernel_us": round(cms * 1e3, 2), "achieved": round(2 * half / (cms * 1e-3) / 1e9, 2), "unit": "GB/s"}
+            del cx, cy
         entry_ = {"workload": n, "desc": w.desc, "ms_per_step": round(sms, 5), "roofline": r}
         if "latency" in w.extra:   # one step with a wait of its own (launch and wake-up latencies included)
             entry_["latency_ms"] = round(_wall_time(torch, w.extra["latency"], 10), 5)
