@@ -349,12 +349,12 @@ def make_workloads(torch, hip, datagen, dev, names):
 # while that file still has the content it was measured on (first 12 hex digits of its SHA-1), else `traffic` is null.
 MEASURED_TRAFFIC_BYTES = {
     "linear2048": (631.7e6, "ttm_linear.hip"), "linear32": (65.7e6, "ttm_linear.hip"), "pack_bfp8": (341.4e6, "ttm_bfp.hip"),
-    "unpack_bfp8": (340.1e6, "ttm_bfp.hip"), "pack_bfp4": (308.1e6, "ttm_bfp.hip"), "unpack_bfp4": (306.5e6, "ttm_bfp.hip"),
+    "unpack_bfp8": (340.1e6, "ttm_bfp.hip"), "pack_bfp4": (306.2e6, "ttm_bfp.hip"), "unpack_bfp4": (306.5e6, "ttm_bfp.hip"),
     "tilize_f32": (537.3e6, "ttm_layout.hip"), "untilize_f32": (537.0e6, "ttm_layout.hip"), "copy": (536.9e6, "ttm_layout.hip"),
     "sdpa_decode32": (270.4e6, "ttm_decode.hip"), "rmsnorm2048": (34.0e6, "ttm_rowwise.hip"),
     "softmax65536": (1073.7e6, "ttm_rowwise.hip"), "reduce65536": (545.3e6, "ttm_rowwise.hip"), "silu_mul512": (44.2e6, "ttm_eltwise.hip"),
 }
-MEASURED_ON = {"ttm_linear.hip": "8321dea48ec6", "ttm_bfp.hip": "5e8fe919a01c", "ttm_layout.hip": "61b650bd867c",
+MEASURED_ON = {"ttm_linear.hip": "8321dea48ec6", "ttm_bfp.hip": "1cd3aa4c76d7", "ttm_layout.hip": "61b650bd867c",
                "ttm_decode.hip": "b17531f29ce4", "ttm_rowwise.hip": "42ca9deff5b2", "ttm_eltwise.hip": "e63e9d74edc6"}
 
 
