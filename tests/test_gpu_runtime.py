@@ -702,6 +702,9 @@ def test_traced_program_replays_as_a_graph(device, orc):
         # unrelated work between replays allocates and frees device memory; the trace's buffers must stay its own
         harness.execute(other, 1, [od["x"], od["norm_w"], bf(od["wg"]), bf(od["wu"]), bf(od["wd"])], device)
     assert (rt.get_stat("TraceCacheMiss"), rt.get_stat("CapturedTrace"), rt.get_stat("ExecutedTrace")) == (1, 1, 4)
+    # the traced function's closing copy into the output slot is folded into the last projection (once in the eager run of
+    # the capture program, once while recording)
+    assert rt.get_stat("FusedCopyIntoSlot") == 2
     # a parameter replaced by the caller (new tensor, new version) is copied into its slot before the replay
     res_t2, res_e2 = resident(traced, main, 2.0), resident(eager, 1, 2.0)
     x = torch.randn((T, H), generator=g).to(torch.bfloat16)
@@ -819,6 +822,7 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
         rt.clear_callbacks()
         if mode == "traced":
             assert rt.get_stat("CapturedTrace") >= 1
+        assert rt.get_stat("FusedCopyIntoSlot") == (2 if mode == "traced" else 0)
         # the Q, K and V projections, both rotary embeddings, the head splits and both cache writes are one fused step (two
         # launches); nothing of this with a callback registered (a traced program runs its body op by op only until the graph
         # is recorded); the head merge behind the attention is folded into the attention kernel

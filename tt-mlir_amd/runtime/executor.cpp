@@ -339,6 +339,40 @@ std::uint32_t soleConsumer(ProgramContext &ctx, std::uint32_t id, std::uint32_t 
   return 0;
 }
 
+// A traced function ends by copying each result into the trace's output slot
+// (lib/Dialect/TTNN/Transforms/TTNNTraceHoistTransform.cpp:452).  When the `copy` that is the only reader of tensor
+// `produced` follows op `from` with nothing but deallocations of other tensors between, and its destination is a live
+// device tensor of the same shape in the plain bf16 tile layout whose buffer is none of `operands`, the producer can write
+// into the destination and the copy be skipped: returns the destination and the copy's index, or an empty tensor.
+Tensor copyDestinationOf(ProgramContext &ctx, std::uint32_t from, const fb::Table &produced, const std::vector<const Tensor *> &operands,
+                         std::uint32_t *copyIndex) {
+  if (!ctx.fuseViews || !decodeFusionEnabled()) return Tensor();
+  const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
+  if (!(layoutFromTensorRef(produced) == plain)) return Tensor();
+  const std::uint32_t id = refId(produced);
+  auto u = ctx.uses.find(id);
+  if (u == ctx.uses.end() || u->second != 1) return Tensor();
+  std::vector<std::uint32_t> freed;
+  std::uint32_t j = from + 1;
+  auto typeOf = [&](std::uint32_t i) { return static_cast<OpType>(ctx.ops[i].scalar<std::uint8_t>(schema::Operation::f_type_type, 0)); };
+  for (; j < ctx.ops.size() && typeOf(j) == OpType::DeallocateOp; ++j)
+    freed.push_back(refId(ctx.ops[j].table(schema::Operation::f_type).table(schema::DeallocateOp::f_in)));
+  if (j >= ctx.ops.size() || typeOf(j) != OpType::CopyOp || ctx.skip.count(j)) return Tensor();
+  fb::Table cop = ctx.ops[j].table(schema::Operation::f_type);
+  fb::Table src = cop.table(schema::CopyOp::f_src), dst = cop.table(schema::CopyOp::f_dst);
+  if (!src || !dst || refId(src) != id || refId(dst) == id) return Tensor();
+  if (std::find(freed.begin(), freed.end(), id) != freed.end() || std::find(freed.begin(), freed.end(), refId(dst)) != freed.end())
+    return Tensor();
+  auto it = ctx.pool.find(refId(dst));
+  if (it == ctx.pool.end() || !isTensorAllocated(it->second) || !(getTensorLayout(it->second) == plain) ||
+      it->second.handle->shape != shapeFromTensorRef(produced))
+    return Tensor();
+  for (const Tensor *t : operands)
+    if (t && t->handle && t->handle->data.get() == it->second.handle->data.get()) return Tensor();
+  *copyIndex = j;
+  return it->second;
+}
+
 // The front of a decode step's attention block: three projections of the same <= 32 tokens (block-float weights) whose
 // results go, each through its own chain of single-consumer ops, to
 //   q: reshape [1, users, heads, D] -> rotary_embedding(token_index)                       -> whoever reads q
@@ -654,6 +688,13 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
         return;
       }
     }
+  }
+  // the last projection of a traced function writes straight into the trace's output slot
+  std::uint32_t copyIndex = 0;
+  if (Tensor slot = copyDestinationOf(ctx, tailOp == TTM_TAIL_NONE ? ctx.opIndex : nextIdx, finalRef, {&a, &b, &bias, &tail}, &copyIndex)) {
+    out = slot;
+    ctx.skip.insert(copyIndex);
+    debug::Stats::get().incrementStat("FusedCopyIntoSlot");
   }
   TTM_CALL(ttm_linear_tail(a.handle->data.get(), TTM_BF16, b.handle->data.get(), ttmDtype(b.handle->dtype), transposeB ? 1 : 0, biasPtr,
                            TTM_BF16, biasLayout, out.handle->data.get(), TTM_BF16, batch, wbatch == 1 ? 1 : batch, M, N, K,
