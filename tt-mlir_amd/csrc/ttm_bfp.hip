@@ -128,8 +128,10 @@ __device__ __forceinline__ u32x4 decode_chunk(const uint32_t (&in)[2], int E) {
 // ------------------------------------------------------------------------------------ strip kernels
 // ELEM = bytes per plain element (4: fp32, 2: bf16).  A tile is CPT = 64*ELEM chunks; a face row is
 // ELEM chunks.  The workgroup handles 1024 chunks = 16/ELEM tiles.
+// Packing bfp8_b from row-major fp32 gains from four workgroups per CU (8192 x 8192: 53.2 -> 50.9 us); every other
+// combination is fastest without a cap.
 template <int W, int ELEM, bool ROWMAJOR, bool PACK>
-__global__ __launch_bounds__(256) void ttm_bfp_strip_k(const void *__restrict__ src_, void *__restrict__ dst_,
+__global__ __launch_bounds__(256) TTM_MAX_WAVES((PACK && ROWMAJOR && W == 7 && ELEM == 4) ? 4 : 8) void ttm_bfp_strip_k(const void *__restrict__ src_, void *__restrict__ dst_,
                                                        int64_t xt, int64_t strips_per_row) {
   constexpr int EPT = 16 / ELEM;
   constexpr int CPT = 64 * ELEM;

@@ -32,6 +32,11 @@ int ttm_set_error(int code, const char *fmt, ...) __attribute__((format(printf, 
 
 int ttm_option(const char *name);  // 0 when unset
 
+// Streaming kernels run fastest with a bounded number of bytes in flight per CU (64 - 96 KiB measured on MI355X): more
+// resident wavefronts than that only lengthen the queues in front of the memory channels.  TTM_MAX_WAVES(n) caps a
+// kernel's wavefronts per SIMD (= 256-lane workgroups per CU) at n; n may depend on template parameters, 8 is no cap.
+#define TTM_MAX_WAVES(n) __attribute__((amdgpu_waves_per_eu((n) < 8 ? (n) : 1, (n))))
+
 // Scratch memory of a stream for kernels that need device memory beyond their operands (split-K partial sums).
 // One grow-only allocation per (device, stream): launches on a stream are ordered, so consecutive users do not overlap.
 // Growing allocates with hipMalloc and is refused while the stream is capturing; an allocation that a captured graph may

@@ -421,8 +421,18 @@ __global__ __launch_bounds__(256) void ttm_rowwise_row_k(RowArgs p, int total_ro
 #ifndef TTM_BAND_EXP
 #define TTM_BAND_EXP expf
 #endif
+// Workgroups per CU by mode and band size (NK x 4 KiB per workgroup), measured at 65536 rows: reductions 4 at 16 KiB
+// (44 -> 40 us for 1024 fp32 columns) and 3 from 32 KiB up (89 -> 82 us for 2048); fp32 softmax 4 at 16 KiB (94 -> 88 us)
+// and 2 from 32 KiB up (195 -> 185 us); RMSNorm 3 at 16 KiB (96 -> 90 us); everything else runs best without a cap.
 template <int MODE, int ELEM, int NK>
-__global__ __launch_bounds__(256) void ttm_rowwise_band_k(RowArgs p) {
+constexpr int band_max_waves() {
+  if (MODE == RW_SUM || MODE == RW_MEAN || MODE == RW_MAX || MODE == RW_MIN) return NK == 4 ? 4 : (NK >= 8 ? 3 : 8);
+  if (MODE == RW_SOFTMAX && ELEM == 4) return NK == 4 ? 4 : (NK >= 8 ? 2 : 8);
+  if (MODE == RW_RMSNORM) return NK == 4 ? 3 : 8;
+  return 8;
+}
+template <int MODE, int ELEM, int NK>
+__global__ __launch_bounds__(256) TTM_MAX_WAVES((band_max_waves<MODE, ELEM, NK>())) void ttm_rowwise_band_k(RowArgs p) {
   constexpr int EPC = 16 / ELEM, RUN = 4 * ELEM;         // chunks per run of four face rows
   constexpr bool IS_MAX = MODE == RW_SOFTMAX || MODE == RW_MAX;
   constexpr bool REDUCE = MODE == RW_SUM || MODE == RW_MEAN || MODE == RW_MAX || MODE == RW_MIN;
