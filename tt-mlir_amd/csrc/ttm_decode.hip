@@ -341,13 +341,15 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
       qf[c] = *(bf16x8 *)&z;
     }
     const int hrow = hk * p.Gt + p.g0;  // mask rows of this block's heads
-    for (int g0 = wave; g0 < ngroups; g0 += 8) {
-      // two groups of 16 keys per pass, all their loads issued before the first product
-      u32x4 kf[2][8];
-      int grp[2];
-      bool kok[2];
+    constexpr int KU = 1;
+    for (int g0 = wave; g0 < ngroups; g0 += 4 * KU) {
+      // KU groups of 16 keys per wavefront and pass, all their loads issued before the first product (one group: 8 KiB per
+      // wavefront in flight; two measured 1.5 % slower, three and four slower still)
+      u32x4 kf[KU][8];
+      int grp[KU];
+      bool kok[KU];
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < KU; ++u) {
         grp[u] = g0 + 4 * u < ngroups ? g0 + 4 * u : g0;   // the tail repeats a valid group and skips its result
         const int key = k0 + grp[u] * 16 + (lane & 15);     // this lane's key column of the B operand
         const uint16_t *kt = kv_tile_row(p.k, p, b, hk, key >> 5, kok[u]);
@@ -358,7 +360,7 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
           if (c < DT) kf[u][c] = kv_load<STREAM>((const u32x4 *)(kt + (int64_t)c * 1024 + in_tile));
       }
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
+      for (int u = 0; u < KU; ++u) {
         if (u == 1 && g0 + 4 >= ngroups) break;
         f32x4v acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll

@@ -458,18 +458,23 @@ __global__ __launch_bounds__(256) TTM_MAX_WAVES((band_max_waves<MODE, ELEM, NK>(
     const int run = min(run_of(k), nruns - 1);
     v[k] = __builtin_nontemporal_load((const u32x4 *)(x + off_of(run) * ELEM));
   }
-  u32x4 wraw[MODE == RW_RMSNORM ? NK : 1], braw[MODE == RW_RMSNORM ? NK : 1];
-  if constexpr (MODE == RW_RMSNORM) {
+  // RMSNorm: the weight and bias chunks of this lane's columns.  Up to eight chunks per lane they are loaded up front, beside
+  // the input; with sixteen that would take every register of a SIMD for a single wavefront (measured 3.2 TB/s at 8192 bf16
+  // columns), so there they are loaded four chunks at a time where they are used (they come from the L2: every row shares them)
+  constexpr bool WB_EARLY = MODE == RW_RMSNORM && NK <= 8;
+  auto wb_load = [&](int k, u32x4 &wv, u32x4 &bv) {
+    const int c0 = col_of(min(run_of(k), nruns - 1));
+    const int64_t tiled = (int64_t)(c0 >> 5) * 1024 + ((c0 >> 4) & 1) * 256 + (c0 & 15);
+    // a null vector reads the input instead (the value is not used): no branch around the loads
+    const uint8_t *wsrc = p.w ? (const uint8_t *)p.w + (p.w_tiled ? tiled : c0) * ELEM : x;
+    const uint8_t *bsrc = p.b ? (const uint8_t *)p.b + (p.b_tiled ? tiled : c0) * ELEM : x;
+    wv = *(const u32x4 *)wsrc;
+    bv = *(const u32x4 *)bsrc;
+  };
+  u32x4 wraw[WB_EARLY ? NK : 1], braw[WB_EARLY ? NK : 1];
+  if constexpr (WB_EARLY) {
 #pragma unroll
-    for (int k = 0; k < NK; ++k) {
-      const int c0 = col_of(min(run_of(k), nruns - 1));
-      const int64_t tiled = (int64_t)(c0 >> 5) * 1024 + ((c0 >> 4) & 1) * 256 + (c0 & 15);
-      // a null vector reads the input instead (the value is not used): no branch around the loads
-      const uint8_t *wsrc = p.w ? (const uint8_t *)p.w + (p.w_tiled ? tiled : c0) * ELEM : x;
-      const uint8_t *bsrc = p.b ? (const uint8_t *)p.b + (p.b_tiled ? tiled : c0) * ELEM : x;
-      wraw[k] = *(const u32x4 *)wsrc;
-      braw[k] = *(const u32x4 *)bsrc;
-    }
+    for (int k = 0; k < NK; ++k) wb_load(k, wraw[k], braw[k]);
   }
   // the lanes of a wavefront that share a row differ in the chunk-part bits (below ELEM) and the run bits (RUN and up)
   auto wave_combine = [&](float a, bool is_max, bool is_min) {
@@ -542,17 +547,29 @@ __global__ __launch_bounds__(256) TTM_MAX_WAVES((band_max_waves<MODE, ELEM, NK>(
       __syncthreads();
       mul = 1.0f / ((red2[0][rl] + red2[1][rl]) + (red2[2][rl] + red2[3][rl]));
     }
+    u32x4 wlate[4], blate[4];
 #pragma unroll
     for (int k = 0; k < NK; ++k) {
+      if constexpr (MODE == RW_RMSNORM && !WB_EARLY) {
+        if (k % 4 == 0) {
+          __builtin_amdgcn_sched_barrier(0);   // the loads of one batch only: the scheduler would hoist all sixteen
+#pragma unroll
+          for (int u = 0; u < 4; ++u) wb_load(min(k + u, NK - 1), wlate[u], blate[u]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
       const int run = run_of(k);
       if (run < nruns) {
         const int c0 = col_of(run);
         float f[EPC];
         if constexpr (MODE == RW_RMSNORM) {
           float w[EPC], b[EPC];
+          // bf16: unpacked again from the raw chunk; without the empty asm the compiler keeps the floats of the first pass
+          // alive across the barrier, twice the registers of the raw chunks
+          if constexpr (ELEM == 2 && NK >= 16) asm volatile("" : "+v"(v[k]));
           unpack_vals<ELEM>(v[k], f);
-          if (p.w) unpack_vals<ELEM>(wraw[k], w);
-          if (p.b) unpack_vals<ELEM>(braw[k], b);
+          if (p.w) unpack_vals<ELEM>(WB_EARLY ? wraw[WB_EARLY ? k : 0] : wlate[k % 4], w);
+          if (p.b) unpack_vals<ELEM>(WB_EARLY ? braw[WB_EARLY ? k : 0] : blate[k % 4], b);
 #pragma unroll
           for (int i = 0; i < EPC; ++i) {
             float y = f[i] * mul;
