@@ -134,7 +134,7 @@ def rowwise_variant(request, hip):
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
 @pytest.mark.parametrize("shape,wl,bias", [((512, 4096), "tile", False), ((64, 96), "tile", True), ((3, 40, 70), "rm", True),
                                            ((1, 33), "tile", False), ((2, 2, 32, 256), "rm", False), ((2048, 1024), "tile", True),
-                                           ((40, 8192), "rm", False)])
+                                           ((40, 8192), "rm", False), ((64, 16384), "tile", True), ((33, 6000), "rm", True)])
 def test_rms_norm(hip, dev, orc, dtype, shape, wl, bias, rowwise_variant):
     tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
     x = datagen.randn(shape, seed=5, dtype=tdt)
@@ -165,7 +165,7 @@ def test_rms_norm(hip, dev, orc, dtype, shape, wl, bias, rowwise_variant):
 
 
 @pytest.mark.parametrize("dtype", ["bf16", "f32"])
-@pytest.mark.parametrize("shape", [(64, 96), (2, 3, 40, 70), (1, 2048), (32, 2048), (1100, 300), (3, 33, 4100)])
+@pytest.mark.parametrize("shape", [(64, 96), (2, 3, 40, 70), (1, 2048), (32, 2048), (1100, 300), (3, 33, 4100), (64, 8192), (33, 12000)])
 def test_softmax_and_reduce_lastdim(hip, dev, orc, dtype, shape, rowwise_variant):
     tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
     hdt = hip.BF16 if dtype == "bf16" else hip.F32

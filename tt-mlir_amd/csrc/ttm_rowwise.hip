@@ -431,12 +431,15 @@ constexpr int band_max_waves() {
   if (MODE == RW_RMSNORM) return NK == 4 ? 3 : 8;
   return 8;
 }
-template <int MODE, int ELEM, int NK>
-__global__ __launch_bounds__(256) TTM_MAX_WAVES((band_max_waves<MODE, ELEM, NK>())) void ttm_rowwise_band_k(RowArgs p) {
+// NT = 512 lanes take bands of up to 32 chunks per 256 lanes (16384 bf16 or 8192 fp32 columns) with sixteen chunks per lane:
+// one such workgroup per CU (128 KiB).
+template <int MODE, int ELEM, int NK, int NT = 256>
+__global__ __launch_bounds__(NT) TTM_MAX_WAVES((NT == 512 ? 2 : band_max_waves<MODE, ELEM, NK>())) void ttm_rowwise_band_k(RowArgs p) {
   constexpr int EPC = 16 / ELEM, RUN = 4 * ELEM;         // chunks per run of four face rows
   constexpr bool IS_MAX = MODE == RW_SOFTMAX || MODE == RW_MAX;
   constexpr bool REDUCE = MODE == RW_SUM || MODE == RW_MEAN || MODE == RW_MAX || MODE == RW_MIN;
-  __shared__ float red[4][4], red2[4][4];
+  constexpr int NW = NT / 64;
+  __shared__ float red[NW][4], red2[NW][4];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int g4 = (int)(blockIdx.x & 7);                  // group of four rows inside the tile row
   const int64_t trow = blockIdx.x >> 3;                  // tile row over all batch entries
@@ -446,8 +449,8 @@ __global__ __launch_bounds__(256) TTM_MAX_WAVES((band_max_waves<MODE, ELEM, NK>(
   const bool row_ok = row < p.rows;
   const int nruns = p.ct * 2, cols = (int)p.cols;        // runs per band: one per (tile, face column)
   const uint8_t *x = (const uint8_t *)p.x + trow * p.ct * 1024 * ELEM;
-  // chunk k of this lane: run tid / RUN + k * (256 / RUN)
-  auto run_of = [&](int k) { return tid / RUN + k * (256 / RUN); };
+  // chunk k of this lane: run tid / RUN + k * (NT / RUN)
+  auto run_of = [&](int k) { return tid / RUN + k * (NT / RUN); };
   auto off_of = [&](int run) { return (int64_t)(run >> 1) * 1024 + ((r >> 4) * 2 + (run & 1)) * 256 + (r & 15) * 16 + part * EPC; };
   auto col_of = [&](int run) { return (run >> 1) * 32 + (run & 1) * 16 + part * EPC; };
   u32x4 v[NK];
@@ -508,8 +511,15 @@ __global__ __launch_bounds__(256) TTM_MAX_WAVES((band_max_waves<MODE, ELEM, NK>(
   __syncthreads();
   float stat;
   {
-    const float a0 = red[0][rl], a1 = red[1][rl], a2 = red[2][rl], a3 = red[3][rl];
-    stat = IS_MAX ? fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)) : (MODE == RW_MIN ? fminf(fminf(a0, a1), fminf(a2, a3)) : (a0 + a1) + (a2 + a3));
+    auto four = [&](int w0) {
+      const float a0 = red[w0][rl], a1 = red[w0 + 1][rl], a2 = red[w0 + 2][rl], a3 = red[w0 + 3][rl];
+      return IS_MAX ? fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)) : (MODE == RW_MIN ? fminf(fminf(a0, a1), fminf(a2, a3)) : (a0 + a1) + (a2 + a3));
+    };
+    stat = four(0);
+    if constexpr (NW == 8) {
+      const float hi = four(4);
+      stat = IS_MAX ? fmaxf(stat, hi) : (MODE == RW_MIN ? fminf(stat, hi) : stat + hi);
+    }
   }
   if constexpr (REDUCE) {
     // output [.., rows, 1] in tile order: one column tile per tile row; this workgroup owns its four rows of it, both faces
@@ -545,7 +555,9 @@ __global__ __launch_bounds__(256) TTM_MAX_WAVES((band_max_waves<MODE, ELEM, NK>(
       sum = wave_combine(sum, false, false);
       if ((lane & ~(RUN - ELEM)) == 0) red2[wave][rl] = sum;
       __syncthreads();
-      mul = 1.0f / ((red2[0][rl] + red2[1][rl]) + (red2[2][rl] + red2[3][rl]));
+      float den = (red2[0][rl] + red2[1][rl]) + (red2[2][rl] + red2[3][rl]);
+      if constexpr (NW == 8) den += (red2[4][rl] + red2[5][rl]) + (red2[6][rl] + red2[7][rl]);
+      mul = 1.0f / den;
     }
     u32x4 wlate[4], blate[4];
 #pragma unroll
@@ -603,6 +615,14 @@ static int launch_rowwise(const RowArgs &p, int dtype, int64_t trows, hipStream_
     // chunks per lane (16384 bf16 or 8192 fp32 columns).  rowwise_variant: 2 forces it, 1 and 3 exclude it.
     const int elem = dtype == TTM_BF16 ? 2 : 4, variant = ttm_option("rowwise_variant");
     const int nk = (int)ttm_cdiv((int64_t)p.ct * 2 * 4 * elem, 256);
+    if (nk > 16 && nk <= 32 && trows * 8 < (1ll << 31) && (variant == 2 || (variant == 0 && trows * 8 >= 256))) {
+      // twice the lanes for bands of 17 - 32 chunks per 256 lanes
+      const dim3 grid((unsigned)(trows * 8)), block(512);
+      if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_band_k<MODE, 2, 16, 512>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((ttm_rowwise_band_k<MODE, 4, 16, 512>), grid, block, 0, s, p);
+      TTM_LAUNCH_CHECK();
+      return TTM_OK;
+    }
     if (nk <= 16 && trows * 8 < (1ll << 31) && (variant == 2 || (variant == 0 && trows * 8 >= 256))) {
       const dim3 grid((unsigned)(trows * 8)), block(256);
 #define TTM_BAND_LAUNCH(E, N) hipLaunchKernelGGL((ttm_rowwise_band_k<MODE, E, N>), grid, block, 0, s, p)
