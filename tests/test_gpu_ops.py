@@ -51,10 +51,14 @@ def test_unary(hip, dev, orc, dtype):
 @pytest.mark.parametrize("layout", ["tile", "row_major"])
 @pytest.mark.parametrize("ashape,bshape", [((64, 96), (64, 96)), ((2, 3, 40, 50), (2, 3, 40, 50)), ((64, 96), (1, 96)),
                                            ((2, 64, 96), (64, 1)), ((2, 1, 33, 70), (1, 3, 1, 70)), ((4, 32, 32), (1,)),
-                                           ((1, 128), (5, 128, 1))])
-def test_binary_broadcast(hip, dev, orc, layout, ashape, bshape):
-    a = datagen.randn(ashape, seed=2, dtype=torch.bfloat16)
-    b = datagen.randn(bshape, seed=3, dtype=torch.bfloat16) + 3.0
+                                           ((1, 128), (5, 128, 1)), ((2, 40, 64), (1, 64)), ((3, 70, 96), (3, 1, 96)),
+                                           ((2, 2, 33, 128), (2, 1, 33, 1))])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_binary_broadcast(hip, dev, orc, layout, ashape, bshape, dtype):
+    """Same-shape, row-vector, column-vector, scalar and batch broadcasting in both layouts and dtypes: the flat kernel, the
+    16-byte-chunk kernel (rows of whole chunks, ragged row counts included) and the element-wise one (ragged columns)."""
+    a = datagen.randn(ashape, seed=2, dtype=dtype)
+    b = datagen.randn(bshape, seed=3, dtype=dtype) + 3.0
     oshape = tuple(np.broadcast_shapes(ashape, bshape))
     rank = len(oshape)
     pad = lambda s: np.array((1,) * (rank - len(s)) + tuple(s), dtype=np.int64)
@@ -64,17 +68,19 @@ def test_binary_broadcast(hip, dev, orc, layout, ashape, bshape):
         if tiled:
             ad, bd = tilize_dev(hip, r2(a), dev), tilize_dev(hip, r2(b), dev)
             Rp, Cp = (oshape[-2] + 31) // 32 * 32, (oshape[-1] + 31) // 32 * 32
-            od = torch.empty(int(np.prod(oshape[:-2], dtype=np.int64)) * Rp * Cp, dtype=torch.bfloat16, device=dev)
+            od = torch.full((int(np.prod(oshape[:-2], dtype=np.int64)) * Rp * Cp,), float("nan"), dtype=dtype, device=dev)
         else:
             ad, bd = a.to(dev), b.to(dev)
-            od = torch.empty(oshape, dtype=torch.bfloat16, device=dev)
+            od = torch.empty(oshape, dtype=dtype, device=dev)
         sa, sb, so = pad(ashape), pad(bshape), pad(oshape)          # keep the shape arrays alive over the call
         hip.call("ttm_eltwise_binary", orc.BINARY[name], hip.ptr(ad), sa.ctypes.data, hip.ptr(bd),
-                 sb.ctypes.data, hip.ptr(od), so.ctypes.data, rank, hip.BF16,
+                 sb.ctypes.data, hip.ptr(od), so.ctypes.data, rank, hip.BF16 if dtype == torch.bfloat16 else hip.F32,
                  hip.TILE if tiled else hip.ROW_MAJOR, hip.current_stream())
         res = untilize_dev(hip, od, oshape, dev) if tiled else od
         torch.cuda.synchronize()
-        want = orc.round_bf16(orc.binary(name, a.float().numpy(), b.float().numpy()))
+        want = orc.binary(name, a.float().numpy(), b.float().numpy())
+        if dtype == torch.bfloat16:
+            want = orc.round_bf16(want)
         assert np.array_equal(res.float().cpu().numpy(), want), name   # one rounding of an exact f32 op: bit exact
         if tiled:  # padding of the tiled result is zero
             full = od.float().cpu().numpy()
@@ -485,7 +491,8 @@ def _i64(v):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("tiled", [False, True])
 @pytest.mark.parametrize("cs,as_,bs", [((3, 40, 70), (3, 40, 70), (3, 40, 70)), ((1, 40, 1), (3, 40, 70), (1, 1, 70)),
-                                       ((2, 3, 1, 33), (1, 3, 35, 33), (1,)), ((64, 64), (64, 64), (1, 1))])
+                                       ((2, 3, 1, 33), (1, 3, 35, 33), (1,)), ((64, 64), (64, 64), (1, 1)),
+                                       ((2, 40, 64), (1, 1, 64), (2, 40, 1)), ((3, 64, 96), (3, 64, 96), (3, 64, 96))])
 def test_where_bit_exact(hip, dev, orc, dtype, tiled, cs, as_, bs):
     """ttm_where against the oracle: same-shape and broadcasting operands (condition, either value, a scalar), ragged
     tiles whose padding must stay zero, both layouts and dtypes; NaN and -0.0 in the condition; the values move as bits."""

@@ -4,6 +4,7 @@
 // 16 bytes per lane; broadcasting binaries decode tile coordinates per element.
 #include <hip/hip_fp16.h>
 
+#include <initializer_list>
 #include <type_traits>
 
 #include "ttm_common.h"
@@ -290,6 +291,97 @@ __global__ __launch_bounds__(256) void ttm_binary_bcast_k(int op, const void *__
   }
 }
 
+// Broadcasting in 16-byte chunks, for outputs whose chunks never straddle a row: tile layout with a multiple of 32 columns,
+// row-major with a multiple of the chunk width.  A chunk is EPC consecutive columns of one row (inside a tile: part of one
+// face row), so per chunk one (row, first column) is decoded and every operand is read either as the 16 bytes at its own
+// offset for that position (its last dim is the output's) or as one element for the whole chunk (its last dim is 1).
+// grid.y numbers the batch entries; rows past R (tile padding) are written as zeros.
+struct ChunkPos {
+  int64_t i0, i1, r, c0, out_chunk;
+  bool live;
+};
+template <int EPC>
+__device__ __forceinline__ ChunkPos chunk_pos(const int64_t (&oshape)[4], int tiled, uint32_t ci, uint32_t chunks_per_plane) {
+  const uint32_t R = (uint32_t)oshape[2], C = (uint32_t)oshape[3];
+  ChunkPos q;
+  const uint32_t batch = blockIdx.y;
+  q.i0 = batch / (uint32_t)oshape[1]; q.i1 = batch % (uint32_t)oshape[1];
+  uint32_t r, c0;
+  if (tiled) {
+    const uint32_t w = ci * EPC, tile = w >> 10, e = w & 1023, face = e >> 8, tcols = C >> 5;
+    r = (tile / tcols) * 32 + (face >> 1) * 16 + ((e >> 4) & 15);
+    c0 = (tile % tcols) * 32 + (face & 1) * 16 + (e & 15);
+  } else {
+    const uint32_t cpr = C / EPC;
+    r = ci / cpr; c0 = (ci % cpr) * EPC;
+  }
+  q.r = r; q.c0 = c0;
+  q.live = r < R;
+  q.out_chunk = (int64_t)batch * chunks_per_plane + ci;
+  return q;
+}
+template <bool BF16, typename F>
+__device__ __forceinline__ void operand_chunk(const void *base, const int64_t (&shape)[4], const ChunkPos &q, int tiled, F (&v)[BF16 ? 8 : 4]) {
+  constexpr int EPC = BF16 ? 8 : 4;
+  const int64_t off = bcast_offset(shape, q.i0, q.i1, q.r, q.c0, tiled);
+  if (shape[3] != 1) {
+    const u32x4 raw = *(const u32x4 *)((const uint8_t *)base + off * (BF16 ? 2 : 4));
+    if constexpr (std::is_same<F, float>::value) {
+      if (BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { v[2 * i] = __uint_as_float(raw[i] << 16); v[2 * i + 1] = __uint_as_float(raw[i] & 0xFFFF0000u); }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(raw[i]);
+      }
+    } else {   // raw bits, one element per entry
+      if (BF16) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { v[2 * i] = raw[i] & 0xFFFFu; v[2 * i + 1] = raw[i] >> 16; }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = raw[i];
+      }
+    }
+  } else {
+    F one;
+    if constexpr (std::is_same<F, float>::value) one = BF16 ? ttm_bf16_to_f32(((const uint16_t *)base)[off]) : ((const float *)base)[off];
+    else one = BF16 ? (F)((const uint16_t *)base)[off] : (F)((const uint32_t *)base)[off];
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) v[i] = one;
+  }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void ttm_binary_chunk_k(int op, const void *__restrict__ a, const void *__restrict__ b,
+                                                          void *__restrict__ out, BcastArgs p, uint32_t chunks_per_plane) {
+  constexpr int EPC = BF16 ? 8 : 4;
+  for (uint32_t ci = blockIdx.x * 256 + threadIdx.x; ci < chunks_per_plane; ci += gridDim.x * 256) {
+    const ChunkPos q = chunk_pos<EPC>(p.oshape, p.tiled, ci, chunks_per_plane);
+    float x[EPC], y[EPC];
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) x[i] = 0.0f;
+    if (q.live) {
+      operand_chunk<BF16>(a, p.ashape, q, p.tiled, x);
+      operand_chunk<BF16>(b, p.bshape, q, p.tiled, y);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) x[i] = binary_op(op, x[i], y[i]);
+    }
+    chunk_store<BF16>(out, q.out_chunk, x);
+  }
+}
+
+// whether the chunked kernels apply: chunks inside rows, everything 16-byte aligned, plane and batch counts within 32 bits
+static bool chunkable(const int64_t (&oshape)[4], int tiled, int es, std::initializer_list<const void *> ptrs) {
+  const int64_t R = oshape[2], C = oshape[3], epc = 16 / es;
+  if (tiled ? (C % 32 != 0) : (C % epc != 0)) return false;
+  const int64_t pr = tiled ? ttm_round_up32(R) : R;
+  if (pr * C >= ((int64_t)1 << 31) || oshape[0] * oshape[1] > 65535 || oshape[0] * oshape[1] < 1) return false;
+  for (const void *q : ptrs)
+    if (((uintptr_t)q & 15) != 0) return false;
+  return true;
+}
+
 TTM_EXPORT int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape,
                                   void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream) {
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_eltwise_binary: dtype must be BFloat16 or Float32 (got %d)", dtype);
@@ -336,6 +428,11 @@ TTM_EXPORT int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape,
       hipLaunchKernelGGL(ttm_binary_flat_k<true>, dim3(grid_for(nchunks)), dim3(256), 0, s, op, a, b, out, nchunks);
     else
       hipLaunchKernelGGL(ttm_binary_flat_k<false>, dim3(grid_for(nchunks)), dim3(256), 0, s, op, a, b, out, nchunks);
+  } else if (chunkable(p.oshape, p.tiled, es, {a, b, out})) {
+    const uint32_t cpp = (uint32_t)(pr * pc * es / 16);
+    const dim3 grid(grid_for(cpp), (unsigned)(p.oshape[0] * p.oshape[1]));
+    if (dtype == TTM_BF16) hipLaunchKernelGGL(ttm_binary_chunk_k<true>, grid, dim3(256), 0, s, op, a, b, out, p, cpp);
+    else hipLaunchKernelGGL(ttm_binary_chunk_k<false>, grid, dim3(256), 0, s, op, a, b, out, p, cpp);
   } else {
     if (dtype == TTM_BF16)
       hipLaunchKernelGGL(ttm_binary_bcast_k<true>, dim3(grid_for(total)), dim3(256), 0, s, op, a, b, out, p, total);
@@ -380,6 +477,34 @@ __global__ __launch_bounds__(256) void ttm_where_k(const void *__restrict__ cond
   }
 }
 
+template <bool BF16>
+__global__ __launch_bounds__(256) void ttm_where_chunk_k(const void *__restrict__ cond, const void *__restrict__ a, const void *__restrict__ b,
+                                                         void *__restrict__ out, WhereArgs p, uint32_t chunks_per_plane) {
+  constexpr int EPC = BF16 ? 8 : 4;
+  for (uint32_t ci = blockIdx.x * 256 + threadIdx.x; ci < chunks_per_plane; ci += gridDim.x * 256) {
+    const ChunkPos q = chunk_pos<EPC>(p.oshape, p.tiled, ci, chunks_per_plane);
+    uint32_t cv[EPC], av[EPC], bv[EPC];
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) av[i] = 0u;
+    if (q.live) {
+      operand_chunk<BF16>(cond, p.cshape, q, p.tiled, cv);
+      operand_chunk<BF16>(a, p.ashape, q, p.tiled, av);
+      operand_chunk<BF16>(b, p.bshape, q, p.tiled, bv);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) av[i] = (cv[i] & (BF16 ? 0x7FFFu : 0x7FFFFFFFu)) != 0 ? av[i] : bv[i];   // +-0 is false, NaN is true
+    }
+    u32x4 o;
+    if (BF16) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = av[2 * i] | (av[2 * i + 1] << 16);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) o[i] = av[i];
+    }
+    ((u32x4 *)out)[q.out_chunk] = o;
+  }
+}
+
 TTM_EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a, const int64_t *a_shape, const void *b,
                          const int64_t *b_shape, void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream) {
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_where: dtype must be BFloat16 or Float32 (got %d)", dtype);
@@ -403,6 +528,15 @@ TTM_EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void
   const int64_t total = p.oshape[0] * p.oshape[1] * pr * pc;
   if (total == 0) return TTM_OK;
   TTM_REQUIRE(cond && a && b && out, "ttm_where: null pointer");
+  const int es = dtype == TTM_BF16 ? 2 : 4;
+  if (chunkable(p.oshape, p.tiled, es, {cond, a, b, out})) {
+    const uint32_t cpp = (uint32_t)(pr * pc * es / 16);
+    const dim3 grid(grid_for(cpp), (unsigned)(p.oshape[0] * p.oshape[1]));
+    if (dtype == TTM_BF16) hipLaunchKernelGGL(ttm_where_chunk_k<true>, grid, dim3(256), 0, (hipStream_t)stream, cond, a, b, out, p, cpp);
+    else hipLaunchKernelGGL(ttm_where_chunk_k<false>, grid, dim3(256), 0, (hipStream_t)stream, cond, a, b, out, p, cpp);
+    TTM_LAUNCH_CHECK();
+    return TTM_OK;
+  }
   if (dtype == TTM_BF16)
     hipLaunchKernelGGL(ttm_where_k<true>, dim3(grid_for(total)), dim3(256), 0, (hipStream_t)stream, cond, a, b, out, p, total);
   else
@@ -445,6 +579,23 @@ __global__ __launch_bounds__(256) void ttm_typecast_k(const void *__restrict__ i
   }
 }
 
+// bf16 <-> fp32 in groups of four elements per lane: 8 bytes of bf16 against 16 of fp32, every instruction of a wavefront
+// touching one contiguous run (the element-wise kernel above moves 2 + 4 bytes per lane and reaches half the bandwidth)
+template <bool WIDEN>
+__global__ __launch_bounds__(256) void ttm_typecast4_k(const void *__restrict__ in, void *__restrict__ out, int64_t groups) {
+  for (int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x; g < groups; g += (int64_t)gridDim.x * 256) {
+    if (WIDEN) {
+      const u32x2 v = __builtin_nontemporal_load((const u32x2 *)in + g);
+      const u32x4 w = {v.x << 16, v.x & 0xFFFF0000u, v.y << 16, v.y & 0xFFFF0000u};
+      __builtin_nontemporal_store(w, (u32x4 *)out + g);
+    } else {
+      const u32x4 w = __builtin_nontemporal_load((const u32x4 *)in + g);
+      const u32x2 v = {ttm_pack_bf16x2(__uint_as_float(w.x), __uint_as_float(w.y)), ttm_pack_bf16x2(__uint_as_float(w.z), __uint_as_float(w.w))};
+      __builtin_nontemporal_store(v, (u32x2 *)out + g);
+    }
+  }
+}
+
 typedef void (*cast_fn)(const void *, void *, int64_t);
 template <int SRC>
 static cast_fn pick_cast_dst(int dst) {
@@ -476,6 +627,13 @@ TTM_EXPORT int ttm_typecast(const void *in, int src_dtype, void *out, int dst_dt
   if (!fn) return ttm_set_error(TTM_ERR_UNSUPPORTED, "ttm_typecast: unsupported conversion %d -> %d", src_dtype, dst_dtype);
   if (n == 0) return TTM_OK;
   TTM_REQUIRE(in && out, "ttm_typecast: null pointer");
+  const bool widen = src_dtype == TTM_BF16 && dst_dtype == TTM_F32, narrow = src_dtype == TTM_F32 && dst_dtype == TTM_BF16;
+  if ((widen || narrow) && n % 4 == 0 && (((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
+    if (widen) hipLaunchKernelGGL(ttm_typecast4_k<true>, dim3(grid_for(n / 4)), dim3(256), 0, (hipStream_t)stream, in, out, n / 4);
+    else hipLaunchKernelGGL(ttm_typecast4_k<false>, dim3(grid_for(n / 4)), dim3(256), 0, (hipStream_t)stream, in, out, n / 4);
+    TTM_LAUNCH_CHECK();
+    return TTM_OK;
+  }
   hipLaunchKernelGGL(fn, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, in, out, n);
   TTM_LAUNCH_CHECK();
   return TTM_OK;
