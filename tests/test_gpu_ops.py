@@ -202,6 +202,24 @@ def test_softmax_and_reduce_lastdim(hip, dev, orc, dtype, shape, rowwise_variant
         assert np.all(np.isfinite(o.float().cpu().numpy()))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(64, 96), (3, 128, 32), (2, 2, 32, 160), (1024, 2048)])
+@pytest.mark.parametrize("dst_order", [False, True])
+def test_tile_transpose_of_whole_tiles(hip, dev, dtype, shape, dst_order):
+    """The transpose of the last two dims between tile-order tensors of whole tiles (the dedicated kernel): the view written
+    in destination order, as the runtime does, and in source order; batched; against torch.transpose."""
+    x = datagen.randn(shape, seed=12, dtype=dtype)
+    xt = tilize_dev(hip, x, dev)
+    tshape = tuple(shape[:-2]) + (shape[-1], shape[-2])
+    xs, ts = strides(shape), strides(tshape)
+    if dst_order:   # view dims run over the destination's shape; the source is read with swapped strides
+        out = view_copy(hip, dev, xt, shape, True, tshape, True, tshape, xs[:-2] + [xs[-1], xs[-2]], ts)
+    else:           # view dims run over the source's shape; the destination is written with swapped strides
+        out = view_copy(hip, dev, xt, shape, True, tshape, True, shape, xs, ts[:-2] + [ts[-1], ts[-2]])
+    torch.cuda.synchronize()
+    assert torch.equal(untilize_dev(hip, out, tshape, dev).cpu(), x.transpose(-1, -2).contiguous())
+
+
 def view_copy(hip, dev, src, src_shape, src_tiled, dst_shape, dst_tiled, extent, sstride, dstride, sbase=0, dbase=0,
               dst=None):
     r2 = lambda s: (1,) * (2 - len(s)) + tuple(s) if len(s) < 2 else tuple(s)

@@ -60,8 +60,12 @@ __global__ __launch_bounds__(256) void ttm_copy_view_k(const T *__restrict__ src
 }
 
 // 16 bytes per lane: the innermost view dimension is contiguous on both sides and everything that positions a
-// group of V = 16 / elem_bytes elements is a multiple of V, so a group never leaves its row or its 16-wide face row
-template <int ELEM, typename I>
+// group of V = 16 / elem_bytes elements is a multiple of V, so a group never leaves its row or its 16-wide face row.
+// DPHYS: the destination is a tile-order tensor that the view covers densely in row-major order (reshape, permute, slice
+// results).  Lanes then take the destination's 16-byte chunks in the order they lie in memory and find their view index
+// from the chunk's position, so that a wavefront's stores are whole lines; in view order consecutive lanes would write
+// one 32- or 64-byte face row each into a different line.  Chunks in the padding of the destination are left alone.
+template <int ELEM, typename I, bool DPHYS>
 __global__ __launch_bounds__(256) void ttm_copy_view_vec_k(const u32x4 *__restrict__ src, u32x4 *__restrict__ dst, ViewArgs p,
                                                            int64_t total) {
   constexpr int V = 16 / ELEM;
@@ -69,6 +73,17 @@ __global__ __launch_bounds__(256) void ttm_copy_view_vec_k(const u32x4 *__restri
   if (!view_position(p, dbase)) return;
   for (int64_t i0 = (int64_t)blockIdx.x * 256 + threadIdx.x; i0 < total; i0 += (int64_t)gridDim.x * 256) {
     I rem = (I)i0, ls = (I)p.sbase, ld = (I)dbase;
+    I dchunk = 0;
+    if constexpr (DPHYS) {
+      // chunk i0 of the destination's memory -> (matrix, row, first column) -> logical index = view index
+      const I ph = (I)i0 * V, tile = ph >> 10, e = ph & 1023, face = e >> 8;
+      const I ptc = ((I)p.dcols + 31) / 32, prt = ((I)p.drows + 31) / 32;
+      const I m = tile / (prt * ptc), tin = tile - m * (prt * ptc), tr = tin / ptc, tc = tin - tr * ptc;
+      const I row = tr * 32 + (face >> 1) * 16 + ((e >> 4) & 15), col = tc * 32 + (face & 1) * 16 + (e & 15);
+      if (row >= (I)p.drows || col >= (I)p.dcols) continue;
+      rem = ((m * (I)p.drows + row) * (I)p.dcols + col) / V;
+      dchunk = (I)i0;
+    }
     {
       const I e = (I)p.extent[p.rank - 1] / V;
       const I q = rem / e, v = rem - q * e;
@@ -84,19 +99,94 @@ __global__ __launch_bounds__(256) void ttm_copy_view_vec_k(const u32x4 *__restri
       ls += v * (I)p.sstride[d];
       ld += v * (I)p.dstride[d];
     }
-    dst[phys_offset<I>(ld, (I)p.drows, (I)p.dcols, p.dtiled) / V] = src[phys_offset<I>(ls, (I)p.srows, (I)p.scols, p.stiled) / V];
+    if constexpr (!DPHYS) dchunk = phys_offset<I>(ld, (I)p.drows, (I)p.dcols, p.dtiled) / V;
+    dst[dchunk] = src[phys_offset<I>(ls, (I)p.srows, (I)p.scols, p.stiled) / V];
   }
 }
 
+// Transpose of the last two dims between tile-order tensors whose extents are multiples of 32: tile (i, j) of the source is
+// tile (j, i) of the destination with its 32 x 32 elements transposed, so every access is a whole tile (2 or 4 KiB
+// contiguous).  One wavefront per tile: every load and store instruction of the wavefront covers 1 KiB contiguous (lane l
+// takes 16-byte chunk 64 i + l of the tile), the elements cross through the wavefront's own 32 x 33-word area of LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void ttm_transpose_tiles_k(const T *__restrict__ src, T *__restrict__ dst, int64_t tiles, int rt, int ct) {
+  __shared__ uint32_t lds[4][32 * 33];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t = (int64_t)blockIdx.x * 4 + wave;
+  if (t >= tiles) return;   // wavefront-uniform; no barrier below
+  const int64_t per = (int64_t)rt * ct, b = t / per, rem = t - b * per;
+  const int tr = (int)(rem / ct), tc = (int)(rem - (int64_t)tr * ct);
+  const u32x4 *sp = (const u32x4 *)(src + (b * per + (int64_t)tr * ct + tc) * 1024);
+  u32x4 *dp = (u32x4 *)(dst + (b * per + (int64_t)tc * rt + tr) * 1024);
+  constexpr int V = 16 / sizeof(T), NCH = 1024 / V / 64;   // elements per chunk, chunks per lane
+  uint32_t *w = lds[wave];
+  u32x4 q[NCH];
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) q[i] = __builtin_nontemporal_load(sp + i * 64 + lane);
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int e0 = (i * 64 + lane) * V, f = e0 >> 8, r = (e0 >> 4) & 15, c0 = e0 & 15;
+    uint32_t *row = w + (16 * (f >> 1) + r) * 33 + 16 * (f & 1) + c0;
+#pragma unroll
+    for (int j = 0; j < V; ++j) row[j] = sizeof(T) == 2 ? (q[i][j / 2] >> (16 * (j & 1))) & 0xFFFFu : q[i][j];
+  }
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    // chunk of the transposed tile: face (fr, fc), row r, columns c0 .. c0 + V - 1 = source elements (16 fc + c0 + j, 16 fr + r)
+    const int e0 = (i * 64 + lane) * V, f = e0 >> 8, r = (e0 >> 4) & 15, c0 = e0 & 15;
+    const uint32_t *col = w + (16 * (f & 1) + c0) * 33 + 16 * (f >> 1) + r;
+    uint32_t e[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) e[j] = col[j * 33];
+    u32x4 o;
+    if (sizeof(T) == 2) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = e[2 * j] | (e[2 * j + 1] << 16);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o[j] = e[j];
+    }
+    __builtin_nontemporal_store(o, dp + i * 64 + lane);
+  }
+}
+
+// whether a view is the transpose of the last two dims of a dense tile-order tensor (either way of writing it: view dims
+// in source order with a transposed destination, or in destination order with a transposed source); *batches = the rest
+static bool is_tile_transpose(const ViewArgs &p, int elem_bytes, int64_t *batches) {
+  if (p.rank < 2 || !p.stiled || !p.dtiled || p.index || (elem_bytes != 2 && elem_bytes != 4) || p.sbase != 0 || p.dbase != 0) return false;
+  const int64_t R = p.srows, C = p.scols;
+  if (R % 32 != 0 || C % 32 != 0 || p.drows != C || p.dcols != R) return false;
+  const int a = p.rank - 2, b = p.rank - 1;
+  const bool src_order = p.extent[a] == R && p.extent[b] == C && p.sstride[a] == C && p.sstride[b] == 1 && p.dstride[a] == 1 && p.dstride[b] == R;
+  const bool dst_order = p.extent[a] == C && p.extent[b] == R && p.sstride[a] == 1 && p.sstride[b] == C && p.dstride[a] == R && p.dstride[b] == 1;
+  if (!src_order && !dst_order) return false;
+  int64_t n = 1;   // the leading dims must number the matrices densely and alike on both sides
+  for (int d = p.rank - 3; d >= 0; --d) {
+    if (p.extent[d] != 1 && (p.sstride[d] != n * R * C || p.dstride[d] != n * R * C)) return false;
+    n *= p.extent[d];
+  }
+  *batches = n;
+  return true;
+}
+
 template <typename I>
-static void launch_copy_view(const void *src, void *dst, const ViewArgs &p, int elem_bytes, bool vec, int64_t total, hipStream_t s) {
+static void launch_copy_view(const void *src, void *dst, const ViewArgs &p, int elem_bytes, bool vec, int64_t dphys_chunks, int64_t total,
+                             hipStream_t s) {
+  if (vec && dphys_chunks > 0) {   // in the order of the destination's memory: every chunk of it, padding included
+    int64_t vblocks = ttm_cdiv(dphys_chunks, 256);
+    unsigned vgrid = (unsigned)(vblocks > 262144 ? 262144 : vblocks);
+    if (elem_bytes == 4) hipLaunchKernelGGL((ttm_copy_view_vec_k<4, I, true>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, dphys_chunks);
+    else if (elem_bytes == 2) hipLaunchKernelGGL((ttm_copy_view_vec_k<2, I, true>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, dphys_chunks);
+    else hipLaunchKernelGGL((ttm_copy_view_vec_k<1, I, true>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, dphys_chunks);
+    return;
+  }
   if (vec) {
     const int64_t groups = total / (16 / elem_bytes);
     int64_t vblocks = ttm_cdiv(groups, 256);
     unsigned vgrid = (unsigned)(vblocks > 262144 ? 262144 : vblocks);
-    if (elem_bytes == 4) hipLaunchKernelGGL((ttm_copy_view_vec_k<4, I>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
-    else if (elem_bytes == 2) hipLaunchKernelGGL((ttm_copy_view_vec_k<2, I>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
-    else hipLaunchKernelGGL((ttm_copy_view_vec_k<1, I>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
+    if (elem_bytes == 4) hipLaunchKernelGGL((ttm_copy_view_vec_k<4, I, false>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
+    else if (elem_bytes == 2) hipLaunchKernelGGL((ttm_copy_view_vec_k<2, I, false>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
+    else hipLaunchKernelGGL((ttm_copy_view_vec_k<1, I, false>), dim3(vgrid), dim3(256), 0, s, (const u32x4 *)src, (u32x4 *)dst, p, groups);
     return;
   }
   int64_t blocks = ttm_cdiv(total, 256);
@@ -130,6 +220,16 @@ static int copy_view_entry(const void *src, int64_t src_rows, int64_t src_cols, 
   p.index = index; p.istride = index_stride; p.ilimit = index_limit;
   if (index) TTM_REQUIRE(index_stride >= 0 && index_limit >= 1, "ttm_copy_view_at: index stride must be >= 0 and the limit >= 1");
   hipStream_t s = (hipStream_t)stream;
+  int64_t matrices = 0;
+  if (is_tile_transpose(p, elem_bytes, &matrices) && ((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0 &&
+      matrices * (src_rows / 32) * (src_cols / 32) < ((int64_t)1 << 32)) {
+    const int rt = (int)(src_rows / 32), ct = (int)(src_cols / 32);
+    const int64_t tiles = matrices * rt * ct;
+    if (elem_bytes == 2) hipLaunchKernelGGL(ttm_transpose_tiles_k<uint16_t>, dim3((unsigned)ttm_cdiv(tiles, 4)), dim3(256), 0, s, (const uint16_t *)src, (uint16_t *)dst, tiles, rt, ct);
+    else hipLaunchKernelGGL(ttm_transpose_tiles_k<uint32_t>, dim3((unsigned)ttm_cdiv(tiles, 4)), dim3(256), 0, s, (const uint32_t *)src, (uint32_t *)dst, tiles, rt, ct);
+    TTM_LAUNCH_CHECK();
+    return TTM_OK;
+  }
   const int64_t V = 16 / elem_bytes;
   bool vec = rank >= 1 && src_stride[rank - 1] == 1 && dst_stride[rank - 1] == 1 && extent[rank - 1] % V == 0 &&
              src_base % V == 0 && dst_base % V == 0 && src_cols % V == 0 && dst_cols % V == 0 &&
@@ -153,8 +253,20 @@ static int copy_view_entry(const void *src, int64_t src_rows, int64_t src_cols, 
     return batches * ttm_round_up32(rows) * ttm_round_up32(cols);
   };
   narrow = narrow && padded_reach(smax, src_rows, src_cols) < ((int64_t)1 << 31) && padded_reach(dmax, dst_rows, dst_cols) < ((int64_t)1 << 31);
-  if (narrow) launch_copy_view<uint32_t>(src, dst, p, elem_bytes, vec, total, s);
-  else launch_copy_view<int64_t>(src, dst, p, elem_bytes, vec, total, s);
+  // destination in tile order, covered densely and in row-major order by the view, from its first element on: the vector
+  // kernel may walk the destination's memory instead of the view
+  int64_t dphys_chunks = 0;
+  if (vec && p.dtiled && !index && dst_base == 0 && total % (dst_rows * dst_cols) == 0) {
+    bool dense = true;
+    int64_t acc = 1;
+    for (int d = rank - 1; d >= 0 && dense; --d) {
+      dense = extent[d] == 1 || dst_stride[d] == acc;
+      acc *= extent[d];
+    }
+    if (dense) dphys_chunks = total / (dst_rows * dst_cols) * ttm_round_up32(dst_rows) * ttm_round_up32(dst_cols) / V;
+  }
+  if (narrow) launch_copy_view<uint32_t>(src, dst, p, elem_bytes, vec, dphys_chunks, total, s);
+  else launch_copy_view<int64_t>(src, dst, p, elem_bytes, vec, dphys_chunks, total, s);
   TTM_LAUNCH_CHECK();
   return TTM_OK;
 }
