@@ -561,10 +561,11 @@ def test_embedding_bit_exact(hip, dev, orc, dtype, rows, vocab, dim, unsigned):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
-@pytest.mark.parametrize("rows,cols", [(32, 128256), (5, 63), (1, 1), (9, 64), (130, 1000)])
+@pytest.mark.parametrize("rows,cols", [(32, 128256), (5, 63), (1, 1), (9, 64), (130, 1000), (7, 50003), (600, 8192), (3, 8193)])
 def test_argmax_first_largest(hip, dev, orc, dtype, rows, cols):
-    """ttm_argmax against the oracle: a vocabulary-sized row, fewer columns than lanes, ties (bf16 rows of 128 256 random
-    values have many; the first index wins), a NaN (counts as largest), -inf rows."""
+    """ttm_argmax against the oracle: a vocabulary-sized row (the two-step kernel; rows of whole 16-byte groups and not),
+    fewer columns than lanes, ties (bf16 rows of 128 256 random values have many; the first index wins, also across the
+    slices of a row), NaNs (count as largest, the first one wins), -inf rows."""
     x = datagen.randn((rows, cols), seed=170, dtype=dtype)
     if cols > 40:
         x[0, 7] = x[0, 33] = 50.0
@@ -572,6 +573,13 @@ def test_argmax_first_largest(hip, dev, orc, dtype, rows, cols):
             x[1, 20] = float("nan")
         if rows > 2:
             x[2, :] = float("-inf")
+    if cols > 8000:   # the same maximum in the first and in the last slice; NaNs in two slices; a maximum in the last column
+        if rows > 3:
+            x[3, 100] = x[3, cols - 5] = 60.0
+        if rows > 4:
+            x[4, cols - 3] = x[4, 4000] = float("nan")
+        if rows > 5:
+            x[5, cols - 1] = 70.0
     xd = x.to(dev)
     out = torch.full((rows,), -1, dtype=torch.int32, device=dev)
     hip.call("ttm_argmax", hip.ptr(xd), hip.BF16 if dtype == torch.bfloat16 else hip.F32, hip.ptr(out), rows, cols, hip.current_stream())

@@ -49,6 +49,97 @@ __global__ __launch_bounds__(256) void ttm_argmax_k(const void *__restrict__ in,
   if (lane == 0) out[row] = (int32_t)(at == INT64_MAX ? 0 : at);
 }
 
+// Long rows (a vocabulary) in two steps: grid (parts, rows) workgroups each scan one slice of a row, 16 bytes per load where
+// the row starts allow it, and leave (value, index) of their first largest element; a second kernel merges the parts of a
+// row.  Candidates compare as in the one-wavefront kernel: NaN beats numbers, equal values go to the smaller index.
+struct ArgBest {
+  float v;
+  int32_t at;     // -1: nothing seen yet
+};
+__device__ __forceinline__ void arg_take(ArgBest &b, float x, int32_t c) {
+  const bool bnan = b.v != b.v, xnan = x != x;
+  if (b.at < 0 || (!bnan && (xnan || x > b.v))) { b.v = x; b.at = c; }   // strictly better: columns come in increasing order
+}
+__device__ __forceinline__ void arg_merge(ArgBest &b, float ov, int32_t oa) {
+  if (oa < 0) return;
+  const bool bnan = b.v != b.v, onan = ov != ov;
+  bool take;
+  if (b.at < 0) take = true;
+  else if (onan != bnan) take = onan;
+  else if (onan) take = oa < b.at;
+  else take = ov > b.v || (ov == b.v && oa < b.at);
+  if (take) { b.v = ov; b.at = oa; }
+}
+__device__ __forceinline__ void arg_wave_merge(ArgBest &b) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    const float ov = __shfl_xor(b.v, o);
+    const int32_t oa = __shfl_xor(b.at, o);
+    arg_merge(b, ov, oa);
+  }
+}
+
+template <bool BF16, bool VEC>
+__global__ __launch_bounds__(256) void ttm_argmax_part_k(const void *__restrict__ in, float *__restrict__ part_v, int32_t *__restrict__ part_at,
+                                                         int64_t cols, int64_t slice) {
+  __shared__ float sv[4];
+  __shared__ int32_t sa[4];
+  constexpr int V = BF16 ? 8 : 4;
+  const int64_t row = blockIdx.y, c0 = (int64_t)blockIdx.x * slice, c1 = min(c0 + slice, cols);
+  ArgBest b = {0.0f, -1};
+  if (VEC) {   // slice and row starts are multiples of V elements
+    const u32x4 *base = (const u32x4 *)((const uint8_t *)in + (row * cols + c0) * (BF16 ? 2 : 4));
+    const int64_t nv = (c1 - c0) / V;
+    for (int64_t g0 = threadIdx.x; g0 < nv; g0 += 1024) {   // four loads in flight per lane
+      u32x4 q[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) q[u] = __builtin_nontemporal_load(base + min(g0 + 256 * u, nv - 1));
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t g = g0 + 256 * u;
+        if (g < nv) {
+          const int32_t c = (int32_t)(c0 + g * V);
+#pragma unroll
+          for (int j = 0; j < V; ++j) {
+            const float x = BF16 ? __uint_as_float((j & 1) ? (q[u][j / 2] & 0xFFFF0000u) : (q[u][j / 2] << 16)) : __uint_as_float(q[u][j]);
+            arg_take(b, x, c + j);
+          }
+        }
+      }
+    }
+    for (int64_t c = c0 + nv * V + threadIdx.x; c < c1; c += 256) {   // the last, partial group of the row
+      const float x = BF16 ? __uint_as_float((uint32_t)((const uint16_t *)in)[row * cols + c] << 16) : ((const float *)in)[row * cols + c];
+      arg_merge(b, x, (int32_t)c);
+    }
+  } else {
+    for (int64_t c = c0 + threadIdx.x; c < c1; c += 256) {
+      const float x = BF16 ? __uint_as_float((uint32_t)((const uint16_t *)in)[row * cols + c] << 16) : ((const float *)in)[row * cols + c];
+      arg_take(b, x, (int32_t)c);
+    }
+  }
+  arg_wave_merge(b);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (lane == 0) { sv[wave] = b.v; sa[wave] = b.at; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) arg_merge(b, sv[w], sa[w]);
+    part_v[row * gridDim.x + blockIdx.x] = b.v;
+    part_at[row * gridDim.x + blockIdx.x] = b.at;
+  }
+}
+
+// one wavefront per row over its parts
+__global__ __launch_bounds__(256) void ttm_argmax_merge_k(const float *__restrict__ part_v, const int32_t *__restrict__ part_at, int32_t *__restrict__ out,
+                                                          int64_t rows, int parts) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  ArgBest b = {0.0f, -1};
+  for (int i = lane; i < parts; i += 64) arg_merge(b, part_v[row * parts + i], part_at[row * parts + i]);
+  arg_wave_merge(b);
+  if (lane == 0) out[row] = b.at < 0 ? 0 : b.at;
+}
+
 template <int DT>
 __global__ __launch_bounds__(256) void ttm_arange_k(void *__restrict__ out, int64_t n, double start, double step) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
@@ -98,6 +189,33 @@ TTM_EXPORT int ttm_argmax(const void *in, int dtype, int32_t *out, int64_t rows,
   if (rows == 0) return TTM_OK;
   TTM_REQUIRE(in && out, "ttm_argmax: null pointer");
   TTM_REQUIRE((rows + 3) / 4 <= 0x7FFFFFFF, "ttm_argmax: too many rows");
+  // rows too long for one wavefront each: slices of at least 2048 columns, enough of them for about 2048 workgroups
+  if (cols >= 8192 && rows <= 65535) {
+    const int es = dtype == TTM_BF16 ? 2 : 4, V = 16 / es;
+    int64_t parts = ttm_cdiv(2048, rows);
+    if (parts > cols / 2048) parts = cols / 2048;
+    if (parts < 1) parts = 1;
+    int64_t slice = ttm_cdiv(ttm_cdiv(cols, parts), V) * V;
+    parts = ttm_cdiv(cols, slice);
+    void *ws = nullptr;
+    if (int rc = ttm_stream_workspace((hipStream_t)stream, (size_t)(rows * parts) * 8, &ws)) return rc;
+    float *pv = (float *)ws;
+    int32_t *pa = (int32_t *)(pv + rows * parts);
+    const bool vec = ((uintptr_t)in & 15) == 0 && (cols * es) % 16 == 0;
+    const dim3 pgrid((unsigned)parts, (unsigned)rows);
+    hipStream_t s = (hipStream_t)stream;
+    if (dtype == TTM_BF16) {
+      if (vec) hipLaunchKernelGGL((ttm_argmax_part_k<true, true>), pgrid, dim3(256), 0, s, in, pv, pa, cols, slice);
+      else hipLaunchKernelGGL((ttm_argmax_part_k<true, false>), pgrid, dim3(256), 0, s, in, pv, pa, cols, slice);
+    } else {
+      if (vec) hipLaunchKernelGGL((ttm_argmax_part_k<false, true>), pgrid, dim3(256), 0, s, in, pv, pa, cols, slice);
+      else hipLaunchKernelGGL((ttm_argmax_part_k<false, false>), pgrid, dim3(256), 0, s, in, pv, pa, cols, slice);
+    }
+    TTM_LAUNCH_CHECK();
+    hipLaunchKernelGGL(ttm_argmax_merge_k, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, pv, pa, out, rows, (int)parts);
+    TTM_LAUNCH_CHECK();
+    return TTM_OK;
+  }
   const dim3 grid((unsigned)((rows + 3) / 4));
   if (dtype == TTM_BF16) hipLaunchKernelGGL(ttm_argmax_k<true>, grid, dim3(256), 0, (hipStream_t)stream, in, out, rows, cols);
   else hipLaunchKernelGGL(ttm_argmax_k<false>, grid, dim3(256), 0, (hipStream_t)stream, in, out, rows, cols);
