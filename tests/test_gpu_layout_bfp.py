@@ -51,16 +51,25 @@ def test_tilize_untilize_bit_exact(hip, dev, orc, shape, dtype, variant):
     assert np.array_equal(back.cpu().numpy().view(x.dtype).view(np.uint8), x.view(np.uint8))
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (5, 7), (33, 31), (3, 17, 40), (1, 100), (40, 4096)])
-def test_tilize_ragged_zero_padded(hip, dev, orc, shape):
-    x = np.random.default_rng(1).standard_normal(shape).astype(np.float32)
+@pytest.mark.parametrize("dtype", [np.float32, np.uint16, np.uint8])
+@pytest.mark.parametrize("shape", [(1, 1), (5, 7), (33, 31), (3, 17, 40), (1, 100), (40, 4096), (3, 500, 1000), (2, 70, 1002), (65, 33),
+                                   (2, 2, 31, 64)])
+def test_tilize_ragged_zero_padded(hip, dev, orc, shape, dtype):
+    """Shapes that are not multiples of 32 in 4-, 2- and 1-byte elements: rows whose row-major start is 16-byte aligned in
+    every row, in every other row, in none; batches; the padding of the tiles is zero, untilize leaves nothing outside the
+    row-major tensor (the buffer is longer than it and must keep its fill)."""
+    rng = np.random.default_rng(1)
+    x = rng.standard_normal(shape).astype(np.float32) if dtype == np.float32 else rng.integers(1, 250, shape).astype(dtype)
     t = run_tilize(hip, dev, x)
-    assert np.array_equal(t.cpu().numpy().view(np.uint32), orc.tilize(x).view(np.uint32))
-    back = torch.zeros(shape, dtype=torch.float32, device=dev)
+    assert np.array_equal(t.cpu().numpy().view(dtype), orc.tilize(x).view(dtype).reshape(-1))
+    n = int(np.prod(shape))
+    back = torch.full((n + 64,), 7, dtype=t.dtype, device=dev)
     b, r, c = orc._split3(shape)
-    hip.call("ttm_untilize", hip.ptr(t), hip.ptr(back), b, r, c, 4, hip.current_stream())
+    hip.call("ttm_untilize", hip.ptr(t), hip.ptr(back), b, r, c, x.dtype.itemsize, hip.current_stream())
     torch.cuda.synchronize()
-    assert np.array_equal(back.cpu().numpy(), x)
+    got = back.cpu().numpy().view(dtype)
+    assert np.array_equal(got[:n].reshape(shape), x)
+    assert np.all(got[n:] == np.asarray(7, dtype=back.cpu().numpy().dtype).view(dtype))
 
 
 def test_c1_operands_layout(hip, dev, orc):

@@ -160,6 +160,74 @@ __global__ __launch_bounds__(256) void ttm_tile_scalar_k(const T *__restrict__ s
   }
 }
 
+// ------------------------------------------------------------------------------------ ragged shapes, 16 bytes at a time
+// Rows or columns that are not multiples of 32.  Lanes walk the tile-order side in 16-byte chunks (V elements of one face
+// row: one row, V consecutive columns), so that side is read or written in whole lines; the row-major side of a chunk is
+// one 16-byte access when it lies inside the row and its address allows it, else up to V element accesses.  grid.y numbers
+// the matrices.  Tilize writes zeros into the padding; untilize skips it.
+template <typename T, bool TILIZE>
+__global__ __launch_bounds__(256) void ttm_tile_ragged_k(const T *__restrict__ src, T *__restrict__ dst, uint32_t rows, uint32_t cols,
+                                                         uint32_t pr, uint32_t pc) {
+  constexpr uint32_t V = 16 / sizeof(T);
+  const uint32_t chunks = pr / V * pc, ct = pc / 32;
+  const int64_t b = blockIdx.y;
+  const T *rm_src = src + b * rows * (int64_t)cols;
+  T *rm_dst = dst + b * rows * (int64_t)cols;
+  const chunk_t *t_src = (const chunk_t *)(src + b * pr * (int64_t)pc);
+  chunk_t *t_dst = (chunk_t *)(dst + b * pr * (int64_t)pc);
+  for (uint32_t ch = blockIdx.x * 256 + threadIdx.x; ch < chunks; ch += gridDim.x * 256) {
+    const uint32_t e0 = ch * V, tile = e0 >> 10, e = e0 & 1023, face = e >> 8;
+    const uint32_t tr = tile / ct, tc = tile - tr * ct;
+    const uint32_t r = tr * 32 + (face >> 1) * 16 + ((e >> 4) & 15), c0 = tc * 32 + (face & 1) * 16 + (e & 15);
+    const bool row_in = r < rows;
+    const int64_t off = (int64_t)r * cols + c0;
+    if (TILIZE) {
+      chunk_t v = {0, 0, 0, 0};
+      if (row_in && c0 < cols) {
+        const T *p = rm_src + off;
+        if (c0 + V <= cols && ((uintptr_t)p & 15) == 0) {
+          v = __builtin_nontemporal_load((const chunk_t *)p);
+        } else {
+          T t[V];
+#pragma unroll
+          for (uint32_t j = 0; j < V; ++j) t[j] = c0 + j < cols ? p[j] : T(0);
+          v = *(const chunk_t *)t;
+        }
+      }
+      __builtin_nontemporal_store(v, t_dst + ch);
+    } else if (row_in && c0 < cols) {
+      const chunk_t v = __builtin_nontemporal_load(t_src + ch);
+      T *p = rm_dst + off;
+      if (c0 + V <= cols && ((uintptr_t)p & 15) == 0) {
+        __builtin_nontemporal_store(v, (chunk_t *)p);
+      } else {
+        T t[V];
+        *(chunk_t *)t = v;
+#pragma unroll
+        for (uint32_t j = 0; j < V; ++j)
+          if (c0 + j < cols) p[j] = t[j];
+      }
+    }
+  }
+}
+
+// Untilize of a ragged shape whose rows are whole 16-byte chunks (cols a multiple of V, destination 16-byte aligned): lanes
+// walk the row-major destination, so the stores are whole lines, and fetch each chunk from its face row on the tile side.
+template <typename T>
+__global__ __launch_bounds__(256) void ttm_untilize_rows_k(const T *__restrict__ src, T *__restrict__ dst, uint32_t rows, uint32_t cols,
+                                                           uint32_t pr, uint32_t pc) {
+  constexpr uint32_t V = 16 / sizeof(T);
+  const uint32_t cpr = cols / V, chunks = rows * cpr, ct = pc / 32;
+  const int64_t b = blockIdx.y;
+  const chunk_t *t_src = (const chunk_t *)(src + b * pr * (int64_t)pc);
+  chunk_t *o = (chunk_t *)(dst + b * rows * (int64_t)cols);
+  for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < chunks; i += gridDim.x * 256) {
+    const uint32_t r = i / cpr, c0 = (i - r * cpr) * V;
+    const uint32_t e = ((r >> 5) * ct + (c0 >> 5)) * 1024 + (((r >> 4) & 1) * 2 + ((c0 >> 4) & 1)) * 256 + (r & 15) * 16 + (c0 & 15);
+    __builtin_nontemporal_store(__builtin_nontemporal_load(t_src + e / V), o + i);
+  }
+}
+
 template <bool TILIZE>
 static int run_layout(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int elem,
                       void *stream, const char *who) {
@@ -171,6 +239,34 @@ static int run_layout(const void *src, void *dst, int64_t batch, int64_t rows, i
   hipStream_t s = (hipStream_t)stream;
   const int64_t pr = ttm_round_up32(rows), pc = ttm_round_up32(cols);
   const bool aligned = rows == pr && cols == pc && ((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0;
+  if (!aligned && batch <= 65535 && pr * pc < ((int64_t)1 << 31) && rows * cols < ((int64_t)1 << 31) &&
+      ((uintptr_t)(TILIZE ? dst : src) & 15) == 0 &&   // the tile-order side moves in whole 16-byte chunks
+      (TILIZE || elem > 1 || cols % 16 == 0)) {       // bytes into rows that are not whole chunks: the element-wise kernel is faster
+    if (!TILIZE && cols % (16 / elem) == 0 && ((uintptr_t)dst & 15) == 0) {
+      const int64_t rchunks = rows * cols * elem / 16;
+      const dim3 rgrid((unsigned)(ttm_cdiv(rchunks, 256) > 262144 ? 262144 : ttm_cdiv(rchunks, 256)), (unsigned)batch);
+#define ROWS(T) \
+  hipLaunchKernelGGL((ttm_untilize_rows_k<T>), rgrid, dim3(256), 0, s, (const T *)src, (T *)dst, (uint32_t)rows, (uint32_t)cols, (uint32_t)pr, \
+                     (uint32_t)pc)
+      if (elem == 4) ROWS(uint32_t);
+      else if (elem == 2) ROWS(uint16_t);
+      else ROWS(uint8_t);
+#undef ROWS
+      TTM_LAUNCH_CHECK();
+      return TTM_OK;
+    }
+    const int64_t chunks = pr * pc * elem / 16;
+    const dim3 grid((unsigned)(ttm_cdiv(chunks, 256) > 262144 ? 262144 : ttm_cdiv(chunks, 256)), (unsigned)batch);
+#define RAGGED(T) \
+  hipLaunchKernelGGL((ttm_tile_ragged_k<T, TILIZE>), grid, dim3(256), 0, s, (const T *)src, (T *)dst, (uint32_t)rows, (uint32_t)cols, \
+                     (uint32_t)pr, (uint32_t)pc)
+    if (elem == 4) RAGGED(uint32_t);
+    else if (elem == 2) RAGGED(uint16_t);
+    else RAGGED(uint8_t);
+#undef RAGGED
+    TTM_LAUNCH_CHECK();
+    return TTM_OK;
+  }
   if (!aligned) {
     int64_t n = batch * pr * pc;
     unsigned blocks = (unsigned)(ttm_cdiv(n, 256) > 1048576 ? 1048576 : ttm_cdiv(n, 256));
