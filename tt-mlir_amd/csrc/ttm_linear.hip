@@ -1171,6 +1171,43 @@ template <bool BFP4>
 __global__ __launch_bounds__(256) TTM_MAX_WAVES(3) void ttm_linear_image_k(const uint8_t *W, int64_t w_batch, uint8_t *img, int64_t img_batch, int Nt, int Kt) {
   linear_image_body<BFP4>(W + (int64_t)blockIdx.z * w_batch, img + (int64_t)blockIdx.z * img_batch, Nt, Kt, blockIdx.x);
 }
+// The same images from bf16 weights, [K, N] tiles (NK = false) or [N, K] tiles (NK = true): a permutation, no arithmetic.
+// With the weights in this form the second pass serves them exactly like block-float ones (seven-wide blocks, split K).
+template <bool NK>
+__global__ __launch_bounds__(256) TTM_MAX_WAVES(3) void ttm_linear_image_bf16_k(const uint8_t *W, int64_t w_batch, uint8_t *img, int64_t img_batch, int Nt, int Kt) {
+  W += (int64_t)blockIdx.z * w_batch;
+  img += (int64_t)blockIdx.z * img_batch;
+  const int tid = threadIdx.x, h = tid >> 5, wq = tid & 31;
+  const int ks = blockIdx.y, nt = 4 * (int)blockIdx.x + (h & 3), kt = 2 * ks + (h >> 2);
+  if (nt >= Nt) return;
+  const int face = wq >> 3, khalf = (wq >> 2) & 1, quad = wq & 3;   // face: (k half of the tile) * 2 + (n half)
+  u32x4 out[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) out[j] = u32x4{0, 0, 0, 0};
+  if (kt < Kt) {
+    if (NK) {   // [N, K] tiles: the eight k of a column are 16 contiguous bytes
+      const uint8_t *t = W + ((int64_t)nt * Kt + kt) * 2048 + ((face & 1) * 2 + (face >> 1)) * 512 + khalf * 16;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) out[j] = *(const u32x4 *)(t + (quad * 4 + j) * 32);
+    } else {    // [K, N] tiles: eight rows of four columns, regrouped by column
+      const uint8_t *t = W + ((int64_t)kt * Nt + nt) * 2048 + face * 512 + khalf * 256 + quad * 8;
+      u32x2 r[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) r[i] = *(const u32x2 *)(t + i * 32);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        out[0][i] = __builtin_amdgcn_perm(r[2 * i + 1].x, r[2 * i].x, 0x05040100u);
+        out[1][i] = __builtin_amdgcn_perm(r[2 * i + 1].x, r[2 * i].x, 0x07060302u);
+        out[2][i] = __builtin_amdgcn_perm(r[2 * i + 1].y, r[2 * i].y, 0x05040100u);
+        out[3][i] = __builtin_amdgcn_perm(r[2 * i + 1].y, r[2 * i].y, 0x07060302u);
+      }
+    }
+  }
+  u32x4 *dst = (u32x4 *)(img + ((int64_t)ks * Nt + nt) * 4096);
+  const int kc = (h >> 2) * 4 + (face >> 1) * 2 + khalf, n0 = (face & 1) * 16 + quad * 4;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) dst[lds_chunk(n0 + j, kc)] = out[j];
+}
 // the members of a group launch: grid.x numbers the members' groups of four column tiles one after another
 struct ImageGroup {
   const uint8_t *W[4];
@@ -1679,7 +1716,9 @@ static int set_lds_limit(K kernel, int bytes) {
 template <int WF>
 static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
   constexpr bool BFP = WF == WF_BFP8 || WF == WF_BFP4;
-  if (a.Mt == 1 || a.Mt * 32 <= ttm_option("linear_small_m_max")) {
+  // up to linear_small_m_max rows (64) the small kernels run once per row tile; bf16 weights leave them after one row tile
+  // (from two on the image route is faster: [14336, 4096] at M = 64 116 us against 75 us)
+  if (a.Mt == 1 || (BFP && a.Mt * 32 <= ttm_option("linear_small_m_max"))) {
     // the small kernel handles one row tile per launch
     LinearArgs p = a;
     const bool decode = BFP && ttm_option("linear_variant") != 1 && (int64_t)a.Nt * 1088 < (int64_t)1 << 32;
@@ -1745,18 +1784,25 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
   int variant = ttm_option("linear_variant");
   // the main kernels keep per-lane 32-bit offsets into one batch entry of the activations ([N,K] weights too)
   const bool fits32 = (int64_t)a.Mt * a.Kt * 2048 < (int64_t)1 << 32 && (int64_t)a.Nt * a.Kt * 2048 < (int64_t)1 << 32;
-  if (variant == 0) variant = !fits32 ? 1 : (BFP ? 6 : 5);
+  if (variant == 0) variant = !fits32 ? 1 : 6;
+  // bf16 weights reach the LDS-direct kernel through images of one weight set, which it addresses with 32 bits
+  if (!BFP && variant == 6 && (int64_t)((a.Kt + 1) / 2 + 1) * a.Nt * 4096 >= ((int64_t)1 << 31)) variant = 5;
   if ((variant == 5 || variant == 6) && !fits32) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear: operand too large for the selected kernel variant");
-  if (variant == 6 && !BFP) variant = 5;
   if (a.group_n > 1 && variant != 6) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear_group: the selected kernel variant has no group form");
   const int lds_bytes = 2 * 4096 * 16;
-  if constexpr (BFP) {
+  {
     if (variant == 6) {
-      static bool attr = false;
+      // bf16 weights always take two passes: the first rewrites them as the same images (a permutation), which gives them
+      // the block-float path's second pass with its seven-wide blocks and split K; the register-staged kernel that served
+      // them before (linear_variant = 5) has neither and loops over K at a third of the speed
+      constexpr int WI = BFP ? WF : WF_BFP8;   // the second pass only sees images
       const int lds6 = 131072 + (WF == WF_BFP8 ? 32768 : 16384);
-      if (!attr) {
-        if (int rc = set_lds_limit(ttm_linear_dma_k<WF>, lds6)) return rc;
-        attr = true;
+      if constexpr (BFP) {
+        static bool attr = false;
+        if (!attr) {
+          if (int rc = set_lds_limit(ttm_linear_dma_k<WF>, lds6)) return rc;
+          attr = true;
+        }
       }
       LinearArgs p = a;
       const int cus = device_cu_count();
@@ -1780,8 +1826,8 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       const int ksteps = (a.Kt + 1) / 2;
       const int64_t sets = a.w_batch == 0 ? 1 : batch;
       const int64_t img_set = (int64_t)(ksteps + 1) * a.Nt * 4096;   // a group: the members' image sets back to back
-      bool two_pass = ttm_option("linear_two_pass") == 2;
-      if (ttm_option("linear_two_pass") == 0) {
+      bool two_pass = ttm_option("linear_two_pass") == 2 || !BFP;
+      if (BFP && ttm_option("linear_two_pass") == 0) {
         static const double width_cost[5] = {0, 0, 0.78, 0.92, 1.0};
         const int64_t rounds = ((int64_t)p.n_blocks * slices * batch + cus - 1) / cus;
         const double fused = rounds * width_cost[p.ntw] * ((ksteps + slices - 1) / slices + 12) * 1.65;
@@ -1808,10 +1854,13 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       if (two_pass) {
         static bool attr2 = false;
         if (!attr2) {
-          if (int rc = set_lds_limit(ttm_linear_img_k<WF>, 131072)) return rc;
+          if (int rc = set_lds_limit(ttm_linear_img_k<WI>, 131072)) return rc;
           attr2 = true;
         }
-        if (a.group_n > 1) {
+        if constexpr (!BFP) {
+          hipLaunchKernelGGL((ttm_linear_image_bf16_k<WF == WF_BF16_NK>), dim3((a.Nt + 3) / 4, ksteps + 1, (unsigned)sets), dim3(256), 0, s, a.W,
+                             a.w_batch, ws, img_set, a.Nt, a.Kt);
+        } else if (a.group_n > 1) {
           ImageGroup g = {};
           g.n = a.group_n;
           uint8_t *at = ws;
@@ -1828,8 +1877,8 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         p.W = ws;
         p.w_batch = a.w_batch == 0 ? 0 : img_set;
         p.img_zero_step = ksteps;
-        hipLaunchKernelGGL((ttm_linear_img_k<WF>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), 131072, s, p);
-      } else {
+        hipLaunchKernelGGL((ttm_linear_img_k<WI>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), 131072, s, p);
+      } else if constexpr (BFP) {
         hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), lds6, s, p);
       }
       if (slices > 1)
