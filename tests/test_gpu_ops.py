@@ -335,8 +335,12 @@ def test_copy_view_at_positions_the_destination_from_device_memory(hip, dev, ele
     # odd and ragged key-tile counts for the 64-keys-per-pass kernel, masks on its second half, causal with Sq != Sk
     (1, 2, 2, 160, 96, 128, False, None), (1, 4, 1, 33, 33, 128, True, None), (1, 2, 2, 96, 224, 64, False, "bh"),
     (2, 4, 4, 130, 190, 128, False, "b1"), (1, 4, 2, 192, 320, 128, True, None), (1, 2, 1, 320, 192, 32, True, None),
-    (1, 8, 2, 1024, 1024, 128, True, None)])
-@pytest.mark.parametrize("variant", [0, 1, 3, 4])   # automatic, 32-key kernel, eight-wavefront kernel forced / forbidden
+    (1, 8, 2, 1024, 1024, 128, True, None),
+    # few query blocks against many keys: the keys of a query block shared among workgroups and merged by a second kernel
+    # (variant 5 keeps them in one workgroup); ragged key counts, masks, a causal chunk, shares without any visible key
+    (1, 8, 2, 128, 2048, 128, False, None), (1, 4, 2, 100, 1500, 64, False, "bh"), (2, 2, 2, 64, 1100, 128, False, "b1"),
+    (1, 4, 4, 128, 1024, 128, True, None), (1, 2, 1, 40, 4096, 32, False, None)])
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5])   # automatic, 32-key kernel, eight-wavefront kernel forced / forbidden, no key shares
 def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask, variant):
     if variant == 1 and Sq * Sk >= 512 * 512:
         pytest.skip("the 32-key kernel is covered by the small shapes")
@@ -434,6 +438,7 @@ def test_sdpa_heads_inner_equals_the_head_major_call(hip, dev, B, Hq, Hkv, Sq, S
     (1, 4, 2, 300, 300, 64, True, 100, True, None, 0), (2, 2, 2, 96, 160, 128, False, 40, False, None, 0),
     (1, 2, 1, 200, 200, 32, False, 0, False, None, 0), (1, 2, 2, 160, 160, 64, False, 65, True, "b1", 0),
     (1, 8, 2, 512, 512, 128, True, 129, True, None, 15), (1, 2, 2, 70, 70, 64, True, 1000, True, None, 0),
+    (1, 4, 2, 128, 2048, 128, False, 600, True, None, 0), (1, 4, 4, 96, 1536, 64, True, 200, True, None, 9),   # key shares
     (1, 2, 2, 128, 128, 128, True, None, True, None, 0), (2, 3, 3, 64, 100, 64, False, None, True, "bh", 0),
     (1, 1, 1, 100, 300, 256, False, 33, True, None, 0), (1, 4, 4, 640, 640, 64, True, 32, False, None, 9),
     (1, 2, 2, 1024, 1024, 128, True, 200, True, None, 0),

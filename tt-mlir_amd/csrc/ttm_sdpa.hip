@@ -33,6 +33,12 @@ struct SdpaArgs {
   // S / 32 * pitch, batch = H * head.  [B, S, H * D] (heads side by side, as a projection leaves them): pitch = H * D / 32
   // tiles, head = D / 32 tiles, batch = S / 32 * pitch.  Same 32 x 32 tiles either way.
   int64_t q_pitch, q_head, q_batch, k_pitch, k_head, k_batch, v_pitch, v_head, v_batch, o_pitch, o_head, o_batch;
+  // Few query blocks against many keys (a chunk of a long prefill, cross attention): the keys of a query block are divided
+  // among ksplits workgroups, which leave their running maximum, sum and unnormalised output per query tile here, in the
+  // order (split, b, h, query tile); ttm_sdpa_combine_k merges them.  ksplits = 1: the workgroup writes the output itself.
+  int ksplits;
+  float *part_o;    // [slots][D / 32][1024] fp32, elements of a tile in tile order
+  float *part_ml;   // [slots][32][2]: running maximum (log2 domain) and sum of each query of the tile
 };
 
 constexpr int kNoLimit = 1 << 29;
@@ -459,7 +465,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // that has only one workgroup per CU (a single sequence of a few thousand tokens) then still keeps two wavefronts on every
 // SIMD, so that one's softmax overlaps the other's matrix products; staging K and V is shared by twice as many lanes.
 template <int DT>  // head_dim / 32
-__device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *ldsK, uint16_t *ldsV) {
+__device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *ldsK, uint16_t *ldsV, int ks = 0) {
   constexpr int NT = 512, CHUNKS = DT * 256, NCH = (CHUNKS + NT - 1) / NT;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int qw = wave & 3, kh = wave >> 2;
@@ -488,7 +494,12 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
   const int q_glob = qt * 32 + l31, q_last = qt * 32 + 31;
 
   const int kt_begin = first_key_tile(p, qb * 128), kt_end = end_key_tile(p, min(qb * 4 + 4, p.sqt) * 32 - 1);
-  const int kb_begin = kt_begin >> 1, kb_end = (kt_end + 1) >> 1;
+  int kb_begin = kt_begin >> 1, kb_end = (kt_end + 1) >> 1;
+  if (p.ksplits > 1) {   // this workgroup's share of the query block's keys (workgroup-uniform)
+    const int chunk = (kb_end - kb_begin + p.ksplits - 1) / p.ksplits;
+    kb_begin += ks * chunk;
+    kb_end = min(kb_end, kb_begin + chunk);
+  }
   u32x4 kreg[NCH], vreg[NCH];
   auto load_block = [&](int kb) {
 #pragma unroll
@@ -514,7 +525,7 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
   };
   constexpr float LOG2E = 1.4426950408889634f;
   const float scale2 = p.scale * LOG2E;
-  if (kh == 0) sink_start(p, h, scale2, m_run, l_run);   // the sink belongs to one of the two halves only
+  if (kh == 0 && ks == 0) sink_start(p, h, scale2, m_run, l_run);   // the sink belongs to one of the two halves (and one key share) only
   for (int kb = kb_begin; kb < kb_end; ++kb) {
     __syncthreads();  // previous block fully consumed
 #pragma unroll
@@ -629,6 +640,7 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
     a0 = __builtin_amdgcn_exp2f(m_run - m_use);
     a1 = __builtin_amdgcn_exp2f(m1 - m_use);
     l_run = l_run * a0 + l1 * a1;
+    m_run = m;   // what the merged sum and output are relative to (a key share hands it on)
   }
 #pragma unroll
   for (int r4 = 0; r4 < 4; ++r4) {
@@ -648,6 +660,19 @@ __device__ __forceinline__ void sdpa64_split_block(const SdpaArgs &p, int qb, in
     __syncthreads();
   }
   if (kh != 0 || !wave_ok) return;   // no barrier follows inside this block; the next block starts with one
+  if (p.ksplits > 1) {   // one share of the keys: leave (max, sum, unnormalised output) for ttm_sdpa_combine_k
+    const int64_t slot_q = (((int64_t)ks * p.B + b) * p.Hq + h) * p.sqt + qt;
+    if (hh == 0) { p.part_ml[slot_q * 64 + 2 * l31] = m_run; p.part_ml[slot_q * 64 + 2 * l31 + 1] = l_run; }
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int din = g * 8 + hh * 4;
+        *(f32x4 *)(p.part_o + (slot_q * DT + d) * 1024 + ((l31 >> 4) * 2 + (din >> 4)) * 256 + (l31 & 15) * 16 + (din & 15)) =
+            f32x4{o[d][g * 4], o[d][g * 4 + 1], o[d][g * 4 + 2], o[d][g * 4 + 3]};
+      }
+    return;
+  }
   const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
   const bool q_ok = q_glob < p.Sq;
 #pragma unroll
@@ -670,13 +695,43 @@ __global__ __launch_bounds__(512) void ttm_sdpa64_split_k(SdpaArgs p, int paired
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[64 * D * 2];
   __shared__ __attribute__((aligned(16))) uint16_t ldsV[D * kSdpaVPitch];
   const int nqb = (p.sqt + 3) / 4, h = blockIdx.y, b = blockIdx.z;
-  if (!paired) {
-    sdpa64_split_block<DT>(p, nqb - 1 - (int)blockIdx.x, h, b, ldsK, ldsV);
+  if (!paired) {   // with key shares grid.x numbers (query block, share)
+    const int xb = (int)blockIdx.x / p.ksplits, ks = (int)blockIdx.x - xb * p.ksplits;
+    sdpa64_split_block<DT>(p, nqb - 1 - xb, h, b, ldsK, ldsV, ks);
     return;
   }
   const int heavy = nqb - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
   sdpa64_split_block<DT>(p, heavy, h, b, ldsK, ldsV);
   if (light < heavy) sdpa64_split_block<DT>(p, light, h, b, ldsK, ldsV);   // workgroup-uniform
+}
+
+// Merges the key shares of ttm_sdpa64_split_k: one workgroup per (b, h, query tile).  With M = max_s m_s, every output is
+// sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M); a share that saw no key has m = -inf and weighs nothing; a row without any
+// visible key gives zeros, as the single-workgroup path does.
+template <int DT>
+__global__ __launch_bounds__(256) void ttm_sdpa_combine_k(SdpaArgs p) {
+  const int qt = blockIdx.x, h = blockIdx.y, b = blockIdx.z, tid = threadIdx.x;
+  const int64_t slots = (int64_t)p.B * p.Hq * p.sqt, slot0 = ((int64_t)b * p.Hq + h) * p.sqt + qt;
+  uint8_t *op = p.out + b * p.o_batch + h * p.o_head + qt * p.o_pitch;
+  for (int g = tid; g < DT * 256; g += 256) {   // groups of four consecutive columns of one query
+    const int d = g >> 8, e = (g & 255) * 4, row = ((e >> 8) >> 1) * 16 + ((e >> 4) & 15);
+    float M = -INFINITY;
+    for (int ks = 0; ks < p.ksplits; ++ks) M = fmaxf(M, p.part_ml[(slot0 + ks * slots) * 64 + 2 * row]);
+    f32x4 num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.0f;
+    for (int ks = 0; ks < p.ksplits; ++ks) {
+      const int64_t sl = slot0 + ks * slots;
+      const float m = p.part_ml[sl * 64 + 2 * row], w = m == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m - M);
+      den += p.part_ml[sl * 64 + 2 * row + 1] * w;
+      num += *(const f32x4 *)(p.part_o + (sl * DT + d) * 1024 + e) * w;
+    }
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    const bool q_ok = qt * 32 + row < p.Sq;
+    u32x2 ov;
+    ov.x = q_ok ? pack_bf16_rne(num[0] * inv, num[1] * inv) : 0u;
+    ov.y = q_ok ? pack_bf16_rne(num[2] * inv, num[3] * inv) : 0u;
+    *(u32x2 *)(op + d * 2048 + e * 2) = ov;
+  }
 }
 
 static int sdpa_entry(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B,
@@ -731,14 +786,43 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
   if (hipGetDevice(&devid) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, devid) != hipSuccess || cus <= 0) cus = 256;
   const int64_t wgs = (int64_t)grid64.x * grid64.y * grid64.z;
   const bool split = wide && D <= 128 && (variant == 3 || (variant == 0 && wgs <= (int64_t)cus));
+  p.ksplits = 1; p.part_o = nullptr; p.part_ml = nullptr;
   if (split) {
     const dim3 block8(512);
+    // few workgroups against many keys (not the paired causal launch, whose query blocks carry equal work already): the
+    // keys of a query block are shared out until the device is full, at least four 64-key passes per share
+    int64_t ks = 1;
+    if (!paired && wgs * 2 <= (int64_t)cus && ttm_option("sdpa_variant") != 5) {
+      ks = (int64_t)cus / wgs;
+      if (ks > p.skt / 8) ks = p.skt / 8;
+      if (ks > 16) ks = 16;
+      if (ks < 1) ks = 1;
+    }
+    dim3 g = grid64;
+    if (ks > 1) {
+      const int64_t slots = (int64_t)B * Hq * p.sqt * ks;
+      void *ws = nullptr;
+      if (int rc = ttm_stream_workspace(s, (size_t)slots * (D * 32 + 64) * sizeof(float), &ws)) return rc;
+      p.ksplits = (int)ks;
+      p.part_o = (float *)ws;
+      p.part_ml = p.part_o + slots * D * 32;
+      g.x = (unsigned)(grid64.x * ks);
+    }
     switch (D) {
-    case 32: hipLaunchKernelGGL(ttm_sdpa64_split_k<1>, grid64, block8, 0, s, p, paired); break;
-    case 64: hipLaunchKernelGGL(ttm_sdpa64_split_k<2>, grid64, block8, 0, s, p, paired); break;
-    default: hipLaunchKernelGGL(ttm_sdpa64_split_k<4>, grid64, block8, 0, s, p, paired); break;
+    case 32: hipLaunchKernelGGL(ttm_sdpa64_split_k<1>, g, block8, 0, s, p, paired); break;
+    case 64: hipLaunchKernelGGL(ttm_sdpa64_split_k<2>, g, block8, 0, s, p, paired); break;
+    default: hipLaunchKernelGGL(ttm_sdpa64_split_k<4>, g, block8, 0, s, p, paired); break;
     }
     TTM_LAUNCH_CHECK();
+    if (ks > 1) {
+      const dim3 cg((unsigned)p.sqt, (unsigned)Hq, (unsigned)B);
+      switch (D) {
+      case 32: hipLaunchKernelGGL(ttm_sdpa_combine_k<1>, cg, dim3(256), 0, s, p); break;
+      case 64: hipLaunchKernelGGL(ttm_sdpa_combine_k<2>, cg, dim3(256), 0, s, p); break;
+      default: hipLaunchKernelGGL(ttm_sdpa_combine_k<4>, cg, dim3(256), 0, s, p); break;
+      }
+      TTM_LAUNCH_CHECK();
+    }
     return TTM_OK;
   }
   switch (D) {
