@@ -504,40 +504,77 @@ __global__ __launch_bounds__(256) void ttm_sdpa_decode_k(DecodeArgs p) {
   }  // nkeys != 0
 }
 
-// merges the slots of one (b, kv head): out = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M)
+// merges the slots of one query head: out = sum_s o_s exp(m_s - M) / sum_s l_s exp(m_s - M).  grid (B * Hkv, G), 256 lanes:
+// the weights exp(m_s - M) of the slices are formed once in LDS; 256 / D lanes share a column and take every (256 / D)-th
+// slice, so that a long cache cut into many slices for a few users (one user, 32768 positions: 64 slices) is merged by all
+// lanes of 32 workgroups instead of by eight workgroups looping over the slices.
+constexpr int kMaxCombineSlices = 1024;
 __global__ __launch_bounds__(256) void ttm_sdpa_decode_combine_k(DecodeArgs p) {
-  const int bh = blockIdx.x, tid0 = threadIdx.x;
+  __shared__ float wgt[kMaxCombineSlices];
+  __shared__ float red[256];
+  __shared__ float stats[2];
+  const int bh = blockIdx.x, tid = threadIdx.x;
   const int b = bh / p.Hkv, hk = bh % p.Hkv;
-  const int G = p.G, D = p.D;
-  const float *base = p.part + (size_t)bh * p.splits * G * (D + 2);
-  for (int i = tid0; i < G * D; i += 256) {
-    const int g = i / D, c = i % D;
-    const int h = hk * p.Gt + p.g0 + g;
-    const float sinkv = p.sink ? ttm_bf16_to_f32(p.sink[ttm_tiled_offset(h, 0, 1)]) * p.scale : -INFINITY;
-    float M = sinkv;
-    for (int s = 0; s < p.splits; ++s) M = fmaxf(M, base[((size_t)s * G + g) * (D + 2) + D]);
-    float num = 0.0f, den = p.sink ? __expf(sinkv - M) : 0.0f;
-    for (int s = 0; s < p.splits; ++s) {
-      const float *sl = base + ((size_t)s * G + g) * (D + 2);
-      const float w = (sl[D] == -INFINITY) ? 0.0f : __expf(sl[D] - M);
-      num += sl[c] * w;
-      den += sl[D + 1] * w;
-    }
-    const uint16_t val = ttm_f32_to_bf16(den > 0.0f ? num / den : 0.0f);
-    if (p.concat_heads) p.out[ttm_tiled_offset(b, h * D + c, (p.H * D) >> 5)] = val;
-    else p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(h, c, D >> 5)] = val;
+  const int G = p.G, D = p.D, S = p.splits;
+  for (int g = blockIdx.y; g < G; g += gridDim.y) {   // grid.y = G: one head per workgroup (workgroup-uniform)
+  const float *base = p.part + (size_t)bh * S * G * (D + 2) + (size_t)g * (D + 2);   // slice s: + s * G * (D + 2)
+  const size_t sstride = (size_t)G * (D + 2);
+  const int h = hk * p.Gt + p.g0 + g;
+  const float sinkv = p.sink ? ttm_bf16_to_f32(p.sink[ttm_tiled_offset(h, 0, 1)]) * p.scale : -INFINITY;
+  // M = max over the slices (and the sink)
+  float m = sinkv;
+  for (int s = tid; s < S; s += 256) m = fmaxf(m, base[s * sstride + D]);
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o));
+  if ((tid & 63) == 0) red[tid >> 6] = m;
+  __syncthreads();
+  const float M = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  // weights and the denominator
+  float den = 0.0f;
+  for (int s = tid; s < S; s += 256) {
+    const float ms = base[s * sstride + D];
+    const float w = ms == -INFINITY ? 0.0f : __expf(ms - M);
+    wgt[s] = w;
+    den += base[s * sstride + D + 1] * w;
   }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) den += __shfl_xor(den, o);
+  if ((tid & 63) == 0) red[tid >> 6] = den;
+  __syncthreads();
+  if (tid == 0) stats[0] = (red[0] + red[1]) + (red[2] + red[3]) + (p.sink ? __expf(sinkv - M) : 0.0f);
+  __syncthreads();
+  den = stats[0];
+  // numerators: lane (c, sub) sums the slices sub, sub + nsub, ... of column c
+  const int nsub = 256 / D > 0 ? 256 / D : 1;
+  for (int c0 = 0; c0 < D; c0 += 256) {   // one round unless D > 256
+    const int c = c0 + (tid % (D < 256 ? D : 256)), sub = D < 256 ? tid / D : 0;
+    float num = 0.0f;
+    if (c < D && sub < nsub)
+      for (int s = sub; s < S; s += nsub) num += base[s * sstride + c] * wgt[s];
+    red[tid] = num;
+    __syncthreads();
+    if (c < D && sub == 0) {
+      for (int u = 1; u < nsub; ++u) num += red[tid + u * D];
+      const uint16_t val = ttm_f32_to_bf16(den > 0.0f ? num / den : 0.0f);
+      if (p.concat_heads) p.out[ttm_tiled_offset(b, h * D + c, (p.H * D) >> 5)] = val;
+      else p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(h, c, D >> 5)] = val;
+    }
+    __syncthreads();
+  }
+  }  // heads of this workgroup
+  if (blockIdx.y != 0) return;   // the padding belongs to the first head's workgroup
   if (p.concat_heads) {   // padding rows below the last user, this kv head's columns
     if (b == p.B - 1) {
       const int pad = (int)ttm_round_up32(p.B) - p.B;
-      for (int i = tid0; i < pad * G * D; i += 256)
+      for (int i = tid; i < pad * G * D; i += 256)
         p.out[ttm_tiled_offset(p.B + i / (G * D), (hk * p.Gt + p.g0) * D + i % (G * D), (p.H * D) >> 5)] = 0;
     }
     return;
   }
   if (hk == p.Hkv - 1 && p.g0 + G == p.Gt) {   // padding rows of the last head tile
     const int pad = (int)ttm_round_up32(p.H) - p.H;
-    for (int i = tid0; i < pad * D; i += 256)
+    for (int i = tid; i < pad * D; i += 256)
       p.out[(int64_t)b * ttm_round_up32(p.H) * D + ttm_tiled_offset(p.H + i / D, i % D, D >> 5)] = 0;
   }
 }
@@ -724,6 +761,8 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
   if (ttm_cdiv(seq, splits) > max_keys) splits = ttm_cdiv(seq, max_keys);
   const int64_t keys = ttm_round_up32(ttm_cdiv(seq, splits));
   splits = ttm_cdiv(seq, keys);
+  TTM_REQUIRE(splits <= kMaxCombineSlices, "ttm_sdpa_decode: a cache of %lld positions takes %lld key slices, the merge handles %d", (long long)seq,
+              (long long)splits, kMaxCombineSlices);
   DecodeArgs p;
   p.q = (const uint16_t *)q; p.k = (const uint16_t *)k; p.v = (const uint16_t *)v; p.mask = (const uint16_t *)mask;
   p.cur_pos = cur_pos; p.page_table = page_table; p.out = (uint16_t *)out;
@@ -756,7 +795,7 @@ static int sdpa_decode_entry(const void *q, const void *k, const void *v, const 
     if (Gt <= kMaxG) hipLaunchKernelGGL(ttm_sdpa_decode_k<true>, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
     else hipLaunchKernelGGL(ttm_sdpa_decode_k<false>, dim3((unsigned)splits, (unsigned)(batch * kv_heads)), dim3(256), lds, s, p);
     TTM_LAUNCH_CHECK();
-    hipLaunchKernelGGL(ttm_sdpa_decode_combine_k, dim3((unsigned)(batch * kv_heads)), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(ttm_sdpa_decode_combine_k, dim3((unsigned)(batch * kv_heads), (unsigned)p.G), dim3(256), 0, s, p);
     TTM_LAUNCH_CHECK();
   }
   return TTM_OK;
