@@ -348,14 +348,14 @@ def make_workloads(torch, hip, datagen, dev, names):
 # and its share of the images again).  Each figure belongs to one version of a kernel source file: it is reported only
 # while that file still has the content it was measured on (first 12 hex digits of its SHA-1), else `traffic` is null.
 MEASURED_TRAFFIC_BYTES = {
-    "linear2048": (629.8e6, "ttm_linear.hip"), "linear32": (65.7e6, "ttm_linear.hip"), "pack_bfp8": (340.5e6, "ttm_bfp.hip"),
+    "linear2048": (629.5e6, "ttm_linear.hip"), "linear32": (65.7e6, "ttm_linear.hip"), "pack_bfp8": (340.4e6, "ttm_bfp.hip"),
     "unpack_bfp8": (340.1e6, "ttm_bfp.hip"), "pack_bfp4": (306.2e6, "ttm_bfp.hip"), "unpack_bfp4": (306.5e6, "ttm_bfp.hip"),
     "tilize_f32": (537.3e6, "ttm_layout.hip"), "untilize_f32": (537.0e6, "ttm_layout.hip"), "copy": (536.9e6, "ttm_layout.hip"),
     "sdpa_decode32": (270.3e6, "ttm_decode.hip"), "rmsnorm2048": (34.0e6, "ttm_rowwise.hip"),
-    "softmax65536": (1073.8e6, "ttm_rowwise.hip"), "reduce65536": (545.3e6, "ttm_rowwise.hip"), "silu_mul512": (44.2e6, "ttm_eltwise.hip"),
+    "softmax65536": (1073.8e6, "ttm_rowwise.hip"), "reduce65536": (545.2e6, "ttm_rowwise.hip"), "silu_mul512": (44.2e6, "ttm_eltwise.hip"),
 }
-MEASURED_ON = {"ttm_linear.hip": "23b79a5f349d", "ttm_bfp.hip": "8e9736544aea", "ttm_layout.hip": "cd2e71a9cab2",
-               "ttm_decode.hip": "563e2f3f8425", "ttm_rowwise.hip": "1ed7fe325f08", "ttm_eltwise.hip": "e63e9d74edc6"}
+MEASURED_ON = {"ttm_linear.hip": "e4074d055f65", "ttm_bfp.hip": "8e9736544aea", "ttm_layout.hip": "c2d080a6c0c5",
+               "ttm_decode.hip": "8bbb69b8561a", "ttm_rowwise.hip": "ad15392e8bae", "ttm_eltwise.hip": "56692d4eb0d8"}
 
 
 def measured_traffic(name):
