@@ -186,6 +186,42 @@ static unary_masked_fn pick_unary_masked(int op) {
 #undef U
 }
 
+// the same in 16-byte chunks: a chunk lies in one face row, so one (row, first column) decides which of its elements are
+// padding; grid.y numbers the matrices
+template <int OP, bool BF16>
+__global__ __launch_bounds__(256) void ttm_unary_masked_chunk_k(const void *__restrict__ in, void *__restrict__ out, uint32_t chunks_per_plane,
+                                                                uint32_t rows, uint32_t cols, float param, float param2) {
+  constexpr int EPC = BF16 ? 8 : 4;
+  const uint32_t tcols = (cols + 31) >> 5;
+  const int64_t base = (int64_t)blockIdx.y * chunks_per_plane;
+  for (uint32_t ci = blockIdx.x * 256 + threadIdx.x; ci < chunks_per_plane; ci += gridDim.x * 256) {
+    const uint32_t w = ci * EPC, tile = w >> 10, e = w & 1023, face = e >> 8;
+    const uint32_t r = (tile / tcols) * 32 + (face >> 1) * 16 + ((e >> 4) & 15), c0 = (tile % tcols) * 32 + (face & 1) * 16 + (e & 15);
+    float f[EPC];
+#pragma unroll
+    for (int i = 0; i < EPC; ++i) f[i] = 0.0f;
+    if (r < rows && c0 < cols) {
+      chunk_load<BF16>(in, base + ci, f);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) f[i] = c0 + i < cols ? unary_op<OP>(f[i], param, param2) : 0.0f;
+    }
+    chunk_store<BF16>(out, base + ci, f);
+  }
+}
+typedef void (*unary_chunk_fn)(const void *, void *, uint32_t, uint32_t, uint32_t, float, float);
+template <bool BF16>
+static unary_chunk_fn pick_unary_masked_chunk(int op) {
+#define U(OP) case OP: return ttm_unary_masked_chunk_k<OP, BF16>;
+  switch (op) {
+    U(U_ABS) U(U_CEIL) U(U_COS) U(U_FLOOR) U(U_GELU) U(U_ISFINITE) U(U_LOGICALNOT) U(U_NEG) U(U_RELU) U(U_SQRT)
+    U(U_RSQRT) U(U_SIGMOID) U(U_SIN) U(U_RECIPROCAL) U(U_SIGN) U(U_TAN) U(U_TANH) U(U_ATAN) U(U_EXP) U(U_ERF)
+    U(U_ERFC) U(U_LOG) U(U_EXPM1) U(U_LEAKYRELU) U(U_RELU6) U(U_SILU) U(U_HARDSIGMOID) U(U_MISH) U(U_ACOS) U(U_ASIN)
+    U(U_ASINH) U(U_CBRT) U(U_CLAMP) U(U_LOG1P)
+  default: return nullptr;
+  }
+#undef U
+}
+
 static unsigned grid_for(int64_t nchunks) {
   int64_t b = ttm_cdiv(nchunks, 256);
   return (unsigned)(b > 262144 ? 262144 : (b < 1 ? 1 : b));
@@ -201,6 +237,16 @@ static int unary_entry(int op, const void *in, void *out, int dtype, int layout,
   const int64_t n = batch * pr * pc;
   if (n == 0) return TTM_OK;
   TTM_REQUIRE(in && out, "ttm_eltwise_unary: null pointer");
+  if (tiled && (pr != rows || pc != cols) && batch <= 65535 && pr * pc < ((int64_t)1 << 31) &&
+      (((uintptr_t)in | (uintptr_t)out) & 15) == 0) {
+    unary_chunk_fn fn = dtype == TTM_BF16 ? pick_unary_masked_chunk<true>(op) : pick_unary_masked_chunk<false>(op);
+    if (!fn) return ttm_set_error(TTM_ERR_UNSUPPORTED, "ttm_eltwise_unary: unsupported op %d", op);
+    const uint32_t cpp = (uint32_t)(pr * pc * (dtype == TTM_BF16 ? 2 : 4) / 16);
+    hipLaunchKernelGGL(fn, dim3(grid_for(cpp), (unsigned)batch), dim3(256), 0, (hipStream_t)stream, in, out, cpp, (uint32_t)rows, (uint32_t)cols,
+                       param, param2);
+    TTM_LAUNCH_CHECK();
+    return TTM_OK;
+  }
   if (tiled && (pr != rows || pc != cols)) {
     unary_masked_fn fn = dtype == TTM_BF16 ? pick_unary_masked<true>(op) : pick_unary_masked<false>(op);
     if (!fn) return ttm_set_error(TTM_ERR_UNSUPPORTED, "ttm_eltwise_unary: unsupported op %d", op);
@@ -291,14 +337,15 @@ __global__ __launch_bounds__(256) void ttm_binary_bcast_k(int op, const void *__
   }
 }
 
-// Broadcasting in 16-byte chunks, for outputs whose chunks never straddle a row: tile layout with a multiple of 32 columns,
-// row-major with a multiple of the chunk width.  A chunk is EPC consecutive columns of one row (inside a tile: part of one
+// Broadcasting in 16-byte chunks, for outputs whose chunks never straddle a row: tile layout (ragged extents included: the
+// columns of a chunk that lie in the padding are written as zeros), row-major with a multiple of the chunk width.  A chunk is EPC consecutive columns of one row (inside a tile: part of one
 // face row), so per chunk one (row, first column) is decoded and every operand is read either as the 16 bytes at its own
 // offset for that position (its last dim is the output's) or as one element for the whole chunk (its last dim is 1).
 // grid.y numbers the batch entries; rows past R (tile padding) are written as zeros.
 struct ChunkPos {
   int64_t i0, i1, r, c0, out_chunk;
-  bool live;
+  bool live;    // the chunk holds at least one element of the tensor
+  int valid;    // how many of its EPC columns do (fewer than EPC only in the last tile column of a ragged tile tensor)
 };
 template <int EPC>
 __device__ __forceinline__ ChunkPos chunk_pos(const int64_t (&oshape)[4], int tiled, uint32_t ci, uint32_t chunks_per_plane) {
@@ -308,7 +355,7 @@ __device__ __forceinline__ ChunkPos chunk_pos(const int64_t (&oshape)[4], int ti
   q.i0 = batch / (uint32_t)oshape[1]; q.i1 = batch % (uint32_t)oshape[1];
   uint32_t r, c0;
   if (tiled) {
-    const uint32_t w = ci * EPC, tile = w >> 10, e = w & 1023, face = e >> 8, tcols = C >> 5;
+    const uint32_t w = ci * EPC, tile = w >> 10, e = w & 1023, face = e >> 8, tcols = (C + 31) >> 5;
     r = (tile / tcols) * 32 + (face >> 1) * 16 + ((e >> 4) & 15);
     c0 = (tile % tcols) * 32 + (face & 1) * 16 + (e & 15);
   } else {
@@ -316,7 +363,8 @@ __device__ __forceinline__ ChunkPos chunk_pos(const int64_t (&oshape)[4], int ti
     r = ci / cpr; c0 = (ci % cpr) * EPC;
   }
   q.r = r; q.c0 = c0;
-  q.live = r < R;
+  q.live = r < R && c0 < C;
+  q.valid = q.live ? (int)min(C - c0, (uint32_t)EPC) : 0;
   q.out_chunk = (int64_t)batch * chunks_per_plane + ci;
   return q;
 }
@@ -365,7 +413,7 @@ __global__ __launch_bounds__(256) void ttm_binary_chunk_k(int op, const void *__
       operand_chunk<BF16>(a, p.ashape, q, p.tiled, x);
       operand_chunk<BF16>(b, p.bshape, q, p.tiled, y);
 #pragma unroll
-      for (int i = 0; i < EPC; ++i) x[i] = binary_op(op, x[i], y[i]);
+      for (int i = 0; i < EPC; ++i) x[i] = i < q.valid ? binary_op(op, x[i], y[i]) : 0.0f;
     }
     chunk_store<BF16>(out, q.out_chunk, x);
   }
@@ -374,9 +422,9 @@ __global__ __launch_bounds__(256) void ttm_binary_chunk_k(int op, const void *__
 // whether the chunked kernels apply: chunks inside rows, everything 16-byte aligned, plane and batch counts within 32 bits
 static bool chunkable(const int64_t (&oshape)[4], int tiled, int es, std::initializer_list<const void *> ptrs) {
   const int64_t R = oshape[2], C = oshape[3], epc = 16 / es;
-  if (tiled ? (C % 32 != 0) : (C % epc != 0)) return false;
-  const int64_t pr = tiled ? ttm_round_up32(R) : R;
-  if (pr * C >= ((int64_t)1 << 31) || oshape[0] * oshape[1] > 65535 || oshape[0] * oshape[1] < 1) return false;
+  if (!tiled && C % epc != 0) return false;   // tile order: any extents, a chunk lies in one face row whatever they are
+  const int64_t pr = tiled ? ttm_round_up32(R) : R, pcc = tiled ? ttm_round_up32(C) : C;
+  if (pr * pcc >= ((int64_t)1 << 31) || oshape[0] * oshape[1] > 65535 || oshape[0] * oshape[1] < 1) return false;
   for (const void *q : ptrs)
     if (((uintptr_t)q & 15) != 0) return false;
   return true;
@@ -491,7 +539,8 @@ __global__ __launch_bounds__(256) void ttm_where_chunk_k(const void *__restrict_
       operand_chunk<BF16>(a, p.ashape, q, p.tiled, av);
       operand_chunk<BF16>(b, p.bshape, q, p.tiled, bv);
 #pragma unroll
-      for (int i = 0; i < EPC; ++i) av[i] = (cv[i] & (BF16 ? 0x7FFFu : 0x7FFFFFFFu)) != 0 ? av[i] : bv[i];   // +-0 is false, NaN is true
+      for (int i = 0; i < EPC; ++i)   // +-0 is false, NaN is true; columns in the padding stay zero
+        av[i] = i >= q.valid ? 0u : ((cv[i] & (BF16 ? 0x7FFFu : 0x7FFFFFFFu)) != 0 ? av[i] : bv[i]);
     }
     u32x4 o;
     if (BF16) {
