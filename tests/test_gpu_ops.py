@@ -87,19 +87,28 @@ def test_binary_broadcast(hip, dev, orc, layout, ashape, bshape, dtype):
             assert np.count_nonzero(full) == np.count_nonzero(want)
 
 
-def test_unary_keeps_tile_padding_zero(hip, dev, orc):
-    x = datagen.randn((2, 40, 50), seed=21, dtype=torch.bfloat16)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("shape", [(2, 40, 50), (3, 70, 64), (1, 32, 33), (2, 1, 1)])
+def test_unary_keeps_tile_padding_zero(hip, dev, orc, shape, dtype):
+    """Ops with f(0) != 0 on tile tensors with ragged rows, ragged columns or both: the padding stays zero."""
+    x = datagen.randn(shape, seed=21, dtype=dtype)
     xt = tilize_dev(hip, x, dev)
     for name in ("exp", "reciprocal", "gelu"):
         out = torch.full_like(xt, float("nan"))
-        hip.call("ttm_eltwise_unary", orc.UNARY[name], hip.ptr(xt), hip.ptr(out), hip.BF16, hip.TILE, 2, 40, 50, 0.0,
-                 hip.current_stream())
+        hip.call("ttm_eltwise_unary", orc.UNARY[name], hip.ptr(xt), hip.ptr(out), hip.BF16 if dtype == torch.bfloat16 else hip.F32, hip.TILE,
+                 shape[0], shape[1], shape[2], 0.0, hip.current_stream())
         torch.cuda.synchronize()
-        want = orc.round_bf16(orc.unary(name, x.float().numpy()))
+        want = orc.unary(name, x.float().numpy())
+        if dtype == torch.bfloat16:
+            want = orc.round_bf16(want)
         full = out.float().cpu().numpy()
         wt = orc.tilize(want)
         assert np.array_equal(full == 0, wt == 0)                               # padding (and only padding) is zero
-        assert np.max(bf16_ulps(untilize_dev(hip, out, x.shape, dev).float().cpu().numpy(), want)) <= 1.0
+        got = untilize_dev(hip, out, x.shape, dev).float().cpu().numpy()
+        if dtype == torch.bfloat16:
+            assert np.max(bf16_ulps(got, want)) <= 1.0
+        else:
+            assert np.allclose(got, want, rtol=1e-5, atol=1e-6)
 
 
 def test_typecast(hip, dev, orc):
