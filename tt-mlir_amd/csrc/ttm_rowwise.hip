@@ -607,6 +607,189 @@ __global__ __launch_bounds__(NT) TTM_MAX_WAVES((NT == 512 ? 2 : band_max_waves<M
   }
 }
 
+// ------------------------------------------------------------------------------------------------ few, very wide rows
+// A vocabulary-sized row for a handful of tokens: too few tile rows to fill the device with one workgroup each.  grid
+// (slices, tile rows): a workgroup takes a range of column tiles of one tile row (all 32 rows of it).  Lane t holds the
+// same 16-byte chunk position in every tile it visits, hence one row; the eight lanes that share a row are combined
+// through LDS.  Step one leaves per (row, slice) the statistics - (max, sum of exp relative to it) for softmax, the sum of
+// squares for RMSNorm, the partial result for the reductions; step two forms each row's total from all slices and, for
+// softmax and RMSNorm, reads the slice again and writes the output.  stats: [tile row][32][slices][2] floats.
+template <int ELEM>
+struct WideLane {
+  static constexpr int EPC = 16 / ELEM, CPT = 1024 / EPC, TPI = 256 / CPT;   // chunks per tile, tiles per step of a workgroup
+  int e, r, col_in, sub;
+  __device__ __forceinline__ WideLane(int tid) {
+    const int c = tid % CPT;
+    sub = tid / CPT;
+    e = c * EPC;
+    const int face = e >> 8;
+    r = (face >> 1) * 16 + ((e >> 4) & 15);
+    col_in = (face & 1) * 16 + (e & 15);
+  }
+  // LDS slot of the i-th of the eight lanes that hold row rr
+  static __device__ __forceinline__ int partner(int rr, int i) {
+    const int q = i % ELEM, f1 = (i / ELEM) & 1, sb = i / (2 * ELEM);
+    return sb * CPT + ((rr >> 4) * 2 + f1) * (16 * ELEM) + (rr & 15) * ELEM + q;
+  }
+};
+
+template <int MODE, int ELEM>
+__global__ __launch_bounds__(256) void ttm_rowwise_wide_stats_k(RowArgs p, float *__restrict__ stats, int slices, int tiles_per_slice) {
+  using L = WideLane<ELEM>;
+  constexpr int EPC = L::EPC;
+  constexpr bool IS_MAX = MODE == RW_SOFTMAX || MODE == RW_MAX;
+  __shared__ float sa[256], sb[256];
+  const int tid = threadIdx.x, slice = blockIdx.x, cols = (int)p.cols;
+  const int64_t trow = blockIdx.y;
+  const L ln(tid);
+  const uint8_t *x = (const uint8_t *)p.x + trow * p.ct * 1024 * ELEM;
+  const int t0 = slice * tiles_per_slice, t1 = min(p.ct, t0 + tiles_per_slice);
+  float a = IS_MAX ? -INFINITY : (MODE == RW_MIN ? INFINITY : 0.0f), l = 0.0f;
+  constexpr int UN = 4;   // loads in flight per lane: unconditional, clamped to the slice (a branch around a load serialises them)
+  for (int tb = t0 + ln.sub; tb < t1; tb += UN * L::TPI) {
+    u32x4 raw[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) raw[u] = __builtin_nontemporal_load((const u32x4 *)(x + ((int64_t)min(tb + u * L::TPI, t1 - 1) * 1024 + ln.e) * ELEM));
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+    const int t = tb + u * L::TPI;
+    if (t >= t1) break;
+    float f[EPC];
+    unpack_vals<ELEM>(raw[u], f);
+    const int c0 = t * 32 + ln.col_in;
+    if (MODE == RW_SOFTMAX) {
+      float cm = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) cm = c0 + i < cols ? fmaxf(cm, f[i]) : cm;
+      if (cm > a) { l *= expf(a - cm); a = cm; }   // a = -inf at first: l is 0 and stays 0
+      if (a != -INFINITY) {
+#pragma unroll
+        for (int i = 0; i < EPC; ++i) l += c0 + i < cols ? expf(f[i] - a) : 0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) {
+        const bool ok = c0 + i < cols;
+        if (MODE == RW_RMSNORM) a += ok ? f[i] * f[i] : 0.0f;
+        else if (MODE == RW_MAX) a = ok ? fmaxf(a, f[i]) : a;
+        else if (MODE == RW_MIN) a = ok ? fminf(a, f[i]) : a;
+        else a += ok ? f[i] : 0.0f;
+      }
+    }
+    }
+  }
+  sa[tid] = a; sb[tid] = l;
+  __syncthreads();
+  if (tid < 32) {
+    float A = IS_MAX ? -INFINITY : (MODE == RW_MIN ? INFINITY : 0.0f), Lsum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float v = sa[L::partner(tid, i)];
+      A = IS_MAX ? fmaxf(A, v) : (MODE == RW_MIN ? fminf(A, v) : A + v);
+    }
+    if (MODE == RW_SOFTMAX) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int k = L::partner(tid, i);
+        Lsum += sa[k] == -INFINITY ? 0.0f : sb[k] * expf(sa[k] - A);
+      }
+    }
+    float *o = stats + ((trow * 32 + tid) * slices + slice) * 2;
+    o[0] = A; o[1] = Lsum;
+  }
+}
+
+// row totals from the slices, by the whole workgroup: lane (row = tid % 32, part = tid / 32) folds every eighth slice of its
+// row, the eight parts of a row meet in LDS.  Softmax folds (max, sum relative to that max) pairs.
+template <int MODE>
+__device__ __forceinline__ void wide_fold(float &A, float &Ls, float v, float w) {
+  if (MODE == RW_SOFTMAX) {
+    if (v > A) { Ls = Ls * expf(A - v) + w; A = v; }   // A = -inf: Ls is 0 and exp gives 0
+    else if (v != -INFINITY) Ls += w * expf(v - A);
+  } else if (MODE == RW_MAX) A = fmaxf(A, v);
+  else if (MODE == RW_MIN) A = fminf(A, v);
+  else A += v;
+}
+template <int MODE>
+__device__ __forceinline__ void wide_totals(const float *st, int slices, float *ga, float *gb, float *ta, float *tb) {
+  constexpr bool IS_MAX = MODE == RW_SOFTMAX || MODE == RW_MAX;
+  const int tid = threadIdx.x, rr = tid & 31, part = tid >> 5;
+  float A = IS_MAX ? -INFINITY : (MODE == RW_MIN ? INFINITY : 0.0f), Ls = 0.0f;
+  for (int s = part; s < slices; s += 8) wide_fold<MODE>(A, Ls, st[((int64_t)rr * slices + s) * 2], st[((int64_t)rr * slices + s) * 2 + 1]);
+  ta[tid] = A; tb[tid] = Ls;
+  __syncthreads();
+  if (tid < 32) {
+    for (int k = 1; k < 8; ++k) wide_fold<MODE>(A, Ls, ta[tid + 32 * k], tb[tid + 32 * k]);
+    ga[tid] = A; gb[tid] = Ls;
+  }
+  __syncthreads();
+}
+
+template <int MODE, int ELEM>   // softmax or RMSNorm
+__global__ __launch_bounds__(256) void ttm_rowwise_wide_apply_k(RowArgs p, const float *__restrict__ stats, int slices, int tiles_per_slice) {
+  using L = WideLane<ELEM>;
+  constexpr int EPC = L::EPC;
+  __shared__ float ga[32], gb[32], ta[256], tb[256];
+  const int tid = threadIdx.x, slice = blockIdx.x, cols = (int)p.cols;
+  const int64_t trow = blockIdx.y;
+  wide_totals<MODE>(stats + trow * 32 * slices * 2, slices, ga, gb, ta, tb);
+  const L ln(tid);
+  const bool row_ok = (trow % p.rt) * 32 + ln.r < p.rows;
+  const float A = ga[ln.r];
+  const float mul = MODE == RW_RMSNORM ? 1.0f / sqrtf(A / (float)cols + p.eps) : 1.0f / gb[ln.r];
+  const uint8_t *x = (const uint8_t *)p.x + trow * p.ct * 1024 * ELEM;
+  uint8_t *o = (uint8_t *)p.out + trow * p.ct * 1024 * ELEM;
+  const int t0 = slice * tiles_per_slice, t1 = min(p.ct, t0 + tiles_per_slice);
+  constexpr int UN = 4;
+  for (int tb = t0 + ln.sub; tb < t1; tb += UN * L::TPI) {
+    u32x4 raw[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) raw[u] = __builtin_nontemporal_load((const u32x4 *)(x + ((int64_t)min(tb + u * L::TPI, t1 - 1) * 1024 + ln.e) * ELEM));
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+    const int t = tb + u * L::TPI;
+    if (t >= t1) break;
+    const int64_t off = (int64_t)t * 1024 + ln.e;
+    float f[EPC];
+    unpack_vals<ELEM>(raw[u], f);
+    const int c0 = t * 32 + ln.col_in;
+    if (MODE == RW_RMSNORM) {
+      float w[EPC], b[EPC];
+      const int cc = min(c0, ((cols + EPC - 1) / EPC - 1) * EPC);   // the padding of the last tile has no weight: reread a valid chunk
+      if (p.w) load_vec<ELEM>(p.w, p.w_tiled, cc, w);
+      if (p.b) load_vec<ELEM>(p.b, p.b_tiled, cc, b);
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) {
+        float y = f[i] * mul;
+        if (p.w) y *= w[i];
+        if (p.b) y += b[i];
+        f[i] = (row_ok && c0 + i < cols) ? y : 0.0f;
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < EPC; ++i) f[i] = (row_ok && c0 + i < cols) ? expf(f[i] - A) * mul : 0.0f;
+    }
+    store_vals<ELEM>(o, off, f);
+    }
+  }
+}
+
+template <int MODE, int ELEM>   // reductions: the [.., rows, 1] output tile of every tile row
+__global__ __launch_bounds__(256) void ttm_rowwise_wide_finish_k(RowArgs p, const float *__restrict__ stats, int slices) {
+  using L = WideLane<ELEM>;
+  __shared__ float ga[32], gb[32], ta[256], tb[256];
+  const int tid = threadIdx.x;
+  const int64_t trow = blockIdx.x;
+  wide_totals<MODE>(stats + trow * 32 * slices * 2, slices, ga, gb, ta, tb);
+  if (tid < L::CPT) {
+    const L ln(tid);
+    u32x4 z = {0, 0, 0, 0};
+    const float total = MODE == RW_MEAN ? ga[ln.r] / (float)p.cols : ga[ln.r];
+    if (ln.col_in == 0 && (trow % p.rt) * 32 + ln.r < p.rows) z.x = ELEM == 2 ? (uint32_t)ttm_f32_to_bf16(total) : __float_as_uint(total);
+    *(u32x4 *)((uint8_t *)p.out + (trow * 1024 + ln.e) * ELEM) = z;
+  }
+}
+
 template <int MODE>
 static int launch_rowwise(const RowArgs &p, int dtype, int64_t trows, hipStream_t s) {
   TTM_REQUIRE(trows < (1ll << 29), "row-wise kernel: tensor too large");
@@ -632,6 +815,33 @@ static int launch_rowwise(const RowArgs &p, int dtype, int64_t trows, hipStream_
       if (dtype == TTM_BF16) TTM_BAND_NK(2); else TTM_BAND_NK(4);
 #undef TTM_BAND_NK
 #undef TTM_BAND_LAUNCH
+      TTM_LAUNCH_CHECK();
+      return TTM_OK;
+    }
+  }
+  // few tile rows of very wide rows: slices of at least eight column tiles, enough of them for about 512 workgroups
+  const bool row_kernel_fits = (MODE == RW_RMSNORM || MODE == RW_SOFTMAX) && p.ct * 2 * (dtype == TTM_BF16 ? 2 : 4) <= 8 * 256;
+  if (p.ct >= 256 && !row_kernel_fits && trows * 2 <= 256 && ttm_option("rowwise_variant") == 0) {
+    int slices = (int)(512 / trows);
+    if (slices > p.ct / 8) slices = p.ct / 8;
+    if (slices > 256) slices = 256;
+    if (slices < 1) slices = 1;
+    const int tps = (int)ttm_cdiv(p.ct, slices);
+    slices = (int)ttm_cdiv(p.ct, tps);
+    void *ws = nullptr;
+    if (int rc = ttm_stream_workspace(s, (size_t)(trows * 32 * slices * 2) * sizeof(float), &ws)) return rc;
+    const dim3 grid((unsigned)slices, (unsigned)trows);
+    if (trows <= 65535) {
+      if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_wide_stats_k<MODE, 2>), grid, dim3(256), 0, s, p, (float *)ws, slices, tps);
+      else hipLaunchKernelGGL((ttm_rowwise_wide_stats_k<MODE, 4>), grid, dim3(256), 0, s, p, (float *)ws, slices, tps);
+      TTM_LAUNCH_CHECK();
+      if constexpr (MODE == RW_RMSNORM || MODE == RW_SOFTMAX) {
+        if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_wide_apply_k<MODE, 2>), grid, dim3(256), 0, s, p, (const float *)ws, slices, tps);
+        else hipLaunchKernelGGL((ttm_rowwise_wide_apply_k<MODE, 4>), grid, dim3(256), 0, s, p, (const float *)ws, slices, tps);
+      } else {
+        if (dtype == TTM_BF16) hipLaunchKernelGGL((ttm_rowwise_wide_finish_k<MODE, 2>), dim3((unsigned)trows), dim3(256), 0, s, p, (const float *)ws, slices);
+        else hipLaunchKernelGGL((ttm_rowwise_wide_finish_k<MODE, 4>), dim3((unsigned)trows), dim3(256), 0, s, p, (const float *)ws, slices);
+      }
       TTM_LAUNCH_CHECK();
       return TTM_OK;
     }
