@@ -73,6 +73,17 @@ int ttrt_tensor_is_allocated(const ttrt_tensor *t, int *allocated);
 int ttrt_tensor_set_retain(ttrt_tensor *t, int retain);
 int ttrt_tensor_get_retain(const ttrt_tensor *t, int *retain);
 int ttrt_tensor_deallocate(ttrt_tensor *t, int force);                         /* deallocateTensor (runtime.h:244) */
+/* createEmptyTensor (runtime.h:107-110): uninitialised tensor in the given layout; dev may be NULL for host storage */
+int ttrt_tensor_create_empty(ttrt_device *dev, const ttrt_layout *layout, const uint32_t *shape, int rank, ttrt_tensor **out);
+/* hasLayout (runtime.h:230); getTensorLayout (232) is the layout ttrt_tensor_desc reports */
+int ttrt_tensor_has_layout(const ttrt_tensor *t, const ttrt_layout *layout, int *has);
+/* getTensorVolume / getTensorElementSize / getTensorStride (runtime.h:142-146): elements, bytes per element (1 for
+ * block-float types) and the contiguous stride in elements; stride receives up to 8 entries, any pointer may be NULL */
+int ttrt_tensor_extent(const ttrt_tensor *t, uint32_t *volume, uint32_t *element_size, int64_t *stride);
+/* dumpTensor / loadTensor (runtime.h:304-308): the file keeps the tensor's own layout (tile order, block-float bytes);
+ * a device tensor is read back first.  load: dev NULL gives a host tensor, else the tensor is moved to that device. */
+int ttrt_tensor_dump(const ttrt_tensor *t, const char *path);
+int ttrt_tensor_load(const char *path, ttrt_device *dev, ttrt_tensor **out);
 
 /* getLayout (runtime.h:234-235), toLayout (227-228; retain: -1 unset, 0, 1), toHost (221-222), wait (212-217),
  * memcpy(void*, Tensor, optional<DataType>) (237-238; target_dtype -1 = none), memcpy(Tensor, Tensor) (240) */
@@ -110,6 +121,13 @@ int ttrt_hook_update(void *hook_ctx, uint32_t global_id, const ttrt_tensor *src)
 int ttrt_hook_program_index(void *hook_ctx, uint32_t *index);
 /* location string of the operation a hook is running for (getOpLocInfo, runtime.h:248) */
 int ttrt_hook_loc(void *hook_ctx, char *buf, size_t len);
+/* shape and data type of one of the operation's operands or results, from the binary alone (TensorRef::get_shape /
+ * get_dtype: getTensorRefShape, runtime.h:263, and getTensorRefDataType); fails if global_id is neither */
+int ttrt_hook_ref_desc(void *hook_ctx, uint32_t global_id, uint32_t *shape, int *rank, int *dtype);
+/* walkProgram (runtime.h:294-297): cb for every operation of the program in order; nothing runs and no device is needed.
+ * Inside cb the hook context answers ttrt_hook_loc / input_refs / output_refs / ref_desc; there is no tensor pool, so
+ * ttrt_hook_output and ttrt_hook_retrieve give NULL and ttrt_hook_update / ttrt_hook_program_index fail. */
+int ttrt_walk_program(const ttrt_binary *bin, uint32_t program, ttrt_op_callback cb, void *user);
 int ttrt_stat(const char *name, int64_t *value);
 int ttrt_stats_clear(void);
 

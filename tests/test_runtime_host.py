@@ -282,3 +282,145 @@ def test_schema_constants_are_what_the_generator_makes_of_the_schema_text():
     spec.loader.exec_module(gen)
     for fname, text in gen.generate(ref).items():
         assert open(os.path.join(rtdir, fname)).read() == text, fname + " differs from the generator's output"
+
+
+def _program_with_recorded_descs():
+    """A two-program binary written with the program builder, and per program the (op name, input descs, output descs)
+    the builder reported while writing it: what the walk must find in the flatbuffer."""
+    pb = rt.ProgramBuilder()
+    want = []
+    pb.begin_program("prep", private=True)
+    w = pb.input((96, 40), DT.BFloat16)
+    wq = pb.typecast(w, DT.BFP_BFloat8)
+    pb.output(wq)
+    pb.end_program()
+    want.append([("TypecastOp", [w], [wq], pb)])
+    pb.begin_program("main")
+    x = pb.input((2, 33, 96), DT.BFloat16)
+    g = pb.input((96,), DT.BFloat16)
+    wi = pb.input((96, 40), DT.BFP_BFloat8)
+    n = pb.rms_norm(x, g, eps=1e-5)
+    y = pb.matmul(n, wi)
+    s = pb.softmax(y, dim=-1)
+    r = pb.reduction(0, s, [2], keep_dim=True)
+    t = pb.transpose(y, 1, 2)
+    pb.output(r)
+    pb.output(t)
+    pb.end_program()
+    want.append([("RMSNormOp", [x, g], [n], pb), ("MatmulOp", [n, wi], [y], pb), ("SoftmaxOp", [y], [s], pb),
+                 ("ReductionOp", [s], [r], pb), ("TransposeOp", [y], [t], pb)])
+    descs = {i: pb.desc(i) for ops in want for _, ins, outs, _ in ops for i in ins + outs}
+    return rt.Binary.load_from_memory(pb.finish()), [[(name, ins, outs) for name, ins, outs, _ in ops] for ops in want], descs
+
+
+def test_walk_program_reports_every_operation_with_its_tensor_refs():
+    # the reference's own check of walkProgram (test/python/chisel/test_walk_program.py:14-54): every operation in order,
+    # the shapes of its operand and result references equal to the shapes of the program that was compiled
+    binary, want, descs = _program_with_recorded_descs()
+    for program, ops in enumerate(want):
+        seen = []
+
+        def visit(idx, name, dbg, hook):
+            ins, outs = hook.input_refs(), hook.output_refs()
+            seen.append((idx, name, ins, outs))
+            for gid in ins + outs:
+                shape, dtype = hook.ref_desc(gid)
+                assert tuple(shape) == tuple(descs[gid][0]) and dtype == descs[gid][1].dtype
+            assert hook.loc() == 'loc("%s"("op%d"))' % (binary.get_program_name(program), idx) and dbg.startswith("ttnn.")
+            assert hook.output() is None and hook.retrieve(ins[0]) is None   # nothing runs: there is no tensor pool
+            with pytest.raises(rt.RuntimeError_, match="no program context"):
+                hook.program_index()
+            with pytest.raises(rt.RuntimeError_, match="neither an operand nor a result"):
+                hook.ref_desc(10 ** 6)
+        rt.walk_program(binary, program, visit)
+        assert [(n, i, o) for _, n, i, o in seen] == ops
+        assert [i for i, _, _, _ in seen] == list(range(len(ops)))
+
+
+def test_walk_program_errors():
+    binary, _, _ = _program_with_recorded_descs()
+    with pytest.raises(rt.RuntimeError_, match="program index out of range"):
+        rt.walk_program(binary, 2, lambda *a: None)
+
+    class Stop(Exception):
+        pass
+    calls = []
+
+    def boom(idx, *a):
+        calls.append(idx)
+        raise Stop()
+    with pytest.raises(Stop):
+        rt.walk_program(binary, 1, boom)
+    assert calls == [0]   # the first exception ends the walk for the caller
+
+
+@pytest.mark.parametrize("dtype,np_dtype", [(DT.Float32, np.float32), (DT.BFloat16, np.uint16), (DT.Int32, np.int32), (DT.UInt8, np.uint8)])
+def test_dump_and_load_tensor_round_trip(tmp_path, dtype, np_dtype):
+    rng = np.random.default_rng(3)
+    a = rng.integers(0, 200, size=(3, 5, 7)).astype(np_dtype)
+    t = rt.create_owned_host_tensor(a, dtype)
+    path = tmp_path / "t.tensor"
+    rt.dump_tensor(t, path)
+    back = rt.load_tensor(path)
+    assert back.get_shape() == [3, 5, 7] and back.get_layout() == rt.Layout(ST.Host, TL.RowMajor, dtype)
+    assert np.array_equal(rt.to_numpy(back), a)
+    assert back.get_data_buffer() == bytearray(a.tobytes())
+    # container: magic, version, dtype, layout, rank, extents, payload size, payload
+    raw = path.read_bytes()
+    assert raw[:4] == b"TTMT" and struct.unpack("<5I", raw[4:24]) == (1, dtype, TL.RowMajor, 3, 3)
+    assert struct.unpack("<2I", raw[24:32]) == (5, 7) and struct.unpack("<Q", raw[32:40])[0] == a.nbytes
+    assert raw[40:] == a.tobytes()
+
+
+def test_load_tensor_rejects_damaged_files(tmp_path):
+    a = np.arange(24, dtype=np.float32).reshape(4, 6)
+    path = tmp_path / "t.tensor"
+    rt.dump_tensor(rt.create_owned_host_tensor(a, DT.Float32), path)
+    raw = path.read_bytes()
+
+    def load(data):
+        p = tmp_path / "bad.tensor"
+        p.write_bytes(data)
+        return rt.load_tensor(p)
+    with pytest.raises(rt.RuntimeError_, match="not a tensor file"):
+        load(b"XXXX" + raw[4:])
+    with pytest.raises(rt.RuntimeError_, match="unknown tensor file version"):
+        load(raw[:4] + struct.pack("<I", 9) + raw[8:])
+    with pytest.raises(rt.RuntimeError_, match="ends inside its payload"):
+        load(raw[:-8])
+    with pytest.raises(rt.RuntimeError_, match="ends inside its header"):
+        load(raw[:18])
+    with pytest.raises(rt.RuntimeError_, match="payload size does not match"):
+        load(raw[:28] + struct.pack("<I", 7) + raw[32:])           # second extent 6 -> 7
+    with pytest.raises(rt.RuntimeError_, match="unknown data type"):
+        load(raw[:8] + struct.pack("<I", 99) + raw[12:])
+    with pytest.raises(rt.RuntimeError_, match="never stored in"):
+        load(raw[:8] + struct.pack("<I", DT.Float64) + raw[12:])
+    with pytest.raises(rt.RuntimeError_, match="block-float data outside the tile layout"):
+        load(raw[:8] + struct.pack("<I", DT.BFP_BFloat8) + raw[12:])
+    with pytest.raises(rt.RuntimeError_, match="cannot open"):
+        rt.load_tensor(tmp_path / "absent.tensor")
+    with pytest.raises(rt.RuntimeError_, match="cannot open"):
+        rt.dump_tensor(rt.create_owned_host_tensor(a, DT.Float32), tmp_path / "no_such_dir" / "t.tensor")
+
+
+def test_tensor_accessors_and_empty_host_tensors():
+    a = np.zeros((2, 3, 40), dtype=np.float32)
+    t = rt.create_owned_host_tensor(a, DT.Float32)
+    assert t.get_shape() == [2, 3, 40] and t.get_stride() == [120, 40, 1]
+    assert t.get_volume() == 240 and t.get_element_size() == 4 and t.get_dtype() == DT.Float32
+    assert t.has_layout(rt.Layout(ST.Host, TL.RowMajor, DT.Float32))
+    assert not t.has_layout(rt.Layout(ST.Host, TL.Tile, DT.Float32))
+    assert not t.has_layout(rt.Layout(ST.Device, TL.RowMajor, DT.Float32))
+    assert not t.has_layout(rt.Layout(ST.Host, TL.RowMajor, DT.BFloat16))
+    # host storage needs no device; the tile layout pads both trailing extents to 32, block-float tiles are 1088 / 576 bytes
+    e = rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.RowMajor, DT.BFloat16), (4, 10))
+    assert e.is_allocated() and e.desc() == ((4, 10), rt.Layout(ST.Host, TL.RowMajor, DT.BFloat16), 80)
+    e = rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.Float32), (2, 33, 40))
+    assert e.desc()[2] == 2 * 64 * 64 * 4
+    e = rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.BFP_BFloat8), (33, 40))
+    assert e.desc()[2] == 4 * 1088 and e.get_element_size() == 1
+    e = rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.BFP_BFloat4), (64, 64))
+    assert e.desc()[2] == 4 * 576
+    with pytest.raises(rt.RuntimeError_, match="null argument: device"):
+        rt.create_empty_tensor(None, rt.Layout(ST.Device, TL.Tile, DT.BFloat16), (32, 32))

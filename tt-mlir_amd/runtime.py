@@ -222,6 +222,39 @@ class Tensor:
         _call("ttrt_tensor_is_allocated", self.h, ctypes.byref(v))
         return bool(v.value)
 
+    # the accessors of the reference's Tensor binding (runtime/python/runtime/runtime.cpp:213-262)
+    def get_shape(self):
+        return list(self.desc()[0])
+
+    def get_layout(self):
+        return self.desc()[1]
+
+    def get_dtype(self):
+        return self.desc()[1].dtype
+
+    def has_layout(self, layout):
+        v = ctypes.c_int()
+        _call("ttrt_tensor_has_layout", self.h, ctypes.byref(layout), ctypes.byref(v))
+        return bool(v.value)
+
+    def _extent(self):
+        vol, esz, stride = ctypes.c_uint32(), ctypes.c_uint32(), (ctypes.c_int64 * 8)()
+        _call("ttrt_tensor_extent", self.h, ctypes.byref(vol), ctypes.byref(esz), stride)
+        return vol.value, esz.value, list(stride[: len(self.desc()[0])])
+
+    def get_volume(self):
+        return self._extent()[0]
+
+    def get_element_size(self):
+        return self._extent()[1]
+
+    def get_stride(self):
+        return self._extent()[2]
+
+    def get_data_buffer(self):
+        """The tensor's bytes, read back and untilized if it lives on the device (getTensorDataBuffer)."""
+        return bytearray(to_numpy(self).tobytes())
+
     def set_retain(self, retain):
         _call("ttrt_tensor_set_retain", self.h, int(retain))
 
@@ -289,6 +322,26 @@ def from_torch(t, borrowed=False):
     a = t.contiguous()
     arr = a.view(view).numpy().view(np.uint16) if view is not None else a.numpy()
     return _host(arr, dt, borrowed)
+
+
+def create_empty_tensor(device, layout, shape):
+    """Uninitialised tensor in `layout` (createEmptyTensor); `device` may be None for host storage."""
+    sh, rank = _shape_arg(shape)
+    h = ctypes.c_void_p()
+    _call("ttrt_tensor_create_empty", device.h if device is not None else None, ctypes.byref(layout), sh, rank, ctypes.byref(h))
+    return Tensor(h)
+
+
+def dump_tensor(tensor, file_path):
+    """Write the tensor to a file in its own layout (dumpTensor)."""
+    _call("ttrt_tensor_dump", tensor.h, os.fsencode(file_path))
+
+
+def load_tensor(file_path, device=None):
+    """Read a tensor written by dump_tensor; on the host, or on `device` when one is given (loadTensor)."""
+    h = ctypes.c_void_p()
+    _call("ttrt_tensor_load", os.fsencode(file_path), device.h if device is not None else None, ctypes.byref(h))
+    return Tensor(h)
 
 
 def get_layout(binary, program, input_index):
@@ -425,6 +478,12 @@ class HookContext:
         _call("ttrt_hook_program_index", self._h, ctypes.byref(i))
         return i.value
 
+    def ref_desc(self, global_id):
+        """(shape, dtype) of one of the op's operands or results as the binary declares it (TensorRef.get_shape / get_dtype)."""
+        shape, rank, dt = (ctypes.c_uint32 * 8)(), ctypes.c_int(), ctypes.c_int()
+        _call("ttrt_hook_ref_desc", self._h, global_id, shape, ctypes.byref(rank), ctypes.byref(dt))
+        return list(shape[: rank.value]), dt.value
+
 
 def _op_trampoline(fn):
     def tramp(idx, name, dbg, hook, user):
@@ -452,6 +511,22 @@ def set_program_callbacks(pre=None, post=None):
         return _PROGRAM_CB_TYPE(lambda idx, hook, user: fn(idx, HookContext(hook)))
     _cb_keep["pre_program"], _cb_keep["post_program"] = wrap(pre), wrap(post)
     _call("ttrt_set_program_callbacks", _cb_keep["pre_program"], _cb_keep["post_program"], None)
+
+
+def walk_program(binary, program_index, fn):
+    """fn(op_index, op_name, debug_info, hook: HookContext) for every operation of the program in order; nothing runs
+    (walkProgram).  The hook answers loc / input_refs / output_refs / ref_desc; there is no tensor pool behind it."""
+    raised = []
+
+    def guarded(idx, name, dbg, hook):   # an exception cannot cross the C frames: keep the first, re-raise it afterwards
+        if not raised:
+            try:
+                fn(idx, name, dbg, hook)
+            except BaseException as e:
+                raised.append(e)
+    _call("ttrt_walk_program", binary.h, program_index, _op_trampoline(guarded), None)
+    if raised:
+        raise raised[0]
 
 
 def clear_callbacks():

@@ -183,6 +183,41 @@ TTRT_EXPORT int ttrt_tensor_deallocate(ttrt_tensor *t, int force) {
   return guard([&] { need(t, "tensor"); deallocateTensor(t->t, force != 0); });
 }
 
+TTRT_EXPORT int ttrt_tensor_create_empty(ttrt_device *dev, const ttrt_layout *layout, const uint32_t *shape, int rank, ttrt_tensor **out) {
+  return guard([&] {
+    need(layout, "layout"); need(out, "out");
+    Layout l = toLayoutStruct(*layout);
+    if (l.storageType == StorageType::Device) need(dev, "device");
+    auto s = shapeVec(shape, rank);
+    *out = new ttrt_tensor{createEmptyTensor(dev ? dev->d : Device{}, l, s, utils::calculateStride(s),
+                                              utils::isBlockFormatDataType(l.dataType) ? 1 : utils::dataTypeElementSize(l.dataType))};
+  });
+}
+TTRT_EXPORT int ttrt_tensor_has_layout(const ttrt_tensor *t, const ttrt_layout *layout, int *has) {
+  return guard([&] { need(t, "tensor"); need(layout, "layout"); need(has, "has"); *has = hasLayout(t->t, toLayoutStruct(*layout)); });
+}
+TTRT_EXPORT int ttrt_tensor_extent(const ttrt_tensor *t, uint32_t *volume, uint32_t *element_size, int64_t *stride) {
+  return guard([&] {
+    need(t, "tensor");
+    if (volume) *volume = getTensorVolume(t->t);
+    if (element_size) *element_size = getTensorElementSize(t->t);
+    if (stride) {
+      auto st = getTensorStride(t->t);
+      if (st.size() > 8) throw std::runtime_error("tensor rank above 8");
+      for (size_t i = 0; i < st.size(); ++i) stride[i] = st[i];
+    }
+  });
+}
+TTRT_EXPORT int ttrt_tensor_dump(const ttrt_tensor *t, const char *path) {
+  return guard([&] { need(t, "tensor"); need(path, "path"); dumpTensor(t->t, path); });
+}
+TTRT_EXPORT int ttrt_tensor_load(const char *path, ttrt_device *dev, ttrt_tensor **out) {
+  return guard([&] {
+    need(path, "path"); need(out, "out");
+    *out = new ttrt_tensor{loadTensor(path, dev ? std::optional<Device>(dev->d) : std::nullopt)};
+  });
+}
+
 TTRT_EXPORT int ttrt_get_layout(const ttrt_binary *bin, uint32_t program, uint32_t input, ttrt_layout *layout) {
   return guard([&] { need(bin, "binary"); need(layout, "layout"); *layout = fromLayoutStruct(getLayout(bin->b, program, input)); });
 }
@@ -316,6 +351,31 @@ TTRT_EXPORT int ttrt_hook_loc(void *hook_ctx, char *buf, size_t len) {
   return guard([&] {
     need(hook_ctx, "hook context");
     copyStr(getOpLocInfo(static_cast<HookCtx *>(hook_ctx)->oc), buf, len);
+  });
+}
+TTRT_EXPORT int ttrt_hook_ref_desc(void *hook_ctx, uint32_t global_id, uint32_t *shape, int *rank, int *dtype) {
+  return guard([&] {
+    need(hook_ctx, "hook context");
+    const OpContext &oc = static_cast<HookCtx *>(hook_ctx)->oc;
+    for (const auto &refs : {getOpInputRefs(oc), getOpOutputRefs(oc)})
+      for (const TensorRef &r : refs)
+        if (getTensorRefGlobalId(r) == global_id) {
+          writeShape(getTensorRefShape(r), shape, rank);
+          if (dtype) *dtype = static_cast<int>(getTensorRefDataType(r));
+          return;
+        }
+    fatal("hook: tensor " + std::to_string(global_id) + " is neither an operand nor a result of this operation");
+  });
+}
+TTRT_EXPORT int ttrt_walk_program(const ttrt_binary *bin, uint32_t program, ttrt_op_callback cb, void *user) {
+  return guard([&] {
+    need(bin, "binary"); need(reinterpret_cast<const void *>(cb), "callback");
+    walkProgram(bin->b, program, [&](OpContext oc) {
+      HookCtx h{CallbackContext{}, oc};
+      auto type = static_cast<ttmlir_amd::schema::OpType>(oc.op.scalar<std::uint8_t>(ttmlir_amd::schema::Operation::f_type_type, 0));
+      std::string dbg = getOpDebugString(oc);
+      cb(oc.index, ttmlir_amd::schema::opTypeName(type), dbg.c_str(), &h, user);
+    });
   });
 }
 TTRT_EXPORT int ttrt_stat(const char *name, int64_t *value) {

@@ -2311,6 +2311,13 @@ std::vector<TensorRef> getOpInputRefs(OpContext oc) { return wrapRefs(opRefs(oc.
 std::vector<std::uint32_t> getTensorRefShape(TensorRef ref) { return shapeFromTensorRef(ref.table); }
 ::tt::target::DataType getTensorRefDataType(TensorRef ref) { return layoutFromTensorRef(ref.table).dataType; }
 std::uint32_t getTensorRefGlobalId(TensorRef ref) { return ref.table.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0); }
+void walkProgram(Binary binary, std::uint32_t programIndex, const OpWalkFn &callback) {
+  TTRT_ASSERT(binary.handle != nullptr, "walkProgram: null binary");
+  auto programs = binary.handle->root.tables(schema::TTNNBinary::f_programs);
+  TTRT_ASSERT(programIndex < programs.size(), "walkProgram: program index out of range");
+  auto ops = programs[programIndex].tables(schema::Program::f_operations);
+  for (std::uint32_t i = 0; i < ops.size(); ++i) callback(OpContext{ops[i], i});
+}
 size_t getProgramIndex(CallbackContext cc) {
   auto *ctx = static_cast<ProgramContext *>(cc.programContext);
   TTRT_ASSERT(ctx != nullptr, "getProgramIndex: no program context");

@@ -730,6 +730,72 @@ Tensor fromDevice(const Tensor &d) {
   return h;
 }
 
+// ---- dumpTensor / loadTensor (runtime/include/tt/runtime/runtime.h:304-308; runtime/lib/ttnn/runtime.cpp:2613-2633).
+// The reference passes the tensor to its device library's flatbuffer tensor writer, whose format is not part of the
+// reference's sources.  The container here: "TTMT", version, data type, layout, rank, the extents, the payload size (all
+// little-endian, 32 bits except the 64-bit size), then the payload in the tensor's own layout, so tile order and
+// block-float bytes come back exactly as they were.
+namespace {
+constexpr char kTensorFileMagic[4] = {'T', 'T', 'M', 'T'};
+constexpr std::uint32_t kTensorFileVersion = 1;
+}  // namespace
+
+void dumpTensor(Tensor tensor, const std::string &filePath) {
+  TTRT_ASSERT(isTensorAllocated(tensor), "dumpTensor: tensor is deallocated");
+  Tensor h = tensor.handle->storage == StorageType::Device ? fromDevice(tensor) : tensor;
+  const TensorImpl &t = *h.handle;
+  TTRT_ASSERT(t.shape.size() <= 8, "dumpTensor: tensor rank above 8");
+  std::ofstream f(filePath, std::ios::binary | std::ios::trunc);
+  TTRT_ASSERT(f.good(), "dumpTensor: cannot open '" + filePath + "' for writing");
+  auto put32 = [&](std::uint32_t v) { f.write(reinterpret_cast<const char *>(&v), 4); };
+  f.write(kTensorFileMagic, 4);
+  put32(kTensorFileVersion);
+  put32(static_cast<std::uint32_t>(t.dtype));
+  put32(static_cast<std::uint32_t>(t.layout));
+  put32(static_cast<std::uint32_t>(t.shape.size()));
+  for (std::uint32_t e : t.shape) put32(e);
+  const std::uint64_t bytes = t.bytes;
+  f.write(reinterpret_cast<const char *>(&bytes), 8);
+  f.write(static_cast<const char *>(t.data.get()), static_cast<std::streamsize>(t.bytes));
+  f.flush();
+  TTRT_ASSERT(f.good(), "dumpTensor: writing '" + filePath + "' failed");
+}
+
+Tensor loadTensor(const std::string &filePath, std::optional<Device> device) {
+  std::ifstream f(filePath, std::ios::binary);
+  TTRT_ASSERT(f.good(), "loadTensor: cannot open '" + filePath + "'");
+  auto get32 = [&]() {
+    std::uint32_t v = 0;
+    f.read(reinterpret_cast<char *>(&v), 4);
+    TTRT_ASSERT(f.gcount() == 4, "loadTensor: '" + filePath + "' ends inside its header");
+    return v;
+  };
+  char magic[4] = {};
+  f.read(magic, 4);
+  TTRT_ASSERT(f.gcount() == 4 && std::memcmp(magic, kTensorFileMagic, 4) == 0, "loadTensor: '" + filePath + "' is not a tensor file");
+  const std::uint32_t version = get32();
+  TTRT_ASSERT(version == kTensorFileVersion, "loadTensor: unknown tensor file version " + std::to_string(version));
+  const std::uint32_t dtype = get32(), layout = get32(), rank = get32();
+  TTRT_ASSERT(dtype <= static_cast<std::uint32_t>(DataType::Bool), "loadTensor: unknown data type " + std::to_string(dtype));
+  TTRT_ASSERT(layout <= static_cast<std::uint32_t>(TensorLayout::Tile), "loadTensor: unknown layout " + std::to_string(layout));
+  TTRT_ASSERT(rank <= 8, "loadTensor: tensor rank above 8");
+  std::vector<std::uint32_t> shape(rank);
+  for (auto &e : shape) e = get32();
+  std::uint64_t bytes = 0;
+  f.read(reinterpret_cast<char *>(&bytes), 8);
+  TTRT_ASSERT(f.gcount() == 8, "loadTensor: '" + filePath + "' ends inside its header");
+  const DataType dt = static_cast<DataType>(dtype);
+  const TensorLayout lay = static_cast<TensorLayout>(layout);
+  TTRT_ASSERT(utils::isSupportedDataType(dt), "loadTensor: the file holds a data type tensors are never stored in");
+  TTRT_ASSERT(!utils::isBlockFormatDataType(dt) || lay == TensorLayout::Tile, "loadTensor: block-float data outside the tile layout");
+  TTRT_ASSERT(bytes == tensorBytes(shape, dt, lay), "loadTensor: the payload size does not match the shape, data type and layout");
+  Tensor t = makeHostTensor(shape, dt, lay);
+  f.read(static_cast<char *>(t.handle->data.get()), static_cast<std::streamsize>(bytes));
+  TTRT_ASSERT(static_cast<std::uint64_t>(f.gcount()) == bytes, "loadTensor: '" + filePath + "' ends inside its payload");
+  if (device.has_value()) return toDevice(t, device->handle);
+  return t;
+}
+
 // Device-side change of layout and/or dtype; the order mirrors LayoutConverter
 // (runtime/lib/ttnn/types/layout_converter.cpp:196-215, 363-379): tilize / untilize and typecast are
 // separate steps except for block-float targets, where the pack kernel tilizes on the fly.

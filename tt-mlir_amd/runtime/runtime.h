@@ -201,6 +201,16 @@ void updateTensorInPool(CallbackContext programContextHandle, TensorRef tensorRe
 void updateTensorInPool(CallbackContext programContextHandle, std::uint32_t globalId, Tensor srcTensor);
 size_t getProgramIndex(CallbackContext programContextHandle);
 
+// every operation of a program in its order, nothing is run (runtime.h:294-297; runtime/lib/ttnn/runtime.cpp:2530-2540):
+// the OpContext answers getOpDebugString / getOpLocInfo / getOpInputRefs / getOpOutputRefs
+using OpWalkFn = std::function<void(OpContext)>;
+void walkProgram(Binary executableHandle, std::uint32_t programIndex, const OpWalkFn &callback);
+
 std::vector<Tensor> submit(Device deviceHandle, Binary executableHandle, std::uint32_t programIndex, std::vector<Tensor> &inputs);
+
+// a tensor to a file and back (runtime.h:304-308).  The file keeps the tensor's own layout: tile order and block-float
+// bytes are stored as they are.  loadTensor gives a host tensor, or a device tensor when a device is passed.
+void dumpTensor(Tensor tensor, const std::string &filePath);
+Tensor loadTensor(const std::string &filePath, std::optional<Device> device = std::nullopt);
 
 }  // namespace tt::runtime
