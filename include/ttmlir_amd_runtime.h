@@ -124,8 +124,13 @@ int ttrt_hook_loc(void *hook_ctx, char *buf, size_t len);
 /* shape and data type of one of the operation's operands or results, from the binary alone (TensorRef::get_shape /
  * get_dtype: getTensorRefShape, runtime.h:263, and getTensorRefDataType); fails if global_id is neither */
 int ttrt_hook_ref_desc(void *hook_ctx, uint32_t global_id, uint32_t *shape, int *rank, int *dtype);
+/* invokeCpuOp (runtime.h:285-292): the function behind the CpuOp the hook runs for, on caller-supplied host tensors that
+ * match the op's declared inputs in number, shape and data type; outputs receives up to max_outputs new host tensors.
+ * The function needs the program's embedded library, not its tensor pool: the call also works inside ttrt_walk_program. */
+int ttrt_hook_invoke_cpu_op(void *hook_ctx, ttrt_tensor *const *inputs, uint32_t num_inputs, ttrt_tensor **outputs,
+                            uint32_t max_outputs, uint32_t *num_outputs);
 /* walkProgram (runtime.h:294-297): cb for every operation of the program in order; nothing runs and no device is needed.
- * Inside cb the hook context answers ttrt_hook_loc / input_refs / output_refs / ref_desc; there is no tensor pool, so
+ * Inside cb the hook context answers ttrt_hook_loc / input_refs / output_refs / ref_desc / invoke_cpu_op; there is no tensor pool, so
  * ttrt_hook_output and ttrt_hook_retrieve give NULL and ttrt_hook_update / ttrt_hook_program_index fail. */
 int ttrt_walk_program(const ttrt_binary *bin, uint32_t program, ttrt_op_callback cb, void *user);
 int ttrt_stat(const char *name, int64_t *value);

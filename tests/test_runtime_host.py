@@ -424,3 +424,69 @@ def test_tensor_accessors_and_empty_host_tensors():
     assert e.desc()[2] == 4 * 576
     with pytest.raises(rt.RuntimeError_, match="null argument: device"):
         rt.create_empty_tensor(None, rt.Layout(ST.Device, TL.Tile, DT.BFloat16), (32, 32))
+
+
+def test_invoke_cpu_op_on_caller_inputs(tmp_path):
+    """invokeCpuOp (runtime/lib/ttnn/runtime.cpp:2598-2611, runtime/lib/ttnn/operations/cpu/cpu.cpp:240-300): the function of a
+    CpuOp on tensors the caller brings, checked against the op's declared inputs.  It needs the program's embedded library
+    and nothing of a running program, so it is reachable from a walk of the binary: the whole CpuOp path (library from the
+    binary's bytes, WrappedTensor packing, ownership of what the callee allocated) runs here without a device."""
+    import subprocess
+    src = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "cpu_hoisted_ops.c")
+    so = tmp_path / "hoisted.so"
+    subprocess.run(["gcc", "-shared", "-fPIC", "-O1", "-o", str(so), src], check=True)
+    host = lambda shape, dt: (shape, rt.Layout(ST.Host, TL.RowMajor, dt))
+    pb = rt.ProgramBuilder()
+    pb.begin_program("hoisted")
+    pb.add_dylib(7, so.read_bytes())
+    a = pb.input((6, 5), DT.Float32, TL.RowMajor, ST.Host)
+    c = pb.input((6, 5), DT.Float32, TL.RowMajor, ST.Host)
+    v = pb.input((9,), DT.Float32, TL.RowMajor, ST.Host)
+    s0, s1 = pb.cpu_op(7, "cpu_hoisted_add_rowsum_0a1b2c3d_helper", [a, c], [host((6, 5), DT.Float32), host((6,), DT.Int32)])
+    d0, d1 = pb.cpu_op(7, "cpu_hoisted_alias_helper", [v], [host((9,), DT.Float32), host((9,), DT.Float32)])
+    (bad,) = pb.cpu_op(7, "no_such_helper", [v], [host((9,), DT.Float32)])
+    (bad2,) = pb.cpu_op(8, "cpu_hoisted_alias_helper", [v], [host((9,), DT.Float32)])
+    n = pb.unary(0, v)
+    for t in (s0, s1, d0, d1, bad, bad2, n):
+        pb.output(t)
+    pb.end_program()
+    binary = rt.Binary.load_from_memory(pb.finish())
+    rng = np.random.default_rng(5)
+    xa, xc, xv = (rng.standard_normal(s).astype(np.float32) for s in ((6, 5), (6, 5), (9,)))
+    f32 = lambda x: rt.create_owned_host_tensor(x, DT.Float32)
+    results = {}
+
+    def visit(idx, name, dbg, hook):
+        if idx == 0:
+            outs = hook.invoke_cpu_op([f32(xa), f32(xc)])
+            results[0] = [rt.to_numpy(o) for o in outs]
+            assert [o.get_layout() for o in outs] == [rt.Layout(ST.Host, TL.RowMajor, DT.Float32), rt.Layout(ST.Host, TL.RowMajor, DT.Int32)]
+            for wrong, msg in (([f32(xa)], "input count mismatch: got 1, expected 2"),
+                               ([f32(xa), f32(xc[:5])], "input 1 has the wrong shape"),
+                               ([f32(xa), rt.create_owned_host_tensor(xc.astype(np.int32), DT.Int32)], "input 1 has the wrong data type"),
+                               ([f32(xa), rt.create_owned_host_tensor(xc.view(np.uint32).astype(np.uint16), DT.BFloat16)], "must have 4-byte elements"),
+                               ([f32(xa), rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.Float32), (6, 5))], "must be a row-major host tensor")):
+                with pytest.raises(rt.RuntimeError_, match=msg):
+                    hook.invoke_cpu_op(wrong)
+        elif idx == 1:
+            for _ in range(3):   # two outputs that share one buffer: freed once, every time
+                outs = hook.invoke_cpu_op([f32(xv)])
+                results[1] = [rt.to_numpy(o) for o in outs]
+                del outs
+        elif idx == 2:
+            with pytest.raises(rt.RuntimeError_, match="could not find requested op"):
+                hook.invoke_cpu_op([f32(xv)])
+        elif idx == 3:
+            with pytest.raises(rt.RuntimeError_, match="could not find dylib corresponding to id: 8"):
+                hook.invoke_cpu_op([f32(xv)])
+        else:
+            with pytest.raises(rt.RuntimeError_, match="opContext must wrap a CpuOp, got EltwiseUnaryOp"):
+                hook.invoke_cpu_op([f32(xv)])
+    rt.walk_program(binary, 0, visit)
+    want = xa + xc
+    assert np.array_equal(results[0][0], want)
+    rows = np.zeros(6, dtype=np.float32)
+    for col in range(5):   # the callee's order of additions
+        rows = rows + want[:, col]
+    assert np.array_equal(results[0][1], rows.astype(np.int32))
+    assert np.array_equal(results[1][0], 2 * xv) and np.array_equal(results[1][1], 2 * xv)

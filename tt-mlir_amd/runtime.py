@@ -478,6 +478,13 @@ class HookContext:
         _call("ttrt_hook_program_index", self._h, ctypes.byref(i))
         return i.value
 
+    def invoke_cpu_op(self, inputs):
+        """Run the function behind the CpuOp this hook is at on host Tensors `inputs`; the list of its outputs (invokeCpuOp)."""
+        arr = (ctypes.c_void_p * max(1, len(inputs)))(*[t.h for t in inputs])
+        outs, n = (ctypes.c_void_p * 16)(), ctypes.c_uint32()
+        _call("ttrt_hook_invoke_cpu_op", self._h, arr, len(inputs), outs, 16, ctypes.byref(n))
+        return [Tensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
+
     def ref_desc(self, global_id):
         """(shape, dtype) of one of the op's operands or results as the binary declares it (TensorRef.get_shape / get_dtype)."""
         shape, rank, dt = (ctypes.c_uint32 * 8)(), ctypes.c_int(), ctypes.c_int()

@@ -265,6 +265,8 @@ TTRT_EXPORT int ttrt_submit(ttrt_device *dev, const ttrt_binary *bin, uint32_t p
 struct HookCtx {
   CallbackContext cc;
   OpContext oc;
+  const ttrt_binary *walked = nullptr;   // set by ttrt_walk_program: no program runs, cc is empty
+  uint32_t walkedProgram = 0;
 };
 static debug::CallbackFn wrapOpCallback(ttrt_op_callback cb, void *user) {
   return debug::CallbackFn([cb, user](Binary, CallbackContext cc, OpContext oc) {
@@ -367,11 +369,27 @@ TTRT_EXPORT int ttrt_hook_ref_desc(void *hook_ctx, uint32_t global_id, uint32_t 
     fatal("hook: tensor " + std::to_string(global_id) + " is neither an operand nor a result of this operation");
   });
 }
+TTRT_EXPORT int ttrt_hook_invoke_cpu_op(void *hook_ctx, ttrt_tensor *const *inputs, uint32_t num_inputs, ttrt_tensor **outputs,
+                                        uint32_t max_outputs, uint32_t *num_outputs) {
+  return guard([&] {
+    need(hook_ctx, "hook context"); need(num_outputs, "num_outputs");
+    auto *h = static_cast<HookCtx *>(hook_ctx);
+    std::vector<Tensor> ins;
+    for (uint32_t i = 0; i < num_inputs; ++i) {
+      need(inputs[i], "input tensor");
+      ins.push_back(inputs[i]->t);
+    }
+    std::vector<Tensor> outs = h->walked ? invokeCpuOpOf(h->walked->b, h->walkedProgram, h->oc, ins) : invokeCpuOp(h->cc, h->oc, ins);
+    if (outs.size() > max_outputs) throw std::runtime_error("the CpuOp returns more outputs than the caller's buffer holds");
+    *num_outputs = static_cast<uint32_t>(outs.size());
+    for (size_t i = 0; i < outs.size(); ++i) outputs[i] = new ttrt_tensor{outs[i]};
+  });
+}
 TTRT_EXPORT int ttrt_walk_program(const ttrt_binary *bin, uint32_t program, ttrt_op_callback cb, void *user) {
   return guard([&] {
     need(bin, "binary"); need(reinterpret_cast<const void *>(cb), "callback");
     walkProgram(bin->b, program, [&](OpContext oc) {
-      HookCtx h{CallbackContext{}, oc};
+      HookCtx h{CallbackContext{}, oc, bin, program};
       auto type = static_cast<ttmlir_amd::schema::OpType>(oc.op.scalar<std::uint8_t>(ttmlir_amd::schema::Operation::f_type_type, 0));
       std::string dbg = getOpDebugString(oc);
       cb(oc.index, ttmlir_amd::schema::opTypeName(type), dbg.c_str(), &h, user);

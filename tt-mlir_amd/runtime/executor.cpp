@@ -1933,14 +1933,14 @@ void *loadLibraryFromMemory(const std::uint8_t *data, size_t size) {
 
 // handles by (binary id, program index, dylib id); a binary's libraries stay loaded for the life of the process (the
 // reference unloads them with the program executor; code pages of a few KiB are not worth the unload hazards)
-WrappedFunc cpuFunction(ProgramContext &ctx, std::uint32_t dylibId, const std::string &name) {
+WrappedFunc cpuFunction(const Binary &binary, std::uint32_t programIndex, std::uint32_t dylibId, const std::string &name) {
   static std::mutex mu;
   static auto *handles = new std::map<std::tuple<std::uint64_t, std::uint32_t, std::uint32_t>, void *>;
   std::lock_guard<std::mutex> g(mu);
-  const auto key = std::make_tuple(ctx.binary.id(), ctx.programIndex, dylibId);
+  const auto key = std::make_tuple(binary.id(), programIndex, dylibId);
   auto it = handles->find(key);
   if (it == handles->end()) {
-    fb::Table program = ctx.binary.handle->root.tables(schema::TTNNBinary::f_programs)[ctx.programIndex];
+    fb::Table program = binary.handle->root.tables(schema::TTNNBinary::f_programs)[programIndex];
     auto libs = program.tables(schema::Program::f_dylibs);
     void *h = nullptr;
     for (std::uint32_t i = 0; i < libs.size() && !h; ++i) {
@@ -1956,20 +1956,25 @@ WrappedFunc cpuFunction(ProgramContext &ctx, std::uint32_t dylibId, const std::s
   return fn;
 }
 
-void runCpu(const fb::Table &op, ProgramContext &ctx) {
+// the function of a CpuOp on the given host tensors (runtime/lib/ttnn/operations/cpu/cpu.cpp:240-300): needs the binary
+// for the program's libraries, nothing else of a running program
+std::vector<Tensor> callCpuFunction(const Binary &binary, std::uint32_t programIndex, const fb::Table &op, const std::vector<Tensor> &inputs) {
   auto ins = op.tables(schema::CpuOp::f_ins), outs = op.tables(schema::CpuOp::f_outs);
-  WrappedFunc fn = cpuFunction(ctx, op.scalar<std::uint32_t>(schema::CpuOp::f_dylib_id, 0), std::string(op.string(schema::CpuOp::f_func_name)));
-  std::vector<Tensor> held;   // inputs stay alive over the call
+  TTRT_ASSERT(inputs.size() == ins.size(),
+              "CpuOp: input count mismatch: got " + std::to_string(inputs.size()) + ", expected " + std::to_string(ins.size()));
+  WrappedFunc fn = cpuFunction(binary, programIndex, op.scalar<std::uint32_t>(schema::CpuOp::f_dylib_id, 0), std::string(op.string(schema::CpuOp::f_func_name)));
   std::vector<std::vector<std::int64_t>> sizesAndStrides;
   std::vector<WrappedTensor> packed;
   sizesAndStrides.reserve(ins.size());
   for (std::uint32_t i = 0; i < ins.size(); ++i) {
-    Tensor t = ctx.get(ins[i], "cpu op input");
+    const Tensor &t = inputs[i];
+    TTRT_ASSERT(isTensorAllocated(t), "CpuOp: input " + std::to_string(i) + " is deallocated");
     // the compiler brings operands of a hoisted function to the host as dense row-major f32 / i32 / u32
     // (lib/Dialect/TTIR/Transforms/HoistCPUOps/HoistCPUOps.cpp:76-108); anything else here is a malformed program
     TTRT_ASSERT(t.handle->storage == StorageType::Host && t.handle->layout == TensorLayout::RowMajor,
                 "CpuOp: input " + std::to_string(i) + " must be a row-major host tensor");
     TTRT_ASSERT(utils::dataTypeElementSize(t.handle->dtype) == 4, "CpuOp: input " + std::to_string(i) + " must have 4-byte elements");
+    TTRT_ASSERT(t.handle->dtype == layoutFromTensorRef(ins[i]).dataType, "CpuOp: input " + std::to_string(i) + " has the wrong data type");
     const std::vector<std::uint32_t> shape = shapeFromTensorRef(ins[i]);
     TTRT_ASSERT(shape == t.handle->shape, "CpuOp: input " + std::to_string(i) + " has the wrong shape");
     std::vector<std::int64_t> ss(2 * shape.size());
@@ -1982,10 +1987,10 @@ void runCpu(const fb::Table &op, ProgramContext &ctx) {
     sizesAndStrides.push_back(std::move(ss));
     void *data = t.handle->data.get();
     packed.push_back(WrappedTensor{data, data, 0, sizesAndStrides.back().data()});
-    held.push_back(t);
   }
   WrappedTensor *result = fn(packed.data());
   TTRT_ASSERT(result != nullptr || outs.size() == 0, "CpuOp: the function returned no outputs");
+  std::vector<Tensor> outputs;
   std::map<void *, std::shared_ptr<void>> seen;   // outputs that alias one buffer share its owner
   for (std::uint32_t i = 0; i < outs.size(); ++i) {
     const WrappedTensor &w = result[i];
@@ -2000,10 +2005,19 @@ void runCpu(const fb::Table &op, ProgramContext &ctx) {
     if (it == seen.end()) it = seen.emplace(w.start, std::shared_ptr<void>(w.alignedStart, [start = w.start](void *) { std::free(start); })).first;
     t->data = it->second;
     t->version = nextTensorVersion();
-    ctx.put(outs[i], Tensor{t});
+    outputs.push_back(Tensor{t});
   }
   if (outs.size() > 0) std::free(result[0].sizesAndStrides);   // one block for all outputs
   std::free(result);
+  return outputs;
+}
+
+void runCpu(const fb::Table &op, ProgramContext &ctx) {
+  auto ins = op.tables(schema::CpuOp::f_ins), outs = op.tables(schema::CpuOp::f_outs);
+  std::vector<Tensor> inputs;   // held over the call
+  for (std::uint32_t i = 0; i < ins.size(); ++i) inputs.push_back(ctx.get(ins[i], "cpu op input"));
+  std::vector<Tensor> outputs = callCpuFunction(ctx.binary, ctx.programIndex, op, inputs);
+  for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], outputs[i]);
 }
 
 // ---- traces (runtime/lib/ttnn/operations/trace/*.cpp): a trace is a HIP graph recorded on the device's stream
@@ -2317,6 +2331,18 @@ void walkProgram(Binary binary, std::uint32_t programIndex, const OpWalkFn &call
   TTRT_ASSERT(programIndex < programs.size(), "walkProgram: program index out of range");
   auto ops = programs[programIndex].tables(schema::Program::f_operations);
   for (std::uint32_t i = 0; i < ops.size(); ++i) callback(OpContext{ops[i], i});
+}
+std::vector<Tensor> invokeCpuOpOf(const Binary &binary, std::uint32_t programIndex, OpContext oc, const std::vector<Tensor> &inputs) {
+  TTRT_ASSERT(binary.handle != nullptr, "invokeCpuOp: null binary");
+  TTRT_ASSERT(programIndex < binary.handle->root.tables(schema::TTNNBinary::f_programs).size(), "invokeCpuOp: program index out of range");
+  const auto type = static_cast<OpType>(oc.op.scalar<std::uint8_t>(schema::Operation::f_type_type, 0));
+  TTRT_ASSERT(type == OpType::CpuOp, std::string("invokeCpuOp: opContext must wrap a CpuOp, got ") + schema::opTypeName(type));
+  return callCpuFunction(binary, programIndex, oc.op.table(schema::Operation::f_type), inputs);
+}
+std::vector<Tensor> invokeCpuOp(CallbackContext cc, OpContext oc, const std::vector<Tensor> &inputs) {
+  auto *ctx = static_cast<ProgramContext *>(cc.programContext);
+  TTRT_ASSERT(ctx != nullptr, "invokeCpuOp: no program context");
+  return invokeCpuOpOf(ctx->binary, static_cast<std::uint32_t>(ctx->programIndex), oc, inputs);
 }
 size_t getProgramIndex(CallbackContext cc) {
   auto *ctx = static_cast<ProgramContext *>(cc.programContext);

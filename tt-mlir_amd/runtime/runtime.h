@@ -200,6 +200,9 @@ std::optional<Tensor> retrieveTensorFromPool(CallbackContext programContextHandl
 void updateTensorInPool(CallbackContext programContextHandle, TensorRef tensorRef, Tensor srcTensor);
 void updateTensorInPool(CallbackContext programContextHandle, std::uint32_t globalId, Tensor srcTensor);
 size_t getProgramIndex(CallbackContext programContextHandle);
+// the function behind a CpuOp on caller-supplied host tensors, which must match the op's declared inputs in number, shape
+// and data type (runtime.h:285-292; runtime/lib/ttnn/runtime.cpp:2598-2611)
+std::vector<Tensor> invokeCpuOp(CallbackContext programContextHandle, OpContext opContextHandle, const std::vector<Tensor> &inputs);
 
 // every operation of a program in its order, nothing is run (runtime.h:294-297; runtime/lib/ttnn/runtime.cpp:2530-2540):
 // the OpContext answers getOpDebugString / getOpLocInfo / getOpInputRefs / getOpOutputRefs

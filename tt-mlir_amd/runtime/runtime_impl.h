@@ -109,6 +109,8 @@ Tensor makeHostTensor(const std::vector<std::uint32_t> &shape, DataType dtype, T
 
 // layout / dtype / storage conversion used by toLayout, toHost and the layout op runners
 Tensor convertOnDevice(const Tensor &src, TensorLayout layout, DataType dtype);
+// invokeCpuOp without a running program: all it needs of one is the binary whose program carries the library
+std::vector<Tensor> invokeCpuOpOf(const Binary &binary, std::uint32_t programIndex, OpContext opContext, const std::vector<Tensor> &inputs);
 Tensor toDevice(const Tensor &hostTensor, const std::shared_ptr<DeviceState> &dev);
 Tensor fromDevice(const Tensor &deviceTensor);
 
