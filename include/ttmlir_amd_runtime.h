@@ -77,9 +77,10 @@ int ttrt_tensor_deallocate(ttrt_tensor *t, int force);                         /
 int ttrt_tensor_create_empty(ttrt_device *dev, const ttrt_layout *layout, const uint32_t *shape, int rank, ttrt_tensor **out);
 /* hasLayout (runtime.h:230); getTensorLayout (232) is the layout ttrt_tensor_desc reports */
 int ttrt_tensor_has_layout(const ttrt_tensor *t, const ttrt_layout *layout, int *has);
-/* getTensorVolume / getTensorElementSize / getTensorStride (runtime.h:142-146): elements, bytes per element (1 for
- * block-float types) and the contiguous stride in elements; stride receives up to 8 entries, any pointer may be NULL */
-int ttrt_tensor_extent(const ttrt_tensor *t, uint32_t *volume, uint32_t *element_size, int64_t *stride);
+/* getTensorVolume / getTensorLogicalVolume / getTensorElementSize / getTensorStride (runtime.h:142-146): elements in
+ * storage (the tile layout's padding included), product of the shape, bytes per element (1 for block-float types) and the
+ * contiguous stride in elements; stride receives up to 8 entries, any pointer may be NULL */
+int ttrt_tensor_extent(const ttrt_tensor *t, uint32_t *volume, uint32_t *logical_volume, uint32_t *element_size, int64_t *stride);
 /* dumpTensor / loadTensor (runtime.h:304-308): the file keeps the tensor's own layout (tile order, block-float bytes);
  * a device tensor is read back first.  load: dev NULL gives a host tensor, else the tensor is moved to that device. */
 int ttrt_tensor_dump(const ttrt_tensor *t, const char *path);

@@ -408,7 +408,7 @@ def test_tensor_accessors_and_empty_host_tensors():
     a = np.zeros((2, 3, 40), dtype=np.float32)
     t = rt.create_owned_host_tensor(a, DT.Float32)
     assert t.get_shape() == [2, 3, 40] and t.get_stride() == [120, 40, 1]
-    assert t.get_volume() == 240 and t.get_element_size() == 4 and t.get_dtype() == DT.Float32
+    assert t.get_volume() == 240 and t.get_logical_volume() == 240 and t.get_element_size() == 4 and t.get_dtype() == DT.Float32
     assert t.has_layout(rt.Layout(ST.Host, TL.RowMajor, DT.Float32))
     assert not t.has_layout(rt.Layout(ST.Host, TL.Tile, DT.Float32))
     assert not t.has_layout(rt.Layout(ST.Device, TL.RowMajor, DT.Float32))
@@ -417,7 +417,7 @@ def test_tensor_accessors_and_empty_host_tensors():
     e = rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.RowMajor, DT.BFloat16), (4, 10))
     assert e.is_allocated() and e.desc() == ((4, 10), rt.Layout(ST.Host, TL.RowMajor, DT.BFloat16), 80)
     e = rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.Float32), (2, 33, 40))
-    assert e.desc()[2] == 2 * 64 * 64 * 4
+    assert e.desc()[2] == 2 * 64 * 64 * 4 and e.get_volume() == 2 * 64 * 64 and e.get_logical_volume() == 2 * 33 * 40
     e = rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.BFP_BFloat8), (33, 40))
     assert e.desc()[2] == 4 * 1088 and e.get_element_size() == 1
     e = rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.BFP_BFloat4), (64, 64))

@@ -238,18 +238,22 @@ class Tensor:
         return bool(v.value)
 
     def _extent(self):
-        vol, esz, stride = ctypes.c_uint32(), ctypes.c_uint32(), (ctypes.c_int64 * 8)()
-        _call("ttrt_tensor_extent", self.h, ctypes.byref(vol), ctypes.byref(esz), stride)
-        return vol.value, esz.value, list(stride[: len(self.desc()[0])])
+        vol, lvol, esz, stride = ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32(), (ctypes.c_int64 * 8)()
+        _call("ttrt_tensor_extent", self.h, ctypes.byref(vol), ctypes.byref(lvol), ctypes.byref(esz), stride)
+        return vol.value, lvol.value, esz.value, list(stride[: len(self.desc()[0])])
 
     def get_volume(self):
+        """Elements in storage: the tile layout's padding counts."""
         return self._extent()[0]
 
-    def get_element_size(self):
+    def get_logical_volume(self):
         return self._extent()[1]
 
-    def get_stride(self):
+    def get_element_size(self):
         return self._extent()[2]
+
+    def get_stride(self):
+        return self._extent()[3]
 
     def get_data_buffer(self):
         """The tensor's bytes, read back and untilized if it lives on the device (getTensorDataBuffer)."""

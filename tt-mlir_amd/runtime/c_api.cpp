@@ -196,10 +196,11 @@ TTRT_EXPORT int ttrt_tensor_create_empty(ttrt_device *dev, const ttrt_layout *la
 TTRT_EXPORT int ttrt_tensor_has_layout(const ttrt_tensor *t, const ttrt_layout *layout, int *has) {
   return guard([&] { need(t, "tensor"); need(layout, "layout"); need(has, "has"); *has = hasLayout(t->t, toLayoutStruct(*layout)); });
 }
-TTRT_EXPORT int ttrt_tensor_extent(const ttrt_tensor *t, uint32_t *volume, uint32_t *element_size, int64_t *stride) {
+TTRT_EXPORT int ttrt_tensor_extent(const ttrt_tensor *t, uint32_t *volume, uint32_t *logical_volume, uint32_t *element_size, int64_t *stride) {
   return guard([&] {
     need(t, "tensor");
     if (volume) *volume = getTensorVolume(t->t);
+    if (logical_volume) *logical_volume = getTensorLogicalVolume(t->t);
     if (element_size) *element_size = getTensorElementSize(t->t);
     if (stride) {
       auto st = getTensorStride(t->t);

@@ -668,7 +668,11 @@ DataType getTensorDataType(Tensor t) { return t.handle->dtype; }
 std::uint32_t getTensorElementSize(Tensor t) {
   return utils::isBlockFormatDataType(t.handle->dtype) ? 1 : utils::dataTypeElementSize(t.handle->dtype);
 }
-std::uint32_t getTensorVolume(Tensor t) { return static_cast<std::uint32_t>(volume(t.handle->shape)); }
+// physical volume: the elements the storage holds, the tile layout's padding included (runtime/lib/ttnn/runtime.cpp:542-552)
+std::uint32_t getTensorVolume(Tensor t) {
+  return static_cast<std::uint32_t>(t.handle->layout == TensorLayout::Tile ? paddedVolume(t.handle->shape) : volume(t.handle->shape));
+}
+std::uint32_t getTensorLogicalVolume(Tensor t) { return static_cast<std::uint32_t>(volume(t.handle->shape)); }
 std::vector<std::uint32_t> getTensorShape(Tensor t) { return t.handle->shape; }
 std::vector<std::int64_t> getTensorStride(Tensor t) { return utils::calculateStride(t.handle->shape); }
 TensorDesc getTensorDesc(Tensor t) { return TensorDesc{t.handle->shape, getTensorStride(t), t.handle->dtype}; }

@@ -167,7 +167,8 @@ bool isTensorAllocated(Tensor tensor);
 ::tt::target::DataType getTensorDataType(Tensor tensor);
 std::vector<std::byte> getTensorDataBuffer(Tensor tensor);
 std::uint32_t getTensorElementSize(Tensor tensor);
-std::uint32_t getTensorVolume(Tensor tensor);
+std::uint32_t getTensorVolume(Tensor tensor);          // elements in storage, tile padding included
+std::uint32_t getTensorLogicalVolume(Tensor tensor);   // product of the shape
 std::vector<std::uint32_t> getTensorShape(Tensor tensor);
 std::vector<std::int64_t> getTensorStride(Tensor tensor);
 TensorDesc getTensorDesc(Tensor tensor);
