@@ -490,3 +490,42 @@ def test_invoke_cpu_op_on_caller_inputs(tmp_path):
         rows = rows + want[:, col]
     assert np.array_equal(results[0][1], rows.astype(np.int32))
     assert np.array_equal(results[1][0], 2 * xv) and np.array_equal(results[1][1], 2 * xv)
+
+
+def _damaged_binaries_never_crash_the_reader(seed, cases):
+    """Body of the test below, run in a child process: a reader that walks off a damaged buffer would take the
+    process down, and that must show as a failed test rather than a dead test run."""
+    import random
+    rnd = random.Random(seed)
+    bases = [programs.c1_matmul(), programs.c4_mlp(tokens=64, hidden=128, ffn=256)]
+    loaded = 0
+    for _ in range(cases):
+        data = bytearray(rnd.choice(bases))
+        for _ in range(rnd.choice([1, 1, 2, 4, 8])):
+            pos, mode = rnd.randrange(len(data)), rnd.randrange(4)
+            data[pos] = (rnd.randrange(256), data[pos] ^ (1 << rnd.randrange(8)), 0xFF, 0)[mode]
+        if rnd.random() < 0.1:
+            data = data[: rnd.randrange(len(data))]
+        try:
+            b = rt.Binary.load_from_memory(bytes(data))
+            for p in range(min(b.get_num_programs(), 4)):
+                b.get_program_name(p), b.get_program_inputs(p), b.get_program_outputs(p)
+                b.get_program_ops_as_text(p), b.get_program_ops_as_json(p), b.get_program_inputs_as_json(p)
+                rt.walk_program(b, p, lambda i, name, dbg, h: [h.ref_desc(g) for g in h.input_refs() + h.output_refs()] + [h.loc()])
+            loaded += 1
+        except rt.RuntimeError_:
+            pass
+    return loaded
+
+
+def test_damaged_binaries_are_rejected_or_read_but_never_crash():
+    # bit flips, byte stamps and truncations of two valid binaries: every access either raises the runtime's error or
+    # returns; the offsets a flatbuffer is made of are all checked against the buffer before they are followed
+    import subprocess
+    import sys
+    code = ("import sys; sys.path.insert(0, %r); sys.path.insert(0, %r); import conftest, test_runtime_host as t; "
+            "print(sum(t._damaged_binaries_never_crash_the_reader(s, 400) for s in (11, 12, 13)))") % (
+        os.path.dirname(os.path.abspath(__file__)), os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, "the reader crashed on a damaged binary (exit %d): %s" % (r.returncode, r.stderr[-400:])
+    assert 0 < int(r.stdout.strip().splitlines()[-1]) < 1200   # some damage is harmless, some must be caught

@@ -70,7 +70,7 @@ def declared_functions():
 
 def _ck(status, what):
     if status != 0:
-        raise RuntimeError_("%s: %s" % (what, lib().ttrt_last_error().decode()))
+        raise RuntimeError_("%s: %s" % (what, lib().ttrt_last_error().decode("utf-8", "replace")))
 
 
 def _call(name, *args):
@@ -110,7 +110,7 @@ class Binary:
     def get_program_name(self, i):
         buf = ctypes.create_string_buffer(256)
         _call("ttrt_binary_program_name", self.h, i, buf, 256)
-        return buf.value.decode()
+        return buf.value.decode("utf-8", "replace")
 
     def is_program_private(self, i):
         v = ctypes.c_int()
@@ -136,7 +136,7 @@ class Binary:
     def get_program_ops_as_text(self, program):
         buf = ctypes.create_string_buffer(1 << 16)
         _call("ttrt_binary_ops_text", self.h, program, buf, 1 << 16)
-        return buf.value.decode()
+        return buf.value.decode("utf-8", "replace")
 
     def _json(self, program, which):
         import json
@@ -144,7 +144,7 @@ class Binary:
         _call("ttrt_binary_program_json", self.h, program, which, None, 0, ctypes.byref(need))
         buf = ctypes.create_string_buffer(need.value + 1)
         _call("ttrt_binary_program_json", self.h, program, which, buf, need.value + 1, None)
-        return json.loads(buf.value.decode())
+        return json.loads(buf.value.decode("utf-8", "replace"))
 
     def get_program_inputs_as_json(self, program):
         """Parsed JSON view of the program's input TensorRefs (Binary.getProgramInputsAsJson)."""
@@ -175,12 +175,12 @@ class Binary:
             arr = (raw.view(np.uint16).astype(np.uint32) << 16).view(np.float32).reshape(shp)
         else:
             arr = raw.view(_NP_DTYPE[dtype.value]).reshape(shp)
-        return name.value.decode(), arr
+        return name.value.decode("utf-8", "replace"), arr
 
     def info(self):
         ident, ver = ctypes.create_string_buffer(5), ctypes.create_string_buffer(64)
         _call("ttrt_binary_info", self.h, ident, ver, 64)
-        return ident.value.decode(), ver.value.decode()
+        return ident.value.decode("utf-8", "replace"), ver.value.decode("utf-8", "replace")
 
     def __del__(self):
         try:
@@ -196,7 +196,7 @@ class Device:
     def name(self):
         buf = ctypes.create_string_buffer(256)
         _call("ttrt_device_name", self.h, buf, 256)
-        return buf.value.decode()
+        return buf.value.decode("utf-8", "replace")
 
 
 class Tensor:
@@ -453,7 +453,7 @@ class HookContext:
     def loc(self):
         buf = ctypes.create_string_buffer(512)
         _call("ttrt_hook_loc", self._h, buf, 512)
-        return buf.value.decode()
+        return buf.value.decode("utf-8", "replace")
 
     def _refs(self, fn):
         ids, n = (ctypes.c_uint32 * 64)(), ctypes.c_uint32()
@@ -498,7 +498,7 @@ class HookContext:
 
 def _op_trampoline(fn):
     def tramp(idx, name, dbg, hook, user):
-        fn(idx, name.decode(), dbg.decode(), HookContext(hook))
+        fn(idx, name.decode("utf-8", "replace"), dbg.decode("utf-8", "replace"), HookContext(hook))
     return _CB_TYPE(tramp)
 
 
@@ -590,7 +590,7 @@ class ProgramBuilder:
     def last_op_loc(self):
         buf = ctypes.create_string_buffer(512)
         _call("ttrt_pb_last_op_loc", self.h, buf, 512)
-        return buf.value.decode()
+        return buf.value.decode("utf-8", "replace")
 
     def golden(self, loc, array, dtype, name=""):
         """Embed an expected tensor for the op at `loc`: numpy array (bf16 as uint16 bits) of runtime dtype `dtype`."""
