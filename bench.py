@@ -359,7 +359,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 MEASURED_ON = {"ttm_linear.hip": ("e4074d055f65",), "ttm_bfp.hip": ("8e9736544aea",), "ttm_layout.hip": ("c2d080a6c0c5",),
                "ttm_decode.hip": ("8bbb69b8561a",), "ttm_rowwise.hip": ("ad15392e8bae", "ff3e580c91ab"),
-               "ttm_eltwise.hip": ("56692d4eb0d8", "538c0c60dffa")}
+               "ttm_eltwise.hip": ("56692d4eb0d8", "538c0c60dffa", "3bec0c51416e")}
 
 
 def measured_traffic(name):

@@ -310,7 +310,9 @@ static inline float unary_f32(int op, float x, float p) {
   case U_ISFINITE: return isfinite(x) ? 1.0f : 0.0f;
   case U_LOGICALNOT: return x == 0.0f ? 1.0f : 0.0f;
   case U_NEG: return -x;
-  case U_RELU: return x > 0.0f ? x : 0.0f;
+  /* max(x, 0) with NaN kept, as linalg.max / arith.maximumf (lib/Conversion/TTIRToLinalg/EltwiseUnary.cpp:508-541) and
+   * torch.relu (tools/golden/mapping.py:7437, 9052) have it; -0.0 gives +0.0 as maximumf does (torch keeps -0.0) */
+  case U_RELU: return x > 0.0f ? x : (x != x ? x : 0.0f);
   case U_SQRT: return sqrtf(x);
   case U_RSQRT: return 1.0f / sqrtf(x);
   case U_SIGMOID: return 1.0f / (1.0f + expf(-x));

@@ -60,6 +60,43 @@ def test_unary_matches_torch(orc, name, fn):
     assert np.allclose(orc.unary(name, x), want, rtol=2e-6, atol=2e-7)
 
 
+def test_remaining_unary_ops_match_torch_on_ordinary_and_special_values(orc):
+    """tan / atan / erfc / expm1 / leaky_relu / relu6 / isfinite / logical_not against the torch routines the goldens call
+    (tools/golden/mapping.py:3954-3971 leaky_relu, 2586-2605 and 5076-5079 logical_not, 5868-5872 isfinite), and every unary op
+    on the values where a plausible mistake shows: both zeros, both infinities, NaN, the knees of the piecewise ops."""
+    x = rnd((1000,), 27, 3.0)
+    t = torch.from_numpy(x).double()
+    for name, want in (("tan", torch.tan(t)), ("atan", torch.atan(t)), ("erfc", torch.erfc(t)), ("expm1", torch.expm1(t)),
+                       ("relu6", F.relu6(t))):
+        assert np.allclose(orc.unary(name, x), want.float().numpy(), rtol=3e-6, atol=2e-7), name
+    for slope in (0.01, 0.2, -0.5):
+        assert np.array_equal(orc.unary("leaky_relu", x, slope), F.leaky_relu(torch.from_numpy(x), negative_slope=slope).numpy())
+    sp = np.array([0.0, -0.0, 1.0, -1.0, 6.0, 6.5, -3.0, 3.0, np.inf, -np.inf, np.nan, 1e-30, -1e-30], dtype=np.float32)
+    ts = torch.from_numpy(sp)
+    assert np.array_equal(orc.unary("isfinite", sp), torch.isfinite(ts).float().numpy())
+    assert np.array_equal(orc.unary("logical_not", sp), torch.logical_not(ts).float().numpy())   # NaN and the infinities are true
+    fns = dict(abs=torch.abs, neg=torch.neg, relu=torch.relu, relu6=F.relu6, sign=torch.sign, floor=torch.floor, ceil=torch.ceil,
+               sigmoid=torch.sigmoid, silu=F.silu, gelu=F.gelu, tanh=torch.tanh, erf=torch.erf, erfc=torch.erfc, exp=torch.exp,
+               expm1=torch.expm1, atan=torch.atan, hardsigmoid=F.hardsigmoid, sqrt=torch.sqrt, rsqrt=torch.rsqrt,
+               reciprocal=torch.reciprocal, log=torch.log, log1p=torch.log1p, asinh=torch.asinh)
+    for name, fn in fns.items():
+        got, want = orc.unary(name, sp), fn(ts.double()).float().numpy()   # in double: torch's own fp32 gelu is off by 1e-4 at -3
+        assert np.allclose(got, want, rtol=1e-5, atol=1e-37, equal_nan=True), (name, got, want)
+        both = np.isfinite(got) & (got == 0)
+        # relu(-0.0): +0.0 like arith.maximumf of the reference's CPU lowering, where torch.relu keeps -0.0
+        if name != "relu":
+            assert np.array_equal(np.signbit(got[both]), np.signbit(want[both])), (name, got, want)
+
+
+def test_comparison_binaries_match_numpy_including_nan(orc):
+    a = np.array([[1.0, 2.0, np.nan, -0.0, np.inf, 3.0]], dtype=np.float32)
+    b = np.array([[1.0], [3.0], [np.nan], [0.0], [np.inf], [-np.inf]], dtype=np.float32)
+    with np.errstate(invalid="ignore"):
+        for name, fn in (("eq", np.equal), ("ne", np.not_equal), ("ge", np.greater_equal), ("gt", np.greater), ("le", np.less_equal),
+                         ("lt", np.less)):
+            assert np.array_equal(orc.binary(name, a, b), fn(a, b).astype(np.float32)), name
+
+
 def test_gelu_doc_example(orc):
     # include/ttmlir/Dialect/TTIR/IR/TTIROps.td:529-537: gelu([1, -1, 0...]) -> [0.8413, -0.1587, 0]
     y = orc.unary("gelu", np.array([1.0, -1.0, 0.0], dtype=np.float32))

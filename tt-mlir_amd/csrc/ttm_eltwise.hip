@@ -32,7 +32,7 @@ __device__ __forceinline__ float unary_op(float x, float p, float p2 = 0.0f) {
   case U_ISFINITE: return isfinite(x) ? 1.0f : 0.0f;
   case U_LOGICALNOT: return x == 0.0f ? 1.0f : 0.0f;
   case U_NEG: return -x;
-  case U_RELU: return x > 0.0f ? x : 0.0f;
+  case U_RELU: return x > 0.0f ? x : (x != x ? x : 0.0f);   // NaN stays NaN, as arith.maximumf and torch.relu have it
   case U_SQRT: return sqrtf(x);
   case U_RSQRT: return 1.0f / sqrtf(x);
   case U_SIGMOID: return 1.0f / (1.0f + expf(-x));
