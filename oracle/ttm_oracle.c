@@ -488,8 +488,11 @@ void orc_reduce_f32(int op, const float *x, float *out, int64_t outer, int64_t d
       float acc = (op == 2) ? -INFINITY : (op == 3 ? INFINITY : 0.0f);
       for (int64_t d = 0; d < dim; ++d) {
         float v = p[d * inner];
-        if (op == 2) acc = v > acc ? v : acc;
-        else if (op == 3) acc = v < acc ? v : acc;
+        /* a NaN anywhere gives NaN: torch.max / torch.min of the goldens (tools/golden/mapping.py:5189-5220, 2815-2856) and
+         * tosa.reduce_max / reduce_min of the CPU lowering (lib/Conversion/TTIRToLinalg/Reduction.cpp:133-136), whose
+         * default is to propagate */
+        if (op == 2) acc = (v > acc || v != v) ? v : acc;
+        else if (op == 3) acc = (v < acc || v != v) ? v : acc;
         else acc += v;
       }
       if (op == 1) acc = acc / (float)dim;

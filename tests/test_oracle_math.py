@@ -136,6 +136,22 @@ def test_softmax_and_reduce(orc):
     assert orc.reduce("sum", x, -1, keepdim=True).shape == (3, 5, 1)
 
 
+def test_rowwise_ops_on_special_values_match_torch(orc):
+    """NaN, infinities and signed zeros through the reductions, softmax, RMSNorm and argmax: a NaN anywhere in a row makes
+    max and min NaN (torch.max / torch.min, tools/golden/mapping.py:5189-5220, 2815-2856), a row of -inf gives a NaN softmax,
+    the first NaN wins argmax."""
+    x = np.array([[1.0, np.nan, 3.0, -2.0], [np.inf, 1.0, 2.0, 0.0], [-np.inf, -np.inf, 1.0, 0.0], [-np.inf] * 4,
+                  [np.inf, np.inf, 0.0, 0.0], [0.0, -0.0, 0.0, -0.0], [5.0, 4.0, np.nan, np.nan]], dtype=np.float32)
+    t = torch.from_numpy(x)
+    for op, fn in (("sum", lambda t: t.sum(-1)), ("mean", lambda t: t.mean(-1)), ("max", lambda t: t.max(-1).values),
+                   ("min", lambda t: t.min(-1).values)):
+        assert np.array_equal(orc.reduce(op, x, -1), fn(t).numpy(), equal_nan=True), op
+        assert np.array_equal(orc.reduce(op, x.T.copy(), 0), fn(t).numpy(), equal_nan=True), op
+    assert np.allclose(orc.softmax(x, -1), F.softmax(t, -1).numpy(), rtol=1e-6, equal_nan=True)
+    assert np.array_equal(orc.rms_norm(x, None, None, 1e-5), F.rms_norm(t, (4,), None, 1e-5).numpy(), equal_nan=True)
+    assert np.array_equal(orc.argmax(x, -1), t.argmax(-1).numpy())
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_sdpa_matches_torch(orc, causal):
     B, Hq, Hkv, S, D = 2, 4, 2, 24, 16
