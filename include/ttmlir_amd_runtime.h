@@ -67,6 +67,11 @@ int ttrt_device_name(ttrt_device *dev, char *buf, size_t len);
  * (contiguous) and counts elements */
 int ttrt_tensor_create_host(const void *data, const uint32_t *shape, int rank, const int64_t *stride, uint32_t itemsize,
                             int dtype, int borrowed, ttrt_tensor **out);
+/* createUnsafeBorrowedHostTensor (runtime.h:70-76): a borrowed tensor over the buffer of an owned row-major host tensor,
+ * no copy; it must not be used after the owner's buffer is gone */
+int ttrt_tensor_create_unsafe_borrowed(const ttrt_tensor *owned, ttrt_tensor **out);
+/* address of a host tensor's buffer (NULL once deallocated); what the reference's tests read through getRawHostDataPtr */
+int ttrt_tensor_host_data(const ttrt_tensor *t, void **data);
 void ttrt_tensor_free(ttrt_tensor *t);
 int ttrt_tensor_desc(const ttrt_tensor *t, uint32_t *shape, int *rank, ttrt_layout *layout, uint64_t *bytes);
 int ttrt_tensor_is_allocated(const ttrt_tensor *t, int *allocated);

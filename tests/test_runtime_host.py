@@ -529,3 +529,30 @@ def test_damaged_binaries_are_rejected_or_read_but_never_crash():
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, "the reader crashed on a damaged binary (exit %d): %s" % (r.returncode, r.stderr[-400:])
     assert 0 < int(r.stdout.strip().splitlines()[-1]) < 1200   # some damage is harmless, some must be caught
+
+
+def test_reference_gtest_dump_and_load_float32_tensor(tmp_path):
+    # runtime/test/ttnn/gtest/test_tensor_serialization.cpp:40-78 (TestDumpAndLoadFloat32Tensor), its data and its checks
+    data = np.array([1.0, 2.5, 3.14159, -1.0, 0.0, 42.0, -3.14159, 1e6, -1e-6], dtype=np.float32).reshape(3, 3)
+    original = rt.create_owned_host_tensor(data, DT.Float32)
+    path = tmp_path / "test_float32_tensor.bin"
+    rt.dump_tensor(original, path)
+    loaded = rt.load_tensor(path)
+    assert original.get_shape() == loaded.get_shape() == [3, 3]
+    assert original.get_dtype() == loaded.get_dtype() == DT.Float32
+    a, b = original.get_data_buffer(), loaded.get_data_buffer()
+    assert len(a) == len(b) == 36 and a == b
+
+
+def test_reference_gtest_unsafe_borrowed_host_tensor_aliases_owned_buffer():
+    # runtime/test/ttnn/gtest/test_unsafe_borrowed_host_tensor.cpp:26-51 (AliasesOwnedBuffer)
+    owned = rt.create_owned_host_tensor(np.array([[1.0, 2.0], [3.0, 4.0]], dtype=np.float32), DT.Float32)
+    borrowed = rt.create_unsafe_borrowed_host_tensor(owned)
+    assert rt.host_data_ptr(owned) == rt.host_data_ptr(borrowed) != 0
+    assert owned.get_shape() == borrowed.get_shape() and owned.get_dtype() == borrowed.get_dtype()
+    # one buffer: what is copied into the owner is what the borrower reads
+    rt.memcpy_tensor(owned, rt.create_owned_host_tensor(np.full((2, 2), 7.0, dtype=np.float32), DT.Float32))
+    assert np.array_equal(rt.to_numpy(borrowed), np.full((2, 2), 7.0, dtype=np.float32))
+    # only row-major host tensors have a buffer that can be borrowed this way (runtime/lib/ttnn/runtime.cpp:287-298)
+    with pytest.raises(rt.RuntimeError_, match="requires ROW_MAJOR layout"):
+        rt.create_unsafe_borrowed_host_tensor(rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.Float32), (32, 32)))

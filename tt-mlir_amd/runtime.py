@@ -328,6 +328,21 @@ def from_torch(t, borrowed=False):
     return _host(arr, dt, borrowed)
 
 
+def create_unsafe_borrowed_host_tensor(owned):
+    """A borrowed Tensor over the buffer of an owned row-major host Tensor, no copy (createUnsafeBorrowedHostTensor); the
+    returned object keeps `owned` alive, which is what the C++ caller has to see to itself."""
+    h = ctypes.c_void_p()
+    _call("ttrt_tensor_create_unsafe_borrowed", owned.h, ctypes.byref(h))
+    return Tensor(h, keepalive=owned)
+
+
+def host_data_ptr(tensor):
+    """Address of a host tensor's buffer, 0 once it is deallocated."""
+    p = ctypes.c_void_p()
+    _call("ttrt_tensor_host_data", tensor.h, ctypes.byref(p))
+    return p.value or 0
+
+
 def create_empty_tensor(device, layout, shape):
     """Uninitialised tensor in `layout` (createEmptyTensor); `device` may be None for host storage."""
     sh, rank = _shape_arg(shape)
@@ -386,6 +401,11 @@ def deallocate_tensor(tensor, force=False):
 def memcpy(dst_array, src_tensor, target_dtype=None):
     """memcpy(void*, Tensor, optional<DataType>) into a numpy array."""
     _call("ttrt_memcpy_out", ctypes.c_void_p(dst_array.ctypes.data), src_tensor.h, -1 if target_dtype is None else target_dtype)
+
+
+def memcpy_tensor(dst_tensor, src_tensor):
+    """memcpy(Tensor, Tensor): the payload of src into dst, same size and data type."""
+    _call("ttrt_memcpy_tensor", dst_tensor.h, src_tensor.h)
 
 
 def to_numpy(tensor, target_dtype=None):

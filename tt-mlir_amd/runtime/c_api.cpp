@@ -161,6 +161,16 @@ TTRT_EXPORT int ttrt_tensor_create_host(const void *data, const uint32_t *shape,
     *out = new ttrt_tensor{t};
   });
 }
+TTRT_EXPORT int ttrt_tensor_create_unsafe_borrowed(const ttrt_tensor *owned, ttrt_tensor **out) {
+  return guard([&] { need(owned, "tensor"); need(out, "out"); *out = new ttrt_tensor{createUnsafeBorrowedHostTensor(owned->t)}; });
+}
+TTRT_EXPORT int ttrt_tensor_host_data(const ttrt_tensor *t, void **data) {
+  return guard([&] {
+    need(t, "tensor"); need(data, "data");
+    if (t->t.handle->storage != StorageType::Host) throw std::runtime_error("the tensor is not on the host");
+    *data = t->t.handle->data.get();
+  });
+}
 TTRT_EXPORT void ttrt_tensor_free(ttrt_tensor *t) { delete t; }
 TTRT_EXPORT int ttrt_tensor_desc(const ttrt_tensor *t, uint32_t *shape, int *rank, ttrt_layout *layout, uint64_t *bytes) {
   return guard([&] {

@@ -657,6 +657,13 @@ Tensor createBorrowedHostTensor(void *data, const std::vector<std::uint32_t> &sh
   return Tensor{t};
 }
 
+Tensor createUnsafeBorrowedHostTensor(Tensor owned) {
+  TTRT_ASSERT(isTensorAllocated(owned) && owned.handle->storage == StorageType::Host, "createUnsafeBorrowedHostTensor requires a host tensor");
+  TTRT_ASSERT(owned.handle->layout == TensorLayout::RowMajor, "createUnsafeBorrowedHostTensor requires ROW_MAJOR layout");
+  const TensorDesc desc = getTensorDesc(owned);
+  return createBorrowedHostTensor(owned.handle->data.get(), desc.shape, desc.stride, utils::dataTypeElementSize(desc.dataType), desc.dataType);
+}
+
 Tensor createEmptyTensor(Device device, Layout layout, const std::vector<std::uint32_t> &shape, const std::vector<std::int64_t> &,
                          std::uint32_t) {
   if (layout.storageType == StorageType::Device) return makeDeviceTensor(device.handle, shape, layout.dataType, layout.layout);

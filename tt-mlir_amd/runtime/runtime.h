@@ -160,6 +160,9 @@ Tensor createBorrowedHostTensor(void *data, const std::vector<std::uint32_t> &sh
                                 std::uint32_t itemsize, ::tt::target::DataType dataType);
 Tensor createOwnedHostTensor(const void *data, const std::vector<std::uint32_t> &shape, const std::vector<std::int64_t> &stride,
                              std::uint32_t itemsize, ::tt::target::DataType dataType);
+// borrowed host tensor over the buffer of an owned row-major host tensor, no copy; it must not outlive the owner's buffer
+// (runtime.h:70-76; runtime/lib/ttnn/runtime.cpp:283-304)
+Tensor createUnsafeBorrowedHostTensor(Tensor ownedHostTensor);
 Tensor createEmptyTensor(Device device, Layout layout, const std::vector<std::uint32_t> &shape,
                          const std::vector<std::int64_t> &stride, std::uint32_t itemsize);
 
