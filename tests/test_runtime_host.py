@@ -429,7 +429,9 @@ def test_tensor_accessors_and_empty_host_tensors():
 def test_invoke_cpu_op_on_caller_inputs(tmp_path):
     """invokeCpuOp (runtime/lib/ttnn/runtime.cpp:2598-2611, runtime/lib/ttnn/operations/cpu/cpu.cpp:240-300): the function of a
     CpuOp on tensors the caller brings, checked against the op's declared inputs.  It needs the program's embedded library
-    and nothing of a running program, so it is reachable from a walk of the binary: the whole CpuOp path (library from the
+    and nothing of a running program, so it is reachable from a walk of the binary (the reference's test of the call,
+    runtime/test/ttnn/python/n150/test_cpu_hoisting_api.py:44-120, makes it from a post-op hook of a running program and
+    checks the sum of two caller-supplied tensors, as here): the whole CpuOp path (library from the
     binary's bytes, WrappedTensor packing, ownership of what the callee allocated) runs here without a device."""
     import subprocess
     src = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "cpu_hoisted_ops.c")
@@ -556,3 +558,22 @@ def test_reference_gtest_unsafe_borrowed_host_tensor_aliases_owned_buffer():
     # only row-major host tensors have a buffer that can be borrowed this way (runtime/lib/ttnn/runtime.cpp:287-298)
     with pytest.raises(rt.RuntimeError_, match="requires ROW_MAJOR layout"):
         rt.create_unsafe_borrowed_host_tensor(rt.create_empty_tensor(None, rt.Layout(ST.Host, TL.Tile, DT.Float32), (32, 32)))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_reference_tensor_buffer_api(dtype):
+    # runtime/test/ttnn/python/n150/test_runtime_api.py:22-57 (test_tensor_buffer_api): a borrowed host tensor reports the
+    # shape, stride, element size, volume, data type and bytes of the memory it was made from
+    import torch
+    tdt = getattr(torch, dtype)
+    t = torch.randn((64, 128), dtype=tdt)
+    rtt = rt.from_torch(t, borrowed=True)
+    desc = rtt.get_tensor_desc()
+    assert desc.shape == rtt.get_shape() and desc.stride == rtt.get_stride()
+    assert desc.dtype == rtt.get_dtype() and desc.item_size == rtt.get_element_size()
+    assert rtt.get_shape() == [64, 128] and rtt.get_stride() == list(t.stride())
+    assert rtt.get_element_size() == t.element_size() and rtt.get_volume() == t.numel()
+    assert rtt.get_dtype() == (DT.Float32 if dtype == "float32" else DT.BFloat16)
+    raw = rtt.get_data_buffer()
+    assert len(raw) == rtt.get_volume() * rtt.get_element_size()
+    assert torch.equal(torch.frombuffer(raw, dtype=tdt).reshape(rtt.get_shape()), t)

@@ -255,6 +255,12 @@ class Tensor:
     def get_stride(self):
         return self._extent()[3]
 
+    def get_tensor_desc(self):
+        """shape / stride / dtype / item_size in one object, as the reference's TensorDesc binding has them."""
+        import types
+        return types.SimpleNamespace(shape=self.get_shape(), stride=self.get_stride(), dtype=self.get_dtype(),
+                                     item_size=self.get_element_size())
+
     def get_data_buffer(self):
         """The tensor's bytes, read back and untilized if it lives on the device (getTensorDataBuffer)."""
         return bytearray(to_numpy(self).tobytes())
