@@ -17,6 +17,10 @@
  *    tiles, row-major over tiles, each tile 4 faces of 16x16 (face order (0,0) (0,1) (1,0) (1,1)),
  *    zero padded (lib/Dialect/TTCore/IR/TTCoreOpsTypes.cpp:1857-1903).  Block-float tiles are
  *    1088 B (bfp8_b) / 576 B (bfp4_b): 64 shared-exponent bytes then the mantissas (:1875-1887).
+ *  - the entry points take logical extents and no buffer sizes: a TILE operand or result of logical
+ *    shape [batch, R, C] must be backed by the whole padded tensor, batch * ceil(R/32) * ceil(C/32)
+ *    tiles, and the kernels read and write all of it (a [1, C] tensor is one full tile row of 32
+ *    rows).  A buffer sized for the logical extents alone is read and written past its end.
  */
 #ifndef TTMLIR_AMD_HIP_H
 #define TTMLIR_AMD_HIP_H
@@ -211,7 +215,9 @@ int ttm_typecast(const void *in, int src_dtype, void *out, int dst_dtype, int64_
 /* ---- row-wise ops on TILE tensors [batch, rows, cols], reduced over the last dim, fp32 math.
  * rms_norm: ::ttnn::rms_norm (runtime/lib/ttnn/operations/normalization/rms_norm.cpp:10-49;
  *   op order lib/Dialect/TTIR/Transforms/DecomposeComposites.cpp:47-111); weight / bias are [cols]
- *   vectors of the same dtype, TILE (a [1,cols] tensor) or ROW_MAJOR, may be NULL.
+ *   vectors of the same dtype, TILE (a [1,cols] tensor) or ROW_MAJOR, may be NULL.  A ROW_MAJOR vector is read in
+ *   16-byte chunks up to the next multiple of 32 elements (what lies past cols is never used): its allocation must
+ *   reach that far, as every allocation of at least 128-byte granularity does.
  * softmax: ::ttnn::softmax over the last dim, always max-subtracted
  *   (normalization/softmax.cpp:12-36; lib/Conversion/TTIRToLinalg/TTIRToLinalg.cpp:944-1017).
  * reduce: ::ttnn::sum/mean/max/min over the last dim (reduction/reduction.cpp:13-63); op is
