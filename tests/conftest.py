@@ -26,6 +26,9 @@ def orc():
 def hip():
     from ttmlir_amd import hip as h
     h.lib()  # raises if the native library is missing: no fallback
+    # a kernel that runs past a buffer faults the whole device: every pointer a test hands over is checked against the
+    # extent the kernels touch before the call goes out
+    h.check_buffers(True)
     return h
 
 

@@ -42,3 +42,59 @@ def test_no_oracle_in_product_path():
                 src = open(os.path.join(d, f), errors="ignore").read()
                 assert not re.search(r"(import|from)\s+oracle|libttm_oracle|oracle[./]|load_oracle", src), \
                     "product file reaches into the oracle: " + f
+
+
+def test_buffer_extent_check_of_the_python_binding(hip):
+    """The entry points take logical extents and no buffer sizes.  With check_buffers on, a pointer made by hip.ptr() must have
+    the bytes behind it that the kernels touch: a [1, C] tile tensor is a full tile row of 32 rows, a reduction's result a
+    full [.., rows, 1] tile per tile row.  The check raises before the library is called (no GPU needed to see it)."""
+    import pytest
+    import torch
+    was_on = hip._check_buffers
+    hip.check_buffers(True)
+    try:
+        C = 128256
+        one_row = torch.zeros(1, C, dtype=torch.bfloat16)               # 256 KB where the kernels read 32 padded rows
+        padded = torch.zeros(32, (C + 31) // 32 * 32, dtype=torch.bfloat16)
+        with pytest.raises(hip.TTMError, match="tile input .argument 0. has 256512 bytes, the kernels touch 8208384"):
+            hip.call("ttm_softmax_lastdim", hip.ptr(one_row), hip.ptr(padded), hip.BF16, 1, 1, C, None)
+        with pytest.raises(hip.TTMError, match="tile output .argument 1."):
+            hip.call("ttm_softmax_lastdim", hip.ptr(padded), hip.ptr(one_row), hip.BF16, 1, 1, C, None)
+        with pytest.raises(hip.TTMError, match="tile output .*rows, 1"):
+            hip.call("ttm_reduce_lastdim", 0, hip.ptr(padded), hip.ptr(torch.zeros(32, dtype=torch.bfloat16)), hip.BF16, 1, 32, C, None)
+        with pytest.raises(hip.TTMError, match="weight .argument 1."):
+            hip.call("ttm_rms_norm", hip.ptr(padded), hip.ptr(torch.zeros(C, dtype=torch.bfloat16)), hip.TILE, None, hip.TILE, hip.ptr(padded),
+                     hip.BF16, 1, 32, C, 1e-5, None)
+        with pytest.raises(hip.TTMError, match="row-major output"):
+            hip.call("ttm_untilize", hip.ptr(padded), hip.ptr(one_row), 1, 32, C, 2, None)
+        with pytest.raises(hip.TTMError, match="ttm_eltwise_unary: the input"):
+            hip.call("ttm_eltwise_unary", 0, hip.ptr(torch.zeros(40, 50)), hip.ptr(torch.zeros(64, 64)), hip.F32, hip.TILE, 1, 40, 50, 0.0, None)
+        # buffers of the right size pass the check, as does anything that is not a pointer made by ptr()
+        ok = [("ttm_softmax_lastdim", (hip.ptr(padded), hip.ptr(padded), hip.BF16, 1, 32, C, None)),
+              ("ttm_softmax_lastdim", (hip.ptr(padded), hip.ptr(padded), hip.BF16, 1, 1, C, None)),
+              ("ttm_reduce_lastdim", (0, hip.ptr(padded), hip.ptr(torch.zeros(32 * 32, dtype=torch.bfloat16)), hip.BF16, 1, 32, C, None)),
+              ("ttm_rms_norm", (hip.ptr(padded), hip.ptr(torch.zeros(C, dtype=torch.bfloat16)), hip.ROW_MAJOR, None, hip.TILE, hip.ptr(padded),
+                                hip.BF16, 1, 32, C, 1e-5, None)),
+              ("ttm_rms_norm", (hip.ptr(padded), hip.ptr(padded), hip.TILE, None, hip.TILE, hip.ptr(padded), hip.BF16, 1, 32, C, 1e-5, None)),
+              ("ttm_tilize", (hip.ptr(torch.zeros(2, 40, 50)), hip.ptr(torch.zeros(2 * 64 * 64)), 2, 40, 50, 4, None)),
+              ("ttm_eltwise_unary", (0, hip.ptr(torch.zeros(40, 50)), hip.ptr(torch.zeros(40, 50)), hip.F32, hip.ROW_MAJOR, 1, 40, 50, 0.0, None)),
+              ("ttm_tilize", (None, ctypes.c_void_p(16), 0, 32, 32, 4, None)), ("ttm_sdpa", ())]
+        for name, args in ok:
+            hip._verify_extents(name, args)
+        # block-float operands count tiles of 1088 / 576 bytes; the weights of a linear are [K, N] tiles
+        a, w = torch.zeros(32 * 64, dtype=torch.bfloat16), torch.zeros(2 * 3 * 1088, dtype=torch.uint8)
+        out = torch.zeros(32 * 96, dtype=torch.bfloat16)
+        lin = lambda a_, w_, o_, N: ("ttm_linear", (hip.ptr(a_), hip.BF16, hip.ptr(w_), hip.BFP8B, 0, None, hip.BF16, hip.TILE, hip.ptr(o_), hip.BF16,
+                                                    1, 1, 20, N, 64, 0, None))
+        hip._verify_extents(*lin(a, w, out, 96))
+        with pytest.raises(hip.TTMError, match="weights .*has 6528 bytes, the kernels touch 8704"):
+            hip._verify_extents(*lin(a, w, torch.zeros(32 * 128, dtype=torch.bfloat16), 128))
+        with pytest.raises(hip.TTMError, match="block-float output .*has 100 bytes, the kernels touch 2304"):
+            hip.call("ttm_bfp_pack", hip.ptr(torch.zeros(40, 50)), hip.F32, hip.ROW_MAJOR, hip.ptr(torch.zeros(100, dtype=torch.uint8)), hip.BFP4B,
+                     1, 40, 50, None)
+        # off (the library's default): the call goes to the library, whose own argument check answers
+        hip.check_buffers(False)
+        with pytest.raises(hip.TTMError, match="elem_bytes"):
+            hip.call("ttm_tilize", hip.ptr(torch.zeros(4)), hip.ptr(torch.zeros(4)), 1, 32, 32, 3, None)
+    finally:
+        hip.check_buffers(was_on)

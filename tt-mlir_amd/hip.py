@@ -73,14 +73,109 @@ def check(status, what=""):
         raise TTMError("%s failed (%d): %s" % (what or "ttm call", status, msg))
 
 
+class _Ptr(ctypes.c_void_p):
+    """A device address that remembers how many bytes follow it in its tensor."""
+    nbytes = None
+
+
+_ELEM_BYTES = {F32: 4, F16: 2, BF16: 2, U32: 4, U16: 2, U8: 1, I32: 4}
+
+
+def _pad32(n):
+    return (int(n) + 31) // 32 * 32
+
+
+def _tile_bytes(batch, rows, cols, elem):
+    return int(batch) * _pad32(rows) * _pad32(cols) * elem
+
+
+def _plain_bytes(batch, rows, cols, elem):
+    return int(batch) * int(rows) * int(cols) * elem
+
+
+def _vec_bytes(layout, cols, elem):   # a [cols] weight / bias vector: one tile row of 32 rows, or the plain vector
+    return 32 * _pad32(cols) * elem if layout == TILE else int(cols) * elem
+
+
+# The entry points take logical extents and no buffer sizes; a tile tensor must be backed by its whole padded extent.
+# Per entry point: (argument index, bytes the kernels touch from that pointer on, what it is).
+_EXTENTS = {
+    "ttm_tilize": lambda a: [(0, _plain_bytes(a[2], a[3], a[4], a[5]), "row-major input"), (1, _tile_bytes(a[2], a[3], a[4], a[5]), "tile output")],
+    "ttm_untilize": lambda a: [(0, _tile_bytes(a[2], a[3], a[4], a[5]), "tile input"), (1, _plain_bytes(a[2], a[3], a[4], a[5]), "row-major output")],
+    "ttm_softmax_lastdim": lambda a: [(i, _tile_bytes(a[3], a[4], a[5], _ELEM_BYTES[a[2]]), w) for i, w in ((0, "tile input"), (1, "tile output"))],
+    "ttm_reduce_lastdim": lambda a: [(1, _tile_bytes(a[4], a[5], a[6], _ELEM_BYTES[a[3]]), "tile input"),
+                                     (2, _tile_bytes(a[4], a[5], 1, _ELEM_BYTES[a[3]]), "tile output [.., rows, 1]")],
+    "ttm_rms_norm": lambda a: [(0, _tile_bytes(a[7], a[8], a[9], _ELEM_BYTES[a[6]]), "tile input"),
+                               (1, _vec_bytes(a[2], a[9], _ELEM_BYTES[a[6]]), "weight"), (3, _vec_bytes(a[4], a[9], _ELEM_BYTES[a[6]]), "bias"),
+                               (5, _tile_bytes(a[7], a[8], a[9], _ELEM_BYTES[a[6]]), "tile output")],
+    "ttm_eltwise_unary": lambda a: [(i, (_tile_bytes if a[4] == TILE else _plain_bytes)(a[5], a[6], a[7], _ELEM_BYTES[a[3]]), w)
+                                    for i, w in ((1, "input"), (2, "output"))],
+}
+
+
+def _tiles(batch, rows, cols):
+    return int(batch) * (_pad32(rows) // 32) * (_pad32(cols) // 32)
+
+
+def _operand_bytes(dtype, batch, rows, cols):   # a tile tensor of a plain or block-float dtype
+    if dtype in (BFP8B, BFP4B):
+        return _tiles(batch, rows, cols) * (1088 if dtype == BFP8B else 576)
+    return _tile_bytes(batch, rows, cols, _ELEM_BYTES[dtype])
+
+
+_EXTENTS.update({
+    # (src, src_dtype, src_layout, dst, fmt, batch, rows, cols)
+    "ttm_bfp_pack": lambda a: [(0, (_tile_bytes if a[2] == TILE else _plain_bytes)(a[5], a[6], a[7], _ELEM_BYTES[a[1]]), "input"),
+                               (3, _operand_bytes(a[4], a[5], a[6], a[7]), "block-float output")],
+    # (src, fmt, dst, dst_dtype, dst_layout, batch, rows, cols)
+    "ttm_bfp_unpack": lambda a: [(0, _operand_bytes(a[1], a[5], a[6], a[7]), "block-float input"),
+                                 (2, (_tile_bytes if a[4] == TILE else _plain_bytes)(a[5], a[6], a[7], _ELEM_BYTES[a[3]]), "output")],
+    # (a, a_dtype, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, act)
+    "ttm_linear": lambda a: [(0, _operand_bytes(a[1], a[10], a[12], a[14]), "activations [batch, M, K]"),
+                             (2, _operand_bytes(a[3], a[11], a[14], a[13]), "weights [w_batch, K, N]"),
+                             (5, _vec_bytes(a[7], a[13], _ELEM_BYTES[a[6]]), "bias"),
+                             (8, _operand_bytes(a[9], a[10], a[12], a[13]), "output [batch, M, N]")],
+    # (in, src_dtype, out, dst_dtype, n)
+    "ttm_typecast": lambda a: [(0, int(a[4]) * _ELEM_BYTES[a[1]], "input"), (2, int(a[4]) * _ELEM_BYTES[a[3]], "output")],
+    "ttm_copy_kernel": lambda a: [(0, int(a[2]), "source"), (1, int(a[2]), "destination")],
+    # (in, dtype, out, rows, cols): row-major on both sides
+    "ttm_argmax": lambda a: [(0, int(a[3]) * int(a[4]) * _ELEM_BYTES[a[1]], "input"), (2, int(a[3]) * 4, "int32 output")],
+})
+_check_buffers = os.environ.get("TTMLIR_AMD_CHECK_BUFFERS", "0") == "1"
+
+
+def check_buffers(on=True):
+    """Switch the host-side check of buffer extents on or off (TTMLIR_AMD_CHECK_BUFFERS=1 switches it on at import): before a
+    call of one of the entry points listed in _EXTENTS, every pointer made by ptr() must have at least the bytes behind it
+    that the kernels will touch.  A kernel that runs past a buffer faults the whole device, so the check belongs in front
+    of any call whose buffers were sized by hand."""
+    global _check_buffers
+    _check_buffers = bool(on)
+
+
+def _verify_extents(name, args):
+    spec = _EXTENTS.get(name)
+    if spec is None:
+        return
+    for idx, need, what in spec(args):
+        p = args[idx]
+        if isinstance(p, _Ptr) and p.nbytes is not None and p.nbytes < need:
+            raise TTMError("%s: the %s (argument %d) has %d bytes, the kernels touch %d from its address on (tile tensors are "
+                           "padded to whole 32 x 32 tiles)" % (name, what, idx, p.nbytes, need))
+
+
 def call(name, *args):
+    if _check_buffers:
+        _verify_extents(name, args)
     check(getattr(lib(), name)(*args), name)
 
 
 def ptr(t):
-    """Device address of a torch tensor (must be contiguous)."""
+    """Device address of a torch tensor (must be contiguous); it carries the tensor's size for check_buffers."""
     assert t.is_contiguous()
-    return ctypes.c_void_p(t.data_ptr())
+    p = _Ptr(t.data_ptr())
+    p.nbytes = t.numel() * t.element_size()
+    return p
 
 
 def current_stream():
