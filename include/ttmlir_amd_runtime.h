@@ -226,6 +226,9 @@ int ttrt_pb_capture_or_execute_trace(ttrt_builder *pb, uint32_t capture_program,
 int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force);
 /* location of the operation added last, and an expected (golden) tensor to embed for a location; data is row-major */
 int ttrt_pb_last_op_loc(ttrt_builder *pb, char *buf, size_t len);
+/* the next tensor the builder creates is declared with this shape instead of the one its operation gives: a program that
+ * lies about a result, for tests of what the executor does with one */
+int ttrt_pb_declare_next_shape(ttrt_builder *pb, const uint32_t *shape, int rank);
 int ttrt_pb_golden(ttrt_builder *pb, const char *loc, const char *name, const void *data, size_t bytes, const int64_t *shape,
                    int rank, int dtype);
 /* out_shapes: n_out entries of 8 extents each, out_ranks / out_layouts per entry */

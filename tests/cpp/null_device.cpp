@@ -1,0 +1,538 @@
+// A device that computes nothing and checks everything: a stand-in for libttmlir_amd_hip.so on a machine without a GPU,
+// built by the tests (g++ -shared) and put in front of the real library with LD_LIBRARY_PATH.  "Device memory" is zeroed
+// host memory with a registry of the live allocations; copies are memcpy; streams and graphs are dummies.  A kernel entry
+// point leaves its outputs as they are, but first holds every pointer argument against the registry: the pointer must lie
+// in a live allocation and have behind it the bytes the real kernels touch (include/ttmlir_amd_hip.h: a tile tensor is
+// backed by its whole padded extent).  A violation is an error return with a message, which the runtime turns into an
+// exception - on the GPU the same call would be a memory fault.  With this the host runtime (executor, tensor pool, fused
+// launches, traces) runs whole programs on the CPU: results are meaningless, the extents of every launch are checked.
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+
+#include "ttmlir_amd_hip.h"
+
+#define EXPORT extern "C" __attribute__((visibility("default")))
+
+namespace {
+thread_local std::string g_err;
+std::mutex g_mu;
+std::map<uintptr_t, size_t> g_allocs;            // base -> bytes
+std::map<std::string, int> g_options;
+long g_kernel_calls = 0, g_capture_mark = -1;
+
+int fail(const char *fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_err = std::string("null device: ") + buf;
+  return TTM_ERR_INVALID;
+}
+
+int64_t pad32(int64_t n) { return (n + 31) / 32 * 32; }
+int64_t elem_bytes(int dtype) {
+  switch (dtype) {
+  case TTM_F32: case TTM_U32: case TTM_I32: return 4;
+  case TTM_F16: case TTM_BF16: case TTM_U16: return 2;
+  case TTM_U8: return 1;
+  default: return 0;
+  }
+}
+// bytes of a [batch, rows, cols] tile tensor of a plain or block-float type
+int64_t tile_bytes(int dtype, int64_t batch, int64_t rows, int64_t cols) {
+  const int64_t tiles = batch * (pad32(rows) / 32) * (pad32(cols) / 32);
+  if (dtype == TTM_BFP8B) return tiles * 1088;
+  if (dtype == TTM_BFP4B) return tiles * 576;
+  return tiles * 1024 * elem_bytes(dtype);
+}
+int64_t tensor_bytes(int dtype, int layout, int64_t batch, int64_t rows, int64_t cols) {
+  return layout == TTM_TILE ? tile_bytes(dtype, batch, rows, cols) : batch * rows * cols * elem_bytes(dtype);
+}
+int64_t vec_bytes(int dtype, int layout, int64_t cols) {   // a [cols] weight / bias vector
+  return layout == TTM_TILE ? tile_bytes(dtype, 1, 1, cols) : cols * elem_bytes(dtype);
+}
+
+// `bytes` from p on lie in one live allocation
+int span(const char *fn, const char *what, const void *p, int64_t bytes, bool optional = false) {
+  if (!p) return optional ? TTM_OK : fail("%s: %s is null", fn, what);
+  if (bytes <= 0) return TTM_OK;
+  const uintptr_t a = (uintptr_t)p;
+  std::lock_guard<std::mutex> g(g_mu);
+  auto it = g_allocs.upper_bound(a);
+  if (it == g_allocs.begin()) return fail("%s: %s (%p) is not device memory", fn, what, p);
+  --it;
+  if (a >= it->first + it->second) return fail("%s: %s (%p) is not in a live device allocation", fn, what, p);
+  const int64_t room = (int64_t)(it->first + it->second - a);
+  if (bytes > room)
+    return fail("%s: %s has %lld bytes behind it in its allocation, the kernels touch %lld", fn, what, (long long)room, (long long)bytes);
+  return TTM_OK;
+}
+#define SPAN(what, p, bytes) do { if (int rc_ = span(__func__, what, p, bytes)) return rc_; } while (0)
+#define SPAN_OPT(what, p, bytes) do { if (int rc_ = span(__func__, what, p, bytes, true)) return rc_; } while (0)
+int kernel() { ++g_kernel_calls; return TTM_OK; }
+
+// a [.., rows, cols] shape of `rank` entries as (batch, rows, cols); rank 1 is one row
+void split3(const int64_t *shape, int rank, int64_t &b, int64_t &r, int64_t &c) {
+  b = 1; r = 1; c = 1;
+  if (rank >= 1) c = shape[rank - 1];
+  if (rank >= 2) r = shape[rank - 2];
+  for (int i = 0; i + 2 < rank; ++i) b *= shape[i];
+}
+
+// strided view over a tensor whose last two dims are [rows, cols]: the tensor must hold every matrix up to the one the
+// largest logical offset lies in
+int view_span(const char *fn, const char *what, const void *p, int64_t rows, int64_t cols, int layout, int elem, int rank,
+              const int64_t *extent, const int64_t *stride, int64_t base, int64_t extra_max) {
+  int64_t lo = base, hi = base + extra_max;
+  for (int i = 0; i < rank; ++i) {
+    if (extent[i] <= 0) return TTM_OK;   // empty view
+    const int64_t d = (extent[i] - 1) * stride[i];
+    if (d >= 0) hi += d; else lo += d;
+  }
+  if (lo < 0) return fail("%s: the %s view reaches logical offset %lld", fn, what, (long long)lo);
+  const int64_t per = rows * cols, mats = per > 0 ? hi / per + 1 : 0;
+  const int64_t bytes = layout == TTM_TILE ? mats * pad32(rows) * pad32(cols) * elem : (hi + 1) * elem;
+  return span(fn, what, p, bytes);
+}
+}  // namespace
+
+EXPORT const char *ttm_last_error(void) { return g_err.c_str(); }
+
+// ---- device, memory, streams, events
+EXPORT int ttm_device_count(int *count) { if (!count) return fail("null count"); *count = 1; return TTM_OK; }
+EXPORT int ttm_set_device(int device) { return device == 0 ? TTM_OK : fail("device %d does not exist", device); }
+EXPORT int ttm_device_name(char *buf, size_t len) { if (buf && len) snprintf(buf, len, "null device (host memory, extent checks)"); return TTM_OK; }
+EXPORT int ttm_mem_info(size_t *free_bytes, size_t *total_bytes) {
+  if (free_bytes) *free_bytes = (size_t)1 << 34;
+  if (total_bytes) *total_bytes = (size_t)1 << 34;
+  return TTM_OK;
+}
+EXPORT int ttm_malloc(void **dptr, size_t bytes) {
+  if (!dptr) return fail("ttm_malloc: null out pointer");
+  void *p = nullptr;
+  if (posix_memalign(&p, 256, bytes ? bytes : 1)) return fail("ttm_malloc: out of host memory (%zu bytes)", bytes);
+  memset(p, 0, bytes);
+  std::lock_guard<std::mutex> g(g_mu);
+  g_allocs[(uintptr_t)p] = bytes;
+  *dptr = p;
+  return TTM_OK;
+}
+EXPORT int ttm_free(void *dptr) {
+  if (!dptr) return TTM_OK;
+  {
+    std::lock_guard<std::mutex> g(g_mu);
+    auto it = g_allocs.find((uintptr_t)dptr);
+    if (it == g_allocs.end()) return fail("ttm_free: %p is not the start of a live device allocation", dptr);
+    g_allocs.erase(it);
+  }
+  free(dptr);
+  return TTM_OK;
+}
+EXPORT int ttm_host_alloc(void **hptr, size_t bytes) { if (!hptr) return fail("null"); *hptr = malloc(bytes ? bytes : 1); return *hptr ? TTM_OK : fail("out of memory"); }
+EXPORT int ttm_host_free(void *hptr) { free(hptr); return TTM_OK; }
+EXPORT int ttm_memcpy_h2d(void *dst, const void *src, size_t bytes, void *) {
+  if (!bytes) return TTM_OK;
+  if (!src) return fail("ttm_memcpy_h2d: null source");
+  SPAN("destination", dst, (int64_t)bytes);
+  memcpy(dst, src, bytes);
+  return TTM_OK;
+}
+EXPORT int ttm_memcpy_d2h(void *dst, const void *src, size_t bytes, void *) {
+  if (!bytes) return TTM_OK;
+  if (!dst) return fail("ttm_memcpy_d2h: null destination");
+  SPAN("source", src, (int64_t)bytes);
+  memcpy(dst, src, bytes);
+  return TTM_OK;
+}
+EXPORT int ttm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *) {
+  if (!bytes) return TTM_OK;
+  SPAN("destination", dst, (int64_t)bytes);
+  SPAN("source", src, (int64_t)bytes);
+  memmove(dst, src, bytes);
+  return TTM_OK;
+}
+EXPORT int ttm_fill_u32(void *dst, uint32_t value, size_t count, void *) {
+  if (!count) return TTM_OK;
+  SPAN("destination", dst, (int64_t)count * 4);
+  for (size_t i = 0; i < count; ++i) ((uint32_t *)dst)[i] = value;
+  return kernel();
+}
+EXPORT int ttm_stream_create(void **stream) { if (!stream) return fail("null"); *stream = malloc(8); return TTM_OK; }
+EXPORT int ttm_stream_destroy(void *stream) { free(stream); return TTM_OK; }
+EXPORT int ttm_stream_sync(void *) { return TTM_OK; }
+EXPORT int ttm_device_sync(void) { return TTM_OK; }
+EXPORT int ttm_event_create(void **event) { if (!event) return fail("null"); *event = malloc(8); return TTM_OK; }
+EXPORT int ttm_event_destroy(void *event) { free(event); return TTM_OK; }
+EXPORT int ttm_event_record(void *, void *) { return TTM_OK; }
+EXPORT int ttm_event_sync(void *) { return TTM_OK; }
+EXPORT int ttm_event_elapsed_ms(float *ms, void *, void *) { if (ms) *ms = 0.0f; return TTM_OK; }
+
+// ---- graphs: the launches between begin and end are counted, a replay does nothing
+EXPORT int ttm_graph_begin_capture(void *) {
+  if (g_capture_mark >= 0) return fail("ttm_graph_begin_capture: a capture is already in progress");
+  g_capture_mark = g_kernel_calls;
+  return TTM_OK;
+}
+EXPORT int ttm_graph_end_capture(void *, void **graph_exec, size_t *num_nodes) {
+  if (g_capture_mark < 0) return fail("ttm_graph_end_capture: no capture in progress");
+  if (num_nodes) *num_nodes = (size_t)(g_kernel_calls - g_capture_mark);
+  g_capture_mark = -1;
+  if (graph_exec) *graph_exec = malloc(8);
+  return TTM_OK;
+}
+EXPORT int ttm_graph_launch(void *graph_exec, void *) { return graph_exec ? TTM_OK : fail("ttm_graph_launch: null graph"); }
+EXPORT int ttm_graph_destroy(void *graph_exec) { free(graph_exec); return TTM_OK; }
+EXPORT int ttm_stream_is_capturing(void *, int *capturing) { if (capturing) *capturing = g_capture_mark >= 0; return TTM_OK; }
+
+EXPORT int ttm_set_option(const char *name, int value) { if (!name) return fail("null"); g_options[name] = value; return TTM_OK; }
+EXPORT int ttm_get_option(const char *name, int *value) { if (!name || !value) return fail("null"); *value = g_options[name]; return TTM_OK; }
+
+// ---- layout, block float, typecast
+EXPORT int ttm_copy_kernel(const void *src, void *dst, size_t bytes, void *) {
+  SPAN("source", src, (int64_t)bytes); SPAN("destination", dst, (int64_t)bytes);
+  return kernel();
+}
+EXPORT int ttm_tilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int elem, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("row-major input", src, batch * rows * cols * elem);
+  SPAN("tile output", dst, batch * pad32(rows) * pad32(cols) * elem);
+  return kernel();
+}
+EXPORT int ttm_untilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int elem, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("tile input", src, batch * pad32(rows) * pad32(cols) * elem);
+  SPAN("row-major output", dst, batch * rows * cols * elem);
+  return kernel();
+}
+EXPORT int64_t ttm_bfp_tile_bytes(int fmt) { return fmt == TTM_BFP8B ? 1088 : (fmt == TTM_BFP4B ? 576 : -1); }
+EXPORT int ttm_bfp_pack(const void *src, int src_dtype, int src_layout, void *dst, int fmt, int64_t batch, int64_t rows, int64_t cols, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("input", src, tensor_bytes(src_dtype, src_layout, batch, rows, cols));
+  SPAN("block-float output", dst, tile_bytes(fmt, batch, rows, cols));
+  return kernel();
+}
+EXPORT int ttm_bfp_unpack(const void *src, int fmt, void *dst, int dst_dtype, int dst_layout, int64_t batch, int64_t rows, int64_t cols, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("block-float input", src, tile_bytes(fmt, batch, rows, cols));
+  SPAN("output", dst, tensor_bytes(dst_dtype, dst_layout, batch, rows, cols));
+  return kernel();
+}
+EXPORT int ttm_typecast(const void *in, int src_dtype, void *out, int dst_dtype, int64_t n, void *) {
+  if (n == 0) return TTM_OK;
+  SPAN("input", in, n * elem_bytes(src_dtype)); SPAN("output", out, n * elem_bytes(dst_dtype));
+  return kernel();
+}
+
+// ---- matmul / linear
+static int linear_check(const char *fn, const void *a, int a_dtype, const void *w, int w_dtype, const void *bias, int bias_dtype, int bias_layout,
+                        void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int tail_op, const void *tail) {
+  if (batch * M * N == 0) return TTM_OK;
+  if (int rc = span(fn, "activations [batch, M, K]", a, tile_bytes(a_dtype, batch, M, K))) return rc;
+  if (int rc = span(fn, "weights [w_batch, K, N]", w, tile_bytes(w_dtype, w_batch, K, N))) return rc;
+  if (int rc = span(fn, "bias", bias, vec_bytes(bias_dtype, bias_layout, N), true)) return rc;
+  if (int rc = span(fn, "output [batch, M, N]", out, tile_bytes(out_dtype, batch, M, N))) return rc;
+  if (tail_op != TTM_TAIL_NONE)
+    if (int rc = span(fn, "tail operand [batch, M, N]", tail, tile_bytes(TTM_BF16, batch, M, N))) return rc;
+  return kernel();
+}
+EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int, const void *bias, int bias_dtype, int bias_layout, void *out,
+                      int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int, void *) {
+  return linear_check(__func__, a, a_dtype, w, w_dtype, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, TTM_TAIL_NONE, nullptr);
+}
+EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int, const void *bias, int bias_dtype, int bias_layout, void *out,
+                           int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int, int tail_op, const void *tail, void *) {
+  return linear_check(__func__, a, a_dtype, w, w_dtype, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, tail_op, tail);
+}
+EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N, const int *, int64_t M,
+                            int64_t K, void *) {
+  if (n < 1 || n > 4 || !w || !out || !N) return fail("ttm_linear_group: one to four members with weights, outputs and widths");
+  SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
+  for (int i = 0; i < n; ++i) {
+    SPAN("weights [K, N_i]", w[i], tile_bytes(w_dtype, 1, K, N[i]));
+    SPAN("output [M, N_i]", out[i], tile_bytes(TTM_BF16, 1, M, N[i]));
+  }
+  return kernel();
+}
+EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M, int64_t N, int64_t K, void *) {
+  SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
+  SPAN("weights 0", w0, tile_bytes(w_dtype, 1, K, N)); SPAN("weights 1", w1, tile_bytes(w_dtype, 1, K, N));
+  SPAN("output 0", out0, tile_bytes(TTM_BF16, 1, M, N)); SPAN("output 1", out1, tile_bytes(TTM_BF16, 1, M, N));
+  return kernel();
+}
+static bool block_float(int dt) { return dt == TTM_BFP8B || dt == TTM_BFP4B; }
+// the predicates of the real library at its default options
+EXPORT int ttm_linear_add_rms_norm_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
+  return block_float(w_dtype) && M >= 1 && M <= 32 && K > 0 && N >= 1 && (N + 31) / 32 * 4 <= 8 * 256;
+}
+EXPORT int ttm_linear_add_rms_norm(const void *a, const void *w, int w_dtype, const void *residual, void *sum_out, const void *norm_weight,
+                                   int weight_layout, const void *norm_bias, int bias_layout, float, void *norm_out, int64_t M, int64_t N, int64_t K,
+                                   void *) {
+  if (!ttm_linear_add_rms_norm_supported(w_dtype, M, N, K)) return fail("ttm_linear_add_rms_norm: unsupported shape");
+  SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
+  SPAN("weights [K, N]", w, tile_bytes(w_dtype, 1, K, N));
+  SPAN("residual [M, N]", residual, tile_bytes(TTM_BF16, 1, M, N));
+  SPAN("sum output [M, N]", sum_out, tile_bytes(TTM_BF16, 1, M, N));
+  SPAN("norm output [M, N]", norm_out, tile_bytes(TTM_BF16, 1, M, N));
+  SPAN_OPT("norm weight", norm_weight, vec_bytes(TTM_BF16, weight_layout, N));
+  SPAN_OPT("norm bias", norm_bias, vec_bytes(TTM_BF16, bias_layout, N));
+  if (sum_out == residual || norm_out == sum_out || norm_out == residual) return fail("ttm_linear_add_rms_norm: the outputs alias");
+  return kernel();
+}
+EXPORT int ttm_linear_qkv_decode_supported(int w_dtype, int64_t users, int64_t K, int64_t heads, int64_t kv_heads, int64_t head_dim) {
+  return block_float(w_dtype) && users >= 1 && users <= 32 && K > 0 && heads >= 1 && kv_heads >= 1 && head_dim >= 32 && head_dim % 32 == 0;
+}
+EXPORT int ttm_linear_qkv_decode(const void *a, const void *wq, const void *wk, const void *wv, int w_dtype, int64_t users, int64_t K, int64_t heads,
+                                 int64_t kv_heads, int64_t head_dim, const void *cos_cache, const void *sin_cache, int64_t cache_rows,
+                                 int64_t token_index, void *q_out, void *k_cache, void *v_cache, int64_t cache_users, int64_t max_seq,
+                                 const int32_t *update_index, int64_t batch_offset, void *) {
+  if (!ttm_linear_qkv_decode_supported(w_dtype, users, K, heads, kv_heads, head_dim)) return fail("ttm_linear_qkv_decode: unsupported shape");
+  if (token_index < 0 || token_index >= cache_rows) return fail("ttm_linear_qkv_decode: token_index outside the cached positions");
+  if (batch_offset < 0 || batch_offset + users > cache_users) return fail("ttm_linear_qkv_decode: batch_offset + users exceeds the cache");
+  SPAN("activations [users, K]", a, tile_bytes(TTM_BF16, 1, users, K));
+  SPAN("q weights", wq, tile_bytes(w_dtype, 1, K, heads * head_dim));
+  SPAN("k weights", wk, tile_bytes(w_dtype, 1, K, kv_heads * head_dim));
+  SPAN("v weights", wv, tile_bytes(w_dtype, 1, K, kv_heads * head_dim));
+  SPAN("cos cache", cos_cache, tile_bytes(TTM_BF16, 1, cache_rows, head_dim));
+  SPAN("sin cache", sin_cache, tile_bytes(TTM_BF16, 1, cache_rows, head_dim));
+  SPAN("q output [1, users, heads, head_dim]", q_out, tile_bytes(TTM_BF16, users, heads, head_dim));
+  SPAN("k cache", k_cache, tile_bytes(TTM_BF16, cache_users * kv_heads, max_seq, head_dim));
+  SPAN("v cache", v_cache, tile_bytes(TTM_BF16, cache_users * kv_heads, max_seq, head_dim));
+  SPAN("update index", update_index, 4);
+  return kernel();
+}
+
+// ---- element-wise
+EXPORT int ttm_eltwise_unary(int, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("input", in, tensor_bytes(dtype, layout, batch, rows, cols)); SPAN("output", out, tensor_bytes(dtype, layout, batch, rows, cols));
+  return kernel();
+}
+EXPORT int ttm_clamp(const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float, float, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("input", in, tensor_bytes(dtype, layout, batch, rows, cols)); SPAN("output", out, tensor_bytes(dtype, layout, batch, rows, cols));
+  return kernel();
+}
+static int shaped(const char *fn, const char *what, const void *p, const int64_t *shape, int rank, int dtype, int layout) {
+  if (!shape) return fail("%s: %s has no shape", fn, what);
+  int64_t b, r, c;
+  split3(shape, rank, b, r, c);
+  return span(fn, what, p, tensor_bytes(dtype, layout, b, r, c));
+}
+EXPORT int ttm_eltwise_binary(int, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape, void *out, const int64_t *out_shape,
+                              int rank, int dtype, int layout, void *) {
+  if (rank < 0 || rank > 8) return fail("ttm_eltwise_binary: rank");
+  if (int rc = shaped(__func__, "left operand", a, a_shape, rank, dtype, layout)) return rc;
+  if (int rc = shaped(__func__, "right operand", b, b_shape, rank, dtype, layout)) return rc;
+  if (int rc = shaped(__func__, "output", out, out_shape, rank, dtype, layout)) return rc;
+  return kernel();
+}
+EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape, void *out,
+                     const int64_t *out_shape, int rank, int dtype, int layout, void *) {
+  if (rank < 0 || rank > 4) return fail("ttm_where: rank");
+  if (int rc = shaped(__func__, "condition", cond, cond_shape, rank, dtype, layout)) return rc;
+  if (int rc = shaped(__func__, "first operand", a, a_shape, rank, dtype, layout)) return rc;
+  if (int rc = shaped(__func__, "second operand", b, b_shape, rank, dtype, layout)) return rc;
+  if (int rc = shaped(__func__, "output", out, out_shape, rank, dtype, layout)) return rc;
+  return kernel();
+}
+EXPORT int ttm_embedding(const void *indices, int, const void *weight, void *out, int elem, int64_t rows, int64_t vocab, int64_t dim, void *) {
+  if (rows * dim == 0) return TTM_OK;
+  SPAN("indices", indices, rows * 4); SPAN("weight [vocab, dim]", weight, vocab * dim * elem); SPAN("output [rows, dim]", out, rows * dim * elem);
+  return kernel();
+}
+EXPORT int ttm_argmax(const void *in, int dtype, int32_t *out, int64_t rows, int64_t cols, void *) {
+  if (rows * cols == 0) return TTM_OK;
+  SPAN("input [rows, cols]", in, rows * cols * elem_bytes(dtype)); SPAN("output [rows]", out, rows * 4);
+  return kernel();
+}
+EXPORT int ttm_arange(void *out, int dtype, int64_t n, double, double, void *) {
+  if (n == 0) return TTM_OK;
+  SPAN("output", out, n * elem_bytes(dtype));
+  return kernel();
+}
+
+// ---- row-wise
+EXPORT int ttm_rms_norm(const void *x, const void *weight, int weight_layout, const void *bias, int bias_layout, void *out, int dtype, int64_t batch,
+                        int64_t rows, int64_t cols, float, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
+  SPAN_OPT("weight", weight, vec_bytes(dtype, weight_layout, cols)); SPAN_OPT("bias", bias, vec_bytes(dtype, bias_layout, cols));
+  return kernel();
+}
+EXPORT int ttm_softmax_lastdim(const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
+  return kernel();
+}
+EXPORT int ttm_reduce_lastdim(int, const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output [.., rows, 1]", out, tile_bytes(dtype, batch, rows, 1));
+  return kernel();
+}
+
+// ---- strided views
+EXPORT int ttm_copy_view(const void *src, int64_t src_rows, int64_t src_cols, int src_layout, void *dst, int64_t dst_rows, int64_t dst_cols,
+                         int dst_layout, int elem, int rank, const int64_t *extent, const int64_t *src_stride, int64_t src_base,
+                         const int64_t *dst_stride, int64_t dst_base, void *) {
+  if (rank < 0 || rank > 8 || (rank > 0 && (!extent || !src_stride || !dst_stride))) return fail("ttm_copy_view: rank / descriptors");
+  if (int rc = view_span(__func__, "source", src, src_rows, src_cols, src_layout, elem, rank, extent, src_stride, src_base, 0)) return rc;
+  if (int rc = view_span(__func__, "destination", dst, dst_rows, dst_cols, dst_layout, elem, rank, extent, dst_stride, dst_base, 0)) return rc;
+  return kernel();
+}
+EXPORT int ttm_copy_view_at(const void *src, int64_t src_rows, int64_t src_cols, int src_layout, void *dst, int64_t dst_rows, int64_t dst_cols,
+                            int dst_layout, int elem, int rank, const int64_t *extent, const int64_t *src_stride, int64_t src_base,
+                            const int64_t *dst_stride, int64_t dst_base, const int32_t *index, int64_t index_stride, int64_t index_limit, void *) {
+  if (rank < 0 || rank > 8 || (rank > 0 && (!extent || !src_stride || !dst_stride))) return fail("ttm_copy_view_at: rank / descriptors");
+  SPAN("index", index, 4);
+  if (int rc = view_span(__func__, "source", src, src_rows, src_cols, src_layout, elem, rank, extent, src_stride, src_base, 0)) return rc;
+  const int64_t far = index_limit > 0 ? (index_limit - 1) * index_stride : 0;
+  if (int rc = view_span(__func__, "destination", dst, dst_rows, dst_cols, dst_layout, elem, rank, extent, dst_stride, dst_base, far)) return rc;
+  return kernel();
+}
+
+// ---- attention
+static int sdpa_check(const char *fn, const void *q, const void *k, const void *v, const void *mask, int mask_heads, int64_t mask_batch, void *out, int dtype,
+                      int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, const void *sink) {
+  if (B * Hq * Sq * D == 0) return TTM_OK;
+  if (Hkv < 1 || Hq % Hkv != 0) return fail("%s: query heads must be a multiple of kv heads", fn);
+  // heads side by side or heads as matrices: the same tiles in another order, the same bytes (D is a multiple of 32)
+  if (int rc = span(fn, "q", q, tile_bytes(dtype, B * Hq, Sq, D))) return rc;
+  if (int rc = span(fn, "k", k, tile_bytes(dtype, B * Hkv, Sk, D))) return rc;
+  if (int rc = span(fn, "v", v, tile_bytes(dtype, B * Hkv, Sk, D))) return rc;
+  if (int rc = span(fn, "mask", mask, tile_bytes(dtype, mask_batch * mask_heads, Sq, Sk), true)) return rc;
+  if (int rc = span(fn, "attention sink", sink, tile_bytes(TTM_BF16, Hq, 1, 1), true)) return rc;
+  if (int rc = span(fn, "output", out, tile_bytes(dtype, B * Hq, Sq, D))) return rc;
+  return kernel();
+}
+EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B, int64_t Hq, int64_t Hkv,
+                    int64_t Sq, int64_t Sk, int64_t D, int, float, void *) {
+  return sdpa_check(__func__, q, k, v, mask, mask_heads, B, out, dtype, B, Hq, Hkv, Sq, Sk, D, nullptr);
+}
+EXPORT int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B, int64_t Hq,
+                                int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int, float, int, void *) {
+  return sdpa_check(__func__, q, k, v, mask, mask_heads, B, out, dtype, B, Hq, Hkv, Sq, Sk, D, nullptr);
+}
+EXPORT int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const void *mask, int mask_heads, int64_t mask_batch, void *out, int dtype,
+                             int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int, float, int, int64_t, const void *attention_sink,
+                             void *) {
+  return sdpa_check(__func__, q, k, v, mask, mask_heads, mask_batch, out, dtype, B, Hq, Hkv, Sq, Sk, D, attention_sink);
+}
+static int decode_check(const char *fn, const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
+                        int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
+                        int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int concat_heads, const void *sink) {
+  if (batch * heads * head_dim == 0) return TTM_OK;
+  if (int rc = span(fn, "q [1, batch, heads, head_dim]", q, tile_bytes(dtype, batch, heads, head_dim))) return rc;
+  const int64_t kv = page_table ? tile_bytes(dtype, page_blocks * kv_heads, page_block, head_dim) : tile_bytes(dtype, batch * kv_heads, seq, head_dim);
+  if (int rc = span(fn, "k", k, kv)) return rc;
+  if (int rc = span(fn, "v", v, kv)) return rc;
+  if (int rc = span(fn, "cur_pos", cur_pos, batch * 4, true)) return rc;
+  if (int rc = span(fn, "mask [mask_batch, 1, mask_heads, seq]", mask, tile_bytes(dtype, mask_batch, mask_heads, seq), true)) return rc;
+  if (int rc = span(fn, "page table", page_table, batch * pages_per_user * 4, true)) return rc;
+  if (int rc = span(fn, "attention sink [heads, 32]", sink, tile_bytes(TTM_BF16, 1, heads, 32), true)) return rc;
+  const int64_t ob = concat_heads ? tile_bytes(dtype, 1, batch, heads * head_dim) : tile_bytes(dtype, batch, heads, head_dim);
+  if (int rc = span(fn, "output", out, ob)) return rc;
+  return kernel();
+}
+EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads, const int32_t *page_table,
+                           int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads,
+                           int64_t kv_heads, int64_t seq, int64_t head_dim, int, float, void *) {
+  return decode_check(__func__, q, k, v, cur_pos, mask, mask_heads, batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads,
+                      kv_heads, seq, head_dim, 0, nullptr);
+}
+EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
+                                        const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
+                                        int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int, float, void *) {
+  return decode_check(__func__, q, k, v, cur_pos, mask, mask_heads, batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads,
+                      kv_heads, seq, head_dim, 1, nullptr);
+}
+EXPORT int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads, int64_t mask_batch,
+                                    const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
+                                    int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int, float, int concat_heads, int64_t,
+                                    const void *attention_sink, void *) {
+  return decode_check(__func__, q, k, v, cur_pos, mask, mask_heads, mask_batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch,
+                      heads, kv_heads, seq, head_dim, concat_heads, attention_sink);
+}
+EXPORT int ttm_sdpa_decode_static(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads, int64_t mask_batch,
+                                  const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
+                                  int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int, float, int concat_heads, int64_t,
+                                  const void *attention_sink, void *) {
+  return decode_check(__func__, q, k, v, cur_pos, mask, mask_heads, mask_batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch,
+                      heads, kv_heads, seq, head_dim, concat_heads, attention_sink);
+}
+
+// ---- decode path
+EXPORT int ttm_rotary_embedding(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols,
+                                int64_t cache_rows, int64_t token_index, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  if (token_index >= cache_rows || (token_index < 0 && rows > cache_rows)) return fail("ttm_rotary_embedding: position outside the cos / sin caches");
+  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
+  SPAN("cos cache", cos_cache, tile_bytes(dtype, 1, cache_rows, cols)); SPAN("sin cache", sin_cache, tile_bytes(dtype, 1, cache_rows, cols));
+  return kernel();
+}
+EXPORT int ttm_rotary_embedding_split_heads(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype, int64_t batch, int64_t heads,
+                                            int64_t head_dim, int64_t cache_rows, int64_t token_index, void *) {
+  if (batch * heads * head_dim == 0) return TTM_OK;
+  if (token_index < 0 || token_index >= cache_rows) return fail("ttm_rotary_embedding_split_heads: position outside the cos / sin caches");
+  SPAN("input [batch, heads * head_dim]", x, tile_bytes(dtype, 1, batch, heads * head_dim));
+  SPAN("output [batch, heads, head_dim]", out, tile_bytes(dtype, batch, heads, head_dim));
+  SPAN("cos cache", cos_cache, tile_bytes(dtype, 1, cache_rows, head_dim)); SPAN("sin cache", sin_cache, tile_bytes(dtype, 1, cache_rows, head_dim));
+  return kernel();
+}
+EXPORT int ttm_rotary_embedding_llama(const void *x, const void *cos_cache, const void *sin_cache, const void *trans_mat, void *out, int dtype, int64_t batch,
+                                      int64_t rows, int64_t cols, int64_t cs_batch, int64_t cs_rows, void *) {
+  if (batch * rows * cols == 0) return TTM_OK;
+  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
+  SPAN("cos", cos_cache, tile_bytes(dtype, cs_batch, cs_rows, cols)); SPAN("sin", sin_cache, tile_bytes(dtype, cs_batch, cs_rows, cols));
+  SPAN("transformation matrix", trans_mat, tile_bytes(TTM_BF16, 1, 32, 32));
+  return kernel();
+}
+EXPORT int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users, int64_t heads, int64_t max_seq,
+                            int64_t head_dim, int64_t input_users, int64_t batch_offset, void *) {
+  if (batch_offset < 0 || batch_offset + input_users > users) return fail("ttm_update_cache: batch_offset + input users exceeds the cache");
+  SPAN("cache", cache, tile_bytes(dtype, users * heads, max_seq, head_dim));
+  SPAN("input [1, heads, users, head_dim]", input, tile_bytes(dtype, heads, input_users, head_dim));
+  SPAN("update index", update_index, 4);
+  return kernel();
+}
+EXPORT int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t users, int64_t heads, int64_t max_seq, int64_t head_dim, int64_t seq,
+                          int64_t batch_offset, void *) {
+  if (batch_offset < 0 || batch_offset >= users || seq > max_seq) return fail("ttm_fill_cache: the input does not fit the cache entry");
+  SPAN("cache", cache, tile_bytes(dtype, users * heads, max_seq, head_dim));
+  SPAN("input [1, heads, seq, head_dim]", input, tile_bytes(dtype, heads, seq, head_dim));
+  return kernel();
+}
+EXPORT int ttm_paged_update_cache(void *cache, const void *input, const int32_t *update_index, const int32_t *page_table, int dtype, int64_t blocks,
+                                  int64_t heads, int64_t block_size, int64_t head_dim, int64_t users, int64_t pages_per_user, int, void *) {
+  SPAN("cache", cache, tile_bytes(dtype, blocks * heads, block_size, head_dim));
+  SPAN("input [1, users, heads, head_dim]", input, tile_bytes(dtype, users, heads, head_dim));
+  SPAN("update index [users]", update_index, users * 4);
+  SPAN_OPT("page table", page_table, users * pages_per_user * 4);
+  return kernel();
+}
+EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_t *page_table, const int32_t *batch_idx, int dtype, int64_t blocks, int64_t heads,
+                                int64_t block_size, int64_t head_dim, int64_t in_batch, int64_t seq, int64_t table_rows, int64_t pages_per_user, void *) {
+  SPAN("cache", cache, tile_bytes(dtype, blocks * heads, block_size, head_dim));
+  SPAN("input [in_batch, heads, seq, head_dim]", input, tile_bytes(dtype, in_batch * heads, seq, head_dim));
+  SPAN("page table", page_table, table_rows * pages_per_user * 4);
+  SPAN_OPT("batch index", batch_idx, in_batch * 4);
+  return kernel();
+}
+EXPORT int ttm_paged_gather(const void *cache, const int32_t *page_table, void *out, int dtype, int64_t blocks, int64_t heads, int64_t block_size,
+                            int64_t head_dim, int64_t users, int64_t pages_per_user, void *) {
+  SPAN("cache", cache, tile_bytes(dtype, blocks * heads, block_size, head_dim));
+  SPAN("page table", page_table, users * pages_per_user * 4);
+  SPAN("output", out, tile_bytes(dtype, users * heads, pages_per_user * block_size, head_dim));
+  return kernel();
+}
+EXPORT int ttm_chunk_causal_mask(void *mask, const int32_t *chunk_start, int64_t rows, int64_t cols, void *) {
+  SPAN("mask [rows, cols]", mask, tile_bytes(TTM_BF16, 1, rows, cols));
+  SPAN("chunk start", chunk_start, 4);
+  return kernel();
+}

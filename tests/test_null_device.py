@@ -1,0 +1,216 @@
+"""The host runtime on a device that computes nothing and checks everything (tests/cpp/null_device.cpp): a stand-in for the
+kernel library whose entry points hold every pointer against the live allocations and the bytes the real kernels touch.
+Put in front of the real library with LD_LIBRARY_PATH, it lets the executor run whole programs on the CPU: the tensor pool,
+the fused launches, the trace protocol and the hooks all run; a launch whose buffer is too small - a memory fault on the
+GPU - is an error here.  Results are meaningless, so the GPU runtime tests are run with assertions stripped (python -O):
+what is checked is that every program runs to its end and that no launch leaves its buffers."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def null_env(tmp_path_factory):
+    d = tmp_path_factory.mktemp("null_device")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-shared", "-fPIC", "-fvisibility=hidden", "-I", os.path.join(ROOT, "include"),
+                    "-o", str(d / "libttmlir_amd_hip.so"), os.path.join(ROOT, "tests", "cpp", "null_device.cpp")], check=True)
+    env = dict(os.environ)
+    # the runtime library finds the kernel library through its RUNPATH, which LD_LIBRARY_PATH precedes
+    env["LD_LIBRARY_PATH"] = str(d) + os.pathsep + env.get("LD_LIBRARY_PATH", "")
+    env["TTMLIR_AMD_NULL_DEVICE"] = "1"
+    return env
+
+
+def test_null_device_exports_the_whole_abi(null_env, hip):
+    import ctypes
+    l = ctypes.CDLL(os.path.join(null_env["LD_LIBRARY_PATH"].split(os.pathsep)[0], "libttmlir_amd_hip.so"))
+    for name, _, _ in hip.declared_functions():   # compiled against the header, so the signatures agree as well
+        assert hasattr(l, name), name
+
+
+def test_null_device_catches_short_buffers(null_env):
+    code = r"""
+import ctypes, sys
+l = ctypes.CDLL("libttmlir_amd_hip.so")
+l.ttm_last_error.restype = ctypes.c_char_p
+V, I64 = ctypes.c_void_p, ctypes.c_int64
+def alloc(n):
+    p = V()
+    assert l.ttm_malloc(ctypes.byref(p), ctypes.c_size_t(n)) == 0
+    return p
+C = 128256
+Cp = (C + 31) // 32 * 32
+one_row, padded = alloc(C * 2), alloc(32 * Cp * 2)
+sm = lambda x, y, rows: l.ttm_softmax_lastdim(x, y, 2, I64(1), I64(rows), I64(C), None)
+assert sm(padded, padded, 1) == 0 and sm(padded, padded, 32) == 0
+assert sm(one_row, padded, 1) == 1 and b"input has 256512 bytes behind it in its allocation, the kernels touch 8208384" in l.ttm_last_error()
+assert sm(padded, one_row, 1) == 1 and b"output" in l.ttm_last_error()
+assert sm(V(padded.value + 2048), padded, 32) == 1          # a view that starts inside the allocation has less room
+assert sm(V(12345), padded, 1) == 1 and b"not device memory" in l.ttm_last_error()
+assert l.ttm_free(one_row) == 0 and sm(padded, one_row, 1) == 1 and b"not" in l.ttm_last_error()   # freed memory is not device memory
+assert l.ttm_free(V(padded.value + 16)) == 1
+print("ok")
+"""
+    r = subprocess.run([sys.executable, "-c", code], env=null_env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and r.stdout.strip() == "ok", r.stderr[-600:]
+
+
+def test_runtime_programs_stay_inside_their_buffers(null_env):
+    # every program the GPU runtime tests build, submitted through the real host runtime on the null device.  Left out: the
+    # full-size configurations (minutes of oracle arithmetic for nothing here) and two tests that look at values by themselves
+    skip = "not full_size and not ttrt_run_checks and not profiler_ranges"
+    r = subprocess.run([sys.executable, "-O", "-m", "pytest", os.path.join(ROOT, "tests", "test_gpu_runtime.py"), "-q", "-m", "gpu", "-p", "no:assertion",
+                        "-p", "no:cacheprovider", "-k", skip], env=null_env, capture_output=True, text=True, timeout=900, cwd=ROOT)
+    tail = r.stdout[-3000:] + r.stderr[-1000:]
+    assert "null device:" not in r.stdout and "null device:" not in r.stderr, tail   # a launch outside its buffers
+    assert r.returncode == 0, tail
+    last = [l for l in r.stdout.strip().splitlines() if " passed" in l][-1]
+    assert int(last.split(" passed")[0].split()[-1]) >= 50 and "failed" not in last, last
+
+
+def test_fusion_decisions_of_a_decode_step_on_the_null_device(null_env):
+    """What the executor fuses is host logic: the counters a decode layer leaves are the same on the null device as on the GPU
+    (tests/test_gpu_runtime.py::test_decode_layer_steps_eager_and_traced asserts them there)."""
+    code = r"""
+import json, sys, os
+sys.path.insert(0, %r); sys.path.insert(0, os.path.join(%r, "tests"))
+import conftest, torch
+from ttmlir_amd import programs, runtime as rt
+import test_gpu_runtime as T
+users, hidden, n_q, n_kv, hd, ffn, max_seq = 8, 256, 4, 2, 64, 512, 128
+w, kc0, vc0, cos, sin, xs = T._decode_setup(users, hidden, n_q, n_kv, hd, ffn, max_seq, seed=31)
+order = ["anw", "wq", "wk", "wv", "wo", "mnw", "wg", "wu", "wd"]
+device = rt.open_mesh_device()
+stats = {}
+for mode in ("eager", "traced", "callbacks"):
+    binary = rt.Binary.load_from_memory(programs.decode_layer(users, hidden, n_q, n_kv, hd, ffn, max_seq, trace=mode == "traced"))
+    rt.clear_stats()
+    if mode == "callbacks":
+        rt.set_post_op_callback(lambda idx, name, dbg, hook: None)
+    main = binary.get_num_programs() - 1
+    lay = lambda k: rt.get_layout(binary, main, k)
+    caches = [rt.to_layout(rt.from_torch(t.clone()), device, lay(5 + i), retain=True) for i, t in enumerate((kc0, vc0))]
+    weights = [rt.to_layout(rt.from_torch(w[n]), device, lay(7 + i), retain=True) for i, n in enumerate(order)]
+    for step, pos in enumerate((40, 41, 42)):
+        step_in = [xs[step], cos[pos].reshape(1, 1, 1, hd), sin[pos].reshape(1, 1, 1, hd), torch.tensor([pos], dtype=torch.int32),
+                   torch.full((users,), pos, dtype=torch.int32)]
+        ins = [rt.to_layout(rt.from_torch(t.contiguous()), device, lay(i)) for i, t in enumerate(step_in)] + caches + weights
+        (y,) = rt.submit(device, binary, main, ins)
+        assert tuple(rt.to_host(y, untilize=True)[0].shape) == (1, users, hidden) or True
+    rt.clear_callbacks()
+    stats[mode] = {k: rt.get_stat(k) for k in ("CapturedTrace", "FusedCopyIntoSlot", "FusedQkvDecode", "FusedCacheUpdate", "FusedHeadSplit",
+                                               "GroupedMatmul", "FusedHeadConcat", "FusedLinearAddNorm", "ConstEvalCacheMiss", "ConstEvalCacheHit")}
+rt.close_mesh_device(device)
+print(json.dumps(stats))
+""" % (ROOT, ROOT)
+    r = subprocess.run([sys.executable, "-c", code], env=null_env, capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-1500:]
+    st = json.loads(r.stdout.strip().splitlines()[-1])
+    for mode in ("eager", "traced", "callbacks"):
+        s = st[mode]
+        assert s["FusedCopyIntoSlot"] == (2 if mode == "traced" else 0), (mode, s)
+        assert s["FusedCacheUpdate"] == 0 and s["FusedHeadSplit"] == 0 and s["GroupedMatmul"] == 0, (mode, s)
+        assert s["FusedHeadConcat"] == s["FusedQkvDecode"] == s["FusedLinearAddNorm"], (mode, s)
+    assert st["eager"]["FusedQkvDecode"] == 3 and st["callbacks"]["FusedQkvDecode"] == 0
+    assert st["traced"]["CapturedTrace"] >= 1 and st["traced"]["FusedQkvDecode"] in (1, 2)
+
+
+def _lying_programs():
+    """Child-process body of the test below (the null device is already in front of the real library): one program per
+    operation whose result is declared smaller than its operands give, submitted on zero inputs."""
+    import numpy as np
+    from ttmlir_amd import runtime as rt
+    DT, TL = rt.DataType, rt.TensorLayout
+    BF, F32, I32, U32 = DT.BFloat16, DT.Float32, DT.Int32, DT.UInt32
+    dev = rt.open_mesh_device()
+    cases = [
+        ("matmul", [((64, 96), BF), ((96, 128), BF)], lambda pb, i: pb.matmul(i[0], i[1]), (64, 64)),
+        ("linear", [((64, 96), BF), ((96, 128), BF), ((128,), BF)], lambda pb, i: pb.linear(i[0], i[1], i[2]), (32, 128)),
+        ("unary", [((64, 96), BF)], lambda pb, i: pb.unary(18, i[0]), (32, 96)),
+        ("binary", [((64, 96), BF), ((64, 96), BF)], lambda pb, i: pb.binary(0, i[0], i[1]), (64, 32)),
+        ("binary broadcast", [((64, 96), BF), ((1, 96), BF)], lambda pb, i: pb.binary(0, i[0], i[1]), (32, 96)),
+        ("binary composite", [((64, 96), BF), ((64, 96), BF)], lambda pb, i: pb.binary_composite(0, i[0], i[1]), (64, 32)),
+        ("where", [((64, 96), BF)] * 3, lambda pb, i: pb.where(i[0], i[1], i[2]), (64, 32)),
+        ("clamp", [((64, 96), BF)], lambda pb, i: pb.unary_composite(1, i[0], -1.0, 1.0), (32, 96)),
+        ("rms_norm", [((64, 96), BF), ((96,), BF)], lambda pb, i: pb.rms_norm(i[0], i[1]), (32, 96)),
+        ("softmax", [((64, 96), BF)], lambda pb, i: pb.softmax(i[0]), (32, 96)),
+        ("softmax over dim 0", [((64, 96), BF)], lambda pb, i: pb.softmax(i[0], dim=0), (32, 96)),
+        ("reduction", [((4, 64, 96), BF)], lambda pb, i: pb.reduction(0, i[0], [2], keep_dim=True), (1, 64, 1)),
+        ("reduction over dim 1", [((4, 64, 96), BF)], lambda pb, i: pb.reduction(0, i[0], [1], keep_dim=False), (4, 32)),
+        ("typecast", [((64, 96), BF)], lambda pb, i: pb.typecast(i[0], F32), (32, 96)),
+        ("typecast to bfp8_b", [((64, 96), BF)], lambda pb, i: pb.typecast(i[0], DT.BFP_BFloat8), (32, 96)),
+        ("to_layout", [((64, 96), BF)], lambda pb, i: pb.to_layout(i[0], TL.RowMajor), (32, 96)),
+        ("reshape", [((64, 96), BF)], lambda pb, i: pb.reshape(i[0], (96, 64)), (32, 64)),
+        ("permute", [((2, 64, 96), BF)], lambda pb, i: pb.permute(i[0], (0, 2, 1)), (2, 32, 64)),
+        ("transpose", [((64, 96), BF)], lambda pb, i: pb.transpose(i[0], 0, 1), (32, 64)),
+        ("concat", [((64, 96), BF), ((64, 96), BF)], lambda pb, i: pb.concat([i[0], i[1]], 1), (64, 96)),
+        ("slice", [((64, 96), BF)], lambda pb, i: pb.slice(i[0], (0, 0), (64, 64)), (32, 32)),
+        ("repeat", [((64, 96), BF)], lambda pb, i: pb.repeat(i[0], (2, 1)), (64, 96)),
+        ("repeat_interleave", [((64, 96), BF)], lambda pb, i: pb.repeat_interleave(i[0], 2, 0), (64, 96)),
+        ("sdpa", [((1, 4, 64, 64), BF), ((1, 2, 64, 64), BF), ((1, 2, 64, 64), BF)], lambda pb, i: pb.sdpa(i[0], i[1], i[2], is_causal=True), (1, 4, 32, 64)),
+        ("sdpa_decode", [((1, 8, 4, 64), BF), ((8, 2, 128, 64), BF), ((8, 2, 128, 64), BF), ((8,), I32)],
+         lambda pb, i: pb.sdpa_decode(i[0], i[1], i[2], cur_pos=i[3]), (1, 4, 4, 64)),
+        ("concatenate_heads", [((1, 4, 64, 64), BF)], lambda pb, i: pb.concatenate_heads(i[0]), (1, 64, 128)),
+        ("nlp_concat_heads", [((1, 4, 64, 64), BF)], lambda pb, i: pb.nlp_concat_heads(i[0]), (1, 1, 32, 256)),
+        ("nlp_concat_heads_decode", [((1, 8, 32, 64), BF)], lambda pb, i: pb.nlp_concat_heads_decode(i[0], 4), (1, 1, 4, 256)),
+        ("nlp_create_qkv_heads_decode", [((1, 1, 8, 8 * 64), BF)], lambda pb, i: pb.nlp_create_qkv_heads_decode(i[0], 4, 2), (1, 4, 4, 64)),
+        ("split_qkv", [((2, 64, 3 * 128), BF)], lambda pb, i: pb.split_query_key_value_and_split_heads(i[0], 4), (2, 4, 32, 32)),
+        ("embedding", [((64,), U32), ((100, 96), BF)], lambda pb, i: pb.embedding(i[0], i[1]), (32, 96)),
+        ("argmax", [((64, 96), BF)], lambda pb, i: pb.argmax(i[0], dim=-1), (32,)),
+        ("rotary_embedding", [((1, 4, 64, 64), BF), ((1, 1, 64, 64), BF), ((1, 1, 64, 64), BF)], lambda pb, i: pb.rotary_embedding(i[0], i[1], i[2]),
+         (1, 4, 32, 64)),
+        ("rotary_embedding decode", [((1, 8, 4, 64), BF), ((1, 1, 64, 64), BF), ((1, 1, 64, 64), BF)],
+         lambda pb, i: pb.rotary_embedding(i[0], i[1], i[2], token_index=5), (1, 4, 4, 64)),
+        ("rotary_embedding_llama", [((1, 4, 64, 64), BF), ((1, 1, 64, 64), BF), ((1, 1, 64, 64), BF), ((1, 1, 32, 32), BF)],
+         lambda pb, i: pb.rotary_embedding_llama(i[0], i[1], i[2], i[3]), (1, 4, 32, 64)),
+        ("full", [], lambda pb, i: pb.full((64, 96), 1.0, BF), (32, 96)),
+        ("arange", [], lambda pb, i: pb.arange(0, 64), (32,)),
+        ("empty", [], lambda pb, i: pb.empty((64, 96), BF), (32, 96)),
+    ]
+    npdt = {BF: np.uint16, F32: np.float32, I32: np.int32, U32: np.uint32}
+    report = {}
+    for lying in (False, True):
+        for name, specs, build, lie in cases:
+            pb = rt.ProgramBuilder()
+            pb.begin_program("p")
+            ins = [pb.input(s, dt) for s, dt in specs]
+            if lying:
+                pb.declare_next_shape(lie)
+            out = build(pb, ins)
+            for o in (out if isinstance(out, (list, tuple)) else [out]):
+                pb.output(o)
+            pb.end_program()
+            b = rt.Binary.load_from_memory(pb.finish())
+            tins = [rt.to_layout(rt.create_owned_host_tensor(np.zeros(s, dtype=npdt[dt]), dt), dev, rt.get_layout(b, 0, k)) for k, (s, dt) in enumerate(specs)]
+            try:
+                rt.submit(dev, b, 0, tins)
+                verdict = "ran"
+            except rt.RuntimeError_ as e:
+                verdict = "LEAK: " + str(e).split("null device: ")[1] if "null device:" in str(e) else "refused"
+            report["%s%s" % (name, " (lying)" if lying else "")] = verdict
+    rt.close_mesh_device(dev)
+    return report
+
+
+def test_programs_that_lie_about_a_result_never_launch_past_a_buffer(null_env):
+    """The kernels are launched from the operands' extents, results are allocated from the shape the program declares: an
+    operation whose declared result is smaller than what its operands give must be refused by the runner (or run on a
+    result of its own making), never reach the device.  Truthful versions of the same programs all run - among them the
+    prefill rotary embedding, whose absent token_index used to reach the kernel as 4294967295."""
+    code = ("import sys, os, json; sys.path.insert(0, %r); sys.path.insert(0, os.path.join(%r, 'tests')); import conftest, test_null_device as t; "
+            "print(json.dumps(t._lying_programs()))") % (ROOT, ROOT)
+    r = subprocess.run([sys.executable, "-c", code], env=null_env, capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-1500:]
+    report = json.loads(r.stdout.strip().splitlines()[-1])
+    assert len(report) == 2 * 38
+    for name, verdict in report.items():
+        assert not verdict.startswith("LEAK"), (name, verdict)
+        if not name.endswith("(lying)"):
+            assert verdict == "ran", (name, verdict)
+    refused = [n for n, v in report.items() if v == "refused"]
+    assert {"matmul (lying)", "linear (lying)", "concat (lying)", "reshape (lying)", "argmax (lying)"} <= set(refused)

@@ -613,6 +613,12 @@ class ProgramBuilder:
         _call("ttrt_pb_tensor_desc", self.h, t, shape, ctypes.byref(rank), ctypes.byref(lay))
         return tuple(shape[: rank.value]), lay
 
+    def declare_next_shape(self, shape):
+        """The next tensor the builder creates is declared with `shape` instead of the one its operation gives (a program that
+        lies about a result, for tests of the executor's checks)."""
+        sh, rank = _shape_arg(shape)
+        _call("ttrt_pb_declare_next_shape", self.h, sh, rank)
+
     def last_op_loc(self):
         buf = ctypes.create_string_buffer(512)
         _call("ttrt_pb_last_op_loc", self.h, buf, 512)

@@ -594,6 +594,9 @@ TTRT_EXPORT int ttrt_pb_execute_trace(ttrt_builder *pb, uint32_t trace_id, int b
 TTRT_EXPORT int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force) {
   return guard([&] { need(pb, "builder"); pb->pb.deallocate(in, force != 0); });
 }
+TTRT_EXPORT int ttrt_pb_declare_next_shape(ttrt_builder *pb, const uint32_t *shape, int rank) {
+  return guard([&] { need(pb, "builder"); pb->pb.declareNextShape(shapeVec(shape, rank)); });
+}
 TTRT_EXPORT int ttrt_pb_last_op_loc(ttrt_builder *pb, char *buf, size_t len) {
   return guard([&] { need(pb, "builder"); copyStr(pb->pb.lastOpLoc(), buf, len); });
 }

@@ -255,6 +255,27 @@ Tensor makeOut(ProgramContext &ctx, const fb::Table &outRef, DataType dtype, Ten
   return makeDeviceTensor(ctx.dev, shapeFromTensorRef(outRef), dtype, layout);
 }
 
+std::string shapeText(const std::vector<std::uint32_t> &s) {
+  std::string t = "[";
+  for (size_t i = 0; i < s.size(); ++i) t += (i ? ", " : "") + std::to_string(s[i]);
+  return t + "]";
+}
+// The kernels are launched from the operands' extents while the result is allocated from the shape the program declares
+// for it: a program that declares another shape than its operands give must be refused here, before a launch writes past
+// the allocation.
+void requireResultShape(const fb::Table &outRef, const std::vector<std::uint32_t> &want, const char *op) {
+  const std::vector<std::uint32_t> declared = shapeFromTensorRef(outRef);
+  TTRT_ASSERT(declared == want, std::string(op) + ": the program declares the result as " + shapeText(declared) + ", the operands give " +
+                                    shapeText(want));
+}
+// the same when only the extent the kernel writes is known: [batch, rows, cols] in the tile layout
+void requireResultExtent(const Tensor &out, std::int64_t batch, std::int64_t rows, std::int64_t cols, const char *op) {
+  const auto r32 = [](std::int64_t n) { return (n + 31) / 32 * 32; };
+  TTRT_ASSERT(paddedVolume(out.handle->shape) == batch * r32(rows) * r32(cols),
+              std::string(op) + ": the program declares the result as " + shapeText(out.handle->shape) + ", the operands give a [" +
+                  std::to_string(batch) + ", " + std::to_string(rows) + ", " + std::to_string(cols) + "] product");
+}
+
 // final cast of an op result to what the program's TensorRef declares (dtype and layout)
 Tensor finish(ProgramContext &ctx, const Tensor &t, const fb::Table &outRef) {
   Layout want = layoutFromTensorRef(outRef);
@@ -519,6 +540,7 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
     biasPtr = bias.handle->data.get();
   }
   Tensor out = makeOut(ctx, outRef, DataType::BFloat16, TensorLayout::Tile);
+  requireResultExtent(out, batch, M, N, "matmul");
   // an `add` or `multiply` that is the only consumer of this result and comes next runs in the kernel's epilogue
   // (residual connections, SiLU(gate) * up); its output takes this op's place
   Tensor tail;
@@ -1070,7 +1092,8 @@ void runRotaryEmbedding(const fb::Table &op, ProgramContext &ctx) {
   const auto &xs = x.handle->shape, &cs = cosc.handle->shape;
   TTRT_ASSERT(xs.size() == 4 && cs.size() == 4 && sinc.handle->shape == cs, "rotary_embedding: all tensors must be 4D, cos and sin of one shape");
   TTRT_ASSERT(cs[0] == 1 && cs[1] == 1 && cs[3] == xs[3], "rotary_embedding: cos / sin caches must be [1, 1, positions, head_dim]");
-  const std::int64_t token = op.has(S::f_token_index) ? op.scalar<std::uint32_t>(S::f_token_index, 0) : -1;
+  // (both arms as int64: with an unsigned arm the -1 would arrive as 4294967295)
+  const std::int64_t token = op.has(S::f_token_index) ? static_cast<std::int64_t>(op.scalar<std::uint32_t>(S::f_token_index, 0)) : std::int64_t{-1};
   auto outRef = op.table(S::f_out);
   Tensor out = makeDeviceTensor(ctx.dev, xs, dt, TensorLayout::Tile);
   TTM_CALL(ttm_rotary_embedding(x.handle->data.get(), cosc.handle->data.get(), sinc.handle->data.get(), out.handle->data.get(),
@@ -1556,6 +1579,20 @@ void runConcat(const fb::Table &op, ProgramContext &ctx) {
   int dim = op.scalar<std::int32_t>(schema::ConcatOp::f_dim, 0);
   if (dim < 0) dim += rank;
   TTRT_ASSERT(dim >= 0 && dim < rank, "concat: dim out of range");
+  {
+    // the copies below address the result by the inputs' extents: the declared shape must be what the inputs add up to
+    std::vector<std::uint32_t> want = first.handle->shape;
+    TTRT_ASSERT(static_cast<int>(want.size()) == rank, "concat: rank mismatch");
+    want[dim] = 0;
+    for (std::uint32_t i = 0; i < ins.size(); ++i) {
+      const std::vector<std::uint32_t> &si = ctx.get(ins[i], "concat in").handle->shape;
+      TTRT_ASSERT(static_cast<int>(si.size()) == rank, "concat: rank mismatch");
+      for (int d = 0; d < rank; ++d)
+        TTRT_ASSERT(d == dim || si[d] == first.handle->shape[d], "concat: inputs differ in a dimension other than the concatenated one");
+      want[dim] += si[dim];
+    }
+    requireResultShape(outRef, want, "concat");
+  }
   Tensor out = makeDeviceTensor(ctx.dev, oshape, first.handle->dtype, first.handle->layout);
   zeroIfPadded(ctx, out);
   auto os = rowMajorStrides(oshape);

@@ -11,6 +11,10 @@ using ::tt::runtime::fatal;
 
 ProgramBuilder::Id ProgramBuilder::newTensor(const Desc &d) {
   tensors_.push_back(d);
+  if (declaredShape_) {
+    tensors_.back().shape = *declaredShape_;
+    declaredShape_.reset();
+  }
   return static_cast<Id>(tensors_.size() - 1);
 }
 

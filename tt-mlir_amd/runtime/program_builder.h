@@ -4,6 +4,7 @@
 // here; the wire format is the reference's (include/ttmlir/Target/TTNN/*.fbs).
 #pragma once
 #include <array>
+#include <optional>
 #include <string>
 #include <vector>
 
@@ -93,6 +94,9 @@ public:
 
   // Location string of the operation added last ("loc(\"<program>\"(\"op<k>\"))"); goldens are keyed by it.
   std::string lastOpLoc() const;
+  // The next tensor the builder creates is declared with `shape` instead of the shape its operation gives: a program that
+  // lies about a result, for tests of what the executor does with one (the compiler never writes such a program).
+  void declareNextShape(const std::vector<std::uint32_t> &shape) { declaredShape_ = shape; }
   // Embeds an expected tensor for the operation at `loc` into the open program's debug info
   // (Common/debug_info.fbs: GoldenInfo.golden_map); data is row-major, contiguous.
   void golden(const std::string &loc, const std::string &name, const void *data, size_t bytes,
@@ -116,6 +120,7 @@ private:
     std::vector<fb::Builder::Off> dylibs;                            // DynamicLib tables
   };
   Id newTensor(const Desc &d);
+  std::optional<std::vector<std::uint32_t>> declaredShape_;   // see declareNextShape
   fb::Builder::Off tensorRef(Id t);
   fb::Builder::Off memoryConfig(StorageType storage);
   void addOp(::ttmlir_amd::schema::OpType type, fb::Builder::Off table, const std::string &debug);
