@@ -214,3 +214,49 @@ def test_programs_that_lie_about_a_result_never_launch_past_a_buffer(null_env):
             assert verdict == "ran", (name, verdict)
     refused = [n for n, v in report.items() if v == "refused"]
     assert {"matmul (lying)", "linear (lying)", "concat (lying)", "reshape (lying)", "argmax (lying)"} <= set(refused)
+
+
+def test_full_size_programs_on_the_null_device(null_env):
+    """The benchmark's whole-program workloads at their real shapes (configs 3, 4, 5 and the 32-user decode step, eager and
+    traced) through the executor on the null device: every launch inside its buffers, and the launches the executor fuses at
+    these shapes (what the GPU profiles show as 11 launches per decode step)."""
+    code = r"""
+import sys, os, json
+sys.path.insert(0, %r); sys.path.insert(0, os.path.join(%r, "tests"))
+import conftest, numpy as np
+from ttmlir_amd import programs, runtime as rt
+DT = rt.DataType
+npdt = {DT.BFloat16: np.uint16, DT.Float32: np.float32, DT.Int32: np.int32, DT.UInt32: np.uint32}
+dev = rt.open_mesh_device()
+keys = ("GroupedMatmul", "FusedLinearTail", "FusedQkvDecode", "FusedLinearAddNorm", "FusedHeadConcat", "CapturedTrace", "ConstEvalCacheMiss", "ConstEvalCacheHit")
+report = {}
+def run(name, data, steps=1):
+    b = rt.Binary.load_from_memory(data)
+    main = b.get_num_programs() - 1
+    ins = [rt.to_layout(rt.create_owned_host_tensor(np.zeros(shape, dtype=npdt[lay.dtype]), lay.dtype), dev, lay, retain=True)
+           for shape, lay in b.get_program_inputs(main)]
+    rt.clear_stats()
+    for _ in range(steps):
+        outs = rt.submit(dev, b, main, ins)
+    report[name] = dict(shapes=[list(o.shape) for o in outs], **{k: rt.get_stat(k) for k in keys})
+run("c3_2048", programs.c3_linear(2048))
+run("c3_32", programs.c3_linear(32))
+run("c4", programs.c4_mlp())
+run("c5", programs.c5_decoder())
+run("decode32", programs.decode_layer(), steps=3)
+run("decode32_traced", programs.decode_layer(trace=True), steps=3)
+rt.close_mesh_device(dev)
+print(json.dumps(report))
+""" % (ROOT, ROOT)
+    r = subprocess.run([sys.executable, "-c", code], env=null_env, capture_output=True, text=True, timeout=900, cwd=ROOT)
+    assert r.returncode == 0, (r.stdout[-500:], r.stderr[-1500:])
+    rep = json.loads(r.stdout.strip().splitlines()[-1])
+    assert rep["c3_2048"]["shapes"] == [[2048, 14336]] and rep["c3_32"]["shapes"] == [[32, 14336]]
+    assert rep["c4"]["shapes"] == [[512, 4096]] and rep["c4"]["GroupedMatmul"] == 1            # gate and up in one launch
+    assert rep["c5"]["shapes"] == [[1, 2048, 4096]]
+    assert rep["c5"]["GroupedMatmul"] == 1 and rep["c5"]["FusedLinearTail"] == 3               # two residual adds and SiLU(gate) * up
+    d = rep["decode32"]                                                                         # three steps
+    assert d["shapes"] == [[32, 4096]] and d["FusedQkvDecode"] == 3 and d["FusedLinearAddNorm"] == 3 and d["FusedHeadConcat"] == 3
+    assert d["ConstEvalCacheMiss"] == 1 and d["ConstEvalCacheHit"] == 2
+    t = rep["decode32_traced"]                                                                  # eager run + recording, then replays
+    assert t["CapturedTrace"] == 1 and t["FusedQkvDecode"] == 2 and t["FusedLinearAddNorm"] == 2
