@@ -66,12 +66,14 @@ int span(const char *fn, const char *what, const void *p, int64_t bytes, bool op
   const uintptr_t a = (uintptr_t)p;
   std::lock_guard<std::mutex> g(g_mu);
   auto it = g_allocs.upper_bound(a);
-  if (it == g_allocs.begin()) return fail("%s: %s (%p) is not device memory", fn, what, p);
+  // every message of this function says "out of bounds": on the GPU the call would be a memory fault, not an error return
+  if (it == g_allocs.begin()) return fail("out of bounds: %s: %s (%p) is not device memory", fn, what, p);
   --it;
-  if (a >= it->first + it->second) return fail("%s: %s (%p) is not in a live device allocation", fn, what, p);
+  if (a >= it->first + it->second) return fail("out of bounds: %s: %s (%p) is not in a live device allocation", fn, what, p);
   const int64_t room = (int64_t)(it->first + it->second - a);
   if (bytes > room)
-    return fail("%s: %s has %lld bytes behind it in its allocation, the kernels touch %lld", fn, what, (long long)room, (long long)bytes);
+    return fail("out of bounds: %s: %s has %lld bytes behind it in its allocation, the kernels touch %lld", fn, what, (long long)room,
+                (long long)bytes);
   return TTM_OK;
 }
 #define SPAN(what, p, bytes) do { if (int rc_ = span(__func__, what, p, bytes)) return rc_; } while (0)
@@ -96,7 +98,7 @@ int view_span(const char *fn, const char *what, const void *p, int64_t rows, int
     const int64_t d = (extent[i] - 1) * stride[i];
     if (d >= 0) hi += d; else lo += d;
   }
-  if (lo < 0) return fail("%s: the %s view reaches logical offset %lld", fn, what, (long long)lo);
+  if (lo < 0) return fail("out of bounds: %s: the %s view reaches logical offset %lld", fn, what, (long long)lo);
   const int64_t per = rows * cols, mats = per > 0 ? hi / per + 1 : 0;
   const int64_t bytes = layout == TTM_TILE ? mats * pad32(rows) * pad32(cols) * elem : (hi + 1) * elem;
   return span(fn, what, p, bytes);
@@ -325,9 +327,17 @@ static int shaped(const char *fn, const char *what, const void *p, const int64_t
   split3(shape, rank, b, r, c);
   return span(fn, what, p, tensor_bytes(dtype, layout, b, r, c));
 }
+// the real library refuses operands that do not broadcast to the output
+static int broadcasts(const char *fn, const int64_t *shape, const int64_t *out_shape, int rank) {
+  for (int d = 0; d < rank; ++d)
+    if (shape && out_shape && shape[d] != out_shape[d] && shape[d] != 1) return fail("%s: shapes do not broadcast at dim %d", fn, d);
+  return TTM_OK;
+}
 EXPORT int ttm_eltwise_binary(int, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape, void *out, const int64_t *out_shape,
                               int rank, int dtype, int layout, void *) {
   if (rank < 0 || rank > 8) return fail("ttm_eltwise_binary: rank");
+  if (int rc = broadcasts(__func__, a_shape, out_shape, rank)) return rc;
+  if (int rc = broadcasts(__func__, b_shape, out_shape, rank)) return rc;
   if (int rc = shaped(__func__, "left operand", a, a_shape, rank, dtype, layout)) return rc;
   if (int rc = shaped(__func__, "right operand", b, b_shape, rank, dtype, layout)) return rc;
   if (int rc = shaped(__func__, "output", out, out_shape, rank, dtype, layout)) return rc;
@@ -336,6 +346,8 @@ EXPORT int ttm_eltwise_binary(int, const void *a, const int64_t *a_shape, const 
 EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape, void *out,
                      const int64_t *out_shape, int rank, int dtype, int layout, void *) {
   if (rank < 0 || rank > 4) return fail("ttm_where: rank");
+  for (const int64_t *sh : {cond_shape, a_shape, b_shape})
+    if (int rc = broadcasts(__func__, sh, out_shape, rank)) return rc;
   if (int rc = shaped(__func__, "condition", cond, cond_shape, rank, dtype, layout)) return rc;
   if (int rc = shaped(__func__, "first operand", a, a_shape, rank, dtype, layout)) return rc;
   if (int rc = shaped(__func__, "second operand", b, b_shape, rank, dtype, layout)) return rc;

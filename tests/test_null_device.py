@@ -48,7 +48,7 @@ Cp = (C + 31) // 32 * 32
 one_row, padded = alloc(C * 2), alloc(32 * Cp * 2)
 sm = lambda x, y, rows: l.ttm_softmax_lastdim(x, y, 2, I64(1), I64(rows), I64(C), None)
 assert sm(padded, padded, 1) == 0 and sm(padded, padded, 32) == 0
-assert sm(one_row, padded, 1) == 1 and b"input has 256512 bytes behind it in its allocation, the kernels touch 8208384" in l.ttm_last_error()
+assert sm(one_row, padded, 1) == 1 and b"out of bounds: ttm_softmax_lastdim: input has 256512 bytes behind it in its allocation, the kernels touch 8208384" in l.ttm_last_error()
 assert sm(padded, one_row, 1) == 1 and b"output" in l.ttm_last_error()
 assert sm(V(padded.value + 2048), padded, 32) == 1          # a view that starts inside the allocation has less room
 assert sm(V(12345), padded, 1) == 1 and b"not device memory" in l.ttm_last_error()
@@ -67,7 +67,7 @@ def test_runtime_programs_stay_inside_their_buffers(null_env):
     r = subprocess.run([sys.executable, "-O", "-m", "pytest", os.path.join(ROOT, "tests", "test_gpu_runtime.py"), "-q", "-m", "gpu", "-p", "no:assertion",
                         "-p", "no:cacheprovider", "-k", skip], env=null_env, capture_output=True, text=True, timeout=900, cwd=ROOT)
     tail = r.stdout[-3000:] + r.stderr[-1000:]
-    assert "null device:" not in r.stdout and "null device:" not in r.stderr, tail   # a launch outside its buffers
+    assert "out of bounds" not in r.stdout and "out of bounds" not in r.stderr, tail   # a launch outside its buffers
     assert r.returncode == 0, tail
     last = [l for l in r.stdout.strip().splitlines() if " passed" in l][-1]
     assert int(last.split(" passed")[0].split()[-1]) >= 50 and "failed" not in last, last
@@ -191,7 +191,7 @@ def _lying_programs():
                 rt.submit(dev, b, 0, tins)
                 verdict = "ran"
             except rt.RuntimeError_ as e:
-                verdict = "LEAK: " + str(e).split("null device: ")[1] if "null device:" in str(e) else "refused"
+                verdict = "LEAK: " + str(e).split("out of bounds: ")[1] if "out of bounds" in str(e) else "refused"
             report["%s%s" % (name, " (lying)" if lying else "")] = verdict
     rt.close_mesh_device(dev)
     return report
@@ -212,8 +212,10 @@ def test_programs_that_lie_about_a_result_never_launch_past_a_buffer(null_env):
         assert not verdict.startswith("LEAK"), (name, verdict)
         if not name.endswith("(lying)"):
             assert verdict == "ran", (name, verdict)
-    refused = [n for n, v in report.items() if v == "refused"]
-    assert {"matmul (lying)", "linear (lying)", "concat (lying)", "reshape (lying)", "argmax (lying)"} <= set(refused)
+    # a full or empty tensor has no operands: the declared shape is its shape.  Everything else is refused, by the runner or
+    # where its result enters the tensor pool under a reference that declares another shape
+    still_run = {n for n, v in report.items() if n.endswith("(lying)") and v == "ran"}
+    assert still_run == {"full (lying)", "empty (lying)"}, still_run
 
 
 def test_full_size_programs_on_the_null_device(null_env):

@@ -59,10 +59,8 @@ struct ProgramContext {
     TTRT_ASSERT(isTensorAllocated(it->second), std::string("tensor ") + std::to_string(id) + " (" + what + ") was deallocated");
     return it->second;
   }
-  void put(const fb::Table &ref, Tensor t) {
-    std::uint32_t id = ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
-    pool[id] = std::move(t);
-  }
+  void put(const fb::Table &ref, Tensor t);
+
   void *stream() const { return dev->stream; }
 };
 
@@ -255,6 +253,19 @@ Tensor makeOut(ProgramContext &ctx, const fb::Table &outRef, DataType dtype, Ten
   return makeDeviceTensor(ctx.dev, shapeFromTensorRef(outRef), dtype, layout);
 }
 
+std::string shapeText(const std::vector<std::uint32_t> &s);
+// A tensor enters the pool under the reference the program declares for it.  Its shape must be the declared one: later
+// operations size their launches from the tensors they find here, and a program whose declarations do not agree with
+// what its operations produce is refused at the first such result rather than run on shapes it did not state.
+void ProgramContext::put(const fb::Table &ref, Tensor t) {
+  std::uint32_t id = ref.scalar<std::uint32_t>(schema::TensorRef::f_global_id, 0);
+  if (t.handle) {
+    const std::vector<std::uint32_t> declared = shapeFromTensorRef(ref);
+    TTRT_ASSERT(t.handle->shape == declared, "tensor " + std::to_string(id) + ": the program declares the shape " + shapeText(declared) +
+                                                 ", the operation produced " + shapeText(t.handle->shape));
+  }
+  pool[id] = std::move(t);
+}
 std::string shapeText(const std::vector<std::uint32_t> &s) {
   std::string t = "[";
   for (size_t i = 0; i < s.size(); ++i) t += (i ? ", " : "") + std::to_string(s[i]);
