@@ -1216,3 +1216,23 @@ def test_head_split_and_merge_ops(device):
     for i, (g_, w_) in enumerate(zip(got, want)):
         assert tuple(g_.shape) == tuple(w_.shape), i
         assert torch.equal(g_, w_.contiguous()), i
+
+
+def test_prefill_rotary_embedding_program(device, orc):
+    """RotaryEmbeddingOp without a token_index (prefill: row s of the input uses row s of the caches) through the executor,
+    bit exact against the oracle as the kernel alone is (tests/test_gpu_decode.py::test_rotary_embedding).  The absent
+    attribute once reached the kernel as 4294967295 instead of -1."""
+    B, H, S, D = 1, 4, 96, 64
+    x = datagen.randn((B, H, S, D), seed=140, dtype=torch.bfloat16)
+    ang = datagen.randn((1, 1, S, D // 2), seed=141, dtype=torch.float32) * 2.0
+    cos = torch.cat([ang.cos(), ang.cos()], -1).to(torch.bfloat16)
+    sin = torch.cat([ang.sin(), ang.sin()], -1).to(torch.bfloat16)
+    pb = rt.ProgramBuilder()
+    pb.begin_program("prefill_rope")
+    ids = [pb.input(tuple(t.shape), DT.BFloat16) for t in (x, cos, sin)]
+    pb.output(pb.rotary_embedding(*ids))
+    pb.end_program()
+    (y,) = harness.execute(rt.Binary.load_from_memory(pb.finish()), 0, [x, cos, sin], device)
+    f = lambda t: t.float().numpy()
+    want = orc.round_bf16(orc.rotary_embedding(f(x), f(cos), f(sin), token_index=None))
+    assert tuple(y.shape) == (B, H, S, D) and np.array_equal(f(y), want)
