@@ -262,3 +262,52 @@ print(json.dumps(report))
     assert d["ConstEvalCacheMiss"] == 1 and d["ConstEvalCacheHit"] == 2
     t = rep["decode32_traced"]                                                                  # eager run + recording, then replays
     assert t["CapturedTrace"] == 1 and t["FusedQkvDecode"] == 2 and t["FusedLinearAddNorm"] == 2
+
+
+def test_const_eval_entries_live_as_long_as_their_inputs(null_env):
+    """The reference's tests of its const-eval cache (runtime/test/ttnn/gtest/test_tensor_cache_lifetime.cpp:46-163), at the
+    level of programs: an entry per set of input versions (CacheSanitySameProgramDifferentTensors: a second weight tensor
+    gets its own entry and leaves the first alone), removed when a tensor it was computed from is destroyed
+    (CacheEntryRemovedOnTensorDestruction), any one of them (MultipleInputTensorsRemoveCacheEntry)."""
+    code = r"""
+import sys, os, json, gc
+sys.path.insert(0, %r); sys.path.insert(0, os.path.join(%r, "tests"))
+import conftest, numpy as np
+from ttmlir_amd import programs, runtime as rt
+DT = rt.DataType
+dev = rt.open_mesh_device()
+stats = lambda: tuple(rt.get_stat(k) for k in ("ConstEvalCacheMiss", "ConstEvalCacheHit", "ConstEvalCacheEvicted"))
+log = {}
+# one weight tensor: config 3 (the weights are packed to bfp8_b by a const-eval program)
+M, K, N = 64, 128, 160
+b = rt.Binary.load_from_memory(programs.c3_linear(M, K, N))
+lay = lambda i: rt.get_layout(b, 1, i)
+mk = lambda shape, i: rt.to_layout(rt.create_owned_host_tensor(np.zeros(shape, dtype=np.uint16), DT.BFloat16), dev, lay(i), retain=True)
+a, bias = mk((M, K), 0), mk((N,), 2)
+wA, wB = mk((K, N), 1), mk((K, N), 1)
+rt.clear_stats()
+run = lambda w: rt.submit(dev, b, 1, [a, w, bias])
+run(wA); log["A"] = stats()
+run(wB); log["B"] = stats()               # another tensor, another version: its own entry
+run(wA); log["A again"] = stats()         # the first entry is still there
+run(wB); log["B again"] = stats()
+del wB; gc.collect(); log["B destroyed"] = stats()
+run(wA); log["A after B died"] = stats()
+del wA; gc.collect(); log["A destroyed"] = stats()
+# several inputs: config 4 packs three weight tensors in one const-eval program; destroying one of them removes the entry
+b4 = rt.Binary.load_from_memory(programs.c4_mlp(64, 128, 256))
+ins = [rt.to_layout(rt.create_owned_host_tensor(np.zeros(s, dtype=np.uint16), l.dtype), dev, l, retain=True) for s, l in b4.get_program_inputs(1)]
+rt.clear_stats()
+rt.submit(dev, b4, 1, ins); rt.submit(dev, b4, 1, ins); log["mlp twice"] = stats()
+victim = ins.pop(3); rest = list(ins)      # the up-projection weights
+del victim; gc.collect(); log["one of three destroyed"] = stats()
+rt.close_mesh_device(dev)
+print(json.dumps(log))
+""" % (ROOT, ROOT)
+    r = subprocess.run([sys.executable, "-c", code], env=null_env, capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-1500:]
+    log = json.loads(r.stdout.strip().splitlines()[-1])
+    assert log["A"] == [1, 0, 0] and log["B"] == [2, 0, 0]
+    assert log["A again"] == [2, 1, 0] and log["B again"] == [2, 2, 0]
+    assert log["B destroyed"] == [2, 2, 1] and log["A after B died"] == [2, 3, 1] and log["A destroyed"] == [2, 3, 2]
+    assert log["mlp twice"] == [1, 1, 0] and log["one of three destroyed"] == [1, 1, 1]

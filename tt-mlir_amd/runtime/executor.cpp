@@ -1921,13 +1921,17 @@ void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
     inputs.push_back(ctx.get(ins[i], "load_cached in"));
     versions.push_back(inputs.back().handle->version);
   }
-  auto key = std::make_pair(ctx.binary.id(), prog);
+  const ConstEvalKey key{ctx.binary.id(), prog, versions};
   {
-    std::lock_guard<std::mutex> g(ctx.dev->constEvalMu);
-    auto it = ctx.dev->constEval.find(key);
-    if (it != ctx.dev->constEval.end() && it->second.inputVersions == versions) {
+    std::vector<Tensor> cached;
+    {
+      std::lock_guard<std::mutex> g(ctx.dev->constEvalMu);
+      auto it = ctx.dev->constEval.find(key);
+      if (it != ctx.dev->constEval.end()) cached = it->second.outputs;
+    }
+    if (!cached.empty()) {
       debug::Stats::get().incrementStat("ConstEvalCacheHit");
-      for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], it->second.outputs.at(i));
+      for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], cached.at(i));
       return;
     }
   }
@@ -1936,8 +1940,30 @@ void runLoadCached(const fb::Table &op, ProgramContext &ctx) {
   TTRT_ASSERT(results.size() == outs.size(), "load_cached: callee returned a different number of outputs");
   for (auto &t : results) setTensorRetain(t, true);
   {
+    ConstEvalEntry replaced;   // destroyed after the lock is released
     std::lock_guard<std::mutex> g(ctx.dev->constEvalMu);
-    ctx.dev->constEval[key] = ConstEvalEntry{versions, results};
+    ConstEvalEntry &slot = ctx.dev->constEval[key];
+    replaced = std::move(slot);
+    slot = ConstEvalEntry{versions, results};
+  }
+  // The entry can be asked for only while all the tensors it was computed from exist (a version belongs to one tensor):
+  // when one of them is destroyed the entry goes with it, as in the reference (global_tensor_cache.cpp, store()).
+  std::weak_ptr<DeviceState> device = ctx.dev;
+  for (Tensor &in : inputs) {
+    std::lock_guard<std::mutex> g(in.handle->destroyMu);
+    in.handle->onDestroy.push_back([device, key] {
+      auto d = device.lock();
+      if (!d) return;
+      ConstEvalEntry dropped;   // destroyed after the lock is released
+      {
+        std::lock_guard<std::mutex> g2(d->constEvalMu);
+        auto it = d->constEval.find(key);
+        if (it == d->constEval.end()) return;
+        dropped = std::move(it->second);
+        d->constEval.erase(it);
+      }
+      debug::Stats::get().incrementStat("ConstEvalCacheEvicted");
+    });
   }
   for (std::uint32_t i = 0; i < outs.size(); ++i) ctx.put(outs[i], results[i]);
 }

@@ -234,6 +234,12 @@ DeviceRegistry &deviceRegistry() {
 }
 }  // namespace
 
+TensorImpl::~TensorImpl() {
+  for (auto &f : onDestroy) {
+    try { f(); } catch (...) { /* a destructor must not throw */ }
+  }
+}
+
 BinaryImpl::~BinaryImpl() {
   std::vector<std::shared_ptr<DeviceState>> devs;
   {
@@ -248,7 +254,7 @@ BinaryImpl::~BinaryImpl() {
     {
       std::lock_guard<std::mutex> g(d->constEvalMu);
       for (auto it = d->constEval.begin(); it != d->constEval.end();) {
-        if (it->first.first == id) { dropped.push_back(std::move(it->second)); it = d->constEval.erase(it); } else ++it;
+        if (std::get<0>(it->first) == id) { dropped.push_back(std::move(it->second)); it = d->constEval.erase(it); } else ++it;
       }
     }
     if (!d->open) continue;
@@ -556,9 +562,11 @@ void closeMeshDevice(Device d) {
   d.handle->traceCache.clear();
   {
     // const-eval results are memory of this device: they go back to the pool before the pool returns it to the driver
-    std::map<std::pair<std::uint64_t, std::uint32_t>, ConstEvalEntry> dropped;
-    std::lock_guard<std::mutex> g(d.handle->constEvalMu);
-    dropped.swap(d.handle->constEval);
+    std::map<ConstEvalKey, ConstEvalEntry> dropped;   // destroyed after the lock is released
+    {
+      std::lock_guard<std::mutex> g(d.handle->constEvalMu);
+      dropped.swap(d.handle->constEval);
+    }
   }
   pool().release();
   TTM_CALL(ttm_stream_destroy(d.handle->stream));

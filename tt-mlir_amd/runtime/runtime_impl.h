@@ -1,10 +1,12 @@
 // Internal state behind the opaque handles of runtime.h.
 #pragma once
 #include <atomic>
+#include <functional>
 #include <map>
 #include <mutex>
 #include <tuple>
 #include <utility>
+#include <vector>
 
 #include "runtime.h"
 #include "ttmlir_amd_hip.h"
@@ -39,6 +41,8 @@ struct ConstEvalEntry {
   std::vector<std::uint64_t> inputVersions;
   std::vector<Tensor> outputs;
 };
+// binary id, const-eval program, versions of the tensors it ran on
+using ConstEvalKey = std::tuple<std::uint64_t, std::uint32_t, std::vector<std::uint64_t>>;
 
 struct DeviceState {
   int deviceId = 0;
@@ -54,11 +58,13 @@ struct DeviceState {
   std::uint32_t nextTraceId = 1;
   std::map<std::uint32_t, TraceData> traces;      // by trace id: graphs recorded on this device
   std::map<TraceKey, std::uint32_t> traceCache;   // capture_or_execute_trace -> trace id
-  // const-eval results by (binary id, program index).  They are device memory of this device, so they live and die with it
-  // (the reference keys its cache by device id as well, load_cached.cpp:24-38): dropped at closeMeshDevice, and per binary
-  // when the binary is destroyed.
+  // const-eval results by (binary id, program index, input versions), one entry per combination as in the reference's
+  // GlobalTensorCache (device id, function hash, input versions; runtime/lib/ttnn/operations/cache/load_cached.cpp:24-38).
+  // They are device memory of this device, so they live and die with it: dropped at closeMeshDevice, per binary when the
+  // binary is destroyed, and singly when one of the tensors an entry was computed from is destroyed (nobody can ask for
+  // it again).  Entries are always destroyed outside the lock: their tensors may carry such callbacks themselves.
   std::mutex constEvalMu;
-  std::map<std::pair<std::uint64_t, std::uint32_t>, ConstEvalEntry> constEval;
+  std::map<ConstEvalKey, ConstEvalEntry> constEval;
   ~DeviceState();
 };
 
@@ -84,6 +90,11 @@ struct TensorImpl {
   std::atomic<bool> retain{false};
   std::shared_ptr<DeviceState> device;  // for device tensors
   std::uint64_t version = 0;
+  // run when the tensor is destroyed: const-eval results computed from it are dropped with it
+  // (runtime/lib/ttnn/operations/cache/global_tensor_cache.cpp, registerOnDestroyCallback)
+  std::mutex destroyMu;
+  std::vector<std::function<void()>> onDestroy;
+  ~TensorImpl();
 };
 
 struct BinaryImpl {
