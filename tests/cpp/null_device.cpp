@@ -6,6 +6,7 @@
 // backed by its whole padded extent).  A violation is an error return with a message, which the runtime turns into an
 // exception - on the GPU the same call would be a memory fault.  With this the host runtime (executor, tensor pool, fused
 // launches, traces) runs whole programs on the CPU: results are meaningless, the extents of every launch are checked.
+#include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
@@ -24,7 +25,7 @@ thread_local std::string g_err;
 std::mutex g_mu;
 std::map<uintptr_t, size_t> g_allocs;            // base -> bytes
 std::map<std::string, int> g_options;
-long g_kernel_calls = 0, g_capture_mark = -1;
+std::atomic<long> g_kernel_calls{0}, g_capture_mark{-1};
 
 int fail(const char *fmt, ...) {
   char buf[512];
@@ -179,12 +180,12 @@ EXPORT int ttm_event_elapsed_ms(float *ms, void *, void *) { if (ms) *ms = 0.0f;
 // ---- graphs: the launches between begin and end are counted, a replay does nothing
 EXPORT int ttm_graph_begin_capture(void *) {
   if (g_capture_mark >= 0) return fail("ttm_graph_begin_capture: a capture is already in progress");
-  g_capture_mark = g_kernel_calls;
+  g_capture_mark = g_kernel_calls.load();
   return TTM_OK;
 }
 EXPORT int ttm_graph_end_capture(void *, void **graph_exec, size_t *num_nodes) {
   if (g_capture_mark < 0) return fail("ttm_graph_end_capture: no capture in progress");
-  if (num_nodes) *num_nodes = (size_t)(g_kernel_calls - g_capture_mark);
+  if (num_nodes) *num_nodes = (size_t)(g_kernel_calls.load() - g_capture_mark.load());
   g_capture_mark = -1;
   if (graph_exec) *graph_exec = malloc(8);
   return TTM_OK;

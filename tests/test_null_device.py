@@ -311,3 +311,26 @@ print(json.dumps(log))
     assert log["A again"] == [2, 1, 0] and log["B again"] == [2, 2, 0]
     assert log["B destroyed"] == [2, 2, 1] and log["A after B died"] == [2, 3, 1] and log["A destroyed"] == [2, 3, 2]
     assert log["mlp twice"] == [1, 1, 0] and log["one of three destroyed"] == [1, 1, 1]
+
+
+def test_runtime_under_thread_sanitizer_on_the_null_device(tmp_path):
+    """tests/cpp/runtime_stress.cpp: six threads submit a program with a const-eval part on one device, creating and
+    destroying weight tensors as they go, while a seventh reads statistics.  The runtime's sources and the null device are
+    built with -fsanitize=thread: no data race, no deadlock, and every const-eval entry is evicted with its tensor."""
+    rtsrc = os.path.join(ROOT, "tt-mlir_amd", "runtime")
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", rtsrc]
+    common = ["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-pthread", "-fsanitize=thread"]
+    jobs = [subprocess.Popen(common + inc + ["-c", os.path.join(rtsrc, f), "-o", str(tmp_path / (f + ".o"))])
+            for f in sorted(os.listdir(rtsrc)) if f.endswith(".cpp")]
+    jobs.append(subprocess.Popen(common + ["-shared", "-fvisibility=hidden"] + inc + ["-o", str(tmp_path / "libttmlir_amd_hip.so"),
+                                           os.path.join(ROOT, "tests", "cpp", "null_device.cpp")]))
+    assert all(j.wait() == 0 for j in jobs)
+    objs = [str(p) for p in tmp_path.glob("*.o")]
+    subprocess.run(common + inc + [os.path.join(ROOT, "tests", "cpp", "runtime_stress.cpp")] + objs +
+                   ["-L", str(tmp_path), "-lttmlir_amd_hip", "-ldl", "-o", str(tmp_path / "stress")], check=True)
+    env = dict(os.environ, LD_LIBRARY_PATH=str(tmp_path), TSAN_OPTIONS="halt_on_error=0 exitcode=66")
+    r = subprocess.run([str(tmp_path / "stress")], env=env, capture_output=True, text=True, timeout=600)
+    assert "ThreadSanitizer" not in r.stderr, r.stderr[-3000:]
+    assert r.returncode == 0, (r.stdout, r.stderr[-1000:])
+    words = r.stdout.split()
+    assert words[0] == "submits" and int(words[1]) == 360 and int(words[3]) == int(words[7]) > 0   # miss == evicted
