@@ -313,13 +313,15 @@ print(json.dumps(log))
     assert log["mlp twice"] == [1, 1, 0] and log["one of three destroyed"] == [1, 1, 1]
 
 
-def test_runtime_under_thread_sanitizer_on_the_null_device(tmp_path):
+@pytest.mark.parametrize("sanitizer", ["thread", "address,undefined"])
+def test_runtime_under_sanitizers_on_the_null_device(tmp_path, sanitizer):
     """tests/cpp/runtime_stress.cpp: six threads submit a program with a const-eval part on one device, creating and
     destroying weight tensors as they go, while a seventh reads statistics.  The runtime's sources and the null device are
-    built with -fsanitize=thread: no data race, no deadlock, and every const-eval entry is evicted with its tensor."""
+    built with -fsanitize=thread (no data race, no deadlock) and with -fsanitize=address,undefined (no bad access, no
+    undefined behaviour, no leak); every const-eval entry is evicted with its tensor."""
     rtsrc = os.path.join(ROOT, "tt-mlir_amd", "runtime")
     inc = ["-I", os.path.join(ROOT, "include"), "-I", rtsrc]
-    common = ["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-pthread", "-fsanitize=thread"]
+    common = ["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-pthread", "-fsanitize=" + sanitizer, "-fno-sanitize-recover=undefined"]
     jobs = [subprocess.Popen(common + inc + ["-c", os.path.join(rtsrc, f), "-o", str(tmp_path / (f + ".o"))])
             for f in sorted(os.listdir(rtsrc)) if f.endswith(".cpp")]
     jobs.append(subprocess.Popen(common + ["-shared", "-fvisibility=hidden"] + inc + ["-o", str(tmp_path / "libttmlir_amd_hip.so"),
@@ -328,9 +330,10 @@ def test_runtime_under_thread_sanitizer_on_the_null_device(tmp_path):
     objs = [str(p) for p in tmp_path.glob("*.o")]
     subprocess.run(common + inc + [os.path.join(ROOT, "tests", "cpp", "runtime_stress.cpp")] + objs +
                    ["-L", str(tmp_path), "-lttmlir_amd_hip", "-ldl", "-o", str(tmp_path / "stress")], check=True)
-    env = dict(os.environ, LD_LIBRARY_PATH=str(tmp_path), TSAN_OPTIONS="halt_on_error=0 exitcode=66")
+    env = dict(os.environ, LD_LIBRARY_PATH=str(tmp_path), TSAN_OPTIONS="halt_on_error=0 exitcode=66", ASAN_OPTIONS="detect_leaks=1",
+               UBSAN_OPTIONS="print_stacktrace=1")
     r = subprocess.run([str(tmp_path / "stress")], env=env, capture_output=True, text=True, timeout=600)
-    assert "ThreadSanitizer" not in r.stderr, r.stderr[-3000:]
+    assert "Sanitizer" not in r.stderr and "runtime error" not in r.stderr, r.stderr[-3000:]
     assert r.returncode == 0, (r.stdout, r.stderr[-1000:])
     words = r.stdout.split()
     assert words[0] == "submits" and int(words[1]) == 360 and int(words[3]) == int(words[7]) > 0   # miss == evicted

@@ -272,6 +272,7 @@ private:
     std::memcpy(&buf_[buf_.size() - used_], p, n);
   }
   void pushZeros(size_t n) {
+    if (!n) return;
     grow(n);
     used_ += static_cast<Off>(n);
     std::memset(&buf_[buf_.size() - used_], 0, n);
