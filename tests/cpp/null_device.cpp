@@ -119,6 +119,7 @@ EXPORT int ttm_mem_info(size_t *free_bytes, size_t *total_bytes) {
 }
 EXPORT int ttm_malloc(void **dptr, size_t bytes) {
   if (!dptr) return fail("ttm_malloc: null out pointer");
+  if (bytes > ((size_t)2 << 30)) return fail("ttm_malloc: %zu bytes are more than this device has", bytes);   // damaged programs ask for anything
   void *p = nullptr;
   if (posix_memalign(&p, 256, bytes ? bytes : 1)) return fail("ttm_malloc: out of host memory (%zu bytes)", bytes);
   memset(p, 0, bytes);

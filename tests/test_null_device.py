@@ -337,3 +337,37 @@ def test_runtime_under_sanitizers_on_the_null_device(tmp_path, sanitizer):
     assert r.returncode == 0, (r.stdout, r.stderr[-1000:])
     words = r.stdout.split()
     assert words[0] == "submits" and int(words[1]) == 360 and int(words[3]) == int(words[7]) > 0   # miss == evicted
+
+
+def test_damaged_programs_through_the_runtime_under_address_sanitizer(tmp_path):
+    """tests/cpp/runtime_fuzz.cpp: four programs (MLP with const-eval, decoder layer, decode layer eager and traced) with a few
+    bytes flipped, 400 copies each, loaded and submitted on the null device with the runtime built under
+    -fsanitize=address,undefined.  A damaged program is refused or runs; it never makes the host runtime touch memory it does
+    not own, overflow an extent, or launch past a buffer."""
+    sys.path.insert(0, ROOT)
+    from ttmlir_amd import programs
+    files = []
+    for name, data in (("c4", programs.c4_mlp(64, 128, 256)), ("c5", programs.c5_decoder(96, 256, 4, 2, 64, 512)),
+                       ("decode", programs.decode_layer(8, 256, 4, 2, 64, 512, 128)),
+                       ("decode_traced", programs.decode_layer(8, 256, 4, 2, 64, 512, 128, trace=True))):
+        files.append(str(tmp_path / (name + ".ttnn")))
+        open(files[-1], "wb").write(data)
+    rtsrc = os.path.join(ROOT, "tt-mlir_amd", "runtime")
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", rtsrc]
+    common = ["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-pthread", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined"]
+    jobs = [subprocess.Popen(common + inc + ["-c", os.path.join(rtsrc, f), "-o", str(tmp_path / (f + ".o"))])
+            for f in sorted(os.listdir(rtsrc)) if f.endswith(".cpp")]
+    jobs.append(subprocess.Popen(common + ["-shared", "-fvisibility=hidden"] + inc + ["-o", str(tmp_path / "libttmlir_amd_hip.so"),
+                                           os.path.join(ROOT, "tests", "cpp", "null_device.cpp")]))
+    assert all(j.wait() == 0 for j in jobs)
+    subprocess.run(common + inc + [os.path.join(ROOT, "tests", "cpp", "runtime_fuzz.cpp")] + [str(p) for p in tmp_path.glob("*.o")] +
+                   ["-L", str(tmp_path), "-lttmlir_amd_hip", "-ldl", "-o", str(tmp_path / "fuzz")], check=True)
+    # a damaged shape may ask for any amount of memory: allocations above 4 GiB fail instead of being tried
+    env = dict(os.environ, LD_LIBRARY_PATH=str(tmp_path), ASAN_OPTIONS="max_allocation_size_mb=4096:allocator_may_return_null=1:detect_leaks=0",
+               UBSAN_OPTIONS="print_stacktrace=1")
+    r = subprocess.run([str(tmp_path / "fuzz"), "400"] + files, env=env, capture_output=True, text=True, timeout=900)
+    assert "Sanitizer" not in r.stderr and "runtime error" not in r.stderr, r.stderr[-3000:]
+    assert r.returncode == 0, (r.stdout[-300:], r.stderr[-1500:])
+    words = r.stdout.strip().splitlines()[-1].split()
+    stats = dict(zip(words[0::2], map(int, words[1::2])))
+    assert stats["out_of_bounds"] == 0 and stats["ran"] >= 4 and stats["refused"] > 100 and stats["loaded"] > 400, stats

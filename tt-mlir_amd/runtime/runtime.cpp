@@ -209,7 +209,23 @@ std::int64_t paddedVolume(const std::vector<std::uint32_t> &shape) {
   Dims3 d = dims3(shape);
   return d.batch * ((d.rows + 31) / 32 * 32) * ((d.cols + 31) / 32 * 32);
 }
+// Every allocation is sized here.  Extents come from the binary or the caller: their padded product is formed with a check
+// at every step, so that an absurd shape (a damaged binary) is an error and not an overflow that allocates a few bytes for
+// a tensor the kernels would then be launched on.
+static void requireRepresentableShape(const std::vector<std::uint32_t> &shape) {
+  TTRT_ASSERT(shape.size() <= 8, "tensor rank above 8");
+  constexpr std::uint64_t kMaxElements = std::uint64_t{1} << 40;   // 1 Ti elements: beyond any device
+  std::uint64_t v = 1;
+  for (size_t i = 0; i < shape.size(); ++i) {
+    const bool tiled = i + 2 >= shape.size();   // the last two extents may be padded to 32
+    const std::uint64_t e = tiled ? (static_cast<std::uint64_t>(shape[i]) + 31) / 32 * 32 : shape[i];
+    if (e == 0) return;                          // an empty tensor
+    TTRT_ASSERT(v <= kMaxElements / e, "tensor shape is too large to allocate");
+    v *= e;
+  }
+}
 size_t tensorBytes(const std::vector<std::uint32_t> &shape, DataType dtype, TensorLayout layout) {
+  requireRepresentableShape(shape);
   if (utils::isBlockFormatDataType(dtype)) {
     TTRT_ASSERT(layout == TensorLayout::Tile, "block-float tensors must be in tile layout");
     return static_cast<size_t>(paddedVolume(shape) / 1024) * utils::blockFormatTileSizeBytes(dtype);
@@ -327,7 +343,11 @@ std::vector<std::uint32_t> shapeFromTensorRef(const fb::Table &ref) {
   auto desc = ref.table(schema::TensorRef::f_desc);
   auto shp = desc.scalars<std::int32_t>(schema::TensorDesc::f_shape);
   std::vector<std::uint32_t> out(shp.size());
-  for (std::uint32_t i = 0; i < shp.size(); ++i) out[i] = static_cast<std::uint32_t>(shp[i]);
+  for (std::uint32_t i = 0; i < shp.size(); ++i) {
+    TTRT_ASSERT(shp[i] >= 0, "the binary declares a tensor with a negative extent");
+    out[i] = static_cast<std::uint32_t>(shp[i]);
+  }
+  requireRepresentableShape(out);   // every shape a binary declares passes here before anything is computed from it
   return out;
 }
 
