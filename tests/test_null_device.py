@@ -371,3 +371,65 @@ def test_damaged_programs_through_the_runtime_under_address_sanitizer(tmp_path):
     words = r.stdout.strip().splitlines()[-1].split()
     stats = dict(zip(words[0::2], map(int, words[1::2])))
     assert stats["out_of_bounds"] == 0 and stats["ran"] >= 4 and stats["refused"] > 100 and stats["loaded"] > 400, stats
+
+
+def test_reference_debug_hook_registration_semantics_on_the_null_device(null_env):
+    """runtime/test/ttnn/python/n150/test_debug_hooks.py: a second registration replaces the callbacks it names
+    (test_multiple_registrations, :275-347) and keeps the others (test_partial_re_registration, :349-412); unregistering
+    silences all (test_unregister_hooks, :202-273); an exception raised in a callback reaches the caller of submit
+    (test_callback_exception_handling, :416-458).  Hooks fire inside submit, which the null device makes possible here."""
+    code = r"""
+import sys, os, json, gc
+sys.path.insert(0, %r); sys.path.insert(0, os.path.join(%r, "tests"))
+import conftest, numpy as np
+from ttmlir_amd import programs, runtime as rt
+DT = rt.DataType
+dev = rt.open_mesh_device()
+b = rt.Binary.load_from_memory(programs.c1_matmul())
+def run():
+    ins = [rt.to_layout(rt.create_owned_host_tensor(np.zeros(s, dtype=np.uint16), l.dtype), dev, l) for s, l in b.get_program_inputs(0)]
+    return rt.submit(dev, b, 0, ins)
+class Tracker:
+    def __init__(self): self.pre_program = self.post_program = self.pre_op = self.post_op = 0
+    def on_pre_program(self, idx, hook): self.pre_program += 1
+    def on_post_program(self, idx, hook): self.post_program += 1
+    def on_pre_op(self, idx, name, dbg, hook): self.pre_op += 1
+    def on_post_op(self, idx, name, dbg, hook): self.post_op += 1
+    def counts(self): return [self.pre_program, self.post_program, self.pre_op, self.post_op]
+log = {}
+t1, t2 = Tracker(), Tracker()
+rt.set_program_callbacks(t1.on_pre_program, t1.on_post_program); run()
+log["first"] = [t1.counts(), t2.counts()]
+rt.set_program_callbacks(t2.on_pre_program, t2.on_post_program); run()
+log["replaced"] = [t1.counts(), t2.counts()]
+rt.clear_callbacks(); run()
+log["unregistered"] = [t1.counts(), t2.counts()]
+t = Tracker()
+rt.set_program_callbacks(t.on_pre_program, t.on_post_program); run()
+log["program only"] = t.counts()
+rt.set_pre_op_callback(t.on_pre_op); rt.set_post_op_callback(t.on_post_op); gc.collect(); run()
+log["merged"] = t.counts()
+rt.set_program_callbacks(post=t2.on_post_program); gc.collect(); run()      # pre stays t's, post becomes t2's
+log["post replaced"] = [t.counts(), t2.counts()]
+rt.clear_callbacks()
+def failing(idx, hook): raise ValueError("Intentional callback failure")
+rt.set_program_callbacks(pre=failing)
+try:
+    run(); log["exception"] = "none"
+except ValueError as e:
+    log["exception"] = str(e)
+rt.clear_callbacks()
+run()                                                                    # and nothing lingers
+rt.close_mesh_device(dev)
+print(json.dumps(log))
+""" % (ROOT, ROOT)
+    r = subprocess.run([sys.executable, "-c", code], env=null_env, capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert r.returncode == 0, r.stderr[-1500:]
+    log = json.loads(r.stdout.strip().splitlines()[-1])
+    assert log["first"] == [[1, 1, 0, 0], [0, 0, 0, 0]]
+    assert log["replaced"] == [[1, 1, 0, 0], [1, 1, 0, 0]] and log["unregistered"] == log["replaced"]
+    assert log["program only"] == [1, 1, 0, 0]
+    n_ops = log["merged"][2]
+    assert log["merged"] == [2, 2, n_ops, n_ops] and n_ops == 7                 # the seven operations of config 1
+    assert log["post replaced"] == [[3, 2, 2 * n_ops, 2 * n_ops], [1, 2, 0, 0]]
+    assert log["exception"] == "Intentional callback failure"

@@ -396,8 +396,15 @@ def submit(device, binary, program, inputs):
     ins = (ctypes.c_void_p * max(1, len(inputs)))(*[t.h for t in inputs])
     outs = (ctypes.c_void_p * 64)()
     n = ctypes.c_uint32()
-    _call("ttrt_submit", device.h, binary.h, program, ins, len(inputs), outs, 64, ctypes.byref(n))
-    return [Tensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
+    del _callback_error[:]
+    try:
+        _call("ttrt_submit", device.h, binary.h, program, ins, len(inputs), outs, 64, ctypes.byref(n))
+    except RuntimeError_:
+        _raise_callback_error()   # the callback's own exception says more than what it led to
+        raise
+    results = [Tensor(ctypes.c_void_p(outs[i])) for i in range(n.value)]
+    _raise_callback_error()
+    return results
 
 
 def deallocate_tensor(tensor, force=False):
@@ -522,9 +529,31 @@ class HookContext:
         return list(shape[: rank.value]), dt.value
 
 
+# An exception cannot cross the C frames between a callback and submit(): the first one a callback raises is kept, the
+# callbacks after it do nothing, and submit() raises it when the program returns (the reference's bindings let it travel
+# through, runtime/test/ttnn/python/n150/test_debug_hooks.py:416-458: the caller sees the callback's exception either way).
+_callback_error = []
+
+
+def _guarded(fn, *args):
+    if _callback_error:
+        return
+    try:
+        fn(*args)
+    except BaseException as e:
+        _callback_error.append(e)
+
+
+def _raise_callback_error():
+    if _callback_error:
+        e = _callback_error[0]
+        del _callback_error[:]
+        raise e
+
+
 def _op_trampoline(fn):
     def tramp(idx, name, dbg, hook, user):
-        fn(idx, name.decode("utf-8", "replace"), dbg.decode("utf-8", "replace"), HookContext(hook))
+        _guarded(fn, idx, name.decode("utf-8", "replace"), dbg.decode("utf-8", "replace"), HookContext(hook))
     return _CB_TYPE(tramp)
 
 
@@ -545,9 +574,15 @@ def set_program_callbacks(pre=None, post=None):
     def wrap(fn):
         if fn is None:
             return _PROGRAM_CB_TYPE()
-        return _PROGRAM_CB_TYPE(lambda idx, hook, user: fn(idx, HookContext(hook)))
-    _cb_keep["pre_program"], _cb_keep["post_program"] = wrap(pre), wrap(post)
-    _call("ttrt_set_program_callbacks", _cb_keep["pre_program"], _cb_keep["post_program"], None)
+        return _PROGRAM_CB_TYPE(lambda idx, hook, user: _guarded(fn, idx, HookContext(hook)))
+    new_pre, new_post = wrap(pre), wrap(post)
+    _call("ttrt_set_program_callbacks", new_pre, new_post, None)
+    # a callback that is not given stays registered (the reference merges registrations,
+    # runtime/test/ttnn/python/n150/test_debug_hooks.py:349-412): its trampoline must stay alive with it
+    if pre is not None:
+        _cb_keep["pre_program"] = new_pre
+    if post is not None:
+        _cb_keep["post_program"] = new_post
 
 
 def walk_program(binary, program_index, fn):
