@@ -1,4 +1,4 @@
-// The sketch of INTEGRATION.md section 1, compiled: a fourth arm of the reference's dispatch that forwards to the C ABI.
+// The integration sketch for the reference's runtime dispatch, compiled: a fourth arm of that dispatch that forwards to the C ABI.
 // The three structs below are stand-ins with the two properties the arm needs of the reference's handle types
 // (runtime/include/tt/runtime/types.h:112-135): a shared_ptr<void> member `handle` and construction from
 // (handle, ..., DeviceRuntime).  Runs on the host: it loads a binary that the Python side wrote and walks its metadata;

@@ -1,5 +1,5 @@
 """C++ translation units compiled and run on the host (no GPU): the device pool's bookkeeping with a mock driver, and the
-integration sketches of INTEGRATION.md compiled against the public headers."""
+sketches of how the reference's runtime would bind this one, compiled against the public headers."""
 import os
 import subprocess
 
@@ -27,7 +27,7 @@ def test_device_pool_bookkeeping(tmp_path):
 
 
 def test_runtime_arm_sketch_compiles_and_runs(tmp_path):
-    """The fourth dispatch arm of INTEGRATION.md: include/ttmlir_amd_runtime_arm.hpp over the C ABI, in its own namespace,
+    """The fourth arm of the reference's runtime dispatch: include/ttmlir_amd_runtime_arm.hpp over the C ABI, in its own namespace,
     linked against the exported ttrt_* symbols only."""
     import sys
     sys.path.insert(0, ROOT)
