@@ -157,7 +157,11 @@ def _verify_extents(name, args):
     spec = _EXTENTS.get(name)
     if spec is None:
         return
-    for idx, need, what in spec(args):
+    try:
+        extents = spec(args)
+    except (KeyError, IndexError, TypeError):
+        return   # arguments the size rules do not cover (an unknown dtype code, a short argument list): the library answers
+    for idx, need, what in extents:
         p = args[idx]
         if isinstance(p, _Ptr) and p.nbytes is not None and p.nbytes < need:
             raise TTMError("%s: the %s (argument %d) has %d bytes, the kernels touch %d from its address on (tile tensors are "
