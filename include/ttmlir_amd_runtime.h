@@ -226,6 +226,11 @@ int ttrt_pb_capture_or_execute_trace(ttrt_builder *pb, uint32_t capture_program,
 int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force);
 /* location of the operation added last, and an expected (golden) tensor to embed for a location; data is row-major */
 int ttrt_pb_last_op_loc(ttrt_builder *pb, char *buf, size_t len);
+/* the next matmul / linear carries a matmul_program_config of this kind (value of the MatmulProgramConfig union,
+ * include/ttmlir/Target/TTNN/operations/matmul.fbs:56-62; 0 = none) whose fused_activation is the UnaryOpType
+ * `fused_activation`, absent when negative: runtime/lib/ttnn/operations/matmul/matmul.cpp:17-44 lets it replace the op's
+ * own activation string */
+int ttrt_pb_set_matmul_program_config(ttrt_builder *pb, int kind, int fused_activation);
 /* the next tensor the builder creates is declared with this shape instead of the one its operation gives: a program that
  * lies about a result, for tests of what the executor does with one */
 int ttrt_pb_declare_next_shape(ttrt_builder *pb, const uint32_t *shape, int rank);

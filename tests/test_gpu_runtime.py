@@ -705,13 +705,65 @@ def test_traced_program_replays_as_a_graph(device, orc):
     # the traced function's closing copy into the output slot is folded into the last projection (once in the eager run of
     # the capture program, once while recording)
     assert rt.get_stat("FusedCopyIntoSlot") == 2
-    # a parameter replaced by the caller (new tensor, new version) is copied into its slot before the replay
+    # parameters replaced by the caller are other tensors at other addresses: another trace is recorded on them, and the
+    # first one, with the const-eval results it reads, is still there when the caller comes back to the original weights
     res_t2, res_e2 = resident(traced, main, 2.0), resident(eager, 1, 2.0)
     x = torch.randn((T, H), generator=g).to(torch.bfloat16)
     y2 = _run_traced(traced, device, x, res_t2)
     assert torch.equal(y2, _run_traced(eager, device, x, res_e2))
-    assert not torch.equal(y2, _run_traced(traced, device, x, res_t))
-    assert rt.get_stat("CapturedTrace") == 1 and rt.get_stat("ExecutedTrace") == 6
+    y1 = _run_traced(traced, device, x, res_t)
+    assert not torch.equal(y2, y1) and torch.equal(y1, _run_traced(eager, device, x, res_e))
+    assert rt.get_stat("CapturedTrace") == 2 and rt.get_stat("ExecutedTrace") == 5
+
+
+def test_traced_program_with_alternating_weight_sets(device, orc):
+    """Weight sets A, B, A, B, ... through a traced program and through the same program run op by op: every result equal
+    and right, each set packed by const-eval once and recorded once, and the caller's tensors left as they were (a trace
+    never writes into a device-resident input: capture_or_execute_trace.cpp:96-150 copies a changed parameter into its
+    slot, and that slot is the previous parameter's own memory)."""
+    T, H, F = 32, 128, 256
+    traced = rt.Binary.load_from_memory(programs.traced_mlp(T, H, F))
+    eager = rt.Binary.load_from_memory(programs.traced_mlp(T, H, F, trace=False))
+    main = traced.get_num_programs() - 1
+    f = lambda t: t.float().numpy()
+    sets = []
+    for seed, scale in ((41, 1.0), (42, 1.5), (43, 0.5)):
+        d = datagen.c4_mlp(T, H, F, seed=seed)
+        ts = [d["norm_w"], bf(d["wg"] * scale), bf(d["wu"]), bf(d["wd"])]
+        on = lambda binary, prog: [rt.to_layout(rt.from_torch(t), device, rt.get_layout(binary, prog, k + 1), retain=True)
+                                   for k, t in enumerate(ts)]
+        sets.append((ts, on(traced, main), on(eager, 1)))
+    rt.clear_stats()
+    g = torch.Generator().manual_seed(9)
+    order = [0, 1, 0, 1, 2, 0, 1, 2]
+    for it, k in enumerate(order):
+        ts, res_t, res_e = sets[k]
+        x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+        y = _run_traced(traced, device, x, res_t)
+        assert torch.equal(y, _run_traced(eager, device, x, res_e)), "submit %d (weight set %d) differs from the op-by-op run" % (it, k)
+        ref = oracle_mlp(orc, f(x), f(ts[0]), f(ts[1]), f(ts[2]), f(ts[3]), 1e-5)
+        assert np.max(np.abs(f(y) - ref)) <= 2.0 ** -9, (it, k)
+    # one capture and one const-eval run per weight set and binary, everything else replayed from the caches
+    assert rt.get_stat("CapturedTrace") == 3 and rt.get_stat("ExecutedTrace") == len(order) - 3
+    assert rt.get_stat("ConstEvalCacheMiss") == 6 and rt.get_stat("ConstEvalCacheHit") == 2 * (len(order) - 3)
+    for ts, res_t, res_e in sets:
+        for t, a, b in zip(ts, res_t, res_e):
+            for dev_t in (a, b):
+                assert torch.equal(rt.to_torch(rt.to_host(dev_t, untilize=True)[0]).reshape(t.shape), t), "a caller's tensor was changed"
+    # a fifth and sixth set push the least recently used traces out; the survivors still replay correctly
+    for seed in (44, 45):
+        d = datagen.c4_mlp(T, H, F, seed=seed)
+        ts = [d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+        res = [rt.to_layout(rt.from_torch(t), device, rt.get_layout(traced, main, k + 1), retain=True) for k, t in enumerate(ts)]
+        x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+        ref = oracle_mlp(orc, f(x), f(ts[0]), f(ts[1]), f(ts[2]), f(ts[3]), 1e-5)
+        assert np.max(np.abs(f(_run_traced(traced, device, x, res)) - ref)) <= 2.0 ** -9
+    assert rt.get_stat("CapturedTrace") == 5 and rt.get_stat("ReleasedTrace") == 1
+    for k, captured in ((0, 6), (2, 6), (1, 7)):   # set 0 was released and is recorded again, which pushes set 1 out
+        ts, res_t, res_e = sets[k]
+        x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+        assert torch.equal(_run_traced(traced, device, x, res_t), _run_traced(eager, device, x, res_e)), k
+        assert rt.get_stat("CapturedTrace") == captured and rt.get_stat("ReleasedTrace") == captured - 4, k
 
 
 def test_traced_program_with_grouped_two_pass_linears(device):

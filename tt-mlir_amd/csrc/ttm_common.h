@@ -77,6 +77,11 @@ __host__ __device__ static inline int64_t ttm_tiled_offset(int64_t r, int64_t c,
   return tile * 1024 + face * 256 + (r & 15) * 16 + (c & 15);
 }
 
+// Maximum and minimum that return NaN when either operand is NaN (one v_maximum3_f32 / v_minimum3_f32 on gfx950), as
+// tosa.reduce_max / arith.maximumf of the CPU lowering and torch.max do; fmaxf / fminf return the other operand.
+__device__ __forceinline__ float ttm_max(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+__device__ __forceinline__ float ttm_min(float a, float b) { return __builtin_elementwise_minimum(a, b); }
+
 __device__ static inline float ttm_bf16_to_f32(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
 // f32 -> bf16, round to nearest even (v_cvt_pk_bf16_f32 on gfx950; NaN stays a quiet NaN)
 typedef __bf16 ttm_bf16x2 __attribute__((ext_vector_type(2)));

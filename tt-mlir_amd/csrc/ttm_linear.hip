@@ -115,7 +115,7 @@ __device__ __forceinline__ float apply_act(float x) {
   if (ACT == TTM_ACT_GELU) return ttm_gelu_fast(x);
   if (ACT == TTM_ACT_SILU) return ttm_silu(x);
   if (ACT == TTM_ACT_SIGMOID) return ttm_sigmoid(x);
-  if (ACT == TTM_ACT_RELU) return fmaxf(x, 0.0f);
+  if (ACT == TTM_ACT_RELU) return ttm_max(x, 0.0f);   // keeps NaN, as arith.maximumf does
   return x;
 }
 

@@ -118,8 +118,8 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
     for (int i = 0; i < EPC; ++i) {
       bool ok = cp.c0 + i < cols;
       if (MODE == RW_RMSNORM) acc += ok ? f[i] * f[i] : 0.0f;
-      else if (IS_MAX) acc = ok ? fmaxf(acc, f[i]) : acc;
-      else if (MODE == RW_MIN) acc = ok ? fminf(acc, f[i]) : acc;
+      else if (IS_MAX) acc = ok ? ttm_max(acc, f[i]) : acc;
+      else if (MODE == RW_MIN) acc = ok ? ttm_min(acc, f[i]) : acc;
       else acc += ok ? f[i] : 0.0f;
     }
   }
@@ -129,7 +129,7 @@ __global__ __launch_bounds__(256) void ttm_rowwise_k(RowArgs p) {
 #pragma unroll
   for (int k = 1; k < J; ++k) {
     float o = part[k][rl];
-    stat = IS_MAX ? fmaxf(stat, o) : (MODE == RW_MIN ? fminf(stat, o) : stat + o);
+    stat = IS_MAX ? ttm_max(stat, o) : (MODE == RW_MIN ? ttm_min(stat, o) : stat + o);
   }
 
   if (MODE == RW_SUM || MODE == RW_MEAN || MODE == RW_MAX || MODE == RW_MIN) {
@@ -230,14 +230,14 @@ __global__ __launch_bounds__(256) void ttm_rowwise_resident_k(RowArgs p) {
     for (int i = 0; i < EPC; ++i) {
       const bool ok = cp.c0 + i < cols;
       if (MODE == RW_RMSNORM) acc += ok ? f[i] * f[i] : 0.0f;
-      else acc = ok ? fmaxf(acc, f[i]) : acc;
+      else acc = ok ? ttm_max(acc, f[i]) : acc;
     }
   }
   part[j][rl] = acc;
   __syncthreads();
   float stat = part[0][rl];
 #pragma unroll
-  for (int k = 1; k < J; ++k) stat = MODE == RW_SOFTMAX ? fmaxf(stat, part[k][rl]) : stat + part[k][rl];
+  for (int k = 1; k < J; ++k) stat = MODE == RW_SOFTMAX ? ttm_max(stat, part[k][rl]) : stat + part[k][rl];
   float mul = 0.0f;
   if (MODE == RW_RMSNORM) mul = 1.0f / sqrtf(stat / (float)cols + p.eps);
   else {
@@ -352,15 +352,15 @@ __global__ __launch_bounds__(256) void ttm_rowwise_row_k(RowArgs p, int total_ro
       for (int i = 0; i < EPC; ++i) {
         const bool ok = c0 + i < cols;
         if (MODE == RW_RMSNORM) acc += ok ? f[i] * f[i] : 0.0f;
-        else acc = ok ? fmaxf(acc, f[i]) : acc;
+        else acc = ok ? ttm_max(acc, f[i]) : acc;
       }
     }
   }
 #pragma unroll
-  for (int s = 32; s > 0; s >>= 1) acc = MODE == RW_SOFTMAX ? fmaxf(acc, __shfl_xor(acc, s)) : acc + __shfl_xor(acc, s);
+  for (int s = 32; s > 0; s >>= 1) acc = MODE == RW_SOFTMAX ? ttm_max(acc, __shfl_xor(acc, s)) : acc + __shfl_xor(acc, s);
   if (lane == 0) red[wave] = acc;
   __syncthreads();
-  const float stat = MODE == RW_SOFTMAX ? fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])) : red[0] + red[1] + red[2] + red[3];
+  const float stat = MODE == RW_SOFTMAX ? ttm_max(ttm_max(red[0], red[1]), ttm_max(red[2], red[3])) : red[0] + red[1] + red[2] + red[3];
   float mul;
   if (MODE == RW_RMSNORM) {
     mul = 1.0f / sqrtf(stat / (float)cols + p.eps);
@@ -485,7 +485,7 @@ __global__ __launch_bounds__(NT) TTM_MAX_WAVES((NT == 512 ? 2 : band_max_waves<M
     for (int sft = 1; sft < 64; sft <<= 1) {
       if (sft >= ELEM && sft < RUN) continue;            // the row bits
       const float o = __shfl_xor(a, sft);
-      a = is_max ? fmaxf(a, o) : (is_min ? fminf(a, o) : a + o);
+      a = is_max ? ttm_max(a, o) : (is_min ? ttm_min(a, o) : a + o);
     }
     return a;
   };
@@ -501,8 +501,8 @@ __global__ __launch_bounds__(NT) TTM_MAX_WAVES((NT == 512 ? 2 : band_max_waves<M
     for (int i = 0; i < EPC; ++i) {
       const bool ok = c0 + i < lim;
       if (MODE == RW_RMSNORM) acc += ok ? f[i] * f[i] : 0.0f;
-      else if (IS_MAX) acc = ok ? fmaxf(acc, f[i]) : acc;
-      else if (MODE == RW_MIN) acc = ok ? fminf(acc, f[i]) : acc;
+      else if (IS_MAX) acc = ok ? ttm_max(acc, f[i]) : acc;
+      else if (MODE == RW_MIN) acc = ok ? ttm_min(acc, f[i]) : acc;
       else acc += ok ? f[i] : 0.0f;
     }
   }
@@ -513,12 +513,12 @@ __global__ __launch_bounds__(NT) TTM_MAX_WAVES((NT == 512 ? 2 : band_max_waves<M
   {
     auto four = [&](int w0) {
       const float a0 = red[w0][rl], a1 = red[w0 + 1][rl], a2 = red[w0 + 2][rl], a3 = red[w0 + 3][rl];
-      return IS_MAX ? fmaxf(fmaxf(a0, a1), fmaxf(a2, a3)) : (MODE == RW_MIN ? fminf(fminf(a0, a1), fminf(a2, a3)) : (a0 + a1) + (a2 + a3));
+      return IS_MAX ? ttm_max(ttm_max(a0, a1), ttm_max(a2, a3)) : (MODE == RW_MIN ? ttm_min(ttm_min(a0, a1), ttm_min(a2, a3)) : (a0 + a1) + (a2 + a3));
     };
     stat = four(0);
     if constexpr (NW == 8) {
       const float hi = four(4);
-      stat = IS_MAX ? fmaxf(stat, hi) : (MODE == RW_MIN ? fminf(stat, hi) : stat + hi);
+      stat = IS_MAX ? ttm_max(stat, hi) : (MODE == RW_MIN ? ttm_min(stat, hi) : stat + hi);
     }
   }
   if constexpr (REDUCE) {
@@ -660,7 +660,7 @@ __global__ __launch_bounds__(256) void ttm_rowwise_wide_stats_k(RowArgs p, float
     if (MODE == RW_SOFTMAX) {
       float cm = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < EPC; ++i) cm = c0 + i < cols ? fmaxf(cm, f[i]) : cm;
+      for (int i = 0; i < EPC; ++i) cm = c0 + i < cols ? ttm_max(cm, f[i]) : cm;
       if (cm > a) { l *= expf(a - cm); a = cm; }   // a = -inf at first: l is 0 and stays 0
       if (a != -INFINITY) {
 #pragma unroll
@@ -671,8 +671,8 @@ __global__ __launch_bounds__(256) void ttm_rowwise_wide_stats_k(RowArgs p, float
       for (int i = 0; i < EPC; ++i) {
         const bool ok = c0 + i < cols;
         if (MODE == RW_RMSNORM) a += ok ? f[i] * f[i] : 0.0f;
-        else if (MODE == RW_MAX) a = ok ? fmaxf(a, f[i]) : a;
-        else if (MODE == RW_MIN) a = ok ? fminf(a, f[i]) : a;
+        else if (MODE == RW_MAX) a = ok ? ttm_max(a, f[i]) : a;
+        else if (MODE == RW_MIN) a = ok ? ttm_min(a, f[i]) : a;
         else a += ok ? f[i] : 0.0f;
       }
     }
@@ -685,7 +685,7 @@ __global__ __launch_bounds__(256) void ttm_rowwise_wide_stats_k(RowArgs p, float
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const float v = sa[L::partner(tid, i)];
-      A = IS_MAX ? fmaxf(A, v) : (MODE == RW_MIN ? fminf(A, v) : A + v);
+      A = IS_MAX ? ttm_max(A, v) : (MODE == RW_MIN ? ttm_min(A, v) : A + v);
     }
     if (MODE == RW_SOFTMAX) {
 #pragma unroll
@@ -706,8 +706,8 @@ __device__ __forceinline__ void wide_fold(float &A, float &Ls, float v, float w)
   if (MODE == RW_SOFTMAX) {
     if (v > A) { Ls = Ls * expf(A - v) + w; A = v; }   // A = -inf: Ls is 0 and exp gives 0
     else if (v != -INFINITY) Ls += w * expf(v - A);
-  } else if (MODE == RW_MAX) A = fmaxf(A, v);
-  else if (MODE == RW_MIN) A = fminf(A, v);
+  } else if (MODE == RW_MAX) A = ttm_max(A, v);
+  else if (MODE == RW_MIN) A = ttm_min(A, v);
   else A += v;
 }
 template <int MODE>

@@ -683,6 +683,11 @@ class ProgramBuilder:
     def from_device(self, t):
         return self._op("ttrt_pb_from_device", t)
 
+    def set_matmul_program_config(self, kind, fused_activation=-1):
+        """The next matmul / linear carries a program config of this kind (1-4, the MatmulProgramConfig union) whose
+        fused_activation is the given UnaryOpType (absent when negative)."""
+        _call("ttrt_pb_set_matmul_program_config", self.h, int(kind), int(fused_activation))
+
     def matmul(self, a, b, transpose_a=False, transpose_b=False, activation="", out_dtype=DataType.BFloat16):
         return self._op("ttrt_pb_matmul", a, b, int(transpose_a), int(transpose_b), activation.encode(), out_dtype)
 

@@ -594,6 +594,9 @@ TTRT_EXPORT int ttrt_pb_execute_trace(ttrt_builder *pb, uint32_t trace_id, int b
 TTRT_EXPORT int ttrt_pb_deallocate(ttrt_builder *pb, uint32_t in, int force) {
   return guard([&] { need(pb, "builder"); pb->pb.deallocate(in, force != 0); });
 }
+TTRT_EXPORT int ttrt_pb_set_matmul_program_config(ttrt_builder *pb, int kind, int fused_activation) {
+  return guard([&] { need(pb, "builder"); pb->pb.setMatmulProgramConfig(kind, fused_activation); });
+}
 TTRT_EXPORT int ttrt_pb_declare_next_shape(ttrt_builder *pb, const uint32_t *shape, int rank) {
   return guard([&] { need(pb, "builder"); pb->pb.declareNextShape(shapeVec(shape, rank)); });
 }

@@ -303,6 +303,38 @@ int activationCode(std::string_view s) {
   fatal("unsupported fused activation '" + std::string(s) + "'");
 }
 
+// The activation a matmul / linear op applies (runtime/lib/ttnn/operations/matmul/matmul.cpp:17-44, 64-66, 116-119): the
+// multicast program configs carry a fused_activation of their own, and when one is present it is the one that runs; the
+// op's `activation` string counts only without it.
+std::string matmulActivation(const fb::Table &op, int configTypeSlot, int configSlot, int activationSlot) {
+  const auto kind = static_cast<schema::MatmulProgramConfig>(op.scalar<std::uint8_t>(configTypeSlot, 0));
+  int fusedSlot = -1;
+  switch (kind) {
+  case schema::MatmulProgramConfig::MatmulMultiCoreReuseMultiCastProgramConfig:
+    fusedSlot = schema::MatmulMultiCoreReuseMultiCastProgramConfig::f_fused_activation; break;
+  case schema::MatmulProgramConfig::MatmulMultiCoreReuseMultiCast1DProgramConfig:
+    fusedSlot = schema::MatmulMultiCoreReuseMultiCast1DProgramConfig::f_fused_activation; break;
+  case schema::MatmulProgramConfig::MatmulMultiCoreReuseMultiCastDRAMShardedProgramConfig:
+    fusedSlot = schema::MatmulMultiCoreReuseMultiCastDRAMShardedProgramConfig::f_fused_activation; break;
+  default: break;
+  }
+  if (fusedSlot >= 0) {
+    if (fb::Table config = op.table(configSlot)) {
+      if (fb::Table fused = config.table(fusedSlot)) {
+        const auto type = static_cast<schema::UnaryOpType>(fused.scalar<std::uint32_t>(schema::UnaryWithParam::f_op_type, 0));
+        switch (type) {
+        case schema::UnaryOpType::Gelu: return "gelu";
+        case schema::UnaryOpType::Relu: return "relu";
+        case schema::UnaryOpType::Sigmoid: return "sigmoid";
+        case schema::UnaryOpType::Silu: return "silu";
+        default: fatal("unsupported fused activation in the matmul program config: UnaryOpType " + std::to_string(static_cast<std::uint32_t>(type)));
+        }
+      }
+    }
+  }
+  return std::string(op.string(activationSlot));
+}
+
 // ---- layout ops (runtime/lib/ttnn/operations/layout/*.cpp)
 void runToLayout(const fb::Table &op, ProgramContext &ctx) {
   Tensor in = ctx.get(op.table(schema::ToLayoutOp::f_in), "to_layout in");
@@ -617,18 +649,18 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
       if ((t != OpType::MatmulOp && t != OpType::LinearOp) || ctx.skip.count(j)) break;
       fb::Table a2, b2, out2;
       bool plainOperands;
-      std::string_view act2;
+      std::string act2;
       if (t == OpType::MatmulOp) {
         using M2 = schema::MatmulOp;
         a2 = nop.table(M2::f_a); b2 = nop.table(M2::f_b); out2 = nop.table(M2::f_out);
         plainOperands = !nop.scalar<std::uint8_t>(M2::f_transpose_a, 0) && !nop.scalar<std::uint8_t>(M2::f_transpose_b, 0);
-        act2 = nop.string(M2::f_activation);
+        act2 = matmulActivation(nop, M2::f_matmul_program_config_type, M2::f_matmul_program_config, M2::f_activation);
       } else {
         using L2 = schema::LinearOp;
         a2 = nop.table(L2::f_a); b2 = nop.table(L2::f_b); out2 = nop.table(L2::f_out);
         plainOperands = !nop.scalar<std::uint8_t>(L2::f_transpose_a, 0) && !nop.scalar<std::uint8_t>(L2::f_transpose_b, 0) &&
                         !nop.table(L2::f_bias);
-        act2 = nop.string(L2::f_activation);
+        act2 = matmulActivation(nop, L2::f_matmul_program_config_type, L2::f_matmul_program_config, L2::f_activation);
       }
       if (!a2 || !b2 || !out2 || refId(a2) != refId(aRef) || !plainOperands) break;
       auto wit = ctx.pool.find(refId(b2));
@@ -737,12 +769,16 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
 void runMatmul(const fb::Table &op, ProgramContext &ctx) {
   runMatmulLike(ctx, op.table(schema::MatmulOp::f_a), op.table(schema::MatmulOp::f_b), fb::Table(), op.table(schema::MatmulOp::f_out),
                 op.scalar<std::uint8_t>(schema::MatmulOp::f_transpose_a, 0) != 0,
-                op.scalar<std::uint8_t>(schema::MatmulOp::f_transpose_b, 0) != 0, op.string(schema::MatmulOp::f_activation));
+                op.scalar<std::uint8_t>(schema::MatmulOp::f_transpose_b, 0) != 0,
+                matmulActivation(op, schema::MatmulOp::f_matmul_program_config_type, schema::MatmulOp::f_matmul_program_config,
+                                 schema::MatmulOp::f_activation));
 }
 void runLinear(const fb::Table &op, ProgramContext &ctx) {
   runMatmulLike(ctx, op.table(schema::LinearOp::f_a), op.table(schema::LinearOp::f_b), op.table(schema::LinearOp::f_bias),
                 op.table(schema::LinearOp::f_out), op.scalar<std::uint8_t>(schema::LinearOp::f_transpose_a, 0) != 0,
-                op.scalar<std::uint8_t>(schema::LinearOp::f_transpose_b, 0) != 0, op.string(schema::LinearOp::f_activation));
+                op.scalar<std::uint8_t>(schema::LinearOp::f_transpose_b, 0) != 0,
+                matmulActivation(op, schema::LinearOp::f_matmul_program_config_type, schema::LinearOp::f_matmul_program_config,
+                                 schema::LinearOp::f_activation));
 }
 
 // ---- eltwise (runtime/lib/ttnn/operations/eltwise/{unary,binary}/*.cpp)
@@ -2148,8 +2184,9 @@ void runCopy(const fb::Table &op, ProgramContext &ctx) {
 
 bool inDeviceMemory(const fb::Table &ref) { return layoutFromTensorRef(ref).storageType == StorageType::Device; }
 
-// Copies the current values of the op's inputs into the persistent input slots; a slot whose version equals its
-// input's already holds the data (device-resident inputs are their own slots).
+// Copies the current values of the op's inputs into the persistent input slots.  A slot that is its input's own memory
+// (device-resident inputs pass through the allocation program) needs nothing; any other slot belongs to the trace and is
+// overwritten when its version is not its input's.
 void updateTraceInputSlots(const fb::Table &op, ProgramContext &ctx, std::vector<Tensor> &slots, bool deviceResidentOnly) {
   auto ins = op.tables(schema::CaptureOrExecuteTraceOp::f_inputs);
   TTRT_ASSERT(ins.size() == slots.size(), "capture_or_execute_trace: mismatched number of input slots");
@@ -2157,6 +2194,7 @@ void updateTraceInputSlots(const fb::Table &op, ProgramContext &ctx, std::vector
     const bool resident = inDeviceMemory(ins[i]);
     if (deviceResidentOnly && !resident) continue;
     Tensor &in = ctx.get(ins[i], "trace input");
+    if (in.handle->data.get() == slots[i].handle->data.get()) continue;
     if (in.handle->version == slots[i].handle->version) continue;
     overwriteTensor(ctx, slots[i], in, "trace input slot");
     slots[i].handle->version = in.handle->version;
@@ -2173,7 +2211,10 @@ void runCaptureOrExecuteTrace(const fb::Table &op, ProgramContext &ctx) {
   const std::uint32_t allocateId = op.scalar<std::uint32_t>(schema::CaptureOrExecuteTraceOp::f_allocate_slots_program_id, 0);
   auto ins = op.tables(schema::CaptureOrExecuteTraceOp::f_inputs);
   auto outs = op.tables(schema::CaptureOrExecuteTraceOp::f_outputs);
-  TraceKey key{ctx.binary.id(), ctx.programIndex, captureId, executeId};
+  std::vector<const void *> residentAddresses;
+  for (std::uint32_t i = 0; i < ins.size(); ++i)
+    if (inDeviceMemory(ins[i])) residentAddresses.push_back(ctx.get(ins[i], "trace input").handle->data.get());
+  TraceKey key{ctx.binary.id(), ctx.programIndex, captureId, executeId, residentAddresses};
   auto hit = ctx.dev->traceCache.find(key);
   if (hit == ctx.dev->traceCache.end()) {
     // allocate the persistent slots once: the allocation program takes the device-resident inputs (their own slots)
@@ -2203,13 +2244,33 @@ void runCaptureOrExecuteTrace(const fb::Table &op, ProgramContext &ctx) {
       if (!inDeviceMemory(ins[i])) inputSlots[i].handle->version = ctx.get(ins[i], "trace input").handle->version;
     it->second.inputSlots = std::move(inputSlots);
     it->second.outputSlots = std::move(outputSlots);
+    it->second.lastUse = ++ctx.dev->traceClock;
     ctx.dev->traceCache[key] = traceId;
     publishTraceOutputs(op, ctx, it->second.outputSlots);  // the capture program replayed the trace once
     debug::Stats::get().incrementStat("TraceCacheMiss");
     debug::Stats::get().incrementStat("CapturedTrace");
+    // traces of this op recorded on other resident tensors: the caller may come back to them (weight sets that alternate),
+    // but each keeps its slots and intermediates alive, so only the most recently used ones stay
+    for (;;) {
+      std::uint32_t oldest = 0, count = 0;
+      std::uint64_t oldestUse = ~std::uint64_t(0);
+      for (const auto &kv : ctx.dev->traceCache) {
+        const TraceKey &k = kv.first;
+        if (std::get<0>(k) != std::get<0>(key) || std::get<1>(k) != std::get<1>(key) || std::get<2>(k) != std::get<2>(key) ||
+            std::get<3>(k) != std::get<3>(key))
+          continue;
+        ++count;
+        const std::uint64_t use = ctx.dev->traces.at(kv.second).lastUse;
+        if (use < oldestUse) { oldestUse = use; oldest = kv.second; }
+      }
+      if (count <= kMaxTracesPerOp) break;
+      releaseTrace(ctx.dev, oldest);
+      debug::Stats::get().incrementStat("ReleasedTrace");
+    }
     return;
   }
   TraceData &td = ctx.dev->traces.at(hit->second);
+  td.lastUse = ++ctx.dev->traceClock;
   updateTraceInputSlots(op, ctx, td.inputSlots, /*deviceResidentOnly=*/false);
   std::vector<Tensor> idArg{makeTraceIdTensor(td.traceId)};
   executeProgram(ctx.dev, ctx.binary, executeId, idArg);

@@ -266,17 +266,61 @@ static std::vector<std::uint32_t> matmulShape(const std::vector<std::uint32_t> &
   return out;
 }
 
+void ProgramBuilder::setMatmulProgramConfig(int kind, int fusedActivation) {
+  if (kind < 0 || kind > static_cast<int>(MatmulProgramConfig::MatmulMultiCoreReuseMultiCastDRAMShardedProgramConfig))
+    fatal("ProgramBuilder: unknown matmul program config kind " + std::to_string(kind));
+  pendingMatmulConfig_ = kind;
+  pendingFusedActivation_ = fusedActivation;
+}
+
+// the program config table of the next matmul / linear (include/ttmlir/Target/TTNN/operations/matmul.fbs:5-62); only the
+// fields the runtime reads are written: the fused activation
+Off ProgramBuilder::takeMatmulProgramConfig(std::uint8_t *kindOut) {
+  const auto kind = static_cast<MatmulProgramConfig>(pendingMatmulConfig_);
+  *kindOut = static_cast<std::uint8_t>(pendingMatmulConfig_);
+  const int fused = pendingFusedActivation_;
+  pendingMatmulConfig_ = 0;
+  pendingFusedActivation_ = -1;
+  if (kind == MatmulProgramConfig::NONE) return 0;
+  int numFields = MatmulMultiCoreReuseProgramConfig::kNumFields, fusedSlot = -1;
+  switch (kind) {
+  case MatmulProgramConfig::MatmulMultiCoreReuseMultiCastProgramConfig:
+    numFields = MatmulMultiCoreReuseMultiCastProgramConfig::kNumFields;
+    fusedSlot = MatmulMultiCoreReuseMultiCastProgramConfig::f_fused_activation; break;
+  case MatmulProgramConfig::MatmulMultiCoreReuseMultiCast1DProgramConfig:
+    numFields = MatmulMultiCoreReuseMultiCast1DProgramConfig::kNumFields;
+    fusedSlot = MatmulMultiCoreReuseMultiCast1DProgramConfig::f_fused_activation; break;
+  case MatmulProgramConfig::MatmulMultiCoreReuseMultiCastDRAMShardedProgramConfig:
+    numFields = MatmulMultiCoreReuseMultiCastDRAMShardedProgramConfig::kNumFields;
+    fusedSlot = MatmulMultiCoreReuseMultiCastDRAMShardedProgramConfig::f_fused_activation; break;
+  default: break;
+  }
+  Off unary = 0;
+  if (fused >= 0 && fusedSlot >= 0) {
+    b_.startTable(UnaryWithParam::kNumFields);
+    b_.addScalar<std::uint32_t>(UnaryWithParam::f_op_type, static_cast<std::uint32_t>(fused));
+    unary = b_.endTable();
+  }
+  b_.startTable(numFields);
+  if (unary) b_.addOffset(fusedSlot, unary);
+  return b_.endTable();
+}
+
 ProgramBuilder::Id ProgramBuilder::matmul(Id a, Id b, bool ta, bool tb, const std::string &activation, DataType outDtype) {
   Desc d{matmulShape(desc(a).shape, desc(b).shape, ta, tb), outDtype, TensorLayout::Tile, StorageType::Device};
   Id out = newTensor(d);
   Off ar = tensorRef(a), br = tensorRef(b), orf = tensorRef(out);
   Off act = activation.empty() ? 0 : b_.createString(activation);
+  std::uint8_t configKind = 0;
+  Off config = takeMatmulProgramConfig(&configKind);
   b_.startTable(MatmulOp::kNumFields);
   b_.addOffset(MatmulOp::f_a, ar);
   b_.addOffset(MatmulOp::f_b, br);
   b_.addOffset(MatmulOp::f_out, orf);
   b_.addScalarDefault<std::uint8_t>(MatmulOp::f_transpose_a, ta, 0);
   b_.addScalarDefault<std::uint8_t>(MatmulOp::f_transpose_b, tb, 0);
+  b_.addScalarDefault<std::uint8_t>(MatmulOp::f_matmul_program_config_type, configKind, 0);
+  b_.addOffset(MatmulOp::f_matmul_program_config, config);
   b_.addOffset(MatmulOp::f_activation, act);
   addOp(OpType::MatmulOp, b_.endTable(), "ttnn.matmul " + shapeStr(desc(a).shape) + " x " + shapeStr(desc(b).shape));
   return out;
@@ -290,6 +334,8 @@ ProgramBuilder::Id ProgramBuilder::linear(Id a, Id b, Id bias, bool ta, bool tb,
   b_.addScalar<std::uint8_t>(DeviceComputeKernelConfig::f_math_fidelity, static_cast<std::uint8_t>(MathFidelity::HiFi4));
   b_.addScalar<std::uint8_t>(DeviceComputeKernelConfig::f_fp32_dest_acc_en, 1);
   Off cc = b_.endTable();
+  std::uint8_t configKind = 0;
+  Off config = takeMatmulProgramConfig(&configKind);
   b_.startTable(LinearOp::kNumFields);
   b_.addOffset(LinearOp::f_a, ar);
   b_.addOffset(LinearOp::f_b, br);
@@ -297,6 +343,8 @@ ProgramBuilder::Id ProgramBuilder::linear(Id a, Id b, Id bias, bool ta, bool tb,
   b_.addOffset(LinearOp::f_out, orf);
   b_.addScalarDefault<std::uint8_t>(LinearOp::f_transpose_a, ta, 0);
   b_.addScalarDefault<std::uint8_t>(LinearOp::f_transpose_b, tb, 0);
+  b_.addScalarDefault<std::uint8_t>(LinearOp::f_matmul_program_config_type, configKind, 0);
+  b_.addOffset(LinearOp::f_matmul_program_config, config);
   b_.addOffset(LinearOp::f_activation, act);
   b_.addOffset(LinearOp::f_compute_config, cc);
   addOp(OpType::LinearOp, b_.endTable(), "ttnn.linear " + shapeStr(desc(a).shape) + " x " + shapeStr(desc(b).shape) + (activation.empty() ? "" : " + " + activation));

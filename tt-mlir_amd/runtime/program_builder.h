@@ -35,6 +35,9 @@ public:
   Id typecast(Id in, DataType dtype);
   Id toDevice(Id in);
   Id fromDevice(Id in);
+  // The next matmul / linear carries a matmul_program_config of this kind (the MatmulProgramConfig union's value; 0 = none)
+  // whose fused_activation is the given UnaryOpType, or none when negative.
+  void setMatmulProgramConfig(int kind, int fusedActivation);
   Id matmul(Id a, Id b, bool transposeA, bool transposeB, const std::string &activation, DataType outDtype);
   Id linear(Id a, Id b, Id bias /* 0 = none */, bool transposeA, bool transposeB, const std::string &activation, DataType outDtype);
   Id unary(std::uint32_t type, Id in, bool hasParam, float param);
@@ -121,6 +124,8 @@ private:
   };
   Id newTensor(const Desc &d);
   std::optional<std::vector<std::uint32_t>> declaredShape_;   // see declareNextShape
+  int pendingMatmulConfig_ = 0, pendingFusedActivation_ = -1;  // see setMatmulProgramConfig
+  fb::Builder::Off takeMatmulProgramConfig(std::uint8_t *kindOut);
   fb::Builder::Off tensorRef(Id t);
   fb::Builder::Off memoryConfig(StorageType storage);
   void addOp(::ttmlir_amd::schema::OpType type, fb::Builder::Off table, const std::string &debug);

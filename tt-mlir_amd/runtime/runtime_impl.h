@@ -30,10 +30,16 @@ struct TraceData {
   size_t numNodes = 0;
   std::vector<Tensor> inputSlots, outputSlots;
   std::vector<std::pair<void *, size_t>> blocks;
+  std::uint64_t lastUse = 0;   // DeviceState::traceClock at the last capture or replay
 };
 
-// (binary id, main program, capture program, execute program): MainProgramKey + CaptureExecuteProgramKey of the reference
-using TraceKey = std::tuple<std::uint64_t, std::uint32_t, std::uint32_t, std::uint32_t>;
+// (binary id, main program, capture program, execute program): MainProgramKey + CaptureExecuteProgramKey of the reference,
+// then the device addresses of the device-resident inputs.  A recorded graph names those addresses (resident inputs are
+// their own slots), so a call with other resident tensors is another trace: nothing is ever copied into, or re-versioned
+// in, a tensor the trace does not own (a caller's parameter, a const-eval result that the const-eval cache still serves).
+using TraceKey = std::tuple<std::uint64_t, std::uint32_t, std::uint32_t, std::uint32_t, std::vector<const void *>>;
+// traces kept per capture_or_execute_trace op; the least recently used one is released beyond that
+constexpr size_t kMaxTracesPerOp = 4;
 
 // Results of a const-eval program (runtime/lib/ttnn/operations/cache/load_cached.cpp:20-90): valid while the versions of
 // the tensors it was run on are those of the current inputs.
@@ -57,7 +63,8 @@ struct DeviceState {
   std::uint32_t capturingTraceId = 0;
   std::uint32_t nextTraceId = 1;
   std::map<std::uint32_t, TraceData> traces;      // by trace id: graphs recorded on this device
-  std::map<TraceKey, std::uint32_t> traceCache;   // capture_or_execute_trace -> trace id
+  std::map<TraceKey, std::uint32_t> traceCache;   // capture_or_execute_trace on these resident tensors -> trace id
+  std::uint64_t traceClock = 0;
   // const-eval results by (binary id, program index, input versions), one entry per combination as in the reference's
   // GlobalTensorCache (device id, function hash, input versions; runtime/lib/ttnn/operations/cache/load_cached.cpp:24-38).
   // They are device memory of this device, so they live and die with it: dropped at closeMeshDevice, per binary when the
