@@ -1,20 +1,29 @@
-// A device that computes nothing and checks everything: a stand-in for libttmlir_amd_hip.so on a machine without a GPU,
-// built by the tests (g++ -shared) and put in front of the real library with LD_LIBRARY_PATH.  "Device memory" is zeroed
-// host memory with a registry of the live allocations; copies are memcpy; streams and graphs are dummies.  A kernel entry
-// point leaves its outputs as they are, but first holds every pointer argument against the registry: the pointer must lie
-// in a live allocation and have behind it the bytes the real kernels touch (include/ttmlir_amd_hip.h: a tile tensor is
+// A device in host memory that checks everything and computes the common ops: a stand-in for libttmlir_amd_hip.so on a
+// machine without a GPU, built by the tests (g++ -shared, linked against the CPU oracle) and put in front of the real library
+// with LD_LIBRARY_PATH.  "Device memory" is zeroed host memory with a registry of the live allocations; copies are memcpy;
+// streams are dummies.  Every kernel entry point first holds each pointer argument against the registry: the pointer must
+// lie in a live allocation and have behind it the bytes the real kernels touch (include/ttmlir_amd_hip.h: a tile tensor is
 // backed by its whole padded extent).  A violation is an error return with a message, which the runtime turns into an
-// exception - on the GPU the same call would be a memory fault.  With this the host runtime (executor, tensor pool, fused
-// launches, traces) runs whole programs on the CPU: results are meaningless, the extents of every launch are checked.
+// exception - on the GPU the same call would be a memory fault.
+// Layout conversion, block-float packing, typecasts, copies and views, matmul / linear in all their forms, element-wise ops,
+// RMSNorm, softmax, reductions, embedding, argmax, arange and prefill attention then compute their result on the host with
+// the oracle's arithmetic (f32, one rounding to the output type), so programs made of them give the values the oracle gives;
+// the decode-path kernels leave their outputs as they are.  A "launch" is a closure: between ttm_graph_begin_capture and
+// ttm_graph_end_capture closures are recorded instead of run, as a capturing HIP stream records kernels, and
+// ttm_graph_launch runs the recorded closures against whatever the recorded addresses hold by then.  With this the host
+// runtime (executor, tensor pool, caches, fused launches, traces) runs whole programs on the CPU with checkable values.
 #include <atomic>
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <cstring>
+#include <functional>
 #include <map>
 #include <mutex>
 #include <string>
+#include <vector>
 
 #include "ttmlir_amd_hip.h"
 
@@ -79,7 +88,17 @@ int span(const char *fn, const char *what, const void *p, int64_t bytes, bool op
 }
 #define SPAN(what, p, bytes) do { if (int rc_ = span(__func__, what, p, bytes)) return rc_; } while (0)
 #define SPAN_OPT(what, p, bytes) do { if (int rc_ = span(__func__, what, p, bytes, true)) return rc_; } while (0)
-int kernel() { ++g_kernel_calls; return TTM_OK; }
+
+// a launch: run now, or recorded while a capture is in progress (the runtime serialises the work of a device)
+using Launch = std::function<void()>;
+struct Graph { std::vector<Launch> nodes; };
+std::vector<Launch> *g_recording = nullptr;
+int launch(Launch f) {
+  ++g_kernel_calls;
+  if (g_recording) g_recording->push_back(std::move(f)); else f();
+  return TTM_OK;
+}
+int kernel() { return launch([] {}); }   // an entry point that computes nothing
 
 // a [.., rows, cols] shape of `rank` entries as (batch, rows, cols); rank 1 is one row
 void split3(const int64_t *shape, int rank, int64_t &b, int64_t &r, int64_t &c) {
@@ -103,6 +122,138 @@ int view_span(const char *fn, const char *what, const void *p, int64_t rows, int
   const int64_t per = rows * cols, mats = per > 0 ? hi / per + 1 : 0;
   const int64_t bytes = layout == TTM_TILE ? mats * pad32(rows) * pad32(cols) * elem : (hi + 1) * elem;
   return span(fn, what, p, bytes);
+}
+// ---- host arithmetic.  The oracle (oracle/ttm_oracle.c) supplies the formulas; tensors pass through dense row-major f32.
+extern "C" {
+void orc_tilize(const void *in, void *out, int64_t batch, int64_t rows, int64_t cols, int elem);
+void orc_untilize(const void *in, void *out, int64_t batch, int64_t rows, int64_t cols, int elem);
+void orc_bfp_pack_rm(const float *rm, uint8_t *out, int64_t batch, int64_t rows, int64_t cols, int fmt);
+void orc_bfp_unpack_rm(const uint8_t *in, float *rm, int64_t batch, int64_t rows, int64_t cols, int fmt);
+void orc_f32_to_bf16(const float *in, uint16_t *out, int64_t n);
+void orc_f16_to_bf16(const uint16_t *in, uint16_t *out, int64_t n);
+void orc_bf16_to_f16(const uint16_t *in, uint16_t *out, int64_t n);
+void orc_unary_f32(int op, const float *in, float *out, int64_t n, float param);
+void orc_binary_f32(int op, const float *a, const int64_t *ashape, const float *b, const int64_t *bshape, float *out,
+                    const int64_t *oshape, int rank);
+void orc_linear_f32(const float *A, const float *B, const float *bias, float *C, int64_t M, int64_t N, int64_t K, int transA,
+                    int transB, int act);
+void orc_rmsnorm_f32(const float *x, const float *w, const float *b, float *out, int64_t rows, int64_t cols, float eps);
+void orc_softmax_f32(const float *x, float *out, int64_t outer, int64_t dim, int64_t inner);
+void orc_reduce_f32(int op, const float *x, float *out, int64_t outer, int64_t dim, int64_t inner);
+void orc_sdpa_f32(const float *q, const float *k, const float *v, const float *mask, int mask_heads, float *out, int64_t B,
+                  int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int64_t window,
+                  const float *sink);
+}
+
+using Dense = std::vector<float>;
+int64_t tiled_off(int64_t r, int64_t c, int64_t ct) {
+  return ((r >> 5) * ct + (c >> 5)) * 1024 + (((r >> 4) & 1) * 2 + ((c >> 4) & 1)) * 256 + (r & 15) * 16 + (c & 15);
+}
+// physical element offset of logical (b, r, c) in a [batch, rows, cols] tensor
+int64_t elem_off(int layout, int64_t rows, int64_t cols, int64_t b, int64_t r, int64_t c) {
+  if (layout != TTM_TILE) return (b * rows + r) * cols + c;
+  return b * pad32(rows) * pad32(cols) + tiled_off(r, c, pad32(cols) / 32);
+}
+float bf16_f32(uint16_t h) { uint32_t u = (uint32_t)h << 16; float f; memcpy(&f, &u, 4); return f; }
+uint16_t f32_bf16(float f) { uint16_t h; orc_f32_to_bf16(&f, &h, 1); return h; }
+float round_bf16(float f) { return bf16_f32(f32_bf16(f)); }
+double load_scalar(const void *p, int dtype, int64_t i) {
+  switch (dtype) {
+  case TTM_F32: return ((const float *)p)[i];
+  case TTM_BF16: return bf16_f32(((const uint16_t *)p)[i]);
+  case TTM_F16: { uint16_t b; orc_f16_to_bf16((const uint16_t *)p + i, &b, 1); return bf16_f32(b); }   // callers that need f16 exactly do not exist
+  case TTM_U32: return ((const uint32_t *)p)[i];
+  case TTM_I32: return ((const int32_t *)p)[i];
+  case TTM_U16: return ((const uint16_t *)p)[i];
+  case TTM_U8: return ((const uint8_t *)p)[i];
+  default: return 0.0;
+  }
+}
+template <typename T> T saturate(double v, double lo, double hi) { return v != v ? (T)0 : (T)(v < lo ? lo : (v > hi ? hi : std::trunc(v))); }
+void store_scalar(void *p, int dtype, int64_t i, double v) {
+  switch (dtype) {
+  case TTM_F32: ((float *)p)[i] = (float)v; break;
+  case TTM_BF16: ((uint16_t *)p)[i] = f32_bf16((float)v); break;
+  case TTM_F16: { uint16_t b = f32_bf16((float)v); orc_bf16_to_f16(&b, (uint16_t *)p + i, 1); break; }
+  case TTM_U32: ((uint32_t *)p)[i] = saturate<uint32_t>(v, 0, 4294967295.0); break;
+  case TTM_I32: ((int32_t *)p)[i] = saturate<int32_t>(v, -2147483648.0, 2147483647.0); break;
+  case TTM_U16: ((uint16_t *)p)[i] = saturate<uint16_t>(v, 0, 65535.0); break;
+  case TTM_U8: ((uint8_t *)p)[i] = saturate<uint8_t>(v, 0, 255.0); break;
+  default: break;
+  }
+}
+bool block_float(int dt) { return dt == TTM_BFP8B || dt == TTM_BFP4B; }
+Dense load_dense(const void *p, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols) {
+  Dense d((size_t)(batch * rows * cols));
+  if (block_float(dtype)) {
+    orc_bfp_unpack_rm((const uint8_t *)p, d.data(), batch, rows, cols, dtype == TTM_BFP8B ? 8 : 4);
+    return d;
+  }
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t r = 0; r < rows; ++r)
+      for (int64_t c = 0; c < cols; ++c) d[(size_t)((b * rows + r) * cols + c)] = (float)load_scalar(p, dtype, elem_off(layout, rows, cols, b, r, c));
+  return d;
+}
+// writes the tensor and, in TILE layout, zeros in its padding
+void store_dense(const Dense &d, void *p, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols) {
+  if (block_float(dtype)) {
+    orc_bfp_pack_rm(d.data(), (uint8_t *)p, batch, rows, cols, dtype == TTM_BFP8B ? 8 : 4);
+    return;
+  }
+  if (layout == TTM_TILE) memset(p, 0, (size_t)tile_bytes(dtype, batch, rows, cols));
+  for (int64_t b = 0; b < batch; ++b)
+    for (int64_t r = 0; r < rows; ++r)
+      for (int64_t c = 0; c < cols; ++c) store_scalar(p, dtype, elem_off(layout, rows, cols, b, r, c), d[(size_t)((b * rows + r) * cols + c)]);
+}
+Dense load_vec(const void *p, int dtype, int layout, int64_t cols) { return load_dense(p, dtype, layout, 1, 1, cols); }
+void round_all_bf16(Dense &d) { for (float &f : d) f = round_bf16(f); }
+
+// act(a w + bias) rounded to bf16, then the optional tail op with its own rounding: dense [batch, M, N]
+Dense linear_host(const void *a, const void *w, int w_dtype, int transpose_w, const void *bias, int bias_dtype, int bias_layout, int64_t batch,
+                  int64_t w_batch, int64_t M, int64_t N, int64_t K, int act, int tail_op, const void *tail) {
+  Dense A = load_dense(a, TTM_BF16, TTM_TILE, batch, M, K);
+  Dense W = transpose_w ? load_dense(w, w_dtype, TTM_TILE, w_batch, N, K) : load_dense(w, w_dtype, TTM_TILE, w_batch, K, N);
+  Dense B;
+  if (bias) B = load_vec(bias, bias_dtype, bias_layout, N);
+  Dense C((size_t)(batch * M * N));
+  for (int64_t b = 0; b < batch; ++b)
+    orc_linear_f32(A.data() + b * M * K, W.data() + (w_batch == 1 ? 0 : b) * K * N, bias ? B.data() : nullptr, C.data() + b * M * N, M, N, K, 0,
+                   transpose_w ? 1 : 0, act);
+  round_all_bf16(C);
+  if (tail_op != TTM_TAIL_NONE) {
+    Dense T = load_dense(tail, TTM_BF16, TTM_TILE, batch, M, N);
+    for (size_t i = 0; i < C.size(); ++i) C[i] = round_bf16(tail_op == TTM_TAIL_ADD ? C[i] + T[i] : C[i] * T[i]);
+  }
+  return C;
+}
+Dense rms_norm_host(const Dense &x, const void *weight, int weight_layout, const void *bias, int bias_layout, int dtype, int64_t rows, int64_t cols,
+                    float eps) {
+  Dense w, b, out(x.size());
+  if (weight) w = load_vec(weight, dtype, weight_layout, cols);
+  if (bias) b = load_vec(bias, dtype, bias_layout, cols);
+  orc_rmsnorm_f32(x.data(), weight ? w.data() : nullptr, bias ? b.data() : nullptr, out.data(), rows, cols, eps);
+  return out;
+}
+std::vector<int64_t> vec64(const int64_t *p, int n) { return p ? std::vector<int64_t>(p, p + n) : std::vector<int64_t>(); }
+// a strided view copy on logical indices (include/ttmlir_amd_hip.h, ttm_copy_view)
+void copy_view_host(const void *src, int64_t src_rows, int64_t src_cols, int src_layout, void *dst, int64_t dst_rows, int64_t dst_cols, int dst_layout,
+                    int elem, const std::vector<int64_t> &extent, const std::vector<int64_t> &sstride, int64_t sbase,
+                    const std::vector<int64_t> &dstride, int64_t dbase) {
+  const int rank = (int)extent.size();
+  int64_t n = 1;
+  for (int64_t e : extent) n *= e;
+  auto phys = [](int64_t idx, int64_t rows, int64_t cols, int layout) {
+    const int64_t per = rows * cols;
+    return elem_off(layout, rows, cols, idx / per, (idx % per) / cols, idx % cols);
+  };
+  for (int64_t i = 0; i < n; ++i) {
+    int64_t rem = i, si = sbase, di = dbase;
+    for (int d = rank - 1; d >= 0; --d) {
+      const int64_t c = rem % extent[d]; rem /= extent[d];
+      si += c * sstride[d]; di += c * dstride[d];
+    }
+    memcpy((uint8_t *)dst + phys(di, dst_rows, dst_cols, dst_layout) * elem, (const uint8_t *)src + phys(si, src_rows, src_cols, src_layout) * elem, elem);
+  }
 }
 }  // namespace
 
@@ -159,14 +310,12 @@ EXPORT int ttm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *) {
   if (!bytes) return TTM_OK;
   SPAN("destination", dst, (int64_t)bytes);
   SPAN("source", src, (int64_t)bytes);
-  memmove(dst, src, bytes);
-  return TTM_OK;
+  return launch([=] { memmove(dst, src, bytes); });
 }
 EXPORT int ttm_fill_u32(void *dst, uint32_t value, size_t count, void *) {
   if (!count) return TTM_OK;
   SPAN("destination", dst, (int64_t)count * 4);
-  for (size_t i = 0; i < count; ++i) ((uint32_t *)dst)[i] = value;
-  return kernel();
+  return launch([=] { for (size_t i = 0; i < count; ++i) ((uint32_t *)dst)[i] = value; });
 }
 EXPORT int ttm_stream_create(void **stream) { if (!stream) return fail("null"); *stream = malloc(8); return TTM_OK; }
 EXPORT int ttm_stream_destroy(void *stream) { free(stream); return TTM_OK; }
@@ -178,21 +327,31 @@ EXPORT int ttm_event_record(void *, void *) { return TTM_OK; }
 EXPORT int ttm_event_sync(void *) { return TTM_OK; }
 EXPORT int ttm_event_elapsed_ms(float *ms, void *, void *) { if (ms) *ms = 0.0f; return TTM_OK; }
 
-// ---- graphs: the launches between begin and end are counted, a replay does nothing
+// ---- graphs: the launches between begin and end are recorded, not run; a replay runs them in order
 EXPORT int ttm_graph_begin_capture(void *) {
   if (g_capture_mark >= 0) return fail("ttm_graph_begin_capture: a capture is already in progress");
   g_capture_mark = g_kernel_calls.load();
+  g_recording = new std::vector<Launch>;
   return TTM_OK;
 }
 EXPORT int ttm_graph_end_capture(void *, void **graph_exec, size_t *num_nodes) {
   if (g_capture_mark < 0) return fail("ttm_graph_end_capture: no capture in progress");
   if (num_nodes) *num_nodes = (size_t)(g_kernel_calls.load() - g_capture_mark.load());
   g_capture_mark = -1;
-  if (graph_exec) *graph_exec = malloc(8);
+  Graph *g = new Graph;
+  g->nodes.swap(*g_recording);
+  delete g_recording;
+  g_recording = nullptr;
+  if (graph_exec) *graph_exec = g; else delete g;
   return TTM_OK;
 }
-EXPORT int ttm_graph_launch(void *graph_exec, void *) { return graph_exec ? TTM_OK : fail("ttm_graph_launch: null graph"); }
-EXPORT int ttm_graph_destroy(void *graph_exec) { free(graph_exec); return TTM_OK; }
+EXPORT int ttm_graph_launch(void *graph_exec, void *) {
+  if (!graph_exec) return fail("ttm_graph_launch: null graph");
+  if (g_recording) return fail("ttm_graph_launch: a capture is in progress");
+  for (const Launch &f : ((Graph *)graph_exec)->nodes) f();
+  return TTM_OK;
+}
+EXPORT int ttm_graph_destroy(void *graph_exec) { delete (Graph *)graph_exec; return TTM_OK; }
 EXPORT int ttm_stream_is_capturing(void *, int *capturing) { if (capturing) *capturing = g_capture_mark >= 0; return TTM_OK; }
 
 EXPORT int ttm_set_option(const char *name, int value) { if (!name) return fail("null"); g_options[name] = value; return TTM_OK; }
@@ -201,42 +360,43 @@ EXPORT int ttm_get_option(const char *name, int *value) { if (!name || !value) r
 // ---- layout, block float, typecast
 EXPORT int ttm_copy_kernel(const void *src, void *dst, size_t bytes, void *) {
   SPAN("source", src, (int64_t)bytes); SPAN("destination", dst, (int64_t)bytes);
-  return kernel();
+  return launch([=] { memmove(dst, src, bytes); });
 }
 EXPORT int ttm_tilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int elem, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("row-major input", src, batch * rows * cols * elem);
   SPAN("tile output", dst, batch * pad32(rows) * pad32(cols) * elem);
-  return kernel();
+  return launch([=] { orc_tilize(src, dst, batch, rows, cols, elem); });
 }
 EXPORT int ttm_untilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int elem, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("tile input", src, batch * pad32(rows) * pad32(cols) * elem);
   SPAN("row-major output", dst, batch * rows * cols * elem);
-  return kernel();
+  return launch([=] { orc_untilize(src, dst, batch, rows, cols, elem); });
 }
 EXPORT int64_t ttm_bfp_tile_bytes(int fmt) { return fmt == TTM_BFP8B ? 1088 : (fmt == TTM_BFP4B ? 576 : -1); }
 EXPORT int ttm_bfp_pack(const void *src, int src_dtype, int src_layout, void *dst, int fmt, int64_t batch, int64_t rows, int64_t cols, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("input", src, tensor_bytes(src_dtype, src_layout, batch, rows, cols));
   SPAN("block-float output", dst, tile_bytes(fmt, batch, rows, cols));
-  return kernel();
+  return launch([=] { store_dense(load_dense(src, src_dtype, src_layout, batch, rows, cols), dst, fmt, TTM_TILE, batch, rows, cols); });
 }
 EXPORT int ttm_bfp_unpack(const void *src, int fmt, void *dst, int dst_dtype, int dst_layout, int64_t batch, int64_t rows, int64_t cols, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("block-float input", src, tile_bytes(fmt, batch, rows, cols));
   SPAN("output", dst, tensor_bytes(dst_dtype, dst_layout, batch, rows, cols));
-  return kernel();
+  return launch([=] { store_dense(load_dense(src, fmt, TTM_TILE, batch, rows, cols), dst, dst_dtype, dst_layout, batch, rows, cols); });
 }
 EXPORT int ttm_typecast(const void *in, int src_dtype, void *out, int dst_dtype, int64_t n, void *) {
   if (n == 0) return TTM_OK;
   SPAN("input", in, n * elem_bytes(src_dtype)); SPAN("output", out, n * elem_bytes(dst_dtype));
-  return kernel();
+  return launch([=] { for (int64_t i = 0; i < n; ++i) store_scalar(out, dst_dtype, i, load_scalar(in, src_dtype, i)); });
 }
 
 // ---- matmul / linear
-static int linear_check(const char *fn, const void *a, int a_dtype, const void *w, int w_dtype, const void *bias, int bias_dtype, int bias_layout,
-                        void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int tail_op, const void *tail) {
+static int linear_check(const char *fn, const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias, int bias_dtype,
+                        int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int act, int tail_op,
+                        const void *tail) {
   if (batch * M * N == 0) return TTM_OK;
   if (int rc = span(fn, "activations [batch, M, K]", a, tile_bytes(a_dtype, batch, M, K))) return rc;
   if (int rc = span(fn, "weights [w_batch, K, N]", w, tile_bytes(w_dtype, w_batch, K, N))) return rc;
@@ -244,17 +404,24 @@ static int linear_check(const char *fn, const void *a, int a_dtype, const void *
   if (int rc = span(fn, "output [batch, M, N]", out, tile_bytes(out_dtype, batch, M, N))) return rc;
   if (tail_op != TTM_TAIL_NONE)
     if (int rc = span(fn, "tail operand [batch, M, N]", tail, tile_bytes(TTM_BF16, batch, M, N))) return rc;
-  return kernel();
+  if (a_dtype != TTM_BF16 || out_dtype != TTM_BF16) return kernel();
+  return launch([=] {
+    store_dense(linear_host(a, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, batch, w_batch, M, N, K, act, tail_op, tail), out, TTM_BF16,
+                TTM_TILE, batch, M, N);
+  });
 }
-EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int, const void *bias, int bias_dtype, int bias_layout, void *out,
-                      int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int, void *) {
-  return linear_check(__func__, a, a_dtype, w, w_dtype, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, TTM_TAIL_NONE, nullptr);
+EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias, int bias_dtype, int bias_layout,
+                      void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int act, void *) {
+  return linear_check(__func__, a, a_dtype, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, act,
+                      TTM_TAIL_NONE, nullptr);
 }
-EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int, const void *bias, int bias_dtype, int bias_layout, void *out,
-                           int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int, int tail_op, const void *tail, void *) {
-  return linear_check(__func__, a, a_dtype, w, w_dtype, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, tail_op, tail);
+EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias, int bias_dtype, int bias_layout,
+                           void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int act, int tail_op,
+                           const void *tail, void *) {
+  return linear_check(__func__, a, a_dtype, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, act,
+                      tail_op, tail);
 }
-EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N, const int *, int64_t M,
+EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N, const int *act, int64_t M,
                             int64_t K, void *) {
   if (n < 1 || n > 4 || !w || !out || !N) return fail("ttm_linear_group: one to four members with weights, outputs and widths");
   SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
@@ -262,21 +429,32 @@ EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dt
     SPAN("weights [K, N_i]", w[i], tile_bytes(w_dtype, 1, K, N[i]));
     SPAN("output [M, N_i]", out[i], tile_bytes(TTM_BF16, 1, M, N[i]));
   }
-  return kernel();
+  std::vector<const void *> ws(w, w + n);
+  std::vector<void *> outs(out, out + n);
+  std::vector<int64_t> ns(N, N + n);
+  std::vector<int> acts(n, TTM_ACT_NONE);
+  if (act) acts.assign(act, act + n);
+  return launch([=] {
+    for (int i = 0; i < n; ++i)
+      store_dense(linear_host(a, ws[i], w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, ns[i], K, acts[i], TTM_TAIL_NONE, nullptr), outs[i], TTM_BF16,
+                  TTM_TILE, 1, M, ns[i]);
+  });
 }
 EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M, int64_t N, int64_t K, void *) {
   SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
   SPAN("weights 0", w0, tile_bytes(w_dtype, 1, K, N)); SPAN("weights 1", w1, tile_bytes(w_dtype, 1, K, N));
   SPAN("output 0", out0, tile_bytes(TTM_BF16, 1, M, N)); SPAN("output 1", out1, tile_bytes(TTM_BF16, 1, M, N));
-  return kernel();
+  return launch([=] {
+    store_dense(linear_host(a, w0, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, N, K, TTM_ACT_NONE, TTM_TAIL_NONE, nullptr), out0, TTM_BF16, TTM_TILE, 1, M, N);
+    store_dense(linear_host(a, w1, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, N, K, TTM_ACT_NONE, TTM_TAIL_NONE, nullptr), out1, TTM_BF16, TTM_TILE, 1, M, N);
+  });
 }
-static bool block_float(int dt) { return dt == TTM_BFP8B || dt == TTM_BFP4B; }
 // the predicates of the real library at its default options
 EXPORT int ttm_linear_add_rms_norm_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
   return block_float(w_dtype) && M >= 1 && M <= 32 && K > 0 && N >= 1 && (N + 31) / 32 * 4 <= 8 * 256;
 }
 EXPORT int ttm_linear_add_rms_norm(const void *a, const void *w, int w_dtype, const void *residual, void *sum_out, const void *norm_weight,
-                                   int weight_layout, const void *norm_bias, int bias_layout, float, void *norm_out, int64_t M, int64_t N, int64_t K,
+                                   int weight_layout, const void *norm_bias, int bias_layout, float eps, void *norm_out, int64_t M, int64_t N, int64_t K,
                                    void *) {
   if (!ttm_linear_add_rms_norm_supported(w_dtype, M, N, K)) return fail("ttm_linear_add_rms_norm: unsupported shape");
   SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
@@ -287,7 +465,11 @@ EXPORT int ttm_linear_add_rms_norm(const void *a, const void *w, int w_dtype, co
   SPAN_OPT("norm weight", norm_weight, vec_bytes(TTM_BF16, weight_layout, N));
   SPAN_OPT("norm bias", norm_bias, vec_bytes(TTM_BF16, bias_layout, N));
   if (sum_out == residual || norm_out == sum_out || norm_out == residual) return fail("ttm_linear_add_rms_norm: the outputs alias");
-  return kernel();
+  return launch([=] {
+    Dense x1 = linear_host(a, w, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, N, K, TTM_ACT_NONE, TTM_TAIL_ADD, residual);
+    store_dense(x1, sum_out, TTM_BF16, TTM_TILE, 1, M, N);
+    store_dense(rms_norm_host(x1, norm_weight, weight_layout, norm_bias, bias_layout, TTM_BF16, M, N, eps), norm_out, TTM_BF16, TTM_TILE, 1, M, N);
+  });
 }
 EXPORT int ttm_linear_qkv_decode_supported(int w_dtype, int64_t users, int64_t K, int64_t heads, int64_t kv_heads, int64_t head_dim) {
   return block_float(w_dtype) && users >= 1 && users <= 32 && K > 0 && heads >= 1 && kv_heads >= 1 && head_dim >= 32 && head_dim % 32 == 0;

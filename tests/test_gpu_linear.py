@@ -275,6 +275,41 @@ def test_two_part_grid_with_ragged_remainder(hip, dev, orc, metrics, wfmt_name):
     for cols in (slice(0, 512), slice(65536 - 256, 65536 + 256), slice(N - 300, N)):
         check(orc, metrics, got[:, cols], a, w_eff[:, cols].contiguous(), b[cols], "relu", max_abs=2.0 ** -5)
 
+@pytest.mark.parametrize("wfmt_name,M,K,N,option,value", [
+    ("bfp8", 32, 1200, 200, None, 0),                   # decode kernel
+    ("bfp4", 20, 1200, 200, "linear_decode_split", 3),  # decode kernel with k-slices: activation applied by the reduction
+    ("bf16", 32, 256, 96, None, 0),                     # small-M kernel for bf16 weights
+    ("bfp8", 330, 232, 677, None, 0),                   # LDS-direct main kernel, ragged
+    ("bfp4", 330, 232, 677, "linear_split_k", 2),       # split-K main kernel
+    ("bfp8", 512, 256, 2048, "linear_two_pass", 2),     # image pass + matrix pass
+    ("bf16", 300, 256, 512, None, 0),                   # bf16 weights through the image route
+])
+def test_relu_epilogue_keeps_nan(hip, dev, orc, wfmt_name, M, K, N, option, value):
+    """linear(..., "relu") on activations that hold a NaN: the rows it reaches stay NaN after the fused relu, as with
+    arith.maximumf of the CPU lowering (lib/Conversion/TTIRToLinalg/EltwiseUnary.cpp:508-541) and the oracle; every other
+    output is what it is without the NaN, and negative sums become +0.0."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B, "bf16": hip.BF16}[wfmt_name]
+    a = datagen.randn((M, K), seed=61, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=62, std=0.1)
+    b = datagen.randn((N,), seed=63, std=0.5, dtype=torch.bfloat16)
+    a[3, 5] = float("nan")
+    a[M - 1, K - 1] = float("nan")
+    if option:
+        hip.set_option(option, value)
+    try:
+        got, w_eff = run_linear(hip, dev, a, w, b, "relu", wfmt)
+    finally:
+        if option:
+            hip.set_option(option, 0)
+    with np.errstate(invalid="ignore"):
+        want = orc.round_bf16(orc.linear(a.float().numpy(), w_eff.numpy(), b.float().numpy(), "relu"))
+    got = got.float().numpy()
+    assert np.isnan(want[3]).all() and np.isnan(want[M - 1]).all() and np.isnan(want).sum() == 2 * N
+    assert np.array_equal(np.isnan(got), np.isnan(want)), "NaN rows differ from the oracle's"
+    fin = ~np.isnan(want)
+    assert np.max(np.abs(got[fin] - want[fin])) <= 2.0 ** -5
+    assert not np.signbit(got[fin]).any()                # relu never leaves a -0.0
+
 
 @pytest.mark.parametrize("tail", ["add", "multiply"])
 @pytest.mark.parametrize("wfmt_name,M,K,N,option,value", [

@@ -217,6 +217,90 @@ def test_softmax_and_reduce_lastdim(hip, dev, orc, dtype, shape, rowwise_variant
             assert np.max(bf16_ulps(got, orc.round_bf16(w))) <= 1.0, op
         assert np.all(np.isfinite(o.float().cpu().numpy()))
 
+def _same_specials(got, want, what):
+    """NaN in the same places, the same infinities, and equal values elsewhere up to `tol` bf16 / fp32 handling by the caller."""
+    assert np.array_equal(np.isnan(got), np.isnan(want)), what + ": NaN in other places than in the oracle's result"
+    assert np.array_equal(np.isposinf(got), np.isposinf(want)) and np.array_equal(np.isneginf(got), np.isneginf(want)), what + ": infinities differ"
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f32"])
+@pytest.mark.parametrize("shape", [(64, 96), (2, 40, 70), (32, 2048), (33, 4100), (40, 8200), (3, 50000)])
+def test_rowwise_ops_on_rows_with_nan_inf_and_negative_zero(hip, dev, orc, dtype, shape, rowwise_variant):
+    """NaN, +-Inf and -0.0 through sum / mean / max / min, softmax and RMSNorm in every row-wise kernel: max and min return
+    NaN for a row that holds one (tosa.reduce_max / reduce_min propagate, lib/Conversion/TTIRToLinalg/Reduction.cpp:133-136;
+    torch.max / torch.min of the goldens, tools/golden/mapping.py:5189-5220, 2815-2856), an infinity wins over finite values,
+    a row of -0.0 keeps its sign.  Rows without special values are checked as in the ordinary tests."""
+    tdt = torch.bfloat16 if dtype == "bf16" else torch.float32
+    hdt = hip.BF16 if dtype == "bf16" else hip.F32
+    x = datagen.randn(shape, seed=88, std=2.0, dtype=tdt)
+    R, C = shape[-2], shape[-1]
+    xf = x.reshape(-1, C)
+    nan, inf = float("nan"), float("inf")
+    rows = xf.shape[0]
+    special = {0: [(0, nan)], 1: [(C - 1, nan)], 2: [(C // 2, inf)], 3: [(1, -inf)], 4: [(3, inf), (C - 2, -inf)],
+               5: [(2, nan), (5, inf)], 6: [(C // 3, -inf), (C // 3 + 1, nan)], 9: [(C - 1, inf)], 10: [(0, -inf), (C - 1, -inf)]}
+    for r, cells in special.items():
+        if r < rows:
+            for c, v in cells:
+                xf[r, c] = v
+    if rows > 7:
+        xf[7, :] = -0.0
+    if rows > 8:
+        xf[8, :] = -inf
+    if rows > 11:
+        xf[11, :] = 0.0
+        xf[11, C // 2] = -0.0
+    xt = tilize_dev(hip, x, dev)
+    batch = int(np.prod(shape[:-2], dtype=np.int64))
+    xn = x.float().numpy()
+    Rp = (R + 31) // 32 * 32
+    for op in ("sum", "mean", "max", "min"):
+        o = torch.full((batch * Rp * 32,), 7.0, dtype=tdt, device=dev)
+        hip.call("ttm_reduce_lastdim", orc.REDUCE[op], hip.ptr(xt), hip.ptr(o), hdt, batch, R, C, hip.current_stream())
+        got = untilize_dev(hip, o, tuple(shape[:-1]) + (1,), dev).float().cpu().numpy()
+        with np.errstate(invalid="ignore", over="ignore"):
+            want = orc.reduce(op, xn, -1, keepdim=True)
+        want = orc.round_bf16(want) if dtype == "bf16" else want
+        _same_specials(got, want, op)
+        fin = np.isfinite(want)
+        if op in ("max", "min"):
+            assert np.array_equal(got[fin], want[fin]), op            # exact, zeros of either sign equal
+            if rows > 7:
+                assert np.signbit(got.reshape(-1)[7]), op + " of a row of -0.0"
+        elif dtype == "f32":
+            mag = np.abs(np.where(np.isfinite(xn), xn, 0)).sum(-1, keepdims=True) / (C if op == "mean" else 1)
+            assert np.all(np.abs(got[fin] - want[fin]) <= 1e-6 * np.abs(want[fin]) + 2.0 ** -22 * mag[fin]), op
+        else:
+            assert not fin.any() or np.max(bf16_ulps(got[fin], want[fin])) <= 1.0, op
+    out = torch.full_like(xt, 7.0)
+    hip.call("ttm_softmax_lastdim", hip.ptr(xt), hip.ptr(out), hdt, batch, R, C, hip.current_stream())
+    res = untilize_dev(hip, out, shape, dev).float().cpu().numpy()
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = orc.softmax(xn, -1)
+    want = orc.round_bf16(want) if dtype == "bf16" else want
+    _same_specials(res, want, "softmax")
+    fin = np.isfinite(want)
+    if dtype == "f32":
+        assert np.allclose(res[fin], want[fin], rtol=max(2e-5, 1.2e-7 * C), atol=1e-7)
+    else:
+        assert not fin.any() or np.max(bf16_ulps(res[fin], want[fin])) <= 1.0
+    w = (1.0 + 0.02 * datagen.randn((C,), seed=6)).to(tdt)
+    wd = w.to(dev)
+    out = torch.full_like(xt, 7.0)
+    hip.call("ttm_rms_norm", hip.ptr(xt), hip.ptr(wd), hip.ROW_MAJOR, None, hip.ROW_MAJOR, hip.ptr(out), hdt, batch, R, C, 1e-5,
+             hip.current_stream())
+    res = untilize_dev(hip, out, shape, dev).float().cpu().numpy()
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = orc.rms_norm(xn, w.float().numpy(), None, 1e-5)
+    want = orc.round_bf16(want) if dtype == "bf16" else want
+    _same_specials(res, want, "rms_norm")
+    fin = np.isfinite(want)
+    if dtype == "f32":
+        assert np.allclose(res[fin], want[fin], rtol=2e-5, atol=1e-6)
+    else:
+        assert not fin.any() or np.max(bf16_ulps(res[fin], want[fin])) <= 1.0
+    torch.cuda.synchronize()
+
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("shape", [(64, 96), (3, 128, 32), (2, 2, 32, 160), (1024, 2048)])

@@ -662,6 +662,24 @@ def test_ttrt_run_checks_embedded_goldens_and_saves_artifacts(orc, tmp_path):
     ya, yb = (torch.load(tmp_path / n / "bad" / "run" / "program_1" / "device_output_0.pt", weights_only=True) for n in ("a", "b"))
     assert torch.equal(ya, yb) and bool(ya.float().abs().sum() > 0)
 
+def test_fused_activation_of_the_matmul_program_config(device):
+    """runtime/lib/ttnn/operations/matmul/matmul.cpp:17-44, 64-66: a multicast program config that carries a
+    fused_activation decides the activation, the op's own string counts only without one."""
+    M, K, N = 64, 96, 160
+    a, w, bias = datagen.c3_linear(M, K, N, seed=12)
+    tins = [a, bf(w), bias]
+    GELU, SILU = 2, 51                                          # UnaryOpType (eltwise.fbs)
+    run = lambda **kw: harness.execute(rt.Binary.load_from_memory(programs.c3_linear(M, K, N, **kw)), 1, tins, device)[0]
+    plain, gelu, silu = run(activation=""), run(activation="gelu"), run(activation="silu")
+    assert not torch.equal(plain, gelu) and not torch.equal(gelu, silu)
+    for kind in (2, 3, 4):                                      # the three configs with a fused_activation field
+        assert torch.equal(run(activation="", program_config=(kind, GELU)), gelu), kind
+        assert torch.equal(run(activation="relu", program_config=(kind, SILU)), silu), kind
+        assert torch.equal(run(activation="gelu", program_config=(kind, -1)), gelu), kind
+    assert torch.equal(run(activation="gelu", program_config=(1, SILU)), gelu)    # MatmulMultiCoreReuseProgramConfig has none
+    with pytest.raises(RuntimeError, match="unsupported fused activation in the matmul program config"):
+        run(activation="", program_config=(3, 0))               # Exp
+
 
 def _run_traced(binary, device, x, resident):
     ins = [rt.from_torch(x)] + resident

@@ -661,7 +661,7 @@ __global__ __launch_bounds__(256) void ttm_rowwise_wide_stats_k(RowArgs p, float
       float cm = -INFINITY;
 #pragma unroll
       for (int i = 0; i < EPC; ++i) cm = c0 + i < cols ? ttm_max(cm, f[i]) : cm;
-      if (cm > a) { l *= expf(a - cm); a = cm; }   // a = -inf at first: l is 0 and stays 0
+      if (cm > a || cm != cm) { l *= expf(a - cm); a = cm; }   // a = -inf at first: l is 0 and stays 0; a NaN maximum stays and makes l NaN
       if (a != -INFINITY) {
 #pragma unroll
         for (int i = 0; i < EPC; ++i) l += c0 + i < cols ? expf(f[i] - a) : 0.0f;

@@ -50,8 +50,9 @@ def c1_matmul():
     return pb.finish()
 
 
-def c3_linear(M, K=4096, N=14336, weight_dtype=DT.BFP_BFloat8, activation="gelu"):
-    """Config 3: linear with block-float weights (packed once by a const-eval program), bias + GELU."""
+def c3_linear(M, K=4096, N=14336, weight_dtype=DT.BFP_BFloat8, activation="gelu", program_config=None):
+    """Config 3: linear with block-float weights (packed once by a const-eval program), bias + GELU.
+    program_config: optional (kind, fused UnaryOpType or -1) written as the op's matmul_program_config."""
     pb = rt.ProgramBuilder()
     ce, ce_outs = _consteval_pack(pb, "c3_linear_const_eval_0", [((K, N), weight_dtype)])
     pb.begin_program("c3_linear")
@@ -59,6 +60,8 @@ def c3_linear(M, K=4096, N=14336, weight_dtype=DT.BFP_BFloat8, activation="gelu"
     w = pb.input((K, N), DT.BFloat16)
     bias = pb.input((N,), DT.BFloat16)
     (wq,) = pb.load_cached(ce, "c3_linear_const_eval_0", [w], ce_outs)
+    if program_config is not None:
+        pb.set_matmul_program_config(*program_config)
     y = pb.linear(a, wq, bias, activation=activation)
     pb.output(y)
     pb.end_program()
