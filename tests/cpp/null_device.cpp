@@ -93,8 +93,12 @@ int span(const char *fn, const char *what, const void *p, int64_t bytes, bool op
 using Launch = std::function<void()>;
 struct Graph { std::vector<Launch> nodes; };
 std::vector<Launch> *g_recording = nullptr;
-int launch(Launch f) {
+// TTMLIR_AMD_NULL_DEVICE_COMPUTE=0: arithmetic launches are counted and recorded but do nothing (programs at benchmark
+// sizes, where only the extents matter); copies and fills always run
+const bool g_compute = !(getenv("TTMLIR_AMD_NULL_DEVICE_COMPUTE") && std::string(getenv("TTMLIR_AMD_NULL_DEVICE_COMPUTE")) == "0");
+int launch(Launch f, bool cheap = false) {
   ++g_kernel_calls;
+  if (!g_compute && !cheap) f = [] {};
   if (g_recording) g_recording->push_back(std::move(f)); else f();
   return TTM_OK;
 }
@@ -310,12 +314,12 @@ EXPORT int ttm_memcpy_d2d(void *dst, const void *src, size_t bytes, void *) {
   if (!bytes) return TTM_OK;
   SPAN("destination", dst, (int64_t)bytes);
   SPAN("source", src, (int64_t)bytes);
-  return launch([=] { memmove(dst, src, bytes); });
+  return launch([=] { memmove(dst, src, bytes); }, true);
 }
 EXPORT int ttm_fill_u32(void *dst, uint32_t value, size_t count, void *) {
   if (!count) return TTM_OK;
   SPAN("destination", dst, (int64_t)count * 4);
-  return launch([=] { for (size_t i = 0; i < count; ++i) ((uint32_t *)dst)[i] = value; });
+  return launch([=] { for (size_t i = 0; i < count; ++i) ((uint32_t *)dst)[i] = value; }, true);
 }
 EXPORT int ttm_stream_create(void **stream) { if (!stream) return fail("null"); *stream = malloc(8); return TTM_OK; }
 EXPORT int ttm_stream_destroy(void *stream) { free(stream); return TTM_OK; }
@@ -360,7 +364,7 @@ EXPORT int ttm_get_option(const char *name, int *value) { if (!name || !value) r
 // ---- layout, block float, typecast
 EXPORT int ttm_copy_kernel(const void *src, void *dst, size_t bytes, void *) {
   SPAN("source", src, (int64_t)bytes); SPAN("destination", dst, (int64_t)bytes);
-  return launch([=] { memmove(dst, src, bytes); });
+  return launch([=] { memmove(dst, src, bytes); }, true);
 }
 EXPORT int ttm_tilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int elem, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
@@ -495,15 +499,23 @@ EXPORT int ttm_linear_qkv_decode(const void *a, const void *wq, const void *wk, 
 }
 
 // ---- element-wise
-EXPORT int ttm_eltwise_unary(int, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float, void *) {
+EXPORT int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float param, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("input", in, tensor_bytes(dtype, layout, batch, rows, cols)); SPAN("output", out, tensor_bytes(dtype, layout, batch, rows, cols));
-  return kernel();
+  return launch([=] {
+    Dense x = load_dense(in, dtype, layout, batch, rows, cols), y(x.size());
+    orc_unary_f32(op, x.data(), y.data(), (int64_t)x.size(), param);
+    store_dense(y, out, dtype, layout, batch, rows, cols);
+  });
 }
-EXPORT int ttm_clamp(const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float, float, void *) {
+EXPORT int ttm_clamp(const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float lo, float hi, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("input", in, tensor_bytes(dtype, layout, batch, rows, cols)); SPAN("output", out, tensor_bytes(dtype, layout, batch, rows, cols));
-  return kernel();
+  return launch([=] {
+    Dense x = load_dense(in, dtype, layout, batch, rows, cols);
+    for (float &f : x) f = f != f ? f : std::fmin(std::fmax(f, lo), hi);
+    store_dense(x, out, dtype, layout, batch, rows, cols);
+  });
 }
 static int shaped(const char *fn, const char *what, const void *p, const int64_t *shape, int rank, int dtype, int layout) {
   if (!shape) return fail("%s: %s has no shape", fn, what);
@@ -517,7 +529,7 @@ static int broadcasts(const char *fn, const int64_t *shape, const int64_t *out_s
     if (shape && out_shape && shape[d] != out_shape[d] && shape[d] != 1) return fail("%s: shapes do not broadcast at dim %d", fn, d);
   return TTM_OK;
 }
-EXPORT int ttm_eltwise_binary(int, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape, void *out, const int64_t *out_shape,
+EXPORT int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape, void *out, const int64_t *out_shape,
                               int rank, int dtype, int layout, void *) {
   if (rank < 0 || rank > 8) return fail("ttm_eltwise_binary: rank");
   if (int rc = broadcasts(__func__, a_shape, out_shape, rank)) return rc;
@@ -525,7 +537,25 @@ EXPORT int ttm_eltwise_binary(int, const void *a, const int64_t *a_shape, const 
   if (int rc = shaped(__func__, "left operand", a, a_shape, rank, dtype, layout)) return rc;
   if (int rc = shaped(__func__, "right operand", b, b_shape, rank, dtype, layout)) return rc;
   if (int rc = shaped(__func__, "output", out, out_shape, rank, dtype, layout)) return rc;
-  return kernel();
+  const bool oracle_op = op == 0 || op == 1 || (op >= 3 && op <= 10), extremum = op == 100 || op == 101;   // maximum, minimum
+  if (!oracle_op && !extremum) return kernel();
+  const std::vector<int64_t> as = vec64(a_shape, rank), bs = vec64(b_shape, rank), os = vec64(out_shape, rank);
+  return launch([=] {
+    int64_t ab, ar, ac, bb, br, bc, ob, orr, oc;
+    split3(as.data(), rank, ab, ar, ac); split3(bs.data(), rank, bb, br, bc); split3(os.data(), rank, ob, orr, oc);
+    Dense x = load_dense(a, dtype, layout, ab, ar, ac), y = load_dense(b, dtype, layout, bb, br, bc), z((size_t)(ob * orr * oc));
+    if (oracle_op) {
+      orc_binary_f32(op, x.data(), as.data(), y.data(), bs.data(), z.data(), os.data(), rank);
+    } else {   // select through two comparisons of the oracle, then put NaN where either operand has one
+      Dense ge(z.size()), xe(z.size()), ye(z.size()), zero(1, 0.0f);
+      std::vector<int64_t> ones(rank, 1);
+      orc_binary_f32(op == 100 ? 6 : 8, x.data(), as.data(), y.data(), bs.data(), ge.data(), os.data(), rank);
+      orc_binary_f32(0, x.data(), as.data(), zero.data(), ones.data(), xe.data(), os.data(), rank);   // operands broadcast to the output
+      orc_binary_f32(0, y.data(), bs.data(), zero.data(), ones.data(), ye.data(), os.data(), rank);
+      for (size_t i = 0; i < z.size(); ++i) z[i] = (xe[i] != xe[i] || ye[i] != ye[i]) ? NAN : (ge[i] != 0.0f ? xe[i] : ye[i]);
+    }
+    store_dense(z, out, dtype, layout, ob, orr, oc);
+  });
 }
 EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape, void *out,
                      const int64_t *out_shape, int rank, int dtype, int layout, void *) {
@@ -536,41 +566,80 @@ EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a,
   if (int rc = shaped(__func__, "first operand", a, a_shape, rank, dtype, layout)) return rc;
   if (int rc = shaped(__func__, "second operand", b, b_shape, rank, dtype, layout)) return rc;
   if (int rc = shaped(__func__, "output", out, out_shape, rank, dtype, layout)) return rc;
-  return kernel();
+  const std::vector<int64_t> cs = vec64(cond_shape, rank), as = vec64(a_shape, rank), bs = vec64(b_shape, rank), os = vec64(out_shape, rank);
+  return launch([=] {
+    int64_t cb, cr, cc, ab, ar, ac, bb, br, bc, ob, orr, oc;
+    split3(cs.data(), rank, cb, cr, cc); split3(as.data(), rank, ab, ar, ac); split3(bs.data(), rank, bb, br, bc); split3(os.data(), rank, ob, orr, oc);
+    Dense c = load_dense(cond, dtype, layout, cb, cr, cc), x = load_dense(a, dtype, layout, ab, ar, ac), y = load_dense(b, dtype, layout, bb, br, bc);
+    Dense ce((size_t)(ob * orr * oc)), xe(ce.size()), ye(ce.size()), zero(1, 0.0f), one(1, 1.0f);
+    std::vector<int64_t> ones(rank, 1);
+    orc_binary_f32(5, c.data(), cs.data(), zero.data(), ones.data(), ce.data(), os.data(), rank);   // cond != 0 (true for NaN)
+    orc_binary_f32(1, x.data(), as.data(), one.data(), ones.data(), xe.data(), os.data(), rank);    // operands broadcast to the output
+    orc_binary_f32(1, y.data(), bs.data(), one.data(), ones.data(), ye.data(), os.data(), rank);
+    for (size_t i = 0; i < ce.size(); ++i) xe[i] = ce[i] != 0.0f ? xe[i] : ye[i];
+    store_dense(xe, out, dtype, layout, ob, orr, oc);
+  });
 }
-EXPORT int ttm_embedding(const void *indices, int, const void *weight, void *out, int elem, int64_t rows, int64_t vocab, int64_t dim, void *) {
+EXPORT int ttm_embedding(const void *indices, int index_dtype, const void *weight, void *out, int elem, int64_t rows, int64_t vocab, int64_t dim, void *) {
   if (rows * dim == 0) return TTM_OK;
   SPAN("indices", indices, rows * 4); SPAN("weight [vocab, dim]", weight, vocab * dim * elem); SPAN("output [rows, dim]", out, rows * dim * elem);
-  return kernel();
+  return launch([=] {
+    for (int64_t r = 0; r < rows; ++r) {
+      int64_t i = index_dtype == TTM_U32 ? (int64_t)((const uint32_t *)indices)[r] : (int64_t)((const int32_t *)indices)[r];
+      i = i < 0 ? 0 : (i >= vocab ? vocab - 1 : i);
+      memcpy((uint8_t *)out + r * dim * elem, (const uint8_t *)weight + i * dim * elem, (size_t)(dim * elem));
+    }
+  });
 }
 EXPORT int ttm_argmax(const void *in, int dtype, int32_t *out, int64_t rows, int64_t cols, void *) {
   if (rows * cols == 0) return TTM_OK;
   SPAN("input [rows, cols]", in, rows * cols * elem_bytes(dtype)); SPAN("output [rows]", out, rows * 4);
-  return kernel();
+  return launch([=] {
+    for (int64_t r = 0; r < rows; ++r) {
+      int64_t best = 0;
+      float bv = (float)load_scalar(in, dtype, r * cols);
+      for (int64_t c = 1; c < cols && bv == bv; ++c) {   // the first NaN wins, else the first largest
+        const float v = (float)load_scalar(in, dtype, r * cols + c);
+        if (v != v || v > bv) { bv = v; best = c; }
+      }
+      out[r] = (int32_t)best;
+    }
+  });
 }
-EXPORT int ttm_arange(void *out, int dtype, int64_t n, double, double, void *) {
+EXPORT int ttm_arange(void *out, int dtype, int64_t n, double start, double step, void *) {
   if (n == 0) return TTM_OK;
   SPAN("output", out, n * elem_bytes(dtype));
-  return kernel();
+  return launch([=] { for (int64_t i = 0; i < n; ++i) store_scalar(out, dtype, i, (float)start + (float)i * (float)step); });
 }
 
 // ---- row-wise
 EXPORT int ttm_rms_norm(const void *x, const void *weight, int weight_layout, const void *bias, int bias_layout, void *out, int dtype, int64_t batch,
-                        int64_t rows, int64_t cols, float, void *) {
+                        int64_t rows, int64_t cols, float eps, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
   SPAN_OPT("weight", weight, vec_bytes(dtype, weight_layout, cols)); SPAN_OPT("bias", bias, vec_bytes(dtype, bias_layout, cols));
-  return kernel();
+  return launch([=] {
+    store_dense(rms_norm_host(load_dense(x, dtype, TTM_TILE, batch, rows, cols), weight, weight_layout, bias, bias_layout, dtype, batch * rows, cols, eps),
+                out, dtype, TTM_TILE, batch, rows, cols);
+  });
 }
 EXPORT int ttm_softmax_lastdim(const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
-  return kernel();
+  return launch([=] {
+    Dense in = load_dense(x, dtype, TTM_TILE, batch, rows, cols), y(in.size());
+    orc_softmax_f32(in.data(), y.data(), batch * rows, cols, 1);
+    store_dense(y, out, dtype, TTM_TILE, batch, rows, cols);
+  });
 }
-EXPORT int ttm_reduce_lastdim(int, const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, void *) {
+EXPORT int ttm_reduce_lastdim(int op, const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output [.., rows, 1]", out, tile_bytes(dtype, batch, rows, 1));
-  return kernel();
+  return launch([=] {
+    Dense in = load_dense(x, dtype, TTM_TILE, batch, rows, cols), y((size_t)(batch * rows));
+    orc_reduce_f32(op, in.data(), y.data(), batch * rows, cols, 1);
+    store_dense(y, out, dtype, TTM_TILE, batch, rows, 1);
+  });
 }
 
 // ---- strided views
@@ -580,7 +649,8 @@ EXPORT int ttm_copy_view(const void *src, int64_t src_rows, int64_t src_cols, in
   if (rank < 0 || rank > 8 || (rank > 0 && (!extent || !src_stride || !dst_stride))) return fail("ttm_copy_view: rank / descriptors");
   if (int rc = view_span(__func__, "source", src, src_rows, src_cols, src_layout, elem, rank, extent, src_stride, src_base, 0)) return rc;
   if (int rc = view_span(__func__, "destination", dst, dst_rows, dst_cols, dst_layout, elem, rank, extent, dst_stride, dst_base, 0)) return rc;
-  return kernel();
+  const std::vector<int64_t> ex = vec64(extent, rank), ss = vec64(src_stride, rank), ds = vec64(dst_stride, rank);
+  return launch([=] { copy_view_host(src, src_rows, src_cols, src_layout, dst, dst_rows, dst_cols, dst_layout, elem, ex, ss, src_base, ds, dst_base); });
 }
 EXPORT int ttm_copy_view_at(const void *src, int64_t src_rows, int64_t src_cols, int src_layout, void *dst, int64_t dst_rows, int64_t dst_cols,
                             int dst_layout, int elem, int rank, const int64_t *extent, const int64_t *src_stride, int64_t src_base,
@@ -590,12 +660,30 @@ EXPORT int ttm_copy_view_at(const void *src, int64_t src_rows, int64_t src_cols,
   if (int rc = view_span(__func__, "source", src, src_rows, src_cols, src_layout, elem, rank, extent, src_stride, src_base, 0)) return rc;
   const int64_t far = index_limit > 0 ? (index_limit - 1) * index_stride : 0;
   if (int rc = view_span(__func__, "destination", dst, dst_rows, dst_cols, dst_layout, elem, rank, extent, dst_stride, dst_base, far)) return rc;
-  return kernel();
+  const std::vector<int64_t> ex = vec64(extent, rank), ss = vec64(src_stride, rank), ds = vec64(dst_stride, rank);
+  return launch([=] {
+    const int64_t at = *index;   // read when the launch runs: a replayed graph sees the current position
+    if (at < 0 || at >= index_limit) return;
+    copy_view_host(src, src_rows, src_cols, src_layout, dst, dst_rows, dst_cols, dst_layout, elem, ex, ss, src_base, ds, dst_base + at * index_stride);
+  });
 }
 
 // ---- attention
+// [B, S, H * D] <-> [B, H, S, D]
+static Dense heads_outer(const Dense &x, int64_t B, int64_t H, int64_t S, int64_t D, bool inverse) {
+  Dense y(x.size());
+  for (int64_t b = 0; b < B; ++b)
+    for (int64_t h = 0; h < H; ++h)
+      for (int64_t s_ = 0; s_ < S; ++s_)
+        for (int64_t d = 0; d < D; ++d) {
+          const size_t inner = (size_t)(((b * S + s_) * H + h) * D + d), outer = (size_t)(((b * H + h) * S + s_) * D + d);
+          if (inverse) y[inner] = x[outer]; else y[outer] = x[inner];
+        }
+  return y;
+}
 static int sdpa_check(const char *fn, const void *q, const void *k, const void *v, const void *mask, int mask_heads, int64_t mask_batch, void *out, int dtype,
-                      int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, const void *sink) {
+                      int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, const void *sink, int is_causal = 0, float scale = 0.0f,
+                      int heads_inner = 0, int64_t window = -1) {
   if (B * Hq * Sq * D == 0) return TTM_OK;
   if (Hkv < 1 || Hq % Hkv != 0) return fail("%s: query heads must be a multiple of kv heads", fn);
   // heads side by side or heads as matrices: the same tiles in another order, the same bytes (D is a multiple of 32)
@@ -605,20 +693,35 @@ static int sdpa_check(const char *fn, const void *q, const void *k, const void *
   if (int rc = span(fn, "mask", mask, tile_bytes(dtype, mask_batch * mask_heads, Sq, Sk), true)) return rc;
   if (int rc = span(fn, "attention sink", sink, tile_bytes(TTM_BF16, Hq, 1, 1), true)) return rc;
   if (int rc = span(fn, "output", out, tile_bytes(dtype, B * Hq, Sq, D))) return rc;
-  return kernel();
+  return launch([=] {
+    auto operand = [&](const void *p, int64_t H, int64_t S, bool inner) {
+      return inner ? heads_outer(load_dense(p, dtype, TTM_TILE, B, S, H * D), B, H, S, D, false) : load_dense(p, dtype, TTM_TILE, B * H, S, D);
+    };
+    Dense Q = operand(q, Hq, Sq, heads_inner & 1), K = operand(k, Hkv, Sk, heads_inner & 2), V = operand(v, Hkv, Sk, heads_inner & 4), M, S_, O(Q.size());
+    if (mask) {
+      M = load_dense(mask, dtype, TTM_TILE, mask_batch * mask_heads, Sq, Sk);
+      if (mask_batch == 1 && B > 1) { Dense one = M; for (int64_t b = 1; b < B; ++b) M.insert(M.end(), one.begin(), one.end()); }
+    }
+    if (sink) S_ = load_dense(sink, TTM_BF16, TTM_TILE, Hq, 1, 1);
+    orc_sdpa_f32(Q.data(), K.data(), V.data(), mask ? M.data() : nullptr, mask_heads, O.data(), B, Hq, Hkv, Sq, Sk, D, is_causal, scale, window < 0 ? -1 : window,
+                 sink ? S_.data() : nullptr);
+    if (heads_inner & 8) store_dense(heads_outer(O, B, Hq, Sq, D, true), out, dtype, TTM_TILE, B, Sq, Hq * D);
+    else store_dense(O, out, dtype, TTM_TILE, B * Hq, Sq, D);
+  });
 }
 EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B, int64_t Hq, int64_t Hkv,
-                    int64_t Sq, int64_t Sk, int64_t D, int, float, void *) {
-  return sdpa_check(__func__, q, k, v, mask, mask_heads, B, out, dtype, B, Hq, Hkv, Sq, Sk, D, nullptr);
+                    int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, void *) {
+  return sdpa_check(__func__, q, k, v, mask, mask_heads, B, out, dtype, B, Hq, Hkv, Sq, Sk, D, nullptr, is_causal, scale);
 }
 EXPORT int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out, int dtype, int64_t B, int64_t Hq,
-                                int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int, float, int, void *) {
-  return sdpa_check(__func__, q, k, v, mask, mask_heads, B, out, dtype, B, Hq, Hkv, Sq, Sk, D, nullptr);
+                                int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int heads_inner, void *) {
+  return sdpa_check(__func__, q, k, v, mask, mask_heads, B, out, dtype, B, Hq, Hkv, Sq, Sk, D, nullptr, is_causal, scale, heads_inner);
 }
 EXPORT int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const void *mask, int mask_heads, int64_t mask_batch, void *out, int dtype,
-                             int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int, float, int, int64_t, const void *attention_sink,
-                             void *) {
-  return sdpa_check(__func__, q, k, v, mask, mask_heads, mask_batch, out, dtype, B, Hq, Hkv, Sq, Sk, D, attention_sink);
+                             int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int heads_inner,
+                             int64_t sliding_window, const void *attention_sink, void *) {
+  return sdpa_check(__func__, q, k, v, mask, mask_heads, mask_batch, out, dtype, B, Hq, Hkv, Sq, Sk, D, attention_sink, is_causal, scale, heads_inner,
+                    sliding_window);
 }
 static int decode_check(const char *fn, const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
                         int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,

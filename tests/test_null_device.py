@@ -1,9 +1,11 @@
-"""The host runtime on a device that computes nothing and checks everything (tests/cpp/null_device.cpp): a stand-in for the
-kernel library whose entry points hold every pointer against the live allocations and the bytes the real kernels touch.
-Put in front of the real library with LD_LIBRARY_PATH, it lets the executor run whole programs on the CPU: the tensor pool,
-the fused launches, the trace protocol and the hooks all run; a launch whose buffer is too small - a memory fault on the
-GPU - is an error here.  Results are meaningless, so the GPU runtime tests are run with assertions stripped (python -O):
-what is checked is that every program runs to its end and that no launch leaves its buffers."""
+"""The host runtime on a device in host memory (tests/cpp/null_device.cpp): a stand-in for the kernel library whose entry
+points hold every pointer against the live allocations and the bytes the real kernels touch, and then compute the common ops
+with the oracle's arithmetic (the decode-path kernels compute nothing).  Put in front of the real library with
+LD_LIBRARY_PATH, it lets the executor run whole programs on the CPU: the tensor pool, the caches, the fused launches, the
+trace protocol (recorded launches are closures that a replay runs) and the hooks all run; a launch whose buffer is too small
+- a memory fault on the GPU - is an error here.  The GPU runtime tests whose programs the null device computes run here with
+their assertions on values; all of them run once more with assertions stripped (python -O), where what is checked is that
+every program runs to its end and that no launch leaves its buffers."""
 import json
 import os
 import subprocess
@@ -14,11 +16,19 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
+def _oracle_link():
+    """Linker arguments for the oracle library, whose arithmetic the null device computes with (built if missing)."""
+    sys.path.insert(0, ROOT)
+    import oracle.oracle as orc
+    oracle_dir = os.path.dirname(orc.build())
+    return ["-L", oracle_dir, "-lttm_oracle", "-Wl,-rpath," + oracle_dir]
+
+
 @pytest.fixture(scope="module")
 def null_env(tmp_path_factory):
     d = tmp_path_factory.mktemp("null_device")
     subprocess.run(["g++", "-std=c++17", "-O1", "-shared", "-fPIC", "-fvisibility=hidden", "-I", os.path.join(ROOT, "include"),
-                    "-o", str(d / "libttmlir_amd_hip.so"), os.path.join(ROOT, "tests", "cpp", "null_device.cpp")], check=True)
+                    "-o", str(d / "libttmlir_amd_hip.so"), os.path.join(ROOT, "tests", "cpp", "null_device.cpp")] + _oracle_link(), check=True)
     env = dict(os.environ)
     # the runtime library finds the kernel library through its RUNPATH, which LD_LIBRARY_PATH precedes
     env["LD_LIBRARY_PATH"] = str(d) + os.pathsep + env.get("LD_LIBRARY_PATH", "")
@@ -58,6 +68,26 @@ print("ok")
 """
     r = subprocess.run([sys.executable, "-c", code], env=null_env, capture_output=True, text=True, timeout=120)
     assert r.returncode == 0 and r.stdout.strip() == "ok", r.stderr[-600:]
+
+
+# programs with decode-path kernels (rotary embedding, cache writes, decode and chunked attention): not computed on the host
+NOT_COMPUTED = ("chunked_prefill_attention or rotary_embedding or decode_layer_steps or update_cache_reads or paged_cache_program or "
+                "sliding_window_and_sink")
+
+
+def test_runtime_programs_give_the_oracles_values_on_the_host(null_env):
+    """The GPU runtime tests, assertions and all, on the computing null device: what they assert about values (a traced
+    program against the same program run op by op and against the oracle, const-eval and trace cache behaviour under
+    replaced weights, hooks that read and replace tensors, fused launches against the op-by-op run) is host logic plus
+    arithmetic the oracle defines, so a wrong tensor reaching a launch fails here before it fails on a GPU."""
+    skip = "not full_size and not profiler_ranges and not (%s)" % NOT_COMPUTED
+    r = subprocess.run([sys.executable, "-m", "pytest", os.path.join(ROOT, "tests", "test_gpu_runtime.py"), "-q", "-m", "gpu",
+                        "-p", "no:cacheprovider", "-k", skip], env=null_env, capture_output=True, text=True, timeout=1500, cwd=ROOT)
+    tail = r.stdout[-3000:] + r.stderr[-1000:]
+    assert r.returncode == 0, tail
+    last = [l for l in r.stdout.strip().splitlines() if " passed" in l][-1]
+    assert int(last.split(" passed")[0].split()[-1]) >= 40 and "failed" not in last, last
+    assert "traced_program_with_alternating_weight_sets" not in r.stdout      # ran and passed (failures are listed by name)
 
 
 def test_runtime_programs_stay_inside_their_buffers(null_env):
@@ -250,7 +280,8 @@ run("decode32_traced", programs.decode_layer(trace=True), steps=3)
 rt.close_mesh_device(dev)
 print(json.dumps(report))
 """ % (ROOT, ROOT)
-    r = subprocess.run([sys.executable, "-c", code], env=null_env, capture_output=True, text=True, timeout=900, cwd=ROOT)
+    env = dict(null_env, TTMLIR_AMD_NULL_DEVICE_COMPUTE="0")   # extents only: the arithmetic of these sizes takes minutes on the host
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=900, cwd=ROOT)
     assert r.returncode == 0, (r.stdout[-500:], r.stderr[-1500:])
     rep = json.loads(r.stdout.strip().splitlines()[-1])
     assert rep["c3_2048"]["shapes"] == [[2048, 14336]] and rep["c3_32"]["shapes"] == [[32, 14336]]
@@ -325,7 +356,7 @@ def test_runtime_under_sanitizers_on_the_null_device(tmp_path, sanitizer):
     jobs = [subprocess.Popen(common + inc + ["-c", os.path.join(rtsrc, f), "-o", str(tmp_path / (f + ".o"))])
             for f in sorted(os.listdir(rtsrc)) if f.endswith(".cpp")]
     jobs.append(subprocess.Popen(common + ["-shared", "-fvisibility=hidden"] + inc + ["-o", str(tmp_path / "libttmlir_amd_hip.so"),
-                                           os.path.join(ROOT, "tests", "cpp", "null_device.cpp")]))
+                                           os.path.join(ROOT, "tests", "cpp", "null_device.cpp")] + _oracle_link()))
     assert all(j.wait() == 0 for j in jobs)
     objs = [str(p) for p in tmp_path.glob("*.o")]
     subprocess.run(common + inc + [os.path.join(ROOT, "tests", "cpp", "runtime_stress.cpp")] + objs +
@@ -358,12 +389,12 @@ def test_damaged_programs_through_the_runtime_under_address_sanitizer(tmp_path):
     jobs = [subprocess.Popen(common + inc + ["-c", os.path.join(rtsrc, f), "-o", str(tmp_path / (f + ".o"))])
             for f in sorted(os.listdir(rtsrc)) if f.endswith(".cpp")]
     jobs.append(subprocess.Popen(common + ["-shared", "-fvisibility=hidden"] + inc + ["-o", str(tmp_path / "libttmlir_amd_hip.so"),
-                                           os.path.join(ROOT, "tests", "cpp", "null_device.cpp")]))
+                                           os.path.join(ROOT, "tests", "cpp", "null_device.cpp")] + _oracle_link()))
     assert all(j.wait() == 0 for j in jobs)
     subprocess.run(common + inc + [os.path.join(ROOT, "tests", "cpp", "runtime_fuzz.cpp")] + [str(p) for p in tmp_path.glob("*.o")] +
                    ["-L", str(tmp_path), "-lttmlir_amd_hip", "-ldl", "-o", str(tmp_path / "fuzz")], check=True)
     # a damaged shape may ask for any amount of memory: allocations above 4 GiB fail instead of being tried
-    env = dict(os.environ, LD_LIBRARY_PATH=str(tmp_path), ASAN_OPTIONS="max_allocation_size_mb=4096:allocator_may_return_null=1:detect_leaks=0",
+    env = dict(os.environ, LD_LIBRARY_PATH=str(tmp_path), TTMLIR_AMD_NULL_DEVICE_COMPUTE="0", ASAN_OPTIONS="max_allocation_size_mb=4096:allocator_may_return_null=1:detect_leaks=0",
                UBSAN_OPTIONS="print_stacktrace=1")
     r = subprocess.run([str(tmp_path / "fuzz"), "400"] + files, env=env, capture_output=True, text=True, timeout=900)
     assert "Sanitizer" not in r.stderr and "runtime error" not in r.stderr, r.stderr[-3000:]
