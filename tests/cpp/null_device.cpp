@@ -26,6 +26,7 @@
 #include <vector>
 
 #include "ttmlir_amd_hip.h"
+#include "ttm_extents.h"   // tt-mlir_amd/csrc: the bytes every entry point touches, shared with the kernel library
 
 #define EXPORT extern "C" __attribute__((visibility("default")))
 
@@ -46,28 +47,10 @@ int fail(const char *fmt, ...) {
   return TTM_ERR_INVALID;
 }
 
-int64_t pad32(int64_t n) { return (n + 31) / 32 * 32; }
-int64_t elem_bytes(int dtype) {
-  switch (dtype) {
-  case TTM_F32: case TTM_U32: case TTM_I32: return 4;
-  case TTM_F16: case TTM_BF16: case TTM_U16: return 2;
-  case TTM_U8: return 1;
-  default: return 0;
-  }
-}
-// bytes of a [batch, rows, cols] tile tensor of a plain or block-float type
-int64_t tile_bytes(int dtype, int64_t batch, int64_t rows, int64_t cols) {
-  const int64_t tiles = batch * (pad32(rows) / 32) * (pad32(cols) / 32);
-  if (dtype == TTM_BFP8B) return tiles * 1088;
-  if (dtype == TTM_BFP4B) return tiles * 576;
-  return tiles * 1024 * elem_bytes(dtype);
-}
-int64_t tensor_bytes(int dtype, int layout, int64_t batch, int64_t rows, int64_t cols) {
-  return layout == TTM_TILE ? tile_bytes(dtype, batch, rows, cols) : batch * rows * cols * elem_bytes(dtype);
-}
-int64_t vec_bytes(int dtype, int layout, int64_t cols) {   // a [cols] weight / bias vector
-  return layout == TTM_TILE ? tile_bytes(dtype, 1, 1, cols) : cols * elem_bytes(dtype);
-}
+using ttm_extents::pad32;
+using ttm_extents::elem_bytes;
+using ttm_extents::tile_bytes;
+using ttm_extents::split3;
 
 // `bytes` from p on lie in one live allocation
 int span(const char *fn, const char *what, const void *p, int64_t bytes, bool optional = false) {
@@ -86,8 +69,12 @@ int span(const char *fn, const char *what, const void *p, int64_t bytes, bool op
                 (long long)bytes);
   return TTM_OK;
 }
+struct Chk {   // the checker the shared extent rules call
+  const char *fn;
+  int operator()(const char *what, const void *p, int64_t bytes, bool optional) const { return span(fn, what, p, bytes, optional); }
+};
+#define EXT(rule, ...) do { if (int rc_ = ttm_extents::rule(Chk{__func__}, __VA_ARGS__)) return rc_; } while (0)
 #define SPAN(what, p, bytes) do { if (int rc_ = span(__func__, what, p, bytes)) return rc_; } while (0)
-#define SPAN_OPT(what, p, bytes) do { if (int rc_ = span(__func__, what, p, bytes, true)) return rc_; } while (0)
 
 // a launch: run now, or recorded while a capture is in progress (the runtime serialises the work of a device)
 using Launch = std::function<void()>;
@@ -104,29 +91,14 @@ int launch(Launch f, bool cheap = false) {
 }
 int kernel() { return launch([] {}); }   // an entry point that computes nothing
 
-// a [.., rows, cols] shape of `rank` entries as (batch, rows, cols); rank 1 is one row
-void split3(const int64_t *shape, int rank, int64_t &b, int64_t &r, int64_t &c) {
-  b = 1; r = 1; c = 1;
-  if (rank >= 1) c = shape[rank - 1];
-  if (rank >= 2) r = shape[rank - 2];
-  for (int i = 0; i + 2 < rank; ++i) b *= shape[i];
+// strided view (ttm_copy_view): the shared rule, with its "view reaches below offset 0" case as an error of its own
+int view_span(const char *fn, const char *what, const void *p, int64_t rows, int64_t cols, int layout, int elem, int rank, const int64_t *extent,
+              const int64_t *stride, int64_t base, int64_t extra_max) {
+  bool negative = false;
+  const int rc = ttm_extents::view(Chk{fn}, what, p, rows, cols, layout, elem, rank, extent, stride, base, extra_max, &negative);
+  return negative ? fail("out of bounds: %s: the %s view reaches a negative logical offset", fn, what) : rc;
 }
 
-// strided view over a tensor whose last two dims are [rows, cols]: the tensor must hold every matrix up to the one the
-// largest logical offset lies in
-int view_span(const char *fn, const char *what, const void *p, int64_t rows, int64_t cols, int layout, int elem, int rank,
-              const int64_t *extent, const int64_t *stride, int64_t base, int64_t extra_max) {
-  int64_t lo = base, hi = base + extra_max;
-  for (int i = 0; i < rank; ++i) {
-    if (extent[i] <= 0) return TTM_OK;   // empty view
-    const int64_t d = (extent[i] - 1) * stride[i];
-    if (d >= 0) hi += d; else lo += d;
-  }
-  if (lo < 0) return fail("out of bounds: %s: the %s view reaches logical offset %lld", fn, what, (long long)lo);
-  const int64_t per = rows * cols, mats = per > 0 ? hi / per + 1 : 0;
-  const int64_t bytes = layout == TTM_TILE ? mats * pad32(rows) * pad32(cols) * elem : (hi + 1) * elem;
-  return span(fn, what, p, bytes);
-}
 // ---- host arithmetic.  The oracle (oracle/ttm_oracle.c) supplies the formulas; tensors pass through dense row-major f32.
 extern "C" {
 void orc_tilize(const void *in, void *out, int64_t batch, int64_t rows, int64_t cols, int elem);
@@ -363,37 +335,33 @@ EXPORT int ttm_get_option(const char *name, int *value) { if (!name || !value) r
 
 // ---- layout, block float, typecast
 EXPORT int ttm_copy_kernel(const void *src, void *dst, size_t bytes, void *) {
-  SPAN("source", src, (int64_t)bytes); SPAN("destination", dst, (int64_t)bytes);
+  EXT(copy_kernel, src, dst, bytes);
   return launch([=] { memmove(dst, src, bytes); }, true);
 }
 EXPORT int ttm_tilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int elem, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("row-major input", src, batch * rows * cols * elem);
-  SPAN("tile output", dst, batch * pad32(rows) * pad32(cols) * elem);
+  EXT(tilize, src, dst, batch, rows, cols, elem);
   return launch([=] { orc_tilize(src, dst, batch, rows, cols, elem); });
 }
 EXPORT int ttm_untilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols, int elem, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("tile input", src, batch * pad32(rows) * pad32(cols) * elem);
-  SPAN("row-major output", dst, batch * rows * cols * elem);
+  EXT(untilize, src, dst, batch, rows, cols, elem);
   return launch([=] { orc_untilize(src, dst, batch, rows, cols, elem); });
 }
 EXPORT int64_t ttm_bfp_tile_bytes(int fmt) { return fmt == TTM_BFP8B ? 1088 : (fmt == TTM_BFP4B ? 576 : -1); }
 EXPORT int ttm_bfp_pack(const void *src, int src_dtype, int src_layout, void *dst, int fmt, int64_t batch, int64_t rows, int64_t cols, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("input", src, tensor_bytes(src_dtype, src_layout, batch, rows, cols));
-  SPAN("block-float output", dst, tile_bytes(fmt, batch, rows, cols));
+  EXT(bfp_pack, src, src_dtype, src_layout, dst, fmt, batch, rows, cols);
   return launch([=] { store_dense(load_dense(src, src_dtype, src_layout, batch, rows, cols), dst, fmt, TTM_TILE, batch, rows, cols); });
 }
 EXPORT int ttm_bfp_unpack(const void *src, int fmt, void *dst, int dst_dtype, int dst_layout, int64_t batch, int64_t rows, int64_t cols, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("block-float input", src, tile_bytes(fmt, batch, rows, cols));
-  SPAN("output", dst, tensor_bytes(dst_dtype, dst_layout, batch, rows, cols));
+  EXT(bfp_unpack, src, fmt, dst, dst_dtype, dst_layout, batch, rows, cols);
   return launch([=] { store_dense(load_dense(src, fmt, TTM_TILE, batch, rows, cols), dst, dst_dtype, dst_layout, batch, rows, cols); });
 }
 EXPORT int ttm_typecast(const void *in, int src_dtype, void *out, int dst_dtype, int64_t n, void *) {
   if (n == 0) return TTM_OK;
-  SPAN("input", in, n * elem_bytes(src_dtype)); SPAN("output", out, n * elem_bytes(dst_dtype));
+  EXT(typecast, in, src_dtype, out, dst_dtype, n);
   return launch([=] { for (int64_t i = 0; i < n; ++i) store_scalar(out, dst_dtype, i, load_scalar(in, src_dtype, i)); });
 }
 
@@ -402,12 +370,8 @@ static int linear_check(const char *fn, const void *a, int a_dtype, const void *
                         int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch, int64_t M, int64_t N, int64_t K, int act, int tail_op,
                         const void *tail) {
   if (batch * M * N == 0) return TTM_OK;
-  if (int rc = span(fn, "activations [batch, M, K]", a, tile_bytes(a_dtype, batch, M, K))) return rc;
-  if (int rc = span(fn, "weights [w_batch, K, N]", w, tile_bytes(w_dtype, w_batch, K, N))) return rc;
-  if (int rc = span(fn, "bias", bias, vec_bytes(bias_dtype, bias_layout, N), true)) return rc;
-  if (int rc = span(fn, "output [batch, M, N]", out, tile_bytes(out_dtype, batch, M, N))) return rc;
-  if (tail_op != TTM_TAIL_NONE)
-    if (int rc = span(fn, "tail operand [batch, M, N]", tail, tile_bytes(TTM_BF16, batch, M, N))) return rc;
+  if (int rc = ttm_extents::linear(Chk{fn}, a, a_dtype, w, w_dtype, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, tail_op, tail))
+    return rc;
   if (a_dtype != TTM_BF16 || out_dtype != TTM_BF16) return kernel();
   return launch([=] {
     store_dense(linear_host(a, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, batch, w_batch, M, N, K, act, tail_op, tail), out, TTM_BF16,
@@ -428,11 +392,7 @@ EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtyp
 EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N, const int *act, int64_t M,
                             int64_t K, void *) {
   if (n < 1 || n > 4 || !w || !out || !N) return fail("ttm_linear_group: one to four members with weights, outputs and widths");
-  SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
-  for (int i = 0; i < n; ++i) {
-    SPAN("weights [K, N_i]", w[i], tile_bytes(w_dtype, 1, K, N[i]));
-    SPAN("output [M, N_i]", out[i], tile_bytes(TTM_BF16, 1, M, N[i]));
-  }
+  EXT(linear_group, a, n, w, w_dtype, out, N, M, K);
   std::vector<const void *> ws(w, w + n);
   std::vector<void *> outs(out, out + n);
   std::vector<int64_t> ns(N, N + n);
@@ -445,9 +405,7 @@ EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dt
   });
 }
 EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M, int64_t N, int64_t K, void *) {
-  SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
-  SPAN("weights 0", w0, tile_bytes(w_dtype, 1, K, N)); SPAN("weights 1", w1, tile_bytes(w_dtype, 1, K, N));
-  SPAN("output 0", out0, tile_bytes(TTM_BF16, 1, M, N)); SPAN("output 1", out1, tile_bytes(TTM_BF16, 1, M, N));
+  EXT(linear_pair, a, w0, w1, w_dtype, out0, out1, M, N, K);
   return launch([=] {
     store_dense(linear_host(a, w0, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, N, K, TTM_ACT_NONE, TTM_TAIL_NONE, nullptr), out0, TTM_BF16, TTM_TILE, 1, M, N);
     store_dense(linear_host(a, w1, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, N, K, TTM_ACT_NONE, TTM_TAIL_NONE, nullptr), out1, TTM_BF16, TTM_TILE, 1, M, N);
@@ -461,13 +419,7 @@ EXPORT int ttm_linear_add_rms_norm(const void *a, const void *w, int w_dtype, co
                                    int weight_layout, const void *norm_bias, int bias_layout, float eps, void *norm_out, int64_t M, int64_t N, int64_t K,
                                    void *) {
   if (!ttm_linear_add_rms_norm_supported(w_dtype, M, N, K)) return fail("ttm_linear_add_rms_norm: unsupported shape");
-  SPAN("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K));
-  SPAN("weights [K, N]", w, tile_bytes(w_dtype, 1, K, N));
-  SPAN("residual [M, N]", residual, tile_bytes(TTM_BF16, 1, M, N));
-  SPAN("sum output [M, N]", sum_out, tile_bytes(TTM_BF16, 1, M, N));
-  SPAN("norm output [M, N]", norm_out, tile_bytes(TTM_BF16, 1, M, N));
-  SPAN_OPT("norm weight", norm_weight, vec_bytes(TTM_BF16, weight_layout, N));
-  SPAN_OPT("norm bias", norm_bias, vec_bytes(TTM_BF16, bias_layout, N));
+  EXT(linear_add_rms_norm, a, w, w_dtype, residual, sum_out, norm_weight, weight_layout, norm_bias, bias_layout, norm_out, M, N, K);
   if (sum_out == residual || norm_out == sum_out || norm_out == residual) return fail("ttm_linear_add_rms_norm: the outputs alias");
   return launch([=] {
     Dense x1 = linear_host(a, w, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, N, K, TTM_ACT_NONE, TTM_TAIL_ADD, residual);
@@ -485,23 +437,15 @@ EXPORT int ttm_linear_qkv_decode(const void *a, const void *wq, const void *wk, 
   if (!ttm_linear_qkv_decode_supported(w_dtype, users, K, heads, kv_heads, head_dim)) return fail("ttm_linear_qkv_decode: unsupported shape");
   if (token_index < 0 || token_index >= cache_rows) return fail("ttm_linear_qkv_decode: token_index outside the cached positions");
   if (batch_offset < 0 || batch_offset + users > cache_users) return fail("ttm_linear_qkv_decode: batch_offset + users exceeds the cache");
-  SPAN("activations [users, K]", a, tile_bytes(TTM_BF16, 1, users, K));
-  SPAN("q weights", wq, tile_bytes(w_dtype, 1, K, heads * head_dim));
-  SPAN("k weights", wk, tile_bytes(w_dtype, 1, K, kv_heads * head_dim));
-  SPAN("v weights", wv, tile_bytes(w_dtype, 1, K, kv_heads * head_dim));
-  SPAN("cos cache", cos_cache, tile_bytes(TTM_BF16, 1, cache_rows, head_dim));
-  SPAN("sin cache", sin_cache, tile_bytes(TTM_BF16, 1, cache_rows, head_dim));
-  SPAN("q output [1, users, heads, head_dim]", q_out, tile_bytes(TTM_BF16, users, heads, head_dim));
-  SPAN("k cache", k_cache, tile_bytes(TTM_BF16, cache_users * kv_heads, max_seq, head_dim));
-  SPAN("v cache", v_cache, tile_bytes(TTM_BF16, cache_users * kv_heads, max_seq, head_dim));
-  SPAN("update index", update_index, 4);
+  EXT(linear_qkv_decode, a, wq, wk, wv, w_dtype, users, K, heads, kv_heads, head_dim, cos_cache, sin_cache, cache_rows, q_out, k_cache, v_cache,
+      cache_users, max_seq, update_index);
   return kernel();
 }
 
 // ---- element-wise
 EXPORT int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float param, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("input", in, tensor_bytes(dtype, layout, batch, rows, cols)); SPAN("output", out, tensor_bytes(dtype, layout, batch, rows, cols));
+  EXT(unary, in, out, dtype, layout, batch, rows, cols);
   return launch([=] {
     Dense x = load_dense(in, dtype, layout, batch, rows, cols), y(x.size());
     orc_unary_f32(op, x.data(), y.data(), (int64_t)x.size(), param);
@@ -510,18 +454,12 @@ EXPORT int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int l
 }
 EXPORT int ttm_clamp(const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float lo, float hi, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("input", in, tensor_bytes(dtype, layout, batch, rows, cols)); SPAN("output", out, tensor_bytes(dtype, layout, batch, rows, cols));
+  EXT(unary, in, out, dtype, layout, batch, rows, cols);
   return launch([=] {
     Dense x = load_dense(in, dtype, layout, batch, rows, cols);
     for (float &f : x) f = f != f ? f : std::fmin(std::fmax(f, lo), hi);
     store_dense(x, out, dtype, layout, batch, rows, cols);
   });
-}
-static int shaped(const char *fn, const char *what, const void *p, const int64_t *shape, int rank, int dtype, int layout) {
-  if (!shape) return fail("%s: %s has no shape", fn, what);
-  int64_t b, r, c;
-  split3(shape, rank, b, r, c);
-  return span(fn, what, p, tensor_bytes(dtype, layout, b, r, c));
 }
 // the real library refuses operands that do not broadcast to the output
 static int broadcasts(const char *fn, const int64_t *shape, const int64_t *out_shape, int rank) {
@@ -534,9 +472,7 @@ EXPORT int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape, con
   if (rank < 0 || rank > 8) return fail("ttm_eltwise_binary: rank");
   if (int rc = broadcasts(__func__, a_shape, out_shape, rank)) return rc;
   if (int rc = broadcasts(__func__, b_shape, out_shape, rank)) return rc;
-  if (int rc = shaped(__func__, "left operand", a, a_shape, rank, dtype, layout)) return rc;
-  if (int rc = shaped(__func__, "right operand", b, b_shape, rank, dtype, layout)) return rc;
-  if (int rc = shaped(__func__, "output", out, out_shape, rank, dtype, layout)) return rc;
+  EXT(binary, a, a_shape, b, b_shape, out, out_shape, rank, dtype, layout);
   const bool oracle_op = op == 0 || op == 1 || (op >= 3 && op <= 10), extremum = op == 100 || op == 101;   // maximum, minimum
   if (!oracle_op && !extremum) return kernel();
   const std::vector<int64_t> as = vec64(a_shape, rank), bs = vec64(b_shape, rank), os = vec64(out_shape, rank);
@@ -562,10 +498,7 @@ EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a,
   if (rank < 0 || rank > 4) return fail("ttm_where: rank");
   for (const int64_t *sh : {cond_shape, a_shape, b_shape})
     if (int rc = broadcasts(__func__, sh, out_shape, rank)) return rc;
-  if (int rc = shaped(__func__, "condition", cond, cond_shape, rank, dtype, layout)) return rc;
-  if (int rc = shaped(__func__, "first operand", a, a_shape, rank, dtype, layout)) return rc;
-  if (int rc = shaped(__func__, "second operand", b, b_shape, rank, dtype, layout)) return rc;
-  if (int rc = shaped(__func__, "output", out, out_shape, rank, dtype, layout)) return rc;
+  EXT(where, cond, cond_shape, a, a_shape, b, b_shape, out, out_shape, rank, dtype, layout);
   const std::vector<int64_t> cs = vec64(cond_shape, rank), as = vec64(a_shape, rank), bs = vec64(b_shape, rank), os = vec64(out_shape, rank);
   return launch([=] {
     int64_t cb, cr, cc, ab, ar, ac, bb, br, bc, ob, orr, oc;
@@ -582,7 +515,7 @@ EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a,
 }
 EXPORT int ttm_embedding(const void *indices, int index_dtype, const void *weight, void *out, int elem, int64_t rows, int64_t vocab, int64_t dim, void *) {
   if (rows * dim == 0) return TTM_OK;
-  SPAN("indices", indices, rows * 4); SPAN("weight [vocab, dim]", weight, vocab * dim * elem); SPAN("output [rows, dim]", out, rows * dim * elem);
+  EXT(embedding, indices, weight, out, elem, rows, vocab, dim);
   return launch([=] {
     for (int64_t r = 0; r < rows; ++r) {
       int64_t i = index_dtype == TTM_U32 ? (int64_t)((const uint32_t *)indices)[r] : (int64_t)((const int32_t *)indices)[r];
@@ -593,7 +526,7 @@ EXPORT int ttm_embedding(const void *indices, int index_dtype, const void *weigh
 }
 EXPORT int ttm_argmax(const void *in, int dtype, int32_t *out, int64_t rows, int64_t cols, void *) {
   if (rows * cols == 0) return TTM_OK;
-  SPAN("input [rows, cols]", in, rows * cols * elem_bytes(dtype)); SPAN("output [rows]", out, rows * 4);
+  EXT(argmax, in, dtype, out, rows, cols);
   return launch([=] {
     for (int64_t r = 0; r < rows; ++r) {
       int64_t best = 0;
@@ -608,7 +541,7 @@ EXPORT int ttm_argmax(const void *in, int dtype, int32_t *out, int64_t rows, int
 }
 EXPORT int ttm_arange(void *out, int dtype, int64_t n, double start, double step, void *) {
   if (n == 0) return TTM_OK;
-  SPAN("output", out, n * elem_bytes(dtype));
+  EXT(arange, out, dtype, n);
   return launch([=] { for (int64_t i = 0; i < n; ++i) store_scalar(out, dtype, i, (float)start + (float)i * (float)step); });
 }
 
@@ -616,8 +549,7 @@ EXPORT int ttm_arange(void *out, int dtype, int64_t n, double start, double step
 EXPORT int ttm_rms_norm(const void *x, const void *weight, int weight_layout, const void *bias, int bias_layout, void *out, int dtype, int64_t batch,
                         int64_t rows, int64_t cols, float eps, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
-  SPAN_OPT("weight", weight, vec_bytes(dtype, weight_layout, cols)); SPAN_OPT("bias", bias, vec_bytes(dtype, bias_layout, cols));
+  EXT(rms_norm, x, weight, weight_layout, bias, bias_layout, out, dtype, batch, rows, cols);
   return launch([=] {
     store_dense(rms_norm_host(load_dense(x, dtype, TTM_TILE, batch, rows, cols), weight, weight_layout, bias, bias_layout, dtype, batch * rows, cols, eps),
                 out, dtype, TTM_TILE, batch, rows, cols);
@@ -625,7 +557,7 @@ EXPORT int ttm_rms_norm(const void *x, const void *weight, int weight_layout, co
 }
 EXPORT int ttm_softmax_lastdim(const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
+  EXT(softmax, x, out, dtype, batch, rows, cols);
   return launch([=] {
     Dense in = load_dense(x, dtype, TTM_TILE, batch, rows, cols), y(in.size());
     orc_softmax_f32(in.data(), y.data(), batch * rows, cols, 1);
@@ -634,7 +566,7 @@ EXPORT int ttm_softmax_lastdim(const void *x, void *out, int dtype, int64_t batc
 }
 EXPORT int ttm_reduce_lastdim(int op, const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output [.., rows, 1]", out, tile_bytes(dtype, batch, rows, 1));
+  EXT(reduce, x, out, dtype, batch, rows, cols);
   return launch([=] {
     Dense in = load_dense(x, dtype, TTM_TILE, batch, rows, cols), y((size_t)(batch * rows));
     orc_reduce_f32(op, in.data(), y.data(), batch * rows, cols, 1);
@@ -686,13 +618,7 @@ static int sdpa_check(const char *fn, const void *q, const void *k, const void *
                       int heads_inner = 0, int64_t window = -1) {
   if (B * Hq * Sq * D == 0) return TTM_OK;
   if (Hkv < 1 || Hq % Hkv != 0) return fail("%s: query heads must be a multiple of kv heads", fn);
-  // heads side by side or heads as matrices: the same tiles in another order, the same bytes (D is a multiple of 32)
-  if (int rc = span(fn, "q", q, tile_bytes(dtype, B * Hq, Sq, D))) return rc;
-  if (int rc = span(fn, "k", k, tile_bytes(dtype, B * Hkv, Sk, D))) return rc;
-  if (int rc = span(fn, "v", v, tile_bytes(dtype, B * Hkv, Sk, D))) return rc;
-  if (int rc = span(fn, "mask", mask, tile_bytes(dtype, mask_batch * mask_heads, Sq, Sk), true)) return rc;
-  if (int rc = span(fn, "attention sink", sink, tile_bytes(TTM_BF16, Hq, 1, 1), true)) return rc;
-  if (int rc = span(fn, "output", out, tile_bytes(dtype, B * Hq, Sq, D))) return rc;
+  if (int rc = ttm_extents::sdpa(Chk{fn}, q, k, v, mask, mask_heads, mask_batch, out, dtype, B, Hq, Hkv, Sq, Sk, D, sink)) return rc;
   return launch([=] {
     auto operand = [&](const void *p, int64_t H, int64_t S, bool inner) {
       return inner ? heads_outer(load_dense(p, dtype, TTM_TILE, B, S, H * D), B, H, S, D, false) : load_dense(p, dtype, TTM_TILE, B * H, S, D);
@@ -727,16 +653,9 @@ static int decode_check(const char *fn, const void *q, const void *k, const void
                         int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
                         int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int concat_heads, const void *sink) {
   if (batch * heads * head_dim == 0) return TTM_OK;
-  if (int rc = span(fn, "q [1, batch, heads, head_dim]", q, tile_bytes(dtype, batch, heads, head_dim))) return rc;
-  const int64_t kv = page_table ? tile_bytes(dtype, page_blocks * kv_heads, page_block, head_dim) : tile_bytes(dtype, batch * kv_heads, seq, head_dim);
-  if (int rc = span(fn, "k", k, kv)) return rc;
-  if (int rc = span(fn, "v", v, kv)) return rc;
-  if (int rc = span(fn, "cur_pos", cur_pos, batch * 4, true)) return rc;
-  if (int rc = span(fn, "mask [mask_batch, 1, mask_heads, seq]", mask, tile_bytes(dtype, mask_batch, mask_heads, seq), true)) return rc;
-  if (int rc = span(fn, "page table", page_table, batch * pages_per_user * 4, true)) return rc;
-  if (int rc = span(fn, "attention sink [heads, 32]", sink, tile_bytes(TTM_BF16, 1, heads, 32), true)) return rc;
-  const int64_t ob = concat_heads ? tile_bytes(dtype, 1, batch, heads * head_dim) : tile_bytes(dtype, batch, heads, head_dim);
-  if (int rc = span(fn, "output", out, ob)) return rc;
+  if (int rc = ttm_extents::sdpa_decode(Chk{fn}, q, k, v, cur_pos, mask, mask_heads, mask_batch, page_table, pages_per_user, page_block, page_blocks, out,
+                                        dtype, batch, heads, kv_heads, seq, head_dim, concat_heads, sink))
+    return rc;
   return kernel();
 }
 EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads, const int32_t *page_table,
@@ -771,67 +690,50 @@ EXPORT int ttm_rotary_embedding(const void *x, const void *cos_cache, const void
                                 int64_t cache_rows, int64_t token_index, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   if (token_index >= cache_rows || (token_index < 0 && rows > cache_rows)) return fail("ttm_rotary_embedding: position outside the cos / sin caches");
-  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
-  SPAN("cos cache", cos_cache, tile_bytes(dtype, 1, cache_rows, cols)); SPAN("sin cache", sin_cache, tile_bytes(dtype, 1, cache_rows, cols));
+  EXT(rotary_embedding, x, cos_cache, sin_cache, out, dtype, batch, rows, cols, cache_rows);
   return kernel();
 }
 EXPORT int ttm_rotary_embedding_split_heads(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype, int64_t batch, int64_t heads,
                                             int64_t head_dim, int64_t cache_rows, int64_t token_index, void *) {
   if (batch * heads * head_dim == 0) return TTM_OK;
   if (token_index < 0 || token_index >= cache_rows) return fail("ttm_rotary_embedding_split_heads: position outside the cos / sin caches");
-  SPAN("input [batch, heads * head_dim]", x, tile_bytes(dtype, 1, batch, heads * head_dim));
-  SPAN("output [batch, heads, head_dim]", out, tile_bytes(dtype, batch, heads, head_dim));
-  SPAN("cos cache", cos_cache, tile_bytes(dtype, 1, cache_rows, head_dim)); SPAN("sin cache", sin_cache, tile_bytes(dtype, 1, cache_rows, head_dim));
+  EXT(rotary_embedding_split_heads, x, cos_cache, sin_cache, out, dtype, batch, heads, head_dim, cache_rows);
   return kernel();
 }
 EXPORT int ttm_rotary_embedding_llama(const void *x, const void *cos_cache, const void *sin_cache, const void *trans_mat, void *out, int dtype, int64_t batch,
                                       int64_t rows, int64_t cols, int64_t cs_batch, int64_t cs_rows, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
-  SPAN("input", x, tile_bytes(dtype, batch, rows, cols)); SPAN("output", out, tile_bytes(dtype, batch, rows, cols));
-  SPAN("cos", cos_cache, tile_bytes(dtype, cs_batch, cs_rows, cols)); SPAN("sin", sin_cache, tile_bytes(dtype, cs_batch, cs_rows, cols));
-  SPAN("transformation matrix", trans_mat, tile_bytes(TTM_BF16, 1, 32, 32));
+  EXT(rotary_embedding_llama, x, cos_cache, sin_cache, trans_mat, out, dtype, batch, rows, cols, cs_batch, cs_rows);
   return kernel();
 }
 EXPORT int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users, int64_t heads, int64_t max_seq,
                             int64_t head_dim, int64_t input_users, int64_t batch_offset, void *) {
   if (batch_offset < 0 || batch_offset + input_users > users) return fail("ttm_update_cache: batch_offset + input users exceeds the cache");
-  SPAN("cache", cache, tile_bytes(dtype, users * heads, max_seq, head_dim));
-  SPAN("input [1, heads, users, head_dim]", input, tile_bytes(dtype, heads, input_users, head_dim));
-  SPAN("update index", update_index, 4);
+  EXT(update_cache, cache, input, update_index, dtype, users, heads, max_seq, head_dim, input_users);
   return kernel();
 }
 EXPORT int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t users, int64_t heads, int64_t max_seq, int64_t head_dim, int64_t seq,
                           int64_t batch_offset, void *) {
   if (batch_offset < 0 || batch_offset >= users || seq > max_seq) return fail("ttm_fill_cache: the input does not fit the cache entry");
-  SPAN("cache", cache, tile_bytes(dtype, users * heads, max_seq, head_dim));
-  SPAN("input [1, heads, seq, head_dim]", input, tile_bytes(dtype, heads, seq, head_dim));
+  EXT(fill_cache, cache, input, dtype, users, heads, max_seq, head_dim, seq);
   return kernel();
 }
 EXPORT int ttm_paged_update_cache(void *cache, const void *input, const int32_t *update_index, const int32_t *page_table, int dtype, int64_t blocks,
                                   int64_t heads, int64_t block_size, int64_t head_dim, int64_t users, int64_t pages_per_user, int, void *) {
-  SPAN("cache", cache, tile_bytes(dtype, blocks * heads, block_size, head_dim));
-  SPAN("input [1, users, heads, head_dim]", input, tile_bytes(dtype, users, heads, head_dim));
-  SPAN("update index [users]", update_index, users * 4);
-  SPAN_OPT("page table", page_table, users * pages_per_user * 4);
+  EXT(paged_update_cache, cache, input, update_index, page_table, dtype, blocks, heads, block_size, head_dim, users, pages_per_user);
   return kernel();
 }
 EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_t *page_table, const int32_t *batch_idx, int dtype, int64_t blocks, int64_t heads,
                                 int64_t block_size, int64_t head_dim, int64_t in_batch, int64_t seq, int64_t table_rows, int64_t pages_per_user, void *) {
-  SPAN("cache", cache, tile_bytes(dtype, blocks * heads, block_size, head_dim));
-  SPAN("input [in_batch, heads, seq, head_dim]", input, tile_bytes(dtype, in_batch * heads, seq, head_dim));
-  SPAN("page table", page_table, table_rows * pages_per_user * 4);
-  SPAN_OPT("batch index", batch_idx, in_batch * 4);
+  EXT(paged_fill_cache, cache, input, page_table, batch_idx, dtype, blocks, heads, block_size, head_dim, in_batch, seq, table_rows, pages_per_user);
   return kernel();
 }
 EXPORT int ttm_paged_gather(const void *cache, const int32_t *page_table, void *out, int dtype, int64_t blocks, int64_t heads, int64_t block_size,
                             int64_t head_dim, int64_t users, int64_t pages_per_user, void *) {
-  SPAN("cache", cache, tile_bytes(dtype, blocks * heads, block_size, head_dim));
-  SPAN("page table", page_table, users * pages_per_user * 4);
-  SPAN("output", out, tile_bytes(dtype, users * heads, pages_per_user * block_size, head_dim));
+  EXT(paged_gather, cache, page_table, out, dtype, blocks, heads, block_size, head_dim, users, pages_per_user);
   return kernel();
 }
 EXPORT int ttm_chunk_causal_mask(void *mask, const int32_t *chunk_start, int64_t rows, int64_t cols, void *) {
-  SPAN("mask [rows, cols]", mask, tile_bytes(TTM_BF16, 1, rows, cols));
-  SPAN("chunk start", chunk_start, 4);
+  EXT(chunk_causal_mask, mask, chunk_start, rows, cols);
   return kernel();
 }

@@ -28,7 +28,7 @@ def _oracle_link():
 def null_env(tmp_path_factory):
     d = tmp_path_factory.mktemp("null_device")
     subprocess.run(["g++", "-std=c++17", "-O1", "-shared", "-fPIC", "-fvisibility=hidden", "-I", os.path.join(ROOT, "include"),
-                    "-o", str(d / "libttmlir_amd_hip.so"), os.path.join(ROOT, "tests", "cpp", "null_device.cpp")] + _oracle_link(), check=True)
+                    "-I", os.path.join(ROOT, "tt-mlir_amd", "csrc"), "-o", str(d / "libttmlir_amd_hip.so"), os.path.join(ROOT, "tests", "cpp", "null_device.cpp")] + _oracle_link(), check=True)
     env = dict(os.environ)
     # the runtime library finds the kernel library through its RUNPATH, which LD_LIBRARY_PATH precedes
     env["LD_LIBRARY_PATH"] = str(d) + os.pathsep + env.get("LD_LIBRARY_PATH", "")
@@ -351,7 +351,7 @@ def test_runtime_under_sanitizers_on_the_null_device(tmp_path, sanitizer):
     built with -fsanitize=thread (no data race, no deadlock) and with -fsanitize=address,undefined (no bad access, no
     undefined behaviour, no leak); every const-eval entry is evicted with its tensor."""
     rtsrc = os.path.join(ROOT, "tt-mlir_amd", "runtime")
-    inc = ["-I", os.path.join(ROOT, "include"), "-I", rtsrc]
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", rtsrc, "-I", os.path.join(ROOT, "tt-mlir_amd", "csrc")]
     common = ["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-pthread", "-fsanitize=" + sanitizer, "-fno-sanitize-recover=undefined"]
     jobs = [subprocess.Popen(common + inc + ["-c", os.path.join(rtsrc, f), "-o", str(tmp_path / (f + ".o"))])
             for f in sorted(os.listdir(rtsrc)) if f.endswith(".cpp")]
@@ -384,7 +384,7 @@ def test_damaged_programs_through_the_runtime_under_address_sanitizer(tmp_path):
         files.append(str(tmp_path / (name + ".ttnn")))
         open(files[-1], "wb").write(data)
     rtsrc = os.path.join(ROOT, "tt-mlir_amd", "runtime")
-    inc = ["-I", os.path.join(ROOT, "include"), "-I", rtsrc]
+    inc = ["-I", os.path.join(ROOT, "include"), "-I", rtsrc, "-I", os.path.join(ROOT, "tt-mlir_amd", "csrc")]
     common = ["g++", "-O1", "-g", "-std=c++17", "-fPIC", "-pthread", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined"]
     jobs = [subprocess.Popen(common + inc + ["-c", os.path.join(rtsrc, f), "-o", str(tmp_path / (f + ".o"))])
             for f in sorted(os.listdir(rtsrc)) if f.endswith(".cpp")]

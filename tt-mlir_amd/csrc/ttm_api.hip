@@ -28,6 +28,7 @@ static std::map<std::string, int> &opts() {
   static std::map<std::string, int> m = {
       {"tilize_variant", 0}, {"untilize_variant", 0}, {"pack_variant", 0}, {"unpack_variant", 0},
       {"rowwise_variant", 0}, {"sdpa_variant", 0}, {"linear_variant", 0}, {"linear_small_m_max", 64}, {"linear_ntw", 0}, {"linear_split_k", 0}, {"linear_two_part", 0}, {"linear_decode_split", 0}, {"linear_decode_variant", 0}, {"linear_two_pass", 0},
+      {"check_extents", getenv("TTMLIR_AMD_CHECK_EXTENTS") && getenv("TTMLIR_AMD_CHECK_EXTENTS")[0] == '1' ? 1 : 0},
   };
   return m;
 }
@@ -36,6 +37,26 @@ int ttm_option(const char *name) {
   auto it = opts().find(name);
   return it == opts().end() ? 0 : it->second;
 }
+// ---- operand extents
+bool ttm_check_extents_on() { return ttm_option("check_extents") != 0; }
+int TtmExtentChecker::operator()(const char *what, const void *p, int64_t bytes, bool optional) const {
+  (void)optional;
+  if (!p || bytes <= 0) return TTM_OK;   // a missing operand is the entry point's own argument check to report
+  hipDeviceptr_t base = nullptr;
+  size_t size = 0;
+  if (hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)p) != hipSuccess) {
+    (void)hipGetLastError();   // the failed lookup must not be reported by the next HIP call
+    return ttm_set_error(TTM_ERR_INVALID, "out of bounds: %s: %s (%p) is not device memory", fn, what, p);
+  }
+  const int64_t room = (int64_t)((const uint8_t *)base + size - (const uint8_t *)p);
+  if (bytes > room)
+    return ttm_set_error(TTM_ERR_INVALID,
+                         "out of bounds: %s: %s has %lld bytes behind it in its allocation, the kernels touch %lld (a TILE tensor [batch, R, C] is "
+                         "backed by batch * ceil(R / 32) * ceil(C / 32) whole tiles)",
+                         fn, what, (long long)room, (long long)bytes);
+  return TTM_OK;
+}
+
 TTM_EXPORT int ttm_set_option(const char *name, int value) {
   TTM_REQUIRE(name != nullptr, "ttm_set_option: null name");
   std::lock_guard<std::mutex> g(g_opt_mu);

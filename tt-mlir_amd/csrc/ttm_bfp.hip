@@ -362,10 +362,12 @@ static int run_bfp(const void *src, void *dst, int fmt, int dtype, int layout, i
 
 TTM_EXPORT int ttm_bfp_pack(const void *src, int src_dtype, int src_layout, void *dst, int fmt, int64_t batch,
                             int64_t rows, int64_t cols, void *stream) {
+  TTM_EXTENTS(bfp_pack, src, src_dtype, src_layout, dst, fmt, batch, rows, cols);
   return run_bfp<true>(src, dst, fmt, src_dtype, src_layout, batch, rows, cols, stream, "ttm_bfp_pack");
 }
 
 TTM_EXPORT int ttm_bfp_unpack(const void *src, int fmt, void *dst, int dst_dtype, int dst_layout, int64_t batch,
                               int64_t rows, int64_t cols, void *stream) {
+  TTM_EXTENTS(bfp_unpack, src, fmt, dst, dst_dtype, dst_layout, batch, rows, cols);
   return run_bfp<false>(src, dst, fmt, dst_dtype, dst_layout, batch, rows, cols, stream, "ttm_bfp_unpack");
 }

@@ -5,6 +5,7 @@
 #include <stdio.h>
 
 #include "ttmlir_amd_hip.h"
+#include "ttm_extents.h"
 
 // native clang vectors (usable with the nontemporal load/store builtins)
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -31,6 +32,38 @@ int ttm_set_error(int code, const char *fmt, ...) __attribute__((format(printf, 
 #define TTM_LAUNCH_CHECK() TTM_HIP(hipGetLastError())
 
 int ttm_option(const char *name);  // 0 when unset
+
+// Opt-in host-side check of operand extents (option "check_extents", or TTMLIR_AMD_CHECK_EXTENTS=1 in the environment):
+// before anything is launched, the bytes the kernels touch behind every pointer argument (ttm_extents.h) must lie inside
+// one device allocation (hipMemGetAddressRange); otherwise the entry point returns TTM_ERR_INVALID with the operand, the
+// bytes it has and the bytes the kernels touch in the message, where the launch would have been a GPU memory fault.
+bool ttm_check_extents_on();
+struct TtmExtentChecker {
+  const char *fn;
+  int operator()(const char *what, const void *p, int64_t bytes, bool optional) const;
+};
+#define TTM_EXTENTS(rule, ...)                                                                               \
+  do {                                                                                                       \
+    if (ttm_check_extents_on())                                                                              \
+      if (int rc_ = ttm_extents::rule(TtmExtentChecker{__func__}, __VA_ARGS__)) return rc_;                  \
+  } while (0)
+#define TTM_EXTENTS_SPAN(what, p, bytes)                                                                     \
+  do {                                                                                                       \
+    if (ttm_check_extents_on())                                                                              \
+      if (int rc_ = TtmExtentChecker{__func__}(what, p, bytes, false)) return rc_;                           \
+  } while (0)
+// source and destination of a strided view (ttm_copy_view); `extra` is the largest offset added to the destination base
+#define TTM_EXTENTS_VIEW(src, srows, scols, slay, dst, drows, dcols, dlay, elem, rank, extent, sstride, sbase, dstride, dbase, extra)     \
+  do {                                                                                                                                     \
+    if (ttm_check_extents_on()) {                                                                                                          \
+      bool neg_ = false;                                                                                                                   \
+      int rc_ = ttm_extents::view(TtmExtentChecker{__func__}, "source", src, srows, scols, slay, elem, rank, extent, sstride, sbase, 0, &neg_); \
+      if (!rc_ && !neg_)                                                                                                                   \
+        rc_ = ttm_extents::view(TtmExtentChecker{__func__}, "destination", dst, drows, dcols, dlay, elem, rank, extent, dstride, dbase, extra, &neg_); \
+      if (neg_) return ttm_set_error(TTM_ERR_INVALID, "out of bounds: %s: the view reaches a negative logical offset", __func__);          \
+      if (rc_) return rc_;                                                                                                                 \
+    }                                                                                                                                      \
+  } while (0)
 
 // Streaming kernels run fastest with a bounded number of bytes in flight per CU (64 - 96 KiB measured on MI355X): more
 // resident wavefronts than that only lengthen the queues in front of the memory channels.  TTM_MAX_WAVES(n) caps a

@@ -275,6 +275,8 @@ TTM_EXPORT int ttm_copy_view(const void *src, int64_t src_rows, int64_t src_cols
                              int64_t dst_rows, int64_t dst_cols, int dst_layout, int elem_bytes, int rank,
                              const int64_t *extent, const int64_t *src_stride, int64_t src_base,
                              const int64_t *dst_stride, int64_t dst_base, void *stream) {
+  if (rank >= 0 && rank <= 8 && (rank == 0 || (extent && src_stride && dst_stride)))
+    TTM_EXTENTS_VIEW(src, src_rows, src_cols, src_layout, dst, dst_rows, dst_cols, dst_layout, elem_bytes, rank, extent, src_stride, src_base, dst_stride, dst_base, 0);
   return copy_view_entry(src, src_rows, src_cols, src_layout, dst, dst_rows, dst_cols, dst_layout, elem_bytes, rank, extent, src_stride,
                          src_base, dst_stride, dst_base, nullptr, 0, 0, stream);
 }
@@ -284,6 +286,11 @@ TTM_EXPORT int ttm_copy_view_at(const void *src, int64_t src_rows, int64_t src_c
                                 const int64_t *extent, const int64_t *src_stride, int64_t src_base,
                                 const int64_t *dst_stride, int64_t dst_base, const int32_t *index, int64_t index_stride,
                                 int64_t index_limit, void *stream) {
+  if (rank >= 0 && rank <= 8 && (rank == 0 || (extent && src_stride && dst_stride))) {
+    TTM_EXTENTS_SPAN("index", index, 4);
+    TTM_EXTENTS_VIEW(src, src_rows, src_cols, src_layout, dst, dst_rows, dst_cols, dst_layout, elem_bytes, rank, extent, src_stride, src_base, dst_stride, dst_base,
+                     index_limit > 0 ? (index_limit - 1) * index_stride : 0);
+  }
   TTM_REQUIRE(index, "ttm_copy_view_at: null index pointer");
   return copy_view_entry(src, src_rows, src_cols, src_layout, dst, dst_rows, dst_cols, dst_layout, elem_bytes, rank, extent, src_stride,
                          src_base, dst_stride, dst_base, index, index_stride, index_limit, stream);

@@ -611,18 +611,21 @@ static int rotary_entry(const void *x, const void *cos_cache, const void *sin_ca
 TTM_EXPORT int ttm_rotary_embedding(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype,
                                     int64_t batch, int64_t rows, int64_t cols, int64_t cache_rows, int64_t token_index,
                                     void *stream) {
+  TTM_EXTENTS(rotary_embedding, x, cos_cache, sin_cache, out, dtype, batch, rows, cols, cache_rows);
   return rotary_entry(x, cos_cache, sin_cache, out, dtype, batch, rows, cols, cache_rows, token_index, false, stream);
 }
 
 TTM_EXPORT int ttm_rotary_embedding_split_heads(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype,
                                                 int64_t batch, int64_t heads, int64_t head_dim, int64_t cache_rows,
                                                 int64_t token_index, void *stream) {
+  TTM_EXTENTS(rotary_embedding_split_heads, x, cos_cache, sin_cache, out, dtype, batch, heads, head_dim, cache_rows);
   return rotary_entry(x, cos_cache, sin_cache, out, dtype, batch, heads, head_dim, cache_rows, token_index, true, stream);
 }
 
 TTM_EXPORT int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users,
                                 int64_t heads, int64_t max_seq, int64_t head_dim, int64_t input_users, int64_t batch_offset,
                                 void *stream) {
+  TTM_EXTENTS(update_cache, cache, input, update_index, dtype, users, heads, max_seq, head_dim, input_users);
   TTM_REQUIRE(cache && input && update_index, "ttm_update_cache: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_update_cache: dtype must be BFloat16 or Float32");
   TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_update_cache: head dim must be a positive multiple of 32");
@@ -646,6 +649,7 @@ TTM_EXPORT int ttm_update_cache(void *cache, const void *input, const int32_t *u
 
 TTM_EXPORT int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t users, int64_t heads, int64_t max_seq,
                               int64_t head_dim, int64_t seq, int64_t batch_offset, void *stream) {
+  TTM_EXTENTS(fill_cache, cache, input, dtype, users, heads, max_seq, head_dim, seq);
   TTM_REQUIRE(cache && input, "ttm_fill_cache: null pointer");
   const int eb = ttm_dtype_bytes(dtype);
   TTM_REQUIRE(eb == 2 || eb == 4, "ttm_fill_cache: element size must be 2 or 4 bytes");
@@ -665,6 +669,7 @@ TTM_EXPORT int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t
 TTM_EXPORT int ttm_paged_update_cache(void *cache, const void *input, const int32_t *update_index, const int32_t *page_table,
                                       int dtype, int64_t blocks, int64_t heads, int64_t block_size, int64_t head_dim, int64_t users,
                                       int64_t pages_per_user, int share_cache, void *stream) {
+  TTM_EXTENTS(paged_update_cache, cache, input, update_index, page_table, dtype, blocks, heads, block_size, head_dim, users, pages_per_user);
   TTM_REQUIRE(cache && input && update_index, "ttm_paged_update_cache: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_paged_update_cache: dtype must be BFloat16 or Float32");
   TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_paged_update_cache: head dim must be a positive multiple of 32");
@@ -689,6 +694,7 @@ TTM_EXPORT int ttm_paged_update_cache(void *cache, const void *input, const int3
 TTM_EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_t *page_table, const int32_t *batch_idx, int dtype,
                                     int64_t blocks, int64_t heads, int64_t block_size, int64_t head_dim, int64_t in_batch, int64_t seq,
                                     int64_t table_rows, int64_t pages_per_user, void *stream) {
+  TTM_EXTENTS(paged_fill_cache, cache, input, page_table, batch_idx, dtype, blocks, heads, block_size, head_dim, in_batch, seq, table_rows, pages_per_user);
   TTM_REQUIRE(cache && input && page_table, "ttm_paged_fill_cache: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_paged_fill_cache: dtype must be BFloat16 or Float32");
   TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_paged_fill_cache: head dim must be a positive multiple of 32");
@@ -805,6 +811,7 @@ TTM_EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, cons
                                int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks,
                                void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim,
                                int is_causal, float scale, void *stream) {
+  TTM_EXTENTS(sdpa_decode, q, k, v, cur_pos, mask, mask_heads, batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads, seq, head_dim, 0, nullptr);
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, 0, -1, nullptr, batch, false, stream);
 }
@@ -813,6 +820,7 @@ TTM_EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const 
                                             int mask_heads, const int32_t *page_table, int64_t pages_per_user, int64_t page_block,
                                             int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads,
                                             int64_t seq, int64_t head_dim, int is_causal, float scale, void *stream) {
+  TTM_EXTENTS(sdpa_decode, q, k, v, cur_pos, mask, mask_heads, batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads, seq, head_dim, 1, nullptr);
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, 1, -1, nullptr, batch, false, stream);
 }
@@ -822,6 +830,7 @@ TTM_EXPORT int ttm_sdpa_decode_windowed(const void *q, const void *k, const void
                                         int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads,
                                         int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                                         const void *attention_sink, void *stream) {
+  TTM_EXTENTS(sdpa_decode, q, k, v, cur_pos, mask, mask_heads, mask_batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads, seq, head_dim, concat_heads, attention_sink);
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, false, stream);
 }
@@ -832,12 +841,14 @@ TTM_EXPORT int ttm_sdpa_decode_static(const void *q, const void *k, const void *
                                       int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads, int64_t kv_heads,
                                       int64_t seq, int64_t head_dim, int is_causal, float scale, int concat_heads, int64_t sliding_window,
                                       const void *attention_sink, void *stream) {
+  TTM_EXTENTS(sdpa_decode, q, k, v, cur_pos, mask, mask_heads, mask_batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads, seq, head_dim, concat_heads, attention_sink);
   return sdpa_decode_entry(q, k, v, cur_pos, mask, mask_heads, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads, kv_heads,
                            seq, head_dim, is_causal, scale, concat_heads != 0, sliding_window, attention_sink, mask_batch, true, stream);
 }
 
 TTM_EXPORT int ttm_paged_gather(const void *cache, const int32_t *page_table, void *out, int dtype, int64_t blocks, int64_t heads,
                                 int64_t block_size, int64_t head_dim, int64_t users, int64_t pages_per_user, void *stream) {
+  TTM_EXTENTS(paged_gather, cache, page_table, out, dtype, blocks, heads, block_size, head_dim, users, pages_per_user);
   TTM_REQUIRE(cache && page_table && out, "ttm_paged_gather: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_paged_gather: dtype must be BFloat16 or Float32");
   TTM_REQUIRE(head_dim > 0 && head_dim % 32 == 0, "ttm_paged_gather: head dim must be a positive multiple of 32");
@@ -857,6 +868,7 @@ TTM_EXPORT int ttm_paged_gather(const void *cache, const int32_t *page_table, vo
 }
 
 TTM_EXPORT int ttm_chunk_causal_mask(void *mask, const int32_t *chunk_start, int64_t rows, int64_t cols, void *stream) {
+  TTM_EXTENTS(chunk_causal_mask, mask, chunk_start, rows, cols);
   TTM_REQUIRE(mask && chunk_start, "ttm_chunk_causal_mask: null pointer");
   TTM_REQUIRE(rows > 0 && cols > 0, "ttm_chunk_causal_mask: bad extents");
   const int64_t rp = ttm_round_up32(rows), cp = ttm_round_up32(cols), total8 = rp * cp / 8;
@@ -869,6 +881,7 @@ TTM_EXPORT int ttm_chunk_causal_mask(void *mask, const int32_t *chunk_start, int
 TTM_EXPORT int ttm_rotary_embedding_llama(const void *x, const void *cos_cache, const void *sin_cache, const void *trans_mat, void *out,
                                           int dtype, int64_t batch, int64_t rows, int64_t cols, int64_t cs_batch, int64_t cs_rows,
                                           void *stream) {
+  TTM_EXTENTS(rotary_embedding_llama, x, cos_cache, sin_cache, trans_mat, out, dtype, batch, rows, cols, cs_batch, cs_rows);
   TTM_REQUIRE(x && cos_cache && sin_cache && trans_mat && out, "ttm_rotary_embedding_llama: null pointer");
   TTM_REQUIRE(dtype == TTM_BF16, "ttm_rotary_embedding_llama: tensors must be BFloat16");
   TTM_REQUIRE(batch >= 0 && rows > 0 && cols > 0 && cols % 32 == 0 && cols <= 256,

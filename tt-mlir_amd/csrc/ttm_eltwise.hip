@@ -266,12 +266,14 @@ static int unary_entry(int op, const void *in, void *out, int dtype, int layout,
 
 TTM_EXPORT int ttm_eltwise_unary(int op, const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows,
                                  int64_t cols, float param, void *stream) {
+  TTM_EXTENTS(unary, in, out, dtype, layout, batch, rows, cols);
   TTM_REQUIRE(op != U_CLAMP, "ttm_eltwise_unary: clamp takes two bounds, use ttm_clamp");
   return unary_entry(op, in, out, dtype, layout, batch, rows, cols, param, 0.0f, stream);
 }
 
 TTM_EXPORT int ttm_clamp(const void *in, void *out, int dtype, int layout, int64_t batch, int64_t rows, int64_t cols, float lo, float hi,
                          void *stream) {
+  TTM_EXTENTS(unary, in, out, dtype, layout, batch, rows, cols);
   return unary_entry(U_CLAMP, in, out, dtype, layout, batch, rows, cols, lo, hi, stream);
 }
 
@@ -432,6 +434,7 @@ static bool chunkable(const int64_t (&oshape)[4], int tiled, int es, std::initia
 
 TTM_EXPORT int ttm_eltwise_binary(int op, const void *a, const int64_t *a_shape, const void *b, const int64_t *b_shape,
                                   void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream) {
+  if (rank >= 0 && rank <= 8 && a_shape && b_shape && out_shape) TTM_EXTENTS(binary, a, a_shape, b, b_shape, out, out_shape, rank, dtype, layout);
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_eltwise_binary: dtype must be BFloat16 or Float32 (got %d)", dtype);
   TTM_REQUIRE(layout == TTM_ROW_MAJOR || layout == TTM_TILE, "ttm_eltwise_binary: bad layout");
   TTM_REQUIRE(rank >= 0 && rank <= 8 && a_shape && b_shape && out_shape, "ttm_eltwise_binary: bad rank or null shape");
@@ -556,6 +559,8 @@ __global__ __launch_bounds__(256) void ttm_where_chunk_k(const void *__restrict_
 
 TTM_EXPORT int ttm_where(const void *cond, const int64_t *cond_shape, const void *a, const int64_t *a_shape, const void *b,
                          const int64_t *b_shape, void *out, const int64_t *out_shape, int rank, int dtype, int layout, void *stream) {
+  if (rank >= 0 && rank <= 4 && cond_shape && a_shape && b_shape && out_shape)
+    TTM_EXTENTS(where, cond, cond_shape, a, a_shape, b, b_shape, out, out_shape, rank, dtype, layout);
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_where: dtype must be BFloat16 or Float32 (got %d)", dtype);
   TTM_REQUIRE(layout == TTM_ROW_MAJOR || layout == TTM_TILE, "ttm_where: bad layout");
   TTM_REQUIRE(rank >= 0 && rank <= 4 && cond_shape && a_shape && b_shape && out_shape, "ttm_where: rank must be at most 4, shapes non-null");
@@ -661,6 +666,7 @@ static cast_fn pick_cast_dst(int dst) {
 }
 
 TTM_EXPORT int ttm_typecast(const void *in, int src_dtype, void *out, int dst_dtype, int64_t n, void *stream) {
+  TTM_EXTENTS(typecast, in, src_dtype, out, dst_dtype, n);
   TTM_REQUIRE(n >= 0, "ttm_typecast: negative size");
   cast_fn fn = nullptr;
   switch (src_dtype) {

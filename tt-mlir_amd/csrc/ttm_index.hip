@@ -161,6 +161,7 @@ unsigned grid_of(int64_t items) {
 
 TTM_EXPORT int ttm_embedding(const void *indices, int index_dtype, const void *weight, void *out, int elem_bytes, int64_t rows,
                              int64_t vocab, int64_t dim, void *stream) {
+  TTM_EXTENTS(embedding, indices, weight, out, elem_bytes, rows, vocab, dim);
   TTM_REQUIRE(index_dtype == TTM_I32 || index_dtype == TTM_U32, "ttm_embedding: indices must be Int32 or UInt32 (got %d)", index_dtype);
   TTM_REQUIRE(elem_bytes == 2 || elem_bytes == 4, "ttm_embedding: element size must be 2 or 4 bytes");
   TTM_REQUIRE(rows >= 0 && vocab > 0 && dim > 0, "ttm_embedding: bad extents");
@@ -184,6 +185,7 @@ TTM_EXPORT int ttm_embedding(const void *indices, int index_dtype, const void *w
 }
 
 TTM_EXPORT int ttm_argmax(const void *in, int dtype, int32_t *out, int64_t rows, int64_t cols, void *stream) {
+  TTM_EXTENTS(argmax, in, dtype, out, rows, cols);
   TTM_REQUIRE(dtype == TTM_BF16 || dtype == TTM_F32, "ttm_argmax: dtype must be BFloat16 or Float32 (got %d)", dtype);
   TTM_REQUIRE(rows >= 0 && cols > 0 && cols <= INT32_MAX, "ttm_argmax: bad extents");
   if (rows == 0) return TTM_OK;
@@ -224,6 +226,7 @@ TTM_EXPORT int ttm_argmax(const void *in, int dtype, int32_t *out, int64_t rows,
 }
 
 TTM_EXPORT int ttm_arange(void *out, int dtype, int64_t n, double start, double step, void *stream) {
+  TTM_EXTENTS(arange, out, dtype, n);
   TTM_REQUIRE(n >= 0, "ttm_arange: negative length");
   if (n == 0) return TTM_OK;
   TTM_REQUIRE(out != nullptr, "ttm_arange: null pointer");

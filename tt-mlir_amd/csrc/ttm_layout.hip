@@ -31,6 +31,7 @@ __global__ __launch_bounds__(256) TTM_MAX_WAVES(5) void ttm_copy_kernel_k(const 
 }
 
 TTM_EXPORT int ttm_copy_kernel(const void *src, void *dst, size_t bytes, void *stream) {
+  TTM_EXTENTS(copy_kernel, src, dst, bytes);
   if (bytes == 0) return TTM_OK;
   TTM_REQUIRE(src && dst, "ttm_copy_kernel: null pointer");
   TTM_REQUIRE(bytes % 16 == 0 && ((uintptr_t)src & 15) == 0 && ((uintptr_t)dst & 15) == 0,
@@ -312,10 +313,12 @@ static int run_layout(const void *src, void *dst, int64_t batch, int64_t rows, i
 
 TTM_EXPORT int ttm_tilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols,
                           int elem_bytes, void *stream) {
+  TTM_EXTENTS(tilize, src, dst, batch, rows, cols, elem_bytes);
   return run_layout<true>(src, dst, batch, rows, cols, elem_bytes, stream, "ttm_tilize");
 }
 
 TTM_EXPORT int ttm_untilize(const void *src, void *dst, int64_t batch, int64_t rows, int64_t cols,
                             int elem_bytes, void *stream) {
+  TTM_EXTENTS(untilize, src, dst, batch, rows, cols, elem_bytes);
   return run_layout<false>(src, dst, batch, rows, cols, elem_bytes, stream, "ttm_untilize");
 }

@@ -1907,6 +1907,7 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
 TTM_EXPORT int ttm_linear(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias,
                           int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch,
                           int64_t w_batch, int64_t M, int64_t N, int64_t K, int act, void *stream) {
+  TTM_EXTENTS(linear, a, a_dtype, w, w_dtype, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, TTM_TAIL_NONE, nullptr);
   return ttm_linear_tail(a, a_dtype, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, act,
                          TTM_TAIL_NONE, nullptr, stream);
 }
@@ -1971,6 +1972,7 @@ static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, 
 TTM_EXPORT int ttm_linear_tail(const void *a, int a_dtype, const void *w, int w_dtype, int transpose_w, const void *bias,
                                int bias_dtype, int bias_layout, void *out, int out_dtype, int64_t batch, int64_t w_batch,
                                int64_t M, int64_t N, int64_t K, int act, int tail_op, const void *tail, void *stream) {
+  TTM_EXTENTS(linear, a, a_dtype, w, w_dtype, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, tail_op, tail);
   return linear_entry(a, a_dtype, w, w_dtype, transpose_w, bias, bias_dtype, bias_layout, out, out_dtype, batch, w_batch, M, N, K, act,
                       tail_op, tail, nullptr, stream);
 }
@@ -1983,6 +1985,7 @@ TTM_EXPORT int ttm_linear_add_rms_norm_supported(int w_dtype, int64_t M, int64_t
 TTM_EXPORT int ttm_linear_add_rms_norm(const void *a, const void *w, int w_dtype, const void *residual, void *sum_out, const void *norm_weight,
                                        int weight_layout, const void *norm_bias, int bias_layout, float eps, void *norm_out, int64_t M,
                                        int64_t N, int64_t K, void *stream) {
+  TTM_EXTENTS(linear_add_rms_norm, a, w, w_dtype, residual, sum_out, norm_weight, weight_layout, norm_bias, bias_layout, norm_out, M, N, K);
   TTM_REQUIRE(ttm_linear_add_rms_norm_supported(w_dtype, M, N, K),
               "ttm_linear_add_rms_norm: needs block-float weights, 1..32 rows and at most 16384 columns");
   TTM_REQUIRE(residual && sum_out && norm_out, "ttm_linear_add_rms_norm: null pointer");
@@ -1995,6 +1998,7 @@ TTM_EXPORT int ttm_linear_add_rms_norm(const void *a, const void *w, int w_dtype
 
 TTM_EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M,
                                int64_t N, int64_t K, void *stream) {
+  TTM_EXTENTS(linear_pair, a, w0, w1, w_dtype, out0, out1, M, N, K);
   TTM_REQUIRE(w0 && w1 && out0 && out1 && w0 != w1 && out0 != out1, "ttm_linear_pair: two distinct weight and output tensors are needed");
   TTM_REQUIRE((((uintptr_t)w1 | (uintptr_t)out1) & 15) == 0, "ttm_linear_pair: operands must be 16-byte aligned");
   const int64_t strides[3] = {0, (const uint8_t *)w1 - (const uint8_t *)w0, (uint8_t *)out1 - (uint8_t *)out0};
@@ -2048,6 +2052,7 @@ static int linear_group_entry(const void *a, int n, const void *const *w, int w_
 
 TTM_EXPORT int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N,
                                 const int *act, int64_t M, int64_t K, void *stream) {
+  if (n >= 1 && n <= 4 && w && out && N) TTM_EXTENTS(linear_group, a, n, w, w_dtype, out, N, M, K);
   return linear_group_entry(a, n, w, w_dtype, out, N, act, M, K, nullptr, stream);
 }
 
@@ -2063,6 +2068,7 @@ TTM_EXPORT int ttm_linear_qkv_decode(const void *a, const void *wq, const void *
                                      int64_t cache_rows, int64_t token_index, void *q_out, void *k_cache, void *v_cache,
                                      int64_t cache_users, int64_t max_seq, const int32_t *update_index, int64_t batch_offset,
                                      void *stream) {
+  TTM_EXTENTS(linear_qkv_decode, a, wq, wk, wv, w_dtype, users, K, heads, kv_heads, head_dim, cos_cache, sin_cache, cache_rows, q_out, k_cache, v_cache, cache_users, max_seq, update_index);
   TTM_REQUIRE(ttm_linear_qkv_decode_supported(w_dtype, users, K, heads, kv_heads, head_dim),
               "ttm_linear_qkv_decode: needs block-float weights, 1..32 users and a head_dim that is a multiple of 32");
   TTM_REQUIRE(a && wq && wk && wv && cos_cache && sin_cache && q_out && k_cache && v_cache && update_index, "ttm_linear_qkv_decode: null pointer");

@@ -925,6 +925,7 @@ int ttm_rowwise_rmsnorm_from_partials(const float *partial, int slices, int64_t 
 
 TTM_EXPORT int ttm_rms_norm(const void *x, const void *weight, int weight_layout, const void *bias, int bias_layout,
                             void *out, int dtype, int64_t batch, int64_t rows, int64_t cols, float eps, void *stream) {
+  TTM_EXTENTS(rms_norm, x, weight, weight_layout, bias, bias_layout, out, dtype, batch, rows, cols);
   if (batch == 0 || rows == 0 || cols == 0) return TTM_OK;
   RowArgs p;
   int rc = fill_args(p, x, out, dtype, batch, rows, cols, "ttm_rms_norm");
@@ -936,6 +937,7 @@ TTM_EXPORT int ttm_rms_norm(const void *x, const void *weight, int weight_layout
 
 TTM_EXPORT int ttm_softmax_lastdim(const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols,
                                    void *stream) {
+  TTM_EXTENTS(softmax, x, out, dtype, batch, rows, cols);
   if (batch == 0 || rows == 0 || cols == 0) return TTM_OK;
   RowArgs p;
   int rc = fill_args(p, x, out, dtype, batch, rows, cols, "ttm_softmax_lastdim");
@@ -945,6 +947,7 @@ TTM_EXPORT int ttm_softmax_lastdim(const void *x, void *out, int dtype, int64_t 
 
 TTM_EXPORT int ttm_reduce_lastdim(int op, const void *x, void *out, int dtype, int64_t batch, int64_t rows, int64_t cols,
                                   void *stream) {
+  TTM_EXTENTS(reduce, x, out, dtype, batch, rows, cols);
   TTM_REQUIRE(op >= 0 && op <= 3, "ttm_reduce_lastdim: op must be Sum(0), Mean(1), Max(2) or Min(3), got %d", op);
   if (batch == 0 || rows == 0 || cols == 0) return TTM_OK;
   RowArgs p;

@@ -838,12 +838,14 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
 TTM_EXPORT int ttm_sdpa(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
                         int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                         int is_causal, float scale, void *stream) {
+  TTM_EXTENTS(sdpa, q, k, v, mask, mask_heads, B, out, dtype, B, Hq, Hkv, Sq, Sk, D, nullptr);
   return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, 0, -1, nullptr, B, stream);
 }
 
 TTM_EXPORT int ttm_sdpa_heads_inner(const void *q, const void *k, const void *v, const void *mask, int mask_heads, void *out,
                                     int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                                     int is_causal, float scale, int heads_inner, void *stream) {
+  TTM_EXTENTS(sdpa, q, k, v, mask, mask_heads, B, out, dtype, B, Hq, Hkv, Sq, Sk, D, nullptr);
   return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner, -1, nullptr, B, stream);
 }
 
@@ -851,6 +853,7 @@ TTM_EXPORT int ttm_sdpa_windowed(const void *q, const void *k, const void *v, co
                                  int dtype, int64_t B, int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D,
                                  int is_causal, float scale, int heads_inner, int64_t sliding_window, const void *attention_sink,
                                  void *stream) {
+  TTM_EXTENTS(sdpa, q, k, v, mask, mask_heads, mask_batch, out, dtype, B, Hq, Hkv, Sq, Sk, D, attention_sink);
   return sdpa_entry(q, k, v, mask, mask_heads, out, dtype, B, Hq, Hkv, Sq, Sk, D, is_causal, scale, heads_inner,
                     sliding_window < 0 ? -1 : sliding_window, attention_sink, mask_batch, stream);
 }

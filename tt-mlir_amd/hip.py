@@ -151,6 +151,9 @@ def check_buffers(on=True):
     of any call whose buffers were sized by hand."""
     global _check_buffers
     _check_buffers = bool(on)
+    # the library's own check covers every entry point (the rules above cover the common ones, against the tensor's size,
+    # which is tighter than the allocation the library can see)
+    set_option("check_extents", 1 if on else 0)
 
 
 def _verify_extents(name, args):
@@ -160,7 +163,7 @@ def _verify_extents(name, args):
     try:
         extents = spec(args)
     except (KeyError, IndexError, TypeError):
-        return   # arguments the size rules do not cover (an unknown dtype code, a short argument list): the library answers
+        return   # arguments the size rules do not cover (an unknown dtype code, a short argument list): the library answers, with its own extent check
     for idx, need, what in extents:
         p = args[idx]
         if isinstance(p, _Ptr) and p.nbytes is not None and p.nbytes < need:
