@@ -1,14 +1,12 @@
-// A device in host memory that checks everything and computes the common ops: a stand-in for libttmlir_amd_hip.so on a
+// A device in host memory that checks everything and computes on the host: a stand-in for libttmlir_amd_hip.so on a
 // machine without a GPU, built by the tests (g++ -shared, linked against the CPU oracle) and put in front of the real library
 // with LD_LIBRARY_PATH.  "Device memory" is zeroed host memory with a registry of the live allocations; copies are memcpy;
 // streams are dummies.  Every kernel entry point first holds each pointer argument against the registry: the pointer must
 // lie in a live allocation and have behind it the bytes the real kernels touch (include/ttmlir_amd_hip.h: a tile tensor is
 // backed by its whole padded extent).  A violation is an error return with a message, which the runtime turns into an
 // exception - on the GPU the same call would be a memory fault.
-// Layout conversion, block-float packing, typecasts, copies and views, matmul / linear in all their forms, element-wise ops,
-// RMSNorm, softmax, reductions, embedding, argmax, arange and prefill attention then compute their result on the host with
-// the oracle's arithmetic (f32, one rounding to the output type), so programs made of them give the values the oracle gives;
-// the decode-path kernels leave their outputs as they are.  A "launch" is a closure: between ttm_graph_begin_capture and
+// Every entry point then computes its result on the host with the oracle's arithmetic (f32, one rounding to the output
+// type), so programs give the values the oracle gives.  A "launch" is a closure: between ttm_graph_begin_capture and
 // ttm_graph_end_capture closures are recorded instead of run, as a capturing HIP stream records kernels, and
 // ttm_graph_launch runs the recorded closures against whatever the recorded addresses hold by then.  With this the host
 // runtime (executor, tensor pool, caches, fused launches, traces) runs whole programs on the CPU with checkable values.
@@ -116,6 +114,10 @@ void orc_linear_f32(const float *A, const float *B, const float *bias, float *C,
 void orc_rmsnorm_f32(const float *x, const float *w, const float *b, float *out, int64_t rows, int64_t cols, float eps);
 void orc_softmax_f32(const float *x, float *out, int64_t outer, int64_t dim, int64_t inner);
 void orc_reduce_f32(int op, const float *x, float *out, int64_t outer, int64_t dim, int64_t inner);
+void orc_rotary_embedding_f32(const float *x, const float *cosc, const float *sinc, float *out, int64_t batch, int64_t rows, int64_t D,
+                              int64_t token_index);
+void orc_sdpa_decode_f32(const float *q, const float *k, const float *v, const int32_t *cur_pos, const float *mask, int mask_heads, float *out,
+                         int64_t B, int64_t H, int64_t Hkv, int64_t S, int64_t D, int is_causal, float scale, int64_t window, const float *sink);
 void orc_sdpa_f32(const float *q, const float *k, const float *v, const float *mask, int mask_heads, float *out, int64_t B,
                   int64_t Hq, int64_t Hkv, int64_t Sq, int64_t Sk, int64_t D, int is_causal, float scale, int64_t window,
                   const float *sink);
@@ -439,7 +441,28 @@ EXPORT int ttm_linear_qkv_decode(const void *a, const void *wq, const void *wk, 
   if (batch_offset < 0 || batch_offset + users > cache_users) return fail("ttm_linear_qkv_decode: batch_offset + users exceeds the cache");
   EXT(linear_qkv_decode, a, wq, wk, wv, w_dtype, users, K, heads, kv_heads, head_dim, cos_cache, sin_cache, cache_rows, q_out, k_cache, v_cache,
       cache_users, max_seq, update_index);
-  return kernel();
+  return launch([=] {
+    // the op sequence it replaces: three projections rounded to bf16, rotary embedding of q and k at row token_index, q as
+    // [1, users, heads, head_dim] with zeroed padding rows, k and v rows into the caches at *update_index
+    const int64_t D = head_dim, nq = heads * D, nk = kv_heads * D;
+    Dense Q = linear_host(a, wq, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, users, nq, K, TTM_ACT_NONE, TTM_TAIL_NONE, nullptr);
+    Dense Kp = linear_host(a, wk, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, users, nk, K, TTM_ACT_NONE, TTM_TAIL_NONE, nullptr);
+    Dense Vp = linear_host(a, wv, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, users, nk, K, TTM_ACT_NONE, TTM_TAIL_NONE, nullptr);
+    Dense C = load_dense(cos_cache, TTM_BF16, TTM_TILE, 1, cache_rows, D), S_ = load_dense(sin_cache, TTM_BF16, TTM_TILE, 1, cache_rows, D);
+    Dense Qr(Q.size()), Kr(Kp.size());
+    orc_rotary_embedding_f32(Q.data(), C.data(), S_.data(), Qr.data(), 1, users * heads, D, token_index);
+    orc_rotary_embedding_f32(Kp.data(), C.data(), S_.data(), Kr.data(), 1, users * kv_heads, D, token_index);
+    store_dense(Qr, q_out, TTM_BF16, TTM_TILE, users, heads, D);
+    const int64_t at = *update_index;
+    if (at < 0 || at >= max_seq) return;
+    for (int64_t u = 0; u < users; ++u)
+      for (int64_t h = 0; h < kv_heads; ++h)
+        for (int64_t d = 0; d < D; ++d) {
+          const int64_t off = elem_off(TTM_TILE, max_seq, D, (batch_offset + u) * kv_heads + h, at, d);
+          store_scalar(k_cache, TTM_BF16, off, Kr[(size_t)((u * kv_heads + h) * D + d)]);
+          store_scalar(v_cache, TTM_BF16, off, Vp[(size_t)((u * kv_heads + h) * D + d)]);
+        }
+  });
 }
 
 // ---- element-wise
@@ -651,38 +674,87 @@ EXPORT int ttm_sdpa_windowed(const void *q, const void *k, const void *v, const 
 }
 static int decode_check(const char *fn, const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
                         int64_t mask_batch, const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
-                        int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int concat_heads, const void *sink) {
+                        int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int concat_heads, const void *sink,
+                        int is_causal = 0, float scale = 0.0f, int64_t window = -1) {
   if (batch * heads * head_dim == 0) return TTM_OK;
   if (int rc = ttm_extents::sdpa_decode(Chk{fn}, q, k, v, cur_pos, mask, mask_heads, mask_batch, page_table, pages_per_user, page_block, page_blocks, out,
                                         dtype, batch, heads, kv_heads, seq, head_dim, concat_heads, sink))
     return rc;
-  return kernel();
+  if (kv_heads < 1 || heads % kv_heads != 0) return fail("%s: query heads must be a multiple of kv heads", fn);
+  return launch([=] {
+    const int64_t B = batch, H = heads, Hk = kv_heads, S = seq, D = head_dim;
+    Dense Q = load_dense(q, dtype, TTM_TILE, B, H, D), K((size_t)(B * Hk * S * D)), V(K.size()), O(Q.size());
+    // the keys a user sees, as an additive mask: the caller's mask, the keys past cur_pos (the kernels apply both) and the
+    // positions whose page-table entry names no page
+    const int mh = mask ? mask_heads : 1;
+    Dense M((size_t)(B * mh * S), 0.0f);
+    if (mask) {
+      Dense m = load_dense(mask, dtype, TTM_TILE, mask_batch, mask_heads, S);
+      for (int64_t b = 0; b < B; ++b)
+        for (int64_t i = 0; i < mh * S; ++i) M[(size_t)(b * mh * S + i)] = m[(size_t)((mask_batch == 1 ? 0 : b) * mh * S + i)];
+    }
+    if (page_table) {
+      Dense PK = load_dense(k, dtype, TTM_TILE, page_blocks * Hk, page_block, D), PV = load_dense(v, dtype, TTM_TILE, page_blocks * Hk, page_block, D);
+      for (int64_t b = 0; b < B; ++b)
+        for (int64_t j = 0; j < S; ++j) {
+          const int64_t page = page_table[b * pages_per_user + j / page_block];
+          const bool ok = page >= 0 && page < page_blocks;
+          for (int64_t h = 0; h < Hk; ++h)
+            for (int64_t d = 0; d < D; ++d) {
+              const size_t to = (size_t)(((b * Hk + h) * S + j) * D + d), from = (size_t)((((ok ? page : 0) * Hk + h) * page_block + j % page_block) * D + d);
+              K[to] = ok ? PK[from] : 0.0f;
+              V[to] = ok ? PV[from] : 0.0f;
+            }
+          if (!ok)
+            for (int64_t hh = 0; hh < mh; ++hh) M[(size_t)((b * mh + hh) * S + j)] = -INFINITY;
+        }
+    } else {
+      K = load_dense(k, dtype, TTM_TILE, B * Hk, S, D);
+      V = load_dense(v, dtype, TTM_TILE, B * Hk, S, D);
+    }
+    if (is_causal && cur_pos)
+      for (int64_t b = 0; b < B; ++b)
+        for (int64_t hh = 0; hh < mh; ++hh)
+          for (int64_t j = cur_pos[b] + 1; j < S; ++j)
+            if (j >= 0) M[(size_t)((b * mh + hh) * S + j)] = -INFINITY;
+    for (Dense *t : {&K, &V})
+      for (float &f : *t) f = f != f ? 0.0f : f;   // rows past the position may hold anything: their weight is exactly zero
+    Dense sk;
+    if (sink) {
+      Dense t = load_dense(sink, TTM_BF16, TTM_TILE, 1, H, 32);
+      for (int64_t h = 0; h < H; ++h) sk.push_back(t[(size_t)(h * 32)]);
+    }
+    orc_sdpa_decode_f32(Q.data(), K.data(), V.data(), cur_pos, M.data(), mh, O.data(), B, H, Hk, S, D, is_causal, scale, window < 0 ? -1 : window,
+                        sink ? sk.data() : nullptr);
+    if (concat_heads) store_dense(O, out, dtype, TTM_TILE, 1, B, H * D);
+    else store_dense(O, out, dtype, TTM_TILE, B, H, D);
+  });
 }
 EXPORT int ttm_sdpa_decode(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads, const int32_t *page_table,
                            int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype, int64_t batch, int64_t heads,
-                           int64_t kv_heads, int64_t seq, int64_t head_dim, int, float, void *) {
+                           int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale, void *) {
   return decode_check(__func__, q, k, v, cur_pos, mask, mask_heads, batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads,
-                      kv_heads, seq, head_dim, 0, nullptr);
+                      kv_heads, seq, head_dim, 0, nullptr, is_causal, scale);
 }
 EXPORT int ttm_sdpa_decode_concat_heads(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads,
                                         const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
-                                        int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int, float, void *) {
+                                        int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale, void *) {
   return decode_check(__func__, q, k, v, cur_pos, mask, mask_heads, batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch, heads,
-                      kv_heads, seq, head_dim, 1, nullptr);
+                      kv_heads, seq, head_dim, 1, nullptr, is_causal, scale);
 }
 EXPORT int ttm_sdpa_decode_windowed(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads, int64_t mask_batch,
                                     const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
-                                    int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int, float, int concat_heads, int64_t,
-                                    const void *attention_sink, void *) {
+                                    int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale,
+                                    int concat_heads, int64_t sliding_window, const void *attention_sink, void *) {
   return decode_check(__func__, q, k, v, cur_pos, mask, mask_heads, mask_batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch,
-                      heads, kv_heads, seq, head_dim, concat_heads, attention_sink);
+                      heads, kv_heads, seq, head_dim, concat_heads, attention_sink, is_causal, scale, sliding_window);
 }
 EXPORT int ttm_sdpa_decode_static(const void *q, const void *k, const void *v, const int32_t *cur_pos, const void *mask, int mask_heads, int64_t mask_batch,
                                   const int32_t *page_table, int64_t pages_per_user, int64_t page_block, int64_t page_blocks, void *out, int dtype,
-                                  int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int, float, int concat_heads, int64_t,
-                                  const void *attention_sink, void *) {
+                                  int64_t batch, int64_t heads, int64_t kv_heads, int64_t seq, int64_t head_dim, int is_causal, float scale,
+                                  int concat_heads, int64_t sliding_window, const void *attention_sink, void *) {
   return decode_check(__func__, q, k, v, cur_pos, mask, mask_heads, mask_batch, page_table, pages_per_user, page_block, page_blocks, out, dtype, batch,
-                      heads, kv_heads, seq, head_dim, concat_heads, attention_sink);
+                      heads, kv_heads, seq, head_dim, concat_heads, attention_sink, is_causal, scale, sliding_window);
 }
 
 // ---- decode path
@@ -691,49 +763,131 @@ EXPORT int ttm_rotary_embedding(const void *x, const void *cos_cache, const void
   if (batch * rows * cols == 0) return TTM_OK;
   if (token_index >= cache_rows || (token_index < 0 && rows > cache_rows)) return fail("ttm_rotary_embedding: position outside the cos / sin caches");
   EXT(rotary_embedding, x, cos_cache, sin_cache, out, dtype, batch, rows, cols, cache_rows);
-  return kernel();
+  return launch([=] {
+    Dense X = load_dense(x, dtype, TTM_TILE, batch, rows, cols), C = load_dense(cos_cache, dtype, TTM_TILE, 1, cache_rows, cols),
+          S_ = load_dense(sin_cache, dtype, TTM_TILE, 1, cache_rows, cols), O(X.size());
+    orc_rotary_embedding_f32(X.data(), C.data(), S_.data(), O.data(), batch, rows, cols, token_index);
+    store_dense(O, out, dtype, TTM_TILE, batch, rows, cols);
+  });
 }
 EXPORT int ttm_rotary_embedding_split_heads(const void *x, const void *cos_cache, const void *sin_cache, void *out, int dtype, int64_t batch, int64_t heads,
                                             int64_t head_dim, int64_t cache_rows, int64_t token_index, void *) {
   if (batch * heads * head_dim == 0) return TTM_OK;
   if (token_index < 0 || token_index >= cache_rows) return fail("ttm_rotary_embedding_split_heads: position outside the cos / sin caches");
   EXT(rotary_embedding_split_heads, x, cos_cache, sin_cache, out, dtype, batch, heads, head_dim, cache_rows);
-  return kernel();
+  return launch([=] {   // [batch, heads * head_dim] row-major is [batch * heads, head_dim] row-major
+    Dense X = load_dense(x, dtype, TTM_TILE, 1, batch, heads * head_dim), C = load_dense(cos_cache, dtype, TTM_TILE, 1, cache_rows, head_dim),
+          S_ = load_dense(sin_cache, dtype, TTM_TILE, 1, cache_rows, head_dim), O(X.size());
+    orc_rotary_embedding_f32(X.data(), C.data(), S_.data(), O.data(), 1, batch * heads, head_dim, token_index);
+    store_dense(O, out, dtype, TTM_TILE, batch, heads, head_dim);
+  });
 }
 EXPORT int ttm_rotary_embedding_llama(const void *x, const void *cos_cache, const void *sin_cache, const void *trans_mat, void *out, int dtype, int64_t batch,
                                       int64_t rows, int64_t cols, int64_t cs_batch, int64_t cs_rows, void *) {
   if (batch * rows * cols == 0) return TTM_OK;
   EXT(rotary_embedding_llama, x, cos_cache, sin_cache, trans_mat, out, dtype, batch, rows, cols, cs_batch, cs_rows);
-  return kernel();
+  return launch([=] {   // out = x cos + (x T) sin, T applied to every 32-column tile; f32, one rounding
+    Dense X = load_dense(x, dtype, TTM_TILE, batch, rows, cols), C = load_dense(cos_cache, dtype, TTM_TILE, cs_batch, cs_rows, cols),
+          S_ = load_dense(sin_cache, dtype, TTM_TILE, cs_batch, cs_rows, cols), T = load_dense(trans_mat, TTM_BF16, TTM_TILE, 1, 32, 32), O(X.size());
+    for (int64_t b = 0; b < batch; ++b)
+      for (int64_t r = 0; r < rows; ++r)
+        for (int64_t c = 0; c < cols; ++c) {
+          float rot = 0.0f;
+          for (int64_t j = 0; j < 32; ++j) rot += X[(size_t)((b * rows + r) * cols + c / 32 * 32 + j)] * T[(size_t)(j * 32 + c % 32)];
+          const size_t cs = (size_t)(((b % cs_batch) * cs_rows + (cs_rows == 1 ? 0 : r)) * cols + c);
+          O[(size_t)((b * rows + r) * cols + c)] = X[(size_t)((b * rows + r) * cols + c)] * C[cs] + rot * S_[cs];
+        }
+    store_dense(O, out, dtype, TTM_TILE, batch, rows, cols);
+  });
 }
 EXPORT int ttm_update_cache(void *cache, const void *input, const int32_t *update_index, int dtype, int64_t users, int64_t heads, int64_t max_seq,
                             int64_t head_dim, int64_t input_users, int64_t batch_offset, void *) {
   if (batch_offset < 0 || batch_offset + input_users > users) return fail("ttm_update_cache: batch_offset + input users exceeds the cache");
   EXT(update_cache, cache, input, update_index, dtype, users, heads, max_seq, head_dim, input_users);
-  return kernel();
+  return launch([=] {
+    const int64_t at = *update_index;   // read when the launch runs
+    if (at < 0 || at >= max_seq) return;
+    for (int64_t b = 0; b < input_users; ++b)
+      for (int64_t h = 0; h < heads; ++h)
+        for (int64_t d = 0; d < head_dim; ++d)
+          store_scalar(cache, dtype, elem_off(TTM_TILE, max_seq, head_dim, (batch_offset + b) * heads + h, at, d),
+                       load_scalar(input, dtype, elem_off(TTM_TILE, input_users, head_dim, h, b, d)));
+  });
 }
 EXPORT int ttm_fill_cache(void *cache, const void *input, int dtype, int64_t users, int64_t heads, int64_t max_seq, int64_t head_dim, int64_t seq,
                           int64_t batch_offset, void *) {
   if (batch_offset < 0 || batch_offset >= users || seq > max_seq) return fail("ttm_fill_cache: the input does not fit the cache entry");
   EXT(fill_cache, cache, input, dtype, users, heads, max_seq, head_dim, seq);
-  return kernel();
+  return launch([=] {
+    for (int64_t h = 0; h < heads; ++h)
+      for (int64_t r = 0; r < pad32(seq) && r < max_seq; ++r)   // the rows up to the next multiple of 32 receive the input's zero padding
+        for (int64_t d = 0; d < head_dim; ++d)
+          store_scalar(cache, dtype, elem_off(TTM_TILE, max_seq, head_dim, batch_offset * heads + h, r, d),
+                       r < seq ? load_scalar(input, dtype, elem_off(TTM_TILE, seq, head_dim, h, r, d)) : 0.0);
+  });
 }
 EXPORT int ttm_paged_update_cache(void *cache, const void *input, const int32_t *update_index, const int32_t *page_table, int dtype, int64_t blocks,
-                                  int64_t heads, int64_t block_size, int64_t head_dim, int64_t users, int64_t pages_per_user, int, void *) {
+                                  int64_t heads, int64_t block_size, int64_t head_dim, int64_t users, int64_t pages_per_user, int share_cache, void *) {
   EXT(paged_update_cache, cache, input, update_index, page_table, dtype, blocks, heads, block_size, head_dim, users, pages_per_user);
-  return kernel();
+  return launch([=] {
+    for (int64_t u = 0; u < users; ++u) {
+      const int64_t pos = update_index[u];
+      int64_t block, row;
+      if (page_table) {
+        if (pos < 0 || pos / block_size >= pages_per_user) continue;
+        block = page_table[u * pages_per_user + pos / block_size]; row = pos % block_size;
+      } else {
+        block = share_cache ? 0 : u; row = pos;
+      }
+      if (pos < 0 || block < 0 || block >= blocks || row >= block_size) continue;
+      for (int64_t h = 0; h < heads; ++h)
+        for (int64_t d = 0; d < head_dim; ++d)
+          store_scalar(cache, dtype, elem_off(TTM_TILE, block_size, head_dim, block * heads + h, row, d),
+                       load_scalar(input, dtype, elem_off(TTM_TILE, heads, head_dim, u, h, d)));
+    }
+  });
 }
 EXPORT int ttm_paged_fill_cache(void *cache, const void *input, const int32_t *page_table, const int32_t *batch_idx, int dtype, int64_t blocks, int64_t heads,
                                 int64_t block_size, int64_t head_dim, int64_t in_batch, int64_t seq, int64_t table_rows, int64_t pages_per_user, void *) {
   EXT(paged_fill_cache, cache, input, page_table, batch_idx, dtype, blocks, heads, block_size, head_dim, in_batch, seq, table_rows, pages_per_user);
-  return kernel();
+  return launch([=] {
+    for (int64_t b = 0; b < in_batch; ++b) {
+      const int64_t row = batch_idx ? batch_idx[b] : b;
+      if (row < 0 || row >= table_rows) continue;
+      for (int64_t s_ = 0; s_ < seq; ++s_) {
+        if (s_ / block_size >= pages_per_user) continue;
+        const int64_t block = page_table[row * pages_per_user + s_ / block_size];
+        if (block < 0 || block >= blocks) continue;
+        for (int64_t h = 0; h < heads; ++h)
+          for (int64_t d = 0; d < head_dim; ++d)
+            store_scalar(cache, dtype, elem_off(TTM_TILE, block_size, head_dim, block * heads + h, s_ % block_size, d),
+                         load_scalar(input, dtype, elem_off(TTM_TILE, seq, head_dim, b * heads + h, s_, d)));
+      }
+    }
+  });
 }
 EXPORT int ttm_paged_gather(const void *cache, const int32_t *page_table, void *out, int dtype, int64_t blocks, int64_t heads, int64_t block_size,
                             int64_t head_dim, int64_t users, int64_t pages_per_user, void *) {
   EXT(paged_gather, cache, page_table, out, dtype, blocks, heads, block_size, head_dim, users, pages_per_user);
-  return kernel();
+  return launch([=] {
+    const int64_t S = pages_per_user * block_size;
+    for (int64_t u = 0; u < users; ++u)
+      for (int64_t j = 0; j < S; ++j) {
+        const int64_t block = page_table[u * pages_per_user + j / block_size];
+        const bool ok = block >= 0 && block < blocks;
+        for (int64_t h = 0; h < heads; ++h)
+          for (int64_t d = 0; d < head_dim; ++d)
+            store_scalar(out, dtype, elem_off(TTM_TILE, S, head_dim, u * heads + h, j, d),
+                         ok ? load_scalar(cache, dtype, elem_off(TTM_TILE, block_size, head_dim, block * heads + h, j % block_size, d)) : 0.0);
+      }
+  });
 }
 EXPORT int ttm_chunk_causal_mask(void *mask, const int32_t *chunk_start, int64_t rows, int64_t cols, void *) {
   EXT(chunk_causal_mask, mask, chunk_start, rows, cols);
-  return kernel();
+  return launch([=] {
+    const int64_t start = *chunk_start;
+    memset(mask, 0, (size_t)tile_bytes(TTM_BF16, 1, rows, cols));
+    for (int64_t r = 0; r < rows; ++r)
+      for (int64_t c = 0; c < cols; ++c) store_scalar(mask, TTM_BF16, elem_off(TTM_TILE, rows, cols, 0, r, c), c <= start + r ? 0.0 : -INFINITY);
+  });
 }
