@@ -415,6 +415,65 @@ __device__ __forceinline__ void linear_epilogue_act(const LinearArgs &p, uint8_t
   }
 }
 
+// The same three steps for accumulators of v_mfma_f32_16x16x32_bf16: acc[u][v] is the 16 (n) x 16 (m) tile u of the
+// wavefront's columns and v of its rows; a lane holds m = lane % 16 and n = 4 (lane / 16) + r in register r.
+template <int ACT, int NU, int NV>
+__device__ __forceinline__ void linear_epilogue16(const LinearArgs &p, uint8_t *C, f32x4 (&acc)[NU][NV], int mtw, int ntw, int nt_end, int lane) {
+  const int m16 = lane & 15, n4 = (lane >> 4) * 4;
+#pragma unroll
+  for (int u = 0; u < NU; ++u) {
+    const int nt = ntw + (u >> 1);
+    if (nt >= nt_end) continue;
+    const int n_in = (u & 1) * 16 + n4;
+    float bv[4] = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+      const uint16_t *bp = p.bias_tiled ? p.bias + (int64_t)nt * 1024 + (n_in >> 4) * 256 + (n_in & 15) : p.bias + nt * 32 + n_in;
+      u32x2 raw = *(const u32x2 *)bp;
+      bv[0] = __uint_as_float(raw.x << 16); bv[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+      bv[2] = __uint_as_float(raw.y << 16); bv[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+    }
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int mt = mtw + (v >> 1);
+      if (mt >= p.Mt) continue;
+      const int m_in = (v & 1) * 16 + m16;
+      float x[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) x[r] = apply_act<ACT>(acc[u][v][r] + bv[r]);
+      const int64_t off = ((int64_t)mt * p.Nt + nt) * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
+      *(u32x2 *)(C + off * 2) = finish_quad(p, C + off * 2, x);
+    }
+  }
+}
+template <int NU, int NV>
+__device__ __forceinline__ void linear_store_partial16(const LinearArgs &p, float *P, f32x4 (&acc)[NU][NV], int mtw, int ntw, int nt_end, int lane) {
+  const int m16 = lane & 15, n4 = (lane >> 4) * 4;
+#pragma unroll
+  for (int u = 0; u < NU; ++u) {
+    const int nt = ntw + (u >> 1);
+    if (nt >= nt_end) continue;
+    const int n_in = (u & 1) * 16 + n4;
+#pragma unroll
+    for (int v = 0; v < NV; ++v) {
+      const int mt = mtw + (v >> 1);
+      if (mt >= p.Mt) continue;
+      const int m_in = (v & 1) * 16 + m16;
+      const int64_t off = ((int64_t)mt * p.Nt + nt) * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
+      *(f32x4 *)(P + off) = acc[u][v];
+    }
+  }
+}
+template <int NU, int NV>
+__device__ __forceinline__ void linear_epilogue_act16(const LinearArgs &p, uint8_t *C, f32x4 (&acc)[NU][NV], int mtw, int ntw, int nt_end, int lane) {
+  switch (p.act) {   // uniform
+  case TTM_ACT_GELU: linear_epilogue16<TTM_ACT_GELU>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  case TTM_ACT_SILU: linear_epilogue16<TTM_ACT_SILU>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  case TTM_ACT_SIGMOID: linear_epilogue16<TTM_ACT_SIGMOID>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  case TTM_ACT_RELU: linear_epilogue16<TTM_ACT_RELU>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  default: linear_epilogue16<TTM_ACT_NONE>(p, C, acc, mtw, ntw, nt_end, lane); break;
+  }
+}
+
 template <int WF>
 __global__ __launch_bounds__(256) void ttm_linear_big_k(LinearArgs p) {
   extern __shared__ u32x4 smem[];  // 2 stages x (A 2048 chunks + W 2048 chunks) = 128 KiB
@@ -1073,6 +1132,178 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   else linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wcol, nt_end, lane);
 }
 
+
+// The second pass (weights already bf16 fragment images) with v_mfma_f32_16x16x32_bf16 in place of 32x32x16: the same LDS
+// images, the same staging and barriers, the same 64 (m) x 32 NTW (n) outputs per wavefront, now as 2 NTW x 4 accumulator
+// tiles of 16 x 16.  The smaller shape moves half the accumulator bytes per multiply-add through the register file; under
+// the power cap that is clock: an MFMA-only loop on random bf16 operands sustains 2.02 PFLOP/s with this shape and 1.78
+// with 32x32x16 on the same part (2.45 either way on all-zero operands, where nothing is power-limited), and the vendor
+// library's bf16 GEMM uses it as well.
+// A step (64 k) is two chunks of 32 k.  In a chunk, n tile u multiplies its weight fragment with the four activation
+// fragments of the chunk; weight fragments are requested one tile ahead.  The block barrier sits after n tile 3 of the
+// second chunk: tiles 4 .. 7 of that chunk multiply from fragments requested before the barrier, and the first fragments
+// of the next step are requested right behind it, so the matrix core does not drain at the barrier.
+template <int WF, int NTW, int BN_ = 2 * NTW>
+__device__ __forceinline__ void linear_img16_block(const LinearArgs &p, int bid, int nblk, int nt_first, int nt_end) {
+  static_assert(BN_ == 2 * NTW || (BN_ == 7 && (NTW == 4 || NTW == 3)), "block of 2 NTW column tiles, or the uneven seven");
+  constexpr int MB = 2, BN = BN_, NU = 2 * NTW, NV = 2 * MB;
+  extern __shared__ u32x4 smem[];
+  uint8_t *lds = (uint8_t *)smem;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int wn, wm, wcol;
+  if constexpr (BN_ == 2 * NTW) {
+    wn = wave & 1; wm = wave >> 1; wcol = wn * NTW;
+  } else {
+    const int sd = wave & 3, hf = wave >> 2;
+    wn = (sd & 1) ^ hf; wm = (sd >> 1) + 2 * hf; wcol = wn ? BN_ - NTW : 0;
+  }
+  if (nblk % 8 == 0) bid = (bid & 7) * (nblk >> 3) + (bid >> 3);   // consecutive blocks of one XCD share weight columns
+  const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
+  const int mt0 = mb * 8, nt0 = nt_first + nb * BN;
+  const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
+  const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
+  uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
+  constexpr uint32_t LDS_W = 65536, STAGE = 32768;
+
+  f32x4 acc[NU][NV];
+#pragma unroll
+  for (int u = 0; u < NU; ++u)
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[u][v] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // fragment reads: 16 rows x four 8-k chunks per instruction.  Row bit 4 (the odd 16-row tiles) enters the swizzle, so
+  // even and odd tiles have their own per-lane constant; + 4096 (tile / 2) + STAGE stage.
+  uint32_t rdW[2][2], rdA[2][2];   // [chunk][tile parity]
+#pragma unroll
+  for (int c = 0; c < 2; ++c)
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+      rdW[c][par] = LDS_W + 16u * lds_chunk(wcol * 32 + par * 16 + (lane & 15), 4 * c + (lane >> 4));
+      rdA[c][par] = 16u * lds_chunk(wm * (32 * MB) + par * 16 + (lane & 15), 4 * c + (lane >> 4));
+    }
+  uint32_t dmaA[4];
+  bool dmaA_sub[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r32 = 8 * i + (lane >> 3);
+    const int kc = (lane & 7) ^ lds_swz(r32);
+    dmaA[i] = (uint32_t)(((r32 >> 4) * 2 + ((kc & 3) >> 1)) * 512 + (r32 & 15) * 32 + (kc & 1) * 16);
+    dmaA_sub[i] = (kc >> 2) != 0;
+  }
+  const int64_t a_row = (int64_t)min(mt0 + wave, p.Mt - 1) * p.Kt * 2048;
+  const int kbase = blockIdx.y * p.k_slice, kt_end = min(p.Kt, kbase + p.k_slice);
+  const int ksteps = (kt_end - kbase + 1) / 2;
+
+  auto issue_a = [&](int kt0, uint32_t stage_off, int i0 = 0, int i1 = 4) {
+    kt0 += kbase;
+    const int kt = min(kt0, p.Kt - 1);
+    const uint32_t sub = kt0 + 1 < p.Kt ? 2048u : 0u;
+    const uint8_t *base = A + a_row + (int64_t)kt * 2048;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i >= i0 && i < i1) lds_dma16(base, dmaA[i] + (dmaA_sub[i] ? sub : 0u), lds0 + stage_off + (uint32_t)(wave * 256 + i * 64) * 16u);
+  };
+  auto issue_img = [&](int step, uint32_t stage_off, int i0 = 0, int i1 = 4) {
+    if (wave >= BN) return;
+    const int ksg = (kbase >> 1) + step;
+    const int ksc = kbase + 2 * step < kt_end ? ksg : p.img_zero_step;
+    const uint8_t *base = W + ((int64_t)ksc * p.Nt + min(nt0 + wave, p.Nt - 1)) * 4096;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i >= i0 && i < i1) lds_dma16(base, (uint32_t)(lane * 16 + i * 1024), lds0 + LDS_W + stage_off + (uint32_t)(wave * 4096 + i * 1024));
+  };
+  // A fragment address is a per-lane base plus a constant (tile pair and stage) that belongs in the instruction's offset
+  // field.  The bases pass through an empty asm in every step: seen as loop-invariant, base + constant would be hoisted
+  // into registers of their own - one per tile pair - and those spill.
+  uint32_t bW[2][2], bA[2][2];
+  auto refresh_bases = [&]() {
+#pragma unroll
+    for (int c = 0; c < 2; ++c)
+#pragma unroll
+      for (int par = 0; par < 2; ++par) {
+        bW[c][par] = rdW[c][par]; bA[c][par] = rdA[c][par];
+        asm volatile("" : "+v"(bW[c][par]), "+v"(bA[c][par]));
+      }
+  };
+  auto fetch_w = [&](int c, int u, uint32_t so) { return *(const u32x4 *)(lds + bW[c][u & 1] + ((u >> 1) * 4096 + so)); };
+  auto fetch_a1 = [&](int c, int v, uint32_t so) { return *(const u32x4 *)(lds + bA[c][v & 1] + ((v >> 1) * 4096 + so)); };
+  auto fetch_a = [&](int c, uint32_t so, u32x4 (&a)[NV]) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) a[v] = fetch_a1(c, v, so);
+  };
+  auto mfma_tile = [&](int u, const u32x4 &w, const u32x4 (&a)[NV]) {
+#pragma unroll
+    for (int v = 0; v < NV; ++v) acc[u][v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(const bf16x8 *)&w, *(const bf16x8 *)&a[v], acc[u][v], 0, 0, 0);
+  };
+  auto landed_barrier = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+  };
+
+  // ---- prologue: step 0 staged, step 1 on its way
+  issue_a(0, 0);
+  issue_img(0, 0);
+  landed_barrier();
+  issue_a(2, STAGE);
+  issue_img(1, STAGE);
+  u32x4 fa[2][NV], fw[NU];   // activation fragments of the two chunks; weight fragments of the chunk in flight
+  refresh_bases();
+  fetch_a(0, 0, fa[0]);
+  fw[0] = fetch_w(0, 0, 0);
+
+  auto step = [&](auto stage_c, int ks) {
+    constexpr uint32_t CUR = decltype(stage_c)::value * STAGE, NXT = STAGE - CUR;
+    constexpr int H = NU / 2;
+    refresh_bases();
+    // chunk 0: the next weight fragment is requested one tile ahead; the activation fragments of chunk 1 in its second half
+#pragma unroll
+    for (int u = 0; u < NU; ++u) {
+      if (u == 0 && ks > 0) { issue_a((ks + 1) * 2, NXT, 1, 3); issue_img(ks + 1, NXT, 1, 3); }
+      if (u == H && ks > 0) { issue_a((ks + 1) * 2, NXT, 3, 4); issue_img(ks + 1, NXT, 3, 4); }
+      if (u >= NU - 4) fa[1][u - (NU - 4)] = fetch_a1(1, u - (NU - 4), CUR);
+      fw[(u + 1) % NU] = u + 1 < NU ? fetch_w(0, u + 1, CUR) : fetch_w(1, 0, CUR);
+      mfma_tile(u, fw[u], fa[0]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // chunk 1, first half; the fragments of the second half are all requested before the barrier
+#pragma unroll
+    for (int u = 0; u < H; ++u) {
+      fw[u + 1] = fetch_w(1, u + 1, CUR);
+      if (u + 1 + H < NU) fw[u + 1 + H] = fetch_w(1, u + 1 + H, CUR);
+      mfma_tile(u, fw[u], fa[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    landed_barrier();
+    // stage CUR is free: the first instruction of the step after next
+    issue_a((ks + 2) * 2, CUR, 0, 1);
+    issue_img(ks + 2, CUR, 0, 1);
+    // the five fragments the next step starts from (four of the activations, one of the weights) are requested between
+    // the remaining tiles, as registers come free: fa[0] and fw[0] were last used before the barrier
+#pragma unroll
+    for (int u = H; u < NU; ++u) {
+#pragma unroll
+      for (int f = 0; f < 5; ++f) {
+        if (f * H / 5 != u - H) continue;
+        if (f < 4) fa[0][f] = fetch_a1(0, f, NXT);
+        else fw[0] = fetch_w(0, 0, NXT);
+      }
+      mfma_tile(u, fw[u], fa[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  for (int ks = 0; ks < ksteps; ks += 2) {
+    step(std::integral_constant<int, 0>{}, ks);
+    step(std::integral_constant<int, 1>{}, ks + 1);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+
+  if (p.partial) linear_store_partial16(p, p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * ((int64_t)p.Mt * p.Nt * 1024), acc,
+                                        mt0 + wm * MB, nt0 + wcol, nt_end, lane);
+  else linear_epilogue_act16(p, C, acc, mt0 + wm * MB, nt0 + wcol, nt_end, lane);
+}
+
 // group launch: the block's member becomes an ordinary single launch over that member's columns (p is rebound); the
 // XCD-aware renumbering is applied to the whole grid here, so the body is told not to repeat it (nblk = 1)
 __device__ __forceinline__ void linear_group_rebind(LinearArgs &p, int &bid, int &nblk, int &end) {
@@ -1098,7 +1329,7 @@ __global__ __launch_bounds__(512) void ttm_linear_dma_k(LinearArgs p) {
   else linear_dma_block<WF, 2>(p, bid, nblk, first, end);
 }
 
-template <int WF>
+template <int WF, bool M16 = true>   // M16: v_mfma_f32_16x16x32_bf16 (linear_img16_block); else 32x32x16
 __global__ __launch_bounds__(512) void ttm_linear_img_k(LinearArgs p) {
   int bid = blockIdx.x, nblk = gridDim.x, first = 0, end = p.Nt, ntw = p.ntw;
   if (p.group_n > 1) linear_group_rebind(p, bid, nblk, end);   // workgroup-uniform
@@ -1106,13 +1337,23 @@ __global__ __launch_bounds__(512) void ttm_linear_img_k(LinearArgs p) {
     if (bid < p.n_blocks1) { nblk = p.n_blocks1; end = p.nt_split; }
     else { bid -= p.n_blocks1; nblk -= p.n_blocks1; first = p.nt_split; ntw = p.ntw2; }
   }
-  if (ntw == 7) {   // seven tiles wide: wide and narrow wavefronts (wavefront-uniform branch)
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if ((((wave & 3) & 1) ^ (wave >> 2)) == 0) linear_dma_block<WF, 4, true, 7>(p, bid, nblk, first, end);
-    else linear_dma_block<WF, 3, true, 7>(p, bid, nblk, first, end);
-  } else if (ntw == 4) linear_dma_block<WF, 4, true>(p, bid, nblk, first, end);
-  else if (ntw == 3) linear_dma_block<WF, 3, true>(p, bid, nblk, first, end);
-  else linear_dma_block<WF, 2, true>(p, bid, nblk, first, end);
+  if constexpr (M16) {
+    if (ntw == 7) {   // seven tiles wide: wide and narrow wavefronts (wavefront-uniform branch)
+      const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+      if ((((wave & 3) & 1) ^ (wave >> 2)) == 0) linear_img16_block<WF, 4, 7>(p, bid, nblk, first, end);
+      else linear_img16_block<WF, 3, 7>(p, bid, nblk, first, end);
+    } else if (ntw == 4) linear_img16_block<WF, 4>(p, bid, nblk, first, end);
+    else if (ntw == 3) linear_img16_block<WF, 3>(p, bid, nblk, first, end);
+    else linear_img16_block<WF, 2>(p, bid, nblk, first, end);
+  } else {
+    if (ntw == 7) {
+      const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+      if ((((wave & 3) & 1) ^ (wave >> 2)) == 0) linear_dma_block<WF, 4, true, 7>(p, bid, nblk, first, end);
+      else linear_dma_block<WF, 3, true, 7>(p, bid, nblk, first, end);
+    } else if (ntw == 4) linear_dma_block<WF, 4, true>(p, bid, nblk, first, end);
+    else if (ntw == 3) linear_dma_block<WF, 3, true>(p, bid, nblk, first, end);
+    else linear_dma_block<WF, 2, true>(p, bid, nblk, first, end);
+  }
 }
 
 // First pass of a two-pass launch: block-float tiles -> bf16 LDS fragment images.  img[(ks * Nt + nt) * 4096 ..] is the
