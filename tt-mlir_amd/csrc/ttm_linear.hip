@@ -1140,13 +1140,14 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
 // with 32x32x16 on the same part (2.45 either way on all-zero operands, where nothing is power-limited), and the vendor
 // library's bf16 GEMM uses it as well.
 // A step (64 k) is two chunks of 32 k.  In a chunk, n tile u multiplies its weight fragment with the four activation
-// fragments of the chunk; weight fragments are requested one tile ahead.  The block barrier sits after n tile 3 of the
+// fragments of the chunk; weight fragments are requested two tiles ahead.  The block barrier sits after n tile 3 of the
 // second chunk: tiles 4 .. 7 of that chunk multiply from fragments requested before the barrier, and the first fragments
 // of the next step are requested right behind it, so the matrix core does not drain at the barrier.
 template <int WF, int NTW, int BN_ = 2 * NTW>
 __device__ __forceinline__ void linear_img16_block(const LinearArgs &p, int bid, int nblk, int nt_first, int nt_end) {
   static_assert(BN_ == 2 * NTW || (BN_ == 7 && (NTW == 4 || NTW == 3)), "block of 2 NTW column tiles, or the uneven seven");
   constexpr int MB = 2, BN = BN_, NU = 2 * NTW, NV = 2 * MB;
+  constexpr int PF = 2;   // weight fragments are requested PF tiles ahead (one ahead measured half a percent slower)
   extern __shared__ u32x4 smem[];
   uint8_t *lds = (uint8_t *)smem;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
@@ -1217,18 +1218,14 @@ __device__ __forceinline__ void linear_img16_block(const LinearArgs &p, int bid,
   // A fragment address is a per-lane base plus a constant (tile pair and stage) that belongs in the instruction's offset
   // field.  The bases pass through an empty asm in every step: seen as loop-invariant, base + constant would be hoisted
   // into registers of their own - one per tile pair - and those spill.
-  uint32_t bW[2][2], bA[2][2];
-  auto refresh_bases = [&]() {
+  auto refresh_bases = [&]() {   // the values stay
 #pragma unroll
     for (int c = 0; c < 2; ++c)
 #pragma unroll
-      for (int par = 0; par < 2; ++par) {
-        bW[c][par] = rdW[c][par]; bA[c][par] = rdA[c][par];
-        asm volatile("" : "+v"(bW[c][par]), "+v"(bA[c][par]));
-      }
+      for (int par = 0; par < 2; ++par) asm volatile("" : "+v"(rdW[c][par]), "+v"(rdA[c][par]));
   };
-  auto fetch_w = [&](int c, int u, uint32_t so) { return *(const u32x4 *)(lds + bW[c][u & 1] + ((u >> 1) * 4096 + so)); };
-  auto fetch_a1 = [&](int c, int v, uint32_t so) { return *(const u32x4 *)(lds + bA[c][v & 1] + ((v >> 1) * 4096 + so)); };
+  auto fetch_w = [&](int c, int u, uint32_t so) { return *(const u32x4 *)(lds + rdW[c][u & 1] + ((u >> 1) * 4096 + so)); };
+  auto fetch_a1 = [&](int c, int v, uint32_t so) { return *(const u32x4 *)(lds + rdA[c][v & 1] + ((v >> 1) * 4096 + so)); };
   auto fetch_a = [&](int c, uint32_t so, u32x4 (&a)[NV]) {
 #pragma unroll
     for (int v = 0; v < NV; ++v) a[v] = fetch_a1(c, v, so);
@@ -1251,27 +1248,29 @@ __device__ __forceinline__ void linear_img16_block(const LinearArgs &p, int bid,
   u32x4 fa[2][NV], fw[NU];   // activation fragments of the two chunks; weight fragments of the chunk in flight
   refresh_bases();
   fetch_a(0, 0, fa[0]);
-  fw[0] = fetch_w(0, 0, 0);
+#pragma unroll
+  for (int u = 0; u < PF; ++u) fw[u] = fetch_w(0, u, 0);
 
   auto step = [&](auto stage_c, int ks) {
     constexpr uint32_t CUR = decltype(stage_c)::value * STAGE, NXT = STAGE - CUR;
     constexpr int H = NU / 2;
     refresh_bases();
-    // chunk 0: the next weight fragment is requested one tile ahead; the activation fragments of chunk 1 in its second half
+    // chunk 0: weight fragments are requested PF tiles ahead (fw[0 .. PF - 1] are there on entry); the activation
+    // fragments of chunk 1 in its second half
 #pragma unroll
     for (int u = 0; u < NU; ++u) {
       if (u == 0 && ks > 0) { issue_a((ks + 1) * 2, NXT, 1, 3); issue_img(ks + 1, NXT, 1, 3); }
       if (u == H && ks > 0) { issue_a((ks + 1) * 2, NXT, 3, 4); issue_img(ks + 1, NXT, 3, 4); }
       if (u >= NU - 4) fa[1][u - (NU - 4)] = fetch_a1(1, u - (NU - 4), CUR);
-      fw[(u + 1) % NU] = u + 1 < NU ? fetch_w(0, u + 1, CUR) : fetch_w(1, 0, CUR);
+      fw[(u + PF) % NU] = u + PF < NU ? fetch_w(0, u + PF, CUR) : fetch_w(1, u + PF - NU, CUR);
       mfma_tile(u, fw[u], fa[0]);
       __builtin_amdgcn_sched_barrier(0);
     }
     // chunk 1, first half; the fragments of the second half are all requested before the barrier
 #pragma unroll
     for (int u = 0; u < H; ++u) {
-      fw[u + 1] = fetch_w(1, u + 1, CUR);
-      if (u + 1 + H < NU) fw[u + 1 + H] = fetch_w(1, u + 1 + H, CUR);
+      fw[u + PF] = fetch_w(1, u + PF, CUR);
+      if (u + PF + H < NU) fw[u + PF + H] = fetch_w(1, u + PF + H, CUR);
       mfma_tile(u, fw[u], fa[1]);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -1279,15 +1278,15 @@ __device__ __forceinline__ void linear_img16_block(const LinearArgs &p, int bid,
     // stage CUR is free: the first instruction of the step after next
     issue_a((ks + 2) * 2, CUR, 0, 1);
     issue_img(ks + 2, CUR, 0, 1);
-    // the five fragments the next step starts from (four of the activations, one of the weights) are requested between
-    // the remaining tiles, as registers come free: fa[0] and fw[0] were last used before the barrier
+    // the fragments the next step starts from (four of the activations, PF of the weights) are requested between the
+    // remaining tiles, as registers come free: fa[0] and fw[0 .. PF - 1] were last used before the barrier
 #pragma unroll
     for (int u = H; u < NU; ++u) {
 #pragma unroll
-      for (int f = 0; f < 5; ++f) {
-        if (f * H / 5 != u - H) continue;
+      for (int f = 0; f < 4 + PF; ++f) {
+        if (f * H / (4 + PF) != u - H) continue;
         if (f < 4) fa[0][f] = fetch_a1(0, f, NXT);
-        else fw[0] = fetch_w(0, 0, NXT);
+        else fw[f - 4] = fetch_w(0, f - 4, NXT);
       }
       mfma_tile(u, fw[u], fa[1]);
       __builtin_amdgcn_sched_barrier(0);
@@ -2059,10 +2058,12 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       // Two passes when the conversion is repeated often enough: every block of 256 rows dequantises the weights it
       // multiplies, so with M / 256 row blocks the same conversion runs M / 256 times.  The first pass writes the weights
       // once as bf16 fragment images into the stream's workspace, the second runs the main loop without conversion
-      // (measured at [2048, 4096] x [4096, 14336]: 243 us fused; 30 us for the image pass + 193 us for the second pass).
-      // Modelled: the fused loop costs what plan_dma_grid says, the second pass 0.78 of it, the first pass 3 us +
-      // (tile bytes + 2048) per tile at 5.5 TB/s.  Launches that split K are left fused: measured, their second pass gains
-      // under 10 % ([2048, 14336] x [14336, 4096]: 232 us fused, 242 us in two passes).
+      // (measured at [2048, 4096] x [4096, 14336]: 230 us fused; 26 us for the image pass + 188 us for the second pass).
+      // Modelled: the fused loop costs what plan_dma_grid says, the first pass 3 us + (tile bytes + 2048) per tile at
+      // 5.5 TB/s, and the second pass saves a share of the fused loop that depends on what the conversion cost there:
+      // 0.28 for bfp8_b and 0.22 for bfp4_b, whose conversion is cheaper; for launches that split K 0.18 and 0.08
+      // (measured: [2048, 4096] x [4096, 4096] bfp8_b 87 us fused, 80 us in two passes; [2048, 14336] x [14336, 4096]
+      // bfp4_b 225 us fused, 231 us in two passes; [1024, 4096] x [4096, 14336] bfp8_b 112 against 114 us).
       // linear_two_pass: 0 = by the model, 1 = never, 2 = always.
       const int ksteps = (a.Kt + 1) / 2;
       const int64_t sets = a.w_batch == 0 ? 1 : batch;
@@ -2073,7 +2074,8 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         const int64_t rounds = ((int64_t)p.n_blocks * slices * batch + cus - 1) / cus;
         const double fused = rounds * width_cost[p.ntw] * ((ksteps + slices - 1) / slices + 12) * 1.65;
         const double first = 3.0 + (double)sets * a.Kt * a.Nt * ((WF == WF_BFP8 ? 1088.0 : 576.0) + 2048.0) / 5.5e6;
-        two_pass = slices == 1 && 0.22 * fused > first && img_set < ((int64_t)1 << 31);
+        const double gain = WF == WF_BFP8 ? (slices == 1 ? 0.28 : 0.18) : (slices == 1 ? 0.22 : 0.08);
+        two_pass = gain * fused > first && img_set < ((int64_t)1 << 31);
       }
       const int64_t per = (int64_t)a.Mt * a.Nt * 1024;
       const size_t img_bytes = two_pass ? (size_t)((img_set * sets + 255) / 256 * 256) : 0;
@@ -2118,7 +2120,12 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
         p.W = ws;
         p.w_batch = a.w_batch == 0 ? 0 : img_set;
         p.img_zero_step = ksteps;
-        hipLaunchKernelGGL((ttm_linear_img_k<WI>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), 131072, s, p);
+        if (ttm_option("linear_img_variant") == 1) {   // the 32x32x16 form of the second pass, for comparison
+          if (int rc = set_lds_limit(ttm_linear_img_k<WI, false>, 131072)) return rc;
+          hipLaunchKernelGGL((ttm_linear_img_k<WI, false>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), 131072, s, p);
+        } else {
+          hipLaunchKernelGGL((ttm_linear_img_k<WI>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), 131072, s, p);
+        }
       } else if constexpr (BFP) {
         hipLaunchKernelGGL((ttm_linear_dma_k<WF>), dim3(p.n_blocks, slices, (unsigned)batch), dim3(512), lds6, s, p);
       }
