@@ -440,7 +440,7 @@ def test_copy_view_at_positions_the_destination_from_device_memory(hip, dev, ele
     # (variant 5 keeps them in one workgroup); ragged key counts, masks, a causal chunk, shares without any visible key
     (1, 8, 2, 128, 2048, 128, False, None), (1, 4, 2, 100, 1500, 64, False, "bh"), (2, 2, 2, 64, 1100, 128, False, "b1"),
     (1, 4, 4, 128, 1024, 128, True, None), (1, 2, 1, 40, 4096, 32, False, None)])
-@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5])   # automatic, 32-key kernel, eight-wavefront kernel forced / forbidden, no key shares
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 6])   # automatic, 32-key kernel, eight-wavefront kernel forced / forbidden, no key shares, no pipeline
 def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask, variant):
     if variant == 1 and Sq * Sk >= 512 * 512:
         pytest.skip("the 32-key kernel is covered by the small shapes")
@@ -497,7 +497,7 @@ def test_sdpa_config5_shape(hip, dev, orc):
     assert np.array_equal(res[0, :, 0, :], np.repeat(v.float().numpy()[0, :, 0, :], Hq // Hkv, axis=0))
 
 
-@pytest.mark.parametrize("variant", [0, 1, 4])
+@pytest.mark.parametrize("variant", [0, 1, 4, 6])
 @pytest.mark.parametrize("flags", [15, 1, 6, 8, 9])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", [(1, 8, 2, 256, 256, 128, True), (2, 4, 4, 96, 160, 64, False), (1, 4, 1, 70, 70, 32, True),
                                                       (1, 2, 2, 40, 300, 256, False)])
@@ -532,7 +532,7 @@ def test_sdpa_heads_inner_equals_the_head_major_call(hip, dev, B, Hq, Hkv, Sq, S
     assert torch.equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 4])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 6])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,window,sink,mask,flags", [
     (1, 4, 2, 256, 256, 128, True, 64, False, None, 0), (1, 4, 2, 256, 256, 128, True, 1, False, None, 0),
     (1, 4, 2, 300, 300, 64, True, 100, True, None, 0), (2, 2, 2, 96, 160, 128, False, 40, False, None, 0),

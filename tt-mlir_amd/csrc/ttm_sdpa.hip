@@ -15,6 +15,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef __bf16 sdpa_bf16x2 __attribute__((ext_vector_type(2)));
 
 struct SdpaArgs {
   const uint8_t *q, *k, *v, *mask;
@@ -705,6 +706,391 @@ __global__ __launch_bounds__(512) void ttm_sdpa64_split_k(SdpaArgs p, int paired
   if (light < heavy) sdpa64_split_block<DT>(p, light, h, b, ldsK, ldsV);   // workgroup-uniform
 }
 
+// The eight-wavefront pass as a software pipeline.  ttm_sdpa64_split_k runs a pass as a chain (stage K and V through
+// registers, barrier, fragment reads, scores, softmax, second product, barrier): all wavefronts ask LDS for their
+// fragments at the same time, then the matrix core at the same time, then the vector ALU at the same time.  Here
+//   * K and V go global -> LDS with LDS-direct loads (no staging registers, no ds_write) into a ring of five 64-key
+//     stages, requested three passes ahead and issued one at a time between the MFMAs; one barrier per pass, and a pass has
+//     landed one barrier before it is multiplied;
+//   * a wavefront computes the scores of pass i while it takes the exponentials of pass i - 1: every MFMA of the score
+//     product is followed by one score's share of the softmax, and the second product of pass i - 1 follows with the rest;
+//   * the fragments a step starts with (K of the first 64 columns, V^T of the first 16 keys) are requested at the end of
+//     the step before, across the barrier, so that the reads of the eight wavefronts do not pile up behind it;
+//   * a wavefront's passes are an interval (causal and window limits are bands): first pass scores only, last pass softmax
+//     only, the loop between them is free of conditions;
+//   * the running maximum is only moved when some query's maximum grew by more than 8 (in the log2 domain): sums and
+//     outputs stay relative to the older maximum (probabilities up to 2^8, exact in bf16's range), and the rescale of the
+//     output accumulators, 16 DT multiplies per lane, becomes rare;
+//   * the two halves of a query's maximum and sum are exchanged with v_permlane32_swap instead of through LDS.
+// Same fragment layouts, same arithmetic per score as the kernels above.
+__device__ __forceinline__ void sdpa_dma16(const void *base, uint32_t lane_off, uint32_t lds_addr) {
+  // lds_addr is wavefront-uniform; lane l of the wavefront writes 16 bytes at lds_addr + 16 l
+  asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
+}
+__device__ __forceinline__ float sdpa_max_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sdpa_sum_halves(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+template <bool B> struct SdpaFlag { static constexpr bool value = B; };
+
+template <int DT>  // head_dim / 32: 2 or 4
+__device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *lds) {
+  static_assert(DT == 2 || DT == 4, "64 or 128 columns");
+  constexpr int TROW = DT * 2048;      // one 32-key tile row of K or V
+  constexpr int STAGE = 4 * TROW;      // a 64-key pass: two tile rows of K, then two of V
+  constexpr int NST = 5;               // stages of the ring
+  constexpr int NL = DT;               // LDS-direct loads per wavefront and pass: DT / 2 of K, DT / 2 of V
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int qw = wave & 3, kh = wave >> 2;
+  const int hk = h / (p.Hq / p.Hkv);
+  const int qt = qb * 4 + qw;                           // this wave's query tile
+  const bool wave_ok = qt < p.sqt;
+  const int l31 = lane & 31, hh = lane >> 5;
+  const int64_t q_mat = b * p.q_batch + h * p.q_head, o_mat = b * p.o_batch + h * p.o_head;
+  const int64_t k_mat = b * p.k_batch + hk * p.k_head, v_mat = b * p.v_batch + hk * p.v_head;
+
+  bf16x8 qf[2 * DT];
+#pragma unroll
+  for (int s = 0; s < 2 * DT; ++s) {
+    u32x4 v = {0, 0, 0, 0};
+    if (wave_ok)
+      v = *(const u32x4 *)(p.q + q_mat + qt * p.q_pitch + (s >> 1) * 2048 + ((l31 >> 4) * 2 + (s & 1)) * 512 +
+                           (l31 & 15) * 32 + hh * 16);
+    qf[s] = *(bf16x8 *)&v;
+  }
+  // The fragments are used here, in front of the loops, so that the wait for their loads stands here too: a counted wait
+  // for them further down would also wait for the LDS-direct loads issued there, which the compiler does not count.
+#pragma unroll
+  for (int s = 0; s < 2 * DT; ++s) asm volatile("" : "+v"(qf[s]));
+  f32x16 o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[d][r] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
+  const int q_glob = qt * 32 + l31, q_last = qt * 32 + 31;
+  const int kt_begin = first_key_tile(p, qb * 128), kt_end = end_key_tile(p, min(qb * 4 + 4, p.sqt) * 32 - 1);
+  const int kb_begin = kt_begin >> 1, kb_end = (kt_end + 1) >> 1;
+  // This wavefront's 32 keys of pass kb start at 64 kb + 32 kh; the passes in which one of them is visible to one of its
+  // queries (not behind the causal or window limit, not in front of the window, not past the last key) are an interval.
+  int w_begin, w_end;
+  {
+    const int x = qt * 32 - p.lo_off - 31 - 32 * kh;
+    const int y = min(q_last + p.hi_off, p.Sk - 1) - 32 * kh;
+    w_begin = max(x > 0 ? (x + 63) >> 6 : 0, kb_begin);
+    w_end = min(y >= 0 ? (y >> 6) + 1 : 0, kb_end);
+    if (!wave_ok || w_begin >= w_end) w_begin = w_end = kb_end;
+  }
+
+  // Staging.  The instructions of a wavefront cover 64 consecutive 16-byte chunks of LDS each; chunk c of a pass's K lies
+  // in tile row c / (128 DT).  K is copied as it lies in its tiles; V too, but the faces of the upper 16 columns are
+  // rotated by eight chunks (four rows) so that the transposing reads touch every bank once: the lane that fills a chunk
+  // of such a face fetches the chunk eight further back.
+  const int c0 = wave * 64;                               // with 512 lanes and 128 DT chunks per tile row, load i of a wavefront
+  const int ccl = c0 % (DT * 128) + lane;                 // lies in tile row (c0 + 512 i) / (128 DT) at the same chunk
+  const uint32_t koff = ccl * 16;
+  const uint32_t voff = ((ccl & ~31) + (((ccl & 31) - 8 * ((ccl >> 5) & 1)) & 31)) * 16;
+  const uint8_t *kg = p.k + k_mat, *vg = p.v + v_mat;
+  auto next_stage = [](int st) { return st + STAGE == NST * STAGE ? 0 : st + STAGE; };   // byte offsets of the ring's stages
+  auto dma = [&](int kb, int st_off, int i) {   // load i of this wavefront for pass kb (stage at st_off): K for even i, V for odd
+    const uint32_t st = lds0 + st_off + c0 * 16 + (i >> 1) * 8192;
+    const int tr = (c0 + 512 * (i >> 1)) / (DT * 128);   // 0 or 1
+    const bool second = tr && 2 * kb + 1 < p.skt;         // an odd tile count repeats the last tile; its keys are masked
+    if (i & 1) sdpa_dma16(vg + (int64_t)(2 * kb) * p.v_pitch + (second ? p.v_pitch : 0), voff, st + 2 * TROW);
+    else sdpa_dma16(kg + (int64_t)(2 * kb) * p.k_pitch + (second ? p.k_pitch : 0), koff, st);
+  };
+  // Every pass of the loop requests NL loads, so that the counted wait below always has the same meaning: near the end
+  // the last pass is requested again, into the stage that is free at that point, and never read.
+  auto dma_all = [&](int kb, int st_off) {
+#pragma unroll
+    for (int i = 0; i < NL; ++i) dma(min(kb, kb_end - 1), st_off, i);
+  };
+  // All but this wavefront's last NL loads have landed, hence pass kb + 1 (requested two passes ago), and after the barrier
+  // every wavefront's share of it; and every wavefront is through with pass kb - 2, whose stage pass kb + 3 overwrites.
+  auto sync = [&]() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NL) : "memory");
+    __syncthreads();
+  };
+  // per-lane parts of the fragment addresses inside a stage
+  const int dhalf = (lane >> 4) & 1, s16 = lane & 15;
+  const int kfrag = kh * TROW + (l31 >> 4) * 1024 + (l31 & 15) * 32 + hh * 16;
+  const int vfrag = 2 * TROW + kh * TROW + dhalf * 512;
+  const int vlo = ((4 * hh + (s16 >> 2)) * 32 + 8 * (s16 & 3) + 128 * dhalf) & 511, vhi = (vlo + 256) & 511;
+  const uint8_t *kfp = lds + kfrag, *vlp = lds + vfrag + vlo, *vhp = lds + vfrag + vhi;
+  u32x4 ka[DT];   // K fragments of DT of a pass's 2 DT steps at a time
+  u32x4 va[DT];   // V^T fragments of 16 of a pass's 32 keys at a time
+  auto read_k = [&](const uint8_t *kp, int st) {   // step st of the pass whose stage kp points into
+    ka[st % DT] = *(const u32x4 *)(kp + (st >> 1) * 2048 + (st & 1) * 512);
+  };
+  auto read_v = [&](const uint8_t *vl, const uint8_t *vh, int t, int d) {
+    // V^T fragment: column d * 32 + l31, keys 16 t + 4 hh .. + 3 and eight further on, by two transposing LDS reads
+    // (ds_read_b64_tr_b16: of the 16 lanes of a group, lane 4 u + c receives element c of the rows that lanes
+    // u, u + 4, u + 8, u + 12 address; lane u + 4 j addresses key j of the four, columns 4 u .. + 3)
+    typedef short s16x4 __attribute__((ext_vector_type(4)));
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(vl + d * 2048 + t * 1024));
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)(vh + d * 2048 + t * 1024));
+    const u32x2 l2 = *(const u32x2 *)&lo, h2 = *(const u32x2 *)&hi;
+    va[d] = u32x4{l2.x, l2.y, h2.x, h2.y};
+  };
+  constexpr float LOG2E = 1.4426950408889634f;
+  const float scale2 = p.scale * LOG2E;
+  if (kh == 0) sink_start(p, h, scale2, m_run, l_run);   // the sink belongs to one of the two halves only
+  float m_use = m_run == -INFINITY ? 0.0f : m_run;       // what the exponentials are relative to: zero while nothing is seen
+
+  // The ring as this wavefront walks it: byte offset of the stage of the pass being multiplied and the fragment addresses
+  // in it, in the stage before (V of the pass whose softmax is under way) and, computed in the step, in the stage after.
+  int st_cur = 0;
+  const uint8_t *k_cur = kfp, *vl_prev = vlp, *vh_prev = vhp, *vl_cur = vlp, *vh_cur = vhp;
+  const uint32_t ones = 0x3F803F80u;   // two bf16 ones: v_dot2_f32_bf16 with them adds a pair of probabilities as the matrix core sees them
+
+  // One pipeline step at pass kb: the score product of pass kb into sn (QK) beside the softmax and the second product of
+  // pass kb - 1, whose scores are in sc (SM).  On entry ka holds the K fragments of the first DT steps of pass kb (QK) and
+  // va the V^T fragments of the first 16 keys of pass kb - 1 (SM); on exit they hold those of the next step.  RING: the
+  // step requests pass kb + 3 (not the step behind the last barrier).
+  auto step = [&](auto qk_tag, auto sm_tag, auto ring_tag, int kb, f32x16 &sc, f32x16 &sn) {
+    constexpr bool QK = decltype(qk_tag)::value, SM = decltype(sm_tag)::value, RING = decltype(ring_tag)::value;
+    const int st_next = next_stage(st_cur);
+    const int st_load = next_stage(next_stage(st_next));
+    const int kb_load = min(kb + 3, kb_end - 1);
+    const uint8_t *k_next = kfp + st_next;
+    float mul = scale2, rs = 0.0f;
+    if constexpr (SM) {
+      const int key_base = (kb - 1) * 64 + 32 * kh;
+      const bool edge = key_base + 31 > qt * 32 + p.hi_off || key_base < q_last - p.lo_off || key_base + 32 > p.Sk;   // wavefront-uniform
+      float mx = -INFINITY;
+      if (p.mask || edge) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int kin = g * 8 + hh * 4;
+          const int key0 = key_base + kin;
+          float mk[4] = {0.f, 0.f, 0.f, 0.f};
+          if (p.mask) {
+            const int kt = min(2 * (kb - 1) + kh, p.skt - 1);
+            const int64_t mm = ((int64_t)b * p.mask_b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
+            const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
+                                (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
+            u32x2 raw = *(const u32x2 *)mp;
+            mk[0] = __uint_as_float(raw.x << 16); mk[1] = __uint_as_float(raw.x & 0xFFFF0000u);
+            mk[2] = __uint_as_float(raw.y << 16); mk[3] = __uint_as_float(raw.y & 0xFFFF0000u);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float v = fmaf(sc[g * 4 + r], scale2, mk[r] * LOG2E);
+            const int key = key0 + r;
+            if (key >= p.Sk || key > q_glob + p.hi_off || key < q_glob - p.lo_off) v = -INFINITY;
+            sc[g * 4 + r] = v;
+            mx = fmaxf(mx, v);
+          }
+        }
+        mul = 1.0f;
+      } else {   // plain block: the scale (positive) is folded into the exponent's multiply-add, the maximum is taken first
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[r]);
+        mx *= scale2;
+      }
+      mx = sdpa_max_halves(mx);
+      if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.0f) != 0) {   // some query's maximum grew by more than 2^8: all move
+        const float m_new = fmaxf(m_run, mx);
+        const float m_to = m_new == -INFINITY ? 0.0f : m_new;   // fully masked so far: stay at zero without producing NaN
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_to);
+        l_run *= alpha;
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[d][r] *= alpha;
+        m_run = m_new;
+        m_use = m_to;
+      }
+    }
+    const float neg_m = -m_use;
+    auto elem = [&](int r) { sc[r] = __builtin_amdgcn_exp2f(fmaf(sc[r], mul, neg_m)); };
+    auto pack8 = [&](int r0) {   // eight probabilities as bf16, and their sum as rounded
+      u32x4 pb;
+      pb.x = pack_bf16_rne(sc[r0 + 0], sc[r0 + 1]);
+      pb.y = pack_bf16_rne(sc[r0 + 2], sc[r0 + 3]);
+      pb.z = pack_bf16_rne(sc[r0 + 4], sc[r0 + 5]);
+      pb.w = pack_bf16_rne(sc[r0 + 6], sc[r0 + 7]);
+      const uint32_t w[4] = {pb.x, pb.y, pb.z, pb.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) rs = __builtin_amdgcn_fdot2_f32_bf16(*(const sdpa_bf16x2 *)&w[j], *(const sdpa_bf16x2 *)&ones, rs, false);
+      return pb;
+    };
+    __builtin_amdgcn_sched_barrier(0);
+    // first half of the exponentials, one MFMA of the score product in front of each share; behind the MFMA its K
+    // register is refilled: second half of this pass, then first half of the next
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int st = 0; st < 2 * DT; ++st) {
+      if constexpr (QK) {
+        sn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&ka[st % DT], qf[st], st == 0 ? zero : sn, 0, 0, 0);
+        if (st < DT) read_k(k_cur, st + DT);
+        else read_k(k_next, st - DT);
+      }
+      if constexpr (RING) {   // the ring's loads are spread over the step: the addresser takes one wavefront's at a time
+        if (st == 0) dma(kb_load, st_load, 0);
+        if (st == DT && NL > 2) dma(kb_load, st_load, 2);
+      }
+      if constexpr (SM) {
+#pragma unroll
+        for (int e = 0; e < 8 / (2 * DT); ++e) elem(st * (8 / (2 * DT)) + e);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (SM) {
+      u32x4 pb = pack8(0);
+      __builtin_amdgcn_sched_barrier(0);
+      // second half of the exponentials beside the second product of the first 16 keys; the V^T fragments of the other
+      // 16 keys follow into the same registers
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va[d], *(bf16x8 *)&pb, o[d], 0, 0, 0);
+        read_v(vl_prev, vh_prev, 1, d);
+        if constexpr (RING) {
+          if (d == 0) dma(kb_load, st_load, 1);
+        }
+#pragma unroll
+        for (int e = 0; e < 8 / DT; ++e) elem(8 + d * (8 / DT) + e);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      pb = pack8(8);
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va[d], *(bf16x8 *)&pb, o[d], 0, 0, 0);
+        if constexpr (QK) read_v(vl_cur, vh_cur, 0, d);   // for the next step
+        if constexpr (RING) {
+          if (d == 0 && NL > 2) dma(kb_load, st_load, 3);
+        }
+      }
+      l_run += sdpa_sum_halves(rs);
+    } else {
+#pragma unroll
+      for (int d = 0; d < DT; ++d) read_v(vl_cur, vh_cur, 0, d);
+      if constexpr (RING) {
+        dma(kb_load, st_load, 1);
+        if (NL > 2) dma(kb_load, st_load, 3);
+      }
+    }
+    // one pass on: the stage multiplied next is the one after, the stage of this pass is the one the softmax looks back to
+    st_cur = st_next;
+    k_cur = k_next;
+    vl_prev = vl_cur; vh_prev = vh_cur;
+    vl_cur = vlp + st_next; vh_cur = vhp + st_next;
+  };
+  auto skip = [&](int kb) {   // a pass outside this wavefront's interval: its share of the staging only
+    sync();
+    const int st_next = next_stage(st_cur);
+    dma_all(kb + 3, next_stage(next_stage(st_next)));
+    st_cur = st_next;
+  };
+
+  f32x16 sa, sb;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) sa[r] = sb[r] = 0.0f;
+  {
+    int st = 0;
+    for (int i = 0; i < 3; ++i) { dma_all(kb_begin + i, st); st = next_stage(st); }   // the first pass lies in stage 0
+  }
+  int kb = kb_begin;
+  for (; kb < w_begin; ++kb) skip(kb);
+  if (w_begin < w_end) {
+    sync();
+    k_cur = kfp + st_cur; vl_cur = vlp + st_cur; vh_cur = vhp + st_cur;
+#pragma unroll
+    for (int st = 0; st < DT; ++st) read_k(k_cur, st);
+    step(SdpaFlag<true>{}, SdpaFlag<false>{}, SdpaFlag<true>{}, kb, sb, sa);   // scores of the first pass into sa
+    for (kb = w_begin + 1; kb + 1 < w_end; kb += 2) {
+      sync();
+      step(SdpaFlag<true>{}, SdpaFlag<true>{}, SdpaFlag<true>{}, kb, sa, sb);
+      sync();
+      step(SdpaFlag<true>{}, SdpaFlag<true>{}, SdpaFlag<true>{}, kb + 1, sb, sa);
+    }
+    if (kb < w_end) {
+      sync();
+      step(SdpaFlag<true>{}, SdpaFlag<true>{}, SdpaFlag<true>{}, kb, sa, sb);
+      sa = sb;
+      ++kb;
+    }
+    // kb = w_end: the last pass's softmax and second product; behind the last barrier nothing is requested any more
+    // (other wavefronts may still be reading the stage that would be overwritten)
+    if (kb < kb_end) {
+      sync();
+      step(SdpaFlag<false>{}, SdpaFlag<true>{}, SdpaFlag<true>{}, kb, sa, sb);
+    } else {
+      step(SdpaFlag<false>{}, SdpaFlag<true>{}, SdpaFlag<false>{}, kb, sa, sb);
+    }
+    for (++kb; kb < kb_end; ++kb) skip(kb);
+  }
+  // merge the two key halves of every query tile: the upper half hands over (max, sum) and its output, 4 DT values per
+  // lane at a time (DT * 4 KiB = 256 lanes x DT float4), through the ring, which nobody reads or fills any more
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  float *ml = (float *)(lds + STAGE);
+  f32x4 *ox = (f32x4 *)lds;
+  const int slot = qw * 64 + lane;
+  if (kh == 1) { ml[2 * slot] = m_run; ml[2 * slot + 1] = l_run; }
+  __syncthreads();
+  float a0 = 1.0f, a1 = 0.0f;
+  if (kh == 0) {
+    const float m1 = ml[2 * slot], l1 = ml[2 * slot + 1];
+    const float m = fmaxf(m_run, m1), m_use = m == -INFINITY ? 0.0f : m;
+    a0 = __builtin_amdgcn_exp2f(m_run - m_use);
+    a1 = __builtin_amdgcn_exp2f(m1 - m_use);
+    l_run = l_run * a0 + l1 * a1;
+  }
+#pragma unroll
+  for (int r4 = 0; r4 < 4; ++r4) {
+    if (kh == 1) {
+#pragma unroll
+      for (int d = 0; d < DT; ++d) ox[slot * DT + d] = f32x4{o[d][4 * r4], o[d][4 * r4 + 1], o[d][4 * r4 + 2], o[d][4 * r4 + 3]};
+    }
+    __syncthreads();
+    if (kh == 0) {
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        const f32x4 x = ox[slot * DT + d];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[d][4 * r4 + e] = o[d][4 * r4 + e] * a0 + x[e] * a1;
+      }
+    }
+    __syncthreads();
+  }
+  if (kh != 0 || !wave_ok) return;   // no barrier follows inside this block; the next block starts with one
+  const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
+  const bool q_ok = q_glob < p.Sq;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int din = g * 8 + hh * 4;
+      u32x2 ov;
+      ov.x = q_ok ? pack_bf16_rne(o[d][g * 4 + 0] * inv, o[d][g * 4 + 1] * inv) : 0u;
+      ov.y = q_ok ? pack_bf16_rne(o[d][g * 4 + 2] * inv, o[d][g * 4 + 3] * inv) : 0u;
+      uint8_t *op = p.out + o_mat + qt * p.o_pitch + d * 2048 +
+                    (((l31 >> 4) * 2 + (din >> 4)) * 256 + (l31 & 15) * 16 + (din & 15)) * 2;
+      *(u32x2 *)op = ov;
+    }
+}
+
+template <int DT>
+__global__ __launch_bounds__(512) void ttm_sdpa_pipe_k(SdpaArgs p, int paired) {
+  extern __shared__ u32x4 sdpa_ring[];
+  uint8_t *lds = (uint8_t *)sdpa_ring;
+  const int nqb = (p.sqt + 3) / 4, h = blockIdx.y, b = blockIdx.z;
+  if (!paired) {
+    sdpa_pipe_block<DT>(p, nqb - 1 - (int)blockIdx.x, h, b, lds);
+    return;
+  }
+  const int heavy = nqb - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
+  sdpa_pipe_block<DT>(p, heavy, h, b, lds);
+  if (light < heavy) sdpa_pipe_block<DT>(p, light, h, b, lds);   // workgroup-uniform
+}
+
 // Merges the key shares of ttm_sdpa64_split_k: one workgroup per (b, h, query tile).  With M = max_s m_s, every output is
 // sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M); a share that saw no key has m = -inf and weighs nothing; a row without any
 // visible key gives zeros, as the single-workgroup path does.
@@ -785,7 +1171,7 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
   int cus = 0, devid = 0;
   if (hipGetDevice(&devid) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, devid) != hipSuccess || cus <= 0) cus = 256;
   const int64_t wgs = (int64_t)grid64.x * grid64.y * grid64.z;
-  const bool split = wide && D <= 128 && (variant == 3 || (variant == 0 && wgs <= (int64_t)cus));
+  const bool split = wide && D <= 128 && (variant == 3 || ((variant == 0 || variant == 6) && wgs <= (int64_t)cus));
   p.ksplits = 1; p.part_o = nullptr; p.part_ml = nullptr;
   if (split) {
     const dim3 block8(512);
@@ -807,6 +1193,17 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
       p.part_o = (float *)ws;
       p.part_ml = p.part_o + slots * D * 32;
       g.x = (unsigned)(grid64.x * ks);
+    }
+    // one workgroup per query block (or pair) and 64 or 128 columns: the pipelined form.  sdpa_variant 6 keeps the chained one.
+    if (ks == 1 && (D == 128 || D == 64) && variant != 6) {
+      const int ring = (int)D / 32 * 40960;   // five stages of 64 keys of K and V
+      hipError_t e = D == 128 ? hipFuncSetAttribute((const void *)ttm_sdpa_pipe_k<4>, hipFuncAttributeMaxDynamicSharedMemorySize, ring)
+                              : hipFuncSetAttribute((const void *)ttm_sdpa_pipe_k<2>, hipFuncAttributeMaxDynamicSharedMemorySize, ring);
+      if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "hipFuncSetAttribute(LDS %d): %s", ring, hipGetErrorString(e));
+      if (D == 128) hipLaunchKernelGGL(ttm_sdpa_pipe_k<4>, g, block8, ring, s, p, paired);
+      else hipLaunchKernelGGL(ttm_sdpa_pipe_k<2>, g, block8, ring, s, p, paired);
+      TTM_LAUNCH_CHECK();
+      return TTM_OK;
     }
     switch (D) {
     case 32: hipLaunchKernelGGL(ttm_sdpa64_split_k<1>, g, block8, 0, s, p, paired); break;
