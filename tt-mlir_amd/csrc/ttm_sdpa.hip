@@ -764,10 +764,6 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
                            (l31 & 15) * 32 + hh * 16);
     qf[s] = *(bf16x8 *)&v;
   }
-  // The fragments are used here, in front of the loops, so that the wait for their loads stands here too: a counted wait
-  // for them further down would also wait for the LDS-direct loads issued there, which the compiler does not count.
-#pragma unroll
-  for (int s = 0; s < 2 * DT; ++s) asm volatile("" : "+v"(qf[s]));
   f32x16 o[DT];
 #pragma unroll
   for (int d = 0; d < DT; ++d)
@@ -996,6 +992,11 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
     int st = 0;
     for (int i = 0; i < 3; ++i) { dma_all(kb_begin + i, st); st = next_stage(st); }   // the first pass lies in stage 0
   }
+  // Q is used here, in front of the loops, so that the wait for its loads stands here (and covers the requests above, whose
+  // first passes the first barrier needs anyway): a counted wait for it further down would also wait for the
+  // LDS-direct loads issued there, which the compiler does not count, and drain the ring at every step.
+#pragma unroll
+  for (int s = 0; s < 2 * DT; ++s) asm volatile("" : "+v"(qf[s]));
   int kb = kb_begin;
   for (; kb < w_begin; ++kb) skip(kb);
   if (w_begin < w_end) {
@@ -1026,40 +1027,37 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
     }
     for (++kb; kb < kb_end; ++kb) skip(kb);
   }
-  // merge the two key halves of every query tile: the upper half hands over (max, sum) and its output, 4 DT values per
-  // lane at a time (DT * 4 KiB = 256 lanes x DT float4), through the ring, which nobody reads or fills any more
+  // merge the two key halves of every query tile: the upper half hands over (max, sum) and its output (16 DT values per
+  // lane: 256 lanes x 16 DT floats = DT * 16 KiB) through the ring, which nobody reads or fills any more
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-  float *ml = (float *)(lds + STAGE);
+  float *ml = (float *)(lds + 4 * STAGE);
   f32x4 *ox = (f32x4 *)lds;
   const int slot = qw * 64 + lane;
-  if (kh == 1) { ml[2 * slot] = m_run; ml[2 * slot + 1] = l_run; }
+  if (kh == 1) {
+    ml[2 * slot] = m_run; ml[2 * slot + 1] = l_run;
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4)
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+        ox[(r4 * 256 + slot) * DT + d] = f32x4{o[d][4 * r4], o[d][4 * r4 + 1], o[d][4 * r4 + 2], o[d][4 * r4 + 3]};
+  }
   __syncthreads();
-  float a0 = 1.0f, a1 = 0.0f;
   if (kh == 0) {
     const float m1 = ml[2 * slot], l1 = ml[2 * slot + 1];
-    const float m = fmaxf(m_run, m1), m_use = m == -INFINITY ? 0.0f : m;
-    a0 = __builtin_amdgcn_exp2f(m_run - m_use);
-    a1 = __builtin_amdgcn_exp2f(m1 - m_use);
+    const float m = fmaxf(m_run, m1), m_to = m == -INFINITY ? 0.0f : m;
+    const float a0 = __builtin_amdgcn_exp2f(m_run - m_to), a1 = __builtin_amdgcn_exp2f(m1 - m_to);
     l_run = l_run * a0 + l1 * a1;
-  }
 #pragma unroll
-  for (int r4 = 0; r4 < 4; ++r4) {
-    if (kh == 1) {
-#pragma unroll
-      for (int d = 0; d < DT; ++d) ox[slot * DT + d] = f32x4{o[d][4 * r4], o[d][4 * r4 + 1], o[d][4 * r4 + 2], o[d][4 * r4 + 3]};
-    }
-    __syncthreads();
-    if (kh == 0) {
+    for (int r4 = 0; r4 < 4; ++r4)
 #pragma unroll
       for (int d = 0; d < DT; ++d) {
-        const f32x4 x = ox[slot * DT + d];
+        const f32x4 x = ox[(r4 * 256 + slot) * DT + d];
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[d][4 * r4 + e] = o[d][4 * r4 + e] * a0 + x[e] * a1;
       }
-    }
-    __syncthreads();
   }
+  __syncthreads();   // the next block of the pair fills the ring again
   if (kh != 0 || !wave_ok) return;   // no barrier follows inside this block; the next block starts with one
   const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
   const bool q_ok = q_glob < p.Sq;
@@ -1081,14 +1079,23 @@ template <int DT>
 __global__ __launch_bounds__(512) void ttm_sdpa_pipe_k(SdpaArgs p, int paired) {
   extern __shared__ u32x4 sdpa_ring[];
   uint8_t *lds = (uint8_t *)sdpa_ring;
-  const int nqb = (p.sqt + 3) / 4, h = blockIdx.y, b = blockIdx.z;
-  if (!paired) {
-    sdpa_pipe_block<DT>(p, nqb - 1 - (int)blockIdx.x, h, b, lds);
-    return;
+  const int nqb = (p.sqt + 3) / 4;
+  int x = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  // Workgroups go to the eight XCDs in turn, in the order of their flat index, and every XCD has an L2 of its own.  The
+  // workgroups that read one K / V matrix (the query blocks of the query heads of one kv head) are therefore given flat
+  // indices that are equal modulo 8: an XCD's L2 then holds the K and V of a few kv heads, each read by all its users,
+  // instead of every XCD streaming all of them.
+  if ((p.B * p.Hkv) % 8 == 0) {
+    const int flat = x + (int)gridDim.x * (h + p.Hq * b), gq = p.Hq / p.Hkv, users = (int)gridDim.x * gq;
+    const int xcd = flat % 8, idx = flat / 8;
+    const int group = (idx / users) * 8 + xcd, member = idx % users;   // group: (batch entry, kv head)
+    b = group / p.Hkv;
+    h = (group % p.Hkv) * gq + member % gq;
+    x = member / gq;
   }
-  const int heavy = nqb - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
-  sdpa_pipe_block<DT>(p, heavy, h, b, lds);
-  if (light < heavy) sdpa_pipe_block<DT>(p, light, h, b, lds);   // workgroup-uniform
+  const int heavy = nqb - 1 - x, light = x;
+  const int parts = paired && light < heavy ? 2 : 1;   // workgroup-uniform
+  for (int part = 0; part < parts; ++part) sdpa_pipe_block<DT>(p, part == 0 ? heavy : light, h, b, lds);
 }
 
 // Merges the key shares of ttm_sdpa64_split_k: one workgroup per (b, h, query tile).  With M = max_s m_s, every output is
