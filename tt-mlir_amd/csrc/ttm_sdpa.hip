@@ -65,6 +65,21 @@ __device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
   return ttm_pack_bf16x2(a, b);
 }
 
+// Workgroups go to the eight XCDs in turn, in the order of their flat index, and every XCD has an L2 of its own.  The
+// workgroups that read one K / V matrix (the query blocks of the query heads of one kv head) are therefore given flat
+// indices that are equal modulo 8: an XCD's L2 then holds the K and V of a few kv heads, each read by all its users,
+// instead of every XCD streaming all of them.  x, h, b come in as blockIdx and go out as the block, head and batch entry
+// this workgroup serves (a permutation of the grid; the identity when the matrices do not divide among eight XCDs).
+__device__ __forceinline__ void sdpa_xcd_order(const SdpaArgs &p, int &x, int &h, int &b) {
+  if ((p.B * p.Hkv) % 8 != 0) return;
+  const int flat = x + (int)gridDim.x * (h + p.Hq * b), gq = p.Hq / p.Hkv, users = (int)gridDim.x * gq;
+  const int xcd = flat % 8, idx = flat / 8;
+  const int group = (idx / users) * 8 + xcd, member = idx % users;   // group: (batch entry, kv head)
+  b = group / p.Hkv;
+  h = (group % p.Hkv) * gq + member % gq;
+  x = member / gq;
+}
+
 template <int DT>  // head_dim / 32
 __global__ __launch_bounds__(256) void ttm_sdpa_k(SdpaArgs p) {
   constexpr int D = DT * 32;
@@ -451,12 +466,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   constexpr int D = DT * 32;
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[64 * D * 2];
   __shared__ __attribute__((aligned(16))) uint16_t ldsV[D * kSdpaVPitch];
-  const int nqb = (p.sqt + 3) / 4, h = blockIdx.y, b = blockIdx.z;
+  const int nqb = (p.sqt + 3) / 4;
+  int x = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  sdpa_xcd_order(p, x, h, b);
   if (!paired) {
-    sdpa64_query_block<DT>(p, nqb - 1 - (int)blockIdx.x, h, b, ldsK, ldsV);
+    sdpa64_query_block<DT>(p, nqb - 1 - x, h, b, ldsK, ldsV);
     return;
   }
-  const int heavy = nqb - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
+  const int heavy = nqb - 1 - x, light = x;
   sdpa64_query_block<DT>(p, heavy, h, b, ldsK, ldsV);
   if (light < heavy) sdpa64_query_block<DT>(p, light, h, b, ldsK, ldsV);
 }
@@ -695,13 +712,15 @@ __global__ __launch_bounds__(512) void ttm_sdpa64_split_k(SdpaArgs p, int paired
   constexpr int D = DT * 32;
   __shared__ __attribute__((aligned(16))) uint8_t ldsK[64 * D * 2];
   __shared__ __attribute__((aligned(16))) uint16_t ldsV[D * kSdpaVPitch];
-  const int nqb = (p.sqt + 3) / 4, h = blockIdx.y, b = blockIdx.z;
+  const int nqb = (p.sqt + 3) / 4;
+  int x = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  sdpa_xcd_order(p, x, h, b);
   if (!paired) {   // with key shares grid.x numbers (query block, share)
-    const int xb = (int)blockIdx.x / p.ksplits, ks = (int)blockIdx.x - xb * p.ksplits;
+    const int xb = x / p.ksplits, ks = x - xb * p.ksplits;
     sdpa64_split_block<DT>(p, nqb - 1 - xb, h, b, ldsK, ldsV, ks);
     return;
   }
-  const int heavy = nqb - 1 - (int)blockIdx.x, light = (int)blockIdx.x;
+  const int heavy = nqb - 1 - x, light = x;
   sdpa64_split_block<DT>(p, heavy, h, b, ldsK, ldsV);
   if (light < heavy) sdpa64_split_block<DT>(p, light, h, b, ldsK, ldsV);   // workgroup-uniform
 }
@@ -1081,18 +1100,7 @@ __global__ __launch_bounds__(512) void ttm_sdpa_pipe_k(SdpaArgs p, int paired) {
   uint8_t *lds = (uint8_t *)sdpa_ring;
   const int nqb = (p.sqt + 3) / 4;
   int x = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  // Workgroups go to the eight XCDs in turn, in the order of their flat index, and every XCD has an L2 of its own.  The
-  // workgroups that read one K / V matrix (the query blocks of the query heads of one kv head) are therefore given flat
-  // indices that are equal modulo 8: an XCD's L2 then holds the K and V of a few kv heads, each read by all its users,
-  // instead of every XCD streaming all of them.
-  if ((p.B * p.Hkv) % 8 == 0) {
-    const int flat = x + (int)gridDim.x * (h + p.Hq * b), gq = p.Hq / p.Hkv, users = (int)gridDim.x * gq;
-    const int xcd = flat % 8, idx = flat / 8;
-    const int group = (idx / users) * 8 + xcd, member = idx % users;   // group: (batch entry, kv head)
-    b = group / p.Hkv;
-    h = (group % p.Hkv) * gq + member % gq;
-    x = member / gq;
-  }
+  sdpa_xcd_order(p, x, h, b);
   const int heavy = nqb - 1 - x, light = x;
   const int parts = paired && light < heavy ? 2 : 1;   // workgroup-uniform
   for (int part = 0; part < parts; ++part) sdpa_pipe_block<DT>(p, part == 0 ? heavy : light, h, b, lds);
@@ -1174,11 +1182,14 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
   // eight wavefronts per workgroup (two key halves per query tile) when the launch would otherwise leave every SIMD with a
   // single wavefront: no more workgroups than CUs (only one eight-wavefront workgroup fits a CU, so a larger launch would
   // take a second round where the four-wavefront kernel runs two workgroups side by side).  sdpa_variant 3 forces it, 4
-  // forbids it.
+  // forbids it, 6 keeps the chained form of it.
   int cus = 0, devid = 0;
   if (hipGetDevice(&devid) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, devid) != hipSuccess || cus <= 0) cus = 256;
   const int64_t wgs = (int64_t)grid64.x * grid64.y * grid64.z;
-  const bool split = wide && D <= 128 && (variant == 3 || ((variant == 0 || variant == 6) && wgs <= (int64_t)cus));
+  // (with 64 or 128 columns the eight-wavefront form is the pipelined kernel, which is the faster one at every launch size:
+  // [2, 32 / 8, 4096, 128] causal 293 against 350 us, [1, 32 / 8, 8192, 128] 539 against 665 us)
+  const bool split = wide && D <= 128 && (variant == 3 || ((variant == 0 || variant == 6) && wgs <= (int64_t)cus) ||
+                                          (variant == 0 && (D == 64 || D == 128)));
   p.ksplits = 1; p.part_o = nullptr; p.part_ml = nullptr;
   if (split) {
     const dim3 block8(512);
