@@ -342,38 +342,41 @@ def make_workloads(torch, hip, datagen, dev, names):
 
 
 # HBM bytes per launch of each workload's kernel, from two rocprofv3 --pmc runs (FETCH_SIZE, then WRITE_SIZE) scaled by
-# what the same counters read for the plain copy kernel of known size (factors 1.9998 and 0.9996); these are measured
-# constants of the committed kernels, not computed here.  linear2048 is a two-pass launch: 183.8 MB for the pass that
-# writes the weights as bf16 fragment images plus 447.9 MB for the matrix pass (every XCD's L2 fetches the activations
-# and its share of the images again).  Each figure belongs to one version of a kernel source file: it is reported only
-# while that file still has the content it was measured on (first 12 hex digits of its SHA-1, listed first), else
-# `traffic` is null.  A later version of a file is listed after the measured one only if it added other kernels and the
-# kernels these workloads launch compile to the same instructions in both versions (device assembly of both, compared
-# function by function).
+# what the same counters read for the plain copy kernel of known size (factors 1.9998 and 0.9999); these are measured
+# constants of the committed kernels, not computed here (profiles/bench_kernels_hbm_traffic_pmc.md holds the table and
+# the commands).  linear2048 is a two-pass launch: 181.9 MB for the pass that writes the weights as bf16 fragment images
+# plus 447.6 MB for the matrix pass (every XCD's L2 fetches the activations and its share of the images again).  Each
+# figure belongs to one version of a kernel source file: it is reported only while that file still has the content it
+# was measured on (first 12 hex digits of its SHA-1), else `traffic` is null and `traffic_source` says so.
 MEASURED_TRAFFIC_BYTES = {
-    "linear2048": (629.5e6, "ttm_linear.hip"), "linear32": (65.7e6, "ttm_linear.hip"), "pack_bfp8": (340.4e6, "ttm_bfp.hip"),
-    "unpack_bfp8": (340.1e6, "ttm_bfp.hip"), "pack_bfp4": (306.2e6, "ttm_bfp.hip"), "unpack_bfp4": (306.5e6, "ttm_bfp.hip"),
+    "linear2048": (629.5e6, "ttm_linear.hip"), "linear32": (65.6e6, "ttm_linear.hip"), "pack_bfp8": (340.4e6, "ttm_bfp.hip"),
+    "unpack_bfp8": (340.1e6, "ttm_bfp.hip"), "pack_bfp4": (306.2e6, "ttm_bfp.hip"), "unpack_bfp4": (306.6e6, "ttm_bfp.hip"),
     "tilize_f32": (537.3e6, "ttm_layout.hip"), "untilize_f32": (537.0e6, "ttm_layout.hip"), "copy": (536.9e6, "ttm_layout.hip"),
-    "sdpa_decode32": (270.3e6, "ttm_decode.hip"), "rmsnorm2048": (34.0e6, "ttm_rowwise.hip"),
+    "sdpa_decode32": (270.3e6, "ttm_decode.hip"), "sdpa2048": (42.3e6, "ttm_sdpa.hip"), "rmsnorm2048": (34.0e6, "ttm_rowwise.hip"),
     "softmax65536": (1073.8e6, "ttm_rowwise.hip"), "reduce65536": (545.2e6, "ttm_rowwise.hip"), "silu_mul512": (44.2e6, "ttm_eltwise.hip"),
 }
-MEASURED_ON = {"ttm_linear.hip": ("e4074d055f65",), "ttm_bfp.hip": ("8e9736544aea",), "ttm_layout.hip": ("c2d080a6c0c5",),
-               "ttm_decode.hip": ("8bbb69b8561a",), "ttm_rowwise.hip": ("ad15392e8bae", "ff3e580c91ab"),
-               "ttm_eltwise.hip": ("56692d4eb0d8", "538c0c60dffa", "3bec0c51416e")}
+MEASURED_ON = {"ttm_linear.hip": ("acc4b5e14f2b",), "ttm_bfp.hip": ("cdf35c7592c1",), "ttm_layout.hip": ("a6cf1c428342",),
+               "ttm_decode.hip": ("3bd99843ac98",), "ttm_rowwise.hip": ("0819544c7ff3",), "ttm_eltwise.hip": ("62019175607e",),
+               "ttm_sdpa.hip": ("588f3e389564",)}
+TRAFFIC_HOW = ("rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs), KiB per dispatch scaled by what the same counters "
+               "read for the 256 MiB copy kernel; profiles/bench_kernels_hbm_traffic_pmc.md")
 
 
 def measured_traffic(name):
+    """(bytes per launch, where the figure comes from) or (None, why there is none)."""
     import hashlib
     entry_ = MEASURED_TRAFFIC_BYTES.get(name)
     if entry_ is None:
-        return None
+        return None, "not measured for this workload"
     nbytes, source = entry_
     try:
         with open(os.path.join(ROOT, "tt-mlir_amd", "csrc", source), "rb") as f:
             digest = hashlib.sha1(f.read()).hexdigest()[:12]
     except OSError:
-        return None
-    return nbytes if digest in MEASURED_ON.get(source, ()) else None
+        return None, "kernel source %s not found" % source
+    if digest in MEASURED_ON.get(source, ()):
+        return nbytes, TRAFFIC_HOW
+    return None, "%s has changed since its kernels' counters were read" % source
 
 
 def roofline(w, kernel_ms):
@@ -383,8 +386,9 @@ def roofline(w, kernel_ms):
     else:
         achieved = w.work / (kernel_ms * 1e-3) / 1e12
         peak, unit = MFMA_BF16_PEAK_TFLOPS, "TFLOP/s"
+    traffic, how = measured_traffic(w.name)
     r = {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-         "frac": round(achieved / peak, 4), "traffic": measured_traffic(w.name), "kernel_us": round(kernel_ms * 1e3, 2),
+         "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_source": how, "kernel_us": round(kernel_ms * 1e3, 2),
          "algorithmic_work": w.work, "work_unit": w.unit_work}
     if "dense_flop" in w.extra:   # attention: the dense count beside the FLOPs of the visible pairs that `frac` is made of
         dense = w.extra["dense_flop"] / (kernel_ms * 1e-3) / 1e12

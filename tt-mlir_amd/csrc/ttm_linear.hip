@@ -152,6 +152,12 @@ __device__ __forceinline__ u32x2 finish_quad(const LinearArgs &p, const uint8_t 
 // (rows 8 apart x 2 chunks).
 __device__ __forceinline__ int lds_swz(int row) { return (((row << 1) & 6) | ((row >> 2) & 1)) ^ (((row >> 3) & 3) << 1); }
 __device__ __forceinline__ int lds_chunk(int row, int kc) { return row * 8 + (kc ^ lds_swz(row)); }
+// The images of the two-pass route (written by the image pass, read by the second pass as 16 rows x four chunks per
+// ds_read_b128 for v_mfma_f32_16x16x32_bf16) swizzle the slot by the low three row bits instead: under that read the
+// swizzle above puts pairs of lanes on one bank group (51 against 32 cycles per instruction with eight wavefronts reading),
+// this one none.
+__device__ __forceinline__ int lds_swz16(int row) { return row & 7; }
+__device__ __forceinline__ int lds_chunk16(int row, int kc) { return row * 8 + (kc ^ lds_swz16(row)); }
 
 // high halves of two floats -> packed bf16 pair (lo = a, hi = b); exact for dequantised weights
 __device__ __forceinline__ uint32_t pack_hi(float a, float b) {
@@ -903,7 +909,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   uint32_t rdW[4], rdA[4];   // fragment reads: + 4096 t + STAGE stage
 #pragma unroll
   for (int s = 0; s < 4; ++s) {
-    rdW[s] = LDS_W + 16u * lds_chunk(wcol * 32 + (lane & 31), 2 * s + (lane >> 5));
+    rdW[s] = LDS_W + 16u * (IMG ? lds_chunk16(wcol * 32 + (lane & 31), 2 * s + (lane >> 5)) : lds_chunk(wcol * 32 + (lane & 31), 2 * s + (lane >> 5)));
     rdA[s] = 16u * lds_chunk(wm * (32 * MB) + (lane & 31), 2 * s + (lane >> 5));
   }
   // weight block of this lane: tile slot tid >> 5 of the 2 x 8 tiles of a step (slot = 8 * k-tile + column tile);
@@ -1181,15 +1187,15 @@ __device__ __forceinline__ void linear_img16_block(const LinearArgs &p, int bid,
   for (int c = 0; c < 2; ++c)
 #pragma unroll
     for (int par = 0; par < 2; ++par) {
-      rdW[c][par] = LDS_W + 16u * lds_chunk(wcol * 32 + par * 16 + (lane & 15), 4 * c + (lane >> 4));
-      rdA[c][par] = 16u * lds_chunk(wm * (32 * MB) + par * 16 + (lane & 15), 4 * c + (lane >> 4));
+      rdW[c][par] = LDS_W + 16u * lds_chunk16(wcol * 32 + par * 16 + (lane & 15), 4 * c + (lane >> 4));
+      rdA[c][par] = 16u * lds_chunk16(wm * (32 * MB) + par * 16 + (lane & 15), 4 * c + (lane >> 4));
     }
   uint32_t dmaA[4];
   bool dmaA_sub[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int r32 = 8 * i + (lane >> 3);
-    const int kc = (lane & 7) ^ lds_swz(r32);
+    const int kc = (lane & 7) ^ lds_swz16(r32);
     dmaA[i] = (uint32_t)(((r32 >> 4) * 2 + ((kc & 3) >> 1)) * 512 + (r32 & 15) * 32 + (kc & 1) * 16);
     dmaA_sub[i] = (kc >> 2) != 0;
   }
@@ -1403,7 +1409,7 @@ __device__ __forceinline__ void linear_image_body(const uint8_t *W, uint8_t *img
   u32x4 *dst = (u32x4 *)(img + ((int64_t)ks * Nt + nt) * 4096);
   const int kc = (h >> 2) * 4 + (face >> 1) * 2 + khalf, n0 = (face & 1) * 16 + quad * 4;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) dst[lds_chunk(n0 + j, kc)] = out[j];
+  for (int j = 0; j < 4; ++j) dst[lds_chunk16(n0 + j, kc)] = out[j];
 }
 // three workgroups per CU: the pass is a pure stream (read 1 byte, write 2); [4096, 14336] about 2.5 us faster than without
 // a cap (the group form below measured no faster with one)
@@ -1446,7 +1452,7 @@ __global__ __launch_bounds__(256) TTM_MAX_WAVES(3) void ttm_linear_image_bf16_k(
   u32x4 *dst = (u32x4 *)(img + ((int64_t)ks * Nt + nt) * 4096);
   const int kc = (h >> 2) * 4 + (face >> 1) * 2 + khalf, n0 = (face & 1) * 16 + quad * 4;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) dst[lds_chunk(n0 + j, kc)] = out[j];
+  for (int j = 0; j < 4; ++j) dst[lds_chunk16(n0 + j, kc)] = out[j];
 }
 // the members of a group launch: grid.x numbers the members' groups of four column tiles one after another
 struct ImageGroup {
