@@ -64,6 +64,8 @@ def lib():
             fn = getattr(l, name)
             fn.restype, fn.argtypes = res, argtypes
         _lib = l
+        if _check_buffers:   # switched on by the environment before the library was loaded: the library's own check goes with it
+            l.ttm_set_option(b"check_extents", 1)
     return _lib
 
 
@@ -162,8 +164,15 @@ def _verify_extents(name, args):
         return
     try:
         extents = spec(args)
-    except (KeyError, IndexError, TypeError):
-        return   # arguments the size rules do not cover (an unknown dtype code, a short argument list): the library answers, with its own extent check
+    except (KeyError, IndexError, TypeError) as e:
+        # arguments the size rules here do not cover (an unknown dtype code, a short argument list): the library's own check,
+        # which is on whenever this one is and holds every operand of every entry point against its allocation, answers;
+        # without it the call is refused rather than let through unchecked
+        v = ctypes.c_int(0)
+        lib().ttm_get_option(b"check_extents", ctypes.byref(v))
+        if v.value == 1:
+            return
+        raise TTMError("%s: buffer extents cannot be checked for these arguments (%s: %s)" % (name, type(e).__name__, e))
     for idx, need, what in extents:
         p = args[idx]
         if isinstance(p, _Ptr) and p.nbytes is not None and p.nbytes < need:
