@@ -434,6 +434,78 @@ def cpu_baseline_pack(orc, datagen, rows=8192):
             "sample": "oracle bfp8_b pack of %d x 8192 fp32 rows of config 2, %.2f s" % (rows, dt)}
 
 
+def cpu_baseline_secondary(orc, datagen, name):
+    """The CPU restatement (one thread, scalar loops) on a bounded sample of a secondary workload, in the workload's own
+    unit: algorithmic bytes (or FLOP) of the sample over the time it took.  None for workloads without one function to time
+    (whole programs, the plain copy)."""
+    import numpy as np
+    rng = np.random.default_rng(0)
+    orc.set_threads(1)
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    def entry_(work, dt, unit, sample):
+        scale = 1e12 if unit == "TFLOP/s" else 1e9
+        return {"value": round(work / dt / scale, 6), "unit": unit, "cores": 1, "kind": "port", "sample": "%s, %.2f s" % (sample, dt)}
+
+    if name in ("pack_bfp8", "pack_bfp4", "unpack_bfp8", "unpack_bfp4"):
+        fmt, rows = (8 if name.endswith("8") else 4), 2048
+        x = datagen.c2_outliers(rows, 8192, seed=0).numpy()
+        nbytes = rows * 8192 * 4 + (rows // 32) * 256 * orc.bfp_tile_bytes(fmt)
+        if name.startswith("pack"):
+            return entry_(nbytes, timed(lambda: orc.bfp_pack(x, fmt)), "GB/s", "oracle bfp%d_b pack of %d x 8192 fp32 rows of config 2" % (fmt, rows))
+        packed = orc.bfp_pack(x, fmt)
+        return entry_(nbytes, timed(lambda: orc.bfp_unpack(packed, x.shape, fmt)), "GB/s", "oracle bfp%d_b unpack of %d x 8192 rows of config 2" % (fmt, rows))
+    if name in ("tilize_f32", "untilize_f32"):
+        rows = 4096
+        x = rng.standard_normal((rows, 8192), dtype=np.float32)
+        if name == "tilize_f32":
+            return entry_(2 * x.nbytes, timed(lambda: orc.tilize(x)), "GB/s", "oracle tilize of %d x 8192 fp32 rows of config 2" % rows)
+        t = orc.tilize(x)
+        return entry_(2 * x.nbytes, timed(lambda: orc.untilize(t, x.shape)), "GB/s", "oracle untilize of %d x 8192 fp32 rows of config 2" % rows)
+    if name == "linear32":
+        a, w, bias = datagen.c3_linear(32)
+        weff = orc.bfp_unpack(orc.bfp_pack(w.numpy(), 8), w.shape, 8)
+        an, bn = a.float().numpy(), bias.float().numpy()
+        K, N = w.shape
+        nbytes = (K // 32) * (N // 32) * 1088 + 2 * 32 * K + 2 * 32 * N + 2 * N
+        return entry_(nbytes, timed(lambda: orc.linear(an, weff, bn, "gelu", rowstream=True)), "GB/s",
+                      "oracle scalar f32 linear+bias+GELU, all 32 rows of config 3 (weight bytes counted as bfp8_b tiles)")
+    if name == "sdpa2048":
+        q = rng.standard_normal((1, 1, 2048, 128), dtype=np.float32)
+        k = rng.standard_normal((1, 1, 2048, 128), dtype=np.float32)
+        v = rng.standard_normal((1, 1, 2048, 128), dtype=np.float32)
+        flop = 4.0 * 2048 * 2048 * 128 / 2
+        return entry_(flop, timed(lambda: orc.sdpa(q, k, v, None, is_causal=True)), "TFLOP/s", "oracle causal SDPA, one of the 32 heads of config 5 (FLOPs of the causal triangle)")
+    if name == "sdpa_decode32":
+        users, H, Hkv, S, D = 4, 32, 8, 2048, 128
+        q = rng.standard_normal((1, users, H, D), dtype=np.float32)
+        k = rng.standard_normal((users, Hkv, S, D), dtype=np.float32)
+        v = rng.standard_normal((users, Hkv, S, D), dtype=np.float32)
+        pos = np.full((users,), S - 1, dtype=np.int32)
+        nbytes = 2 * users * Hkv * S * D * 2 + 2 * users * H * D * 2
+        return entry_(nbytes, timed(lambda: orc.sdpa_decode(q, k, v, cur_pos=pos)), "GB/s", "oracle decode attention, 4 of the 32 users (cache bytes counted as bf16)")
+    if name == "rmsnorm2048":
+        x = rng.standard_normal((2048, 4096), dtype=np.float32)
+        w = rng.standard_normal((4096,), dtype=np.float32)
+        return entry_(2 * 2048 * 4096 * 2 + 4096 * 2, timed(lambda: orc.rms_norm(x, w, None, 1e-5)), "GB/s", "oracle RMSNorm of [2048, 4096] (bytes counted as bf16)")
+    if name == "softmax65536":
+        x = rng.standard_normal((4096, 2048), dtype=np.float32)
+        return entry_(2 * x.nbytes, timed(lambda: orc.softmax(x, -1)), "GB/s", "oracle softmax over 4096 of the 65536 rows of 2048 fp32")
+    if name == "reduce65536":
+        x = rng.standard_normal((8192, 2048), dtype=np.float32)
+        return entry_(x.nbytes + 8192 * 32 * 4, timed(lambda: orc.reduce("sum", x, -1, True)), "GB/s", "oracle sum over 8192 of the 65536 rows of 2048 fp32")
+    if name == "silu_mul512":
+        g = rng.standard_normal((512, 14336), dtype=np.float32)
+        u = rng.standard_normal((512, 14336), dtype=np.float32)
+        return entry_(3 * 512 * 14336 * 2, timed(lambda: orc.binary("multiply", orc.round_bf16(orc.unary("silu", g)), u)), "GB/s",
+                      "oracle SiLU(gate) * up on [512, 14336] (bytes counted as bf16)")
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -576,6 +648,10 @@ def main():
         else:
             result["cpu_baseline"] = cpu_baseline_pack(orc, datagen)
         result["cpu_baseline_pack_bfp8"] = cpu_baseline_pack(orc, datagen)
+        for e in secondary:   # the same path on the host cores, on a bounded sample of every kernel workload
+            cb = cpu_baseline_secondary(orc, datagen, e["workload"])
+            if cb is not None:
+                e["cpu_baseline"] = cb
     print(json.dumps(result))
 
 
