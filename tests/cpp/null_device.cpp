@@ -414,6 +414,23 @@ EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_
   });
 }
 // the predicates of the real library at its default options
+EXPORT int ttm_linear_glu_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
+  const int64_t groups = ((N + 31) / 32 + 1) / 2, kt = (K + 31) / 32;
+  return block_float(w_dtype) && M >= 1 && M <= 32 && K > 0 && N >= 1 && std::min<int64_t>(256 / groups, kt / 32) <= 1;
+}
+EXPORT int ttm_linear_glu(const void *a, const void *w_gate, const void *w_up, int w_dtype, void *out, int64_t M, int64_t N, int64_t K, int act_gate,
+                          int act_up, void *) {
+  if (!ttm_linear_glu_supported(w_dtype, M, N, K)) return fail("ttm_linear_glu: unsupported shape");
+  EXT(linear_glu, a, w_gate, w_up, w_dtype, out, M, N, K);
+  return launch([=] {
+    // the op sequence it stands for: the gate projection stored as bf16 tiles, then the up projection with the multiply as its tail
+    std::vector<uint8_t> gate(static_cast<size_t>(((M + 31) / 32) * ((N + 31) / 32)) * 2048);
+    store_dense(linear_host(a, w_gate, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, N, K, act_gate, TTM_TAIL_NONE, nullptr), gate.data(), TTM_BF16,
+                TTM_TILE, 1, M, N);
+    store_dense(linear_host(a, w_up, w_dtype, 0, nullptr, TTM_BF16, TTM_TILE, 1, 1, M, N, K, act_up, TTM_TAIL_MUL, gate.data()), out, TTM_BF16, TTM_TILE, 1,
+                M, N);
+  });
+}
 EXPORT int ttm_linear_add_rms_norm_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
   return block_float(w_dtype) && M >= 1 && M <= 32 && K > 0 && N >= 1 && (N + 31) / 32 * 4 <= 8 * 256;
 }

@@ -520,3 +520,48 @@ def test_linear_add_rms_norm_equals_the_op_sequence(hip, dev, orc, M, K, N, fmt,
     with pytest.raises(hip.TTMError, match="must not alias"):
         hip.call("ttm_linear_add_rms_norm", hip.ptr(at), hip.ptr(wt), wf, hip.ptr(rt_), hip.ptr(rt_), None, hip.TILE, None, hip.TILE, 1e-5,
                  hip.ptr(hf), M, N, K, s)
+
+
+@pytest.mark.parametrize("M,K,N,fmt,acts", [
+    (32, 4096, 14336, "bfp8", ("silu", None)),     # gate and up of the Llama-3-8B decode step
+    (32, 4096, 14336, "bfp4", ("silu", None)),
+    (7, 256, 1000, "bfp8", ("gelu", "relu")),      # ragged rows and columns, an odd number of column tiles
+    (1, 512, 96, "bfp4", (None, "sigmoid")),
+    (32, 1024, 8224, "bfp8", ("silu", None)),      # 129 column pairs: the first width at which K = 1024 is not split
+])
+def test_linear_glu_equals_the_op_sequence(hip, dev, orc, M, K, N, fmt, acts):
+    """ttm_linear_glu against ttm_linear (gate) followed by ttm_linear_tail (up, multiply): bit-identical, padding rows of the
+    output left alone; and against the CPU oracle's linear + multiply with the three bf16 roundings."""
+    from test_gpu_linear import pack_weight
+    wf = hip.BFP8B if fmt == "bfp8" else hip.BFP4B
+    a = datagen.randn((M, K), seed=120, dtype=torch.bfloat16)
+    wg = datagen.randn((K, N), seed=121, dtype=torch.float32) * 0.05
+    wu = datagen.randn((K, N), seed=122, dtype=torch.float32) * 0.05
+    at, wgt, wut = tilize_dev(hip, a, dev), pack_weight(hip, wg, wf, dev), pack_weight(hip, wu, wf, dev)
+    s = hip.current_stream()
+    Np = (N + 31) // 32 * 32
+    gate = torch.zeros((32 * Np,), dtype=torch.bfloat16, device=dev)
+    want = torch.zeros_like(gate)
+    hip.call("ttm_linear", hip.ptr(at), hip.BF16, hip.ptr(wgt), wf, 0, None, hip.BF16, hip.TILE, hip.ptr(gate), hip.BF16, 1, 1, M, N, K,
+             hip.ACT[acts[0]], s)
+    hip.call("ttm_linear_tail", hip.ptr(at), hip.BF16, hip.ptr(wut), wf, 0, None, hip.BF16, hip.TILE, hip.ptr(want), hip.BF16, 1, 1, M, N, K,
+             hip.ACT[acts[1]], 2, hip.ptr(gate), s)
+    assert hip.lib().ttm_linear_glu_supported(wf, M, N, K) == 1
+    got = torch.zeros_like(want)
+    hip.call("ttm_linear_glu", hip.ptr(at), hip.ptr(wgt), hip.ptr(wut), wf, hip.ptr(got), M, N, K, hip.ACT[acts[0]], hip.ACT[acts[1]], s)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert bool(torch.isfinite(got.float()).all())
+    # the oracle on the weights the device multiplies
+    r = lambda x: orc.round_bf16(x)
+    fmtn = 8 if fmt == "bfp8" else 4
+    q = lambda w_: orc.bfp_unpack(orc.bfp_pack(w_.numpy(), fmtn), w_.shape, fmtn)
+    an = a.float().numpy()
+    ref = r(r(orc.linear(an, q(wg), None, acts[0])) * r(orc.linear(an, q(wu), None, acts[1])))
+    out = untilize_dev(hip, got, (32, Np), dev)[:M, :N].float().cpu().numpy()
+    assert np.max(np.abs(out - ref)) <= 2.0 ** -5 * max(1.0, float(np.max(np.abs(ref))))
+    assert hip.lib().ttm_linear_glu_supported(wf, 33, N, K) == 0 and hip.lib().ttm_linear_glu_supported(hip.BF16, M, N, K) == 0
+    # a width at which one projection alone splits K over workgroups stays with the op sequence
+    assert hip.lib().ttm_linear_glu_supported(wf, 32, 4096, 4096) == 0
+    with pytest.raises(hip.TTMError, match="ttm_linear_glu"):
+        hip.call("ttm_linear_glu", hip.ptr(at), hip.ptr(wgt), hip.ptr(wut), wf, hip.ptr(got), 33, N, K, 0, 0, s)

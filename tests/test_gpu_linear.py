@@ -474,6 +474,9 @@ def test_two_pass_launch_with_batches_pairs_and_tails(hip, dev, orc, metrics):
     (32, 1024, (512, 128, 128), {"linear_decode_split": 2}),       # decode kernel, k-slices, reduction that knows the members
     (20, 520, (200, 72, 72, 40), {"linear_decode_split": 1}),      # ragged everywhere, four members, direct epilogue
     (64, 256, (96, 160), {"linear_decode_split": 3}),              # two row tiles
+    (32, 1024, (512, 128, 128), {"linear_decode_split": 2, "linear_decode_wide": 2}),   # the same with 128 columns per workgroup
+    (20, 520, (200, 72, 72, 40), {"linear_decode_split": 1, "linear_decode_wide": 2}),
+    (64, 256, (96, 160), {"linear_decode_split": 3, "linear_decode_wide": 2}),
     (330, 232, (677, 100, 300), {"linear_split_k": 1, "linear_two_pass": 1}),   # fused main kernel
     (512, 256, (1024, 256, 256), {"linear_split_k": 1, "linear_two_pass": 2}),  # two passes: one image launch for all members
     (2048, 128, (2048, 512, 512), {"linear_split_k": 1, "linear_two_pass": 2, "linear_ntw": 7}),   # 7-wide blocks, several rounds
@@ -508,3 +511,31 @@ def test_linear_group_equals_separate_launches(hip, dev, wfmt_name, M, K, Ns, op
             hip.set_option(k, 0)
     for g, w in zip(got, want):
         assert torch.equal(g, w)
+
+
+@pytest.mark.parametrize("wfmt_name", ["bfp8", "bfp4"])
+@pytest.mark.parametrize("M,K,N,with_bias,act", [
+    (32, 512, 1000, True, "gelu"),       # ragged columns, an even number of column tiles
+    (7, 1024, 96, False, "silu"),        # three column tiles: the last workgroup's second tile pair is half there
+    (32, 256, 32, True, None),           # one column tile
+    (64, 2048, 8256, False, "relu"),     # two row tiles, 129 wide workgroups
+    (32, 4096, 28672, True, "gelu"),     # a width at which the wide form is the default
+])
+def test_decode_kernel_wide_workgroups_equal_narrow_ones(hip, dev, wfmt_name, M, K, N, with_bias, act):
+    """The decode kernel with 128 columns per workgroup (linear_decode_wide = 2) against 64 (= 1), neither splitting K: the
+    same k order per output, bit-identical results; the default picks one of the two."""
+    wfmt = {"bfp8": hip.BFP8B, "bfp4": hip.BFP4B}[wfmt_name]
+    a = datagen.randn((M, K), seed=131, dtype=torch.bfloat16)
+    w = datagen.randn((K, N), seed=132, std=0.05)
+    bias = datagen.randn((1, N), seed=133, dtype=torch.bfloat16) if with_bias else None
+    outs = {}
+    try:
+        hip.set_option("linear_decode_split", 1)
+        for wide in (1, 2, 0):
+            hip.set_option("linear_decode_wide", wide)
+            outs[wide] = run_linear(hip, dev, a, w, bias, act, wfmt)[0]
+    finally:
+        hip.set_option("linear_decode_split", 0)
+        hip.set_option("linear_decode_wide", 0)
+    assert torch.equal(outs[1], outs[2]) and torch.equal(outs[0], outs[1])
+    assert bool(torch.isfinite(outs[2].float()).all())

@@ -903,6 +903,8 @@ def test_decode_layer_steps_eager_and_traced(device, orc, metrics):
         assert rt.get_stat("FusedHeadConcat") == qkv
         # the output projection, its residual add and the RMSNorm in front of the MLP are one fused step as well
         assert rt.get_stat("FusedLinearAddNorm") == qkv
+        # and the gate and up projections with the multiply that joins them
+        assert rt.get_stat("FusedLinearGlu") == qkv
     # the replayed graph runs the same kernels on the same data: identical to the op-by-op run, caches included; so is
     # the unfused run
     for other in ("traced", "callbacks"):

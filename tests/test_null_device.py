@@ -129,7 +129,7 @@ for mode in ("eager", "traced", "callbacks"):
         assert tuple(rt.to_host(y, untilize=True)[0].shape) == (1, users, hidden) or True
     rt.clear_callbacks()
     stats[mode] = {k: rt.get_stat(k) for k in ("CapturedTrace", "FusedCopyIntoSlot", "FusedQkvDecode", "FusedCacheUpdate", "FusedHeadSplit",
-                                               "GroupedMatmul", "FusedHeadConcat", "FusedLinearAddNorm", "ConstEvalCacheMiss", "ConstEvalCacheHit")}
+                                               "GroupedMatmul", "FusedHeadConcat", "FusedLinearAddNorm", "FusedLinearGlu", "ConstEvalCacheMiss", "ConstEvalCacheHit")}
 rt.close_mesh_device(device)
 print(json.dumps(stats))
 """ % (ROOT, ROOT)
@@ -140,7 +140,7 @@ print(json.dumps(stats))
         s = st[mode]
         assert s["FusedCopyIntoSlot"] == (2 if mode == "traced" else 0), (mode, s)
         assert s["FusedCacheUpdate"] == 0 and s["FusedHeadSplit"] == 0 and s["GroupedMatmul"] == 0, (mode, s)
-        assert s["FusedHeadConcat"] == s["FusedQkvDecode"] == s["FusedLinearAddNorm"], (mode, s)
+        assert s["FusedHeadConcat"] == s["FusedQkvDecode"] == s["FusedLinearAddNorm"] == s["FusedLinearGlu"], (mode, s)
     assert st["eager"]["FusedQkvDecode"] == 3 and st["callbacks"]["FusedQkvDecode"] == 0
     assert st["traced"]["CapturedTrace"] >= 1 and st["traced"]["FusedQkvDecode"] in (1, 2)
 
@@ -255,7 +255,7 @@ from ttmlir_amd import programs, runtime as rt
 DT = rt.DataType
 npdt = {DT.BFloat16: np.uint16, DT.Float32: np.float32, DT.Int32: np.int32, DT.UInt32: np.uint32}
 dev = rt.open_mesh_device()
-keys = ("GroupedMatmul", "FusedLinearTail", "FusedQkvDecode", "FusedLinearAddNorm", "FusedHeadConcat", "CapturedTrace", "ConstEvalCacheMiss", "ConstEvalCacheHit")
+keys = ("GroupedMatmul", "FusedLinearTail", "FusedQkvDecode", "FusedLinearAddNorm", "FusedLinearGlu", "FusedHeadConcat", "CapturedTrace", "ConstEvalCacheMiss", "ConstEvalCacheHit")
 report = {}
 def run(name, data, steps=1):
     b = rt.Binary.load_from_memory(data)
@@ -285,9 +285,10 @@ print(json.dumps(report))
     assert rep["c5"]["GroupedMatmul"] == 1 and rep["c5"]["FusedLinearTail"] == 3               # two residual adds and SiLU(gate) * up
     d = rep["decode32"]                                                                         # three steps
     assert d["shapes"] == [[32, 4096]] and d["FusedQkvDecode"] == 3 and d["FusedLinearAddNorm"] == 3 and d["FusedHeadConcat"] == 3
+    assert d["FusedLinearGlu"] == 3 and d["FusedLinearTail"] == 6                               # gate, up and their product; the two residual adds
     assert d["ConstEvalCacheMiss"] == 1 and d["ConstEvalCacheHit"] == 2
     t = rep["decode32_traced"]                                                                  # eager run + recording, then replays
-    assert t["CapturedTrace"] == 1 and t["FusedQkvDecode"] == 2 and t["FusedLinearAddNorm"] == 2
+    assert t["CapturedTrace"] == 1 and t["FusedQkvDecode"] == 2 and t["FusedLinearAddNorm"] == 2 and t["FusedLinearGlu"] == 2
 
 
 def test_const_eval_entries_live_as_long_as_their_inputs(null_env):

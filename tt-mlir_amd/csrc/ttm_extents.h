@@ -136,6 +136,14 @@ int linear_pair(Span &&span, const void *a, const void *w0, const void *w1, int 
   return 0;
 }
 template <class Span>
+int linear_glu(Span &&span, const void *a, const void *w_gate, const void *w_up, int w_dtype, void *out, int64_t M, int64_t N, int64_t K) {
+  TTM_EXT(span("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K), false));
+  TTM_EXT(span("gate weights [K, N]", w_gate, tile_bytes(w_dtype, 1, K, N), false));
+  TTM_EXT(span("up weights [K, N]", w_up, tile_bytes(w_dtype, 1, K, N), false));
+  TTM_EXT(span("output [M, N]", out, tile_bytes(TTM_BF16, 1, M, N), false));
+  return 0;
+}
+template <class Span>
 int linear_add_rms_norm(Span &&span, const void *a, const void *w, int w_dtype, const void *residual, void *sum_out, const void *norm_weight,
                         int weight_layout, const void *norm_bias, int bias_layout, void *norm_out, int64_t M, int64_t N, int64_t K) {
   TTM_EXT(span("activations [M, K]", a, tile_bytes(TTM_BF16, 1, M, K), false));

@@ -54,6 +54,7 @@ struct LinearArgs {
   uint8_t *gC[4];
   int gNt[4];
   int gAct[4];                        // per-member activation
+  int glu;                            // gated pair (decode kernel only): C = gC[0] = act0(A gW[0]) x act1(A gW[1]), both [K, gNt[0] * 32]
   int tail;                           // 0 none, 1 add, 2 multiply: element-wise tail with a tensor laid out like the output
   int64_t tail_delta;                 // byte distance from an output element to its tail operand
   const struct QkvFinishArgs *qkv;    // host side only: the decode launch leaves partial sums and ttm_qkv_finish_k ends it
@@ -1637,9 +1638,9 @@ typedef float f32x4v __attribute__((ext_vector_type(4)));
 // or steps, V and S go through the matrix cores into two accumulators, and the result is their difference: twice the
 // MFMAs (which were idle) for less than half the vector instructions.  The two sums are each a few times larger than
 // their difference, so the fp32 rounding error grows by that factor - still four decimal orders below a bf16 result.
-template <bool BFP4, bool TWO_TERM>
+template <bool BFP4, bool TWO_TERM, int NP, bool GLU>
 __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
-  extern __shared__ u32x4 smem[];   // partial sums: 8 wavefronts x 8 x 64 float4 = 64 KiB
+  extern __shared__ u32x4 smem[];   // partial sums: NP x 8 wavefronts x 8 x 64 float4 = NP x 64 KiB
   constexpr int D = 2;
   constexpr uint32_t TB = BFP4 ? 576u : 1088u, FACE = BFP4 ? 128u : 256u, ROW = BFP4 ? 8u : 16u;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -1648,25 +1649,35 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
   const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
   uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
-  if (p.group_n > 1) {   // workgroup-uniform
-    const GroupMember m = group_member(p, cg, 2);
+  static_assert(!GLU || NP == 2, "the gated form multiplies the two tile pairs of a workgroup");
+  if constexpr (GLU) {
+    W = p.gW[0]; C = p.gC[0]; Nt = p.gNt[0];
+  } else if (p.group_n > 1) {   // workgroup-uniform
+    const GroupMember m = group_member(p, cg, 2 * NP);
     W = m.W; C = m.C; Nt = m.Nt; cg = m.local; tile_base = m.tile_base; act = m.act;
   }
+  const uint8_t *W2 = GLU ? p.gW[1] : W;   // GLU: tile pair 1 is the same column pair of the second matrix
   const int q16 = lane & 15, kg = lane >> 4;   // weight operand row and 8-k group of this lane
   const int fc = (q16 >> 2) & 1, quad = q16 & 3, fr = kg >> 1, half = kg & 1;
-  const uint32_t nt_l = (uint32_t)min(2 * cg + (q16 >> 3), Nt - 1);
-  const uint32_t offW = nt_l * TB + 64u + (fr * 2 + fc) * FACE + half * (FACE / 2) + quad * (ROW / 4);   // + ROW i
-  const uint32_t offE = nt_l * TB + (fr * 2 + fc) * 16 + half * 8;
+  uint32_t offW[NP], offE[NP];   // tile pair pr of the workgroup: column tiles 2 NP cg + 2 pr, + 1
+#pragma unroll
+  for (int pr = 0; pr < NP; ++pr) {
+    const uint32_t nt_l = (uint32_t)min(GLU ? 2 * cg + (q16 >> 3) : 2 * NP * cg + 2 * pr + (q16 >> 3), Nt - 1);
+    offW[pr] = nt_l * TB + 64u + (fr * 2 + fc) * FACE + half * (FACE / 2) + quad * (ROW / 4);   // + ROW i
+    offE[pr] = nt_l * TB + (fr * 2 + fc) * 16 + half * 8;
+  }
   const uint32_t offA = fr * 512 + q16 * 32 + half * 16;                                     // + 1024 h
 
-  f32x4v acc[2][4], accs[2][4];   // accs: the sum over the S terms (TWO_TERM)
+  f32x4v acc[NP][2][4], accs[NP][2][4];   // accs: the sum over the S terms (TWO_TERM)
 #pragma unroll
-  for (int h = 0; h < 2; ++h)
+  for (int pr = 0; pr < NP; ++pr)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[h][j] = accs[h][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[pr][h][j] = accs[pr][h][j] = f32x4v{0.f, 0.f, 0.f, 0.f};
 
-  uint32_t rows[D][8], keeps[D];
-  u32x2 ex[D];
+  uint32_t rows[D][NP][8], keeps[D];
+  u32x2 ex[D][NP];
   u32x4 af[D][2];
   // split-K: workgroup y of the grid takes k-tiles [y k_slice, (y + 1) k_slice) and leaves fp32 partial sums
   const int kbase = p.partial ? (int)blockIdx.y * p.k_slice : 0;
@@ -1676,34 +1687,38 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
     const int kt = kbase + wave + 8 * c;
     const int ktc = min(kt, kend - 1);
     const uint32_t keep = kt < kend ? 0xFFFFFFFFu : 0u;   // past the end: zero exponents, zero weights
-    const uint8_t *Wk = W + (int64_t)ktc * Nt * TB;
+    const uint8_t *Wk0 = W + (int64_t)ktc * Nt * TB, *Wk1 = W2 + (int64_t)ktc * Nt * TB;
     const uint8_t *Ak = A + (int64_t)ktc * 2048;
 #pragma unroll
-    for (int i = 0; i < 8; ++i)   // the eight loads share their cache lines: cached loads
-      rows[s][i] = BFP4 ? (uint32_t) * (const uint16_t *)(Wk + offW + i * ROW) : *(const uint32_t *)(Wk + offW + i * ROW);
-    ex[s] = *(const u32x2 *)(Wk + offE);
+    for (int pr = 0; pr < NP; ++pr) {
+      const uint8_t *Wk = pr == 0 ? Wk0 : Wk1;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)   // the eight loads share their cache lines: cached loads
+        rows[s][pr][i] = BFP4 ? (uint32_t) * (const uint16_t *)(Wk + offW[pr] + i * ROW) : *(const uint32_t *)(Wk + offW[pr] + i * ROW);
+      ex[s][pr] = *(const u32x2 *)(Wk + offE[pr]);
+    }
     keeps[s] = keep;   // applied when the slot is consumed: masking here would wait for the load
 #pragma unroll
     for (int h = 0; h < 2; ++h) af[s][h] = *(const u32x4 *)(Ak + offA + h * 1024);
   };
-  auto process = [&](int s) {
+  auto process_pair = [&](int s, int pr) __attribute__((always_inline)) {
     if constexpr (TWO_TERM) {
       if (keeps[s] == 0u) return;   // wavefront-uniform: a k-tile past the end contributes nothing
       // (E + 1) << 7 for the rows 2 ip and 2 ip + 1, in the two halves of a word; E is capped so that the field stays 8 bits
       uint32_t epk[4];
 #pragma unroll
       for (int ip = 0; ip < 4; ++ip) {
-        const uint32_t src = ip < 2 ? ex[s].x : ex[s].y;
+        const uint32_t src = ip < 2 ? ex[s][pr].x : ex[s][pr].y;
         uint32_t e2 = __builtin_amdgcn_perm(0u, src, (ip & 1) ? 0x0c030c02u : 0x0c010c00u);
         typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
         const u16x2 capped = __builtin_elementwise_min(*(const u16x2 *)&e2, u16x2{0xFD, 0xFD});
         e2 = *(const uint32_t *)&capped;
         epk[ip] = (e2 + 0x00010001u) << 7;
       }
-      uint32_t pr[4] = {0u, 0u, 0u, 0u};
+      uint32_t pk[4] = {0u, 0u, 0u, 0u};
       if constexpr (BFP4) {
 #pragma unroll
-        for (int ip = 0; ip < 4; ++ip) pr[ip] = rows[s][2 * ip] | (rows[s][2 * ip + 1] << 16);   // four nibbles per row
+        for (int ip = 0; ip < 4; ++ip) pk[ip] = rows[s][pr][2 * ip] | (rows[s][pr][2 * ip + 1] << 16);   // four nibbles per row
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -1712,11 +1727,11 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
         for (int ip = 0; ip < 4; ++ip) {
           uint32_t sb, v;
           if constexpr (BFP4) {
-            const uint32_t q = pr[ip] >> (4 * j);            // nibble j of either row in bits 0..3 and 16..19
+            const uint32_t q = pk[ip] >> (4 * j);            // nibble j of either row in bits 0..3 and 16..19
             sb = ((q & 0x00080008u) << 12) | epk[ip];
             v = ((q & 0x00070007u) << 4) | sb;
           } else {
-            const uint32_t q = __builtin_amdgcn_perm(rows[s][2 * ip + 1], rows[s][2 * ip], 0x0c040c00u + 0x00010001u * j);
+            const uint32_t q = __builtin_amdgcn_perm(rows[s][pr][2 * ip + 1], rows[s][pr][2 * ip], 0x0c040c00u + 0x00010001u * j);
             sb = ((q & 0x00800080u) << 8) | epk[ip];
             v = (q & 0x007F007Fu) | sb;
           }
@@ -1725,8 +1740,8 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
         }
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&wv, *(bf16x8 *)&af[s][h], acc[h][j], 0, 0, 0);
-          accs[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&ws, *(bf16x8 *)&af[s][h], accs[h][j], 0, 0, 0);
+          acc[pr][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&wv, *(bf16x8 *)&af[s][h], acc[pr][h][j], 0, 0, 0);
+          accs[pr][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&ws, *(bf16x8 *)&af[s][h], accs[pr][h][j], 0, 0, 0);
         }
       }
       return;
@@ -1734,12 +1749,12 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
     float f[8][4];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      uint32_t E = (((i < 4 ? ex[s].x : ex[s].y) & keeps[s]) >> (8 * (i & 3))) & 0xFFu;
+      uint32_t E = (((i < 4 ? ex[s][pr].x : ex[s][pr].y) & keeps[s]) >> (8 * (i & 3))) & 0xFFu;
       // value = magnitude x 2^(E - 127 - 6) (bfp8_b) or 2^(E - 127 - 2) (bfp4_b); smaller exponents flush to zero
       constexpr uint32_t EB = BFP4 ? 2u : 6u, SIGN = BFP4 ? 0x08080808u : 0x80808080u, SH = BFP4 ? 3u : 7u;
       E = max(E, EB);
       const float scale = __uint_as_float((E - EB) << 23), nscale = (BFP4 ? -8.0f : -128.0f) * scale;
-      uint32_t d = rows[s][i];
+      uint32_t d = rows[s][pr][i];
       if (BFP4) {   // nibbles n3 n2 n1 n0 of the low half -> one per byte
         d = (d | (d << 8)) & 0x00FF00FFu;
         d = (d | (d << 4)) & 0x0F0F0F0Fu;
@@ -1754,8 +1769,12 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
       u32x4 w = {pack_hi(f[0][j], f[1][j]), pack_hi(f[2][j], f[3][j]), pack_hi(f[4][j], f[5][j]), pack_hi(f[6][j], f[7][j])};
 #pragma unroll
       for (int h = 0; h < 2; ++h)
-        acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&w, *(bf16x8 *)&af[s][h], acc[h][j], 0, 0, 0);
+        acc[pr][h][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*(bf16x8 *)&w, *(bf16x8 *)&af[s][h], acc[pr][h][j], 0, 0, 0);
     }
+  };
+  auto process = [&](int s) __attribute__((always_inline)) {
+#pragma unroll
+    for (int pr = 0; pr < NP; ++pr) process_pair(s, pr);
   };
 #pragma unroll
   for (int s = 0; s < D; ++s) {
@@ -1776,31 +1795,73 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
 
   if constexpr (TWO_TERM) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int pr = 0; pr < NP; ++pr)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[h][j] -= accs[h][j];
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[pr][h][j] -= accs[pr][h][j];
   }
-  // partial sums -> LDS as float4 (four consecutive n of one m): slot ((wave * 8 + h * 4 + i) * 64 + lane)
+  // partial sums -> LDS as float4 (four consecutive n of one m): slot (((pr * 8 + wave) * 8 + h * 4 + i) * 64 + lane)
   f32x4v *part = (f32x4v *)smem;
 #pragma unroll
-  for (int h = 0; h < 2; ++h)
+  for (int pr = 0; pr < NP; ++pr)
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      part[(wave * 8 + h * 4 + i) * 64 + lane] = f32x4v{acc[h][0][i], acc[h][1][i], acc[h][2][i], acc[h][3][i]};
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        part[((pr * 8 + wave) * 8 + h * 4 + i) * 64 + lane] = f32x4v{acc[pr][h][0][i], acc[pr][h][1][i], acc[pr][h][2][i], acc[pr][h][3][i]};
   __syncthreads();
-  // thread t finishes slot t of the 512: (h, i, lane) = (t >> 8, (t >> 6) & 3, t & 63)
-  f32x4v sum = part[tid];
-#pragma unroll
-  for (int w = 1; w < 8; ++w) sum += part[w * 512 + tid];
   const int h = tid >> 8, i = (tid >> 6) & 3;
-  const int nt = 2 * cg + (kg >> 1);
-  if (nt >= Nt) return;
+  if constexpr (GLU) {
+    // thread t holds the same four outputs of both matrices: out = bf16(bf16(act0(gate)) x bf16(act1(up))), the roundings
+    // of the two projections stored by themselves and of the multiply that would read them
+    f32x4v s0 = part[tid], s1 = part[4096 + tid];
+#pragma unroll
+    for (int w = 1; w < 8; ++w) { s0 += part[w * 512 + tid]; s1 += part[4096 + w * 512 + tid]; }
+    const int nt = 2 * cg + (kg >> 1);
+    if (nt >= Nt) return;
+    const int n_in = 16 * (kg & 1) + 4 * i;
+    const int64_t off = (int64_t)nt * 1024 + (h * 2 + (n_in >> 4)) * 256 + q16 * 16 + (n_in & 15);
+    float v0[4], v1[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float x = s0[r], y = s1[r];
+      switch (p.gAct[0]) {
+      case TTM_ACT_GELU: x = apply_act<TTM_ACT_GELU>(x); break;
+      case TTM_ACT_SILU: x = apply_act<TTM_ACT_SILU>(x); break;
+      case TTM_ACT_SIGMOID: x = apply_act<TTM_ACT_SIGMOID>(x); break;
+      case TTM_ACT_RELU: x = apply_act<TTM_ACT_RELU>(x); break;
+      default: break;
+      }
+      switch (p.gAct[1]) {
+      case TTM_ACT_GELU: y = apply_act<TTM_ACT_GELU>(y); break;
+      case TTM_ACT_SILU: y = apply_act<TTM_ACT_SILU>(y); break;
+      case TTM_ACT_SIGMOID: y = apply_act<TTM_ACT_SIGMOID>(y); break;
+      case TTM_ACT_RELU: y = apply_act<TTM_ACT_RELU>(y); break;
+      default: break;
+      }
+      v0[r] = x; v1[r] = y;
+    }
+    const u32x2 g = {pack_bf16(v0[0], v0[1]), pack_bf16(v0[2], v0[3])}, u = {pack_bf16(v1[0], v1[1]), pack_bf16(v1[2], v1[3])};
+    const float z[4] = {__uint_as_float(g.x << 16) * __uint_as_float(u.x << 16), __uint_as_float(g.x & 0xFFFF0000u) * __uint_as_float(u.x & 0xFFFF0000u),
+                        __uint_as_float(g.y << 16) * __uint_as_float(u.y << 16), __uint_as_float(g.y & 0xFFFF0000u) * __uint_as_float(u.y & 0xFFFF0000u)};
+    *(u32x2 *)(C + off * 2) = u32x2{pack_bf16(z[0], z[1]), pack_bf16(z[2], z[3])};
+    return;
+  }
+#pragma unroll
+  for (int pr = 0; pr < NP; ++pr) {
+  // thread t finishes slot t of the pair's 512: (h, i, lane) = (t >> 8, (t >> 6) & 3, t & 63)
+  f32x4v sum = part[pr * 4096 + tid];
+#pragma unroll
+  for (int w = 1; w < 8; ++w) sum += part[pr * 4096 + w * 512 + tid];
+  const int nt = 2 * NP * cg + 2 * pr + (kg >> 1);
+  if (nt >= Nt) continue;
   const int n_in = 16 * (kg & 1) + 4 * i;
   const int64_t off = (int64_t)nt * 1024 + (h * 2 + (n_in >> 4)) * 256 + q16 * 16 + (n_in & 15);
   if (p.partial) {   // bias, activation and rounding happen in ttm_linear_reduce_k
     const int64_t per = (int64_t)p.Nt * 1024;   // a group's partial sums are laid out as the concatenation
     *(f32x4v *)(p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * per + (int64_t)tile_base * 1024 + off) = sum;
-    return;
+    continue;
   }
   float bv[4] = {0.f, 0.f, 0.f, 0.f};
   if (p.bias) {
@@ -1823,6 +1884,7 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
     v[r] = x;
   }
   *(u32x2 *)(C + off * 2) = finish_quad(p, C + off * 2, v);
+  }
 }
 
 // Ends the decode step's Q / K / V launch.  One lane per four consecutive columns of one user: sums the k-slices, rounds to
@@ -1973,12 +2035,29 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
     // as long as a slice keeps 32 k-tiles (four per wavefront, the depth of its load ring); the slices leave fp32
     // partial sums that ttm_linear_reduce_k finishes.  Measured at M = 32: [4096, 4096] 14.3 -> 10.6 us,
     // [14336, 4096] 38 -> 19 us with 4 slices; 8 slices or splitting a [4096, 14336] weight are slower than not splitting.
-    int slices = 1;
+    int slices = 1, np = 1;
+    int64_t units = a.Nt;   // workgroups along the columns
+    if (a.glu && !decode) return ttm_set_error(TTM_ERR_INVALID, "ttm_linear_glu: the selected kernel variant has no gated form");
     if (decode) {
-      const int64_t groups = (int64_t)column_units(a, 2) * batch;
-      slices = ttm_option("linear_decode_split");
+      const int cus = device_cu_count();
+      if (a.glu) {   // a workgroup's two tile pairs are the same 64 columns of the two matrices
+        np = 2;
+        units = (a.gNt[0] + 1) / 2;
+      } else {
+        // A workgroup owns 64 columns, or 128 (linear_decode_wide: 0 = by the rule, 1 = never, 2 = always): the wide form reads
+        // the activations once per 128 columns and fills a CU with one workgroup where the narrow form needs two, which pays
+        // when it also rounds better to whole rounds of the device.  Measured at M = 32, K = 4096 (narrow / wide, us):
+        // N = 28672 30.7 / 27.3, 32000 31.3 / 28.3, 43008 44.3 / 50.0, 57344 57.3 / 53.3, 128256 121.3 / 114.7; one round of
+        // wide workgroups costs 1.8 narrow ones.  Launches that split K stay narrow (N = 14336 in two slices: 17.3 against 16.1 us).
+        const int wide = ttm_option("linear_decode_wide");
+        const int64_t gn = (int64_t)column_units(a, 2) * batch, gw = (int64_t)column_units(a, 4) * batch;
+        np = wide == 2 || (wide == 0 && gn >= cus && ((gw + cus - 1) / cus) * 9 < ((gn + cus - 1) / cus) * 5) ? 2 : 1;
+        units = column_units(a, 2 * np);
+      }
+      const int64_t groups = units * batch;
+      slices = a.glu ? 1 : ttm_option("linear_decode_split");
       if (slices <= 0) {
-        slices = (int)(device_cu_count() / groups);
+        slices = (int)(cus / groups);
         if (slices > a.Kt / 32) slices = a.Kt / 32;
       }
       if (slices > a.Kt) slices = a.Kt;
@@ -2001,14 +2080,26 @@ static int launch_linear(const LinearArgs &a, int64_t batch, hipStream_t s) {
       p.A = a.A + (int64_t)mt * a.Kt * 2048;
       p.C = a.C + (int64_t)mt * a.Nt * 2048;
       for (int j = 0; j < a.group_n; ++j) p.gC[j] = a.gC[j] + (int64_t)mt * a.gNt[j] * 2048;
-      const dim3 grid(column_units(a, 2), slices, (unsigned)batch);
+      const dim3 grid((unsigned)units, slices, (unsigned)batch);
       const bool two_term = ttm_option("linear_decode_variant") != 1;   // 1 = operands by int -> float conversion
-      if (decode && WF == WF_BFP4) {
-        if (two_term) hipLaunchKernelGGL((ttm_linear_decode_k<true, true>), grid, dim3(512), 65536, s, p);
-        else hipLaunchKernelGGL((ttm_linear_decode_k<true, false>), grid, dim3(512), 65536, s, p);
-      } else if (decode) {
-        if (two_term) hipLaunchKernelGGL((ttm_linear_decode_k<false, true>), grid, dim3(512), 65536, s, p);
-        else hipLaunchKernelGGL((ttm_linear_decode_k<false, false>), grid, dim3(512), 65536, s, p);
+      if (decode) {
+        constexpr bool B4 = WF == WF_BFP4;
+        if (np == 2) {
+          static bool attr = false;
+          if (!attr) {
+            if (int rc = set_lds_limit(ttm_linear_decode_k<B4, true, 2, false>, 131072)) return rc;
+            if (int rc = set_lds_limit(ttm_linear_decode_k<B4, false, 2, false>, 131072)) return rc;
+            if (int rc = set_lds_limit(ttm_linear_decode_k<B4, true, 2, true>, 131072)) return rc;
+            if (int rc = set_lds_limit(ttm_linear_decode_k<B4, false, 2, true>, 131072)) return rc;
+            attr = true;
+          }
+          if (a.glu) {
+            if (two_term) hipLaunchKernelGGL((ttm_linear_decode_k<B4, true, 2, true>), grid, dim3(512), 131072, s, p);
+            else hipLaunchKernelGGL((ttm_linear_decode_k<B4, false, 2, true>), grid, dim3(512), 131072, s, p);
+          } else if (two_term) hipLaunchKernelGGL((ttm_linear_decode_k<B4, true, 2, false>), grid, dim3(512), 131072, s, p);
+          else hipLaunchKernelGGL((ttm_linear_decode_k<B4, false, 2, false>), grid, dim3(512), 131072, s, p);
+        } else if (two_term) hipLaunchKernelGGL((ttm_linear_decode_k<B4, true, 1, false>), grid, dim3(512), 65536, s, p);
+        else hipLaunchKernelGGL((ttm_linear_decode_k<B4, false, 1, false>), grid, dim3(512), 65536, s, p);
       }
       else hipLaunchKernelGGL((ttm_linear_small_k<WF>), dim3(a.Nt, 1, (unsigned)batch), dim3(256), 0, s, p);
       if (a.qkv) {
@@ -2204,7 +2295,7 @@ static int linear_entry(const void *a, int a_dtype, const void *w, int w_dtype, 
   p.k_slice = p.Kt; p.partial = nullptr;
   p.nt_split = p.n_blocks1 = p.ntw2 = 0;
   p.img_zero_step = 0;
-  p.group_n = 0;
+  p.group_n = 0; p.glu = 0;
   for (int j = 0; j < 4; ++j) { p.gW[j] = nullptr; p.gC[j] = nullptr; p.gNt[j] = 0; p.gAct[j] = TTM_ACT_NONE; }
   p.tail = tail_op;
   p.tail_delta = tail ? (const uint8_t *)tail - (const uint8_t *)out : 0;
@@ -2260,6 +2351,52 @@ TTM_EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, in
                       TTM_TAIL_NONE, nullptr, strides, stream);
 }
 
+// The rule of launch_linear for a single projection of this shape: does the decode kernel run it unsplit?
+static bool decode_runs_unsplit(int64_t N, int64_t K) {
+  const int64_t groups = (ttm_cdiv(N, 32) + 1) / 2, kt = ttm_cdiv(K, 32);
+  int64_t slices = ttm_option("linear_decode_split");
+  if (slices <= 0) slices = std::min<int64_t>(device_cu_count() / groups, kt / 32);
+  return slices <= 1;
+}
+
+TTM_EXPORT int ttm_linear_glu_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
+  return (w_dtype == TTM_BFP8B || w_dtype == TTM_BFP4B) && M >= 1 && M <= 32 && K > 0 && N >= 1 && ttm_option("linear_variant") != 1 &&
+         ttm_option("linear_decode_wide") != 1 && ttm_option("linear_small_m_max") >= 32 && ttm_cdiv(N, 32) * 1088 < (int64_t)1 << 32 &&
+         decode_runs_unsplit(N, K);
+}
+
+TTM_EXPORT int ttm_linear_glu(const void *a, const void *w_gate, const void *w_up, int w_dtype, void *out, int64_t M, int64_t N, int64_t K,
+                              int act_gate, int act_up, void *stream) {
+  TTM_EXTENTS(linear_glu, a, w_gate, w_up, w_dtype, out, M, N, K);
+  TTM_REQUIRE(ttm_linear_glu_supported(w_dtype, M, N, K),
+              "ttm_linear_glu: needs block-float weights, 1..32 rows and enough columns for the decode kernel to run unsplit");
+  TTM_REQUIRE(a && w_gate && w_up && out, "ttm_linear_glu: null pointer");
+  TTM_REQUIRE((((uintptr_t)a | (uintptr_t)w_gate | (uintptr_t)w_up | (uintptr_t)out) & 15) == 0, "ttm_linear_glu: operands must be 16-byte aligned");
+  TTM_REQUIRE(act_gate >= TTM_ACT_NONE && act_gate <= TTM_ACT_RELU && act_up >= TTM_ACT_NONE && act_up <= TTM_ACT_RELU,
+              "ttm_linear_glu: unknown activation %d / %d", act_gate, act_up);
+  LinearArgs p;
+  p.A = (const uint8_t *)a; p.W = (const uint8_t *)w_gate; p.bias = nullptr; p.C = (uint8_t *)out;
+  p.Mt = 1; p.Kt = (int)ttm_cdiv(K, 32); p.Nt = (int)ttm_cdiv(N, 32);
+  p.group_n = 0; p.glu = 1;
+  for (int j = 0; j < 4; ++j) { p.gW[j] = nullptr; p.gC[j] = nullptr; p.gNt[j] = 0; p.gAct[j] = TTM_ACT_NONE; }
+  p.gW[0] = (const uint8_t *)w_gate; p.gW[1] = (const uint8_t *)w_up; p.gC[0] = (uint8_t *)out;
+  p.gNt[0] = p.gNt[1] = p.Nt; p.gAct[0] = act_gate; p.gAct[1] = act_up;
+  p.act = TTM_ACT_NONE; p.bias_tiled = 1;
+  p.a_batch = p.w_batch = p.c_batch = 0;
+  p.m_blocks = 1; p.n_blocks = (p.Nt + 7) / 8;
+  p.ntw = 4;
+  p.k_slice = p.Kt; p.partial = nullptr;
+  p.nt_split = p.n_blocks1 = p.ntw2 = 0;
+  p.img_zero_step = 0;
+  p.tail = TTM_TAIL_NONE; p.tail_delta = 0;
+  p.qkv = nullptr; p.norm = nullptr;
+  hipStream_t s = (hipStream_t)stream;
+  const int rc = w_dtype == TTM_BFP8B ? launch_linear<WF_BFP8>(p, 1, s) : launch_linear<WF_BFP4>(p, 1, s);
+  if (rc) return rc;
+  TTM_LAUNCH_CHECK();
+  return TTM_OK;
+}
+
 static int linear_group_entry(const void *a, int n, const void *const *w, int w_dtype, void *const *out, const int64_t *N,
                               const int *act, int64_t M, int64_t K, const QkvFinishArgs *qkv, void *stream) {
   TTM_REQUIRE(n >= 1 && n <= 4, "ttm_linear_group: 1 to 4 members (got %d)", n);
@@ -2279,7 +2416,7 @@ static int linear_group_entry(const void *a, int n, const void *const *w, int w_
   LinearArgs p;
   p.A = (const uint8_t *)a; p.W = (const uint8_t *)w[0]; p.bias = nullptr; p.C = (uint8_t *)out[0];
   p.Mt = (int)ttm_cdiv(M, 32); p.Kt = (int)ttm_cdiv(K, 32); p.Nt = 0;
-  p.group_n = n;
+  p.group_n = n; p.glu = 0;
   for (int j = 0; j < 4; ++j) {
     p.gW[j] = j < n ? (const uint8_t *)w[j] : nullptr;
     p.gC[j] = j < n ? (uint8_t *)out[j] : nullptr;

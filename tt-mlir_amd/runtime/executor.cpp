@@ -678,7 +678,29 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
         if (after < ctx.ops.size() && opType(after) == OpType::EltwiseBinaryOp) {
           fb::Table bop = ctx.ops[after].table(schema::Operation::f_type);
           fb::Table l = bop.table(schema::EltwiseBinaryOp::f_lhs), r = bop.table(schema::EltwiseBinaryOp::f_rhs);
-          if ((l && refId(l) == refId(out2)) || (r && refId(r) == refId(out2))) break;
+          if ((l && refId(l) == refId(out2)) || (r && refId(r) == refId(out2))) {
+            // ... unless that op multiplies the follower's result with this one's (SiLU(gate) * up of a decode step's MLP):
+            // both projections and the multiply are one launch whose workgroups stream the same columns of both matrices
+            fb::Table bout = bop.table(schema::EltwiseBinaryOp::f_out);
+            const std::uint32_t mine = refId(outRef), theirs = refId(out2);
+            auto usesOf = [&](std::uint32_t id) { auto u = ctx.uses.find(id); return u == ctx.uses.end() ? 0u : u->second; };
+            const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
+            if (decodeFusionEnabled() && followers.empty() && as_.size() == 2 && bop.scalar<std::uint32_t>(schema::EltwiseBinaryOp::f_type, 0) == 1 && l && r && bout &&
+                ((refId(l) == mine && refId(r) == theirs) || (refId(l) == theirs && refId(r) == mine)) && usesOf(mine) == 1 &&
+                usesOf(theirs) == 1 && shape2 == outShape && shapeFromTensorRef(bout) == outShape && layoutFromTensorRef(bout) == plain &&
+                wit->second.handle->shape[1] == b.handle->shape[1] && wit->second.handle->data.get() != b.handle->data.get() &&
+                ttm_linear_glu_supported(ttmDtype(b.handle->dtype), M, N, K)) {
+              Tensor gated = makeOut(ctx, bout, DataType::BFloat16, TensorLayout::Tile);
+              TTM_CALL(ttm_linear_glu(a.handle->data.get(), b.handle->data.get(), wit->second.handle->data.get(), ttmDtype(b.handle->dtype),
+                                      gated.handle->data.get(), M, N, K, activationCode(activation), activationCode(act2), ctx.stream()));
+              ctx.put(bout, finish(ctx, gated, bout));
+              ctx.skip.insert(j);
+              ctx.skip.insert(after);
+              debug::Stats::get().incrementStat("FusedLinearGlu");
+              return;
+            }
+            break;
+          }
         }
       }
       bool distinct = wit->second.handle->data.get() != b.handle->data.get();
