@@ -746,6 +746,10 @@ __device__ __forceinline__ void sdpa_dma16(const void *base, uint32_t lane_off, 
   // lds_addr is wavefront-uniform; lane l of the wavefront writes 16 bytes at lds_addr + 16 l
   asm volatile("s_mov_b32 m0, %2\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_addr) : "memory");
 }
+template <int IMM>
+__device__ __forceinline__ void sdpa_dma16_at(const void *base, uint32_t lane_off, uint32_t lds_addr) {   // to lds_addr + IMM
+  asm volatile("s_add_u32 m0, %2, %3\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_off), "s"(base), "s"(lds_addr), "n"(IMM) : "memory", "scc");
+}
 __device__ __forceinline__ float sdpa_max_halves(float x) {
   const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
@@ -755,6 +759,7 @@ __device__ __forceinline__ float sdpa_sum_halves(float x) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 template <bool B> struct SdpaFlag { static constexpr bool value = B; };
+template <int I> struct SdpaIdx { static constexpr int value = I; };
 
 template <int DT>  // head_dim / 32: 2 or 4
 __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *lds) {
@@ -804,27 +809,55 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
   }
 
   // Staging.  The instructions of a wavefront cover 64 consecutive 16-byte chunks of LDS each; chunk c of a pass's K lies
-  // in tile row c / (128 DT).  K is copied as it lies in its tiles; V too, but the faces of the upper 16 columns are
+  // in tile row c / (128 DT).  K is copied as it lies in its tiles (but for the exchange below); V too, but the faces of the upper 16 columns are
   // rotated by eight chunks (four rows) so that the transposing reads touch every bank once: the lane that fills a chunk
   // of such a face fetches the chunk eight further back.
   const int c0 = wave * 64;                               // with 512 lanes and 128 DT chunks per tile row, load i of a wavefront
   const int ccl = c0 % (DT * 128) + lane;                 // lies in tile row (c0 + 512 i) / (128 DT) at the same chunk
-  const uint32_t koff = ccl * 16;
+  // K is copied as it lies in its tiles but for one exchange: in the faces' rows 8..15 the two 16-byte halves of a row swap
+  // places, so that the 16 lanes whose fragment reads go out together (rows 0..15, one half) touch 16 different bank groups
+  // instead of 8 twice.  The lane that fills a chunk fetches its partner's.
+  const uint32_t koff = (ccl ^ ((ccl >> 4) & 1)) * 16;
   const uint32_t voff = ((ccl & ~31) + (((ccl & 31) - 8 * ((ccl >> 5) & 1)) & 31)) * 16;
   const uint8_t *kg = p.k + k_mat, *vg = p.v + v_mat;
   auto next_stage = [](int st) { return st + STAGE == NST * STAGE ? 0 : st + STAGE; };   // byte offsets of the ring's stages
-  auto dma = [&](int kb, int st_off, int i) {   // load i of this wavefront for pass kb (stage at st_off): K for even i, V for odd
-    const uint32_t st = lds0 + st_off + c0 * 16 + (i >> 1) * 8192;
-    const int tr = (c0 + 512 * (i >> 1)) / (DT * 128);   // 0 or 1
-    const bool second = tr && 2 * kb + 1 < p.skt;         // an odd tile count repeats the last tile; its keys are masked
-    if (i & 1) sdpa_dma16(vg + (int64_t)(2 * kb) * p.v_pitch + (second ? p.v_pitch : 0), voff, st + 2 * TROW);
-    else sdpa_dma16(kg + (int64_t)(2 * kb) * p.k_pitch + (second ? p.k_pitch : 0), koff, st);
+  // The ring's loads walk the passes in order, three ahead of the pass being multiplied, so what a load needs is carried
+  // from pass to pass in scalar registers instead of being worked out from the pass number (64-bit multiplies, a chain
+  // of stage selects: 60 scalar instructions per pass, of which a wavefront issues one per four cycles): the addresses
+  // of the pass's first K and V tile rows, its stage, and the distance to its second tile row - zero when an odd tile
+  // count ends inside the pass: the last tile is fetched twice and its keys are masked.  Past the last pass the loads
+  // stay on it while the stage moves on: every pass of the loop requests NL loads, so that the counted wait below
+  // always has the same meaning; what they fetch then lands in the stage that is free at that point and is never read.
+  const uint32_t ld_m0 = lds0 + c0 * 16;
+  int ld_kb = kb_begin, ld_st = 0;
+  const uint8_t *ld_k = kg + (int64_t)(2 * kb_begin) * p.k_pitch, *ld_v = vg + (int64_t)(2 * kb_begin) * p.v_pitch;
+  const bool ld_row1 = DT == 4 || wave >= 4;   // this wavefront's loads of the second half (DT = 4) or all its loads (DT = 2) are tile row 1
+  uint32_t koff1 = koff, voff1 = voff;          // lane offsets for tile row 1
+  auto ld_second = [&]() {
+    const bool second = ld_row1 && 2 * ld_kb + 1 < p.skt;
+    koff1 = koff + (second ? (uint32_t)p.k_pitch : 0u);
+    voff1 = voff + (second ? (uint32_t)p.v_pitch : 0u);
   };
-  // Every pass of the loop requests NL loads, so that the counted wait below always has the same meaning: near the end
-  // the last pass is requested again, into the stage that is free at that point, and never read.
-  auto dma_all = [&](int kb, int st_off) {
-#pragma unroll
-    for (int i = 0; i < NL; ++i) dma(min(kb, kb_end - 1), st_off, i);
+  ld_second();
+  auto dma = [&](auto i_tag) {   // load i of this wavefront for the pass the ring is at: K for even i, V for odd
+    constexpr int i = decltype(i_tag)::value;
+    constexpr bool row1_is_half = DT == 4;   // DT = 4: load i covers tile row i / 2; DT = 2: the wavefront's row
+    const bool r1 = row1_is_half ? (i >> 1) != 0 : true;
+    if constexpr (i & 1) sdpa_dma16_at<(i >> 1) * 8192 + 2 * TROW>(ld_v, r1 ? voff1 : voff, ld_m0 + ld_st);
+    else sdpa_dma16_at<(i >> 1) * 8192>(ld_k, r1 ? koff1 : koff, ld_m0 + ld_st);
+  };
+  auto ld_advance = [&]() {   // on to the next pass
+    const bool more = ld_kb + 1 < kb_end;
+    ld_kb += more ? 1 : 0;
+    ld_k += more ? 2 * p.k_pitch : 0;
+    ld_v += more ? 2 * p.v_pitch : 0;
+    ld_st = next_stage(ld_st);
+    ld_second();
+  };
+  auto dma_all = [&]() {
+    dma(SdpaIdx<0>{}); dma(SdpaIdx<1>{});
+    if constexpr (NL > 2) { dma(SdpaIdx<2>{}); dma(SdpaIdx<3>{}); }
+    ld_advance();
   };
   // All but this wavefront's last NL loads have landed, hence pass kb + 1 (requested two passes ago), and after the barrier
   // every wavefront's share of it; and every wavefront is through with pass kb - 2, whose stage pass kb + 3 overwrites.
@@ -834,7 +867,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
   };
   // per-lane parts of the fragment addresses inside a stage
   const int dhalf = (lane >> 4) & 1, s16 = lane & 15;
-  const int kfrag = kh * TROW + (l31 >> 4) * 1024 + (l31 & 15) * 32 + hh * 16;
+  const int kfrag = kh * TROW + (l31 >> 4) * 1024 + (l31 & 15) * 32 + (hh ^ ((l31 >> 3) & 1)) * 16;
   const int vfrag = 2 * TROW + kh * TROW + dhalf * 512;
   const int vlo = ((4 * hh + (s16 >> 2)) * 32 + 8 * (s16 & 3) + 128 * dhalf) & 511, vhi = (vlo + 256) & 511;
   const uint8_t *kfp = lds + kfrag, *vlp = lds + vfrag + vlo, *vhp = lds + vfrag + vhi;
@@ -871,8 +904,6 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
   auto step = [&](auto qk_tag, auto sm_tag, auto ring_tag, int kb, f32x16 &sc, f32x16 &sn) {
     constexpr bool QK = decltype(qk_tag)::value, SM = decltype(sm_tag)::value, RING = decltype(ring_tag)::value;
     const int st_next = next_stage(st_cur);
-    const int st_load = next_stage(next_stage(st_next));
-    const int kb_load = min(kb + 3, kb_end - 1);
     const uint8_t *k_next = kfp + st_next;
     float mul = scale2, rs = 0.0f;
     if constexpr (SM) {
@@ -948,8 +979,8 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
         else read_k(k_next, st - DT);
       }
       if constexpr (RING) {   // the ring's loads are spread over the step: the addresser takes one wavefront's at a time
-        if (st == 0) dma(kb_load, st_load, 0);
-        if (st == DT && NL > 2) dma(kb_load, st_load, 2);
+        if (st == 0) dma(SdpaIdx<0>{});
+        if constexpr (NL > 2) { if (st == DT) dma(SdpaIdx<2>{}); }
       }
       if constexpr (SM) {
 #pragma unroll
@@ -967,7 +998,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
         o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va[d], *(bf16x8 *)&pb, o[d], 0, 0, 0);
         read_v(vl_prev, vh_prev, 1, d);
         if constexpr (RING) {
-          if (d == 0) dma(kb_load, st_load, 1);
+          if (d == 0) dma(SdpaIdx<1>{});
         }
 #pragma unroll
         for (int e = 0; e < 8 / DT; ++e) elem(8 + d * (8 / DT) + e);
@@ -979,7 +1010,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
         o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*(bf16x8 *)&va[d], *(bf16x8 *)&pb, o[d], 0, 0, 0);
         if constexpr (QK) read_v(vl_cur, vh_cur, 0, d);   // for the next step
         if constexpr (RING) {
-          if (d == 0 && NL > 2) dma(kb_load, st_load, 3);
+          if constexpr (NL > 2) { if (d == 0) dma(SdpaIdx<3>{}); }
         }
       }
       l_run += sdpa_sum_halves(rs);
@@ -987,10 +1018,11 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
 #pragma unroll
       for (int d = 0; d < DT; ++d) read_v(vl_cur, vh_cur, 0, d);
       if constexpr (RING) {
-        dma(kb_load, st_load, 1);
-        if (NL > 2) dma(kb_load, st_load, 3);
+        dma(SdpaIdx<1>{});
+        if constexpr (NL > 2) dma(SdpaIdx<3>{});
       }
     }
+    if constexpr (RING) ld_advance();
     // one pass on: the stage multiplied next is the one after, the stage of this pass is the one the softmax looks back to
     st_cur = st_next;
     k_cur = k_next;
@@ -999,17 +1031,15 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
   };
   auto skip = [&](int kb) {   // a pass outside this wavefront's interval: its share of the staging only
     sync();
-    const int st_next = next_stage(st_cur);
-    dma_all(kb + 3, next_stage(next_stage(st_next)));
-    st_cur = st_next;
+    dma_all();
+    st_cur = next_stage(st_cur);
   };
 
   f32x16 sa, sb;
 #pragma unroll
   for (int r = 0; r < 16; ++r) sa[r] = sb[r] = 0.0f;
   {
-    int st = 0;
-    for (int i = 0; i < 3; ++i) { dma_all(kb_begin + i, st); st = next_stage(st); }   // the first pass lies in stage 0
+    for (int i = 0; i < 3; ++i) dma_all();   // the first pass lies in stage 0
   }
   // Q is used here, in front of the loops, so that the wait for its loads stands here (and covers the requests above, whose
   // first passes the first barrier needs anyway): a counted wait for it further down would also wait for the
@@ -1059,7 +1089,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
     for (int r4 = 0; r4 < 4; ++r4)
 #pragma unroll
       for (int d = 0; d < DT; ++d)
-        ox[(r4 * 256 + slot) * DT + d] = f32x4{o[d][4 * r4], o[d][4 * r4 + 1], o[d][4 * r4 + 2], o[d][4 * r4 + 3]};
+        ox[(r4 * DT + d) * 256 + slot] = f32x4{o[d][4 * r4], o[d][4 * r4 + 1], o[d][4 * r4 + 2], o[d][4 * r4 + 3]};
   }
   __syncthreads();
   if (kh == 0) {
@@ -1071,7 +1101,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
     for (int r4 = 0; r4 < 4; ++r4)
 #pragma unroll
       for (int d = 0; d < DT; ++d) {
-        const f32x4 x = ox[(r4 * 256 + slot) * DT + d];
+        const f32x4 x = ox[(r4 * DT + d) * 256 + slot];
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[d][4 * r4 + e] = o[d][4 * r4 + e] * a0 + x[e] * a1;
       }
@@ -1213,7 +1243,8 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
       g.x = (unsigned)(grid64.x * ks);
     }
     // one workgroup per query block (or pair) and 64 or 128 columns: the pipelined form.  sdpa_variant 6 keeps the chained one.
-    if (ks == 1 && (D == 128 || D == 64) && variant != 6) {
+    // (its ring loads add the distance between two tile rows to a 32-bit lane offset)
+    if (ks == 1 && (D == 128 || D == 64) && variant != 6 && p.k_pitch < ((int64_t)1 << 30) && p.v_pitch < ((int64_t)1 << 30)) {
       const int ring = (int)D / 32 * 40960;   // five stages of 64 keys of K and V
       hipError_t e = D == 128 ? hipFuncSetAttribute((const void *)ttm_sdpa_pipe_k<4>, hipFuncAttributeMaxDynamicSharedMemorySize, ring)
                               : hipFuncSetAttribute((const void *)ttm_sdpa_pipe_k<2>, hipFuncAttributeMaxDynamicSharedMemorySize, ring);
