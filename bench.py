@@ -357,7 +357,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 MEASURED_ON = {"ttm_linear.hip": ("2623b3ecfdda",), "ttm_bfp.hip": ("cdf35c7592c1",), "ttm_layout.hip": ("a6cf1c428342",),
                "ttm_decode.hip": ("3bd99843ac98",), "ttm_rowwise.hip": ("0819544c7ff3",), "ttm_eltwise.hip": ("62019175607e",),
-               "ttm_sdpa.hip": ("46ecf9c3e2fa",)}
+               "ttm_sdpa.hip": ("3c1e7f59da68",)}
 TRAFFIC_HOW = ("rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs), KiB per dispatch scaled by what the same counters "
                "read for the 256 MiB copy kernel; profiles/bench_kernels_hbm_traffic_pmc.md")
 

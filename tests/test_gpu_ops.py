@@ -440,7 +440,7 @@ def test_copy_view_at_positions_the_destination_from_device_memory(hip, dev, ele
     # (variant 5 keeps them in one workgroup); ragged key counts, masks, a causal chunk, shares without any visible key
     (1, 8, 2, 128, 2048, 128, False, None), (1, 4, 2, 100, 1500, 64, False, "bh"), (2, 2, 2, 64, 1100, 128, False, "b1"),
     (1, 4, 4, 128, 1024, 128, True, None), (1, 2, 1, 40, 4096, 32, False, None)])
-@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 6])   # automatic, 32-key kernel, eight-wavefront kernel forced / forbidden, no key shares, no pipeline
+@pytest.mark.parametrize("variant", [0, 1, 3, 4, 5, 6, 7, 8])   # automatic, 32-key kernel, eight-wavefront kernel forced / forbidden, no key shares, no pipeline, four- / eight-wavefront pipeline
 def test_sdpa(hip, dev, orc, B, Hq, Hkv, Sq, Sk, D, causal, mask, variant):
     if variant == 1 and Sq * Sk >= 512 * 512:
         pytest.skip("the 32-key kernel is covered by the small shapes")
@@ -497,7 +497,40 @@ def test_sdpa_config5_shape(hip, dev, orc):
     assert np.array_equal(res[0, :, 0, :], np.repeat(v.float().numpy()[0, :, 0, :], Hq // Hkv, axis=0))
 
 
-@pytest.mark.parametrize("variant", [0, 1, 4, 6])
+def test_sdpa_several_sequences_four_wavefront_form(hip, dev, orc):
+    """Three sequences of 1024 tokens (32 query / 8 kv heads, head dim 128, causal): three query blocks per CU, which the
+    automatic choice gives to the four-wavefront pipelined kernel (two workgroups per CU, 32 keys per pass).  Every output
+    against the oracle, and the forced eight-wavefront form beside it."""
+    import oracle.metrics as metrics
+    B, Hq, Hkv, S, D = 3, 32, 8, 1024, 128
+    q = datagen.randn((B, Hq, S, D), seed=115, dtype=torch.bfloat16)
+    k = datagen.randn((B, Hkv, S, D), seed=116, dtype=torch.bfloat16)
+    v = datagen.randn((B, Hkv, S, D), seed=117, dtype=torch.bfloat16)
+    qt, kt, vt = (tilize_dev(hip, t, dev) for t in (q, k, v))
+    res = {}
+    try:
+        for variant in (0, 7, 8):
+            hip.set_option("sdpa_variant", variant)
+            out = torch.full_like(qt, float("nan"))
+            hip.call("ttm_sdpa", hip.ptr(qt), hip.ptr(kt), hip.ptr(vt), None, 1, hip.ptr(out), hip.BF16, B, Hq, Hkv, S, S, D, 1, 0.0,
+                     hip.current_stream())
+            res[variant] = untilize_dev(hip, out, q.shape, dev).float().cpu().numpy()
+    finally:
+        hip.set_option("sdpa_variant", 0)
+    orc.set_threads(orc.max_threads())
+    try:
+        want = orc.sdpa(q.float().numpy(), k.float().numpy(), v.float().numpy(), None, is_causal=True)
+    finally:
+        orc.set_threads(1)
+    assert np.array_equal(res[0], res[7])        # 768 blocks on 256 CUs: the automatic choice is the four-wavefront form
+    for variant in (7, 8):
+        assert np.all(np.isfinite(res[variant]))
+        assert np.max(np.abs(res[variant] - want)) <= 2.0 ** -6
+        assert metrics.get_pcc(want, res[variant]) >= 0.9999
+        assert np.array_equal(res[variant][:, :, 0, :], np.repeat(v.float().numpy()[:, :, 0, :], Hq // Hkv, axis=1))
+
+
+@pytest.mark.parametrize("variant", [0, 1, 4, 6, 7])
 @pytest.mark.parametrize("flags", [15, 1, 6, 8, 9])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal", [(1, 8, 2, 256, 256, 128, True), (2, 4, 4, 96, 160, 64, False), (1, 4, 1, 70, 70, 32, True),
                                                       (1, 2, 2, 40, 300, 256, False)])
@@ -532,7 +565,7 @@ def test_sdpa_heads_inner_equals_the_head_major_call(hip, dev, B, Hq, Hkv, Sq, S
     assert torch.equal(got, want)
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 6])
+@pytest.mark.parametrize("variant", [0, 1, 2, 3, 4, 6, 7])
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,window,sink,mask,flags", [
     (1, 4, 2, 256, 256, 128, True, 64, False, None, 0), (1, 4, 2, 256, 256, 128, True, 1, False, None, 0),
     (1, 4, 2, 300, 300, 64, True, 100, True, None, 0), (2, 2, 2, 96, 160, 128, False, 40, False, None, 0),

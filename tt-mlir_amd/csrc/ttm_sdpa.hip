@@ -761,11 +761,15 @@ __device__ __forceinline__ float sdpa_sum_halves(float x) {
 template <bool B> struct SdpaFlag { static constexpr bool value = B; };
 template <int I> struct SdpaIdx { static constexpr int value = I; };
 
-template <int DT>  // head_dim / 32: 2 or 4
+// KH = 2: eight wavefronts, 64 keys per pass, the two key halves of a query tile in two wavefronts (merged at the end).
+// KH = 1: four wavefronts, 32 keys per pass, no halves: half the ring, so that two workgroups share a CU and the two
+// wavefronts of a SIMD belong to different workgroups - no common barrier, no merge.
+template <int DT, int KH>  // head_dim / 32: 2 or 4
 __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h, int b, uint8_t *lds) {
-  static_assert(DT == 2 || DT == 4, "64 or 128 columns");
+  static_assert((DT == 2 || DT == 4) && (KH == 1 || KH == 2), "64 or 128 columns");
   constexpr int TROW = DT * 2048;      // one 32-key tile row of K or V
-  constexpr int STAGE = 4 * TROW;      // a 64-key pass: two tile rows of K, then two of V
+  constexpr int STAGE = 2 * KH * TROW; // a pass of 32 KH keys: KH tile rows of K, then of V
+  constexpr int LANES = 256 * KH;
   constexpr int NST = 5;               // stages of the ring
   constexpr int NL = DT;               // LDS-direct loads per wavefront and pass: DT / 2 of K, DT / 2 of V
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) uint8_t *)lds;
@@ -796,15 +800,15 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
   float m_run = -INFINITY, l_run = 0.0f;
   const int q_glob = qt * 32 + l31, q_last = qt * 32 + 31;
   const int kt_begin = first_key_tile(p, qb * 128), kt_end = end_key_tile(p, min(qb * 4 + 4, p.sqt) * 32 - 1);
-  const int kb_begin = kt_begin >> 1, kb_end = (kt_end + 1) >> 1;
-  // This wavefront's 32 keys of pass kb start at 64 kb + 32 kh; the passes in which one of them is visible to one of its
+  const int kb_begin = kt_begin / KH, kb_end = (kt_end + KH - 1) / KH;
+  // This wavefront's 32 keys of pass kb start at 32 KH kb + 32 kh; the passes in which one of them is visible to one of its
   // queries (not behind the causal or window limit, not in front of the window, not past the last key) are an interval.
   int w_begin, w_end;
   {
     const int x = qt * 32 - p.lo_off - 31 - 32 * kh;
     const int y = min(q_last + p.hi_off, p.Sk - 1) - 32 * kh;
-    w_begin = max(x > 0 ? (x + 63) >> 6 : 0, kb_begin);
-    w_end = min(y >= 0 ? (y >> 6) + 1 : 0, kb_end);
+    w_begin = max(x > 0 ? (x + 32 * KH - 1) / (32 * KH) : 0, kb_begin);
+    w_end = min(y >= 0 ? y / (32 * KH) + 1 : 0, kb_end);
     if (!wave_ok || w_begin >= w_end) w_begin = w_end = kb_end;
   }
 
@@ -812,8 +816,9 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
   // in tile row c / (128 DT).  K is copied as it lies in its tiles (but for the exchange below); V too, but the faces of the upper 16 columns are
   // rotated by eight chunks (four rows) so that the transposing reads touch every bank once: the lane that fills a chunk
   // of such a face fetches the chunk eight further back.
-  const int c0 = wave * 64;                               // with 512 lanes and 128 DT chunks per tile row, load i of a wavefront
-  const int ccl = c0 % (DT * 128) + lane;                 // lies in tile row (c0 + 512 i) / (128 DT) at the same chunk
+  const int c0 = wave * 64;                               // with 128 DT chunks per tile row, load i of a wavefront (chunk
+  const int ccl = c0 % (DT * 128) + lane;                 // c0 + LANES (i / 2) + lane of the pass's K or V) lies in tile row
+                                                          // (c0 + LANES (i / 2)) / (128 DT); ccl is its chunk there for i < 2
   // K is copied as it lies in its tiles but for one exchange: in the faces' rows 8..15 the two 16-byte halves of a row swap
   // places, so that the 16 lanes whose fragment reads go out together (rows 0..15, one half) touch 16 different bank groups
   // instead of 8 twice.  The lane that fills a chunk fetches its partner's.
@@ -830,27 +835,30 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
   // always has the same meaning; what they fetch then lands in the stage that is free at that point and is never read.
   const uint32_t ld_m0 = lds0 + c0 * 16;
   int ld_kb = kb_begin, ld_st = 0;
-  const uint8_t *ld_k = kg + (int64_t)(2 * kb_begin) * p.k_pitch, *ld_v = vg + (int64_t)(2 * kb_begin) * p.v_pitch;
-  const bool ld_row1 = DT == 4 || wave >= 4;   // this wavefront's loads of the second half (DT = 4) or all its loads (DT = 2) are tile row 1
-  uint32_t koff1 = koff, voff1 = voff;          // lane offsets for tile row 1
+  const uint8_t *ld_k = kg + (int64_t)(KH * kb_begin) * p.k_pitch, *ld_v = vg + (int64_t)(KH * kb_begin) * p.v_pitch;
+  // KH = 2: this wavefront's loads of the second half (DT = 4) or all its loads (DT = 2) are tile row 1.  KH = 1: the
+  // second half (DT = 4) is the second half of the one tile row, 4096 bytes on.
+  const bool ld_row1 = DT == 4 || wave >= 4;
+  uint32_t koff1 = koff + (KH == 1 ? 4096u : 0u), voff1 = voff + (KH == 1 ? 4096u : 0u);   // lane offsets of that half
   auto ld_second = [&]() {
-    const bool second = ld_row1 && 2 * ld_kb + 1 < p.skt;
-    koff1 = koff + (second ? (uint32_t)p.k_pitch : 0u);
-    voff1 = voff + (second ? (uint32_t)p.v_pitch : 0u);
+    if constexpr (KH == 2) {
+      const bool second = ld_row1 && 2 * ld_kb + 1 < p.skt;
+      koff1 = koff + (second ? (uint32_t)p.k_pitch : 0u);
+      voff1 = voff + (second ? (uint32_t)p.v_pitch : 0u);
+    }
   };
   ld_second();
   auto dma = [&](auto i_tag) {   // load i of this wavefront for the pass the ring is at: K for even i, V for odd
     constexpr int i = decltype(i_tag)::value;
-    constexpr bool row1_is_half = DT == 4;   // DT = 4: load i covers tile row i / 2; DT = 2: the wavefront's row
-    const bool r1 = row1_is_half ? (i >> 1) != 0 : true;
-    if constexpr (i & 1) sdpa_dma16_at<(i >> 1) * 8192 + 2 * TROW>(ld_v, r1 ? voff1 : voff, ld_m0 + ld_st);
-    else sdpa_dma16_at<(i >> 1) * 8192>(ld_k, r1 ? koff1 : koff, ld_m0 + ld_st);
+    constexpr bool r1 = KH == 2 && DT == 2 ? true : (i >> 1) != 0;
+    if constexpr (i & 1) sdpa_dma16_at<(i >> 1) * LANES * 16 + KH * TROW>(ld_v, r1 ? voff1 : voff, ld_m0 + ld_st);
+    else sdpa_dma16_at<(i >> 1) * LANES * 16>(ld_k, r1 ? koff1 : koff, ld_m0 + ld_st);
   };
   auto ld_advance = [&]() {   // on to the next pass
     const bool more = ld_kb + 1 < kb_end;
     ld_kb += more ? 1 : 0;
-    ld_k += more ? 2 * p.k_pitch : 0;
-    ld_v += more ? 2 * p.v_pitch : 0;
+    ld_k += more ? KH * p.k_pitch : 0;
+    ld_v += more ? KH * p.v_pitch : 0;
     ld_st = next_stage(ld_st);
     ld_second();
   };
@@ -868,7 +876,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
   // per-lane parts of the fragment addresses inside a stage
   const int dhalf = (lane >> 4) & 1, s16 = lane & 15;
   const int kfrag = kh * TROW + (l31 >> 4) * 1024 + (l31 & 15) * 32 + (hh ^ ((l31 >> 3) & 1)) * 16;
-  const int vfrag = 2 * TROW + kh * TROW + dhalf * 512;
+  const int vfrag = KH * TROW + kh * TROW + dhalf * 512;
   const int vlo = ((4 * hh + (s16 >> 2)) * 32 + 8 * (s16 & 3) + 128 * dhalf) & 511, vhi = (vlo + 256) & 511;
   const uint8_t *kfp = lds + kfrag, *vlp = lds + vfrag + vlo, *vhp = lds + vfrag + vhi;
   u32x4 ka[DT];   // K fragments of DT of a pass's 2 DT steps at a time
@@ -907,7 +915,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
     const uint8_t *k_next = kfp + st_next;
     float mul = scale2, rs = 0.0f;
     if constexpr (SM) {
-      const int key_base = (kb - 1) * 64 + 32 * kh;
+      const int key_base = (kb - 1) * 32 * KH + 32 * kh;
       const bool edge = key_base + 31 > qt * 32 + p.hi_off || key_base < q_last - p.lo_off || key_base + 32 > p.Sk;   // wavefront-uniform
       float mx = -INFINITY;
       if (p.mask || edge) {
@@ -917,7 +925,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
           const int key0 = key_base + kin;
           float mk[4] = {0.f, 0.f, 0.f, 0.f};
           if (p.mask) {
-            const int kt = min(2 * (kb - 1) + kh, p.skt - 1);
+            const int kt = min(KH * (kb - 1) + kh, p.skt - 1);
             const int64_t mm = ((int64_t)b * p.mask_b * p.mask_heads + (p.mask_heads == 1 ? 0 : h)) * p.sqt * p.skt * 2048;
             const uint8_t *mp = p.mask + mm + ((int64_t)qt * p.skt + kt) * 2048 +
                                 (((l31 >> 4) * 2 + (kin >> 4)) * 256 + (l31 & 15) * 16 + (kin & 15)) * 2;
@@ -1076,9 +1084,10 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
     }
     for (++kb; kb < kb_end; ++kb) skip(kb);
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if constexpr (KH == 2) {
   // merge the two key halves of every query tile: the upper half hands over (max, sum) and its output (16 DT values per
   // lane: 256 lanes x 16 DT floats = DT * 16 KiB) through the ring, which nobody reads or fills any more
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   float *ml = (float *)(lds + 4 * STAGE);
   f32x4 *ox = (f32x4 *)lds;
@@ -1107,6 +1116,7 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
       }
   }
   __syncthreads();   // the next block of the pair fills the ring again
+  }
   if (kh != 0 || !wave_ok) return;   // no barrier follows inside this block; the next block starts with one
   const float inv = l_run > 0.0f ? 1.0f / l_run : 0.0f;
   const bool q_ok = q_glob < p.Sq;
@@ -1124,16 +1134,25 @@ __device__ __forceinline__ void sdpa_pipe_block(const SdpaArgs &p, int qb, int h
     }
 }
 
-template <int DT>
-__global__ __launch_bounds__(512) void ttm_sdpa_pipe_k(SdpaArgs p, int paired) {
+template <int DT, int KH>
+__global__ __launch_bounds__(256 * KH) __attribute__((amdgpu_waves_per_eu(2, 2))) void ttm_sdpa_pipe_k(SdpaArgs p, int paired) {
   extern __shared__ u32x4 sdpa_ring[];
   uint8_t *lds = (uint8_t *)sdpa_ring;
   const int nqb = (p.sqt + 3) / 4;
   int x = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   sdpa_xcd_order(p, x, h, b);
+  if constexpr (KH == 1) {
+    // One query block per workgroup, two workgroups per CU.  Under a causal mask a block's work grows with its number:
+    // the first half of a matrix's workgroups (the first to be placed, one per CU) take the upper blocks from the last
+    // down, the second half (placed beside them) the lower blocks from the first up, so that the two that share a CU
+    // carry about the same work together wherever the dispatcher keeps to that order; nothing depends on it.
+    const int upper = (nqb + 1) / 2;
+    sdpa_pipe_block<DT, 1>(p, x < upper ? nqb - 1 - x : x - upper, h, b, lds);
+    return;
+  }
   const int heavy = nqb - 1 - x, light = x;
   const int parts = paired && light < heavy ? 2 : 1;   // workgroup-uniform
-  for (int part = 0; part < parts; ++part) sdpa_pipe_block<DT>(p, part == 0 ? heavy : light, h, b, lds);
+  for (int part = 0; part < parts; ++part) sdpa_pipe_block<DT, KH>(p, part == 0 ? heavy : light, h, b, lds);
 }
 
 // Merges the key shares of ttm_sdpa64_split_k: one workgroup per (b, h, query tile).  With M = max_s m_s, every output is
@@ -1219,7 +1238,7 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
   // (with 64 or 128 columns the eight-wavefront form is the pipelined kernel, which is the faster one at every launch size:
   // [2, 32 / 8, 4096, 128] causal 293 against 350 us, [1, 32 / 8, 8192, 128] 539 against 665 us)
   const bool split = wide && D <= 128 && (variant == 3 || ((variant == 0 || variant == 6) && wgs <= (int64_t)cus) ||
-                                          (variant == 0 && (D == 64 || D == 128)));
+                                          ((variant == 0 || variant == 7 || variant == 8) && (D == 64 || D == 128)));
   p.ksplits = 1; p.part_o = nullptr; p.part_ml = nullptr;
   if (split) {
     const dim3 block8(512);
@@ -1245,12 +1264,25 @@ static int sdpa_entry(const void *q, const void *k, const void *v, const void *m
     // one workgroup per query block (or pair) and 64 or 128 columns: the pipelined form.  sdpa_variant 6 keeps the chained one.
     // (its ring loads add the distance between two tile rows to a 32-bit lane offset)
     if (ks == 1 && (D == 128 || D == 64) && variant != 6 && p.k_pitch < ((int64_t)1 << 30) && p.v_pitch < ((int64_t)1 << 30)) {
-      const int ring = (int)D / 32 * 40960;   // five stages of 64 keys of K and V
-      hipError_t e = D == 128 ? hipFuncSetAttribute((const void *)ttm_sdpa_pipe_k<4>, hipFuncAttributeMaxDynamicSharedMemorySize, ring)
-                              : hipFuncSetAttribute((const void *)ttm_sdpa_pipe_k<2>, hipFuncAttributeMaxDynamicSharedMemorySize, ring);
+      // The four-wavefront form runs two workgroups per CU side by side, one query block each and 32 keys per pass: the two
+      // wavefronts of a SIMD then share no barrier, nothing is merged at the end, and one workgroup's first and last passes
+      // overlap the other's middle.  It pays for many short query-block columns (several sequences of up to ~3000 tokens,
+      // 128 columns: [2..8, 32 / 8, 2048, 128] causal 5..13 % faster, [1, 32 / 8, 3000, 128] 12 %); a single sequence of 2048
+      // tokens has only two blocks per CU, of very different length, and is 8 % slower that way, 4096 tokens 4 % slower,
+      // 8192 the same.  sdpa_variant 7 forces it, 8 keeps the eight-wavefront form.
+      const int64_t blocks = (int64_t)nqb * Hq * B;
+      const bool four = variant == 7 || (variant == 0 && D == 128 && blocks >= 3 * (int64_t)cus && nqb <= 24);
+      const int ring = (int)D / 32 * (four ? 20480 : 40960);   // five stages of 32 or 64 keys of K and V
+      const void *fn = four ? (D == 128 ? (const void *)ttm_sdpa_pipe_k<4, 1> : (const void *)ttm_sdpa_pipe_k<2, 1>)
+                            : (D == 128 ? (const void *)ttm_sdpa_pipe_k<4, 2> : (const void *)ttm_sdpa_pipe_k<2, 2>);
+      hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, ring);
       if (e != hipSuccess) return ttm_set_error(TTM_ERR_HIP, "hipFuncSetAttribute(LDS %d): %s", ring, hipGetErrorString(e));
-      if (D == 128) hipLaunchKernelGGL(ttm_sdpa_pipe_k<4>, g, block8, ring, s, p, paired);
-      else hipLaunchKernelGGL(ttm_sdpa_pipe_k<2>, g, block8, ring, s, p, paired);
+      if (four) {
+        const dim3 g4((unsigned)nqb, (unsigned)Hq, (unsigned)B);
+        if (D == 128) hipLaunchKernelGGL((ttm_sdpa_pipe_k<4, 1>), g4, dim3(256), ring, s, p, 0);
+        else hipLaunchKernelGGL((ttm_sdpa_pipe_k<2, 1>), g4, dim3(256), ring, s, p, 0);
+      } else if (D == 128) hipLaunchKernelGGL((ttm_sdpa_pipe_k<4, 2>), g, block8, ring, s, p, paired);
+      else hipLaunchKernelGGL((ttm_sdpa_pipe_k<2, 2>), g, block8, ring, s, p, paired);
       TTM_LAUNCH_CHECK();
       return TTM_OK;
     }
