@@ -1619,8 +1619,9 @@ __global__ __launch_bounds__(256) void ttm_linear_small_k(LinearArgs p) {
 // =============================================================================================
 // Decode kernel for bfp8_b weights (M <= 32 per launch): pure weight streaming, no LDS on the way in.
 // A workgroup owns 64 output columns (two weight tiles); its 8 wavefronts take every 8th k-tile and are
-// summed through LDS at the end.  Per k-tile a lane loads the 8 (k) x 4 (n) block it needs as eight
-// 4-byte words, dequantises it in registers and feeds byte j of the words to MFMA j: with
+// summed through LDS at the end.  Per k-tile a lane needs an 8 (k) x 4 (n) block as eight 4-byte words (bfp8_b: the four
+// lanes of a quad fetch the 128-byte line that holds their four blocks as two whole 16-byte rows each and transpose
+// it between them with DPP moves; bfp4_b: eight 2-byte loads), dequantises it in registers and feeds byte j of the words to MFMA j: with
 // v_mfma_f32_16x16x32_bf16 lane l supplies row l % 16 and k = 8 (l / 16) .. + 7 of the 16 x 32 weight
 // operand, and MFMA j's row r stands for column n = 4 r + j, so one accumulator register of the four
 // MFMAs is four consecutive n again.  Loads run two k-tiles ahead (register ring): with eight wavefronts that is
@@ -1642,6 +1643,7 @@ template <bool BFP4, bool TWO_TERM, int NP, bool GLU>
 __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
   extern __shared__ u32x4 smem[];   // partial sums: NP x 8 wavefronts x 8 x 64 float4 = NP x 64 KiB
   constexpr int D = 2;
+  constexpr bool WL = !BFP4;   // whole-row loads and a transpose within lane quads (bfp8_b)
   constexpr uint32_t TB = BFP4 ? 576u : 1088u, FACE = BFP4 ? 128u : 256u, ROW = BFP4 ? 8u : 16u;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1663,7 +1665,7 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
 #pragma unroll
   for (int pr = 0; pr < NP; ++pr) {
     const uint32_t nt_l = (uint32_t)min(GLU ? 2 * cg + (q16 >> 3) : 2 * NP * cg + 2 * pr + (q16 >> 3), Nt - 1);
-    offW[pr] = nt_l * TB + 64u + (fr * 2 + fc) * FACE + half * (FACE / 2) + quad * (ROW / 4);   // + ROW i
+    offW[pr] = nt_l * TB + 64u + (fr * 2 + fc) * FACE + half * (FACE / 2) + quad * (WL ? ROW : ROW / 4);   // + ROW i (WL: row quad, + 4 ROW)
     offE[pr] = nt_l * TB + (fr * 2 + fc) * 16 + half * 8;
   }
   const uint32_t offA = fr * 512 + q16 * 32 + half * 16;                                     // + 1024 h
@@ -1692,16 +1694,46 @@ __global__ __launch_bounds__(512) void ttm_linear_decode_k(LinearArgs p) {
 #pragma unroll
     for (int pr = 0; pr < NP; ++pr) {
       const uint8_t *Wk = pr == 0 ? Wk0 : Wk1;
+      if constexpr (WL) {
+        // the four lanes of a quad need one 128-byte line between them (8 k rows x 16 n bytes, a dword column each): every
+        // lane fetches two whole rows of it (rows quad and quad + 4) and the quad transposes in registers when the slot is
+        // consumed - 2 loads and 32 cache-line look-ups per wavefront and tile pair instead of 8 and 128
+        const u32x4 x = *(const u32x4 *)(Wk + offW[pr]), y = *(const u32x4 *)(Wk + offW[pr] + 64);
+        rows[s][pr][0] = x.x; rows[s][pr][1] = x.y; rows[s][pr][2] = x.z; rows[s][pr][3] = x.w;
+        rows[s][pr][4] = y.x; rows[s][pr][5] = y.y; rows[s][pr][6] = y.z; rows[s][pr][7] = y.w;
+      } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i)   // the eight loads share their cache lines: cached loads
-        rows[s][pr][i] = BFP4 ? (uint32_t) * (const uint16_t *)(Wk + offW[pr] + i * ROW) : *(const uint32_t *)(Wk + offW[pr] + i * ROW);
+        for (int i = 0; i < 8; ++i)   // the eight loads share their cache lines: cached loads
+          rows[s][pr][i] = BFP4 ? (uint32_t) * (const uint16_t *)(Wk + offW[pr] + i * ROW) : *(const uint32_t *)(Wk + offW[pr] + i * ROW);
+      }
       ex[s][pr] = *(const u32x2 *)(Wk + offE[pr]);
     }
     keeps[s] = keep;   // applied when the slot is consumed: masking here would wait for the load
 #pragma unroll
     for (int h = 0; h < 2; ++h) af[s][h] = *(const u32x4 *)(Ak + offA + h * 1024);
   };
+  // 4 x 4 transpose of dwords within every quad of lanes: lane q ends up with dword q of the rows that lanes 0..3 hold
+  auto quad_transpose = [&](uint32_t *v) __attribute__((always_inline)) {
+    const bool odd = (lane & 1) != 0, hi = (lane & 2) != 0;
+#pragma unroll
+    for (int a = 0; a < 4; a += 2) {   // lanes 2 j and 2 j + 1 exchange (v[a + 1] of the even, v[a] of the odd)
+      const uint32_t ta = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[a], 0xB1, 0xF, 0xF, true);
+      const uint32_t tb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[a + 1], 0xB1, 0xF, 0xF, true);
+      v[a + 1] = odd ? v[a + 1] : ta;
+      v[a] = odd ? tb : v[a];
+    }
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {      // lanes j and j + 2 exchange (v[a + 2] of the lower, v[a] of the upper)
+      const uint32_t ta = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[a], 0x4E, 0xF, 0xF, true);
+      const uint32_t tb = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[a + 2], 0x4E, 0xF, 0xF, true);
+      v[a + 2] = hi ? v[a + 2] : ta;
+      v[a] = hi ? tb : v[a];
+    }
+  };
   auto process_pair = [&](int s, int pr) __attribute__((always_inline)) {
+    if constexpr (WL) {
+      if (!TWO_TERM || keeps[s] != 0u) { quad_transpose(&rows[s][pr][0]); quad_transpose(&rows[s][pr][4]); }
+    }
     if constexpr (TWO_TERM) {
       if (keeps[s] == 0u) return;   // wavefront-uniform: a k-tile past the end contributes nothing
       // (E + 1) << 7 for the rows 2 ip and 2 ip + 1, in the two halves of a word; E is capped so that the field stays 8 bits
