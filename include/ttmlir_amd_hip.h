@@ -140,14 +140,18 @@ int ttm_linear_group(const void *a, int n, const void *const *w, int w_dtype, vo
                      const int *act, int64_t M, int64_t K, void *stream);
 int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, void *out0, void *out1, int64_t M, int64_t N,
                     int64_t K, void *stream);
-/* out = round(round(act_gate(a w_gate)) * round(act_up(a w_up))) for M <= 32 rows in one launch: the gate and up projections
- * of a decode step's MLP and the multiply that joins them (SiLU(gate) * up).  a [M, K] and out [M, N] are bf16 tiles, the two
- * weight matrices block-float [K, N] of one format.  A workgroup streams the same 64 columns of both matrices, so the
- * activations pass through a CU once for both and the two results meet in registers; the three bf16 roundings of the op
- * sequence are kept and the result is bit-identical to ttm_linear (act_gate) + ttm_linear_tail (act_up, TTM_TAIL_MUL), which
- * is what it replaces (runtime/lib/ttnn/operations/matmul/matmul.cpp:47-83, eltwise/binary/binary.cpp:38-126).
- * ttm_linear_glu_supported returns 1 when the shapes and the selected kernel variants allow it (block-float weights,
- * M <= 32, and enough columns that one projection alone would not split K over workgroups), else 0. */
+/* out = round(round(act_gate(a w_gate)) * round(act_up(a w_up))) in one launch: the gate and up projections of an MLP and the
+ * multiply that joins them (SiLU(gate) * up).  a [M, K] and out [M, N] are bf16 tiles, the two weight matrices block-float
+ * [K, N] of one format.  Two forms: for M <= 32 rows (a decode step) a workgroup of the decode kernel streams the same 64
+ * columns of both matrices; for 65 <= M <= 1024 rows and BFP_BFloat8 weights a block of the fused main kernel takes four
+ * column tiles of each matrix instead of eight of one.  Either way the activations pass through a CU once for both and the
+ * two results meet in registers; the three bf16 roundings of the op sequence are kept and the result is bit-identical to
+ * ttm_linear (act_gate) + ttm_linear_tail (act_up, TTM_TAIL_MUL) on the same kernel, which is what it replaces
+ * (runtime/lib/ttnn/operations/matmul/matmul.cpp:47-83, eltwise/binary/binary.cpp:38-126).
+ * ttm_linear_glu_supported returns 1 when the shapes and the selected kernel variants allow it, else 0: block-float weights,
+ * M <= 32 and enough columns that one projection alone would not split K over workgroups; or BFP_BFloat8 weights,
+ * 65 <= M <= 1024 and a shape whose pair of projections the library would run in one pass (where it would first rewrite
+ * the weights as bf16 images, that sequence stays the faster one). */
 int ttm_linear_glu_supported(int w_dtype, int64_t M, int64_t N, int64_t K);
 int ttm_linear_glu(const void *a, const void *w_gate, const void *w_up, int w_dtype, void *out, int64_t M, int64_t N, int64_t K,
                    int act_gate, int act_up, void *stream);

@@ -416,6 +416,12 @@ EXPORT int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_
 // the predicates of the real library at its default options
 EXPORT int ttm_linear_glu_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
   const int64_t groups = ((N + 31) / 32 + 1) / 2, kt = (K + 31) / 32;
+  if (w_dtype == TTM_BFP8B && M > 64 && M <= 1024 && K > 0 && N >= 1 && g_options["linear_two_pass"] != 2 && g_options["linear_glu_main"] != 1) {
+    // the gated form of the fused main kernel, where the real library's model keeps the pair of projections in one pass (256 CUs)
+    const int64_t ksteps = (kt + 1) / 2, nt = (N + 31) / 32, blocks = ((M + 255) / 256) * ((2 * nt + 7) / 8), rounds = (blocks + 255) / 256;
+    const double fused = rounds * (ksteps + 12) * 1.65, first = 3.0 + static_cast<double>(kt) * 2 * nt * (1088.0 + 2048.0) / 5.5e6;
+    if (g_options["linear_two_pass"] == 1 || !(0.28 * fused > first)) return 1;
+  }
   return block_float(w_dtype) && M >= 1 && M <= 32 && K > 0 && N >= 1 && std::min<int64_t>(256 / groups, kt / 32) <= 1;
 }
 EXPORT int ttm_linear_glu(const void *a, const void *w_gate, const void *w_up, int w_dtype, void *out, int64_t M, int64_t N, int64_t K, int act_gate,

@@ -565,3 +565,57 @@ def test_linear_glu_equals_the_op_sequence(hip, dev, orc, M, K, N, fmt, acts):
     assert hip.lib().ttm_linear_glu_supported(wf, 32, 4096, 4096) == 0
     with pytest.raises(hip.TTMError, match="ttm_linear_glu"):
         hip.call("ttm_linear_glu", hip.ptr(at), hip.ptr(wgt), hip.ptr(wut), wf, hip.ptr(got), 33, N, K, 0, 0, s)
+
+
+@pytest.mark.parametrize("M,K,N,acts", [
+    (512, 4096, 14336, ("silu", None)),      # gate and up of config 4
+    (100, 256, 1000, ("gelu", "relu")),       # ragged rows and columns: 32 column tiles = four blocks of eight tile slots
+    (1024, 512, 544, (None, "sigmoid")),      # 17 column tiles: the last block holds one tile of either matrix
+    (65, 96, 96, ("silu", None)),             # the smallest row count of the form, a ragged k tile pair
+])
+def test_linear_glu_main_kernel_equals_the_op_sequence(hip, dev, orc, M, K, N, acts):
+    """ttm_linear_glu at 65..1024 rows (the fused main kernel over alternating column tiles of the two bfp8_b matrices, the
+    product taken in the epilogue) against ttm_linear (gate) + ttm_linear_tail (up, multiply) on the same kernel without
+    split K: bit-identical; and against the CPU oracle with the three bf16 roundings."""
+    from test_gpu_linear import pack_weight
+    wf = hip.BFP8B
+    a = datagen.randn((M, K), seed=140, dtype=torch.bfloat16)
+    wg = datagen.randn((K, N), seed=141, dtype=torch.float32) * 0.05
+    wu = datagen.randn((K, N), seed=142, dtype=torch.float32) * 0.05
+    at, wgt, wut = tilize_dev(hip, a, dev), pack_weight(hip, wg, wf, dev), pack_weight(hip, wu, wf, dev)
+    s = hip.current_stream()
+    Mp, Np = (M + 31) // 32 * 32, (N + 31) // 32 * 32
+    gate = torch.zeros((Mp * Np,), dtype=torch.bfloat16, device=dev)
+    want = torch.zeros_like(gate)
+    got = torch.zeros_like(want)
+    try:   # one pass and no split K for the op sequence; with the image pass ruled out the gated form takes every shape it can run
+        hip.set_option("linear_split_k", 1)
+        hip.set_option("linear_two_pass", 1)
+        hip.call("ttm_linear", hip.ptr(at), hip.BF16, hip.ptr(wgt), wf, 0, None, hip.BF16, hip.TILE, hip.ptr(gate), hip.BF16, 1, 1, M, N, K,
+                 hip.ACT[acts[0]], s)
+        hip.call("ttm_linear_tail", hip.ptr(at), hip.BF16, hip.ptr(wut), wf, 0, None, hip.BF16, hip.TILE, hip.ptr(want), hip.BF16, 1, 1, M, N, K,
+                 hip.ACT[acts[1]], 2, hip.ptr(gate), s)
+        assert hip.lib().ttm_linear_glu_supported(wf, M, N, K) == 1
+        hip.call("ttm_linear_glu", hip.ptr(at), hip.ptr(wgt), hip.ptr(wut), wf, hip.ptr(got), M, N, K, hip.ACT[acts[0]], hip.ACT[acts[1]], s)
+        torch.cuda.synchronize()
+    finally:
+        hip.set_option("linear_split_k", 0)
+        hip.set_option("linear_two_pass", 0)
+    g2, w2 = untilize_dev(hip, got, (Mp, Np), dev)[:M, :N], untilize_dev(hip, want, (Mp, Np), dev)[:M, :N]
+    assert torch.equal(g2, w2)
+    assert bool(torch.isfinite(g2.float()).all())
+    r = lambda x: orc.round_bf16(x)
+    q = lambda w_: orc.bfp_unpack(orc.bfp_pack(w_.numpy(), 8), w_.shape, 8)
+    an = a.float().numpy()
+    orc.set_threads(orc.max_threads())
+    try:
+        ref = r(r(orc.linear(an, q(wg), None, acts[0])) * r(orc.linear(an, q(wu), None, acts[1])))
+    finally:
+        orc.set_threads(1)
+    out = g2.float().cpu().numpy()
+    assert np.max(np.abs(out - ref)) <= 2.0 ** -5 * max(1.0, float(np.max(np.abs(ref))))
+    # bfp4_b weights and the token counts between the two forms stay with the op sequence
+    assert hip.lib().ttm_linear_glu_supported(hip.BFP4B, M, N, K) == 0 and hip.lib().ttm_linear_glu_supported(wf, 48, N, K) == 0
+    assert hip.lib().ttm_linear_glu_supported(wf, 2048, N, K) == 0
+    # by default it follows the library's model of the image pass: config 4 stays in one pass, twice its rows take two
+    assert hip.lib().ttm_linear_glu_supported(wf, 512, 14336, 4096) == 1 and hip.lib().ttm_linear_glu_supported(wf, 1024, 14336, 4096) == 0

@@ -147,8 +147,19 @@ def test_c4_mlp_full_size(device, orc, metrics):
     d = datagen.c4_mlp()
     binary = rt.Binary.load_from_memory(programs.c4_mlp())
     tins = [d["x"], d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    rt.clear_stats()
     (y,) = harness.execute(binary, 1, tins, device)
     assert tuple(y.shape) == (512, 4096) and bool(torch.isfinite(y.float()).all())
+    # gate, up and their product are one launch of the gated main kernel; as a group launch and a multiply they give the same bits
+    assert rt.get_stat("FusedLinearGlu") == 1 and rt.get_stat("GroupedMatmul") == 0
+    from ttmlir_amd import hip
+    hip.set_option("linear_glu_main", 1)
+    try:
+        (y_ops,) = harness.execute(binary, 1, tins, device)
+    finally:
+        hip.set_option("linear_glu_main", 0)
+    assert rt.get_stat("FusedLinearGlu") == 1 and rt.get_stat("GroupedMatmul") == 1
+    assert torch.equal(y, y_ops)
     f = lambda t: t.float().numpy()
     orc.set_threads(orc.max_threads())
     try:

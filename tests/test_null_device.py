@@ -280,7 +280,7 @@ print(json.dumps(report))
     assert r.returncode == 0, (r.stdout[-500:], r.stderr[-1500:])
     rep = json.loads(r.stdout.strip().splitlines()[-1])
     assert rep["c3_2048"]["shapes"] == [[2048, 14336]] and rep["c3_32"]["shapes"] == [[32, 14336]]
-    assert rep["c4"]["shapes"] == [[512, 4096]] and rep["c4"]["GroupedMatmul"] == 1            # gate and up in one launch
+    assert rep["c4"]["shapes"] == [[512, 4096]] and rep["c4"]["FusedLinearGlu"] == 1 and rep["c4"]["GroupedMatmul"] == 0   # gate, up and their product in one launch
     assert rep["c5"]["shapes"] == [[1, 2048, 4096]]
     assert rep["c5"]["GroupedMatmul"] == 1 and rep["c5"]["FusedLinearTail"] == 3               # two residual adds and SiLU(gate) * up
     d = rep["decode32"]                                                                         # three steps

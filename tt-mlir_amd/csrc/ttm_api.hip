@@ -27,7 +27,7 @@ static std::mutex g_opt_mu;
 static std::map<std::string, int> &opts() {
   static std::map<std::string, int> m = {
       {"tilize_variant", 0}, {"untilize_variant", 0}, {"pack_variant", 0}, {"unpack_variant", 0},
-      {"rowwise_variant", 0}, {"sdpa_variant", 0}, {"linear_variant", 0}, {"linear_small_m_max", 64}, {"linear_ntw", 0}, {"linear_split_k", 0}, {"linear_two_part", 0}, {"linear_decode_split", 0}, {"linear_decode_wide", 0}, {"linear_decode_variant", 0}, {"linear_two_pass", 0}, {"linear_img_variant", 0},
+      {"rowwise_variant", 0}, {"sdpa_variant", 0}, {"linear_variant", 0}, {"linear_small_m_max", 64}, {"linear_ntw", 0}, {"linear_split_k", 0}, {"linear_two_part", 0}, {"linear_decode_split", 0}, {"linear_decode_wide", 0}, {"linear_glu_main", 0}, {"linear_decode_variant", 0}, {"linear_two_pass", 0}, {"linear_img_variant", 0},
       {"check_extents", getenv("TTMLIR_AMD_CHECK_EXTENTS") && getenv("TTMLIR_AMD_CHECK_EXTENTS")[0] == '1' ? 1 : 0},
   };
   return m;

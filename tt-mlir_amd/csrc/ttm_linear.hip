@@ -365,6 +365,50 @@ __device__ __forceinline__ void linear_store_partial(const LinearArgs &p, float 
   }
 }
 
+// gated launch: the wavefront's accumulator tiles alternate between the two matrices (tile 2 j: columns of the first, tile
+// 2 j + 1: the same columns of the second); out = round(round(act0(first)) x round(act1(second))) into column tile
+// ntw / 2 + j of the output, whose rows are NtR tiles long.  No bias.
+__device__ __forceinline__ float linear_act_rt(int act, float x) {
+  switch (act) {
+  case TTM_ACT_GELU: return apply_act<TTM_ACT_GELU>(x);
+  case TTM_ACT_SILU: return apply_act<TTM_ACT_SILU>(x);
+  case TTM_ACT_SIGMOID: return apply_act<TTM_ACT_SIGMOID>(x);
+  case TTM_ACT_RELU: return apply_act<TTM_ACT_RELU>(x);
+  default: return x;
+  }
+}
+template <int NA, int MB>
+__device__ __forceinline__ void linear_epilogue_glu(const LinearArgs &p, uint8_t *C, f32x16 (&acc)[NA][MB], int mtw, int ntw, int nt_end, int NtR, int lane) {
+  static_assert(NA % 2 == 0, "pairs of column tiles");
+  const int m_in = lane & 31;
+  const int act0 = p.gAct[0], act1 = p.gAct[1];
+#pragma unroll
+  for (int j = 0; j < NA / 2; ++j) {
+    if (ntw + 2 * j >= nt_end) continue;
+    const int nt = (ntw >> 1) + j;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int n_in = g * 8 + (lane >> 5) * 4;
+#pragma unroll
+      for (int b = 0; b < MB; ++b) {
+        const int mt = mtw + b;
+        if (mt >= p.Mt) continue;
+        float x[4], y[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          x[r] = linear_act_rt(act0, acc[2 * j][b][g * 4 + r]);
+          y[r] = linear_act_rt(act1, acc[2 * j + 1][b][g * 4 + r]);
+        }
+        const u32x2 gq = {pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3])}, uq = {pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3])};
+        const float z[4] = {__uint_as_float(gq.x << 16) * __uint_as_float(uq.x << 16), __uint_as_float(gq.x & 0xFFFF0000u) * __uint_as_float(uq.x & 0xFFFF0000u),
+                            __uint_as_float(gq.y << 16) * __uint_as_float(uq.y << 16), __uint_as_float(gq.y & 0xFFFF0000u) * __uint_as_float(uq.y & 0xFFFF0000u)};
+        const int64_t off = ((int64_t)mt * NtR + nt) * 1024 + ((m_in >> 4) * 2 + (n_in >> 4)) * 256 + (m_in & 15) * 16 + (n_in & 15);
+        *(u32x2 *)(C + off * 2) = u32x2{pack_bf16(z[0], z[1]), pack_bf16(z[2], z[3])};
+      }
+    }
+  }
+}
+
 // split-K: sums the slices, then bias, activation and bf16 as in the fused epilogue; one lane per four elements
 __global__ __launch_bounds__(256) void ttm_linear_reduce_k(LinearArgs p, int slices) {
   const int64_t per = (int64_t)p.Mt * p.Nt * 1024;
@@ -870,9 +914,13 @@ __device__ __forceinline__ void lds_dma16(const void *base, uint32_t lane_off, u
 // BN_ = 7 (second pass only) is a block of seven column tiles: the wavefronts of one half take four of them (this body
 // with NTW = 4), those of the other half three (NTW = 3), and the two halves are dealt out so that every SIMD runs one
 // wavefront of each kind.  Both bodies execute the same sequence of barriers.
-template <int WF, int NTW, bool IMG = false, int BN_ = 2 * NTW>
+template <int WF, int NTW, bool IMG = false, int BN_ = 2 * NTW, bool GLU = false>
 __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, int nblk, int nt_first, int nt_end) {
   static_assert(WF == WF_BFP8 || WF == WF_BFP4, "block-float weights only");
+  // GLU: the block's column tiles alternate between two bfp8_b matrices [K, NtR * 32] (p.gW[0], p.gW[1]; tile 2 j holds
+  // columns of the first, 2 j + 1 the same columns of the second; p.Nt = 2 NtR counts both) and the epilogue multiplies the
+  // pairs: act0(A W0) x act1(A W1), e.g. SiLU(gate) x up, without either factor leaving the registers
+  static_assert(!GLU || (WF == WF_BFP8 && !IMG && BN_ == 2 * NTW && NTW % 2 == 0), "the gated form exists for the fused bfp8_b kernel");
   static_assert(BN_ == 2 * NTW || (IMG && BN_ == 7 && (NTW == 4 || NTW == 3)), "uneven blocks exist for the second pass only");
   constexpr int MB = 2;          // row tiles (32 m) per wavefront
   constexpr int BN = BN_;        // column tiles per block
@@ -892,8 +940,10 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   const int nb = bid / p.m_blocks, mb = bid % p.m_blocks;
   const int mt0 = mb * 8, nt0 = nt_first + nb * BN;
   const uint8_t *A = p.A + (int64_t)blockIdx.z * p.a_batch;
-  const uint8_t *W = p.W + (int64_t)blockIdx.z * p.w_batch;
-  uint8_t *C = p.C + (int64_t)blockIdx.z * p.c_batch;
+  const uint8_t *W = GLU ? p.gW[0] : p.W + (int64_t)blockIdx.z * p.w_batch;
+  const uint8_t *W1 = GLU ? p.gW[1] : W;                  // GLU: the matrix of the odd tile slots
+  uint8_t *C = GLU ? p.gC[0] : p.C + (int64_t)blockIdx.z * p.c_batch;
+  const int NtW = GLU ? p.gNt[0] : p.Nt;                  // column tiles of a weight matrix (GLU: p.Nt counts both matrices)
   constexpr uint32_t LDS_W = 65536, LDS_RAW = 131072, STAGE = 32768;
   constexpr uint32_t RAW_TILE = WF == WF_BFP8 ? 1024u : 512u, RAW_STAGE = 16 * RAW_TILE;
   constexpr uint32_t W_TILE = WF == WF_BFP8 ? 1088u : 576u;
@@ -933,7 +983,8 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     if constexpr (WF == WF_BFP8) rawRd = LDS_RAW + tile_l * 1024 + a * 128 + ((a ^ (tile_l & 1)) << 4) + quad * 4;
     else rawRd = LDS_RAW + tile_l * 512 + a * 64 + quad * 2;
   }
-  const uint32_t offWe = (uint32_t)min(nt0 + unt, p.Nt - 1) * W_TILE + face * 16 + khalf * 8;
+  const uint32_t offWe = (uint32_t)min(GLU ? (nt0 + unt) >> 1 : nt0 + unt, NtW - 1) * W_TILE + face * 16 + khalf * 8;
+  const uint8_t *We = GLU && (unt & 1) ? W1 : W;          // per lane: the matrix its tile slot belongs to
   // LDS-direct loads of the activations: wavefront w fills rows 32 w .. 32 w + 31 (row tile mt0 + w) with four
   // instructions of 8 rows each; lane l writes slot l & 7 of row 8 i + (l >> 3), i.e. k-chunk slot ^ swizzle(row)
   uint32_t dmaA[4];
@@ -953,9 +1004,9 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     const int a = lane >> 3;
     dmaW = 64u + (uint32_t)(8 * a + ((lane & 7) ^ a)) * 16u;   // tile parity is folded in at the call site (XOR 16)
 #pragma unroll
-    for (int x = 0; x < 2; ++x) w_col[x] = (int64_t)min(nt0 + 2 * (wave & 3) + x, p.Nt - 1) * W_TILE;
+    for (int x = 0; x < 2; ++x) w_col[x] = (int64_t)min(GLU ? (nt0 + 2 * (wave & 3)) >> 1 : nt0 + 2 * (wave & 3) + x, NtW - 1) * W_TILE;
   } else {
-    dmaW = (uint32_t)(min(nt0 + 2 * (wave & 3) + (lane >> 5), p.Nt - 1) * (int)W_TILE) + 64u + (uint32_t)(lane & 31) * 16u;
+    dmaW = (uint32_t)(min(nt0 + 2 * (wave & 3) + (lane >> 5), NtW - 1) * (int)W_TILE) + 64u + (uint32_t)(lane & 31) * 16u;
   }
 
   // split-K: this block reduces k-tiles [kbase, kt_end); k-tiles past kt_end get zero weights
@@ -990,11 +1041,11 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     if constexpr (IMG) return;
     if (!converts) return;
     const int kt = min(kbase + kt0 + ukt, p.Kt - 1);
-    const uint8_t *row = W + (int64_t)kt * p.Nt * W_TILE;
+    const uint8_t *row = W + (int64_t)kt * NtW * W_TILE;
     if constexpr (WF == WF_BFP8) {
 #pragma unroll
       for (int x = 0; x < 2; ++x)
-        lds_dma16(row + w_col[x], dmaW ^ (x << 4), lds0 + LDS_RAW + stage_off + (uint32_t)(2 * wave + x) * 1024u);
+        lds_dma16((GLU && x ? W1 + (int64_t)kt * NtW * W_TILE : row) + w_col[x], dmaW ^ (x << 4), lds0 + LDS_RAW + stage_off + (uint32_t)(2 * wave + x) * 1024u);
     } else {
       lds_dma16(row, dmaW, lds0 + LDS_RAW + stage_off + (uint32_t)(2 * wave) * 512u);
     }
@@ -1007,7 +1058,7 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
     kt0 += kbase;
     const int kt = min(kt0 + ukt, p.Kt - 1);
     keep = kt0 + ukt >= kt_end ? 0u : 0xFFFFFFFFu;
-    return *(const u32x2 *)(W + (int64_t)kt * p.Nt * W_TILE + offWe);
+    return *(const u32x2 *)(We + (int64_t)kt * NtW * W_TILE + offWe);
   };
   auto fetch = [&](int s2, uint32_t so, u32x4 (&w)[NTW], u32x4 (&a)[MB]) {
 #pragma unroll
@@ -1134,8 +1185,9 @@ __device__ __forceinline__ void linear_dma_block(const LinearArgs &p, int bid, i
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be in flight towards LDS when the block ends
 
-  if (p.partial) linear_store_partial(p, p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * ((int64_t)p.Mt * p.Nt * 1024), acc,
-                                      mt0 + wm * MB, nt0 + wcol, nt_end, lane);
+  if constexpr (GLU) linear_epilogue_glu(p, C, acc, mt0 + wm * MB, nt0 + wcol, nt_end, NtW, lane);
+  else if (p.partial) linear_store_partial(p, p.partial + ((int64_t)blockIdx.z * gridDim.y + blockIdx.y) * ((int64_t)p.Mt * p.Nt * 1024), acc,
+                                           mt0 + wm * MB, nt0 + wcol, nt_end, lane);
   else linear_epilogue_act(p, C, acc, mt0 + wm * MB, nt0 + wcol, nt_end, lane);
 }
 
@@ -1333,6 +1385,11 @@ __global__ __launch_bounds__(512) void ttm_linear_dma_k(LinearArgs p) {
   if (ntw == 4) linear_dma_block<WF, 4>(p, bid, nblk, first, end);
   else if (ntw == 3) linear_dma_block<WF, 3>(p, bid, nblk, first, end);
   else linear_dma_block<WF, 2>(p, bid, nblk, first, end);
+}
+
+// the gated form of the fused kernel (bfp8_b): blocks of eight tile slots = four column tiles of either matrix
+__global__ __launch_bounds__(512) void ttm_linear_dma_glu_k(LinearArgs p) {
+  linear_dma_block<WF_BFP8, 4, false, 8, true>(p, blockIdx.x, gridDim.x, 0, p.Nt);
 }
 
 template <int WF, bool M16 = true>   // M16: v_mfma_f32_16x16x32_bf16 (linear_img16_block); else 32x32x16
@@ -2391,7 +2448,26 @@ static bool decode_runs_unsplit(int64_t N, int64_t K) {
   return slices <= 1;
 }
 
+// Token counts at which the gated form of the fused main kernel is used: those where the two projections would otherwise
+// share one launch and leave their product to an element-wise kernel (a projection alone would split K to fill the device).
+static bool glu_main_ok(int w_dtype, int64_t M, int64_t N, int64_t K) {
+  const int64_t Mt = ttm_cdiv(M, 32), Nt = ttm_cdiv(N, 32), Kt = ttm_cdiv(K, 32);
+  const int variant = ttm_option("linear_variant");
+  if (!(w_dtype == TTM_BFP8B && M > 64 && M <= 1024 && M > ttm_option("linear_small_m_max") && (variant == 0 || variant == 6) &&
+        ttm_option("linear_two_pass") != 2 && ttm_option("linear_glu_main") != 1 && Mt * Kt * 2048 < (int64_t)1 << 32 &&
+        Nt * Kt * 2048 < (int64_t)1 << 32 && Nt * 1088 < (int64_t)1 << 31))
+    return false;
+  if (ttm_option("linear_two_pass") == 1) return true;
+  // where launch_linear's model sends the group of the two projections through the image pass, the two passes and an
+  // element-wise multiply are the faster sequence (the gated kernel converts its weights in every block of 256 rows)
+  const int cus = device_cu_count();
+  const int64_t ksteps = (Kt + 1) / 2, blocks = ttm_cdiv(Mt, 8) * ttm_cdiv(2 * Nt, 8), rounds = (blocks + cus - 1) / cus;
+  const double fused = rounds * (ksteps + 12) * 1.65, first = 3.0 + (double)Kt * 2 * Nt * (1088.0 + 2048.0) / 5.5e6;
+  return !(0.28 * fused > first);
+}
+
 TTM_EXPORT int ttm_linear_glu_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
+  if (M >= 1 && K > 0 && N >= 1 && glu_main_ok(w_dtype, M, N, K)) return 1;
   return (w_dtype == TTM_BFP8B || w_dtype == TTM_BFP4B) && M >= 1 && M <= 32 && K > 0 && N >= 1 && ttm_option("linear_variant") != 1 &&
          ttm_option("linear_decode_wide") != 1 && ttm_option("linear_small_m_max") >= 32 && ttm_cdiv(N, 32) * 1088 < (int64_t)1 << 32 &&
          decode_runs_unsplit(N, K);
@@ -2401,7 +2477,7 @@ TTM_EXPORT int ttm_linear_glu(const void *a, const void *w_gate, const void *w_u
                               int act_gate, int act_up, void *stream) {
   TTM_EXTENTS(linear_glu, a, w_gate, w_up, w_dtype, out, M, N, K);
   TTM_REQUIRE(ttm_linear_glu_supported(w_dtype, M, N, K),
-              "ttm_linear_glu: needs block-float weights, 1..32 rows and enough columns for the decode kernel to run unsplit");
+              "ttm_linear_glu: needs block-float weights and 1..32 rows with enough columns for the decode kernel to run unsplit, or bfp8_b weights and 65..1024 rows");
   TTM_REQUIRE(a && w_gate && w_up && out, "ttm_linear_glu: null pointer");
   TTM_REQUIRE((((uintptr_t)a | (uintptr_t)w_gate | (uintptr_t)w_up | (uintptr_t)out) & 15) == 0, "ttm_linear_glu: operands must be 16-byte aligned");
   TTM_REQUIRE(act_gate >= TTM_ACT_NONE && act_gate <= TTM_ACT_RELU && act_up >= TTM_ACT_NONE && act_up <= TTM_ACT_RELU,
@@ -2423,6 +2499,20 @@ TTM_EXPORT int ttm_linear_glu(const void *a, const void *w_gate, const void *w_u
   p.tail = TTM_TAIL_NONE; p.tail_delta = 0;
   p.qkv = nullptr; p.norm = nullptr;
   hipStream_t s = (hipStream_t)stream;
+  if (M > 32) {   // the fused main kernel over the tile slots of both matrices: blocks of 256 rows x four column tiles of each
+    p.Mt = (int)ttm_cdiv(M, 32);
+    p.Nt = 2 * p.gNt[0];
+    p.m_blocks = (p.Mt + 7) / 8;
+    p.n_blocks = p.m_blocks * ((p.Nt + 7) / 8);
+    static bool attr = false;
+    if (!attr) {
+      if (int rc = set_lds_limit(ttm_linear_dma_glu_k, 131072 + 32768)) return rc;
+      attr = true;
+    }
+    hipLaunchKernelGGL(ttm_linear_dma_glu_k, dim3((unsigned)p.n_blocks), dim3(512), 131072 + 32768, s, p);
+    TTM_LAUNCH_CHECK();
+    return TTM_OK;
+  }
   const int rc = w_dtype == TTM_BFP8B ? launch_linear<WF_BFP8>(p, 1, s) : launch_linear<WF_BFP4>(p, 1, s);
   if (rc) return rc;
   TTM_LAUNCH_CHECK();

@@ -672,7 +672,7 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
       if (shape2.size() != outShape.size() || shape2.empty() || !std::equal(shape2.begin(), shape2.end() - 1, outShape.begin()) ||
           shape2.back() != wit->second.handle->shape[1])
         break;
-      if (!midM) {   // its own element-wise tail, if it has one, is worth more than the shared launch
+      {   // its own element-wise tail, if it has one, is worth more than the shared launch (not at the middle token counts)
         std::uint32_t after = j + 1;
         while (after < ctx.ops.size() && opType(after) == OpType::DeallocateOp) ++after;
         if (after < ctx.ops.size() && opType(after) == OpType::EltwiseBinaryOp) {
@@ -685,7 +685,7 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
             const std::uint32_t mine = refId(outRef), theirs = refId(out2);
             auto usesOf = [&](std::uint32_t id) { auto u = ctx.uses.find(id); return u == ctx.uses.end() ? 0u : u->second; };
             const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
-            if (decodeFusionEnabled() && followers.empty() && as_.size() == 2 && bop.scalar<std::uint32_t>(schema::EltwiseBinaryOp::f_type, 0) == 1 && l && r && bout &&
+            if ((decodeFusionEnabled() || M > 32) && followers.empty() && as_.size() == 2 && bop.scalar<std::uint32_t>(schema::EltwiseBinaryOp::f_type, 0) == 1 && l && r && bout &&
                 ((refId(l) == mine && refId(r) == theirs) || (refId(l) == theirs && refId(r) == mine)) && usesOf(mine) == 1 &&
                 usesOf(theirs) == 1 && shape2 == outShape && shapeFromTensorRef(bout) == outShape && layoutFromTensorRef(bout) == plain &&
                 wit->second.handle->shape[1] == b.handle->shape[1] && wit->second.handle->data.get() != b.handle->data.get() &&
@@ -699,7 +699,7 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
               debug::Stats::get().incrementStat("FusedLinearGlu");
               return;
             }
-            break;
+            if (!midM) break;
           }
         }
       }
