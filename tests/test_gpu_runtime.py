@@ -142,6 +142,31 @@ def test_c4_mlp_program_small(device, orc, metrics):
     assert metrics.get_pcc(want, f(y)) >= 0.999
 
 
+def test_mlp_gate_up_product_in_one_launch_at_mid_token_counts(device, orc):
+    """96 tokens with bfp8_b gate / up weights: with the image pass ruled out the executor binds ttm_linear_glu (the gated main
+    kernel) for the two matmuls and their multiply; ragged widths; the result equals the run that keeps them apart, bit for bit."""
+    from ttmlir_amd import hip
+    T, H, F = 96, 160, 416     # 13 column tiles per matrix: the last block of the gated kernel holds one tile of each
+    d = datagen.c4_mlp(tokens=T, hidden=H, ffn=F, seed=9)
+    binary = rt.Binary.load_from_memory(programs.c4_mlp(T, H, F))
+    tins = [d["x"], d["norm_w"], bf(d["wg"]), bf(d["wu"]), bf(d["wd"])]
+    hip.set_option("linear_two_pass", 1)
+    try:
+        rt.clear_stats()
+        (y,) = harness.execute(binary, 1, tins, device)
+        assert rt.get_stat("FusedLinearGlu") == 1 and rt.get_stat("GroupedMatmul") == 0
+        hip.set_option("linear_glu_main", 1)
+        (y_ops,) = harness.execute(binary, 1, tins, device)
+        assert rt.get_stat("FusedLinearGlu") == 1 and rt.get_stat("GroupedMatmul") == 1
+    finally:
+        hip.set_option("linear_glu_main", 0)
+        hip.set_option("linear_two_pass", 0)
+    assert torch.equal(y, y_ops)
+    f = lambda t: t.float().numpy()
+    want = oracle_mlp(orc, f(d["x"]), f(d["norm_w"]), f(bf(d["wg"])), f(bf(d["wu"])), f(bf(d["wd"])), 1e-5)
+    assert np.max(np.abs(f(y) - want)) <= 2.0 ** -10
+
+
 def test_c4_mlp_full_size(device, orc, metrics):
     """Config 4 at its real shape (512 tokens, 4096 -> 14336 -> 4096), all 512 x 4096 outputs against the oracle."""
     d = datagen.c4_mlp()

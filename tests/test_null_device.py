@@ -33,6 +33,7 @@ def null_env(tmp_path_factory):
     # the runtime library finds the kernel library through its RUNPATH, which LD_LIBRARY_PATH precedes
     env["LD_LIBRARY_PATH"] = str(d) + os.pathsep + env.get("LD_LIBRARY_PATH", "")
     env["TTMLIR_AMD_NULL_DEVICE"] = "1"
+    env["TTMLIR_AMD_HIP_LIB"] = str(d / "libttmlir_amd_hip.so")   # the Python binding's options reach the same library
     return env
 
 
