@@ -355,7 +355,7 @@ MEASURED_TRAFFIC_BYTES = {
     "sdpa_decode32": (270.3e6, "ttm_decode.hip"), "sdpa2048": (42.3e6, "ttm_sdpa.hip"), "rmsnorm2048": (34.0e6, "ttm_rowwise.hip"),
     "softmax65536": (1073.8e6, "ttm_rowwise.hip"), "reduce65536": (545.2e6, "ttm_rowwise.hip"), "silu_mul512": (44.2e6, "ttm_eltwise.hip"),
 }
-MEASURED_ON = {"ttm_linear.hip": ("03b7b80fdaa8",), "ttm_bfp.hip": ("cdf35c7592c1",), "ttm_layout.hip": ("a6cf1c428342",),
+MEASURED_ON = {"ttm_linear.hip": ("875295d3c654",), "ttm_bfp.hip": ("cdf35c7592c1",), "ttm_layout.hip": ("a6cf1c428342",),
                "ttm_decode.hip": ("3bd99843ac98",), "ttm_rowwise.hip": ("0819544c7ff3",), "ttm_eltwise.hip": ("62019175607e",),
                "ttm_sdpa.hip": ("3c1e7f59da68",)}
 TRAFFIC_HOW = ("rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs), KiB per dispatch scaled by what the same counters "

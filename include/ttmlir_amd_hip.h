@@ -150,8 +150,8 @@ int ttm_linear_pair(const void *a, const void *w0, const void *w1, int w_dtype, 
  * (runtime/lib/ttnn/operations/matmul/matmul.cpp:47-83, eltwise/binary/binary.cpp:38-126).
  * ttm_linear_glu_supported returns 1 when the shapes and the selected kernel variants allow it, else 0: block-float weights,
  * M <= 32 and enough columns that one projection alone would not split K over workgroups; or BFP_BFloat8 weights,
- * 65 <= M <= 1024 and a shape whose pair of projections the library would run in one pass (where it would first rewrite
- * the weights as bf16 images, that sequence stays the faster one). */
+ * 65 <= M <= 1024 and a shape at which the library's cost model puts this launch ahead of the grouped projections followed
+ * by a multiply (narrow weight matrices, which are cheap to rewrite as bf16 images first, stay with that sequence). */
 int ttm_linear_glu_supported(int w_dtype, int64_t M, int64_t N, int64_t K);
 int ttm_linear_glu(const void *a, const void *w_gate, const void *w_up, int w_dtype, void *out, int64_t M, int64_t N, int64_t K,
                    int act_gate, int act_up, void *stream);

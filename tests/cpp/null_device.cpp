@@ -420,7 +420,8 @@ EXPORT int ttm_linear_glu_supported(int w_dtype, int64_t M, int64_t N, int64_t K
     // the gated form of the fused main kernel, where the real library's model keeps the pair of projections in one pass (256 CUs)
     const int64_t ksteps = (kt + 1) / 2, nt = (N + 31) / 32, blocks = ((M + 255) / 256) * ((2 * nt + 7) / 8), rounds = (blocks + 255) / 256;
     const double fused = rounds * (ksteps + 12) * 1.65, first = 3.0 + static_cast<double>(kt) * 2 * nt * (1088.0 + 2048.0) / 5.5e6;
-    if (g_options["linear_two_pass"] == 1 || !(0.28 * fused > first)) return 1;
+    const double multiply = 3.0 + 3.0 * static_cast<double>((M + 31) / 32) * nt * 2048.0 / 5.5e6;
+    if (g_options["linear_two_pass"] == 1 || !(0.28 * fused - first > multiply)) return 1;
   }
   return block_float(w_dtype) && M >= 1 && M <= 32 && K > 0 && N >= 1 && std::min<int64_t>(256 / groups, kt / 32) <= 1;
 }

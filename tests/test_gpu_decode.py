@@ -617,5 +617,7 @@ def test_linear_glu_main_kernel_equals_the_op_sequence(hip, dev, orc, M, K, N, a
     # bfp4_b weights and the token counts between the two forms stay with the op sequence
     assert hip.lib().ttm_linear_glu_supported(hip.BFP4B, M, N, K) == 0 and hip.lib().ttm_linear_glu_supported(wf, 48, N, K) == 0
     assert hip.lib().ttm_linear_glu_supported(wf, 2048, N, K) == 0
-    # by default it follows the library's model of the image pass: config 4 stays in one pass, twice its rows take two
-    assert hip.lib().ttm_linear_glu_supported(wf, 512, 14336, 4096) == 1 and hip.lib().ttm_linear_glu_supported(wf, 1024, 14336, 4096) == 0
+    # by default it weighs the library's model of the image pass against the multiply it saves: config 4's shape takes the gated
+    # kernel up to 1024 rows, a square weight (cheap to rewrite as images, few blocks for the gated kernel) does not
+    assert hip.lib().ttm_linear_glu_supported(wf, 512, 14336, 4096) == 1 and hip.lib().ttm_linear_glu_supported(wf, 1024, 14336, 4096) == 1
+    assert hip.lib().ttm_linear_glu_supported(wf, 512, 4096, 4096) == 0

@@ -2458,12 +2458,16 @@ static bool glu_main_ok(int w_dtype, int64_t M, int64_t N, int64_t K) {
         Nt * Kt * 2048 < (int64_t)1 << 32 && Nt * 1088 < (int64_t)1 << 31))
     return false;
   if (ttm_option("linear_two_pass") == 1) return true;
-  // where launch_linear's model sends the group of the two projections through the image pass, the two passes and an
-  // element-wise multiply are the faster sequence (the gated kernel converts its weights in every block of 256 rows)
+  // The other sequence is the group launch of the two projections and an element-wise multiply.  Where launch_linear's model
+  // sends the group through the image pass (the gated kernel converts its weights in every block of 256 rows), that sequence
+  // wins if the image pass gains more than the multiply costs (3 us + three tensors of M x N bf16 at 5.5 TB/s).  Measured,
+  // sequence / gated in us, K x N = 4096 x 14336: M = 128 105 / 101, 512 138 / 125, 768 248 / 226, 1024 311 / 240;
+  // 4096 x 4096: 512 84 / 99, 1024 102 / 110; 1024 x 2816: 1024 35 / 37; 2048 x 8192: 1024 91 / 77; 8192 x 28672: 512 508 / 491.
   const int cus = device_cu_count();
   const int64_t ksteps = (Kt + 1) / 2, blocks = ttm_cdiv(Mt, 8) * ttm_cdiv(2 * Nt, 8), rounds = (blocks + cus - 1) / cus;
   const double fused = rounds * (ksteps + 12) * 1.65, first = 3.0 + (double)Kt * 2 * Nt * (1088.0 + 2048.0) / 5.5e6;
-  return !(0.28 * fused > first);
+  const double multiply = 3.0 + 3.0 * (double)Mt * Nt * 2048.0 / 5.5e6;
+  return !(0.28 * fused - first > multiply);
 }
 
 TTM_EXPORT int ttm_linear_glu_supported(int w_dtype, int64_t M, int64_t N, int64_t K) {
