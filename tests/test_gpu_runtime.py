@@ -254,6 +254,30 @@ def test_c5_decoder_layer_small(device, orc, metrics):
     assert metrics.get_pcc(want, got) >= 0.9999
 
 
+def test_decoder_layer_mlp_takes_the_gated_kernel_on_rank_three_activations(device, orc):
+    """The small decoder layer (activations [1, 96, 256]) with the image pass ruled out: gate, up and their product are one
+    launch although the activations have a batch dimension of one in front; the layer's output equals the run that keeps
+    them apart bit for bit, and the oracle's within the small layer's bar."""
+    from ttmlir_amd import hip
+    d = datagen.c5_decoder(seq=96, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, seed=4)
+    binary = rt.Binary.load_from_memory(programs.c5_decoder(96, 256, 4, 2, 64, 512))
+    tins = [d["x"], d["attn_norm_w"], bf(d["wq"]), bf(d["wk"]), bf(d["wv"]), bf(d["wo"]), d["mlp_norm_w"], bf(d["wg"]), bf(d["wu"]),
+            bf(d["wd"])]
+    hip.set_option("linear_two_pass", 1)
+    try:
+        rt.clear_stats()
+        (y,) = harness.execute(binary, 1, tins, device)
+        assert rt.get_stat("FusedLinearGlu") == 1
+        hip.set_option("linear_glu_main", 1)
+        (y_ops,) = harness.execute(binary, 1, tins, device)
+        assert rt.get_stat("FusedLinearGlu") == 1
+    finally:
+        hip.set_option("linear_glu_main", 0)
+        hip.set_option("linear_two_pass", 0)
+    assert torch.equal(y, y_ops)
+    assert np.max(np.abs(y.float().numpy() - oracle_decoder(orc, d))) <= 2.0 ** -5
+
+
 def test_c5_decoder_layer_small_row_subset(device, orc):
     """The oracle evaluated on a subset of token rows is the full evaluation restricted to those rows, bit for bit."""
     d = datagen.c5_decoder(seq=96, hidden=256, n_q=4, n_kv=2, head_dim=64, ffn=512, seed=4)

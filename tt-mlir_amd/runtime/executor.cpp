@@ -685,7 +685,7 @@ void runMatmulLike(ProgramContext &ctx, const fb::Table &aRef, const fb::Table &
             const std::uint32_t mine = refId(outRef), theirs = refId(out2);
             auto usesOf = [&](std::uint32_t id) { auto u = ctx.uses.find(id); return u == ctx.uses.end() ? 0u : u->second; };
             const Layout plain{StorageType::Device, TensorLayout::Tile, DataType::BFloat16};
-            if ((decodeFusionEnabled() || M > 32) && followers.empty() && as_.size() == 2 && bop.scalar<std::uint32_t>(schema::EltwiseBinaryOp::f_type, 0) == 1 && l && r && bout &&
+            if ((decodeFusionEnabled() || M > 32) && followers.empty() && as_.size() >= 2 && bop.scalar<std::uint32_t>(schema::EltwiseBinaryOp::f_type, 0) == 1 && l && r && bout &&
                 ((refId(l) == mine && refId(r) == theirs) || (refId(l) == theirs && refId(r) == mine)) && usesOf(mine) == 1 &&
                 usesOf(theirs) == 1 && shape2 == outShape && shapeFromTensorRef(bout) == outShape && layoutFromTensorRef(bout) == plain &&
                 wit->second.handle->shape[1] == b.handle->shape[1] && wit->second.handle->data.get() != b.handle->data.get() &&
